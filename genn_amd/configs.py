@@ -1,0 +1,309 @@
+"""Synthetic-input generators for the benchmark configurations (and reduced-scale twins).
+
+Every array comes from :mod:`genn_amd.rng`; a (config, scale, seed) triple therefore names
+one exact network.  Rows are sorted by postsynaptic index, as the reference's built-in
+connectivity snippets and ``set_sparse_connections`` produce them
+(pygenn/genn_groups.py:447-460).
+"""
+import math
+
+import numpy as np
+
+from . import rng
+from .netspec import Net, Pop, CurrentSource, Syn
+
+
+# --------------------------------------------------------------------------------------------
+# connectivity builders (all return rowLength[numPre], ind[numPre,stride])
+# --------------------------------------------------------------------------------------------
+def fixed_probability(seed, stream, n_pre, n_post, p, pad=1):
+    """Bernoulli(p) per (pre,post) pair via geometric skips — the process of
+    include/genn/genn/initSparseConnectivitySnippet.h:170-187, driven by the repo's own
+    generator.  Row r uses counters [r*K, (r+1)*K) of ``stream``."""
+    mean = n_post * p
+    K = int(mean + 8.0 * math.sqrt(mean * (1 - p)) + 16)
+    logq = math.log1p(-p)
+    row_length = np.zeros(n_pre, dtype=np.uint32)
+    rows = []
+    chunk = max(1, (1 << 22) // K)
+    for r0 in range(0, n_pre, chunk):
+        r1 = min(n_pre, r0 + chunk)
+        u = rng.uniform_open(seed, stream, r0 * K, (r1 - r0) * K).reshape(r1 - r0, K)
+        skips = np.floor(np.log(u) / logq).astype(np.int64) + 1
+        pos = np.cumsum(skips, axis=1) - 1
+        valid = pos < n_post
+        if valid[:, -1].any():
+            raise RuntimeError("fixed_probability: candidate budget too small")
+        row_length[r0:r1] = valid.sum(axis=1)
+        rows.append((pos, valid))
+    stride = int(max(1, row_length.max()))
+    stride = ((stride + pad - 1) // pad) * pad
+    ind = np.zeros((n_pre, stride), dtype=np.uint32)
+    r0 = 0
+    for pos, valid in rows:
+        n = pos.shape[0]
+        w = min(stride, pos.shape[1])
+        ind[r0:r0 + n, :w] = np.where(valid[:, :w], pos[:, :w], 0)
+        r0 += n
+    return row_length, ind
+
+
+def fixed_number_post(seed, stream, n_pre, n_post, fanout):
+    """Every row draws ``fanout`` targets uniformly with replacement, then sorts them
+    (shape of FixedNumberPostWithReplacement, initSparseConnectivitySnippet.h:242-276)."""
+    ind = np.empty((n_pre, fanout), dtype=np.uint32)
+    chunk = max(1, (1 << 24) // fanout)
+    for r0 in range(0, n_pre, chunk):
+        r1 = min(n_pre, r0 + chunk)
+        x = rng.randint(seed, stream, r0 * fanout, (r1 - r0) * fanout, n_post).reshape(r1 - r0, fanout)
+        x.sort(axis=1)
+        ind[r0:r1] = x
+    return np.full(n_pre, fanout, dtype=np.uint32), ind
+
+
+def fixed_number_total(seed, stream, n_pre, n_post, total, pad=1):
+    """``total`` (pre,post) pairs uniformly with replacement (multapses allowed), sorted
+    (shape of FixedNumberTotalWithReplacement, initSparseConnectivitySnippet.h:292-370)."""
+    keys = np.empty(total, dtype=np.uint64)
+    chunk = 1 << 24
+    for c0 in range(0, total, chunk):
+        c = min(chunk, total - c0)
+        pre = rng.randint(seed, stream, c0, c, n_pre).astype(np.uint64)
+        post = rng.randint(seed, stream + 0x20000000, c0, c, n_post).astype(np.uint64)
+        keys[c0:c0 + c] = pre * np.uint64(n_post) + post
+    keys.sort()
+    pre = (keys // np.uint64(n_post)).astype(np.int64)
+    post = (keys % np.uint64(n_post)).astype(np.uint32)
+    row_length = np.bincount(pre, minlength=n_pre).astype(np.uint32)
+    stride = int(max(1, row_length.max()))
+    stride = ((stride + pad - 1) // pad) * pad
+    starts = np.concatenate(([0], np.cumsum(row_length)[:-1])).astype(np.int64)
+    within = np.arange(total, dtype=np.int64) - starts[pre]
+    ind = np.zeros((n_pre, stride), dtype=np.uint32)
+    ind[pre, within] = post
+    return row_length, ind, (pre, within)
+
+
+def _fill_rows(row_length, stride, values):
+    """Scatter a flat per-synapse array (row-major over valid entries) into padded layout."""
+    n_pre = len(row_length)
+    out = np.zeros((n_pre, stride), dtype=values.dtype)
+    mask = np.arange(stride)[None, :] < row_length[:, None]
+    out[mask] = values
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# C1: balanced LIF network (Vogels-Abbott shape)
+# --------------------------------------------------------------------------------------------
+def vogels_abbott(n=4000, steps=10000, seed=1234, p=0.02, dt=0.1, ioffset=0.55):
+    n_e = (n * 4) // 5
+    n_i = n - n_e
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=ioffset, TauRefrac=5.0)
+    net = Net(name="va", dt=dt, steps=steps, seed=seed)
+    for k, (name, num) in enumerate((("E", n_e), ("I", n_i))):
+        v0 = (-60.0 + 10.0 * rng.uniform(seed, 1 + k, 0, num)).astype(np.float32)
+        net.pops.append(Pop(name, "lif", num, dict(lif), {"V": v0, "RefracTime": np.zeros(num, np.float32)}))
+    stream = 16
+    for src, n_src, w, tau in (("E", n_e, 0.5, 5.0), ("I", n_i, -2.25, 10.0)):
+        for trg, n_trg in (("E", n_e), ("I", n_i)):
+            rl, ind = fixed_probability(seed, stream, n_src, n_trg, p)
+            stream += 1
+            g = np.where(np.arange(ind.shape[1])[None, :] < rl[:, None], np.float32(w), np.float32(0)).astype(np.float32)
+            net.syns.append(Syn(f"{src}{trg}", src, trg, wum="static", psm="expcurr", tau=tau,
+                                row_stride=ind.shape[1], row_length=rl, ind=ind, g=g))
+    return net
+
+
+def clipped_normal(seed, stream, count, mean, sd, lo, hi):
+    """Normal(mean, sd) resampled until inside [lo, hi] (the rule of NormalClipped,
+    include/genn/genn/initVarSnippet.h:161-176).  Element k tries counters k, k+count, ..."""
+    out = mean + sd * rng.normal(seed, stream, 0, count)
+    bad = np.flatnonzero((out > hi) | (out < lo))
+    attempt = 1
+    while bad.size:
+        # counters of the retry are count*attempt + k, gathered sparsely
+        z = np.empty(bad.size)
+        for j, k in enumerate(bad):       # rare path: a handful of elements per million
+            z[j] = rng.normal(seed, stream, attempt * count + int(k), 1)[0]
+        cand = mean + sd * z
+        ok = (cand <= hi) & (cand >= lo)
+        out[bad[ok]] = cand[ok]
+        bad = bad[~ok]
+        attempt += 1
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# C2: Potjans-Diesmann cortical microcircuit (constants: userproject/potjans_microcircuit.py:27-100)
+# --------------------------------------------------------------------------------------------
+PD_LAYERS = ("23", "4", "5", "6")
+PD_NUM = {"23E": 20683, "23I": 5834, "4E": 21915, "4I": 5479, "5E": 4850, "5I": 1065, "6E": 14395, "6I": 2948}
+PD_PROB = {  # [target][source]
+    "23E": {"23E": 0.1009, "23I": 0.1689, "4E": 0.0437, "4I": 0.0818, "5E": 0.0323, "5I": 0.0, "6E": 0.0076, "6I": 0.0},
+    "23I": {"23E": 0.1346, "23I": 0.1371, "4E": 0.0316, "4I": 0.0515, "5E": 0.0755, "5I": 0.0, "6E": 0.0042, "6I": 0.0},
+    "4E": {"23E": 0.0077, "23I": 0.0059, "4E": 0.0497, "4I": 0.135, "5E": 0.0067, "5I": 0.0003, "6E": 0.0453, "6I": 0.0},
+    "4I": {"23E": 0.0691, "23I": 0.0029, "4E": 0.0794, "4I": 0.1597, "5E": 0.0033, "5I": 0.0, "6E": 0.1057, "6I": 0.0},
+    "5E": {"23E": 0.1004, "23I": 0.0622, "4E": 0.0505, "4I": 0.0057, "5E": 0.0831, "5I": 0.3726, "6E": 0.0204, "6I": 0.0},
+    "5I": {"23E": 0.0548, "23I": 0.0269, "4E": 0.0257, "4I": 0.0022, "5E": 0.06, "5I": 0.3158, "6E": 0.0086, "6I": 0.0},
+    "6E": {"23E": 0.0156, "23I": 0.0066, "4E": 0.0211, "4I": 0.0166, "5E": 0.0572, "5I": 0.0197, "6E": 0.0396, "6I": 0.2252},
+    "6I": {"23E": 0.0364, "23I": 0.001, "4E": 0.0034, "4I": 0.0005, "5E": 0.0277, "5I": 0.008, "6E": 0.0658, "6I": 0.1443}}
+PD_EXT = {"23E": 1600, "23I": 1500, "4E": 2100, "4I": 1900, "5E": 2000, "5I": 1900, "6E": 2900, "6I": 2100}
+PD_RATE = {"23E": 0.971, "23I": 2.868, "4E": 4.746, "4I": 5.396, "5E": 8.142, "5I": 9.078, "6E": 0.991, "6I": 7.523}
+PD_MEAN_W = 87.8e-3
+PD_G = -4.0
+PD_BG_RATE = 8.0
+PD_MEAN_DELAY = {"E": 1.5, "I": 0.75}
+PD_DELAY_SD = {"E": 0.75, "I": 0.375}
+PD_NORM_Q9999 = 3.719016485455709     # scipy.stats.norm.ppf(0.9999)
+
+
+def pd_full_num_inputs(src, trg):
+    n_src, n_trg = PD_NUM[src], PD_NUM[trg]
+    p = PD_PROB[trg][src]
+    if p == 0.0:
+        return 0
+    return int(round(math.log(1.0 - p) / math.log(float(n_trg * n_src - 1) / float(n_trg * n_src))) / n_trg)
+
+
+def pd_mean_weight(src, trg):
+    if src.endswith("E"):
+        return 2.0 * PD_MEAN_W if (src == "4E" and trg == "23E") else PD_MEAN_W
+    return PD_G * PD_MEAN_W
+
+
+def potjans(neuron_scale=1.0, connectivity_scale=1.0, steps=10000, seed=4321, dt=0.1, pad=1):
+    """Background Poisson input (PoissonExp, currentSourceModels.h:107-129) is replaced by a DC
+    source with the same stationary mean, w * tauSyn * rate[1/ms]."""
+    pops = [l + p for l in PD_LAYERS for p in ("E", "I")]
+    max_delay = {k: PD_MEAN_DELAY[k] + PD_DELAY_SD[k] * PD_NORM_Q9999 for k in ("E", "I")}
+    slots = int(round(max(max_delay.values()) / dt))
+    net = Net(name="potjans", dt=dt, steps=steps, fuse_psm=True, seed=seed)
+    size = {}
+    for k, name in enumerate(pops):
+        n = int(round(neuron_scale * PD_NUM[name]))
+        size[name] = n
+        full_in = sum(pd_mean_weight(s, name) * pd_full_num_inputs(s, name) * PD_RATE[s] for s in pops)
+        full_in += PD_MEAN_W * PD_EXT[name] * PD_BG_RATE
+        ioff = 0.001 * 0.5 * (1.0 - math.sqrt(connectivity_scale)) * full_in
+        v0 = (-58.0 + 5.0 * rng.normal(seed, 1 + k, 0, n)).astype(np.float32)
+        net.pops.append(Pop(name, "lif", n,
+                            dict(C=0.25, TauM=10.0, Vrest=-65.0, Vreset=-65.0, Vthresh=-50.0, Ioffset=ioff, TauRefrac=2.0),
+                            {"V": v0, "RefracTime": np.zeros(n, np.float32)}))
+        ext_rate = PD_EXT[name] * connectivity_scale * PD_BG_RATE
+        ext_w = PD_MEAN_W / math.sqrt(connectivity_scale)
+        net.css.append(CurrentSource(name + "_dc", "dc", name, amp=ext_w * 0.5 * ext_rate / 1000.0))
+    stream = 100
+    for trg in pops:
+        for src in pops:
+            stream += 4
+            num_in = pd_full_num_inputs(src, trg) * connectivity_scale
+            total = int(round(num_in * float(size[trg])))
+            if total <= 0:
+                continue
+            mean_w = pd_mean_weight(src, trg) / math.sqrt(connectivity_scale)
+            sd_w = mean_w * 0.05 if (src == "4E" and trg == "23E") else abs(mean_w * 0.1)
+            rl, ind, (pre, within) = fixed_number_total(seed, stream, size[src], size[trg], total, pad=pad)
+            kind = src[-1]
+            fmax = float(np.finfo(np.float32).max)
+            lo, hi = (0.0, fmax) if kind == "E" else (-fmax, 0.0)
+            gv = clipped_normal(seed, stream + 1, total, mean_w, sd_w, lo, hi).astype(np.float32)
+            dv = np.rint(clipped_normal(seed, stream + 2, total, PD_MEAN_DELAY[kind] / dt, PD_DELAY_SD[kind] / dt,
+                                        0.0, max_delay[kind] / dt).astype(np.float32)).astype(np.uint8)
+            g = np.zeros(ind.shape, np.float32)
+            d = np.zeros(ind.shape, np.uint8)
+            g[pre, within] = gv
+            d[pre, within] = dv
+            net.syns.append(Syn(f"{src}_{trg}", src, trg, wum="static_delay", psm="expcurr", tau=0.5,
+                                row_stride=ind.shape[1], row_length=rl, ind=ind, g=g, d=d, max_den_delay=slots))
+    return net
+
+
+# --------------------------------------------------------------------------------------------
+# C3: fixed-fanout Izhikevich network with pregenerated noise current
+# --------------------------------------------------------------------------------------------
+def izhikevich_fanout(n=1_000_000, fanout=1000, steps=1000, seed=777, dt=1.0, with_noise=True):
+    n_e = (n * 4) // 5
+    net = Net(name="izh", dt=dt, steps=steps, seed=seed)
+    v0 = np.full(n, -65.0, np.float32)
+    u0 = (0.2 * v0).astype(np.float32)
+    net.pops.append(Pop("N", "izh", n, dict(a=0.02, b=0.2, c=-65.0, d=8.0), {"V": v0, "U": u0}))
+    rl, ind = fixed_number_post(seed, 10, n, n, fanout)
+    g = np.empty((n, fanout), np.float32)
+    chunk = max(1, (1 << 24) // fanout)
+    for r0 in range(0, n, chunk):
+        r1 = min(n, r0 + chunk)
+        u = rng.uniform(seed, 11, r0 * fanout, (r1 - r0) * fanout).reshape(r1 - r0, fanout)
+        rows = np.arange(r0, r1)[:, None]
+        g[r0:r1] = np.where(rows < n_e, 0.5 * u, u - 1.0).astype(np.float32)
+    net.syns.append(Syn("NN", "N", "N", wum="static", psm="deltacurr", row_stride=fanout, row_length=rl, ind=ind, g=g))
+    if with_noise:
+        noise = (5.0 * rng.uniform(seed, 12, 0, steps * n)).astype(np.float32).reshape(steps, n)
+        net.css.append(CurrentSource("N_noise", "noise", "N", noise=noise))
+    return net
+
+
+# --------------------------------------------------------------------------------------------
+# C4: plastic sparse network with trace STDP (pygenn/genn_model.py:1448-1476)
+# --------------------------------------------------------------------------------------------
+def poisson_spike_source(seed, stream, n, rate_hz, steps, dt, rates=None):
+    """Pregenerated Poisson spike times (ms, on the dt grid) in SpikeSourceArray layout
+    (startSpike/endSpike/spikeTimes, include/genn/genn/neuronModels.h:274-286)."""
+    p = (np.full(n, rate_hz) if rates is None else np.asarray(rates)) * dt / 1000.0
+    u = rng.uniform(seed, stream, 0, n * steps).reshape(n, steps)
+    fire = u < p[:, None]
+    counts = fire.sum(axis=1)
+    end = np.cumsum(counts).astype(np.uint32)
+    start = (end - counts).astype(np.uint32)
+    src, step = np.nonzero(fire)
+    times = (step.astype(np.float64) * dt).astype(np.float32)
+    return start, end, times
+
+
+def plastic_stdp(n=100_000, n_src=1000, steps=10000, seed=99, dt=1.0, fan=500, src_fan=100, src_w=2.0):
+    n_e = (n * 4) // 5
+    n_i = n - n_e
+    net = Net(name="stdp", dt=dt, steps=steps, seed=seed)
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.45, TauRefrac=5.0)
+    for k, (name, num) in enumerate((("E", n_e), ("I", n_i))):
+        v0 = (-60.0 + 10.0 * rng.uniform(seed, 1 + k, 0, num)).astype(np.float32)
+        net.pops.append(Pop(name, "lif", num, dict(lif), {"V": v0, "RefracTime": np.zeros(num, np.float32)}))
+    start, end, times = poisson_spike_source(seed, 5, n_src, 10.0, steps, dt)
+    net.pops.append(Pop("P", "ssa", n_src, {}, {"startSpike": start, "endSpike": end}, spike_times=times))
+    # plastic E->E
+    rl, ind = fixed_probability(seed, 20, n_e, n_e, min(1.0, fan / n_e))
+    mask = np.arange(ind.shape[1])[None, :] < rl[:, None]
+    g = np.zeros(ind.shape, np.float32)
+    g[mask] = (0.5 * rng.uniform(seed, 21, 0, int(rl.sum()))).astype(np.float32) * np.float32(4.0 * 500.0 / max(fan, 1) / 20.0)
+    net.syns.append(Syn("EE", "E", "E", wum="stdp_trace",
+                        wum_params=dict(tauPlus=20.0, tauMinus=20.0, aPlus=0.01, aMinus=0.012, wMin=0.0, wMax=1.0),
+                        psm="expcurr", tau=5.0, row_stride=ind.shape[1], row_length=rl, ind=ind, g=g))
+    # static projections closing the balanced loop
+    for name, src, trg, ns, nt, w, tau, st in (("EI", "E", "I", n_e, n_i, 0.05, 5.0, 22), ("IE", "I", "E", n_i, n_e, -0.25, 10.0, 23),
+                                               ("II", "I", "I", n_i, n_i, -0.25, 10.0, 24)):
+        rl, ind = fixed_probability(seed, st, ns, nt, min(1.0, fan / n_e))
+        g = np.where(np.arange(ind.shape[1])[None, :] < rl[:, None], np.float32(w), np.float32(0)).astype(np.float32)
+        net.syns.append(Syn(name, src, trg, wum="static", psm="expcurr", tau=tau, row_stride=ind.shape[1],
+                            row_length=rl, ind=ind, g=g))
+    rl, ind = fixed_number_post(seed, 25, n_src, n_e, min(src_fan, n_e))
+    g = np.full(ind.shape, np.float32(src_w), np.float32)
+    net.syns.append(Syn("PE", "P", "E", wum="static", psm="expcurr", tau=5.0, row_stride=ind.shape[1],
+                        row_length=rl, ind=ind, g=g))
+    return net
+
+
+# --------------------------------------------------------------------------------------------
+# C5: convolutional spiking layer through TOEPLITZ connectivity
+# --------------------------------------------------------------------------------------------
+def conv_toeplitz(h=64, w=64, ic=16, oc=32, k=3, steps=500, seed=5, dt=1.0, batch_index=0, max_rate=50.0, w_sd=0.1):
+    n_in, n_out = h * w * ic, h * w * oc
+    net = Net(name="conv", dt=dt, steps=steps, seed=seed)
+    rates = max_rate * rng.uniform(seed, 1, 0, n_in)
+    start, end, times = poisson_spike_source(seed, 100 + batch_index, n_in, 0.0, steps, dt, rates=rates)
+    net.pops.append(Pop("In", "ssa", n_in, {}, {"startSpike": start, "endSpike": end}, spike_times=times))
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.0, TauRefrac=5.0)
+    net.pops.append(Pop("Out", "lif", n_out, lif, {"V": np.full(n_out, -60.0, np.float32), "RefracTime": np.zeros(n_out, np.float32)}))
+    kern = (w_sd * rng.normal(seed, 2, 0, k * k * ic * oc)).astype(np.float32).reshape(k, k, ic, oc)
+    net.syns.append(Syn("Conv", "In", "Out", matrix="conv2d", wum="static", psm="expcurr", tau=5.0, g=kern,
+                        conv=dict(conv_kh=k, conv_kw=k, conv_ih=h, conv_iw=w, conv_ic=ic, conv_oh=h, conv_ow=w, conv_oc=oc)))
+    return net

@@ -1,0 +1,1004 @@
+// MI355X (gfx950) device layer for GeNN's per-timestep hot path: kernels + C ABI.
+//
+// Kernels (one launch each per timestep, all on the runner's stream):
+//   presynapticUpdateKernel   sparse / Toeplitz presynaptic event propagation into outPost or the
+//                             dendritic-delay ring (replaces updatePresynapticKernel,
+//                             src/genn/genn/code_generator/backendSIMT.cc:694-764 and the strategies in
+//                             presynapticUpdateStrategySIMT.cc:57-162, 167-389, 750-934)
+//   postsynapticUpdateKernel  STDP learnPost through the column remap (backendSIMT.cc:766-803, 1822-1898)
+//   neuronUpdateKernel        PSM apply + current sources + neuron model + threshold + ordered spike
+//                             compaction + recording (backendSIMT.cc:405-662, 1931-1975); also does the
+//                             work of neuronSpikeQueueUpdateKernel (:373-403) and
+//                             synapseDendriticDelayUpdateKernel (:664-692), which need no launch here.
+//   remap*Kernel              deterministic colLength/remap build (replaces backendSIMT.cc:1977-1991)
+//
+// Arithmetic contract: fp32, one rounding per operation, same operation order as the code the
+// reference's SingleThreadedCPU backend generates (build with -ffp-contract=off).  The only
+// permitted divergence is the order of fp32 atomic adds into outPost / denDelay.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "genn_mi355x.h"
+
+namespace
+{
+constexpr int BLOCK = 256;                  // 4 wave64 per work-group
+constexpr int WAVE = 64;
+constexpr uint32_t SPIN_LIMIT = 1u << 22;   // bounded wait of the spike-offset look-back
+constexpr uint32_t REMAP_SORT_MAX = 16384;  // longest column the LDS sort handles (64 KiB)
+
+thread_local std::string g_lastError;
+
+int fail(int code, const std::string &msg)
+{
+    g_lastError = msg;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                              \
+    do {                                                                                           \
+        hipError_t e_ = (expr);                                                                    \
+        if(e_ != hipSuccess) {                                                                     \
+            return fail(GENNMI_EHIP, std::string(#expr) + ": " + hipGetErrorString(e_));           \
+        }                                                                                          \
+    } while(0)
+
+// ------------------------------------------------------------------------------------------------
+// device-side tables
+// ------------------------------------------------------------------------------------------------
+struct StepState             // device-resident; lets a captured graph be replayed unchanged
+{
+    unsigned long long timestep;
+    unsigned long long epoch;           // number of completed steps since runner creation
+    unsigned long long numRecordingTimesteps;
+};
+
+struct StepArgs              // per-launch; either direct values or offsets from *base
+{
+    const StepState *base;
+    unsigned long long k;               // offset added to base->timestep / base->epoch
+    unsigned long long epoch;           // direct
+    float t;                            // direct
+    uint32_t recordingTimestep;         // direct
+};
+
+struct Resolved { float t; uint32_t recT; unsigned long long epoch; };
+
+__device__ __forceinline__ Resolved resolve(const StepArgs &a, float dt)
+{
+    Resolved r;
+    if(a.base) {
+        const unsigned long long ts = a.base->timestep + a.k;
+        // const float t = timestep * DT  (generateRunner.cc:283)
+        r.t = (float)ts * dt;
+        const unsigned long long nr = a.base->numRecordingTimesteps;
+        r.recT = nr ? (uint32_t)(ts % nr) : 0u;
+        r.epoch = a.base->epoch + a.k;
+    }
+    else {
+        r.t = a.t; r.recT = a.recordingTimestep; r.epoch = a.epoch;
+    }
+    return r;
+}
+
+struct NeuronGroupDev
+{
+    gennmi_neuron_update_group_t g;
+    uint32_t startBlock, numBlocks;
+};
+
+struct PreGroupDev
+{
+    gennmi_presynaptic_update_group_t g;
+    uint32_t startBlock, numBlocks;
+    uint32_t lanesPerSpike;             // power of two, 1..64
+    uint32_t vec4;                      // rows are 16-byte aligned and padded: dwordx4 loads
+    int32_t convBH, convBW;
+};
+
+struct PostGroupDev
+{
+    gennmi_postsynaptic_update_group_t g;
+    uint32_t startBlock, numBlocks;
+    uint32_t lanesPerSpike;
+};
+
+// Block -> group: groups occupy consecutive block ranges (the reference pads thread ranges to
+// block multiples for the same reason, backendSIMT.h:244-323).  Table sizes are tens of entries.
+template<typename G>
+__device__ __forceinline__ uint32_t findGroup(const G *groups, uint32_t numGroups, uint32_t block)
+{
+    uint32_t lo = 0, hi = numGroups;
+    while(hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if(groups[mid].startBlock <= block) { lo = mid; } else { hi = mid; }
+    }
+    return lo;
+}
+
+__device__ __forceinline__ void atomicAddF32(float *addr, float v)
+{
+    // gfx950 has a native global_atomic_add_f32; no return value is needed
+    unsafeAtomicAdd(addr, v);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Presynaptic update.  One sub-group of `lanesPerSpike` lanes walks one spike's row; sub-groups
+// take spikes round-robin.  lanesPerSpike = 64 is the "post span" mapping (lanes span the row, so
+// ind/g are read as whole 256-byte lines); small values are the "pre span" mapping (few lanes per
+// spike, many spikes per wave).  Spike list, rowLength and row base are read once per spike.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(BLOCK)
+void presynapticUpdateKernel(const PreGroupDev *groups, uint32_t numGroups, StepArgs args, float dt,
+                             unsigned long long *eventCounter)
+{
+    const Resolved st = resolve(args, dt);
+    const uint32_t gi = findGroup(groups, numGroups, blockIdx.x);
+    const PreGroupDev &G = groups[gi];
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const uint32_t W = G.lanesPerSpike;
+    const uint32_t localBlock = blockIdx.x - G.startBlock;
+    const uint32_t lis = threadIdx.x & (W - 1);
+    const uint32_t subGroup = (localBlock * BLOCK + threadIdx.x) / W;
+    const uint32_t numSubGroups = (G.numBlocks * BLOCK) / W;
+    const uint32_t numSpikes = g.srcSpkCnt[batch];
+    const uint32_t *spk = g.srcSpk + (size_t)batch * g.numSrcNeurons;
+    unsigned long long events = 0;
+
+    if(g.matrix == GENNMI_MATRIX_TOEPLITZ_CONV2D) {
+        // initToeplitzConnectivitySnippet.h:116-137; lanes span the kh*kw*oc diagonals, so
+        // consecutive lanes hit consecutive output channels (consecutive outPost addresses)
+        const int kh = g.conv[0], kw = g.conv[1], iw = g.conv[3], ic = g.conv[4];
+        const int oh = g.conv[5], ow = g.conv[6], oc = g.conv[7];
+        const uint32_t numDiag = (uint32_t)(kh * kw * oc);
+        float *outPost = g.outPost + (size_t)batch * g.numTrgNeurons;
+        for(uint32_t s = subGroup; s < numSpikes; s += numSubGroups) {
+            const uint32_t ipre = spk[s];
+            const int preRow = (int)(ipre / ic) / iw;
+            const int preCol = (int)(ipre / ic) % iw;
+            const int preChan = (int)(ipre % ic);
+            for(uint32_t j = lis; j < numDiag; j += W) {
+                const int kernRow = (int)(j / oc) / kw;
+                const int kernCol = (int)(j / oc) % kw;
+                const int kernOutChan = (int)(j % oc);
+                const int postRow = preRow + kernRow - G.convBH;
+                const int postCol = preCol + kernCol - G.convBW;
+                if(postRow >= 0 && postCol >= 0 && postRow < oh && postCol < ow) {
+                    const int postInd = (postRow * ow * oc) + (postCol * oc) + kernOutChan;
+                    const int kernelInd = ((kh - kernRow - 1) * kw * ic * oc) + ((kw - kernCol - 1) * ic * oc) + (preChan * oc) + kernOutChan;
+                    atomicAddF32(&outPost[postInd], g.g[kernelInd]);
+                    events++;
+                }
+            }
+        }
+    }
+    else {
+        const uint32_t D = g.maxDenDelay;
+        // *denDelayPtr = (*denDelayPtr + 1) % D happens at the start of updateSynapses
+        // (synapseUpdateGroupMerged.cc:480-483); st.epoch counts completed steps, so the pointer
+        // in force during this step is (epoch + 1) % D.
+        const uint32_t denPtr = D ? (uint32_t)((st.epoch + 1) % D) : 0;
+        float *outPost = g.outPost + (size_t)batch * g.numTrgNeurons;
+        float *denDelay = D ? g.denDelay + (size_t)batch * D * g.numTrgNeurons : nullptr;
+        for(uint32_t s = subGroup; s < numSpikes; s += numSubGroups) {
+            const uint32_t idPre = spk[s];
+            const uint32_t npost = g.rowLength[idPre];
+            const size_t rowBase = (size_t)idPre * g.rowStride;
+            if(lis == 0) { events += npost; }
+            if(g.wum == GENNMI_WUM_STATIC_PULSE) {
+                if(G.vec4) {
+                    const uint4 *ind4 = reinterpret_cast<const uint4*>(g.ind + rowBase);
+                    const float4 *g4 = reinterpret_cast<const float4*>(g.g + rowBase);
+                    for(uint32_t j = lis * 4; j < npost; j += W * 4) {
+                        const uint4 ip = ind4[j >> 2];
+                        const float4 w = g4[j >> 2];
+                        atomicAddF32(&outPost[ip.x], w.x);
+                        if(j + 1 < npost) { atomicAddF32(&outPost[ip.y], w.y); }
+                        if(j + 2 < npost) { atomicAddF32(&outPost[ip.z], w.z); }
+                        if(j + 3 < npost) { atomicAddF32(&outPost[ip.w], w.w); }
+                    }
+                }
+                else {
+                    for(uint32_t j = lis; j < npost; j += W) {
+                        atomicAddF32(&outPost[g.ind[rowBase + j]], g.g[rowBase + j]);
+                    }
+                }
+            }
+            else if(g.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY) {
+                // addToPostDelay(g, d): denDelay[((ptr + d) % D) * numPost + idPost] += g  (synapseUpdateGroupMerged.cc:245-251)
+                if(G.vec4) {
+                    const uint4 *ind4 = reinterpret_cast<const uint4*>(g.ind + rowBase);
+                    const float4 *g4 = reinterpret_cast<const float4*>(g.g + rowBase);
+                    const uchar4 *d4 = reinterpret_cast<const uchar4*>(g.d + rowBase);
+                    for(uint32_t j = lis * 4; j < npost; j += W * 4) {
+                        const uint4 ip = ind4[j >> 2];
+                        const float4 w = g4[j >> 2];
+                        const uchar4 dl = d4[j >> 2];
+                        atomicAddF32(&denDelay[(size_t)((denPtr + dl.x) % D) * g.numTrgNeurons + ip.x], w.x);
+                        if(j + 1 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.y) % D) * g.numTrgNeurons + ip.y], w.y); }
+                        if(j + 2 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.z) % D) * g.numTrgNeurons + ip.z], w.z); }
+                        if(j + 3 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.w) % D) * g.numTrgNeurons + ip.w], w.w); }
+                    }
+                }
+                else {
+                    for(uint32_t j = lis; j < npost; j += W) {
+                        const uint32_t slot = (denPtr + g.d[rowBase + j]) % D;
+                        atomicAddF32(&denDelay[(size_t)slot * g.numTrgNeurons + g.ind[rowBase + j]], g.g[rowBase + j]);
+                    }
+                }
+            }
+            else {
+                // trace STDP presynaptic-spike code (pygenn/genn_model.py:1456-1463); every synapse of
+                // the row is owned by exactly one lane, so the read-modify-write of g needs no atomic
+                for(uint32_t j = lis; j < npost; j += W) {
+                    const uint32_t idPost = g.ind[rowBase + j];
+                    const float w = g.g[rowBase + j];
+                    const float stPost = dt + g.trgST[idPost];       // st_post = DT*(backPropSteps+1) + trgST (synapseUpdateGroupMerged.cc:134-142)
+                    atomicAddF32(&outPost[idPost], w);
+                    const float dtSpike = st.t - stPost;
+                    if(dtSpike > 0) {
+                        const float newWeight = w - (g.aMinus * g.postTrace[idPost]);
+                        g.g[rowBase + j] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
+                    }
+                }
+            }
+        }
+    }
+
+    // one counter update per wave
+    for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
+    if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Postsynaptic update (learnPost): one sub-group per postsynaptic spike walks the column through
+// remap (coalesced), gathers g by synapse index.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(BLOCK)
+void postsynapticUpdateKernel(const PostGroupDev *groups, uint32_t numGroups, StepArgs args, float dt)
+{
+    const Resolved st = resolve(args, dt);
+    const uint32_t gi = findGroup(groups, numGroups, blockIdx.x);
+    const PostGroupDev &G = groups[gi];
+    const gennmi_postsynaptic_update_group_t &g = G.g;
+    const uint32_t W = G.lanesPerSpike;
+    const uint32_t localBlock = blockIdx.x - G.startBlock;
+    const uint32_t lis = threadIdx.x & (W - 1);
+    const uint32_t subGroup = (localBlock * BLOCK + threadIdx.x) / W;
+    const uint32_t numSubGroups = (G.numBlocks * BLOCK) / W;
+    const uint32_t numSpikes = g.trgSpkCnt[0];
+    for(uint32_t s = subGroup; s < numSpikes; s += numSubGroups) {
+        const uint32_t spike = g.trgSpk[s];
+        const uint32_t npre = g.colLength[spike];
+        const size_t colBase = (size_t)spike * g.colStride;
+        for(uint32_t i = lis; i < npre; i += W) {
+            const uint32_t rowMajorIndex = g.remap[colBase + i];
+            const uint32_t idPre = rowMajorIndex / g.rowStride;
+            const float stPre = dt + g.srcST[idPre];
+            const float dtSpike = st.t - stPre;
+            if(dtSpike > 0) {
+                const float newWeight = g.g[rowMajorIndex] + (g.aPlus * g.preTrace[idPre]);
+                g.g[rowMajorIndex] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Neuron update.  One lane per neuron.  Spikes are emitted in ascending neuron index (the CPU
+// backend's order, single_threaded_cpu/backend.cc:321, 2119-2133): wave ballot gives the in-wave
+// rank, an LDS scan the in-block rank, and a look-back over per-block counts published in `agg`
+// (tagged with the step so nothing ever needs clearing) the cross-block offset.  Only blocks that
+// emitted spikes, and the last block of each population (which stores spkCnt), look back.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(BLOCK)
+void neuronUpdateKernel(const NeuronGroupDev *groups, uint32_t numGroups, StepArgs args, float dt,
+                        unsigned long long *agg, uint32_t *errorFlag)
+{
+    __shared__ uint32_t shWaveCount[BLOCK / WAVE];
+    __shared__ uint32_t shPrefix;
+
+    const Resolved st = resolve(args, dt);
+    const uint32_t gi = findGroup(groups, numGroups, blockIdx.x);
+    const NeuronGroupDev &G = groups[gi];
+    const gennmi_neuron_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const uint32_t localBlock = blockIdx.x - G.startBlock;
+    const uint32_t n = g.numNeurons;
+    const uint32_t i = localBlock * BLOCK + threadIdx.x;
+    const size_t bi = (size_t)batch * n + i;
+    const uint32_t lane = threadIdx.x & (WAVE - 1);
+    const uint32_t wave = threadIdx.x / WAVE;
+    const float t = st.t;
+
+    bool spiked = false;
+    if(i < n) {
+        if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
+            uint32_t startSpike = g.startSpike[bi];
+            spiked = (startSpike != g.endSpike[bi]) && (t >= g.spikeTimes[startSpike]);
+            if(spiked) { g.startSpike[bi] = startSpike + 1; }
+        }
+        else {
+            float Isyn = 0;
+            float l0 = g.var0[bi], l1 = g.var1[bi];
+            for(uint32_t m = 0; m < g.numPSM; m++) {
+                const gennmi_psm_t &psm = g.psm[m];
+                float linSyn = psm.outPost[bi];
+                if(psm.maxDenDelay) {
+                    // read and clear the front slot of the ring (neuronUpdateGroupMerged.cc:84-101)
+                    const uint32_t ptr = (uint32_t)((st.epoch + 1) % psm.maxDenDelay);
+                    float *front = &psm.denDelay[((size_t)batch * psm.maxDenDelay + ptr) * n + i];
+                    linSyn += *front;
+                    *front = 0.0f;
+                }
+                if(psm.kind == GENNMI_PSM_EXPCURR) {
+                    Isyn += psm.init * linSyn;
+                    linSyn *= psm.expDecay;
+                }
+                else {
+                    Isyn += linSyn;
+                    linSyn = 0.0f;
+                }
+                psm.outPost[bi] = linSyn;
+            }
+            for(uint32_t c = 0; c < g.numCS; c++) {
+                const gennmi_cs_t &cs = g.cs[c];
+                Isyn += (cs.kind == GENNMI_CS_DC) ? cs.amp : cs.array[(size_t)(st.epoch % cs.arraySteps) * n + i];
+            }
+            if(g.model == GENNMI_NEURON_LIF) {
+                if(l1 <= 0.0f) {
+                    const float alpha = ((Isyn + g.params[0]) * g.params[1]) + g.params[2];
+                    l0 = alpha - (g.params[3] * (alpha - l0));
+                }
+                else {
+                    l1 -= dt;
+                }
+            }
+            else {
+                if(l0 >= 30.0f) {
+                    l0 = g.params[2];
+                    l1 += g.params[3];
+                }
+                l0 += 0.5f * (0.04f * l0 * l0 + 5.0f * l0 + 140.0f - l1 + Isyn) * dt;
+                l0 += 0.5f * (0.04f * l0 * l0 + 5.0f * l0 + 140.0f - l1 + Isyn) * dt;
+                l1 += g.params[0] * (g.params[1] * l0 - l1) * dt;
+                if(l0 > 30.0f) { l0 = 30.0f; }
+            }
+            float preTrace = 0, postTrace = 0;
+            if(g.preTrace) { preTrace = g.preTrace[bi] * g.preDecay; }
+            if(g.postTrace) { postTrace = g.postTrace[bi] * g.postDecay; }
+            spiked = (g.model == GENNMI_NEURON_LIF) ? (l1 <= 0.0f && l0 >= g.params[4]) : (l0 >= 29.99f);
+            if(spiked) {
+                preTrace += 1.0f; postTrace += 1.0f;
+                if(g.sT) { g.sT[bi] = t; }
+                if(g.model == GENNMI_NEURON_LIF) { l0 = g.params[5]; l1 = g.params[6]; }
+            }
+            if(g.preTrace) { g.preTrace[bi] = preTrace; }
+            if(g.postTrace) { g.postTrace[bi] = postTrace; }
+            g.var0[bi] = l0; g.var1[bi] = l1;
+        }
+    }
+
+    // keep the user-visible ring pointers current (nothing in the kernels reads them)
+    if(localBlock == 0 && batch == 0 && threadIdx.x < g.numPSM) {
+        const gennmi_psm_t &psm = g.psm[threadIdx.x];
+        if(psm.maxDenDelay && psm.denDelayPtr) { *psm.denDelayPtr = (uint32_t)((st.epoch + 1) % psm.maxDenDelay); }
+    }
+
+    // ---- ordered compaction --------------------------------------------------------------------
+    const unsigned long long ballot = __ballot(spiked);
+    const uint32_t waveCount = __popcll(ballot);
+    const uint32_t laneRank = __popcll(ballot & ((1ull << lane) - 1ull));
+    if(lane == 0) { shWaveCount[wave] = waveCount; }
+
+    // recording: the ballot IS the bitfield (bit i%32 of word i/32, runtime.cc:855-913); every word of
+    // the step is overwritten, so no clearing and no atomicOr (cf. backendSIMT.cc:1948-1953)
+    if(g.recordSpk && (lane & 31) == 0 && i < n) {
+        const uint32_t words = (n + 31) / 32;
+        g.recordSpk[((size_t)st.recT * gridDim.y + batch) * words + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
+    }
+    __syncthreads();
+
+    uint32_t blockCount = 0, waveOffset = 0;
+    #pragma unroll
+    for(uint32_t w = 0; w < BLOCK / WAVE; w++) {
+        const uint32_t c = shWaveCount[w];
+        if(w < wave) { waveOffset += c; }
+        blockCount += c;
+    }
+
+    const uint32_t tag = (uint32_t)(st.epoch + 1);
+    const size_t aggBase = (size_t)batch * gridDim.x + G.startBlock;
+    if(threadIdx.x == 0) {
+        __hip_atomic_store(&agg[aggBase + localBlock], ((unsigned long long)tag << 32) | blockCount,
+                           __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const bool last = (localBlock == G.numBlocks - 1);
+    if(blockCount == 0 && !last) { return; }
+
+    if(wave == 0) {
+        uint32_t sum = 0;
+        bool ok = true;
+        for(uint32_t base = 0; base < localBlock; base += WAVE) {
+            const uint32_t k = base + lane;
+            uint32_t v = 0;
+            if(k < localBlock) {
+                uint32_t spins = 0;
+                while(true) {
+                    const unsigned long long a = __hip_atomic_load(&agg[aggBase + k], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+                    if((uint32_t)(a >> 32) == tag) { v = (uint32_t)a; break; }
+                    if(++spins > SPIN_LIMIT) { ok = false; break; }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+            }
+            sum += v;
+        }
+        for(int off = WAVE / 2; off > 0; off >>= 1) { sum += __shfl_down(sum, off, WAVE); }
+        const bool allOk = (__ballot(!ok) == 0ull);
+        if(lane == 0) {
+            if(!allOk) { atomicOr(errorFlag, 1u); sum = 0xFFFFFFFFu; }
+            shPrefix = sum;
+        }
+    }
+    __syncthreads();
+    const uint32_t prefix = shPrefix;
+    if(prefix == 0xFFFFFFFFu) { return; }       // bounded wait expired: flagged, nothing written
+    if(spiked) { g.spk[(size_t)batch * n + prefix + waveOffset + laneRank] = i; }
+    if(last && threadIdx.x == 0) { g.spkCnt[batch] = prefix + blockCount; }
+}
+
+// Advances the device-resident step state at the end of a captured graph.
+__global__ void advanceStepKernel(StepState *state, unsigned long long steps)
+{
+    if(threadIdx.x == 0 && blockIdx.x == 0) { state->timestep += steps; state->epoch += steps; }
+}
+
+__global__ void fillKernel(float *p, float v, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if(i < n) { p[i] = v; }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Remap build: scatter in arbitrary order, then sort every column ascending, which is the order
+// the CPU backend's row-major traversal produces (single_threaded_cpu/backend.cc:156-179).
+// ------------------------------------------------------------------------------------------------
+__global__ void remapCountKernel(uint32_t numSrc, uint32_t rowStride, const uint32_t *rowLength, const uint32_t *ind,
+                                 uint32_t colStride, uint32_t *colLength, uint32_t *remap, uint32_t *overflow)
+{
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t total = (size_t)numSrc * rowStride;
+    if(idx >= total) { return; }
+    const uint32_t row = (uint32_t)(idx / rowStride), j = (uint32_t)(idx % rowStride);
+    if(j >= rowLength[row]) { return; }
+    const uint32_t post = ind[idx];
+    const uint32_t pos = atomicAdd(&colLength[post], 1u);
+    if(remap) {
+        if(pos < colStride) { remap[(size_t)post * colStride + pos] = (uint32_t)idx; }
+        else { atomicMax(overflow, pos + 1); }
+    }
+}
+
+__global__ __launch_bounds__(BLOCK)
+void remapSortKernel(uint32_t colStride, const uint32_t *colLength, uint32_t *remap)
+{
+    extern __shared__ uint32_t shCol[];
+    const uint32_t col = blockIdx.x;
+    const uint32_t len = min(colLength[col], colStride);
+    if(len < 2) { return; }
+    uint32_t p2 = 1;
+    while(p2 < len) { p2 <<= 1; }
+    uint32_t *column = remap + (size_t)col * colStride;
+    for(uint32_t k = threadIdx.x; k < p2; k += BLOCK) { shCol[k] = (k < len) ? column[k] : 0xFFFFFFFFu; }
+    __syncthreads();
+    for(uint32_t size = 2; size <= p2; size <<= 1) {
+        for(uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+            for(uint32_t k = threadIdx.x; k < p2; k += BLOCK) {
+                const uint32_t partner = k ^ stride;
+                if(partner > k) {
+                    const bool up = ((k & size) == 0);
+                    const uint32_t a = shCol[k], b = shCol[partner];
+                    if((a > b) == up) { shCol[k] = b; shCol[partner] = a; }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    for(uint32_t k = threadIdx.x; k < len; k += BLOCK) { column[k] = shCol[k]; }
+}
+
+uint32_t pow2Floor(uint32_t v) { uint32_t p = 1; while(p * 2 <= v) { p *= 2; } return p; }
+uint32_t pow2Ceil(uint32_t v) { uint32_t p = 1; while(p < v) { p *= 2; } return p; }
+}   // namespace
+
+// ------------------------------------------------------------------------------------------------
+struct gennmi_runner
+{
+    float dt = 0;
+    uint32_t batch = 1;
+    bool finalised = false;
+    hipStream_t stream = nullptr;
+    std::vector<NeuronGroupDev> neuron; std::vector<PreGroupDev> pre; std::vector<PostGroupDev> post;
+    NeuronGroupDev *dNeuron = nullptr; PreGroupDev *dPre = nullptr; PostGroupDev *dPost = nullptr;
+    uint32_t neuronBlocks = 0, preBlocks = 0, postBlocks = 0;
+    unsigned long long *dAgg = nullptr; uint32_t *dError = nullptr; unsigned long long *dEvents = nullptr;
+    StepState *dState = nullptr;
+    unsigned long long epoch = 0;       // completed steps (host mirror)
+    bool synapsesDone = false;          // updateSynapses ran for the current step
+    // graph
+    hipGraphExec_t graphExec = nullptr; unsigned long long graphSteps = 0;
+    // timing
+    bool timing = false;
+    hipEvent_t evA = nullptr, evB = nullptr, evC = nullptr, evD = nullptr;
+    double neuronTime = 0, preTime = 0, postTime = 0;
+    unsigned long long preLaunches = 0, neuronLaunches = 0;
+};
+
+extern "C" {
+
+const char *gennmi_last_error(void) { return g_lastError.c_str(); }
+
+int gennmi_init(int device)
+{
+    int count = 0;
+    HIP_TRY(hipGetDeviceCount(&count));
+    if(device < 0 || device >= count) { return fail(GENNMI_EINVAL, "gennmi_init: no such device"); }
+    HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if(prop.warpSize != WAVE) { return fail(GENNMI_EUNSUPPORTED, "gennmi_init: kernels assume 64-wide wavefronts"); }
+    return GENNMI_OK;
+}
+
+int gennmi_device_name(char *buf, size_t len)
+{
+    int device = 0;
+    HIP_TRY(hipGetDevice(&device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    snprintf(buf, len, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+    return GENNMI_OK;
+}
+
+int gennmi_malloc(void **devPtr, size_t bytes)
+{
+    HIP_TRY(hipMalloc(devPtr, bytes ? bytes : 4));
+    return GENNMI_OK;
+}
+int gennmi_free(void *devPtr) { HIP_TRY(hipFree(devPtr)); return GENNMI_OK; }
+int gennmi_memcpy_to_device(void *dev, const void *host, size_t bytes) { HIP_TRY(hipMemcpy(dev, host, bytes, hipMemcpyHostToDevice)); return GENNMI_OK; }
+int gennmi_memcpy_from_device(void *host, const void *dev, size_t bytes) { HIP_TRY(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost)); return GENNMI_OK; }
+int gennmi_memset(void *dev, int value, size_t bytes) { HIP_TRY(hipMemset(dev, value, bytes)); return GENNMI_OK; }
+int gennmi_fill_f32(float *dev, float value, size_t count)
+{
+    if(count) {
+        fillKernel<<<dim3((unsigned int)((count + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, 0>>>(dev, value, count);
+        HIP_TRY(hipGetLastError());
+        HIP_TRY(hipDeviceSynchronize());
+    }
+    return GENNMI_OK;
+}
+int gennmi_synchronize(void) { HIP_TRY(hipDeviceSynchronize()); return GENNMI_OK; }
+int gennmi_free_device_memory_bytes(size_t *bytes)
+{
+    size_t total = 0;
+    HIP_TRY(hipMemGetInfo(bytes, &total));
+    return GENNMI_OK;
+}
+
+int gennmi_runner_create(gennmi_runner **runner, float dt, uint32_t batchSize)
+{
+    if(!runner || batchSize == 0 || batchSize > 65535) { return fail(GENNMI_EINVAL, "gennmi_runner_create: bad arguments"); }
+    gennmi_runner *r = new gennmi_runner;
+    r->dt = dt; r->batch = batchSize;
+    HIP_TRY(hipStreamCreate(&r->stream));       // blocking stream: ordered against null-stream copies
+    HIP_TRY(hipMalloc(&r->dError, sizeof(uint32_t)));
+    HIP_TRY(hipMemset(r->dError, 0, sizeof(uint32_t)));
+    HIP_TRY(hipMalloc(&r->dEvents, sizeof(unsigned long long)));
+    HIP_TRY(hipMemset(r->dEvents, 0, sizeof(unsigned long long)));
+    HIP_TRY(hipMalloc(&r->dState, sizeof(StepState)));
+    HIP_TRY(hipMemset(r->dState, 0, sizeof(StepState)));
+    *runner = r;
+    return GENNMI_OK;
+}
+
+int gennmi_runner_destroy(gennmi_runner *r)
+{
+    if(!r) { return GENNMI_OK; }
+    hipStreamSynchronize(r->stream);
+    if(r->graphExec) { hipGraphExecDestroy(r->graphExec); }
+    for(hipEvent_t e : {r->evA, r->evB, r->evC, r->evD}) { if(e) { hipEventDestroy(e); } }
+    hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dAgg); hipFree(r->dError); hipFree(r->dEvents); hipFree(r->dState);
+    hipStreamDestroy(r->stream);
+    delete r;
+    return GENNMI_OK;
+}
+
+int gennmi_push_neuron_update_group(gennmi_runner *r, const gennmi_neuron_update_group_t *g, uint32_t *idx)
+{
+    if(!r || !g) { return fail(GENNMI_EINVAL, "push_neuron_update_group: null argument"); }
+    if(r->finalised) { return fail(GENNMI_ESTATE, "push_neuron_update_group: runner already finalised"); }
+    if(g->numNeurons == 0) { return fail(GENNMI_EINVAL, "push_neuron_update_group: empty population"); }
+    if(g->numPSM > GENNMI_MAX_PSM || g->numCS > GENNMI_MAX_CS) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: too many children"); }
+    if(!g->spk || !g->spkCnt) { return fail(GENNMI_EINVAL, "push_neuron_update_group: spike queue missing"); }
+    if(g->model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
+        if(!g->startSpike || !g->endSpike || !g->spikeTimes) { return fail(GENNMI_EINVAL, "push_neuron_update_group: spike source arrays missing"); }
+    }
+    else if(g->model == GENNMI_NEURON_LIF || g->model == GENNMI_NEURON_IZHIKEVICH) {
+        if(!g->var0 || !g->var1) { return fail(GENNMI_EINVAL, "push_neuron_update_group: state variables missing"); }
+    }
+    else { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: unknown neuron model"); }
+    for(uint32_t m = 0; m < g->numPSM; m++) {
+        if(!g->psm[m].outPost) { return fail(GENNMI_EINVAL, "push_neuron_update_group: outPost missing"); }
+        if(g->psm[m].maxDenDelay && !g->psm[m].denDelay) { return fail(GENNMI_EINVAL, "push_neuron_update_group: denDelay missing"); }
+        if(g->psm[m].kind > GENNMI_PSM_DELTACURR) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: unknown postsynaptic model"); }
+    }
+    for(uint32_t c = 0; c < g->numCS; c++) {
+        if(g->cs[c].kind == GENNMI_CS_ARRAY && (!g->cs[c].array || g->cs[c].arraySteps == 0)) { return fail(GENNMI_EINVAL, "push_neuron_update_group: current-source array missing"); }
+        if(g->cs[c].kind > GENNMI_CS_ARRAY) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: unknown current source"); }
+    }
+    NeuronGroupDev d;
+    memset(&d, 0, sizeof(d));
+    d.g = *g;
+    if(idx) { *idx = (uint32_t)r->neuron.size(); }
+    r->neuron.push_back(d);
+    return GENNMI_OK;
+}
+
+int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynaptic_update_group_t *g, uint32_t *idx)
+{
+    if(!r || !g) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: null argument"); }
+    if(r->finalised) { return fail(GENNMI_ESTATE, "push_presynaptic_update_group: runner already finalised"); }
+    if(!g->srcSpk || !g->srcSpkCnt || !g->outPost || !g->g) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: required array missing"); }
+    if(g->numSrcNeurons == 0 || g->numTrgNeurons == 0) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: empty population"); }
+    PreGroupDev d;
+    memset(&d, 0, sizeof(d));
+    d.g = *g;
+    if(g->matrix == GENNMI_MATRIX_SPARSE) {
+        if(!g->rowLength || !g->ind || g->rowStride == 0) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: sparse arrays missing"); }
+        if((uint64_t)g->numSrcNeurons * g->rowStride > 0xFFFFFFFFull) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: synapse index exceeds 32 bits"); }
+        if(g->wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY) {
+            if(!g->d || !g->denDelay || g->maxDenDelay == 0) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: dendritic delay arrays missing"); }
+        }
+        else if(g->wum == GENNMI_WUM_STDP_TRACE) {
+            if(!g->trgST || !g->postTrace) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: STDP arrays missing"); }
+            if(r->batch != 1) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: plastic weights need batch size 1"); }
+        }
+        else if(g->wum != GENNMI_WUM_STATIC_PULSE) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: unknown weight update model"); }
+        if(g->wum != GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY) { d.g.maxDenDelay = 0; }
+    }
+    else if(g->matrix == GENNMI_MATRIX_TOEPLITZ_CONV2D) {
+        const int32_t *c = g->conv;
+        for(int k = 0; k < 8; k++) { if(c[k] <= 0) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: bad conv parameter"); } }
+        if((uint64_t)c[2] * c[3] * c[4] != g->numSrcNeurons || (uint64_t)c[5] * c[6] * c[7] != g->numTrgNeurons) {
+            return fail(GENNMI_EINVAL, "push_presynaptic_update_group: conv shape does not match population sizes");
+        }
+        if(g->wum != GENNMI_WUM_STATIC_PULSE) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: Toeplitz supports StaticPulse only"); }
+        // derived parameters conv_bw / conv_bh (initToeplitzConnectivitySnippet.h:113-114)
+        d.convBW = ((c[3] + c[1] - 1) - c[6]) / 2;
+        d.convBH = ((c[2] + c[0] - 1) - c[5]) / 2;
+        d.g.maxDenDelay = 0;
+    }
+    else { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: unknown matrix type"); }
+    if(idx) { *idx = (uint32_t)r->pre.size(); }
+    r->pre.push_back(d);
+    return GENNMI_OK;
+}
+
+int gennmi_push_postsynaptic_update_group(gennmi_runner *r, const gennmi_postsynaptic_update_group_t *g, uint32_t *idx)
+{
+    if(!r || !g) { return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: null argument"); }
+    if(r->finalised) { return fail(GENNMI_ESTATE, "push_postsynaptic_update_group: runner already finalised"); }
+    if(!g->colLength || !g->remap || !g->g || !g->trgSpk || !g->trgSpkCnt || !g->srcST || !g->preTrace) {
+        return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: required array missing");
+    }
+    if(g->rowStride == 0 || g->colStride == 0) { return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: zero stride"); }
+    if(r->batch != 1) { return fail(GENNMI_EUNSUPPORTED, "push_postsynaptic_update_group: plastic weights need batch size 1"); }
+    PostGroupDev d;
+    memset(&d, 0, sizeof(d));
+    d.g = *g;
+    if(idx) { *idx = (uint32_t)r->post.size(); }
+    r->post.push_back(d);
+    return GENNMI_OK;
+}
+
+int gennmi_runner_finalise(gennmi_runner *r)
+{
+    if(!r) { return fail(GENNMI_EINVAL, "runner_finalise: null runner"); }
+    if(r->finalised) { return fail(GENNMI_ESTATE, "runner_finalise: called twice"); }
+    if(r->neuron.empty()) { return fail(GENNMI_EINVAL, "runner_finalise: no neuron groups"); }
+    int device = 0;
+    HIP_TRY(hipGetDevice(&device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    const uint32_t numCU = (uint32_t)prop.multiProcessorCount;
+
+    uint32_t block = 0;
+    for(auto &n : r->neuron) {
+        n.startBlock = block;
+        n.numBlocks = (n.g.numNeurons + BLOCK - 1) / BLOCK;
+        block += n.numBlocks;
+    }
+    r->neuronBlocks = block;
+
+    // Presynaptic launch geometry.  The number of spikes is only known on the device, so every
+    // group gets enough sub-groups to keep the chip busy when its whole source population fires
+    // within a few steps, capped so that silent groups cost next to nothing.
+    block = 0;
+    const uint32_t maxBlocksPerGroup = std::max(1u, (numCU * 16u) / std::max<uint32_t>(1u, (uint32_t)r->pre.size()));
+    for(auto &p : r->pre) {
+        const uint32_t rowLen = (p.g.matrix == GENNMI_MATRIX_SPARSE) ? p.g.rowStride : (uint32_t)(p.g.conv[0] * p.g.conv[1] * p.g.conv[7]);
+        uint32_t W;
+        if(p.g.span == GENNMI_SPAN_PRE) { W = std::min(64u, pow2Ceil(std::max(1u, p.g.numThreadsPerSpike))); }
+        else if(p.g.span == GENNMI_SPAN_POST) { W = WAVE; }
+        else { W = std::min<uint32_t>(WAVE, std::max(4u, pow2Ceil((rowLen + 3) / 4))); }
+        p.lanesPerSpike = W;
+        p.vec4 = (p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum != GENNMI_WUM_STDP_TRACE && (p.g.rowStride % 4) == 0
+                  && (reinterpret_cast<uintptr_t>(p.g.ind) % 16) == 0 && (reinterpret_cast<uintptr_t>(p.g.g) % 16) == 0
+                  && (p.g.wum != GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY || (reinterpret_cast<uintptr_t>(p.g.d) % 4) == 0)
+                  && W >= 16) ? 1u : 0u;
+        // expected concurrent spikes: a few percent of the source population per step
+        const uint64_t wantSubGroups = std::max<uint64_t>(8, p.g.numSrcNeurons / 16);
+        uint32_t blocks = (uint32_t)std::min<uint64_t>((wantSubGroups * W + BLOCK - 1) / BLOCK, maxBlocksPerGroup);
+        p.startBlock = block;
+        p.numBlocks = std::max(1u, blocks);
+        block += p.numBlocks;
+    }
+    r->preBlocks = block;
+
+    block = 0;
+    for(auto &p : r->post) {
+        p.lanesPerSpike = std::min<uint32_t>(WAVE, std::max(4u, pow2Ceil((p.g.colStride + 3) / 4)));
+        const uint64_t wantSubGroups = std::max<uint64_t>(8, p.g.numTrgNeurons / 16);
+        const uint32_t cap = std::max(1u, (numCU * 16u) / (uint32_t)r->post.size());
+        p.startBlock = block;
+        p.numBlocks = std::max(1u, (uint32_t)std::min<uint64_t>((wantSubGroups * p.lanesPerSpike + BLOCK - 1) / BLOCK, cap));
+        block += p.numBlocks;
+    }
+    r->postBlocks = block;
+
+    HIP_TRY(hipMalloc(&r->dNeuron, r->neuron.size() * sizeof(NeuronGroupDev)));
+    HIP_TRY(hipMemcpy(r->dNeuron, r->neuron.data(), r->neuron.size() * sizeof(NeuronGroupDev), hipMemcpyHostToDevice));
+    if(!r->pre.empty()) {
+        HIP_TRY(hipMalloc(&r->dPre, r->pre.size() * sizeof(PreGroupDev)));
+        HIP_TRY(hipMemcpy(r->dPre, r->pre.data(), r->pre.size() * sizeof(PreGroupDev), hipMemcpyHostToDevice));
+    }
+    if(!r->post.empty()) {
+        HIP_TRY(hipMalloc(&r->dPost, r->post.size() * sizeof(PostGroupDev)));
+        HIP_TRY(hipMemcpy(r->dPost, r->post.data(), r->post.size() * sizeof(PostGroupDev), hipMemcpyHostToDevice));
+    }
+    const size_t aggCount = (size_t)r->neuronBlocks * r->batch;
+    HIP_TRY(hipMalloc(&r->dAgg, aggCount * sizeof(unsigned long long)));
+    HIP_TRY(hipMemset(r->dAgg, 0, aggCount * sizeof(unsigned long long)));
+    HIP_TRY(hipDeviceSynchronize());
+    r->finalised = true;
+    return GENNMI_OK;
+}
+
+static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
+{
+    if(timed) { HIP_TRY(hipEventRecord(r->evA, r->stream)); }
+    if(!r->pre.empty()) {
+        presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dPre, (uint32_t)r->pre.size(), a, r->dt, r->dEvents);
+        if(timed) { HIP_TRY(hipEventRecord(r->evB, r->stream)); }
+    }
+    if(!r->post.empty()) {
+        postsynapticUpdateKernel<<<dim3(r->postBlocks), dim3(BLOCK), 0, r->stream>>>(r->dPost, (uint32_t)r->post.size(), a, r->dt);
+        if(timed) { HIP_TRY(hipEventRecord(r->evC, r->stream)); }
+    }
+    HIP_TRY(hipGetLastError());
+    return GENNMI_OK;
+}
+
+static int launchNeurons(gennmi_runner *r, const StepArgs &a, bool timed)
+{
+    if(timed) { HIP_TRY(hipEventRecord(r->evC, r->stream)); }
+    neuronUpdateKernel<<<dim3(r->neuronBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dNeuron, (uint32_t)r->neuron.size(), a, r->dt, r->dAgg, r->dError);
+    if(timed) { HIP_TRY(hipEventRecord(r->evD, r->stream)); }
+    HIP_TRY(hipGetLastError());
+    return GENNMI_OK;
+}
+
+int gennmi_update_synapses(gennmi_runner *r, float t)
+{
+    if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "update_synapses: runner not finalised"); }
+    StepArgs a{};
+    a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = 0;
+    const int rc = launchSynapses(r, a, r->timing);
+    if(rc) { return rc; }
+    if(r->timing) {
+        float ms = 0;
+        if(!r->pre.empty()) {
+            HIP_TRY(hipEventSynchronize(r->evB));
+            HIP_TRY(hipEventElapsedTime(&ms, r->evA, r->evB));
+            r->preTime += ms * 1e-3; r->preLaunches++;
+        }
+        if(!r->post.empty()) {
+            HIP_TRY(hipEventSynchronize(r->evC));
+            HIP_TRY(hipEventElapsedTime(&ms, r->pre.empty() ? r->evA : r->evB, r->evC));
+            r->postTime += ms * 1e-3;
+        }
+    }
+    r->synapsesDone = true;
+    return GENNMI_OK;
+}
+
+int gennmi_update_neurons(gennmi_runner *r, float t, uint32_t recordingTimestep)
+{
+    if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "update_neurons: runner not finalised"); }
+    StepArgs a{};
+    a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recordingTimestep;
+    const int rc = launchNeurons(r, a, r->timing);
+    if(rc) { return rc; }
+    if(r->timing) {
+        float ms = 0;
+        HIP_TRY(hipEventSynchronize(r->evD));
+        HIP_TRY(hipEventElapsedTime(&ms, r->evC, r->evD));
+        r->neuronTime += ms * 1e-3; r->neuronLaunches++;
+    }
+    r->epoch++;
+    r->synapsesDone = false;
+    return GENNMI_OK;
+}
+
+int gennmi_step_time(gennmi_runner *r, unsigned long long timestep, unsigned long long numRecordingTimesteps)
+{
+    if(!r) { return fail(GENNMI_EINVAL, "step_time: null runner"); }
+    // const float t = timestep * DT  (generateRunner.cc:283)
+    const float t = (float)timestep * r->dt;
+    int rc = gennmi_update_synapses(r, t);
+    if(rc) { return rc; }
+    return gennmi_update_neurons(r, t, numRecordingTimesteps ? (uint32_t)(timestep % numRecordingTimesteps) : 0u);
+}
+
+int gennmi_run_steps(gennmi_runner *r, unsigned long long timestep, unsigned long long numSteps, unsigned long long numRecordingTimesteps)
+{
+    if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "run_steps: runner not finalised"); }
+    constexpr unsigned long long CHUNK = 100;
+    if(r->timing) {
+        for(unsigned long long s = 0; s < numSteps; s++) {
+            const int rc = gennmi_step_time(r, timestep + s, numRecordingTimesteps);
+            if(rc) { return rc; }
+        }
+        return GENNMI_OK;
+    }
+    const StepState hs{timestep, r->epoch, numRecordingTimesteps};
+    HIP_TRY(hipMemcpyAsync(r->dState, &hs, sizeof(hs), hipMemcpyHostToDevice, r->stream));
+    HIP_TRY(hipStreamSynchronize(r->stream));   // hs lives on this stack frame
+    unsigned long long done = 0;
+    while(numSteps - done >= CHUNK) {
+        if(!r->graphExec) {
+            hipGraph_t graph;
+            HIP_TRY(hipStreamBeginCapture(r->stream, hipStreamCaptureModeThreadLocal));
+            int rc = GENNMI_OK;
+            for(unsigned long long k = 0; k < CHUNK && rc == GENNMI_OK; k++) {
+                StepArgs a{};
+                a.base = r->dState; a.k = k;
+                rc = launchSynapses(r, a, false);
+                if(rc == GENNMI_OK) { rc = launchNeurons(r, a, false); }
+            }
+            advanceStepKernel<<<dim3(1), dim3(64), 0, r->stream>>>(r->dState, CHUNK);
+            const hipError_t ce = hipStreamEndCapture(r->stream, &graph);
+            if(rc) { return rc; }
+            if(ce != hipSuccess) { return fail(GENNMI_EHIP, std::string("hipStreamEndCapture: ") + hipGetErrorString(ce)); }
+            HIP_TRY(hipGraphInstantiate(&r->graphExec, graph, nullptr, nullptr, 0));
+            HIP_TRY(hipGraphDestroy(graph));
+            r->graphSteps = CHUNK;
+        }
+        HIP_TRY(hipGraphLaunch(r->graphExec, r->stream));
+        done += CHUNK;
+        r->epoch += CHUNK;
+    }
+    for(; done < numSteps; done++) {
+        StepArgs a{};
+        a.base = r->dState; a.k = 0;
+        int rc = launchSynapses(r, a, false);
+        if(rc == GENNMI_OK) { rc = launchNeurons(r, a, false); }
+        if(rc) { return rc; }
+        advanceStepKernel<<<dim3(1), dim3(64), 0, r->stream>>>(r->dState, 1);
+        r->epoch++;
+    }
+    HIP_TRY(hipGetLastError());
+    return GENNMI_OK;
+}
+
+int gennmi_runner_synchronize(gennmi_runner *r)
+{
+    if(!r) { return fail(GENNMI_EINVAL, "runner_synchronize: null runner"); }
+    HIP_TRY(hipStreamSynchronize(r->stream));
+    uint32_t err = 0;
+    HIP_TRY(hipMemcpy(&err, r->dError, sizeof(err), hipMemcpyDeviceToHost));
+    if(err) { return fail(GENNMI_EDEVICE, "neuronUpdateKernel: bounded wait for spike offsets expired"); }
+    return GENNMI_OK;
+}
+
+int gennmi_runner_set_timing(gennmi_runner *r, int enabled)
+{
+    if(!r) { return fail(GENNMI_EINVAL, "runner_set_timing: null runner"); }
+    if(enabled && !r->evA) {
+        HIP_TRY(hipEventCreate(&r->evA)); HIP_TRY(hipEventCreate(&r->evB));
+        HIP_TRY(hipEventCreate(&r->evC)); HIP_TRY(hipEventCreate(&r->evD));
+    }
+    r->timing = (enabled != 0);
+    return GENNMI_OK;
+}
+
+int gennmi_runner_get_times(gennmi_runner *r, double *neuronUpdateTime, double *presynapticUpdateTime, double *postsynapticUpdateTime)
+{
+    if(!r) { return fail(GENNMI_EINVAL, "runner_get_times: null runner"); }
+    if(neuronUpdateTime) { *neuronUpdateTime = r->neuronTime; }
+    if(presynapticUpdateTime) { *presynapticUpdateTime = r->preTime; }
+    if(postsynapticUpdateTime) { *postsynapticUpdateTime = r->postTime; }
+    return GENNMI_OK;
+}
+
+int gennmi_runner_kernel_stats(gennmi_runner *r, unsigned long long *presynLaunches, double *presynSeconds,
+                               unsigned long long *neuronLaunches, double *neuronSeconds)
+{
+    if(!r) { return fail(GENNMI_EINVAL, "runner_kernel_stats: null runner"); }
+    if(presynLaunches) { *presynLaunches = r->preLaunches; }
+    if(presynSeconds) { *presynSeconds = r->preTime; }
+    if(neuronLaunches) { *neuronLaunches = r->neuronLaunches; }
+    if(neuronSeconds) { *neuronSeconds = r->neuronTime; }
+    return GENNMI_OK;
+}
+
+int gennmi_runner_event_count(gennmi_runner *r, unsigned long long *events)
+{
+    if(!r || !events) { return fail(GENNMI_EINVAL, "runner_event_count: null argument"); }
+    HIP_TRY(hipStreamSynchronize(r->stream));
+    HIP_TRY(hipMemcpy(events, r->dEvents, sizeof(*events), hipMemcpyDeviceToHost));
+    return GENNMI_OK;
+}
+
+int gennmi_max_col_length(uint32_t numSrc, uint32_t numTrg, uint32_t rowStride, const uint32_t *rowLength, const uint32_t *ind, uint32_t *maxColLength)
+{
+    if(!rowLength || !ind || !maxColLength || rowStride == 0) { return fail(GENNMI_EINVAL, "max_col_length: bad arguments"); }
+    uint32_t *dCount = nullptr;
+    HIP_TRY(hipMalloc(&dCount, (size_t)numTrg * sizeof(uint32_t)));
+    HIP_TRY(hipMemset(dCount, 0, (size_t)numTrg * sizeof(uint32_t)));
+    const size_t total = (size_t)numSrc * rowStride;
+    remapCountKernel<<<dim3((unsigned int)((total + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, 0>>>(numSrc, rowStride, rowLength, ind, 0, dCount, nullptr, nullptr);
+    HIP_TRY(hipGetLastError());
+    std::vector<uint32_t> h(numTrg);
+    HIP_TRY(hipMemcpy(h.data(), dCount, (size_t)numTrg * sizeof(uint32_t), hipMemcpyDeviceToHost));
+    HIP_TRY(hipFree(dCount));
+    uint32_t m = 0;
+    for(uint32_t v : h) { m = std::max(m, v); }
+    *maxColLength = m;
+    return GENNMI_OK;
+}
+
+int gennmi_build_remap(uint32_t numSrc, uint32_t numTrg, uint32_t rowStride, uint32_t colStride,
+                       const uint32_t *rowLength, const uint32_t *ind, uint32_t *colLength, uint32_t *remap)
+{
+    if(!rowLength || !ind || !colLength || !remap || rowStride == 0 || colStride == 0) { return fail(GENNMI_EINVAL, "build_remap: bad arguments"); }
+    if(colStride > REMAP_SORT_MAX) { return fail(GENNMI_EUNSUPPORTED, "build_remap: column stride above 16384 is not supported"); }
+    uint32_t *dOverflow = nullptr;
+    HIP_TRY(hipMalloc(&dOverflow, sizeof(uint32_t)));
+    HIP_TRY(hipMemset(dOverflow, 0, sizeof(uint32_t)));
+    HIP_TRY(hipMemset(colLength, 0, (size_t)numTrg * sizeof(uint32_t)));
+    const size_t total = (size_t)numSrc * rowStride;
+    remapCountKernel<<<dim3((unsigned int)((total + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, 0>>>(numSrc, rowStride, rowLength, ind, colStride, colLength, remap, dOverflow);
+    HIP_TRY(hipGetLastError());
+    uint32_t overflow = 0;
+    HIP_TRY(hipMemcpy(&overflow, dOverflow, sizeof(uint32_t), hipMemcpyDeviceToHost));
+    HIP_TRY(hipFree(dOverflow));
+    if(overflow) { return fail(GENNMI_EINVAL, "build_remap: a column holds " + std::to_string(overflow) + " synapses, more than colStride"); }
+    const size_t lds = (size_t)pow2Ceil(colStride) * sizeof(uint32_t);
+    if(lds > 48 * 1024) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(remapSortKernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    }
+    remapSortKernel<<<dim3(numTrg), dim3(BLOCK), lds, 0>>>(colStride, colLength, remap);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipDeviceSynchronize());
+    return GENNMI_OK;
+}
+
+}   // extern "C"

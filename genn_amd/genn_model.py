@@ -1,0 +1,699 @@
+"""Host side of the MI355X backend: a model description with PyGeNN's surface
+(``GeNNModel.add_neuron_population / add_synapse_population / add_current_source / build /
+load / step_time``, pygenn/genn_model.py:159-847) for the fixed set of snippets on the hot path,
+plus the work the reference's ``Runtime`` does around a generated runner: allocate every array
+with the reference's names and sizes (src/genn/genn/runtime/runtime.cc:147-402), push one
+merged-group descriptor per group (runtime.h:573-669), and step.
+
+All device work goes through the C ABI in include/genn_mi355x.h; nothing here computes the
+simulation on the host.
+"""
+import ctypes as C
+import math
+from fractions import Fraction
+
+import numpy as np
+
+from . import _abi
+
+FLT_MAX = np.float32(3.402823466e+38)
+
+
+# --------------------------------------------------------------------------------------------
+# numeric literal handling
+# --------------------------------------------------------------------------------------------
+def lit32(x):
+    """fp32 value of a parameter the reference bakes into generated code as a literal:
+    double -> ``%.9e`` text -> correctly rounded float (src/genn/genn/type.cc:329-350)."""
+    x = float(x)
+    if x == 0.0 or math.isinf(x) or math.isnan(x):
+        return np.float32(x)
+    text = "%.9e" % x
+    exact = Fraction(text)
+    c = np.float32(float(text))
+    best = None
+    for cand in (np.nextafter(c, np.float32(-np.inf)), c, np.nextafter(c, np.float32(np.inf))):
+        if not np.isfinite(cand):
+            continue
+        err = abs(Fraction(float(cand)) - exact)
+        even = (int(np.float32(cand).view(np.uint32)) & 1) == 0
+        key = (err, 0 if even else 1)
+        if best is None or key < best[0]:
+            best = (key, cand)
+    return np.float32(best[1])
+
+
+def field32(x):
+    """fp32 value of a parameter that is heterogeneous across a merged group and therefore
+    travels as a struct field: a plain double->float cast (runtime.h:647-651)."""
+    return np.float32(float(x))
+
+
+def _merge_round(values):
+    """Literal rounding when every group of the merged group agrees, field rounding otherwise
+    (include/genn/genn/code_generator/environment.h:483-511)."""
+    same = all(float(v) == float(values[0]) for v in values)
+    return [lit32(v) if same else field32(v) for v in values]
+
+
+# --------------------------------------------------------------------------------------------
+# snippet initialisers with PyGeNN's names (pygenn/genn_model.py init_* helpers)
+# --------------------------------------------------------------------------------------------
+class _Init:
+    def __init__(self, snippet, params=None, vars=None, pre_vars=None, post_vars=None):
+        self.snippet = snippet
+        self.params = dict(params or {})
+        self.vars = dict(vars or {})
+        self.pre_vars = dict(pre_vars or {})
+        self.post_vars = dict(post_vars or {})
+
+
+def init_postsynaptic(snippet, params=None, vars=None):
+    if snippet not in ("ExpCurr", "DeltaCurr"):
+        raise NotImplementedError(f"postsynaptic model {snippet}")
+    return _Init(snippet, params, vars)
+
+
+def init_weight_update(snippet, params=None, vars=None, pre_vars=None, post_vars=None):
+    if snippet not in ("StaticPulse", "StaticPulseDendriticDelay", "STDPTrace"):
+        raise NotImplementedError(f"weight update model {snippet}")
+    return _Init(snippet, params, vars, pre_vars, post_vars)
+
+
+def init_toeplitz_connectivity(snippet, params=None):
+    if snippet != "Conv2D":
+        raise NotImplementedError(f"toeplitz connectivity {snippet}")
+    return _Init(snippet, params)
+
+
+# --------------------------------------------------------------------------------------------
+# device arrays (the reference's Array objects, src/genn/backends/hip/backend.cc:61-236)
+# --------------------------------------------------------------------------------------------
+class Array:
+    def __init__(self, count, dtype, fill=None):
+        self.dtype = np.dtype(dtype)
+        self.count = int(count)
+        self.view = np.zeros(self.count, dtype=self.dtype) if fill is None else np.full(self.count, fill, dtype=self.dtype)
+        self._dev = C.c_void_p()
+        _abi.check(_abi.load().gennmi_malloc(C.byref(self._dev), self.view.nbytes))
+        self.push_to_device()
+
+    @property
+    def ptr(self):
+        return self._dev.value
+
+    @property
+    def values(self):
+        return self.view
+
+    def push_to_device(self):
+        if self.view.nbytes:
+            _abi.check(_abi.load().gennmi_memcpy_to_device(self._dev, self.view.ctypes.data_as(C.c_void_p), self.view.nbytes))
+
+    def pull_from_device(self):
+        if self.view.nbytes:
+            _abi.check(_abi.load().gennmi_memcpy_from_device(self.view.ctypes.data_as(C.c_void_p), self._dev, self.view.nbytes))
+        return self.view
+
+    def free(self):
+        if self._dev:
+            _abi.load().gennmi_free(self._dev)
+            self._dev = C.c_void_p()
+
+
+class NeuronGroup:
+    def __init__(self, model, name, n, neuron, params, vars):
+        self._model = model
+        self.name = name
+        self.num_neurons = int(n)
+        self.neuron = neuron
+        self.params = dict(params)
+        self.var_init = dict(vars)
+        self.vars = {}
+        self.extra_global_params = {}
+        self.current_sources = []
+        self.in_syn = []
+        self.out_syn = []
+        self.spike_recording_enabled = False
+        self.fused_psm = []          # list of lists of SynapseGroup sharing one outPost
+        self.pre_trace_owner = None
+        self.post_trace_owner = None
+        self.needs_spike_time = False
+
+    @property
+    def size(self):
+        return self.num_neurons
+
+    def set_extra_global_param(self, name, value):
+        self.extra_global_params[name] = np.ascontiguousarray(value)
+
+    @property
+    def spike_recording_data(self):
+        """[(times, ids)] per batch, decoded from the recordSpk bitfield (runtime.cc:855-913)."""
+        return self._model._decode_recording(self)
+
+    @property
+    def current_spikes(self):
+        """Spike queue written by the last step: ids in ascending order (per batch)."""
+        cnt = self.vars["spkCnt"].pull_from_device().copy()
+        spk = self.vars["spk"].pull_from_device().reshape(self._model.batch_size, self.num_neurons)
+        return [spk[b, :cnt[b]].copy() for b in range(self._model.batch_size)]
+
+
+class CurrentSource:
+    def __init__(self, name, kind, pop, params):
+        self.name = name
+        self.kind = kind
+        self.pop = pop
+        self.params = dict(params)
+        self.extra_global_params = {}
+        self.vars = {}
+
+    def set_extra_global_param(self, name, value):
+        self.extra_global_params[name] = np.ascontiguousarray(value, dtype=np.float32)
+
+
+class SynapseGroup:
+    def __init__(self, model, name, matrix_type, src, trg, wu, ps, conn):
+        self._model = model
+        self.name = name
+        self.matrix_type = matrix_type
+        self.src = src
+        self.trg = trg
+        self.wu = wu
+        self.ps = ps
+        self.conn = conn
+        self.vars = {}
+        self.max_dendritic_delay_timesteps = 1
+        self.parallelism_hint = "POSTSYNAPTIC"
+        self.num_threads_per_spike = 1
+        self.row_stride = 0
+        self.col_stride = 0
+        self.row_length_host = None
+        self.ind_host = None
+        self.var_host = {}
+        self.fused_ps_target = self
+
+    # pygenn/genn_groups.py:434-470
+    def set_sparse_connections(self, pre_indices, post_indices):
+        pre = np.asarray(pre_indices, dtype=np.int64)
+        post = np.asarray(post_indices, dtype=np.int64)
+        order = np.lexsort((post, pre))
+        pre, post = pre[order], post[order]
+        n_pre = self.src.num_neurons
+        row_length = np.bincount(pre, minlength=n_pre).astype(np.uint32)
+        stride = int(max(1, row_length.max(initial=0)))
+        starts = np.concatenate(([0], np.cumsum(row_length)[:-1])).astype(np.int64)
+        within = np.arange(len(pre), dtype=np.int64) - starts[pre]
+        ind = np.zeros((n_pre, stride), dtype=np.uint32)
+        ind[pre, within] = post
+        self.set_ragged(row_length, ind)
+        self._coo = (order, pre, within)
+
+    def set_ragged(self, row_length, ind):
+        """Adopt connectivity already in the reference's ragged layout."""
+        ind = np.ascontiguousarray(ind, dtype=np.uint32)
+        self.row_length_host = np.ascontiguousarray(row_length, dtype=np.uint32)
+        self.ind_host = ind.reshape(self.src.num_neurons, -1)
+        self.row_stride = self.ind_host.shape[1]
+
+    def set_var_ragged(self, name, values):
+        self.var_host[name] = np.ascontiguousarray(values)
+
+    def set_var_coo(self, name, values):
+        """Per-synapse values in the order the COO lists were given to set_sparse_connections."""
+        order, pre, within = self._coo
+        dtype = np.uint8 if name == "d" else np.float32
+        out = np.zeros(self.ind_host.shape, dtype=dtype)
+        out[pre, within] = np.asarray(values)[order]
+        self.var_host[name] = out
+
+    @property
+    def num_synapses(self):
+        return int(self.row_length_host.sum())
+
+    def get_var_values(self, name):
+        """Pull a per-synapse variable and return the valid entries in row-major order."""
+        a = self.vars[name].pull_from_device().reshape(self.src.num_neurons, self.row_stride)
+        mask = np.arange(self.row_stride)[None, :] < self.row_length_host[:, None]
+        return a[mask]
+
+
+class GeNNModel:
+    def __init__(self, precision="float", model_name="model", batch_size=1, dt=1.0, device=0):
+        if precision != "float":
+            raise NotImplementedError("only fp32 models are supported")
+        self.name = model_name
+        self.batch_size = int(batch_size)
+        self.dt = float(dt)
+        self.fuse_postsynaptic_models = False
+        self.timing_enabled = False
+        self.neuron_populations = {}
+        self.synapse_populations = {}
+        self.current_sources = {}
+        self.timestep = 0
+        self._runner = C.c_void_p()
+        self._built = False
+        self._loaded = False
+        self._device = device
+        self._arrays = []
+        self.num_recording_timesteps = None
+
+    # ------------------------------------------------------------------ description
+    def add_neuron_population(self, pop_name, num_neurons, neuron, params=None, vars=None):
+        if neuron not in ("LIF", "Izhikevich", "SpikeSourceArray"):
+            raise NotImplementedError(f"neuron model {neuron}")
+        if pop_name in self.neuron_populations:
+            raise ValueError(f"duplicate neuron population {pop_name}")
+        g = NeuronGroup(self, pop_name, num_neurons, neuron, params or {}, vars or {})
+        self.neuron_populations[pop_name] = g
+        return g
+
+    def add_current_source(self, cs_name, current_source_model, pop, params=None, vars=None):
+        if current_source_model not in ("DC", "ArrayNoise"):
+            raise NotImplementedError(f"current source {current_source_model}")
+        cs = CurrentSource(cs_name, current_source_model, pop, params or {})
+        pop.current_sources.append(cs)
+        self.current_sources[cs_name] = cs
+        return cs
+
+    def add_synapse_population(self, pop_name, matrix_type, source, target, weight_update_init, postsynaptic_init,
+                               connectivity_init=None):
+        if matrix_type not in ("SPARSE", "TOEPLITZ"):
+            raise NotImplementedError(f"matrix type {matrix_type}")
+        if matrix_type == "TOEPLITZ" and (connectivity_init is None or connectivity_init.snippet != "Conv2D"):
+            raise ValueError("TOEPLITZ connectivity needs init_toeplitz_connectivity('Conv2D', ...)")
+        s = SynapseGroup(self, pop_name, matrix_type, source, target, weight_update_init, postsynaptic_init, connectivity_init)
+        self.synapse_populations[pop_name] = s
+        source.out_syn.append(s)
+        target.in_syn.append(s)
+        return s
+
+    # ------------------------------------------------------------------ build = finalise + derive constants
+    def build(self):
+        lib = _abi.load()
+        _abi.check(lib.gennmi_init(self._device))
+        for n in self.neuron_populations.values():
+            # fuse postsynaptic models (src/genn/genn/neuronGroup.cc:436): same snippet, same parameters,
+            # same dendritic-delay depth, no state variables
+            # fusing walks the incoming projections from the last one added to the first
+            # (fuseSynapseGroups, src/genn/genn/neuronGroup.cc:41-96), which fixes both the child
+            # order (it decides the order in which Isyn is summed) and the owner of a fused outPost
+            n.fused_psm = []
+            for s in reversed(n.in_syn):
+                key = (s.ps.snippet, tuple(sorted(s.ps.params.items())), self._den_delay(s))
+                target = None
+                if self.fuse_postsynaptic_models:
+                    for grp in n.fused_psm:
+                        o = grp[0]
+                        if (o.ps.snippet, tuple(sorted(o.ps.params.items())), self._den_delay(o)) == key:
+                            target = grp
+                            break
+                if target is None:
+                    n.fused_psm.append([s])
+                    s.fused_ps_target = s
+                else:
+                    target.append(s)
+                    s.fused_ps_target = target[0]
+            if len(n.fused_psm) > _abi.MAX_PSM:
+                raise NotImplementedError(f"{n.name}: more than {_abi.MAX_PSM} postsynaptic models after fusing")
+            if len(n.current_sources) > _abi.MAX_CS:
+                raise NotImplementedError(f"{n.name}: more than {_abi.MAX_CS} current sources")
+            pre = [s for s in n.out_syn if s.wu.snippet == "STDPTrace"]
+            post = [s for s in n.in_syn if s.wu.snippet == "STDPTrace"]
+            if len(pre) > 1 or len(post) > 1:
+                raise NotImplementedError(f"{n.name}: more than one plastic projection per side")
+            n.pre_trace_owner = pre[0] if pre else None
+            n.post_trace_owner = post[0] if post else None
+            n.needs_spike_time = bool(pre or post)
+        self._built = True
+
+    @staticmethod
+    def _den_delay(s):
+        return s.max_dendritic_delay_timesteps if s.wu.snippet == "StaticPulseDendriticDelay" else 0
+
+    def _alloc(self, count, dtype, fill=None):
+        a = Array(count, dtype, fill)
+        self._arrays.append(a)
+        return a
+
+    # ------------------------------------------------------------------ load = allocate + push merged groups
+    def load(self, num_recording_timesteps=None):
+        if not self._built:
+            raise RuntimeError("build() must be called before load()")
+        lib = _abi.load()
+        B = self.batch_size
+        self.num_recording_timesteps = num_recording_timesteps
+        dt32 = lit32(self.dt)
+        _abi.check(lib.gennmi_runner_create(C.byref(self._runner), C.c_float(dt32), B))
+
+        # ---- neuron-group arrays (runtime.cc:156-282)
+        for n in self.neuron_populations.values():
+            N = n.num_neurons
+            if n.neuron == "SpikeSourceArray":
+                for v in ("startSpike", "endSpike"):
+                    a = self._alloc(B * N, np.uint32)
+                    a.view[:] = np.broadcast_to(np.asarray(n.var_init[v], dtype=np.uint32), (B, N)).reshape(-1) \
+                        if np.ndim(n.var_init[v]) < 2 else np.asarray(n.var_init[v], dtype=np.uint32).reshape(-1)
+                    a.push_to_device()
+                    n.vars[v] = a
+                st = np.ascontiguousarray(n.extra_global_params["spikeTimes"], dtype=np.float32)
+                a = self._alloc(max(1, st.size), np.float32)
+                a.view[:st.size] = st
+                a.push_to_device()
+                n.vars["spikeTimes"] = a
+            else:
+                names = ("V", "RefracTime") if n.neuron == "LIF" else ("V", "U")
+                for v in names:
+                    a = self._alloc(B * N, np.float32)
+                    init = np.asarray(n.var_init[v], dtype=np.float32)
+                    a.view[:] = np.broadcast_to(init, (B, N)).reshape(-1) if init.ndim < 2 else init.reshape(-1)
+                    a.push_to_device()
+                    n.vars[v] = a
+            n.vars["spkCnt"] = self._alloc(B, np.uint32)
+            n.vars["spk"] = self._alloc(B * N, np.uint32)
+            if n.spike_recording_enabled:
+                if not num_recording_timesteps:
+                    raise RuntimeError("Cannot use recording system without specifying number of recording timesteps")
+                n.vars["recordSpk"] = self._alloc(((N + 31) // 32) * B * num_recording_timesteps, np.uint32)
+            if n.needs_spike_time:
+                n.vars["sT"] = self._alloc(B * N, np.float32, fill=-FLT_MAX)      # -TIME_MAX, as the reference's initialize()
+            for grp in n.fused_psm:
+                owner = grp[0]
+                owner.vars["outPost"] = self._alloc(B * N, np.float32)
+                D = self._den_delay(owner)
+                if D:
+                    owner.vars["denDelay"] = self._alloc(B * D * N, np.float32)
+                    owner.vars["denDelayPtr"] = self._alloc(1, np.uint32)
+            if n.pre_trace_owner is not None:
+                n.pre_trace_owner.vars["preTrace"] = self._alloc(B * N, np.float32)
+            if n.post_trace_owner is not None:
+                n.post_trace_owner.vars["postTrace"] = self._alloc(B * N, np.float32)
+            for cs in n.current_sources:
+                if cs.kind == "ArrayNoise":
+                    noise = np.ascontiguousarray(cs.extra_global_params["noise"], dtype=np.float32)
+                    if noise.size % N:
+                        raise ValueError(f"{cs.name}: noise array is not a multiple of the population size")
+                    a = self._alloc(noise.size, np.float32)
+                    a.view[:] = noise.reshape(-1)
+                    a.push_to_device()
+                    cs.vars["noise"] = a
+
+        # ---- synapse-group arrays (runtime.cc:330-402)
+        for s in self.synapse_populations.values():
+            if s.matrix_type == "SPARSE":
+                if s.ind_host is None:
+                    raise RuntimeError(f"{s.name}: sparse connectivity has not been set")
+                n_pre = s.src.num_neurons
+                for name, host, dtype in (("rowLength", s.row_length_host, np.uint32), ("ind", s.ind_host, np.uint32)):
+                    a = self._alloc(host.size, dtype)
+                    a.view[:] = host.reshape(-1)
+                    a.push_to_device()
+                    s.vars[name] = a
+                names = ["g"] + (["d"] if s.wu.snippet == "StaticPulseDendriticDelay" else [])
+                for name in names:
+                    dtype = np.uint8 if name == "d" else np.float32
+                    a = self._alloc(n_pre * s.row_stride, dtype)
+                    if name in s.var_host:
+                        a.view[:] = np.asarray(s.var_host[name], dtype=dtype).reshape(-1)
+                    else:
+                        a.view[:] = dtype(s.wu.vars[name])
+                    a.push_to_device()
+                    s.vars[name] = a
+            else:
+                kern = np.ascontiguousarray(s.var_host.get("g", s.wu.vars.get("g")), dtype=np.float32)
+                a = self._alloc(kern.size, np.float32)
+                a.view[:] = kern.reshape(-1)
+                a.push_to_device()
+                s.vars["g"] = a
+
+        self._initialize_sparse()
+        self._push_merged_groups()
+        _abi.check(lib.gennmi_runner_finalise(self._runner))
+        if self.timing_enabled:
+            _abi.check(lib.gennmi_runner_set_timing(self._runner, 1))
+        self._loaded = True
+        self.timestep = 0
+
+    def _initialize_sparse(self):
+        """initializeSparse(): column views for projections with postsynaptic-spike code."""
+        lib = _abi.load()
+        for s in self.synapse_populations.values():
+            if s.wu.snippet != "STDPTrace":
+                continue
+            n_pre, n_post = s.src.num_neurons, s.trg.num_neurons
+            m = C.c_uint32()
+            _abi.check(lib.gennmi_max_col_length(n_pre, n_post, s.row_stride, s.vars["rowLength"].ptr, s.vars["ind"].ptr, C.byref(m)))
+            s.col_stride = max(1, int(m.value)) if not s.col_stride else s.col_stride
+            s.vars["colLength"] = self._alloc(n_post, np.uint32)
+            s.vars["remap"] = self._alloc(n_post * s.col_stride, np.uint32)
+            _abi.check(lib.gennmi_build_remap(n_pre, n_post, s.row_stride, s.col_stride, s.vars["rowLength"].ptr,
+                                              s.vars["ind"].ptr, s.vars["colLength"].ptr, s.vars["remap"].ptr))
+
+    # merged-group membership as the reference would form it (same model code and structure)
+    def _neuron_merge_key(self, n):
+        psm = tuple((grp[0].ps.snippet, self._den_delay(grp[0])) for grp in self._sorted_psm(n))
+        return (n.neuron, psm, tuple(cs.kind for cs in n.current_sources), n.pre_trace_owner is not None,
+                n.post_trace_owner is not None, n.needs_spike_time, n.spike_recording_enabled)
+
+    def _sorted_psm(self, n):
+        # children are ordered by a structure-only digest, ties keep creation order (groupMerged.h:411-454)
+        return sorted(n.fused_psm, key=lambda grp: (grp[0].ps.snippet, self._den_delay(grp[0])))
+
+    def _push_merged_groups(self):
+        lib = _abi.load()
+        B = self.batch_size
+        merged = {}
+        for n in self.neuron_populations.values():
+            merged.setdefault(self._neuron_merge_key(n), []).append(n)
+        for members in merged.values():
+            model = members[0].neuron
+            descs = [_abi.NeuronUpdateGroup() for _ in members]
+            for d, n in zip(descs, members):
+                d.model = {"LIF": _abi.NEURON_LIF, "Izhikevich": _abi.NEURON_IZHIKEVICH, "SpikeSourceArray": _abi.NEURON_SPIKE_SOURCE_ARRAY}[model]
+                d.numNeurons = n.num_neurons
+                d.spkCnt, d.spk = n.vars["spkCnt"].ptr, n.vars["spk"].ptr
+                d.recordSpk = n.vars["recordSpk"].ptr if "recordSpk" in n.vars else None
+                d.sT = n.vars["sT"].ptr if "sT" in n.vars else None
+            if model == "SpikeSourceArray":
+                for d, n in zip(descs, members):
+                    d.startSpike, d.endSpike, d.spikeTimes = n.vars["startSpike"].ptr, n.vars["endSpike"].ptr, n.vars["spikeTimes"].ptr
+            elif model == "LIF":
+                def derived(n):
+                    p = n.params
+                    return [p["Ioffset"], p["TauM"] / p["C"], p["Vrest"], math.exp(-self.dt / p["TauM"]), p["Vthresh"], p["Vreset"], p["TauRefrac"]]
+                cols = list(zip(*[derived(n) for n in members]))
+                rounded = [_merge_round(list(col)) for col in cols]
+                for k, (d, n) in enumerate(zip(descs, members)):
+                    d.var0, d.var1 = n.vars["V"].ptr, n.vars["RefracTime"].ptr
+                    for j in range(7):
+                        d.params[j] = rounded[j][k]
+            else:
+                cols = list(zip(*[[n.params[q] for q in ("a", "b", "c", "d")] for n in members]))
+                rounded = [_merge_round(list(col)) for col in cols]
+                for k, (d, n) in enumerate(zip(descs, members)):
+                    d.var0, d.var1 = n.vars["V"].ptr, n.vars["U"].ptr
+                    for j in range(4):
+                        d.params[j] = rounded[j][k]
+            # postsynaptic-model children
+            num_psm = len(members[0].fused_psm)
+            for m in range(num_psm):
+                owners = [self._sorted_psm(n)[m][0] for n in members]
+                if owners[0].ps.snippet == "ExpCurr":
+                    taus = [o.ps.params["tau"] for o in owners]
+                    decay = _merge_round([math.exp(-self.dt / tau) for tau in taus])
+                    init = _merge_round([(tau * (1.0 - math.exp(-self.dt / tau))) * (1.0 / self.dt) for tau in taus])
+                for k, (d, o) in enumerate(zip(descs, owners)):
+                    p = d.psm[m]
+                    p.outPost = o.vars["outPost"].ptr
+                    D = self._den_delay(o)
+                    p.maxDenDelay = D
+                    if D:
+                        p.denDelay, p.denDelayPtr = o.vars["denDelay"].ptr, o.vars["denDelayPtr"].ptr
+                    if o.ps.snippet == "ExpCurr":
+                        p.kind, p.init, p.expDecay = _abi.PSM_EXPCURR, init[k], decay[k]
+                    else:
+                        p.kind = _abi.PSM_DELTACURR
+            for d in descs:
+                d.numPSM = num_psm
+            # current-source children
+            num_cs = len(members[0].current_sources)
+            for c in range(num_cs):
+                srcs = [n.current_sources[c] for n in members]
+                if srcs[0].kind == "DC":
+                    amps = _merge_round([cs.params["amp"] for cs in srcs])
+                for k, (d, cs, n) in enumerate(zip(descs, srcs, members)):
+                    if cs.kind == "DC":
+                        d.cs[c].kind, d.cs[c].amp = _abi.CS_DC, amps[k]
+                    else:
+                        d.cs[c].kind, d.cs[c].array = _abi.CS_ARRAY, cs.vars["noise"].ptr
+                        d.cs[c].arraySteps = cs.vars["noise"].count // n.num_neurons
+            for d in descs:
+                d.numCS = num_cs
+            # weight-update pre / post children (trace decay is a derived parameter of the WU model)
+            if members[0].pre_trace_owner is not None:
+                dec = _merge_round([math.exp(-self.dt / n.pre_trace_owner.wu.params["tauPlus"]) for n in members])
+                for k, (d, n) in enumerate(zip(descs, members)):
+                    d.preTrace, d.preDecay = n.pre_trace_owner.vars["preTrace"].ptr, dec[k]
+            if members[0].post_trace_owner is not None:
+                dec = _merge_round([math.exp(-self.dt / n.post_trace_owner.wu.params["tauMinus"]) for n in members])
+                for k, (d, n) in enumerate(zip(descs, members)):
+                    d.postTrace, d.postDecay = n.post_trace_owner.vars["postTrace"].ptr, dec[k]
+            for d in descs:
+                _abi.check(lib.gennmi_push_neuron_update_group(self._runner, C.byref(d), None))
+
+        # presynaptic / postsynaptic update groups; merged by weight-update code and matrix type
+        syn_merged = {}
+        for s in self.synapse_populations.values():
+            syn_merged.setdefault((s.matrix_type, s.wu.snippet, self._den_delay(s) > 0), []).append(s)
+        for members in syn_merged.values():
+            stdp = members[0].wu.snippet == "STDPTrace"
+            if stdp:
+                rounded = {q: _merge_round([s.wu.params[q] for s in members]) for q in ("aPlus", "aMinus", "wMin", "wMax")}
+            for k, s in enumerate(members):
+                d = _abi.PresynapticUpdateGroup()
+                d.matrix = _abi.MATRIX_SPARSE if s.matrix_type == "SPARSE" else _abi.MATRIX_TOEPLITZ_CONV2D
+                d.wum = {"StaticPulse": _abi.WUM_STATIC_PULSE, "StaticPulseDendriticDelay": _abi.WUM_STATIC_PULSE_DENDRITIC_DELAY,
+                         "STDPTrace": _abi.WUM_STDP_TRACE}[s.wu.snippet]
+                d.span = {"POSTSYNAPTIC": _abi.SPAN_AUTO, "PRESYNAPTIC": _abi.SPAN_PRE, "WAVE": _abi.SPAN_POST}[s.parallelism_hint]
+                d.numThreadsPerSpike = s.num_threads_per_spike
+                d.numSrcNeurons, d.numTrgNeurons = s.src.num_neurons, s.trg.num_neurons
+                owner = s.fused_ps_target
+                d.outPost = owner.vars["outPost"].ptr
+                d.srcSpkCnt, d.srcSpk = s.src.vars["spkCnt"].ptr, s.src.vars["spk"].ptr
+                d.g = s.vars["g"].ptr
+                if s.matrix_type == "SPARSE":
+                    d.rowStride = s.row_stride
+                    d.rowLength, d.ind = s.vars["rowLength"].ptr, s.vars["ind"].ptr
+                    D = self._den_delay(s)
+                    if D:
+                        d.maxDenDelay = D
+                        d.d = s.vars["d"].ptr
+                        d.denDelay, d.denDelayPtr = owner.vars["denDelay"].ptr, owner.vars["denDelayPtr"].ptr
+                else:
+                    for j, q in enumerate(("conv_kh", "conv_kw", "conv_ih", "conv_iw", "conv_ic", "conv_oh", "conv_ow", "conv_oc")):
+                        d.conv[j] = int(s.conn.params[q])
+                if stdp:
+                    d.trgST, d.postTrace = s.trg.vars["sT"].ptr, s.vars["postTrace"].ptr
+                    d.aMinus, d.wMin, d.wMax = rounded["aMinus"][k], rounded["wMin"][k], rounded["wMax"][k]
+                _abi.check(lib.gennmi_push_presynaptic_update_group(self._runner, C.byref(d), None))
+                if stdp:
+                    q = _abi.PostsynapticUpdateGroup()
+                    q.numSrcNeurons, q.numTrgNeurons = s.src.num_neurons, s.trg.num_neurons
+                    q.rowStride, q.colStride = s.row_stride, s.col_stride
+                    q.colLength, q.remap, q.g = s.vars["colLength"].ptr, s.vars["remap"].ptr, s.vars["g"].ptr
+                    q.trgSpkCnt, q.trgSpk = s.trg.vars["spkCnt"].ptr, s.trg.vars["spk"].ptr
+                    q.srcST, q.preTrace = s.src.vars["sT"].ptr, s.vars["preTrace"].ptr
+                    q.aPlus, q.wMin, q.wMax = rounded["aPlus"][k], rounded["wMin"][k], rounded["wMax"][k]
+                    _abi.check(lib.gennmi_push_postsynaptic_update_group(self._runner, C.byref(q), None))
+
+    # ------------------------------------------------------------------ stepping
+    @property
+    def t(self):
+        return float(np.float32(self.timestep) * lit32(self.dt))
+
+    def step_time(self):
+        nrec = self.num_recording_timesteps or 0
+        _abi.check(_abi.load().gennmi_step_time(self._runner, self.timestep, nrec))
+        self.timestep += 1
+
+    def run(self, num_steps):
+        """num_steps consecutive step_time() calls replayed from captured HIP graphs."""
+        nrec = self.num_recording_timesteps or 0
+        _abi.check(_abi.load().gennmi_run_steps(self._runner, self.timestep, int(num_steps), nrec))
+        self.timestep += int(num_steps)
+
+    def synchronize(self):
+        _abi.check(_abi.load().gennmi_runner_synchronize(self._runner))
+
+    def pull_recording_buffers_from_device(self):
+        self.synchronize()
+        for n in self.neuron_populations.values():
+            if "recordSpk" in n.vars:
+                n.vars["recordSpk"].pull_from_device()
+
+    def _decode_recording(self, n):
+        words = (n.num_neurons + 31) // 32
+        rec = n.vars["recordSpk"].view.reshape(self.num_recording_timesteps, self.batch_size, words)
+        bits = np.unpackbits(rec.view(np.uint8), axis=2, bitorder="little")[:, :, :n.num_neurons]
+        start = self.timestep - self.num_recording_timesteps if self.timestep >= self.num_recording_timesteps else 0
+        out = []
+        for b in range(self.batch_size):
+            steps, ids = np.nonzero(bits[:, b, :])
+            out.append(((start + steps).astype(np.float64) * self.dt, ids.astype(np.uint32)))
+        return out
+
+    @property
+    def synaptic_event_count(self):
+        v = C.c_ulonglong()
+        _abi.check(_abi.load().gennmi_runner_event_count(self._runner, C.byref(v)))
+        return int(v.value)
+
+    def kernel_stats(self):
+        a, b = C.c_ulonglong(), C.c_double()
+        c, d = C.c_ulonglong(), C.c_double()
+        _abi.check(_abi.load().gennmi_runner_kernel_stats(self._runner, C.byref(a), C.byref(b), C.byref(c), C.byref(d)))
+        return {"presyn_launches": a.value, "presyn_seconds": b.value, "neuron_launches": c.value, "neuron_seconds": d.value}
+
+    def set_timing(self, enabled):
+        _abi.check(_abi.load().gennmi_runner_set_timing(self._runner, int(bool(enabled))))
+
+    def unload(self):
+        if self._runner:
+            _abi.load().gennmi_runner_destroy(self._runner)
+            self._runner = C.c_void_p()
+        for a in self._arrays:
+            a.free()
+        self._arrays = []
+        self._loaded = False
+
+
+# --------------------------------------------------------------------------------------------
+def model_from_net(net, batch_size=1, record=True, span=None, device=0):
+    """Build a GeNNModel from a :class:`genn_amd.netspec.Net` (arrays are loaded, never generated here)."""
+    m = GeNNModel("float", net.name, batch_size=batch_size, dt=net.dt, device=device)
+    m.fuse_postsynaptic_models = net.fuse_psm
+    pops = {}
+    for p in net.pops:
+        if p.model == "lif":
+            g = m.add_neuron_population(p.name, p.n, "LIF", p.params, p.vars)
+        elif p.model == "izh":
+            g = m.add_neuron_population(p.name, p.n, "Izhikevich", p.params, p.vars)
+        else:
+            g = m.add_neuron_population(p.name, p.n, "SpikeSourceArray", {}, p.vars)
+            g.set_extra_global_param("spikeTimes", p.spike_times)
+        g.spike_recording_enabled = record
+        pops[p.name] = g
+    for c in net.css:
+        if c.model == "dc":
+            m.add_current_source(c.name, "DC", pops[c.pop], {"amp": c.amp})
+        else:
+            cs = m.add_current_source(c.name, "ArrayNoise", pops[c.pop])
+            cs.set_extra_global_param("noise", c.noise)
+    for s in net.syns:
+        ps = init_postsynaptic("ExpCurr", {"tau": s.tau}) if s.psm == "expcurr" else init_postsynaptic("DeltaCurr")
+        if s.wum == "static":
+            wu = init_weight_update("StaticPulse", {}, {"g": 0.0})
+        elif s.wum == "static_delay":
+            wu = init_weight_update("StaticPulseDendriticDelay", {}, {"g": 0.0, "d": 0})
+        else:
+            wu = init_weight_update("STDPTrace", s.wum_params, {"g": 0.0}, {"preTrace": 0.0}, {"postTrace": 0.0})
+        if s.matrix == "sparse":
+            sg = m.add_synapse_population(s.name, "SPARSE", pops[s.src], pops[s.trg], wu, ps)
+            sg.set_ragged(s.row_length, s.ind)
+            sg.set_var_ragged("g", s.g)
+            if s.d is not None:
+                sg.set_var_ragged("d", s.d)
+            if s.max_den_delay:
+                sg.max_dendritic_delay_timesteps = s.max_den_delay
+            if s.hint_pre:
+                sg.parallelism_hint = "PRESYNAPTIC"
+                sg.num_threads_per_spike = s.threads_per_spike
+            if span is not None:
+                sg.parallelism_hint = span
+        else:
+            sg = m.add_synapse_population(s.name, "TOEPLITZ", pops[s.src], pops[s.trg], wu, ps,
+                                          init_toeplitz_connectivity("Conv2D", s.conv))
+            sg.set_var_ragged("g", s.g)
+    m.build()
+    return m

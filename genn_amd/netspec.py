@@ -1,0 +1,170 @@
+"""Plain-data description of a spiking network: populations, current sources, projections.
+
+This is the one description every executor consumes: the MI355X engine (through the C-ABI),
+the CPU oracle under ``oracle/`` (tests and the bench's CPU baseline only) and, in the
+builder container, the reference's own SingleThreadedCPU backend via ``oracle/ref_driver.cc``
+(which reads the directory written by :func:`write_netspec`).  All arrays use the reference's
+ragged SPARSE layout (``rowLength[numPre]``, ``ind/g/d[numPre*rowStride]`` with identical
+padding; src/genn/genn/runtime/runtime.cc:360-402).
+"""
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+import hashlib
+import os
+
+import numpy as np
+
+NEURON_MODELS = ("lif", "izh", "ssa")
+LIF_PARAMS = ("C", "TauM", "Vrest", "Vreset", "Vthresh", "Ioffset", "TauRefrac")
+IZH_PARAMS = ("a", "b", "c", "d")
+STDP_PARAMS = ("tauPlus", "tauMinus", "aPlus", "aMinus", "wMin", "wMax")
+CONV_PARAMS = ("conv_kh", "conv_kw", "conv_ih", "conv_iw", "conv_ic", "conv_oh", "conv_ow", "conv_oc")
+
+
+@dataclass
+class Pop:
+    name: str
+    model: str                      # "lif" | "izh" | "ssa"
+    n: int
+    params: Dict[str, float] = field(default_factory=dict)
+    vars: Dict[str, np.ndarray] = field(default_factory=dict)   # V/RefracTime, V/U, startSpike/endSpike
+    spike_times: Optional[np.ndarray] = None                    # ssa only (fp32, ms)
+
+
+@dataclass
+class CurrentSource:
+    name: str
+    model: str                      # "dc" | "noise"
+    pop: str
+    amp: float = 0.0
+    noise: Optional[np.ndarray] = None   # fp32 [steps, n] for "noise"
+
+
+@dataclass
+class Syn:
+    name: str
+    src: str
+    trg: str
+    matrix: str = "sparse"          # "sparse" | "conv2d"
+    wum: str = "static"             # "static" | "static_delay" | "stdp_trace"
+    wum_params: Dict[str, float] = field(default_factory=dict)
+    psm: str = "expcurr"            # "expcurr" | "deltacurr"
+    tau: float = 5.0
+    row_stride: int = 0
+    row_length: Optional[np.ndarray] = None   # uint32 [numPre]
+    ind: Optional[np.ndarray] = None          # uint32 [numPre, rowStride]
+    g: Optional[np.ndarray] = None            # fp32 [numPre, rowStride] or kernel [kh,kw,ic,oc]
+    d: Optional[np.ndarray] = None            # uint8 [numPre, rowStride]
+    max_den_delay: int = 0
+    hint_pre: bool = False
+    col_stride: int = 0             # longest column (plastic projections); 0 = let the executor size it
+    threads_per_spike: int = 1
+    conv: Dict[str, int] = field(default_factory=dict)
+
+    @property
+    def num_synapses(self):
+        return int(self.row_length.sum()) if self.row_length is not None else 0
+
+
+@dataclass
+class Net:
+    name: str
+    dt: float
+    steps: int
+    pops: List[Pop] = field(default_factory=list)
+    css: List[CurrentSource] = field(default_factory=list)
+    syns: List[Syn] = field(default_factory=list)
+    fuse_psm: bool = False
+    seed: int = 0
+
+    def pop(self, name):
+        return next(p for p in self.pops if p.name == name)
+
+    def syn(self, name):
+        return next(s for s in self.syns if s.name == name)
+
+    def input_digest(self):
+        """SHA-1 over every input array; stored beside golden outputs to detect generator drift."""
+        h = hashlib.sha1()
+        for p in self.pops:
+            for k in sorted(p.vars):
+                h.update(np.ascontiguousarray(p.vars[k]).tobytes())
+            if p.spike_times is not None:
+                h.update(np.ascontiguousarray(p.spike_times).tobytes())
+        for c in self.css:
+            if c.noise is not None:
+                h.update(np.ascontiguousarray(c.noise).tobytes())
+        for s in self.syns:
+            for a in (s.row_length, s.ind, s.g, s.d):
+                if a is not None:
+                    h.update(np.ascontiguousarray(a).tobytes())
+        return h.hexdigest()
+
+
+def ragged_from_lists(n_pre, pre, post, stride=None, sort=True):
+    """Build (rowLength, ind[numPre,stride], order) from COO lists the way
+    pygenn/genn_groups.py:434-470 does: lexsort by (pre, post), stride = longest row."""
+    pre = np.asarray(pre, dtype=np.int64)
+    post = np.asarray(post, dtype=np.int64)
+    order = np.lexsort((post, pre)) if sort else np.argsort(pre, kind="stable")
+    pre_s, post_s = pre[order], post[order]
+    row_length = np.bincount(pre_s, minlength=n_pre).astype(np.uint32)
+    stride = int(stride if stride is not None else max(1, row_length.max(initial=0)))
+    starts = np.concatenate(([0], np.cumsum(row_length)[:-1])).astype(np.int64)
+    within = np.arange(len(pre_s), dtype=np.int64) - starts[pre_s]
+    ind = np.zeros((n_pre, stride), dtype=np.uint32)
+    ind[pre_s, within] = post_s
+    return row_length, ind, order, (pre_s, within)
+
+
+def write_netspec(net: Net, path: str):
+    """Write the directory format read by oracle/ref_driver.cc."""
+    os.makedirs(path, exist_ok=True)
+    lines = [f"model {net.name}", f"dt {net.dt!r}", f"steps {net.steps}", f"fuse_psm {int(net.fuse_psm)}"]
+    snap = getattr(net, "snap", 0)
+    lines.append(f"snap {snap}")
+    for p in net.pops:
+        if p.model == "lif":
+            ps = " ".join(repr(float(p.params[k])) for k in LIF_PARAMS)
+        elif p.model == "izh":
+            ps = " ".join(repr(float(p.params[k])) for k in IZH_PARAMS)
+        else:
+            ps = ""
+        lines.append(f"pop {p.name} {p.model} {p.n} {ps}".rstrip())
+        for k, v in p.vars.items():
+            suffix = "u32" if v.dtype == np.uint32 else "f32"
+            np.ascontiguousarray(v).tofile(os.path.join(path, f"{p.name}.{k}.{suffix}"))
+        if p.spike_times is not None:
+            np.ascontiguousarray(p.spike_times, dtype=np.float32).tofile(os.path.join(path, f"{p.name}.spikeTimes.f32"))
+    for c in net.css:
+        if c.model == "dc":
+            lines.append(f"cs {c.name} dc {c.pop} {float(c.amp)!r}")
+        else:
+            lines.append(f"cs {c.name} noise {c.pop}")
+            np.ascontiguousarray(c.noise, dtype=np.float32).tofile(os.path.join(path, f"{c.name}.noise.f32"))
+    for s in net.syns:
+        if s.matrix == "sparse":
+            head = f"syn {s.name} sparse {s.src} {s.trg} {s.row_stride}"
+            np.ascontiguousarray(s.row_length, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.rowLength.u32"))
+            np.ascontiguousarray(s.ind, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.ind.u32"))
+        else:
+            head = f"syn {s.name} conv2d {s.src} {s.trg} " + " ".join(str(int(s.conv[k])) for k in CONV_PARAMS)
+        np.ascontiguousarray(s.g, dtype=np.float32).tofile(os.path.join(path, f"{s.name}.g.f32"))
+        if s.wum == "static":
+            w = "static"
+        elif s.wum == "static_delay":
+            w = f"static_delay {s.max_den_delay}"
+            np.ascontiguousarray(s.d, dtype=np.uint8).tofile(os.path.join(path, f"{s.name}.d.u8"))
+        elif s.wum == "stdp_trace":
+            w = "stdp_trace " + " ".join(repr(float(s.wum_params[k])) for k in STDP_PARAMS)
+        else:
+            raise ValueError(s.wum)
+        psm = f"expcurr {float(s.tau)!r}" if s.psm == "expcurr" else "deltacurr"
+        opts = (" hint_pre" if s.hint_pre else "") + (f" tps {s.threads_per_spike}" if s.threads_per_spike > 1 else "")
+        if s.wum == "stdp_trace":
+            mask = np.arange(s.row_stride)[None, :] < s.row_length[:, None]
+            col = s.col_stride or int(np.bincount(s.ind[mask], minlength=net.pop(s.trg).n).max())
+            opts += f" col_stride {max(1, col)}"
+        lines.append(f"{head} {w} {psm}{opts}")
+    with open(os.path.join(path, "net.txt"), "w") as f:
+        f.write("\n".join(lines) + "\n")

@@ -1,0 +1,204 @@
+/*
+ * genn_mi355x.h — C ABI of the MI355X (gfx950) device layer for GeNN's per-timestep hot path.
+ *
+ * Everything a generated runner needs to step a spiking network on one MI355X without
+ * containing any device code itself: the runner is plain host C++ that fills merged-group
+ * descriptors (the counterpart of the reference's pushMerged<Name>Group<i>ToDevice calls) and
+ * calls the entry points below.  Signatures use plain pointers and sizes only.
+ *
+ * Every function returns 0 on success or a negative GENNMI_E* code; gennmi_last_error()
+ * returns a description of the last failure on the calling thread.  The reference signals
+ * the same conditions by throwing std::runtime_error from CHECK_RUNTIME_ERRORS
+ * (src/genn/backends/hip/backend.cc:696-701); a C++ runner turns a non-zero return into that.
+ *
+ * All device pointers are addresses returned by gennmi_malloc (or any hipMalloc'd memory of
+ * the same process).  Memory is owned by the caller — the reference's Runtime owns arrays
+ * through backend Array objects and the runner only receives pointers
+ * (src/genn/genn/runtime/runtime.cc:147-402, include/genn/genn/runtime/runtime.h:573-669).
+ */
+#ifndef GENN_MI355X_H
+#define GENN_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GENNMI_OK            0
+#define GENNMI_EHIP         -1   /* a HIP runtime call failed */
+#define GENNMI_EINVAL       -2   /* descriptor inconsistent with what the kernels assume */
+#define GENNMI_EUNSUPPORTED -3   /* feature outside the supported model set */
+#define GENNMI_ESTATE       -4   /* call order violated (e.g. step before finalise) */
+#define GENNMI_EDEVICE      -5   /* a kernel reported an internal failure (bounded wait expired) */
+
+#define GENNMI_MAX_PSM 8         /* fused postsynaptic models per neuron group */
+#define GENNMI_MAX_CS  4         /* current sources per neuron group */
+
+/* neuron models: include/genn/genn/neuronModels.h:220-257 (LIF), :163-186 (Izhikevich), :274-286 (SpikeSourceArray) */
+enum { GENNMI_NEURON_LIF = 0, GENNMI_NEURON_IZHIKEVICH = 1, GENNMI_NEURON_SPIKE_SOURCE_ARRAY = 2 };
+/* postsynaptic models: include/genn/genn/postsynapticModels.h:91-106 (ExpCurr), DeltaCurr */
+enum { GENNMI_PSM_EXPCURR = 0, GENNMI_PSM_DELTACURR = 1 };
+/* current sources: include/genn/genn/currentSourceModels.h:70-77 (DC); ARRAY injects noise[step*numNeurons+id] */
+enum { GENNMI_CS_DC = 0, GENNMI_CS_ARRAY = 1 };
+/* weight update models: include/genn/genn/weightUpdateModels.h:236-244, :279-287; trace STDP pygenn/genn_model.py:1448-1476 */
+enum { GENNMI_WUM_STATIC_PULSE = 0, GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY = 1, GENNMI_WUM_STDP_TRACE = 2 };
+/* connectivity: ragged SPARSE (runtime.cc:360-402) or TOEPLITZ Conv2D (initToeplitzConnectivitySnippet.h:105-150) */
+enum { GENNMI_MATRIX_SPARSE = 0, GENNMI_MATRIX_TOEPLITZ_CONV2D = 1 };
+/* presynaptic strategies: presynapticUpdateStrategySIMT.cc:57-162 (PreSpan), :167-389 (PostSpan) */
+enum { GENNMI_SPAN_AUTO = 0, GENNMI_SPAN_POST = 1, GENNMI_SPAN_PRE = 2 };
+
+/* ---------------------------------------------------------------------------------------------
+ * Thin device layer.  Replaces the hip* calls the reference emits inline into generated code and
+ * its Array class (src/genn/backends/hip/backend.cc:61-236: allocate/free/push/pull/memset).
+ * ------------------------------------------------------------------------------------------- */
+int gennmi_init(int device);                                   /* hip/backend.cc:290-322 (device select) */
+const char *gennmi_last_error(void);
+int gennmi_device_name(char *buf, size_t len);
+int gennmi_malloc(void **devPtr, size_t bytes);                 /* Array::allocate  hip/backend.cc:86-108 */
+int gennmi_free(void *devPtr);                                  /* Array::free      hip/backend.cc:110-128 */
+int gennmi_memcpy_to_device(void *dev, const void *host, size_t bytes);    /* pushToDevice / pushSlice1DToDevice   :130-176 */
+int gennmi_memcpy_from_device(void *host, const void *dev, size_t bytes);  /* pullFromDevice / pullSlice1DFromDevice :142-198 */
+int gennmi_memset(void *dev, int value, size_t bytes);          /* memsetDeviceObject :200-204 */
+int gennmi_fill_f32(float *dev, float value, size_t count);     /* e.g. sT = -TIME_MAX (initGroupMerged.cc neuron init) */
+int gennmi_synchronize(void);
+int gennmi_free_device_memory_bytes(size_t *bytes);             /* genReturnFreeDeviceMemoryBytes, backendCUDAHIP.cc */
+
+/* ---------------------------------------------------------------------------------------------
+ * Merged-group descriptors.  Field names follow the reference's merged structs
+ * (src/genn/genn/code_generator/backendBase.cc:104-380); one descriptor = one group of one
+ * merged group, i.e. one pushMerged<Name>Group<i>ToDevice(idx, ...) call.
+ * Per-neuron arrays hold batchSize*numNeurons elements, batch-major.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct gennmi_psm_t {             /* one fused postsynaptic model ("InSyn" child, neuronUpdateGroupMerged.cc:66-137) */
+    float *outPost;                       /* [batch*numNeurons] */
+    float *denDelay;                      /* [batch*maxDenDelay*numNeurons] slot-major, or NULL */
+    uint32_t *denDelayPtr;                /* [1] device-resident head pointer, or NULL */
+    float init, expDecay;                 /* ExpCurr derived parameters, already rounded to fp32 */
+    uint32_t kind;                        /* GENNMI_PSM_* */
+    uint32_t maxDenDelay;                 /* 0 = no dendritic delay */
+} gennmi_psm_t;
+
+typedef struct gennmi_cs_t {              /* one current source child (neuronUpdateGroupMerged.cc:20-55) */
+    const float *array;                   /* GENNMI_CS_ARRAY: [numSteps*numNeurons]; row (step % arraySteps) is injected */
+    float amp;                            /* GENNMI_CS_DC */
+    uint32_t kind;
+    uint32_t arraySteps;
+    uint32_t pad_;
+} gennmi_cs_t;
+
+typedef struct gennmi_neuron_update_group_t {      /* MergedNeuronUpdateGroup<i> */
+    uint32_t model;                       /* GENNMI_NEURON_* */
+    uint32_t numNeurons;
+    float *var0, *var1;                   /* LIF: V, RefracTime.  Izhikevich: V, U */
+    uint32_t *startSpike;                 /* SpikeSourceArray state [batch*numNeurons] */
+    const uint32_t *endSpike;             /* [batch*numNeurons] */
+    const float *spikeTimes;              /* shared across batches */
+    /* LIF: Ioffset, Rmembrane, Vrest, ExpTC, Vthresh, Vreset, TauRefrac.  Izhikevich: a, b, c, d. */
+    float params[8];
+    uint32_t numPSM, numCS;
+    gennmi_psm_t psm[GENNMI_MAX_PSM];
+    gennmi_cs_t cs[GENNMI_MAX_CS];
+    float *preTrace, *postTrace;          /* fused WU pre / post variables (OutSynWUMPre / InSynWUMPost children), or NULL */
+    float preDecay, postDecay;
+    float *sT;                            /* spike times [batch*numNeurons] or NULL */
+    uint32_t *spkCnt;                     /* [batch] */
+    uint32_t *spk;                        /* [batch*numNeurons], ascending neuron index within a step */
+    uint32_t *recordSpk;                  /* [numRecordingTimesteps*batch*ceil(numNeurons/32)] or NULL (runtime.cc:169) */
+} gennmi_neuron_update_group_t;
+
+typedef struct gennmi_presynaptic_update_group_t { /* MergedPresynapticUpdateGroup<i> */
+    uint32_t matrix;                      /* GENNMI_MATRIX_* */
+    uint32_t wum;                         /* GENNMI_WUM_* */
+    uint32_t span;                        /* GENNMI_SPAN_* (parallelism hint, synapseGroup.h:42-47) */
+    uint32_t numThreadsPerSpike;          /* PreSpan only (synapseGroup.h:135) */
+    uint32_t numSrcNeurons, numTrgNeurons;
+    uint32_t rowStride;
+    uint32_t maxDenDelay;
+    const uint32_t *rowLength;            /* [numSrcNeurons] */
+    const uint32_t *ind;                  /* [numSrcNeurons*rowStride] */
+    float *g;                             /* [numSrcNeurons*rowStride], or Toeplitz kernel [kh*kw*ic*oc] */
+    const uint8_t *d;                     /* [numSrcNeurons*rowStride] dendritic delay in timesteps */
+    float *outPost;                       /* fused PSM target of this group */
+    float *denDelay;
+    uint32_t *denDelayPtr;
+    const uint32_t *srcSpkCnt, *srcSpk;
+    const float *trgST;                   /* STDP: postsynaptic spike times */
+    const float *postTrace;
+    float aMinus, wMin, wMax;
+    int32_t conv[8];                      /* conv_kh, conv_kw, conv_ih, conv_iw, conv_ic, conv_oh, conv_ow, conv_oc */
+} gennmi_presynaptic_update_group_t;
+
+typedef struct gennmi_postsynaptic_update_group_t { /* MergedPostsynapticUpdateGroup<i> */
+    uint32_t numSrcNeurons, numTrgNeurons;
+    uint32_t rowStride, colStride;
+    const uint32_t *colLength;            /* [numTrgNeurons] */
+    const uint32_t *remap;                /* [numTrgNeurons*colStride] */
+    float *g;
+    const uint32_t *trgSpkCnt, *trgSpk;
+    const float *srcST, *preTrace;
+    float aPlus, wMin, wMax;
+    uint32_t pad_;
+} gennmi_postsynaptic_update_group_t;
+
+/* ---------------------------------------------------------------------------------------------
+ * Runner: the device-side half of one generated librunner.so.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct gennmi_runner gennmi_runner;
+
+/* allocateMem()  generateRunner.cc:241-252.  dt is the fp32 time-precision literal of the model's DT. */
+int gennmi_runner_create(gennmi_runner **runner, float dt, uint32_t batchSize);
+/* freeMem()  generateRunner.cc:256-265 */
+int gennmi_runner_destroy(gennmi_runner *runner);
+
+/* pushMergedNeuronUpdateGroup<i>ToDevice(idx, fields...)  backendCUDAHIP.h:206-238, runtime.h:573-669.
+ * Groups are appended; *idx receives the position.  Pushing is only legal before finalise. */
+int gennmi_push_neuron_update_group(gennmi_runner *runner, const gennmi_neuron_update_group_t *group, uint32_t *idx);
+int gennmi_push_presynaptic_update_group(gennmi_runner *runner, const gennmi_presynaptic_update_group_t *group, uint32_t *idx);
+int gennmi_push_postsynaptic_update_group(gennmi_runner *runner, const gennmi_postsynaptic_update_group_t *group, uint32_t *idx);
+
+/* Validates descriptors against the kernels' assumptions, uploads the descriptor tables, fixes
+ * the launch geometry.  Corresponds to the end of Runtime::allocate (runtime.cc:497-661). */
+int gennmi_runner_finalise(gennmi_runner *runner);
+
+/* initializeSparse(): builds colLength / remap for one SPARSE matrix with the reference's CPU
+ * ordering (ascending idSyn within a column; single_threaded_cpu/backend.cc:156-179), replacing
+ * the order-nondeterministic atomic build of backendSIMT.cc:1977-1991. */
+int gennmi_build_remap(uint32_t numSrcNeurons, uint32_t numTrgNeurons, uint32_t rowStride, uint32_t colStride,
+                       const uint32_t *rowLength, const uint32_t *ind, uint32_t *colLength, uint32_t *remap);
+/* Longest column of a SPARSE matrix (what SynapseGroup::getMaxSourceConnections must cover). */
+int gennmi_max_col_length(uint32_t numSrcNeurons, uint32_t numTrgNeurons, uint32_t rowStride,
+                          const uint32_t *rowLength, const uint32_t *ind, uint32_t *maxColLength);
+
+/* updateSynapses(t)  backendCUDAHIP.cc:548-589: dendritic-delay pointer advance, presynaptic
+ * update, postsynaptic update.  updateNeurons(t, recordingTimestep)  backendCUDAHIP.cc:386-420:
+ * spike-queue reset and neuron update.  Asynchronous on the runner's stream. */
+int gennmi_update_synapses(gennmi_runner *runner, float t);
+int gennmi_update_neurons(gennmi_runner *runner, float t, uint32_t recordingTimestep);
+/* stepTime(timestep, numRecordingTimesteps)  generateRunner.cc:270-299 */
+int gennmi_step_time(gennmi_runner *runner, unsigned long long timestep, unsigned long long numRecordingTimesteps);
+/* numSteps consecutive stepTime calls starting at `timestep`, replayed from a captured HIP
+ * graph so that no per-kernel launch latency is paid (no counterpart in the reference, which
+ * launches 4-7 kernels per step from the host). */
+int gennmi_run_steps(gennmi_runner *runner, unsigned long long timestep, unsigned long long numSteps,
+                     unsigned long long numRecordingTimesteps);
+/* stepTimeFinalise: blocks until everything queued has finished and reports device-side
+ * failures (backendCUDAHIP.cc:1400-1411). */
+int gennmi_runner_synchronize(gennmi_runner *runner);
+
+/* Timers: neuronUpdateTime / presynapticUpdateTime / postsynapticUpdateTime of generateRunner.cc:161-174,
+ * in seconds, accumulated with HIP events while enabled (backendCUDAHIP.cc:36-76, 1479-1504). */
+int gennmi_runner_set_timing(gennmi_runner *runner, int enabled);
+int gennmi_runner_get_times(gennmi_runner *runner, double *neuronUpdateTime, double *presynapticUpdateTime,
+                            double *postsynapticUpdateTime);
+/* Launch counts and average HIP-event duration of the presynaptic kernel since the last reset. */
+int gennmi_runner_kernel_stats(gennmi_runner *runner, unsigned long long *presynLaunches, double *presynSeconds,
+                               unsigned long long *neuronLaunches, double *neuronSeconds);
+/* Synaptic events processed so far per presynaptic group (device counter, enabled with timing). */
+int gennmi_runner_event_count(gennmi_runner *runner, unsigned long long *events);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,376 @@
+// Test infrastructure, not product code.
+//
+// Drives the reference's OWN SingleThreadedCPU backend (built by oracle/Makefile.ref into
+// oracle/_ref/) on a network described by a "netspec" directory written by
+// genn_amd/netspec.py, and dumps spike rasters and state snapshots.  Those dumps become the
+// golden fixtures under tests/golden/ and validate the C restatement in oracle/genn_cpu.c.
+//
+// The flow follows the reference's generator driver (src/genn/generator/generator.cc:55-121):
+// ModelSpecInternal -> finalise -> createBackend -> ModelSpecMerged -> generateAll ->
+// generateMakefile -> make -> Runtime -> allocate / initialize / (load arrays) /
+// initializeSparse / stepTime.  All inputs (connectivity, weights, delays, initial state,
+// spike-source arrays, noise) are LOADED from the netspec; none of the reference's seeded
+// initialisation snippets is used, because their draw order cannot be reproduced elsewhere.
+//
+// usage: ref_driver <netspec dir> <work dir> <out dir>
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <iostream>
+#include <map>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include <plog/Appenders/ConsoleAppender.h>
+#include "path.h"
+#include "logging.h"
+#include "modelSpecInternal.h"
+#include "code_generator/generateMakefile.h"
+#include "code_generator/generateModules.h"
+#include "code_generator/modelSpecMerged.h"
+#include "runtime/runtime.h"
+#include "optimiser.h"
+
+using namespace GeNN;
+using namespace GeNN::CodeGenerator::SingleThreadedCPU;
+
+// ---------------------------------------------------------------------------------------------
+// Models that are not built into the reference (declared the way a user of its C++ API would)
+// ---------------------------------------------------------------------------------------------
+// All-to-all trace STDP: the "stdp_additive_2" example of pygenn/genn_model.py:1448-1476
+class TraceSTDP : public WeightUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(TraceSTDP);
+    SET_PARAMS({"tauPlus", "tauMinus", "aPlus", "aMinus", "wMin", "wMax"});
+    SET_DERIVED_PARAMS({
+        {"tauPlusDecay", [](const ParamValues &p, double dt){ return std::exp(-dt / p.at("tauPlus").cast<double>()); }},
+        {"tauMinusDecay", [](const ParamValues &p, double dt){ return std::exp(-dt / p.at("tauMinus").cast<double>()); }}});
+    SET_VARS({{"g", "scalar"}});
+    SET_PRE_VARS({{"preTrace", "scalar"}});
+    SET_POST_VARS({{"postTrace", "scalar"}});
+    SET_PRE_SPIKE_SYN_CODE(
+        "addToPost(g);\n"
+        "const scalar dt = t - st_post;\n"
+        "if(dt > 0) {\n"
+        "    const scalar newWeight = g - (aMinus * postTrace);\n"
+        "    g = fmin(wMax, fmax(wMin, newWeight));\n"
+        "}\n");
+    SET_POST_SPIKE_SYN_CODE(
+        "const scalar dt = t - st_pre;\n"
+        "if(dt > 0) {\n"
+        "    const scalar newWeight = g + (aPlus * preTrace);\n"
+        "    g = fmin(wMax, fmax(wMin, newWeight));\n"
+        "}\n");
+    SET_PRE_SPIKE_CODE("preTrace += 1.0;\n");
+    SET_PRE_DYNAMICS_CODE("preTrace *= tauPlusDecay;\n");
+    SET_POST_SPIKE_CODE("postTrace += 1.0;\n");
+    SET_POST_DYNAMICS_CODE("postTrace *= tauMinusDecay;\n");
+};
+IMPLEMENT_SNIPPET(TraceSTDP);
+
+// Current source fed from a host-pregenerated array; the driver rewrites the N-element
+// window before every step, so the injected value at step s is noise[s*N + id].
+class ArrayNoise : public CurrentSourceModels::Base
+{
+public:
+    DECLARE_SNIPPET(ArrayNoise);
+    SET_INJECTION_CODE("injectCurrent(noise[id]);\n");
+    SET_EXTRA_GLOBAL_PARAMS({{"noise", "scalar*"}});
+};
+IMPLEMENT_SNIPPET(ArrayNoise);
+
+// ---------------------------------------------------------------------------------------------
+template<typename T>
+static std::vector<T> readFile(const std::string &path, size_t expect = 0)
+{
+    std::ifstream f(path, std::ios::binary | std::ios::ate);
+    if(!f) { throw std::runtime_error("cannot open " + path); }
+    const size_t bytes = (size_t)f.tellg();
+    f.seekg(0);
+    std::vector<T> v(bytes / sizeof(T));
+    f.read(reinterpret_cast<char*>(v.data()), bytes);
+    if(expect && v.size() != expect) {
+        throw std::runtime_error(path + ": expected " + std::to_string(expect) + " elements, got " + std::to_string(v.size()));
+    }
+    return v;
+}
+
+template<typename T>
+static void appendFile(const std::string &path, const T *data, size_t n)
+{
+    std::ofstream f(path, std::ios::binary | std::ios::app);
+    f.write(reinterpret_cast<const char*>(data), n * sizeof(T));
+}
+
+struct PopSpec { std::string name, model; unsigned int n; std::vector<double> p; NeuronGroup *ng = nullptr; };
+struct CSSpec { std::string name, model, pop; std::vector<double> p; CurrentSource *cs = nullptr; };
+struct SynSpec
+{
+    std::string name, matrix, src, trg, wum, psm;
+    unsigned int rowStride = 0, maxDenDelay = 0, tps = 1, colStride = 0;
+    bool hintPre = false;
+    std::vector<double> conv, wumP, psmP;
+    SynapseGroup *sg = nullptr;
+};
+
+int main(int argc, char *argv[])
+{
+    try {
+        if(argc != 4) { std::cerr << "usage: ref_driver <netspec dir> <work dir> <out dir>" << std::endl; return 1; }
+        const std::string in = argv[1], work = argv[2], out = argv[3];
+
+        plog::ConsoleAppender<plog::TxtFormatter> app;
+        Preferences prefs;
+        Logging::init(prefs.gennLogLevel, prefs.codeGeneratorLogLevel, prefs.transpilerLogLevel,
+                      prefs.runtimeLogLevel, &app, &app, &app, &app);
+
+        // ---- parse net.txt -----------------------------------------------------------------
+        std::string name = "net";
+        double dt = 1.0;
+        unsigned int steps = 1, snap = 0, fuse = 0;
+        std::vector<PopSpec> pops; std::vector<CSSpec> css; std::vector<SynSpec> syns;
+        {
+            std::ifstream f(in + "/net.txt");
+            if(!f) { throw std::runtime_error("no net.txt in " + in); }
+            std::string line;
+            while(std::getline(f, line)) {
+                std::istringstream ls(line);
+                std::string k; if(!(ls >> k) || k[0] == '#') { continue; }
+                if(k == "model") ls >> name;
+                else if(k == "dt") ls >> dt;
+                else if(k == "steps") ls >> steps;
+                else if(k == "snap") ls >> snap;
+                else if(k == "fuse_psm") ls >> fuse;
+                else if(k == "pop") { PopSpec p; ls >> p.name >> p.model >> p.n; double v; while(ls >> v) p.p.push_back(v); pops.push_back(p); }
+                else if(k == "cs") { CSSpec c; ls >> c.name >> c.model >> c.pop; double v; while(ls >> v) c.p.push_back(v); css.push_back(c); }
+                else if(k == "syn") {
+                    SynSpec s; ls >> s.name >> s.matrix >> s.src >> s.trg;
+                    if(s.matrix == "sparse") { ls >> s.rowStride; }
+                    else if(s.matrix == "conv2d") { s.conv.resize(8); for(auto &c : s.conv) ls >> c; }
+                    else throw std::runtime_error("matrix " + s.matrix);
+                    ls >> s.wum;
+                    if(s.wum == "static_delay") { ls >> s.maxDenDelay; }
+                    else if(s.wum == "stdp_trace" || s.wum == "stdp") { s.wumP.resize(6); for(auto &c : s.wumP) ls >> c; }
+                    else if(s.wum != "static") throw std::runtime_error("wum " + s.wum);
+                    ls >> s.psm;
+                    if(s.psm == "expcurr") { s.psmP.resize(1); ls >> s.psmP[0]; }
+                    else if(s.psm != "deltacurr") throw std::runtime_error("psm " + s.psm);
+                    std::string o;
+                    while(ls >> o) { if(o == "hint_pre") s.hintPre = true; else if(o == "tps") ls >> s.tps; else if(o == "col_stride") ls >> s.colStride; else throw std::runtime_error("opt " + o); }
+                    syns.push_back(s);
+                }
+                else throw std::runtime_error("unknown key " + k);
+            }
+        }
+
+        // ---- build ModelSpec ---------------------------------------------------------------
+        ModelSpecInternal model;
+        model.setName(name);
+        model.setDT(dt);
+        model.setPrecision(Type::Float);
+        model.setFusePostsynapticModels(fuse != 0);
+        std::map<std::string, PopSpec*> popByName;
+        for(auto &p : pops) {
+            if(p.model == "lif") {
+                p.ng = model.addNeuronPopulation<NeuronModels::LIF>(p.name, p.n,
+                    {{"C", p.p.at(0)}, {"TauM", p.p.at(1)}, {"Vrest", p.p.at(2)}, {"Vreset", p.p.at(3)},
+                     {"Vthresh", p.p.at(4)}, {"Ioffset", p.p.at(5)}, {"TauRefrac", p.p.at(6)}},
+                    {{"V", uninitialisedVar()}, {"RefracTime", uninitialisedVar()}});
+            }
+            else if(p.model == "izh") {
+                p.ng = model.addNeuronPopulation<NeuronModels::Izhikevich>(p.name, p.n,
+                    {{"a", p.p.at(0)}, {"b", p.p.at(1)}, {"c", p.p.at(2)}, {"d", p.p.at(3)}},
+                    {{"V", uninitialisedVar()}, {"U", uninitialisedVar()}});
+            }
+            else if(p.model == "ssa") {
+                p.ng = model.addNeuronPopulation<NeuronModels::SpikeSourceArray>(p.name, p.n, {},
+                    {{"startSpike", uninitialisedVar()}, {"endSpike", uninitialisedVar()}});
+            }
+            else throw std::runtime_error("pop model " + p.model);
+            p.ng->setSpikeRecordingEnabled(true);
+            popByName[p.name] = &p;
+        }
+        for(auto &c : css) {
+            NeuronGroup *ng = popByName.at(c.pop)->ng;
+            if(c.model == "dc") c.cs = model.addCurrentSource<CurrentSourceModels::DC>(c.name, ng, {{"amp", c.p.at(0)}}, {});
+            else if(c.model == "noise") c.cs = model.addCurrentSource<ArrayNoise>(c.name, ng, {}, {});
+            else throw std::runtime_error("cs model " + c.model);
+        }
+        for(auto &s : syns) {
+            NeuronGroup *src = popByName.at(s.src)->ng, *trg = popByName.at(s.trg)->ng;
+            const auto psm = (s.psm == "expcurr") ? initPostsynaptic<PostsynapticModels::ExpCurr>({{"tau", s.psmP[0]}})
+                                                  : initPostsynaptic<PostsynapticModels::DeltaCurr>();
+            WeightUpdateModels::Init wum = initWeightUpdate<WeightUpdateModels::StaticPulse>({}, {{"g", uninitialisedVar()}});
+            if(s.wum == "static_delay") {
+                wum = initWeightUpdate<WeightUpdateModels::StaticPulseDendriticDelay>({}, {{"g", uninitialisedVar()}, {"d", uninitialisedVar()}});
+            }
+            else if(s.wum == "stdp_trace") {
+                wum = initWeightUpdate<TraceSTDP>(
+                    {{"tauPlus", s.wumP[0]}, {"tauMinus", s.wumP[1]}, {"aPlus", s.wumP[2]}, {"aMinus", s.wumP[3]}, {"wMin", s.wumP[4]}, {"wMax", s.wumP[5]}},
+                    {{"g", uninitialisedVar()}}, {{"preTrace", uninitialisedVar()}}, {{"postTrace", uninitialisedVar()}});
+            }
+            else if(s.wum == "stdp") {
+                wum = initWeightUpdate<WeightUpdateModels::STDP>(
+                    {{"tauPlus", s.wumP[0]}, {"tauMinus", s.wumP[1]}, {"Aplus", s.wumP[2]}, {"Aminus", s.wumP[3]}, {"Wmin", s.wumP[4]}, {"Wmax", s.wumP[5]}},
+                    {{"g", uninitialisedVar()}});
+            }
+            if(s.matrix == "sparse") {
+                s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::SPARSE, src, trg, wum, psm);
+                s.sg->setMaxConnections(s.rowStride);
+                if(s.colStride) s.sg->setMaxSourceConnections(s.colStride);
+            }
+            else {
+                s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::TOEPLITZ, src, trg, wum, psm,
+                    initToeplitzConnectivity<InitToeplitzConnectivitySnippet::Conv2D>(
+                        {{"conv_kh", (int)s.conv[0]}, {"conv_kw", (int)s.conv[1]}, {"conv_ih", (int)s.conv[2]}, {"conv_iw", (int)s.conv[3]},
+                         {"conv_ic", (int)s.conv[4]}, {"conv_oh", (int)s.conv[5]}, {"conv_ow", (int)s.conv[6]}, {"conv_oc", (int)s.conv[7]}}));
+            }
+            if(s.maxDenDelay) s.sg->setMaxDendriticDelayTimesteps(s.maxDenDelay);
+            if(s.hintPre) s.sg->setParallelismHint(SynapseGroup::ParallelismHint::PRESYNAPTIC);
+            if(s.tps > 1) s.sg->setNumThreadsPerSpike(s.tps);
+        }
+        model.finalise();
+
+        // ---- generate + build --------------------------------------------------------------
+        const filesystem::path targetPath(work);
+        const filesystem::path outputPath = targetPath / (model.getName() + "_CODE");
+        filesystem::create_directory(outputPath);
+        auto backend = Optimiser::createBackend(model, outputPath, prefs.backendLogLevel, &app, prefs);
+        CodeGenerator::ModelSpecMerged modelMerged(backend, model);
+        const auto moduleNames = CodeGenerator::generateAll(modelMerged, backend, outputPath, true);
+        {
+            std::ofstream makefile((outputPath / "Makefile").str());
+            CodeGenerator::generateMakefile(makefile, backend, moduleNames);
+        }
+        const std::string cmd = "make -s -C \"" + outputPath.str() + "\" -j 8";
+        if(system(cmd.c_str()) != 0) { throw std::runtime_error("build failed: " + cmd); }
+
+        // ---- run ---------------------------------------------------------------------------
+        Runtime::Runtime rt(targetPath, modelMerged, backend);
+        rt.allocate(steps);
+        rt.initialize();
+        auto load = [&](Runtime::ArrayBase *a, const std::string &file) {
+            const auto bytes = readFile<char>(in + "/" + file, a->getSizeBytes());
+            std::copy(bytes.begin(), bytes.end(), reinterpret_cast<char*>(a->getHostPointer()));
+        };
+        for(auto &p : pops) {
+            if(p.model == "lif") { load(rt.getArray(*p.ng, "V"), p.name + ".V.f32"); load(rt.getArray(*p.ng, "RefracTime"), p.name + ".RefracTime.f32"); }
+            else if(p.model == "izh") { load(rt.getArray(*p.ng, "V"), p.name + ".V.f32"); load(rt.getArray(*p.ng, "U"), p.name + ".U.f32"); }
+            else if(p.model == "ssa") {
+                load(rt.getArray(*p.ng, "startSpike"), p.name + ".startSpike.u32");
+                load(rt.getArray(*p.ng, "endSpike"), p.name + ".endSpike.u32");
+                const auto st = readFile<float>(in + "/" + p.name + ".spikeTimes.f32");
+                rt.allocateArray(*p.ng, "spikeTimes", st.size());
+                auto *a = rt.getArray(*p.ng, "spikeTimes");
+                std::copy(st.begin(), st.end(), a->getHostPointer<float>());
+                a->pushToDevice();
+            }
+        }
+        std::map<std::string, std::vector<float>> noise;
+        for(auto &c : css) {
+            if(c.model == "noise") {
+                const unsigned int n = popByName.at(c.pop)->n;
+                noise[c.name] = readFile<float>(in + "/" + c.name + ".noise.f32", (size_t)n * steps);
+                rt.allocateArray(*c.cs, "noise", n);
+            }
+        }
+        for(auto &s : syns) {
+            if(s.matrix == "sparse") {
+                load(rt.getArray(*s.sg, "rowLength"), s.name + ".rowLength.u32");
+                load(rt.getArray(*s.sg, "ind"), s.name + ".ind.u32");
+            }
+            load(rt.getArray(*s.sg, "g"), s.name + ".g.f32");
+            if(s.wum == "static_delay") load(rt.getArray(*s.sg, "d"), s.name + ".d.u8");
+            if(s.wum == "stdp_trace") {
+                rt.getArray(*s.sg, "preTrace")->memsetHostPointer(0);
+                rt.getArray(*s.sg, "postTrace")->memsetHostPointer(0);
+            }
+        }
+        rt.initializeSparse();
+
+        // fuse map + remap dump
+        {
+            std::ofstream fm(out + "/fusemap.txt");
+            for(auto &s : syns) {
+                const auto *sgi = static_cast<const SynapseGroupInternal*>(s.sg);
+                fm << s.name << " " << sgi->getFusedPSTarget().getName() << std::endl;
+                if(s.wum == "stdp_trace" || s.wum == "stdp") {
+                    auto *cl = rt.getArray(*s.sg, "colLength"); auto *rm = rt.getArray(*s.sg, "remap");
+                    appendFile(out + "/" + s.name + ".colLength.u32", cl->getHostPointer<uint32_t>(), cl->getCount());
+                    appendFile(out + "/" + s.name + ".remap.u32", rm->getHostPointer<uint32_t>(), rm->getCount());
+                    std::ofstream(out + "/" + s.name + ".colStride.txt") << sgi->getMaxSourceConnections() << std::endl;
+                }
+            }
+        }
+
+        auto snapshot = [&]() {
+            for(auto &p : pops) {
+                if(p.model == "ssa") continue;
+                appendFile(out + "/" + p.name + ".V.f32", rt.getArray(*p.ng, "V")->getHostPointer<float>(), p.n);
+                if(p.model == "lif") appendFile(out + "/" + p.name + ".RefracTime.f32", rt.getArray(*p.ng, "RefracTime")->getHostPointer<float>(), p.n);
+                if(p.model == "izh") appendFile(out + "/" + p.name + ".U.f32", rt.getArray(*p.ng, "U")->getHostPointer<float>(), p.n);
+            }
+            for(auto &s : syns) {
+                const auto *sgi = static_cast<const SynapseGroupInternal*>(s.sg);
+                if(&sgi->getFusedPSTarget() == sgi) {
+                    auto *a = rt.getArray(*s.sg, "outPost");
+                    appendFile(out + "/" + s.name + ".outPost.f32", a->getHostPointer<float>(), a->getCount());
+                    if(sgi->isDendriticOutputDelayRequired()) {
+                        auto *d = rt.getArray(*s.sg, "denDelay");
+                        appendFile(out + "/" + s.name + ".denDelay.f32", d->getHostPointer<float>(), d->getCount());
+                    }
+                }
+                if(s.wum == "stdp_trace" || s.wum == "stdp") {
+                    auto *a = rt.getArray(*s.sg, "g");
+                    appendFile(out + "/" + s.name + ".g.f32", a->getHostPointer<float>(), a->getCount());
+                }
+                if(s.wum == "stdp_trace") {
+                    auto *a = rt.getArray(*s.sg, "preTrace"); auto *b = rt.getArray(*s.sg, "postTrace");
+                    appendFile(out + "/" + s.name + ".preTrace.f32", a->getHostPointer<float>(), a->getCount());
+                    appendFile(out + "/" + s.name + ".postTrace.f32", b->getHostPointer<float>(), b->getCount());
+                }
+            }
+        };
+
+        for(unsigned int i = 0; i < steps; i++) {
+            for(auto &c : css) {
+                if(c.model == "noise") {
+                    const unsigned int n = popByName.at(c.pop)->n;
+                    auto *a = rt.getArray(*c.cs, "noise");
+                    std::copy_n(noise[c.name].begin() + (size_t)i * n, n, a->getHostPointer<float>());
+                    a->pushToDevice();
+                }
+            }
+            rt.stepTime();
+            if(snap && ((i + 1) % snap) == 0) snapshot();
+        }
+        if(!snap || (steps % snap) != 0) snapshot();
+
+        // spike rasters as (step, id) pairs; the reference reports times in ms = step*dt
+        rt.pullRecordingBuffersFromDevice();
+        for(auto &p : pops) {
+            const auto ev = rt.getRecordedSpikes(*p.ng);
+            // the reference's decode lists the ids of one timestep in bit-scan order; sort them
+            std::vector<std::pair<uint32_t, uint32_t>> sorted;
+            const auto &times = ev.at(0).first; const auto &ids = ev.at(0).second;
+            for(size_t k = 0; k < times.size(); k++) {
+                sorted.emplace_back((uint32_t)std::llround(times[k] / dt), ids[k]);
+            }
+            std::sort(sorted.begin(), sorted.end());
+            std::vector<uint32_t> pairs;
+            for(const auto &s : sorted) { pairs.push_back(s.first); pairs.push_back(s.second); }
+            appendFile(out + "/" + p.name + ".spikes.u32", pairs.data(), pairs.size());
+        }
+        std::cout << "ref_driver: " << name << " ran " << steps << " steps" << std::endl;
+    }
+    catch(const std::exception &e) {
+        std::cerr << "ref_driver error: " << e.what() << std::endl;
+        return 1;
+    }
+    return 0;
+}
