@@ -122,11 +122,8 @@ def clipped_normal(seed, stream, count, mean, sd, lo, hi):
     bad = np.flatnonzero((out > hi) | (out < lo))
     attempt = 1
     while bad.size:
-        # counters of the retry are count*attempt + k, gathered sparsely
-        z = np.empty(bad.size)
-        for j, k in enumerate(bad):       # rare path: a handful of elements per million
-            z[j] = rng.normal(seed, stream, attempt * count + int(k), 1)[0]
-        cand = mean + sd * z
+        # retry number `attempt` of element k uses counter count*attempt + k
+        cand = mean + sd * rng.normal_at(seed, stream, np.uint64(attempt) * np.uint64(count) + bad.astype(np.uint64))
         ok = (cand <= hi) & (cand >= lo)
         out[bad[ok]] = cand[ok]
         bad = bad[~ok]
@@ -260,11 +257,12 @@ def poisson_spike_source(seed, stream, n, rate_hz, steps, dt, rates=None):
     return start, end, times
 
 
-def plastic_stdp(n=100_000, n_src=1000, steps=10000, seed=99, dt=1.0, fan=500, src_fan=100, src_w=2.0):
+def plastic_stdp(n=100_000, n_src=1000, steps=10000, seed=99, dt=1.0, fan=500, src_fan=100, src_w=2.0,
+                 ioffset=0.45, w_ei=0.25, w_ie=-1.0, w_ii=-1.0):
     n_e = (n * 4) // 5
     n_i = n - n_e
     net = Net(name="stdp", dt=dt, steps=steps, seed=seed)
-    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.45, TauRefrac=5.0)
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=ioffset, TauRefrac=5.0)
     for k, (name, num) in enumerate((("E", n_e), ("I", n_i))):
         v0 = (-60.0 + 10.0 * rng.uniform(seed, 1 + k, 0, num)).astype(np.float32)
         net.pops.append(Pop(name, "lif", num, dict(lif), {"V": v0, "RefracTime": np.zeros(num, np.float32)}))
@@ -274,13 +272,13 @@ def plastic_stdp(n=100_000, n_src=1000, steps=10000, seed=99, dt=1.0, fan=500, s
     rl, ind = fixed_probability(seed, 20, n_e, n_e, min(1.0, fan / n_e))
     mask = np.arange(ind.shape[1])[None, :] < rl[:, None]
     g = np.zeros(ind.shape, np.float32)
-    g[mask] = (0.5 * rng.uniform(seed, 21, 0, int(rl.sum()))).astype(np.float32) * np.float32(4.0 * 500.0 / max(fan, 1) / 20.0)
+    g[mask] = (0.5 * rng.uniform(seed, 21, 0, int(rl.sum()))).astype(np.float32)
     net.syns.append(Syn("EE", "E", "E", wum="stdp_trace",
                         wum_params=dict(tauPlus=20.0, tauMinus=20.0, aPlus=0.01, aMinus=0.012, wMin=0.0, wMax=1.0),
                         psm="expcurr", tau=5.0, row_stride=ind.shape[1], row_length=rl, ind=ind, g=g))
     # static projections closing the balanced loop
-    for name, src, trg, ns, nt, w, tau, st in (("EI", "E", "I", n_e, n_i, 0.05, 5.0, 22), ("IE", "I", "E", n_i, n_e, -0.25, 10.0, 23),
-                                               ("II", "I", "I", n_i, n_i, -0.25, 10.0, 24)):
+    for name, src, trg, ns, nt, w, tau, st in (("EI", "E", "I", n_e, n_i, w_ei, 5.0, 22), ("IE", "I", "E", n_i, n_e, w_ie, 10.0, 23),
+                                               ("II", "I", "I", n_i, n_i, w_ii, 10.0, 24)):
         rl, ind = fixed_probability(seed, st, ns, nt, min(1.0, fan / n_e))
         g = np.where(np.arange(ind.shape[1])[None, :] < rl[:, None], np.float32(w), np.float32(0)).astype(np.float32)
         net.syns.append(Syn(name, src, trg, wum="static", psm="expcurr", tau=tau, row_stride=ind.shape[1],

@@ -319,14 +319,16 @@ void neuronUpdateKernel(const NeuronGroupDev *groups, uint32_t numGroups, StepAr
 
     bool spiked = false;
     if(i < n) {
+        // order of operations: neuronUpdateGroupMerged.cc:552-773 — PSMs, current sources, sim code,
+        // WU pre/post dynamics, threshold, then (on a spike) WU pre/post spike code, sT, reset
+        float l0 = 0, l1 = 0;
+        uint32_t startSpike = 0;
         if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
-            uint32_t startSpike = g.startSpike[bi];
-            spiked = (startSpike != g.endSpike[bi]) && (t >= g.spikeTimes[startSpike]);
-            if(spiked) { g.startSpike[bi] = startSpike + 1; }
+            startSpike = g.startSpike[bi];
         }
         else {
             float Isyn = 0;
-            float l0 = g.var0[bi], l1 = g.var1[bi];
+            l0 = g.var0[bi]; l1 = g.var1[bi];
             for(uint32_t m = 0; m < g.numPSM; m++) {
                 const gennmi_psm_t &psm = g.psm[m];
                 float linSyn = psm.outPost[bi];
@@ -370,19 +372,22 @@ void neuronUpdateKernel(const NeuronGroupDev *groups, uint32_t numGroups, StepAr
                 l1 += g.params[0] * (g.params[1] * l0 - l1) * dt;
                 if(l0 > 30.0f) { l0 = 30.0f; }
             }
-            float preTrace = 0, postTrace = 0;
-            if(g.preTrace) { preTrace = g.preTrace[bi] * g.preDecay; }
-            if(g.postTrace) { postTrace = g.postTrace[bi] * g.postDecay; }
-            spiked = (g.model == GENNMI_NEURON_LIF) ? (l1 <= 0.0f && l0 >= g.params[4]) : (l0 >= 29.99f);
-            if(spiked) {
-                preTrace += 1.0f; postTrace += 1.0f;
-                if(g.sT) { g.sT[bi] = t; }
-                if(g.model == GENNMI_NEURON_LIF) { l0 = g.params[5]; l1 = g.params[6]; }
-            }
-            if(g.preTrace) { g.preTrace[bi] = preTrace; }
-            if(g.postTrace) { g.postTrace[bi] = postTrace; }
-            g.var0[bi] = l0; g.var1[bi] = l1;
         }
+        float preTrace = 0, postTrace = 0;
+        if(g.preTrace) { preTrace = g.preTrace[bi] * g.preDecay; }
+        if(g.postTrace) { postTrace = g.postTrace[bi] * g.postDecay; }
+        if(g.model == GENNMI_NEURON_LIF) { spiked = (l1 <= 0.0f && l0 >= g.params[4]); }
+        else if(g.model == GENNMI_NEURON_IZHIKEVICH) { spiked = (l0 >= 29.99f); }
+        else { spiked = (startSpike != g.endSpike[bi]) && (t >= g.spikeTimes[startSpike]); }
+        if(spiked) {
+            preTrace += 1.0f; postTrace += 1.0f;
+            if(g.sT) { g.sT[bi] = t; }
+            if(g.model == GENNMI_NEURON_LIF) { l0 = g.params[5]; l1 = g.params[6]; }
+            else if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) { g.startSpike[bi] = startSpike + 1; }
+        }
+        if(g.preTrace) { g.preTrace[bi] = preTrace; }
+        if(g.postTrace) { g.postTrace[bi] = postTrace; }
+        if(g.model != GENNMI_NEURON_SPIKE_SOURCE_ARRAY) { g.var0[bi] = l0; g.var1[bi] = l1; }
     }
 
     // keep the user-visible ring pointers current (nothing in the kernels reads them)

@@ -386,9 +386,9 @@ class GeNNModel:
                     owner.vars["denDelay"] = self._alloc(B * D * N, np.float32)
                     owner.vars["denDelayPtr"] = self._alloc(1, np.uint32)
             if n.pre_trace_owner is not None:
-                n.pre_trace_owner.vars["preTrace"] = self._alloc(B * N, np.float32)
+                n.pre_trace_owner.vars["preTrace"] = self._alloc(B * N, np.float32, fill=n.pre_trace_owner.wu.pre_vars.get("preTrace", 0.0))
             if n.post_trace_owner is not None:
-                n.post_trace_owner.vars["postTrace"] = self._alloc(B * N, np.float32)
+                n.post_trace_owner.vars["postTrace"] = self._alloc(B * N, np.float32, fill=n.post_trace_owner.wu.post_vars.get("postTrace", 0.0))
             for cs in n.current_sources:
                 if cs.kind == "ArrayNoise":
                     noise = np.ascontiguousarray(cs.extra_global_params["noise"], dtype=np.float32)
@@ -595,6 +595,17 @@ class GeNNModel:
     def step_time(self):
         nrec = self.num_recording_timesteps or 0
         _abi.check(_abi.load().gennmi_step_time(self._runner, self.timestep, nrec))
+        self.timestep += 1
+
+    def update_synapses(self):
+        """First half of step_time(): the runner's updateSynapses(t) on its own."""
+        _abi.check(_abi.load().gennmi_update_synapses(self._runner, C.c_float(np.float32(self.timestep) * lit32(self.dt))))
+
+    def update_neurons(self):
+        """Second half of step_time(): the runner's updateNeurons(t, recordingTimestep); advances time."""
+        nrec = self.num_recording_timesteps or 0
+        _abi.check(_abi.load().gennmi_update_neurons(self._runner, C.c_float(np.float32(self.timestep) * lit32(self.dt)),
+                                                     (self.timestep % nrec) if nrec else 0))
         self.timestep += 1
 
     def run(self, num_steps):

@@ -25,12 +25,24 @@ def _mix(z):
     return z ^ (z >> np.uint64(31))
 
 
-def words(seed, stream, start, count):
-    """``count`` 64-bit words of stream ``stream`` beginning at counter ``start``."""
+def words_at(seed, stream, ctr):
+    """64-bit words of stream ``stream`` at the counters in ``ctr`` (any uint64 array)."""
     with np.errstate(over="ignore"):
         base = np.uint64(seed) * GOLDEN + np.uint64(stream) * STREAM_MULT
-        ctr = np.arange(start, start + count, dtype=np.uint64)
-        return _mix(_mix(base + ctr) + GOLDEN)
+        return _mix(_mix(base + np.asarray(ctr, dtype=np.uint64)) + GOLDEN)
+
+
+def words(seed, stream, start, count):
+    """``count`` 64-bit words of stream ``stream`` beginning at counter ``start``."""
+    return words_at(seed, stream, np.arange(start, start + count, dtype=np.uint64))
+
+
+def normal_at(seed, stream, ctr):
+    """Standard normals at arbitrary counters; normal(seed, stream, a, n) == normal_at(seed, stream, arange(a, a+n))."""
+    ctr = np.asarray(ctr, dtype=np.uint64)
+    u1 = ((words_at(seed, stream, ctr + np.uint64(0)) >> np.uint64(40)).astype(np.float64) + 1.0) * (1.0 / 16777216.0)
+    u2 = (words_at(seed, stream + 0x40000000, ctr) >> np.uint64(40)).astype(np.float64) * (1.0 / 16777216.0)
+    return np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
 
 
 def uniform(seed, stream, start, count):
@@ -51,6 +63,4 @@ def randint(seed, stream, start, count, n):
 
 def normal(seed, stream, start, count):
     """Standard normals (Box-Muller, cosine branch) as fp64."""
-    u1 = uniform_open(seed, stream, 2 * start, count)
-    u2 = uniform(seed, stream + 0x40000000, 2 * start, count)
-    return np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
+    return normal_at(seed, stream, np.arange(start, start + count, dtype=np.uint64))

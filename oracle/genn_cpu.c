@@ -330,9 +330,14 @@ void gc_update_neurons(gc_net *net, float t, uint32_t recordingTimestep)
             int spiked;
             if(p->model == GC_SSA) {
                 uint32_t startSpike = p->startSpike[i];
+                if(p->preTrace) { p->preTrace[i] *= p->preDecay; }
+                if(p->postTrace) { p->postTrace[i] *= p->postDecay; }
                 spiked = (startSpike != p->endSpike[i] && t >= p->spikeTimes[startSpike]);
                 if(spiked) {
+                    if(p->preTrace) { p->preTrace[i] += 1.0f; }
+                    if(p->postTrace) { p->postTrace[i] += 1.0f; }
                     if(rec) { rec[i / 32] |= (1u << (i % 32)); }
+                    if(p->sT) { p->sT[i] = t; }
                     p->spk[p->spkCnt++] = i;
                     startSpike++;
                 }

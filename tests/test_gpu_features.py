@@ -1,0 +1,182 @@
+"""The reference's feature tests for the hot path (tests/features/test_event_propagation.py,
+test_recording.py), restated against the MI355X engine.  They pin the path with closed-form
+answers: binary decode of one-hot spike sources, a dendritic-delay ramp that must sum to
+exactly 10.0 at step 11, the Sobel fixtures of the Toeplitz test, and a decode through the
+column remap.  The reference reads a custom "x = Isyn" neuron; here the same quantity is read
+as outPost between updateSynapses and updateNeurons (with DeltaCurr, Isyn IS outPost)."""
+import os
+
+import numpy as np
+import pytest
+
+from genn_amd.genn_model import init_postsynaptic, init_toeplitz_connectivity, init_weight_update
+
+pytestmark = pytest.mark.gpu
+
+FIXTURES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_fixtures")
+LIF = {"C": 1.0, "TauM": 20.0, "Vrest": -60.0, "Vreset": -60.0, "Vthresh": 1e9, "Ioffset": 0.0, "TauRefrac": 5.0}
+
+
+def _silent_pop(model, name, n):
+    return model.add_neuron_population(name, n, "LIF", LIF, {"V": np.full(n, -60.0, np.float32), "RefracTime": np.zeros(n, np.float32)})
+
+
+def _decoder_lists(n_src=16, n_trg=4):
+    pre, post = [], []
+    for i in range(n_src):
+        for j in range(n_trg):
+            if ((i + 1) & (1 << j)) != 0:
+                pre.append(i)
+                post.append(j)
+    return np.asarray(pre), np.asarray(post)
+
+
+# tests/features/test_event_propagation.py:65-260
+def test_forward(make_model):
+    model = make_model("float", "test_forward", dt=1.0)
+    ss = model.add_neuron_population("SpikeSource", 16, "SpikeSourceArray", {},
+                                     {"startSpike": np.arange(16), "endSpike": np.arange(1, 17)})
+    ss.set_extra_global_param("spikeTimes", np.arange(16.0))
+    pre, post = _decoder_lists()
+    outputs = []
+    for name, hint, tps in (("Sparse", "POSTSYNAPTIC", 1), ("SparsePreSpan", "PRESYNAPTIC", 1),
+                            ("SparseHybrid", "PRESYNAPTIC", 2), ("SparseWave", "WAVE", 1)):
+        n = _silent_pop(model, "Post" + name, 4)
+        s = model.add_synapse_population(name + "Synapse", "SPARSE", ss, n,
+                                         init_weight_update("StaticPulse", {}, {"g": 1.0}), init_postsynaptic("DeltaCurr"))
+        s.set_sparse_connections(pre, post)
+        s.parallelism_hint = hint
+        s.num_threads_per_spike = tps
+        outputs.append(s)
+    model.build()
+    model.load()
+    place = 2 ** np.arange(4)
+    while model.timestep < 16:
+        model.update_synapses()
+        for s in outputs:
+            x = s.vars["outPost"].pull_from_device()
+            value = np.sum(place[np.isclose(np.ones(4), x)])
+            # spikes emitted in timestep n arrive in timestep n+1
+            expect = model.timestep if model.timestep > 0 else 0
+            assert value == expect, f"{s.name} decoding incorrect ({value} rather than {expect})"
+        model.update_neurons()
+
+
+# tests/features/test_event_propagation.py:262-329 (batch sizes 1 and 5, conftest.py:38-64)
+@pytest.mark.parametrize("batch_size", [1, 5])
+def test_forward_den_delay(make_model, batch_size):
+    model = make_model("float", "test_forward_den_delay", dt=1.0, batch_size=batch_size)
+    ss = model.add_neuron_population("SpikeSource", 10, "SpikeSourceArray", {},
+                                     {"startSpike": np.arange(10), "endSpike": np.arange(1, 11)})
+    ss.set_extra_global_param("spikeTimes", np.arange(10.0))
+    delay = np.arange(9, -1, -1)
+    outputs = []
+    for name, hint in (("Sparse", "POSTSYNAPTIC"), ("SparsePreSpan", "PRESYNAPTIC")):
+        n = _silent_pop(model, "Post" + name, 1)
+        s = model.add_synapse_population(name + "Synapse", "SPARSE", ss, n,
+                                         init_weight_update("StaticPulseDendriticDelay", {}, {"g": 1.0, "d": 0}),
+                                         init_postsynaptic("DeltaCurr"))
+        s.max_dendritic_delay_timesteps = 10
+        s.set_sparse_connections(np.arange(10), np.zeros(10, dtype=int))
+        s.set_var_coo("d", delay)
+        s.parallelism_hint = hint
+        outputs.append(s)
+    model.build()
+    model.load()
+    # Isyn of the neuron update in timestep n is outPost + the ring's front slot; the neuron kernel
+    # folds the front slot in and DeltaCurr clears it, so observe the front slot before it runs
+    while model.timestep < 11:
+        model.update_synapses()
+        ptr = (model.timestep + 1) % 10
+        correct = 10.0 if model.timestep == 10 else 0.0
+        for s in outputs:
+            ring = s.vars["denDelay"].pull_from_device().reshape(batch_size, 10, 1)
+            assert np.allclose(ring[:, ptr, 0], correct), f"{s.name} decoding incorrect ({ring[:, ptr, 0]} rather than {correct})"
+        model.update_neurons()
+        for s in outputs:
+            assert s.vars["denDelayPtr"].pull_from_device()[0] == ptr
+
+
+# tests/features/test_event_propagation.py:387-485 with the reference's own fixtures
+def test_forward_kernel(make_model):
+    vertical = np.asarray([[1.0, 0.0, -1.0], [2.0, 0.0, -2.0], [1.0, 0.0, -1.0]])
+    horizontal = np.asarray([[1.0, 2.0, 1.0], [0.0, 0.0, 0.0], [-1.0, -2.0, -1.0]])
+    model = make_model("float", "test_forward_kernel", dt=1.0)
+    pattern = np.load(os.path.join(FIXTURES, "test_pattern.npy"))
+    end = np.cumsum(np.bincount(pattern, minlength=64 * 64))
+    start = np.concatenate(([0], end[:-1]))
+    pre = model.add_neuron_population("SpikeSource", 64 * 64, "SpikeSourceArray", {}, {"startSpike": start, "endSpike": end})
+    pre.set_extra_global_param("spikeTimes", np.zeros(len(pattern)))
+    params = {"conv_kh": 3, "conv_kw": 3, "conv_ih": 64, "conv_iw": 64, "conv_ic": 1, "conv_oh": 62, "conv_ow": 62, "conv_oc": 1}
+    syn = {}
+    for name, kern in (("Horiz", horizontal), ("Vert", vertical)):
+        post = _silent_pop(model, "Post" + name, 62 * 62)
+        syn[name] = model.add_synapse_population("Toeplitz" + name, "TOEPLITZ", pre, post,
+                                                 init_weight_update("StaticPulse", {}, {"g": kern.flatten()}),
+                                                 init_postsynaptic("DeltaCurr"), init_toeplitz_connectivity("Conv2D", params))
+    model.build()
+    model.load()
+    model.step_time()
+    model.update_synapses()
+    assert np.allclose(syn["Horiz"].vars["outPost"].pull_from_device(), np.load(os.path.join(FIXTURES, "horizontal_output.npy")))
+    assert np.allclose(syn["Vert"].vars["outPost"].pull_from_device(), np.load(os.path.join(FIXTURES, "vertical_output.npy")))
+
+
+# learnPost through the column remap, as a decode in the style of test_event_propagation.py:848-955:
+# postsynaptic spike j must touch exactly the synapses {i -> j : bit i of j+1 set}
+def test_learn_post_decode(make_model):
+    model = make_model("float", "test_learn_post", dt=1.0)
+    pre_pop = _silent_pop(model, "Pre", 4)
+    post_pop = model.add_neuron_population("SpikeSource", 16, "SpikeSourceArray", {},
+                                           {"startSpike": np.arange(16), "endSpike": np.arange(1, 17)})
+    post_pop.set_extra_global_param("spikeTimes", np.arange(16.0))
+    post_inds, pre_inds = _decoder_lists()        # (source index 0..15, bit 0..3) -> post j, pre i
+    stdp = {"tauPlus": 1e30, "tauMinus": 1e30, "aPlus": 1.0, "aMinus": 0.0, "wMin": 0.0, "wMax": 100.0}
+    s = model.add_synapse_population("Plastic", "SPARSE", pre_pop, post_pop,
+                                     init_weight_update("STDPTrace", stdp, {"g": 0.0}, {"preTrace": 1.0}, {"postTrace": 0.0}),
+                                     init_postsynaptic("DeltaCurr"))
+    s.set_sparse_connections(pre_inds, post_inds)
+    model.build()
+    model.load()
+    col_length = s.vars["colLength"].pull_from_device()
+    assert np.array_equal(col_length, [bin((j + 1) & 15).count("1") for j in range(16)])
+    place = 2 ** np.arange(4)
+    seen = np.zeros((4, s.row_stride), np.float32)
+    while model.timestep < 16:
+        model.step_time()
+        g = s.vars["g"].pull_from_device().reshape(4, s.row_stride)
+        changed = (g != seen)
+        seen = g.copy()
+        rows, cols = np.nonzero(changed)
+        value = int(np.sum(place[rows]))
+        assert value == model.timestep - 1, f"learnPost decoding incorrect ({value} rather than {model.timestep - 1})"
+        if len(rows):
+            assert np.all(s.ind_host[rows, cols] == model.timestep - 2)
+            assert np.allclose(g[rows, cols], 1.0)
+
+
+# tests/features/test_recording.py:56-134 — bitfield round trip, batched, ragged population size
+@pytest.mark.parametrize("batch_size", [1, 3])
+def test_spike_recording(make_model, batch_size):
+    n = 100
+    rng = np.random.default_rng(7)
+    model = make_model("float", "test_spike_recording", dt=1.0, batch_size=batch_size)
+    spikes = [[np.sort(rng.choice(50, rng.integers(0, 6), replace=False)).astype(np.float32) for _ in range(n)] for _ in range(batch_size)]
+    times = np.concatenate([np.concatenate(b) if any(len(x) for x in b) else np.zeros(0, np.float32) for b in spikes])
+    counts = np.array([[len(x) for x in b] for b in spikes]).reshape(-1)
+    end = np.cumsum(counts).astype(np.uint32).reshape(batch_size, n)
+    start = (end.reshape(-1) - counts).astype(np.uint32).reshape(batch_size, n)
+    pop = model.add_neuron_population("SpikeSource", n, "SpikeSourceArray", {}, {"startSpike": start, "endSpike": end})
+    pop.set_extra_global_param("spikeTimes", times)
+    pop.spike_recording_enabled = True
+    model.build()
+    model.load(num_recording_timesteps=50)
+    for _ in range(50):
+        model.step_time()
+    model.pull_recording_buffers_from_device()
+    data = pop.spike_recording_data
+    for b in range(batch_size):
+        rec_t, rec_id = data[b]
+        want = sorted((float(t), i) for i in range(n) for t in spikes[b][i])
+        got = sorted(zip(rec_t.tolist(), rec_id.tolist()))
+        assert got == want

@@ -1,17 +1,179 @@
-"""GPU parity: the MI355X engine against the CPU oracle on the same seeded inputs, through the C ABI."""
+"""GPU parity: the MI355X engine against the CPU oracle on the same seeded inputs, through the C ABI.
+
+Bars: connectivity-derived arrays (colLength/remap) and per-step spike queues bit-exact; state within
+1e-5 relative — bit-exact wherever no fp32 sum can be reordered (one weight value per outPost);
+rasters identical over the first 100 ms of simulated time."""
 import numpy as np
 import pytest
 
 from genn_amd import configs
+from genn_amd.genn_model import model_from_net
+from oracle.genn_cpu import OracleNet
+from parity import compare_state, run_side_by_side
 
 pytestmark = pytest.mark.gpu
 
 
 def test_balanced_lif_bit_exact():
-    """C1 shape at full size: one constant weight per projection and one outPost per projection,
-    so atomic reordering cannot change a bit — everything must be identical."""
-    from parity import run_side_by_side
+    """C1 at full size.  One constant weight per projection and one outPost per projection: atomic
+    reordering cannot change a bit, so spike queues AND all state must be identical for the run."""
     net = configs.vogels_abbott(n=4000, steps=1000)
     model, oracle, counts = run_side_by_side(net, check_every=100, exact=True)
     assert counts["E"] > 1000 and counts["I"] > 200
+    model.unload()
+
+
+@pytest.mark.parametrize("span", ["POSTSYNAPTIC", "PRESYNAPTIC", "WAVE"])
+def test_balanced_lif_strategies(span):
+    """Row-per-spike, few-lanes-per-spike and wave-per-spike mappings give identical results."""
+    net = configs.vogels_abbott(n=1500, steps=300, p=0.05)
+    model, oracle, counts = run_side_by_side(net, check_every=50, exact=True, span=span)
+    assert counts["E"] > 100
+    model.unload()
+
+
+def test_microcircuit_dendritic_delay():
+    """C2 shape at 5 % of the neurons with full in-degree: 8 populations, all postsynaptic models of a
+    target fused into one ring buffer of 43 slots.  Weights differ, so sums may be reordered:
+    rasters must be identical for the first 100 ms (1000 steps), state within 1e-5."""
+    net = configs.potjans(neuron_scale=0.05, connectivity_scale=1.0, steps=1000)
+    model, oracle, counts = run_side_by_side(net, check_every=100, exact=False, exact_steps=1000)
+    assert sum(counts.values()) > 500
+    model.unload()
+
+
+def test_izhikevich_fanout_noise():
+    """C3 shape: Izhikevich neurons, fixed fanout with replacement (multapses), DeltaCurr input,
+    per-step noise current from a pregenerated array.  dt = 1 ms, first 100 ms = 100 steps."""
+    net = configs.izhikevich_fanout(n=20000, fanout=100, steps=200)
+    model, oracle, counts = run_side_by_side(net, check_every=20, exact=False, exact_steps=100)
+    assert counts["N"] > 1000
+    model.unload()
+
+
+def test_plastic_stdp_learn_post():
+    """C4 shape: trace STDP on E->E with learnPost through the column remap, SpikeSourceArray drive."""
+    net = configs.plastic_stdp(n=5000, n_src=100, steps=200, fan=250, src_fan=50)
+    model = model_from_net(net)
+    model.load(num_recording_timesteps=net.steps)
+    sg = model.synapse_populations["EE"]
+    oracle = OracleNet(net, col_stride={"EE": sg.col_stride})
+    # the column view must equal the CPU build bit for bit (ascending synapse index within a column)
+    col_length = sg.vars["colLength"].pull_from_device()
+    assert np.array_equal(col_length, oracle.col_length("EE"))
+    assert sg.col_stride == col_length.max()
+    remap = sg.vars["remap"].pull_from_device().reshape(-1, sg.col_stride)
+    want = oracle.remap("EE").reshape(-1, sg.col_stride)
+    mask = np.arange(sg.col_stride)[None, :] < col_length[:, None]
+    assert np.array_equal(remap[mask], want[mask])
+    spikes = 0
+    for step in range(net.steps):
+        model.step_time()
+        oracle.step()
+        for p in net.pops:
+            got = model.neuron_populations[p.name].current_spikes[0]
+            want_s = oracle.spikes(p.name)
+            if step < 100:
+                assert np.array_equal(got, want_s), f"step {step}: spike queue of {p.name} differs"
+            spikes += len(want_s)
+        if step < 100 and (step + 1) % 20 == 0:
+            compare_state(net, model, oracle, f"step {step}", exact=False)
+    assert spikes > 2000
+    model.unload()
+
+
+def test_toeplitz_conv_layer():
+    """C5 shape at 16x16x4 -> 16x16x8 (batch 1; the oracle, like the reference's CPU backend, has no batch)."""
+    net = configs.conv_toeplitz(h=16, w=16, ic=4, oc=8, steps=150, w_sd=0.5)
+    net.pop("Out").params["Ioffset"] = 0.4
+    model, oracle, counts = run_side_by_side(net, check_every=25, exact=False, exact_steps=100)
+    assert counts["Out"] > 100 and counts["In"] > 1000
+    model.unload()
+
+
+def test_toeplitz_batches_are_independent():
+    """Batch b of a batched run equals a batch-1 run of the oracle fed batch b's spike trains."""
+    B = 3
+    nets = [configs.conv_toeplitz(h=8, w=8, ic=2, oc=4, steps=60, w_sd=0.6, batch_index=b) for b in range(B)]
+    for net in nets:
+        net.pop("Out").params["Ioffset"] = 0.4
+    base = nets[0]
+    # spikeTimes is shared by all batches; startSpike / endSpike select each batch's slice (test_recording.py:56-103)
+    times = np.concatenate([n.pop("In").spike_times for n in nets])
+    offs = np.cumsum([0] + [len(n.pop("In").spike_times) for n in nets])
+    start = np.stack([n.pop("In").vars["startSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32)
+    end = np.stack([n.pop("In").vars["endSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32)
+    import copy
+    batched = copy.deepcopy(base)
+    batched.pop("In").vars = {"startSpike": start, "endSpike": end}
+    batched.pop("In").spike_times = times
+    model = model_from_net(batched, batch_size=B)
+    model.load(num_recording_timesteps=base.steps)
+    oracles = [OracleNet(n) for n in nets]
+    total = 0
+    for step in range(base.steps):
+        model.step_time()
+        got = {name: model.neuron_populations[name].current_spikes for name in ("In", "Out")}
+        for b, o in enumerate(oracles):
+            o.step()
+            for name in ("In", "Out"):
+                assert np.array_equal(got[name][b], o.spikes(name)), f"step {step} batch {b}: {name} spikes differ"
+                total += len(o.spikes(name))
+    assert total > 500
+    v = model.neuron_populations["Out"].vars["V"].pull_from_device().reshape(B, -1)
+    for b, o in enumerate(oracles):
+        np.testing.assert_allclose(v[b], o.var("Out", 0), rtol=1e-5)
+    model.unload()
+
+
+def test_graph_replay_matches_stepping():
+    """run() replays captured HIP graphs; every replay must leave the state eager stepping leaves.
+    Replays are interleaved with eager steps and synchronisations."""
+    net = configs.vogels_abbott(n=2000, steps=730, p=0.04)
+    eager = model_from_net(net)
+    eager.load(num_recording_timesteps=net.steps)
+    graph = model_from_net(net)
+    graph.load(num_recording_timesteps=net.steps)
+    for chunk in (250, 3, 200, 77, 200):           # 200/250 -> graph replays (+ remainder), 3/77 -> single steps
+        graph.run(chunk)
+        graph.synchronize()
+        for _ in range(chunk):
+            eager.step_time()
+        eager.synchronize()
+        for name in ("E", "I"):
+            for var in ("V", "RefracTime"):
+                assert np.array_equal(graph.neuron_populations[name].vars[var].pull_from_device(),
+                                      eager.neuron_populations[name].vars[var].pull_from_device()), f"{name}.{var} after {graph.timestep} steps"
+            assert np.array_equal(graph.neuron_populations[name].current_spikes[0], eager.neuron_populations[name].current_spikes[0])
+    assert graph.timestep == eager.timestep == 730
+    graph.pull_recording_buffers_from_device()
+    eager.pull_recording_buffers_from_device()
+    for name in ("E", "I"):
+        assert np.array_equal(graph.neuron_populations[name].vars["recordSpk"].view, eager.neuron_populations[name].vars["recordSpk"].view)
+    t, ids = graph.neuron_populations["E"].spike_recording_data[0]
+    assert len(ids) > 500
+    assert graph.synaptic_event_count == eager.synaptic_event_count
+    graph.unload()
+    eager.unload()
+
+
+@pytest.mark.parametrize("n", [1, 31, 64, 65, 257, 1000])
+def test_ragged_population_sizes(n):
+    """Population sizes around the wave (64), recording-word (32) and work-group (256) boundaries;
+    includes empty rows and a population in which every neuron fires in the same step."""
+    from genn_amd.netspec import Net, Pop, Syn
+    from genn_amd import rng
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=1.0, TauRefrac=2.0)
+    net = Net(name="ragged", dt=1.0, steps=60)
+    v0 = np.full(n, -50.5, np.float32)             # everyone crosses threshold in step 0
+    net.pops.append(Pop("A", "lif", n, dict(lif), {"V": v0, "RefracTime": np.zeros(n, np.float32)}))
+    m = max(1, n // 2)
+    net.pops.append(Pop("B", "lif", m, dict(lif, Ioffset=0.2), {"V": np.full(m, -60.0, np.float32), "RefracTime": np.zeros(m, np.float32)}))
+    stride = 5
+    row_length = (rng.randint(3, 1, 0, n, stride + 1)).astype(np.uint32)      # 0..5, some rows empty
+    ind = np.sort(rng.randint(3, 2, 0, n * stride, m).reshape(n, stride), axis=1).astype(np.uint32)
+    g = np.full((n, stride), 1.5, np.float32)
+    net.syns.append(Syn("AB", "A", "B", wum="static", psm="expcurr", tau=5.0, row_stride=stride, row_length=row_length, ind=ind, g=g))
+    model, oracle, counts = run_side_by_side(net, check_every=10, exact=True)
+    assert counts["A"] >= n
     model.unload()
