@@ -1,0 +1,159 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-timestep hot path on one MI355X.
+
+Workload (default): the full-scale cortical microcircuit — 77,169 LIF neurons in 8 populations,
+298,624,465 synapses in 54 SPARSE projections with fp32 weights and uint8 dendritic delays into a
+43-slot ring, DC background, dt = 0.1 ms.  A "step" is one simulation timestep
+(updateSynapses + updateNeurons).  Inputs are synthetic (repo-owned seeded generator) and already
+resident in HBM when the timed region starts.
+
+Prints ONE JSON line: whole-job synaptic events per second, plus
+  roofline      the presynaptic-update kernel against the HBM roofline (algorithmic bytes per event
+                x events per launch / average launch duration from HIP events on the kernel's stream)
+  cpu_baseline  the single-threaded CPU oracle timed on this host on a bounded sample of the same network
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+# algorithmic bytes per synaptic event: ind 4 + g 4 + fp32 read-modify-write of the target 8 (+ 1 delay byte)
+BYTES_PER_EVENT = {"static": 16, "static_delay": 17, "stdp_trace": 28, "conv2d": 8}
+
+
+def build_net(name, steps):
+    from genn_amd import configs
+    if name == "potjans":
+        return configs.potjans(steps=steps), "C2 potjans_microcircuit 77169 neurons 298.6M synapses dt=0.1ms"
+    if name == "potjans_small":
+        return configs.potjans(neuron_scale=0.1, connectivity_scale=1.0, steps=steps), "potjans 10% neurons full in-degree"
+    if name == "va":
+        return configs.vogels_abbott(steps=steps), "C1 balanced LIF 4000 neurons p=0.02 dt=0.1ms"
+    if name == "izh":
+        return configs.izhikevich_fanout(steps=steps, noise_steps=64), "C3 izhikevich 1e6 neurons fanout 1000 dt=1ms (noise rows cycled)"
+    if name == "izh_small":
+        return configs.izhikevich_fanout(n=100_000, fanout=1000, steps=steps, noise_steps=64), "izhikevich 1e5 neurons fanout 1000"
+    if name == "stdp":
+        return configs.plastic_stdp(steps=steps), "C4 plastic STDP 100k neurons fanout 500 dt=1ms"
+    raise SystemExit(f"unknown workload {name}")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10000)
+    ap.add_argument("--warmup", type=int, default=2000)
+    ap.add_argument("--workload", default="potjans")
+    ap.add_argument("--cpu-steps", type=int, default=None, help="steps of the CPU baseline sample (default: sized for ~10-20 s)")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--profile-steps", type=int, default=2000, help="eager steps with HIP events around every kernel")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
+                         "(the hot path is single-GPU; see DESIGN.md for how it would shard)")
+
+    import numpy as np
+    from genn_amd.genn_model import model_from_net
+
+    total_steps = args.warmup + args.steps + args.profile_steps
+    t0 = time.time()
+    net, label = build_net(args.workload, total_steps)
+    gen_s = time.time() - t0
+    num_neurons = sum(p.n for p in net.pops)
+    num_synapses = sum(s.num_synapses for s in net.syns)
+    kinds = {("conv2d" if s.matrix == "conv2d" else s.wum) for s in net.syns}
+    bytes_per_event = max(BYTES_PER_EVENT[k] for k in kinds) if len(kinds) == 1 else None
+
+    t0 = time.time()
+    model = model_from_net(net, record=True)
+    model.load(num_recording_timesteps=args.warmup + args.steps)
+    model.synchronize()
+    load_s = time.time() - t0
+
+    # ---- warm-up (also captures the step graph), then the timed region
+    model.run(args.warmup)
+    model.synchronize()
+    ev0 = model.synaptic_event_count
+    t0 = time.perf_counter()
+    model.run(args.steps)
+    model.synchronize()
+    wall = time.perf_counter() - t0
+    events = model.synaptic_event_count - ev0
+
+    model.pull_recording_buffers_from_device()
+    rates = {}
+    for p in net.pops:
+        _, ids = model.neuron_populations[p.name].spike_recording_data[0]
+        rates[p.name] = round(len(ids) / p.n / ((args.warmup + args.steps) * net.dt / 1000.0), 3)
+
+    # ---- per-kernel durations: eager stepping with HIP events around each launch on the runner's stream
+    roofline = None
+    if args.profile_steps > 0:
+        model.num_recording_timesteps = None
+        model.set_timing(True)
+        evp0 = model.synaptic_event_count
+        for _ in range(args.profile_steps):
+            model.step_time()
+        model.synchronize()
+        st = model.kernel_stats()
+        evp = model.synaptic_event_count - evp0
+        model.set_timing(False)
+        if st["presyn_launches"]:
+            avg_s = st["presyn_seconds"] / st["presyn_launches"]
+            ev_per_launch = evp / st["presyn_launches"]
+            bpe = bytes_per_event or max(BYTES_PER_EVENT[k] for k in kinds)
+            achieved = ev_per_launch * bpe / avg_s / 1e9
+            roofline = {"bound": "hbm", "kernel": "presynapticUpdateKernel", "achieved": round(achieved, 3), "peak": HBM_PEAK_GBS,
+                        "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6), "traffic": None,
+                        "bytes_per_event": bpe, "events_per_launch": round(ev_per_launch, 1), "avg_launch_us": round(avg_s * 1e6, 3),
+                        "neuron_kernel_avg_us": round(st["neuron_seconds"] / max(1, st["neuron_launches"]) * 1e6, 3),
+                        "neuron_kernel_gbs": round(num_neurons * 32 / (st["neuron_seconds"] / max(1, st["neuron_launches"])) / 1e9, 3)}
+    model.unload()
+
+    # ---- CPU baseline: the single-threaded oracle on the same network, bounded sample from t = 0
+    cpu = None
+    if not args.no_cpu:
+        from oracle.genn_cpu import OracleNet
+        oracle = OracleNet(net)
+        probe = 20
+        t0 = time.perf_counter()
+        oracle.run(probe)
+        per_step = (time.perf_counter() - t0) / probe
+        cpu_steps = args.cpu_steps or int(max(100, min(args.warmup + args.steps, 15.0 / max(per_step, 1e-6))))
+        ev_before = oracle.events()
+        t0 = time.perf_counter()
+        oracle.run(cpu_steps)
+        cpu_wall = time.perf_counter() - t0
+        cpu_events = oracle.events() - ev_before
+        cpu = {"value": round(cpu_events / cpu_wall, 1), "unit": "events/s", "cores": 1, "kind": "port",
+               "sample": f"steps {probe}..{probe + cpu_steps} of the same network from t=0 ({cpu_events} events in {cpu_wall:.2f} s)",
+               "wall_s_per_sim_s": round(cpu_wall / (cpu_steps * net.dt / 1000.0), 3),
+               "host_cores": os.cpu_count()}
+        oracle.close()
+
+    sim_s = args.steps * net.dt / 1000.0
+    out = {
+        "metric": "synaptic_events_per_s", "value": round(events / wall, 1), "unit": "events/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall / args.steps * 1e3, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": label, "neurons": num_neurons, "synapses": num_synapses, "dt_ms": net.dt, "seed": net.seed,
+                   "stepping": "hipGraph replay, 100 steps per graph"},
+        "gsop_per_s": round(events / wall / 1e9, 4),
+        "neuron_updates_per_s": round(num_neurons * args.steps / wall, 1),
+        "wall_s_per_sim_s": round(wall / sim_s, 4),
+        "events_per_step": round(events / args.steps, 1),
+        "algorithmic_gb_per_s_wallclock": round(events * (bytes_per_event or 16) / wall / 1e9, 3),
+        "firing_rates_hz": rates,
+        "setup_s": {"generate": round(gen_s, 1), "load": round(load_s, 1)},
+        "roofline": roofline, "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

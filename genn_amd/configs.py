@@ -1,102 +1,27 @@
 """Synthetic-input generators for the benchmark configurations (and reduced-scale twins).
 
-Every array comes from :mod:`genn_amd.rng`; a (config, scale, seed) triple therefore names
-one exact network.  Rows are sorted by postsynaptic index, as the reference's built-in
-connectivity snippets and ``set_sparse_connections`` produce them
-(pygenn/genn_groups.py:447-460).
+Every array comes from the repo's counter-based generator (:mod:`genn_amd.rng` for small
+arrays, :mod:`genn_amd.netgen` — the same streams, multi-threaded C — for per-synapse ones); a
+(config, scale, seed) triple therefore names one exact network.  Rows are sorted by
+postsynaptic index, as the reference's built-in connectivity snippets and
+``set_sparse_connections`` produce them (pygenn/genn_groups.py:447-460).
 """
 import math
 
 import numpy as np
 
-from . import rng
+from . import netgen, rng
 from .netspec import Net, Pop, CurrentSource, Syn
 
 
-# --------------------------------------------------------------------------------------------
-# connectivity builders (all return rowLength[numPre], ind[numPre,stride])
-# --------------------------------------------------------------------------------------------
-def fixed_probability(seed, stream, n_pre, n_post, p, pad=1):
-    """Bernoulli(p) per (pre,post) pair via geometric skips — the process of
-    include/genn/genn/initSparseConnectivitySnippet.h:170-187, driven by the repo's own
-    generator.  Row r uses counters [r*K, (r+1)*K) of ``stream``."""
-    mean = n_post * p
-    K = int(mean + 8.0 * math.sqrt(mean * (1 - p)) + 16)
-    logq = math.log1p(-p)
-    row_length = np.zeros(n_pre, dtype=np.uint32)
-    rows = []
-    chunk = max(1, (1 << 22) // K)
-    for r0 in range(0, n_pre, chunk):
-        r1 = min(n_pre, r0 + chunk)
-        u = rng.uniform_open(seed, stream, r0 * K, (r1 - r0) * K).reshape(r1 - r0, K)
-        skips = np.floor(np.log(u) / logq).astype(np.int64) + 1
-        pos = np.cumsum(skips, axis=1) - 1
-        valid = pos < n_post
-        if valid[:, -1].any():
-            raise RuntimeError("fixed_probability: candidate budget too small")
-        row_length[r0:r1] = valid.sum(axis=1)
-        rows.append((pos, valid))
-    stride = int(max(1, row_length.max()))
-    stride = ((stride + pad - 1) // pad) * pad
-    ind = np.zeros((n_pre, stride), dtype=np.uint32)
-    r0 = 0
-    for pos, valid in rows:
-        n = pos.shape[0]
-        w = min(stride, pos.shape[1])
-        ind[r0:r0 + n, :w] = np.where(valid[:, :w], pos[:, :w], 0)
-        r0 += n
-    return row_length, ind
-
-
-def fixed_number_post(seed, stream, n_pre, n_post, fanout):
-    """Every row draws ``fanout`` targets uniformly with replacement, then sorts them
-    (shape of FixedNumberPostWithReplacement, initSparseConnectivitySnippet.h:242-276)."""
-    ind = np.empty((n_pre, fanout), dtype=np.uint32)
-    chunk = max(1, (1 << 24) // fanout)
-    for r0 in range(0, n_pre, chunk):
-        r1 = min(n_pre, r0 + chunk)
-        x = rng.randint(seed, stream, r0 * fanout, (r1 - r0) * fanout, n_post).reshape(r1 - r0, fanout)
-        x.sort(axis=1)
-        ind[r0:r1] = x
-    return np.full(n_pre, fanout, dtype=np.uint32), ind
-
-
-def fixed_number_total(seed, stream, n_pre, n_post, total, pad=1):
-    """``total`` (pre,post) pairs uniformly with replacement (multapses allowed), sorted
-    (shape of FixedNumberTotalWithReplacement, initSparseConnectivitySnippet.h:292-370)."""
-    keys = np.empty(total, dtype=np.uint64)
-    chunk = 1 << 24
-    for c0 in range(0, total, chunk):
-        c = min(chunk, total - c0)
-        pre = rng.randint(seed, stream, c0, c, n_pre).astype(np.uint64)
-        post = rng.randint(seed, stream + 0x20000000, c0, c, n_post).astype(np.uint64)
-        keys[c0:c0 + c] = pre * np.uint64(n_post) + post
-    keys.sort()
-    pre = (keys // np.uint64(n_post)).astype(np.int64)
-    post = (keys % np.uint64(n_post)).astype(np.uint32)
-    row_length = np.bincount(pre, minlength=n_pre).astype(np.uint32)
-    stride = int(max(1, row_length.max()))
-    stride = ((stride + pad - 1) // pad) * pad
-    starts = np.concatenate(([0], np.cumsum(row_length)[:-1])).astype(np.int64)
-    within = np.arange(total, dtype=np.int64) - starts[pre]
-    ind = np.zeros((n_pre, stride), dtype=np.uint32)
-    ind[pre, within] = post
-    return row_length, ind, (pre, within)
-
-
-def _fill_rows(row_length, stride, values):
-    """Scatter a flat per-synapse array (row-major over valid entries) into padded layout."""
-    n_pre = len(row_length)
-    out = np.zeros((n_pre, stride), dtype=values.dtype)
-    mask = np.arange(stride)[None, :] < row_length[:, None]
-    out[mask] = values
-    return out
+def _const_rows(row_length, stride, value):
+    return np.where(np.arange(stride)[None, :] < row_length[:, None], np.float32(value), np.float32(0)).astype(np.float32)
 
 
 # --------------------------------------------------------------------------------------------
 # C1: balanced LIF network (Vogels-Abbott shape)
 # --------------------------------------------------------------------------------------------
-def vogels_abbott(n=4000, steps=10000, seed=1234, p=0.02, dt=0.1, ioffset=0.55):
+def vogels_abbott(n=4000, steps=10000, seed=1234, p=0.02, dt=0.1, ioffset=0.55, pad=1):
     n_e = (n * 4) // 5
     n_i = n - n_e
     lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=ioffset, TauRefrac=5.0)
@@ -107,28 +32,11 @@ def vogels_abbott(n=4000, steps=10000, seed=1234, p=0.02, dt=0.1, ioffset=0.55):
     stream = 16
     for src, n_src, w, tau in (("E", n_e, 0.5, 5.0), ("I", n_i, -2.25, 10.0)):
         for trg, n_trg in (("E", n_e), ("I", n_i)):
-            rl, ind = fixed_probability(seed, stream, n_src, n_trg, p)
+            rl, ind = netgen.fixed_probability(seed, stream, n_src, n_trg, p, pad=pad)
             stream += 1
-            g = np.where(np.arange(ind.shape[1])[None, :] < rl[:, None], np.float32(w), np.float32(0)).astype(np.float32)
             net.syns.append(Syn(f"{src}{trg}", src, trg, wum="static", psm="expcurr", tau=tau,
-                                row_stride=ind.shape[1], row_length=rl, ind=ind, g=g))
+                                row_stride=ind.shape[1], row_length=rl, ind=ind, g=_const_rows(rl, ind.shape[1], w)))
     return net
-
-
-def clipped_normal(seed, stream, count, mean, sd, lo, hi):
-    """Normal(mean, sd) resampled until inside [lo, hi] (the rule of NormalClipped,
-    include/genn/genn/initVarSnippet.h:161-176).  Element k tries counters k, k+count, ..."""
-    out = mean + sd * rng.normal(seed, stream, 0, count)
-    bad = np.flatnonzero((out > hi) | (out < lo))
-    attempt = 1
-    while bad.size:
-        # retry number `attempt` of element k uses counter count*attempt + k
-        cand = mean + sd * rng.normal_at(seed, stream, np.uint64(attempt) * np.uint64(count) + bad.astype(np.uint64))
-        ok = (cand <= hi) & (cand >= lo)
-        out[bad[ok]] = cand[ok]
-        bad = bad[~ok]
-        attempt += 1
-    return out
 
 
 # --------------------------------------------------------------------------------------------
@@ -169,9 +77,11 @@ def pd_mean_weight(src, trg):
     return PD_G * PD_MEAN_W
 
 
-def potjans(neuron_scale=1.0, connectivity_scale=1.0, steps=10000, seed=4321, dt=0.1, pad=1):
-    """Background Poisson input (PoissonExp, currentSourceModels.h:107-129) is replaced by a DC
-    source with the same stationary mean, w * tauSyn * rate[1/ms]."""
+def potjans(neuron_scale=1.0, connectivity_scale=1.0, steps=10000, seed=4321, dt=0.1, pad=4):
+    """Scaling rules are those of the reference script (userproject/potjans_microcircuit.py:105-147,
+    193-200).  The Poisson background (PoissonExp, currentSourceModels.h:107-129) is replaced by a
+    DC source with the same stationary mean, w * tauSyn * rate[1/ms].  Rows are padded to
+    ``pad`` entries so that row starts are 16-byte aligned."""
     pops = [l + p for l in PD_LAYERS for p in ("E", "I")]
     max_delay = {k: PD_MEAN_DELAY[k] + PD_DELAY_SD[k] * PD_NORM_Q9999 for k in ("E", "I")}
     slots = int(round(max(max_delay.values()) / dt))
@@ -191,52 +101,45 @@ def potjans(neuron_scale=1.0, connectivity_scale=1.0, steps=10000, seed=4321, dt
         ext_w = PD_MEAN_W / math.sqrt(connectivity_scale)
         net.css.append(CurrentSource(name + "_dc", "dc", name, amp=ext_w * 0.5 * ext_rate / 1000.0))
     stream = 100
+    fmax = float(np.finfo(np.float32).max)
     for trg in pops:
         for src in pops:
-            stream += 4
+            stream += 8
             num_in = pd_full_num_inputs(src, trg) * connectivity_scale
             total = int(round(num_in * float(size[trg])))
             if total <= 0:
                 continue
             mean_w = pd_mean_weight(src, trg) / math.sqrt(connectivity_scale)
             sd_w = mean_w * 0.05 if (src == "4E" and trg == "23E") else abs(mean_w * 0.1)
-            rl, ind, (pre, within) = fixed_number_total(seed, stream, size[src], size[trg], total, pad=pad)
+            rl, ind = netgen.fixed_number_total(seed, stream, size[src], size[trg], total, pad=pad)
+            stride = ind.shape[1]
             kind = src[-1]
-            fmax = float(np.finfo(np.float32).max)
             lo, hi = (0.0, fmax) if kind == "E" else (-fmax, 0.0)
-            gv = clipped_normal(seed, stream + 1, total, mean_w, sd_w, lo, hi).astype(np.float32)
-            dv = np.rint(clipped_normal(seed, stream + 2, total, PD_MEAN_DELAY[kind] / dt, PD_DELAY_SD[kind] / dt,
-                                        0.0, max_delay[kind] / dt).astype(np.float32)).astype(np.uint8)
-            g = np.zeros(ind.shape, np.float32)
-            d = np.zeros(ind.shape, np.uint8)
-            g[pre, within] = gv
-            d[pre, within] = dv
+            g = netgen.rows_clipped_normal(seed, stream + 2, rl, stride, mean_w, sd_w, lo, hi)
+            d = netgen.rows_clipped_normal_delay(seed, stream + 4, rl, stride, PD_MEAN_DELAY[kind] / dt, PD_DELAY_SD[kind] / dt,
+                                                 0.0, max_delay[kind] / dt)
             net.syns.append(Syn(f"{src}_{trg}", src, trg, wum="static_delay", psm="expcurr", tau=0.5,
-                                row_stride=ind.shape[1], row_length=rl, ind=ind, g=g, d=d, max_den_delay=slots))
+                                row_stride=stride, row_length=rl, ind=ind, g=g, d=d, max_den_delay=slots))
     return net
 
 
 # --------------------------------------------------------------------------------------------
 # C3: fixed-fanout Izhikevich network with pregenerated noise current
 # --------------------------------------------------------------------------------------------
-def izhikevich_fanout(n=1_000_000, fanout=1000, steps=1000, seed=777, dt=1.0, with_noise=True):
+def izhikevich_fanout(n=1_000_000, fanout=1000, steps=1000, seed=777, dt=1.0, noise_steps=None):
+    """Regular-spiking Izhikevich neurons, 80/20 excitatory/inhibitory by row, DeltaCurr input.
+    ``noise_steps`` rows of U[0,5) noise are generated and cycled (default: one row per step)."""
     n_e = (n * 4) // 5
     net = Net(name="izh", dt=dt, steps=steps, seed=seed)
     v0 = np.full(n, -65.0, np.float32)
-    u0 = (0.2 * v0).astype(np.float32)
+    u0 = (np.float32(0.2) * v0).astype(np.float32)
     net.pops.append(Pop("N", "izh", n, dict(a=0.02, b=0.2, c=-65.0, d=8.0), {"V": v0, "U": u0}))
-    rl, ind = fixed_number_post(seed, 10, n, n, fanout)
-    g = np.empty((n, fanout), np.float32)
-    chunk = max(1, (1 << 24) // fanout)
-    for r0 in range(0, n, chunk):
-        r1 = min(n, r0 + chunk)
-        u = rng.uniform(seed, 11, r0 * fanout, (r1 - r0) * fanout).reshape(r1 - r0, fanout)
-        rows = np.arange(r0, r1)[:, None]
-        g[r0:r1] = np.where(rows < n_e, 0.5 * u, u - 1.0).astype(np.float32)
+    rl, ind = netgen.fixed_number_post(seed, 10, n, n, fanout)
+    g = netgen.rows_uniform(seed, 11, rl, fanout, n_e, 0.5, 0.0, 1.0, -1.0)
     net.syns.append(Syn("NN", "N", "N", wum="static", psm="deltacurr", row_stride=fanout, row_length=rl, ind=ind, g=g))
-    if with_noise:
-        noise = (5.0 * rng.uniform(seed, 12, 0, steps * n)).astype(np.float32).reshape(steps, n)
-        net.css.append(CurrentSource("N_noise", "noise", "N", noise=noise))
+    rows = steps if noise_steps is None else noise_steps
+    noise = netgen.uniform_f32(seed, 12, 0, rows * n, 5.0, 0.0).reshape(rows, n)
+    net.css.append(CurrentSource("N_noise", "noise", "N", noise=noise))
     return net
 
 
@@ -247,18 +150,20 @@ def poisson_spike_source(seed, stream, n, rate_hz, steps, dt, rates=None):
     """Pregenerated Poisson spike times (ms, on the dt grid) in SpikeSourceArray layout
     (startSpike/endSpike/spikeTimes, include/genn/genn/neuronModels.h:274-286)."""
     p = (np.full(n, rate_hz) if rates is None else np.asarray(rates)) * dt / 1000.0
-    u = rng.uniform(seed, stream, 0, n * steps).reshape(n, steps)
-    fire = u < p[:, None]
+    u = netgen.uniform_f32(seed, stream, 0, n * steps).reshape(n, steps)
+    fire = u < p[:, None].astype(np.float32)
     counts = fire.sum(axis=1)
     end = np.cumsum(counts).astype(np.uint32)
     start = (end - counts).astype(np.uint32)
-    src, step = np.nonzero(fire)
+    _, step = np.nonzero(fire)
     times = (step.astype(np.float64) * dt).astype(np.float32)
     return start, end, times
 
 
 def plastic_stdp(n=100_000, n_src=1000, steps=10000, seed=99, dt=1.0, fan=500, src_fan=100, src_w=2.0,
                  ioffset=0.45, w_ei=0.25, w_ie=-1.0, w_ii=-1.0):
+    """80 % excitatory neurons with plastic E->E (fanout ~``fan``, g0 ~ U[0,0.5], clipped to [0,1]); the
+    static E->I, I->E, I->I projections close a balanced loop; Poisson sources drive E."""
     n_e = (n * 4) // 5
     n_i = n - n_e
     net = Net(name="stdp", dt=dt, steps=steps, seed=seed)
@@ -268,38 +173,36 @@ def plastic_stdp(n=100_000, n_src=1000, steps=10000, seed=99, dt=1.0, fan=500, s
         net.pops.append(Pop(name, "lif", num, dict(lif), {"V": v0, "RefracTime": np.zeros(num, np.float32)}))
     start, end, times = poisson_spike_source(seed, 5, n_src, 10.0, steps, dt)
     net.pops.append(Pop("P", "ssa", n_src, {}, {"startSpike": start, "endSpike": end}, spike_times=times))
-    # plastic E->E
-    rl, ind = fixed_probability(seed, 20, n_e, n_e, min(1.0, fan / n_e))
-    mask = np.arange(ind.shape[1])[None, :] < rl[:, None]
-    g = np.zeros(ind.shape, np.float32)
-    g[mask] = (0.5 * rng.uniform(seed, 21, 0, int(rl.sum()))).astype(np.float32)
+    p_conn = min(1.0, fan / n_e)
+    rl, ind = netgen.fixed_probability(seed, 20, n_e, n_e, p_conn)
+    g = netgen.rows_uniform(seed, 21, rl, ind.shape[1], n_e, 0.5, 0.0, 0.5, 0.0)
     net.syns.append(Syn("EE", "E", "E", wum="stdp_trace",
                         wum_params=dict(tauPlus=20.0, tauMinus=20.0, aPlus=0.01, aMinus=0.012, wMin=0.0, wMax=1.0),
                         psm="expcurr", tau=5.0, row_stride=ind.shape[1], row_length=rl, ind=ind, g=g))
-    # static projections closing the balanced loop
     for name, src, trg, ns, nt, w, tau, st in (("EI", "E", "I", n_e, n_i, w_ei, 5.0, 22), ("IE", "I", "E", n_i, n_e, w_ie, 10.0, 23),
                                                ("II", "I", "I", n_i, n_i, w_ii, 10.0, 24)):
-        rl, ind = fixed_probability(seed, st, ns, nt, min(1.0, fan / n_e))
-        g = np.where(np.arange(ind.shape[1])[None, :] < rl[:, None], np.float32(w), np.float32(0)).astype(np.float32)
+        rl, ind = netgen.fixed_probability(seed, st, ns, nt, p_conn)
         net.syns.append(Syn(name, src, trg, wum="static", psm="expcurr", tau=tau, row_stride=ind.shape[1],
-                            row_length=rl, ind=ind, g=g))
-    rl, ind = fixed_number_post(seed, 25, n_src, n_e, min(src_fan, n_e))
-    g = np.full(ind.shape, np.float32(src_w), np.float32)
+                            row_length=rl, ind=ind, g=_const_rows(rl, ind.shape[1], w)))
+    rl, ind = netgen.fixed_number_post(seed, 25, n_src, n_e, min(src_fan, n_e))
     net.syns.append(Syn("PE", "P", "E", wum="static", psm="expcurr", tau=5.0, row_stride=ind.shape[1],
-                        row_length=rl, ind=ind, g=g))
+                        row_length=rl, ind=ind, g=np.full(ind.shape, np.float32(src_w), np.float32)))
     return net
 
 
 # --------------------------------------------------------------------------------------------
 # C5: convolutional spiking layer through TOEPLITZ connectivity
 # --------------------------------------------------------------------------------------------
-def conv_toeplitz(h=64, w=64, ic=16, oc=32, k=3, steps=500, seed=5, dt=1.0, batch_index=0, max_rate=50.0, w_sd=0.1):
+def conv_toeplitz(h=64, w=64, ic=16, oc=32, k=3, steps=500, seed=5, dt=1.0, batch_index=0, max_rate=50.0, w_sd=0.1,
+                  ioffset=0.0):
+    """Rate-coded Poisson sources (rates U[0,max_rate) Hz, one spike train per batch index) into a LIF
+    layer through Conv2D k x k, stride 1, same padding; kernel weights N(0, w_sd)."""
     n_in, n_out = h * w * ic, h * w * oc
     net = Net(name="conv", dt=dt, steps=steps, seed=seed)
     rates = max_rate * rng.uniform(seed, 1, 0, n_in)
     start, end, times = poisson_spike_source(seed, 100 + batch_index, n_in, 0.0, steps, dt, rates=rates)
     net.pops.append(Pop("In", "ssa", n_in, {}, {"startSpike": start, "endSpike": end}, spike_times=times))
-    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.0, TauRefrac=5.0)
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=ioffset, TauRefrac=5.0)
     net.pops.append(Pop("Out", "lif", n_out, lif, {"V": np.full(n_out, -60.0, np.float32), "RefracTime": np.zeros(n_out, np.float32)}))
     kern = (w_sd * rng.normal(seed, 2, 0, k * k * ic * oc)).astype(np.float32).reshape(k, k, ic, oc)
     net.syns.append(Syn("Conv", "In", "Out", matrix="conv2d", wum="static", psm="expcurr", tau=5.0, g=kern,

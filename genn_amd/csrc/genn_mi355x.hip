@@ -19,8 +19,10 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "genn_mi355x.h"
@@ -108,38 +110,40 @@ struct PostGroupDev
     uint32_t lanesPerSpike;
 };
 
-// Block -> group: groups occupy consecutive block ranges (the reference pads thread ranges to
-// block multiples for the same reason, backendSIMT.h:244-323).  Table sizes are tens of entries.
-template<typename G>
-__device__ __forceinline__ uint32_t findGroup(const G *groups, uint32_t numGroups, uint32_t block)
-{
-    uint32_t lo = 0, hi = numGroups;
-    while(hi - lo > 1) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if(groups[mid].startBlock <= block) { lo = mid; } else { hi = mid; }
-    }
-    return lo;
-}
+// Block -> group: groups occupy consecutive block ranges (the reference pads thread ranges to block
+// multiples for the same reason, backendSIMT.h:244-323).  Every block has its own copy of its group's
+// descriptor in a table indexed by blockIdx.x.
 
-__device__ __forceinline__ void atomicAddF32(float *addr, float v)
+// Pointers reach the kernels through descriptor tables, so the compiler cannot know their address
+// space; these casts let it emit global_load / global_atomic instead of flat instructions.
+#define GLOBAL_AS __attribute__((address_space(1)))
+template<typename T>
+__device__ __forceinline__ GLOBAL_AS T *asGlobal(T *p) { return (GLOBAL_AS T*)p; }
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint8_t u8x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void atomicAddF32(GLOBAL_AS float *addr, float v)
 {
-    // gfx950 has a native global_atomic_add_f32; no return value is needed
-    unsafeAtomicAdd(addr, v);
+    // gfx950 has a native global_atomic_add_f32; the old value is not needed
+    __builtin_amdgcn_global_atomic_fadd_f32(addr, v);
 }
 
 // ------------------------------------------------------------------------------------------------
-// Presynaptic update.  One sub-group of `lanesPerSpike` lanes walks one spike's row; sub-groups
-// take spikes round-robin.  lanesPerSpike = 64 is the "post span" mapping (lanes span the row, so
-// ind/g are read as whole 256-byte lines); small values are the "pre span" mapping (few lanes per
-// spike, many spikes per wave).  Spike list, rowLength and row base are read once per spike.
+// Presynaptic update.  The unit of work is (spike, chunk of its row): a sub-group of
+// `lanesPerSpike` lanes handles `span` consecutive synapses of one row, so a long row is spread
+// over many wavefronts instead of being walked serially, and every load of ind / g / d is one
+// contiguous segment (dwordx4 per lane when rows are padded to 4 entries and 16-byte aligned).
+// lanesPerSpike = 64 is the "post span" mapping (lanes span the row); small values are the
+// "pre span" mapping (few lanes per spike, many spikes per wavefront).  Work items are dealt
+// round-robin to the sub-groups of the synapse group's blocks, so the launch geometry is fixed
+// while the spike count lives on the device.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(BLOCK)
-void presynapticUpdateKernel(const PreGroupDev *groups, uint32_t numGroups, StepArgs args, float dt,
-                             unsigned long long *eventCounter)
+void presynapticUpdateKernel(const PreGroupDev *blocks, StepArgs args, float dt, unsigned long long *eventCounter)
 {
     const Resolved st = resolve(args, dt);
-    const uint32_t gi = findGroup(groups, numGroups, blockIdx.x);
-    const PreGroupDev &G = groups[gi];
+    const PreGroupDev &G = blocks[blockIdx.x];
     const gennmi_presynaptic_update_group_t &g = G.g;
     const uint32_t batch = blockIdx.y;
     const uint32_t W = G.lanesPerSpike;
@@ -147,8 +151,9 @@ void presynapticUpdateKernel(const PreGroupDev *groups, uint32_t numGroups, Step
     const uint32_t lis = threadIdx.x & (W - 1);
     const uint32_t subGroup = (localBlock * BLOCK + threadIdx.x) / W;
     const uint32_t numSubGroups = (G.numBlocks * BLOCK) / W;
-    const uint32_t numSpikes = g.srcSpkCnt[batch];
-    const uint32_t *spk = g.srcSpk + (size_t)batch * g.numSrcNeurons;
+    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
+    GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
     unsigned long long events = 0;
 
     if(g.matrix == GENNMI_MATRIX_TOEPLITZ_CONV2D) {
@@ -157,13 +162,17 @@ void presynapticUpdateKernel(const PreGroupDev *groups, uint32_t numGroups, Step
         const int kh = g.conv[0], kw = g.conv[1], iw = g.conv[3], ic = g.conv[4];
         const int oh = g.conv[5], ow = g.conv[6], oc = g.conv[7];
         const uint32_t numDiag = (uint32_t)(kh * kw * oc);
-        float *outPost = g.outPost + (size_t)batch * g.numTrgNeurons;
-        for(uint32_t s = subGroup; s < numSpikes; s += numSubGroups) {
+        const uint32_t chunksPerRow = (numDiag + W - 1) / W;
+        const unsigned long long numItems = (unsigned long long)numSpikes * chunksPerRow;
+        GLOBAL_AS const float *kernel = asGlobal(g.g);
+        for(unsigned long long item = subGroup; item < numItems; item += numSubGroups) {
+            const uint32_t s = (uint32_t)(item / chunksPerRow);
+            const uint32_t j = (uint32_t)(item % chunksPerRow) * W + lis;
             const uint32_t ipre = spk[s];
-            const int preRow = (int)(ipre / ic) / iw;
-            const int preCol = (int)(ipre / ic) % iw;
-            const int preChan = (int)(ipre % ic);
-            for(uint32_t j = lis; j < numDiag; j += W) {
+            if(j < numDiag) {
+                const int preRow = (int)(ipre / ic) / iw;
+                const int preCol = (int)(ipre / ic) % iw;
+                const int preChan = (int)(ipre % ic);
                 const int kernRow = (int)(j / oc) / kw;
                 const int kernCol = (int)(j / oc) % kw;
                 const int kernOutChan = (int)(j % oc);
@@ -172,7 +181,7 @@ void presynapticUpdateKernel(const PreGroupDev *groups, uint32_t numGroups, Step
                 if(postRow >= 0 && postCol >= 0 && postRow < oh && postCol < ow) {
                     const int postInd = (postRow * ow * oc) + (postCol * oc) + kernOutChan;
                     const int kernelInd = ((kh - kernRow - 1) * kw * ic * oc) + ((kw - kernCol - 1) * ic * oc) + (preChan * oc) + kernOutChan;
-                    atomicAddF32(&outPost[postInd], g.g[kernelInd]);
+                    atomicAddF32(&outPost[postInd], kernel[kernelInd]);
                     events++;
                 }
             }
@@ -184,70 +193,83 @@ void presynapticUpdateKernel(const PreGroupDev *groups, uint32_t numGroups, Step
         // (synapseUpdateGroupMerged.cc:480-483); st.epoch counts completed steps, so the pointer
         // in force during this step is (epoch + 1) % D.
         const uint32_t denPtr = D ? (uint32_t)((st.epoch + 1) % D) : 0;
-        float *outPost = g.outPost + (size_t)batch * g.numTrgNeurons;
-        float *denDelay = D ? g.denDelay + (size_t)batch * D * g.numTrgNeurons : nullptr;
-        for(uint32_t s = subGroup; s < numSpikes; s += numSubGroups) {
-            const uint32_t idPre = spk[s];
-            const uint32_t npost = g.rowLength[idPre];
+        GLOBAL_AS float *denDelay = D ? asGlobal(g.denDelay) + (size_t)batch * D * g.numTrgNeurons : nullptr;
+        GLOBAL_AS const uint32_t *rowLength = asGlobal(g.rowLength);
+        GLOBAL_AS const uint32_t *ind = asGlobal(g.ind);
+        GLOBAL_AS float *weight = asGlobal(g.g);
+        GLOBAL_AS const uint8_t *delay = asGlobal(g.d);
+        const uint32_t numTrg = g.numTrgNeurons;
+        const uint32_t perLane = G.vec4 ? 4u : 1u;
+        const uint32_t span = W * perLane;
+        const uint32_t chunksPerRow = (g.rowStride + span - 1) / span;
+        const unsigned long long numItems = (unsigned long long)numSpikes * chunksPerRow;
+        // Loads are issued ahead of the values that decide whether they are needed, so that the
+        // dependent chain per item is spike id -> {rowLength, row chunk} -> atomics: the spike id of
+        // the NEXT item is fetched while the current one is processed (spk always holds
+        // numSrcNeurons entries, so any index below that is readable), and the row chunk is read
+        // together with rowLength (rows are padded to rowStride, so any j < rowStride is readable).
+        const uint32_t lastSrc = g.numSrcNeurons - 1;
+        uint32_t idPreNext = spk[min((uint32_t)(subGroup / chunksPerRow), lastSrc)];
+        for(unsigned long long item = subGroup; item < numItems; item += numSubGroups) {
+            const uint32_t chunk = (uint32_t)(item % chunksPerRow);
+            const uint32_t idPre = idPreNext;
+            idPreNext = spk[min((uint32_t)((item + numSubGroups) / chunksPerRow), lastSrc)];
             const size_t rowBase = (size_t)idPre * g.rowStride;
-            if(lis == 0) { events += npost; }
+            const uint32_t j = chunk * span + lis * perLane;
+            const bool inRow = (j < g.rowStride);
+            const uint32_t npost = rowLength[idPre];
             if(g.wum == GENNMI_WUM_STATIC_PULSE) {
                 if(G.vec4) {
-                    const uint4 *ind4 = reinterpret_cast<const uint4*>(g.ind + rowBase);
-                    const float4 *g4 = reinterpret_cast<const float4*>(g.g + rowBase);
-                    for(uint32_t j = lis * 4; j < npost; j += W * 4) {
-                        const uint4 ip = ind4[j >> 2];
-                        const float4 w = g4[j >> 2];
-                        atomicAddF32(&outPost[ip.x], w.x);
-                        if(j + 1 < npost) { atomicAddF32(&outPost[ip.y], w.y); }
-                        if(j + 2 < npost) { atomicAddF32(&outPost[ip.z], w.z); }
-                        if(j + 3 < npost) { atomicAddF32(&outPost[ip.w], w.w); }
+                    u32x4 ip = {0, 0, 0, 0}; f32x4 w = {0, 0, 0, 0};
+                    if(inRow) {
+                        ip = *reinterpret_cast<GLOBAL_AS const u32x4*>(ind + rowBase + j);
+                        w = *reinterpret_cast<GLOBAL_AS const f32x4*>(weight + rowBase + j);
                     }
+                    if(j < npost) { atomicAddF32(&outPost[ip.x], w.x); }
+                    if(j + 1 < npost) { atomicAddF32(&outPost[ip.y], w.y); }
+                    if(j + 2 < npost) { atomicAddF32(&outPost[ip.z], w.z); }
+                    if(j + 3 < npost) { atomicAddF32(&outPost[ip.w], w.w); }
                 }
                 else {
-                    for(uint32_t j = lis; j < npost; j += W) {
-                        atomicAddF32(&outPost[g.ind[rowBase + j]], g.g[rowBase + j]);
-                    }
+                    uint32_t ip = 0; float w = 0;
+                    if(inRow) { ip = ind[rowBase + j]; w = weight[rowBase + j]; }
+                    if(j < npost) { atomicAddF32(&outPost[ip], w); }
                 }
             }
             else if(g.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY) {
                 // addToPostDelay(g, d): denDelay[((ptr + d) % D) * numPost + idPost] += g  (synapseUpdateGroupMerged.cc:245-251)
                 if(G.vec4) {
-                    const uint4 *ind4 = reinterpret_cast<const uint4*>(g.ind + rowBase);
-                    const float4 *g4 = reinterpret_cast<const float4*>(g.g + rowBase);
-                    const uchar4 *d4 = reinterpret_cast<const uchar4*>(g.d + rowBase);
-                    for(uint32_t j = lis * 4; j < npost; j += W * 4) {
-                        const uint4 ip = ind4[j >> 2];
-                        const float4 w = g4[j >> 2];
-                        const uchar4 dl = d4[j >> 2];
-                        atomicAddF32(&denDelay[(size_t)((denPtr + dl.x) % D) * g.numTrgNeurons + ip.x], w.x);
-                        if(j + 1 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.y) % D) * g.numTrgNeurons + ip.y], w.y); }
-                        if(j + 2 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.z) % D) * g.numTrgNeurons + ip.z], w.z); }
-                        if(j + 3 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.w) % D) * g.numTrgNeurons + ip.w], w.w); }
+                    u32x4 ip = {0, 0, 0, 0}; f32x4 w = {0, 0, 0, 0}; u8x4 dl = {0, 0, 0, 0};
+                    if(inRow) {
+                        ip = *reinterpret_cast<GLOBAL_AS const u32x4*>(ind + rowBase + j);
+                        w = *reinterpret_cast<GLOBAL_AS const f32x4*>(weight + rowBase + j);
+                        dl = *reinterpret_cast<GLOBAL_AS const u8x4*>(delay + rowBase + j);
                     }
+                    if(j < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.x) % D) * numTrg + ip.x], w.x); }
+                    if(j + 1 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.y) % D) * numTrg + ip.y], w.y); }
+                    if(j + 2 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.z) % D) * numTrg + ip.z], w.z); }
+                    if(j + 3 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.w) % D) * numTrg + ip.w], w.w); }
                 }
                 else {
-                    for(uint32_t j = lis; j < npost; j += W) {
-                        const uint32_t slot = (denPtr + g.d[rowBase + j]) % D;
-                        atomicAddF32(&denDelay[(size_t)slot * g.numTrgNeurons + g.ind[rowBase + j]], g.g[rowBase + j]);
-                    }
+                    uint32_t ip = 0; float w = 0; uint32_t dl = 0;
+                    if(inRow) { ip = ind[rowBase + j]; w = weight[rowBase + j]; dl = delay[rowBase + j]; }
+                    if(j < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl) % D) * numTrg + ip], w); }
                 }
             }
-            else {
+            else if(j < npost) {
                 // trace STDP presynaptic-spike code (pygenn/genn_model.py:1456-1463); every synapse of
                 // the row is owned by exactly one lane, so the read-modify-write of g needs no atomic
-                for(uint32_t j = lis; j < npost; j += W) {
-                    const uint32_t idPost = g.ind[rowBase + j];
-                    const float w = g.g[rowBase + j];
-                    const float stPost = dt + g.trgST[idPost];       // st_post = DT*(backPropSteps+1) + trgST (synapseUpdateGroupMerged.cc:134-142)
-                    atomicAddF32(&outPost[idPost], w);
-                    const float dtSpike = st.t - stPost;
-                    if(dtSpike > 0) {
-                        const float newWeight = w - (g.aMinus * g.postTrace[idPost]);
-                        g.g[rowBase + j] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
-                    }
+                const uint32_t idPost = ind[rowBase + j];
+                const float w = weight[rowBase + j];
+                const float stPost = dt + asGlobal(g.trgST)[idPost];   // st_post = DT*(backPropSteps+1) + trgST (synapseUpdateGroupMerged.cc:134-142)
+                atomicAddF32(&outPost[idPost], w);
+                const float dtSpike = st.t - stPost;
+                if(dtSpike > 0) {
+                    const float newWeight = w - (g.aMinus * asGlobal(g.postTrace)[idPost]);
+                    weight[rowBase + j] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
                 }
             }
+            if(lis == 0 && chunk == 0) { events += npost; }
         }
     }
 
@@ -261,11 +283,10 @@ void presynapticUpdateKernel(const PreGroupDev *groups, uint32_t numGroups, Step
 // remap (coalesced), gathers g by synapse index.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(BLOCK)
-void postsynapticUpdateKernel(const PostGroupDev *groups, uint32_t numGroups, StepArgs args, float dt)
+void postsynapticUpdateKernel(const PostGroupDev *blocks, StepArgs args, float dt)
 {
     const Resolved st = resolve(args, dt);
-    const uint32_t gi = findGroup(groups, numGroups, blockIdx.x);
-    const PostGroupDev &G = groups[gi];
+    const PostGroupDev &G = blocks[blockIdx.x];
     const gennmi_postsynaptic_update_group_t &g = G.g;
     const uint32_t W = G.lanesPerSpike;
     const uint32_t localBlock = blockIdx.x - G.startBlock;
@@ -298,15 +319,14 @@ void postsynapticUpdateKernel(const PostGroupDev *groups, uint32_t numGroups, St
 // emitted spikes, and the last block of each population (which stores spkCnt), look back.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(BLOCK)
-void neuronUpdateKernel(const NeuronGroupDev *groups, uint32_t numGroups, StepArgs args, float dt,
+void neuronUpdateKernel(const NeuronGroupDev *blocks, StepArgs args, float dt,
                         unsigned long long *agg, uint32_t *errorFlag)
 {
     __shared__ uint32_t shWaveCount[BLOCK / WAVE];
     __shared__ uint32_t shPrefix;
 
     const Resolved st = resolve(args, dt);
-    const uint32_t gi = findGroup(groups, numGroups, blockIdx.x);
-    const NeuronGroupDev &G = groups[gi];
+    const NeuronGroupDev &G = blocks[blockIdx.x];
     const gennmi_neuron_update_group_t &g = G.g;
     const uint32_t batch = blockIdx.y;
     const uint32_t localBlock = blockIdx.x - G.startBlock;
@@ -421,8 +441,10 @@ void neuronUpdateKernel(const NeuronGroupDev *groups, uint32_t numGroups, StepAr
     const uint32_t tag = (uint32_t)(st.epoch + 1);
     const size_t aggBase = (size_t)batch * gridDim.x + G.startBlock;
     if(threadIdx.x == 0) {
+        // the count itself is all that is communicated, so a relaxed device-scope store suffices
+        // (release would write back the whole L2 from every block)
         __hip_atomic_store(&agg[aggBase + localBlock], ((unsigned long long)tag << 32) | blockCount,
-                           __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     const bool last = (localBlock == G.numBlocks - 1);
     if(blockCount == 0 && !last) { return; }
@@ -436,7 +458,7 @@ void neuronUpdateKernel(const NeuronGroupDev *groups, uint32_t numGroups, StepAr
             if(k < localBlock) {
                 uint32_t spins = 0;
                 while(true) {
-                    const unsigned long long a = __hip_atomic_load(&agg[aggBase + k], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+                    const unsigned long long a = __hip_atomic_load(&agg[aggBase + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     if((uint32_t)(a >> 32) == tag) { v = (uint32_t)a; break; }
                     if(++spins > SPIN_LIMIT) { ok = false; break; }
                     __builtin_amdgcn_s_sleep(1);
@@ -733,10 +755,11 @@ int gennmi_runner_finalise(gennmi_runner *r)
     r->neuronBlocks = block;
 
     // Presynaptic launch geometry.  The number of spikes is only known on the device, so every
-    // group gets enough sub-groups to keep the chip busy when its whole source population fires
-    // within a few steps, capped so that silent groups cost next to nothing.
+    // group gets a fixed share of a block budget and deals its (spike, chunk) work items round-robin.
     block = 0;
-    const uint32_t maxBlocksPerGroup = std::max(1u, (numCU * 16u) / std::max<uint32_t>(1u, (uint32_t)r->pre.size()));
+    const char *envBudget = getenv("GENNMI_PRESYN_BLOCKS_PER_CU");
+    const uint32_t blocksPerCU = envBudget ? std::max(1, atoi(envBudget)) : 4u;
+    const uint32_t maxBlocksPerGroup = std::max(2u, (numCU * blocksPerCU) / std::max<uint32_t>(1u, (uint32_t)r->pre.size()));
     for(auto &p : r->pre) {
         const uint32_t rowLen = (p.g.matrix == GENNMI_MATRIX_SPARSE) ? p.g.rowStride : (uint32_t)(p.g.conv[0] * p.g.conv[1] * p.g.conv[7]);
         uint32_t W;
@@ -748,8 +771,10 @@ int gennmi_runner_finalise(gennmi_runner *r)
                   && (reinterpret_cast<uintptr_t>(p.g.ind) % 16) == 0 && (reinterpret_cast<uintptr_t>(p.g.g) % 16) == 0
                   && (p.g.wum != GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY || (reinterpret_cast<uintptr_t>(p.g.d) % 4) == 0)
                   && W >= 16) ? 1u : 0u;
-        // expected concurrent spikes: a few percent of the source population per step
-        const uint64_t wantSubGroups = std::max<uint64_t>(8, p.g.numSrcNeurons / 16);
+        const uint32_t span = W * (p.vec4 ? 4u : 1u);
+        const uint64_t chunksPerRow = (rowLen + span - 1) / span;
+        // enough sub-groups for ~1.5 % of the source population firing in one step
+        const uint64_t wantSubGroups = std::max<uint64_t>(8, ((uint64_t)p.g.numSrcNeurons * chunksPerRow) / 64);
         uint32_t blocks = (uint32_t)std::min<uint64_t>((wantSubGroups * W + BLOCK - 1) / BLOCK, maxBlocksPerGroup);
         p.startBlock = block;
         p.numBlocks = std::max(1u, blocks);
@@ -768,16 +793,22 @@ int gennmi_runner_finalise(gennmi_runner *r)
     }
     r->postBlocks = block;
 
-    HIP_TRY(hipMalloc(&r->dNeuron, r->neuron.size() * sizeof(NeuronGroupDev)));
-    HIP_TRY(hipMemcpy(r->dNeuron, r->neuron.data(), r->neuron.size() * sizeof(NeuronGroupDev), hipMemcpyHostToDevice));
-    if(!r->pre.empty()) {
-        HIP_TRY(hipMalloc(&r->dPre, r->pre.size() * sizeof(PreGroupDev)));
-        HIP_TRY(hipMemcpy(r->dPre, r->pre.data(), r->pre.size() * sizeof(PreGroupDev), hipMemcpyHostToDevice));
-    }
-    if(!r->post.empty()) {
-        HIP_TRY(hipMalloc(&r->dPost, r->post.size() * sizeof(PostGroupDev)));
-        HIP_TRY(hipMemcpy(r->dPost, r->post.data(), r->post.size() * sizeof(PostGroupDev), hipMemcpyHostToDevice));
-    }
+    // One descriptor copy per block, indexed by blockIdx.x: a block finds everything it needs with a
+    // single round of scalar loads (the reference bisects a start-ID table and then loads the merged
+    // struct, backendSIMT.h:244-323 — two to four dependent loads before any work starts).
+    auto uploadPerBlock = [](const auto &groups, uint32_t totalBlocks, auto **dTable) -> hipError_t {
+        using T = typename std::remove_reference<decltype(groups[0])>::type;
+        std::vector<typename std::remove_const<T>::type> table;
+        table.reserve(totalBlocks);
+        for(const auto &g : groups) { for(uint32_t b = 0; b < g.numBlocks; b++) { table.push_back(g); } }
+        if(table.empty()) { *dTable = nullptr; return hipSuccess; }
+        hipError_t e = hipMalloc(dTable, table.size() * sizeof(table[0]));
+        if(e != hipSuccess) { return e; }
+        return hipMemcpy(*dTable, table.data(), table.size() * sizeof(table[0]), hipMemcpyHostToDevice);
+    };
+    HIP_TRY(uploadPerBlock(r->neuron, r->neuronBlocks, &r->dNeuron));
+    HIP_TRY(uploadPerBlock(r->pre, r->preBlocks, &r->dPre));
+    HIP_TRY(uploadPerBlock(r->post, r->postBlocks, &r->dPost));
     const size_t aggCount = (size_t)r->neuronBlocks * r->batch;
     HIP_TRY(hipMalloc(&r->dAgg, aggCount * sizeof(unsigned long long)));
     HIP_TRY(hipMemset(r->dAgg, 0, aggCount * sizeof(unsigned long long)));
@@ -790,11 +821,11 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
 {
     if(timed) { HIP_TRY(hipEventRecord(r->evA, r->stream)); }
     if(!r->pre.empty()) {
-        presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dPre, (uint32_t)r->pre.size(), a, r->dt, r->dEvents);
+        presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dPre, a, r->dt, r->dEvents);
         if(timed) { HIP_TRY(hipEventRecord(r->evB, r->stream)); }
     }
     if(!r->post.empty()) {
-        postsynapticUpdateKernel<<<dim3(r->postBlocks), dim3(BLOCK), 0, r->stream>>>(r->dPost, (uint32_t)r->post.size(), a, r->dt);
+        postsynapticUpdateKernel<<<dim3(r->postBlocks), dim3(BLOCK), 0, r->stream>>>(r->dPost, a, r->dt);
         if(timed) { HIP_TRY(hipEventRecord(r->evC, r->stream)); }
     }
     HIP_TRY(hipGetLastError());
@@ -804,7 +835,7 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
 static int launchNeurons(gennmi_runner *r, const StepArgs &a, bool timed)
 {
     if(timed) { HIP_TRY(hipEventRecord(r->evC, r->stream)); }
-    neuronUpdateKernel<<<dim3(r->neuronBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dNeuron, (uint32_t)r->neuron.size(), a, r->dt, r->dAgg, r->dError);
+    neuronUpdateKernel<<<dim3(r->neuronBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dNeuron, a, r->dt, r->dAgg, r->dError);
     if(timed) { HIP_TRY(hipEventRecord(r->evD, r->stream)); }
     HIP_TRY(hipGetLastError());
     return GENNMI_OK;
