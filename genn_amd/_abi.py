@@ -80,6 +80,7 @@ SYMBOLS = {
     "gennmi_fill_f32": (C.c_int, [C.c_void_p, C.c_float, C.c_size_t]),
     "gennmi_synchronize": (C.c_int, []),
     "gennmi_free_device_memory_bytes": (C.c_int, [C.POINTER(C.c_size_t)]),
+    "gennmi_abi_struct_sizes": (C.c_int, [C.POINTER(C.c_size_t * 5)]),
     "gennmi_runner_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_float, C.c_uint32]),
     "gennmi_runner_destroy": (C.c_int, [C.c_void_p]),
     "gennmi_push_neuron_update_group": (C.c_int, [C.c_void_p, C.POINTER(NeuronUpdateGroup), C.POINTER(C.c_uint32)]),

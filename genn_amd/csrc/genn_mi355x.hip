@@ -619,6 +619,14 @@ int gennmi_free_device_memory_bytes(size_t *bytes)
     return GENNMI_OK;
 }
 
+int gennmi_abi_struct_sizes(size_t sizes[5])
+{
+    if(!sizes) { return fail(GENNMI_EINVAL, "abi_struct_sizes: null argument"); }
+    sizes[0] = sizeof(gennmi_psm_t); sizes[1] = sizeof(gennmi_cs_t); sizes[2] = sizeof(gennmi_neuron_update_group_t);
+    sizes[3] = sizeof(gennmi_presynaptic_update_group_t); sizes[4] = sizeof(gennmi_postsynaptic_update_group_t);
+    return GENNMI_OK;
+}
+
 int gennmi_runner_create(gennmi_runner **runner, float dt, uint32_t batchSize)
 {
     if(!runner || batchSize == 0 || batchSize > 65535) { return fail(GENNMI_EINVAL, "gennmi_runner_create: bad arguments"); }

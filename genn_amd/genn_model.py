@@ -291,8 +291,6 @@ class GeNNModel:
 
     # ------------------------------------------------------------------ build = finalise + derive constants
     def build(self):
-        lib = _abi.load()
-        _abi.check(lib.gennmi_init(self._device))
         for n in self.neuron_populations.values():
             # fuse postsynaptic models (src/genn/genn/neuronGroup.cc:436): same snippet, same parameters,
             # same dendritic-delay depth, no state variables
@@ -342,6 +340,7 @@ class GeNNModel:
         if not self._built:
             raise RuntimeError("build() must be called before load()")
         lib = _abi.load()
+        _abi.check(lib.gennmi_init(self._device))
         B = self.batch_size
         self.num_recording_timesteps = num_recording_timesteps
         dt32 = lit32(self.dt)

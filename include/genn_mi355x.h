@@ -64,6 +64,11 @@ int gennmi_memset(void *dev, int value, size_t bytes);          /* memsetDeviceO
 int gennmi_fill_f32(float *dev, float value, size_t count);     /* e.g. sT = -TIME_MAX (initGroupMerged.cc neuron init) */
 int gennmi_synchronize(void);
 int gennmi_free_device_memory_bytes(size_t *bytes);             /* genReturnFreeDeviceMemoryBytes, backendCUDAHIP.cc */
+/* sizeof() of the five descriptor structs below, in declaration order (psm, cs, neuron update, presynaptic
+ * update, postsynaptic update), so that a binding in another language can verify its struct layout.  Needs
+ * no device.  The reference gets the same guarantee from generating both sides of every push call from one
+ * field list (groupMerged.h:214-227). */
+int gennmi_abi_struct_sizes(size_t sizes[5]);
 
 /* ---------------------------------------------------------------------------------------------
  * Merged-group descriptors.  Field names follow the reference's merged structs

@@ -413,6 +413,9 @@ void gc_step(gc_net *net)
     net->timestep++;
 }
 
+/* for callers that run the two halves of a step separately */
+void gc_advance(gc_net *net) { net->timestep++; }
+
 void gc_run(gc_net *net, uint64_t steps) { for(uint64_t i = 0; i < steps; i++) { gc_step(net); } }
 
 /* ------------------------------------------------------------------------------------------ */

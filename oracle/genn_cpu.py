@@ -49,6 +49,9 @@ def lib():
         l.gc_add_syn_conv2d.restype = i32; l.gc_add_syn_conv2d.argtypes = [vp, i32, i32, i32, vp, vp]
         l.gc_build_remap.restype = None; l.gc_build_remap.argtypes = [vp, i32]
         l.gc_step.restype = None; l.gc_step.argtypes = [vp]
+        l.gc_advance.restype = None; l.gc_advance.argtypes = [vp]
+        l.gc_update_synapses.restype = None; l.gc_update_synapses.argtypes = [vp, f32]
+        l.gc_update_neurons.restype = None; l.gc_update_neurons.argtypes = [vp, f32, u32]
         l.gc_run.restype = None; l.gc_run.argtypes = [vp, u64]
         l.gc_spike_count.restype = u32; l.gc_spike_count.argtypes = [vp, i32]
         for name in ("gc_spikes", "gc_start_spike", "gc_record", "gc_pre_trace", "gc_post_trace", "gc_spike_time"):

@@ -1,0 +1,28 @@
+"""Definitions of the golden cases: small networks of each configuration's shape.  Shared by
+make_golden.py (which runs the reference's own CPU backend on them, in the builder container)
+and by the tests (which regenerate the same inputs and compare against the stored outputs)."""
+from genn_amd import configs
+
+
+def va_small():
+    return configs.vogels_abbott(n=400, steps=300, p=0.1), 50
+
+
+def potjans_small():
+    return configs.potjans(neuron_scale=0.02, connectivity_scale=0.2, steps=400), 50
+
+
+def izhikevich_small():
+    return configs.izhikevich_fanout(n=500, fanout=50, steps=200), 25
+
+
+def stdp_small():
+    return configs.plastic_stdp(n=500, n_src=50, steps=200, fan=60, src_fan=40), 25
+
+
+def conv_small():
+    return configs.conv_toeplitz(h=8, w=8, ic=2, oc=4, steps=100, w_sd=0.6, ioffset=0.4), 25
+
+
+CASES = {"va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+         "stdp_small": stdp_small, "conv_small": conv_small}

@@ -1,0 +1,70 @@
+#!/usr/bin/env python3
+"""Writes the golden fixtures tests/golden/<case>.npz by running the REFERENCE's own
+SingleThreadedCPU backend (oracle/_ref/ref_driver, built by oracle/Makefile.ref from the sources
+under /root/reference) on each case of cases.py.  Runs only where the reference tree is mounted;
+the fixtures it writes are data: the digest of the inputs, spike rasters, and state snapshots.
+
+    python tests/golden/make_golden.py [case ...]
+"""
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, HERE)
+
+from genn_amd.netspec import write_netspec  # noqa: E402
+from cases import CASES  # noqa: E402
+
+DRIVER = os.path.join(ROOT, "oracle", "_ref", "ref_driver")
+
+
+def make(name):
+    net, snap = CASES[name]()
+    net.snap = snap
+    tmp = tempfile.mkdtemp(prefix="golden_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(net, spec)
+        subprocess.check_call([DRIVER, spec, work, out], stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        data = {"input_digest": np.array(net.input_digest()), "snap": np.array(snap), "steps": np.array(net.steps)}
+        fuse = dict(line.split() for line in open(os.path.join(out, "fusemap.txt")))
+        data["fusemap"] = np.array([f"{k}={v}" for k, v in fuse.items()])
+        for p in net.pops:
+            data[f"spikes.{p.name}"] = np.fromfile(os.path.join(out, f"{p.name}.spikes.u32"), np.uint32).reshape(-1, 2)
+            for var in ("V", "RefracTime", "U"):
+                f = os.path.join(out, f"{p.name}.{var}.f32")
+                if os.path.exists(f):
+                    data[f"{var}.{p.name}"] = np.fromfile(f, np.float32).reshape(-1, p.n)
+        for s in net.syns:
+            for var, dtype in (("outPost", np.float32), ("denDelay", np.float32), ("g", np.float32), ("preTrace", np.float32),
+                               ("postTrace", np.float32), ("colLength", np.uint32), ("remap", np.uint32)):
+                f = os.path.join(out, f"{s.name}.{var}.{'u32' if dtype == np.uint32 else 'f32'}")
+                if os.path.exists(f):
+                    a = np.fromfile(f, dtype)
+                    if var in ("g", "denDelay", "outPost", "preTrace", "postTrace"):
+                        a = a.reshape(net.steps // snap, -1)[-1] if var in ("g", "denDelay") else a.reshape(net.steps // snap, -1)
+                    data[f"{var}.{s.name}"] = a
+            f = os.path.join(out, f"{s.name}.colStride.txt")
+            if os.path.exists(f):
+                data[f"colStride.{s.name}"] = np.array(int(open(f).read()))
+        np.savez_compressed(os.path.join(HERE, name + ".npz"), **data)
+        total = sum(len(data[f"spikes.{p.name}"]) for p in net.pops)
+        print(f"{name}: {total} spikes, {os.path.getsize(os.path.join(HERE, name + '.npz')) / 1024:.0f} KiB")
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
+if __name__ == "__main__":
+    if not os.path.exists(DRIVER):
+        raise SystemExit("oracle/_ref/ref_driver is missing: run `make -f Makefile.ref` in oracle/ (needs /root/reference)")
+    for case in (sys.argv[1:] or list(CASES)):
+        make(case)
