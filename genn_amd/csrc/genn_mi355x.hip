@@ -88,10 +88,25 @@ __device__ __forceinline__ Resolved resolve(const StepArgs &a, float dt)
     return r;
 }
 
+// Synapses whose dendritic delay is a multiple of the ring depth land in the slot the target reads in
+// the very step that delivers them.  When a runner handles them in the neuron update (see
+// gennmi_runner_finalise), each population carries one of these per outgoing delayed projection:
+// the positions of such synapses within every row.
+struct ZeroDelayEntry
+{
+    float *ringElem;                    // &denDelay[ipost] of the target ring (slot 0, batch 0)
+    const float *weight;                // &g[idSyn]: read at delivery time, so pushed weights are honoured
+    uint32_t numTrgNeurons, maxDenDelay;
+};
+
 struct NeuronGroupDev
 {
     gennmi_neuron_update_group_t g;
     uint32_t startBlock, numBlocks;
+    const uint32_t *zeroStart;          // [N+1] CSR offsets into zeroEntries (all outgoing projections merged), or NULL
+    const ZeroDelayEntry *zeroEntries;
+    uint32_t *shadowSpk;                // [2][batch*N] engine-private double-buffered copy of the spike queue, or NULL
+    uint32_t *shadowCnt;                // [2][batch]
 };
 
 struct PreGroupDev
@@ -101,6 +116,9 @@ struct PreGroupDev
     uint32_t lanesPerSpike;             // power of two, 1..64
     uint32_t vec4;                      // rows are 16-byte aligned and padded: dwordx4 loads
     int32_t convBH, convBW;
+    uint32_t skipZeroDelay, pad_;       // synapses with d % D == 0 are delivered by the neuron update instead
+    const uint32_t *shadowSpk;          // the source population's shadow queue (read instead of srcSpk when set)
+    const uint32_t *shadowCnt;
 };
 
 struct PostGroupDev
@@ -139,20 +157,23 @@ __device__ __forceinline__ void atomicAddF32(GLOBAL_AS float *addr, float v)
 // round-robin to the sub-groups of the synapse group's blocks, so the launch geometry is fixed
 // while the spike count lives on the device.
 // ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(BLOCK)
-void presynapticUpdateKernel(const PreGroupDev *blocks, StepArgs args, float dt, unsigned long long *eventCounter)
+__device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t blockInKernel, const Resolved &st, float dt,
+                                                unsigned long long *eventCounter)
 {
-    const Resolved st = resolve(args, dt);
-    const PreGroupDev &G = blocks[blockIdx.x];
     const gennmi_presynaptic_update_group_t &g = G.g;
     const uint32_t batch = blockIdx.y;
     const uint32_t W = G.lanesPerSpike;
-    const uint32_t localBlock = blockIdx.x - G.startBlock;
+    const uint32_t localBlock = blockInKernel - G.startBlock;
     const uint32_t lis = threadIdx.x & (W - 1);
     const uint32_t subGroup = (localBlock * BLOCK + threadIdx.x) / W;
     const uint32_t numSubGroups = (G.numBlocks * BLOCK) / W;
-    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
-    GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    // spikes of the previous step: the population's own queue, or (when this launch may run next to the
+    // neuron update that refills that queue) the shadow copy written one step ago
+    const uint32_t parity = (uint32_t)((st.epoch + 1) & 1);
+    GLOBAL_AS const uint32_t *cntPtr = G.shadowSpk ? asGlobal(G.shadowCnt) + (size_t)parity * gridDim.y : asGlobal(g.srcSpkCnt);
+    GLOBAL_AS const uint32_t *spk = G.shadowSpk ? asGlobal(G.shadowSpk) + ((size_t)parity * gridDim.y + batch) * g.numSrcNeurons
+                                                : asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    const uint32_t numSpikes = cntPtr[batch];
     GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
     unsigned long long events = 0;
 
@@ -245,15 +266,18 @@ void presynapticUpdateKernel(const PreGroupDev *blocks, StepArgs args, float dt,
                         w = *reinterpret_cast<GLOBAL_AS const f32x4*>(weight + rowBase + j);
                         dl = *reinterpret_cast<GLOBAL_AS const u8x4*>(delay + rowBase + j);
                     }
-                    if(j < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.x) % D) * numTrg + ip.x], w.x); }
-                    if(j + 1 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.y) % D) * numTrg + ip.y], w.y); }
-                    if(j + 2 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.z) % D) * numTrg + ip.z], w.z); }
-                    if(j + 3 < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl.w) % D) * numTrg + ip.w], w.w); }
+                    const uint32_t s0 = (denPtr + dl.x) % D, s1 = (denPtr + dl.y) % D, s2 = (denPtr + dl.z) % D, s3 = (denPtr + dl.w) % D;
+                    const bool skip = (G.skipZeroDelay != 0);       // slot == denPtr <=> d % D == 0
+                    if(j < npost && !(skip && s0 == denPtr)) { atomicAddF32(&denDelay[(size_t)s0 * numTrg + ip.x], w.x); }
+                    if(j + 1 < npost && !(skip && s1 == denPtr)) { atomicAddF32(&denDelay[(size_t)s1 * numTrg + ip.y], w.y); }
+                    if(j + 2 < npost && !(skip && s2 == denPtr)) { atomicAddF32(&denDelay[(size_t)s2 * numTrg + ip.z], w.z); }
+                    if(j + 3 < npost && !(skip && s3 == denPtr)) { atomicAddF32(&denDelay[(size_t)s3 * numTrg + ip.w], w.w); }
                 }
                 else {
                     uint32_t ip = 0; float w = 0; uint32_t dl = 0;
                     if(inRow) { ip = ind[rowBase + j]; w = weight[rowBase + j]; dl = delay[rowBase + j]; }
-                    if(j < npost) { atomicAddF32(&denDelay[(size_t)((denPtr + dl) % D) * numTrg + ip], w); }
+                    const uint32_t slot = (denPtr + dl) % D;
+                    if(j < npost && !(G.skipZeroDelay && slot == denPtr)) { atomicAddF32(&denDelay[(size_t)slot * numTrg + ip], w); }
                 }
             }
             else if(j < npost) {
@@ -276,6 +300,12 @@ void presynapticUpdateKernel(const PreGroupDev *blocks, StepArgs args, float dt,
     // one counter update per wave
     for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
     if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+__global__ __launch_bounds__(BLOCK)
+void presynapticUpdateKernel(const PreGroupDev *blocks, StepArgs args, float dt, unsigned long long *eventCounter)
+{
+    presynapticBody(blocks[blockIdx.x], blockIdx.x, resolve(args, dt), dt, eventCounter);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -318,18 +348,15 @@ void postsynapticUpdateKernel(const PostGroupDev *blocks, StepArgs args, float d
 // (tagged with the step so nothing ever needs clearing) the cross-block offset.  Only blocks that
 // emitted spikes, and the last block of each population (which stores spkCnt), look back.
 // ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(BLOCK)
-void neuronUpdateKernel(const NeuronGroupDev *blocks, StepArgs args, float dt,
-                        unsigned long long *agg, uint32_t *errorFlag)
+__device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blockInKernel, uint32_t totalNeuronBlocks,
+                                           const Resolved &st, float dt, unsigned long long *agg, uint32_t *errorFlag)
 {
     __shared__ uint32_t shWaveCount[BLOCK / WAVE];
     __shared__ uint32_t shPrefix;
 
-    const Resolved st = resolve(args, dt);
-    const NeuronGroupDev &G = blocks[blockIdx.x];
     const gennmi_neuron_update_group_t &g = G.g;
     const uint32_t batch = blockIdx.y;
-    const uint32_t localBlock = blockIdx.x - G.startBlock;
+    const uint32_t localBlock = blockInKernel - G.startBlock;
     const uint32_t n = g.numNeurons;
     const uint32_t i = localBlock * BLOCK + threadIdx.x;
     const size_t bi = (size_t)batch * n + i;
@@ -338,6 +365,8 @@ void neuronUpdateKernel(const NeuronGroupDev *blocks, StepArgs args, float dt,
     const float t = st.t;
 
     bool spiked = false;
+    uint32_t z0 = 0, z1 = 0;
+    if(G.zeroStart && i < n) { z0 = asGlobal(G.zeroStart)[i]; z1 = asGlobal(G.zeroStart)[i + 1]; }
     if(i < n) {
         // order of operations: neuronUpdateGroupMerged.cc:552-773 — PSMs, current sources, sim code,
         // WU pre/post dynamics, threshold, then (on a spike) WU pre/post spike code, sT, reset
@@ -439,7 +468,7 @@ void neuronUpdateKernel(const NeuronGroupDev *blocks, StepArgs args, float dt,
     }
 
     const uint32_t tag = (uint32_t)(st.epoch + 1);
-    const size_t aggBase = (size_t)batch * gridDim.x + G.startBlock;
+    const size_t aggBase = (size_t)batch * totalNeuronBlocks + G.startBlock;
     if(threadIdx.x == 0) {
         // the count itself is all that is communicated, so a relaxed device-scope store suffices
         // (release would write back the whole L2 from every block)
@@ -448,6 +477,25 @@ void neuronUpdateKernel(const NeuronGroupDev *blocks, StepArgs args, float dt,
     }
     const bool last = (localBlock == G.numBlocks - 1);
     if(blockCount == 0 && !last) { return; }
+
+    // Synapses with d % D == 0 of the neurons that just fired belong in the slot their targets read in the
+    // NEXT step, (epoch + 2) % D, which nothing reads or clears during this step — so the presynaptic update of
+    // the next step (which skips them) may run concurrently with that step's neuron update.  The wavefront
+    // delivers them cooperatively, one fired neuron at a time, lanes striding over its merged list.
+    auto deliverZeroDelay = [&]() {
+        unsigned long long pending = ballot;
+        while(pending) {
+            const int src = __ffsll((long long)pending) - 1;
+            pending &= pending - 1;
+            const uint32_t s0 = __shfl(z0, src, WAVE), s1 = __shfl(z1, src, WAVE);
+            for(uint32_t k = s0 + lane; k < s1; k += WAVE) {
+                const ZeroDelayEntry e = G.zeroEntries[k];
+                const uint32_t slot = (uint32_t)((st.epoch + 2) % e.maxDenDelay);
+                atomicAddF32(asGlobal(e.ringElem) + ((size_t)batch * e.maxDenDelay + slot) * e.numTrgNeurons, *asGlobal(e.weight));
+            }
+        }
+    };
+    if(G.zeroStart && wave != 0) { deliverZeroDelay(); }
 
     if(wave == 0) {
         uint32_t sum = 0;
@@ -478,6 +526,51 @@ void neuronUpdateKernel(const NeuronGroupDev *blocks, StepArgs args, float dt,
     if(prefix == 0xFFFFFFFFu) { return; }       // bounded wait expired: flagged, nothing written
     if(spiked) { g.spk[(size_t)batch * n + prefix + waveOffset + laneRank] = i; }
     if(last && threadIdx.x == 0) { g.spkCnt[batch] = prefix + blockCount; }
+    if(G.shadowSpk) {
+        const uint32_t parity = (uint32_t)(st.epoch & 1);
+        if(spiked) { G.shadowSpk[((size_t)parity * gridDim.y + batch) * n + prefix + waveOffset + laneRank] = i; }
+        if(last && threadIdx.x == 0) { G.shadowCnt[(size_t)parity * gridDim.y + batch] = prefix + blockCount; }
+    }
+    if(G.zeroStart && wave == 0) { deliverZeroDelay(); }
+}
+
+__global__ __launch_bounds__(BLOCK)
+void neuronUpdateKernel(const NeuronGroupDev *blocks, StepArgs args, float dt,
+                        unsigned long long *agg, uint32_t *errorFlag)
+{
+    neuronBody(blocks[blockIdx.x], blockIdx.x, gridDim.x, resolve(args, dt), dt, agg, errorFlag);
+}
+
+// One launch per timestep for networks whose projections all go through the dendritic-delay ring: the
+// neuron update of step t and the presynaptic update of step t touch disjoint ring slots once zero-delay
+// synapses are delivered by the spiking neuron itself, and the presynaptic update reads the shadow spike
+// queue of step t-1 while the neuron update refills the visible one.  Neuron blocks come first so that
+// their look-back chain starts early.
+__global__ __launch_bounds__(BLOCK)
+void stepFusedKernel(const NeuronGroupDev *neuronBlocks, uint32_t numNeuronBlocks, const PreGroupDev *preBlocks,
+                     StepArgs args, float dt, unsigned long long *agg, uint32_t *errorFlag, unsigned long long *eventCounter)
+{
+    const Resolved st = resolve(args, dt);
+    if(blockIdx.x < numNeuronBlocks) { neuronBody(neuronBlocks[blockIdx.x], blockIdx.x, numNeuronBlocks, st, dt, agg, errorFlag); }
+    else { presynapticBody(preBlocks[blockIdx.x - numNeuronBlocks], blockIdx.x - numNeuronBlocks, st, dt, eventCounter); }
+}
+
+// Per row: count the synapses with d % D == 0 and, when `entries` is given, append them at offset[row].
+__global__ void zeroDelayScanKernel(uint32_t numSrc, uint32_t rowStride, const uint32_t *rowLength, const uint8_t *d, uint32_t D,
+                                    const uint32_t *ind, const float *g, float *denDelay, uint32_t numTrg,
+                                    uint32_t *zeroLen, const uint32_t *offset, ZeroDelayEntry *entries)
+{
+    const uint32_t row = blockIdx.x * blockDim.x + threadIdx.x;
+    if(row >= numSrc) { return; }
+    const size_t base = (size_t)row * rowStride;
+    uint32_t count = 0;
+    for(uint32_t j = 0; j < rowLength[row]; j++) {
+        if((d[base + j] % D) == 0) {
+            if(entries) { entries[offset[row] + count] = ZeroDelayEntry{denDelay + ind[base + j], g + base + j, numTrg, D}; }
+            count++;
+        }
+    }
+    if(zeroLen) { zeroLen[row] = count; }
 }
 
 // Advances the device-resident step state at the end of a captured graph.
@@ -558,6 +651,8 @@ struct gennmi_runner
     StepState *dState = nullptr;
     unsigned long long epoch = 0;       // completed steps (host mirror)
     bool synapsesDone = false;          // updateSynapses ran for the current step
+    bool fusedStep = false;             // zero-delay synapses are delivered by the neuron update; one launch per step
+    std::vector<void*> owned;           // engine-private device allocations (shadow queues, zero-delay lists)
     // graph
     hipGraphExec_t graphExec = nullptr; unsigned long long graphSteps = 0;
     // timing
@@ -649,6 +744,7 @@ int gennmi_runner_destroy(gennmi_runner *r)
     hipStreamSynchronize(r->stream);
     if(r->graphExec) { hipGraphExecDestroy(r->graphExec); }
     for(hipEvent_t e : {r->evA, r->evB, r->evC, r->evD}) { if(e) { hipEventDestroy(e); } }
+    for(void *q : r->owned) { hipFree(q); }
     hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dAgg); hipFree(r->dError); hipFree(r->dEvents); hipFree(r->dState);
     hipStreamDestroy(r->stream);
     delete r;
@@ -814,6 +910,68 @@ int gennmi_runner_finalise(gennmi_runner *r)
         if(e != hipSuccess) { return e; }
         return hipMemcpy(*dTable, table.data(), table.size() * sizeof(table[0]), hipMemcpyHostToDevice);
     };
+    // ---- single-launch step: possible when every projection is a SPARSE dendritic-delay one with ring depth >= 2
+    // and nothing is plastic
+    const char *envFused = getenv("GENNMI_FUSED_STEP");
+    bool eligible = !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty();
+    for(const auto &p : r->pre) {
+        eligible = eligible && p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY
+                   && p.g.maxDenDelay >= 2;
+        bool found = false;
+        for(const auto &n : r->neuron) { found = found || (n.g.spk == p.g.srcSpk && n.g.numNeurons == p.g.numSrcNeurons); }
+        eligible = eligible && found;
+    }
+    if(eligible) {
+        auto devAlloc = [r](void **q, size_t bytes) -> hipError_t {
+            hipError_t e = hipMalloc(q, bytes ? bytes : 4);
+            if(e == hipSuccess) { r->owned.push_back(*q); e = hipMemset(*q, 0, bytes ? bytes : 4); }
+            return e;
+        };
+        for(auto &n : r->neuron) {
+            HIP_TRY(devAlloc((void**)&n.shadowSpk, 2 * (size_t)r->batch * n.g.numNeurons * sizeof(uint32_t)));
+            HIP_TRY(devAlloc((void**)&n.shadowCnt, 2 * (size_t)r->batch * sizeof(uint32_t)));
+            std::vector<PreGroupDev*> outs;
+            for(auto &p : r->pre) { if(p.g.srcSpk == n.g.spk) { outs.push_back(&p); } }
+            if(outs.empty()) { continue; }
+            const uint32_t N = n.g.numNeurons;
+            const dim3 grid((N + BLOCK - 1) / BLOCK);
+            uint32_t *dLen = nullptr;
+            HIP_TRY(devAlloc((void**)&dLen, (size_t)N * sizeof(uint32_t)));
+            std::vector<std::vector<uint32_t>> len(outs.size(), std::vector<uint32_t>(N));
+            for(size_t o = 0; o < outs.size(); o++) {
+                const auto &q = outs[o]->g;
+                zeroDelayScanKernel<<<grid, dim3(BLOCK), 0, 0>>>(N, q.rowStride, q.rowLength, q.d, q.maxDenDelay, q.ind, q.g, q.denDelay,
+                                                                 q.numTrgNeurons, dLen, nullptr, nullptr);
+                HIP_TRY(hipGetLastError());
+                HIP_TRY(hipMemcpy(len[o].data(), dLen, (size_t)N * sizeof(uint32_t), hipMemcpyDeviceToHost));
+            }
+            std::vector<uint32_t> start(N + 1, 0);
+            for(uint32_t i = 0; i < N; i++) {
+                uint64_t sum = start[i];
+                for(size_t o = 0; o < outs.size(); o++) { sum += len[o][i]; }
+                if(sum > 0xFFFFFFFFull) { return fail(GENNMI_EUNSUPPORTED, "runner_finalise: too many zero-delay synapses"); }
+                start[i + 1] = (uint32_t)sum;
+            }
+            uint32_t *dStart = nullptr, *dOffset = nullptr; ZeroDelayEntry *dEntries = nullptr;
+            HIP_TRY(devAlloc((void**)&dStart, (size_t)(N + 1) * sizeof(uint32_t)));
+            HIP_TRY(hipMemcpy(dStart, start.data(), (size_t)(N + 1) * sizeof(uint32_t), hipMemcpyHostToDevice));
+            HIP_TRY(devAlloc((void**)&dOffset, (size_t)N * sizeof(uint32_t)));
+            HIP_TRY(devAlloc((void**)&dEntries, (size_t)std::max(1u, start[N]) * sizeof(ZeroDelayEntry)));
+            std::vector<uint32_t> offset(start.begin(), start.begin() + N);
+            for(size_t o = 0; o < outs.size(); o++) {
+                auto &q = outs[o]->g;
+                HIP_TRY(hipMemcpy(dOffset, offset.data(), (size_t)N * sizeof(uint32_t), hipMemcpyHostToDevice));
+                zeroDelayScanKernel<<<grid, dim3(BLOCK), 0, 0>>>(N, q.rowStride, q.rowLength, q.d, q.maxDenDelay, q.ind, q.g, q.denDelay,
+                                                                 q.numTrgNeurons, nullptr, dOffset, dEntries);
+                HIP_TRY(hipGetLastError());
+                HIP_TRY(hipDeviceSynchronize());
+                for(uint32_t i = 0; i < N; i++) { offset[i] += len[o][i]; }
+                outs[o]->skipZeroDelay = 1; outs[o]->shadowSpk = n.shadowSpk; outs[o]->shadowCnt = n.shadowCnt;
+            }
+            n.zeroStart = dStart; n.zeroEntries = dEntries;
+        }
+        r->fusedStep = true;
+    }
     HIP_TRY(uploadPerBlock(r->neuron, r->neuronBlocks, &r->dNeuron));
     HIP_TRY(uploadPerBlock(r->pre, r->preBlocks, &r->dPre));
     HIP_TRY(uploadPerBlock(r->post, r->postBlocks, &r->dPost));
@@ -838,6 +996,24 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
     }
     HIP_TRY(hipGetLastError());
     return GENNMI_OK;
+}
+
+static int launchNeurons(gennmi_runner *r, const StepArgs &a, bool timed);
+
+static int launchFusedStep(gennmi_runner *r, const StepArgs &a)
+{
+    stepFusedKernel<<<dim3(r->neuronBlocks + r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(
+        r->dNeuron, r->neuronBlocks, r->dPre, a, r->dt, r->dAgg, r->dError, r->dEvents);
+    HIP_TRY(hipGetLastError());
+    return GENNMI_OK;
+}
+
+// one whole timestep: a single launch where the runner allows it, else synapse kernels then the neuron kernel
+static int launchStep(gennmi_runner *r, const StepArgs &a)
+{
+    if(r->fusedStep) { return launchFusedStep(r, a); }
+    const int rc = launchSynapses(r, a, false);
+    return rc ? rc : launchNeurons(r, a, false);
 }
 
 static int launchNeurons(gennmi_runner *r, const StepArgs &a, bool timed)
@@ -896,9 +1072,18 @@ int gennmi_step_time(gennmi_runner *r, unsigned long long timestep, unsigned lon
     if(!r) { return fail(GENNMI_EINVAL, "step_time: null runner"); }
     // const float t = timestep * DT  (generateRunner.cc:283)
     const float t = (float)timestep * r->dt;
+    const uint32_t recT = numRecordingTimesteps ? (uint32_t)(timestep % numRecordingTimesteps) : 0u;
+    if(r->finalised && r->fusedStep && !r->timing) {
+        StepArgs a{};
+        a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recT;
+        const int rc = launchFusedStep(r, a);
+        if(rc) { return rc; }
+        r->epoch++;
+        return GENNMI_OK;
+    }
     int rc = gennmi_update_synapses(r, t);
     if(rc) { return rc; }
-    return gennmi_update_neurons(r, t, numRecordingTimesteps ? (uint32_t)(timestep % numRecordingTimesteps) : 0u);
+    return gennmi_update_neurons(r, t, recT);
 }
 
 int gennmi_run_steps(gennmi_runner *r, unsigned long long timestep, unsigned long long numSteps, unsigned long long numRecordingTimesteps)
@@ -924,8 +1109,7 @@ int gennmi_run_steps(gennmi_runner *r, unsigned long long timestep, unsigned lon
             for(unsigned long long k = 0; k < CHUNK && rc == GENNMI_OK; k++) {
                 StepArgs a{};
                 a.base = r->dState; a.k = k;
-                rc = launchSynapses(r, a, false);
-                if(rc == GENNMI_OK) { rc = launchNeurons(r, a, false); }
+                rc = launchStep(r, a);
             }
             advanceStepKernel<<<dim3(1), dim3(64), 0, r->stream>>>(r->dState, CHUNK);
             const hipError_t ce = hipStreamEndCapture(r->stream, &graph);
@@ -942,8 +1126,7 @@ int gennmi_run_steps(gennmi_runner *r, unsigned long long timestep, unsigned lon
     for(; done < numSteps; done++) {
         StepArgs a{};
         a.base = r->dState; a.k = 0;
-        int rc = launchSynapses(r, a, false);
-        if(rc == GENNMI_OK) { rc = launchNeurons(r, a, false); }
+        const int rc = launchStep(r, a);
         if(rc) { return rc; }
         advanceStepKernel<<<dim3(1), dim3(64), 0, r->stream>>>(r->dState, 1);
         r->epoch++;
@@ -990,6 +1173,14 @@ int gennmi_runner_kernel_stats(gennmi_runner *r, unsigned long long *presynLaunc
     if(presynSeconds) { *presynSeconds = r->preTime; }
     if(neuronLaunches) { *neuronLaunches = r->neuronLaunches; }
     if(neuronSeconds) { *neuronSeconds = r->neuronTime; }
+    return GENNMI_OK;
+}
+
+int gennmi_runner_get_info(gennmi_runner *r, uint32_t info[4])
+{
+    if(!r || !info) { return fail(GENNMI_EINVAL, "runner_get_info: null argument"); }
+    if(!r->finalised) { return fail(GENNMI_ESTATE, "runner_get_info: runner not finalised"); }
+    info[0] = r->fusedStep ? 1u : 0u; info[1] = r->neuronBlocks; info[2] = r->preBlocks; info[3] = r->postBlocks;
     return GENNMI_OK;
 }
 

@@ -645,6 +645,11 @@ class GeNNModel:
         _abi.check(_abi.load().gennmi_runner_kernel_stats(self._runner, C.byref(a), C.byref(b), C.byref(c), C.byref(d)))
         return {"presyn_launches": a.value, "presyn_seconds": b.value, "neuron_launches": c.value, "neuron_seconds": d.value}
 
+    def runner_info(self):
+        info = (C.c_uint32 * 4)()
+        _abi.check(_abi.load().gennmi_runner_get_info(self._runner, C.byref(info)))
+        return {"single_launch_step": bool(info[0]), "neuron_blocks": info[1], "presyn_blocks": info[2], "postsyn_blocks": info[3]}
+
     def set_timing(self, enabled):
         _abi.check(_abi.load().gennmi_runner_set_timing(self._runner, int(bool(enabled))))
 

@@ -200,7 +200,14 @@ int gennmi_runner_get_times(gennmi_runner *runner, double *neuronUpdateTime, dou
 /* Launch counts and average HIP-event duration of the presynaptic kernel since the last reset. */
 int gennmi_runner_kernel_stats(gennmi_runner *runner, unsigned long long *presynLaunches, double *presynSeconds,
                                unsigned long long *neuronLaunches, double *neuronSeconds);
-/* Synaptic events processed so far per presynaptic group (device counter, enabled with timing). */
+/* Launch plan chosen by gennmi_runner_finalise: info[0] = 1 if a whole timestep is one launch (all projections go
+ * through a dendritic-delay ring; synapses with d % D == 0 are then delivered by the spiking neuron one launch
+ * earlier, into the slot read in the next step — the visible difference is the content of that one ring slot
+ * between steps; GENNMI_FUSED_STEP=0 in the environment keeps the reference's placement), info[1..3] = blocks of
+ * the neuron, presynaptic and postsynaptic kernels.  The reference logs the analogous choice of presynaptic
+ * strategy (backendSIMT.cc:736). */
+int gennmi_runner_get_info(gennmi_runner *runner, uint32_t info[4]);
+/* Synaptic events processed so far, summed over presynaptic groups (device counter). */
 int gennmi_runner_event_count(gennmi_runner *runner, unsigned long long *events);
 
 #ifdef __cplusplus

@@ -68,7 +68,16 @@ def compare_state(net, model, oracle, where, exact):
         if sg.fused_ps_target is sg:
             assert_close(sg.vars["outPost"].pull_from_device(), oracle.out_post(s.name), f"{where}: outPost of {s.name}", exact, accumulator=True)
             if "denDelay" in sg.vars:
-                assert_close(sg.vars["denDelay"].pull_from_device(), oracle.den_delay(s.name), f"{where}: denDelay of {s.name}", exact, accumulator=True)
+                got, want = sg.vars["denDelay"].pull_from_device().copy(), oracle.den_delay(s.name).copy()
+                if model.runner_info()["single_launch_step"]:
+                    # zero-delay synapses of the last step's spikes already sit in the slot that will be read next
+                    # (the reference adds them at the start of the next step): leave that slot out here; the
+                    # neuron state compared above depends on every slot's total
+                    D, n = s.max_den_delay, net.pop(s.trg).n
+                    nxt = (model.timestep + 1) % D
+                    got.reshape(D, n)[nxt] = 0
+                    want.reshape(D, n)[nxt] = 0
+                assert_close(got, want, f"{where}: denDelay of {s.name}", exact, accumulator=True)
         if s.wum == "stdp_trace":
             assert_close(sg.vars["g"].pull_from_device(), oracle.syn_g(s.name), f"{where}: g of {s.name}", exact)
             assert_close(sg.vars["preTrace"].pull_from_device(), oracle.pre_trace(s.src), f"{where}: preTrace of {s.name}", exact)

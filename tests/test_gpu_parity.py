@@ -38,7 +38,19 @@ def test_microcircuit_dendritic_delay():
     rasters must be identical for the first 100 ms (1000 steps), state within 1e-5."""
     net = configs.potjans(neuron_scale=0.05, connectivity_scale=1.0, steps=1000)
     model, oracle, counts = run_side_by_side(net, check_every=100, exact=False, exact_steps=1000)
+    assert model.runner_info()["single_launch_step"]
     assert sum(counts.values()) > 500
+    model.unload()
+
+
+def test_microcircuit_two_launch_step(monkeypatch):
+    """Same network with the single-launch step switched off: synapse and neuron kernels run back to back and
+    every ring slot must match the oracle, including the one read next."""
+    monkeypatch.setenv("GENNMI_FUSED_STEP", "0")
+    net = configs.potjans(neuron_scale=0.05, connectivity_scale=1.0, steps=300)
+    model, oracle, counts = run_side_by_side(net, check_every=50, exact=False, exact_steps=300)
+    assert not model.runner_info()["single_launch_step"]
+    assert sum(counts.values()) > 100
     model.unload()
 
 
@@ -153,6 +165,40 @@ def test_graph_replay_matches_stepping():
     t, ids = graph.neuron_populations["E"].spike_recording_data[0]
     assert len(ids) > 500
     assert graph.synaptic_event_count == eager.synaptic_event_count
+    graph.unload()
+    eager.unload()
+
+
+def test_graph_replay_single_launch_step():
+    """Graph replay of the one-launch-per-step plan (dendritic-delay network) against eager stepping and the oracle:
+    rasters identical, membrane potentials within tolerance (weights differ, so atomic order may differ)."""
+    net = configs.potjans(neuron_scale=0.04, connectivity_scale=1.0, steps=450)
+    eager = model_from_net(net)
+    eager.load(num_recording_timesteps=net.steps)
+    graph = model_from_net(net)
+    graph.load(num_recording_timesteps=net.steps)
+    assert graph.runner_info()["single_launch_step"]
+    oracle = OracleNet(net, num_recording_timesteps=net.steps)
+    for chunk in (200, 50, 200):
+        graph.run(chunk)
+        graph.synchronize()
+        for _ in range(chunk):
+            eager.step_time()
+        oracle.run(chunk)
+        for p in net.pops:
+            want = oracle.var(p.name, 0)
+            for m in (graph, eager):
+                np.testing.assert_allclose(m.neuron_populations[p.name].vars["V"].pull_from_device(), want, rtol=1e-5)
+    graph.pull_recording_buffers_from_device()
+    eager.pull_recording_buffers_from_device()
+    spikes = 0
+    for p in net.pops:
+        want = oracle.record(p.name, net.steps)
+        assert np.array_equal(graph.neuron_populations[p.name].vars["recordSpk"].view, want)
+        assert np.array_equal(eager.neuron_populations[p.name].vars["recordSpk"].view, want)
+        spikes += int(np.unpackbits(want.view(np.uint8)).sum())
+    assert spikes > 200
+    assert graph.synaptic_event_count == eager.synaptic_event_count == oracle.events()
     graph.unload()
     eager.unload()
 
