@@ -51,7 +51,7 @@ def main():
     ap.add_argument("--workload", default="potjans")
     ap.add_argument("--cpu-steps", type=int, default=None, help="steps of the CPU baseline sample (default: sized for ~10-20 s)")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--profile-steps", type=int, default=2000, help="eager steps with HIP events around every kernel")
+    ap.add_argument("--profile-steps", type=int, default=2000, help="extra steps replayed with HIP event nodes around every kernel (multiple of 100)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
@@ -91,28 +91,39 @@ def main():
         _, ids = model.neuron_populations[p.name].spike_recording_data[0]
         rates[p.name] = round(len(ids) / p.n / ((args.warmup + args.steps) * net.dt / 1000.0), 3)
 
-    # ---- per-kernel durations: eager stepping with HIP events around each launch on the runner's stream
+    # ---- per-kernel durations: the same graph replay with HIP event nodes between the kernels of every step
+    # (events on the runner's stream; durations are those of back-to-back execution)
     roofline = None
+    info = model.runner_info()
     if args.profile_steps > 0:
-        model.num_recording_timesteps = None
         model.set_timing(True)
         evp0 = model.synaptic_event_count
-        for _ in range(args.profile_steps):
-            model.step_time()
+        model.run(args.profile_steps)
         model.synchronize()
         st = model.kernel_stats()
         evp = model.synaptic_event_count - evp0
         model.set_timing(False)
-        if st["presyn_launches"]:
+        bpe = bytes_per_event or max(BYTES_PER_EVENT[k] for k in kinds)
+        neuron_bytes = sum(p.n * (0 if p.model == "ssa" else 32) for p in net.pops)     # 32 B per LIF/Izhikevich update (state + one PSM)
+        if info["single_launch_step"] and st["step_launches"]:
+            avg_s = st["step_seconds"] / st["step_launches"]
+            ev_per_launch = evp / st["step_launches"]
+            achieved = (ev_per_launch * bpe + neuron_bytes) / avg_s / 1e9
+            roofline = {"bound": "hbm", "kernel": "stepFusedKernel (presynaptic + neuron update of one timestep)",
+                        "achieved": round(achieved, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6),
+                        "traffic": None, "bytes_per_event": bpe, "events_per_launch": round(ev_per_launch, 1),
+                        "neuron_bytes_per_launch": neuron_bytes, "avg_launch_us": round(avg_s * 1e6, 3)}
+        elif st["presyn_launches"]:
             avg_s = st["presyn_seconds"] / st["presyn_launches"]
             ev_per_launch = evp / st["presyn_launches"]
-            bpe = bytes_per_event or max(BYTES_PER_EVENT[k] for k in kinds)
             achieved = ev_per_launch * bpe / avg_s / 1e9
-            roofline = {"bound": "hbm", "kernel": "presynapticUpdateKernel", "achieved": round(achieved, 3), "peak": HBM_PEAK_GBS,
-                        "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6), "traffic": None,
+            navg = st["neuron_seconds"] / max(1, st["neuron_launches"])
+            roofline = {"bound": "hbm", "kernel": "presynapticUpdateKernel (+ presynapticTileKernel)", "achieved": round(achieved, 3),
+                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6), "traffic": None,
                         "bytes_per_event": bpe, "events_per_launch": round(ev_per_launch, 1), "avg_launch_us": round(avg_s * 1e6, 3),
-                        "neuron_kernel_avg_us": round(st["neuron_seconds"] / max(1, st["neuron_launches"]) * 1e6, 3),
-                        "neuron_kernel_gbs": round(num_neurons * 32 / (st["neuron_seconds"] / max(1, st["neuron_launches"])) / 1e9, 3)}
+                        "neuron_kernel_avg_us": round(navg * 1e6, 3), "neuron_kernel_gbs": round(neuron_bytes / navg / 1e9, 3)}
+            if st["postsyn_launches"]:
+                roofline["postsyn_kernel_avg_us"] = round(st["postsyn_seconds"] / st["postsyn_launches"] * 1e6, 3)
     model.unload()
 
     # ---- CPU baseline: the single-threaded oracle on the same network, bounded sample from t = 0
@@ -142,7 +153,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall / args.steps * 1e3, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": label, "neurons": num_neurons, "synapses": num_synapses, "dt_ms": net.dt, "seed": net.seed,
-                   "stepping": "hipGraph replay, 100 steps per graph"},
+                   "stepping": "hipGraph replay, 100 steps per graph, " + ("1 launch per step" if info["single_launch_step"] else "2-3 launches per step")},
         "gsop_per_s": round(events / wall / 1e9, 4),
         "neuron_updates_per_s": round(num_neurons * args.steps / wall, 1),
         "wall_s_per_sim_s": round(wall / sim_s, 4),

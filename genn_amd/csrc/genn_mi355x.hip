@@ -116,9 +116,22 @@ struct PreGroupDev
     uint32_t lanesPerSpike;             // power of two, 1..64
     uint32_t vec4;                      // rows are 16-byte aligned and padded: dwordx4 loads
     int32_t convBH, convBW;
-    uint32_t skipZeroDelay, pad_;       // synapses with d % D == 0 are delivered by the neuron update instead
+    uint32_t skipZeroDelay;             // synapses with d % D == 0 are delivered by the neuron update instead
+    uint32_t tileThreshold;             // != 0: leave the step to the tile kernel when numSpikes*rowStride reaches it
     const uint32_t *shadowSpk;          // the source population's shadow queue (read instead of srcSpk when set)
     const uint32_t *shadowCnt;
+};
+
+// Dense-activity path of a static SPARSE projection without delay: one block accumulates the events that
+// fall into one tile of postsynaptic neurons in LDS and flushes the tile with lane-consecutive atomics.
+struct TileGroupDev
+{
+    gennmi_presynaptic_update_group_t g;
+    const uint16_t *tileOff;            // [numSrc*(numTiles+1)] first position of every row whose target is >= tile*tileSize
+    uint32_t numTiles, tileSize;
+    uint32_t tile, split, numSplits;    // this block: which tile, which share of the spikes
+    uint32_t lanes;                     // lanes per (spike, tile) segment, power of two
+    uint32_t threshold, pad_;
 };
 
 struct PostGroupDev
@@ -174,6 +187,7 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
     GLOBAL_AS const uint32_t *spk = G.shadowSpk ? asGlobal(G.shadowSpk) + ((size_t)parity * gridDim.y + batch) * g.numSrcNeurons
                                                 : asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
     const uint32_t numSpikes = cntPtr[batch];
+    if(G.tileThreshold && (unsigned long long)numSpikes * g.rowStride >= G.tileThreshold) { return; }
     GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
     unsigned long long events = 0;
 
@@ -300,6 +314,76 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
     // one counter update per wave
     for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
     if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Tile kernel.  Scattered fp32 atomics cost one memory transaction each (≈20 G/s measured on this part,
+// whatever the array size), lane-consecutive ones ≈280 G/s.  When a step carries enough events
+// (numSpikes*rowStride >= numTrg), a block therefore owns a tile of postsynaptic neurons in LDS: it walks
+// its share of the spike list, reads only the segment of each row that falls into its tile (rows are
+// sorted by target; tileOff holds the segment boundaries), adds into LDS, and finally flushes the tile
+// with consecutive lanes on consecutive addresses.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(BLOCK)
+void presynapticTileKernel(const TileGroupDev *blocks, unsigned long long *eventCounter)
+{
+    extern __shared__ float shTile[];
+    const TileGroupDev &G = blocks[blockIdx.x];
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
+    if((unsigned long long)numSpikes * g.rowStride < G.threshold) { return; }      // the scatter kernel took this step
+    const uint32_t tileStart = G.tile * G.tileSize;
+    const uint32_t tileLen = min(G.tileSize, g.numTrgNeurons - tileStart);
+    for(uint32_t k = threadIdx.x; k < tileLen; k += BLOCK) { shTile[k] = 0.0f; }
+    __syncthreads();
+
+    GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    GLOBAL_AS const uint16_t *off = asGlobal(G.tileOff);
+    GLOBAL_AS const uint32_t *ind = asGlobal(g.ind);
+    GLOBAL_AS const float *weight = asGlobal(g.g);
+    const uint32_t L = G.lanes;
+    const uint32_t lis = threadIdx.x & (L - 1);
+    const uint32_t perBlock = BLOCK / L;
+    const uint32_t stride = perBlock * G.numSplits;
+    unsigned long long events = 0;
+    for(uint32_t s = G.split * perBlock + threadIdx.x / L; s < numSpikes; s += stride) {
+        const uint32_t idPre = spk[s];
+        const size_t o = (size_t)idPre * (G.numTiles + 1) + G.tile;
+        const uint32_t a = off[o], b = off[o + 1];
+        const size_t rowBase = (size_t)idPre * g.rowStride;
+        for(uint32_t j = a + lis; j < b; j += L) {
+            unsafeAtomicAdd(&shTile[ind[rowBase + j] - tileStart], weight[rowBase + j]);
+        }
+        if(lis == 0) { events += b - a; }
+    }
+    __syncthreads();
+    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons + tileStart;
+    for(uint32_t k = threadIdx.x; k < tileLen; k += BLOCK) {
+        const float v = shTile[k];
+        if(v != 0.0f) { atomicAddF32(&outPost[k], v); }
+    }
+    for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
+    if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// Segment boundaries of every row for the tile kernel; also verifies that rows are sorted by target.
+__global__ void tileOffsetKernel(uint32_t numSrc, uint32_t rowStride, const uint32_t *rowLength, const uint32_t *ind,
+                                 uint32_t tileSize, uint32_t numTiles, uint16_t *off, uint32_t *unsorted)
+{
+    const uint32_t row = blockIdx.x * blockDim.x + threadIdx.x;
+    if(row >= numSrc) { return; }
+    const uint32_t len = rowLength[row];
+    const uint32_t *r = ind + (size_t)row * rowStride;
+    uint16_t *o = off + (size_t)row * (numTiles + 1);
+    uint32_t t = 0, prev = 0;
+    for(uint32_t j = 0; j < len; j++) {
+        const uint32_t p = r[j];
+        if(p < prev) { atomicOr(unsorted, 1u); }
+        prev = p;
+        while(t <= numTiles && (unsigned long long)t * tileSize <= p) { o[t++] = (uint16_t)j; }
+    }
+    while(t <= numTiles) { o[t++] = (uint16_t)len; }
 }
 
 __global__ __launch_bounds__(BLOCK)
@@ -652,14 +736,17 @@ struct gennmi_runner
     unsigned long long epoch = 0;       // completed steps (host mirror)
     bool synapsesDone = false;          // updateSynapses ran for the current step
     bool fusedStep = false;             // zero-delay synapses are delivered by the neuron update; one launch per step
+    TileGroupDev *dTile = nullptr; uint32_t tileBlocks = 0, tileFloats = 0;
     std::vector<void*> owned;           // engine-private device allocations (shadow queues, zero-delay lists)
     // graph
     hipGraphExec_t graphExec = nullptr; unsigned long long graphSteps = 0;
     // timing
     bool timing = false;
-    hipEvent_t evA = nullptr, evB = nullptr, evC = nullptr, evD = nullptr;
     double neuronTime = 0, preTime = 0, postTime = 0;
-    unsigned long long preLaunches = 0, neuronLaunches = 0;
+    unsigned long long preLaunches = 0, neuronLaunches = 0, postLaunches = 0, stepLaunches = 0;
+    double stepTime = 0;                // single-launch steps
+    struct Pending { hipEvent_t a, b; int kind; };          // kind: 0 presynaptic, 1 postsynaptic, 2 neuron, 3 single-launch step
+    std::vector<hipEvent_t> eventPool; size_t eventNext = 0; std::vector<Pending> pending;
 };
 
 extern "C" {
@@ -743,8 +830,9 @@ int gennmi_runner_destroy(gennmi_runner *r)
     if(!r) { return GENNMI_OK; }
     hipStreamSynchronize(r->stream);
     if(r->graphExec) { hipGraphExecDestroy(r->graphExec); }
-    for(hipEvent_t e : {r->evA, r->evB, r->evC, r->evD}) { if(e) { hipEventDestroy(e); } }
+    for(hipEvent_t e : r->eventPool) { hipEventDestroy(e); }
     for(void *q : r->owned) { hipFree(q); }
+    hipFree(r->dTile);
     hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dAgg); hipFree(r->dError); hipFree(r->dEvents); hipFree(r->dState);
     hipStreamDestroy(r->stream);
     delete r;
@@ -910,6 +998,51 @@ int gennmi_runner_finalise(gennmi_runner *r)
         if(e != hipSuccess) { return e; }
         return hipMemcpy(*dTable, table.data(), table.size() * sizeof(table[0]), hipMemcpyHostToDevice);
     };
+    // ---- tile path for static, delay-free SPARSE projections whose rows are sorted by target
+    {
+        const char *envTile = getenv("GENNMI_TILE_FLOATS");
+        const uint32_t tileFloats = envTile ? (uint32_t)std::max(0, atoi(envTile)) : 8192u;
+        std::vector<TileGroupDev> tiles;
+        for(auto &p : r->pre) {
+            if(tileFloats == 0 || p.g.matrix != GENNMI_MATRIX_SPARSE || p.g.wum != GENNMI_WUM_STATIC_PULSE || p.g.rowStride > 65535) { continue; }
+            const uint32_t tileSize = std::min(tileFloats, p.g.numTrgNeurons);
+            const uint32_t numTiles = (p.g.numTrgNeurons + tileSize - 1) / tileSize;
+            uint16_t *dOff = nullptr; uint32_t *dFlag = nullptr;
+            HIP_TRY(hipMalloc(&dOff, (size_t)p.g.numSrcNeurons * (numTiles + 1) * sizeof(uint16_t)));
+            r->owned.push_back(dOff);
+            HIP_TRY(hipMalloc(&dFlag, sizeof(uint32_t)));
+            HIP_TRY(hipMemset(dFlag, 0, sizeof(uint32_t)));
+            tileOffsetKernel<<<dim3((p.g.numSrcNeurons + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, 0>>>(
+                p.g.numSrcNeurons, p.g.rowStride, p.g.rowLength, p.g.ind, tileSize, numTiles, dOff, dFlag);
+            HIP_TRY(hipGetLastError());
+            uint32_t unsorted = 0;
+            HIP_TRY(hipMemcpy(&unsorted, dFlag, sizeof(uint32_t), hipMemcpyDeviceToHost));
+            HIP_TRY(hipFree(dFlag));
+            if(unsorted) { continue; }          // rows not sorted by target: the scatter kernel handles every step
+            p.tileThreshold = std::max(1u, p.g.numTrgNeurons);
+            const char *envSplit = getenv("GENNMI_TILE_BLOCKS_PER_CU");
+            const uint32_t blocksPerCUTile = envSplit ? (uint32_t)std::max(1, atoi(envSplit)) : 2u;
+            const uint32_t numSplits = std::max(1u, std::min(256u, (blocksPerCUTile * numCU) / numTiles));
+            const uint32_t avgSeg = std::max(1u, p.g.rowStride / numTiles);
+            TileGroupDev t{};
+            t.g = p.g; t.tileOff = dOff; t.numTiles = numTiles; t.tileSize = tileSize; t.numSplits = numSplits;
+            t.lanes = std::min<uint32_t>(WAVE, pow2Ceil((avgSeg + 1) / 2)); t.threshold = p.tileThreshold;
+            for(uint32_t tile = 0; tile < numTiles; tile++) {
+                for(uint32_t split = 0; split < numSplits; split++) { t.tile = tile; t.split = split; tiles.push_back(t); }
+            }
+            r->tileFloats = std::max(r->tileFloats, tileSize);
+        }
+        if(!tiles.empty()) {
+            HIP_TRY(hipMalloc(&r->dTile, tiles.size() * sizeof(TileGroupDev)));
+            HIP_TRY(hipMemcpy(r->dTile, tiles.data(), tiles.size() * sizeof(TileGroupDev), hipMemcpyHostToDevice));
+            r->tileBlocks = (uint32_t)tiles.size();
+            if((size_t)r->tileFloats * sizeof(float) > 48 * 1024) {
+                HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(presynapticTileKernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            (int)(r->tileFloats * sizeof(float))));
+            }
+        }
+    }
+
     // ---- single-launch step: possible when every projection is a SPARSE dendritic-delay one with ring depth >= 2
     // and nothing is plastic
     const char *envFused = getenv("GENNMI_FUSED_STEP");
@@ -983,16 +1116,55 @@ int gennmi_runner_finalise(gennmi_runner *r)
     return GENNMI_OK;
 }
 
+// Timing: events are taken from a pool and recorded on the runner's stream around each kernel; elapsed times are
+// only read (after one synchronisation) when the pool is full or statistics are requested.
+static int drainTimers(gennmi_runner *r)
+{
+    if(r->pending.empty()) { return GENNMI_OK; }
+    HIP_TRY(hipStreamSynchronize(r->stream));
+    for(const auto &p : r->pending) {
+        float ms = 0;
+        HIP_TRY(hipEventElapsedTime(&ms, p.a, p.b));
+        const double sec = ms * 1e-3;
+        if(p.kind == 0) { r->preTime += sec; r->preLaunches++; }
+        else if(p.kind == 1) { r->postTime += sec; r->postLaunches++; }
+        else if(p.kind == 2) { r->neuronTime += sec; r->neuronLaunches++; }
+        else { r->stepTime += sec; r->stepLaunches++; }
+    }
+    r->pending.clear();
+    r->eventNext = 0;
+    return GENNMI_OK;
+}
+
+static int stamp(gennmi_runner *r, hipEvent_t *out)
+{
+    if(r->eventNext == r->eventPool.size()) {
+        hipEvent_t e;
+        HIP_TRY(hipEventCreate(&e));
+        r->eventPool.push_back(e);
+    }
+    *out = r->eventPool[r->eventNext++];
+    HIP_TRY(hipEventRecord(*out, r->stream));
+    return GENNMI_OK;
+}
+
 static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
 {
-    if(timed) { HIP_TRY(hipEventRecord(r->evA, r->stream)); }
+    hipEvent_t e0 = nullptr, e1 = nullptr, e2 = nullptr;
+    if(timed) {
+        if(r->pending.size() >= 2048) { const int rc = drainTimers(r); if(rc) { return rc; } }
+        const int rc = stamp(r, &e0); if(rc) { return rc; }
+    }
     if(!r->pre.empty()) {
         presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dPre, a, r->dt, r->dEvents);
-        if(timed) { HIP_TRY(hipEventRecord(r->evB, r->stream)); }
+        if(r->tileBlocks) {
+            presynapticTileKernel<<<dim3(r->tileBlocks, r->batch), dim3(BLOCK), r->tileFloats * sizeof(float), r->stream>>>(r->dTile, r->dEvents);
+        }
+        if(timed) { const int rc = stamp(r, &e1); if(rc) { return rc; } r->pending.push_back({e0, e1, 0}); }
     }
     if(!r->post.empty()) {
         postsynapticUpdateKernel<<<dim3(r->postBlocks), dim3(BLOCK), 0, r->stream>>>(r->dPost, a, r->dt);
-        if(timed) { HIP_TRY(hipEventRecord(r->evC, r->stream)); }
+        if(timed) { const int rc = stamp(r, &e2); if(rc) { return rc; } r->pending.push_back({e1 ? e1 : e0, e2, 1}); }
     }
     HIP_TRY(hipGetLastError());
     return GENNMI_OK;
@@ -1018,9 +1190,10 @@ static int launchStep(gennmi_runner *r, const StepArgs &a)
 
 static int launchNeurons(gennmi_runner *r, const StepArgs &a, bool timed)
 {
-    if(timed) { HIP_TRY(hipEventRecord(r->evC, r->stream)); }
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if(timed) { const int rc = stamp(r, &e0); if(rc) { return rc; } }
     neuronUpdateKernel<<<dim3(r->neuronBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dNeuron, a, r->dt, r->dAgg, r->dError);
-    if(timed) { HIP_TRY(hipEventRecord(r->evD, r->stream)); }
+    if(timed) { const int rc = stamp(r, &e1); if(rc) { return rc; } r->pending.push_back({e0, e1, 2}); }
     HIP_TRY(hipGetLastError());
     return GENNMI_OK;
 }
@@ -1032,19 +1205,6 @@ int gennmi_update_synapses(gennmi_runner *r, float t)
     a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = 0;
     const int rc = launchSynapses(r, a, r->timing);
     if(rc) { return rc; }
-    if(r->timing) {
-        float ms = 0;
-        if(!r->pre.empty()) {
-            HIP_TRY(hipEventSynchronize(r->evB));
-            HIP_TRY(hipEventElapsedTime(&ms, r->evA, r->evB));
-            r->preTime += ms * 1e-3; r->preLaunches++;
-        }
-        if(!r->post.empty()) {
-            HIP_TRY(hipEventSynchronize(r->evC));
-            HIP_TRY(hipEventElapsedTime(&ms, r->pre.empty() ? r->evA : r->evB, r->evC));
-            r->postTime += ms * 1e-3;
-        }
-    }
     r->synapsesDone = true;
     return GENNMI_OK;
 }
@@ -1056,12 +1216,6 @@ int gennmi_update_neurons(gennmi_runner *r, float t, uint32_t recordingTimestep)
     a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recordingTimestep;
     const int rc = launchNeurons(r, a, r->timing);
     if(rc) { return rc; }
-    if(r->timing) {
-        float ms = 0;
-        HIP_TRY(hipEventSynchronize(r->evD));
-        HIP_TRY(hipEventElapsedTime(&ms, r->evC, r->evD));
-        r->neuronTime += ms * 1e-3; r->neuronLaunches++;
-    }
     r->epoch++;
     r->synapsesDone = false;
     return GENNMI_OK;
@@ -1073,11 +1227,17 @@ int gennmi_step_time(gennmi_runner *r, unsigned long long timestep, unsigned lon
     // const float t = timestep * DT  (generateRunner.cc:283)
     const float t = (float)timestep * r->dt;
     const uint32_t recT = numRecordingTimesteps ? (uint32_t)(timestep % numRecordingTimesteps) : 0u;
-    if(r->finalised && r->fusedStep && !r->timing) {
+    if(r->finalised && r->fusedStep) {
         StepArgs a{};
         a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recT;
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        if(r->timing) {
+            if(r->pending.size() >= 2048) { const int rc = drainTimers(r); if(rc) { return rc; } }
+            const int rc = stamp(r, &e0); if(rc) { return rc; }
+        }
         const int rc = launchFusedStep(r, a);
         if(rc) { return rc; }
+        if(r->timing) { const int rc2 = stamp(r, &e1); if(rc2) { return rc2; } r->pending.push_back({e0, e1, 3}); }
         r->epoch++;
         return GENNMI_OK;
     }
@@ -1090,17 +1250,19 @@ int gennmi_run_steps(gennmi_runner *r, unsigned long long timestep, unsigned lon
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "run_steps: runner not finalised"); }
     constexpr unsigned long long CHUNK = 100;
-    if(r->timing) {
-        for(unsigned long long s = 0; s < numSteps; s++) {
-            const int rc = gennmi_step_time(r, timestep + s, numRecordingTimesteps);
-            if(rc) { return rc; }
-        }
-        return GENNMI_OK;
-    }
     const StepState hs{timestep, r->epoch, numRecordingTimesteps};
     HIP_TRY(hipMemcpyAsync(r->dState, &hs, sizeof(hs), hipMemcpyHostToDevice, r->stream));
     HIP_TRY(hipStreamSynchronize(r->stream));   // hs lives on this stack frame
     unsigned long long done = 0;
+    if(r->timing) {
+        // individually launched steps with HIP events around every kernel; nothing waits until the statistics
+        // are read, so the device stays busy and the clocks stay up
+        for(; done < numSteps; done++) {
+            const int rc = gennmi_step_time(r, timestep + done, numRecordingTimesteps);
+            if(rc) { return rc; }
+        }
+        return GENNMI_OK;
+    }
     while(numSteps - done >= CHUNK) {
         if(!r->graphExec) {
             hipGraph_t graph;
@@ -1148,10 +1310,7 @@ int gennmi_runner_synchronize(gennmi_runner *r)
 int gennmi_runner_set_timing(gennmi_runner *r, int enabled)
 {
     if(!r) { return fail(GENNMI_EINVAL, "runner_set_timing: null runner"); }
-    if(enabled && !r->evA) {
-        HIP_TRY(hipEventCreate(&r->evA)); HIP_TRY(hipEventCreate(&r->evB));
-        HIP_TRY(hipEventCreate(&r->evC)); HIP_TRY(hipEventCreate(&r->evD));
-    }
+    if(!enabled) { const int rc = drainTimers(r); if(rc) { return rc; } }
     r->timing = (enabled != 0);
     return GENNMI_OK;
 }
@@ -1159,20 +1318,21 @@ int gennmi_runner_set_timing(gennmi_runner *r, int enabled)
 int gennmi_runner_get_times(gennmi_runner *r, double *neuronUpdateTime, double *presynapticUpdateTime, double *postsynapticUpdateTime)
 {
     if(!r) { return fail(GENNMI_EINVAL, "runner_get_times: null runner"); }
+    { const int rc = drainTimers(r); if(rc) { return rc; } }
     if(neuronUpdateTime) { *neuronUpdateTime = r->neuronTime; }
     if(presynapticUpdateTime) { *presynapticUpdateTime = r->preTime; }
     if(postsynapticUpdateTime) { *postsynapticUpdateTime = r->postTime; }
     return GENNMI_OK;
 }
 
-int gennmi_runner_kernel_stats(gennmi_runner *r, unsigned long long *presynLaunches, double *presynSeconds,
-                               unsigned long long *neuronLaunches, double *neuronSeconds)
+int gennmi_runner_kernel_stats(gennmi_runner *r, double stats[8])
 {
-    if(!r) { return fail(GENNMI_EINVAL, "runner_kernel_stats: null runner"); }
-    if(presynLaunches) { *presynLaunches = r->preLaunches; }
-    if(presynSeconds) { *presynSeconds = r->preTime; }
-    if(neuronLaunches) { *neuronLaunches = r->neuronLaunches; }
-    if(neuronSeconds) { *neuronSeconds = r->neuronTime; }
+    if(!r || !stats) { return fail(GENNMI_EINVAL, "runner_kernel_stats: null argument"); }
+    { const int rc = drainTimers(r); if(rc) { return rc; } }
+    stats[0] = (double)r->preLaunches; stats[1] = r->preTime;
+    stats[2] = (double)r->neuronLaunches; stats[3] = r->neuronTime;
+    stats[4] = (double)r->postLaunches; stats[5] = r->postTime;
+    stats[6] = (double)r->stepLaunches; stats[7] = r->stepTime;
     return GENNMI_OK;
 }
 

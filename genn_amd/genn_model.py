@@ -640,10 +640,10 @@ class GeNNModel:
         return int(v.value)
 
     def kernel_stats(self):
-        a, b = C.c_ulonglong(), C.c_double()
-        c, d = C.c_ulonglong(), C.c_double()
-        _abi.check(_abi.load().gennmi_runner_kernel_stats(self._runner, C.byref(a), C.byref(b), C.byref(c), C.byref(d)))
-        return {"presyn_launches": a.value, "presyn_seconds": b.value, "neuron_launches": c.value, "neuron_seconds": d.value}
+        st = (C.c_double * 8)()
+        _abi.check(_abi.load().gennmi_runner_kernel_stats(self._runner, C.byref(st)))
+        return {"presyn_launches": int(st[0]), "presyn_seconds": st[1], "neuron_launches": int(st[2]), "neuron_seconds": st[3],
+                "postsyn_launches": int(st[4]), "postsyn_seconds": st[5], "step_launches": int(st[6]), "step_seconds": st[7]}
 
     def runner_info(self):
         info = (C.c_uint32 * 4)()

@@ -197,9 +197,11 @@ int gennmi_runner_synchronize(gennmi_runner *runner);
 int gennmi_runner_set_timing(gennmi_runner *runner, int enabled);
 int gennmi_runner_get_times(gennmi_runner *runner, double *neuronUpdateTime, double *presynapticUpdateTime,
                             double *postsynapticUpdateTime);
-/* Launch counts and average HIP-event duration of the presynaptic kernel since the last reset. */
-int gennmi_runner_kernel_stats(gennmi_runner *runner, unsigned long long *presynLaunches, double *presynSeconds,
-                               unsigned long long *neuronLaunches, double *neuronSeconds);
+/* Launch counts and summed HIP-event durations (seconds) since the runner was created, measured while timing is
+ * enabled: stats = {presynaptic launches, seconds, neuron launches, seconds, postsynaptic launches, seconds,
+ * single-launch steps, seconds}.  Events are recorded on the runner's stream around every kernel and only read
+ * (after one synchronisation) when statistics are requested, so timed stepping does not idle the device. */
+int gennmi_runner_kernel_stats(gennmi_runner *runner, double stats[8]);
 /* Launch plan chosen by gennmi_runner_finalise: info[0] = 1 if a whole timestep is one launch (all projections go
  * through a dendritic-delay ring; synapses with d % D == 0 are then delivered by the spiking neuron one launch
  * earlier, into the slot read in the next step — the visible difference is the content of that one ring slot

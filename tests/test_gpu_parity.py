@@ -54,6 +54,30 @@ def test_microcircuit_two_launch_step(monkeypatch):
     model.unload()
 
 
+@pytest.mark.parametrize("tile_floats", ["8192", "600", "64"])
+def test_dense_activity_tile_path(tile_floats, monkeypatch):
+    """Steps that carry at least one event per target are handled by the tile kernel (LDS accumulation per tile
+    of postsynaptic neurons).  Integer-valued weights and DeltaCurr input make every fp32 sum exact in any
+    order, so the whole trajectory must be bit-identical to the oracle; tile sizes that do and do not divide the
+    population, and multapses, are covered."""
+    from genn_amd.netspec import Net, Pop, Syn
+    from genn_amd import netgen
+    monkeypatch.setenv("GENNMI_TILE_FLOATS", tile_floats)
+    n, m, fan = 3000, 1111, 40
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.7, TauRefrac=2.0)
+    net = Net(name="dense", dt=1.0, steps=80)
+    v0 = (-60.0 + 10.0 * np.linspace(0, 1, n)).astype(np.float32)
+    net.pops.append(Pop("A", "lif", n, dict(lif), {"V": v0, "RefracTime": np.zeros(n, np.float32)}))
+    net.pops.append(Pop("B", "lif", m, dict(lif, Ioffset=0.0), {"V": np.full(m, -60.0, np.float32), "RefracTime": np.zeros(m, np.float32)}))
+    rl, ind = netgen.fixed_number_post(11, 3, n, m, fan)
+    g = np.round(netgen.rows_uniform(11, 4, rl, fan, n, 3.0, 0.0, 3.0, 0.0)).astype(np.float32) * 0.25      # multiples of 1/4 mV-ish: exact sums
+    net.syns.append(Syn("AB", "A", "B", wum="static", psm="deltacurr", row_stride=fan, row_length=rl, ind=ind, g=g))
+    model, oracle, counts = run_side_by_side(net, check_every=10, exact=True)
+    assert counts["A"] > 2 * n and counts["B"] > m            # ~100 spikes per step x 40 targets >> 1111 targets: tile steps
+    assert model.synaptic_event_count == oracle.events()
+    model.unload()
+
+
 def test_izhikevich_fanout_noise():
     """C3 shape: Izhikevich neurons, fixed fanout with replacement (multapses), DeltaCurr input,
     per-step noise current from a pregenerated array.  dt = 1 ms, first 100 ms = 100 steps."""
@@ -204,9 +228,11 @@ def test_graph_replay_single_launch_step():
 
 
 @pytest.mark.parametrize("n", [1, 31, 64, 65, 257, 1000])
-def test_ragged_population_sizes(n):
+def test_ragged_population_sizes(n, monkeypatch):
     """Population sizes around the wave (64), recording-word (32) and work-group (256) boundaries;
-    includes empty rows and a population in which every neuron fires in the same step."""
+    includes empty rows and a population in which every neuron fires in the same step.  The tile path is
+    switched off: it adds LDS partial sums to outPost, which re-associates the sum (tested separately)."""
+    monkeypatch.setenv("GENNMI_TILE_FLOATS", "0")
     from genn_amd.netspec import Net, Pop, Syn
     from genn_amd import rng
     lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=1.0, TauRefrac=2.0)
