@@ -40,6 +40,20 @@ def build_net(name, steps):
         return configs.izhikevich_fanout(n=100_000, fanout=1000, steps=steps, noise_steps=64), "izhikevich 1e5 neurons fanout 1000"
     if name == "stdp":
         return configs.plastic_stdp(steps=steps), "C4 plastic STDP 100k neurons fanout 500 dt=1ms"
+    if name == "conv":
+        import copy
+        import numpy as np
+        B = 16
+        nets = [configs.conv_toeplitz(steps=steps, batch_index=b, w_sd=0.1, ioffset=0.3) for b in range(B)]
+        times = np.concatenate([n.pop("In").spike_times for n in nets])
+        offs = np.cumsum([0] + [len(n.pop("In").spike_times) for n in nets])
+        net = copy.deepcopy(nets[0])
+        net.pop("In").vars = {"startSpike": np.stack([n.pop("In").vars["startSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32),
+                              "endSpike": np.stack([n.pop("In").vars["endSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32)}
+        net.pop("In").spike_times = times
+        net.batch_size = B
+        net.batch_nets = nets
+        return net, "C5 conv2d 3x3 64x64x16 -> 64x64x32 TOEPLITZ, batch 16, dt=1ms"
     raise SystemExit(f"unknown workload {name}")
 
 
@@ -70,7 +84,8 @@ def main():
     bytes_per_event = max(BYTES_PER_EVENT[k] for k in kinds) if len(kinds) == 1 else None
 
     t0 = time.time()
-    model = model_from_net(net, record=True)
+    batch = getattr(net, "batch_size", 1)
+    model = model_from_net(net, batch_size=batch, record=True)
     model.load(num_recording_timesteps=args.warmup + args.steps)
     model.synchronize()
     load_s = time.time() - t0
@@ -80,16 +95,19 @@ def main():
     model.synchronize()
     ev0 = model.synaptic_event_count
     t0 = time.perf_counter()
+    model.stream_mark(0)
     model.run(args.steps)
+    model.stream_mark(1)
     model.synchronize()
     wall = time.perf_counter() - t0
+    region_s = model.stream_elapsed()          # HIP events on the runner's stream around the timed region
     events = model.synaptic_event_count - ev0
 
     model.pull_recording_buffers_from_device()
     rates = {}
     for p in net.pops:
-        _, ids = model.neuron_populations[p.name].spike_recording_data[0]
-        rates[p.name] = round(len(ids) / p.n / ((args.warmup + args.steps) * net.dt / 1000.0), 3)
+        data = model.neuron_populations[p.name].spike_recording_data
+        rates[p.name] = round(sum(len(ids) for _, ids in data) / batch / p.n / ((args.warmup + args.steps) * net.dt / 1000.0), 3)
 
     # ---- per-kernel durations: the same graph replay with HIP event nodes between the kernels of every step
     # (events on the runner's stream; durations are those of back-to-back execution)
@@ -105,14 +123,17 @@ def main():
         model.set_timing(False)
         bpe = bytes_per_event or max(BYTES_PER_EVENT[k] for k in kinds)
         neuron_bytes = sum(p.n * (0 if p.model == "ssa" else 32) for p in net.pops)     # 32 B per LIF/Izhikevich update (state + one PSM)
-        if info["single_launch_step"] and st["step_launches"]:
-            avg_s = st["step_seconds"] / st["step_launches"]
-            ev_per_launch = evp / st["step_launches"]
+        if info["single_launch_step"]:
+            # the timed region consists of this kernel only (one launch per step, back to back inside the replayed
+            # graphs, plus one 1-thread node per 100 steps), so HIP events around the region give its average duration
+            avg_s = region_s / args.steps
+            ev_per_launch = events / args.steps
             achieved = (ev_per_launch * bpe + neuron_bytes) / avg_s / 1e9
             roofline = {"bound": "hbm", "kernel": "stepFusedKernel (presynaptic + neuron update of one timestep)",
                         "achieved": round(achieved, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6),
                         "traffic": None, "bytes_per_event": bpe, "events_per_launch": round(ev_per_launch, 1),
-                        "neuron_bytes_per_launch": neuron_bytes, "avg_launch_us": round(avg_s * 1e6, 3)}
+                        "neuron_bytes_per_launch": neuron_bytes, "avg_launch_us": round(avg_s * 1e6, 3),
+                        "avg_launch_us_individually_launched": round(st["step_seconds"] / max(1, st["step_launches"]) * 1e6, 3)}
         elif st["presyn_launches"]:
             avg_s = st["presyn_seconds"] / st["presyn_launches"]
             ev_per_launch = evp / st["presyn_launches"]
@@ -130,7 +151,8 @@ def main():
     cpu = None
     if not args.no_cpu:
         from oracle.genn_cpu import OracleNet
-        oracle = OracleNet(net)
+        # the reference's CPU backend (and the oracle) has no batch dimension: batch 0 is timed and the figure is per batch
+        oracle = OracleNet(net.batch_nets[0] if batch > 1 else net)
         probe = 20
         t0 = time.perf_counter()
         oracle.run(probe)
@@ -155,7 +177,7 @@ def main():
         "config": {"workload": label, "neurons": num_neurons, "synapses": num_synapses, "dt_ms": net.dt, "seed": net.seed,
                    "stepping": "hipGraph replay, 100 steps per graph, " + ("1 launch per step" if info["single_launch_step"] else "2-3 launches per step")},
         "gsop_per_s": round(events / wall / 1e9, 4),
-        "neuron_updates_per_s": round(num_neurons * args.steps / wall, 1),
+        "neuron_updates_per_s": round(num_neurons * batch * args.steps / wall, 1),
         "wall_s_per_sim_s": round(wall / sim_s, 4),
         "events_per_step": round(events / args.steps, 1),
         "algorithmic_gb_per_s_wallclock": round(events * (bytes_per_event or 16) / wall / 1e9, 3),

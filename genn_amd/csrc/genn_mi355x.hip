@@ -117,7 +117,8 @@ struct PreGroupDev
     uint32_t vec4;                      // rows are 16-byte aligned and padded: dwordx4 loads
     int32_t convBH, convBW;
     uint32_t skipZeroDelay;             // synapses with d % D == 0 are delivered by the neuron update instead
-    uint32_t tileThreshold;             // != 0: leave the step to the tile kernel when numSpikes*rowStride reaches it
+    uint32_t tileThreshold;             // != 0: leave the step to the tile kernel when numSpikes*workPerSpike reaches it
+    uint32_t workPerSpike, pad2_;       // rowStride (SPARSE) or kh*kw*oc (Toeplitz)
     const uint32_t *shadowSpk;          // the source population's shadow queue (read instead of srcSpk when set)
     const uint32_t *shadowCnt;
 };
@@ -131,6 +132,16 @@ struct TileGroupDev
     uint32_t numTiles, tileSize;
     uint32_t tile, split, numSplits;    // this block: which tile, which share of the spikes
     uint32_t lanes;                     // lanes per (spike, tile) segment, power of two
+    uint32_t threshold, pad_;
+};
+
+// Dense-activity path of a Toeplitz Conv2D projection: a block owns rowsPerTile output rows (all columns and
+// channels) in LDS next to a copy of the kernel weights.
+struct ConvTileDev
+{
+    gennmi_presynaptic_update_group_t g;
+    int32_t convBH, convBW;
+    uint32_t rowsPerTile, tileRow0;
     uint32_t threshold, pad_;
 };
 
@@ -153,6 +164,8 @@ __device__ __forceinline__ GLOBAL_AS T *asGlobal(T *p) { return (GLOBAL_AS T*)p;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint8_t u8x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4u __attribute__((ext_vector_type(4), aligned(4)));     // dword-aligned only: segments start anywhere in a row
+typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
 
 __device__ __forceinline__ void atomicAddF32(GLOBAL_AS float *addr, float v)
 {
@@ -187,7 +200,7 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
     GLOBAL_AS const uint32_t *spk = G.shadowSpk ? asGlobal(G.shadowSpk) + ((size_t)parity * gridDim.y + batch) * g.numSrcNeurons
                                                 : asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
     const uint32_t numSpikes = cntPtr[batch];
-    if(G.tileThreshold && (unsigned long long)numSpikes * g.rowStride >= G.tileThreshold) { return; }
+    if(G.tileThreshold && (unsigned long long)numSpikes * G.workPerSpike >= G.tileThreshold) { return; }
     GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
     unsigned long long events = 0;
 
@@ -324,7 +337,7 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
 // sorted by target; tileOff holds the segment boundaries), adds into LDS, and finally flushes the tile
 // with consecutive lanes on consecutive addresses.
 // ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(BLOCK)
+__global__ __launch_bounds__(1024)
 void presynapticTileKernel(const TileGroupDev *blocks, unsigned long long *eventCounter)
 {
     extern __shared__ float shTile[];
@@ -335,7 +348,7 @@ void presynapticTileKernel(const TileGroupDev *blocks, unsigned long long *event
     if((unsigned long long)numSpikes * g.rowStride < G.threshold) { return; }      // the scatter kernel took this step
     const uint32_t tileStart = G.tile * G.tileSize;
     const uint32_t tileLen = min(G.tileSize, g.numTrgNeurons - tileStart);
-    for(uint32_t k = threadIdx.x; k < tileLen; k += BLOCK) { shTile[k] = 0.0f; }
+    for(uint32_t k = threadIdx.x; k < tileLen; k += blockDim.x) { shTile[k] = 0.0f; }
     __syncthreads();
 
     GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
@@ -344,27 +357,114 @@ void presynapticTileKernel(const TileGroupDev *blocks, unsigned long long *event
     GLOBAL_AS const float *weight = asGlobal(g.g);
     const uint32_t L = G.lanes;
     const uint32_t lis = threadIdx.x & (L - 1);
-    const uint32_t perBlock = BLOCK / L;
+    const uint32_t perBlock = blockDim.x / L;
     const uint32_t stride = perBlock * G.numSplits;
+    const uint32_t lastSrc = g.numSrcNeurons - 1;
     unsigned long long events = 0;
-    for(uint32_t s = G.split * perBlock + threadIdx.x / L; s < numSpikes; s += stride) {
-        const uint32_t idPre = spk[s];
-        const size_t o = (size_t)idPre * (G.numTiles + 1) + G.tile;
-        const uint32_t a = off[o], b = off[o + 1];
+    // software pipeline over this sub-group's spikes: the spike id is fetched two iterations ahead and the
+    // segment boundaries one iteration ahead (spk holds numSrcNeurons entries, so clamped indices are readable)
+    uint32_t s = G.split * perBlock + threadIdx.x / L;
+    uint32_t id0 = spk[min(s, lastSrc)], id1 = spk[min(s + stride, lastSrc)];
+    size_t o0 = (size_t)id0 * (G.numTiles + 1) + G.tile;
+    uint32_t a0 = off[o0], b0 = off[o0 + 1];
+    for(; s < numSpikes; s += stride) {
+        const uint32_t idPre = id0, a = a0, b = b0;
+        id0 = id1;
+        id1 = spk[min(s + 2 * stride, lastSrc)];
+        o0 = (size_t)id0 * (G.numTiles + 1) + G.tile;
+        a0 = off[o0]; b0 = off[o0 + 1];
         const size_t rowBase = (size_t)idPre * g.rowStride;
-        for(uint32_t j = a + lis; j < b; j += L) {
-            unsafeAtomicAdd(&shTile[ind[rowBase + j] - tileStart], weight[rowBase + j]);
+        for(uint32_t j = a + 4 * lis; j < b; j += 4 * L) {
+            if(j + 4 <= b) {
+                const u32x4u ip = *reinterpret_cast<GLOBAL_AS const u32x4u*>(ind + rowBase + j);
+                const f32x4u w = *reinterpret_cast<GLOBAL_AS const f32x4u*>(weight + rowBase + j);
+                unsafeAtomicAdd(&shTile[ip.x - tileStart], w.x);
+                unsafeAtomicAdd(&shTile[ip.y - tileStart], w.y);
+                unsafeAtomicAdd(&shTile[ip.z - tileStart], w.z);
+                unsafeAtomicAdd(&shTile[ip.w - tileStart], w.w);
+            }
+            else {
+                for(uint32_t jj = j; jj < b; jj++) { unsafeAtomicAdd(&shTile[ind[rowBase + jj] - tileStart], weight[rowBase + jj]); }
+            }
         }
         if(lis == 0) { events += b - a; }
     }
     __syncthreads();
     GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons + tileStart;
-    for(uint32_t k = threadIdx.x; k < tileLen; k += BLOCK) {
+    for(uint32_t k = threadIdx.x; k < tileLen; k += blockDim.x) {
         const float v = shTile[k];
         if(v != 0.0f) { atomicAddF32(&outPost[k], v); }
     }
     for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
     if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// Toeplitz Conv2D counterpart of the tile kernel: every block scans the (short) spike list, keeps the spikes whose
+// kernel footprint touches its output rows, and one wavefront at a time adds a spike's kh*kw*oc contributions
+// into LDS.  The block owns its rows exclusively, so the flush is a plain read-modify-write without atomics.
+__global__ __launch_bounds__(BLOCK)
+void presynapticConvTileKernel(const ConvTileDev *blocks, unsigned long long *eventCounter)
+{
+    extern __shared__ float shConv[];
+    const ConvTileDev &G = blocks[blockIdx.x];
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const int kh = g.conv[0], kw = g.conv[1], iw = g.conv[3], ic = g.conv[4];
+    const int oh = g.conv[5], ow = g.conv[6], oc = g.conv[7];
+    const uint32_t numDiag = (uint32_t)(kh * kw * oc);
+    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
+    if((unsigned long long)numSpikes * numDiag < G.threshold) { return; }      // the scatter kernel took this step
+    const int row0 = (int)G.tileRow0;
+    const int rows = min((int)G.rowsPerTile, oh - row0);
+    const uint32_t tileLen = (uint32_t)(rows * ow * oc);
+    const uint32_t kernelLen = (uint32_t)(kh * kw * ic * oc);
+    float *tile = shConv;
+    float *kern = tile + G.rowsPerTile * ow * oc;
+    uint32_t *diag = reinterpret_cast<uint32_t*>(kern + kernelLen);
+    for(uint32_t k = threadIdx.x; k < tileLen; k += BLOCK) { tile[k] = 0.0f; }
+    for(uint32_t k = threadIdx.x; k < kernelLen; k += BLOCK) { kern[k] = asGlobal(g.g)[k]; }
+    for(uint32_t j = threadIdx.x; j < numDiag; j += BLOCK) {
+        // kernel diagonal j -> (kernRow, kernCol, outChan), initToeplitzConnectivitySnippet.h:117-119
+        diag[j] = ((j / oc) / kw) << 20 | ((j / oc) % kw) << 10 | (j % oc);
+    }
+    __syncthreads();
+
+    GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    const uint32_t lane = threadIdx.x & (WAVE - 1);
+    unsigned long long events = 0;
+    for(uint32_t base = 0; base < numSpikes; base += BLOCK) {
+        const uint32_t s = base + threadIdx.x;
+        const uint32_t ipre = (s < numSpikes) ? spk[s] : 0u;
+        const int myRow = (int)(ipre / ic) / iw;
+        // rows this spike can reach: [myRow - bh, myRow - bh + kh - 1]
+        const bool relevant = (s < numSpikes) && (myRow - G.convBH + kh - 1 >= row0) && (myRow - G.convBH < row0 + rows);
+        unsigned long long pending = __ballot(relevant);
+        while(pending) {
+            const int src = __ffsll((long long)pending) - 1;
+            pending &= pending - 1;
+            const uint32_t id = __shfl(ipre, src, WAVE);
+            const int preRow = (int)(id / ic) / iw, preCol = (int)(id / ic) % iw, preChan = (int)(id % ic);
+            for(uint32_t j = lane; j < numDiag; j += WAVE) {
+                const uint32_t e = diag[j];
+                const int kernRow = (int)(e >> 20), kernCol = (int)((e >> 10) & 1023), ch = (int)(e & 1023);
+                const int postRow = preRow + kernRow - G.convBH;
+                const int postCol = preCol + kernCol - G.convBW;
+                if(postRow >= row0 && postRow < row0 + rows && postCol >= 0 && postCol < ow) {
+                    unsafeAtomicAdd(&tile[((postRow - row0) * ow + postCol) * oc + ch],
+                                    kern[((kh - kernRow - 1) * kw + (kw - kernCol - 1)) * ic * oc + preChan * oc + ch]);
+                    events++;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons + (size_t)row0 * ow * oc;
+    for(uint32_t k = threadIdx.x; k < tileLen; k += BLOCK) {
+        const float v = tile[k];
+        if(v != 0.0f) { outPost[k] += v; }
+    }
+    for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
+    if(lane == 0 && events) { atomicAdd(eventCounter, events); }
 }
 
 // Segment boundaries of every row for the tile kernel; also verifies that rows are sorted by target.
@@ -560,7 +660,8 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     const bool last = (localBlock == G.numBlocks - 1);
-    if(blockCount == 0 && !last) { return; }
+    const bool groupLeader = ((localBlock % WAVE) == WAVE - 1) || last;
+    if(blockCount == 0 && !groupLeader) { return; }
 
     // Synapses with d % D == 0 of the neurons that just fired belong in the slot their targets read in the
     // NEXT step, (epoch + 2) % D, which nothing reads or clears during this step — so the presynaptic update of
@@ -582,23 +683,44 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
     if(G.zeroStart && wave != 0) { deliverZeroDelay(); }
 
     if(wave == 0) {
-        uint32_t sum = 0;
+        // Two-level offset: blocks of a population form groups of 64.  The last block of a group sums the
+        // group's 64 counts and publishes the group total in the second half of `agg`; a block's offset is the
+        // sum of the counts of the earlier blocks of its group plus the totals of the earlier groups.  Every
+        // wait is for a value that depends only on other blocks having published their own count, so there is
+        // no chain of blocks waiting for each other's results, whatever the population size.
+        unsigned long long *groupAgg = agg + (size_t)totalNeuronBlocks * gridDim.y;
+        const uint32_t group = localBlock / WAVE, inGroup = localBlock % WAVE;
+        const size_t groupBase = aggBase + (size_t)group * WAVE;
         bool ok = true;
-        for(uint32_t base = 0; base < localBlock; base += WAVE) {
-            const uint32_t k = base + lane;
-            uint32_t v = 0;
-            if(k < localBlock) {
-                uint32_t spins = 0;
-                while(true) {
-                    const unsigned long long a = __hip_atomic_load(&agg[aggBase + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if((uint32_t)(a >> 32) == tag) { v = (uint32_t)a; break; }
-                    if(++spins > SPIN_LIMIT) { ok = false; break; }
-                    __builtin_amdgcn_s_sleep(1);
-                }
+        auto waitFor = [&](const unsigned long long *p) -> uint32_t {
+            uint32_t spins = 0;
+            while(true) {
+                const unsigned long long a = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if((uint32_t)(a >> 32) == tag) { return (uint32_t)a; }
+                if(++spins > SPIN_LIMIT) { ok = false; return 0u; }
+                __builtin_amdgcn_s_sleep(1);
             }
-            sum += v;
+        };
+        // counts of the earlier blocks of this group (lane == inGroup contributes this block's own count)
+        uint32_t v = 0;
+        if(lane < inGroup) { v = waitFor(&agg[groupBase + lane]); }
+        uint32_t intra = v;
+        for(int off = WAVE / 2; off > 0; off >>= 1) { intra += __shfl_down(intra, off, WAVE); }
+        intra = __shfl(intra, 0, WAVE);
+        if(inGroup == WAVE - 1 || last) {
+            if(lane == 0 && ok) {
+                __hip_atomic_store(&groupAgg[aggBase + group], ((unsigned long long)tag << 32) | (intra + blockCount),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
-        for(int off = WAVE / 2; off > 0; off >>= 1) { sum += __shfl_down(sum, off, WAVE); }
+        uint32_t sum = 0;
+        if(blockCount != 0 || last) {
+            for(uint32_t base = 0; base < group; base += WAVE) {
+                if(base + lane < group) { sum += waitFor(&groupAgg[aggBase + base + lane]); }
+            }
+            for(int off = WAVE / 2; off > 0; off >>= 1) { sum += __shfl_down(sum, off, WAVE); }
+            sum += intra;
+        }
         const bool allOk = (__ballot(!ok) == 0ull);
         if(lane == 0) {
             if(!allOk) { atomicOr(errorFlag, 1u); sum = 0xFFFFFFFFu; }
@@ -736,7 +858,8 @@ struct gennmi_runner
     unsigned long long epoch = 0;       // completed steps (host mirror)
     bool synapsesDone = false;          // updateSynapses ran for the current step
     bool fusedStep = false;             // zero-delay synapses are delivered by the neuron update; one launch per step
-    TileGroupDev *dTile = nullptr; uint32_t tileBlocks = 0, tileFloats = 0;
+    TileGroupDev *dTile = nullptr; uint32_t tileBlocks = 0, tileFloats = 0, tileThreads = BLOCK;
+    ConvTileDev *dConvTile = nullptr; uint32_t convTileBlocks = 0; size_t convTileBytes = 0;
     std::vector<void*> owned;           // engine-private device allocations (shadow queues, zero-delay lists)
     // graph
     hipGraphExec_t graphExec = nullptr; unsigned long long graphSteps = 0;
@@ -747,6 +870,7 @@ struct gennmi_runner
     double stepTime = 0;                // single-launch steps
     struct Pending { hipEvent_t a, b; int kind; };          // kind: 0 presynaptic, 1 postsynaptic, 2 neuron, 3 single-launch step
     std::vector<hipEvent_t> eventPool; size_t eventNext = 0; std::vector<Pending> pending;
+    hipEvent_t marks[2] = {nullptr, nullptr};               // gennmi_runner_stream_mark
 };
 
 extern "C" {
@@ -831,8 +955,9 @@ int gennmi_runner_destroy(gennmi_runner *r)
     hipStreamSynchronize(r->stream);
     if(r->graphExec) { hipGraphExecDestroy(r->graphExec); }
     for(hipEvent_t e : r->eventPool) { hipEventDestroy(e); }
+    for(hipEvent_t e : r->marks) { if(e) { hipEventDestroy(e); } }
     for(void *q : r->owned) { hipFree(q); }
-    hipFree(r->dTile);
+    hipFree(r->dTile); hipFree(r->dConvTile);
     hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dAgg); hipFree(r->dError); hipFree(r->dEvents); hipFree(r->dState);
     hipStreamDestroy(r->stream);
     delete r;
@@ -1001,9 +1126,33 @@ int gennmi_runner_finalise(gennmi_runner *r)
     // ---- tile path for static, delay-free SPARSE projections whose rows are sorted by target
     {
         const char *envTile = getenv("GENNMI_TILE_FLOATS");
-        const uint32_t tileFloats = envTile ? (uint32_t)std::max(0, atoi(envTile)) : 8192u;
+        const uint32_t tileFloats = envTile ? (uint32_t)std::max(0, atoi(envTile)) : 16384u;
+        const char *envThreads = getenv("GENNMI_TILE_THREADS");
+        r->tileThreads = envThreads ? (uint32_t)std::min(1024, std::max(64, atoi(envThreads))) : (tileFloats > 16384 ? 1024u : (tileFloats > 8192 ? 512u : (uint32_t)BLOCK));
         std::vector<TileGroupDev> tiles;
+        std::vector<ConvTileDev> convTiles;
         for(auto &p : r->pre) {
+            p.workPerSpike = (p.g.matrix == GENNMI_MATRIX_SPARSE) ? p.g.rowStride : (uint32_t)(p.g.conv[0] * p.g.conv[1] * p.g.conv[7]);
+            if(tileFloats != 0 && p.g.matrix == GENNMI_MATRIX_TOEPLITZ_CONV2D && r->pre.size() == 1
+               && p.g.conv[0] < 4096 && p.g.conv[1] < 1024 && p.g.conv[7] < 1024) {
+                const int32_t *c = p.g.conv;
+                const size_t rowFloats = (size_t)c[6] * c[7];
+                const size_t fixedFloats = (size_t)c[0] * c[1] * c[4] * c[7] + (size_t)c[0] * c[1] * c[7];
+                const size_t budgetFloats = 60 * 1024 / sizeof(float);
+                if(fixedFloats + rowFloats <= budgetFloats) {
+                    // as many rows per block as fit in LDS, but enough blocks to cover the chip about twice
+                    uint32_t rowsPerTile = (uint32_t)std::min<size_t>((budgetFloats - fixedFloats) / rowFloats, (size_t)c[5]);
+                    const uint32_t wantBlocks = std::max(1u, (2 * numCU) / r->batch);
+                    rowsPerTile = std::max(1u, std::min(rowsPerTile, ((uint32_t)c[5] + wantBlocks - 1) / wantBlocks));
+                    ConvTileDev t{};
+                    t.g = p.g; t.convBH = p.convBH; t.convBW = p.convBW; t.rowsPerTile = rowsPerTile;
+                    p.tileThreshold = std::max(1u, p.g.numTrgNeurons / 4);
+                    t.threshold = p.tileThreshold;
+                    for(uint32_t row0 = 0; row0 < (uint32_t)c[5]; row0 += rowsPerTile) { t.tileRow0 = row0; convTiles.push_back(t); }
+                    r->convTileBytes = (fixedFloats + rowsPerTile * rowFloats) * sizeof(float);
+                }
+                continue;
+            }
             if(tileFloats == 0 || p.g.matrix != GENNMI_MATRIX_SPARSE || p.g.wum != GENNMI_WUM_STATIC_PULSE || p.g.rowStride > 65535) { continue; }
             const uint32_t tileSize = std::min(tileFloats, p.g.numTrgNeurons);
             const uint32_t numTiles = (p.g.numTrgNeurons + tileSize - 1) / tileSize;
@@ -1021,16 +1170,25 @@ int gennmi_runner_finalise(gennmi_runner *r)
             if(unsorted) { continue; }          // rows not sorted by target: the scatter kernel handles every step
             p.tileThreshold = std::max(1u, p.g.numTrgNeurons);
             const char *envSplit = getenv("GENNMI_TILE_BLOCKS_PER_CU");
-            const uint32_t blocksPerCUTile = envSplit ? (uint32_t)std::max(1, atoi(envSplit)) : 2u;
-            const uint32_t numSplits = std::max(1u, std::min(256u, (blocksPerCUTile * numCU) / numTiles));
+            const uint32_t blocksPerCUTile = envSplit ? (uint32_t)std::max(1, atoi(envSplit)) : 4u;
+            const uint32_t numSplits = std::max(1u, std::min(256u, (blocksPerCUTile * numCU * BLOCK / r->tileThreads) / numTiles));
             const uint32_t avgSeg = std::max(1u, p.g.rowStride / numTiles);
             TileGroupDev t{};
             t.g = p.g; t.tileOff = dOff; t.numTiles = numTiles; t.tileSize = tileSize; t.numSplits = numSplits;
-            t.lanes = std::min<uint32_t>(WAVE, pow2Ceil((avgSeg + 1) / 2)); t.threshold = p.tileThreshold;
+            t.lanes = std::min<uint32_t>(WAVE, pow2Ceil((avgSeg + 7) / 8)); t.threshold = p.tileThreshold;
             for(uint32_t tile = 0; tile < numTiles; tile++) {
                 for(uint32_t split = 0; split < numSplits; split++) { t.tile = tile; t.split = split; tiles.push_back(t); }
             }
             r->tileFloats = std::max(r->tileFloats, tileSize);
+        }
+        if(!convTiles.empty()) {
+            HIP_TRY(hipMalloc(&r->dConvTile, convTiles.size() * sizeof(ConvTileDev)));
+            HIP_TRY(hipMemcpy(r->dConvTile, convTiles.data(), convTiles.size() * sizeof(ConvTileDev), hipMemcpyHostToDevice));
+            r->convTileBlocks = (uint32_t)convTiles.size();
+            if(r->convTileBytes > 48 * 1024) {
+                HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(presynapticConvTileKernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            (int)r->convTileBytes));
+            }
         }
         if(!tiles.empty()) {
             HIP_TRY(hipMalloc(&r->dTile, tiles.size() * sizeof(TileGroupDev)));
@@ -1108,7 +1266,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
     HIP_TRY(uploadPerBlock(r->neuron, r->neuronBlocks, &r->dNeuron));
     HIP_TRY(uploadPerBlock(r->pre, r->preBlocks, &r->dPre));
     HIP_TRY(uploadPerBlock(r->post, r->postBlocks, &r->dPost));
-    const size_t aggCount = (size_t)r->neuronBlocks * r->batch;
+    const size_t aggCount = 2 * (size_t)r->neuronBlocks * r->batch;       // per-block counts, then per-group totals
     HIP_TRY(hipMalloc(&r->dAgg, aggCount * sizeof(unsigned long long)));
     HIP_TRY(hipMemset(r->dAgg, 0, aggCount * sizeof(unsigned long long)));
     HIP_TRY(hipDeviceSynchronize());
@@ -1158,7 +1316,10 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
     if(!r->pre.empty()) {
         presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dPre, a, r->dt, r->dEvents);
         if(r->tileBlocks) {
-            presynapticTileKernel<<<dim3(r->tileBlocks, r->batch), dim3(BLOCK), r->tileFloats * sizeof(float), r->stream>>>(r->dTile, r->dEvents);
+            presynapticTileKernel<<<dim3(r->tileBlocks, r->batch), dim3(r->tileThreads), r->tileFloats * sizeof(float), r->stream>>>(r->dTile, r->dEvents);
+        }
+        if(r->convTileBlocks) {
+            presynapticConvTileKernel<<<dim3(r->convTileBlocks, r->batch), dim3(BLOCK), r->convTileBytes, r->stream>>>(r->dConvTile, r->dEvents);
         }
         if(timed) { const int rc = stamp(r, &e1); if(rc) { return rc; } r->pending.push_back({e0, e1, 0}); }
     }
@@ -1333,6 +1494,24 @@ int gennmi_runner_kernel_stats(gennmi_runner *r, double stats[8])
     stats[2] = (double)r->neuronLaunches; stats[3] = r->neuronTime;
     stats[4] = (double)r->postLaunches; stats[5] = r->postTime;
     stats[6] = (double)r->stepLaunches; stats[7] = r->stepTime;
+    return GENNMI_OK;
+}
+
+int gennmi_runner_stream_mark(gennmi_runner *r, int which)
+{
+    if(!r || which < 0 || which > 1) { return fail(GENNMI_EINVAL, "runner_stream_mark: bad arguments"); }
+    if(!r->marks[which]) { HIP_TRY(hipEventCreate(&r->marks[which])); }
+    HIP_TRY(hipEventRecord(r->marks[which], r->stream));
+    return GENNMI_OK;
+}
+
+int gennmi_runner_stream_elapsed(gennmi_runner *r, double *seconds)
+{
+    if(!r || !seconds || !r->marks[0] || !r->marks[1]) { return fail(GENNMI_EINVAL, "runner_stream_elapsed: both marks must have been recorded"); }
+    HIP_TRY(hipEventSynchronize(r->marks[1]));
+    float ms = 0;
+    HIP_TRY(hipEventElapsedTime(&ms, r->marks[0], r->marks[1]));
+    *seconds = ms * 1e-3;
     return GENNMI_OK;
 }
 

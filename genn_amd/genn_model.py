@@ -645,6 +645,14 @@ class GeNNModel:
         return {"presyn_launches": int(st[0]), "presyn_seconds": st[1], "neuron_launches": int(st[2]), "neuron_seconds": st[3],
                 "postsyn_launches": int(st[4]), "postsyn_seconds": st[5], "step_launches": int(st[6]), "step_seconds": st[7]}
 
+    def stream_mark(self, which):
+        _abi.check(_abi.load().gennmi_runner_stream_mark(self._runner, int(which)))
+
+    def stream_elapsed(self):
+        v = C.c_double()
+        _abi.check(_abi.load().gennmi_runner_stream_elapsed(self._runner, C.byref(v)))
+        return v.value
+
     def runner_info(self):
         info = (C.c_uint32 * 4)()
         _abi.check(_abi.load().gennmi_runner_get_info(self._runner, C.byref(info)))

@@ -202,6 +202,11 @@ int gennmi_runner_get_times(gennmi_runner *runner, double *neuronUpdateTime, dou
  * single-launch steps, seconds}.  Events are recorded on the runner's stream around every kernel and only read
  * (after one synchronisation) when statistics are requested, so timed stepping does not idle the device. */
 int gennmi_runner_kernel_stats(gennmi_runner *runner, double stats[8]);
+/* Two HIP events on the runner's stream: mark(0) before and mark(1) after a region of queued work, then
+ * elapsed() = device time between them (blocks until mark 1 has completed).  This is the Timer of
+ * backendCUDAHIP.cc:36-76 for a caller-chosen region, e.g. a whole gennmi_run_steps replay. */
+int gennmi_runner_stream_mark(gennmi_runner *runner, int which);
+int gennmi_runner_stream_elapsed(gennmi_runner *runner, double *seconds);
 /* Launch plan chosen by gennmi_runner_finalise: info[0] = 1 if a whole timestep is one launch (all projections go
  * through a dendritic-delay ring; synapses with d % D == 0 are then delivered by the spiking neuron one launch
  * earlier, into the slot read in the next step — the visible difference is the content of that one ring slot
