@@ -52,7 +52,8 @@ typedef struct {
 typedef struct {
     int kind;
     float amp;
-    const float *noise;     /* [steps * n], row s is injected at step s */
+    const float *noise;     /* [noiseSteps * n]: row s % noiseSteps is what the host pushes before step s */
+    uint64_t noiseSteps;
 } gc_cs;
 
 typedef struct {
@@ -142,11 +143,12 @@ int gc_add_psm(gc_net *net, int pop, int kind, float init, float expDecay, uint3
     return p->numPSM++;
 }
 
-int gc_add_cs(gc_net *net, int pop, int kind, float amp, const float *noise)
+int gc_add_cs(gc_net *net, int pop, int kind, float amp, const float *noise, uint64_t noiseSteps)
 {
     gc_pop *p = &net->pops[pop];
     if(p->numCS == GC_MAX_CHILD) { return -1; }
     p->cs[p->numCS].kind = kind; p->cs[p->numCS].amp = amp; p->cs[p->numCS].noise = noise;
+    p->cs[p->numCS].noiseSteps = noiseSteps ? noiseSteps : 1;
     return p->numCS++;
 }
 
@@ -365,7 +367,7 @@ void gc_update_neurons(gc_net *net, float t, uint32_t recordingTimestep)
                 psm->outPost[i] = linSyn;
             }
             for(int c = 0; c < p->numCS; c++) {
-                Isyn += (p->cs[c].kind == GC_CS_DC) ? p->cs[c].amp : p->cs[c].noise[(size_t)step * p->n + i];
+                Isyn += (p->cs[c].kind == GC_CS_DC) ? p->cs[c].amp : p->cs[c].noise[(size_t)(step % p->cs[c].noiseSteps) * p->n + i];
             }
             if(p->model == GC_LIF) {
                 /* p = {Ioffset, Rmembrane, Vrest, ExpTC, Vthresh, Vreset, TauRefrac} ; l0 = V, l1 = RefracTime */

@@ -43,7 +43,7 @@ def lib():
         l.gc_create.restype = vp; l.gc_create.argtypes = [f32, u64]
         l.gc_add_pop.restype = i32; l.gc_add_pop.argtypes = [vp, i32, u32, vp, i32, vp, vp, vp]
         l.gc_add_psm.restype = i32; l.gc_add_psm.argtypes = [vp, i32, i32, f32, f32, u32]
-        l.gc_add_cs.restype = i32; l.gc_add_cs.argtypes = [vp, i32, i32, f32, vp]
+        l.gc_add_cs.restype = i32; l.gc_add_cs.argtypes = [vp, i32, i32, f32, vp, u64]
         l.gc_add_syn_sparse.restype = i32; l.gc_add_syn_sparse.argtypes = [vp, i32, i32, i32, i32, u32, vp, vp, vp, vp, i32]
         l.gc_set_stdp_trace.restype = None; l.gc_set_stdp_trace.argtypes = [vp, i32, f32, f32, f32, f32, f32, f32, u32]
         l.gc_add_syn_conv2d.restype = i32; l.gc_add_syn_conv2d.argtypes = [vp, i32, i32, i32, vp, vp]
@@ -98,6 +98,7 @@ class OracleNet:
         self.l = lib()
         self.net = net
         self.keep = []               # arrays the C side borrows
+        self.num_rec = num_recording_timesteps
         self.h = self.l.gc_create(C.c_float(literal_f32(net.dt)), num_recording_timesteps)
         self.pop_id, self.syn_id, self.psm_id = {}, {}, {}
         dt = net.dt
@@ -180,11 +181,11 @@ class OracleNet:
                 for j, p in enumerate(members):
                     c = css[j][ci]
                     if c.model == "dc":
-                        self.l.gc_add_cs(self.h, self.pop_id[p.name], GC_CS_DC, C.c_float(amps[j]), None)
+                        self.l.gc_add_cs(self.h, self.pop_id[p.name], GC_CS_DC, C.c_float(amps[j]), None, 0)
                     else:
                         a = _as(c.noise, np.float32)
                         self.keep.append(a)
-                        self.l.gc_add_cs(self.h, self.pop_id[p.name], GC_CS_NOISE, 0.0, a.ctypes.data)
+                        self.l.gc_add_cs(self.h, self.pop_id[p.name], GC_CS_NOISE, 0.0, a.ctypes.data, a.size // p.n)
 
         for s in net.syns:
             src, trg = self.pop_id[s.src], self.pop_id[s.trg]
@@ -221,6 +222,21 @@ class OracleNet:
 
     def run(self, steps):
         self.l.gc_run(self.h, steps)
+
+    @property
+    def timestep(self):
+        return int(self.l.gc_timestep(self.h))
+
+    def update_synapses(self):
+        """First half of step(): the runner's updateSynapses(t)."""
+        self.l.gc_update_synapses(self.h, C.c_float(np.float32(self.timestep) * np.float32(literal_f32(self.net.dt))))
+
+    def update_neurons(self):
+        """Second half of step(): updateNeurons(t, recordingTimestep); advances time."""
+        ts = self.timestep
+        self.l.gc_update_neurons(self.h, C.c_float(np.float32(ts) * np.float32(literal_f32(self.net.dt))),
+                                 (ts % self.num_rec) if self.num_rec else 0)
+        self.l.gc_advance(self.h)
 
     def _arr(self, ptr, n, dtype):
         if not ptr or n == 0:

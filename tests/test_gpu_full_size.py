@@ -1,0 +1,176 @@
+"""GPU parity at the full sizes the throughput figures are quoted on.
+
+Each network is generated at its published size, run for (at least) its first 100 ms of simulated time
+through the captured-graph path (`run`) — the path the benchmark times — and compared with the CPU
+oracle run over the same steps:
+
+* the recorded spike raster (every neuron, every step) must be identical bit for bit,
+* the number of synaptic events delivered must be identical, and must equal the sum of the row lengths
+  of the recorded spikes (conservation: no event lost or duplicated by any kernel or work split),
+* neuron state must agree within 1e-5 relative (accumulators relative to their peak magnitude).
+"""
+import numpy as np
+import pytest
+
+from genn_amd import configs
+from genn_amd.genn_model import model_from_net
+from oracle.genn_cpu import OracleNet
+from parity import compare_state
+
+pytestmark = pytest.mark.gpu
+
+
+def _raster_bits(words, n, steps):
+    """recordSpk words of one population -> bool[steps, n]."""
+    w = (n + 31) // 32
+    return np.unpackbits(np.ascontiguousarray(words).view(np.uint8).reshape(steps, w * 4), axis=1, bitorder="little")[:, :n]
+
+
+def _events_from_raster(net, rasters):
+    """Sum over recorded spikes of the row length of every outgoing SPARSE projection.  Spikes of the last step
+    are delivered by the step after it, so they are left out."""
+    total = 0
+    for s in net.syns:
+        if s.matrix != "sparse":
+            continue
+        per_neuron = rasters[s.src][:-1].sum(axis=0, dtype=np.int64)
+        total += int((per_neuron * s.row_length.astype(np.int64)).sum())
+    return total
+
+
+def _run_both(net, steps, col_stride_of=()):
+    model = model_from_net(net)
+    model.load(num_recording_timesteps=steps)
+    col_stride = {name: model.synapse_populations[name].col_stride for name in col_stride_of} or None
+    oracle = OracleNet(net, num_recording_timesteps=steps, col_stride=col_stride)
+    model.run(steps)
+    oracle.run(steps)
+    model.pull_recording_buffers_from_device()
+    rasters = {}
+    for p in net.pops:
+        got = model.neuron_populations[p.name].vars["recordSpk"].view
+        want = oracle.record(p.name, steps)
+        if not np.array_equal(got, want):
+            g, w = _raster_bits(got, p.n, steps), _raster_bits(want, p.n, steps)
+            first = int(np.nonzero((g != w).any(axis=1))[0][0])
+            raise AssertionError(f"raster of {p.name} differs first at step {first}")
+        rasters[p.name] = _raster_bits(want, p.n, steps)
+    return model, oracle, rasters
+
+
+def test_microcircuit_full_size_first_100ms():
+    """77,169 neurons, 298,624,465 synapses, dt 0.1 ms: 1000 steps."""
+    net = configs.potjans(steps=1000)
+    assert sum(p.n for p in net.pops) == 77169
+    assert sum(int(s.row_length.sum()) for s in net.syns) == 298624465
+    model, oracle, rasters = _run_both(net, 1000)
+    assert model.runner_info()["single_launch_step"]
+    spikes = sum(int(r.sum()) for r in rasters.values())
+    assert spikes > 10000
+    assert model.synaptic_event_count == oracle.events() == _events_from_raster(net, rasters)
+    compare_state(net, model, oracle, "after 1000 steps", exact=False)
+    model.unload()
+
+
+def test_izhikevich_full_size_first_100ms():
+    """1,000,000 neurons, 10^9 synapses, dt 1 ms: 100 steps, covering the silent start, the sparse regime (scatter
+    kernel) and the population burst (hundreds of thousands of spikes per step, tile kernel).
+
+    During the burst every neuron sums hundreds of differently-valued weights per step, in an order atomics do not
+    fix; a neuron whose potential lands within rounding of the 30 mV threshold can then fire one step apart on the two
+    executors, after which free-running trajectories separate chaotically.  The comparison is therefore made in lock
+    step, each half of a step on its own and from the SAME state: the presynaptic update's input sums must agree
+    within 1e-5 of the array's peak; the engine's sums are then copied into the oracle, and from those identical
+    inputs the neuron update must produce identical spike queues and V, U within 1e-5 (then copied likewise).  Every
+    step of the full-size run is checked this way, and the event counters must agree exactly at the end."""
+    net = configs.izhikevich_fanout(steps=100, noise_steps=64)
+    n = net.pops[0].n
+    assert n == 1_000_000 and int(net.syns[0].row_length.sum()) == 1_000_000_000
+    model = model_from_net(net)
+    model.load(num_recording_timesteps=100)
+    oracle = OracleNet(net, num_recording_timesteps=100)
+    pop, syn = model.neuron_populations["N"], model.synapse_populations[net.syns[0].name]
+    dense_steps = sparse_steps = 0
+    events = 0
+    for step in range(100):
+        num_in = len(oracle.spikes("N"))
+        events += num_in * 1000
+        model.update_synapses()
+        oracle.update_synapses()
+        got, want = syn.vars["outPost"].pull_from_device(), oracle.out_post(net.syns[0].name)
+        peak = max(1e-3, float(np.abs(want).max()))
+        err = float(np.abs(got.astype(np.float64) - want).max()) / peak
+        assert err <= 1e-5, f"step {step}: input sums differ by {err:.3e} of peak ({num_in} spikes)"
+        # carry the engine's sums over, so the neuron update is compared from identical inputs
+        want[:] = got
+        model.update_neurons()
+        oracle.update_neurons()
+        got_s, want_s = pop.current_spikes[0], oracle.spikes("N")
+        flips = np.setxor1d(got_s, want_s)
+        dense = num_in * 1000 >= n
+        dense_steps += dense
+        sparse_steps += (0 < num_in * 1000 < n)
+        assert len(flips) == 0, f"step {step}: spike queues differ from identical inputs ({len(flips)} neurons)"
+        for k, name in enumerate(("V", "U")):
+            g, w = pop.vars[name].pull_from_device(), oracle.var("N", k)
+            rel = np.abs(g.astype(np.float64) - w) / np.maximum(np.abs(w), 1e-3)
+            assert rel.max() <= 1e-5, f"step {step}: {name} max relative error {rel.max():.3e}"
+            w[:] = g
+    assert dense_steps >= 10 and sparse_steps >= 10, (dense_steps, sparse_steps)
+    assert model.synaptic_event_count == oracle.events() == events
+    model.unload()
+
+
+def test_plastic_stdp_full_size_first_100ms():
+    """100,000 neurons with trace STDP on E->E (learnPost through the column remap), dt 1 ms: 100 steps."""
+    net = configs.plastic_stdp(steps=100)
+    assert sum(p.n for p in net.pops if p.model != "ssa") == 100_000
+    model, oracle, rasters = _run_both(net, 100, col_stride_of=("EE",))
+    sg = model.synapse_populations["EE"]
+    col_length = sg.vars["colLength"].pull_from_device()
+    assert np.array_equal(col_length, oracle.col_length("EE"))
+    remap = sg.vars["remap"].pull_from_device().reshape(-1, sg.col_stride)
+    want = oracle.remap("EE").reshape(-1, sg.col_stride)
+    mask = np.arange(sg.col_stride)[None, :] < col_length[:, None]
+    assert np.array_equal(remap[mask], want[mask])
+    assert sum(int(r.sum()) for r in rasters.values()) > 10000
+    assert model.synaptic_event_count == oracle.events()
+    compare_state(net, model, oracle, "after 100 steps", exact=False)
+    model.unload()
+
+
+def test_toeplitz_conv_full_size_batch16():
+    """64x64x16 -> 64x64x32, 3x3 kernels, batch 16, dt 1 ms: 100 steps; batch b must equal a batch-1 oracle run
+    fed batch b's input spike trains."""
+    import copy
+    B, steps = 16, 100
+    nets = [configs.conv_toeplitz(steps=steps, batch_index=b) for b in range(B)]
+    times = np.concatenate([n.pop("In").spike_times for n in nets])
+    offs = np.cumsum([0] + [len(n.pop("In").spike_times) for n in nets])
+    start = np.stack([n.pop("In").vars["startSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32)
+    end = np.stack([n.pop("In").vars["endSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32)
+    batched = copy.deepcopy(nets[0])
+    batched.pop("In").vars = {"startSpike": start, "endSpike": end}
+    batched.pop("In").spike_times = times
+    model = model_from_net(batched, batch_size=B)
+    model.load(num_recording_timesteps=steps)
+    model.run(steps)
+    model.pull_recording_buffers_from_device()
+    v = model.neuron_populations["Out"].vars["V"].pull_from_device().reshape(B, -1)
+    total = 0
+    for b, net in enumerate(nets):
+        oracle = OracleNet(net, num_recording_timesteps=steps)
+        oracle.run(steps)
+        for name in ("In", "Out"):
+            n = net.pop(name).n
+            words = (n + 31) // 32
+            got = model.neuron_populations[name].vars["recordSpk"].view.reshape(steps, B, words)[:, b, :]
+            want = oracle.record(name, steps).reshape(steps, words)
+            assert np.array_equal(got, want), f"batch {b}: raster of {name} differs"
+            total += int(_raster_bits(want, n, steps).sum())
+        want_v = oracle.var("Out", 0)
+        err = np.abs(v[b].astype(np.float64) - want_v) / np.maximum(np.abs(want_v), 1e-3)
+        assert err.max() <= 1e-5, f"batch {b}: V max relative error {err.max():.3e}"
+        oracle.close()
+    assert total > 100000
+    model.unload()
