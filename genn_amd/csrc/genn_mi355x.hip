@@ -71,6 +71,13 @@ struct StepArgs              // per-launch; either direct values or offsets from
 
 struct Resolved { float t; uint32_t recT; unsigned long long epoch; };
 
+// step counter modulo a 32-bit period: 64-bit division is a long software routine on this part, and the
+// counter fits 32 bits for the first 4e9 steps
+__device__ __forceinline__ uint32_t modStep(unsigned long long x, uint32_t d)
+{
+    return (x >> 32) ? (uint32_t)(x % d) : ((uint32_t)x % d);
+}
+
 __device__ __forceinline__ Resolved resolve(const StepArgs &a, float dt)
 {
     Resolved r;
@@ -79,7 +86,7 @@ __device__ __forceinline__ Resolved resolve(const StepArgs &a, float dt)
         // const float t = timestep * DT  (generateRunner.cc:283)
         r.t = (float)ts * dt;
         const unsigned long long nr = a.base->numRecordingTimesteps;
-        r.recT = nr ? (uint32_t)(ts % nr) : 0u;
+        r.recT = nr ? (((ts | nr) >> 32) ? (uint32_t)(ts % nr) : ((uint32_t)ts % (uint32_t)nr)) : 0u;
         r.epoch = a.base->epoch + a.k;
     }
     else {
@@ -199,6 +206,11 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
     GLOBAL_AS const uint32_t *cntPtr = G.shadowSpk ? asGlobal(G.shadowCnt) + (size_t)parity * gridDim.y : asGlobal(g.srcSpkCnt);
     GLOBAL_AS const uint32_t *spk = G.shadowSpk ? asGlobal(G.shadowSpk) + ((size_t)parity * gridDim.y + batch) * g.numSrcNeurons
                                                 : asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    // the first spike id this sub-group would handle is fetched together with the count, not after it (the
+    // queue always holds numSrcNeurons entries, so any index below that is readable)
+    const uint32_t sparseSpan = W * (G.vec4 ? 4u : 1u);
+    const uint32_t sparseChunksPerRow = (g.rowStride + sparseSpan - 1) / sparseSpan;
+    const uint32_t firstSpike = (g.matrix == GENNMI_MATRIX_SPARSE) ? spk[min(subGroup / max(sparseChunksPerRow, 1u), g.numSrcNeurons - 1)] : 0u;
     const uint32_t numSpikes = cntPtr[batch];
     if(G.tileThreshold && (unsigned long long)numSpikes * G.workPerSpike >= G.tileThreshold) { return; }
     GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
@@ -211,12 +223,15 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
         const int oh = g.conv[5], ow = g.conv[6], oc = g.conv[7];
         const uint32_t numDiag = (uint32_t)(kh * kw * oc);
         const uint32_t chunksPerRow = (numDiag + W - 1) / W;
-        const unsigned long long numItems = (unsigned long long)numSpikes * chunksPerRow;
         GLOBAL_AS const float *kernel = asGlobal(g.g);
-        for(unsigned long long item = subGroup; item < numItems; item += numSubGroups) {
-            const uint32_t s = (uint32_t)(item / chunksPerRow);
-            const uint32_t j = (uint32_t)(item % chunksPerRow) * W + lis;
+        // item = subGroup + k*numSubGroups, split into (spike, chunk) incrementally: no division in the loop
+        const uint32_t stepSpike = numSubGroups / chunksPerRow, stepChunk = numSubGroups % chunksPerRow;
+        uint32_t chunk = subGroup % chunksPerRow;
+        for(unsigned long long s = subGroup / chunksPerRow; s < numSpikes; ) {
+            const uint32_t j = chunk * W + lis;
             const uint32_t ipre = spk[s];
+            s += stepSpike; chunk += stepChunk;
+            if(chunk >= chunksPerRow) { chunk -= chunksPerRow; s++; }
             if(j < numDiag) {
                 const int preRow = (int)(ipre / ic) / iw;
                 const int preCol = (int)(ipre / ic) % iw;
@@ -240,7 +255,7 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
         // *denDelayPtr = (*denDelayPtr + 1) % D happens at the start of updateSynapses
         // (synapseUpdateGroupMerged.cc:480-483); st.epoch counts completed steps, so the pointer
         // in force during this step is (epoch + 1) % D.
-        const uint32_t denPtr = D ? (uint32_t)((st.epoch + 1) % D) : 0;
+        const uint32_t denPtr = D ? modStep(st.epoch + 1, D) : 0;
         GLOBAL_AS float *denDelay = D ? asGlobal(g.denDelay) + (size_t)batch * D * g.numTrgNeurons : nullptr;
         GLOBAL_AS const uint32_t *rowLength = asGlobal(g.rowLength);
         GLOBAL_AS const uint32_t *ind = asGlobal(g.ind);
@@ -250,18 +265,22 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
         const uint32_t perLane = G.vec4 ? 4u : 1u;
         const uint32_t span = W * perLane;
         const uint32_t chunksPerRow = (g.rowStride + span - 1) / span;
-        const unsigned long long numItems = (unsigned long long)numSpikes * chunksPerRow;
         // Loads are issued ahead of the values that decide whether they are needed, so that the
         // dependent chain per item is spike id -> {rowLength, row chunk} -> atomics: the spike id of
         // the NEXT item is fetched while the current one is processed (spk always holds
         // numSrcNeurons entries, so any index below that is readable), and the row chunk is read
         // together with rowLength (rows are padded to rowStride, so any j < rowStride is readable).
         const uint32_t lastSrc = g.numSrcNeurons - 1;
-        uint32_t idPreNext = spk[min((uint32_t)(subGroup / chunksPerRow), lastSrc)];
-        for(unsigned long long item = subGroup; item < numItems; item += numSubGroups) {
-            const uint32_t chunk = (uint32_t)(item % chunksPerRow);
+        uint32_t idPreNext = firstSpike;
+        // item = subGroup + k*numSubGroups, split into (spike, chunk) incrementally: no division in the loop
+        const uint32_t stepSpike = numSubGroups / chunksPerRow, stepChunk = numSubGroups % chunksPerRow;
+        uint32_t chunkNext = subGroup % chunksPerRow;
+        for(unsigned long long sNext = subGroup / chunksPerRow; sNext < numSpikes; ) {
+            const uint32_t chunk = chunkNext;
             const uint32_t idPre = idPreNext;
-            idPreNext = spk[min((uint32_t)((item + numSubGroups) / chunksPerRow), lastSrc)];
+            sNext += stepSpike; chunkNext += stepChunk;
+            if(chunkNext >= chunksPerRow) { chunkNext -= chunksPerRow; sNext++; }
+            idPreNext = spk[(uint32_t)min(sNext, (unsigned long long)lastSrc)];
             const size_t rowBase = (size_t)idPre * g.rowStride;
             const uint32_t j = chunk * span + lis * perLane;
             const bool inRow = (j < g.rowStride);
@@ -338,7 +357,7 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
 // with consecutive lanes on consecutive addresses.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(1024)
-void presynapticTileKernel(const TileGroupDev *blocks, unsigned long long *eventCounter)
+void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, unsigned long long *eventCounter)
 {
     extern __shared__ float shTile[];
     const TileGroupDev &G = blocks[blockIdx.x];
@@ -403,7 +422,7 @@ void presynapticTileKernel(const TileGroupDev *blocks, unsigned long long *event
 // kernel footprint touches its output rows, and one wavefront at a time adds a spike's kh*kw*oc contributions
 // into LDS.  The block owns its rows exclusively, so the flush is a plain read-modify-write without atomics.
 __global__ __launch_bounds__(BLOCK)
-void presynapticConvTileKernel(const ConvTileDev *blocks, unsigned long long *eventCounter)
+void presynapticConvTileKernel(const ConvTileDev * __restrict__ blocks, unsigned long long *eventCounter)
 {
     extern __shared__ float shConv[];
     const ConvTileDev &G = blocks[blockIdx.x];
@@ -487,7 +506,7 @@ __global__ void tileOffsetKernel(uint32_t numSrc, uint32_t rowStride, const uint
 }
 
 __global__ __launch_bounds__(BLOCK)
-void presynapticUpdateKernel(const PreGroupDev *blocks, StepArgs args, float dt, unsigned long long *eventCounter)
+void presynapticUpdateKernel(const PreGroupDev * __restrict__ blocks, StepArgs args, float dt, unsigned long long *eventCounter)
 {
     presynapticBody(blocks[blockIdx.x], blockIdx.x, resolve(args, dt), dt, eventCounter);
 }
@@ -497,7 +516,7 @@ void presynapticUpdateKernel(const PreGroupDev *blocks, StepArgs args, float dt,
 // remap (coalesced), gathers g by synapse index.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(BLOCK)
-void postsynapticUpdateKernel(const PostGroupDev *blocks, StepArgs args, float dt)
+void postsynapticUpdateKernel(const PostGroupDev * __restrict__ blocks, StepArgs args, float dt)
 {
     const Resolved st = resolve(args, dt);
     const PostGroupDev &G = blocks[blockIdx.x];
@@ -560,31 +579,58 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
             startSpike = g.startSpike[bi];
         }
         else {
-            float Isyn = 0;
-            l0 = g.var0[bi]; l1 = g.var1[bi];
-            for(uint32_t m = 0; m < g.numPSM; m++) {
-                const gennmi_psm_t &psm = g.psm[m];
-                float linSyn = psm.outPost[bi];
-                if(psm.maxDenDelay) {
-                    // read and clear the front slot of the ring (neuronUpdateGroupMerged.cc:84-101)
-                    const uint32_t ptr = (uint32_t)((st.epoch + 1) % psm.maxDenDelay);
-                    float *front = &psm.denDelay[((size_t)batch * psm.maxDenDelay + ptr) * n + i];
-                    linSyn += *front;
-                    *front = 0.0f;
+            // Every load of this neuron's inputs is issued before the first store: the pointers come out of a
+            // descriptor in memory, so a store in between would force the compiler to re-read the descriptor
+            // and would serialise the loads, and each dependent access costs about a microsecond at the start of
+            // a launch (nothing is cached yet).  Sums keep the reference's order (PSMs, then current sources).
+            float lin[GENNMI_MAX_PSM], front[GENNMI_MAX_PSM], inj[GENNMI_MAX_CS];
+            const uint32_t numPSM = g.numPSM, numCS = g.numCS;
+            l0 = asGlobal(g.var0)[bi]; l1 = asGlobal(g.var1)[bi];
+            #pragma unroll
+            for(uint32_t m = 0; m < GENNMI_MAX_PSM; m++) {
+                lin[m] = 0.0f; front[m] = 0.0f;
+                if(m < numPSM) {
+                    lin[m] = asGlobal(g.psm[m].outPost)[bi];
+                    const uint32_t D = g.psm[m].maxDenDelay;
+                    if(D) { front[m] = asGlobal(g.psm[m].denDelay)[((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i]; }
                 }
-                if(psm.kind == GENNMI_PSM_EXPCURR) {
-                    Isyn += psm.init * linSyn;
-                    linSyn *= psm.expDecay;
-                }
-                else {
-                    Isyn += linSyn;
-                    linSyn = 0.0f;
-                }
-                psm.outPost[bi] = linSyn;
             }
-            for(uint32_t c = 0; c < g.numCS; c++) {
-                const gennmi_cs_t &cs = g.cs[c];
-                Isyn += (cs.kind == GENNMI_CS_DC) ? cs.amp : cs.array[(size_t)(st.epoch % cs.arraySteps) * n + i];
+            #pragma unroll
+            for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) {
+                inj[c] = 0.0f;
+                if(c < numCS) {
+                    inj[c] = (g.cs[c].kind == GENNMI_CS_DC) ? g.cs[c].amp
+                                                            : asGlobal(g.cs[c].array)[(size_t)modStep(st.epoch, g.cs[c].arraySteps) * n + i];
+                }
+            }
+            float Isyn = 0;
+            #pragma unroll
+            for(uint32_t m = 0; m < GENNMI_MAX_PSM; m++) {
+                if(m < numPSM) {
+                    // read and clear the front slot of the ring (neuronUpdateGroupMerged.cc:84-101)
+                    float linSyn = lin[m];
+                    const uint32_t D = g.psm[m].maxDenDelay;
+                    if(D) { linSyn += front[m]; }
+                    if(g.psm[m].kind == GENNMI_PSM_EXPCURR) {
+                        Isyn += g.psm[m].init * linSyn;
+                        linSyn *= g.psm[m].expDecay;
+                    }
+                    else {
+                        Isyn += linSyn;
+                        linSyn = 0.0f;
+                    }
+                    lin[m] = linSyn;
+                }
+            }
+            #pragma unroll
+            for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) { if(c < numCS) { Isyn += inj[c]; } }
+            #pragma unroll
+            for(uint32_t m = 0; m < GENNMI_MAX_PSM; m++) {
+                if(m < numPSM) {
+                    const uint32_t D = g.psm[m].maxDenDelay;
+                    if(D) { asGlobal(g.psm[m].denDelay)[((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i] = 0.0f; }
+                    asGlobal(g.psm[m].outPost)[bi] = lin[m];
+                }
             }
             if(g.model == GENNMI_NEURON_LIF) {
                 if(l1 <= 0.0f) {
@@ -626,7 +672,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
     // keep the user-visible ring pointers current (nothing in the kernels reads them)
     if(localBlock == 0 && batch == 0 && threadIdx.x < g.numPSM) {
         const gennmi_psm_t &psm = g.psm[threadIdx.x];
-        if(psm.maxDenDelay && psm.denDelayPtr) { *psm.denDelayPtr = (uint32_t)((st.epoch + 1) % psm.maxDenDelay); }
+        if(psm.maxDenDelay && psm.denDelayPtr) { *psm.denDelayPtr = modStep(st.epoch + 1, psm.maxDenDelay); }
     }
 
     // ---- ordered compaction --------------------------------------------------------------------
@@ -675,7 +721,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
             const uint32_t s0 = __shfl(z0, src, WAVE), s1 = __shfl(z1, src, WAVE);
             for(uint32_t k = s0 + lane; k < s1; k += WAVE) {
                 const ZeroDelayEntry e = G.zeroEntries[k];
-                const uint32_t slot = (uint32_t)((st.epoch + 2) % e.maxDenDelay);
+                const uint32_t slot = modStep(st.epoch + 2, e.maxDenDelay);
                 atomicAddF32(asGlobal(e.ringElem) + ((size_t)batch * e.maxDenDelay + slot) * e.numTrgNeurons, *asGlobal(e.weight));
             }
         }
@@ -741,7 +787,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
 }
 
 __global__ __launch_bounds__(BLOCK)
-void neuronUpdateKernel(const NeuronGroupDev *blocks, StepArgs args, float dt,
+void neuronUpdateKernel(const NeuronGroupDev * __restrict__ blocks, StepArgs args, float dt,
                         unsigned long long *agg, uint32_t *errorFlag)
 {
     neuronBody(blocks[blockIdx.x], blockIdx.x, gridDim.x, resolve(args, dt), dt, agg, errorFlag);
@@ -753,11 +799,16 @@ void neuronUpdateKernel(const NeuronGroupDev *blocks, StepArgs args, float dt,
 // queue of step t-1 while the neuron update refills the visible one.  Neuron blocks come first so that
 // their look-back chain starts early.
 __global__ __launch_bounds__(BLOCK)
-void stepFusedKernel(const NeuronGroupDev *neuronBlocks, uint32_t numNeuronBlocks, const PreGroupDev *preBlocks,
+void stepFusedKernel(const NeuronGroupDev * __restrict__ neuronBlocks, uint32_t numNeuronBlocks, const PreGroupDev * __restrict__ preBlocks,
                      StepArgs args, float dt, unsigned long long *agg, uint32_t *errorFlag, unsigned long long *eventCounter)
 {
     const Resolved st = resolve(args, dt);
-    if(blockIdx.x < numNeuronBlocks) { neuronBody(neuronBlocks[blockIdx.x], blockIdx.x, numNeuronBlocks, st, dt, agg, errorFlag); }
+    if(blockIdx.x < numNeuronBlocks) {
+        // the neuron blocks are the critical path (other blocks wait for their spike counts): let their
+        // instructions issue ahead of the presynaptic blocks that share the compute unit
+        __builtin_amdgcn_s_setprio(3);
+        neuronBody(neuronBlocks[blockIdx.x], blockIdx.x, numNeuronBlocks, st, dt, agg, errorFlag);
+    }
     else { presynapticBody(preBlocks[blockIdx.x - numNeuronBlocks], blockIdx.x - numNeuronBlocks, st, dt, eventCounter); }
 }
 
@@ -1072,11 +1123,15 @@ int gennmi_runner_finalise(gennmi_runner *r)
     r->neuronBlocks = block;
 
     // Presynaptic launch geometry.  The number of spikes is only known on the device, so every
-    // group gets a fixed share of a block budget and deals its (spike, chunk) work items round-robin.
+    // group gets a fixed number of blocks and deals its (spike, chunk) work items round-robin to their
+    // sub-groups.  A group wants enough sub-groups for ~1.5 % of its source population firing in one step; when
+    // the groups together want more than the budget, it is shared in proportion (work per step scales with
+    // source size x row length, whatever the rates turn out to be).
     block = 0;
     const char *envBudget = getenv("GENNMI_PRESYN_BLOCKS_PER_CU");
     const uint32_t blocksPerCU = envBudget ? std::max(1, atoi(envBudget)) : 4u;
-    const uint32_t maxBlocksPerGroup = std::max(2u, (numCU * blocksPerCU) / std::max<uint32_t>(1u, (uint32_t)r->pre.size()));
+    const uint64_t budget = (uint64_t)numCU * blocksPerCU;
+    std::vector<uint64_t> wantBlocks;
     for(auto &p : r->pre) {
         const uint32_t rowLen = (p.g.matrix == GENNMI_MATRIX_SPARSE) ? p.g.rowStride : (uint32_t)(p.g.conv[0] * p.g.conv[1] * p.g.conv[7]);
         uint32_t W;
@@ -1090,11 +1145,16 @@ int gennmi_runner_finalise(gennmi_runner *r)
                   && W >= 16) ? 1u : 0u;
         const uint32_t span = W * (p.vec4 ? 4u : 1u);
         const uint64_t chunksPerRow = (rowLen + span - 1) / span;
-        // enough sub-groups for ~1.5 % of the source population firing in one step
         const uint64_t wantSubGroups = std::max<uint64_t>(8, ((uint64_t)p.g.numSrcNeurons * chunksPerRow) / 64);
-        uint32_t blocks = (uint32_t)std::min<uint64_t>((wantSubGroups * W + BLOCK - 1) / BLOCK, maxBlocksPerGroup);
+        wantBlocks.push_back(std::min<uint64_t>((wantSubGroups * W + BLOCK - 1) / BLOCK, budget));
+    }
+    uint64_t wantTotal = 0;
+    for(uint64_t w : wantBlocks) { wantTotal += w; }
+    for(size_t k = 0; k < r->pre.size(); k++) {
+        auto &p = r->pre[k];
+        const uint64_t blocks = (wantTotal <= budget) ? wantBlocks[k] : (wantBlocks[k] * budget + wantTotal - 1) / wantTotal;
         p.startBlock = block;
-        p.numBlocks = std::max(1u, blocks);
+        p.numBlocks = (uint32_t)std::max<uint64_t>(1, blocks);
         block += p.numBlocks;
     }
     r->preBlocks = block;
