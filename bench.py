@@ -24,6 +24,14 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # algorithmic bytes per synaptic event: ind 4 + g 4 + fp32 read-modify-write of the target 8 (+ 1 delay byte)
 BYTES_PER_EVENT = {"static": 16, "static_delay": 17, "stdp_trace": 28, "conv2d": 8}
+# HBM bytes per launch of the dominant kernel, from hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each
+# scaled by what the same counter reads for the library's 256 MiB copy kernel); recorded with the commands that
+# produced them in profiles/<kernel>_<workload>.md.  They are measurements of an earlier run of the same workload,
+# not of this one; workloads without an entry report null.
+MEASURED_TRAFFIC_BYTES = {
+    "potjans": {"bytes_per_launch": 5.76e6, "source": "profiles/stepFusedKernel_potjans_full.md (median launch: 3172.6 KiB read + 2447.8 KiB written)"},
+    "izh": {"bytes_per_launch": 2.43e8, "source": "profiles/presynapticTileKernel_izhikevich_1M_full.md (average launch of presynapticTileKernel + presynapticUpdateKernel over the first 500 steps)"},
+}
 
 
 def build_net(name, steps):
@@ -66,6 +74,9 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=None, help="steps of the CPU baseline sample (default: sized for ~10-20 s)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--profile-steps", type=int, default=2000, help="extra steps replayed with HIP event nodes around every kernel (multiple of 100)")
+    ap.add_argument("--yardstick-mib", type=int, default=0,
+                    help="also run the library's plain copy kernel on this many MiB (5 launches, 2x this traffic each), so a "
+                         "hardware-counter run has a kernel of known HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
@@ -145,6 +156,16 @@ def main():
                         "neuron_kernel_avg_us": round(navg * 1e6, 3), "neuron_kernel_gbs": round(neuron_bytes / navg / 1e9, 3)}
             if st["postsyn_launches"]:
                 roofline["postsyn_kernel_avg_us"] = round(st["postsyn_seconds"] / st["postsyn_launches"] * 1e6, 3)
+    if args.yardstick_mib > 0:
+        from genn_amd.genn_model import Array
+        count = args.yardstick_mib * (1 << 20) // 4
+        a, b = Array(count, np.float32, fill=1.0), Array(count, np.float32)
+        for _ in range(5):
+            b.copy_on_device(a)
+        a.free(); b.free()
+    if roofline is not None and args.workload in MEASURED_TRAFFIC_BYTES:
+        roofline["traffic"] = MEASURED_TRAFFIC_BYTES[args.workload]["bytes_per_launch"]
+        roofline["traffic_source"] = MEASURED_TRAFFIC_BYTES[args.workload]["source"]
     model.unload()
 
     # ---- CPU baseline: the single-threaded oracle on the same network, bounded sample from t = 0
@@ -153,16 +174,21 @@ def main():
         from oracle.genn_cpu import OracleNet
         # the reference's CPU backend (and the oracle) has no batch dimension: batch 0 is timed and the figure is per batch
         oracle = OracleNet(net.batch_nets[0] if batch > 1 else net)
-        probe = 20
-        t0 = time.perf_counter()
-        oracle.run(probe)
-        per_step = (time.perf_counter() - t0) / probe
-        cpu_steps = args.cpu_steps or int(max(100, min(args.warmup + args.steps, 15.0 / max(per_step, 1e-6))))
-        ev_before = oracle.events()
-        t0 = time.perf_counter()
-        oracle.run(cpu_steps)
-        cpu_wall = time.perf_counter() - t0
-        cpu_events = oracle.events() - ev_before
+        # activity is not stationary (silent start, bursts), so the sample is bounded by time, not sized from a probe:
+        # blocks of steps until ~12 s of CPU work or the GPU run's step count, whichever comes first
+        cpu_budget_s, block = 12.0, 10
+        limit = args.cpu_steps or (args.warmup + args.steps)
+        cpu_steps, cpu_wall = 0, 0.0
+        while cpu_steps < limit and (args.cpu_steps or cpu_wall < cpu_budget_s):
+            n = min(block, limit - cpu_steps)
+            t0 = time.perf_counter()
+            oracle.run(n)
+            cpu_wall += time.perf_counter() - t0
+            cpu_steps += n
+            if cpu_wall < 1.0:
+                block = min(block * 2, 2000)
+        cpu_events = oracle.events()
+        probe = 0
         cpu = {"value": round(cpu_events / cpu_wall, 1), "unit": "events/s", "cores": 1, "kind": "port",
                "sample": f"steps {probe}..{probe + cpu_steps} of the same network from t=0 ({cpu_events} events in {cpu_wall:.2f} s)",
                "wall_s_per_sim_s": round(cpu_wall / (cpu_steps * net.dt / 1000.0), 3),

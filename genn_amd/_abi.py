@@ -78,6 +78,7 @@ SYMBOLS = {
     "gennmi_memcpy_from_device": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "gennmi_memset": (C.c_int, [C.c_void_p, C.c_int, C.c_size_t]),
     "gennmi_fill_f32": (C.c_int, [C.c_void_p, C.c_float, C.c_size_t]),
+    "gennmi_copy_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "gennmi_synchronize": (C.c_int, []),
     "gennmi_free_device_memory_bytes": (C.c_int, [C.POINTER(C.c_size_t)]),
     "gennmi_abi_struct_sizes": (C.c_int, [C.POINTER(C.c_size_t * 5)]),

@@ -836,6 +836,18 @@ __global__ void advanceStepKernel(StepState *state, unsigned long long steps)
     if(threadIdx.x == 0 && blockIdx.x == 0) { state->timestep += steps; state->epoch += steps; }
 }
 
+// four floats per lane; dwordx4 when both pointers are 16-byte aligned (hipMalloc'd arrays are), else scalar
+__global__ void copyKernel(float *dst, const float *src, size_t n)
+{
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if(i + 4 <= n && ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15) == 0) {
+        *reinterpret_cast<f32x4*>(dst + i) = *reinterpret_cast<const f32x4*>(src + i);
+    }
+    else {
+        for(size_t k = i; k < n && k < i + 4; k++) { dst[k] = src[k]; }
+    }
+}
+
 __global__ void fillKernel(float *p, float v, size_t n)
 {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -963,6 +975,17 @@ int gennmi_fill_f32(float *dev, float value, size_t count)
 {
     if(count) {
         fillKernel<<<dim3((unsigned int)((count + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, 0>>>(dev, value, count);
+        HIP_TRY(hipGetLastError());
+        HIP_TRY(hipDeviceSynchronize());
+    }
+    return GENNMI_OK;
+}
+int gennmi_copy_f32(float *dst, const float *src, size_t count)
+{
+    if(count) {
+        if(!dst || !src) { return fail(GENNMI_EINVAL, "copy_f32: null pointer"); }
+        const size_t lanes = (count + 3) / 4;
+        copyKernel<<<dim3((unsigned int)((lanes + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, 0>>>(dst, src, count);
         HIP_TRY(hipGetLastError());
         HIP_TRY(hipDeviceSynchronize());
     }

@@ -115,6 +115,12 @@ class Array:
             _abi.check(_abi.load().gennmi_memcpy_from_device(self.view.ctypes.data_as(C.c_void_p), self._dev, self.view.nbytes))
         return self.view
 
+    def copy_on_device(self, src):
+        """Device-to-device copy of another fp32 Array of the same length (host views are left alone)."""
+        if self.dtype != np.float32 or src.dtype != np.float32 or src.count != self.count:
+            raise ValueError("copy_on_device needs two float32 arrays of equal length")
+        _abi.check(_abi.load().gennmi_copy_f32(self._dev, src._dev, self.count))
+
     def free(self):
         if self._dev:
             _abi.load().gennmi_free(self._dev)

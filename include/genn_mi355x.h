@@ -62,6 +62,11 @@ int gennmi_memcpy_to_device(void *dev, const void *host, size_t bytes);    /* pu
 int gennmi_memcpy_from_device(void *host, const void *dev, size_t bytes);  /* pullFromDevice / pullSlice1DFromDevice :142-198 */
 int gennmi_memset(void *dev, int value, size_t bytes);          /* memsetDeviceObject :200-204 */
 int gennmi_fill_f32(float *dev, float value, size_t count);     /* e.g. sT = -TIME_MAX (initGroupMerged.cc neuron init) */
+/* Device-to-device copy of `count` floats by a plain kernel (one 16-byte load and store per lane).  No counterpart
+ * in the reference, whose arrays are only copied between host and device; it exists for host code that
+ * snapshots state on the device, and as the traffic yardstick hardware counters are scaled by (a launch moves
+ * exactly 8*count bytes). */
+int gennmi_copy_f32(float *dst, const float *src, size_t count);
 int gennmi_synchronize(void);
 int gennmi_free_device_memory_bytes(size_t *bytes);             /* genReturnFreeDeviceMemoryBytes, backendCUDAHIP.cc */
 /* sizeof() of the five descriptor structs below, in declaration order (psm, cs, neuron update, presynaptic

@@ -180,3 +180,19 @@ def test_spike_recording(make_model, batch_size):
         want = sorted((float(t), i) for i in range(n) for t in spikes[b][i])
         got = sorted(zip(rec_t.tolist(), rec_id.tolist()))
         assert got == want
+
+
+@pytest.mark.parametrize("count", [1, 3, 4, 1023, 1 << 20])
+def test_device_copy(count):
+    """gennmi_copy_f32: every element copied, nothing beyond `count` touched (odd counts take the scalar tail)."""
+    from genn_amd import _abi
+    from genn_amd.genn_model import Array
+    _abi.check(_abi.load().gennmi_init(0))
+    src, dst = Array(count + 8, np.float32), Array(count + 8, np.float32, fill=-1.0)
+    src.view[:] = np.arange(count + 8, dtype=np.float32)
+    src.push_to_device()
+    _abi.check(_abi.load().gennmi_copy_f32(dst.ptr, src.ptr, count))
+    got = dst.pull_from_device()
+    assert np.array_equal(got[:count], src.view[:count])
+    assert np.all(got[count:] == -1.0)
+    src.free(); dst.free()
