@@ -357,7 +357,7 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
 // with consecutive lanes on consecutive addresses.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(1024)
-void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, unsigned long long *eventCounter)
+void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs args, float dt, unsigned long long *eventCounter)
 {
     extern __shared__ float shTile[];
     const TileGroupDev &G = blocks[blockIdx.x];
@@ -373,7 +373,19 @@ void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, unsigned lo
     GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
     GLOBAL_AS const uint16_t *off = asGlobal(G.tileOff);
     GLOBAL_AS const uint32_t *ind = asGlobal(g.ind);
-    GLOBAL_AS const float *weight = asGlobal(g.g);
+    GLOBAL_AS float *weight = asGlobal(g.g);
+    // trace-STDP rows: besides delivering the (old) weight, every event applies the presynaptic-spike rule to its own
+    // synapse (pygenn/genn_model.py:1456-1463); a synapse belongs to exactly one tile, so g needs no atomic here either
+    const bool stdp = (g.wum == GENNMI_WUM_STDP_TRACE);
+    const float t = stdp ? resolve(args, dt).t : 0.0f;
+    GLOBAL_AS const float *trgST = asGlobal(g.trgST);
+    GLOBAL_AS const float *postTrace = asGlobal(g.postTrace);
+    auto depress = [&](uint32_t idPost, float w) -> float {
+        const float stPost = dt + trgST[idPost];
+        const float dtSpike = t - stPost;
+        if(dtSpike > 0) { return fminf(g.wMax, fmaxf(g.wMin, w - (g.aMinus * postTrace[idPost]))); }
+        return w;
+    };
     const uint32_t L = G.lanes;
     const uint32_t lis = threadIdx.x & (L - 1);
     const uint32_t perBlock = blockDim.x / L;
@@ -397,13 +409,23 @@ void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, unsigned lo
             if(j + 4 <= b) {
                 const u32x4u ip = *reinterpret_cast<GLOBAL_AS const u32x4u*>(ind + rowBase + j);
                 const f32x4u w = *reinterpret_cast<GLOBAL_AS const f32x4u*>(weight + rowBase + j);
+                if(stdp) {
+                    f32x4u nw;
+                    nw.x = depress(ip.x, w.x); nw.y = depress(ip.y, w.y); nw.z = depress(ip.z, w.z); nw.w = depress(ip.w, w.w);
+                    *reinterpret_cast<GLOBAL_AS f32x4u*>(weight + rowBase + j) = nw;
+                }
                 unsafeAtomicAdd(&shTile[ip.x - tileStart], w.x);
                 unsafeAtomicAdd(&shTile[ip.y - tileStart], w.y);
                 unsafeAtomicAdd(&shTile[ip.z - tileStart], w.z);
                 unsafeAtomicAdd(&shTile[ip.w - tileStart], w.w);
             }
             else {
-                for(uint32_t jj = j; jj < b; jj++) { unsafeAtomicAdd(&shTile[ind[rowBase + jj] - tileStart], weight[rowBase + jj]); }
+                for(uint32_t jj = j; jj < b; jj++) {
+                    const uint32_t idPost = ind[rowBase + jj];
+                    const float w = weight[rowBase + jj];
+                    if(stdp) { weight[rowBase + jj] = depress(idPost, w); }
+                    unsafeAtomicAdd(&shTile[idPost - tileStart], w);
+                }
             }
         }
         if(lis == 0) { events += b - a; }
@@ -1206,13 +1228,13 @@ int gennmi_runner_finalise(gennmi_runner *r)
         if(e != hipSuccess) { return e; }
         return hipMemcpy(*dTable, table.data(), table.size() * sizeof(table[0]), hipMemcpyHostToDevice);
     };
-    // ---- tile path for static, delay-free SPARSE projections whose rows are sorted by target
+    // ---- tile path for delay-free SPARSE projections (static or trace-STDP weights) whose rows are sorted by target
     {
         const char *envTile = getenv("GENNMI_TILE_FLOATS");
         const uint32_t tileFloats = envTile ? (uint32_t)std::max(0, atoi(envTile)) : 16384u;
         const char *envThreads = getenv("GENNMI_TILE_THREADS");
         r->tileThreads = envThreads ? (uint32_t)std::min(1024, std::max(64, atoi(envThreads))) : (tileFloats > 16384 ? 1024u : (tileFloats > 8192 ? 512u : (uint32_t)BLOCK));
-        std::vector<TileGroupDev> tiles;
+        std::vector<TileGroupDev> tiles, tileGroups;
         std::vector<ConvTileDev> convTiles;
         for(auto &p : r->pre) {
             p.workPerSpike = (p.g.matrix == GENNMI_MATRIX_SPARSE) ? p.g.rowStride : (uint32_t)(p.g.conv[0] * p.g.conv[1] * p.g.conv[7]);
@@ -1236,7 +1258,8 @@ int gennmi_runner_finalise(gennmi_runner *r)
                 }
                 continue;
             }
-            if(tileFloats == 0 || p.g.matrix != GENNMI_MATRIX_SPARSE || p.g.wum != GENNMI_WUM_STATIC_PULSE || p.g.rowStride > 65535) { continue; }
+            if(tileFloats == 0 || p.g.matrix != GENNMI_MATRIX_SPARSE || p.g.rowStride > 65535
+               || (p.g.wum != GENNMI_WUM_STATIC_PULSE && p.g.wum != GENNMI_WUM_STDP_TRACE)) { continue; }
             const uint32_t tileSize = std::min(tileFloats, p.g.numTrgNeurons);
             const uint32_t numTiles = (p.g.numTrgNeurons + tileSize - 1) / tileSize;
             uint16_t *dOff = nullptr; uint32_t *dFlag = nullptr;
@@ -1252,17 +1275,27 @@ int gennmi_runner_finalise(gennmi_runner *r)
             HIP_TRY(hipFree(dFlag));
             if(unsorted) { continue; }          // rows not sorted by target: the scatter kernel handles every step
             p.tileThreshold = std::max(1u, p.g.numTrgNeurons);
-            const char *envSplit = getenv("GENNMI_TILE_BLOCKS_PER_CU");
-            const uint32_t blocksPerCUTile = envSplit ? (uint32_t)std::max(1, atoi(envSplit)) : 4u;
-            const uint32_t numSplits = std::max(1u, std::min(256u, (blocksPerCUTile * numCU * BLOCK / r->tileThreads) / numTiles));
             const uint32_t avgSeg = std::max(1u, p.g.rowStride / numTiles);
             TileGroupDev t{};
-            t.g = p.g; t.tileOff = dOff; t.numTiles = numTiles; t.tileSize = tileSize; t.numSplits = numSplits;
+            t.g = p.g; t.tileOff = dOff; t.numTiles = numTiles; t.tileSize = tileSize;
             t.lanes = std::min<uint32_t>(WAVE, pow2Ceil((avgSeg + 7) / 8)); t.threshold = p.tileThreshold;
-            for(uint32_t tile = 0; tile < numTiles; tile++) {
-                for(uint32_t split = 0; split < numSplits; split++) { t.tile = tile; t.split = split; tiles.push_back(t); }
-            }
+            tileGroups.push_back(t);
             r->tileFloats = std::max(r->tileFloats, tileSize);
+        }
+        if(!tileGroups.empty()) {
+            // Every group gets a whole resident round of the chip (GENNMI_TILE_BLOCKS_PER_CU x 256 threads per compute
+            // unit): activity is bursty, a burst in one projection should find all compute units, and the blocks of
+            // groups whose step went to the scatter kernel leave after reading one counter.
+            const char *envSplit = getenv("GENNMI_TILE_BLOCKS_PER_CU");
+            const uint32_t blocksPerCUTile = envSplit ? (uint32_t)std::max(1, atoi(envSplit)) : 4u;
+            const uint32_t budget = blocksPerCUTile * numCU * BLOCK / r->tileThreads;
+            for(auto &t : tileGroups) {
+                const uint32_t numSplits = std::max(1u, std::min(256u, budget / t.numTiles));
+                t.numSplits = numSplits;
+                for(uint32_t tile = 0; tile < t.numTiles; tile++) {
+                    for(uint32_t split = 0; split < numSplits; split++) { t.tile = tile; t.split = split; tiles.push_back(t); }
+                }
+            }
         }
         if(!convTiles.empty()) {
             HIP_TRY(hipMalloc(&r->dConvTile, convTiles.size() * sizeof(ConvTileDev)));
@@ -1399,7 +1432,7 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
     if(!r->pre.empty()) {
         presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dPre, a, r->dt, r->dEvents);
         if(r->tileBlocks) {
-            presynapticTileKernel<<<dim3(r->tileBlocks, r->batch), dim3(r->tileThreads), r->tileFloats * sizeof(float), r->stream>>>(r->dTile, r->dEvents);
+            presynapticTileKernel<<<dim3(r->tileBlocks, r->batch), dim3(r->tileThreads), r->tileFloats * sizeof(float), r->stream>>>(r->dTile, a, r->dt, r->dEvents);
         }
         if(r->convTileBlocks) {
             presynapticConvTileKernel<<<dim3(r->convTileBlocks, r->batch), dim3(BLOCK), r->convTileBytes, r->stream>>>(r->dConvTile, r->dEvents);
