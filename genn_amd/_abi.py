@@ -8,6 +8,7 @@ import os
 
 MAX_PSM = 8
 MAX_CS = 4
+MAX_EXTRA_SPK = 3
 
 NEURON_LIF, NEURON_IZHIKEVICH, NEURON_SPIKE_SOURCE_ARRAY = 0, 1, 2
 PSM_EXPCURR, PSM_DELTACURR = 0, 1
@@ -42,7 +43,9 @@ class NeuronUpdateGroup(C.Structure):
                 ("psm", Psm * MAX_PSM), ("cs", Cs * MAX_CS),
                 ("preTrace", p_f32), ("postTrace", p_f32),
                 ("preDecay", C.c_float), ("postDecay", C.c_float),
-                ("sT", p_f32), ("spkCnt", p_u32), ("spk", p_u32), ("recordSpk", p_u32)]
+                ("sT", p_f32), ("spkCnt", p_u32), ("spk", p_u32), ("recordSpk", p_u32),
+                ("numExtraSpk", C.c_uint32), ("pad_", C.c_uint32),
+                ("extraSpkCnt", p_u32 * MAX_EXTRA_SPK), ("extraSpk", p_u32 * MAX_EXTRA_SPK)]
 
 
 class PresynapticUpdateGroup(C.Structure):
@@ -79,6 +82,11 @@ SYMBOLS = {
     "gennmi_memset": (C.c_int, [C.c_void_p, C.c_int, C.c_size_t]),
     "gennmi_fill_f32": (C.c_int, [C.c_void_p, C.c_float, C.c_size_t]),
     "gennmi_copy_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "gennmi_register_mirror": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "gennmi_unregister_mirror": (C.c_int, [C.c_void_p]),
+    "gennmi_mirror_device_pointer": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "gennmi_push_mirrors": (C.c_int, []),
+    "gennmi_step": (C.c_int, [C.c_void_p, C.c_float, C.c_uint32]),
     "gennmi_synchronize": (C.c_int, []),
     "gennmi_free_device_memory_bytes": (C.c_int, [C.POINTER(C.c_size_t)]),
     "gennmi_abi_struct_sizes": (C.c_int, [C.POINTER(C.c_size_t * 5)]),

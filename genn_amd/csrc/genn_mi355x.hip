@@ -23,6 +23,8 @@
 #include <cstring>
 #include <string>
 #include <type_traits>
+#include <map>
+#include <mutex>
 #include <vector>
 
 #include "genn_mi355x.h"
@@ -800,6 +802,12 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
     if(prefix == 0xFFFFFFFFu) { return; }       // bounded wait expired: flagged, nothing written
     if(spiked) { g.spk[(size_t)batch * n + prefix + waveOffset + laneRank] = i; }
     if(last && threadIdx.x == 0) { g.spkCnt[batch] = prefix + blockCount; }
+    // further copies of the queue (one population can feed several spike arrays: its own outgoing projections
+    // and, for learnPost, the incoming plastic ones; runtime.cc:267-278)
+    for(uint32_t q = 0; q < g.numExtraSpk; q++) {
+        if(spiked) { g.extraSpk[q][(size_t)batch * n + prefix + waveOffset + laneRank] = i; }
+        if(last && threadIdx.x == 0) { g.extraSpkCnt[q][batch] = prefix + blockCount; }
+    }
     if(G.shadowSpk) {
         const uint32_t parity = (uint32_t)(st.epoch & 1);
         if(spiked) { G.shadowSpk[((size_t)parity * gridDim.y + batch) * n + prefix + waveOffset + laneRank] = i; }
@@ -1014,6 +1022,49 @@ int gennmi_copy_f32(float *dst, const float *src, size_t count)
     return GENNMI_OK;
 }
 int gennmi_synchronize(void) { HIP_TRY(hipDeviceSynchronize()); return GENNMI_OK; }
+
+// ---- host mirrors: host buffer <-> device buffer pairs, for callers whose generated code only knows host pointers
+namespace
+{
+struct Mirror { void *dev; size_t bytes; };
+std::map<uintptr_t, Mirror> g_mirrors;      // keyed by host base address
+std::mutex g_mirrorMutex;
+}
+int gennmi_register_mirror(const void *host, void *dev, size_t bytes)
+{
+    if(!host || !dev || bytes == 0) { return fail(GENNMI_EINVAL, "register_mirror: null pointer or empty buffer"); }
+    std::lock_guard<std::mutex> lock(g_mirrorMutex);
+    g_mirrors[reinterpret_cast<uintptr_t>(host)] = Mirror{dev, bytes};
+    return GENNMI_OK;
+}
+int gennmi_unregister_mirror(const void *host)
+{
+    std::lock_guard<std::mutex> lock(g_mirrorMutex);
+    if(g_mirrors.erase(reinterpret_cast<uintptr_t>(host)) == 0) { return fail(GENNMI_EINVAL, "unregister_mirror: unknown host pointer"); }
+    return GENNMI_OK;
+}
+int gennmi_mirror_device_pointer(const void *host, void **dev)
+{
+    if(!dev) { return fail(GENNMI_EINVAL, "mirror_device_pointer: null result pointer"); }
+    *dev = nullptr;
+    if(!host) { return GENNMI_OK; }        // absent arrays stay absent
+    std::lock_guard<std::mutex> lock(g_mirrorMutex);
+    const uintptr_t h = reinterpret_cast<uintptr_t>(host);
+    auto it = g_mirrors.upper_bound(h);
+    if(it == g_mirrors.begin()) { return fail(GENNMI_EINVAL, "mirror_device_pointer: host pointer is not inside a registered buffer"); }
+    --it;
+    if(h - it->first >= it->second.bytes) { return fail(GENNMI_EINVAL, "mirror_device_pointer: host pointer is not inside a registered buffer"); }
+    *dev = static_cast<char*>(it->second.dev) + (h - it->first);
+    return GENNMI_OK;
+}
+int gennmi_push_mirrors(void)
+{
+    std::lock_guard<std::mutex> lock(g_mirrorMutex);
+    for(const auto &m : g_mirrors) {
+        HIP_TRY(hipMemcpy(m.second.dev, reinterpret_cast<const void*>(m.first), m.second.bytes, hipMemcpyHostToDevice));
+    }
+    return GENNMI_OK;
+}
 int gennmi_free_device_memory_bytes(size_t *bytes)
 {
     size_t total = 0;
@@ -1082,6 +1133,10 @@ int gennmi_push_neuron_update_group(gennmi_runner *r, const gennmi_neuron_update
     for(uint32_t c = 0; c < g->numCS; c++) {
         if(g->cs[c].kind == GENNMI_CS_ARRAY && (!g->cs[c].array || g->cs[c].arraySteps == 0)) { return fail(GENNMI_EINVAL, "push_neuron_update_group: current-source array missing"); }
         if(g->cs[c].kind > GENNMI_CS_ARRAY) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: unknown current source"); }
+    }
+    if(g->numExtraSpk > GENNMI_MAX_EXTRA_SPK) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: too many spike arrays"); }
+    for(uint32_t q = 0; q < g->numExtraSpk; q++) {
+        if(!g->extraSpkCnt[q] || !g->extraSpk[q]) { return fail(GENNMI_EINVAL, "push_neuron_update_group: extra spike array missing"); }
     }
     NeuronGroupDev d;
     memset(&d, 0, sizeof(d));
@@ -1504,9 +1559,15 @@ int gennmi_step_time(gennmi_runner *r, unsigned long long timestep, unsigned lon
     // const float t = timestep * DT  (generateRunner.cc:283)
     const float t = (float)timestep * r->dt;
     const uint32_t recT = numRecordingTimesteps ? (uint32_t)(timestep % numRecordingTimesteps) : 0u;
-    if(r->finalised && r->fusedStep) {
+    return gennmi_step(r, t, recT);
+}
+
+int gennmi_step(gennmi_runner *r, float t, uint32_t recordingTimestep)
+{
+    if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "step: runner not finalised"); }
+    if(r->fusedStep) {
         StepArgs a{};
-        a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recT;
+        a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recordingTimestep;
         hipEvent_t e0 = nullptr, e1 = nullptr;
         if(r->timing) {
             if(r->pending.size() >= 2048) { const int rc = drainTimers(r); if(rc) { return rc; } }
@@ -1518,9 +1579,9 @@ int gennmi_step_time(gennmi_runner *r, unsigned long long timestep, unsigned lon
         r->epoch++;
         return GENNMI_OK;
     }
-    int rc = gennmi_update_synapses(r, t);
+    const int rc = gennmi_update_synapses(r, t);
     if(rc) { return rc; }
-    return gennmi_update_neurons(r, t, recT);
+    return gennmi_update_neurons(r, t, recordingTimestep);
 }
 
 int gennmi_run_steps(gennmi_runner *r, unsigned long long timestep, unsigned long long numSteps, unsigned long long numRecordingTimesteps)

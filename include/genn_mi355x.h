@@ -35,6 +35,7 @@ extern "C" {
 
 #define GENNMI_MAX_PSM 8         /* fused postsynaptic models per neuron group */
 #define GENNMI_MAX_CS  4         /* current sources per neuron group */
+#define GENNMI_MAX_EXTRA_SPK 3   /* spike arrays per neuron group beyond the first */
 
 /* neuron models: include/genn/genn/neuronModels.h:220-257 (LIF), :163-186 (Izhikevich), :274-286 (SpikeSourceArray) */
 enum { GENNMI_NEURON_LIF = 0, GENNMI_NEURON_IZHIKEVICH = 1, GENNMI_NEURON_SPIKE_SOURCE_ARRAY = 2 };
@@ -68,6 +69,16 @@ int gennmi_fill_f32(float *dev, float value, size_t count);     /* e.g. sT = -TI
  * exactly 8*count bytes). */
 int gennmi_copy_f32(float *dst, const float *src, size_t count);
 int gennmi_synchronize(void);
+/* Host mirrors.  GeNN's Runtime serialises HOST pointers into merged-group structs for backends that report
+ * isArrayDeviceObjectRequired() == false (runtime.cc:700-720, 1027-1044) — which lets the generated initialize() /
+ * initializeSparse() run the reference's own host-side initialisation code on those pointers.  An Array
+ * (BackendBase::createArray, hip/backend.cc:61-236) registers its host buffer with the device buffer behind it;
+ * generated code translates a host pointer (anywhere inside a registered buffer) to the device address, and
+ * gennmi_push_mirrors() uploads every registered buffer (end of initialize() / initializeSparse()). */
+int gennmi_register_mirror(const void *host, void *dev, size_t bytes);
+int gennmi_unregister_mirror(const void *host);
+int gennmi_mirror_device_pointer(const void *host, void **dev);   /* NULL host -> NULL device, no error */
+int gennmi_push_mirrors(void);
 int gennmi_free_device_memory_bytes(size_t *bytes);             /* genReturnFreeDeviceMemoryBytes, backendCUDAHIP.cc */
 /* sizeof() of the five descriptor structs below, in declaration order (psm, cs, neuron update, presynaptic
  * update, postsynaptic update), so that a binding in another language can verify its struct layout.  Needs
@@ -116,6 +127,11 @@ typedef struct gennmi_neuron_update_group_t {      /* MergedNeuronUpdateGroup<i>
     uint32_t *spkCnt;                     /* [batch] */
     uint32_t *spk;                        /* [batch*numNeurons], ascending neuron index within a step */
     uint32_t *recordSpk;                  /* [numRecordingTimesteps*batch*ceil(numNeurons/32)] or NULL (runtime.cc:169) */
+    /* further spike arrays that receive the same queue: the reference keeps one srcSpk per fused outgoing spike
+     * owner and one trgSpk per incoming projection with learnPost (runtime.cc:267-278, "SynSpike" children) */
+    uint32_t numExtraSpk, pad_;
+    uint32_t *extraSpkCnt[GENNMI_MAX_EXTRA_SPK];
+    uint32_t *extraSpk[GENNMI_MAX_EXTRA_SPK];
 } gennmi_neuron_update_group_t;
 
 typedef struct gennmi_presynaptic_update_group_t { /* MergedPresynapticUpdateGroup<i> */
@@ -186,6 +202,10 @@ int gennmi_max_col_length(uint32_t numSrcNeurons, uint32_t numTrgNeurons, uint32
  * spike-queue reset and neuron update.  Asynchronous on the runner's stream. */
 int gennmi_update_synapses(gennmi_runner *runner, float t);
 int gennmi_update_neurons(gennmi_runner *runner, float t, uint32_t recordingTimestep);
+/* updateSynapses(t) + updateNeurons(t, recordingTimestep) as one call, which lets delay networks take the
+ * single-launch plan; a generated runner whose stepTime() body is fixed by generateRunner.cc:270-299 defers
+ * updateSynapses and calls this from updateNeurons. */
+int gennmi_step(gennmi_runner *runner, float t, uint32_t recordingTimestep);
 /* stepTime(timestep, numRecordingTimesteps)  generateRunner.cc:270-299 */
 int gennmi_step_time(gennmi_runner *runner, unsigned long long timestep, unsigned long long numRecordingTimesteps);
 /* numSteps consecutive stepTime calls starting at `timestep`, replayed from a captured HIP
