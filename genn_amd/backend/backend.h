@@ -1,0 +1,128 @@
+#pragma once
+// GeNN::CodeGenerator::MI355X::Backend — plugs the MI355X device library (include/genn_mi355x.h) into GeNN's code
+// generator as one more backend (interface: include/genn/genn/code_generator/backendBase.h:127-486; selected like
+// include/genn/backends/single_threaded_cpu/backend.h or hip/backend.h).
+//
+// Division of labour:
+//  * initialize() / initializeSparse() are the reference's own host-side initialisation code, generated through
+//    the generic *InitGroupMerged::generateInit machinery, running on the arrays' host buffers; every buffer is then
+//    uploaded.  Runtime hands merged groups HOST pointers because isArrayDeviceObjectRequired() is false.
+//  * updateSynapses() / updateNeurons() do not run generated model code: each merged update group is recognised as
+//    one of the models the device library implements and translated, once, into a descriptor
+//    (gennmi_*_update_group_t); anything else is rejected at code-generation time with std::runtime_error.
+#include <memory>
+#include <string>
+
+#include "backendExport.h"
+#include "code_generator/backendBase.h"
+#include "code_generator/environment.h"
+
+namespace filesystem { class path; }
+
+namespace GeNN::CodeGenerator::MI355X
+{
+struct Preferences : public PreferencesBase
+{
+    //! HIP device ordinal handed to gennmi_init() by the generated allocateMem()
+    int deviceID = 0;
+
+    //! Where the generated Makefile finds genn_mi355x.h and libgenn_mi355x.so
+    //! (empty: the GENN_MI355X_ROOT environment variable at code-generation time)
+    std::string installRoot;
+
+    void updateHash(boost::uuids::detail::sha1 &hash) const
+    {
+        PreferencesBase::updateHash(hash);
+        Utils::updateHash(deviceID, hash);
+    }
+};
+
+class State : public Runtime::StateBase
+{
+};
+
+class BACKEND_EXPORT Backend : public BackendBase
+{
+public:
+    Backend(const Preferences &preferences);
+
+    //--------------------------------------------------------------------------
+    // BackendBase virtuals
+    //--------------------------------------------------------------------------
+    virtual void genNeuronUpdate(CodeStream &os, FileStreamCreator streamCreator, ModelSpecMerged &modelMerged,
+                                 BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const final;
+    virtual void genSynapseUpdate(CodeStream &os, FileStreamCreator streamCreator, ModelSpecMerged &modelMerged,
+                                  BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const final;
+    virtual void genCustomUpdate(CodeStream &os, FileStreamCreator streamCreator, ModelSpecMerged &modelMerged,
+                                 BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const final;
+    virtual void genInit(CodeStream &os, FileStreamCreator streamCreator, ModelSpecMerged &modelMerged,
+                         BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const final;
+
+    virtual size_t getSynapticMatrixRowStride(const SynapseGroupInternal &sg) const final;
+
+    virtual void genDefinitionsPreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const final;
+    virtual void genRunnerPreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const final;
+    virtual void genAllocateMemPreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const final;
+    virtual void genFreeMemPreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const final;
+    virtual void genStepTimeFinalisePreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const final;
+
+    virtual std::unique_ptr<GeNN::Runtime::StateBase> createState(const Runtime::Runtime &runtime) const final;
+    virtual std::unique_ptr<Runtime::ArrayBase> createArray(const Type::ResolvedType &type, size_t count,
+                                                            VarLocation location, bool uninitialized) const final;
+    virtual std::unique_ptr<Runtime::ArrayBase> createPopulationRNG(size_t count) const final;
+
+    virtual void genLazyVariableDynamicAllocation(CodeStream &os, const Type::ResolvedType &type, const std::string &name,
+                                                  VarLocation loc, const std::string &countVarName) const final;
+    virtual void genLazyVariableDynamicPush(CodeStream &os, const Type::ResolvedType &type, const std::string &name,
+                                            VarLocation loc, const std::string &countVarName) const final;
+    virtual void genLazyVariableDynamicPull(CodeStream &os, const Type::ResolvedType &type, const std::string &name,
+                                            VarLocation loc, const std::string &countVarName) const final;
+    virtual void genMergedDynamicVariablePush(CodeStream &os, const std::string &suffix, size_t mergedGroupIdx,
+                                              const std::string &groupIdx, const std::string &fieldName,
+                                              const std::string &egpName) const final;
+
+    virtual void genPopVariableInit(EnvironmentExternalBase &env, HandlerEnv handler) const final;
+    virtual void genVariableInit(EnvironmentExternalBase &env, const std::string &count, const std::string &indexVarName,
+                                 HandlerEnv handler) const final;
+    virtual void genSparseSynapseVariableRowInit(EnvironmentExternalBase &env, HandlerEnv handler) const final;
+    virtual void genDenseSynapseVariableRowInit(EnvironmentExternalBase &env, HandlerEnv handler) const final;
+    virtual void genKernelSynapseVariableInit(EnvironmentExternalBase &env, SynapseInitGroupMerged &sg, HandlerEnv handler) const final;
+    virtual void genKernelCustomUpdateVariableInit(EnvironmentExternalBase &env, CustomWUUpdateInitGroupMerged &cu, HandlerEnv handler) const final;
+
+    virtual std::string getAtomicOperation(const std::string &lhsPointer, const std::string &rhsValue,
+                                           const Type::ResolvedType &type, AtomicOperation op = AtomicOperation::ADD) const final;
+    virtual std::string getRestrictKeyword() const final { return " __restrict__"; }
+
+    virtual void genGlobalDeviceRNG(CodeStream &definitions, CodeStream &runner, CodeStream &allocations, CodeStream &free) const final;
+    virtual void genTimer(CodeStream &definitions, CodeStream &runner, CodeStream &allocations, CodeStream &free,
+                          CodeStream &stepTimeFinalise, const std::string &name, bool updateInStepTime) const final;
+    virtual void genReturnFreeDeviceMemoryBytes(CodeStream &os) const final;
+    virtual void genAssert(CodeStream &os, const std::string &condition) const final;
+
+    virtual bool shouldUseNMakeBuildSystem() const final { return false; }
+    virtual void genMakefilePreamble(std::ostream &os) const final;
+    virtual void genMakefileLinkRule(std::ostream &os) const final;
+    virtual void genMakefileCompileRule(std::ostream &os) const final;
+    virtual void genNMakefilePreamble(std::ostream &os) const final;
+    virtual void genNMakefileLinkRule(std::ostream &os) const final;
+    virtual void genNMakefileCompileRule(std::ostream &os) const final;
+    virtual void genMSBuildConfigProperties(std::ostream &os) const final;
+    virtual void genMSBuildImportProps(std::ostream &os) const final;
+    virtual void genMSBuildItemDefinitions(std::ostream &os) const final;
+    virtual void genMSBuildCompileModule(const std::string &moduleName, std::ostream &os) const final;
+    virtual void genMSBuildImportTarget(std::ostream &os) const final;
+
+    //! Merged groups are given host pointers (see the header comment); generated code maps them to device addresses
+    virtual bool isArrayDeviceObjectRequired() const final { return false; }
+    virtual bool isArrayHostObjectRequired() const final { return false; }
+    virtual bool isGlobalHostRNGRequired(const ModelSpecInternal &model) const final;
+    virtual bool isGlobalDeviceRNGRequired(const ModelSpecInternal &model) const final { return false; }
+    virtual bool isPopulationRNGInitialisedOnDevice() const final { return false; }
+    //! learnPost walks columns through colLength / remap (built by gennmi_build_remap in initializeSparse())
+    virtual bool isPostsynapticRemapRequired() const final { return true; }
+    virtual bool isHostReductionRequired() const final { return false; }
+    virtual size_t getDeviceMemoryBytes() const final;
+    virtual MemorySpaces getMergedGroupMemorySpaces(const ModelSpecMerged &modelMerged) const final { return {}; }
+    virtual boost::uuids::detail::sha1::digest_type getHashDigest() const final;
+};
+}   // namespace GeNN::CodeGenerator::MI355X
