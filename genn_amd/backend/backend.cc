@@ -217,3 +217,883 @@ std::string tableU32(const std::vector<uint64_t> &values)
     return os.str();
 }
 }   // anonymous namespace
+
+//--------------------------------------------------------------------------
+// GeNN::CodeGenerator::MI355X::Backend
+//--------------------------------------------------------------------------
+namespace GeNN::CodeGenerator::MI355X
+{
+Backend::Backend(const Preferences &preferences)
+:   BackendBase(preferences)
+{
+}
+//--------------------------------------------------------------------------
+// updateNeurons: one descriptor per group of every merged neuron update group, built once by
+// gennmiBuildNeuronGroups(); the call itself advances the whole timestep (see gennmi_step)
+//--------------------------------------------------------------------------
+void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelMerged,
+                              BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const
+{
+    const ModelSpecInternal &model = modelMerged.getModel();
+    const unsigned int batchSize = model.getBatchSize();
+    const auto scalar = model.getPrecision();
+    if(scalar != Type::Float || model.getTimePrecision() != Type::Float) {
+        throw std::runtime_error("MI355X backend: only single-precision models are supported");
+    }
+
+    std::ostringstream bodyStream;
+    CodeStream body(bodyStream);
+    EnvironmentLibrary libEnv(body, StandardLibrary::getMathsFunctions());
+
+    body << "void gennmiBuildNeuronGroups()";
+    {
+        CodeStream::Scope b(body);
+        EnvironmentExternal funcEnv(libEnv);
+        modelMerged.genMergedNeuronUpdateGroups(
+            *this, memorySpaces,
+            [this, &funcEnv, batchSize, scalar](auto &n)
+            {
+                const auto &arch = n.getArchetype();
+                const size_t numGroups = n.getGroups().size();
+                const unsigned int neuronModel = recogniseNeuron(arch.getModel(), arch.getName());
+                if(arch.isDelayRequired()) { unsupported("axonal or back-propagation delay on population '" + arch.getName() + "'"); }
+                if(arch.isSimRNGRequired()) { unsupported("random numbers in the update of population '" + arch.getName() + "'"); }
+                if(arch.isPrevSpikeTimeRequired()) { unsupported("previous spike times of population '" + arch.getName() + "'"); }
+                if(!n.getMergedSpikeEventGroups().empty()) { unsupported("spike-like events of population '" + arch.getName() + "'"); }
+                if(!n.getMergedOutSynPreOutputGroups().empty()) { unsupported("presynaptic output into population '" + arch.getName() + "'"); }
+
+                // values of one quantity across the groups of this merged group
+                auto perGroup = [&n](auto fn)
+                {
+                    std::vector<Type::NumericValue> v;
+                    for(const auto &g : n.getGroups()) { v.push_back(fn(g.get())); }
+                    return v;
+                };
+
+                CodeStream::Scope b(funcEnv.getStream());
+                funcEnv.getStream() << "// merged neuron update group " << n.getIndex() << std::endl;
+                funcEnv.getStream() << "for(unsigned int g = 0; g < " << numGroups << "; g++)";
+                CodeStream::Scope b2(funcEnv.getStream());
+                funcEnv.getStream() << "const auto *group = &mergedNeuronUpdateGroup" << n.getIndex() << "[g];" << std::endl;
+                EnvironmentGroupMergedField<NeuronUpdateGroupMerged> env(funcEnv, n);
+                buildStandardEnvironment(env, batchSize);
+                CodeStream &out = env.getStream();
+
+                // pointer fields of the merged struct, added under the names the reference's own backends use
+                auto var = [&env](const std::string &name, const Type::ResolvedType &type, bool dynamic = false)
+                {
+                    env.addField(type.createPointer(), "_mi_" + name, name,
+                                 [name](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, name); },
+                                 "", dynamic ? GroupMergedFieldType::DYNAMIC : GroupMergedFieldType::STANDARD);
+                    return "gennmiDev(" + env["_mi_" + name] + ")";
+                };
+
+                out << "gennmi_neuron_update_group_t d = {};" << std::endl;
+                out << "d.model = " << neuronModel << "u;" << std::endl;
+                out << "static const uint32_t numNeurons[] = " << tableU32([&n]{ std::vector<uint64_t> v; for(const auto &g : n.getGroups()) { v.push_back(g.get().getNumNeurons()); } return v; }()) << ";" << std::endl;
+                out << "d.numNeurons = numNeurons[g];" << std::endl;
+
+                std::vector<std::string> paramNames;
+                if(neuronModel == GENNMI_NEURON_LIF) {
+                    out << "d.var0 = " << var("V", scalar) << "; d.var1 = " << var("RefracTime", scalar) << ";" << std::endl;
+                    paramNames = {"Ioffset", "Rmembrane", "Vrest", "ExpTC", "Vthresh", "Vreset", "TauRefrac"};
+                }
+                else if(neuronModel == GENNMI_NEURON_IZHIKEVICH) {
+                    out << "d.var0 = " << var("V", scalar) << "; d.var1 = " << var("U", scalar) << ";" << std::endl;
+                    paramNames = {"a", "b", "c", "d"};
+                }
+                else {
+                    out << "d.startSpike = " << var("startSpike", Type::Uint32) << "; d.endSpike = " << var("endSpike", Type::Uint32) << ";" << std::endl;
+                    out << "d.spikeTimes = " << var("spikeTimes", scalar, true) << ";" << std::endl;
+                }
+                for(size_t k = 0; k < paramNames.size(); k++) {
+                    const std::string &p = paramNames[k];
+                    out << "{ static const float v[] = " << table(perGroup([&p](const NeuronGroupInternal &g)
+                        {
+                            const auto it = g.getParams().find(p);
+                            return (it != g.getParams().end()) ? it->second : g.getDerivedParams().at(p);
+                        }), scalar) << "; d.params[" << k << "] = v[g]; }" << std::endl;
+                }
+
+                // fused postsynaptic models, in the order the reference applies them
+                const auto &psms = n.getMergedInSynPSMGroups();
+                if(psms.size() > GENNMI_MAX_PSM) { unsupported("more than 8 postsynaptic models on population '" + arch.getName() + "'"); }
+                out << "d.numPSM = " << psms.size() << "u;" << std::endl;
+                for(size_t k = 0; k < psms.size(); k++) {
+                    auto &child = const_cast<NeuronUpdateGroupMerged::InSynPSM&>(psms[k]);
+                    const auto &sg = child.getArchetype();
+                    const unsigned int kind = recognisePSM(sg.getPSInitialiser().getSnippet(), sg.getName());
+                    if(sg.getPostTargetVar() != "Isyn") { unsupported("postsynaptic target variable '" + sg.getPostTargetVar() + "'"); }
+                    const std::string sfx = "InSyn" + std::to_string(child.getIndex());
+                    const std::string dst = "d.psm[" + std::to_string(k) + "]";
+                    EnvironmentGroupMergedField<NeuronUpdateGroupMerged::InSynPSM, NeuronUpdateGroupMerged> penv(env, child, n);
+                    auto childPtr = [&penv, &sfx](const std::string &name, const Type::ResolvedType &type)
+                    {
+                        penv.addField(type.createPointer(), "_mi_" + name, name + sfx,
+                                      [name](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, name); });
+                        return "gennmiDev(" + penv["_mi_" + name] + ")";
+                    };
+                    auto childValues = [&child](auto fn)
+                    {
+                        std::vector<Type::NumericValue> v;
+                        for(const auto &g : child.getGroups()) { v.push_back(fn(g.get())); }
+                        return v;
+                    };
+                    CodeStream &pout = penv.getStream();
+                    pout << dst << ".outPost = " << childPtr("outPost", scalar) << "; " << dst << ".kind = " << kind << "u;" << std::endl;
+                    if(sg.isDendriticOutputDelayRequired()) {
+                        pout << dst << ".denDelay = " << childPtr("denDelay", scalar) << "; " << dst << ".denDelayPtr = " << childPtr("denDelayPtr", Type::Uint32) << ";" << std::endl;
+                        pout << "{ static const uint32_t v[] = " << tableU32([&child]{ std::vector<uint64_t> v; for(const auto &g : child.getGroups()) { v.push_back(g.get().getMaxDendriticDelayTimesteps()); } return v; }())
+                             << "; " << dst << ".maxDenDelay = v[g]; }" << std::endl;
+                    }
+                    if(kind == GENNMI_PSM_EXPCURR) {
+                        for(const char *p : {"init", "expDecay"}) {
+                            pout << "{ static const float v[] = " << table(childValues([p](const SynapseGroupInternal &g){ return g.getPSInitialiser().getDerivedParams().at(p); }), scalar)
+                                 << "; " << dst << "." << p << " = v[g]; }" << std::endl;
+                        }
+                    }
+                }
+
+                // current sources
+                const auto &css = n.getMergedCurrentSourceGroups();
+                if(css.size() > GENNMI_MAX_CS) { unsupported("more than 4 current sources on population '" + arch.getName() + "'"); }
+                out << "d.numCS = " << css.size() << "u;" << std::endl;
+                for(size_t k = 0; k < css.size(); k++) {
+                    auto &child = const_cast<NeuronUpdateGroupMerged::CurrentSource&>(css[k]);
+                    const auto &cs = child.getArchetype();
+                    const std::string dst = "d.cs[" + std::to_string(k) + "]";
+                    if(cs.getTargetVar() != "Isyn") { unsupported("current source target variable '" + cs.getTargetVar() + "'"); }
+                    EnvironmentGroupMergedField<NeuronUpdateGroupMerged::CurrentSource, NeuronUpdateGroupMerged> cenv(env, child, n);
+                    CodeStream &cout = cenv.getStream();
+                    if(same(cs.getModel()->getInjectionCode(), CurrentSourceModels::DC::getInstance()->getInjectionCode())) {
+                        std::vector<Type::NumericValue> amps;
+                        for(const auto &g : child.getGroups()) { amps.push_back(g.get().getParams().at("amp")); }
+                        cout << "{ static const float v[] = " << table(amps, scalar) << "; " << dst << ".kind = " << GENNMI_CS_DC << "u; " << dst << ".amp = v[g]; }" << std::endl;
+                    }
+                    // one value per neuron read from an array the host refills before every step
+                    else if(same(cs.getModel()->getInjectionCode(), "injectCurrent(noise[id]);") && cs.getModel()->getExtraGlobalParams().size() == 1) {
+                        cenv.addField(scalar.createPointer(), "_mi_noise", "noiseCS" + std::to_string(child.getIndex()),
+                                      [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, "noise"); },
+                                      "", GroupMergedFieldType::DYNAMIC);
+                        cout << dst << ".kind = " << GENNMI_CS_ARRAY << "u; " << dst << ".arraySteps = 1u; " << dst << ".array = gennmiDev(" << cenv["_mi_noise"] << ");" << std::endl;
+                    }
+                    else {
+                        unsupported("current source model of '" + cs.getName() + "'");
+                    }
+                }
+
+                // trace variables of plastic projections leaving / entering the population
+                const auto &wuPre = n.getMergedOutSynWUMPreCodeGroups();
+                const auto &wuPost = n.getMergedInSynWUMPostCodeGroups();
+                if(wuPre.size() > 1 || wuPost.size() > 1) { unsupported("more than one plastic projection per side of population '" + arch.getName() + "'"); }
+                if(!wuPre.empty()) {
+                    auto &child = const_cast<NeuronUpdateGroupMerged::OutSynWUMPreCode&>(wuPre[0]);
+                    if(!isTraceSTDP(child.getArchetype().getWUInitialiser().getSnippet())) { unsupported("presynaptic weight-update code of '" + child.getArchetype().getName() + "'"); }
+                    EnvironmentGroupMergedField<NeuronUpdateGroupMerged::OutSynWUMPreCode, NeuronUpdateGroupMerged> wenv(env, child, n);
+                    wenv.addField(scalar.createPointer(), "_mi_preTrace", "preTraceOutSynWUMPre" + std::to_string(child.getIndex()),
+                                  [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, "preTrace"); });
+                    std::vector<Type::NumericValue> decay;
+                    for(const auto &g : child.getGroups()) { decay.push_back(g.get().getWUInitialiser().getDerivedParams().at("tauPlusDecay")); }
+                    wenv.getStream() << "{ static const float v[] = " << table(decay, scalar) << "; d.preTrace = gennmiDev(" << wenv["_mi_preTrace"] << "); d.preDecay = v[g]; }" << std::endl;
+                }
+                if(!wuPost.empty()) {
+                    auto &child = const_cast<NeuronUpdateGroupMerged::InSynWUMPostCode&>(wuPost[0]);
+                    if(!isTraceSTDP(child.getArchetype().getWUInitialiser().getSnippet())) { unsupported("postsynaptic weight-update code of '" + child.getArchetype().getName() + "'"); }
+                    EnvironmentGroupMergedField<NeuronUpdateGroupMerged::InSynWUMPostCode, NeuronUpdateGroupMerged> wenv(env, child, n);
+                    wenv.addField(scalar.createPointer(), "_mi_postTrace", "postTraceInSynWUMPost" + std::to_string(child.getIndex()),
+                                  [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, "postTrace"); });
+                    std::vector<Type::NumericValue> decay;
+                    for(const auto &g : child.getGroups()) { decay.push_back(g.get().getWUInitialiser().getDerivedParams().at("tauMinusDecay")); }
+                    wenv.getStream() << "{ static const float v[] = " << table(decay, scalar) << "; d.postTrace = gennmiDev(" << wenv["_mi_postTrace"] << "); d.postDecay = v[g]; }" << std::endl;
+                }
+
+                // spike arrays: the first is the queue proper, the others receive copies
+                const auto &spikes = n.getMergedSpikeGroups();
+                if(spikes.size() > 1 + GENNMI_MAX_EXTRA_SPK) { unsupported("more than 4 spike arrays on population '" + arch.getName() + "'"); }
+                for(size_t k = 0; k < spikes.size(); k++) {
+                    auto &child = const_cast<NeuronUpdateGroupMerged::SynSpike&>(spikes[k]);
+                    const std::string sfx = "SynSpike" + std::to_string(child.getIndex());
+                    EnvironmentGroupMergedField<NeuronUpdateGroupMerged::SynSpike, NeuronUpdateGroupMerged> senv(env, child, n);
+                    senv.addField(Type::Uint32.createPointer(), "_mi_spkCnt", "spkCnt" + sfx,
+                                  [&n](const auto &runtime, const auto &g, size_t i) { return runtime.getFusedEventArray(n, i, g, "SpkCnt"); });
+                    senv.addField(Type::Uint32.createPointer(), "_mi_spk", "spk" + sfx,
+                                  [&n](const auto &runtime, const auto &g, size_t i) { return runtime.getFusedEventArray(n, i, g, "Spk"); });
+                    const std::string cnt = "gennmiDev(" + senv["_mi_spkCnt"] + ")", spk = "gennmiDev(" + senv["_mi_spk"] + ")";
+                    if(k == 0) {
+                        senv.getStream() << "d.spkCnt = " << cnt << "; d.spk = " << spk << ";" << std::endl;
+                    }
+                    else {
+                        senv.getStream() << "d.extraSpkCnt[" << (k - 1) << "] = " << cnt << "; d.extraSpk[" << (k - 1) << "] = " << spk << ";" << std::endl;
+                    }
+                }
+                if(spikes.empty()) {
+                    // nothing reads this population's spikes: the kernel still needs a queue to write
+                    out << "d.spkCnt = gennmiScratch(" << batchSize << "u * (numNeurons[g] + 1u)); d.spk = d.spkCnt + " << batchSize << "u;" << std::endl;
+                }
+                else {
+                    out << "d.numExtraSpk = " << (spikes.size() - 1) << "u;" << std::endl;
+                }
+                if(arch.isSpikeTimeRequired()) { out << "d.sT = gennmiDev(" << env["_st"] << ");" << std::endl; }
+                if(arch.isSpikeRecordingEnabled()) { out << "d.recordSpk = gennmiDev(" << env["_record_spk"] << ");" << std::endl; }
+                out << "GENNMI_CHECK(gennmi_push_neuron_update_group(gennmiRunner, &d, nullptr));" << std::endl;
+            });
+    }
+    body << std::endl;
+
+    body << "void updateNeurons(" << model.getTimePrecision().getName() << " t";
+    if(model.isRecordingInUse()) {
+        body << ", unsigned int recordingTimestep";
+    }
+    body << ")";
+    {
+        CodeStream::Scope b(body);
+        body << "gennmiEnsureFinalised();" << std::endl;
+        body << "GENNMI_CHECK(gennmi_step(gennmiRunner, t, " << (model.isRecordingInUse() ? "recordingTimestep" : "0u") << "));" << std::endl;
+    }
+
+    modelMerged.genMergedNeuronUpdateGroupStructs(os, *this);
+    modelMerged.genMergedNeuronUpdateGroupHostStructArrayPush(os, *this);
+    preambleHandler(os);
+    os << bodyStream.str();
+}
+//--------------------------------------------------------------------------
+// updateSynapses: descriptors for presynaptic and postsynaptic update groups.  The call itself only notes that
+// the synaptic half of the step is due; gennmi_step() runs both halves from updateNeurons() (stepTime() always
+// calls the two back to back, generateRunner.cc:270-299), which lets delay networks use a single launch.
+//--------------------------------------------------------------------------
+void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelMerged,
+                               BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const
+{
+    const ModelSpecInternal &model = modelMerged.getModel();
+    const unsigned int batchSize = model.getBatchSize();
+    const auto scalar = model.getPrecision();
+
+    std::ostringstream bodyStream;
+    CodeStream body(bodyStream);
+    EnvironmentLibrary libEnv(body, StandardLibrary::getMathsFunctions());
+
+    body << "void gennmiBuildSynapseGroups()";
+    {
+        CodeStream::Scope b(body);
+        EnvironmentExternal funcEnv(libEnv);
+
+        modelMerged.genMergedSynapseDynamicsGroups(
+            *this, memorySpaces,
+            [](auto &s) { unsupported("synapse dynamics code of projection '" + s.getArchetype().getName() + "'"); });
+
+        modelMerged.genMergedPresynapticUpdateGroups(
+            *this, memorySpaces,
+            [this, &funcEnv, batchSize, scalar](auto &s)
+            {
+                const auto &arch = s.getArchetype();
+                const auto *wum = arch.getWUInitialiser().getSnippet();
+                const unsigned int wumKind = recogniseWUM(wum, arch.getName());
+                if(arch.getAxonalDelaySteps() != 0 || arch.getSrcNeuronGroup()->isDelayRequired() || arch.getTrgNeuronGroup()->isDelayRequired()) {
+                    unsupported("axonal or back-propagation delay on projection '" + arch.getName() + "'");
+                }
+                if(arch.isPreSpikeEventRequired() || arch.isPostSpikeEventRequired()) { unsupported("spike-like events on projection '" + arch.getName() + "'"); }
+                if(wumKind == GENNMI_WUM_STDP_TRACE && batchSize != 1) { unsupported("plastic weights with a batch size above 1"); }
+
+                const auto matrixType = arch.getMatrixType();
+                const bool sparse = (matrixType & SynapseMatrixConnectivity::SPARSE) && (matrixType & SynapseMatrixWeight::INDIVIDUAL);
+                const bool toeplitz = (matrixType & SynapseMatrixConnectivity::TOEPLITZ) && (matrixType & SynapseMatrixWeight::KERNEL);
+                if(!sparse && !toeplitz) { unsupported("matrix type of projection '" + arch.getName() + "' (SPARSE with individual weights or TOEPLITZ with kernel weights)"); }
+                if(sparse && arch.getSparseIndType() != Type::Uint32) { unsupported("narrow sparse index type of projection '" + arch.getName() + "'"); }
+                if(toeplitz) {
+                    const auto *conn = arch.getToeplitzConnectivityInitialiser().getSnippet();
+                    if(conn != InitToeplitzConnectivitySnippet::Conv2D::getInstance() || wumKind != GENNMI_WUM_STATIC_PULSE) {
+                        unsupported("Toeplitz connectivity of projection '" + arch.getName() + "' (Conv2D with StaticPulse)");
+                    }
+                }
+
+                CodeStream::Scope b(funcEnv.getStream());
+                funcEnv.getStream() << "// merged presynaptic update group " << s.getIndex() << std::endl;
+                funcEnv.getStream() << "for(unsigned int g = 0; g < " << s.getGroups().size() << "; g++)";
+                CodeStream::Scope b2(funcEnv.getStream());
+                funcEnv.getStream() << "const auto *group = &mergedPresynapticUpdateGroup" << s.getIndex() << "[g];" << std::endl;
+                EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> env(funcEnv, s);
+                buildStandardEnvironment(env, batchSize);
+                CodeStream &out = env.getStream();
+
+                auto values = [&s](auto fn)
+                {
+                    std::vector<Type::NumericValue> v;
+                    for(const auto &g : s.getGroups()) { v.push_back(fn(g.get())); }
+                    return v;
+                };
+                auto counts = [&s](auto fn)
+                {
+                    std::vector<uint64_t> v;
+                    for(const auto &g : s.getGroups()) { v.push_back(fn(g.get())); }
+                    return v;
+                };
+                auto wuVar = [&env](const std::string &name, const Type::ResolvedType &type)
+                {
+                    env.addField(type.createPointer(), "_mi_" + name, name,
+                                 [name](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, name); });
+                    return "gennmiDev(" + env["_mi_" + name] + ")";
+                };
+
+                out << "gennmi_presynaptic_update_group_t d = {};" << std::endl;
+                out << "d.matrix = " << (sparse ? GENNMI_MATRIX_SPARSE : GENNMI_MATRIX_TOEPLITZ_CONV2D) << "u; d.wum = " << wumKind << "u;" << std::endl;
+                if(arch.getParallelismHint() == SynapseGroup::ParallelismHint::PRESYNAPTIC) {
+                    out << "d.span = " << GENNMI_SPAN_PRE << "u; d.numThreadsPerSpike = " << arch.getNumThreadsPerSpike() << "u;" << std::endl;
+                }
+                else {
+                    out << "d.span = " << GENNMI_SPAN_AUTO << "u;" << std::endl;
+                }
+                out << "{ static const uint32_t a[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getSrcNeuronGroup()->getNumNeurons(); }))
+                    << ", b[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getTrgNeuronGroup()->getNumNeurons(); }))
+                    << ", c[] = " << tableU32(counts([this](const SynapseGroupInternal &g){ return getSynapticMatrixRowStride(g); }))
+                    << "; d.numSrcNeurons = a[g]; d.numTrgNeurons = b[g]; d.rowStride = c[g]; }" << std::endl;
+                out << "d.srcSpkCnt = gennmiDev(" << env["_src_spk_cnt"] << "); d.srcSpk = gennmiDev(" << env["_src_spk"] << ");" << std::endl;
+                out << "d.outPost = gennmiDev(" << env["_out_post"] << "); d.g = " << wuVar("g", scalar) << ";" << std::endl;
+                if(sparse) {
+                    out << "d.rowLength = gennmiDev(" << env["_row_length"] << "); d.ind = gennmiDev(" << env["_ind"] << ");" << std::endl;
+                }
+                else {
+                    const auto &names = std::vector<std::string>{"conv_kh", "conv_kw", "conv_ih", "conv_iw", "conv_ic", "conv_oh", "conv_ow", "conv_oc"};
+                    for(size_t k = 0; k < names.size(); k++) {
+                        out << "{ static const int32_t v[] = " << tableU32(counts([&names, k](const SynapseGroupInternal &g)
+                            { return (uint64_t)g.getToeplitzConnectivityInitialiser().getParams().at(names[k]).template cast<int>(); }))
+                            << "; d.conv[" << k << "] = v[g]; }" << std::endl;
+                    }
+                }
+                if(wumKind == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY) {
+                    out << "d.d = " << wuVar("d", Type::Uint8) << "; d.denDelay = gennmiDev(" << env["_den_delay"] << "); d.denDelayPtr = gennmiDev(" << env["_den_delay_ptr"] << ");" << std::endl;
+                    out << "{ static const uint32_t v[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getMaxDendriticDelayTimesteps(); })) << "; d.maxDenDelay = v[g]; }" << std::endl;
+                }
+                if(wumKind == GENNMI_WUM_STDP_TRACE) {
+                    env.addField(scalar.createPointer(), "_mi_postTrace", "postTrace",
+                                 [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g.getFusedWUPostTarget(), "postTrace"); });
+                    out << "d.trgST = gennmiDev(" << env["_trg_st"] << "); d.postTrace = gennmiDev(" << env["_mi_postTrace"] << ");" << std::endl;
+                    for(const char *p : {"aMinus", "wMin", "wMax"}) {
+                        out << "{ static const float v[] = " << table(values([p](const SynapseGroupInternal &g){ return g.getWUInitialiser().getParams().at(p); }), scalar)
+                            << "; d." << p << " = v[g]; }" << std::endl;
+                    }
+                }
+                out << "GENNMI_CHECK(gennmi_push_presynaptic_update_group(gennmiRunner, &d, nullptr));" << std::endl;
+            });
+
+        modelMerged.genMergedPostsynapticUpdateGroups(
+            *this, memorySpaces,
+            [this, &funcEnv, batchSize, scalar](auto &s)
+            {
+                const auto &arch = s.getArchetype();
+                if(!isTraceSTDP(arch.getWUInitialiser().getSnippet())) { unsupported("postsynaptic-spike code of projection '" + arch.getName() + "'"); }
+                if(!(arch.getMatrixType() & SynapseMatrixConnectivity::SPARSE)) { unsupported("postsynaptic learning on a non-SPARSE projection"); }
+
+                CodeStream::Scope b(funcEnv.getStream());
+                funcEnv.getStream() << "// merged postsynaptic update group " << s.getIndex() << std::endl;
+                funcEnv.getStream() << "for(unsigned int g = 0; g < " << s.getGroups().size() << "; g++)";
+                CodeStream::Scope b2(funcEnv.getStream());
+                funcEnv.getStream() << "const auto *group = &mergedPostsynapticUpdateGroup" << s.getIndex() << "[g];" << std::endl;
+                EnvironmentGroupMergedField<PostsynapticUpdateGroupMerged> env(funcEnv, s);
+                buildStandardEnvironment(env, batchSize);
+                CodeStream &out = env.getStream();
+                auto counts = [&s](auto fn)
+                {
+                    std::vector<uint64_t> v;
+                    for(const auto &g : s.getGroups()) { v.push_back(fn(g.get())); }
+                    return v;
+                };
+                env.addField(scalar.createPointer(), "_mi_g", "g", [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, "g"); });
+                env.addField(scalar.createPointer(), "_mi_preTrace", "preTrace",
+                             [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g.getFusedWUPreTarget(), "preTrace"); });
+                out << "gennmi_postsynaptic_update_group_t d = {};" << std::endl;
+                out << "{ static const uint32_t a[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getSrcNeuronGroup()->getNumNeurons(); }))
+                    << ", b[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getTrgNeuronGroup()->getNumNeurons(); }))
+                    << ", c[] = " << tableU32(counts([this](const SynapseGroupInternal &g){ return getSynapticMatrixRowStride(g); }))
+                    << ", e[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getMaxSourceConnections(); }))
+                    << "; d.numSrcNeurons = a[g]; d.numTrgNeurons = b[g]; d.rowStride = c[g]; d.colStride = e[g]; }" << std::endl;
+                out << "d.colLength = gennmiDev(" << env["_col_length"] << "); d.remap = gennmiDev(" << env["_remap"] << "); d.g = gennmiDev(" << env["_mi_g"] << ");" << std::endl;
+                out << "d.trgSpkCnt = gennmiDev(" << env["_trg_spk_cnt"] << "); d.trgSpk = gennmiDev(" << env["_trg_spk"] << ");" << std::endl;
+                out << "d.srcST = gennmiDev(" << env["_src_st"] << "); d.preTrace = gennmiDev(" << env["_mi_preTrace"] << ");" << std::endl;
+                for(const char *p : {"aPlus", "wMin", "wMax"}) {
+                    std::vector<Type::NumericValue> v;
+                    for(const auto &g : s.getGroups()) { v.push_back(g.get().getWUInitialiser().getParams().at(p)); }
+                    out << "{ static const float v[] = " << table(v, scalar) << "; d." << p << " = v[g]; }" << std::endl;
+                }
+                out << "GENNMI_CHECK(gennmi_push_postsynaptic_update_group(gennmiRunner, &d, nullptr));" << std::endl;
+            });
+    }
+    body << std::endl;
+    body << "void updateSynapses(" << model.getTimePrecision().getName() << ")";
+    {
+        CodeStream::Scope b(body);
+        body << "// runs as part of updateNeurons()" << std::endl;
+    }
+
+    modelMerged.genMergedPresynapticUpdateGroupStructs(os, *this);
+    modelMerged.genMergedPostsynapticUpdateGroupStructs(os, *this);
+    modelMerged.genMergedPresynapticUpdateGroupHostStructArrayPush(os, *this);
+    modelMerged.genMergedPostsynapticUpdateGroupHostStructArrayPush(os, *this);
+    preambleHandler(os);
+    os << bodyStream.str();
+}
+//--------------------------------------------------------------------------
+void Backend::genCustomUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelMerged,
+                              BackendBase::MemorySpaces&, HostHandler preambleHandler) const
+{
+    const ModelSpecInternal &model = modelMerged.getModel();
+    if(!model.getCustomUpdates().empty() || !model.getCustomWUUpdates().empty() || !model.getCustomConnectivityUpdates().empty()) {
+        unsupported("custom updates");
+    }
+    preambleHandler(os);
+}
+//--------------------------------------------------------------------------
+// initialize() / initializeSparse(): the reference's generic initialisation code, generated as plain host loops over
+// the arrays' host buffers (merged init groups carry host pointers), followed by an upload of every buffer.
+// initializeSparse() additionally builds the column view of plastic projections on the device.
+//--------------------------------------------------------------------------
+void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelMerged,
+                      BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const
+{
+    const ModelSpecInternal &model = modelMerged.getModel();
+    const unsigned int batchSize = model.getBatchSize();
+
+    std::ostringstream bodyStream;
+    CodeStream body(bodyStream);
+    EnvironmentLibrary rngEnv(body, StandardLibrary::getHostRNGFunctions(model.getPrecision()));
+    EnvironmentLibrary initEnv(rngEnv, StandardLibrary::getMathsFunctions());
+
+    // "for every group of this merged group" wrapper shared by all init groups
+    auto forEachGroup = [](EnvironmentExternalBase &funcEnv, const std::string &structName, size_t index, size_t numGroups, auto emit)
+    {
+        CodeStream::Scope b(funcEnv.getStream());
+        funcEnv.getStream() << "// merged " << structName << " " << index << std::endl;
+        funcEnv.getStream() << "for(unsigned int g = 0; g < " << numGroups << "; g++)";
+        CodeStream::Scope b2(funcEnv.getStream());
+        funcEnv.getStream() << "const auto *group = &merged" << structName << index << "[g];" << std::endl;
+        emit();
+    };
+
+    body << "void initialize()";
+    {
+        CodeStream::Scope b(body);
+        EnvironmentExternal funcEnv(initEnv);
+        funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
+
+        modelMerged.genMergedNeuronInitGroups(
+            *this, memorySpaces,
+            [&](auto &n)
+            {
+                forEachGroup(funcEnv, "NeuronInitGroup", n.getIndex(), n.getGroups().size(), [&]
+                {
+                    EnvironmentGroupMergedField<NeuronInitGroupMerged> env(funcEnv, n);
+                    buildStandardEnvironment(env, batchSize);
+                    n.generateInit(*this, env, batchSize);
+                });
+            });
+        modelMerged.genMergedSynapseInitGroups(
+            *this, memorySpaces,
+            [&](auto &s)
+            {
+                forEachGroup(funcEnv, "SynapseInitGroup", s.getIndex(), s.getGroups().size(), [&]
+                {
+                    EnvironmentGroupMergedField<SynapseInitGroupMerged> env(funcEnv, s);
+                    buildStandardEnvironment(env, batchSize);
+                    s.generateInit(*this, env, batchSize);
+                });
+            });
+        modelMerged.genMergedSynapseConnectivityInitGroups(
+            *this, memorySpaces,
+            [&](auto &s)
+            {
+                const auto &arch = s.getArchetype();
+                const auto &connect = arch.getSparseConnectivityInitialiser();
+                if(!(arch.getMatrixType() & SynapseMatrixConnectivity::SPARSE) || !arch.getKernelSize().empty()) {
+                    unsupported("connectivity initialisation of projection '" + arch.getName() + "' (SPARSE without kernel only)");
+                }
+                const bool byRow = !Utils::areTokensEmpty(connect.getRowBuildCodeTokens());
+                forEachGroup(funcEnv, "SynapseConnectivityInitGroup", s.getIndex(), s.getGroups().size(), [&]
+                {
+                    EnvironmentGroupMergedField<SynapseConnectivityInitGroupMerged> env(funcEnv, s);
+                    buildStandardEnvironment(env, batchSize);
+                    // rows start empty whatever an earlier initialize() left behind
+                    env.printLine("std::fill_n($(_row_length), $(num_pre), 0u);");
+                    if(byRow) {
+                        env.print("for(unsigned int i = 0; i < $(num_pre); i++)");
+                        env.add(Type::Uint32.addConst(), "id_pre", "i");
+                        env.add(Type::Uint32.addConst(), "id_post_begin", "0");
+                    }
+                    else {
+                        env.print("for(unsigned int j = 0; j < $(num_post); j++)");
+                        env.add(Type::Uint32.addConst(), "id_post", "j");
+                        env.add(Type::Uint32.addConst(), "id_pre_begin", "0");
+                    }
+                    env.add(Type::Uint32.addConst(), "id_thread", "0");
+                    env.add(Type::Uint32.addConst(), "num_threads", "1");
+                    CodeStream::Scope loop(env.getStream());
+
+                    // addSynapse(other end of the synapse): append to the row
+                    std::ostringstream addStream;
+                    CodeStream add(addStream);
+                    {
+                        CodeStream::Scope a(add);
+                        EnvironmentExternal addEnv(env, add);
+                        if(byRow) {
+                            addEnv.add(Type::Uint32.addConst(), "id_post", "idPost", {addEnv.addInitialiser("const unsigned int idPost = $(0);")});
+                        }
+                        else {
+                            addEnv.add(Type::Uint32.addConst(), "id_pre", "idPre", {addEnv.addInitialiser("const unsigned int idPre = $(0);")});
+                        }
+                        addEnv.printLine("$(_ind)[($(id_pre) * $(_row_stride)) + $(_row_length)[$(id_pre)]] = $(id_post);");
+                        addEnv.printLine("$(_row_length)[$(id_pre)]++;");
+                    }
+                    env.add(Type::ResolvedType::createFunction(Type::Void, {Type::Uint32}), "addSynapse", addStream.str());
+                    if(byRow) {
+                        s.generateSparseRowInit(env);
+                    }
+                    else {
+                        s.generateSparseColumnInit(env);
+                    }
+                });
+            });
+        funcEnv.getStream() << "GENNMI_CHECK(gennmi_push_mirrors());" << std::endl;
+    }
+    body << std::endl;
+
+    // column views to build once connectivity is on the device: (merged group index, number of groups)
+    std::vector<std::pair<size_t, size_t>> remapGroups;
+    body << "void initializeSparse()";
+    {
+        CodeStream::Scope b(body);
+        EnvironmentExternal funcEnv(initEnv);
+        funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
+
+        std::ostringstream remapStream;
+        CodeStream remap(remapStream);
+        modelMerged.genMergedSynapseSparseInitGroups(
+            *this, memorySpaces,
+            [&](auto &s)
+            {
+                const bool learnPost = s.getArchetype().isPostSpikeRequired() || s.getArchetype().isPostSpikeEventRequired();
+                forEachGroup(funcEnv, "SynapseSparseInitGroup", s.getIndex(), s.getGroups().size(), [&]
+                {
+                    EnvironmentGroupMergedField<SynapseSparseInitGroupMerged> env(funcEnv, s);
+                    buildStandardEnvironment(env, batchSize);
+                    if(s.getArchetype().isWUVarInitRequired()) {
+                        env.print("for(unsigned int i = 0; i < $(num_pre); i++)");
+                        CodeStream::Scope loop(env.getStream());
+                        env.add(Type::Uint32.addConst(), "id_pre", "i");
+                        env.add(Type::Uint32.addConst(), "row_len", "$(_row_length)[i]");
+                        s.generateInit(*this, env, batchSize);
+                    }
+                    if(learnPost) {
+                        // evaluated here so the fields exist; executed after the upload below
+                        remap << "for(unsigned int g = 0; g < " << s.getGroups().size() << "; g++)";
+                        CodeStream::Scope r(remap);
+                        remap << "const auto *group = &mergedSynapseSparseInitGroup" << s.getIndex() << "[g];" << std::endl;
+                        remap << "GENNMI_CHECK(gennmi_build_remap(" << env["num_pre"] << ", " << env["num_post"] << ", " << env["_row_stride"] << ", " << env["_col_stride"]
+                              << ", gennmiDev(" << env["_row_length"] << "), gennmiDev(" << env["_ind"] << "), gennmiDev(" << env["_col_length"] << "), gennmiDev(" << env["_remap"] << ")));" << std::endl;
+                    }
+                });
+            });
+        funcEnv.getStream() << "GENNMI_CHECK(gennmi_push_mirrors());" << std::endl;
+        funcEnv.getStream() << remapStream.str();
+    }
+
+    modelMerged.genMergedNeuronInitGroupStructs(os, *this);
+    modelMerged.genMergedSynapseInitGroupStructs(os, *this);
+    modelMerged.genMergedSynapseConnectivityInitGroupStructs(os, *this);
+    modelMerged.genMergedSynapseSparseInitGroupStructs(os, *this);
+    modelMerged.genMergedNeuronInitGroupHostStructArrayPush(os, *this);
+    modelMerged.genMergedSynapseInitGroupHostStructArrayPush(os, *this);
+    modelMerged.genMergedSynapseConnectivityInitGroupHostStructArrayPush(os, *this);
+    modelMerged.genMergedSynapseSparseInitGroupHostStructArrayPush(os, *this);
+    preambleHandler(os);
+    os << bodyStream.str();
+}
+//--------------------------------------------------------------------------
+// Loop shapes of the generic initialisation code: plain host loops
+//--------------------------------------------------------------------------
+void Backend::genPopVariableInit(EnvironmentExternalBase &env, HandlerEnv handler) const
+{
+    handler(env);
+}
+void Backend::genVariableInit(EnvironmentExternalBase &env, const std::string &count, const std::string &indexVarName, HandlerEnv handler) const
+{
+    env.getStream() << "for(unsigned int k = 0; k < (" << env[count] << "); k++)";
+    CodeStream::Scope b(env.getStream());
+    EnvironmentExternal varEnv(env);
+    varEnv.add(Type::Uint32, indexVarName, "k");
+    handler(varEnv);
+}
+void Backend::genSparseSynapseVariableRowInit(EnvironmentExternalBase &env, HandlerEnv handler) const
+{
+    env.print("for(unsigned int j = 0; j < $(_row_length)[$(id_pre)]; j++)");
+    CodeStream::Scope b(env.getStream());
+    EnvironmentExternal varEnv(env);
+    varEnv.add(Type::Uint32, "id_syn", "idSyn", {varEnv.addInitialiser("const unsigned int idSyn = ($(id_pre) * $(_row_stride)) + j;")});
+    varEnv.add(Type::Uint32, "id_post", "idPost", {varEnv.addInitialiser("const unsigned int idPost = $(_ind)[$(id_syn)];")});
+    handler(varEnv);
+}
+void Backend::genDenseSynapseVariableRowInit(EnvironmentExternalBase &env, HandlerEnv handler) const
+{
+    env.print("for(unsigned int j = 0; j < $(num_post); j++)");
+    CodeStream::Scope b(env.getStream());
+    EnvironmentExternal varEnv(env);
+    varEnv.add(Type::Uint32, "id_syn", "idSyn", {varEnv.addInitialiser("const unsigned int idSyn = ($(id_pre) * $(_row_stride)) + j;")});
+    varEnv.add(Type::Uint32, "id_post", "j");
+    handler(varEnv);
+}
+void Backend::genKernelSynapseVariableInit(EnvironmentExternalBase &env, SynapseInitGroupMerged &sg, HandlerEnv handler) const
+{
+    // one nested loop per kernel dimension, innermost last; id_syn is the row-major kernel index
+    EnvironmentExternal loopEnv(env);
+    const size_t numDims = sg.getArchetype().getKernelSize().size();
+    std::string index;
+    for(size_t d = 0; d < numDims; d++) {
+        const std::string v = "k" + std::to_string(d);
+        loopEnv.getStream() << "for(unsigned int " << v << " = 0; " << v << " < " << getKernelSize(sg, d) << "; " << v << "++)" << CodeStream::OB(500 + d);
+        loopEnv.add(Type::Uint32.addConst(), "id_kernel_" + std::to_string(d), v);
+        index = index.empty() ? v : ("(" + index + ") * " + getKernelSize(sg, d) + " + " + v);
+    }
+    {
+        EnvironmentExternal varEnv(static_cast<EnvironmentExternalBase&>(loopEnv));
+        varEnv.add(Type::Uint32.addConst(), "id_syn", "idSyn", {varEnv.addInitialiser("const unsigned int idSyn = " + index + ";")});
+        handler(varEnv);
+    }
+    for(size_t d = numDims; d > 0; d--) {
+        loopEnv.getStream() << CodeStream::CB(500 + d - 1);
+    }
+}
+void Backend::genKernelCustomUpdateVariableInit(EnvironmentExternalBase&, CustomWUUpdateInitGroupMerged&, HandlerEnv) const
+{
+    unsupported("custom updates");
+}
+//--------------------------------------------------------------------------
+size_t Backend::getSynapticMatrixRowStride(const SynapseGroupInternal &sg) const
+{
+    if(sg.getMatrixType() & SynapseMatrixConnectivity::SPARSE) {
+        // rows padded to 4 entries start on 16-byte boundaries, which the row loads of the kernels exploit
+        return padSize(sg.getMaxConnections(), 4);
+    }
+    else if(sg.getMatrixType() & SynapseMatrixConnectivity::TOEPLITZ) {
+        return sg.getMaxConnections();
+    }
+    else if(sg.getMatrixType() & SynapseMatrixConnectivity::BITMASK) {
+        return padSize(sg.getTrgNeuronGroup()->getNumNeurons(), 32);
+    }
+    else {
+        return sg.getTrgNeuronGroup()->getNumNeurons();
+    }
+}
+//--------------------------------------------------------------------------
+void Backend::genDefinitionsPreamble(CodeStream &os, const ModelSpecMerged&) const
+{
+    os << "// Standard C++ includes" << std::endl;
+    for(const char *h : {"algorithm", "cassert", "cmath", "cstdint", "cstring", "iostream", "random", "stdexcept", "string", "vector"}) {
+        os << "#include <" << h << ">" << std::endl;
+    }
+    os << std::endl;
+    os << "// MI355X device library" << std::endl;
+    os << "#include \"genn_mi355x.h\"" << std::endl;
+    os << "#define GENNMI_CHECK(call) do { if((call) != GENNMI_OK) { throw std::runtime_error(std::string(__FILE__) + \": \" + std::to_string(__LINE__) + \": \" + gennmi_last_error()); } } while(0)" << std::endl;
+    os << std::endl;
+    os << "extern gennmi_runner *gennmiRunner;" << std::endl;
+    os << "void gennmiBuildNeuronGroups();" << std::endl;
+    os << "void gennmiBuildSynapseGroups();" << std::endl;
+    os << "void gennmiEnsureFinalised();" << std::endl;
+    os << "uint32_t *gennmiScratch(size_t count);" << std::endl;
+    os << "// merged groups hold host pointers; kernels need the device buffers registered behind them" << std::endl;
+    os << "template<typename T> inline T *gennmiDev(T *host)";
+    {
+        CodeStream::Scope b(os);
+        os << "void *dev = nullptr;" << std::endl;
+        os << "GENNMI_CHECK(gennmi_mirror_device_pointer((const void*)host, &dev));" << std::endl;
+        os << "return (T*)dev;" << std::endl;
+    }
+    os << "using std::min;" << std::endl;
+    os << "using std::max;" << std::endl;
+    os << std::endl;
+}
+//--------------------------------------------------------------------------
+void Backend::genRunnerPreamble(CodeStream &os, const ModelSpecMerged&) const
+{
+    os << "gennmi_runner *gennmiRunner = nullptr;" << std::endl;
+    os << "static bool gennmiFinalised = false;" << std::endl;
+    os << "static std::vector<void*> gennmiScratchBuffers;" << std::endl;
+    os << "uint32_t *gennmiScratch(size_t count)";
+    {
+        CodeStream::Scope b(os);
+        os << "void *p = nullptr;" << std::endl;
+        os << "GENNMI_CHECK(gennmi_malloc(&p, count * sizeof(uint32_t)));" << std::endl;
+        os << "GENNMI_CHECK(gennmi_memset(p, 0, count * sizeof(uint32_t)));" << std::endl;
+        os << "gennmiScratchBuffers.push_back(p);" << std::endl;
+        os << "return (uint32_t*)p;" << std::endl;
+    }
+    os << "// every merged update group becomes descriptors of the device library, once, before the first step" << std::endl;
+    os << "void gennmiEnsureFinalised()";
+    {
+        CodeStream::Scope b(os);
+        os << "if(gennmiFinalised) { return; }" << std::endl;
+        os << "gennmiBuildNeuronGroups();" << std::endl;
+        os << "gennmiBuildSynapseGroups();" << std::endl;
+        os << "GENNMI_CHECK(gennmi_runner_finalise(gennmiRunner));" << std::endl;
+        os << "gennmiFinalised = true;" << std::endl;
+    }
+    os << std::endl;
+}
+//--------------------------------------------------------------------------
+void Backend::genAllocateMemPreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const
+{
+    const ModelSpecInternal &model = modelMerged.getModel();
+    os << "GENNMI_CHECK(gennmi_init(" << getPreferences<Preferences>().deviceID << "));" << std::endl;
+    os << "GENNMI_CHECK(gennmi_runner_create(&gennmiRunner, " << Type::writeNumeric(model.getDT(), model.getTimePrecision()) << ", " << model.getBatchSize() << "u));" << std::endl;
+    if(model.isTimingEnabled()) {
+        os << "GENNMI_CHECK(gennmi_runner_set_timing(gennmiRunner, 1));" << std::endl;
+    }
+}
+//--------------------------------------------------------------------------
+void Backend::genFreeMemPreamble(CodeStream &os, const ModelSpecMerged&) const
+{
+    os << "if(gennmiRunner) { GENNMI_CHECK(gennmi_runner_destroy(gennmiRunner)); gennmiRunner = nullptr; }" << std::endl;
+    os << "for(void *p : gennmiScratchBuffers) { gennmi_free(p); }" << std::endl;
+    os << "gennmiScratchBuffers.clear();" << std::endl;
+    os << "gennmiFinalised = false;" << std::endl;
+}
+//--------------------------------------------------------------------------
+void Backend::genStepTimeFinalisePreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const
+{
+    // the reference's device backends synchronise here too when timing (backendCUDAHIP.cc:1400-1411)
+    if(modelMerged.getModel().isTimingEnabled()) {
+        os << "GENNMI_CHECK(gennmi_runner_synchronize(gennmiRunner));" << std::endl;
+        os << "GENNMI_CHECK(gennmi_runner_get_times(gennmiRunner, &neuronUpdateTime, &presynapticUpdateTime, &postsynapticUpdateTime));" << std::endl;
+    }
+}
+//--------------------------------------------------------------------------
+std::unique_ptr<GeNN::Runtime::StateBase> Backend::createState(const Runtime::Runtime&) const
+{
+    return std::make_unique<State>();
+}
+std::unique_ptr<Runtime::ArrayBase> Backend::createArray(const Type::ResolvedType &type, size_t count,
+                                                         VarLocation location, bool uninitialized) const
+{
+    return std::make_unique<Array>(type, count, location, uninitialized);
+}
+std::unique_ptr<Runtime::ArrayBase> Backend::createPopulationRNG(size_t) const
+{
+    return std::unique_ptr<Runtime::ArrayBase>();
+}
+//--------------------------------------------------------------------------
+// Extra global parameters allocated from generated host code (initializeHost): plain host arrays
+//--------------------------------------------------------------------------
+void Backend::genLazyVariableDynamicAllocation(CodeStream &os, const Type::ResolvedType &type, const std::string &name,
+                                               VarLocation, const std::string &countVarName) const
+{
+    const auto &valueType = type.isPointer() ? *type.getPointer().valueType : type;
+    os << (type.isPointer() ? "*" : "") << "$(_" << name << ") = new " << valueType.getValue().name << "[" << countVarName << "];" << std::endl;
+}
+void Backend::genLazyVariableDynamicPush(CodeStream&, const Type::ResolvedType&, const std::string&, VarLocation, const std::string&) const
+{
+}
+void Backend::genLazyVariableDynamicPull(CodeStream&, const Type::ResolvedType&, const std::string&, VarLocation, const std::string&) const
+{
+}
+void Backend::genMergedDynamicVariablePush(CodeStream &os, const std::string &suffix, size_t mergedGroupIdx,
+                                           const std::string &groupIdx, const std::string &fieldName,
+                                           const std::string &egpName) const
+{
+    os << "merged" << suffix << "Group" << mergedGroupIdx << "[" << groupIdx << "]." << fieldName << " = " << egpName << ";" << std::endl;
+}
+//--------------------------------------------------------------------------
+std::string Backend::getAtomicOperation(const std::string &lhsPointer, const std::string &rhsValue,
+                                        const Type::ResolvedType&, AtomicOperation op) const
+{
+    // only host-side initialisation code is generated, and it is single-threaded
+    return "(*(" + lhsPointer + ") " + ((op == AtomicOperation::ADD) ? "+=" : "|=") + " (" + rhsValue + "))";
+}
+void Backend::genGlobalDeviceRNG(CodeStream&, CodeStream&, CodeStream&, CodeStream&) const
+{
+    unsupported("a device random number generator");
+}
+void Backend::genTimer(CodeStream&, CodeStream&, CodeStream&, CodeStream&, CodeStream&, const std::string&, bool) const
+{
+    // kernel durations are accumulated inside the device library (gennmi_runner_set_timing / get_times)
+}
+void Backend::genReturnFreeDeviceMemoryBytes(CodeStream &os) const
+{
+    os << "size_t freeBytes = 0;" << std::endl;
+    os << "GENNMI_CHECK(gennmi_free_device_memory_bytes(&freeBytes));" << std::endl;
+    os << "return freeBytes;" << std::endl;
+}
+void Backend::genAssert(CodeStream &os, const std::string &condition) const
+{
+    os << "assert(" << condition << ");" << std::endl;
+}
+//--------------------------------------------------------------------------
+// Build system: the runner is host C++ linked against the device library
+//--------------------------------------------------------------------------
+void Backend::genMakefilePreamble(std::ostream &os) const
+{
+    std::string root = getPreferences<Preferences>().installRoot;
+    if(root.empty()) {
+        const char *env = std::getenv("GENN_MI355X_ROOT");
+        root = env ? env : GENNMI_DEFAULT_ROOT;
+    }
+    std::string cxxFlags = "-c -fPIC -std=c++17 -MMD -MP -I\"" + root + "/include\" " + getPreferences().userCxxFlagsGNU;
+    cxxFlags += getPreferences().debugCode ? " -O0 -g" : " -O2";
+    os << "CXXFLAGS := " << cxxFlags << std::endl;
+    os << "LINKFLAGS := -shared" << std::endl;
+    os << "LINKLIBS := -L\"" << root << "/genn_amd/lib\" -lgenn_mi355x -Wl,-rpath,\"" << root << "/genn_amd/lib\"" << std::endl;
+    os << std::endl;
+}
+void Backend::genMakefileLinkRule(std::ostream &os) const
+{
+    os << "\t@$(CXX) $(LINKFLAGS) -o $@ $(OBJECTS) $(LINKLIBS)" << std::endl;
+}
+void Backend::genMakefileCompileRule(std::ostream &os) const
+{
+    os << "%.o: %.cc %.d" << std::endl;
+    os << "\t@$(CXX) $(CXXFLAGS) -o $@ $<" << std::endl;
+}
+void Backend::genNMakefilePreamble(std::ostream&) const { unsupported("NMake"); }
+void Backend::genNMakefileLinkRule(std::ostream&) const { unsupported("NMake"); }
+void Backend::genNMakefileCompileRule(std::ostream&) const { unsupported("NMake"); }
+void Backend::genMSBuildConfigProperties(std::ostream&) const {}
+void Backend::genMSBuildImportProps(std::ostream&) const {}
+void Backend::genMSBuildItemDefinitions(std::ostream&) const {}
+void Backend::genMSBuildCompileModule(const std::string&, std::ostream&) const {}
+void Backend::genMSBuildImportTarget(std::ostream&) const {}
+//--------------------------------------------------------------------------
+bool Backend::isGlobalHostRNGRequired(const ModelSpecInternal &model) const
+{
+    // initialisation runs on the host, so any random initialisation draws from the host generator
+    const auto &ngs = model.getNeuronGroups();
+    const auto &sgs = model.getSynapseGroups();
+    return std::any_of(ngs.cbegin(), ngs.cend(), [](const auto &n){ return n.second.isInitRNGRequired(); })
+        || std::any_of(sgs.cbegin(), sgs.cend(), [](const auto &s){ return s.second.isWUInitRNGRequired() || s.second.getSparseConnectivityInitialiser().isRNGRequired()
+                                                                          || s.second.getSparseConnectivityInitialiser().isHostRNGRequired(); });
+}
+size_t Backend::getDeviceMemoryBytes() const
+{
+    size_t bytes = 0;
+    return (gennmi_free_device_memory_bytes(&bytes) == GENNMI_OK) ? bytes : 0;
+}
+boost::uuids::detail::sha1::digest_type Backend::getHashDigest() const
+{
+    boost::uuids::detail::sha1 hash;
+    Utils::updateHash("MI355X", hash);
+    getPreferences<Preferences>().updateHash(hash);
+    return hash.get_digest();
+}
+//--------------------------------------------------------------------------
+// GeNN::CodeGenerator::MI355X::Optimiser
+//--------------------------------------------------------------------------
+namespace Optimiser
+{
+Backend createBackend(const ModelSpecInternal&, const filesystem::path&, plog::Severity backendLevel,
+                      plog::IAppender *backendAppender, const Preferences &preferences)
+{
+    if(plog::get<Logging::CHANNEL_BACKEND>() == nullptr) {
+        plog::init<Logging::CHANNEL_BACKEND>(backendLevel, backendAppender);
+    }
+    else {
+        plog::get<Logging::CHANNEL_BACKEND>()->setMaxSeverity(backendLevel);
+    }
+    return Backend(preferences);
+}
+}   // namespace Optimiser
+}   // namespace GeNN::CodeGenerator::MI355X

@@ -36,7 +36,13 @@
 #include "optimiser.h"
 
 using namespace GeNN;
+// The same driver runs the network on the MI355X backend when built with -DDRIVER_BACKEND_MI355X (and the
+// include path of that backend's optimiser.h first); array layouts are converted to the backend's row stride.
+#ifdef DRIVER_BACKEND_MI355X
+using namespace GeNN::CodeGenerator::MI355X;
+#else
 using namespace GeNN::CodeGenerator::SingleThreadedCPU;
+#endif
 
 // ---------------------------------------------------------------------------------------------
 // Models that are not built into the reference (declared the way a user of its C++ API would)
@@ -279,13 +285,25 @@ int main(int argc, char *argv[])
                 rt.allocateArray(*c.cs, "noise", n);
             }
         }
+        // per-synapse arrays are stored with the netspec's row stride; the backend may use a larger one
+        auto backendStride = [&](const SynSpec &s) { return backend.getSynapticMatrixRowStride(*static_cast<const SynapseGroupInternal*>(s.sg)); };
+        auto loadRows = [&](Runtime::ArrayBase *a, const std::string &file, const SynSpec &s, auto zero) {
+            using T = decltype(zero);
+            const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
+            const auto rows = readFile<T>(in + "/" + file, numPre * s.rowStride);
+            auto *dst = a->getHostPointer<T>();
+            for(size_t i = 0; i < numPre; i++) { std::copy_n(rows.begin() + i * s.rowStride, s.rowStride, dst + i * stride); }
+        };
         for(auto &s : syns) {
             if(s.matrix == "sparse") {
                 load(rt.getArray(*s.sg, "rowLength"), s.name + ".rowLength.u32");
-                load(rt.getArray(*s.sg, "ind"), s.name + ".ind.u32");
+                loadRows(rt.getArray(*s.sg, "ind"), s.name + ".ind.u32", s, uint32_t(0));
+                loadRows(rt.getArray(*s.sg, "g"), s.name + ".g.f32", s, float(0));
+                if(s.wum == "static_delay") loadRows(rt.getArray(*s.sg, "d"), s.name + ".d.u8", s, uint8_t(0));
             }
-            load(rt.getArray(*s.sg, "g"), s.name + ".g.f32");
-            if(s.wum == "static_delay") load(rt.getArray(*s.sg, "d"), s.name + ".d.u8");
+            else {
+                load(rt.getArray(*s.sg, "g"), s.name + ".g.f32");
+            }
             if(s.wum == "stdp_trace") {
                 rt.getArray(*s.sg, "preTrace")->memsetHostPointer(0);
                 rt.getArray(*s.sg, "postTrace")->memsetHostPointer(0);
@@ -301,16 +319,24 @@ int main(int argc, char *argv[])
                 fm << s.name << " " << sgi->getFusedPSTarget().getName() << std::endl;
                 if(s.wum == "stdp_trace" || s.wum == "stdp") {
                     auto *cl = rt.getArray(*s.sg, "colLength"); auto *rm = rt.getArray(*s.sg, "remap");
+                    cl->pullFromDevice(); rm->pullFromDevice();
                     appendFile(out + "/" + s.name + ".colLength.u32", cl->getHostPointer<uint32_t>(), cl->getCount());
-                    appendFile(out + "/" + s.name + ".remap.u32", rm->getHostPointer<uint32_t>(), rm->getCount());
+                    // synapse indices are written in terms of the netspec's row stride
+                    std::vector<uint32_t> remap(rm->getHostPointer<uint32_t>(), rm->getHostPointer<uint32_t>() + rm->getCount());
+                    const uint32_t stride = (uint32_t)backendStride(s);
+                    for(auto &r : remap) { r = (r / stride) * s.rowStride + (r % stride); }
+                    appendFile(out + "/" + s.name + ".remap.u32", remap.data(), remap.size());
                     std::ofstream(out + "/" + s.name + ".colStride.txt") << sgi->getMaxSourceConnections() << std::endl;
                 }
             }
         }
 
+        auto pulled = [](Runtime::ArrayBase *a) { a->pullFromDevice(); return a; };
         auto snapshot = [&]() {
             for(auto &p : pops) {
                 if(p.model == "ssa") continue;
+                pulled(rt.getArray(*p.ng, "V"));
+                pulled(rt.getArray(*p.ng, p.model == "lif" ? "RefracTime" : "U"));
                 appendFile(out + "/" + p.name + ".V.f32", rt.getArray(*p.ng, "V")->getHostPointer<float>(), p.n);
                 if(p.model == "lif") appendFile(out + "/" + p.name + ".RefracTime.f32", rt.getArray(*p.ng, "RefracTime")->getHostPointer<float>(), p.n);
                 if(p.model == "izh") appendFile(out + "/" + p.name + ".U.f32", rt.getArray(*p.ng, "U")->getHostPointer<float>(), p.n);
@@ -318,19 +344,20 @@ int main(int argc, char *argv[])
             for(auto &s : syns) {
                 const auto *sgi = static_cast<const SynapseGroupInternal*>(s.sg);
                 if(&sgi->getFusedPSTarget() == sgi) {
-                    auto *a = rt.getArray(*s.sg, "outPost");
+                    auto *a = pulled(rt.getArray(*s.sg, "outPost"));
                     appendFile(out + "/" + s.name + ".outPost.f32", a->getHostPointer<float>(), a->getCount());
                     if(sgi->isDendriticOutputDelayRequired()) {
-                        auto *d = rt.getArray(*s.sg, "denDelay");
+                        auto *d = pulled(rt.getArray(*s.sg, "denDelay"));
                         appendFile(out + "/" + s.name + ".denDelay.f32", d->getHostPointer<float>(), d->getCount());
                     }
                 }
                 if(s.wum == "stdp_trace" || s.wum == "stdp") {
-                    auto *a = rt.getArray(*s.sg, "g");
-                    appendFile(out + "/" + s.name + ".g.f32", a->getHostPointer<float>(), a->getCount());
+                    auto *a = pulled(rt.getArray(*s.sg, "g"));
+                    const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
+                    for(size_t i = 0; i < numPre; i++) { appendFile(out + "/" + s.name + ".g.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
                 }
                 if(s.wum == "stdp_trace") {
-                    auto *a = rt.getArray(*s.sg, "preTrace"); auto *b = rt.getArray(*s.sg, "postTrace");
+                    auto *a = pulled(rt.getArray(*s.sg, "preTrace")); auto *b = pulled(rt.getArray(*s.sg, "postTrace"));
                     appendFile(out + "/" + s.name + ".preTrace.f32", a->getHostPointer<float>(), a->getCount());
                     appendFile(out + "/" + s.name + ".postTrace.f32", b->getHostPointer<float>(), b->getCount());
                 }
