@@ -127,8 +127,9 @@ struct SynSpec
 int main(int argc, char *argv[])
 {
     try {
-        if(argc != 4) { std::cerr << "usage: ref_driver <netspec dir> <work dir> <out dir>" << std::endl; return 1; }
+        if(argc != 4 && argc != 5) { std::cerr << "usage: ref_driver <netspec dir> <work dir> <out dir> [--generate-only]" << std::endl; return 1; }
         const std::string in = argv[1], work = argv[2], out = argv[3];
+        const bool generateOnly = (argc == 5 && std::string(argv[4]) == "--generate-only");
 
         plog::ConsoleAppender<plog::TxtFormatter> app;
         Preferences prefs;
@@ -255,6 +256,10 @@ int main(int argc, char *argv[])
         }
         const std::string cmd = "make -s -C \"" + outputPath.str() + "\" -j 8";
         if(system(cmd.c_str()) != 0) { throw std::runtime_error("build failed: " + cmd); }
+        if(generateOnly) {
+            std::cout << "ref_driver: generated and built " << outputPath.str() << std::endl;
+            return 0;
+        }
 
         // ---- run ---------------------------------------------------------------------------
         Runtime::Runtime rt(targetPath, modelMerged, backend);

@@ -1,0 +1,72 @@
+"""Code generation through the GeNN backend adapter, without a GPU: the reference's generator, given
+`GeNN::CodeGenerator::MI355X::Backend`, must produce a runner that compiles with the host compiler alone and
+exports exactly the entry points Runtime binds (runtime.cc:87-94, generateRunner.cc:308-321) plus one
+pushMerged<Name>Group<i>ToDevice per merged group."""
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+sys.path.insert(0, os.path.join(HERE, "golden"))
+
+from cases import CASES  # noqa: E402
+from genn_amd.netspec import write_netspec  # noqa: E402
+
+DRIVER = os.path.join(ROOT, "oracle", "_ref", "mi355x_driver")
+pytestmark = pytest.mark.skipif(not os.path.exists(DRIVER), reason="oracle/_ref/mi355x_driver is not built (needs the reference tree at build time)")
+
+
+def _generate(case):
+    net, snap = CASES[case]()
+    net.snap = snap
+    tmp = tempfile.mkdtemp(prefix="adapter_gen_")
+    spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+    for d in (work, out):
+        os.makedirs(d)
+    write_netspec(net, spec)
+    res = subprocess.run([DRIVER, spec, work, out, "--generate-only"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    assert res.returncode == 0, res.stdout[-3000:]
+    code = os.path.join(work, net.name + "_CODE")
+    return net, tmp, code
+
+
+def _exports(lib):
+    out = subprocess.run(["nm", "-D", "--defined-only", lib], stdout=subprocess.PIPE, text=True, check=True).stdout
+    return {line.split()[-1] for line in out.splitlines() if " T " in line}
+
+
+@pytest.mark.parametrize("case", ["stdp_small", "potjans_small", "conv_small"])
+def test_generated_runner_exports_reference_entry_points(case):
+    net, tmp, code = _generate(case)
+    try:
+        exports = _exports(os.path.join(code, "librunner.so"))
+        for name in ("allocateMem", "freeMem", "initialize", "initializeSparse", "initializeHost", "stepTime", "updateNeurons", "updateSynapses"):
+            assert name in exports, f"{name} missing from the generated runner"
+        pushes = {e for e in exports if e.startswith("pushMerged")}
+        assert any(e.startswith("pushMergedNeuronUpdateGroup") for e in pushes)
+        assert any(e.startswith("pushMergedPresynapticUpdateGroup") for e in pushes)
+        if case == "stdp_small":
+            assert any(e.startswith("pushMergedPostsynapticUpdateGroup") for e in pushes)
+            assert "pushMergedNeuronUpdate0spikeTimesToDevice" in exports or any("spikeTimes" in e for e in pushes)
+        # the runner is host code: no device code object, only a link against the device library
+        ldd = subprocess.run(["ldd", os.path.join(code, "librunner.so")], stdout=subprocess.PIPE, text=True).stdout
+        assert "libgenn_mi355x.so" in ldd
+        neuron = open(os.path.join(code, "neuronUpdate.cc")).read()
+        assert "gennmi_push_neuron_update_group" in neuron and "gennmi_step" in neuron and "__global__" not in neuron
+        synapse = open(os.path.join(code, "synapseUpdate.cc")).read()
+        assert synapse.count("gennmi_push_presynaptic_update_group") >= 1
+        if case == "potjans_small":
+            assert "d.maxDenDelay" in synapse and "d.denDelay" in synapse
+        if case == "conv_small":
+            assert "d.conv[7]" in synapse
+        init = open(os.path.join(code, "init.cc")).read()
+        assert "gennmi_push_mirrors" in init
+        if case == "stdp_small":
+            assert "gennmi_build_remap" in init
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
