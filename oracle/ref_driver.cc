@@ -14,6 +14,7 @@
 //
 // usage: ref_driver <netspec dir> <work dir> <out dir>
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -369,6 +370,7 @@ int main(int argc, char *argv[])
             }
         };
 
+        const auto loopStart = std::chrono::steady_clock::now();
         for(unsigned int i = 0; i < steps; i++) {
             for(auto &c : css) {
                 if(c.model == "noise") {
@@ -381,6 +383,11 @@ int main(int argc, char *argv[])
             rt.stepTime();
             if(snap && ((i + 1) % snap) == 0) snapshot();
         }
+        // a blocking pull drains whatever the backend still has queued, so the loop time below is complete
+        if(!pops.empty() && pops.front().model != "ssa") { rt.getArray(*pops.front().ng, "V")->pullFromDevice(); }
+        const double loopSeconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - loopStart).count();
+        std::cout << "ref_driver: stepping loop " << loopSeconds << " s for " << steps << " steps ("
+                  << loopSeconds / steps * 1e6 << " us per Runtime::stepTime, snapshots included)" << std::endl;
         if(!snap || (steps % snap) != 0) snapshot();
 
         // spike rasters as (step, id) pairs; the reference reports times in ms = step*dt

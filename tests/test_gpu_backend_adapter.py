@@ -103,3 +103,38 @@ def test_adapter_matches_reference_backend(case):
                 _close(got, want, key, accumulator=True)
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_adapter_full_size_microcircuit_first_100ms():
+    """77,169 neurons / 298,624,465 synapses through the reference's Runtime::stepTime on the MI355X backend, 1000
+    steps: rasters must be those of the CPU oracle, final membrane potentials within 1e-5."""
+    from genn_amd import configs
+    from oracle.genn_cpu import OracleNet
+    net = configs.potjans(steps=1000)
+    net.snap = 0
+    tmp = tempfile.mkdtemp(prefix="adapter_full_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(net, spec)
+        print(f"adapter full-size microcircuit: running {DRIVER}", flush=True)
+        res = subprocess.run([DRIVER, spec, work, out], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=280)
+        assert res.returncode == 0, res.stdout[-3000:]
+        oracle = OracleNet(net, num_recording_timesteps=net.steps)
+        oracle.run(net.steps)
+        total = 0
+        for p in net.pops:
+            got = np.fromfile(os.path.join(out, f"{p.name}.spikes.u32"), np.uint32).reshape(-1, 2)
+            words = (p.n + 31) // 32
+            bits = np.unpackbits(oracle.record(p.name, net.steps).view(np.uint8).reshape(net.steps, words * 4), axis=1, bitorder="little")[:, :p.n]
+            steps, ids = np.nonzero(bits)
+            want = np.stack([steps, ids], axis=1).astype(np.uint32)
+            assert np.array_equal(got, want), f"raster of {p.name} differs ({len(got)} vs {len(want)} spikes)"
+            total += len(want)
+            v = np.fromfile(os.path.join(out, f"{p.name}.V.f32"), np.float32)
+            _close(v, oracle.var(p.name, 0), f"V of {p.name}")
+        assert total > 10000
+        oracle.close()
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
