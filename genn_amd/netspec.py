@@ -123,6 +123,8 @@ def write_netspec(net: Net, path: str):
     lines = [f"model {net.name}", f"dt {net.dt!r}", f"steps {net.steps}", f"fuse_psm {int(net.fuse_psm)}"]
     snap = getattr(net, "snap", 0)
     lines.append(f"snap {snap}")
+    if getattr(net, "batch_size", 1) != 1:
+        lines.append(f"batch {int(net.batch_size)}")
     for p in net.pops:
         if p.model == "lif":
             ps = " ".join(repr(float(p.params[k])) for k in LIF_PARAMS)

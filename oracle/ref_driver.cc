@@ -140,7 +140,7 @@ int main(int argc, char *argv[])
         // ---- parse net.txt -----------------------------------------------------------------
         std::string name = "net";
         double dt = 1.0;
-        unsigned int steps = 1, snap = 0, fuse = 0;
+        unsigned int steps = 1, snap = 0, fuse = 0, batch = 1;
         std::vector<PopSpec> pops; std::vector<CSSpec> css; std::vector<SynSpec> syns;
         {
             std::ifstream f(in + "/net.txt");
@@ -154,6 +154,7 @@ int main(int argc, char *argv[])
                 else if(k == "steps") ls >> steps;
                 else if(k == "snap") ls >> snap;
                 else if(k == "fuse_psm") ls >> fuse;
+                else if(k == "batch") ls >> batch;
                 else if(k == "pop") { PopSpec p; ls >> p.name >> p.model >> p.n; double v; while(ls >> v) p.p.push_back(v); pops.push_back(p); }
                 else if(k == "cs") { CSSpec c; ls >> c.name >> c.model >> c.pop; double v; while(ls >> v) c.p.push_back(v); css.push_back(c); }
                 else if(k == "syn") {
@@ -180,6 +181,7 @@ int main(int argc, char *argv[])
         ModelSpecInternal model;
         model.setName(name);
         model.setDT(dt);
+        model.setBatchSize(batch);
         model.setPrecision(Type::Float);
         model.setFusePostsynapticModels(fuse != 0);
         std::map<std::string, PopSpec*> popByName;
@@ -266,9 +268,15 @@ int main(int argc, char *argv[])
         Runtime::Runtime rt(targetPath, modelMerged, backend);
         rt.allocate(steps);
         rt.initialize();
+        // a file holds either the whole array or one batch's worth, which is then replicated
         auto load = [&](Runtime::ArrayBase *a, const std::string &file) {
-            const auto bytes = readFile<char>(in + "/" + file, a->getSizeBytes());
-            std::copy(bytes.begin(), bytes.end(), reinterpret_cast<char*>(a->getHostPointer()));
+            const auto bytes = readFile<char>(in + "/" + file);
+            if(bytes.empty() || (a->getSizeBytes() % bytes.size()) != 0) {
+                throw std::runtime_error(file + ": " + std::to_string(bytes.size()) + " bytes do not tile an array of " + std::to_string(a->getSizeBytes()));
+            }
+            for(size_t o = 0; o < a->getSizeBytes(); o += bytes.size()) {
+                std::copy(bytes.begin(), bytes.end(), reinterpret_cast<char*>(a->getHostPointer()) + o);
+            }
         };
         for(auto &p : pops) {
             if(p.model == "lif") { load(rt.getArray(*p.ng, "V"), p.name + ".V.f32"); load(rt.getArray(*p.ng, "RefracTime"), p.name + ".RefracTime.f32"); }
@@ -343,9 +351,9 @@ int main(int argc, char *argv[])
                 if(p.model == "ssa") continue;
                 pulled(rt.getArray(*p.ng, "V"));
                 pulled(rt.getArray(*p.ng, p.model == "lif" ? "RefracTime" : "U"));
-                appendFile(out + "/" + p.name + ".V.f32", rt.getArray(*p.ng, "V")->getHostPointer<float>(), p.n);
-                if(p.model == "lif") appendFile(out + "/" + p.name + ".RefracTime.f32", rt.getArray(*p.ng, "RefracTime")->getHostPointer<float>(), p.n);
-                if(p.model == "izh") appendFile(out + "/" + p.name + ".U.f32", rt.getArray(*p.ng, "U")->getHostPointer<float>(), p.n);
+                appendFile(out + "/" + p.name + ".V.f32", rt.getArray(*p.ng, "V")->getHostPointer<float>(), (size_t)p.n * batch);
+                if(p.model == "lif") appendFile(out + "/" + p.name + ".RefracTime.f32", rt.getArray(*p.ng, "RefracTime")->getHostPointer<float>(), (size_t)p.n * batch);
+                if(p.model == "izh") appendFile(out + "/" + p.name + ".U.f32", rt.getArray(*p.ng, "U")->getHostPointer<float>(), (size_t)p.n * batch);
             }
             for(auto &s : syns) {
                 const auto *sgi = static_cast<const SynapseGroupInternal*>(s.sg);
@@ -394,16 +402,19 @@ int main(int argc, char *argv[])
         rt.pullRecordingBuffersFromDevice();
         for(auto &p : pops) {
             const auto ev = rt.getRecordedSpikes(*p.ng);
-            // the reference's decode lists the ids of one timestep in bit-scan order; sort them
-            std::vector<std::pair<uint32_t, uint32_t>> sorted;
-            const auto &times = ev.at(0).first; const auto &ids = ev.at(0).second;
-            for(size_t k = 0; k < times.size(); k++) {
-                sorted.emplace_back((uint32_t)std::llround(times[k] / dt), ids[k]);
+            // the reference's decode lists the ids of one timestep in bit-scan order; sort them.
+            // One file per batch: <pop>.spikes.u32 for batch 0, <pop>.spikes.b<k>.u32 for the others
+            for(unsigned int bi = 0; bi < batch; bi++) {
+                std::vector<std::pair<uint32_t, uint32_t>> sorted;
+                const auto &times = ev.at(bi).first; const auto &ids = ev.at(bi).second;
+                for(size_t k = 0; k < times.size(); k++) {
+                    sorted.emplace_back((uint32_t)std::llround(times[k] / dt), ids[k]);
+                }
+                std::sort(sorted.begin(), sorted.end());
+                std::vector<uint32_t> pairs;
+                for(const auto &s : sorted) { pairs.push_back(s.first); pairs.push_back(s.second); }
+                appendFile(out + "/" + p.name + ".spikes" + (bi ? ".b" + std::to_string(bi) : std::string()) + ".u32", pairs.data(), pairs.size());
             }
-            std::sort(sorted.begin(), sorted.end());
-            std::vector<uint32_t> pairs;
-            for(const auto &s : sorted) { pairs.push_back(s.first); pairs.push_back(s.second); }
-            appendFile(out + "/" + p.name + ".spikes.u32", pairs.data(), pairs.size());
         }
         std::cout << "ref_driver: " << name << " ran " << steps << " steps" << std::endl;
     }

@@ -138,3 +138,48 @@ def test_adapter_full_size_microcircuit_first_100ms():
         oracle.close()
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_adapter_batched_toeplitz_layer():
+    """Batch size 3 through the adapter (the reference's CPU backend has no batch): shared kernel weights and spike
+    times, per-batch spike-source windows; batch b must equal a batch-1 oracle run fed batch b's input."""
+    import copy
+    from genn_amd import configs
+    from oracle.genn_cpu import OracleNet
+    B = 3
+    nets = [configs.conv_toeplitz(h=8, w=8, ic=2, oc=4, steps=60, w_sd=0.6, batch_index=b, ioffset=0.4) for b in range(B)]
+    times = np.concatenate([n.pop("In").spike_times for n in nets])
+    offs = np.cumsum([0] + [len(n.pop("In").spike_times) for n in nets])
+    batched = copy.deepcopy(nets[0])
+    batched.pop("In").vars = {"startSpike": np.stack([n.pop("In").vars["startSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32),
+                              "endSpike": np.stack([n.pop("In").vars["endSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32)}
+    batched.pop("In").spike_times = times
+    batched.batch_size = B
+    batched.snap = 0
+    tmp = tempfile.mkdtemp(prefix="adapter_batch_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(batched, spec)
+        print(f"adapter batched conv: running {DRIVER}", flush=True)
+        res = subprocess.run([DRIVER, spec, work, out], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+        assert res.returncode == 0, res.stdout[-3000:]
+        total = 0
+        for b, net in enumerate(nets):
+            oracle = OracleNet(net, num_recording_timesteps=net.steps)
+            oracle.run(net.steps)
+            for p in net.pops:
+                got = np.fromfile(os.path.join(out, f"{p.name}.spikes{'.b%d' % b if b else ''}.u32"), np.uint32).reshape(-1, 2)
+                words = (p.n + 31) // 32
+                bits = np.unpackbits(oracle.record(p.name, net.steps).view(np.uint8).reshape(net.steps, words * 4), axis=1, bitorder="little")[:, :p.n]
+                steps, ids = np.nonzero(bits)
+                assert np.array_equal(got, np.stack([steps, ids], axis=1).astype(np.uint32)), f"batch {b}: raster of {p.name} differs"
+                total += len(ids)
+            n_out = net.pop("Out").n
+            v = np.fromfile(os.path.join(out, "Out.V.f32"), np.float32).reshape(-1, B, n_out)[-1, b]
+            _close(v, oracle.var("Out", 0), f"batch {b}: V of Out")
+            oracle.close()
+        assert total > 300
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
