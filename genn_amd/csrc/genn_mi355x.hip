@@ -1333,7 +1333,9 @@ int gennmi_runner_finalise(gennmi_runner *r)
             const uint32_t avgSeg = std::max(1u, p.g.rowStride / numTiles);
             TileGroupDev t{};
             t.g = p.g; t.tileOff = dOff; t.numTiles = numTiles; t.tileSize = tileSize;
-            t.lanes = std::min<uint32_t>(WAVE, pow2Ceil((avgSeg + 7) / 8)); t.threshold = p.tileThreshold;
+            const char *envLanes = getenv("GENNMI_TILE_LANES");
+            t.lanes = envLanes ? std::min<uint32_t>(WAVE, pow2Ceil((uint32_t)std::max(1, atoi(envLanes)))) : std::min<uint32_t>(WAVE, pow2Ceil((avgSeg + 7) / 8));
+            t.threshold = p.tileThreshold;
             tileGroups.push_back(t);
             r->tileFloats = std::max(r->tileFloats, tileSize);
         }
