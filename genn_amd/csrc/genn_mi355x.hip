@@ -33,6 +33,8 @@ namespace
 {
 constexpr int BLOCK = 256;                  // 4 wave64 per work-group
 constexpr int WAVE = 64;
+constexpr int CONV_TILE_SPIKES = 2048;      // spikes staged in LDS at a time by the Conv2D tile kernel
+constexpr int CONV_TILE_THREADS = 512;      // work-group size of the Conv2D tile kernel (8 wave64 share one LDS tile)
 constexpr uint32_t SPIN_LIMIT = 1u << 22;   // bounded wait of the spike-offset look-back
 constexpr uint32_t REMAP_SORT_MAX = 16384;  // longest column the LDS sort handles (64 KiB)
 
@@ -442,10 +444,9 @@ void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs ar
     if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
 }
 
-// Toeplitz Conv2D counterpart of the tile kernel: every block scans the (short) spike list, keeps the spikes whose
-// kernel footprint touches its output rows, and one wavefront at a time adds a spike's kh*kw*oc contributions
-// into LDS.  The block owns its rows exclusively, so the flush is a plain read-modify-write without atomics.
-__global__ __launch_bounds__(BLOCK)
+// Toeplitz Conv2D counterpart of the tile kernel: every block finds the run of spikes whose kernel footprint touches
+// its output rows and accumulates their contributions in an LDS tile, each wavefront in its own band of columns.  The block owns its rows exclusively, so the flush is a plain read-modify-write without atomics.
+__global__ __launch_bounds__(CONV_TILE_THREADS)
 void presynapticConvTileKernel(const ConvTileDev * __restrict__ blocks, unsigned long long *eventCounter)
 {
     extern __shared__ float shConv[];
@@ -463,48 +464,87 @@ void presynapticConvTileKernel(const ConvTileDev * __restrict__ blocks, unsigned
     const uint32_t kernelLen = (uint32_t)(kh * kw * ic * oc);
     float *tile = shConv;
     float *kern = tile + G.rowsPerTile * ow * oc;
-    uint32_t *diag = reinterpret_cast<uint32_t*>(kern + kernelLen);
-    for(uint32_t k = threadIdx.x; k < tileLen; k += BLOCK) { tile[k] = 0.0f; }
-    for(uint32_t k = threadIdx.x; k < kernelLen; k += BLOCK) { kern[k] = asGlobal(g.g)[k]; }
-    for(uint32_t j = threadIdx.x; j < numDiag; j += BLOCK) {
-        // kernel diagonal j -> (kernRow, kernCol, outChan), initToeplitzConnectivitySnippet.h:117-119
-        diag[j] = ((j / oc) / kw) << 20 | ((j / oc) % kw) << 10 | (j % oc);
-    }
+    uint32_t *stage = reinterpret_cast<uint32_t*>(kern + kernelLen);
+    __shared__ uint32_t shLo, shHi;
+    if(threadIdx.x == 0) { shLo = 0u; shHi = 0u; }
+    for(uint32_t k = threadIdx.x; k < tileLen; k += blockDim.x) { tile[k] = 0.0f; }
+    for(uint32_t k = threadIdx.x; k < kernelLen; k += blockDim.x) { kern[k] = asGlobal(g.g)[k]; }
     __syncthreads();
 
+    // The queue is in ascending neuron index, i.e. sorted by input row, so the spikes whose kernel footprint reaches
+    // this block's output rows — input rows [row0 + bh - kh + 1, row0 + rows + bh) — form one contiguous run
+    // [lo, hi): count the spikes in front of either bound.
     GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
     const uint32_t lane = threadIdx.x & (WAVE - 1);
+    const uint32_t wave = threadIdx.x / WAVE, numWaves = blockDim.x / WAVE;
+    const int firstRow = row0 + G.convBH - kh + 1, endRow = row0 + rows + G.convBH;
+    uint32_t below = 0, upto = 0;
+    for(uint32_t s = threadIdx.x; s < numSpikes; s += blockDim.x) {
+        const int myRow = (int)(spk[s] / ic) / iw;
+        below += (myRow < firstRow) ? 1u : 0u;
+        upto += (myRow < endRow) ? 1u : 0u;
+    }
+    for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { below += __shfl_down(below, o2, WAVE); upto += __shfl_down(upto, o2, WAVE); }
+    if(lane == 0) { atomicAdd(&shLo, below); atomicAdd(&shHi, upto); }
+    __syncthreads();
+    const uint32_t lo = shLo, hi = shHi;
     unsigned long long events = 0;
-    for(uint32_t base = 0; base < numSpikes; base += BLOCK) {
-        const uint32_t s = base + threadIdx.x;
-        const uint32_t ipre = (s < numSpikes) ? spk[s] : 0u;
-        const int myRow = (int)(ipre / ic) / iw;
-        // rows this spike can reach: [myRow - bh, myRow - bh + kh - 1]
-        const bool relevant = (s < numSpikes) && (myRow - G.convBH + kh - 1 >= row0) && (myRow - G.convBH < row0 + rows);
-        unsigned long long pending = __ballot(relevant);
-        while(pending) {
-            const int src = __ffsll((long long)pending) - 1;
-            pending &= pending - 1;
-            const uint32_t id = __shfl(ipre, src, WAVE);
-            const int preRow = (int)(id / ic) / iw, preCol = (int)(id / ic) % iw, preChan = (int)(id % ic);
-            for(uint32_t j = lane; j < numDiag; j += WAVE) {
-                const uint32_t e = diag[j];
-                const int kernRow = (int)(e >> 20), kernCol = (int)((e >> 10) & 1023), ch = (int)(e & 1023);
-                const int postRow = preRow + kernRow - G.convBH;
-                const int postCol = preCol + kernCol - G.convBW;
-                if(postRow >= row0 && postRow < row0 + rows && postCol >= 0 && postCol < ow) {
-                    unsafeAtomicAdd(&tile[((postRow - row0) * ow + postCol) * oc + ch],
-                                    kern[((kh - kernRow - 1) * kw + (kw - kernCol - 1)) * ic * oc + preChan * oc + ch]);
-                    events++;
+    // The run is staged in LDS (decoded to row / column / channel) CONV_TILE_SPIKES at a time.  LDS float atomics
+    // retire about one lane per clock, so none are used: every wavefront owns a band of output columns, picks the
+    // staged spikes whose footprint touches its band (64 tested at a time), and adds their contributions to its own
+    // columns with plain read-modify-write.  Per output element the contributions arrive in queue order, the order of
+    // the CPU backend's loop.
+    const int colsPerWave = (ow + (int)numWaves - 1) / (int)numWaves;
+    const int col0 = (int)wave * colsPerWave, col1 = min(ow, col0 + colsPerWave);
+    for(uint32_t base = lo; base < hi; base += CONV_TILE_SPIKES) {
+        const uint32_t count = min((uint32_t)CONV_TILE_SPIKES, hi - base);
+        __syncthreads();
+        for(uint32_t k = threadIdx.x; k < count; k += blockDim.x) {
+            const uint32_t id = spk[base + k];
+            const uint32_t preRow = (id / ic) / iw, preCol = (id / ic) % iw, preChan = id % ic;
+            // a queue that is not sorted would put foreign spikes inside the run: they are marked and skipped
+            const bool relevant = ((int)preRow >= firstRow) && ((int)preRow < endRow);
+            stage[k] = relevant ? (preRow << 20 | preCol << 10 | preChan) : 0xFFFFFFFFu;
+        }
+        __syncthreads();
+        for(uint32_t sb = 0; sb < count && col0 < col1; sb += WAVE) {
+            const uint32_t mine = (sb + lane < count) ? stage[sb + lane] : 0xFFFFFFFFu;
+            const int myCol = (int)((mine >> 10) & 1023) - G.convBW;       // first output column this spike reaches
+            unsigned long long pending = __ballot(mine != 0xFFFFFFFFu && myCol + kw - 1 >= col0 && myCol < col1);
+            while(pending) {
+                const int src = __ffsll((long long)pending) - 1;
+                pending &= pending - 1;
+                // everything about the spike and the kernel position is wavefront-uniform (scalar registers, scalar
+                // branches); only the output channels are spread over the lanes
+                const uint32_t pre = __builtin_amdgcn_readlane(mine, src);
+                const int preRow = (int)(pre >> 20), preCol = (int)((pre >> 10) & 1023), preChan = (int)(pre & 1023);
+                for(int kernRow = 0; kernRow < kh; kernRow++) {
+                    const int postRow = preRow + kernRow - G.convBH;
+                    if(postRow < row0 || postRow >= row0 + rows) { continue; }
+                    for(int kernCol = 0; kernCol < kw; kernCol++) {
+                        const int postCol = preCol + kernCol - G.convBW;
+                        if(postCol < col0 || postCol >= col1) { continue; }
+                        const float *weights = kern + (((kh - kernRow - 1) * kw + (kw - kernCol - 1)) * ic + preChan) * oc;
+                        float *target = tile + ((postRow - row0) * ow + postCol) * oc;
+                        for(int ch = (int)lane; ch < oc; ch += WAVE) { target[ch] += weights[ch]; }
+                        if(lane == 0) { events += (unsigned long long)oc; }
+                    }
                 }
             }
         }
     }
     __syncthreads();
     GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons + (size_t)row0 * ow * oc;
-    for(uint32_t k = threadIdx.x; k < tileLen; k += BLOCK) {
-        const float v = tile[k];
-        if(v != 0.0f) { outPost[k] += v; }
+    // the block owns these rows, so plain read-modify-write; loads of a batch of elements are issued together
+    for(uint32_t k0 = 0; k0 < tileLen; k0 += 8 * blockDim.x) {
+        float old[8];
+        #pragma unroll
+        for(int u = 0; u < 8; u++) { const uint32_t k = k0 + u * blockDim.x + threadIdx.x; old[u] = (k < tileLen) ? outPost[k] : 0.0f; }
+        #pragma unroll
+        for(int u = 0; u < 8; u++) {
+            const uint32_t k = k0 + u * blockDim.x + threadIdx.x;
+            if(k < tileLen) { const float v = tile[k]; if(v != 0.0f) { outPost[k] = old[u] + v; } }
+        }
     }
     for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
     if(lane == 0 && events) { atomicAdd(eventCounter, events); }
@@ -1294,10 +1334,11 @@ int gennmi_runner_finalise(gennmi_runner *r)
         for(auto &p : r->pre) {
             p.workPerSpike = (p.g.matrix == GENNMI_MATRIX_SPARSE) ? p.g.rowStride : (uint32_t)(p.g.conv[0] * p.g.conv[1] * p.g.conv[7]);
             if(tileFloats != 0 && p.g.matrix == GENNMI_MATRIX_TOEPLITZ_CONV2D && r->pre.size() == 1
-               && p.g.conv[0] < 4096 && p.g.conv[1] < 1024 && p.g.conv[7] < 1024) {
+               && p.g.conv[0] < 1024 && p.g.conv[1] < 1024 && p.g.conv[7] < 1024
+               && p.g.conv[2] < 1024 && p.g.conv[3] < 1024 && p.g.conv[4] < 1024) {        // rows, columns and channels are packed 10 bits each
                 const int32_t *c = p.g.conv;
                 const size_t rowFloats = (size_t)c[6] * c[7];
-                const size_t fixedFloats = (size_t)c[0] * c[1] * c[4] * c[7] + (size_t)c[0] * c[1] * c[7];
+                const size_t fixedFloats = (size_t)c[0] * c[1] * c[4] * c[7] + CONV_TILE_SPIKES;      // kernel weights + staged spikes
                 const size_t budgetFloats = 60 * 1024 / sizeof(float);
                 if(fixedFloats + rowFloats <= budgetFloats) {
                     // as many rows per block as fit in LDS, but enough blocks to cover the chip about twice
@@ -1492,7 +1533,7 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
             presynapticTileKernel<<<dim3(r->tileBlocks, r->batch), dim3(r->tileThreads), r->tileFloats * sizeof(float), r->stream>>>(r->dTile, a, r->dt, r->dEvents);
         }
         if(r->convTileBlocks) {
-            presynapticConvTileKernel<<<dim3(r->convTileBlocks, r->batch), dim3(BLOCK), r->convTileBytes, r->stream>>>(r->dConvTile, r->dEvents);
+            presynapticConvTileKernel<<<dim3(r->convTileBlocks, r->batch), dim3(CONV_TILE_THREADS), r->convTileBytes, r->stream>>>(r->dConvTile, r->dEvents);
         }
         if(timed) { const int rc = stamp(r, &e1); if(rc) { return rc; } r->pending.push_back({e0, e1, 0}); }
     }
