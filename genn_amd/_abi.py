@@ -66,7 +66,8 @@ class PostsynapticUpdateGroup(C.Structure):
                 ("colLength", p_u32), ("remap", p_u32), ("g", p_f32),
                 ("trgSpkCnt", p_u32), ("trgSpk", p_u32),
                 ("srcST", p_f32), ("preTrace", p_f32),
-                ("aPlus", C.c_float), ("wMin", C.c_float), ("wMax", C.c_float), ("pad_", C.c_uint32)]
+                ("aPlus", C.c_float), ("wMin", C.c_float), ("wMax", C.c_float), ("pad_", C.c_uint32),
+                ("rowLength", p_u32), ("ind", p_u32)]
 
 
 # every symbol include/genn_mi355x.h declares: (restype, argtypes)

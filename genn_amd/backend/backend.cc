@@ -609,6 +609,7 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                 out << "d.colLength = gennmiDev(" << env["_col_length"] << "); d.remap = gennmiDev(" << env["_remap"] << "); d.g = gennmiDev(" << env["_mi_g"] << ");" << std::endl;
                 out << "d.trgSpkCnt = gennmiDev(" << env["_trg_spk_cnt"] << "); d.trgSpk = gennmiDev(" << env["_trg_spk"] << ");" << std::endl;
                 out << "d.srcST = gennmiDev(" << env["_src_st"] << "); d.preTrace = gennmiDev(" << env["_mi_preTrace"] << ");" << std::endl;
+                out << "d.rowLength = gennmiDev(" << env["_row_length"] << "); d.ind = gennmiDev(" << env["_ind"] << ");" << std::endl;
                 for(const char *p : {"aPlus", "wMin", "wMax"}) {
                     std::vector<Type::NumericValue> v;
                     for(const auto &g : s.getGroups()) { v.push_back(g.get().getWUInitialiser().getParams().at(p)); }

@@ -118,6 +118,7 @@ struct NeuronGroupDev
     const ZeroDelayEntry *zeroEntries;
     uint32_t *shadowSpk;                // [2][batch*N] engine-private double-buffered copy of the spike queue, or NULL
     uint32_t *shadowCnt;                // [2][batch]
+    uint32_t *spikeBitmap;              // [ceil(N/32)] engine-private bitmap of this step's spikes (populations with learnPost), or NULL
 };
 
 struct PreGroupDev
@@ -161,6 +162,8 @@ struct PostGroupDev
     gennmi_postsynaptic_update_group_t g;
     uint32_t startBlock, numBlocks;
     uint32_t lanesPerSpike;
+    uint32_t denseThreshold;            // != 0: steps with at least this many postsynaptic spikes walk the rows instead
+    const uint32_t *spikeBitmap;        // [ceil(numTrg/32)] this step's postsynaptic spikes, written by the neuron update
 };
 
 // Block -> group: groups occupy consecutive block ranges (the reference pads thread ranges to block
@@ -591,6 +594,51 @@ void postsynapticUpdateKernel(const PostGroupDev * __restrict__ blocks, StepArgs
     const uint32_t subGroup = (localBlock * BLOCK + threadIdx.x) / W;
     const uint32_t numSubGroups = (G.numBlocks * BLOCK) / W;
     const uint32_t numSpikes = g.trgSpkCnt[0];
+    if(G.denseThreshold && numSpikes >= G.denseThreshold) {
+        // A large share of the target population fired: nearly every row holds synapses to update, so walk the rows
+        // once (coalesced ind / g) and test each synapse's target against the spike bitmap, instead of one scattered
+        // read-modify-write per (spike, column entry).  Same arithmetic per synapse; every synapse is visited once.
+        extern __shared__ uint32_t shBits[];
+        const uint32_t words = (g.numTrgNeurons + 31) / 32;
+        for(uint32_t k = threadIdx.x; k < words; k += BLOCK) { shBits[k] = asGlobal(G.spikeBitmap)[k]; }
+        __syncthreads();
+        const uint32_t lane = threadIdx.x & (WAVE - 1);
+        const uint32_t numWaves = G.numBlocks * (BLOCK / WAVE);
+        GLOBAL_AS const uint32_t *ind = asGlobal(g.ind);
+        GLOBAL_AS float *weight = asGlobal(g.g);
+        // per-row scalars of the NEXT row are fetched while the current one is processed (indices clamped: readable)
+        const uint32_t lastRow = g.numSrcNeurons - 1;
+        uint32_t row = localBlock * (BLOCK / WAVE) + threadIdx.x / WAVE;
+        uint32_t lenNext = asGlobal(g.rowLength)[min(row, lastRow)];
+        float stNext = asGlobal(g.srcST)[min(row, lastRow)], traceNext = asGlobal(g.preTrace)[min(row, lastRow)];
+        for(; row < g.numSrcNeurons; row += numWaves) {
+            const uint32_t len = lenNext;
+            const float stPre = dt + stNext;
+            const float step = g.aPlus * traceNext;
+            const uint32_t nextRow = min(row + numWaves, lastRow);
+            lenNext = asGlobal(g.rowLength)[nextRow]; stNext = asGlobal(g.srcST)[nextRow]; traceNext = asGlobal(g.preTrace)[nextRow];
+            const float dtSpike = st.t - stPre;
+            if(!(dtSpike > 0) || len == 0) { continue; }
+            const size_t rowBase = (size_t)row * g.rowStride;
+            // up to four strides of the row in flight per lane
+            for(uint32_t j0 = lane; j0 < len; j0 += 4 * WAVE) {
+                uint32_t idPost[4]; float w[4];
+                #pragma unroll
+                for(int u = 0; u < 4; u++) {
+                    const uint32_t j = j0 + u * WAVE;
+                    idPost[u] = (j < len) ? ind[rowBase + j] : 0xFFFFFFFFu;
+                    w[u] = (j < len) ? weight[rowBase + j] : 0.0f;
+                }
+                #pragma unroll
+                for(int u = 0; u < 4; u++) {
+                    if(idPost[u] != 0xFFFFFFFFu && ((shBits[idPost[u] >> 5] >> (idPost[u] & 31)) & 1u)) {
+                        weight[rowBase + j0 + u * WAVE] = fminf(g.wMax, fmaxf(g.wMin, w[u] + step));
+                    }
+                }
+            }
+        }
+        return;
+    }
     for(uint32_t s = subGroup; s < numSpikes; s += numSubGroups) {
         const uint32_t spike = g.trgSpk[s];
         const uint32_t npre = g.colLength[spike];
@@ -751,6 +799,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
         const uint32_t words = (n + 31) / 32;
         g.recordSpk[((size_t)st.recT * gridDim.y + batch) * words + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
     }
+    if(G.spikeBitmap && (lane & 31) == 0 && i < n) { G.spikeBitmap[i >> 5] = (uint32_t)(ballot >> (lane & 32)); }
     __syncthreads();
 
     uint32_t blockCount = 0, waveOffset = 0;
@@ -992,6 +1041,7 @@ struct gennmi_runner
     bool synapsesDone = false;          // updateSynapses ran for the current step
     bool fusedStep = false;             // zero-delay synapses are delivered by the neuron update; one launch per step
     TileGroupDev *dTile = nullptr; uint32_t tileBlocks = 0, tileFloats = 0, tileThreads = BLOCK;
+    uint32_t postLdsBytes = 0;
     ConvTileDev *dConvTile = nullptr; uint32_t convTileBlocks = 0; size_t convTileBytes = 0;
     std::vector<void*> owned;           // engine-private device allocations (shadow queues, zero-delay lists)
     // graph
@@ -1235,6 +1285,7 @@ int gennmi_push_postsynaptic_update_group(gennmi_runner *r, const gennmi_postsyn
     }
     if(g->rowStride == 0 || g->colStride == 0) { return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: zero stride"); }
     if(r->batch != 1) { return fail(GENNMI_EUNSUPPORTED, "push_postsynaptic_update_group: plastic weights need batch size 1"); }
+    if((g->rowLength == nullptr) != (g->ind == nullptr)) { return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: rowLength and ind go together"); }
     PostGroupDev d;
     memset(&d, 0, sizeof(d));
     d.g = *g;
@@ -1477,6 +1528,30 @@ int gennmi_runner_finalise(gennmi_runner *r)
         }
         r->fusedStep = true;
     }
+    // ---- dense-activity path of learnPost: the neuron update of the target population keeps a bitmap of the step's
+    // spikes, and steps in which at least 1/8 of the targets fired walk the rows
+    for(auto &p : r->post) {
+        const uint32_t words = (p.g.numTrgNeurons + 31) / 32;
+        if(!p.g.rowLength || !p.g.ind || words * sizeof(uint32_t) > 60 * 1024) { continue; }
+        for(auto &n : r->neuron) {
+            bool feeds = (n.g.spk == p.g.trgSpk);
+            for(uint32_t q = 0; q < n.g.numExtraSpk; q++) { feeds = feeds || (n.g.extraSpk[q] == p.g.trgSpk); }
+            if(!feeds || n.g.numNeurons != p.g.numTrgNeurons) { continue; }
+            if(!n.spikeBitmap) {
+                HIP_TRY(hipMalloc((void**)&n.spikeBitmap, words * sizeof(uint32_t)));
+                HIP_TRY(hipMemset(n.spikeBitmap, 0, words * sizeof(uint32_t)));
+                r->owned.push_back(n.spikeBitmap);
+            }
+            p.spikeBitmap = n.spikeBitmap;
+            const char *envDiv = getenv("GENNMI_POST_DENSE_DIVISOR");      // rows are walked from numTrg / divisor spikes on (0: never)
+            const uint32_t divisor = envDiv ? (uint32_t)std::max(0, atoi(envDiv)) : 8u;
+            p.denseThreshold = divisor ? std::max(1u, p.g.numTrgNeurons / divisor) : 0u;
+            r->postLdsBytes = std::max<uint32_t>(r->postLdsBytes, words * sizeof(uint32_t));
+        }
+    }
+    if(r->postLdsBytes > 48 * 1024) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(postsynapticUpdateKernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)r->postLdsBytes));
+    }
     HIP_TRY(uploadPerBlock(r->neuron, r->neuronBlocks, &r->dNeuron));
     HIP_TRY(uploadPerBlock(r->pre, r->preBlocks, &r->dPre));
     HIP_TRY(uploadPerBlock(r->post, r->postBlocks, &r->dPost));
@@ -1538,7 +1613,7 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
         if(timed) { const int rc = stamp(r, &e1); if(rc) { return rc; } r->pending.push_back({e0, e1, 0}); }
     }
     if(!r->post.empty()) {
-        postsynapticUpdateKernel<<<dim3(r->postBlocks), dim3(BLOCK), 0, r->stream>>>(r->dPost, a, r->dt);
+        postsynapticUpdateKernel<<<dim3(r->postBlocks), dim3(BLOCK), r->postLdsBytes, r->stream>>>(r->dPost, a, r->dt);
         if(timed) { const int rc = stamp(r, &e2); if(rc) { return rc; } r->pending.push_back({e1 ? e1 : e0, e2, 1}); }
     }
     HIP_TRY(hipGetLastError());

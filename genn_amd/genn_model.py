@@ -589,6 +589,7 @@ class GeNNModel:
                     q.colLength, q.remap, q.g = s.vars["colLength"].ptr, s.vars["remap"].ptr, s.vars["g"].ptr
                     q.trgSpkCnt, q.trgSpk = s.trg.vars["spkCnt"].ptr, s.trg.vars["spk"].ptr
                     q.srcST, q.preTrace = s.src.vars["sT"].ptr, s.vars["preTrace"].ptr
+                    q.rowLength, q.ind = s.vars["rowLength"].ptr, s.vars["ind"].ptr
                     q.aPlus, q.wMin, q.wMax = rounded["aPlus"][k], rounded["wMin"][k], rounded["wMax"][k]
                     _abi.check(lib.gennmi_push_postsynaptic_update_group(self._runner, C.byref(q), None))
 

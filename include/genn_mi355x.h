@@ -166,6 +166,10 @@ typedef struct gennmi_postsynaptic_update_group_t { /* MergedPostsynapticUpdateG
     const float *srcST, *preTrace;
     float aPlus, wMin, wMax;
     uint32_t pad_;
+    /* row view of the same matrix (optional, both or neither): lets a step in which a large share of the target
+     * population fired walk the rows once, coalesced, instead of one gather per (spike, column entry) */
+    const uint32_t *rowLength;            /* [numSrcNeurons] */
+    const uint32_t *ind;                  /* [numSrcNeurons*rowStride] */
 } gennmi_postsynaptic_update_group_t;
 
 /* ---------------------------------------------------------------------------------------------

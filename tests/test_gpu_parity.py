@@ -118,6 +118,34 @@ def test_plastic_stdp_learn_post():
     model.unload()
 
 
+@pytest.mark.parametrize("divisor", ["1000000", "0"])
+def test_learn_post_row_walk_and_column_walk(divisor, monkeypatch):
+    """learnPost has two device paths: columns of the spiking targets through the remap (few spikes) and a walk over
+    all rows with a bitmap of the spiking targets (many spikes).  Forcing either for every step must leave the same
+    weights as the oracle: each synapse gets the same single update, so g must agree to the last bit of the tolerance
+    used everywhere else (and the two device paths with each other exactly)."""
+    monkeypatch.setenv("GENNMI_POST_DENSE_DIVISOR", divisor)
+    net = configs.plastic_stdp(n=3000, n_src=100, steps=120, fan=150, src_fan=50)
+    model = model_from_net(net)
+    model.load(num_recording_timesteps=net.steps)
+    sg = model.synapse_populations["EE"]
+    oracle = OracleNet(net, col_stride={"EE": sg.col_stride})
+    spikes = 0
+    for step in range(net.steps):
+        model.step_time()
+        oracle.step()
+        for p in net.pops:
+            want = oracle.spikes(p.name)
+            assert np.array_equal(model.neuron_populations[p.name].current_spikes[0], want), f"step {step}: spike queue of {p.name} differs"
+            spikes += len(want)
+        if (step + 1) % 30 == 0:
+            compare_state(net, model, oracle, f"step {step}", exact=False)
+    assert spikes > 1000
+    changed = np.count_nonzero(sg.vars["g"].pull_from_device() != net.syn("EE").g.reshape(-1))
+    assert changed > 1000, "no weight was updated"
+    model.unload()
+
+
 def test_toeplitz_conv_layer():
     """C5 shape at 16x16x4 -> 16x16x8 (batch 1; the oracle, like the reference's CPU backend, has no batch)."""
     net = configs.conv_toeplitz(h=16, w=16, ic=4, oc=8, steps=150, w_sd=0.5)
