@@ -73,6 +73,9 @@ def main():
     ap.add_argument("--workload", default="potjans")
     ap.add_argument("--cpu-steps", type=int, default=None, help="steps of the CPU baseline sample (default: sized for ~10-20 s)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--reference-steps", type=int, default=2000,
+                    help="steps of the extra CPU leg on the reference's own SingleThreadedCPU backend (oracle/_ref/ref_driver, "
+                         "only where that prebuilt driver exists; 0 disables)")
     ap.add_argument("--profile-steps", type=int, default=2000, help="extra steps replayed with HIP event nodes around every kernel (multiple of 100)")
     ap.add_argument("--yardstick-mib", type=int, default=0,
                     help="also run the library's plain copy kernel on this many MiB (5 launches, 2x this traffic each), so a "
@@ -194,6 +197,37 @@ def main():
                "wall_s_per_sim_s": round(cpu_wall / (cpu_steps * net.dt / 1000.0), 3),
                "host_cores": os.cpu_count()}
         oracle.close()
+
+    # ---- the same network on the reference's OWN SingleThreadedCPU backend (generated code compiled -O3), where
+    # the prebuilt driver exists: wall-clock of its Runtime::stepTime loop over a bounded number of steps
+    if cpu is not None and args.reference_steps > 0 and batch == 1:
+        driver = os.path.join(ROOT, "oracle", "_ref", "ref_driver")
+        if os.path.exists(driver):
+            import re
+            import shutil
+            import subprocess
+            import tempfile
+            from genn_amd.netspec import write_netspec
+            tmp = tempfile.mkdtemp(prefix="bench_ref_")
+            try:
+                spec, work, out_dir = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+                os.makedirs(work); os.makedirs(out_dir)
+                old_steps, net.steps, net.snap = net.steps, args.reference_steps, 0
+                write_netspec(net, spec)
+                net.steps = old_steps
+                res = subprocess.run([driver, spec, work, out_dir, "--cxxflags=-O3"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+                m = re.search(r"stepping loop ([0-9.eE+-]+) s for (\d+) steps", res.stdout)
+                if res.returncode == 0 and m:
+                    ref_wall, ref_steps = float(m.group(1)), int(m.group(2))
+                    cpu["reference_backend"] = {"kind": "reference", "what": "genn-team/genn SingleThreadedCPU backend through Runtime::stepTime, generated code built -O3",
+                                                "steps": ref_steps, "wall_s": round(ref_wall, 3),
+                                                "wall_s_per_sim_s": round(ref_wall / (ref_steps * net.dt / 1000.0), 3), "cores": 1}
+                else:
+                    cpu["reference_backend"] = {"error": res.stdout[-300:]}
+            except Exception as e:      # the baseline is a reported extra: never let it take the bench line down
+                cpu["reference_backend"] = {"error": repr(e)}
+            finally:
+                shutil.rmtree(tmp, ignore_errors=True)
 
     sim_s = args.steps * net.dt / 1000.0
     out = {

@@ -128,12 +128,20 @@ struct SynSpec
 int main(int argc, char *argv[])
 {
     try {
-        if(argc != 4 && argc != 5) { std::cerr << "usage: ref_driver <netspec dir> <work dir> <out dir> [--generate-only]" << std::endl; return 1; }
+        if(argc < 4) { std::cerr << "usage: ref_driver <netspec dir> <work dir> <out dir> [--generate-only] [--cxxflags=<flags>]" << std::endl; return 1; }
         const std::string in = argv[1], work = argv[2], out = argv[3];
-        const bool generateOnly = (argc == 5 && std::string(argv[4]) == "--generate-only");
+        bool generateOnly = false;
+        std::string userCxxFlags;
+        for(int a = 4; a < argc; a++) {
+            const std::string opt = argv[a];
+            if(opt == "--generate-only") { generateOnly = true; }
+            else if(opt.rfind("--cxxflags=", 0) == 0) { userCxxFlags = opt.substr(11); }      // e.g. -O3: same results as the default build, faster
+            else { std::cerr << "unknown option " << opt << std::endl; return 1; }
+        }
 
         plog::ConsoleAppender<plog::TxtFormatter> app;
         Preferences prefs;
+        prefs.userCxxFlagsGNU = userCxxFlags;
         Logging::init(prefs.gennLogLevel, prefs.codeGeneratorLogLevel, prefs.transpilerLogLevel,
                       prefs.runtimeLogLevel, &app, &app, &app, &app);
 
