@@ -70,6 +70,10 @@ class PostsynapticUpdateGroup(C.Structure):
                 ("rowLength", p_u32), ("ind", p_u32)]
 
 
+INIT_SNIPPETS = {"Constant": 0, "Uniform": 1, "Normal": 2, "NormalClipped": 3, "NormalClippedDelay": 4, "Exponential": 5,
+                 "Gamma": 6, "Binomial": 7}
+ELEMENT_TYPES = {"float32": 0, "uint32": 1, "int32": 2, "uint16": 3, "uint8": 4}
+
 # every symbol include/genn_mi355x.h declares: (restype, argtypes)
 _ULL = C.c_ulonglong
 SYMBOLS = {
@@ -99,6 +103,14 @@ SYMBOLS = {
     "gennmi_runner_finalise": (C.c_int, [C.c_void_p]),
     "gennmi_build_remap": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "gennmi_max_col_length": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]),
+    "gennmi_init_var": (C.c_int, [C.c_void_p, C.c_uint32, C.c_size_t, C.c_uint32, C.POINTER(C.c_double * 4), C.c_uint64, C.c_uint32]),
+    "gennmi_init_sparse_fixed_probability": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_double, C.c_int, C.c_uint64, C.c_uint32,
+                                                       C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]),
+    "gennmi_init_sparse_fixed_number_post": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_uint64, C.c_uint32,
+                                                       C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]),
+    "gennmi_init_sparse_one_to_one": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]),
+    "gennmi_philox4x32": (C.c_int, [C.POINTER(C.c_uint32 * 4), C.POINTER(C.c_uint32 * 2), C.POINTER(C.c_uint32 * 4)]),
+    "gennmi_init_random_words": (C.c_int, [C.c_void_p, C.c_size_t, C.c_uint64, C.c_uint32]),
     "gennmi_update_synapses": (C.c_int, [C.c_void_p, C.c_float]),
     "gennmi_update_neurons": (C.c_int, [C.c_void_p, C.c_float, C.c_uint32]),
     "gennmi_step_time": (C.c_int, [C.c_void_p, _ULL, _ULL]),

@@ -1056,6 +1056,12 @@ struct gennmi_runner
     hipEvent_t marks[2] = {nullptr, nullptr};               // gennmi_runner_stream_mark
 };
 
+namespace gennmi_detail
+{
+// error reporting for the library's other translation units
+int fail(int code, const std::string &msg) { return ::fail(code, msg); }
+}
+
 extern "C" {
 
 const char *gennmi_last_error(void) { return g_lastError.c_str(); }

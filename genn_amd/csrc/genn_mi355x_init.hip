@@ -1,0 +1,455 @@
+// On-device initialisation for the MI355X (gfx950) device layer: the reference's built-in
+// connectivity snippets (include/genn/genn/initSparseConnectivitySnippet.h:107-330) and value
+// snippets (include/genn/genn/initVarSnippet.h:87-262), which its GPU backends run inside
+// initializeKernel / initializeSparseKernel (src/genn/genn/code_generator/backendSIMT.cc:1482-1779).
+//
+// The reference gives every thread a hiprand Philox state and lets one thread walk one row
+// (src/genn/backends/hip/backend.cc:32-50); the draws a given synapse sees therefore depend on the
+// backend, and the reference's own tests only ask for the right distribution
+// (tests/features/test_connect_init.py, test_rng.py).  Here every draw is a pure function of
+// (seed, stream, row or element, draw number) through Philox4x32-10, so a result does not depend on
+// the launch geometry, and a wavefront can generate a row twice (count, then write) without storing it:
+//
+//   * a row belongs to one wave64, so the row's `ind` entries leave the wave as whole cache lines;
+//   * FixedProbability: the geometric-skip walk of the snippet runs independently inside each lane's
+//     slice of the row (Bernoulli trials of different pairs are independent), lane counts are
+//     prefix-summed across the wave;
+//   * FixedNumber*WithReplacement: the snippet draws ascending targets one after the other from the
+//     first order statistic of what is left; the same joint distribution — sorted uniforms — is
+//     produced in parallel as normalised prefix sums of n+1 exponential spacings;
+//   * value snippets stream: one Philox call per four elements, 16-byte stores.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <string>
+
+#include "genn_mi355x.h"
+
+namespace gennmi_detail { int fail(int code, const std::string &msg); }
+
+namespace
+{
+constexpr int WAVE = 64;
+constexpr int BLOCK = 256;
+
+#define HIP_TRY(expr)                                                                                          \
+    do {                                                                                                       \
+        hipError_t e_ = (expr);                                                                                \
+        if(e_ != hipSuccess) {                                                                                 \
+            return gennmi_detail::fail(GENNMI_EHIP, std::string(#expr) + ": " + hipGetErrorString(e_));       \
+        }                                                                                                      \
+    } while(0)
+
+// Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11)
+struct Words { uint32_t w[4]; };
+
+__host__ __device__ inline uint32_t mulHi(uint32_t a, uint32_t b) { return (uint32_t)(((unsigned long long)a * b) >> 32); }
+
+__host__ __device__ inline Words philox4x32(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1)
+{
+    #pragma unroll
+    for(int round = 0; round < 10; round++) {
+        const uint32_t hi0 = mulHi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+        const uint32_t hi1 = mulHi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+        c0 = hi1 ^ c1 ^ k0;
+        c1 = lo1;
+        c2 = hi0 ^ c3 ^ k1;
+        c3 = lo0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    return Words{{c0, c1, c2, c3}};
+}
+
+// A stream of draws: key = the 64-bit seed, counter = (index low, index high, sub-counter, stream number).
+struct Stream
+{
+    uint32_t k0, k1, stream;
+    __host__ __device__ Words at(unsigned long long index, uint32_t sub) const
+    {
+        return philox4x32((uint32_t)index, (uint32_t)(index >> 32), sub, stream, k0, k1);
+    }
+};
+
+__device__ __forceinline__ float uniformHalfOpen(uint32_t x) { return (float)(x >> 8) * (1.0f / 16777216.0f); }              // [0, 1)
+__device__ __forceinline__ float uniformOpen(uint32_t x) { return ((float)(x >> 8) + 0.5f) * (1.0f / 16777216.0f); }         // (0, 1)
+
+// four standard normals from four words (Box-Muller, both branches)
+__device__ __forceinline__ void normals(const Words &r, float n[4])
+{
+    #pragma unroll
+    for(int p = 0; p < 2; p++) {
+        const float radius = sqrtf(-2.0f * logf(uniformOpen(r.w[2 * p])));
+        float s, c;
+        sincospif(2.0f * uniformHalfOpen(r.w[2 * p + 1]), &s, &c);
+        n[2 * p] = radius * c;
+        n[2 * p + 1] = radius * s;
+    }
+}
+
+template<typename T> struct Quad;
+template<> struct Quad<float> { typedef float4 type; };
+template<> struct Quad<uint32_t> { typedef uint4 type; };
+template<> struct Quad<int32_t> { typedef int4 type; };
+template<> struct Quad<uint16_t> { typedef ushort4 type; };
+template<> struct Quad<uint8_t> { typedef uchar4 type; };
+
+// Marsaglia & Tsang (2000) for shape >= 1; shape < 1 through gamma(a + 1) * u^(1/a)
+__device__ float gammaDraw(const Stream &s, unsigned long long element, float a)
+{
+    const float boost = (a < 1.0f) ? 1.0f : 0.0f;
+    const float d = (a + boost) - (1.0f / 3.0f);
+    const float c = 1.0f / sqrtf(9.0f * d);
+    for(uint32_t attempt = 0; ; attempt++) {
+        const Words r = s.at(element, attempt);
+        float n[4];
+        normals(r, n);
+        // words 0 and 1 give the normal, word 3 the acceptance uniform, word 2 the uniform of the shape < 1 correction
+        const float x = n[0];
+        float v = 1.0f + c * x;
+        if(v <= 0.0f) { continue; }
+        v = v * v * v;
+        const float u = uniformOpen(r.w[3]);
+        if(u < 1.0f - 0.0331f * (x * x) * (x * x) || logf(u) < 0.5f * x * x + d * (1.0f - v + logf(v))) {
+            float g = d * v;
+            if(boost != 0.0f) { g *= powf(uniformOpen(r.w[2]), 1.0f / a); }
+            return g;
+        }
+    }
+}
+
+// Binomial(n, p) by inversion of the CDF from k = 0 (Kachitvichyanukul & Schmeiser's BINV recurrence), applied to
+// slices of n short enough that (1-p)^slice stays a normal double; the slices' counts add up
+__device__ uint32_t binomialDraw(const Stream &s, unsigned long long element, uint32_t n, double p)
+{
+    if(p <= 0.0 || n == 0) { return 0; }
+    if(p >= 1.0) { return n; }
+    const bool flip = p > 0.5;
+    const double pp = flip ? 1.0 - p : p;
+    const double logQ = log1p(-pp);
+    const uint32_t maxSlice = (uint32_t)fmin(4.0e9, fmax(1.0, floor(-600.0 / logQ)));
+    const double ratio = pp / (1.0 - pp);
+    uint32_t total = 0, done = 0, call = 0;
+    while(done < n) {
+        const uint32_t m = min(maxSlice, n - done);
+        const Words r = s.at(element, call++);
+        double u = ((double)r.w[0] * 4294967296.0 + (double)r.w[1] + 0.5) * (1.0 / 18446744073709551616.0);
+        double pmf = exp((double)m * logQ);
+        uint32_t k = 0;
+        while(u > pmf && k < m) {
+            u -= pmf;
+            k++;
+            pmf *= ratio * (double)(m - k + 1) / (double)k;
+        }
+        total += k;
+        done += m;
+    }
+    return flip ? n - total : total;
+}
+
+struct VarInit { uint32_t snippet; float p[4]; double p64[2]; };
+
+// value of element `e` whose group of four shares the Philox call `r` (attempt 0); slot = e % 4
+__device__ __forceinline__ float drawValue(const VarInit &v, const Stream &s, unsigned long long group, int slot, const Words &r, const float n[4])
+{
+    switch(v.snippet) {
+    case GENNMI_INIT_CONSTANT:
+        return v.p[0];
+    case GENNMI_INIT_UNIFORM: {
+        const float scale = v.p[1] - v.p[0];
+        return v.p[0] + (uniformHalfOpen(r.w[slot]) * scale);
+    }
+    case GENNMI_INIT_NORMAL:
+        return v.p[0] + (n[slot] * v.p[1]);
+    case GENNMI_INIT_NORMAL_CLIPPED:
+    case GENNMI_INIT_NORMAL_CLIPPED_DELAY: {
+        float value = v.p[0] + (n[slot] * v.p[1]);
+        for(uint32_t attempt = 1; value > v.p[3] || value < v.p[2]; attempt++) {
+            float retry[4];
+            normals(s.at(group, attempt), retry);
+            value = v.p[0] + (retry[slot] * v.p[1]);
+        }
+        return (v.snippet == GENNMI_INIT_NORMAL_CLIPPED_DELAY) ? rintf(value) : value;
+    }
+    case GENNMI_INIT_EXPONENTIAL:
+        return v.p[0] * -logf(uniformOpen(r.w[slot]));
+    default:
+        return 0.0f;
+    }
+}
+
+template<typename T>
+__global__ __launch_bounds__(BLOCK)
+void initVarKernel(T *out, unsigned long long count, VarInit v, Stream s)
+{
+    typedef typename Quad<T>::type Q;
+    const unsigned long long groups = (count + 3) / 4;
+    for(unsigned long long g = (unsigned long long)blockIdx.x * BLOCK + threadIdx.x; g < groups; g += (unsigned long long)gridDim.x * BLOCK) {
+        T value[4];
+        if(v.snippet == GENNMI_INIT_GAMMA || v.snippet == GENNMI_INIT_BINOMIAL) {
+            for(int k = 0; k < 4; k++) {
+                const unsigned long long e = g * 4 + k;
+                if(e < count) {
+                    value[k] = (v.snippet == GENNMI_INIT_GAMMA) ? (T)(v.p[1] * gammaDraw(s, e, v.p[0]))
+                                                               : (T)binomialDraw(s, e, (uint32_t)v.p64[0], v.p64[1]);
+                }
+            }
+        }
+        else {
+            const Words r = s.at(g, 0);
+            float n[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if(v.snippet == GENNMI_INIT_NORMAL || v.snippet == GENNMI_INIT_NORMAL_CLIPPED || v.snippet == GENNMI_INIT_NORMAL_CLIPPED_DELAY) {
+                normals(r, n);
+            }
+            #pragma unroll
+            for(int k = 0; k < 4; k++) { value[k] = (T)drawValue(v, s, g, k, r, n); }
+        }
+        if(g * 4 + 3 < count) {
+            Q q;
+            q.x = value[0]; q.y = value[1]; q.z = value[2]; q.w = value[3];
+            *reinterpret_cast<Q*>(out + g * 4) = q;
+        }
+        else {
+            for(int k = 0; k < 4 && g * 4 + k < count; k++) { out[g * 4 + k] = value[k]; }
+        }
+    }
+}
+
+__global__ __launch_bounds__(BLOCK)
+void randomWordsKernel(uint32_t *out, unsigned long long count, Stream s)
+{
+    const unsigned long long groups = (count + 3) / 4;
+    for(unsigned long long g = (unsigned long long)blockIdx.x * BLOCK + threadIdx.x; g < groups; g += (unsigned long long)gridDim.x * BLOCK) {
+        const Words r = s.at(g, 0);
+        for(int k = 0; k < 4 && g * 4 + k < count; k++) { out[g * 4 + k] = r.w[k]; }
+    }
+}
+
+// ---- wave64 scans
+__device__ __forceinline__ uint32_t waveInclusiveScan(uint32_t v, int lane)
+{
+    #pragma unroll
+    for(int d = 1; d < WAVE; d <<= 1) {
+        const uint32_t o = __shfl_up(v, d, WAVE);
+        if(lane >= d) { v += o; }
+    }
+    return v;
+}
+__device__ __forceinline__ double waveInclusiveScan(double v, int lane)
+{
+    #pragma unroll
+    for(int d = 1; d < WAVE; d <<= 1) {
+        const double o = __shfl_up(v, d, WAVE);
+        if(lane >= d) { v += o; }
+    }
+    return v;
+}
+
+__device__ uint32_t g_rowOverflow;      // rows that wanted more entries than rowStride, last connectivity launch
+
+// FixedProbability / FixedProbabilityNoAutapse (initSparseConnectivitySnippet.h:170-187, 208-230): one row per wave64.
+// Lane l owns post indices [l*slice, (l+1)*slice) and walks them with the snippet's geometric skips
+// `prev += 1 + (int)(log(u) * probLogRecip)`; the walk is memoryless, so restarting it at a slice boundary, or
+// stepping over the diagonal without emitting (the snippet redraws instead), leaves the distribution unchanged.
+__global__ __launch_bounds__(BLOCK)
+void fixedProbabilityKernel(uint32_t numPre, uint32_t numPost, uint32_t rowStride, float probLogRecip, int noAutapse, Stream s,
+                            uint32_t *rowLength, uint32_t *ind)
+{
+    const int lane = threadIdx.x & (WAVE - 1);
+    const uint32_t row = blockIdx.x * (BLOCK / WAVE) + threadIdx.x / WAVE;
+    if(row >= numPre) { return; }
+    const uint32_t slice = (numPost + WAVE - 1) / WAVE;
+    const uint32_t begin = min(numPost, (uint32_t)lane * slice), end = min(numPost, begin + slice);
+    uint32_t offset = 0;
+    for(int pass = 0; pass < 2; pass++) {
+        uint32_t count = 0, draw = 0;
+        long long j = (long long)begin - 1;
+        Words r;
+        while(true) {
+            if((draw & 3u) == 0) { r = s.at(((unsigned long long)row << 32) | (draw >> 2), (uint32_t)lane); }
+            const float skip = logf(uniformOpen(r.w[draw & 3u])) * probLogRecip;
+            draw++;
+            if(skip >= (float)(end - begin)) { break; }
+            j += 1 + (int)skip;
+            if(j >= (long long)end) { break; }
+            if(noAutapse && j == (long long)row) { continue; }
+            if(pass == 1 && offset + count < rowStride) { ind[(size_t)row * rowStride + offset + count] = (uint32_t)j; }
+            count++;
+        }
+        if(pass == 0) {
+            const uint32_t inclusive = waveInclusiveScan(count, lane);
+            offset = inclusive - count;
+            const uint32_t total = __shfl(inclusive, WAVE - 1, WAVE);
+            if(lane == 0) {
+                rowLength[row] = min(total, rowStride);
+                if(total > rowStride) { atomicAdd(&g_rowOverflow, 1u); }
+            }
+        }
+    }
+}
+
+// FixedNumberPostWithReplacement / FixedNumberTotalWithReplacement (initSparseConnectivitySnippet.h:242-276, 292-370): one row
+// per wave64.  The snippet's loop `x += (1 - x) * (1 - pow(u, 1/c))` for c = n..1 draws the n order statistics of n uniforms in
+// ascending order.  The same joint law is S_k / S_{n+1} with S the prefix sums of n+1 unit exponentials, which a wave computes
+// 64 draws at a time with a scan: first the total, then — regenerating the same draws — the normalised prefix sums.
+__global__ __launch_bounds__(BLOCK)
+void fixedNumberPostKernel(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t num, const uint32_t *rowLengthIn, Stream s,
+                           uint32_t *rowLength, uint32_t *ind)
+{
+    const int lane = threadIdx.x & (WAVE - 1);
+    const uint32_t row = blockIdx.x * (BLOCK / WAVE) + threadIdx.x / WAVE;
+    if(row >= numPre) { return; }
+    uint32_t n = rowLengthIn ? rowLengthIn[row] : num;
+    if(n > rowStride) {
+        if(lane == 0) { atomicAdd(&g_rowOverflow, 1u); }
+        n = rowStride;
+    }
+    double total = 0.0;
+    for(int pass = 0; pass < 2; pass++) {
+        double carry = 0.0;
+        // draws 0..n: spacing k ends at target k; spacing n is the gap between the largest target and 1
+        for(uint32_t base = 0; base <= n; base += WAVE) {
+            const uint32_t k = base + lane;
+            const Words r = s.at(((unsigned long long)row << 32) | (k >> 2), 0);
+            const double spacing = (k <= n) ? (double)-logf(uniformOpen(r.w[k & 3u])) : 0.0;
+            const double inclusive = carry + waveInclusiveScan(spacing, lane);
+            if(pass == 1 && k < n) {
+                const uint32_t post = (uint32_t)((inclusive / total) * (double)numPost);
+                ind[(size_t)row * rowStride + k] = min(post, numPost - 1);
+            }
+            carry = __shfl(inclusive, WAVE - 1, WAVE);
+        }
+        total = carry;
+    }
+    if(lane == 0) { rowLength[row] = n; }
+}
+
+// OneToOne (initSparseConnectivitySnippet.h:107-118)
+__global__ void oneToOneKernel(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t *rowLength, uint32_t *ind)
+{
+    const uint32_t row = blockIdx.x * blockDim.x + threadIdx.x;
+    if(row < numPre) {
+        const bool valid = row < numPost;
+        rowLength[row] = valid ? 1u : 0u;
+        if(valid) { ind[(size_t)row * rowStride] = row; }
+    }
+}
+
+Stream makeStream(uint64_t seed, uint32_t stream) { return Stream{(uint32_t)seed, (uint32_t)(seed >> 32), stream}; }
+
+int finishConnectivity(uint32_t *overflowRows)
+{
+    HIP_TRY(hipGetLastError());
+    uint32_t overflow = 0;
+    HIP_TRY(hipMemcpyFromSymbol(&overflow, HIP_SYMBOL(g_rowOverflow), sizeof(uint32_t)));
+    if(overflowRows) { *overflowRows = overflow; }
+    if(overflow) {
+        return gennmi_detail::fail(GENNMI_EINVAL, std::to_string(overflow) + " row(s) drew more synapses than rowStride holds; the rows were truncated");
+    }
+    return GENNMI_OK;
+}
+
+int clearOverflow()
+{
+    const uint32_t zero = 0;
+    HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(g_rowOverflow), &zero, sizeof(uint32_t)));
+    return GENNMI_OK;
+}
+
+template<typename T>
+int launchInitVar(void *dev, size_t count, const VarInit &v, const Stream &s)
+{
+    const unsigned long long groups = (count + 3) / 4;
+    const unsigned int blocks = (unsigned int)std::min<unsigned long long>((groups + BLOCK - 1) / BLOCK, 256ull * 32ull);
+    hipLaunchKernelGGL(initVarKernel<T>, dim3(blocks), dim3(BLOCK), 0, 0, (T*)dev, (unsigned long long)count, v, s);
+    HIP_TRY(hipGetLastError());
+    return GENNMI_OK;
+}
+}   // anonymous namespace
+
+extern "C" {
+
+int gennmi_philox4x32(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4])
+{
+    const Words r = philox4x32(counter[0], counter[1], counter[2], counter[3], key[0], key[1]);
+    for(int k = 0; k < 4; k++) { out[k] = r.w[k]; }
+    return GENNMI_OK;
+}
+
+int gennmi_init_random_words(uint32_t *dev, size_t count, uint64_t seed, uint32_t stream)
+{
+    if(count == 0) { return GENNMI_OK; }
+    const unsigned long long groups = (count + 3) / 4;
+    const unsigned int blocks = (unsigned int)std::min<unsigned long long>((groups + BLOCK - 1) / BLOCK, 256ull * 32ull);
+    hipLaunchKernelGGL(randomWordsKernel, dim3(blocks), dim3(BLOCK), 0, 0, dev, (unsigned long long)count, makeStream(seed, stream));
+    HIP_TRY(hipGetLastError());
+    return GENNMI_OK;
+}
+
+int gennmi_init_var(void *dev, uint32_t elementType, size_t count, uint32_t snippet, const double params[4], uint64_t seed, uint32_t stream)
+{
+    if(count == 0) { return GENNMI_OK; }
+    if(snippet > GENNMI_INIT_BINOMIAL) { return gennmi_detail::fail(GENNMI_EUNSUPPORTED, "unknown value-initialisation snippet"); }
+    if((uintptr_t)dev % 16) { return gennmi_detail::fail(GENNMI_EINVAL, "array to initialise is not 16-byte aligned"); }
+    VarInit v;
+    v.snippet = snippet;
+    for(int k = 0; k < 4; k++) { v.p[k] = (float)params[k]; }
+    v.p64[0] = params[0];
+    v.p64[1] = params[1];
+    if((snippet == GENNMI_INIT_NORMAL_CLIPPED || snippet == GENNMI_INIT_NORMAL_CLIPPED_DELAY) && !(v.p[2] < v.p[3])) {
+        return gennmi_detail::fail(GENNMI_EINVAL, "clipped normal needs min < max");
+    }
+    if(snippet == GENNMI_INIT_GAMMA && !(v.p[0] > 0.0f)) { return gennmi_detail::fail(GENNMI_EINVAL, "gamma shape must be positive"); }
+    if(snippet == GENNMI_INIT_BINOMIAL && !(params[0] >= 0.0 && params[0] < 4294967296.0 && params[1] >= 0.0 && params[1] <= 1.0)) {
+        return gennmi_detail::fail(GENNMI_EINVAL, "binomial needs 0 <= n < 2^32 and 0 <= p <= 1");
+    }
+    const Stream s = makeStream(seed, stream);
+    switch(elementType) {
+    case GENNMI_TYPE_F32: return launchInitVar<float>(dev, count, v, s);
+    case GENNMI_TYPE_U32: return launchInitVar<uint32_t>(dev, count, v, s);
+    case GENNMI_TYPE_I32: return launchInitVar<int32_t>(dev, count, v, s);
+    case GENNMI_TYPE_U16: return launchInitVar<uint16_t>(dev, count, v, s);
+    case GENNMI_TYPE_U8: return launchInitVar<uint8_t>(dev, count, v, s);
+    default: return gennmi_detail::fail(GENNMI_EUNSUPPORTED, "unknown element type");
+    }
+}
+
+int gennmi_init_sparse_fixed_probability(uint32_t numPre, uint32_t numPost, uint32_t rowStride, double prob, int noAutapse,
+                                         uint64_t seed, uint32_t stream, uint32_t *rowLength, uint32_t *ind, uint32_t *overflowRows)
+{
+    if(!(prob >= 0.0 && prob <= 1.0)) { return gennmi_detail::fail(GENNMI_EINVAL, "connection probability outside [0, 1]"); }
+    if(numPre == 0 || numPost == 0 || rowStride == 0) { return gennmi_detail::fail(GENNMI_EINVAL, "empty matrix"); }
+    if(numPost > 0x7fffffffu || rowStride > 0x7fffffffu) { return gennmi_detail::fail(GENNMI_EINVAL, "more than 2^31-1 postsynaptic neurons or row entries"); }
+    if(int rc = clearOverflow()) { return rc; }
+    // probLogRecip = 1 / log(1 - prob) as the snippet's derived parameter; prob = 0 gives -inf (every skip leaves the row),
+    // prob = 1 gives -0 (every skip is 0: all pairs connect)
+    const float probLogRecip = (prob == 0.0) ? -INFINITY : (float)(1.0 / std::log(1.0 - prob));
+    const unsigned int blocks = (numPre + (BLOCK / WAVE) - 1) / (BLOCK / WAVE);
+    hipLaunchKernelGGL(fixedProbabilityKernel, dim3(blocks), dim3(BLOCK), 0, 0, numPre, numPost, rowStride, probLogRecip, noAutapse,
+                       makeStream(seed, stream), rowLength, ind);
+    return finishConnectivity(overflowRows);
+}
+
+int gennmi_init_sparse_fixed_number_post(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t num, const uint32_t *rowLengthIn,
+                                         uint64_t seed, uint32_t stream, uint32_t *rowLength, uint32_t *ind, uint32_t *overflowRows)
+{
+    if(numPre == 0 || numPost == 0 || rowStride == 0) { return gennmi_detail::fail(GENNMI_EINVAL, "empty matrix"); }
+    if(!rowLengthIn && num > rowStride) { return gennmi_detail::fail(GENNMI_EINVAL, "num exceeds rowStride"); }
+    if(rowStride > 0x7fffffffu) { return gennmi_detail::fail(GENNMI_EINVAL, "more than 2^31-1 row entries"); }
+    if(int rc = clearOverflow()) { return rc; }
+    const unsigned int blocks = (numPre + (BLOCK / WAVE) - 1) / (BLOCK / WAVE);
+    hipLaunchKernelGGL(fixedNumberPostKernel, dim3(blocks), dim3(BLOCK), 0, 0, numPre, numPost, rowStride, num, rowLengthIn,
+                       makeStream(seed, stream), rowLength, ind);
+    return finishConnectivity(overflowRows);
+}
+
+int gennmi_init_sparse_one_to_one(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t *rowLength, uint32_t *ind)
+{
+    if(numPre == 0 || numPost == 0 || rowStride == 0) { return gennmi_detail::fail(GENNMI_EINVAL, "empty matrix"); }
+    hipLaunchKernelGGL(oneToOneKernel, dim3((numPre + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, 0, numPre, numPost, rowStride, rowLength, ind);
+    HIP_TRY(hipGetLastError());
+    return GENNMI_OK;
+}
+
+}   // extern "C"

@@ -86,17 +86,85 @@ def init_toeplitz_connectivity(snippet, params=None):
     return _Init(snippet, params)
 
 
+# initSparseConnectivitySnippet.h:107-370; maximum row length as each snippet's SET_CALC_MAX_ROW_LENGTH_FUNC
+_SPARSE_SNIPPETS = ("OneToOne", "FixedProbability", "FixedProbabilityNoAutapse", "FixedNumberPostWithReplacement",
+                    "FixedNumberTotalWithReplacement")
+
+
+def init_sparse_connectivity(snippet, params=None):
+    """Connectivity built on the device at load() (pygenn.init_sparse_connectivity)."""
+    if snippet not in _SPARSE_SNIPPETS:
+        raise NotImplementedError(f"sparse connectivity snippet {snippet}")
+    return _Init(snippet, params)
+
+
+def binomial_inverse_cdf(cdf, n, p):
+    """GeNN::binomialInverseCDF (src/genn/genn/binomial.cc:37-110): the reference's unit test holds it to scipy's
+    binom.ppf (tests/unit/binomial.cc)."""
+    from scipy import stats
+    return int(stats.binom.ppf(cdf, n, p))
+
+
+def max_row_length(snippet, params, num_pre, num_post):
+    if snippet == "OneToOne":
+        return 1
+    if snippet in ("FixedProbability", "FixedProbabilityNoAutapse"):
+        # initSparseConnectivitySnippet.h:135-142
+        return max(1, binomial_inverse_cdf(0.9999 ** (1.0 / num_pre), num_post, float(params["prob"])))
+    if snippet == "FixedNumberPostWithReplacement":
+        return int(params["num"])
+    if snippet == "FixedNumberTotalWithReplacement":
+        # :372-381: rows are binomial(num, 1/numPre)
+        return max(1, binomial_inverse_cdf(0.9999 ** (1.0 / num_pre), int(params["num"]), 1.0 / num_pre))
+    raise NotImplementedError(snippet)
+
+
+class VarInit:
+    """Value snippet evaluated on the device at load() (pygenn.init_var; initVarSnippet.h:87-262)."""
+    _PARAMS = {"Constant": ("constant",), "Uniform": ("min", "max"), "Normal": ("mean", "sd"),
+               "NormalClipped": ("mean", "sd", "min", "max"), "NormalClippedDelay": ("mean", "sd", "min", "max"),
+               "Exponential": ("lambda",), "Gamma": ("a", "b"), "Binomial": ("n", "p")}
+
+    def __init__(self, snippet, params):
+        if snippet not in self._PARAMS:
+            raise NotImplementedError(f"variable initialisation snippet {snippet}")
+        missing = [k for k in self._PARAMS[snippet] if k not in params]
+        if missing:
+            raise ValueError(f"{snippet}: missing parameter(s) {missing}")
+        self.snippet = snippet
+        self.params = dict(params)
+
+    def values(self, dt):
+        v = [float(self.params[k]) for k in self._PARAMS[self.snippet]]
+        if self.snippet == "NormalClippedDelay":
+            v = [x / dt for x in v]          # the snippet's derived parameters (initVarSnippet.h:204-208)
+        return v + [0.0] * (4 - len(v))
+
+
+def init_var(snippet, params=None):
+    return VarInit(snippet, params or {})
+
+
 # --------------------------------------------------------------------------------------------
 # device arrays (the reference's Array objects, src/genn/backends/hip/backend.cc:61-236)
 # --------------------------------------------------------------------------------------------
 class Array:
-    def __init__(self, count, dtype, fill=None):
+    def __init__(self, count, dtype, fill=None, device_only=False):
+        """``device_only`` arrays (those a device kernel initialises) get their host copy on the first pull."""
         self.dtype = np.dtype(dtype)
         self.count = int(count)
-        self.view = np.zeros(self.count, dtype=self.dtype) if fill is None else np.full(self.count, fill, dtype=self.dtype)
         self._dev = C.c_void_p()
-        _abi.check(_abi.load().gennmi_malloc(C.byref(self._dev), self.view.nbytes))
-        self.push_to_device()
+        _abi.check(_abi.load().gennmi_malloc(C.byref(self._dev), self.count * self.dtype.itemsize))
+        self._view = None
+        if not device_only:
+            self._view = np.zeros(self.count, dtype=self.dtype) if fill is None else np.full(self.count, fill, dtype=self.dtype)
+            self.push_to_device()
+
+    @property
+    def view(self):
+        if self._view is None:
+            self._view = np.zeros(self.count, dtype=self.dtype)
+        return self._view
 
     @property
     def ptr(self):
@@ -114,6 +182,12 @@ class Array:
         if self.view.nbytes:
             _abi.check(_abi.load().gennmi_memcpy_from_device(self.view.ctypes.data_as(C.c_void_p), self._dev, self.view.nbytes))
         return self.view
+
+    def init_on_device(self, init, seed, stream, dt):
+        """Fill from a value snippet (gennmi_init_var); the host copy is not touched."""
+        params = (C.c_double * 4)(*init.values(dt))
+        _abi.check(_abi.load().gennmi_init_var(self._dev, _abi.ELEMENT_TYPES[self.dtype.name], self.count,
+                                               _abi.INIT_SNIPPETS[init.snippet], C.byref(params), seed, stream))
 
     def copy_on_device(self, src):
         """Device-to-device copy of another fp32 Array of the same length (host views are left alone)."""
@@ -234,6 +308,18 @@ class SynapseGroup:
         out[pre, within] = np.asarray(values)[order]
         self.var_host[name] = out
 
+    def pull_connectivity_from_device(self):
+        """Host copies of rowLength / ind (needed after on-device connectivity initialisation)."""
+        self.row_length_host = self.vars["rowLength"].pull_from_device().copy()
+        self.ind_host = self.vars["ind"].pull_from_device().reshape(self.src.num_neurons, self.row_stride)
+
+    def get_sparse_pre_inds(self):
+        return np.repeat(np.arange(self.src.num_neurons, dtype=np.uint32), self.row_length_host)
+
+    def get_sparse_post_inds(self):
+        mask = np.arange(self.row_stride)[None, :] < self.row_length_host[:, None]
+        return self.ind_host[mask]
+
     @property
     def num_synapses(self):
         return int(self.row_length_host.sum())
@@ -264,6 +350,8 @@ class GeNNModel:
         self._device = device
         self._arrays = []
         self.num_recording_timesteps = None
+        self.seed = 0                       # seeds every on-device initialisation snippet (ModelSpec::setSeed)
+        self._init_streams = 0              # one generator stream per array initialised on the device, in creation order
 
     # ------------------------------------------------------------------ description
     def add_neuron_population(self, pop_name, num_neurons, neuron, params=None, vars=None):
@@ -336,10 +424,19 @@ class GeNNModel:
     def _den_delay(s):
         return s.max_dendritic_delay_timesteps if s.wu.snippet == "StaticPulseDendriticDelay" else 0
 
-    def _alloc(self, count, dtype, fill=None):
-        a = Array(count, dtype, fill)
+    def _alloc(self, count, dtype, fill=None, device_only=False):
+        a = Array(count, dtype, fill, device_only)
         self._arrays.append(a)
         return a
+
+    def _alloc_device_init(self, count, dtype, init):
+        a = self._alloc(count, dtype, device_only=True)
+        a.init_on_device(init, self.seed, self._next_stream(), self.dt)
+        return a
+
+    def _next_stream(self):
+        self._init_streams += 1
+        return self._init_streams
 
     # ------------------------------------------------------------------ load = allocate + push merged groups
     def load(self, num_recording_timesteps=None):
@@ -370,6 +467,9 @@ class GeNNModel:
             else:
                 names = ("V", "RefracTime") if n.neuron == "LIF" else ("V", "U")
                 for v in names:
+                    if isinstance(n.var_init[v], VarInit):
+                        n.vars[v] = self._alloc_device_init(B * N, np.float32, n.var_init[v])
+                        continue
                     a = self._alloc(B * N, np.float32)
                     init = np.asarray(n.var_init[v], dtype=np.float32)
                     a.view[:] = np.broadcast_to(init, (B, N)).reshape(-1) if init.ndim < 2 else init.reshape(-1)
@@ -407,17 +507,23 @@ class GeNNModel:
         # ---- synapse-group arrays (runtime.cc:330-402)
         for s in self.synapse_populations.values():
             if s.matrix_type == "SPARSE":
-                if s.ind_host is None:
-                    raise RuntimeError(f"{s.name}: sparse connectivity has not been set")
                 n_pre = s.src.num_neurons
-                for name, host, dtype in (("rowLength", s.row_length_host, np.uint32), ("ind", s.ind_host, np.uint32)):
-                    a = self._alloc(host.size, dtype)
-                    a.view[:] = host.reshape(-1)
-                    a.push_to_device()
-                    s.vars[name] = a
+                if s.ind_host is None and s.conn is not None:
+                    self._init_connectivity_on_device(s)
+                elif s.ind_host is None:
+                    raise RuntimeError(f"{s.name}: sparse connectivity has not been set")
+                else:
+                    for name, host, dtype in (("rowLength", s.row_length_host, np.uint32), ("ind", s.ind_host, np.uint32)):
+                        a = self._alloc(host.size, dtype)
+                        a.view[:] = host.reshape(-1)
+                        a.push_to_device()
+                        s.vars[name] = a
                 names = ["g"] + (["d"] if s.wu.snippet == "StaticPulseDendriticDelay" else [])
                 for name in names:
                     dtype = np.uint8 if name == "d" else np.float32
+                    if name not in s.var_host and isinstance(s.wu.vars[name], VarInit):
+                        s.vars[name] = self._alloc_device_init(n_pre * s.row_stride, dtype, s.wu.vars[name])
+                        continue
                     a = self._alloc(n_pre * s.row_stride, dtype)
                     if name in s.var_host:
                         a.view[:] = np.asarray(s.var_host[name], dtype=dtype).reshape(-1)
@@ -439,6 +545,34 @@ class GeNNModel:
             _abi.check(lib.gennmi_runner_set_timing(self._runner, 1))
         self._loaded = True
         self.timestep = 0
+
+    def _init_connectivity_on_device(self, s):
+        """Built-in connectivity snippets on the device (the reference's initializeSparse path for GPU backends)."""
+        lib = _abi.load()
+        n_pre, n_post = s.src.num_neurons, s.trg.num_neurons
+        snippet, params = s.conn.snippet, s.conn.params
+        s.row_stride = max_row_length(snippet, params, n_pre, n_post)
+        s.vars["rowLength"] = self._alloc(n_pre, np.uint32, device_only=True)
+        s.vars["ind"] = self._alloc(n_pre * s.row_stride, np.uint32, device_only=True)
+        row_length, ind = s.vars["rowLength"].ptr, s.vars["ind"].ptr
+        stream = self._next_stream()
+        if snippet == "OneToOne":
+            _abi.check(lib.gennmi_init_sparse_one_to_one(n_pre, n_post, s.row_stride, row_length, ind))
+        elif snippet in ("FixedProbability", "FixedProbabilityNoAutapse"):
+            _abi.check(lib.gennmi_init_sparse_fixed_probability(n_pre, n_post, s.row_stride, float(params["prob"]),
+                                                                int(snippet.endswith("NoAutapse")), self.seed, stream, row_length, ind, None))
+        elif snippet == "FixedNumberPostWithReplacement":
+            _abi.check(lib.gennmi_init_sparse_fixed_number_post(n_pre, n_post, s.row_stride, int(params["num"]), None,
+                                                                self.seed, stream, row_length, ind, None))
+        else:
+            # FixedNumberTotalWithReplacement: the row lengths are one multinomial draw, made on the host as the
+            # snippet's host init code does (initSparseConnectivitySnippet.h:312-358), then handed to the device
+            rng = np.random.Generator(np.random.Philox(key=[self.seed, stream]))
+            lengths = rng.multinomial(int(params["num"]), np.full(n_pre, 1.0 / n_pre)).astype(np.uint32)
+            s.vars["rowLength"].view[:] = lengths
+            s.vars["rowLength"].push_to_device()
+            _abi.check(lib.gennmi_init_sparse_fixed_number_post(n_pre, n_post, s.row_stride, 0, row_length,
+                                                                self.seed, stream, row_length, ind, None))
 
     def _initialize_sparse(self):
         """initializeSparse(): column views for projections with postsynaptic-spike code."""

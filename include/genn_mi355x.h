@@ -197,6 +197,43 @@ int gennmi_runner_finalise(gennmi_runner *runner);
  * the order-nondeterministic atomic build of backendSIMT.cc:1977-1991. */
 int gennmi_build_remap(uint32_t numSrcNeurons, uint32_t numTrgNeurons, uint32_t rowStride, uint32_t colStride,
                        const uint32_t *rowLength, const uint32_t *ind, uint32_t *colLength, uint32_t *remap);
+/* ---------------------------------------------------------------------------------------------
+ * On-device initialisation: what the reference's GPU backends run in initializeKernel /
+ * initializeSparseKernel (src/genn/genn/code_generator/backendSIMT.cc:1482-1779) for its built-in snippets.
+ * Every draw is Philox4x32-10 of (seed, stream, element or row, draw number), so results do not depend on
+ * the launch geometry; like the reference's GPU backends (hiprand Philox, src/genn/backends/hip/backend.cc:32-50)
+ * the values differ from the CPU backend's std::mt19937 draws and agree with them in distribution only
+ * (the reference tests that much: tests/features/test_connect_init.py, test_rng.py).  All launches go to the
+ * null stream; the connectivity calls return after the kernel has finished.
+ * ------------------------------------------------------------------------------------------- */
+/* value snippets, include/genn/genn/initVarSnippet.h: Constant :87-95 {constant}; Uniform :120-130 {min, max};
+ * Normal :140-148 {mean, sd}; NormalClipped :161-175 {mean, sd, min, max}; NormalClippedDelay :190-209 {mean, sd, min, max
+ * already divided by dt, as the snippet's derived parameters}; Exponential :218-226 {lambda}; Gamma :236-244 {a, b};
+ * Binomial :254-262 {n, p} */
+enum { GENNMI_INIT_CONSTANT = 0, GENNMI_INIT_UNIFORM = 1, GENNMI_INIT_NORMAL = 2, GENNMI_INIT_NORMAL_CLIPPED = 3,
+       GENNMI_INIT_NORMAL_CLIPPED_DELAY = 4, GENNMI_INIT_EXPONENTIAL = 5, GENNMI_INIT_GAMMA = 6, GENNMI_INIT_BINOMIAL = 7 };
+enum { GENNMI_TYPE_F32 = 0, GENNMI_TYPE_U32 = 1, GENNMI_TYPE_I32 = 2, GENNMI_TYPE_U16 = 3, GENNMI_TYPE_U8 = 4 };
+/* genVariableInit / genSparseSynapseVariableRowInit (backendBase.h:246-251): fills `count` elements of a 16-byte aligned
+ * device array; values are computed in fp32 and converted to the element type.  Per-synapse variables of a SPARSE
+ * matrix are filled over the whole numPre*rowStride range, padding included (padding is never read). */
+int gennmi_init_var(void *dev, uint32_t elementType, size_t count, uint32_t snippet, const double params[4], uint64_t seed, uint32_t stream);
+/* FixedProbability (initSparseConnectivitySnippet.h:170-187) and FixedProbabilityNoAutapse (:208-230): rows ascending.
+ * Rows that draw more than rowStride entries are truncated, counted in *overflowRows (may be NULL) and make the call
+ * return GENNMI_EINVAL; the reference sizes rowStride so that this has probability 1e-4 per matrix (:135-142). */
+int gennmi_init_sparse_fixed_probability(uint32_t numPre, uint32_t numPost, uint32_t rowStride, double prob, int noAutapse,
+                                         uint64_t seed, uint32_t stream, uint32_t *rowLength, uint32_t *ind, uint32_t *overflowRows);
+/* FixedNumberPostWithReplacement (:242-276): `num` ascending targets per row.  With rowLengthIn != NULL (device array of
+ * numPre counts) row r draws rowLengthIn[r] targets instead: FixedNumberTotalWithReplacement (:292-370), whose row lengths
+ * the reference too draws on the host (its host init code) and hands to the device.  rowLengthIn may alias rowLength. */
+int gennmi_init_sparse_fixed_number_post(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t num, const uint32_t *rowLengthIn,
+                                         uint64_t seed, uint32_t stream, uint32_t *rowLength, uint32_t *ind, uint32_t *overflowRows);
+/* OneToOne (:107-118) */
+int gennmi_init_sparse_one_to_one(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t *rowLength, uint32_t *ind);
+/* The generator itself, for known-answer tests: one Philox4x32-10 block on the host, and the raw words of a stream
+ * on the device (word i = output i%4 of counter (i/4, 0, 0, stream) under key = seed). */
+int gennmi_philox4x32(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
+int gennmi_init_random_words(uint32_t *dev, size_t count, uint64_t seed, uint32_t stream);
+
 /* Longest column of a SPARSE matrix (what SynapseGroup::getMaxSourceConnections must cover). */
 int gennmi_max_col_length(uint32_t numSrcNeurons, uint32_t numTrgNeurons, uint32_t rowStride,
                           const uint32_t *rowLength, const uint32_t *ind, uint32_t *maxColLength);

@@ -117,3 +117,28 @@ def test_bench_refuses_more_than_one_gpu():
     import sys
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+
+
+def test_philox_known_answers():
+    """The generator under the on-device initialisation snippets, through the library's host entry point and the numpy
+    restatement the GPU tests compare device output with: both must give the published known-answer vectors."""
+    import ctypes as C
+    from philox_ref import KNOWN_ANSWERS, philox4x32
+    lib = _abi.load()
+    for counter, key, want in KNOWN_ANSWERS:
+        out = (C.c_uint32 * 4)()
+        assert lib.gennmi_philox4x32(C.byref((C.c_uint32 * 4)(*counter)), C.byref((C.c_uint32 * 2)(*key)), C.byref(out)) == 0
+        assert tuple(out) == want
+        assert tuple(int(w) for w in philox4x32(*counter, *key)) == want
+
+
+def test_max_row_length_follows_the_snippets():
+    """Row strides of the built-in connectivity snippets against the known answers of the reference's unit test for
+    binomialInverseCDF (tests/unit/binomial.cc:15-35: square matrices of 1, 1000 and 10^6 neurons at three probabilities)."""
+    from genn_amd.genn_model import max_row_length
+    table = {0.02: (1, 47, 20897), 0.1: (1, 153, 101914), 1.0: (1, 1000, 1000000)}
+    for prob, want in table.items():
+        for size, stride in zip((1, 1000, 1000000), want):
+            assert max_row_length("FixedProbability", {"prob": prob}, size, size) == stride
+    assert max_row_length("FixedNumberPostWithReplacement", {"num": 37}, 100, 100) == 37
+    assert max_row_length("OneToOne", {}, 100, 100) == 1
