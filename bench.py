@@ -65,6 +65,53 @@ def build_net(name, steps):
     raise SystemExit(f"unknown workload {name}")
 
 
+def bench_init(args):
+    """--workload init_izhikevich: on-device initialisation at the size of the 10^6-neuron configuration — 10^6 rows of
+    1000 ascending targets (FixedNumberPostWithReplacement) and 10^9 uniform weights.  A step builds both arrays once
+    (8 GB written); connectivity and weights are timed separately with the host clock around synchronous calls."""
+    import ctypes as C
+    import numpy as np
+    from genn_amd import _abi
+    from genn_amd.genn_model import Array
+    lib = _abi.load()
+    _abi.check(lib.gennmi_init(0))
+    num, fan_out = 1_000_000, 1000
+    row_length, ind, g = Array(num, np.uint32, device_only=True), Array(num * fan_out, np.uint32, device_only=True), Array(num * fan_out, np.float32, device_only=True)
+    params = (C.c_double * 4)(0.0, 0.5, 0.0, 0.0)
+    steps = min(args.steps, 20)
+    warmup = min(args.warmup, 2)
+    t_conn = t_var = 0.0
+    for it in range(warmup + steps):
+        t0 = time.perf_counter()
+        _abi.check(lib.gennmi_init_sparse_fixed_number_post(num, num, fan_out, fan_out, None, 1234, 1 + it, row_length.ptr, ind.ptr, None))
+        _abi.check(lib.gennmi_synchronize())
+        t1 = time.perf_counter()
+        _abi.check(lib.gennmi_init_var(g.ptr, _abi.ELEMENT_TYPES["float32"], num * fan_out, _abi.INIT_SNIPPETS["Uniform"], C.byref(params), 1234, 1000 + it))
+        _abi.check(lib.gennmi_synchronize())
+        t2 = time.perf_counter()
+        if it >= warmup:
+            t_conn += t1 - t0
+            t_var += t2 - t1
+    # spot check of the last build: a block of rows is ascending and in range
+    sample = np.empty(4096 * fan_out, dtype=np.uint32)
+    _abi.check(lib.gennmi_memcpy_from_device(sample.ctypes.data_as(C.c_void_p), ind.ptr, sample.nbytes))
+    rows = sample.reshape(4096, fan_out).astype(np.int64)
+    assert np.all(np.diff(rows, axis=1) >= 0) and rows.max() < num
+    synapses = num * fan_out
+    per_step = (t_conn + t_var) / steps
+    out = {"metric": "synapses_initialised_per_s", "value": round(synapses / per_step, 1), "unit": "synapses/s", "n_gpus": 1,
+           "steps": steps, "warmup": warmup, "ms_per_step": round(per_step * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "u32+f32", "data": "synthetic",
+           "config": {"workload": "on-device initialisation, 10^6 x 1000 FixedNumberPostWithReplacement + Uniform weights", "synapses": synapses},
+           "connectivity_ms": round(t_conn / steps * 1e3, 3), "weights_ms": round(t_var / steps * 1e3, 3),
+           "roofline": {"bound": "hbm", "kernel": "fixedNumberPostKernel (4 B written per synapse)", "achieved": round(4.0 * synapses / (t_conn / steps) / 1e9, 1),
+                        "peak": 8000.0, "unit": "GB/s", "frac": round(4.0 * synapses / (t_conn / steps) / 8e12, 4), "traffic": None,
+                        "weights_kernel": {"kernel": "initVarKernel<float>", "achieved": round(4.0 * synapses / (t_var / steps) / 1e9, 1),
+                                           "frac": round(4.0 * synapses / (t_var / steps) / 8e12, 4)}},
+           "cpu_baseline": None}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -84,6 +131,9 @@ def main():
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
                          "(the hot path is single-GPU; see DESIGN.md for how it would shard)")
+
+    if args.workload == "init_izhikevich":
+        return bench_init(args)
 
     import numpy as np
     from genn_amd.genn_model import model_from_net

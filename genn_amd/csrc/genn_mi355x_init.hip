@@ -292,7 +292,7 @@ void fixedProbabilityKernel(uint32_t numPre, uint32_t numPost, uint32_t rowStrid
 // FixedNumberPostWithReplacement / FixedNumberTotalWithReplacement (initSparseConnectivitySnippet.h:242-276, 292-370): one row
 // per wave64.  The snippet's loop `x += (1 - x) * (1 - pow(u, 1/c))` for c = n..1 draws the n order statistics of n uniforms in
 // ascending order.  The same joint law is S_k / S_{n+1} with S the prefix sums of n+1 unit exponentials, which a wave computes
-// 64 draws at a time with a scan: first the total, then — regenerating the same draws — the normalised prefix sums.
+// 256 draws at a time with a scan: first the total, then — regenerating the same draws — the normalised prefix sums.
 __global__ __launch_bounds__(BLOCK)
 void fixedNumberPostKernel(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t num, const uint32_t *rowLengthIn, Stream s,
                            uint32_t *rowLength, uint32_t *ind)
@@ -305,22 +305,39 @@ void fixedNumberPostKernel(uint32_t numPre, uint32_t numPost, uint32_t rowStride
         if(lane == 0) { atomicAdd(&g_rowOverflow, 1u); }
         n = rowStride;
     }
-    double total = 0.0;
+    // draws 0..n: spacing k ends at target k; spacing n is the gap between the largest target and 1.  A lane takes the four
+    // draws of one generator call, so a wave covers 256 draws per round and stores 1 KiB of the row at a time.
+    uint32_t *rowInd = ind + (size_t)row * rowStride;
+    const bool vectorStores = ((rowStride & 3u) == 0) && (((uintptr_t)ind & 15u) == 0);
+    double scale = 0.0;
     for(int pass = 0; pass < 2; pass++) {
         double carry = 0.0;
-        // draws 0..n: spacing k ends at target k; spacing n is the gap between the largest target and 1
-        for(uint32_t base = 0; base <= n; base += WAVE) {
-            const uint32_t k = base + lane;
+        for(uint32_t base = 0; base <= n; base += 4 * WAVE) {
+            const uint32_t k = base + 4 * lane;
             const Words r = s.at(((unsigned long long)row << 32) | (k >> 2), 0);
-            const double spacing = (k <= n) ? (double)-logf(uniformOpen(r.w[k & 3u])) : 0.0;
-            const double inclusive = carry + waveInclusiveScan(spacing, lane);
-            if(pass == 1 && k < n) {
-                const uint32_t post = (uint32_t)((inclusive / total) * (double)numPost);
-                ind[(size_t)row * rowStride + k] = min(post, numPost - 1);
+            double prefix[4];
+            double sum = 0.0;
+            #pragma unroll
+            for(int i = 0; i < 4; i++) {
+                sum += (k + i <= n) ? (double)-logf(uniformOpen(r.w[i])) : 0.0;
+                prefix[i] = sum;
             }
-            carry = __shfl(inclusive, WAVE - 1, WAVE);
+            const double inclusive = waveInclusiveScan(sum, lane);
+            const double before = carry + (inclusive - sum);
+            if(pass == 1 && k < n) {
+                uint32_t post[4];
+                #pragma unroll
+                for(int i = 0; i < 4; i++) { post[i] = min((uint32_t)((before + prefix[i]) * scale), numPost - 1); }
+                if(vectorStores && k + 3 < n) {
+                    *reinterpret_cast<uint4*>(rowInd + k) = make_uint4(post[0], post[1], post[2], post[3]);
+                }
+                else {
+                    for(int i = 0; i < 4 && k + i < n; i++) { rowInd[k + i] = post[i]; }
+                }
+            }
+            carry += __shfl(inclusive, WAVE - 1, WAVE);
         }
-        total = carry;
+        scale = (double)numPost / carry;
     }
     if(lane == 0) { rowLength[row] = n; }
 }
