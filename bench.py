@@ -187,7 +187,18 @@ def main():
         model.set_timing(False)
         bpe = bytes_per_event or max(BYTES_PER_EVENT[k] for k in kinds)
         neuron_bytes = sum(p.n * (0 if p.model == "ssa" else 32) for p in net.pops)     # 32 B per LIF/Izhikevich update (state + one PSM)
-        if info["single_launch_step"]:
+        if info["resident_plan"]:
+            # the timed region is ONE launch of residentKernel that performs all K steps (preceded by an 8-byte-per-tile
+            # memset), so HIP events around the region give that launch's duration; a launch moves K steps' worth of
+            # algorithmic bytes
+            achieved = (events * bpe + neuron_bytes * args.steps) / region_s / 1e9
+            roofline = {"bound": "hbm", "kernel": "residentKernel (all timesteps of the timed region in one launch)",
+                        "achieved": round(achieved, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6),
+                        "traffic": None, "bytes_per_event": bpe, "events_per_launch": events, "steps_per_launch": args.steps,
+                        "neuron_bytes_per_launch": neuron_bytes * args.steps, "avg_launch_us": round(region_s * 1e6, 3),
+                        "us_per_step": round(region_s / args.steps * 1e6, 3),
+                        "avg_launch_us_one_step_per_launch": round(st["step_seconds"] / max(1, st["step_launches"]) * 1e6, 3) if st["step_launches"] else None}
+        elif info["single_launch_step"]:
             # the timed region consists of this kernel only (one launch per step, back to back inside the replayed
             # graphs, plus one 1-thread node per 100 steps), so HIP events around the region give its average duration
             avg_s = region_s / args.steps
@@ -216,7 +227,7 @@ def main():
         for _ in range(5):
             b.copy_on_device(a)
         a.free(); b.free()
-    if roofline is not None and args.workload in MEASURED_TRAFFIC_BYTES:
+    if roofline is not None and args.workload in MEASURED_TRAFFIC_BYTES and not (info["resident_plan"] and args.workload == "potjans"):
         roofline["traffic"] = MEASURED_TRAFFIC_BYTES[args.workload]["bytes_per_launch"]
         roofline["traffic_source"] = MEASURED_TRAFFIC_BYTES[args.workload]["source"]
     model.unload()
@@ -285,7 +296,8 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall / args.steps * 1e3, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": label, "neurons": num_neurons, "synapses": num_synapses, "dt_ms": net.dt, "seed": net.seed,
-                   "stepping": "hipGraph replay, 100 steps per graph, " + ("1 launch per step" if info["single_launch_step"] else "2-3 launches per step")},
+                   "stepping": ("resident plan: one launch for all timed steps, state in registers/LDS" if info["resident_plan"] else
+                                "hipGraph replay, 100 steps per graph, " + ("1 launch per step" if info["single_launch_step"] else "2-3 launches per step"))},
         "gsop_per_s": round(events / wall / 1e9, 4),
         "neuron_updates_per_s": round(num_neurons * batch * args.steps / wall, 1),
         "wall_s_per_sim_s": round(wall / sim_s, 4),

@@ -26,7 +26,11 @@
 
 #include "genn_mi355x.h"
 
-namespace gennmi_detail { int fail(int code, const std::string &msg); }
+namespace gennmi_detail
+{
+int fail(int code, const std::string &msg);
+void noteDeviceWrite(const void *dev, size_t bytes);     // lets runners that hold copies of weights refresh them
+}
 
 namespace
 {
@@ -422,6 +426,7 @@ int gennmi_init_var(void *dev, uint32_t elementType, size_t count, uint32_t snip
         return gennmi_detail::fail(GENNMI_EINVAL, "binomial needs 0 <= n < 2^32 and 0 <= p <= 1");
     }
     const Stream s = makeStream(seed, stream);
+    gennmi_detail::noteDeviceWrite(dev, count * 4);
     switch(elementType) {
     case GENNMI_TYPE_F32: return launchInitVar<float>(dev, count, v, s);
     case GENNMI_TYPE_U32: return launchInitVar<uint32_t>(dev, count, v, s);

@@ -190,14 +190,18 @@ def test_toeplitz_batches_are_independent():
     model.unload()
 
 
-def test_graph_replay_matches_stepping():
-    """run() replays captured HIP graphs; every replay must leave the state eager stepping leaves.
-    Replays are interleaved with eager steps and synchronisations."""
+@pytest.mark.parametrize("resident", ["1", "0"])
+def test_graph_replay_matches_stepping(resident, monkeypatch):
+    """run() either keeps the network resident on the chip for the whole chunk (one launch) or, with that plan switched
+    off, replays captured HIP graphs; either way every chunk must leave the state eager stepping leaves.
+    Chunks are interleaved with eager steps and synchronisations."""
+    monkeypatch.setenv("GENNMI_RESIDENT", resident)
     net = configs.vogels_abbott(n=2000, steps=730, p=0.04)
     eager = model_from_net(net)
     eager.load(num_recording_timesteps=net.steps)
     graph = model_from_net(net)
     graph.load(num_recording_timesteps=net.steps)
+    assert graph.runner_info()["resident_plan"] == (resident == "1")
     for chunk in (250, 3, 200, 77, 200):           # 200/250 -> graph replays (+ remainder), 3/77 -> single steps
         graph.run(chunk)
         graph.synchronize()
@@ -221,15 +225,18 @@ def test_graph_replay_matches_stepping():
     eager.unload()
 
 
-def test_graph_replay_single_launch_step():
-    """Graph replay of the one-launch-per-step plan (dendritic-delay network) against eager stepping and the oracle:
-    rasters identical, membrane potentials within tolerance (weights differ, so atomic order may differ)."""
+@pytest.mark.parametrize("resident", ["1", "0"])
+def test_graph_replay_single_launch_step(resident, monkeypatch):
+    """Chunks of steps of a dendritic-delay network — resident plan, or graph replay of the one-launch-per-step plan —
+    against eager stepping (one launch per step, which hands front-slot synapses over one step early) and the oracle:
+    rasters identical, membrane potentials within tolerance (weights differ, so the order of additions may differ)."""
+    monkeypatch.setenv("GENNMI_RESIDENT", resident)
     net = configs.potjans(neuron_scale=0.04, connectivity_scale=1.0, steps=450)
     eager = model_from_net(net)
     eager.load(num_recording_timesteps=net.steps)
     graph = model_from_net(net)
     graph.load(num_recording_timesteps=net.steps)
-    assert graph.runner_info()["single_launch_step"]
+    assert graph.runner_info()["single_launch_step"] and graph.runner_info()["resident_plan"] == (resident == "1")
     oracle = OracleNet(net, num_recording_timesteps=net.steps)
     for chunk in (200, 50, 200):
         graph.run(chunk)
