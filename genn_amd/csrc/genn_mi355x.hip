@@ -1054,6 +1054,7 @@ constexpr uint32_t RES_FRONT_MAX = 4;        // front-slot synapses held inline 
 constexpr uint32_t RES_SEG_OVERFLOW = 1u << 24, RES_SEG_NO_DELAY = 1u << 25;
 constexpr uint32_t RES_PAIR_GROUP = 16;      // pairs a wavefront expands at a time
 constexpr int RES_SEQ_SHIFT = 41;            // word = seq << 41 | count << 32 | id
+constexpr uint32_t RES_REPLICAS = 8;         // copies of the word array, one per XCD, so that polling spreads over memory channels
 
 struct ResProj
 {
@@ -1136,7 +1137,7 @@ __global__ __launch_bounds__(BLOCK)
 void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const NeuronGroupDev * __restrict__ groups,
                     const uint8_t * __restrict__ tileGroup, unsigned long long *tags, uint32_t *side,
                     unsigned long long timestep0, unsigned long long epoch0, unsigned long long numRecordingTimesteps, uint32_t numSteps,
-                    float dt, uint32_t zeroDelaySplit, uint32_t *errorFlag, unsigned long long *eventCounter)
+                    float dt, uint32_t zeroDelaySplit, uint32_t *errorFlag, unsigned long long *eventCounter, uint32_t replicaStride)
 {
     extern __shared__ float lds[];                       // inSyn rows and ring slices of this tile
     __shared__ unsigned long long shTag[RES_MAX_TILES];
@@ -1151,6 +1152,10 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     __shared__ uint32_t shWave[BLOCK / WAVE];
     __shared__ uint32_t shScalar[4];
 
+    // every tile publishes its word into all copies of the word array and reads the copy of its own XCD
+    uint32_t xcc = 0;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    const unsigned long long *myTags = tags + (size_t)(xcc & (RES_REPLICAS - 1)) * replicaStride;
     const ResTile &T = tiles[blockIdx.x];
     const NeuronGroupDev &G = groups[T.group];
     const gennmi_neuron_update_group_t &g = G.g;
@@ -1225,9 +1230,9 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         }
         __syncthreads();
-        if(tid == 0) {
+        if(tid < RES_REPLICAS) {
             const unsigned long long word = ((unsigned long long)seq << RES_SEQ_SHIFT) | ((unsigned long long)count << 32) | (count == 1 ? shOwn[0] : 0u);
-            __hip_atomic_store(&tags[(size_t)parity * numTiles + blockIdx.x], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&tags[(size_t)tid * replicaStride + (size_t)parity * numTiles + blockIdx.x], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     };
 
@@ -1258,7 +1263,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             #pragma unroll
             for(uint32_t q = 0; q < WATCH; q++) {
                 if(pending & (1u << q)) {
-                    word[q] = __hip_atomic_load(&tags[(size_t)parity * numTiles + tid + q * BLOCK], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    word[q] = __hip_atomic_load(&myTags[(size_t)parity * numTiles + tid + q * BLOCK], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
             #pragma unroll
@@ -1582,7 +1587,7 @@ struct gennmi_runner
     bool resident = false;
     ResTile *dResTiles = nullptr; NeuronGroupDev *dResGroups = nullptr; uint8_t *dResTileGroup = nullptr;
     unsigned long long *dResTags = nullptr; uint32_t *dResSide = nullptr;
-    uint32_t resTiles = 0; size_t resLdsBytes = 0;
+    uint32_t resTiles = 0, resReplicaStride = 0; size_t resLdsBytes = 0;
     std::vector<u32x4*> resSegs;        // segment table of each presynaptic group, in push order
     std::vector<uint32_t> resSegTiles;  // tiles of its target population
     bool resStale = false;              // connectivity or weights were written since the tables were built
@@ -2009,7 +2014,8 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
     HIP_TRY(upload((void**)&r->dResTiles, tiles.data(), tiles.size() * sizeof(ResTile)));
     HIP_TRY(upload((void**)&r->dResGroups, groups.data(), groups.size() * sizeof(NeuronGroupDev)));
     HIP_TRY(upload((void**)&r->dResTileGroup, tileGroup.data(), tileGroup.size()));
-    HIP_TRY(hipMalloc(&r->dResTags, 2 * tiles.size() * sizeof(unsigned long long)));
+    r->resReplicaStride = (uint32_t)((2 * tiles.size() + 511) / 512 * 512);          // in words: copies start 4 KiB-aligned
+    HIP_TRY(hipMalloc(&r->dResTags, (size_t)RES_REPLICAS * r->resReplicaStride * sizeof(unsigned long long)));
     r->owned.push_back(r->dResTags);
     HIP_TRY(hipMalloc(&r->dResSide, 2 * tiles.size() * RES_T * sizeof(uint32_t)));
     r->owned.push_back(r->dResSide);
@@ -2042,10 +2048,10 @@ static int launchResident(gennmi_runner *r, unsigned long long timestep, unsigne
     }
     for(unsigned long long done = 0; done < numSteps; ) {
         const uint32_t chunk = (uint32_t)std::min(MAX_STEPS, numSteps - done);
-        HIP_TRY(hipMemsetAsync(r->dResTags, 0, 2 * (size_t)r->resTiles * sizeof(unsigned long long), r->stream));
+        HIP_TRY(hipMemsetAsync(r->dResTags, 0, (size_t)RES_REPLICAS * r->resReplicaStride * sizeof(unsigned long long), r->stream));
         residentKernel<<<dim3(r->resTiles), dim3(BLOCK), r->resLdsBytes, r->stream>>>(
             r->dResTiles, r->resTiles, r->dResGroups, r->dResTileGroup, r->dResTags, r->dResSide, timestep + done, r->epoch, numRecordingTimesteps,
-            chunk, r->dt, r->fusedStep ? 1u : 0u, r->dError, r->dEvents);
+            chunk, r->dt, r->fusedStep ? 1u : 0u, r->dError, r->dEvents, r->resReplicaStride);
         HIP_TRY(hipGetLastError());
         done += chunk;
         r->epoch += chunk;
