@@ -10,6 +10,9 @@
 //                             compaction + recording (backendSIMT.cc:405-662, 1931-1975); also does the
 //                             work of neuronSpikeQueueUpdateKernel (:373-403) and
 //                             synapseDendriticDelayUpdateKernel (:664-692), which need no launch here.
+//   residentKernel            many timesteps of a network that fits the chip in ONE launch: neuron state in registers,
+//                             inSyn and dendritic-delay rings in LDS, spikes exchanged between work-groups through
+//                             one word per tile (no counterpart in the reference)
 //   remap*Kernel              deterministic colLength/remap build (replaces backendSIMT.cc:1977-1991)
 //
 // Arithmetic contract: fp32, one rounding per operation, same operation order as the code the

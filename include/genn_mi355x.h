@@ -249,9 +249,10 @@ int gennmi_update_neurons(gennmi_runner *runner, float t, uint32_t recordingTime
 int gennmi_step(gennmi_runner *runner, float t, uint32_t recordingTimestep);
 /* stepTime(timestep, numRecordingTimesteps)  generateRunner.cc:270-299 */
 int gennmi_step_time(gennmi_runner *runner, unsigned long long timestep, unsigned long long numRecordingTimesteps);
-/* numSteps consecutive stepTime calls starting at `timestep`, replayed from a captured HIP
- * graph so that no per-kernel launch latency is paid (no counterpart in the reference, which
- * launches 4-7 kernels per step from the host). */
+/* numSteps consecutive stepTime calls starting at `timestep` without a host round trip per step (no counterpart
+ * in the reference, which launches 4-7 kernels per step from the host): one launch that keeps the network resident
+ * on the chip where the runner's plan allows it (see gennmi_runner_get_info), else replays of a captured HIP graph
+ * of 100 steps.  Either way the arrays are left as numSteps calls of gennmi_step_time would leave them. */
 int gennmi_run_steps(gennmi_runner *runner, unsigned long long timestep, unsigned long long numSteps,
                      unsigned long long numRecordingTimesteps);
 /* stepTimeFinalise: blocks until everything queued has finished and reports device-side
@@ -273,7 +274,9 @@ int gennmi_runner_kernel_stats(gennmi_runner *runner, double stats[8]);
  * backendCUDAHIP.cc:36-76 for a caller-chosen region, e.g. a whole gennmi_run_steps replay. */
 int gennmi_runner_stream_mark(gennmi_runner *runner, int which);
 int gennmi_runner_stream_elapsed(gennmi_runner *runner, double *seconds);
-/* Launch plan chosen by gennmi_runner_finalise: info[0] = 1 if a whole timestep is one launch (all projections go
+/* Launch plan chosen by gennmi_runner_finalise: bit 1 of info[0] is set if gennmi_run_steps keeps the network resident on
+ * the chip (many steps per launch: batch 1, static SPARSE projections with ascending rows between LIF / Izhikevich
+ * populations, all tiles of 256 neurons resident at once; GENNMI_RESIDENT=0 disables it); bit 0 if a whole timestep is one launch (all projections go
  * through a dendritic-delay ring; synapses with d % D == 0 are then delivered by the spiking neuron one launch
  * earlier, into the slot read in the next step — the visible difference is the content of that one ring slot
  * between steps; GENNMI_FUSED_STEP=0 in the environment keeps the reference's placement), info[1..3] = blocks of
