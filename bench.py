@@ -30,6 +30,7 @@ BYTES_PER_EVENT = {"static": 16, "static_delay": 17, "stdp_trace": 28, "conv2d":
 # not of this one; workloads without an entry report null.
 MEASURED_TRAFFIC_BYTES = {
     "potjans": {"bytes_per_launch": 5.76e6, "source": "profiles/stepFusedKernel_potjans_full.md (median launch: 3172.6 KiB read + 2447.8 KiB written)"},
+    "potjans_resident": {"bytes_per_step": 3.90e6, "source": "profiles/residentKernel_potjans_full.md (10,000-step launch: 38.05 GB read + 0.97 GB written)"},
     "izh": {"bytes_per_launch": 2.43e8, "source": "profiles/presynapticTileKernel_izhikevich_1M_full.md (average launch of presynapticTileKernel + presynapticUpdateKernel over the first 500 steps)"},
 }
 
@@ -227,7 +228,10 @@ def main():
         for _ in range(5):
             b.copy_on_device(a)
         a.free(); b.free()
-    if roofline is not None and args.workload in MEASURED_TRAFFIC_BYTES and not (info["resident_plan"] and args.workload == "potjans"):
+    if roofline is not None and info["resident_plan"] and args.workload == "potjans":
+        roofline["traffic"] = MEASURED_TRAFFIC_BYTES["potjans_resident"]["bytes_per_step"] * args.steps
+        roofline["traffic_source"] = MEASURED_TRAFFIC_BYTES["potjans_resident"]["source"]
+    elif roofline is not None and args.workload in MEASURED_TRAFFIC_BYTES:
         roofline["traffic"] = MEASURED_TRAFFIC_BYTES[args.workload]["bytes_per_launch"]
         roofline["traffic_source"] = MEASURED_TRAFFIC_BYTES[args.workload]["source"]
     model.unload()

@@ -1056,7 +1056,8 @@ constexpr uint32_t RES_PAIR_CAP = 1024;      // (spike, projection) pairs staged
 constexpr uint32_t RES_FRONT_MAX = 4;        // front-slot synapses held inline in a segment entry
 constexpr uint32_t RES_SEG_OVERFLOW = 1u << 24, RES_SEG_NO_DELAY = 1u << 25;
 constexpr uint32_t RES_PAIR_GROUP = 16;      // pairs a wavefront expands at a time
-constexpr int RES_SEQ_SHIFT = 41;            // word = seq << 41 | count << 32 | id
+constexpr int RES_SEQ_SHIFT = 41;            // word = seq << 41 | count << 32 | up to four tile-local neuron indices, 8 bits each
+constexpr uint32_t RES_WORD_IDS = 4;         // spikes of a tile and step that travel inside its word (more: side buffer)
 constexpr uint32_t RES_REPLICAS = 8;         // copies of the word array, one per XCD, so that polling spreads over memory channels
 
 struct ResProj
@@ -1225,7 +1226,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
 
     auto publish = [&](uint32_t seq, uint32_t count) {
         const uint32_t parity = seq & 1u;
-        if(count >= 2) {
+        if(count > RES_WORD_IDS) {
             for(uint32_t r = tid; r < count; r += BLOCK) {
                 __hip_atomic_store(&side[((size_t)parity * numTiles + blockIdx.x) * RES_T + r], shOwn[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
@@ -1234,17 +1235,20 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         }
         __syncthreads();
         if(tid < RES_REPLICAS) {
-            const unsigned long long word = ((unsigned long long)seq << RES_SEQ_SHIFT) | ((unsigned long long)count << 32) | (count == 1 ? shOwn[0] : 0u);
+            uint32_t locals = 0;
+            for(uint32_t e = 0; e < min(count, RES_WORD_IDS); e++) { locals |= (shOwn[e] - T.first) << (8 * e); }
+            const unsigned long long word = ((unsigned long long)seq << RES_SEQ_SHIFT) | ((unsigned long long)count << 32) | locals;
             __hip_atomic_store(&tags[(size_t)tid * replicaStride + (size_t)parity * numTiles + blockIdx.x], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     };
 
     // source tiles this thread watches (tile tid, tid + 256, ...) and how many of this tile's projections each feeds
     constexpr uint32_t WATCH = RES_MAX_TILES / BLOCK;
-    uint32_t watchProj0[WATCH], watchNumProj[WATCH];
+    uint32_t watchProj0[WATCH], watchNumProj[WATCH], watchFirst[WATCH];
     #pragma unroll
     for(uint32_t q = 0; q < WATCH; q++) {
         const uint32_t k = tid + q * BLOCK;
+        watchFirst[q] = (k < numTiles) ? tiles[k].first : 0u;
         const uint32_t s = (k < numTiles) ? shTileGroup[k] : 0u;
         watchProj0[q] = shProjStart[s];
         watchNumProj[q] = (k < numTiles) ? shProjStart[s + 1] - shProjStart[s] : 0u;
@@ -1292,8 +1296,8 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             uint32_t pos = atomicAdd(&shScalar[0], c * np);
             if(pos + c * np > RES_PAIR_CAP) { continue; }
             for(uint32_t e = 0; e < c; e++) {
-                const uint32_t id = (c == 1) ? (uint32_t)word[q]
-                                             : __hip_atomic_load(&side[((size_t)parity * numTiles + tid + q * BLOCK) * RES_T + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const uint32_t id = (c <= RES_WORD_IDS) ? watchFirst[q] + (((uint32_t)word[q] >> (8 * e)) & 0xFFu)
+                                                        : __hip_atomic_load(&side[((size_t)parity * numTiles + tid + q * BLOCK) * RES_T + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 for(uint32_t j = 0; j < np; j++) { shPair[pos++] = make_uint2(id, shProjIdx[watchProj0[q] + j]); }
             }
         }
@@ -1404,8 +1408,8 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
                 if(c == 0 || np == 0) { continue; }
                 if(pos + c * np <= chunk0 || pos >= chunk0 + RES_PAIR_CAP) { pos += c * np; continue; }
                 for(uint32_t q = 0; q < c; q++) {
-                    const uint32_t id = (c == 1) ? (uint32_t)tag
-                                                 : __hip_atomic_load(&side[((size_t)parity * numTiles + k) * RES_T + q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const uint32_t id = (c <= RES_WORD_IDS) ? tiles[k].first + (((uint32_t)tag >> (8 * q)) & 0xFFu)
+                                                            : __hip_atomic_load(&side[((size_t)parity * numTiles + k) * RES_T + q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     for(uint32_t j = 0; j < np; j++, pos++) {
                         if(pos >= chunk0 && pos < chunk0 + RES_PAIR_CAP) { shPair[pos - chunk0] = make_uint2(id, shProjIdx[p0 + j]); }
                     }
