@@ -38,7 +38,7 @@ constexpr int BLOCK = 256;                  // 4 wave64 per work-group
 constexpr int WAVE = 64;
 constexpr int CONV_TILE_SPIKES = 2048;      // spikes staged in LDS at a time by the Conv2D tile kernel
 constexpr int CONV_TILE_THREADS = 512;      // work-group size of the Conv2D tile kernel (8 wave64 share one LDS tile)
-constexpr uint32_t SPIN_LIMIT = 1u << 22;   // bounded wait of the spike-offset look-back
+constexpr uint32_t SPIN_LIMIT = 1u << 22;   // default bound of every wait for another work-group (polls)
 constexpr uint32_t REMAP_SORT_MAX = 16384;  // longest column the LDS sort handles (64 KiB)
 
 thread_local std::string g_lastError;
@@ -56,6 +56,10 @@ int fail(int code, const std::string &msg)
             return fail(GENNMI_EHIP, std::string(#expr) + ": " + hipGetErrorString(e_));           \
         }                                                                                          \
     } while(0)
+
+// Polls a work-group spends waiting for another one before it raises the error flag and leaves.  Set from
+// GENNMI_SPIN_LIMIT when a runner is finalised; tests of the failure path set it to 0 so that the first missed poll expires.
+__constant__ uint32_t c_spinLimit = SPIN_LIMIT;
 
 // ------------------------------------------------------------------------------------------------
 // device-side tables
@@ -859,7 +863,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
             while(true) {
                 const unsigned long long a = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if((uint32_t)(a >> 32) == tag) { return (uint32_t)a; }
-                if(++spins > SPIN_LIMIT) { ok = false; return 0u; }
+                if(++spins > c_spinLimit) { ok = false; return 0u; }
                 __builtin_amdgcn_s_sleep(1);
             }
         };
@@ -1045,7 +1049,7 @@ uint32_t pow2Ceil(uint32_t v) { uint32_t p = 1; while(p < v) { p *= 2; } return 
 // tile can run at most one step ahead of the slowest one, because it needs every tile's word of step s before
 // it can publish its own word of step s+1.
 //
-// The wait for the other tiles' words is bounded (SPIN_LIMIT polls) and also watches the error flag, so a launch
+// The wait for the other tiles' words is bounded (c_spinLimit polls) and also watches the error flag, so a launch
 // whose work-groups are not all resident ends with an error instead of hanging.
 // ------------------------------------------------------------------------------------------------
 constexpr uint32_t RES_T = BLOCK;            // neurons per tile = threads per work-group
@@ -1279,7 +1283,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             }
             if(!pending) { break; }
             ++spins;
-            if(spins > SPIN_LIMIT || ((spins & 255u) == 0 && __hip_atomic_load(errorFlag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) { ok = false; break; }
+            if(spins > c_spinLimit || ((spins & 255u) == 0 && __hip_atomic_load(errorFlag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) { ok = false; break; }
             __builtin_amdgcn_s_sleep(1);
         }
         #pragma unroll
@@ -2331,6 +2335,14 @@ int gennmi_runner_finalise(gennmi_runner *r)
     HIP_TRY(hipMalloc(&r->dAgg, aggCount * sizeof(unsigned long long)));
     HIP_TRY(hipMemset(r->dAgg, 0, aggCount * sizeof(unsigned long long)));
     { const int rc = setupResident(r, numCU); if(rc) { return rc; } }
+    if(const char *envSpin = getenv("GENNMI_SPIN_LIMIT")) {
+        const uint32_t limit = (uint32_t)std::max(0ll, atoll(envSpin));
+        HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(c_spinLimit), &limit, sizeof(limit)));
+    }
+    else {
+        const uint32_t limit = SPIN_LIMIT;
+        HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(c_spinLimit), &limit, sizeof(limit)));
+    }
     HIP_TRY(hipDeviceSynchronize());
     r->finalised = true;
     return GENNMI_OK;
@@ -2533,7 +2545,7 @@ int gennmi_runner_synchronize(gennmi_runner *r)
     HIP_TRY(hipStreamSynchronize(r->stream));
     uint32_t err = 0;
     HIP_TRY(hipMemcpy(&err, r->dError, sizeof(err), hipMemcpyDeviceToHost));
-    if(err) { return fail(GENNMI_EDEVICE, "neuronUpdateKernel: bounded wait for spike offsets expired"); }
+    if(err) { return fail(GENNMI_EDEVICE, "a kernel's bounded wait for other work-groups expired (spike offsets or spike exchange); state is undefined"); }
     return GENNMI_OK;
 }
 

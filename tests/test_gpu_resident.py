@@ -152,3 +152,29 @@ def test_plan_can_be_switched_off(monkeypatch):
 
     model, oracle, spikes = _run_chunks(net, (120,), check, resident=False)
     model.unload()
+
+
+@pytest.mark.parametrize("resident", ["1", "0"])
+def test_expired_wait_is_reported_not_hung(resident, monkeypatch):
+    """Failure path, forced from the host: with a wait bound of zero polls the first word (resident plan) or spike
+    count (per-step plans) that has not arrived when it is first looked at makes the work-group raise the device error
+    flag and leave; every kernel still ends normally, and the next synchronisation reports the error."""
+    from genn_amd import configs
+    from genn_amd._abi import GennmiError
+    monkeypatch.setenv("GENNMI_SPIN_LIMIT", "0")
+    monkeypatch.setenv("GENNMI_RESIDENT", resident)
+    net = configs.potjans(neuron_scale=0.05, connectivity_scale=1.0, steps=2000)
+    model = model_from_net(net)
+    model.load(num_recording_timesteps=2000)
+    assert model.runner_info()["resident_plan"] == (resident == "1")
+    model.run(2000)
+    with pytest.raises(GennmiError, match="bounded wait"):
+        model.synchronize()
+    model.unload()
+    # the bound is per process: restore the default for whatever runs next
+    monkeypatch.delenv("GENNMI_SPIN_LIMIT")
+    model = model_from_net(net)
+    model.load(num_recording_timesteps=100)
+    model.run(100)
+    model.synchronize()
+    model.unload()
