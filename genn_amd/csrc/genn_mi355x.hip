@@ -1151,6 +1151,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     __shared__ unsigned long long shTag[RES_MAX_TILES];
     __shared__ uint2 shPair[RES_PAIR_CAP];               // (presynaptic neuron, projection)
     __shared__ uint2 shSeg[RES_PAIR_CAP];                // (first idSyn, length | flags) of each staged pair
+    __shared__ uint32_t shFlagged;                       // staged pairs whose row has to be walked before the update
     __shared__ ResProj shProj[RES_MAX_PROJ];
     __shared__ uint32_t shProjPtr[RES_MAX_PROJ];         // this step's front slot of each projection's ring
     __shared__ uint32_t shProjStart[RES_MAX_GROUPS + 1]; // projections of this tile by source group
@@ -1228,6 +1229,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     __syncthreads();
     uint32_t ownCount = shScalar[1];
 
+    // (callers synchronise the work-group after filling shOwn)
     auto publish = [&](uint32_t seq, uint32_t count) {
         const uint32_t parity = seq & 1u;
         if(count > RES_WORD_IDS) {
@@ -1236,8 +1238,8 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             }
             // the ids must have reached memory before the word that announces them
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            __syncthreads();
         }
-        __syncthreads();
         if(tid < RES_REPLICAS) {
             uint32_t locals = 0;
             for(uint32_t e = 0; e < min(count, RES_WORD_IDS); e++) { locals |= (shOwn[e] - T.first) << (8 * e); }
@@ -1261,14 +1263,14 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     // Waits for every tile's word of sequence number seq (false when the bounded wait expired somewhere) and stages the
     // (spike, projection) pairs that concern this tile in shPair; shScalar[0] receives their number, which may exceed
     // RES_PAIR_CAP (then only the claims that fitted were written and the caller takes the chunked path).
-    auto poll = [&](uint32_t seq) -> bool {
+    auto poll = [&](uint32_t seq, unsigned long long epoch) -> bool {
         const uint32_t parity = seq & 1u;
         bool ok = true;
         unsigned long long word[WATCH];
         uint32_t pending = 0;
         #pragma unroll
         for(uint32_t q = 0; q < WATCH; q++) { word[q] = 0; if(tid + q * BLOCK < numTiles) { pending |= 1u << q; } }
-        if(tid == 0) { shScalar[0] = 0; }
+        if(tid == 0) { shScalar[0] = 0; shFlagged = 0; }
         uint32_t spins = 0;
         while(pending) {
             #pragma unroll
@@ -1293,6 +1295,8 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             if(tid == 0) { atomicOr(errorFlag, 1u); }
             return false;
         }
+        // front slot of every projection's ring in the step this exchange feeds
+        if(tid < T.numProj) { shProjPtr[tid] = shProj[tid].D ? modStep(epoch + 1, shProj[tid].D) : 0u; }
         #pragma unroll
         for(uint32_t q = 0; q < WATCH; q++) {
             const uint32_t c = (uint32_t)(word[q] >> 32) & 0x1FFu, np = watchNumProj[q];
@@ -1322,6 +1326,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             GLOBAL_AS const u32x4 *entry = asGlobal(P.seg) + 2 * ((size_t)pr.x * T.tilesInGroup + T.tileInGroup);
             const u32x4 lo4 = entry[0], hi4 = entry[1];
             shSeg[q] = make_uint2(lo4.x, lo4.y);
+            if(lo4.y & (RES_SEG_OVERFLOW | RES_SEG_NO_DELAY)) { atomicAdd(&shFlagged, 1u); }
             if(count) { events += lo4.y & 0xFFFFu; }
             if(skipInline) { continue; }
             const uint32_t numFront = (lo4.y >> 16) & 0xFFu;
@@ -1432,9 +1437,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     // (inline in the segment entries; row walks only for segments that say so).  `convention` is PASS_ALL normally,
     // PASS_LATER when a previous launch has already delivered the due synapses of these spikes, PASS_DUE when only those
     // are wanted.  Returns the number of staged pairs whose remaining synapses deliverLater() has to add, or 0.
-    auto deliverDue = [&](uint32_t seq, unsigned long long epoch, uint32_t convention) -> uint32_t {
-        if(tid < T.numProj) { shProjPtr[tid] = shProj[tid].D ? modStep(epoch + 1, shProj[tid].D) : 0u; }
-        __syncthreads();
+    auto deliverDue = [&](uint32_t seq, uint32_t convention) -> uint32_t {
         const uint32_t total = shScalar[0];
         if(total > RES_PAIR_CAP) {
             processChunked(seq, total, convention, convention != PASS_DUE);
@@ -1442,7 +1445,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         }
         readSegments(total, convention == PASS_LATER, convention != PASS_DUE);
         __syncthreads();
-        if(convention != PASS_LATER) { process(total, PASS_DUE, true); }
+        if(convention != PASS_LATER && shFlagged) { process(total, PASS_DUE, true); }
         return (convention == PASS_DUE) ? 0u : total;
     };
     // the rest of those pairs' synapses: none of them is read before the next step
@@ -1456,8 +1459,8 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     uint32_t k = 0;
     for(; k < numSteps; k++) {
         const unsigned long long epoch = epoch0 + k;
-        if(!poll(k + 1)) { ok = false; break; }
-        const uint32_t later = deliverDue(k + 1, epoch, (zeroDelaySplit && k == 0) ? PASS_LATER : PASS_ALL);
+        if(!poll(k + 1, epoch)) { ok = false; break; }
+        const uint32_t later = deliverDue(k + 1, (zeroDelaySplit && k == 0) ? PASS_LATER : PASS_ALL);
         __syncthreads();
 
         // neuron update: same operations in the same order as neuronBody
@@ -1537,10 +1540,10 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
 
     // ---- after the last step: everybody's last spikes give the position of this tile's spikes in the population's
     // queue; a runner that delivers front-slot synapses one step early (single-launch plan) wants them in the ring now
-    if(ok && !poll(numSteps + 1)) { ok = false; }
-    if(!ok) { return; }
     const unsigned long long epochEnd = epoch0 + numSteps;       // completed steps
-    if(zeroDelaySplit) { deliverDue(numSteps + 1, epochEnd, PASS_DUE); }
+    if(ok && !poll(numSteps + 1, epochEnd)) { ok = false; }
+    if(!ok) { return; }
+    if(zeroDelaySplit) { deliverDue(numSteps + 1, PASS_DUE); }
     __syncthreads();
 
     if(mine) { asGlobal(g.var0)[i] = l0; asGlobal(g.var1)[i] = l1; }
