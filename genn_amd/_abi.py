@@ -13,8 +13,8 @@ MAX_EXTRA_SPK = 3
 NEURON_LIF, NEURON_IZHIKEVICH, NEURON_SPIKE_SOURCE_ARRAY = 0, 1, 2
 PSM_EXPCURR, PSM_DELTACURR = 0, 1
 CS_DC, CS_ARRAY = 0, 1
-WUM_STATIC_PULSE, WUM_STATIC_PULSE_DENDRITIC_DELAY, WUM_STDP_TRACE = 0, 1, 2
-MATRIX_SPARSE, MATRIX_TOEPLITZ_CONV2D = 0, 1
+WUM_STATIC_PULSE, WUM_STATIC_PULSE_DENDRITIC_DELAY, WUM_STDP_TRACE, WUM_STATIC_PULSE_CONSTANT_WEIGHT = 0, 1, 2, 3
+MATRIX_SPARSE, MATRIX_TOEPLITZ_CONV2D, MATRIX_DENSE, MATRIX_BITMASK = 0, 1, 2, 3
 SPAN_AUTO, SPAN_POST, SPAN_PRE = 0, 1, 2
 
 LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
@@ -57,7 +57,8 @@ class PresynapticUpdateGroup(C.Structure):
                 ("srcSpkCnt", p_u32), ("srcSpk", p_u32),
                 ("trgST", p_f32), ("postTrace", p_f32),
                 ("aMinus", C.c_float), ("wMin", C.c_float), ("wMax", C.c_float),
-                ("conv", C.c_int32 * 8)]
+                ("conv", C.c_int32 * 8),
+                ("gp", p_u32), ("constantWeight", C.c_float), ("pad2_", C.c_uint32)]
 
 
 class PostsynapticUpdateGroup(C.Structure):

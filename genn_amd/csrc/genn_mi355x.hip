@@ -363,6 +363,65 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
 }
 
 // ------------------------------------------------------------------------------------------------
+// DENSE and BITMASK projections (single_threaded_cpu/backend.cc:1985-2021 is the sequential definition).  One lane
+// per postsynaptic neuron walks the spike queue: weights of a spike's row are lane-consecutive (DENSE: g[idPre*numTrg
+// + idPost]) or one bit each (BITMASK, most significant bit first), so there is nothing to scatter and no atomic —
+// a lane that owns its outPost element alone continues the sum from the value that is there, in queue order, which is
+// the CPU backend's order bit for bit.  When several projections feed one outPost the lane's partial sum is added
+// with one (lane-consecutive) atomic instead.
+// ------------------------------------------------------------------------------------------------
+struct DenseGroupDev
+{
+    gennmi_presynaptic_update_group_t g;
+    uint32_t startBlock, numBlocks;
+    uint32_t exclusive;                 // no other projection adds to this outPost
+    uint32_t pad_;
+};
+
+__global__ __launch_bounds__(BLOCK)
+void presynapticDenseKernel(const DenseGroupDev * __restrict__ blocks, unsigned long long *eventCounter)
+{
+    const DenseGroupDev &G = blocks[blockIdx.x];
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const uint32_t j = (blockIdx.x - G.startBlock) * BLOCK + threadIdx.x;
+    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
+    if(numSpikes == 0) { return; }
+    GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
+    unsigned long long events = 0;
+    if(j < g.numTrgNeurons) {
+        float acc = G.exclusive ? outPost[j] : 0.0f;
+        if(g.matrix == GENNMI_MATRIX_DENSE) {
+            const bool constant = (g.wum == GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT);
+            GLOBAL_AS const float *weight = asGlobal(g.g);
+            // four rows in flight; the additions keep queue order
+            uint32_t s = 0;
+            for(; s + 4 <= numSpikes; s += 4) {
+                float w[4];
+                #pragma unroll
+                for(int u = 0; u < 4; u++) { w[u] = constant ? g.constantWeight : weight[(size_t)spk[s + u] * g.numTrgNeurons + j]; }
+                #pragma unroll
+                for(int u = 0; u < 4; u++) { acc += w[u]; }
+            }
+            for(; s < numSpikes; s++) { acc += constant ? g.constantWeight : weight[(size_t)spk[s] * g.numTrgNeurons + j]; }
+            if(j == 0) { events = (unsigned long long)numSpikes * g.numTrgNeurons; }
+        }
+        else {
+            GLOBAL_AS const uint32_t *gp = asGlobal(g.gp);
+            for(uint32_t s = 0; s < numSpikes; s++) {
+                const unsigned long long gid = (unsigned long long)spk[s] * g.rowStride + j;
+                if(gp[gid >> 5] & (0x80000000u >> (gid & 31))) { acc += g.constantWeight; events++; }
+            }
+        }
+        if(G.exclusive) { outPost[j] = acc; }
+        else if(acc != 0.0f) { atomicAddF32(&outPost[j], acc); }
+    }
+    for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
+    if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Tile kernel.  Scattered fp32 atomics cost one memory transaction each (≈20 G/s measured on this part,
 // whatever the array size), lane-consecutive ones ≈280 G/s.  When a step carries enough events
 // (numSpikes*rowStride >= numTrg), a block therefore owns a tile of postsynaptic neurons in LDS: it walks
@@ -1586,6 +1645,7 @@ struct gennmi_runner
     bool finalised = false;
     hipStream_t stream = nullptr;
     std::vector<NeuronGroupDev> neuron; std::vector<PreGroupDev> pre; std::vector<PostGroupDev> post;
+    std::vector<DenseGroupDev> dense; DenseGroupDev *dDense = nullptr; uint32_t denseBlocks = 0;
     NeuronGroupDev *dNeuron = nullptr; PreGroupDev *dPre = nullptr; PostGroupDev *dPost = nullptr;
     uint32_t neuronBlocks = 0, preBlocks = 0, postBlocks = 0;
     unsigned long long *dAgg = nullptr; uint32_t *dError = nullptr; unsigned long long *dEvents = nullptr;
@@ -1808,7 +1868,7 @@ int gennmi_runner_destroy(gennmi_runner *r)
     for(hipEvent_t e : r->marks) { if(e) { hipEventDestroy(e); } }
     for(void *q : r->owned) { hipFree(q); }
     hipFree(r->dTile); hipFree(r->dConvTile);
-    hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dAgg); hipFree(r->dError); hipFree(r->dEvents); hipFree(r->dState);
+    hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dDense); hipFree(r->dAgg); hipFree(r->dError); hipFree(r->dEvents); hipFree(r->dState);
     hipStreamDestroy(r->stream);
     delete r;
     return GENNMI_OK;
@@ -1853,8 +1913,29 @@ int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynap
 {
     if(!r || !g) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: null argument"); }
     if(r->finalised) { return fail(GENNMI_ESTATE, "push_presynaptic_update_group: runner already finalised"); }
-    if(!g->srcSpk || !g->srcSpkCnt || !g->outPost || !g->g) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: required array missing"); }
+    if(!g->srcSpk || !g->srcSpkCnt || !g->outPost) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: required array missing"); }
     if(g->numSrcNeurons == 0 || g->numTrgNeurons == 0) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: empty population"); }
+    if(g->matrix == GENNMI_MATRIX_DENSE || g->matrix == GENNMI_MATRIX_BITMASK) {
+        const bool constant = (g->wum == GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT);
+        if(g->matrix == GENNMI_MATRIX_DENSE) {
+            if(!constant && g->wum != GENNMI_WUM_STATIC_PULSE) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: DENSE supports StaticPulse and StaticPulseConstantWeight"); }
+            if(!constant && !g->g) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: dense weights missing"); }
+        }
+        else {
+            if(!constant) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: BITMASK needs StaticPulseConstantWeight"); }
+            if(!g->gp || g->rowStride < g->numTrgNeurons || (g->rowStride % 32) != 0) {
+                return fail(GENNMI_EINVAL, "push_presynaptic_update_group: bitmask words missing or row stride not numTrg padded to 32");
+            }
+        }
+        DenseGroupDev dd;
+        memset(&dd, 0, sizeof(dd));
+        dd.g = *g;
+        dd.g.maxDenDelay = 0;
+        if(idx) { *idx = (uint32_t)(r->pre.size() + r->dense.size()); }
+        r->dense.push_back(dd);
+        return GENNMI_OK;
+    }
+    if(!g->g) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: required array missing"); }
     PreGroupDev d;
     memset(&d, 0, sizeof(d));
     d.g = *g;
@@ -1914,7 +1995,7 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
 {
     const char *env = getenv("GENNMI_RESIDENT");
     if(env && atoi(env) == 0) { return GENNMI_OK; }
-    if(r->batch != 1 || !r->post.empty() || r->pre.empty() || r->neuron.size() > RES_MAX_GROUPS) { return GENNMI_OK; }
+    if(r->batch != 1 || !r->post.empty() || r->pre.empty() || !r->dense.empty() || r->neuron.size() > RES_MAX_GROUPS) { return GENNMI_OK; }
     for(const auto &n : r->neuron) {
         const auto &g = n.g;
         if((g.model != GENNMI_NEURON_LIF && g.model != GENNMI_NEURON_IZHIKEVICH) || g.preTrace || g.postTrace || g.sT) { return GENNMI_OK; }
@@ -2140,6 +2221,18 @@ int gennmi_runner_finalise(gennmi_runner *r)
     }
     r->postBlocks = block;
 
+    // DENSE / BITMASK projections: one lane per postsynaptic neuron; a group owns its outPost unless another dense or
+    // bitmask group adds to the same one (sparse groups have finished by the time this kernel starts)
+    block = 0;
+    for(auto &d : r->dense) {
+        d.startBlock = block;
+        d.numBlocks = (d.g.numTrgNeurons + BLOCK - 1) / BLOCK;
+        block += d.numBlocks;
+        d.exclusive = 1;
+        for(const auto &o : r->dense) { if(&o != &d && o.g.outPost == d.g.outPost) { d.exclusive = 0; } }
+    }
+    r->denseBlocks = block;
+
     // One descriptor copy per block, indexed by blockIdx.x: a block finds everything it needs with a
     // single round of scalar loads (the reference bisects a start-ID table and then loads the merged
     // struct, backendSIMT.h:244-323 — two to four dependent loads before any work starts).
@@ -2248,7 +2341,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
     // ---- single-launch step: possible when every projection is a SPARSE dendritic-delay one with ring depth >= 2
     // and nothing is plastic
     const char *envFused = getenv("GENNMI_FUSED_STEP");
-    bool eligible = !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty();
+    bool eligible = !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty() && r->dense.empty();
     for(const auto &p : r->pre) {
         eligible = eligible && p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY
                    && p.g.maxDenDelay >= 2;
@@ -2334,6 +2427,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
     HIP_TRY(uploadPerBlock(r->neuron, r->neuronBlocks, &r->dNeuron));
     HIP_TRY(uploadPerBlock(r->pre, r->preBlocks, &r->dPre));
     HIP_TRY(uploadPerBlock(r->post, r->postBlocks, &r->dPost));
+    HIP_TRY(uploadPerBlock(r->dense, r->denseBlocks, &r->dDense));
     const size_t aggCount = 2 * (size_t)r->neuronBlocks * r->batch;       // per-block counts, then per-group totals
     HIP_TRY(hipMalloc(&r->dAgg, aggCount * sizeof(unsigned long long)));
     HIP_TRY(hipMemset(r->dAgg, 0, aggCount * sizeof(unsigned long long)));
@@ -2390,8 +2484,13 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
         if(r->pending.size() >= 2048) { const int rc = drainTimers(r); if(rc) { return rc; } }
         const int rc = stamp(r, &e0); if(rc) { return rc; }
     }
-    if(!r->pre.empty()) {
-        presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dPre, a, r->dt, r->dEvents);
+    if(!r->pre.empty() || r->denseBlocks) {
+        if(r->preBlocks) {
+            presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dPre, a, r->dt, r->dEvents);
+        }
+        if(r->denseBlocks) {
+            presynapticDenseKernel<<<dim3(r->denseBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dDense, r->dEvents);
+        }
         if(r->tileBlocks) {
             presynapticTileKernel<<<dim3(r->tileBlocks, r->batch), dim3(r->tileThreads), r->tileFloats * sizeof(float), r->stream>>>(r->dTile, a, r->dt, r->dEvents);
         }

@@ -75,7 +75,7 @@ def init_postsynaptic(snippet, params=None, vars=None):
 
 
 def init_weight_update(snippet, params=None, vars=None, pre_vars=None, post_vars=None):
-    if snippet not in ("StaticPulse", "StaticPulseDendriticDelay", "STDPTrace"):
+    if snippet not in ("StaticPulse", "StaticPulseConstantWeight", "StaticPulseDendriticDelay", "STDPTrace"):
         raise NotImplementedError(f"weight update model {snippet}")
     return _Init(snippet, params, vars, pre_vars, post_vars)
 
@@ -272,12 +272,22 @@ class SynapseGroup:
         self.row_length_host = None
         self.ind_host = None
         self.var_host = {}
+        self.gp_host = None
         self.fused_ps_target = self
 
     # pygenn/genn_groups.py:434-470
     def set_sparse_connections(self, pre_indices, post_indices):
         pre = np.asarray(pre_indices, dtype=np.int64)
         post = np.asarray(post_indices, dtype=np.int64)
+        if self.matrix_type == "BITMASK":
+            # one bit per pair, gid = idPre*rowStride + idPost with the row stride padded to 32, most significant bit of a
+            # word first (single_threaded_cpu/backend.cc:1393-1404, 2003-2006)
+            stride = (self.trg.num_neurons + 31) // 32 * 32
+            bits = np.zeros(self.src.num_neurons * stride, dtype=np.uint8)
+            bits[pre * stride + post] = 1
+            self.gp_host = np.packbits(bits, bitorder="big").view(">u4").astype(np.uint32)
+            self.row_stride = stride
+            return
         order = np.lexsort((post, pre))
         pre, post = pre[order], post[order]
         n_pre = self.src.num_neurons
@@ -373,8 +383,12 @@ class GeNNModel:
 
     def add_synapse_population(self, pop_name, matrix_type, source, target, weight_update_init, postsynaptic_init,
                                connectivity_init=None):
-        if matrix_type not in ("SPARSE", "TOEPLITZ"):
+        if matrix_type not in ("SPARSE", "TOEPLITZ", "DENSE", "BITMASK"):
             raise NotImplementedError(f"matrix type {matrix_type}")
+        if matrix_type == "BITMASK" and weight_update_init.snippet != "StaticPulseConstantWeight":
+            raise ValueError("BITMASK connectivity has no per-synapse variables: use StaticPulseConstantWeight")
+        if matrix_type == "DENSE" and weight_update_init.snippet not in ("StaticPulse", "StaticPulseConstantWeight"):
+            raise NotImplementedError(f"DENSE connectivity with {weight_update_init.snippet}")
         if matrix_type == "TOEPLITZ" and (connectivity_init is None or connectivity_init.snippet != "Conv2D"):
             raise ValueError("TOEPLITZ connectivity needs init_toeplitz_connectivity('Conv2D', ...)")
         s = SynapseGroup(self, pop_name, matrix_type, source, target, weight_update_init, postsynaptic_init, connectivity_init)
@@ -518,7 +532,10 @@ class GeNNModel:
                         a.view[:] = host.reshape(-1)
                         a.push_to_device()
                         s.vars[name] = a
-                names = ["g"] + (["d"] if s.wu.snippet == "StaticPulseDendriticDelay" else [])
+                if s.wu.snippet == "StaticPulseConstantWeight":
+                    # the sparse kernels read a weight per synapse: the one weight is written out
+                    s.vars["g"] = self._alloc(n_pre * s.row_stride, np.float32, fill=np.float32(lit32(s.wu.params["g"])))
+                names = [] if s.wu.snippet == "StaticPulseConstantWeight" else ["g"] + (["d"] if s.wu.snippet == "StaticPulseDendriticDelay" else [])
                 for name in names:
                     dtype = np.uint8 if name == "d" else np.float32
                     if name not in s.var_host and isinstance(s.wu.vars[name], VarInit):
@@ -531,6 +548,25 @@ class GeNNModel:
                         a.view[:] = dtype(s.wu.vars[name])
                     a.push_to_device()
                     s.vars[name] = a
+            elif s.matrix_type == "DENSE":
+                if s.wu.snippet == "StaticPulse":
+                    count = s.src.num_neurons * s.trg.num_neurons
+                    init = s.var_host.get("g", s.wu.vars.get("g"))
+                    if isinstance(init, VarInit):
+                        s.vars["g"] = self._alloc_device_init(count, np.float32, init)
+                    else:
+                        a = self._alloc(count, np.float32)
+                        a.view[:] = np.broadcast_to(np.asarray(init, dtype=np.float32).reshape(-1), (count,)) if np.size(init) in (1, count) \
+                            else np.asarray(init, dtype=np.float32).reshape(-1)
+                        a.push_to_device()
+                        s.vars["g"] = a
+            elif s.matrix_type == "BITMASK":
+                if s.gp_host is None:
+                    raise RuntimeError(f"{s.name}: bitmask connectivity has not been set")
+                a = self._alloc(s.gp_host.size, np.uint32)
+                a.view[:] = s.gp_host
+                a.push_to_device()
+                s.vars["gp"] = a
             else:
                 kern = np.ascontiguousarray(s.var_host.get("g", s.wu.vars.get("g")), dtype=np.float32)
                 a = self._alloc(kern.size, np.float32)
@@ -689,19 +725,32 @@ class GeNNModel:
             stdp = members[0].wu.snippet == "STDPTrace"
             if stdp:
                 rounded = {q: _merge_round([s.wu.params[q] for s in members]) for q in ("aPlus", "aMinus", "wMin", "wMax")}
+            if members[0].wu.snippet == "StaticPulseConstantWeight":
+                consts = _merge_round([s.wu.params["g"] for s in members])
             for k, s in enumerate(members):
                 d = _abi.PresynapticUpdateGroup()
-                d.matrix = _abi.MATRIX_SPARSE if s.matrix_type == "SPARSE" else _abi.MATRIX_TOEPLITZ_CONV2D
+                d.matrix = {"SPARSE": _abi.MATRIX_SPARSE, "TOEPLITZ": _abi.MATRIX_TOEPLITZ_CONV2D, "DENSE": _abi.MATRIX_DENSE,
+                            "BITMASK": _abi.MATRIX_BITMASK}[s.matrix_type]
                 d.wum = {"StaticPulse": _abi.WUM_STATIC_PULSE, "StaticPulseDendriticDelay": _abi.WUM_STATIC_PULSE_DENDRITIC_DELAY,
-                         "STDPTrace": _abi.WUM_STDP_TRACE}[s.wu.snippet]
+                         "STDPTrace": _abi.WUM_STDP_TRACE, "StaticPulseConstantWeight": _abi.WUM_STATIC_PULSE_CONSTANT_WEIGHT}[s.wu.snippet]
+                if s.wu.snippet == "StaticPulseConstantWeight":
+                    d.constantWeight = consts[k]
+                    if s.matrix_type == "SPARSE":
+                        d.wum = _abi.WUM_STATIC_PULSE
                 d.span = {"POSTSYNAPTIC": _abi.SPAN_AUTO, "PRESYNAPTIC": _abi.SPAN_PRE, "WAVE": _abi.SPAN_POST}[s.parallelism_hint]
                 d.numThreadsPerSpike = s.num_threads_per_spike
                 d.numSrcNeurons, d.numTrgNeurons = s.src.num_neurons, s.trg.num_neurons
                 owner = s.fused_ps_target
                 d.outPost = owner.vars["outPost"].ptr
                 d.srcSpkCnt, d.srcSpk = s.src.vars["spkCnt"].ptr, s.src.vars["spk"].ptr
-                d.g = s.vars["g"].ptr
-                if s.matrix_type == "SPARSE":
+                if "g" in s.vars:
+                    d.g = s.vars["g"].ptr
+                if s.matrix_type == "BITMASK":
+                    d.rowStride = s.row_stride
+                    d.gp = s.vars["gp"].ptr
+                if s.matrix_type in ("DENSE", "BITMASK"):
+                    pass
+                elif s.matrix_type == "SPARSE":
                     d.rowStride = s.row_stride
                     d.rowLength, d.ind = s.vars["rowLength"].ptr, s.vars["ind"].ptr
                     D = self._den_delay(s)
@@ -840,12 +889,23 @@ def model_from_net(net, batch_size=1, record=True, span=None, device=0):
             wu = init_weight_update("StaticPulse", {}, {"g": 0.0})
         elif s.wum == "static_delay":
             wu = init_weight_update("StaticPulseDendriticDelay", {}, {"g": 0.0, "d": 0})
+        elif s.wum == "static_const":
+            wu = init_weight_update("StaticPulseConstantWeight", {"g": s.wum_params["g"]})
         else:
             wu = init_weight_update("STDPTrace", s.wum_params, {"g": 0.0}, {"preTrace": 0.0}, {"postTrace": 0.0})
-        if s.matrix == "sparse":
+        if s.matrix == "dense":
+            sg = m.add_synapse_population(s.name, "DENSE", pops[s.src], pops[s.trg], wu, ps)
+            if s.g is not None:
+                sg.set_var_ragged("g", s.g)
+        elif s.matrix == "bitmask":
+            sg = m.add_synapse_population(s.name, "BITMASK", pops[s.src], pops[s.trg], wu, ps)
+            sg.gp_host = np.ascontiguousarray(s.gp, dtype=np.uint32)
+            sg.row_stride = s.row_stride
+        elif s.matrix == "sparse":
             sg = m.add_synapse_population(s.name, "SPARSE", pops[s.src], pops[s.trg], wu, ps)
             sg.set_ragged(s.row_length, s.ind)
-            sg.set_var_ragged("g", s.g)
+            if s.wum != "static_const":
+                sg.set_var_ragged("g", s.g)
             if s.d is not None:
                 sg.set_var_ragged("d", s.d)
             if s.max_den_delay:

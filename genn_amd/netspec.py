@@ -45,15 +45,16 @@ class Syn:
     name: str
     src: str
     trg: str
-    matrix: str = "sparse"          # "sparse" | "conv2d"
-    wum: str = "static"             # "static" | "static_delay" | "stdp_trace"
+    matrix: str = "sparse"          # "sparse" | "conv2d" | "dense" | "bitmask"
+    wum: str = "static"             # "static" | "static_delay" | "stdp_trace" | "static_const" (one weight, wum_params["g"])
     wum_params: Dict[str, float] = field(default_factory=dict)
     psm: str = "expcurr"            # "expcurr" | "deltacurr"
     tau: float = 5.0
     row_stride: int = 0
     row_length: Optional[np.ndarray] = None   # uint32 [numPre]
     ind: Optional[np.ndarray] = None          # uint32 [numPre, rowStride]
-    g: Optional[np.ndarray] = None            # fp32 [numPre, rowStride] or kernel [kh,kw,ic,oc]
+    g: Optional[np.ndarray] = None            # fp32 [numPre, rowStride], dense [numPre, numPost], or kernel [kh,kw,ic,oc]
+    gp: Optional[np.ndarray] = None           # bitmask: uint32 words, bit idPre*rowStride + idPost, most significant bit first
     d: Optional[np.ndarray] = None            # uint8 [numPre, rowStride]
     max_den_delay: int = 0
     hint_pre: bool = False
@@ -63,6 +64,10 @@ class Syn:
 
     @property
     def num_synapses(self):
+        if self.matrix == "bitmask":
+            return int(np.unpackbits(np.ascontiguousarray(self.gp).view(np.uint8)).sum())
+        if self.matrix == "dense":
+            return int(self.g.size) if self.g is not None else 0
         return int(self.row_length.sum()) if self.row_length is not None else 0
 
 

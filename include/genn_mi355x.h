@@ -44,9 +44,14 @@ enum { GENNMI_PSM_EXPCURR = 0, GENNMI_PSM_DELTACURR = 1 };
 /* current sources: include/genn/genn/currentSourceModels.h:70-77 (DC); ARRAY injects noise[step*numNeurons+id] */
 enum { GENNMI_CS_DC = 0, GENNMI_CS_ARRAY = 1 };
 /* weight update models: include/genn/genn/weightUpdateModels.h:236-244, :279-287; trace STDP pygenn/genn_model.py:1448-1476 */
-enum { GENNMI_WUM_STATIC_PULSE = 0, GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY = 1, GENNMI_WUM_STDP_TRACE = 2 };
+enum { GENNMI_WUM_STATIC_PULSE = 0, GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY = 1, GENNMI_WUM_STDP_TRACE = 2,
+       GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT = 3 /* weightUpdateModels.h:202-213: one weight for the whole projection */ };
 /* connectivity: ragged SPARSE (runtime.cc:360-402) or TOEPLITZ Conv2D (initToeplitzConnectivitySnippet.h:105-150) */
-enum { GENNMI_MATRIX_SPARSE = 0, GENNMI_MATRIX_TOEPLITZ_CONV2D = 1 };
+enum { GENNMI_MATRIX_SPARSE = 0, GENNMI_MATRIX_TOEPLITZ_CONV2D = 1,
+       /* DENSE: g[numSrc*numTrg], idSyn = idPre*numTrg + idPost; BITMASK: one bit per pair, most significant bit first,
+        * gid = idPre*rowStride + idPost with rowStride = numTrg padded to 32 (single_threaded_cpu/backend.cc:1393-1404,
+        * 1985-2021; runtime.cc:340-357) */
+       GENNMI_MATRIX_DENSE = 2, GENNMI_MATRIX_BITMASK = 3 };
 /* presynaptic strategies: presynapticUpdateStrategySIMT.cc:57-162 (PreSpan), :167-389 (PostSpan) */
 enum { GENNMI_SPAN_AUTO = 0, GENNMI_SPAN_POST = 1, GENNMI_SPAN_PRE = 2 };
 
@@ -154,6 +159,9 @@ typedef struct gennmi_presynaptic_update_group_t { /* MergedPresynapticUpdateGro
     const float *postTrace;
     float aMinus, wMin, wMax;
     int32_t conv[8];                      /* conv_kh, conv_kw, conv_ih, conv_iw, conv_ic, conv_oh, conv_ow, conv_oc */
+    const uint32_t *gp;                   /* BITMASK: [ceil(numSrcNeurons*rowStride / 32)] connectivity words */
+    float constantWeight;                 /* GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT: the parameter g (DENSE and BITMASK) */
+    uint32_t pad2_;
 } gennmi_presynaptic_update_group_t;
 
 typedef struct gennmi_postsynaptic_update_group_t { /* MergedPostsynapticUpdateGroup<i> */

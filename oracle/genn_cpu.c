@@ -12,6 +12,8 @@
  *                                                    src/genn/genn/code_generator/synapseUpdateGroupMerged.cc:480-483
  *                        sparse presynaptic loop     backend.cc:1884-1929, synapseUpdateGroupMerged.cc:49-217, 245-251
  *                        Toeplitz presynaptic loop   backend.cc:1788-1883, include/genn/genn/initToeplitzConnectivitySnippet.h:116-137
+ *                        dense / bitmask loop        backend.cc:1985-2021 (bit gid = idPre*rowStride + idPost, most significant bit
+ *                                                    first; row stride = numPost padded to 32, backend.cc:1393-1404)
  *                        postsynaptic (learnPost)    backend.cc:2029-2095
  *   gc_update_neurons    spike queue reset           src/genn/genn/code_generator/neuronUpdateGroupMerged.cc:947-975
  *                        neuron loop + op order      backend.cc:187-398, neuronUpdateGroupMerged.cc:552-773 (PSM :66-137, CS :20-55,
@@ -25,7 +27,9 @@
  *
  * Parity pins: golden vectors written by the reference's own CPU backend (tests/golden/, made
  * by tests/golden/make_golden.py through oracle/ref_driver.cc), the closed-form decode tables
- * of the reference's tests/features/test_event_propagation.py, and its Toeplitz fixtures.
+ * of the reference's tests/features/test_event_propagation.py, and its Toeplitz fixtures.  The dense / bitmask loop has no
+ * golden vector from the reference's backend: it is pinned by that decode table (test_event_propagation.py:237-260 holds
+ * for its DENSE and BITMASK projections too) and by brute force against a matrix-vector product (tests/test_oracle_golden.py).
  */
 #include <math.h>
 #include <stdint.h>
@@ -35,7 +39,7 @@
 enum { GC_LIF = 0, GC_IZH = 1, GC_SSA = 2 };
 enum { GC_EXPCURR = 0, GC_DELTACURR = 1 };
 enum { GC_STATIC = 0, GC_STATIC_DELAY = 1, GC_STDP_TRACE = 2 };
-enum { GC_SPARSE = 0, GC_CONV2D = 1 };
+enum { GC_SPARSE = 0, GC_CONV2D = 1, GC_DENSE = 2, GC_BITMASK = 3 };
 enum { GC_CS_DC = 0, GC_CS_NOISE = 1 };
 
 #define GC_MAX_CHILD 16
@@ -80,6 +84,8 @@ typedef struct {
     uint32_t *colLength, *remap;
     float aPlus, aMinus, wMin, wMax;
     int conv[8]; int conv_bh, conv_bw;
+    const uint32_t *gp;     /* BITMASK connectivity words */
+    float constantWeight;   /* StaticPulseConstantWeight (weightUpdateModels.h:202-213): used when g is NULL */
     uint64_t events;        /* synaptic events processed so far (bookkeeping, not in the reference) */
 } gc_syn;
 
@@ -209,6 +215,23 @@ int gc_add_syn_conv2d(gc_net *net, int src, int trg, int psm, const int *conv, c
     return net->numSyns - 1;
 }
 
+/* DENSE (g != NULL: individual weights [numPre*numPost]; else the constant) or BITMASK (gp, rowStride = numPost padded to 32) */
+int gc_add_syn_dense(gc_net *net, int src, int trg, int psm, const float *g, float constantWeight)
+{
+    gc_syn *s = gc_new_syn(net);
+    s->matrix = GC_DENSE; s->wum = GC_STATIC; s->src = src; s->trg = trg; s->psm = psm;
+    s->g = (float*)g; s->constantWeight = constantWeight;
+    return net->numSyns - 1;
+}
+
+int gc_add_syn_bitmask(gc_net *net, int src, int trg, int psm, const uint32_t *gp, uint32_t rowStride, float constantWeight)
+{
+    gc_syn *s = gc_new_syn(net);
+    s->matrix = GC_BITMASK; s->wum = GC_STATIC; s->src = src; s->trg = trg; s->psm = psm;
+    s->gp = gp; s->rowStride = rowStride; s->constantWeight = constantWeight;
+    return net->numSyns - 1;
+}
+
 /* backend.cc:156-179 — row-major traversal, so each column lists its synapses in ascending idSyn */
 void gc_build_remap(gc_net *net, int syn)
 {
@@ -263,6 +286,27 @@ void gc_update_synapses(gc_net *net, float t)
                         const int32_t postInd = (postRow * ow * oc) + (postCol * oc) + kernOutChan;
                         const uint32_t kernelInd = (uint32_t)((flipKernRow * kw * ic * oc) + (flipKernCol * ic * oc) + (preChan * oc) + kernOutChan);
                         psm->outPost[postInd] += s->g[kernelInd];
+                        s->events++;
+                    }
+                }
+            }
+            continue;
+        }
+        if(s->matrix == GC_DENSE || s->matrix == GC_BITMASK) {
+            /* backend.cc:1985-2021: for every spike, every postsynaptic neuron in ascending order */
+            for(uint32_t i = 0; i < src->spkCnt; i++) {
+                const uint32_t idPre = src->spk[i];
+                for(uint32_t ipost = 0; ipost < trg->n; ipost++) {
+                    if(s->matrix == GC_BITMASK) {
+                        const uint64_t gid = ((uint64_t)idPre * s->rowStride) + ipost;
+                        if(s->gp[gid / 32] & (0x80000000u >> (gid & 31))) {
+                            psm->outPost[ipost] += s->constantWeight;
+                            s->events++;
+                        }
+                    }
+                    else {
+                        const size_t idSyn = ((size_t)idPre * trg->n) + ipost;
+                        psm->outPost[ipost] += s->g ? s->g[idSyn] : s->constantWeight;
                         s->events++;
                     }
                 }

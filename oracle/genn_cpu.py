@@ -47,6 +47,8 @@ def lib():
         l.gc_add_syn_sparse.restype = i32; l.gc_add_syn_sparse.argtypes = [vp, i32, i32, i32, i32, u32, vp, vp, vp, vp, i32]
         l.gc_set_stdp_trace.restype = None; l.gc_set_stdp_trace.argtypes = [vp, i32, f32, f32, f32, f32, f32, f32, u32]
         l.gc_add_syn_conv2d.restype = i32; l.gc_add_syn_conv2d.argtypes = [vp, i32, i32, i32, vp, vp]
+        l.gc_add_syn_dense.restype = i32; l.gc_add_syn_dense.argtypes = [vp, i32, i32, i32, vp, C.c_float]
+        l.gc_add_syn_bitmask.restype = i32; l.gc_add_syn_bitmask.argtypes = [vp, i32, i32, i32, vp, u32, C.c_float]
         l.gc_build_remap.restype = None; l.gc_build_remap.argtypes = [vp, i32]
         l.gc_step.restype = None; l.gc_step.argtypes = [vp]
         l.gc_advance.restype = None; l.gc_advance.argtypes = [vp]
@@ -190,10 +192,13 @@ class OracleNet:
         for s in net.syns:
             src, trg = self.pop_id[s.src], self.pop_id[s.trg]
             if s.matrix == "sparse":
-                rl, ind, g = _as(s.row_length, np.uint32), _as(s.ind, np.uint32), _as(s.g, np.float32)
+                rl, ind = _as(s.row_length, np.uint32), _as(s.ind, np.uint32)
+                # StaticPulseConstantWeight (weightUpdateModels.h:202-213) adds its parameter g for every synapse: same loop,
+                # same value everywhere
+                g = np.full(ind.shape, literal_f32(s.wum_params["g"]), np.float32) if s.wum == "static_const" else _as(s.g, np.float32)
                 d = _as(s.d, np.uint8) if s.d is not None else None
                 self.keep += [rl, ind, g, d]
-                wum = {"static": GC_STATIC, "static_delay": GC_STATIC_DELAY, "stdp_trace": GC_STDP_TRACE}[s.wum]
+                wum = {"static": GC_STATIC, "static_const": GC_STATIC, "static_delay": GC_STATIC_DELAY, "stdp_trace": GC_STDP_TRACE}[s.wum]
                 sid = self.l.gc_add_syn_sparse(self.h, src, trg, self.psm_id[s.name], wum, s.row_stride, rl.ctypes.data, ind.ctypes.data,
                                                g.ctypes.data, d.ctypes.data if d is not None else None, int(s.wum == "stdp_trace"))
                 if s.wum == "stdp_trace":
@@ -209,6 +214,16 @@ class OracleNet:
                     self.l.gc_build_remap(self.h, sid)
                     self.col_stride = getattr(self, "col_stride", {})
                     self.col_stride[s.name] = max(1, stride)
+            elif s.matrix == "dense":
+                g = _as(s.g, np.float32) if s.g is not None else None
+                self.keep.append(g)
+                sid = self.l.gc_add_syn_dense(self.h, src, trg, self.psm_id[s.name], g.ctypes.data if g is not None else None,
+                                              C.c_float(literal_f32(s.wum_params.get("g", 0.0))))
+            elif s.matrix == "bitmask":
+                gp = _as(s.gp, np.uint32)
+                self.keep.append(gp)
+                sid = self.l.gc_add_syn_bitmask(self.h, src, trg, self.psm_id[s.name], gp.ctypes.data, s.row_stride,
+                                                C.c_float(literal_f32(s.wum_params["g"])))
             else:
                 conv = np.array([s.conv[k] for k in ("conv_kh", "conv_kw", "conv_ih", "conv_iw", "conv_ic", "conv_oh", "conv_ow", "conv_oc")], dtype=np.int32)
                 kern = _as(s.g, np.float32)

@@ -48,6 +48,23 @@ def test_forward(make_model):
         s.parallelism_hint = hint
         s.num_threads_per_spike = tps
         outputs.append(s)
+    # the reference's other decoder projections: constant weight (SPARSE, BITMASK), DENSE with individual weights
+    n = _silent_pop(model, "PostSparseConstantWeight", 4)
+    s = model.add_synapse_population("SparseConstantWeightSynapse", "SPARSE", ss, n,
+                                     init_weight_update("StaticPulseConstantWeight", {"g": 1.0}), init_postsynaptic("DeltaCurr"))
+    s.set_sparse_connections(pre, post)
+    outputs.append(s)
+    n = _silent_pop(model, "PostBitmask", 4)
+    s = model.add_synapse_population("BitmaskSynapse", "BITMASK", ss, n,
+                                     init_weight_update("StaticPulseConstantWeight", {"g": 1.0}), init_postsynaptic("DeltaCurr"))
+    s.set_sparse_connections(pre, post)
+    outputs.append(s)
+    dense = np.zeros((16, 4), np.float32)
+    dense[pre, post] = 1.0
+    n = _silent_pop(model, "PostDense", 4)
+    s = model.add_synapse_population("DenseSynapse", "DENSE", ss, n,
+                                     init_weight_update("StaticPulse", {}, {"g": dense.flatten()}), init_postsynaptic("DeltaCurr"))
+    outputs.append(s)
     model.build()
     model.load()
     place = 2 ** np.arange(4)

@@ -190,6 +190,69 @@ def test_toeplitz_batches_are_independent():
     model.unload()
 
 
+def _bitmask_words(n_pre, n_post, mask):
+    stride = (n_post + 31) // 32 * 32
+    bits = np.zeros((n_pre, stride), np.uint8)
+    bits[:, :n_post] = mask
+    return np.packbits(bits.reshape(-1), bitorder="big").view(">u4").astype(np.uint32), stride
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+def test_dense_and_bitmask_projections(fuse):
+    """DENSE (individual and constant weights), BITMASK and constant-weight SPARSE projections in a recurrent LIF network
+    whose populations are not multiples of the wavefront or of a connectivity word.  A lane that owns its outPost
+    element continues the sum in spike-queue order, the CPU backend's order, so without fusing everything is identical;
+    with fused postsynaptic models several projections share an outPost (partial sums, one atomic each) and state is
+    held to 1e-5."""
+    from genn_amd import rng
+    from genn_amd.netspec import Net, Pop, Syn
+    n_a, n_b = 300, 77
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.6, TauRefrac=2.0)
+    net = Net(name="dense_bitmask", dt=1.0, steps=200, fuse_psm=fuse)
+    net.pops.append(Pop("A", "lif", n_a, dict(lif), {"V": (-60.0 + 9.0 * rng.uniform(9, 1, 0, n_a)).astype(np.float32), "RefracTime": np.zeros(n_a, np.float32)}))
+    net.pops.append(Pop("B", "lif", n_b, dict(lif, Ioffset=0.45), {"V": (-60.0 + 9.0 * rng.uniform(9, 2, 0, n_b)).astype(np.float32), "RefracTime": np.zeros(n_b, np.float32)}))
+    g_ab = (0.02 * rng.normal(9, 3, 0, n_a * n_b)).astype(np.float32).reshape(n_a, n_b)
+    net.syns.append(Syn("AB_dense", "A", "B", matrix="dense", wum="static", psm="expcurr", tau=5.0, g=g_ab))
+    mask = rng.uniform(9, 4, 0, n_b * n_a).reshape(n_b, n_a) < 0.2
+    gp, stride = _bitmask_words(n_b, n_a, mask)
+    net.syns.append(Syn("BA_bitmask", "B", "A", matrix="bitmask", wum="static_const", wum_params={"g": -0.08}, psm="expcurr", tau=5.0, gp=gp, row_stride=stride))
+    net.syns.append(Syn("AA_dense_const", "A", "A", matrix="dense", wum="static_const", wum_params={"g": 0.0005}, psm="expcurr", tau=5.0))
+    ind = np.sort(rng.randint(9, 5, 0, n_b * 20, n_b).reshape(n_b, 20), axis=1).astype(np.uint32)
+    net.syns.append(Syn("BB_sparse_const", "B", "B", wum="static_const", wum_params={"g": 0.03}, psm="expcurr", tau=5.0,
+                        row_stride=20, row_length=np.full(n_b, 20, np.uint32), ind=ind))
+    model, oracle, counts = run_side_by_side(net, check_every=20, exact=not fuse, exact_steps=100)
+    assert counts["A"] > 1000 and counts["B"] > 50
+    assert model.synaptic_event_count == oracle.events()
+    model.unload()
+
+
+def test_dense_projection_batched():
+    """Batch of 3 through a DENSE projection: weights are shared, spike queues and outPost are per batch."""
+    from genn_amd.genn_model import GeNNModel, init_postsynaptic, init_weight_update
+    B, n_src, n_trg = 3, 40, 70
+    model = GeNNModel("float", "dense_batch", batch_size=B, dt=1.0)
+    start = np.stack([np.arange(n_src), np.arange(n_src), np.arange(n_src)]).astype(np.uint32)
+    # batch b's source i fires at step (i + b) % 7
+    times = np.stack([(np.arange(n_src) + b) % 7 for b in range(B)]).astype(np.float32)
+    src = model.add_neuron_population("S", n_src, "SpikeSourceArray", {}, {"startSpike": start + np.arange(B)[:, None] * n_src,
+                                                                          "endSpike": start + np.arange(B)[:, None] * n_src + 1})
+    src.set_extra_global_param("spikeTimes", times.reshape(-1))
+    lif = {"C": 1.0, "TauM": 20.0, "Vrest": -60.0, "Vreset": -60.0, "Vthresh": 1e9, "Ioffset": 0.0, "TauRefrac": 5.0}
+    trg = model.add_neuron_population("T", n_trg, "LIF", lif, {"V": -60.0, "RefracTime": 0.0})
+    w = np.arange(n_src * n_trg, dtype=np.float32).reshape(n_src, n_trg) % 13 - 6
+    s = model.add_synapse_population("ST", "DENSE", src, trg, init_weight_update("StaticPulse", {}, {"g": w.flatten()}), init_postsynaptic("DeltaCurr"))
+    model.build()
+    model.load()
+    for step in range(9):
+        model.update_synapses()
+        got = s.vars["outPost"].pull_from_device().reshape(B, n_trg)
+        for b in range(B):
+            fired = (times[b] == step - 1) if step > 0 else np.zeros(n_src, bool)
+            assert np.array_equal(got[b], w.T @ fired.astype(np.float32)), f"step {step}, batch {b}"
+        model.update_neurons()
+    model.unload()
+
+
 @pytest.mark.parametrize("resident", ["1", "0"])
 def test_graph_replay_matches_stepping(resident, monkeypatch):
     """run() either keeps the network resident on the chip for the whole chunk (one launch) or, with that plan switched

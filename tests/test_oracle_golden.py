@@ -248,6 +248,65 @@ def test_oracle_propagation_equals_dense_product():
     assert np.array_equal(o.out_post("SP"), dense.T @ fire.astype(np.float32))
 
 
+def _bitmask_words(n_pre, n_post, pre, post):
+    """BITMASK connectivity words: bit idPre*rowStride + idPost (row stride = numPost padded to 32), most significant bit
+    of a word first (single_threaded_cpu/backend.cc:1393-1404, 2003-2006)."""
+    stride = (n_post + 31) // 32 * 32
+    bits = np.zeros(n_pre * stride, np.uint8)
+    bits[np.asarray(pre) * stride + np.asarray(post)] = 1
+    return np.packbits(bits, bitorder="big").view(">u4").astype(np.uint32), stride
+
+
+# tests/features/test_event_propagation.py:65-260 — the decode table holds for the DENSE, BITMASK and constant-weight
+# projections of that test too
+@pytest.mark.parametrize("kind", ["dense", "dense_const_all", "bitmask", "sparse_const"])
+def test_oracle_forward_decode_other_matrix_types(kind):
+    pre, post = map(np.asarray, zip(*[(i, j) for i in range(16) for j in range(4) if (i + 1) & (1 << j)]))
+    net = Net("fwd", dt=1.0, steps=16, pops=[_one_hot_source("S", 16), _silent("P", 4)])
+    if kind == "dense":
+        g = np.zeros((16, 4), np.float32)
+        g[pre, post] = 1.0
+        net.syns.append(Syn("SP", "S", "P", matrix="dense", wum="static", psm="deltacurr", g=g))
+    elif kind == "dense_const_all":
+        net.syns.append(Syn("SP", "S", "P", matrix="dense", wum="static_const", wum_params={"g": 1.0}, psm="deltacurr"))
+    elif kind == "bitmask":
+        gp, stride = _bitmask_words(16, 4, pre, post)
+        net.syns.append(Syn("SP", "S", "P", matrix="bitmask", wum="static_const", wum_params={"g": 1.0}, psm="deltacurr", gp=gp, row_stride=stride))
+    else:
+        rl, ind, _ = _ragged(16, pre, post)
+        net.syns.append(Syn("SP", "S", "P", wum="static_const", wum_params={"g": 1.0}, psm="deltacurr", row_stride=ind.shape[1], row_length=rl, ind=ind))
+    o = OracleNet(net)
+    place = 2 ** np.arange(4)
+    for step in range(16):
+        o.l.gc_update_synapses(o.h, np.float32(step))
+        value = int(np.sum(place[np.isclose(o.out_post("SP"), 1.0)]))
+        assert value == (15 if kind == "dense_const_all" and step > 0 else step)
+        o.l.gc_update_neurons(o.h, np.float32(step), 0)
+        o.l.gc_advance(o.h)
+
+
+def test_oracle_dense_and_bitmask_equal_matrix_products():
+    """Brute force: one step through a DENSE matrix is W^T s, through a BITMASK one g * B^T s (small integers: sums exact)."""
+    rng = np.random.default_rng(5)
+    n_pre, n_post = 41, 37                      # more than one connectivity word per row, with padding bits
+    dense = rng.integers(-4, 5, (n_pre, n_post)).astype(np.float32)
+    mask = rng.random((n_pre, n_post)) < 0.4
+    fire = rng.random(n_pre) < 0.5
+    end = np.cumsum(fire).astype(np.uint32)
+    start = (end - fire).astype(np.uint32)
+    gp, stride = _bitmask_words(n_pre, n_post, *np.nonzero(mask))
+    net = Net("dense", dt=1.0, steps=2)
+    net.pops.append(Pop("S", "ssa", n_pre, {}, {"startSpike": start, "endSpike": end}, spike_times=np.zeros(int(fire.sum()), np.float32)))
+    net.pops += [_silent("P", n_post), _silent("Q", n_post)]
+    net.syns.append(Syn("SP", "S", "P", matrix="dense", wum="static", psm="deltacurr", g=dense))
+    net.syns.append(Syn("SQ", "S", "Q", matrix="bitmask", wum="static_const", wum_params={"g": 3.0}, psm="deltacurr", gp=gp, row_stride=stride))
+    o = OracleNet(net)
+    o.step()
+    o.l.gc_update_synapses(o.h, np.float32(1.0))
+    assert np.array_equal(o.out_post("SP"), dense.T @ fire.astype(np.float32))
+    assert np.array_equal(o.out_post("SQ"), 3.0 * (mask.T.astype(np.float32) @ fire.astype(np.float32)))
+
+
 def test_oracle_recording_bitfield():
     n = 70
     fire_at = np.arange(n) % 7
