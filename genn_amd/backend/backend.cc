@@ -177,6 +177,9 @@ unsigned int recogniseWUM(const WeightUpdateModels::Base *m, const std::string &
                        && m->getPreDynamicsCode().empty() && m->getPostDynamicsCode().empty();
     if(plain && same(m->getPreSpikeSynCode(), WeightUpdateModels::StaticPulse::getInstance()->getPreSpikeSynCode())
        && m->getVars().size() == 1) { return GENNMI_WUM_STATIC_PULSE; }
+    // StaticPulseConstantWeight (weightUpdateModels.h:202-213): the same code with g a parameter instead of a variable
+    if(plain && same(m->getPreSpikeSynCode(), WeightUpdateModels::StaticPulseConstantWeight::getInstance()->getPreSpikeSynCode())
+       && m->getVars().empty() && m->getParams().size() == 1 && m->getParams()[0].name == "g") { return GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT; }
     if(plain && same(m->getPreSpikeSynCode(), WeightUpdateModels::StaticPulseDendriticDelay::getInstance()->getPreSpikeSynCode())) {
         return GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY;
     }
@@ -497,7 +500,15 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                 const auto matrixType = arch.getMatrixType();
                 const bool sparse = (matrixType & SynapseMatrixConnectivity::SPARSE) && (matrixType & SynapseMatrixWeight::INDIVIDUAL);
                 const bool toeplitz = (matrixType & SynapseMatrixConnectivity::TOEPLITZ) && (matrixType & SynapseMatrixWeight::KERNEL);
-                if(!sparse && !toeplitz) { unsupported("matrix type of projection '" + arch.getName() + "' (SPARSE with individual weights or TOEPLITZ with kernel weights)"); }
+                const bool dense = (matrixType & SynapseMatrixConnectivity::DENSE) && (matrixType & SynapseMatrixWeight::INDIVIDUAL);
+                const bool bitmask = (matrixType & SynapseMatrixConnectivity::BITMASK) != 0;
+                const bool constantWeight = (wumKind == GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT);
+                if(!sparse && !toeplitz && !dense && !bitmask) {
+                    unsupported("matrix type of projection '" + arch.getName() + "' (SPARSE, DENSE, BITMASK or TOEPLITZ with kernel weights)");
+                }
+                if(dense && wumKind != GENNMI_WUM_STATIC_PULSE && !constantWeight) { unsupported("weight update model of DENSE projection '" + arch.getName() + "'"); }
+                if(bitmask && !constantWeight) { unsupported("weight update model of BITMASK projection '" + arch.getName() + "' (StaticPulseConstantWeight)"); }
+                if(toeplitz && constantWeight) { unsupported("constant weight on Toeplitz projection '" + arch.getName() + "'"); }
                 if(sparse && arch.getSparseIndType() != Type::Uint32) { unsupported("narrow sparse index type of projection '" + arch.getName() + "'"); }
                 if(toeplitz) {
                     const auto *conn = arch.getToeplitzConnectivityInitialiser().getSnippet();
@@ -535,7 +546,8 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                 };
 
                 out << "gennmi_presynaptic_update_group_t d = {};" << std::endl;
-                out << "d.matrix = " << (sparse ? GENNMI_MATRIX_SPARSE : GENNMI_MATRIX_TOEPLITZ_CONV2D) << "u; d.wum = " << wumKind << "u;" << std::endl;
+                out << "d.matrix = " << (sparse ? GENNMI_MATRIX_SPARSE : (dense ? GENNMI_MATRIX_DENSE : (bitmask ? GENNMI_MATRIX_BITMASK : GENNMI_MATRIX_TOEPLITZ_CONV2D)))
+                    << "u; d.wum = " << ((sparse && constantWeight) ? (unsigned int)GENNMI_WUM_STATIC_PULSE : wumKind) << "u;" << std::endl;
                 if(arch.getParallelismHint() == SynapseGroup::ParallelismHint::PRESYNAPTIC) {
                     out << "d.span = " << GENNMI_SPAN_PRE << "u; d.numThreadsPerSpike = " << arch.getNumThreadsPerSpike() << "u;" << std::endl;
                 }
@@ -547,11 +559,26 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                     << ", c[] = " << tableU32(counts([this](const SynapseGroupInternal &g){ return getSynapticMatrixRowStride(g); }))
                     << "; d.numSrcNeurons = a[g]; d.numTrgNeurons = b[g]; d.rowStride = c[g]; }" << std::endl;
                 out << "d.srcSpkCnt = gennmiDev(" << env["_src_spk_cnt"] << "); d.srcSpk = gennmiDev(" << env["_src_spk"] << ");" << std::endl;
-                out << "d.outPost = gennmiDev(" << env["_out_post"] << "); d.g = " << wuVar("g", scalar) << ";" << std::endl;
+                out << "d.outPost = gennmiDev(" << env["_out_post"] << ");" << std::endl;
+                if(constantWeight) {
+                    out << "{ static const float v[] = " << table(values([](const SynapseGroupInternal &g){ return g.getWUInitialiser().getParams().at("g"); }), scalar)
+                        << "; d.constantWeight = v[g]; }" << std::endl;
+                    if(sparse) {
+                        // the sparse kernels read a weight per synapse: the one weight is written out once, on the device
+                        out << "{ const size_t count = (size_t)d.numSrcNeurons * d.rowStride; float *w = reinterpret_cast<float*>(gennmiScratch(count));" << std::endl;
+                        out << "  GENNMI_CHECK(gennmi_fill_f32(w, d.constantWeight, count)); d.g = w; }" << std::endl;
+                    }
+                }
+                else {
+                    out << "d.g = " << wuVar("g", scalar) << ";" << std::endl;
+                }
                 if(sparse) {
                     out << "d.rowLength = gennmiDev(" << env["_row_length"] << "); d.ind = gennmiDev(" << env["_ind"] << ");" << std::endl;
                 }
-                else {
+                else if(bitmask) {
+                    out << "d.gp = gennmiDev(" << env["_gp"] << ");" << std::endl;
+                }
+                else if(toeplitz) {
                     const auto &names = std::vector<std::string>{"conv_kh", "conv_kw", "conv_ih", "conv_iw", "conv_ic", "conv_oh", "conv_ow", "conv_oc"};
                     for(size_t k = 0; k < names.size(); k++) {
                         out << "{ static const int32_t v[] = " << tableU32(counts([&names, k](const SynapseGroupInternal &g)

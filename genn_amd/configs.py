@@ -208,3 +208,28 @@ def conv_toeplitz(h=64, w=64, ic=16, oc=32, k=3, steps=500, seed=5, dt=1.0, batc
     net.syns.append(Syn("Conv", "In", "Out", matrix="conv2d", wum="static", psm="expcurr", tau=5.0, g=kern,
                         conv=dict(conv_kh=k, conv_kw=k, conv_ih=h, conv_iw=w, conv_ic=ic, conv_oh=h, conv_ow=w, conv_oc=oc)))
     return net
+
+
+def dense_bitmask(n_a=300, n_b=77, steps=200, seed=9, dt=1.0, fuse=False):
+    """Recurrent LIF network over the remaining matrix types: DENSE with individual weights (A -> B), BITMASK with a
+    constant weight (B -> A), DENSE with a constant weight (A -> A) and SPARSE with a constant weight (B -> B).  Sizes
+    that are no multiple of a wavefront or of a 32-bit connectivity word."""
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.6, TauRefrac=2.0)
+    net = Net(name="dense_bitmask", dt=dt, steps=steps, fuse_psm=fuse, seed=seed)
+    net.pops.append(Pop("A", "lif", n_a, dict(lif), {"V": (-60.0 + 9.0 * rng.uniform(seed, 1, 0, n_a)).astype(np.float32),
+                                                     "RefracTime": np.zeros(n_a, np.float32)}))
+    net.pops.append(Pop("B", "lif", n_b, dict(lif, Ioffset=0.45), {"V": (-60.0 + 9.0 * rng.uniform(seed, 2, 0, n_b)).astype(np.float32),
+                                                                   "RefracTime": np.zeros(n_b, np.float32)}))
+    g_ab = (0.02 * rng.normal(seed, 3, 0, n_a * n_b)).astype(np.float32).reshape(n_a, n_b)
+    net.syns.append(Syn("AB_dense", "A", "B", matrix="dense", wum="static", psm="expcurr", tau=5.0, g=g_ab))
+    stride = (n_a + 31) // 32 * 32
+    bits = np.zeros((n_b, stride), np.uint8)
+    bits[:, :n_a] = rng.uniform(seed, 4, 0, n_b * n_a).reshape(n_b, n_a) < 0.2
+    gp = np.packbits(bits.reshape(-1), bitorder="big").view(">u4").astype(np.uint32)       # most significant bit of a word first
+    net.syns.append(Syn("BA_bitmask", "B", "A", matrix="bitmask", wum="static_const", wum_params={"g": -0.08}, psm="expcurr", tau=5.0,
+                        gp=gp, row_stride=stride))
+    net.syns.append(Syn("AA_dense_const", "A", "A", matrix="dense", wum="static_const", wum_params={"g": 0.0005}, psm="expcurr", tau=5.0))
+    ind = np.sort(rng.randint(seed, 5, 0, n_b * 20, n_b).reshape(n_b, 20), axis=1).astype(np.uint32)
+    net.syns.append(Syn("BB_sparse_const", "B", "B", wum="static_const", wum_params={"g": 0.03}, psm="expcurr", tau=5.0,
+                        row_stride=20, row_length=np.full(n_b, 20, np.uint32), ind=ind))
+    return net

@@ -100,7 +100,7 @@ class Net:
             if c.noise is not None:
                 h.update(np.ascontiguousarray(c.noise).tobytes())
         for s in self.syns:
-            for a in (s.row_length, s.ind, s.g, s.d):
+            for a in (s.row_length, s.ind, s.g, s.d, s.gp):
                 if a is not None:
                     h.update(np.ascontiguousarray(a).tobytes())
         return h.hexdigest()
@@ -154,11 +154,19 @@ def write_netspec(net: Net, path: str):
             head = f"syn {s.name} sparse {s.src} {s.trg} {s.row_stride}"
             np.ascontiguousarray(s.row_length, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.rowLength.u32"))
             np.ascontiguousarray(s.ind, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.ind.u32"))
+        elif s.matrix == "dense":
+            head = f"syn {s.name} dense {s.src} {s.trg}"
+        elif s.matrix == "bitmask":
+            head = f"syn {s.name} bitmask {s.src} {s.trg}"
+            np.ascontiguousarray(s.gp, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.gp.u32"))
         else:
             head = f"syn {s.name} conv2d {s.src} {s.trg} " + " ".join(str(int(s.conv[k])) for k in CONV_PARAMS)
-        np.ascontiguousarray(s.g, dtype=np.float32).tofile(os.path.join(path, f"{s.name}.g.f32"))
+        if s.wum != "static_const":
+            np.ascontiguousarray(s.g, dtype=np.float32).tofile(os.path.join(path, f"{s.name}.g.f32"))
         if s.wum == "static":
             w = "static"
+        elif s.wum == "static_const":
+            w = f"static_const {float(s.wum_params['g'])!r}"
         elif s.wum == "static_delay":
             w = f"static_delay {s.max_den_delay}"
             np.ascontiguousarray(s.d, dtype=np.uint8).tofile(os.path.join(path, f"{s.name}.d.u8"))

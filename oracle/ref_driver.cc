@@ -169,10 +169,11 @@ int main(int argc, char *argv[])
                     SynSpec s; ls >> s.name >> s.matrix >> s.src >> s.trg;
                     if(s.matrix == "sparse") { ls >> s.rowStride; }
                     else if(s.matrix == "conv2d") { s.conv.resize(8); for(auto &c : s.conv) ls >> c; }
-                    else throw std::runtime_error("matrix " + s.matrix);
+                    else if(s.matrix != "dense" && s.matrix != "bitmask") throw std::runtime_error("matrix " + s.matrix);
                     ls >> s.wum;
                     if(s.wum == "static_delay") { ls >> s.maxDenDelay; }
                     else if(s.wum == "stdp_trace" || s.wum == "stdp") { s.wumP.resize(6); for(auto &c : s.wumP) ls >> c; }
+                    else if(s.wum == "static_const") { s.wumP.resize(1); ls >> s.wumP[0]; }
                     else if(s.wum != "static") throw std::runtime_error("wum " + s.wum);
                     ls >> s.psm;
                     if(s.psm == "expcurr") { s.psmP.resize(1); ls >> s.psmP[0]; }
@@ -224,7 +225,10 @@ int main(int argc, char *argv[])
             const auto psm = (s.psm == "expcurr") ? initPostsynaptic<PostsynapticModels::ExpCurr>({{"tau", s.psmP[0]}})
                                                   : initPostsynaptic<PostsynapticModels::DeltaCurr>();
             WeightUpdateModels::Init wum = initWeightUpdate<WeightUpdateModels::StaticPulse>({}, {{"g", uninitialisedVar()}});
-            if(s.wum == "static_delay") {
+            if(s.wum == "static_const") {
+                wum = initWeightUpdate<WeightUpdateModels::StaticPulseConstantWeight>({{"g", s.wumP[0]}});
+            }
+            else if(s.wum == "static_delay") {
                 wum = initWeightUpdate<WeightUpdateModels::StaticPulseDendriticDelay>({}, {{"g", uninitialisedVar()}, {"d", uninitialisedVar()}});
             }
             else if(s.wum == "stdp_trace") {
@@ -241,6 +245,12 @@ int main(int argc, char *argv[])
                 s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::SPARSE, src, trg, wum, psm);
                 s.sg->setMaxConnections(s.rowStride);
                 if(s.colStride) s.sg->setMaxSourceConnections(s.colStride);
+            }
+            else if(s.matrix == "dense") {
+                s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::DENSE, src, trg, wum, psm);
+            }
+            else if(s.matrix == "bitmask") {
+                s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::BITMASK, src, trg, wum, psm);
             }
             else {
                 s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::TOEPLITZ, src, trg, wum, psm,
@@ -320,10 +330,13 @@ int main(int argc, char *argv[])
             if(s.matrix == "sparse") {
                 load(rt.getArray(*s.sg, "rowLength"), s.name + ".rowLength.u32");
                 loadRows(rt.getArray(*s.sg, "ind"), s.name + ".ind.u32", s, uint32_t(0));
-                loadRows(rt.getArray(*s.sg, "g"), s.name + ".g.f32", s, float(0));
+                if(s.wum != "static_const") loadRows(rt.getArray(*s.sg, "g"), s.name + ".g.f32", s, float(0));
                 if(s.wum == "static_delay") loadRows(rt.getArray(*s.sg, "d"), s.name + ".d.u8", s, uint8_t(0));
             }
-            else {
+            else if(s.matrix == "bitmask") {
+                load(rt.getArray(*s.sg, "gp"), s.name + ".gp.u32");
+            }
+            else if(s.wum != "static_const") {
                 load(rt.getArray(*s.sg, "g"), s.name + ".g.f32");
             }
             if(s.wum == "stdp_trace") {

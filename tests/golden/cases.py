@@ -24,5 +24,9 @@ def conv_small():
     return configs.conv_toeplitz(h=8, w=8, ic=2, oc=4, steps=100, w_sd=0.6, ioffset=0.4), 25
 
 
-CASES = {"va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+def dense_small():
+    return configs.dense_bitmask(), 25
+
+
+CASES = {"dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
          "stdp_small": stdp_small, "conv_small": conv_small}

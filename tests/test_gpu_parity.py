@@ -190,13 +190,6 @@ def test_toeplitz_batches_are_independent():
     model.unload()
 
 
-def _bitmask_words(n_pre, n_post, mask):
-    stride = (n_post + 31) // 32 * 32
-    bits = np.zeros((n_pre, stride), np.uint8)
-    bits[:, :n_post] = mask
-    return np.packbits(bits.reshape(-1), bitorder="big").view(">u4").astype(np.uint32), stride
-
-
 @pytest.mark.parametrize("fuse", [False, True])
 def test_dense_and_bitmask_projections(fuse):
     """DENSE (individual and constant weights), BITMASK and constant-weight SPARSE projections in a recurrent LIF network
@@ -204,22 +197,7 @@ def test_dense_and_bitmask_projections(fuse):
     element continues the sum in spike-queue order, the CPU backend's order, so without fusing everything is identical;
     with fused postsynaptic models several projections share an outPost (partial sums, one atomic each) and state is
     held to 1e-5."""
-    from genn_amd import rng
-    from genn_amd.netspec import Net, Pop, Syn
-    n_a, n_b = 300, 77
-    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.6, TauRefrac=2.0)
-    net = Net(name="dense_bitmask", dt=1.0, steps=200, fuse_psm=fuse)
-    net.pops.append(Pop("A", "lif", n_a, dict(lif), {"V": (-60.0 + 9.0 * rng.uniform(9, 1, 0, n_a)).astype(np.float32), "RefracTime": np.zeros(n_a, np.float32)}))
-    net.pops.append(Pop("B", "lif", n_b, dict(lif, Ioffset=0.45), {"V": (-60.0 + 9.0 * rng.uniform(9, 2, 0, n_b)).astype(np.float32), "RefracTime": np.zeros(n_b, np.float32)}))
-    g_ab = (0.02 * rng.normal(9, 3, 0, n_a * n_b)).astype(np.float32).reshape(n_a, n_b)
-    net.syns.append(Syn("AB_dense", "A", "B", matrix="dense", wum="static", psm="expcurr", tau=5.0, g=g_ab))
-    mask = rng.uniform(9, 4, 0, n_b * n_a).reshape(n_b, n_a) < 0.2
-    gp, stride = _bitmask_words(n_b, n_a, mask)
-    net.syns.append(Syn("BA_bitmask", "B", "A", matrix="bitmask", wum="static_const", wum_params={"g": -0.08}, psm="expcurr", tau=5.0, gp=gp, row_stride=stride))
-    net.syns.append(Syn("AA_dense_const", "A", "A", matrix="dense", wum="static_const", wum_params={"g": 0.0005}, psm="expcurr", tau=5.0))
-    ind = np.sort(rng.randint(9, 5, 0, n_b * 20, n_b).reshape(n_b, 20), axis=1).astype(np.uint32)
-    net.syns.append(Syn("BB_sparse_const", "B", "B", wum="static_const", wum_params={"g": 0.03}, psm="expcurr", tau=5.0,
-                        row_stride=20, row_length=np.full(n_b, 20, np.uint32), ind=ind))
+    net = configs.dense_bitmask(fuse=fuse)
     model, oracle, counts = run_side_by_side(net, check_every=20, exact=not fuse, exact_steps=100)
     assert counts["A"] > 1000 and counts["B"] > 50
     assert model.synaptic_event_count == oracle.events()
