@@ -23,7 +23,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 # algorithmic bytes per synaptic event: ind 4 + g 4 + fp32 read-modify-write of the target 8 (+ 1 delay byte)
-BYTES_PER_EVENT = {"static": 16, "static_delay": 17, "stdp_trace": 28, "conv2d": 8}
+BYTES_PER_EVENT = {"dense": 4,          # one weight read per (spike, target); outPost is read and written once per target and step
+                   "static": 16, "static_delay": 17, "stdp_trace": 28, "conv2d": 8}
 # HBM bytes per launch of the dominant kernel, from hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each
 # scaled by what the same counter reads for the library's 256 MiB copy kernel); recorded with the commands that
 # produced them in profiles/<kernel>_<workload>.md.  They are measurements of an earlier run of the same workload,
@@ -43,6 +44,8 @@ def build_net(name, steps):
         return configs.potjans(neuron_scale=0.1, connectivity_scale=1.0, steps=steps), "potjans 10% neurons full in-degree"
     if name == "va":
         return configs.vogels_abbott(steps=steps), "C1 balanced LIF 4000 neurons p=0.02 dt=0.1ms"
+    if name == "dense":
+        return configs.dense_layer(steps=steps), "dense layer 8192 Poisson sources (50 Hz) -> 8192 LIF, DENSE individual weights, dt=1ms"
     if name == "izh":
         return configs.izhikevich_fanout(steps=steps, noise_steps=64), "C3 izhikevich 1e6 neurons fanout 1000 dt=1ms (noise rows cycled)"
     if name == "izh_small":
@@ -145,7 +148,7 @@ def main():
     gen_s = time.time() - t0
     num_neurons = sum(p.n for p in net.pops)
     num_synapses = sum(s.num_synapses for s in net.syns)
-    kinds = {("conv2d" if s.matrix == "conv2d" else s.wum) for s in net.syns}
+    kinds = {(s.matrix if s.matrix in ("conv2d", "dense", "bitmask") else s.wum) for s in net.syns}
     bytes_per_event = max(BYTES_PER_EVENT[k] for k in kinds) if len(kinds) == 1 else None
 
     t0 = time.time()
@@ -215,7 +218,7 @@ def main():
             ev_per_launch = evp / st["presyn_launches"]
             achieved = ev_per_launch * bpe / avg_s / 1e9
             navg = st["neuron_seconds"] / max(1, st["neuron_launches"])
-            roofline = {"bound": "hbm", "kernel": "presynapticUpdateKernel (+ presynapticTileKernel)", "achieved": round(achieved, 3),
+            roofline = {"bound": "hbm", "kernel": "presynapticDenseKernel" if kinds == {"dense"} else "presynapticUpdateKernel (+ presynapticTileKernel)", "achieved": round(achieved, 3),
                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6), "traffic": None,
                         "bytes_per_event": bpe, "events_per_launch": round(ev_per_launch, 1), "avg_launch_us": round(avg_s * 1e6, 3),
                         "neuron_kernel_avg_us": round(navg * 1e6, 3), "neuron_kernel_gbs": round(neuron_bytes / navg / 1e9, 3)}

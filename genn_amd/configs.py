@@ -233,3 +233,16 @@ def dense_bitmask(n_a=300, n_b=77, steps=200, seed=9, dt=1.0, fuse=False):
     net.syns.append(Syn("BB_sparse_const", "B", "B", wum="static_const", wum_params={"g": 0.03}, psm="expcurr", tau=5.0,
                         row_stride=20, row_length=np.full(n_b, 20, np.uint32), ind=ind))
     return net
+
+
+def dense_layer(n_in=8192, n_out=8192, rate_hz=50.0, steps=1000, seed=17, dt=1.0, w_sd=0.02):
+    """A fully connected spiking layer: Poisson sources (rate_hz per source) into LIF neurons through a DENSE matrix
+    with individual weights ~ N(0, w_sd); the shape of the dense layers of rate-coded classifiers."""
+    net = Net(name="dense_layer", dt=dt, steps=steps, seed=seed)
+    start, end, times = poisson_spike_source(seed, 1, n_in, rate_hz, steps, dt)
+    net.pops.append(Pop("In", "ssa", n_in, {}, {"startSpike": start, "endSpike": end}, spike_times=times))
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.3, TauRefrac=2.0)
+    net.pops.append(Pop("Out", "lif", n_out, lif, {"V": np.full(n_out, -60.0, np.float32), "RefracTime": np.zeros(n_out, np.float32)}))
+    g = netgen.normal_f32(seed, 2, 0, n_in * n_out, 0.0, w_sd).reshape(n_in, n_out)
+    net.syns.append(Syn("InOut", "In", "Out", matrix="dense", wum="static", psm="expcurr", tau=5.0, g=g))
+    return net

@@ -367,16 +367,18 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
 // per postsynaptic neuron walks the spike queue: weights of a spike's row are lane-consecutive (DENSE: g[idPre*numTrg
 // + idPost]) or one bit each (BITMASK, most significant bit first), so there is nothing to scatter and no atomic —
 // a lane that owns its outPost element alone continues the sum from the value that is there, in queue order, which is
-// the CPU backend's order bit for bit.  When several projections feed one outPost the lane's partial sum is added
-// with one (lane-consecutive) atomic instead.
+// the CPU backend's order bit for bit.  When several projections feed one outPost, or a step carries so many spikes
+// that the queue is shared between several blocks, the lane's partial sum is added with one (lane-consecutive) atomic.
 // ------------------------------------------------------------------------------------------------
 struct DenseGroupDev
 {
     gennmi_presynaptic_update_group_t g;
-    uint32_t startBlock, numBlocks;
+    uint32_t startBlock, numBlocks;     // numBlocks = column blocks x slices
     uint32_t exclusive;                 // no other projection adds to this outPost
-    uint32_t pad_;
+    uint32_t slices;                    // blocks that may share the spike queue of one block of columns
 };
+
+constexpr uint32_t DENSE_SPIKES_PER_SLICE = 16;     // a step with fewer spikes than this per slice uses fewer slices
 
 __global__ __launch_bounds__(BLOCK)
 void presynapticDenseKernel(const DenseGroupDev * __restrict__ blocks, unsigned long long *eventCounter)
@@ -384,37 +386,46 @@ void presynapticDenseKernel(const DenseGroupDev * __restrict__ blocks, unsigned 
     const DenseGroupDev &G = blocks[blockIdx.x];
     const gennmi_presynaptic_update_group_t &g = G.g;
     const uint32_t batch = blockIdx.y;
-    const uint32_t j = (blockIdx.x - G.startBlock) * BLOCK + threadIdx.x;
+    const uint32_t local = blockIdx.x - G.startBlock;
+    const uint32_t slice = local % G.slices;
+    const uint32_t j = (local / G.slices) * BLOCK + threadIdx.x;
     const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
-    if(numSpikes == 0) { return; }
+    // The queue is cut into as many contiguous pieces as there are slices with at least 16 spikes each; with one
+    // piece the lane continues the sum from outPost itself (exact queue order), with more every piece adds its partial sum.
+    const uint32_t active = min(G.slices, max(1u, numSpikes / DENSE_SPIKES_PER_SLICE));
+    if(numSpikes == 0 || slice >= active) { return; }
+    const uint32_t perSlice = (numSpikes + active - 1) / active;
+    const uint32_t first = slice * perSlice, last = min(numSpikes, first + perSlice);
+    if(first >= numSpikes) { return; }          // rounding up perSlice can leave the last pieces empty
+    const bool continueSum = G.exclusive && active == 1;
     GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
     GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
     unsigned long long events = 0;
     if(j < g.numTrgNeurons) {
-        float acc = G.exclusive ? outPost[j] : 0.0f;
+        float acc = continueSum ? outPost[j] : 0.0f;
         if(g.matrix == GENNMI_MATRIX_DENSE) {
             const bool constant = (g.wum == GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT);
             GLOBAL_AS const float *weight = asGlobal(g.g);
-            // four rows in flight; the additions keep queue order
-            uint32_t s = 0;
-            for(; s + 4 <= numSpikes; s += 4) {
-                float w[4];
+            // eight rows in flight; the additions keep queue order
+            uint32_t s = first;
+            for(; s + 8 <= last; s += 8) {
+                float w[8];
                 #pragma unroll
-                for(int u = 0; u < 4; u++) { w[u] = constant ? g.constantWeight : weight[(size_t)spk[s + u] * g.numTrgNeurons + j]; }
+                for(int u = 0; u < 8; u++) { w[u] = constant ? g.constantWeight : weight[(size_t)spk[s + u] * g.numTrgNeurons + j]; }
                 #pragma unroll
-                for(int u = 0; u < 4; u++) { acc += w[u]; }
+                for(int u = 0; u < 8; u++) { acc += w[u]; }
             }
-            for(; s < numSpikes; s++) { acc += constant ? g.constantWeight : weight[(size_t)spk[s] * g.numTrgNeurons + j]; }
-            if(j == 0) { events = (unsigned long long)numSpikes * g.numTrgNeurons; }
+            for(; s < last; s++) { acc += constant ? g.constantWeight : weight[(size_t)spk[s] * g.numTrgNeurons + j]; }
+            if(j == 0) { events = (unsigned long long)(last - first) * g.numTrgNeurons; }
         }
         else {
             GLOBAL_AS const uint32_t *gp = asGlobal(g.gp);
-            for(uint32_t s = 0; s < numSpikes; s++) {
+            for(uint32_t s = first; s < last; s++) {
                 const unsigned long long gid = (unsigned long long)spk[s] * g.rowStride + j;
                 if(gp[gid >> 5] & (0x80000000u >> (gid & 31))) { acc += g.constantWeight; events++; }
             }
         }
-        if(G.exclusive) { outPost[j] = acc; }
+        if(continueSum) { outPost[j] = acc; }
         else if(acc != 0.0f) { atomicAddF32(&outPost[j], acc); }
     }
     for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
@@ -2225,8 +2236,11 @@ int gennmi_runner_finalise(gennmi_runner *r)
     // bitmask group adds to the same one (sparse groups have finished by the time this kernel starts)
     block = 0;
     for(auto &d : r->dense) {
+        const uint32_t columnBlocks = (d.g.numTrgNeurons + BLOCK - 1) / BLOCK;
+        // enough blocks to cover the chip a few times when a step carries many spikes
+        d.slices = std::max(1u, std::min({64u, (4u * numCU + columnBlocks - 1) / columnBlocks, (d.g.numSrcNeurons + DENSE_SPIKES_PER_SLICE - 1) / DENSE_SPIKES_PER_SLICE}));
         d.startBlock = block;
-        d.numBlocks = (d.g.numTrgNeurons + BLOCK - 1) / BLOCK;
+        d.numBlocks = columnBlocks * d.slices;
         block += d.numBlocks;
         d.exclusive = 1;
         for(const auto &o : r->dense) { if(&o != &d && o.g.outPost == d.g.outPost) { d.exclusive = 0; } }

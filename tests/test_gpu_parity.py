@@ -204,6 +204,20 @@ def test_dense_and_bitmask_projections(fuse):
     model.unload()
 
 
+def test_dense_layer_many_spikes_per_step():
+    """A DENSE layer in which a step carries hundreds of spikes: the queue is cut into pieces handled by different blocks,
+    each adding a partial sum.  Weights are multiples of 2^-10 and the postsynaptic model keeps nothing between steps, so
+    every sum is exact in any order and state, spikes and event counts must still be identical."""
+    net = configs.dense_layer(n_in=2100, n_out=530, rate_hz=120.0, steps=60, w_sd=0.03)
+    syn = net.syns[0]
+    syn.g = (np.rint(syn.g * 1024.0) / 1024.0).astype(np.float32)
+    syn.psm = "deltacurr"
+    model, oracle, counts = run_side_by_side(net, check_every=10, exact=True)
+    assert counts["In"] > 60 * 200 and counts["Out"] > 50
+    assert model.synaptic_event_count == oracle.events() == (counts["In"] - len(oracle.spikes("In"))) * 530
+    model.unload()
+
+
 def test_dense_projection_batched():
     """Batch of 3 through a DENSE projection: weights are shared, spike queues and outPost are per batch."""
     from genn_amd.genn_model import GeNNModel, init_postsynaptic, init_weight_update
