@@ -44,7 +44,7 @@ class NeuronUpdateGroup(C.Structure):
                 ("preTrace", p_f32), ("postTrace", p_f32),
                 ("preDecay", C.c_float), ("postDecay", C.c_float),
                 ("sT", p_f32), ("spkCnt", p_u32), ("spk", p_u32), ("recordSpk", p_u32),
-                ("numExtraSpk", C.c_uint32), ("pad_", C.c_uint32),
+                ("numExtraSpk", C.c_uint32), ("numDelaySlots", C.c_uint32),
                 ("extraSpkCnt", p_u32 * MAX_EXTRA_SPK), ("extraSpk", p_u32 * MAX_EXTRA_SPK)]
 
 
@@ -58,7 +58,8 @@ class PresynapticUpdateGroup(C.Structure):
                 ("trgST", p_f32), ("postTrace", p_f32),
                 ("aMinus", C.c_float), ("wMin", C.c_float), ("wMax", C.c_float),
                 ("conv", C.c_int32 * 8),
-                ("gp", p_u32), ("constantWeight", C.c_float), ("pad2_", C.c_uint32)]
+                ("gp", p_u32), ("constantWeight", C.c_float), ("axonalDelaySteps", C.c_uint32),
+                ("numSrcDelaySlots", C.c_uint32), ("pad3_", C.c_uint32)]
 
 
 class PostsynapticUpdateGroup(C.Structure):

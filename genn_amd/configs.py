@@ -21,7 +21,9 @@ def _const_rows(row_length, stride, value):
 # --------------------------------------------------------------------------------------------
 # C1: balanced LIF network (Vogels-Abbott shape)
 # --------------------------------------------------------------------------------------------
-def vogels_abbott(n=4000, steps=10000, seed=1234, p=0.02, dt=0.1, ioffset=0.55, pad=1):
+def vogels_abbott(n=4000, steps=10000, seed=1234, p=0.02, dt=0.1, ioffset=0.55, pad=1, axonal_delays=None):
+    """Balanced LIF network (E/I 4:1, fixed connection probability).  `axonal_delays`: axonal delay in timesteps per
+    projection name ("EE", "EI", "IE", "II"), default none."""
     n_e = (n * 4) // 5
     n_i = n - n_e
     lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=ioffset, TauRefrac=5.0)
@@ -35,7 +37,8 @@ def vogels_abbott(n=4000, steps=10000, seed=1234, p=0.02, dt=0.1, ioffset=0.55, 
             rl, ind = netgen.fixed_probability(seed, stream, n_src, n_trg, p, pad=pad)
             stream += 1
             net.syns.append(Syn(f"{src}{trg}", src, trg, wum="static", psm="expcurr", tau=tau,
-                                row_stride=ind.shape[1], row_length=rl, ind=ind, g=_const_rows(rl, ind.shape[1], w)))
+                                row_stride=ind.shape[1], row_length=rl, ind=ind, g=_const_rows(rl, ind.shape[1], w),
+                                axonal_delay_steps=int((axonal_delays or {}).get(f"{src}{trg}", 0))))
     return net
 
 

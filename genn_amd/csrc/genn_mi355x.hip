@@ -217,15 +217,20 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
     // spikes of the previous step: the population's own queue, or (when this launch may run next to the
     // neuron update that refills that queue) the shadow copy written one step ago
     const uint32_t parity = (uint32_t)((st.epoch + 1) & 1);
-    GLOBAL_AS const uint32_t *cntPtr = G.shadowSpk ? asGlobal(G.shadowCnt) + (size_t)parity * gridDim.y : asGlobal(g.srcSpkCnt);
+    // axonal delay: the source's queue is a ring of slots; this projection reads the slot written axonalDelaySteps + 1
+    // updates ago, (spkQuePtr + slots - delay) % slots with spkQuePtr = epoch % slots (backendBase.cc:207-216)
+    const uint32_t slots = max(1u, g.numSrcDelaySlots);
+    const uint32_t readSlot = (slots > 1) ? modStep(st.epoch + slots - g.axonalDelaySteps, slots) : 0u;
+    GLOBAL_AS const uint32_t *cntPtr = G.shadowSpk ? asGlobal(G.shadowCnt) + (size_t)parity * gridDim.y + batch
+                                                   : asGlobal(g.srcSpkCnt) + ((size_t)batch * slots + readSlot);
     GLOBAL_AS const uint32_t *spk = G.shadowSpk ? asGlobal(G.shadowSpk) + ((size_t)parity * gridDim.y + batch) * g.numSrcNeurons
-                                                : asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+                                                : asGlobal(g.srcSpk) + ((size_t)batch * slots + readSlot) * g.numSrcNeurons;
     // the first spike id this sub-group would handle is fetched together with the count, not after it (the
     // queue always holds numSrcNeurons entries, so any index below that is readable)
     const uint32_t sparseSpan = W * (G.vec4 ? 4u : 1u);
     const uint32_t sparseChunksPerRow = (g.rowStride + sparseSpan - 1) / sparseSpan;
     const uint32_t firstSpike = (g.matrix == GENNMI_MATRIX_SPARSE) ? spk[min(subGroup / max(sparseChunksPerRow, 1u), g.numSrcNeurons - 1)] : 0u;
-    const uint32_t numSpikes = cntPtr[batch];
+    const uint32_t numSpikes = cntPtr[0];
     if(G.tileThreshold && (unsigned long long)numSpikes * G.workPerSpike >= G.tileThreshold) { return; }
     GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
     unsigned long long events = 0;
@@ -966,8 +971,12 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
     __syncthreads();
     const uint32_t prefix = shPrefix;
     if(prefix == 0xFFFFFFFFu) { return; }       // bounded wait expired: flagged, nothing written
-    if(spiked) { g.spk[(size_t)batch * n + prefix + waveOffset + laneRank] = i; }
-    if(last && threadIdx.x == 0) { g.spkCnt[batch] = prefix + blockCount; }
+    // with axonal delay the queue is a ring of slots and this step writes slot (epoch + 1) % slots: the reference's
+    // spkQuePtr after the increment at the start of its updateNeurons (neuronUpdateGroupMerged.cc:947-953)
+    const uint32_t delaySlots = max(1u, g.numDelaySlots);
+    const size_t queue = (size_t)batch * delaySlots + ((delaySlots > 1) ? modStep(st.epoch + 1, delaySlots) : 0u);
+    if(spiked) { g.spk[queue * n + prefix + waveOffset + laneRank] = i; }
+    if(last && threadIdx.x == 0) { g.spkCnt[queue] = prefix + blockCount; }
     // further copies of the queue (one population can feed several spike arrays: its own outgoing projections
     // and, for learnPost, the incoming plastic ones; runtime.cc:267-278)
     for(uint32_t q = 0; q < g.numExtraSpk; q++) {
@@ -1892,6 +1901,9 @@ int gennmi_push_neuron_update_group(gennmi_runner *r, const gennmi_neuron_update
     if(g->numNeurons == 0) { return fail(GENNMI_EINVAL, "push_neuron_update_group: empty population"); }
     if(g->numPSM > GENNMI_MAX_PSM || g->numCS > GENNMI_MAX_CS) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: too many children"); }
     if(!g->spk || !g->spkCnt) { return fail(GENNMI_EINVAL, "push_neuron_update_group: spike queue missing"); }
+    if(g->numDelaySlots > 1 && (g->numExtraSpk || g->preTrace || g->postTrace || g->sT)) {
+        return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: axonal delay slots together with plasticity or further spike arrays");
+    }
     if(g->model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
         if(!g->startSpike || !g->endSpike || !g->spikeTimes) { return fail(GENNMI_EINVAL, "push_neuron_update_group: spike source arrays missing"); }
     }
@@ -1938,6 +1950,7 @@ int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynap
                 return fail(GENNMI_EINVAL, "push_presynaptic_update_group: bitmask words missing or row stride not numTrg padded to 32");
             }
         }
+        if(g->numSrcDelaySlots > 1 || g->axonalDelaySteps) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: axonal delay on a DENSE or BITMASK projection"); }
         DenseGroupDev dd;
         memset(&dd, 0, sizeof(dd));
         dd.g = *g;
@@ -1947,6 +1960,11 @@ int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynap
         return GENNMI_OK;
     }
     if(!g->g) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: required array missing"); }
+    if(g->numSrcDelaySlots > 1) {
+        if(g->axonalDelaySteps >= g->numSrcDelaySlots) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: axonal delay does not fit the source's delay slots"); }
+        if(g->wum == GENNMI_WUM_STDP_TRACE) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: axonal delay on a plastic projection"); }
+    }
+    else if(g->axonalDelaySteps) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: axonal delay without delay slots"); }
     PreGroupDev d;
     memset(&d, 0, sizeof(d));
     d.g = *g;
@@ -2009,7 +2027,7 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
     if(r->batch != 1 || !r->post.empty() || r->pre.empty() || !r->dense.empty() || r->neuron.size() > RES_MAX_GROUPS) { return GENNMI_OK; }
     for(const auto &n : r->neuron) {
         const auto &g = n.g;
-        if((g.model != GENNMI_NEURON_LIF && g.model != GENNMI_NEURON_IZHIKEVICH) || g.preTrace || g.postTrace || g.sT) { return GENNMI_OK; }
+        if((g.model != GENNMI_NEURON_LIF && g.model != GENNMI_NEURON_IZHIKEVICH) || g.preTrace || g.postTrace || g.sT || g.numDelaySlots > 1) { return GENNMI_OK; }
         for(uint32_t c = 0; c < g.numCS; c++) { if(g.cs[c].kind != GENNMI_CS_DC) { return GENNMI_OK; } }
     }
     // tiles and their LDS layout
@@ -2176,6 +2194,14 @@ int gennmi_runner_finalise(gennmi_runner *r)
     HIP_TRY(hipGetDeviceProperties(&prop, device));
     const uint32_t numCU = (uint32_t)prop.multiProcessorCount;
 
+    // a projection's view of its source's delay slots must be the source's own
+    for(const auto &p : r->pre) {
+        for(const auto &n : r->neuron) {
+            if(n.g.spk == p.g.srcSpk && std::max(1u, n.g.numDelaySlots) != std::max(1u, p.g.numSrcDelaySlots)) {
+                return fail(GENNMI_EINVAL, "runner_finalise: a projection and its source population disagree on the number of delay slots");
+            }
+        }
+    }
     uint32_t block = 0;
     for(auto &n : r->neuron) {
         n.startBlock = block;
@@ -2270,6 +2296,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
         std::vector<ConvTileDev> convTiles;
         for(auto &p : r->pre) {
             p.workPerSpike = (p.g.matrix == GENNMI_MATRIX_SPARSE) ? p.g.rowStride : (uint32_t)(p.g.conv[0] * p.g.conv[1] * p.g.conv[7]);
+            if(p.g.numSrcDelaySlots > 1) { continue; }       // the tile kernels read the queue without delay slots
             if(tileFloats != 0 && p.g.matrix == GENNMI_MATRIX_TOEPLITZ_CONV2D && r->pre.size() == 1
                && p.g.conv[0] < 1024 && p.g.conv[1] < 1024 && p.g.conv[7] < 1024
                && p.g.conv[2] < 1024 && p.g.conv[3] < 1024 && p.g.conv[4] < 1024) {        // rows, columns and channels are packed 10 bits each
@@ -2358,7 +2385,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
     bool eligible = !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty() && r->dense.empty();
     for(const auto &p : r->pre) {
         eligible = eligible && p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY
-                   && p.g.maxDenDelay >= 2;
+                   && p.g.maxDenDelay >= 2 && p.g.numSrcDelaySlots <= 1;
         bool found = false;
         for(const auto &n : r->neuron) { found = found || (n.g.spk == p.g.srcSpk && n.g.numNeurons == p.g.numSrcNeurons); }
         eligible = eligible && found;

@@ -219,6 +219,7 @@ class NeuronGroup:
         self.pre_trace_owner = None
         self.post_trace_owner = None
         self.needs_spike_time = False
+        self.num_delay_slots = 1     # longest axonal delay of the outgoing projections + 1, set by build()
 
     @property
     def size(self):
@@ -235,9 +236,13 @@ class NeuronGroup:
     @property
     def current_spikes(self):
         """Spike queue written by the last step: ids in ascending order (per batch)."""
-        cnt = self.vars["spkCnt"].pull_from_device().copy()
-        spk = self.vars["spk"].pull_from_device().reshape(self._model.batch_size, self.num_neurons)
-        return [spk[b, :cnt[b]].copy() for b in range(self._model.batch_size)]
+        # with axonal delay the queue is a ring of slots; the last step wrote slot timestep % slots (pygenn's current_spikes
+        # reads spkQuePtr the same way, genn_groups.py)
+        slots, B = self.num_delay_slots, self._model.batch_size
+        slot = self._model.timestep % slots
+        cnt = self.vars["spkCnt"].pull_from_device().reshape(B, slots)[:, slot].copy()
+        spk = self.vars["spk"].pull_from_device().reshape(B, slots, self.num_neurons)[:, slot]
+        return [spk[b, :cnt[b]].copy() for b in range(B)]
 
 
 class CurrentSource:
@@ -267,6 +272,7 @@ class SynapseGroup:
         self.max_dendritic_delay_timesteps = 1
         self.parallelism_hint = "POSTSYNAPTIC"
         self.num_threads_per_spike = 1
+        self.axonal_delay_steps = 0
         self.row_stride = 0
         self.col_stride = 0
         self.row_length_host = None
@@ -429,6 +435,7 @@ class GeNNModel:
             post = [s for s in n.in_syn if s.wu.snippet == "STDPTrace"]
             if len(pre) > 1 or len(post) > 1:
                 raise NotImplementedError(f"{n.name}: more than one plastic projection per side")
+            n.num_delay_slots = max([s.axonal_delay_steps for s in n.out_syn], default=0) + 1
             n.pre_trace_owner = pre[0] if pre else None
             n.post_trace_owner = post[0] if post else None
             n.needs_spike_time = bool(pre or post)
@@ -489,8 +496,8 @@ class GeNNModel:
                     a.view[:] = np.broadcast_to(init, (B, N)).reshape(-1) if init.ndim < 2 else init.reshape(-1)
                     a.push_to_device()
                     n.vars[v] = a
-            n.vars["spkCnt"] = self._alloc(B, np.uint32)
-            n.vars["spk"] = self._alloc(B * N, np.uint32)
+            n.vars["spkCnt"] = self._alloc(B * n.num_delay_slots, np.uint32)
+            n.vars["spk"] = self._alloc(B * n.num_delay_slots * N, np.uint32)
             if n.spike_recording_enabled:
                 if not num_recording_timesteps:
                     raise RuntimeError("Cannot use recording system without specifying number of recording timesteps")
@@ -629,7 +636,7 @@ class GeNNModel:
     def _neuron_merge_key(self, n):
         psm = tuple((grp[0].ps.snippet, self._den_delay(grp[0])) for grp in self._sorted_psm(n))
         return (n.neuron, psm, tuple(cs.kind for cs in n.current_sources), n.pre_trace_owner is not None,
-                n.post_trace_owner is not None, n.needs_spike_time, n.spike_recording_enabled)
+                n.post_trace_owner is not None, n.needs_spike_time, n.spike_recording_enabled, n.num_delay_slots)
 
     def _sorted_psm(self, n):
         # children are ordered by a structure-only digest, ties keep creation order (groupMerged.h:411-454)
@@ -648,6 +655,7 @@ class GeNNModel:
                 d.model = {"LIF": _abi.NEURON_LIF, "Izhikevich": _abi.NEURON_IZHIKEVICH, "SpikeSourceArray": _abi.NEURON_SPIKE_SOURCE_ARRAY}[model]
                 d.numNeurons = n.num_neurons
                 d.spkCnt, d.spk = n.vars["spkCnt"].ptr, n.vars["spk"].ptr
+                d.numDelaySlots = n.num_delay_slots
                 d.recordSpk = n.vars["recordSpk"].ptr if "recordSpk" in n.vars else None
                 d.sT = n.vars["sT"].ptr if "sT" in n.vars else None
             if model == "SpikeSourceArray":
@@ -743,6 +751,7 @@ class GeNNModel:
                 owner = s.fused_ps_target
                 d.outPost = owner.vars["outPost"].ptr
                 d.srcSpkCnt, d.srcSpk = s.src.vars["spkCnt"].ptr, s.src.vars["spk"].ptr
+                d.axonalDelaySteps, d.numSrcDelaySlots = s.axonal_delay_steps, s.src.num_delay_slots
                 if "g" in s.vars:
                     d.g = s.vars["g"].ptr
                 if s.matrix_type == "BITMASK":
@@ -910,6 +919,7 @@ def model_from_net(net, batch_size=1, record=True, span=None, device=0):
                 sg.set_var_ragged("d", s.d)
             if s.max_den_delay:
                 sg.max_dendritic_delay_timesteps = s.max_den_delay
+            sg.axonal_delay_steps = s.axonal_delay_steps
             if s.hint_pre:
                 sg.parallelism_hint = "PRESYNAPTIC"
                 sg.num_threads_per_spike = s.threads_per_spike

@@ -60,6 +60,7 @@ class Syn:
     hint_pre: bool = False
     col_stride: int = 0             # longest column (plastic projections); 0 = let the executor size it
     threads_per_spike: int = 1
+    axonal_delay_steps: int = 0     # spikes reach the projection this many timesteps late (SynapseGroup::setAxonalDelaySteps)
     conv: Dict[str, int] = field(default_factory=dict)
 
     @property
@@ -176,6 +177,8 @@ def write_netspec(net: Net, path: str):
             raise ValueError(s.wum)
         psm = f"expcurr {float(s.tau)!r}" if s.psm == "expcurr" else "deltacurr"
         opts = (" hint_pre" if s.hint_pre else "") + (f" tps {s.threads_per_spike}" if s.threads_per_spike > 1 else "")
+        if s.axonal_delay_steps:
+            opts += f" axonal_delay {int(s.axonal_delay_steps)}"
         if s.wum == "stdp_trace":
             mask = np.arange(s.row_stride)[None, :] < s.row_length[:, None]
             col = s.col_stride or int(np.bincount(s.ind[mask], minlength=net.pop(s.trg).n).max())

@@ -129,12 +129,16 @@ typedef struct gennmi_neuron_update_group_t {      /* MergedNeuronUpdateGroup<i>
     float *preTrace, *postTrace;          /* fused WU pre / post variables (OutSynWUMPre / InSynWUMPost children), or NULL */
     float preDecay, postDecay;
     float *sT;                            /* spike times [batch*numNeurons] or NULL */
-    uint32_t *spkCnt;                     /* [batch] */
-    uint32_t *spk;                        /* [batch*numNeurons], ascending neuron index within a step */
+    uint32_t *spkCnt;                     /* [batch * max(1, numDelaySlots)] */
+    uint32_t *spk;                        /* [batch * max(1, numDelaySlots) * numNeurons], ascending neuron index within a step */
     uint32_t *recordSpk;                  /* [numRecordingTimesteps*batch*ceil(numNeurons/32)] or NULL (runtime.cc:169) */
     /* further spike arrays that receive the same queue: the reference keeps one srcSpk per fused outgoing spike
      * owner and one trgSpk per incoming projection with learnPost (runtime.cc:267-278, "SynSpike" children) */
-    uint32_t numExtraSpk, pad_;
+    uint32_t numExtraSpk;
+    /* Axonal delay (backendBase.cc:128-162, neuronUpdateGroupMerged.cc:947-953): with numDelaySlots > 1 the queue is a ring
+     * of slots, slot-major within a batch; the step that follows k completed steps writes slot (k + 1) % numDelaySlots
+     * (the reference's spkQuePtr after its increment at the start of updateNeurons).  0 or 1: no delay. */
+    uint32_t numDelaySlots;
     uint32_t *extraSpkCnt[GENNMI_MAX_EXTRA_SPK];
     uint32_t *extraSpk[GENNMI_MAX_EXTRA_SPK];
 } gennmi_neuron_update_group_t;
@@ -161,7 +165,11 @@ typedef struct gennmi_presynaptic_update_group_t { /* MergedPresynapticUpdateGro
     int32_t conv[8];                      /* conv_kh, conv_kw, conv_ih, conv_iw, conv_ic, conv_oh, conv_ow, conv_oc */
     const uint32_t *gp;                   /* BITMASK: [ceil(numSrcNeurons*rowStride / 32)] connectivity words */
     float constantWeight;                 /* GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT: the parameter g (DENSE and BITMASK) */
-    uint32_t pad2_;
+    /* Axonal delay: the projection reads the source's slot (spkQuePtr + numSrcDelaySlots - axonalDelaySteps) %
+     * numSrcDelaySlots (backendBase.cc:207-216), i.e. the spikes emitted axonalDelaySteps + 1 steps before the step that
+     * delivers them.  numSrcDelaySlots must equal the source group's numDelaySlots (0 or 1: no ring). */
+    uint32_t axonalDelaySteps;
+    uint32_t numSrcDelaySlots, pad3_;
 } gennmi_presynaptic_update_group_t;
 
 typedef struct gennmi_postsynaptic_update_group_t { /* MergedPostsynapticUpdateGroup<i> */

@@ -72,7 +72,11 @@ typedef struct {
     /* fused WU pre / post trace variables (one each is all the configurations need) */
     float *preTrace, *postTrace; float preDecay, postDecay;
     float *sT;              /* spike times, allocated when a WU model reads st_pre / st_post */
-    uint32_t *spk, spkCnt;
+    uint32_t *spk, spkCnt;  /* the queue written by the last neuron update (slot spkQuePtr of the ring below, if there is one) */
+    /* axonal delay (backendBase.cc:128-162): ring of numDelaySlots queues, slot-major; spkQuePtr advances at the start of
+     * every neuron update (neuronUpdateGroupMerged.cc:947-953) */
+    uint32_t numDelaySlots, spkQuePtr;
+    uint32_t *spkRing, *spkCntRing;
     uint32_t *recordSpk;    /* [numRec * ceil(n/32)] or NULL */
 } gc_pop;
 
@@ -84,6 +88,7 @@ typedef struct {
     uint32_t *colLength, *remap;
     float aPlus, aMinus, wMin, wMax;
     int conv[8]; int conv_bh, conv_bw;
+    uint32_t delaySteps;    /* axonal delay in timesteps: reads slot (spkQuePtr + slots - delaySteps) % slots of the source */
     const uint32_t *gp;     /* BITMASK connectivity words */
     float constantWeight;   /* StaticPulseConstantWeight (weightUpdateModels.h:202-213): used when g is NULL */
     uint64_t events;        /* synaptic events processed so far (bookkeeping, not in the reference) */
@@ -136,6 +141,21 @@ int gc_add_pop(gc_net *net, int model, uint32_t n, const float *params, int numP
     if(net->numRec) { p->recordSpk = (uint32_t*)calloc(net->numRec * ((n + 31) / 32), sizeof(uint32_t)); }
     return net->numPops++;
 }
+
+/* numDelaySlots = longest axonal delay of the population's outgoing projections + 1 (neuronGroup.cc checkNumDelaySlots) */
+void gc_set_delay_slots(gc_net *net, int pop, uint32_t numDelaySlots)
+{
+    gc_pop *p = &net->pops[pop];
+    if(numDelaySlots > 1) {
+        p->numDelaySlots = numDelaySlots;
+        p->spkRing = (uint32_t*)calloc((size_t)numDelaySlots * (p->n ? p->n : 1), sizeof(uint32_t));
+        p->spkCntRing = (uint32_t*)calloc(numDelaySlots, sizeof(uint32_t));
+        free(p->spk);
+        p->spk = p->spkRing;
+    }
+}
+
+void gc_set_axonal_delay(gc_net *net, int syn, uint32_t delaySteps) { net->syns[syn].delaySteps = delaySteps; }
 
 int gc_add_psm(gc_net *net, int pop, int kind, float init, float expDecay, uint32_t maxDenDelay)
 {
@@ -264,6 +284,14 @@ void gc_update_synapses(gc_net *net, float t)
         gc_syn *s = &net->syns[k];
         const gc_pop *src = &net->pops[s->src];
         gc_pop *trg = &net->pops[s->trg];
+        /* axonal delay: slot (spkQuePtr + slots - delaySteps) % slots of the source's ring (backendBase.cc:207-216) */
+        const uint32_t *srcSpk = src->spk;
+        uint32_t srcSpkCnt = src->spkCnt;
+        if(src->numDelaySlots > 1) {
+            const uint32_t slot = (src->spkQuePtr + src->numDelaySlots - s->delaySteps) % src->numDelaySlots;
+            srcSpk = src->spkRing + (size_t)slot * src->n;
+            srcSpkCnt = src->spkCntRing[slot];
+        }
         gc_psm *psm = &trg->psm[s->psm];
         if(s->matrix == GC_CONV2D) {
             const int kh = s->conv[0], kw = s->conv[1], iw = s->conv[3], ic = s->conv[4];
@@ -275,8 +303,8 @@ void gc_update_synapses(gc_net *net, float t)
                 const int32_t kernOutChan = (int32_t)(j % oc);
                 const int32_t flipKernRow = kh - kernRow - 1;
                 const int32_t flipKernCol = kw - kernCol - 1;
-                for(uint32_t i = 0; i < src->spkCnt; i++) {
-                    const uint32_t ipre = src->spk[i];
+                for(uint32_t i = 0; i < srcSpkCnt; i++) {
+                    const uint32_t ipre = srcSpk[i];
                     const int32_t preRow = (int32_t)(ipre / ic) / iw;
                     const int32_t preCol = (int32_t)(ipre / ic) % iw;
                     const int32_t preChan = (int32_t)(ipre % ic);
@@ -294,8 +322,8 @@ void gc_update_synapses(gc_net *net, float t)
         }
         if(s->matrix == GC_DENSE || s->matrix == GC_BITMASK) {
             /* backend.cc:1985-2021: for every spike, every postsynaptic neuron in ascending order */
-            for(uint32_t i = 0; i < src->spkCnt; i++) {
-                const uint32_t idPre = src->spk[i];
+            for(uint32_t i = 0; i < srcSpkCnt; i++) {
+                const uint32_t idPre = srcSpk[i];
                 for(uint32_t ipost = 0; ipost < trg->n; ipost++) {
                     if(s->matrix == GC_BITMASK) {
                         const uint64_t gid = ((uint64_t)idPre * s->rowStride) + ipost;
@@ -313,8 +341,8 @@ void gc_update_synapses(gc_net *net, float t)
             }
             continue;
         }
-        for(uint32_t i = 0; i < src->spkCnt; i++) {
-            const uint32_t idPre = src->spk[i];
+        for(uint32_t i = 0; i < srcSpkCnt; i++) {
+            const uint32_t idPre = srcSpk[i];
             const uint32_t npost = s->rowLength[idPre];
             s->events += npost;
             for(uint32_t j = 0; j < npost; j++) {
@@ -366,7 +394,14 @@ void gc_update_synapses(gc_net *net, float t)
 void gc_update_neurons(gc_net *net, float t, uint32_t recordingTimestep)
 {
     const uint64_t step = net->timestep;
-    for(int k = 0; k < net->numPops; k++) { net->pops[k].spkCnt = 0; }
+    for(int k = 0; k < net->numPops; k++) {
+        gc_pop *p = &net->pops[k];
+        if(p->numDelaySlots > 1) {
+            p->spkQuePtr = (p->spkQuePtr + 1) % p->numDelaySlots;
+            p->spk = p->spkRing + (size_t)p->spkQuePtr * p->n;
+        }
+        p->spkCnt = 0;
+    }
     for(int k = 0; k < net->numPops; k++) {
         gc_pop *p = &net->pops[k];
         const uint32_t numRecordingWords = (p->n + 31) / 32;
@@ -448,6 +483,7 @@ void gc_update_neurons(gc_net *net, float t, uint32_t recordingTimestep)
             }
             p->v0[i] = l0; p->v1[i] = l1;
         }
+        if(p->numDelaySlots > 1) { p->spkCntRing[p->spkQuePtr] = p->spkCnt; }
     }
 }
 
@@ -491,7 +527,8 @@ void gc_destroy(gc_net *net)
         gc_pop *p = &net->pops[k];
         free(p->v0); free(p->v1); free(p->startSpike); free((void*)p->endSpike);
         for(int m = 0; m < p->numPSM; m++) { free(p->psm[m].outPost); free(p->psm[m].denDelay); }
-        free(p->preTrace); free(p->postTrace); free(p->sT); free(p->spk); free(p->recordSpk);
+        free(p->preTrace); free(p->postTrace); free(p->sT); free(p->recordSpk);
+        if(p->spkRing) { free(p->spkRing); free(p->spkCntRing); } else { free(p->spk); }
     }
     for(int k = 0; k < net->numSyns; k++) { free(net->syns[k].colLength); free(net->syns[k].remap); }
     free(net->pops); free(net->syns); free(net);

@@ -47,6 +47,8 @@ def lib():
         l.gc_add_syn_sparse.restype = i32; l.gc_add_syn_sparse.argtypes = [vp, i32, i32, i32, i32, u32, vp, vp, vp, vp, i32]
         l.gc_set_stdp_trace.restype = None; l.gc_set_stdp_trace.argtypes = [vp, i32, f32, f32, f32, f32, f32, f32, u32]
         l.gc_add_syn_conv2d.restype = i32; l.gc_add_syn_conv2d.argtypes = [vp, i32, i32, i32, vp, vp]
+        l.gc_set_delay_slots.restype = None; l.gc_set_delay_slots.argtypes = [vp, i32, u32]
+        l.gc_set_axonal_delay.restype = None; l.gc_set_axonal_delay.argtypes = [vp, i32, u32]
         l.gc_add_syn_dense.restype = i32; l.gc_add_syn_dense.argtypes = [vp, i32, i32, i32, vp, C.c_float]
         l.gc_add_syn_bitmask.restype = i32; l.gc_add_syn_bitmask.argtypes = [vp, i32, i32, i32, vp, u32, C.c_float]
         l.gc_build_remap.restype = None; l.gc_build_remap.argtypes = [vp, i32]
@@ -128,7 +130,8 @@ class OracleNet:
             psm = tuple((g[0][0], g[0][2]) for g in fused[p.name])
             pre = any(s.wum == "stdp_trace" for s in out_syn[p.name])
             post = any(s.wum == "stdp_trace" for s in in_syn[p.name])
-            return (p.model, psm, cs, pre, post)
+            slots = max([s.axonal_delay_steps for s in out_syn[p.name]], default=0) + 1
+            return (p.model, psm, cs, pre, post, slots)
 
         merged = {}
         for p in net.pops:
@@ -160,6 +163,12 @@ class OracleNet:
             pr = params[p.name]
             self.pop_id[p.name] = self.l.gc_add_pop(self.h, model, p.n, pr.ctypes.data if pr.size else None, pr.size,
                                                     v0.ctypes.data, v1.ctypes.data, stp)
+
+        # delay slots: longest axonal delay among a population's outgoing projections, plus one
+        for p in net.pops:
+            slots = max([s.axonal_delay_steps for s in out_syn[p.name]], default=0) + 1
+            if slots > 1:
+                self.l.gc_set_delay_slots(self.h, self.pop_id[p.name], slots)
 
         # postsynaptic-model children with merged-group rounding, matched by child index
         for members in merged.values():
@@ -230,6 +239,8 @@ class OracleNet:
                 self.keep += [conv, kern]
                 sid = self.l.gc_add_syn_conv2d(self.h, src, trg, self.psm_id[s.name], conv.ctypes.data, kern.ctypes.data)
             self.syn_id[s.name] = sid
+            if s.axonal_delay_steps:
+                self.l.gc_set_axonal_delay(self.h, sid, s.axonal_delay_steps)
 
     # ---- stepping and state -----------------------------------------------------------------
     def step(self):

@@ -119,7 +119,7 @@ struct CSSpec { std::string name, model, pop; std::vector<double> p; CurrentSour
 struct SynSpec
 {
     std::string name, matrix, src, trg, wum, psm;
-    unsigned int rowStride = 0, maxDenDelay = 0, tps = 1, colStride = 0;
+    unsigned int rowStride = 0, maxDenDelay = 0, tps = 1, colStride = 0, axonalDelay = 0;
     bool hintPre = false;
     std::vector<double> conv, wumP, psmP;
     SynapseGroup *sg = nullptr;
@@ -179,7 +179,7 @@ int main(int argc, char *argv[])
                     if(s.psm == "expcurr") { s.psmP.resize(1); ls >> s.psmP[0]; }
                     else if(s.psm != "deltacurr") throw std::runtime_error("psm " + s.psm);
                     std::string o;
-                    while(ls >> o) { if(o == "hint_pre") s.hintPre = true; else if(o == "tps") ls >> s.tps; else if(o == "col_stride") ls >> s.colStride; else throw std::runtime_error("opt " + o); }
+                    while(ls >> o) { if(o == "hint_pre") s.hintPre = true; else if(o == "tps") ls >> s.tps; else if(o == "col_stride") ls >> s.colStride; else if(o == "axonal_delay") ls >> s.axonalDelay; else throw std::runtime_error("opt " + o); }
                     syns.push_back(s);
                 }
                 else throw std::runtime_error("unknown key " + k);
@@ -259,6 +259,7 @@ int main(int argc, char *argv[])
                          {"conv_ic", (int)s.conv[4]}, {"conv_oh", (int)s.conv[5]}, {"conv_ow", (int)s.conv[6]}, {"conv_oc", (int)s.conv[7]}}));
             }
             if(s.maxDenDelay) s.sg->setMaxDendriticDelayTimesteps(s.maxDenDelay);
+            if(s.axonalDelay) s.sg->setAxonalDelaySteps(s.axonalDelay);
             if(s.hintPre) s.sg->setParallelismHint(SynapseGroup::ParallelismHint::PRESYNAPTIC);
             if(s.tps > 1) s.sg->setNumThreadsPerSpike(s.tps);
         }

@@ -24,9 +24,14 @@ def conv_small():
     return configs.conv_toeplitz(h=8, w=8, ic=2, oc=4, steps=100, w_sd=0.6, ioffset=0.4), 25
 
 
+def va_delay_small():
+    # axonal delays: E's ring has 4 slots (longest outgoing delay 3), I's has 6; IE reads the newest slot of a ring
+    return configs.vogels_abbott(n=400, steps=300, p=0.1, axonal_delays={"EE": 3, "EI": 1, "IE": 0, "II": 5}), 50
+
+
 def dense_small():
     return configs.dense_bitmask(), 25
 
 
-CASES = {"dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+CASES = {"va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
          "stdp_small": stdp_small, "conv_small": conv_small}

@@ -190,6 +190,31 @@ def test_toeplitz_batches_are_independent():
     model.unload()
 
 
+@pytest.mark.parametrize("span", ["POSTSYNAPTIC", "PRESYNAPTIC"])
+def test_axonal_delays(span):
+    """Balanced LIF network with axonal delays of 3, 1, 0 and 5 timesteps: the spike queue of a population is a ring of
+    slots (4 for E, 6 for I) and every projection reads the slot its delay selects.  One weight per outPost, so the whole
+    state must be identical to the oracle's, stepped one launch at a time and through graph replay."""
+    delays = {"EE": 3, "EI": 1, "IE": 0, "II": 5}
+    net = configs.vogels_abbott(n=2000, steps=600, p=0.04, axonal_delays=delays)
+    model, oracle, counts = run_side_by_side(net, check_every=100, exact=True, span=span)
+    assert counts["E"] > 300 and counts["I"] > 50
+    info = model.runner_info()
+    assert not info["resident_plan"] and not info["single_launch_step"]
+    # the same network through run(): graph replays of the two-launch step
+    replay = model_from_net(net, span=span)
+    replay.load(num_recording_timesteps=600)
+    replay.run(600)
+    replay.synchronize()
+    for p in net.pops:
+        for name in ("V", "RefracTime"):
+            assert np.array_equal(replay.neuron_populations[p.name].vars[name].pull_from_device(), model.neuron_populations[p.name].vars[name].pull_from_device())
+        assert np.array_equal(replay.neuron_populations[p.name].current_spikes[0], oracle.spikes(p.name))
+    assert replay.synaptic_event_count == model.synaptic_event_count == oracle.events()
+    replay.unload()
+    model.unload()
+
+
 @pytest.mark.parametrize("fuse", [False, True])
 def test_dense_and_bitmask_projections(fuse):
     """DENSE (individual and constant weights), BITMASK and constant-weight SPARSE projections in a recurrent LIF network
