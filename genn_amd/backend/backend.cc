@@ -248,18 +248,25 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
     CodeStream body(bodyStream);
     EnvironmentLibrary libEnv(body, StandardLibrary::getMathsFunctions());
 
+    // host-side advance of the spike-queue pointers of populations with axonal delay slots, run by updateNeurons()
+    std::ostringstream queueStream;
+    CodeStream queue(queueStream);
+
     body << "void gennmiBuildNeuronGroups()";
     {
         CodeStream::Scope b(body);
         EnvironmentExternal funcEnv(libEnv);
         modelMerged.genMergedNeuronUpdateGroups(
             *this, memorySpaces,
-            [this, &funcEnv, batchSize, scalar](auto &n)
+            [this, &funcEnv, &queue, batchSize, scalar](auto &n)
             {
                 const auto &arch = n.getArchetype();
                 const size_t numGroups = n.getGroups().size();
                 const unsigned int neuronModel = recogniseNeuron(arch.getModel(), arch.getName());
-                if(arch.isDelayRequired()) { unsupported("axonal or back-propagation delay on population '" + arch.getName() + "'"); }
+                // axonal delay slots: supported for populations whose spikes feed static projections only
+                if(arch.isDelayRequired() && (arch.isSpikeTimeRequired() || !n.getMergedOutSynWUMPreCodeGroups().empty() || !n.getMergedInSynWUMPostCodeGroups().empty())) {
+                    unsupported("delay slots together with plasticity on population '" + arch.getName() + "'");
+                }
                 if(arch.isSimRNGRequired()) { unsupported("random numbers in the update of population '" + arch.getName() + "'"); }
                 if(arch.isPrevSpikeTimeRequired()) { unsupported("previous spike times of population '" + arch.getName() + "'"); }
                 if(!n.getMergedSpikeEventGroups().empty()) { unsupported("spike-like events of population '" + arch.getName() + "'"); }
@@ -436,6 +443,18 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
                 else {
                     out << "d.numExtraSpk = " << (spikes.size() - 1) << "u;" << std::endl;
                 }
+                if(arch.isDelayRequired()) {
+                    if(spikes.size() > 1) { unsupported("delay slots with more than one spike array on population '" + arch.getName() + "'"); }
+                    out << "d.numDelaySlots = " << arch.getNumDelaySlots() << "u;" << std::endl;
+                    // the reference advances spkQuePtr at the start of its neuron update (neuronUpdateGroupMerged.cc:947-953);
+                    // the kernels derive the slot from the step count, the host copy is kept in step for whoever reads it
+                    queue << "for(unsigned int g = 0; g < " << numGroups << "; g++)";
+                    {
+                        CodeStream::Scope q(queue);
+                        queue << "const auto *group = &mergedNeuronUpdateGroup" << n.getIndex() << "[g];" << std::endl;
+                        queue << "*" << env["_spk_que_ptr"] << " = (*" << env["_spk_que_ptr"] << " + 1) % " << arch.getNumDelaySlots() << ";" << std::endl;
+                    }
+                }
                 if(arch.isSpikeTimeRequired()) { out << "d.sT = gennmiDev(" << env["_st"] << ");" << std::endl; }
                 if(arch.isSpikeRecordingEnabled()) { out << "d.recordSpk = gennmiDev(" << env["_record_spk"] << ");" << std::endl; }
                 out << "GENNMI_CHECK(gennmi_push_neuron_update_group(gennmiRunner, &d, nullptr));" << std::endl;
@@ -451,6 +470,7 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
     {
         CodeStream::Scope b(body);
         body << "gennmiEnsureFinalised();" << std::endl;
+        body << queueStream.str();
         body << "GENNMI_CHECK(gennmi_step(gennmiRunner, t, " << (model.isRecordingInUse() ? "recordingTimestep" : "0u") << "));" << std::endl;
     }
 
@@ -491,8 +511,9 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                 const auto &arch = s.getArchetype();
                 const auto *wum = arch.getWUInitialiser().getSnippet();
                 const unsigned int wumKind = recogniseWUM(wum, arch.getName());
-                if(arch.getAxonalDelaySteps() != 0 || arch.getSrcNeuronGroup()->isDelayRequired() || arch.getTrgNeuronGroup()->isDelayRequired()) {
-                    unsupported("axonal or back-propagation delay on projection '" + arch.getName() + "'");
+                const bool srcDelay = arch.getSrcNeuronGroup()->isDelayRequired();
+                if(arch.getBackPropDelaySteps() != 0 || (wumKind == GENNMI_WUM_STDP_TRACE && (srcDelay || arch.getTrgNeuronGroup()->isDelayRequired()))) {
+                    unsupported("back-propagation delay, or delay slots on a plastic projection ('" + arch.getName() + "')");
                 }
                 if(arch.isPreSpikeEventRequired() || arch.isPostSpikeEventRequired()) { unsupported("spike-like events on projection '" + arch.getName() + "'"); }
                 if(wumKind == GENNMI_WUM_STDP_TRACE && batchSize != 1) { unsupported("plastic weights with a batch size above 1"); }
@@ -559,6 +580,12 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                     << ", c[] = " << tableU32(counts([this](const SynapseGroupInternal &g){ return getSynapticMatrixRowStride(g); }))
                     << "; d.numSrcNeurons = a[g]; d.numTrgNeurons = b[g]; d.rowStride = c[g]; }" << std::endl;
                 out << "d.srcSpkCnt = gennmiDev(" << env["_src_spk_cnt"] << "); d.srcSpk = gennmiDev(" << env["_src_spk"] << ");" << std::endl;
+                if(srcDelay) {
+                    if(dense || bitmask) { unsupported("axonal delay on DENSE or BITMASK projection '" + arch.getName() + "'"); }
+                    out << "{ static const uint32_t a[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getAxonalDelaySteps(); }))
+                        << ", b[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getSrcNeuronGroup()->getNumDelaySlots(); }))
+                        << "; d.axonalDelaySteps = a[g]; d.numSrcDelaySlots = b[g]; }" << std::endl;
+                }
                 out << "d.outPost = gennmiDev(" << env["_out_post"] << ");" << std::endl;
                 if(constantWeight) {
                     out << "{ static const float v[] = " << table(values([](const SynapseGroupInternal &g){ return g.getWUInitialiser().getParams().at("g"); }), scalar)
