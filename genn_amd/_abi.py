@@ -14,7 +14,8 @@ NEURON_LIF, NEURON_IZHIKEVICH, NEURON_SPIKE_SOURCE_ARRAY = 0, 1, 2
 PSM_EXPCURR, PSM_DELTACURR = 0, 1
 CS_DC, CS_ARRAY = 0, 1
 WUM_STATIC_PULSE, WUM_STATIC_PULSE_DENDRITIC_DELAY, WUM_STDP_TRACE, WUM_STATIC_PULSE_CONSTANT_WEIGHT = 0, 1, 2, 3
-MATRIX_SPARSE, MATRIX_TOEPLITZ_CONV2D, MATRIX_DENSE, MATRIX_BITMASK = 0, 1, 2, 3
+MATRIX_SPARSE, MATRIX_TOEPLITZ_CONV2D, MATRIX_DENSE, MATRIX_BITMASK, MATRIX_PROCEDURAL = 0, 1, 2, 3, 4
+CONNECT_SNIPPETS = {"FixedProbability": 0, "FixedProbabilityNoAutapse": 1, "FixedNumberPostWithReplacement": 2}
 SPAN_AUTO, SPAN_POST, SPAN_PRE = 0, 1, 2
 
 LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
@@ -48,6 +49,12 @@ class NeuronUpdateGroup(C.Structure):
                 ("extraSpkCnt", p_u32 * MAX_EXTRA_SPK), ("extraSpk", p_u32 * MAX_EXTRA_SPK)]
 
 
+class Procedural(C.Structure):
+    _fields_ = [("seed", C.c_uint64), ("connectivity", C.c_uint32), ("connectivityStream", C.c_uint32), ("prob", C.c_double),
+                ("num", C.c_uint32), ("weightSnippet", C.c_uint32), ("weightStream", C.c_uint32), ("pad_", C.c_uint32),
+                ("weightParams", C.c_double * 4)]
+
+
 class PresynapticUpdateGroup(C.Structure):
     _fields_ = [("matrix", C.c_uint32), ("wum", C.c_uint32), ("span", C.c_uint32), ("numThreadsPerSpike", C.c_uint32),
                 ("numSrcNeurons", C.c_uint32), ("numTrgNeurons", C.c_uint32),
@@ -59,7 +66,7 @@ class PresynapticUpdateGroup(C.Structure):
                 ("aMinus", C.c_float), ("wMin", C.c_float), ("wMax", C.c_float),
                 ("conv", C.c_int32 * 8),
                 ("gp", p_u32), ("constantWeight", C.c_float), ("axonalDelaySteps", C.c_uint32),
-                ("numSrcDelaySlots", C.c_uint32), ("pad3_", C.c_uint32)]
+                ("numSrcDelaySlots", C.c_uint32), ("pad3_", C.c_uint32), ("procedural", Procedural)]
 
 
 class PostsynapticUpdateGroup(C.Structure):

@@ -31,6 +31,7 @@
 #include <vector>
 
 #include "genn_mi355x.h"
+#include "genn_mi355x_rows.h"
 
 namespace
 {
@@ -435,6 +436,61 @@ void presynapticDenseKernel(const DenseGroupDev * __restrict__ blocks, unsigned 
     }
     for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
     if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// ------------------------------------------------------------------------------------------------
+// PROCEDURAL connectivity (the reference's PostSpan/PreSpan procedural strategies, presynapticUpdateStrategySIMT.cc:391-560,
+// re-run the connectivity snippet with a per-row generator state).  Here a wavefront regenerates the row of a spiking
+// neuron with exactly the code and draws the initialisation kernels use (genn_mi355x_rows.h), so a procedural projection
+// behaves synapse for synapse like the stored matrix the same seed would have produced — without reading a byte of
+// connectivity: the only memory traffic of an event is its atomic.
+// ------------------------------------------------------------------------------------------------
+struct ProcGroupDev
+{
+    gennmi_presynaptic_update_group_t g;
+    uint32_t startBlock, numBlocks;
+    gennmi_rows::Stream connectivity, weight;
+    gennmi_rows::VarInit weightInit;
+    float probLogRecip;
+    uint32_t pad_;
+};
+
+__global__ __launch_bounds__(BLOCK)
+void presynapticProceduralKernel(const ProcGroupDev * __restrict__ blocks, unsigned long long *eventCounter)
+{
+    using namespace gennmi_rows;
+    const ProcGroupDev &G = blocks[blockIdx.x];
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const uint32_t lane = threadIdx.x & (WAVE - 1);
+    const uint32_t waveIdx = (blockIdx.x - G.startBlock) * (BLOCK / WAVE) + threadIdx.x / WAVE;
+    const uint32_t numWaves = G.numBlocks * (BLOCK / WAVE);
+    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
+    GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
+    const uint32_t rowStride = g.rowStride;
+    unsigned long long events = 0;
+    for(uint32_t s = waveIdx; s < numSpikes; s += numWaves) {
+        const uint32_t row = spk[s];
+        const unsigned long long firstElement = (unsigned long long)row * rowStride;
+        if(g.procedural.connectivity == GENNMI_CONNECT_FIXED_NUMBER_POST) {
+            const uint32_t n = min(g.procedural.num, rowStride);
+            fixedNumberPostRow(row, g.numTrgNeurons, n, G.connectivity, lane, [&](uint32_t k, const uint32_t post[4]) {
+                for(int i = 0; i < 4 && k + i < n; i++) { atomicAddF32(&outPost[post[i]], valueAt(G.weightInit, G.weight, firstElement + k + i)); }
+            });
+            if(lane == 0) { events += n; }
+        }
+        else {
+            const uint32_t total = fixedProbabilityRow(row, g.numTrgNeurons, G.probLogRecip,
+                                                       g.procedural.connectivity == GENNMI_CONNECT_FIXED_PROBABILITY_NO_AUTAPSE, G.connectivity, lane,
+                                                       [&](uint32_t k, uint32_t post) {
+                if(k < rowStride) { atomicAddF32(&outPost[post], valueAt(G.weightInit, G.weight, firstElement + k)); }
+            });
+            if(lane == 0) { events += min(total, rowStride); }
+        }
+    }
+    for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
+    if(lane == 0 && events) { atomicAdd(eventCounter, events); }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1666,6 +1722,7 @@ struct gennmi_runner
     hipStream_t stream = nullptr;
     std::vector<NeuronGroupDev> neuron; std::vector<PreGroupDev> pre; std::vector<PostGroupDev> post;
     std::vector<DenseGroupDev> dense; DenseGroupDev *dDense = nullptr; uint32_t denseBlocks = 0;
+    std::vector<ProcGroupDev> proc; ProcGroupDev *dProc = nullptr; uint32_t procBlocks = 0;
     NeuronGroupDev *dNeuron = nullptr; PreGroupDev *dPre = nullptr; PostGroupDev *dPost = nullptr;
     uint32_t neuronBlocks = 0, preBlocks = 0, postBlocks = 0;
     unsigned long long *dAgg = nullptr; uint32_t *dError = nullptr; unsigned long long *dEvents = nullptr;
@@ -1888,7 +1945,7 @@ int gennmi_runner_destroy(gennmi_runner *r)
     for(hipEvent_t e : r->marks) { if(e) { hipEventDestroy(e); } }
     for(void *q : r->owned) { hipFree(q); }
     hipFree(r->dTile); hipFree(r->dConvTile);
-    hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dDense); hipFree(r->dAgg); hipFree(r->dError); hipFree(r->dEvents); hipFree(r->dState);
+    hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dDense); hipFree(r->dProc); hipFree(r->dAgg); hipFree(r->dError); hipFree(r->dEvents); hipFree(r->dState);
     hipStreamDestroy(r->stream);
     delete r;
     return GENNMI_OK;
@@ -1938,6 +1995,31 @@ int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynap
     if(r->finalised) { return fail(GENNMI_ESTATE, "push_presynaptic_update_group: runner already finalised"); }
     if(!g->srcSpk || !g->srcSpkCnt || !g->outPost) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: required array missing"); }
     if(g->numSrcNeurons == 0 || g->numTrgNeurons == 0) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: empty population"); }
+    if(g->matrix == GENNMI_MATRIX_PROCEDURAL) {
+        const gennmi_procedural_t &q = g->procedural;
+        if(g->wum != GENNMI_WUM_STATIC_PULSE && g->wum != GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT) {
+            return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: PROCEDURAL supports StaticPulse and StaticPulseConstantWeight");
+        }
+        if(g->numSrcDelaySlots > 1 || g->axonalDelaySteps) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: axonal delay on a PROCEDURAL projection"); }
+        if(g->rowStride == 0 || g->numTrgNeurons > 0x7fffffffu) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: procedural row stride or target count out of range"); }
+        if(q.connectivity > GENNMI_CONNECT_FIXED_NUMBER_POST) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: unknown procedural connectivity"); }
+        if(q.connectivity != GENNMI_CONNECT_FIXED_NUMBER_POST && !(q.prob >= 0.0 && q.prob <= 1.0)) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: connection probability outside [0, 1]"); }
+        if(q.connectivity == GENNMI_CONNECT_FIXED_NUMBER_POST && q.num > g->rowStride) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: num exceeds rowStride"); }
+        if(q.weightSnippet > GENNMI_INIT_EXPONENTIAL) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: procedural weights support Constant, Uniform, Normal, NormalClipped and Exponential"); }
+        ProcGroupDev pd;
+        memset(&pd, 0, sizeof(pd));
+        pd.g = *g;
+        pd.g.maxDenDelay = 0;
+        pd.connectivity = gennmi_rows::Stream{(uint32_t)q.seed, (uint32_t)(q.seed >> 32), q.connectivityStream};
+        pd.weight = gennmi_rows::Stream{(uint32_t)q.seed, (uint32_t)(q.seed >> 32), q.weightStream};
+        pd.weightInit.snippet = (g->wum == GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT) ? (uint32_t)GENNMI_INIT_CONSTANT : q.weightSnippet;
+        for(int k = 0; k < 4; k++) { pd.weightInit.p[k] = (float)q.weightParams[k]; }
+        if(g->wum == GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT) { pd.weightInit.p[0] = g->constantWeight; }
+        pd.probLogRecip = (q.prob == 0.0) ? -INFINITY : (float)(1.0 / std::log(1.0 - q.prob));
+        if(idx) { *idx = (uint32_t)(r->pre.size() + r->dense.size() + r->proc.size()); }
+        r->proc.push_back(pd);
+        return GENNMI_OK;
+    }
     if(g->matrix == GENNMI_MATRIX_DENSE || g->matrix == GENNMI_MATRIX_BITMASK) {
         const bool constant = (g->wum == GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT);
         if(g->matrix == GENNMI_MATRIX_DENSE) {
@@ -2024,7 +2106,7 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
 {
     const char *env = getenv("GENNMI_RESIDENT");
     if(env && atoi(env) == 0) { return GENNMI_OK; }
-    if(r->batch != 1 || !r->post.empty() || r->pre.empty() || !r->dense.empty() || r->neuron.size() > RES_MAX_GROUPS) { return GENNMI_OK; }
+    if(r->batch != 1 || !r->post.empty() || r->pre.empty() || !r->dense.empty() || !r->proc.empty() || r->neuron.size() > RES_MAX_GROUPS) { return GENNMI_OK; }
     for(const auto &n : r->neuron) {
         const auto &g = n.g;
         if((g.model != GENNMI_NEURON_LIF && g.model != GENNMI_NEURON_IZHIKEVICH) || g.preTrace || g.postTrace || g.sT || g.numDelaySlots > 1) { return GENNMI_OK; }
@@ -2273,6 +2355,16 @@ int gennmi_runner_finalise(gennmi_runner *r)
     }
     r->denseBlocks = block;
 
+    // PROCEDURAL projections: a wavefront per spike; enough wavefronts for ~1.5 % of the source population firing at once
+    block = 0;
+    for(auto &p : r->proc) {
+        const uint32_t wantWaves = std::max(8u, p.g.numSrcNeurons / 64);
+        p.startBlock = block;
+        p.numBlocks = std::max(1u, std::min((wantWaves + (BLOCK / WAVE) - 1) / (BLOCK / WAVE), 8u * numCU / std::max<uint32_t>(1, (uint32_t)r->proc.size())));
+        block += p.numBlocks;
+    }
+    r->procBlocks = block;
+
     // One descriptor copy per block, indexed by blockIdx.x: a block finds everything it needs with a
     // single round of scalar loads (the reference bisects a start-ID table and then loads the merged
     // struct, backendSIMT.h:244-323 — two to four dependent loads before any work starts).
@@ -2382,7 +2474,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
     // ---- single-launch step: possible when every projection is a SPARSE dendritic-delay one with ring depth >= 2
     // and nothing is plastic
     const char *envFused = getenv("GENNMI_FUSED_STEP");
-    bool eligible = !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty() && r->dense.empty();
+    bool eligible = !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty() && r->dense.empty() && r->proc.empty();
     for(const auto &p : r->pre) {
         eligible = eligible && p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY
                    && p.g.maxDenDelay >= 2 && p.g.numSrcDelaySlots <= 1;
@@ -2469,6 +2561,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
     HIP_TRY(uploadPerBlock(r->pre, r->preBlocks, &r->dPre));
     HIP_TRY(uploadPerBlock(r->post, r->postBlocks, &r->dPost));
     HIP_TRY(uploadPerBlock(r->dense, r->denseBlocks, &r->dDense));
+    HIP_TRY(uploadPerBlock(r->proc, r->procBlocks, &r->dProc));
     const size_t aggCount = 2 * (size_t)r->neuronBlocks * r->batch;       // per-block counts, then per-group totals
     HIP_TRY(hipMalloc(&r->dAgg, aggCount * sizeof(unsigned long long)));
     HIP_TRY(hipMemset(r->dAgg, 0, aggCount * sizeof(unsigned long long)));
@@ -2525,7 +2618,10 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
         if(r->pending.size() >= 2048) { const int rc = drainTimers(r); if(rc) { return rc; } }
         const int rc = stamp(r, &e0); if(rc) { return rc; }
     }
-    if(!r->pre.empty() || r->denseBlocks) {
+    if(!r->pre.empty() || r->denseBlocks || r->procBlocks) {
+        if(r->procBlocks) {
+            presynapticProceduralKernel<<<dim3(r->procBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dProc, r->dEvents);
+        }
         if(r->preBlocks) {
             presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dPre, a, r->dt, r->dEvents);
         }

@@ -25,6 +25,7 @@
 #include <string>
 
 #include "genn_mi355x.h"
+#include "genn_mi355x_rows.h"
 
 namespace gennmi_detail
 {
@@ -34,7 +35,7 @@ void noteDeviceWrite(const void *dev, size_t bytes);     // lets runners that ho
 
 namespace
 {
-constexpr int WAVE = 64;
+using namespace gennmi_rows;
 constexpr int BLOCK = 256;
 
 #define HIP_TRY(expr)                                                                                          \
@@ -44,53 +45,6 @@ constexpr int BLOCK = 256;
             return gennmi_detail::fail(GENNMI_EHIP, std::string(#expr) + ": " + hipGetErrorString(e_));       \
         }                                                                                                      \
     } while(0)
-
-// Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11)
-struct Words { uint32_t w[4]; };
-
-__host__ __device__ inline uint32_t mulHi(uint32_t a, uint32_t b) { return (uint32_t)(((unsigned long long)a * b) >> 32); }
-
-__host__ __device__ inline Words philox4x32(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1)
-{
-    #pragma unroll
-    for(int round = 0; round < 10; round++) {
-        const uint32_t hi0 = mulHi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
-        const uint32_t hi1 = mulHi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
-        c0 = hi1 ^ c1 ^ k0;
-        c1 = lo1;
-        c2 = hi0 ^ c3 ^ k1;
-        c3 = lo0;
-        k0 += 0x9E3779B9u;
-        k1 += 0xBB67AE85u;
-    }
-    return Words{{c0, c1, c2, c3}};
-}
-
-// A stream of draws: key = the 64-bit seed, counter = (index low, index high, sub-counter, stream number).
-struct Stream
-{
-    uint32_t k0, k1, stream;
-    __host__ __device__ Words at(unsigned long long index, uint32_t sub) const
-    {
-        return philox4x32((uint32_t)index, (uint32_t)(index >> 32), sub, stream, k0, k1);
-    }
-};
-
-__device__ __forceinline__ float uniformHalfOpen(uint32_t x) { return (float)(x >> 8) * (1.0f / 16777216.0f); }              // [0, 1)
-__device__ __forceinline__ float uniformOpen(uint32_t x) { return ((float)(x >> 8) + 0.5f) * (1.0f / 16777216.0f); }         // (0, 1)
-
-// four standard normals from four words (Box-Muller, both branches)
-__device__ __forceinline__ void normals(const Words &r, float n[4])
-{
-    #pragma unroll
-    for(int p = 0; p < 2; p++) {
-        const float radius = sqrtf(-2.0f * logf(uniformOpen(r.w[2 * p])));
-        float s, c;
-        sincospif(2.0f * uniformHalfOpen(r.w[2 * p + 1]), &s, &c);
-        n[2 * p] = radius * c;
-        n[2 * p + 1] = radius * s;
-    }
-}
 
 template<typename T> struct Quad;
 template<> struct Quad<float> { typedef float4 type; };
@@ -152,37 +106,6 @@ __device__ uint32_t binomialDraw(const Stream &s, unsigned long long element, ui
     return flip ? n - total : total;
 }
 
-struct VarInit { uint32_t snippet; float p[4]; double p64[2]; };
-
-// value of element `e` whose group of four shares the Philox call `r` (attempt 0); slot = e % 4
-__device__ __forceinline__ float drawValue(const VarInit &v, const Stream &s, unsigned long long group, int slot, const Words &r, const float n[4])
-{
-    switch(v.snippet) {
-    case GENNMI_INIT_CONSTANT:
-        return v.p[0];
-    case GENNMI_INIT_UNIFORM: {
-        const float scale = v.p[1] - v.p[0];
-        return v.p[0] + (uniformHalfOpen(r.w[slot]) * scale);
-    }
-    case GENNMI_INIT_NORMAL:
-        return v.p[0] + (n[slot] * v.p[1]);
-    case GENNMI_INIT_NORMAL_CLIPPED:
-    case GENNMI_INIT_NORMAL_CLIPPED_DELAY: {
-        float value = v.p[0] + (n[slot] * v.p[1]);
-        for(uint32_t attempt = 1; value > v.p[3] || value < v.p[2]; attempt++) {
-            float retry[4];
-            normals(s.at(group, attempt), retry);
-            value = v.p[0] + (retry[slot] * v.p[1]);
-        }
-        return (v.snippet == GENNMI_INIT_NORMAL_CLIPPED_DELAY) ? rintf(value) : value;
-    }
-    case GENNMI_INIT_EXPONENTIAL:
-        return v.p[0] * -logf(uniformOpen(r.w[slot]));
-    default:
-        return 0.0f;
-    }
-}
-
 template<typename T>
 __global__ __launch_bounds__(BLOCK)
 void initVarKernel(T *out, unsigned long long count, VarInit v, Stream s)
@@ -230,78 +153,32 @@ void randomWordsKernel(uint32_t *out, unsigned long long count, Stream s)
     }
 }
 
-// ---- wave64 scans
-__device__ __forceinline__ uint32_t waveInclusiveScan(uint32_t v, int lane)
-{
-    #pragma unroll
-    for(int d = 1; d < WAVE; d <<= 1) {
-        const uint32_t o = __shfl_up(v, d, WAVE);
-        if(lane >= d) { v += o; }
-    }
-    return v;
-}
-__device__ __forceinline__ double waveInclusiveScan(double v, int lane)
-{
-    #pragma unroll
-    for(int d = 1; d < WAVE; d <<= 1) {
-        const double o = __shfl_up(v, d, WAVE);
-        if(lane >= d) { v += o; }
-    }
-    return v;
-}
-
 __device__ uint32_t g_rowOverflow;      // rows that wanted more entries than rowStride, last connectivity launch
 
-// FixedProbability / FixedProbabilityNoAutapse (initSparseConnectivitySnippet.h:170-187, 208-230): one row per wave64.
-// Lane l owns post indices [l*slice, (l+1)*slice) and walks them with the snippet's geometric skips
-// `prev += 1 + (int)(log(u) * probLogRecip)`; the walk is memoryless, so restarting it at a slice boundary, or
-// stepping over the diagonal without emitting (the snippet redraws instead), leaves the distribution unchanged.
+// FixedProbability / FixedProbabilityNoAutapse: one row per wave64, generated by fixedProbabilityRow() and stored
 __global__ __launch_bounds__(BLOCK)
 void fixedProbabilityKernel(uint32_t numPre, uint32_t numPost, uint32_t rowStride, float probLogRecip, int noAutapse, Stream s,
                             uint32_t *rowLength, uint32_t *ind)
 {
-    const int lane = threadIdx.x & (WAVE - 1);
+    const uint32_t lane = threadIdx.x & (WAVE - 1);
     const uint32_t row = blockIdx.x * (BLOCK / WAVE) + threadIdx.x / WAVE;
     if(row >= numPre) { return; }
-    const uint32_t slice = (numPost + WAVE - 1) / WAVE;
-    const uint32_t begin = min(numPost, (uint32_t)lane * slice), end = min(numPost, begin + slice);
-    uint32_t offset = 0;
-    for(int pass = 0; pass < 2; pass++) {
-        uint32_t count = 0, draw = 0;
-        long long j = (long long)begin - 1;
-        Words r;
-        while(true) {
-            if((draw & 3u) == 0) { r = s.at(((unsigned long long)row << 32) | (draw >> 2), (uint32_t)lane); }
-            const float skip = logf(uniformOpen(r.w[draw & 3u])) * probLogRecip;
-            draw++;
-            if(skip >= (float)(end - begin)) { break; }
-            j += 1 + (int)skip;
-            if(j >= (long long)end) { break; }
-            if(noAutapse && j == (long long)row) { continue; }
-            if(pass == 1 && offset + count < rowStride) { ind[(size_t)row * rowStride + offset + count] = (uint32_t)j; }
-            count++;
-        }
-        if(pass == 0) {
-            const uint32_t inclusive = waveInclusiveScan(count, lane);
-            offset = inclusive - count;
-            const uint32_t total = __shfl(inclusive, WAVE - 1, WAVE);
-            if(lane == 0) {
-                rowLength[row] = min(total, rowStride);
-                if(total > rowStride) { atomicAdd(&g_rowOverflow, 1u); }
-            }
-        }
+    uint32_t *rowInd = ind + (size_t)row * rowStride;
+    const uint32_t total = fixedProbabilityRow(row, numPost, probLogRecip, noAutapse != 0, s, lane,
+                                               [&](uint32_t k, uint32_t post) { if(k < rowStride) { rowInd[k] = post; } });
+    if(lane == 0) {
+        rowLength[row] = min(total, rowStride);
+        if(total > rowStride) { atomicAdd(&g_rowOverflow, 1u); }
     }
 }
 
-// FixedNumberPostWithReplacement / FixedNumberTotalWithReplacement (initSparseConnectivitySnippet.h:242-276, 292-370): one row
-// per wave64.  The snippet's loop `x += (1 - x) * (1 - pow(u, 1/c))` for c = n..1 draws the n order statistics of n uniforms in
-// ascending order.  The same joint law is S_k / S_{n+1} with S the prefix sums of n+1 unit exponentials, which a wave computes
-// 256 draws at a time with a scan: first the total, then — regenerating the same draws — the normalised prefix sums.
+// FixedNumberPostWithReplacement / FixedNumberTotalWithReplacement: one row per wave64, generated by fixedNumberPostRow() and
+// stored 1 KiB of the row at a time
 __global__ __launch_bounds__(BLOCK)
 void fixedNumberPostKernel(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t num, const uint32_t *rowLengthIn, Stream s,
                            uint32_t *rowLength, uint32_t *ind)
 {
-    const int lane = threadIdx.x & (WAVE - 1);
+    const uint32_t lane = threadIdx.x & (WAVE - 1);
     const uint32_t row = blockIdx.x * (BLOCK / WAVE) + threadIdx.x / WAVE;
     if(row >= numPre) { return; }
     uint32_t n = rowLengthIn ? rowLengthIn[row] : num;
@@ -309,40 +186,16 @@ void fixedNumberPostKernel(uint32_t numPre, uint32_t numPost, uint32_t rowStride
         if(lane == 0) { atomicAdd(&g_rowOverflow, 1u); }
         n = rowStride;
     }
-    // draws 0..n: spacing k ends at target k; spacing n is the gap between the largest target and 1.  A lane takes the four
-    // draws of one generator call, so a wave covers 256 draws per round and stores 1 KiB of the row at a time.
     uint32_t *rowInd = ind + (size_t)row * rowStride;
     const bool vectorStores = ((rowStride & 3u) == 0) && (((uintptr_t)ind & 15u) == 0);
-    double scale = 0.0;
-    for(int pass = 0; pass < 2; pass++) {
-        double carry = 0.0;
-        for(uint32_t base = 0; base <= n; base += 4 * WAVE) {
-            const uint32_t k = base + 4 * lane;
-            const Words r = s.at(((unsigned long long)row << 32) | (k >> 2), 0);
-            double prefix[4];
-            double sum = 0.0;
-            #pragma unroll
-            for(int i = 0; i < 4; i++) {
-                sum += (k + i <= n) ? (double)-logf(uniformOpen(r.w[i])) : 0.0;
-                prefix[i] = sum;
-            }
-            const double inclusive = waveInclusiveScan(sum, lane);
-            const double before = carry + (inclusive - sum);
-            if(pass == 1 && k < n) {
-                uint32_t post[4];
-                #pragma unroll
-                for(int i = 0; i < 4; i++) { post[i] = min((uint32_t)((before + prefix[i]) * scale), numPost - 1); }
-                if(vectorStores && k + 3 < n) {
-                    *reinterpret_cast<uint4*>(rowInd + k) = make_uint4(post[0], post[1], post[2], post[3]);
-                }
-                else {
-                    for(int i = 0; i < 4 && k + i < n; i++) { rowInd[k + i] = post[i]; }
-                }
-            }
-            carry += __shfl(inclusive, WAVE - 1, WAVE);
+    fixedNumberPostRow(row, numPost, n, s, lane, [&](uint32_t k, const uint32_t post[4]) {
+        if(vectorStores && k + 3 < n) {
+            *reinterpret_cast<uint4*>(rowInd + k) = make_uint4(post[0], post[1], post[2], post[3]);
         }
-        scale = (double)numPost / carry;
-    }
+        else {
+            for(int i = 0; i < 4 && k + i < n; i++) { rowInd[k + i] = post[i]; }
+        }
+    });
     if(lane == 0) { rowLength[row] = n; }
 }
 

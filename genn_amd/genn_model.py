@@ -279,6 +279,7 @@ class SynapseGroup:
         self.ind_host = None
         self.var_host = {}
         self.gp_host = None
+        self.procedural_streams = None
         self.fused_ps_target = self
 
     # pygenn/genn_groups.py:434-470
@@ -389,8 +390,14 @@ class GeNNModel:
 
     def add_synapse_population(self, pop_name, matrix_type, source, target, weight_update_init, postsynaptic_init,
                                connectivity_init=None):
-        if matrix_type not in ("SPARSE", "TOEPLITZ", "DENSE", "BITMASK"):
+        if matrix_type not in ("SPARSE", "TOEPLITZ", "DENSE", "BITMASK", "PROCEDURAL"):
             raise NotImplementedError(f"matrix type {matrix_type}")
+        if matrix_type == "PROCEDURAL":
+            if connectivity_init is None or connectivity_init.snippet not in _abi.CONNECT_SNIPPETS:
+                raise NotImplementedError("PROCEDURAL connectivity needs init_sparse_connectivity with FixedProbability, "
+                                          "FixedProbabilityNoAutapse or FixedNumberPostWithReplacement")
+            if weight_update_init.snippet not in ("StaticPulse", "StaticPulseConstantWeight"):
+                raise NotImplementedError(f"PROCEDURAL connectivity with {weight_update_init.snippet}")
         if matrix_type == "BITMASK" and weight_update_init.snippet != "StaticPulseConstantWeight":
             raise ValueError("BITMASK connectivity has no per-synapse variables: use StaticPulseConstantWeight")
         if matrix_type == "DENSE" and weight_update_init.snippet not in ("StaticPulse", "StaticPulseConstantWeight"):
@@ -555,6 +562,12 @@ class GeNNModel:
                         a.view[:] = dtype(s.wu.vars[name])
                     a.push_to_device()
                     s.vars[name] = a
+            elif s.matrix_type == "PROCEDURAL":
+                # nothing is stored: the generator streams the stored matrix would have used are reserved in the same order
+                s.row_stride = max_row_length(s.conn.snippet, s.conn.params, s.src.num_neurons, s.trg.num_neurons)
+                s.procedural_streams = [self._next_stream(), 0]
+                if s.wu.snippet == "StaticPulse" and isinstance(s.wu.vars["g"], VarInit):
+                    s.procedural_streams[1] = self._next_stream()
             elif s.matrix_type == "DENSE":
                 if s.wu.snippet == "StaticPulse":
                     count = s.src.num_neurons * s.trg.num_neurons
@@ -738,7 +751,7 @@ class GeNNModel:
             for k, s in enumerate(members):
                 d = _abi.PresynapticUpdateGroup()
                 d.matrix = {"SPARSE": _abi.MATRIX_SPARSE, "TOEPLITZ": _abi.MATRIX_TOEPLITZ_CONV2D, "DENSE": _abi.MATRIX_DENSE,
-                            "BITMASK": _abi.MATRIX_BITMASK}[s.matrix_type]
+                            "BITMASK": _abi.MATRIX_BITMASK, "PROCEDURAL": _abi.MATRIX_PROCEDURAL}[s.matrix_type]
                 d.wum = {"StaticPulse": _abi.WUM_STATIC_PULSE, "StaticPulseDendriticDelay": _abi.WUM_STATIC_PULSE_DENDRITIC_DELAY,
                          "STDPTrace": _abi.WUM_STDP_TRACE, "StaticPulseConstantWeight": _abi.WUM_STATIC_PULSE_CONSTANT_WEIGHT}[s.wu.snippet]
                 if s.wu.snippet == "StaticPulseConstantWeight":
@@ -757,7 +770,24 @@ class GeNNModel:
                 if s.matrix_type == "BITMASK":
                     d.rowStride = s.row_stride
                     d.gp = s.vars["gp"].ptr
-                if s.matrix_type in ("DENSE", "BITMASK"):
+                if s.matrix_type == "PROCEDURAL":
+                    d.rowStride = s.row_stride
+                    q = d.procedural
+                    q.seed = self.seed
+                    q.connectivity = _abi.CONNECT_SNIPPETS[s.conn.snippet]
+                    q.connectivityStream, q.weightStream = s.procedural_streams
+                    q.prob = float(s.conn.params.get("prob", 0.0))
+                    q.num = int(s.conn.params.get("num", 0))
+                    if s.wu.snippet == "StaticPulse":
+                        init = s.wu.vars["g"]
+                        if isinstance(init, VarInit):
+                            q.weightSnippet = _abi.INIT_SNIPPETS[init.snippet]
+                            for j, v in enumerate(init.values(self.dt)):
+                                q.weightParams[j] = v
+                        else:
+                            q.weightSnippet = _abi.INIT_SNIPPETS["Constant"]
+                            q.weightParams[0] = float(init)
+                if s.matrix_type in ("DENSE", "BITMASK", "PROCEDURAL"):
                     pass
                 elif s.matrix_type == "SPARSE":
                     d.rowStride = s.row_stride

@@ -51,7 +51,11 @@ enum { GENNMI_MATRIX_SPARSE = 0, GENNMI_MATRIX_TOEPLITZ_CONV2D = 1,
        /* DENSE: g[numSrc*numTrg], idSyn = idPre*numTrg + idPost; BITMASK: one bit per pair, most significant bit first,
         * gid = idPre*rowStride + idPost with rowStride = numTrg padded to 32 (single_threaded_cpu/backend.cc:1393-1404,
         * 1985-2021; runtime.cc:340-357) */
-       GENNMI_MATRIX_DENSE = 2, GENNMI_MATRIX_BITMASK = 3 };
+       GENNMI_MATRIX_DENSE = 2, GENNMI_MATRIX_BITMASK = 3,
+       /* PROCEDURAL (synapseMatrixType.h:60-66; presynapticUpdateStrategySIMT.cc:391-560): nothing is stored, the row of a
+        * spiking neuron — and its weights — are regenerated from the initialisation snippets' generator when needed */
+       GENNMI_MATRIX_PROCEDURAL = 4 };
+enum { GENNMI_CONNECT_FIXED_PROBABILITY = 0, GENNMI_CONNECT_FIXED_PROBABILITY_NO_AUTAPSE = 1, GENNMI_CONNECT_FIXED_NUMBER_POST = 2 };
 /* presynaptic strategies: presynapticUpdateStrategySIMT.cc:57-162 (PreSpan), :167-389 (PostSpan) */
 enum { GENNMI_SPAN_AUTO = 0, GENNMI_SPAN_POST = 1, GENNMI_SPAN_PRE = 2 };
 
@@ -143,6 +147,20 @@ typedef struct gennmi_neuron_update_group_t {      /* MergedNeuronUpdateGroup<i>
     uint32_t *extraSpk[GENNMI_MAX_EXTRA_SPK];
 } gennmi_neuron_update_group_t;
 
+/* What gennmi_init_sparse_* and gennmi_init_var would have stored for a projection, for GENNMI_MATRIX_PROCEDURAL: the row
+ * of presynaptic neuron r is row r of that connectivity call (same seed and stream), truncated to rowStride entries, and
+ * the weight of its k-th synapse is element r*rowStride + k of that gennmi_init_var call. */
+typedef struct gennmi_procedural_t {
+    uint64_t seed;
+    uint32_t connectivity;                /* GENNMI_CONNECT_* */
+    uint32_t connectivityStream;
+    double prob;                          /* FixedProbability[NoAutapse] */
+    uint32_t num;                         /* FixedNumberPostWithReplacement */
+    uint32_t weightSnippet;               /* GENNMI_INIT_CONSTANT .. GENNMI_INIT_EXPONENTIAL */
+    uint32_t weightStream, pad_;
+    double weightParams[4];
+} gennmi_procedural_t;
+
 typedef struct gennmi_presynaptic_update_group_t { /* MergedPresynapticUpdateGroup<i> */
     uint32_t matrix;                      /* GENNMI_MATRIX_* */
     uint32_t wum;                         /* GENNMI_WUM_* */
@@ -170,6 +188,7 @@ typedef struct gennmi_presynaptic_update_group_t { /* MergedPresynapticUpdateGro
      * delivers them.  numSrcDelaySlots must equal the source group's numDelaySlots (0 or 1: no ring). */
     uint32_t axonalDelaySteps;
     uint32_t numSrcDelaySlots, pad3_;
+    gennmi_procedural_t procedural;       /* GENNMI_MATRIX_PROCEDURAL only (rowStride = the stride the stored matrix would have) */
 } gennmi_presynaptic_update_group_t;
 
 typedef struct gennmi_postsynaptic_update_group_t { /* MergedPostsynapticUpdateGroup<i> */
