@@ -9,11 +9,12 @@ import os
 MAX_PSM = 8
 MAX_CS = 4
 MAX_EXTRA_SPK = 3
+MAX_SPK_EVENT = 2
 
 NEURON_LIF, NEURON_IZHIKEVICH, NEURON_SPIKE_SOURCE_ARRAY = 0, 1, 2
 PSM_EXPCURR, PSM_DELTACURR = 0, 1
 CS_DC, CS_ARRAY = 0, 1
-WUM_STATIC_PULSE, WUM_STATIC_PULSE_DENDRITIC_DELAY, WUM_STDP_TRACE, WUM_STATIC_PULSE_CONSTANT_WEIGHT = 0, 1, 2, 3
+WUM_STATIC_PULSE, WUM_STATIC_PULSE_DENDRITIC_DELAY, WUM_STDP_TRACE, WUM_STATIC_PULSE_CONSTANT_WEIGHT, WUM_STATIC_GRADED = 0, 1, 2, 3, 4
 MATRIX_SPARSE, MATRIX_TOEPLITZ_CONV2D, MATRIX_DENSE, MATRIX_BITMASK, MATRIX_PROCEDURAL = 0, 1, 2, 3, 4
 CONNECT_SNIPPETS = {"FixedProbability": 0, "FixedProbabilityNoAutapse": 1, "FixedNumberPostWithReplacement": 2}
 SPAN_AUTO, SPAN_POST, SPAN_PRE = 0, 1, 2
@@ -35,6 +36,10 @@ class Cs(C.Structure):
     _fields_ = [("array", p_f32), ("amp", C.c_float), ("kind", C.c_uint32), ("arraySteps", C.c_uint32), ("pad_", C.c_uint32)]
 
 
+class SpikeEvent(C.Structure):
+    _fields_ = [("spkCntEvent", p_u32), ("spkEvent", p_u32), ("threshold", C.c_float), ("pad_", C.c_uint32)]
+
+
 class NeuronUpdateGroup(C.Structure):
     _fields_ = [("model", C.c_uint32), ("numNeurons", C.c_uint32),
                 ("var0", p_f32), ("var1", p_f32),
@@ -46,7 +51,8 @@ class NeuronUpdateGroup(C.Structure):
                 ("preDecay", C.c_float), ("postDecay", C.c_float),
                 ("sT", p_f32), ("spkCnt", p_u32), ("spk", p_u32), ("recordSpk", p_u32),
                 ("numExtraSpk", C.c_uint32), ("numDelaySlots", C.c_uint32),
-                ("extraSpkCnt", p_u32 * MAX_EXTRA_SPK), ("extraSpk", p_u32 * MAX_EXTRA_SPK)]
+                ("extraSpkCnt", p_u32 * MAX_EXTRA_SPK), ("extraSpk", p_u32 * MAX_EXTRA_SPK),
+                ("numSpkEvent", C.c_uint32), ("pad2_", C.c_uint32), ("spkEvent", SpikeEvent * MAX_SPK_EVENT)]
 
 
 class Procedural(C.Structure):
@@ -66,7 +72,8 @@ class PresynapticUpdateGroup(C.Structure):
                 ("aMinus", C.c_float), ("wMin", C.c_float), ("wMax", C.c_float),
                 ("conv", C.c_int32 * 8),
                 ("gp", p_u32), ("constantWeight", C.c_float), ("axonalDelaySteps", C.c_uint32),
-                ("numSrcDelaySlots", C.c_uint32), ("pad3_", C.c_uint32), ("procedural", Procedural)]
+                ("numSrcDelaySlots", C.c_uint32), ("pad3_", C.c_uint32), ("procedural", Procedural),
+                ("srcV", p_f32), ("gradedEpre", C.c_float), ("gradedVslope", C.c_float)]
 
 
 class PostsynapticUpdateGroup(C.Structure):

@@ -170,6 +170,28 @@ bool isTraceSTDP(const WeightUpdateModels::Base *m)
         && same(m->getPreDynamicsCode(), "preTrace *= tauPlusDecay;") && same(m->getPostDynamicsCode(), "postTrace *= tauMinusDecay;")
         && m->getSynapseDynamicsCode().empty() && m->getPreEventSynCode().empty() && m->getPostEventSynCode().empty();
 }
+// StaticGraded (weightUpdateModels.h:308-319): spike-like events while V > Epre, each adding
+// fmax(0, g * tanh((V_pre - Epre) / Vslope) * dt).  The built-in's event code spells the presynaptic potential `V_pre`;
+// a model with the same code that spells it `V` — the name the 5.4.0 generator gives a presynaptic neuron variable
+// reference in synapse code — is the same model.
+bool isStaticGraded(const WeightUpdateModels::Base *m)
+{
+    const auto *builtin = WeightUpdateModels::StaticGraded::getInstance();
+    auto respelt = [](std::string code)
+    {
+        for(size_t at = code.find("V_pre"); at != std::string::npos; at = code.find("V_pre", at)) { code.replace(at, 5, "V"); }
+        return code;
+    };
+    const bool onlyEvents = m->getPreSpikeSynCode().empty() && m->getPostSpikeSynCode().empty() && m->getSynapseDynamicsCode().empty()
+                            && m->getPostEventSynCode().empty() && m->getPreSpikeCode().empty() && m->getPostSpikeCode().empty()
+                            && m->getPreDynamicsCode().empty() && m->getPostDynamicsCode().empty() && m->getPostEventThresholdConditionCode().empty();
+    const auto refs = m->getPreNeuronVarRefs();
+    return onlyEvents && same(m->getPreEventThresholdConditionCode(), builtin->getPreEventThresholdConditionCode())
+           && (same(m->getPreEventSynCode(), builtin->getPreEventSynCode()) || same(m->getPreEventSynCode(), respelt(builtin->getPreEventSynCode())))
+           && m->getVars().size() == 1 && m->getVars()[0].name == "g" && refs.size() == 1 && refs[0].name == "V"
+           && m->getParams().size() == 2 && m->getPreVars().empty() && m->getPostVars().empty();
+}
+
 unsigned int recogniseWUM(const WeightUpdateModels::Base *m, const std::string &name)
 {
     const bool plain = m->getPostSpikeSynCode().empty() && m->getSynapseDynamicsCode().empty() && m->getPreEventSynCode().empty()
@@ -184,6 +206,7 @@ unsigned int recogniseWUM(const WeightUpdateModels::Base *m, const std::string &
         return GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY;
     }
     if(isTraceSTDP(m)) { return GENNMI_WUM_STDP_TRACE; }
+    if(isStaticGraded(m)) { return GENNMI_WUM_STATIC_GRADED; }
     unsupported("weight update model of projection '" + name + "'");
 }
 
@@ -269,7 +292,11 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
                 }
                 if(arch.isSimRNGRequired()) { unsupported("random numbers in the update of population '" + arch.getName() + "'"); }
                 if(arch.isPrevSpikeTimeRequired()) { unsupported("previous spike times of population '" + arch.getName() + "'"); }
-                if(!n.getMergedSpikeEventGroups().empty()) { unsupported("spike-like events of population '" + arch.getName() + "'"); }
+                if(n.getMergedSpikeEventGroups().size() > GENNMI_MAX_SPK_EVENT) { unsupported("more than 2 spike-like event conditions on population '" + arch.getName() + "'"); }
+                if(!n.getMergedSpikeEventGroups().empty() && (arch.isDelayRequired() || arch.isSpikeEventTimeRequired() || arch.isPrevSpikeEventTimeRequired()
+                                                              || arch.isSpikeEventRecordingEnabled())) {
+                    unsupported("delay slots, event times or event recording with spike-like events on population '" + arch.getName() + "'");
+                }
                 if(!n.getMergedOutSynPreOutputGroups().empty()) { unsupported("presynaptic output into population '" + arch.getName() + "'"); }
 
                 // values of one quantity across the groups of this merged group
@@ -455,6 +482,27 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
                         queue << "*" << env["_spk_que_ptr"] << " = (*" << env["_spk_que_ptr"] << " + 1) % " << arch.getNumDelaySlots() << ";" << std::endl;
                     }
                 }
+                // spike-like event queues ("SynSpikeEvent" children): recognised condition V > Epre of an outgoing graded projection
+                const auto &events = n.getMergedSpikeEventGroups();
+                for(size_t k = 0; k < events.size(); k++) {
+                    auto &child = const_cast<NeuronUpdateGroupMerged::SynSpikeEvent&>(events[k]);
+                    const auto &carch = child.getArchetype();
+                    if(carch.getSrcNeuronGroup() != &arch || !isStaticGraded(carch.getWUInitialiser().getSnippet())) {
+                        unsupported("spike-like event condition of projection '" + carch.getName() + "'");
+                    }
+                    const std::string sfx = "SynSpikeEvent" + std::to_string(child.getIndex());
+                    EnvironmentGroupMergedField<NeuronUpdateGroupMerged::SynSpikeEvent, NeuronUpdateGroupMerged> eenv(env, child, n);
+                    eenv.addField(Type::Uint32.createPointer(), "_mi_spkCntEvent", "spkCntEvent" + sfx,
+                                  [&n](const auto &runtime, const auto &g, size_t i) { return runtime.getFusedEventArray(n, i, g, "SpkCntEvent"); });
+                    eenv.addField(Type::Uint32.createPointer(), "_mi_spkEvent", "spkEvent" + sfx,
+                                  [&n](const auto &runtime, const auto &g, size_t i) { return runtime.getFusedEventArray(n, i, g, "SpkEvent"); });
+                    std::vector<Type::NumericValue> thresholds;
+                    for(const auto &g : child.getGroups()) { thresholds.push_back(g.get().getWUInitialiser().getParams().at("Epre")); }
+                    eenv.getStream() << "{ static const float v[] = " << table(thresholds, scalar) << "; d.spkEvent[" << k << "].spkCntEvent = gennmiDev("
+                                     << eenv["_mi_spkCntEvent"] << "); d.spkEvent[" << k << "].spkEvent = gennmiDev(" << eenv["_mi_spkEvent"]
+                                     << "); d.spkEvent[" << k << "].threshold = v[g]; }" << std::endl;
+                }
+                out << "d.numSpkEvent = " << events.size() << "u;" << std::endl;
                 if(arch.isSpikeTimeRequired()) { out << "d.sT = gennmiDev(" << env["_st"] << ");" << std::endl; }
                 if(arch.isSpikeRecordingEnabled()) { out << "d.recordSpk = gennmiDev(" << env["_record_spk"] << ");" << std::endl; }
                 out << "GENNMI_CHECK(gennmi_push_neuron_update_group(gennmiRunner, &d, nullptr));" << std::endl;
@@ -515,7 +563,9 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                 if(arch.getBackPropDelaySteps() != 0 || (wumKind == GENNMI_WUM_STDP_TRACE && (srcDelay || arch.getTrgNeuronGroup()->isDelayRequired()))) {
                     unsupported("back-propagation delay, or delay slots on a plastic projection ('" + arch.getName() + "')");
                 }
-                if(arch.isPreSpikeEventRequired() || arch.isPostSpikeEventRequired()) { unsupported("spike-like events on projection '" + arch.getName() + "'"); }
+                const bool graded = (wumKind == GENNMI_WUM_STATIC_GRADED);
+                if((arch.isPreSpikeEventRequired() && !graded) || arch.isPostSpikeEventRequired()) { unsupported("spike-like events on projection '" + arch.getName() + "'"); }
+                if(graded && srcDelay) { unsupported("delay slots on the source of graded projection '" + arch.getName() + "'"); }
                 if(wumKind == GENNMI_WUM_STDP_TRACE && batchSize != 1) { unsupported("plastic weights with a batch size above 1"); }
 
                 const auto matrixType = arch.getMatrixType();
@@ -527,6 +577,7 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                 if(!sparse && !toeplitz && !dense && !bitmask) {
                     unsupported("matrix type of projection '" + arch.getName() + "' (SPARSE, DENSE, BITMASK or TOEPLITZ with kernel weights)");
                 }
+                if(graded && !sparse) { unsupported("graded synapses on a non-SPARSE projection ('" + arch.getName() + "')"); }
                 if(dense && wumKind != GENNMI_WUM_STATIC_PULSE && !constantWeight) { unsupported("weight update model of DENSE projection '" + arch.getName() + "'"); }
                 if(bitmask && !constantWeight) { unsupported("weight update model of BITMASK projection '" + arch.getName() + "' (StaticPulseConstantWeight)"); }
                 if(toeplitz && constantWeight) { unsupported("constant weight on Toeplitz projection '" + arch.getName() + "'"); }
@@ -579,7 +630,19 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                     << ", b[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getTrgNeuronGroup()->getNumNeurons(); }))
                     << ", c[] = " << tableU32(counts([this](const SynapseGroupInternal &g){ return getSynapticMatrixRowStride(g); }))
                     << "; d.numSrcNeurons = a[g]; d.numTrgNeurons = b[g]; d.rowStride = c[g]; }" << std::endl;
-                out << "d.srcSpkCnt = gennmiDev(" << env["_src_spk_cnt"] << "); d.srcSpk = gennmiDev(" << env["_src_spk"] << ");" << std::endl;
+                if(graded) {
+                    // driven by the source's event queue; V_pre is the source population's V
+                    out << "d.srcSpkCnt = gennmiDev(" << env["_src_spk_cnt_event"] << "); d.srcSpk = gennmiDev(" << env["_src_spk_event"] << ");" << std::endl;
+                    env.addField(scalar.createPointer(), "_mi_srcV", "V",
+                                 [](const auto &runtime, const auto &g, size_t) { return g.getWUMPreNeuronVarReferences().at("V").getTargetArray(runtime); });
+                    out << "d.srcV = gennmiDev(" << env["_mi_srcV"] << ");" << std::endl;
+                    out << "{ static const float a[] = " << table(values([](const SynapseGroupInternal &g){ return g.getWUInitialiser().getParams().at("Epre"); }), scalar)
+                        << ", b[] = " << table(values([](const SynapseGroupInternal &g){ return g.getWUInitialiser().getParams().at("Vslope"); }), scalar)
+                        << "; d.gradedEpre = a[g]; d.gradedVslope = b[g]; }" << std::endl;
+                }
+                else {
+                    out << "d.srcSpkCnt = gennmiDev(" << env["_src_spk_cnt"] << "); d.srcSpk = gennmiDev(" << env["_src_spk"] << ");" << std::endl;
+                }
                 if(srcDelay) {
                     if(dense || bitmask) { unsupported("axonal delay on DENSE or BITMASK projection '" + arch.getName() + "'"); }
                     out << "{ static const uint32_t a[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getAxonalDelaySteps(); }))

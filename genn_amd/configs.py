@@ -238,6 +238,36 @@ def dense_bitmask(n_a=300, n_b=77, steps=200, seed=9, dt=1.0, fuse=False):
     return net
 
 
+def graded(n_a=300, n_b=130, n_c=64, steps=200, seed=13, dt=0.5):
+    """Graded (spike-like event) transmission next to ordinary spikes: two LIF populations and an Izhikevich one, three
+    StaticGraded projections with different thresholds and slopes (two of them leave population A, so it keeps two event
+    queues) and one spiking inhibitory projection back."""
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.6, TauRefrac=2.0)
+    net = Net(name="graded", dt=dt, steps=steps, seed=seed)
+    net.pops.append(Pop("A", "lif", n_a, dict(lif), {"V": (-60.0 + 9.0 * rng.uniform(seed, 1, 0, n_a)).astype(np.float32),
+                                                     "RefracTime": np.zeros(n_a, np.float32)}))
+    net.pops.append(Pop("B", "lif", n_b, dict(lif, Ioffset=0.35), {"V": (-60.0 + 5.0 * rng.uniform(seed, 2, 0, n_b)).astype(np.float32),
+                                                                   "RefracTime": np.zeros(n_b, np.float32)}))
+    net.pops.append(Pop("C", "izh", n_c, dict(a=0.02, b=0.2, c=-65.0, d=8.0),
+                        {"V": (-65.0 + 10.0 * rng.uniform(seed, 3, 0, n_c)).astype(np.float32), "U": np.full(n_c, -13.0, np.float32)}))
+    net.css.append(CurrentSource("C_dc", "dc", "C", amp=6.0))
+
+    def sparse(name, src, trg, n_src, n_trg, stride, stream, lo, hi, **kw):
+        ind = np.sort(rng.randint(seed, stream, 0, n_src * stride, n_trg).reshape(n_src, stride), axis=1).astype(np.uint32)
+        row_length = (stride - rng.randint(seed, stream + 1, 0, n_src, 4)).astype(np.uint32)          # ragged rows
+        g = (lo + (hi - lo) * rng.uniform(seed, stream + 2, 0, n_src * stride)).astype(np.float32).reshape(n_src, stride)
+        return Syn(name, src, trg, psm="expcurr", row_stride=stride, row_length=row_length, ind=ind, g=g, **kw)
+
+    net.syns.append(sparse("AB_graded", "A", "B", n_a, n_b, 24, 10, 0.0, 0.04, wum="static_graded",
+                           wum_params={"Epre": -54.3, "Vslope": 7.3}, tau=5.0))
+    net.syns.append(sparse("AA_graded", "A", "A", n_a, n_a, 16, 20, -0.01, 0.03, wum="static_graded",
+                           wum_params={"Epre": -52.0, "Vslope": 4.1}, tau=8.0))
+    net.syns.append(sparse("CB_graded", "C", "B", n_c, n_b, 40, 30, 0.0, 0.02, wum="static_graded",
+                           wum_params={"Epre": -40.0, "Vslope": 20.0}, tau=5.0))
+    net.syns.append(sparse("BA_spikes", "B", "A", n_b, n_a, 30, 40, -0.6, -0.2, wum="static", tau=10.0))
+    return net
+
+
 def dense_layer(n_in=8192, n_out=8192, rate_hz=50.0, steps=1000, seed=17, dt=1.0, w_sd=0.02):
     """A fully connected spiking layer: Poisson sources (rate_hz per source) into LIF neurons through a DENSE matrix
     with individual weights ~ N(0, w_sd); the shape of the dense layers of rate-coded classifiers."""

@@ -127,6 +127,7 @@ struct NeuronGroupDev
     uint32_t *shadowSpk;                // [2][batch*N] engine-private double-buffered copy of the spike queue, or NULL
     uint32_t *shadowCnt;                // [2][batch]
     uint32_t *spikeBitmap;              // [ceil(N/32)] engine-private bitmap of this step's spikes (populations with learnPost), or NULL
+    unsigned long long *aggEvent;       // look-back area of the spike-like event queues (groups with events), or NULL
 };
 
 struct PreGroupDev
@@ -344,6 +345,18 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
                     if(inRow) { ip = ind[rowBase + j]; w = weight[rowBase + j]; dl = delay[rowBase + j]; }
                     const uint32_t slot = (denPtr + dl) % D;
                     if(j < npost && !(G.skipZeroDelay && slot == denPtr)) { atomicAddF32(&denDelay[(size_t)slot * numTrg + ip], w); }
+                }
+            }
+            else if(g.wum == GENNMI_WUM_STATIC_GRADED) {
+                // event code of weightUpdateModels.h:318: addToPost(fmax(0.0, g * tanh((V_pre - Epre) / Vslope) * dt)).  The CPU
+                // backend's generated code evaluates tanh, the products and the maximum in double (only the double versions of
+                // tanh and fmax are in scope there); so does this, rounding once before the fp32 atomic.
+                const float vPre = asGlobal(g.srcV)[(size_t)batch * g.numSrcNeurons + idPre];
+                const double release = tanh((double)((vPre - g.gradedEpre) / g.gradedVslope));
+                for(uint32_t q = 0; q < perLane; q++) {
+                    if(inRow && j + q < npost) {
+                        atomicAddF32(&outPost[ind[rowBase + j + q]], (float)fmax(0.0, (double)weight[rowBase + j + q] * release * (double)dt));
+                    }
                 }
             }
             else if(j < npost) {
@@ -795,6 +808,77 @@ void postsynapticUpdateKernel(const PostGroupDev * __restrict__ blocks, StepArgs
 }
 
 // ------------------------------------------------------------------------------------------------
+// Ordered append of the flagged neurons of a population to a queue, for spike-like events: the scheme the neuron
+// update uses for true spikes (ballot rank in the wave, LDS scan in the block, look-back over per-block counts tagged
+// with the step, blocks in groups of 64 with a published group total), as a function every block of the population
+// calls with all its threads.  `counts` and `groupTotals` hold one entry per (batch, neuron block of the launch).
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void appendOrdered(bool flag, uint32_t id, uint32_t localBlock, uint32_t numBlocks, size_t aggBase,
+                                              unsigned long long *counts, unsigned long long *groupTotals, uint32_t tag,
+                                              uint32_t *queue, uint32_t *queueCount, uint32_t *errorFlag)
+{
+    __shared__ uint32_t shCount[BLOCK / WAVE];
+    __shared__ uint32_t shOffset;
+    const uint32_t lane = threadIdx.x & (WAVE - 1);
+    const uint32_t wave = threadIdx.x / WAVE;
+    const unsigned long long ballot = __ballot(flag);
+    const uint32_t laneRank = __popcll(ballot & ((1ull << lane) - 1ull));
+    if(lane == 0) { shCount[wave] = __popcll(ballot); }
+    __syncthreads();
+    uint32_t blockCount = 0, waveOffset = 0;
+    #pragma unroll
+    for(uint32_t w = 0; w < BLOCK / WAVE; w++) {
+        const uint32_t c = shCount[w];
+        if(w < wave) { waveOffset += c; }
+        blockCount += c;
+    }
+    if(threadIdx.x == 0) {
+        __hip_atomic_store(&counts[aggBase + localBlock], ((unsigned long long)tag << 32) | blockCount, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const bool last = (localBlock == numBlocks - 1);
+    if(wave == 0) {
+        const uint32_t group = localBlock / WAVE, inGroup = localBlock % WAVE;
+        const size_t groupBase = aggBase + (size_t)group * WAVE;
+        bool ok = true;
+        auto waitFor = [&](const unsigned long long *p) -> uint32_t {
+            uint32_t spins = 0;
+            while(true) {
+                const unsigned long long a = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if((uint32_t)(a >> 32) == tag) { return (uint32_t)a; }
+                if(++spins > c_spinLimit) { ok = false; return 0u; }
+                __builtin_amdgcn_s_sleep(1);
+            }
+        };
+        uint32_t intra = (lane < inGroup) ? waitFor(&counts[groupBase + lane]) : 0u;
+        for(int off = WAVE / 2; off > 0; off >>= 1) { intra += __shfl_down(intra, off, WAVE); }
+        intra = __shfl(intra, 0, WAVE);
+        if((inGroup == WAVE - 1 || last) && lane == 0 && ok) {
+            __hip_atomic_store(&groupTotals[aggBase + group], ((unsigned long long)tag << 32) | (intra + blockCount), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        uint32_t sum = 0;
+        if(blockCount != 0 || last) {
+            for(uint32_t base = 0; base < group; base += WAVE) {
+                if(base + lane < group) { sum += waitFor(&groupTotals[aggBase + base + lane]); }
+            }
+            for(int off = WAVE / 2; off > 0; off >>= 1) { sum += __shfl_down(sum, off, WAVE); }
+            sum += intra;
+        }
+        const bool allOk = (__ballot(!ok) == 0ull);
+        if(lane == 0) {
+            if(!allOk) { atomicOr(errorFlag, 1u); sum = 0xFFFFFFFFu; }
+            shOffset = sum;
+        }
+    }
+    __syncthreads();
+    const uint32_t prefix = shOffset;
+    if(prefix != 0xFFFFFFFFu) {
+        if(flag) { queue[prefix + waveOffset + laneRank] = id; }
+        if(last && threadIdx.x == 0) { *queueCount = prefix + blockCount; }
+    }
+    __syncthreads();            // the shared words are reused by the next call
+}
+
+// ------------------------------------------------------------------------------------------------
 // Neuron update.  One lane per neuron.  Spikes are emitted in ascending neuron index (the CPU
 // backend's order, single_threaded_cpu/backend.cc:321, 2119-2133): wave ballot gives the in-wave
 // rank, an LDS scan the in-block rank, and a look-back over per-block counts published in `agg`
@@ -818,6 +902,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
     const float t = st.t;
 
     bool spiked = false;
+    float vEvent = 0.0f;
     uint32_t z0 = 0, z1 = 0;
     if(G.zeroStart && i < n) { z0 = asGlobal(G.zeroStart)[i]; z1 = asGlobal(G.zeroStart)[i + 1]; }
     if(i < n) {
@@ -908,6 +993,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
         if(g.model == GENNMI_NEURON_LIF) { spiked = (l1 <= 0.0f && l0 >= g.params[4]); }
         else if(g.model == GENNMI_NEURON_IZHIKEVICH) { spiked = (l0 >= 29.99f); }
         else { spiked = (startSpike != g.endSpike[bi]) && (t >= g.spikeTimes[startSpike]); }
+        vEvent = l0;           // spike-like event conditions see the updated V before any reset (neuronUpdateGroupMerged.cc:677-683)
         if(spiked) {
             preTrace += 1.0f; postTrace += 1.0f;
             if(g.sT) { g.sT[bi] = t; }
@@ -923,6 +1009,17 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
     if(localBlock == 0 && batch == 0 && threadIdx.x < g.numPSM) {
         const gennmi_psm_t &psm = g.psm[threadIdx.x];
         if(psm.maxDenDelay && psm.denDelayPtr) { *psm.denDelayPtr = modStep(st.epoch + 1, psm.maxDenDelay); }
+    }
+
+    // ---- spike-like events: one ordered queue per event condition ----------------------------------
+    if(g.numSpkEvent) {
+        const size_t perArea = (size_t)totalNeuronBlocks * gridDim.y;
+        for(uint32_t e = 0; e < g.numSpkEvent; e++) {
+            unsigned long long *counts = G.aggEvent + (size_t)e * 2 * perArea;
+            appendOrdered(i < n && vEvent > g.spkEvent[e].threshold, i, localBlock, G.numBlocks, (size_t)batch * totalNeuronBlocks + G.startBlock,
+                          counts, counts + perArea, (uint32_t)(st.epoch + 1), g.spkEvent[e].spkEvent + (size_t)batch * n,
+                          g.spkEvent[e].spkCntEvent + batch, errorFlag);
+        }
     }
 
     // ---- ordered compaction --------------------------------------------------------------------
@@ -1981,6 +2078,13 @@ int gennmi_push_neuron_update_group(gennmi_runner *r, const gennmi_neuron_update
     for(uint32_t q = 0; q < g->numExtraSpk; q++) {
         if(!g->extraSpkCnt[q] || !g->extraSpk[q]) { return fail(GENNMI_EINVAL, "push_neuron_update_group: extra spike array missing"); }
     }
+    if(g->numSpkEvent > GENNMI_MAX_SPK_EVENT) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: too many spike-like event conditions"); }
+    if(g->numSpkEvent && (g->model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY || g->numDelaySlots > 1)) {
+        return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: spike-like events need a LIF or Izhikevich group without delay slots");
+    }
+    for(uint32_t e = 0; e < g->numSpkEvent; e++) {
+        if(!g->spkEvent[e].spkCntEvent || !g->spkEvent[e].spkEvent) { return fail(GENNMI_EINVAL, "push_neuron_update_group: event queue missing"); }
+    }
     NeuronGroupDev d;
     memset(&d, 0, sizeof(d));
     d.g = *g;
@@ -2060,6 +2164,10 @@ int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynap
             if(!g->trgST || !g->postTrace) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: STDP arrays missing"); }
             if(r->batch != 1) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: plastic weights need batch size 1"); }
         }
+        else if(g->wum == GENNMI_WUM_STATIC_GRADED) {
+            if(!g->srcV || !(g->gradedVslope != 0.0f)) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: graded synapses need the source's V and a non-zero Vslope"); }
+            if(g->numSrcDelaySlots > 1) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: axonal delay on a graded projection"); }
+        }
         else if(g->wum != GENNMI_WUM_STATIC_PULSE) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: unknown weight update model"); }
         if(g->wum != GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY) { d.g.maxDenDelay = 0; }
     }
@@ -2109,7 +2217,7 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
     if(r->batch != 1 || !r->post.empty() || r->pre.empty() || !r->dense.empty() || !r->proc.empty() || r->neuron.size() > RES_MAX_GROUPS) { return GENNMI_OK; }
     for(const auto &n : r->neuron) {
         const auto &g = n.g;
-        if((g.model != GENNMI_NEURON_LIF && g.model != GENNMI_NEURON_IZHIKEVICH) || g.preTrace || g.postTrace || g.sT || g.numDelaySlots > 1) { return GENNMI_OK; }
+        if((g.model != GENNMI_NEURON_LIF && g.model != GENNMI_NEURON_IZHIKEVICH) || g.preTrace || g.postTrace || g.sT || g.numDelaySlots > 1 || g.numSpkEvent) { return GENNMI_OK; }
         for(uint32_t c = 0; c < g.numCS; c++) { if(g.cs[c].kind != GENNMI_CS_DC) { return GENNMI_OK; } }
     }
     // tiles and their LDS layout
@@ -2473,8 +2581,10 @@ int gennmi_runner_finalise(gennmi_runner *r)
 
     // ---- single-launch step: possible when every projection is a SPARSE dendritic-delay one with ring depth >= 2
     // and nothing is plastic
+    bool anyEvents = false;
+    for(const auto &n : r->neuron) { anyEvents = anyEvents || n.g.numSpkEvent != 0; }
     const char *envFused = getenv("GENNMI_FUSED_STEP");
-    bool eligible = !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty() && r->dense.empty() && r->proc.empty();
+    bool eligible = !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty() && r->dense.empty() && r->proc.empty() && !anyEvents;
     for(const auto &p : r->pre) {
         eligible = eligible && p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY
                    && p.g.maxDenDelay >= 2 && p.g.numSrcDelaySlots <= 1;
@@ -2556,6 +2666,15 @@ int gennmi_runner_finalise(gennmi_runner *r)
     }
     if(r->postLdsBytes > 48 * 1024) {
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(postsynapticUpdateKernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)r->postLdsBytes));
+    }
+    // look-back area of the spike-like event queues: per event slot, per-block counts then per-group totals
+    if(anyEvents) {
+        const size_t count = (size_t)GENNMI_MAX_SPK_EVENT * 2 * r->neuronBlocks * r->batch;
+        unsigned long long *area = nullptr;
+        HIP_TRY(hipMalloc(&area, count * sizeof(unsigned long long)));
+        r->owned.push_back(area);
+        HIP_TRY(hipMemset(area, 0, count * sizeof(unsigned long long)));
+        for(auto &n : r->neuron) { n.aggEvent = area; }
     }
     HIP_TRY(uploadPerBlock(r->neuron, r->neuronBlocks, &r->dNeuron));
     HIP_TRY(uploadPerBlock(r->pre, r->preBlocks, &r->dPre));

@@ -75,7 +75,7 @@ def init_postsynaptic(snippet, params=None, vars=None):
 
 
 def init_weight_update(snippet, params=None, vars=None, pre_vars=None, post_vars=None):
-    if snippet not in ("StaticPulse", "StaticPulseConstantWeight", "StaticPulseDendriticDelay", "STDPTrace"):
+    if snippet not in ("StaticPulse", "StaticPulseConstantWeight", "StaticPulseDendriticDelay", "STDPTrace", "StaticGraded"):
         raise NotImplementedError(f"weight update model {snippet}")
     return _Init(snippet, params, vars, pre_vars, post_vars)
 
@@ -220,6 +220,7 @@ class NeuronGroup:
         self.post_trace_owner = None
         self.needs_spike_time = False
         self.num_delay_slots = 1     # longest axonal delay of the outgoing projections + 1, set by build()
+        self.event_thresholds = []   # one spike-like event queue per distinct threshold of the outgoing graded projections
 
     @property
     def size(self):
@@ -398,6 +399,11 @@ class GeNNModel:
                                           "FixedProbabilityNoAutapse or FixedNumberPostWithReplacement")
             if weight_update_init.snippet not in ("StaticPulse", "StaticPulseConstantWeight"):
                 raise NotImplementedError(f"PROCEDURAL connectivity with {weight_update_init.snippet}")
+        if weight_update_init.snippet == "StaticGraded":
+            if matrix_type != "SPARSE":
+                raise NotImplementedError("StaticGraded needs SPARSE connectivity")
+            if source.neuron == "SpikeSourceArray":
+                raise ValueError("StaticGraded references the presynaptic variable V, which a spike source does not have")
         if matrix_type == "BITMASK" and weight_update_init.snippet != "StaticPulseConstantWeight":
             raise ValueError("BITMASK connectivity has no per-synapse variables: use StaticPulseConstantWeight")
         if matrix_type == "DENSE" and weight_update_init.snippet not in ("StaticPulse", "StaticPulseConstantWeight"):
@@ -443,6 +449,13 @@ class GeNNModel:
             if len(pre) > 1 or len(post) > 1:
                 raise NotImplementedError(f"{n.name}: more than one plastic projection per side")
             n.num_delay_slots = max([s.axonal_delay_steps for s in n.out_syn], default=0) + 1
+            # projections whose event condition and parameters agree share one queue (neuronGroup.cc:505-517)
+            n.event_thresholds = []
+            for s in n.out_syn:
+                if s.wu.snippet == "StaticGraded" and float(s.wu.params["Epre"]) not in n.event_thresholds:
+                    n.event_thresholds.append(float(s.wu.params["Epre"]))
+            if len(n.event_thresholds) > _abi.MAX_SPK_EVENT:
+                raise NotImplementedError(f"{n.name}: more than {_abi.MAX_SPK_EVENT} spike-like event conditions")
             n.pre_trace_owner = pre[0] if pre else None
             n.post_trace_owner = post[0] if post else None
             n.needs_spike_time = bool(pre or post)
@@ -505,6 +518,9 @@ class GeNNModel:
                     n.vars[v] = a
             n.vars["spkCnt"] = self._alloc(B * n.num_delay_slots, np.uint32)
             n.vars["spk"] = self._alloc(B * n.num_delay_slots * N, np.uint32)
+            for e in range(len(n.event_thresholds)):
+                n.vars[f"spkCntEvent{e}"] = self._alloc(B, np.uint32)
+                n.vars[f"spkEvent{e}"] = self._alloc(B * N, np.uint32)
             if n.spike_recording_enabled:
                 if not num_recording_timesteps:
                     raise RuntimeError("Cannot use recording system without specifying number of recording timesteps")
@@ -649,7 +665,7 @@ class GeNNModel:
     def _neuron_merge_key(self, n):
         psm = tuple((grp[0].ps.snippet, self._den_delay(grp[0])) for grp in self._sorted_psm(n))
         return (n.neuron, psm, tuple(cs.kind for cs in n.current_sources), n.pre_trace_owner is not None,
-                n.post_trace_owner is not None, n.needs_spike_time, n.spike_recording_enabled, n.num_delay_slots)
+                n.post_trace_owner is not None, n.needs_spike_time, n.spike_recording_enabled, n.num_delay_slots, len(n.event_thresholds))
 
     def _sorted_psm(self, n):
         # children are ordered by a structure-only digest, ties keep creation order (groupMerged.h:411-454)
@@ -691,6 +707,13 @@ class GeNNModel:
                     d.var0, d.var1 = n.vars["V"].ptr, n.vars["U"].ptr
                     for j in range(4):
                         d.params[j] = rounded[j][k]
+            # spike-like event children
+            for e in range(len(members[0].event_thresholds)):
+                thresholds = _merge_round([n.event_thresholds[e] for n in members])
+                for k, (d, n) in enumerate(zip(descs, members)):
+                    d.numSpkEvent = len(n.event_thresholds)
+                    d.spkEvent[e].spkCntEvent, d.spkEvent[e].spkEvent = n.vars[f"spkCntEvent{e}"].ptr, n.vars[f"spkEvent{e}"].ptr
+                    d.spkEvent[e].threshold = thresholds[k]
             # postsynaptic-model children
             num_psm = len(members[0].fused_psm)
             for m in range(num_psm):
@@ -748,12 +771,15 @@ class GeNNModel:
                 rounded = {q: _merge_round([s.wu.params[q] for s in members]) for q in ("aPlus", "aMinus", "wMin", "wMax")}
             if members[0].wu.snippet == "StaticPulseConstantWeight":
                 consts = _merge_round([s.wu.params["g"] for s in members])
+            if members[0].wu.snippet == "StaticGraded":
+                graded = {q: _merge_round([s.wu.params[q] for s in members]) for q in ("Epre", "Vslope")}
             for k, s in enumerate(members):
                 d = _abi.PresynapticUpdateGroup()
                 d.matrix = {"SPARSE": _abi.MATRIX_SPARSE, "TOEPLITZ": _abi.MATRIX_TOEPLITZ_CONV2D, "DENSE": _abi.MATRIX_DENSE,
                             "BITMASK": _abi.MATRIX_BITMASK, "PROCEDURAL": _abi.MATRIX_PROCEDURAL}[s.matrix_type]
                 d.wum = {"StaticPulse": _abi.WUM_STATIC_PULSE, "StaticPulseDendriticDelay": _abi.WUM_STATIC_PULSE_DENDRITIC_DELAY,
-                         "STDPTrace": _abi.WUM_STDP_TRACE, "StaticPulseConstantWeight": _abi.WUM_STATIC_PULSE_CONSTANT_WEIGHT}[s.wu.snippet]
+                         "STDPTrace": _abi.WUM_STDP_TRACE, "StaticPulseConstantWeight": _abi.WUM_STATIC_PULSE_CONSTANT_WEIGHT,
+                         "StaticGraded": _abi.WUM_STATIC_GRADED}[s.wu.snippet]
                 if s.wu.snippet == "StaticPulseConstantWeight":
                     d.constantWeight = consts[k]
                     if s.matrix_type == "SPARSE":
@@ -765,6 +791,12 @@ class GeNNModel:
                 d.outPost = owner.vars["outPost"].ptr
                 d.srcSpkCnt, d.srcSpk = s.src.vars["spkCnt"].ptr, s.src.vars["spk"].ptr
                 d.axonalDelaySteps, d.numSrcDelaySlots = s.axonal_delay_steps, s.src.num_delay_slots
+                if s.wu.snippet == "StaticGraded":
+                    # the projection is driven by the source's event queue for its threshold, not by its spikes
+                    e = s.src.event_thresholds.index(float(s.wu.params["Epre"]))
+                    d.srcSpkCnt, d.srcSpk = s.src.vars[f"spkCntEvent{e}"].ptr, s.src.vars[f"spkEvent{e}"].ptr
+                    d.srcV = s.src.vars["V"].ptr
+                    d.gradedEpre, d.gradedVslope = graded["Epre"][k], graded["Vslope"][k]
                 if "g" in s.vars:
                     d.g = s.vars["g"].ptr
                 if s.matrix_type == "BITMASK":
@@ -930,6 +962,8 @@ def model_from_net(net, batch_size=1, record=True, span=None, device=0):
             wu = init_weight_update("StaticPulseDendriticDelay", {}, {"g": 0.0, "d": 0})
         elif s.wum == "static_const":
             wu = init_weight_update("StaticPulseConstantWeight", {"g": s.wum_params["g"]})
+        elif s.wum == "static_graded":
+            wu = init_weight_update("StaticGraded", s.wum_params, {"g": 0.0})
         else:
             wu = init_weight_update("STDPTrace", s.wum_params, {"g": 0.0}, {"preTrace": 0.0}, {"postTrace": 0.0})
         if s.matrix == "dense":

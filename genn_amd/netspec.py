@@ -47,6 +47,7 @@ class Syn:
     trg: str
     matrix: str = "sparse"          # "sparse" | "conv2d" | "dense" | "bitmask"
     wum: str = "static"             # "static" | "static_delay" | "stdp_trace" | "static_const" (one weight, wum_params["g"])
+                                    # | "static_graded" (spike-like events, wum_params["Epre"], ["Vslope"]; source must have a V)
     wum_params: Dict[str, float] = field(default_factory=dict)
     psm: str = "expcurr"            # "expcurr" | "deltacurr"
     tau: float = 5.0
@@ -173,6 +174,8 @@ def write_netspec(net: Net, path: str):
             np.ascontiguousarray(s.d, dtype=np.uint8).tofile(os.path.join(path, f"{s.name}.d.u8"))
         elif s.wum == "stdp_trace":
             w = "stdp_trace " + " ".join(repr(float(s.wum_params[k])) for k in STDP_PARAMS)
+        elif s.wum == "static_graded":
+            w = f"static_graded {float(s.wum_params['Epre'])!r} {float(s.wum_params['Vslope'])!r}"
         else:
             raise ValueError(s.wum)
         psm = f"expcurr {float(s.tau)!r}" if s.psm == "expcurr" else "deltacurr"

@@ -45,7 +45,10 @@ enum { GENNMI_PSM_EXPCURR = 0, GENNMI_PSM_DELTACURR = 1 };
 enum { GENNMI_CS_DC = 0, GENNMI_CS_ARRAY = 1 };
 /* weight update models: include/genn/genn/weightUpdateModels.h:236-244, :279-287; trace STDP pygenn/genn_model.py:1448-1476 */
 enum { GENNMI_WUM_STATIC_PULSE = 0, GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY = 1, GENNMI_WUM_STDP_TRACE = 2,
-       GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT = 3 /* weightUpdateModels.h:202-213: one weight for the whole projection */ };
+       GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT = 3, /* weightUpdateModels.h:202-213: one weight for the whole projection */
+       /* weightUpdateModels.h:308-319: no spike code; while the presynaptic V exceeds Epre the neuron emits a spike-like
+        * event every step, and each event adds fmax(0, g * tanh((V_pre - Epre) / Vslope) * dt) per synapse */
+       GENNMI_WUM_STATIC_GRADED = 4 };
 /* connectivity: ragged SPARSE (runtime.cc:360-402) or TOEPLITZ Conv2D (initToeplitzConnectivitySnippet.h:105-150) */
 enum { GENNMI_MATRIX_SPARSE = 0, GENNMI_MATRIX_TOEPLITZ_CONV2D = 1,
        /* DENSE: g[numSrc*numTrg], idSyn = idPre*numTrg + idPost; BITMASK: one bit per pair, most significant bit first,
@@ -118,6 +121,18 @@ typedef struct gennmi_cs_t {              /* one current source child (neuronUpd
     uint32_t pad_;
 } gennmi_cs_t;
 
+/* Spike-like events ("SynSpikeEvent" children, neuronUpdateGroupMerged.cc:189-330): after the neuron's sim code and
+ * before its threshold test, a neuron whose V exceeds `threshold` is appended to this queue (ascending neuron index, like
+ * true spikes; backend.cc genEmitEvent).  The queue is rewritten every step.  Projections whose weight update model has
+ * an event threshold read it as their srcSpk / srcSpkCnt. */
+#define GENNMI_MAX_SPK_EVENT 2
+typedef struct gennmi_spike_event_t {
+    uint32_t *spkCntEvent;                /* [batch] */
+    uint32_t *spkEvent;                   /* [batch*numNeurons] */
+    float threshold;                      /* StaticGraded: Epre */
+    uint32_t pad_;
+} gennmi_spike_event_t;
+
 typedef struct gennmi_neuron_update_group_t {      /* MergedNeuronUpdateGroup<i> */
     uint32_t model;                       /* GENNMI_NEURON_* */
     uint32_t numNeurons;
@@ -145,6 +160,8 @@ typedef struct gennmi_neuron_update_group_t {      /* MergedNeuronUpdateGroup<i>
     uint32_t numDelaySlots;
     uint32_t *extraSpkCnt[GENNMI_MAX_EXTRA_SPK];
     uint32_t *extraSpk[GENNMI_MAX_EXTRA_SPK];
+    uint32_t numSpkEvent, pad2_;          /* LIF and Izhikevich groups without delay slots only */
+    gennmi_spike_event_t spkEvent[GENNMI_MAX_SPK_EVENT];
 } gennmi_neuron_update_group_t;
 
 /* What gennmi_init_sparse_* and gennmi_init_var would have stored for a projection, for GENNMI_MATRIX_PROCEDURAL: the row
@@ -189,6 +206,10 @@ typedef struct gennmi_presynaptic_update_group_t { /* MergedPresynapticUpdateGro
     uint32_t axonalDelaySteps;
     uint32_t numSrcDelaySlots, pad3_;
     gennmi_procedural_t procedural;       /* GENNMI_MATRIX_PROCEDURAL only (rowStride = the stride the stored matrix would have) */
+    /* GENNMI_WUM_STATIC_GRADED (SPARSE only): srcSpk / srcSpkCnt are the source's event queue for threshold Epre; V_pre is
+     * read when the event is delivered, i.e. after the update (and reset) that emitted it */
+    const float *srcV;                    /* [batch*numSrcNeurons] the source population's V */
+    float gradedEpre, gradedVslope;
 } gennmi_presynaptic_update_group_t;
 
 typedef struct gennmi_postsynaptic_update_group_t { /* MergedPostsynapticUpdateGroup<i> */

@@ -14,10 +14,13 @@
  *                        Toeplitz presynaptic loop   backend.cc:1788-1883, include/genn/genn/initToeplitzConnectivitySnippet.h:116-137
  *                        dense / bitmask loop        backend.cc:1985-2021 (bit gid = idPre*rowStride + idPost, most significant bit
  *                                                    first; row stride = numPost padded to 32, backend.cc:1393-1404)
+ *                        spike-like events           backend.cc:537-540 + the sparse loop with the event code of
+ *                                                    include/genn/genn/weightUpdateModels.h:308-319 (StaticGraded)
  *                        postsynaptic (learnPost)    backend.cc:2029-2095
  *   gc_update_neurons    spike queue reset           src/genn/genn/code_generator/neuronUpdateGroupMerged.cc:947-975
  *                        neuron loop + op order      backend.cc:187-398, neuronUpdateGroupMerged.cc:552-773 (PSM :66-137, CS :20-55,
  *                                                    WU pre/post :333-459), spike emission backend.cc:2119-2133
+ *                        event conditions            neuronUpdateGroupMerged.cc:215-330, 677-683; emission backend.cc genEmitEvent
  *                        model arithmetic            include/genn/genn/neuronModels.h:163-186 (Izhikevich), :220-257 (LIF), :274-286
  *                                                    (SpikeSourceArray); postsynapticModels.h:91-106 (ExpCurr), DeltaCurr;
  *                                                    currentSourceModels.h:70-77 (DC); weightUpdateModels.h:236-287;
@@ -38,11 +41,18 @@
 
 enum { GC_LIF = 0, GC_IZH = 1, GC_SSA = 2 };
 enum { GC_EXPCURR = 0, GC_DELTACURR = 1 };
-enum { GC_STATIC = 0, GC_STATIC_DELAY = 1, GC_STDP_TRACE = 2 };
+enum { GC_STATIC = 0, GC_STATIC_DELAY = 1, GC_STDP_TRACE = 2, GC_STATIC_GRADED = 3 };
 enum { GC_SPARSE = 0, GC_CONV2D = 1, GC_DENSE = 2, GC_BITMASK = 3 };
 enum { GC_CS_DC = 0, GC_CS_NOISE = 1 };
 
 #define GC_MAX_CHILD 16
+#define GC_MAX_EVENT 4
+
+/* one spike-like event queue of a population ("SynSpikeEvent" child): condition V > threshold */
+typedef struct {
+    float threshold;
+    uint32_t *spkEvent, spkCntEvent;
+} gc_event;
 
 typedef struct {
     int kind;            /* GC_EXPCURR / GC_DELTACURR */
@@ -78,6 +88,7 @@ typedef struct {
     uint32_t numDelaySlots, spkQuePtr;
     uint32_t *spkRing, *spkCntRing;
     uint32_t *recordSpk;    /* [numRec * ceil(n/32)] or NULL */
+    int numEvents; gc_event events[GC_MAX_EVENT];
 } gc_pop;
 
 typedef struct {
@@ -91,6 +102,7 @@ typedef struct {
     uint32_t delaySteps;    /* axonal delay in timesteps: reads slot (spkQuePtr + slots - delaySteps) % slots of the source */
     const uint32_t *gp;     /* BITMASK connectivity words */
     float constantWeight;   /* StaticPulseConstantWeight (weightUpdateModels.h:202-213): used when g is NULL */
+    int event; float epre, vslope;   /* StaticGraded: which of the source's event queues it reads, and its parameters */
     uint64_t events;        /* synaptic events processed so far (bookkeeping, not in the reference) */
 } gc_syn;
 
@@ -201,6 +213,24 @@ int gc_add_syn_sparse(gc_net *net, int src, int trg, int psm, int wum, uint32_t 
     return net->numSyns - 1;
 }
 
+/* StaticGraded (weightUpdateModels.h:308-319) on a SPARSE projection added with wum = GC_STATIC_GRADED: the source population
+ * gets an event queue for the condition V > Epre — one per distinct threshold, as the reference fuses the event queues of
+ * projections whose condition and parameters agree (neuronGroup.cc:505-517) */
+void gc_set_static_graded(gc_net *net, int syn, float epre, float vslope)
+{
+    gc_syn *s = &net->syns[syn];
+    gc_pop *p = &net->pops[s->src];
+    s->epre = epre; s->vslope = vslope;
+    for(int e = 0; e < p->numEvents; e++) {
+        if(p->events[e].threshold == epre) { s->event = e; return; }
+    }
+    s->event = p->numEvents;
+    p->events[p->numEvents].threshold = epre;
+    p->events[p->numEvents].spkEvent = (uint32_t*)calloc(p->n ? p->n : 1, sizeof(uint32_t));
+    p->events[p->numEvents].spkCntEvent = 0;
+    p->numEvents++;
+}
+
 /* sT is initialised to -TIME_MAX (= -FLT_MAX) exactly as the reference's generated initialize() does */
 static void gc_need_st(gc_pop *p)
 {
@@ -293,6 +323,27 @@ void gc_update_synapses(gc_net *net, float t)
             srcSpkCnt = src->spkCntRing[slot];
         }
         gc_psm *psm = &trg->psm[s->psm];
+        if(s->wum == GC_STATIC_GRADED) {
+            /* spike-like events (backend.cc:537-540, the same row loop as true spikes with the event code); V_pre is the
+             * source's V as it stands now, i.e. after the update — and reset — of the step that emitted the event */
+            const gc_event *ev = &src->events[s->event];
+            for(uint32_t i = 0; i < ev->spkCntEvent; i++) {
+                const uint32_t idPre = ev->spkEvent[i];
+                const uint32_t npost = s->rowLength[idPre];
+                s->events += npost;
+                for(uint32_t j = 0; j < npost; j++) {
+                    const uint32_t idSyn = (idPre * s->rowStride) + j;
+                    /* The generated C++ reads `outPost[idPost] += fmax(0.0f, g[idSyn] * tanh((V[idPre] - Epre) / Vslope) * DT)` and
+                     * includes only <cmath>, which leaves the double versions of tanh and fmax as the only ones in the global
+                     * namespace: the argument is an fp32 quotient, everything after it — the product, the maximum and the
+                     * addition to outPost — is double arithmetic, rounded to fp32 by the store. */
+                    const float x = (src->v0[idPre] - s->epre) / s->vslope;
+                    const double release = fmax((double)0.0f, (double)s->g[idSyn] * tanh((double)x) * (double)net->dt);
+                    psm->outPost[s->ind[idSyn]] = (float)((double)psm->outPost[s->ind[idSyn]] + release);
+                }
+            }
+            continue;
+        }
         if(s->matrix == GC_CONV2D) {
             const int kh = s->conv[0], kw = s->conv[1], iw = s->conv[3], ic = s->conv[4];
             const int oh = s->conv[5], ow = s->conv[6], oc = s->conv[7];
@@ -401,6 +452,7 @@ void gc_update_neurons(gc_net *net, float t, uint32_t recordingTimestep)
             p->spk = p->spkRing + (size_t)p->spkQuePtr * p->n;
         }
         p->spkCnt = 0;
+        for(int e = 0; e < p->numEvents; e++) { p->events[e].spkCntEvent = 0; }
     }
     for(int k = 0; k < net->numPops; k++) {
         gc_pop *p = &net->pops[k];
@@ -472,6 +524,10 @@ void gc_update_neurons(gc_net *net, float t, uint32_t recordingTimestep)
             /* WU pre / post dynamics run every step, before the threshold test */
             if(p->preTrace) { p->preTrace[i] *= p->preDecay; }
             if(p->postTrace) { p->postTrace[i] *= p->postDecay; }
+            /* spike-like event conditions: after the sim code, before the threshold test (neuronUpdateGroupMerged.cc:677-683) */
+            for(int e = 0; e < p->numEvents; e++) {
+                if(l0 > p->events[e].threshold) { p->events[e].spkEvent[p->events[e].spkCntEvent++] = i; }
+            }
             spiked = (p->model == GC_LIF) ? (l1 <= 0.0f && l0 >= p->p[4]) : (l0 >= 29.99f);
             if(spiked) {
                 if(p->preTrace) { p->preTrace[i] += 1.0f; }
@@ -517,6 +573,9 @@ uint32_t *gc_record(gc_net *net, int pop) { return net->pops[pop].recordSpk; }
 float *gc_syn_g(gc_net *net, int syn) { return net->syns[syn].g; }
 uint32_t *gc_col_length(gc_net *net, int syn) { return net->syns[syn].colLength; }
 uint32_t *gc_remap(gc_net *net, int syn) { return net->syns[syn].remap; }
+uint32_t gc_event_count(const gc_net *net, int pop, int event) { return net->pops[pop].events[event].spkCntEvent; }
+const uint32_t *gc_events(const gc_net *net, int pop, int event) { return net->pops[pop].events[event].spkEvent; }
+int gc_syn_event_queue(const gc_net *net, int syn) { return net->syns[syn].event; }
 uint64_t gc_syn_events(const gc_net *net, int syn) { return net->syns[syn].events; }
 uint64_t gc_timestep(const gc_net *net) { return net->timestep; }
 
@@ -529,6 +588,7 @@ void gc_destroy(gc_net *net)
         for(int m = 0; m < p->numPSM; m++) { free(p->psm[m].outPost); free(p->psm[m].denDelay); }
         free(p->preTrace); free(p->postTrace); free(p->sT); free(p->recordSpk);
         if(p->spkRing) { free(p->spkRing); free(p->spkCntRing); } else { free(p->spk); }
+        for(int e = 0; e < p->numEvents; e++) { free(p->events[e].spkEvent); }
     }
     for(int k = 0; k < net->numSyns; k++) { free(net->syns[k].colLength); free(net->syns[k].remap); }
     free(net->pops); free(net->syns); free(net);

@@ -22,7 +22,7 @@ SRC = os.path.join(HERE, "genn_cpu.c")
 
 GC_LIF, GC_IZH, GC_SSA = 0, 1, 2
 GC_EXPCURR, GC_DELTACURR = 0, 1
-GC_STATIC, GC_STATIC_DELAY, GC_STDP_TRACE = 0, 1, 2
+GC_STATIC, GC_STATIC_DELAY, GC_STDP_TRACE, GC_STATIC_GRADED = 0, 1, 2, 3
 GC_CS_DC, GC_CS_NOISE = 0, 1
 
 
@@ -67,6 +67,10 @@ def lib():
         for name in ("gc_syn_g", "gc_col_length", "gc_remap"):
             getattr(l, name).restype = vp; getattr(l, name).argtypes = [vp, i32]
         l.gc_syn_events.restype = u64; l.gc_syn_events.argtypes = [vp, i32]
+        l.gc_set_static_graded.restype = None; l.gc_set_static_graded.argtypes = [vp, i32, f32, f32]
+        l.gc_event_count.restype = u32; l.gc_event_count.argtypes = [vp, i32, i32]
+        l.gc_events.restype = vp; l.gc_events.argtypes = [vp, i32, i32]
+        l.gc_syn_event_queue.restype = i32; l.gc_syn_event_queue.argtypes = [vp, i32]
         l.gc_timestep.restype = u64; l.gc_timestep.argtypes = [vp]
         l.gc_destroy.restype = None; l.gc_destroy.argtypes = [vp]
         _lib = l
@@ -131,7 +135,8 @@ class OracleNet:
             pre = any(s.wum == "stdp_trace" for s in out_syn[p.name])
             post = any(s.wum == "stdp_trace" for s in in_syn[p.name])
             slots = max([s.axonal_delay_steps for s in out_syn[p.name]], default=0) + 1
-            return (p.model, psm, cs, pre, post, slots)
+            events = len({float(s.wum_params["Epre"]) for s in out_syn[p.name] if s.wum == "static_graded"})
+            return (p.model, psm, cs, pre, post, slots, events)
 
         merged = {}
         for p in net.pops:
@@ -207,9 +212,16 @@ class OracleNet:
                 g = np.full(ind.shape, literal_f32(s.wum_params["g"]), np.float32) if s.wum == "static_const" else _as(s.g, np.float32)
                 d = _as(s.d, np.uint8) if s.d is not None else None
                 self.keep += [rl, ind, g, d]
-                wum = {"static": GC_STATIC, "static_const": GC_STATIC, "static_delay": GC_STATIC_DELAY, "stdp_trace": GC_STDP_TRACE}[s.wum]
+                wum = {"static": GC_STATIC, "static_const": GC_STATIC, "static_delay": GC_STATIC_DELAY, "stdp_trace": GC_STDP_TRACE,
+                       "static_graded": GC_STATIC_GRADED}[s.wum]
                 sid = self.l.gc_add_syn_sparse(self.h, src, trg, self.psm_id[s.name], wum, s.row_stride, rl.ctypes.data, ind.ctypes.data,
                                                g.ctypes.data, d.ctypes.data if d is not None else None, int(s.wum == "stdp_trace"))
+                if s.wum == "static_graded":
+                    # Epre and Vslope are literals when every graded projection has the same value, struct fields otherwise
+                    graded = [x for x in net.syns if x.wum == "static_graded" and x.matrix == "sparse"]
+                    k = graded.index(s)
+                    self.l.gc_set_static_graded(self.h, sid, C.c_float(_round_group([x.wum_params["Epre"] for x in graded])[k]),
+                                                C.c_float(_round_group([x.wum_params["Vslope"] for x in graded])[k]))
                 if s.wum == "stdp_trace":
                     q = s.wum_params
                     stride = (col_stride or {}).get(s.name)
@@ -308,6 +320,12 @@ class OracleNet:
     def record(self, pop, num_rec):
         n = self.net.pop(pop).n
         return self._arr(self.l.gc_record(self.h, self.pop_id[pop]), num_rec * ((n + 31) // 32), np.uint32)
+
+    def spike_events(self, syn):
+        """The spike-like event queue a graded projection read last / will read next (ids in ascending order)."""
+        s = self.net.syn(syn)
+        pop, q = self.pop_id[s.src], self.l.gc_syn_event_queue(self.h, self.syn_id[syn])
+        return self._arr(self.l.gc_events(self.h, pop, q), self.l.gc_event_count(self.h, pop, q), np.uint32).copy()
 
     def events(self):
         return sum(self.l.gc_syn_events(self.h, i) for i in self.syn_id.values())

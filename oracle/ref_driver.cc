@@ -80,6 +80,22 @@ public:
 };
 IMPLEMENT_SNIPPET(TraceSTDP);
 
+// The built-in WeightUpdateModels::StaticGraded (weightUpdateModels.h:308-319) with one identifier changed: its event code
+// reads the presynaptic potential as `V_pre`, but the 5.4.0 code generator exposes a presynaptic neuron variable reference
+// under its own name (`V`; synapseUpdateGroupMerged.cc:62-69), so the built-in does not transpile ("Undefined identifier"
+// at 'V_pre').  Everything else is the built-in's.
+class GradedSynapse : public WeightUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(GradedSynapse);
+    SET_PARAMS({"Epre", "Vslope"});
+    SET_VARS({{"g", "scalar", VarAccess::READ_ONLY}});
+    SET_PRE_NEURON_VAR_REFS({{"V", "scalar", VarAccessMode::READ_ONLY}});
+    SET_PRE_EVENT_THRESHOLD_CONDITION_CODE("V > Epre");
+    SET_PRE_EVENT_SYN_CODE("addToPost(fmax(0.0, g * tanh((V - Epre) / Vslope) * dt));\n");
+};
+IMPLEMENT_SNIPPET(GradedSynapse);
+
 // Current source fed from a host-pregenerated array; the driver rewrites the N-element
 // window before every step, so the injected value at step s is noise[s*N + id].
 class ArrayNoise : public CurrentSourceModels::Base
@@ -174,6 +190,7 @@ int main(int argc, char *argv[])
                     if(s.wum == "static_delay") { ls >> s.maxDenDelay; }
                     else if(s.wum == "stdp_trace" || s.wum == "stdp") { s.wumP.resize(6); for(auto &c : s.wumP) ls >> c; }
                     else if(s.wum == "static_const") { s.wumP.resize(1); ls >> s.wumP[0]; }
+                    else if(s.wum == "static_graded") { s.wumP.resize(2); ls >> s.wumP[0] >> s.wumP[1]; }
                     else if(s.wum != "static") throw std::runtime_error("wum " + s.wum);
                     ls >> s.psm;
                     if(s.psm == "expcurr") { s.psmP.resize(1); ls >> s.psmP[0]; }
@@ -227,6 +244,15 @@ int main(int argc, char *argv[])
             WeightUpdateModels::Init wum = initWeightUpdate<WeightUpdateModels::StaticPulse>({}, {{"g", uninitialisedVar()}});
             if(s.wum == "static_const") {
                 wum = initWeightUpdate<WeightUpdateModels::StaticPulseConstantWeight>({{"g", s.wumP[0]}});
+            }
+            else if(s.wum == "static_graded") {
+#ifdef DRIVER_BACKEND_MI355X
+                // the adapter recognises the built-in as it stands (it never transpiles the event code)
+                wum = initWeightUpdate<WeightUpdateModels::StaticGraded>(
+#else
+                wum = initWeightUpdate<GradedSynapse>(
+#endif
+                    {{"Epre", s.wumP[0]}, {"Vslope", s.wumP[1]}}, {{"g", uninitialisedVar()}}, {}, {}, {{"V", std::string("V")}});
             }
             else if(s.wum == "static_delay") {
                 wum = initWeightUpdate<WeightUpdateModels::StaticPulseDendriticDelay>({}, {{"g", uninitialisedVar()}, {"d", uninitialisedVar()}});

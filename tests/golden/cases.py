@@ -33,5 +33,9 @@ def dense_small():
     return configs.dense_bitmask(), 25
 
 
-CASES = {"va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+def graded_small():
+    return configs.graded(), 25
+
+
+CASES = {"graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
          "stdp_small": stdp_small, "conv_small": conv_small}
