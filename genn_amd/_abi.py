@@ -10,11 +10,12 @@ MAX_PSM = 8
 MAX_CS = 4
 MAX_EXTRA_SPK = 3
 MAX_SPK_EVENT = 2
+MAX_PRE_OUTPUT = 2
 
 NEURON_LIF, NEURON_IZHIKEVICH, NEURON_SPIKE_SOURCE_ARRAY = 0, 1, 2
 PSM_EXPCURR, PSM_DELTACURR = 0, 1
 CS_DC, CS_ARRAY = 0, 1
-WUM_STATIC_PULSE, WUM_STATIC_PULSE_DENDRITIC_DELAY, WUM_STDP_TRACE, WUM_STATIC_PULSE_CONSTANT_WEIGHT, WUM_STATIC_GRADED = 0, 1, 2, 3, 4
+WUM_STATIC_PULSE, WUM_STATIC_PULSE_DENDRITIC_DELAY, WUM_STDP_TRACE, WUM_STATIC_PULSE_CONSTANT_WEIGHT, WUM_STATIC_GRADED, WUM_STATIC_PULSE_REVERSE = 0, 1, 2, 3, 4, 5
 MATRIX_SPARSE, MATRIX_TOEPLITZ_CONV2D, MATRIX_DENSE, MATRIX_BITMASK, MATRIX_PROCEDURAL = 0, 1, 2, 3, 4
 CONNECT_SNIPPETS = {"FixedProbability": 0, "FixedProbabilityNoAutapse": 1, "FixedNumberPostWithReplacement": 2}
 SPAN_AUTO, SPAN_POST, SPAN_PRE = 0, 1, 2
@@ -52,7 +53,8 @@ class NeuronUpdateGroup(C.Structure):
                 ("sT", p_f32), ("spkCnt", p_u32), ("spk", p_u32), ("recordSpk", p_u32),
                 ("numExtraSpk", C.c_uint32), ("numDelaySlots", C.c_uint32),
                 ("extraSpkCnt", p_u32 * MAX_EXTRA_SPK), ("extraSpk", p_u32 * MAX_EXTRA_SPK),
-                ("numSpkEvent", C.c_uint32), ("pad2_", C.c_uint32), ("spkEvent", SpikeEvent * MAX_SPK_EVENT)]
+                ("numSpkEvent", C.c_uint32), ("numPreOutput", C.c_uint32), ("spkEvent", SpikeEvent * MAX_SPK_EVENT),
+                ("outPre", p_f32 * MAX_PRE_OUTPUT)]
 
 
 class Procedural(C.Structure):
@@ -73,7 +75,7 @@ class PresynapticUpdateGroup(C.Structure):
                 ("conv", C.c_int32 * 8),
                 ("gp", p_u32), ("constantWeight", C.c_float), ("axonalDelaySteps", C.c_uint32),
                 ("numSrcDelaySlots", C.c_uint32), ("pad3_", C.c_uint32), ("procedural", Procedural),
-                ("srcV", p_f32), ("gradedEpre", C.c_float), ("gradedVslope", C.c_float)]
+                ("srcV", p_f32), ("gradedEpre", C.c_float), ("gradedVslope", C.c_float), ("outPre", p_f32)]
 
 
 class PostsynapticUpdateGroup(C.Structure):

@@ -207,6 +207,8 @@ unsigned int recogniseWUM(const WeightUpdateModels::Base *m, const std::string &
     }
     if(isTraceSTDP(m)) { return GENNMI_WUM_STDP_TRACE; }
     if(isStaticGraded(m)) { return GENNMI_WUM_STATIC_GRADED; }
+    // presynaptic output: the static_pulse_reverse model of the reference's tests/features/test_event_propagation.py:584-590
+    if(plain && same(m->getPreSpikeSynCode(), "addToPre(g);") && m->getVars().size() == 1 && m->getVars()[0].name == "g") { return GENNMI_WUM_STATIC_PULSE_REVERSE; }
     unsupported("weight update model of projection '" + name + "'");
 }
 
@@ -297,7 +299,7 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
                                                               || arch.isSpikeEventRecordingEnabled())) {
                     unsupported("delay slots, event times or event recording with spike-like events on population '" + arch.getName() + "'");
                 }
-                if(!n.getMergedOutSynPreOutputGroups().empty()) { unsupported("presynaptic output into population '" + arch.getName() + "'"); }
+                if(n.getMergedOutSynPreOutputGroups().size() > GENNMI_MAX_PRE_OUTPUT) { unsupported("more than 2 presynaptic outputs into population '" + arch.getName() + "'"); }
 
                 // values of one quantity across the groups of this merged group
                 auto perGroup = [&n](auto fn)
@@ -503,6 +505,17 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
                                      << "); d.spkEvent[" << k << "].threshold = v[g]; }" << std::endl;
                 }
                 out << "d.numSpkEvent = " << events.size() << "u;" << std::endl;
+                // presynaptic output of outgoing projections ("OutSynPreOutput" children, neuronUpdateGroupMerged.cc:148-165)
+                const auto &reverse = n.getMergedOutSynPreOutputGroups();
+                for(size_t k = 0; k < reverse.size(); k++) {
+                    auto &child = const_cast<NeuronUpdateGroupMerged::OutSynPreOutput&>(reverse[k]);
+                    if(child.getArchetype().getPreTargetVar() != "Isyn") { unsupported("presynaptic output into a variable other than Isyn ('" + child.getArchetype().getName() + "')"); }
+                    EnvironmentGroupMergedField<NeuronUpdateGroupMerged::OutSynPreOutput, NeuronUpdateGroupMerged> renv(env, child, n);
+                    renv.addField(scalar.createPointer(), "_mi_outPre", "outPreOutSyn" + std::to_string(child.getIndex()),
+                                  [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, "outPre"); });
+                    renv.getStream() << "d.outPre[" << k << "] = gennmiDev(" << renv["_mi_outPre"] << ");" << std::endl;
+                }
+                out << "d.numPreOutput = " << reverse.size() << "u;" << std::endl;
                 if(arch.isSpikeTimeRequired()) { out << "d.sT = gennmiDev(" << env["_st"] << ");" << std::endl; }
                 if(arch.isSpikeRecordingEnabled()) { out << "d.recordSpk = gennmiDev(" << env["_record_spk"] << ");" << std::endl; }
                 out << "GENNMI_CHECK(gennmi_push_neuron_update_group(gennmiRunner, &d, nullptr));" << std::endl;
@@ -650,6 +663,10 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                         << "; d.axonalDelaySteps = a[g]; d.numSrcDelaySlots = b[g]; }" << std::endl;
                 }
                 out << "d.outPost = gennmiDev(" << env["_out_post"] << ");" << std::endl;
+                if(wumKind == GENNMI_WUM_STATIC_PULSE_REVERSE) {
+                    if(!sparse || srcDelay) { unsupported("presynaptic output on a non-SPARSE or axonally delayed projection ('" + arch.getName() + "')"); }
+                    out << "d.outPre = gennmiDev(" << env["_out_pre"] << ");" << std::endl;
+                }
                 if(constantWeight) {
                     out << "{ static const float v[] = " << table(values([](const SynapseGroupInternal &g){ return g.getWUInitialiser().getParams().at("g"); }), scalar)
                         << "; d.constantWeight = v[g]; }" << std::endl;

@@ -268,6 +268,30 @@ def graded(n_a=300, n_b=130, n_c=64, steps=200, seed=13, dt=0.5):
     return net
 
 
+def reverse(n_a=260, n_b=90, steps=200, seed=21, dt=1.0):
+    """Presynaptic ("reverse") output: population A spikes, and every synapse of its projection to B adds its weight to
+    the spiking neuron's own input (`addToPre(g)`), here a self-inhibition that grows with the neuron's out-degree; B
+    projects back the ordinary way, and has a reverse projection of its own onto a sparser matrix."""
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.7, TauRefrac=2.0)
+    net = Net(name="reverse", dt=dt, steps=steps, seed=seed)
+    net.pops.append(Pop("A", "lif", n_a, dict(lif), {"V": (-60.0 + 9.5 * rng.uniform(seed, 1, 0, n_a)).astype(np.float32),
+                                                     "RefracTime": np.zeros(n_a, np.float32)}))
+    net.pops.append(Pop("B", "lif", n_b, dict(lif, Ioffset=0.58), {"V": (-60.0 + 9.5 * rng.uniform(seed, 2, 0, n_b)).astype(np.float32),
+                                                                   "RefracTime": np.zeros(n_b, np.float32)}))
+
+    def sparse(name, src, trg, n_src, n_trg, stride, stream, lo, hi, wum):
+        ind = np.sort(rng.randint(seed, stream, 0, n_src * stride, n_trg).reshape(n_src, stride), axis=1).astype(np.uint32)
+        row_length = (stride - rng.randint(seed, stream + 1, 0, n_src, stride // 2)).astype(np.uint32)    # ragged: half to full rows
+        g = (lo + (hi - lo) * rng.uniform(seed, stream + 2, 0, n_src * stride)).astype(np.float32).reshape(n_src, stride)
+        return Syn(name, src, trg, psm="expcurr", tau=5.0, row_stride=stride, row_length=row_length, ind=ind, g=g, wum=wum)
+
+    net.syns.append(sparse("AB_reverse", "A", "B", n_a, n_b, 36, 10, -0.8, 0.1, "static_reverse"))
+    net.syns.append(sparse("AB_forward", "A", "B", n_a, n_b, 12, 20, 0.0, 0.08, "static"))
+    net.syns.append(sparse("BA_forward", "B", "A", n_b, n_a, 20, 30, -0.2, 0.1, "static"))
+    net.syns.append(sparse("BA_reverse", "B", "A", n_b, n_a, 7, 40, -1.5, 0.0, "static_reverse"))
+    return net
+
+
 def dense_layer(n_in=8192, n_out=8192, rate_hz=50.0, steps=1000, seed=17, dt=1.0, w_sd=0.02):
     """A fully connected spiking layer: Poisson sources (rate_hz per source) into LIF neurons through a DENSE matrix
     with individual weights ~ N(0, w_sd); the shape of the dense layers of rate-coded classifiers."""

@@ -347,6 +347,14 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
                     if(j < npost && !(G.skipZeroDelay && slot == denPtr)) { atomicAddF32(&denDelay[(size_t)slot * numTrg + ip], w); }
                 }
             }
+            else if(g.wum == GENNMI_WUM_STATIC_PULSE_REVERSE) {
+                // addToPre(g): the weights of the row go to the spiking neuron itself; a lane sums its share, the lanes of the
+                // (spike, chunk) item combine theirs, one atomic per item
+                float sum = 0.0f;
+                for(uint32_t q = 0; q < perLane; q++) { if(inRow && j + q < npost) { sum += weight[rowBase + j + q]; } }
+                for(uint32_t off = W / 2; off > 0; off >>= 1) { sum += __shfl_xor(sum, off, WAVE); }
+                if(lis == 0 && sum != 0.0f) { atomicAddF32(asGlobal(g.outPre) + (size_t)batch * g.numSrcNeurons + idPre, sum); }
+            }
             else if(g.wum == GENNMI_WUM_STATIC_GRADED) {
                 // event code of weightUpdateModels.h:318: addToPost(fmax(0.0, g * tanh((V_pre - Epre) / Vslope) * dt)).  The CPU
                 // backend's generated code evaluates tanh, the products and the maximum in double (only the double versions of
@@ -918,8 +926,10 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
             // descriptor in memory, so a store in between would force the compiler to re-read the descriptor
             // and would serialise the loads, and each dependent access costs about a microsecond at the start of
             // a launch (nothing is cached yet).  Sums keep the reference's order (PSMs, then current sources).
-            float lin[GENNMI_MAX_PSM], front[GENNMI_MAX_PSM], inj[GENNMI_MAX_CS];
-            const uint32_t numPSM = g.numPSM, numCS = g.numCS;
+            float lin[GENNMI_MAX_PSM], front[GENNMI_MAX_PSM], inj[GENNMI_MAX_CS], rev[GENNMI_MAX_PRE_OUTPUT];
+            const uint32_t numPSM = g.numPSM, numCS = g.numCS, numRev = g.numPreOutput;
+            #pragma unroll
+            for(uint32_t q = 0; q < GENNMI_MAX_PRE_OUTPUT; q++) { rev[q] = (q < numRev) ? asGlobal(g.outPre[q])[bi] : 0.0f; }
             l0 = asGlobal(g.var0)[bi]; l1 = asGlobal(g.var1)[bi];
             #pragma unroll
             for(uint32_t m = 0; m < GENNMI_MAX_PSM; m++) {
@@ -957,8 +967,13 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
                     lin[m] = linSyn;
                 }
             }
+            // presynaptic output of the outgoing projections: after the postsynaptic models, before the current sources
+            #pragma unroll
+            for(uint32_t q = 0; q < GENNMI_MAX_PRE_OUTPUT; q++) { if(q < numRev) { Isyn += rev[q]; } }
             #pragma unroll
             for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) { if(c < numCS) { Isyn += inj[c]; } }
+            #pragma unroll
+            for(uint32_t q = 0; q < GENNMI_MAX_PRE_OUTPUT; q++) { if(q < numRev) { asGlobal(g.outPre[q])[bi] = 0.0f; } }
             #pragma unroll
             for(uint32_t m = 0; m < GENNMI_MAX_PSM; m++) {
                 if(m < numPSM) {
@@ -2078,6 +2093,9 @@ int gennmi_push_neuron_update_group(gennmi_runner *r, const gennmi_neuron_update
     for(uint32_t q = 0; q < g->numExtraSpk; q++) {
         if(!g->extraSpkCnt[q] || !g->extraSpk[q]) { return fail(GENNMI_EINVAL, "push_neuron_update_group: extra spike array missing"); }
     }
+    if(g->numPreOutput > GENNMI_MAX_PRE_OUTPUT) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: too many presynaptic outputs"); }
+    if(g->numPreOutput && g->model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: presynaptic output into a spike source"); }
+    for(uint32_t q = 0; q < g->numPreOutput; q++) { if(!g->outPre[q]) { return fail(GENNMI_EINVAL, "push_neuron_update_group: outPre missing"); } }
     if(g->numSpkEvent > GENNMI_MAX_SPK_EVENT) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: too many spike-like event conditions"); }
     if(g->numSpkEvent && (g->model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY || g->numDelaySlots > 1)) {
         return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: spike-like events need a LIF or Izhikevich group without delay slots");
@@ -2097,7 +2115,7 @@ int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynap
 {
     if(!r || !g) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: null argument"); }
     if(r->finalised) { return fail(GENNMI_ESTATE, "push_presynaptic_update_group: runner already finalised"); }
-    if(!g->srcSpk || !g->srcSpkCnt || !g->outPost) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: required array missing"); }
+    if(!g->srcSpk || !g->srcSpkCnt || (!g->outPost && g->wum != GENNMI_WUM_STATIC_PULSE_REVERSE)) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: required array missing"); }
     if(g->numSrcNeurons == 0 || g->numTrgNeurons == 0) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: empty population"); }
     if(g->matrix == GENNMI_MATRIX_PROCEDURAL) {
         const gennmi_procedural_t &q = g->procedural;
@@ -2164,6 +2182,9 @@ int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynap
             if(!g->trgST || !g->postTrace) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: STDP arrays missing"); }
             if(r->batch != 1) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: plastic weights need batch size 1"); }
         }
+        else if(g->wum == GENNMI_WUM_STATIC_PULSE_REVERSE) {
+            if(!g->outPre) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: outPre missing"); }
+        }
         else if(g->wum == GENNMI_WUM_STATIC_GRADED) {
             if(!g->srcV || !(g->gradedVslope != 0.0f)) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: graded synapses need the source's V and a non-zero Vslope"); }
             if(g->numSrcDelaySlots > 1) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: axonal delay on a graded projection"); }
@@ -2217,7 +2238,7 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
     if(r->batch != 1 || !r->post.empty() || r->pre.empty() || !r->dense.empty() || !r->proc.empty() || r->neuron.size() > RES_MAX_GROUPS) { return GENNMI_OK; }
     for(const auto &n : r->neuron) {
         const auto &g = n.g;
-        if((g.model != GENNMI_NEURON_LIF && g.model != GENNMI_NEURON_IZHIKEVICH) || g.preTrace || g.postTrace || g.sT || g.numDelaySlots > 1 || g.numSpkEvent) { return GENNMI_OK; }
+        if((g.model != GENNMI_NEURON_LIF && g.model != GENNMI_NEURON_IZHIKEVICH) || g.preTrace || g.postTrace || g.sT || g.numDelaySlots > 1 || g.numSpkEvent || g.numPreOutput) { return GENNMI_OK; }
         for(uint32_t c = 0; c < g.numCS; c++) { if(g.cs[c].kind != GENNMI_CS_DC) { return GENNMI_OK; } }
     }
     // tiles and their LDS layout

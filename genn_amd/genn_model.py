@@ -75,7 +75,7 @@ def init_postsynaptic(snippet, params=None, vars=None):
 
 
 def init_weight_update(snippet, params=None, vars=None, pre_vars=None, post_vars=None):
-    if snippet not in ("StaticPulse", "StaticPulseConstantWeight", "StaticPulseDendriticDelay", "STDPTrace", "StaticGraded"):
+    if snippet not in ("StaticPulse", "StaticPulseConstantWeight", "StaticPulseDendriticDelay", "STDPTrace", "StaticGraded", "StaticPulseReverse"):
         raise NotImplementedError(f"weight update model {snippet}")
     return _Init(snippet, params, vars, pre_vars, post_vars)
 
@@ -220,6 +220,7 @@ class NeuronGroup:
         self.post_trace_owner = None
         self.needs_spike_time = False
         self.num_delay_slots = 1     # longest axonal delay of the outgoing projections + 1, set by build()
+        self.pre_output_syn = []     # outgoing projections whose code calls addToPre
         self.event_thresholds = []   # one spike-like event queue per distinct threshold of the outgoing graded projections
 
     @property
@@ -399,6 +400,8 @@ class GeNNModel:
                                           "FixedProbabilityNoAutapse or FixedNumberPostWithReplacement")
             if weight_update_init.snippet not in ("StaticPulse", "StaticPulseConstantWeight"):
                 raise NotImplementedError(f"PROCEDURAL connectivity with {weight_update_init.snippet}")
+        if weight_update_init.snippet == "StaticPulseReverse" and (matrix_type != "SPARSE" or source.neuron == "SpikeSourceArray"):
+            raise NotImplementedError("StaticPulseReverse needs SPARSE connectivity and a source population with an input current")
         if weight_update_init.snippet == "StaticGraded":
             if matrix_type != "SPARSE":
                 raise NotImplementedError("StaticGraded needs SPARSE connectivity")
@@ -454,6 +457,9 @@ class GeNNModel:
             for s in n.out_syn:
                 if s.wu.snippet == "StaticGraded" and float(s.wu.params["Epre"]) not in n.event_thresholds:
                     n.event_thresholds.append(float(s.wu.params["Epre"]))
+            n.pre_output_syn = [s for s in n.out_syn if s.wu.snippet == "StaticPulseReverse"]
+            if len(n.pre_output_syn) > _abi.MAX_PRE_OUTPUT:
+                raise NotImplementedError(f"{n.name}: more than {_abi.MAX_PRE_OUTPUT} projections with presynaptic output")
             if len(n.event_thresholds) > _abi.MAX_SPK_EVENT:
                 raise NotImplementedError(f"{n.name}: more than {_abi.MAX_SPK_EVENT} spike-like event conditions")
             n.pre_trace_owner = pre[0] if pre else None
@@ -518,6 +524,8 @@ class GeNNModel:
                     n.vars[v] = a
             n.vars["spkCnt"] = self._alloc(B * n.num_delay_slots, np.uint32)
             n.vars["spk"] = self._alloc(B * n.num_delay_slots * N, np.uint32)
+            for s in n.pre_output_syn:
+                s.vars["outPre"] = self._alloc(B * N, np.float32)
             for e in range(len(n.event_thresholds)):
                 n.vars[f"spkCntEvent{e}"] = self._alloc(B, np.uint32)
                 n.vars[f"spkEvent{e}"] = self._alloc(B * N, np.uint32)
@@ -665,7 +673,7 @@ class GeNNModel:
     def _neuron_merge_key(self, n):
         psm = tuple((grp[0].ps.snippet, self._den_delay(grp[0])) for grp in self._sorted_psm(n))
         return (n.neuron, psm, tuple(cs.kind for cs in n.current_sources), n.pre_trace_owner is not None,
-                n.post_trace_owner is not None, n.needs_spike_time, n.spike_recording_enabled, n.num_delay_slots, len(n.event_thresholds))
+                n.post_trace_owner is not None, n.needs_spike_time, n.spike_recording_enabled, n.num_delay_slots, len(n.event_thresholds), len(n.pre_output_syn))
 
     def _sorted_psm(self, n):
         # children are ordered by a structure-only digest, ties keep creation order (groupMerged.h:411-454)
@@ -707,6 +715,10 @@ class GeNNModel:
                     d.var0, d.var1 = n.vars["V"].ptr, n.vars["U"].ptr
                     for j in range(4):
                         d.params[j] = rounded[j][k]
+            for d, n in zip(descs, members):
+                d.numPreOutput = len(n.pre_output_syn)
+                for q, s in enumerate(n.pre_output_syn):
+                    d.outPre[q] = s.vars["outPre"].ptr
             # spike-like event children
             for e in range(len(members[0].event_thresholds)):
                 thresholds = _merge_round([n.event_thresholds[e] for n in members])
@@ -779,7 +791,7 @@ class GeNNModel:
                             "BITMASK": _abi.MATRIX_BITMASK, "PROCEDURAL": _abi.MATRIX_PROCEDURAL}[s.matrix_type]
                 d.wum = {"StaticPulse": _abi.WUM_STATIC_PULSE, "StaticPulseDendriticDelay": _abi.WUM_STATIC_PULSE_DENDRITIC_DELAY,
                          "STDPTrace": _abi.WUM_STDP_TRACE, "StaticPulseConstantWeight": _abi.WUM_STATIC_PULSE_CONSTANT_WEIGHT,
-                         "StaticGraded": _abi.WUM_STATIC_GRADED}[s.wu.snippet]
+                         "StaticGraded": _abi.WUM_STATIC_GRADED, "StaticPulseReverse": _abi.WUM_STATIC_PULSE_REVERSE}[s.wu.snippet]
                 if s.wu.snippet == "StaticPulseConstantWeight":
                     d.constantWeight = consts[k]
                     if s.matrix_type == "SPARSE":
@@ -791,6 +803,8 @@ class GeNNModel:
                 d.outPost = owner.vars["outPost"].ptr
                 d.srcSpkCnt, d.srcSpk = s.src.vars["spkCnt"].ptr, s.src.vars["spk"].ptr
                 d.axonalDelaySteps, d.numSrcDelaySlots = s.axonal_delay_steps, s.src.num_delay_slots
+                if s.wu.snippet == "StaticPulseReverse":
+                    d.outPre = s.vars["outPre"].ptr
                 if s.wu.snippet == "StaticGraded":
                     # the projection is driven by the source's event queue for its threshold, not by its spikes
                     e = s.src.event_thresholds.index(float(s.wu.params["Epre"]))
@@ -964,6 +978,8 @@ def model_from_net(net, batch_size=1, record=True, span=None, device=0):
             wu = init_weight_update("StaticPulseConstantWeight", {"g": s.wum_params["g"]})
         elif s.wum == "static_graded":
             wu = init_weight_update("StaticGraded", s.wum_params, {"g": 0.0})
+        elif s.wum == "static_reverse":
+            wu = init_weight_update("StaticPulseReverse", {}, {"g": 0.0})
         else:
             wu = init_weight_update("STDPTrace", s.wum_params, {"g": 0.0}, {"preTrace": 0.0}, {"postTrace": 0.0})
         if s.matrix == "dense":

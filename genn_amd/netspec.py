@@ -47,6 +47,7 @@ class Syn:
     trg: str
     matrix: str = "sparse"          # "sparse" | "conv2d" | "dense" | "bitmask"
     wum: str = "static"             # "static" | "static_delay" | "stdp_trace" | "static_const" (one weight, wum_params["g"])
+                                    # | "static_reverse" (addToPre(g): the row's weights go back to the spiking neuron)
                                     # | "static_graded" (spike-like events, wum_params["Epre"], ["Vslope"]; source must have a V)
     wum_params: Dict[str, float] = field(default_factory=dict)
     psm: str = "expcurr"            # "expcurr" | "deltacurr"
@@ -165,8 +166,8 @@ def write_netspec(net: Net, path: str):
             head = f"syn {s.name} conv2d {s.src} {s.trg} " + " ".join(str(int(s.conv[k])) for k in CONV_PARAMS)
         if s.wum != "static_const":
             np.ascontiguousarray(s.g, dtype=np.float32).tofile(os.path.join(path, f"{s.name}.g.f32"))
-        if s.wum == "static":
-            w = "static"
+        if s.wum in ("static", "static_reverse"):
+            w = s.wum
         elif s.wum == "static_const":
             w = f"static_const {float(s.wum_params['g'])!r}"
         elif s.wum == "static_delay":

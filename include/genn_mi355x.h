@@ -48,7 +48,10 @@ enum { GENNMI_WUM_STATIC_PULSE = 0, GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY = 1,
        GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT = 3, /* weightUpdateModels.h:202-213: one weight for the whole projection */
        /* weightUpdateModels.h:308-319: no spike code; while the presynaptic V exceeds Epre the neuron emits a spike-like
         * event every step, and each event adds fmax(0, g * tanh((V_pre - Epre) / Vslope) * dt) per synapse */
-       GENNMI_WUM_STATIC_GRADED = 4 };
+       GENNMI_WUM_STATIC_GRADED = 4,
+       /* presynaptic-spike code `addToPre(g);` (the static_pulse_reverse model of tests/features/test_event_propagation.py:584-590):
+        * every synapse of a spiking neuron's row adds its weight to that neuron's own outPre (SPARSE only) */
+       GENNMI_WUM_STATIC_PULSE_REVERSE = 5 };
 /* connectivity: ragged SPARSE (runtime.cc:360-402) or TOEPLITZ Conv2D (initToeplitzConnectivitySnippet.h:105-150) */
 enum { GENNMI_MATRIX_SPARSE = 0, GENNMI_MATRIX_TOEPLITZ_CONV2D = 1,
        /* DENSE: g[numSrc*numTrg], idSyn = idPre*numTrg + idPost; BITMASK: one bit per pair, most significant bit first,
@@ -126,6 +129,7 @@ typedef struct gennmi_cs_t {              /* one current source child (neuronUpd
  * true spikes; backend.cc genEmitEvent).  The queue is rewritten every step.  Projections whose weight update model has
  * an event threshold read it as their srcSpk / srcSpkCnt. */
 #define GENNMI_MAX_SPK_EVENT 2
+#define GENNMI_MAX_PRE_OUTPUT 2
 typedef struct gennmi_spike_event_t {
     uint32_t *spkCntEvent;                /* [batch] */
     uint32_t *spkEvent;                   /* [batch*numNeurons] */
@@ -160,8 +164,12 @@ typedef struct gennmi_neuron_update_group_t {      /* MergedNeuronUpdateGroup<i>
     uint32_t numDelaySlots;
     uint32_t *extraSpkCnt[GENNMI_MAX_EXTRA_SPK];
     uint32_t *extraSpk[GENNMI_MAX_EXTRA_SPK];
-    uint32_t numSpkEvent, pad2_;          /* LIF and Izhikevich groups without delay slots only */
+    uint32_t numSpkEvent;                 /* LIF and Izhikevich groups without delay slots only */
+    /* Presynaptic output ("OutSynPreOutput" children, neuronUpdateGroupMerged.cc:148-165): after the postsynaptic models and
+     * before the current sources, Isyn += outPre[id]; outPre[id] = 0 for each outgoing projection whose code calls addToPre */
+    uint32_t numPreOutput;
     gennmi_spike_event_t spkEvent[GENNMI_MAX_SPK_EVENT];
+    float *outPre[GENNMI_MAX_PRE_OUTPUT]; /* [batch*numNeurons] each */
 } gennmi_neuron_update_group_t;
 
 /* What gennmi_init_sparse_* and gennmi_init_var would have stored for a projection, for GENNMI_MATRIX_PROCEDURAL: the row
@@ -210,6 +218,7 @@ typedef struct gennmi_presynaptic_update_group_t { /* MergedPresynapticUpdateGro
      * read when the event is delivered, i.e. after the update (and reset) that emitted it */
     const float *srcV;                    /* [batch*numSrcNeurons] the source population's V */
     float gradedEpre, gradedVslope;
+    float *outPre;                        /* GENNMI_WUM_STATIC_PULSE_REVERSE: [batch*numSrcNeurons], the source's presynaptic output */
 } gennmi_presynaptic_update_group_t;
 
 typedef struct gennmi_postsynaptic_update_group_t { /* MergedPostsynapticUpdateGroup<i> */

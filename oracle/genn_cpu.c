@@ -14,6 +14,7 @@
  *                        Toeplitz presynaptic loop   backend.cc:1788-1883, include/genn/genn/initToeplitzConnectivitySnippet.h:116-137
  *                        dense / bitmask loop        backend.cc:1985-2021 (bit gid = idPre*rowStride + idPost, most significant bit
  *                                                    first; row stride = numPost padded to 32, backend.cc:1393-1404)
+ *                        presynaptic output          addToPre backend.cc:1822; consumed neuronUpdateGroupMerged.cc:148-165, 591-595
  *                        spike-like events           backend.cc:537-540 + the sparse loop with the event code of
  *                                                    include/genn/genn/weightUpdateModels.h:308-319 (StaticGraded)
  *                        postsynaptic (learnPost)    backend.cc:2029-2095
@@ -41,7 +42,7 @@
 
 enum { GC_LIF = 0, GC_IZH = 1, GC_SSA = 2 };
 enum { GC_EXPCURR = 0, GC_DELTACURR = 1 };
-enum { GC_STATIC = 0, GC_STATIC_DELAY = 1, GC_STDP_TRACE = 2, GC_STATIC_GRADED = 3 };
+enum { GC_STATIC = 0, GC_STATIC_DELAY = 1, GC_STDP_TRACE = 2, GC_STATIC_GRADED = 3, GC_STATIC_REVERSE = 4 };
 enum { GC_SPARSE = 0, GC_CONV2D = 1, GC_DENSE = 2, GC_BITMASK = 3 };
 enum { GC_CS_DC = 0, GC_CS_NOISE = 1 };
 
@@ -89,6 +90,8 @@ typedef struct {
     uint32_t *spkRing, *spkCntRing;
     uint32_t *recordSpk;    /* [numRec * ceil(n/32)] or NULL */
     int numEvents; gc_event events[GC_MAX_EVENT];
+    /* presynaptic output of outgoing projections whose code calls addToPre ("OutSynPreOutput" children) */
+    int numPreOutput; float *outPre[GC_MAX_EVENT];
 } gc_pop;
 
 typedef struct {
@@ -103,6 +106,7 @@ typedef struct {
     const uint32_t *gp;     /* BITMASK connectivity words */
     float constantWeight;   /* StaticPulseConstantWeight (weightUpdateModels.h:202-213): used when g is NULL */
     int event; float epre, vslope;   /* StaticGraded: which of the source's event queues it reads, and its parameters */
+    int preOutput;          /* GC_STATIC_REVERSE: which outPre of the source it adds to */
     uint64_t events;        /* synaptic events processed so far (bookkeeping, not in the reference) */
 } gc_syn;
 
@@ -229,6 +233,15 @@ void gc_set_static_graded(gc_net *net, int syn, float epre, float vslope)
     p->events[p->numEvents].spkEvent = (uint32_t*)calloc(p->n ? p->n : 1, sizeof(uint32_t));
     p->events[p->numEvents].spkCntEvent = 0;
     p->numEvents++;
+}
+
+/* A SPARSE projection added with wum = GC_STATIC_REVERSE (presynaptic-spike code `addToPre(g);`): the source gets an outPre */
+void gc_set_static_reverse(gc_net *net, int syn)
+{
+    gc_syn *s = &net->syns[syn];
+    gc_pop *p = &net->pops[s->src];
+    s->preOutput = p->numPreOutput;
+    p->outPre[p->numPreOutput++] = (float*)calloc(p->n ? p->n : 1, sizeof(float));
 }
 
 /* sT is initialised to -TIME_MAX (= -FLT_MAX) exactly as the reference's generated initialize() does */
@@ -402,6 +415,10 @@ void gc_update_synapses(gc_net *net, float t)
                 if(s->wum == GC_STATIC) {
                     psm->outPost[idPost] += s->g[idSyn];
                 }
+                else if(s->wum == GC_STATIC_REVERSE) {
+                    /* addToPre(x): outPre[idPre] += x (backend.cc:1822) */
+                    net->pops[s->src].outPre[s->preOutput][idPre] += s->g[idSyn];
+                }
                 else if(s->wum == GC_STATIC_DELAY) {
                     psm->denDelay[(size_t)((psm->denDelayPtr + s->d[idSyn]) % psm->maxDenDelay) * trg->n + idPost] += s->g[idSyn];
                 }
@@ -497,6 +514,11 @@ void gc_update_neurons(gc_net *net, float t, uint32_t recordingTimestep)
                 }
                 psm->outPost[i] = linSyn;
             }
+            /* presynaptic output: after the incoming postsynaptic models, before the current sources (neuronUpdateGroupMerged.cc:585-600) */
+            for(int q = 0; q < p->numPreOutput; q++) {
+                Isyn += p->outPre[q][i];
+                p->outPre[q][i] = 0.0f;
+            }
             for(int c = 0; c < p->numCS; c++) {
                 Isyn += (p->cs[c].kind == GC_CS_DC) ? p->cs[c].amp : p->cs[c].noise[(size_t)(step % p->cs[c].noiseSteps) * p->n + i];
             }
@@ -573,6 +595,7 @@ uint32_t *gc_record(gc_net *net, int pop) { return net->pops[pop].recordSpk; }
 float *gc_syn_g(gc_net *net, int syn) { return net->syns[syn].g; }
 uint32_t *gc_col_length(gc_net *net, int syn) { return net->syns[syn].colLength; }
 uint32_t *gc_remap(gc_net *net, int syn) { return net->syns[syn].remap; }
+float *gc_out_pre(gc_net *net, int syn) { return net->pops[net->syns[syn].src].outPre[net->syns[syn].preOutput]; }
 uint32_t gc_event_count(const gc_net *net, int pop, int event) { return net->pops[pop].events[event].spkCntEvent; }
 const uint32_t *gc_events(const gc_net *net, int pop, int event) { return net->pops[pop].events[event].spkEvent; }
 int gc_syn_event_queue(const gc_net *net, int syn) { return net->syns[syn].event; }
@@ -589,6 +612,7 @@ void gc_destroy(gc_net *net)
         free(p->preTrace); free(p->postTrace); free(p->sT); free(p->recordSpk);
         if(p->spkRing) { free(p->spkRing); free(p->spkCntRing); } else { free(p->spk); }
         for(int e = 0; e < p->numEvents; e++) { free(p->events[e].spkEvent); }
+        for(int q = 0; q < p->numPreOutput; q++) { free(p->outPre[q]); }
     }
     for(int k = 0; k < net->numSyns; k++) { free(net->syns[k].colLength); free(net->syns[k].remap); }
     free(net->pops); free(net->syns); free(net);

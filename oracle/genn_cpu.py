@@ -22,7 +22,7 @@ SRC = os.path.join(HERE, "genn_cpu.c")
 
 GC_LIF, GC_IZH, GC_SSA = 0, 1, 2
 GC_EXPCURR, GC_DELTACURR = 0, 1
-GC_STATIC, GC_STATIC_DELAY, GC_STDP_TRACE, GC_STATIC_GRADED = 0, 1, 2, 3
+GC_STATIC, GC_STATIC_DELAY, GC_STDP_TRACE, GC_STATIC_GRADED, GC_STATIC_REVERSE = 0, 1, 2, 3, 4
 GC_CS_DC, GC_CS_NOISE = 0, 1
 
 
@@ -68,6 +68,8 @@ def lib():
             getattr(l, name).restype = vp; getattr(l, name).argtypes = [vp, i32]
         l.gc_syn_events.restype = u64; l.gc_syn_events.argtypes = [vp, i32]
         l.gc_set_static_graded.restype = None; l.gc_set_static_graded.argtypes = [vp, i32, f32, f32]
+        l.gc_set_static_reverse.restype = None; l.gc_set_static_reverse.argtypes = [vp, i32]
+        l.gc_out_pre.restype = vp; l.gc_out_pre.argtypes = [vp, i32]
         l.gc_event_count.restype = u32; l.gc_event_count.argtypes = [vp, i32, i32]
         l.gc_events.restype = vp; l.gc_events.argtypes = [vp, i32, i32]
         l.gc_syn_event_queue.restype = i32; l.gc_syn_event_queue.argtypes = [vp, i32]
@@ -136,7 +138,8 @@ class OracleNet:
             post = any(s.wum == "stdp_trace" for s in in_syn[p.name])
             slots = max([s.axonal_delay_steps for s in out_syn[p.name]], default=0) + 1
             events = len({float(s.wum_params["Epre"]) for s in out_syn[p.name] if s.wum == "static_graded"})
-            return (p.model, psm, cs, pre, post, slots, events)
+            reverse = sum(s.wum == "static_reverse" for s in out_syn[p.name])
+            return (p.model, psm, cs, pre, post, slots, events, reverse)
 
         merged = {}
         for p in net.pops:
@@ -213,9 +216,11 @@ class OracleNet:
                 d = _as(s.d, np.uint8) if s.d is not None else None
                 self.keep += [rl, ind, g, d]
                 wum = {"static": GC_STATIC, "static_const": GC_STATIC, "static_delay": GC_STATIC_DELAY, "stdp_trace": GC_STDP_TRACE,
-                       "static_graded": GC_STATIC_GRADED}[s.wum]
+                       "static_graded": GC_STATIC_GRADED, "static_reverse": GC_STATIC_REVERSE}[s.wum]
                 sid = self.l.gc_add_syn_sparse(self.h, src, trg, self.psm_id[s.name], wum, s.row_stride, rl.ctypes.data, ind.ctypes.data,
                                                g.ctypes.data, d.ctypes.data if d is not None else None, int(s.wum == "stdp_trace"))
+                if s.wum == "static_reverse":
+                    self.l.gc_set_static_reverse(self.h, sid)
                 if s.wum == "static_graded":
                     # Epre and Vslope are literals when every graded projection has the same value, struct fields otherwise
                     graded = [x for x in net.syns if x.wum == "static_graded" and x.matrix == "sparse"]
@@ -320,6 +325,10 @@ class OracleNet:
     def record(self, pop, num_rec):
         n = self.net.pop(pop).n
         return self._arr(self.l.gc_record(self.h, self.pop_id[pop]), num_rec * ((n + 31) // 32), np.uint32)
+
+    def out_pre(self, syn):
+        s = self.net.syn(syn)
+        return self._arr(self.l.gc_out_pre(self.h, self.syn_id[syn]), self.net.pop(s.src).n, np.float32)
 
     def spike_events(self, syn):
         """The spike-like event queue a graded projection read last / will read next (ids in ascending order)."""

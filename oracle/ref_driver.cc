@@ -96,6 +96,16 @@ public:
 };
 IMPLEMENT_SNIPPET(GradedSynapse);
 
+// Presynaptic ("reverse") output: the static_pulse_reverse model of tests/features/test_event_propagation.py:584-590
+class StaticPulseReverse : public WeightUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(StaticPulseReverse);
+    SET_VARS({{"g", "scalar", VarAccess::READ_ONLY}});
+    SET_PRE_SPIKE_SYN_CODE("addToPre(g);\n");
+};
+IMPLEMENT_SNIPPET(StaticPulseReverse);
+
 // Current source fed from a host-pregenerated array; the driver rewrites the N-element
 // window before every step, so the injected value at step s is noise[s*N + id].
 class ArrayNoise : public CurrentSourceModels::Base
@@ -191,7 +201,7 @@ int main(int argc, char *argv[])
                     else if(s.wum == "stdp_trace" || s.wum == "stdp") { s.wumP.resize(6); for(auto &c : s.wumP) ls >> c; }
                     else if(s.wum == "static_const") { s.wumP.resize(1); ls >> s.wumP[0]; }
                     else if(s.wum == "static_graded") { s.wumP.resize(2); ls >> s.wumP[0] >> s.wumP[1]; }
-                    else if(s.wum != "static") throw std::runtime_error("wum " + s.wum);
+                    else if(s.wum != "static" && s.wum != "static_reverse") throw std::runtime_error("wum " + s.wum);
                     ls >> s.psm;
                     if(s.psm == "expcurr") { s.psmP.resize(1); ls >> s.psmP[0]; }
                     else if(s.psm != "deltacurr") throw std::runtime_error("psm " + s.psm);
@@ -244,6 +254,9 @@ int main(int argc, char *argv[])
             WeightUpdateModels::Init wum = initWeightUpdate<WeightUpdateModels::StaticPulse>({}, {{"g", uninitialisedVar()}});
             if(s.wum == "static_const") {
                 wum = initWeightUpdate<WeightUpdateModels::StaticPulseConstantWeight>({{"g", s.wumP[0]}});
+            }
+            else if(s.wum == "static_reverse") {
+                wum = initWeightUpdate<StaticPulseReverse>({}, {{"g", uninitialisedVar()}});
             }
             else if(s.wum == "static_graded") {
 #ifdef DRIVER_BACKEND_MI355X

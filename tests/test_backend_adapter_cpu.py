@@ -40,7 +40,7 @@ def _exports(lib):
     return {line.split()[-1] for line in out.splitlines() if " T " in line}
 
 
-@pytest.mark.parametrize("case", ["stdp_small", "potjans_small", "conv_small", "dense_small", "va_delay_small", "graded_small"])
+@pytest.mark.parametrize("case", ["stdp_small", "potjans_small", "conv_small", "dense_small", "va_delay_small", "graded_small", "reverse_small"])
 def test_generated_runner_exports_reference_entry_points(case):
     net, tmp, code = _generate(case)
     try:

@@ -99,3 +99,52 @@ def test_graded_synapses_through_run():
     compare_state(net, model, oracle, "after run(230)", exact=False)
     assert model.synaptic_event_count == oracle.events()
     model.unload()
+
+
+# ---- presynaptic ("reverse") output: addToPre --------------------------------------------------------------------------
+def _reverse_lock_step(net, steps, exact):
+    from parity import assert_close
+    model = model_from_net(net)
+    model.load(num_recording_timesteps=steps)
+    info = model.runner_info()
+    assert not info["single_launch_step"] and not info["resident_plan"]
+    oracle = OracleNet(net, num_recording_timesteps=steps)
+    spikes, fed_back = 0, 0.0
+    for step in range(steps):
+        model.update_synapses()
+        oracle.update_synapses()
+        for name in ("AB_reverse", "BA_reverse"):
+            got = model.synapse_populations[name].vars["outPre"].pull_from_device()
+            want = oracle.out_pre(name)
+            assert_close(got, want, f"step {step}: outPre of {name}", exact, accumulator=True)
+            fed_back += float(np.abs(want).sum())
+        model.update_neurons()
+        oracle.update_neurons()
+        for name in ("AB_reverse", "BA_reverse"):
+            assert not model.synapse_populations[name].vars["outPre"].pull_from_device().any(), "outPre is consumed by the neuron update"
+        for p in net.pops:
+            want = oracle.spikes(p.name)
+            assert np.array_equal(model.neuron_populations[p.name].current_spikes[0], want), f"step {step}: spike queue of {p.name}"
+            spikes += len(want)
+        if (step + 1) % 10 == 0:
+            compare_state(net, model, oracle, f"step {step}", exact=False)
+    assert model.synaptic_event_count == oracle.events()
+    assert spikes > 500 and fed_back > 100.0
+    model.unload()
+
+
+def test_reverse_output_exact_with_dyadic_weights():
+    """Weights that are multiples of 1/8: the sum of a row is exact in any order and outPre starts every step at zero, so
+    outPre must equal the oracle's bit for bit although the GPU adds a row's weights by wavefront reduction.  (The
+    forward projections' ExpCurr accumulators carry a decayed remainder, so they stay within tolerance only.)"""
+    net = configs.reverse()
+    for s in net.syns:
+        s.g = (np.round(s.g * 8.0) / 8.0).astype(np.float32)
+    _reverse_lock_step(net, 100, exact=True)
+
+
+def test_reverse_output_matches_the_oracle():
+    """The fixture's network (arbitrary weights): identical spike queues over the first 100 steps, outPre and state within
+    1e-5 (a row's weights are summed in a different order)."""
+    net = configs.reverse()
+    _reverse_lock_step(net, 100, exact=False)
