@@ -116,6 +116,75 @@ def bench_init(args):
     print(json.dumps(out))
 
 
+def bench_procedural(args, stored):
+    """--workload izh_procedural / izh_stored: the 10^6-neuron, 10^9-synapse Izhikevich network with its connectivity and
+    weights regenerated for every spike (PROCEDURAL: nothing stored), or its stored twin built on the device from the same
+    seed (SPARSE).  800,000 excitatory and 200,000 inhibitory neurons; every neuron has 800 + 200 targets
+    (FixedNumberPostWithReplacement per target population), weights U[0, 0.5) from excitatory and U[-1, 0) from inhibitory
+    rows; DeltaCurr input; a cycled array of U[0, 5) noise."""
+    import numpy as np
+    from genn_amd import netgen
+    from genn_amd.genn_model import GeNNModel, init_postsynaptic, init_sparse_connectivity, init_var, init_weight_update
+    n_e, n_i, rows = 800_000, 200_000, 8
+    t0 = time.time()
+    model = GeNNModel("float", "izh_procedural", dt=1.0)
+    model.seed = 777
+    izh = dict(a=0.02, b=0.2, c=-65.0, d=8.0)
+    pops = {"E": model.add_neuron_population("E", n_e, "Izhikevich", izh, {"V": -65.0, "U": -13.0}),
+            "I": model.add_neuron_population("I", n_i, "Izhikevich", izh, {"V": -65.0, "U": -13.0})}
+    for k, (name, n) in enumerate((("E", n_e), ("I", n_i))):
+        cs = model.add_current_source(name + "_noise", "ArrayNoise", pops[name])
+        cs.set_extra_global_param("noise", netgen.uniform_f32(777, 12 + k, 0, rows * n, 5.0, 0.0).reshape(rows, n))
+        pops[name].spike_recording_enabled = True
+    matrix = "SPARSE" if stored else "PROCEDURAL"
+    for src, lo, hi in (("E", 0.0, 0.5), ("I", -1.0, 0.0)):
+        for trg, num in (("E", 800), ("I", 200)):
+            model.add_synapse_population(src + trg, matrix, pops[src], pops[trg],
+                                         init_weight_update("StaticPulse", {}, {"g": init_var("Uniform", {"min": lo, "max": hi})}),
+                                         init_postsynaptic("DeltaCurr"), init_sparse_connectivity("FixedNumberPostWithReplacement", {"num": num}))
+    model.build()
+    model.load(num_recording_timesteps=args.warmup + args.steps)
+    model.synchronize()
+    load_s = time.time() - t0
+    model.run(args.warmup)
+    model.synchronize()
+    ev0 = model.synaptic_event_count
+    t0 = time.perf_counter()
+    model.run(args.steps)
+    model.synchronize()
+    wall = time.perf_counter() - t0
+    events = model.synaptic_event_count - ev0
+    model.pull_recording_buffers_from_device()
+    rates = {name: round(len(p.spike_recording_data[0][1]) / p.num_neurons / ((args.warmup + args.steps) / 1000.0), 3) for name, p in pops.items()}
+    roofline = None
+    if args.profile_steps > 0:
+        model.set_timing(True)
+        evp0 = model.synaptic_event_count
+        model.run(args.profile_steps)
+        model.synchronize()
+        st = model.kernel_stats()
+        evp = model.synaptic_event_count - evp0
+        avg_s = st["presyn_seconds"] / max(1, st["presyn_launches"])
+        # algorithmic bytes per event: the fp32 read-modify-write of outPost, plus the stored index and weight if there are any
+        bpe = 16 if stored else 8
+        achieved = evp / max(1, st["presyn_launches"]) * bpe / avg_s / 1e9
+        roofline = {"bound": "hbm", "kernel": "presynapticUpdateKernel (+ presynapticTileKernel)" if stored else "presynapticProceduralKernel",
+                    "achieved": round(achieved, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6), "traffic": None,
+                    "bytes_per_event": bpe, "events_per_launch": round(evp / max(1, st["presyn_launches"]), 1), "avg_launch_us": round(avg_s * 1e6, 3),
+                    "events_per_s_in_kernel": round(evp / st["presyn_seconds"], 1) if st["presyn_seconds"] else None,
+                    "neuron_kernel_avg_us": round(st["neuron_seconds"] / max(1, st["neuron_launches"]) * 1e6, 3)}
+    model.unload()
+    print(json.dumps({
+        "metric": "synaptic_events_per_s", "value": round(events / wall, 1), "unit": "events/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall / args.steps * 1e3, 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "10^6 Izhikevich neurons, 10^9 synapses, " + ("stored on the device (SPARSE, built there)" if stored else "PROCEDURAL (regenerated per spike)"),
+                   "neurons": n_e + n_i, "synapses": (n_e + n_i) * 1000, "dt_ms": 1.0, "seed": 777},
+        "gsop_per_s": round(events / wall / 1e9, 4), "wall_s_per_sim_s": round(wall / (args.steps / 1000.0), 4),
+        "events_per_step": round(events / args.steps, 1), "firing_rates_hz": rates, "setup_s": {"build_and_load": round(load_s, 2)},
+        "roofline": roofline, "cpu_baseline": None}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -138,6 +207,8 @@ def main():
 
     if args.workload == "init_izhikevich":
         return bench_init(args)
+    if args.workload in ("izh_procedural", "izh_stored"):
+        return bench_procedural(args, stored=(args.workload == "izh_stored"))
 
     import numpy as np
     from genn_amd.genn_model import model_from_net

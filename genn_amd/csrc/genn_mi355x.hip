@@ -480,28 +480,54 @@ __global__ __launch_bounds__(BLOCK)
 void presynapticProceduralKernel(const ProcGroupDev * __restrict__ blocks, unsigned long long *eventCounter)
 {
     using namespace gennmi_rows;
+    constexpr uint32_t MAX_ROUNDS = 64;                 // rows of up to 16,383 targets are shared between the block's waves
+    __shared__ double shRoundTotal[MAX_ROUNDS];
     const ProcGroupDev &G = blocks[blockIdx.x];
     const gennmi_presynaptic_update_group_t &g = G.g;
     const uint32_t batch = blockIdx.y;
     const uint32_t lane = threadIdx.x & (WAVE - 1);
-    const uint32_t waveIdx = (blockIdx.x - G.startBlock) * (BLOCK / WAVE) + threadIdx.x / WAVE;
-    const uint32_t numWaves = G.numBlocks * (BLOCK / WAVE);
+    const uint32_t wave = threadIdx.x / WAVE;
+    const uint32_t localBlock = blockIdx.x - G.startBlock;
     const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
     GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
     GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
     const uint32_t rowStride = g.rowStride;
     unsigned long long events = 0;
-    for(uint32_t s = waveIdx; s < numSpikes; s += numWaves) {
-        const uint32_t row = spk[s];
-        const unsigned long long firstElement = (unsigned long long)row * rowStride;
-        if(g.procedural.connectivity == GENNMI_CONNECT_FIXED_NUMBER_POST) {
-            const uint32_t n = min(g.procedural.num, rowStride);
-            fixedNumberPostRow(row, g.numTrgNeurons, n, G.connectivity, lane, [&](uint32_t k, const uint32_t post[4]) {
-                for(int i = 0; i < 4 && k + i < n; i++) { atomicAddF32(&outPost[post[i]], valueAt(G.weightInit, G.weight, firstElement + k + i)); }
-            });
-            if(lane == 0) { events += n; }
+    if(g.procedural.connectivity == GENNMI_CONNECT_FIXED_NUMBER_POST) {
+        const uint32_t n = min(g.procedural.num, rowStride);
+        // a group of four synapses shares one generator call for its weights when the row starts on a multiple of four
+        const bool aligned = (rowStride & 3u) == 0;
+        auto deliver = [&](unsigned long long firstElement, uint32_t k, const uint32_t post[4]) {
+            float w[4];
+            if(aligned) { valuesAt4(G.weightInit, G.weight, firstElement + k, w); }
+            else { for(int i = 0; i < 4; i++) { w[i] = valueAt(G.weightInit, G.weight, firstElement + k + i); } }
+            for(int i = 0; i < 4 && k + i < n; i++) { atomicAddF32(&outPost[post[i]], w[i]); }
+        };
+        if(n / (4 * WAVE) + 1 > 1 && n / (4 * WAVE) + 1 <= MAX_ROUNDS) {
+            // long rows: one spike per block, the block's waves share the row's rounds of 256 draws
+            for(uint32_t s = localBlock; s < numSpikes; s += G.numBlocks) {
+                const uint32_t row = spk[s];
+                const unsigned long long firstElement = (unsigned long long)row * rowStride;
+                fixedNumberPostRowBlock<BLOCK / WAVE>(row, g.numTrgNeurons, n, G.connectivity, lane, wave, shRoundTotal, MAX_ROUNDS,
+                                                      [&](uint32_t k, const uint32_t post[4]) { deliver(firstElement, k, post); });
+                if(threadIdx.x == 0) { events += n; }
+            }
         }
         else {
+            const uint32_t numWaves = G.numBlocks * (BLOCK / WAVE);
+            for(uint32_t s = localBlock * (BLOCK / WAVE) + wave; s < numSpikes; s += numWaves) {
+                const uint32_t row = spk[s];
+                const unsigned long long firstElement = (unsigned long long)row * rowStride;
+                fixedNumberPostRow(row, g.numTrgNeurons, n, G.connectivity, lane, [&](uint32_t k, const uint32_t post[4]) { deliver(firstElement, k, post); });
+                if(lane == 0) { events += n; }
+            }
+        }
+    }
+    else {
+        const uint32_t numWaves = G.numBlocks * (BLOCK / WAVE);
+        for(uint32_t s = localBlock * (BLOCK / WAVE) + wave; s < numSpikes; s += numWaves) {
+            const uint32_t row = spk[s];
+            const unsigned long long firstElement = (unsigned long long)row * rowStride;
             const uint32_t total = fixedProbabilityRow(row, g.numTrgNeurons, G.probLogRecip,
                                                        g.procedural.connectivity == GENNMI_CONNECT_FIXED_PROBABILITY_NO_AUTAPSE, G.connectivity, lane,
                                                        [&](uint32_t k, uint32_t post) {

@@ -126,6 +126,18 @@ __device__ __forceinline__ float valueAt(const VarInit &v, const Stream &s, unsi
     return drawValue(v, s, group, (int)(e & 3), r, n);
 }
 
+// elements e0..e0+3 at once (e0 a multiple of four): the four share one generator call
+__device__ __forceinline__ void valuesAt4(const VarInit &v, const Stream &s, unsigned long long e0, float out[4])
+{
+    if(v.snippet == GENNMI_INIT_CONSTANT) { out[0] = out[1] = out[2] = out[3] = v.p[0]; return; }
+    const unsigned long long group = e0 >> 2;
+    const Words r = s.at(group, 0);
+    float n[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if(v.snippet == GENNMI_INIT_NORMAL || v.snippet == GENNMI_INIT_NORMAL_CLIPPED || v.snippet == GENNMI_INIT_NORMAL_CLIPPED_DELAY) { normals(r, n); }
+    #pragma unroll
+    for(int i = 0; i < 4; i++) { out[i] = drawValue(v, s, group, i, r, n); }
+}
+
 // FixedProbability / FixedProbabilityNoAutapse (include/genn/genn/initSparseConnectivitySnippet.h:170-187, 208-230), one row
 // by one wave64.  Lane l owns post indices [l*slice, (l+1)*slice) and walks them with the snippet's geometric skips
 // `prev += 1 + (int)(log(u) * probLogRecip)`; the walk is memoryless, so restarting it at a slice boundary, or stepping over
@@ -171,6 +183,28 @@ __device__ __forceinline__ uint32_t fixedProbabilityRow(uint32_t row, uint32_t n
 template<typename Sink>
 __device__ __forceinline__ void fixedNumberPostRow(uint32_t row, uint32_t numPost, uint32_t n, const Stream &s, uint32_t lane, Sink sink)
 {
+    if(n < 4 * WAVE) {
+        // a single round of draws: nothing to regenerate, the spacings stay in registers while the total is formed
+        const uint32_t k = 4 * lane;
+        const Words r = s.at(((unsigned long long)row << 32) | (k >> 2), 0);
+        double prefix[4];
+        double sum = 0.0;
+        #pragma unroll
+        for(int i = 0; i < 4; i++) {
+            sum += (k + i <= n) ? (double)-logf(uniformOpen(r.w[i])) : 0.0;
+            prefix[i] = sum;
+        }
+        const double inclusive = waveInclusiveScan(sum, (int)lane);
+        const double scale = (double)numPost / (0.0 + __shfl(inclusive, WAVE - 1, WAVE));
+        if(k < n) {
+            const double before = 0.0 + (inclusive - sum);
+            uint32_t post[4];
+            #pragma unroll
+            for(int i = 0; i < 4; i++) { post[i] = min((uint32_t)((before + prefix[i]) * scale), numPost - 1); }
+            sink(k, post);
+        }
+        return;
+    }
     double scale = 0.0;
     for(int pass = 0; pass < 2; pass++) {
         double carry = 0.0;
@@ -196,6 +230,86 @@ __device__ __forceinline__ void fixedNumberPostRow(uint32_t row, uint32_t numPos
         }
         scale = (double)numPost / carry;
     }
+}
+
+// The same row by the BLOCK_WAVES wavefronts of one work-group: wave w takes rounds w, w + BLOCK_WAVES, ... of 256 draws.  The
+// totals of the rounds go through `roundTotal` (LDS, one double per round, at most maxRounds), and every wave then adds them
+// up in round order — the additions, and so every bit of the result, are those of the one-wave version above.
+// Call with all threads of the block; returns false (nothing done) if the row has more rounds than maxRounds.
+template<uint32_t BLOCK_WAVES, typename Sink>
+__device__ __forceinline__ bool fixedNumberPostRowBlock(uint32_t row, uint32_t numPost, uint32_t n, const Stream &s, uint32_t lane, uint32_t wave,
+                                                        double *roundTotal, uint32_t maxRounds, Sink sink)
+{
+    const uint32_t rounds = n / (4 * WAVE) + 1;          // draws 0..n
+    if(rounds > maxRounds) { return false; }
+    if(rounds <= BLOCK_WAVES) {
+        // at most one round per wave: its spacings stay in registers while the totals are exchanged
+        const uint32_t round = wave;
+        const uint32_t k = round * 4 * WAVE + 4 * lane;
+        double prefix[4] = {0.0, 0.0, 0.0, 0.0};
+        double sum = 0.0, inclusive = 0.0;
+        if(round < rounds) {
+            const Words r = s.at(((unsigned long long)row << 32) | (k >> 2), 0);
+            #pragma unroll
+            for(int i = 0; i < 4; i++) {
+                sum += (k + i <= n) ? (double)-logf(uniformOpen(r.w[i])) : 0.0;
+                prefix[i] = sum;
+            }
+            inclusive = waveInclusiveScan(sum, (int)lane);
+            if(lane == WAVE - 1) { roundTotal[round] = inclusive; }
+        }
+        __syncthreads();
+        if(round < rounds && k < n) {
+            double total = 0.0, carry = 0.0;
+            for(uint32_t q = 0; q < rounds; q++) {
+                if(q == round) { carry = total; }
+                total += roundTotal[q];
+            }
+            const double scale = (double)numPost / total;
+            const double before = carry + (inclusive - sum);
+            uint32_t post[4];
+            #pragma unroll
+            for(int i = 0; i < 4; i++) { post[i] = min((uint32_t)((before + prefix[i]) * scale), numPost - 1); }
+            sink(k, post);
+        }
+        __syncthreads();
+        return true;
+    }
+    for(int pass = 0; pass < 2; pass++) {
+        double scale = 0.0;
+        if(pass == 1) {
+            __syncthreads();
+            double total = 0.0;
+            for(uint32_t r = 0; r < rounds; r++) { total += roundTotal[r]; }
+            scale = (double)numPost / total;
+        }
+        for(uint32_t round = wave; round < rounds; round += BLOCK_WAVES) {
+            const uint32_t k = round * 4 * WAVE + 4 * lane;
+            const Words r = s.at(((unsigned long long)row << 32) | (k >> 2), 0);
+            double prefix[4];
+            double sum = 0.0;
+            #pragma unroll
+            for(int i = 0; i < 4; i++) {
+                sum += (k + i <= n) ? (double)-logf(uniformOpen(r.w[i])) : 0.0;
+                prefix[i] = sum;
+            }
+            const double inclusive = waveInclusiveScan(sum, (int)lane);
+            if(pass == 0) {
+                if(lane == WAVE - 1) { roundTotal[round] = inclusive; }
+            }
+            else if(k < n) {
+                double carry = 0.0;
+                for(uint32_t q = 0; q < round; q++) { carry += roundTotal[q]; }
+                const double before = carry + (inclusive - sum);
+                uint32_t post[4];
+                #pragma unroll
+                for(int i = 0; i < 4; i++) { post[i] = min((uint32_t)((before + prefix[i]) * scale), numPost - 1); }
+                sink(k, post);
+            }
+        }
+    }
+    __syncthreads();            // roundTotal is reused by the next row
+    return true;
 }
 }   // namespace gennmi_rows
 
