@@ -203,7 +203,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
-                         "(the hot path is single-GPU; see DESIGN.md for how it would shard)")
+                         "(the hot path is single-GPU: sharded by postsynaptic neuron it would exchange only the spike lists each step)")
 
     if args.workload == "init_izhikevich":
         return bench_init(args)

@@ -128,6 +128,8 @@ struct NeuronGroupDev
     uint32_t *shadowCnt;                // [2][batch]
     uint32_t *spikeBitmap;              // [ceil(N/32)] engine-private bitmap of this step's spikes (populations with learnPost), or NULL
     unsigned long long *aggEvent;       // look-back area of the spike-like event queues (groups with events), or NULL
+    float *nextSpikeTime;               // spike sources: engine-private copy of spikeTimes[startSpike] per neuron (+inf: none left)
+    size_t spikeTimesBytes;             // spike sources: bytes from spikeTimes to the end of its allocation (host bookkeeping)
 };
 
 struct PreGroupDev
@@ -944,8 +946,11 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
         // WU pre/post dynamics, threshold, then (on a spike) WU pre/post spike code, sT, reset
         float l0 = 0, l1 = 0;
         uint32_t startSpike = 0;
+        float nextTime = 0.0f;
         if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
-            startSpike = g.startSpike[bi];
+            // one coalesced read instead of startSpike, endSpike and a gather from spikeTimes: the time of the neuron's next
+            // spike is kept beside the state and refreshed only when the neuron fires
+            nextTime = asGlobal(G.nextSpikeTime)[bi];
         }
         else {
             // Every load of this neuron's inputs is issued before the first store: the pointers come out of a
@@ -1033,13 +1038,17 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
         if(g.postTrace) { postTrace = g.postTrace[bi] * g.postDecay; }
         if(g.model == GENNMI_NEURON_LIF) { spiked = (l1 <= 0.0f && l0 >= g.params[4]); }
         else if(g.model == GENNMI_NEURON_IZHIKEVICH) { spiked = (l0 >= 29.99f); }
-        else { spiked = (startSpike != g.endSpike[bi]) && (t >= g.spikeTimes[startSpike]); }
+        else { spiked = (t >= nextTime); }       // startSpike != endSpike && t >= spikeTimes[startSpike] (neuronModels.h:274-286)
         vEvent = l0;           // spike-like event conditions see the updated V before any reset (neuronUpdateGroupMerged.cc:677-683)
         if(spiked) {
             preTrace += 1.0f; postTrace += 1.0f;
             if(g.sT) { g.sT[bi] = t; }
             if(g.model == GENNMI_NEURON_LIF) { l0 = g.params[5]; l1 = g.params[6]; }
-            else if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) { g.startSpike[bi] = startSpike + 1; }
+            else if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
+                startSpike = g.startSpike[bi] + 1;
+                g.startSpike[bi] = startSpike;
+                G.nextSpikeTime[bi] = (startSpike != g.endSpike[bi]) ? g.spikeTimes[startSpike] : INFINITY;
+            }
         }
         if(g.preTrace) { g.preTrace[bi] = preTrace; }
         if(g.postTrace) { g.postTrace[bi] = postTrace; }
@@ -1230,6 +1239,16 @@ __global__ void zeroDelayScanKernel(uint32_t numSrc, uint32_t rowStride, const u
 }
 
 // Advances the device-resident step state at the end of a captured graph.
+// spike sources: (re)build the per-neuron copy of the next spike time from the arrays the user owns
+__global__ void nextSpikeTimeKernel(const uint32_t *startSpike, const uint32_t *endSpike, const float *spikeTimes, float *next, size_t count)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if(i < count) {
+        const uint32_t s = startSpike[i];
+        next[i] = (s != endSpike[i]) ? spikeTimes[s] : INFINITY;
+    }
+}
+
 __global__ void advanceStepKernel(StepState *state, unsigned long long steps)
 {
     if(threadIdx.x == 0 && blockIdx.x == 0) { state->timestep += steps; state->epoch += steps; }
@@ -1879,6 +1898,7 @@ struct gennmi_runner
     uint32_t resTiles = 0, resReplicaStride = 0; size_t resLdsBytes = 0;
     std::vector<u32x4*> resSegs;        // segment table of each presynaptic group, in push order
     std::vector<uint32_t> resSegTiles;  // tiles of its target population
+    bool sourcesStale = false;          // startSpike / endSpike / spikeTimes of a spike source were written since nextSpikeTime was built
     bool resStale = false;              // connectivity or weights were written since the tables were built
     // graph
     hipGraphExec_t graphExec = nullptr; unsigned long long graphSteps = 0;
@@ -1902,6 +1922,12 @@ static void noteDeviceWrite(const void *dev, size_t bytes)
     std::lock_guard<std::mutex> lock(g_runnersMutex);
     const uintptr_t a = reinterpret_cast<uintptr_t>(dev), b = a + bytes;
     for(gennmi_runner *r : g_runners) {
+        for(const auto &n : r->neuron) {
+            if(n.g.model != GENNMI_NEURON_SPIKE_SOURCE_ARRAY || r->sourcesStale) { continue; }
+            const size_t perNeuron = (size_t)r->batch * n.g.numNeurons * sizeof(uint32_t);
+            const uintptr_t st = reinterpret_cast<uintptr_t>(n.g.startSpike), en = reinterpret_cast<uintptr_t>(n.g.endSpike);
+            if((a < st + perNeuron && st < b) || (a < en + perNeuron && en < b) || (a < reinterpret_cast<uintptr_t>(n.g.spikeTimes) + n.spikeTimesBytes && reinterpret_cast<uintptr_t>(n.g.spikeTimes) < b)) { r->sourcesStale = true; }
+        }
         if(!r->resident || r->resStale) { continue; }
         for(const auto &p : r->pre) {
             const size_t entries = (size_t)p.g.numSrcNeurons * p.g.rowStride;
@@ -2714,6 +2740,17 @@ int gennmi_runner_finalise(gennmi_runner *r)
     if(r->postLdsBytes > 48 * 1024) {
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(postsynapticUpdateKernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)r->postLdsBytes));
     }
+    // spike sources: per-neuron copy of the next spike time, built before the first step and again after writes to the arrays
+    for(auto &n : r->neuron) {
+        if(n.g.model != GENNMI_NEURON_SPIKE_SOURCE_ARRAY) { continue; }
+        // spikeTimes comes without a length: everything up to the end of its allocation counts as the array
+        hipDeviceptr_t base = nullptr; size_t size = 0;
+        HIP_TRY(hipMemGetAddressRange(&base, &size, const_cast<float*>(n.g.spikeTimes)));
+        n.spikeTimesBytes = (reinterpret_cast<uintptr_t>(base) + size) - reinterpret_cast<uintptr_t>(n.g.spikeTimes);
+        HIP_TRY(hipMalloc(&n.nextSpikeTime, (size_t)r->batch * n.g.numNeurons * sizeof(float)));
+        r->owned.push_back(n.nextSpikeTime);
+        r->sourcesStale = true;
+    }
     // look-back area of the spike-like event queues: per event slot, per-block counts then per-group totals
     if(anyEvents) {
         const size_t count = (size_t)GENNMI_MAX_SPK_EVENT * 2 * r->neuronBlocks * r->batch;
@@ -2774,6 +2811,26 @@ static int stamp(gennmi_runner *r, hipEvent_t *out)
     }
     *out = r->eventPool[r->eventNext++];
     HIP_TRY(hipEventRecord(*out, r->stream));
+    return GENNMI_OK;
+}
+
+// spike sources: bring the per-neuron copies of the next spike time up to date with arrays written since they were built
+static int refreshSpikeSources(gennmi_runner *r)
+{
+    bool stale;
+    {
+        std::lock_guard<std::mutex> lock(g_runnersMutex);
+        stale = r->sourcesStale;
+        r->sourcesStale = false;
+    }
+    if(!stale) { return GENNMI_OK; }
+    for(const auto &n : r->neuron) {
+        if(n.g.model != GENNMI_NEURON_SPIKE_SOURCE_ARRAY) { continue; }
+        const size_t count = (size_t)r->batch * n.g.numNeurons;
+        nextSpikeTimeKernel<<<dim3((unsigned int)((count + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, r->stream>>>(n.g.startSpike, n.g.endSpike, n.g.spikeTimes,
+                                                                                                              n.nextSpikeTime, count);
+        HIP_TRY(hipGetLastError());
+    }
     return GENNMI_OK;
 }
 
@@ -2852,6 +2909,7 @@ int gennmi_update_synapses(gennmi_runner *r, float t)
 int gennmi_update_neurons(gennmi_runner *r, float t, uint32_t recordingTimestep)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "update_neurons: runner not finalised"); }
+    { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
     StepArgs a{};
     a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recordingTimestep;
     const int rc = launchNeurons(r, a, r->timing);
@@ -2873,6 +2931,7 @@ int gennmi_step_time(gennmi_runner *r, unsigned long long timestep, unsigned lon
 int gennmi_step(gennmi_runner *r, float t, uint32_t recordingTimestep)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "step: runner not finalised"); }
+    { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
     if(r->fusedStep) {
         StepArgs a{};
         a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recordingTimestep;
@@ -2895,6 +2954,7 @@ int gennmi_step(gennmi_runner *r, float t, uint32_t recordingTimestep)
 int gennmi_run_steps(gennmi_runner *r, unsigned long long timestep, unsigned long long numSteps, unsigned long long numRecordingTimesteps)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "run_steps: runner not finalised"); }
+    { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
     constexpr unsigned long long CHUNK = 100;
     const StepState hs{timestep, r->epoch, numRecordingTimesteps};
     HIP_TRY(hipMemcpyAsync(r->dState, &hs, sizeof(hs), hipMemcpyHostToDevice, r->stream));

@@ -9,7 +9,7 @@ import os
 import numpy as np
 import pytest
 
-from genn_amd.genn_model import init_postsynaptic, init_toeplitz_connectivity, init_weight_update
+from genn_amd.genn_model import GeNNModel, init_postsynaptic, init_toeplitz_connectivity, init_weight_update
 
 pytestmark = pytest.mark.gpu
 
@@ -213,3 +213,49 @@ def test_device_copy(count):
     assert np.array_equal(got[:count], src.view[:count])
     assert np.all(got[count:] == -1.0)
     src.free(); dst.free()
+
+
+@pytest.mark.parametrize("replay", [False, True])
+def test_spike_source_arrays_rewritten_between_steps(replay):
+    """The neuron update keeps the time of each source's next spike beside its state instead of gathering
+    spikeTimes[startSpike] every step; that copy must follow the user's arrays.  After 25 steps the host rewinds startSpike
+    and shifts spikeTimes by 30 ms (the way new input is fed to a SpikeSourceArray): the same pattern must come out again,
+    30 steps later, through single steps and through replayed graphs."""
+    n, first = 300, 25
+    rng = np.random.default_rng(12)
+    per = rng.integers(0, 4, n)                                  # 0..3 spikes per source
+    end = np.cumsum(per).astype(np.uint32)
+    start = (end - per).astype(np.uint32)
+    times = np.concatenate([np.sort(rng.choice(20, k, replace=False)) for k in per] + [np.zeros(0)]).astype(np.float32)
+    model = GeNNModel("float", "rewrite", dt=1.0)
+    src = model.add_neuron_population("S", n, "SpikeSourceArray", {}, {"startSpike": start, "endSpike": end})
+    src.set_extra_global_param("spikeTimes", np.concatenate([times, [0.0]]))
+    src.spike_recording_enabled = True
+    model.build()
+    model.load(num_recording_timesteps=80)
+
+    def expected(offset):
+        want = np.zeros((80, n), bool)
+        for i in range(n):
+            for t in times[start[i]:end[i]]:
+                want[int(t) + offset, i] = True
+        return want
+
+    for _ in range(first):
+        model.step_time()
+    assert np.array_equal(src.vars["startSpike"].pull_from_device(), end)            # every source has used up its list
+    src.vars["spikeTimes"].view[:len(times)] = times + 30.0
+    src.vars["spikeTimes"].push_to_device()
+    src.vars["startSpike"].view[:] = start
+    src.vars["startSpike"].push_to_device()
+    if replay:
+        model.run(55)
+    else:
+        for _ in range(55):
+            model.step_time()
+    model.pull_recording_buffers_from_device()
+    words = src.vars["recordSpk"].view.reshape(80, -1)
+    got = np.unpackbits(words.view(np.uint8), axis=1, bitorder="little")[:, :n].astype(bool)
+    assert np.array_equal(got, expected(0) | expected(30))
+    assert got.sum() == 2 * per.sum() and per.sum() > 300
+    model.unload()
