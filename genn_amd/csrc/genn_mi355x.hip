@@ -844,30 +844,15 @@ void postsynapticUpdateKernel(const PostGroupDev * __restrict__ blocks, StepArgs
 }
 
 // ------------------------------------------------------------------------------------------------
-// Ordered append of the flagged neurons of a population to a queue, for spike-like events: the scheme the neuron
-// update uses for true spikes (ballot rank in the wave, LDS scan in the block, look-back over per-block counts tagged
-// with the step, blocks in groups of 64 with a published group total), as a function every block of the population
-// calls with all its threads.  `counts` and `groupTotals` hold one entry per (batch, neuron block of the launch).
-// ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ void appendOrdered(bool flag, uint32_t id, uint32_t localBlock, uint32_t numBlocks, size_t aggBase,
-                                              unsigned long long *counts, unsigned long long *groupTotals, uint32_t tag,
-                                              uint32_t *queue, uint32_t *queueCount, uint32_t *errorFlag)
+// Offset of a block's entries in its population's queue: the block publishes its count, then (wave 0) sums the counts of
+// the earlier blocks of its group of 64 and the published totals of the earlier groups.  Every thread of the block calls
+// this between two barriers of its own; returns 0xFFFFFFFF after a bounded wait expired (error flag raised).
+__device__ __forceinline__ uint32_t blockQueueOffset(uint32_t blockCount, uint32_t localBlock, uint32_t numBlocks, size_t aggBase,
+                                                    unsigned long long *counts, unsigned long long *groupTotals, uint32_t tag,
+                                                    uint32_t *shOffset, uint32_t *errorFlag)
 {
-    __shared__ uint32_t shCount[BLOCK / WAVE];
-    __shared__ uint32_t shOffset;
     const uint32_t lane = threadIdx.x & (WAVE - 1);
     const uint32_t wave = threadIdx.x / WAVE;
-    const unsigned long long ballot = __ballot(flag);
-    const uint32_t laneRank = __popcll(ballot & ((1ull << lane) - 1ull));
-    if(lane == 0) { shCount[wave] = __popcll(ballot); }
-    __syncthreads();
-    uint32_t blockCount = 0, waveOffset = 0;
-    #pragma unroll
-    for(uint32_t w = 0; w < BLOCK / WAVE; w++) {
-        const uint32_t c = shCount[w];
-        if(w < wave) { waveOffset += c; }
-        blockCount += c;
-    }
     if(threadIdx.x == 0) {
         __hip_atomic_store(&counts[aggBase + localBlock], ((unsigned long long)tag << 32) | blockCount, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -902,14 +887,42 @@ __device__ __forceinline__ void appendOrdered(bool flag, uint32_t id, uint32_t l
         const bool allOk = (__ballot(!ok) == 0ull);
         if(lane == 0) {
             if(!allOk) { atomicOr(errorFlag, 1u); sum = 0xFFFFFFFFu; }
-            shOffset = sum;
+            *shOffset = sum;
         }
     }
     __syncthreads();
-    const uint32_t prefix = shOffset;
+    return *shOffset;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Ordered append of the flagged neurons of a population to a queue, for spike-like events: the scheme the neuron
+// update uses for true spikes (ballot rank in the wave, LDS scan in the block, look-back over per-block counts tagged
+// with the step, blocks in groups of 64 with a published group total), as a function every block of the population
+// calls with all its threads.  `counts` and `groupTotals` hold one entry per (batch, neuron block of the launch).
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void appendOrdered(bool flag, uint32_t id, uint32_t localBlock, uint32_t numBlocks, size_t aggBase,
+                                              unsigned long long *counts, unsigned long long *groupTotals, uint32_t tag,
+                                              uint32_t *queue, uint32_t *queueCount, uint32_t *errorFlag)
+{
+    __shared__ uint32_t shCount[BLOCK / WAVE];
+    __shared__ uint32_t shOffset;
+    const uint32_t lane = threadIdx.x & (WAVE - 1);
+    const uint32_t wave = threadIdx.x / WAVE;
+    const unsigned long long ballot = __ballot(flag);
+    const uint32_t laneRank = __popcll(ballot & ((1ull << lane) - 1ull));
+    if(lane == 0) { shCount[wave] = __popcll(ballot); }
+    __syncthreads();
+    uint32_t blockCount = 0, waveOffset = 0;
+    #pragma unroll
+    for(uint32_t w = 0; w < BLOCK / WAVE; w++) {
+        const uint32_t c = shCount[w];
+        if(w < wave) { waveOffset += c; }
+        blockCount += c;
+    }
+    const uint32_t prefix = blockQueueOffset(blockCount, localBlock, numBlocks, aggBase, counts, groupTotals, tag, &shOffset, errorFlag);
     if(prefix != 0xFFFFFFFFu) {
         if(flag) { queue[prefix + waveOffset + laneRank] = id; }
-        if(last && threadIdx.x == 0) { *queueCount = prefix + blockCount; }
+        if(localBlock == numBlocks - 1 && threadIdx.x == 0) { *queueCount = prefix + blockCount; }
     }
     __syncthreads();            // the shared words are reused by the next call
 }
@@ -1199,6 +1212,172 @@ void neuronUpdateKernel(const NeuronGroupDev * __restrict__ blocks, StepArgs arg
                         unsigned long long *agg, uint32_t *errorFlag)
 {
     neuronBody(blocks[blockIdx.x], blockIdx.x, gridDim.x, resolve(args, dt), dt, agg, errorFlag);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Neuron update for large populations.  With one neuron per lane a population of millions is many rounds of resident
+// work-groups, and every round pays the whole dependent chain (descriptor, inputs, count published, look-back, queue).
+// Here a wavefront takes NPL consecutive chunks of 64 neurons: all inputs of all chunks are requested before anything is
+// stored, so a lane has NPL times the bytes in flight and the launch has 1/NPL of the work-groups.  Same arithmetic per
+// neuron and the same ordered queue as neuronBody (chunks of a wave are consecutive neurons, so chunk-major rank is neuron
+// order); the subset of features large populations use: LIF, Izhikevich and spike-source groups with up to two
+// postsynaptic models and one current source, spike recording; no traces, spike times, delay slots, further spike arrays,
+// events or presynaptic output (the host picks this kernel only when every group fits).
+// ------------------------------------------------------------------------------------------------
+constexpr uint32_t BULK_MAX_PSM = 2, BULK_MAX_CS = 1;
+
+template<int NPL>
+__device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t blockInKernel, uint32_t totalNeuronBlocks,
+                                               const Resolved &st, float dt, unsigned long long *agg, uint32_t *errorFlag)
+{
+    __shared__ uint32_t shWaveCount[BLOCK / WAVE];
+    __shared__ uint32_t shPrefix;
+    const gennmi_neuron_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const uint32_t localBlock = blockInKernel - G.startBlock;
+    const uint32_t n = g.numNeurons;
+    const uint32_t lane = threadIdx.x & (WAVE - 1);
+    const uint32_t wave = threadIdx.x / WAVE;
+    const float t = st.t;
+    const uint32_t first = (localBlock * (BLOCK / WAVE) + wave) * (WAVE * NPL) + lane;      // this lane's neuron in chunk 0
+    const uint32_t numPSM = g.numPSM, numCS = g.numCS;
+
+    float l0[NPL], l1[NPL], lin[NPL][BULK_MAX_PSM], front[NPL][BULK_MAX_PSM], inj[NPL];
+    bool spiked[NPL];
+    // ---- every input of every chunk first
+    #pragma unroll
+    for(int j = 0; j < NPL; j++) {
+        const uint32_t i = first + j * WAVE;
+        const size_t bi = (size_t)batch * n + i;
+        l0[j] = l1[j] = inj[j] = 0.0f;
+        #pragma unroll
+        for(uint32_t m = 0; m < BULK_MAX_PSM; m++) { lin[j][m] = front[j][m] = 0.0f; }
+        spiked[j] = false;
+        if(i < n) {
+            if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
+                l0[j] = asGlobal(G.nextSpikeTime)[bi];
+            }
+            else {
+                l0[j] = asGlobal(g.var0)[bi]; l1[j] = asGlobal(g.var1)[bi];
+                #pragma unroll
+                for(uint32_t m = 0; m < BULK_MAX_PSM; m++) {
+                    if(m < numPSM) {
+                        lin[j][m] = asGlobal(g.psm[m].outPost)[bi];
+                        const uint32_t D = g.psm[m].maxDenDelay;
+                        if(D) { front[j][m] = asGlobal(g.psm[m].denDelay)[((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i]; }
+                    }
+                }
+                if(numCS) {
+                    inj[j] = (g.cs[0].kind == GENNMI_CS_DC) ? g.cs[0].amp
+                                                            : asGlobal(g.cs[0].array)[(size_t)modStep(st.epoch, g.cs[0].arraySteps) * n + i];
+                }
+            }
+        }
+    }
+    // ---- update and store, chunk by chunk (operations and their order as in neuronBody)
+    #pragma unroll
+    for(int j = 0; j < NPL; j++) {
+        const uint32_t i = first + j * WAVE;
+        const size_t bi = (size_t)batch * n + i;
+        if(i >= n) { continue; }
+        if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
+            spiked[j] = (t >= l0[j]);
+            if(spiked[j]) {
+                const uint32_t startSpike = g.startSpike[bi] + 1;
+                g.startSpike[bi] = startSpike;
+                G.nextSpikeTime[bi] = (startSpike != g.endSpike[bi]) ? g.spikeTimes[startSpike] : INFINITY;
+            }
+            continue;
+        }
+        float Isyn = 0;
+        #pragma unroll
+        for(uint32_t m = 0; m < BULK_MAX_PSM; m++) {
+            if(m < numPSM) {
+                float linSyn = lin[j][m];
+                const uint32_t D = g.psm[m].maxDenDelay;
+                if(D) { linSyn += front[j][m]; }
+                if(g.psm[m].kind == GENNMI_PSM_EXPCURR) {
+                    Isyn += g.psm[m].init * linSyn;
+                    linSyn *= g.psm[m].expDecay;
+                }
+                else {
+                    Isyn += linSyn;
+                    linSyn = 0.0f;
+                }
+                if(D) { asGlobal(g.psm[m].denDelay)[((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i] = 0.0f; }
+                asGlobal(g.psm[m].outPost)[bi] = linSyn;
+            }
+        }
+        if(numCS) { Isyn += inj[j]; }
+        float v0 = l0[j], v1 = l1[j];
+        if(g.model == GENNMI_NEURON_LIF) {
+            if(v1 <= 0.0f) {
+                const float alpha = ((Isyn + g.params[0]) * g.params[1]) + g.params[2];
+                v0 = alpha - (g.params[3] * (alpha - v0));
+            }
+            else {
+                v1 -= dt;
+            }
+            spiked[j] = (v1 <= 0.0f && v0 >= g.params[4]);
+            if(spiked[j]) { v0 = g.params[5]; v1 = g.params[6]; }
+        }
+        else {
+            if(v0 >= 30.0f) {
+                v0 = g.params[2];
+                v1 += g.params[3];
+            }
+            v0 += 0.5f * (0.04f * v0 * v0 + 5.0f * v0 + 140.0f - v1 + Isyn) * dt;
+            v0 += 0.5f * (0.04f * v0 * v0 + 5.0f * v0 + 140.0f - v1 + Isyn) * dt;
+            v1 += g.params[0] * (g.params[1] * v0 - v1) * dt;
+            if(v0 > 30.0f) { v0 = 30.0f; }
+            spiked[j] = (v0 >= 29.99f);
+        }
+        g.var0[bi] = v0; g.var1[bi] = v1;
+    }
+    if(localBlock == 0 && batch == 0 && threadIdx.x < g.numPSM) {
+        const gennmi_psm_t &psm = g.psm[threadIdx.x];
+        if(psm.maxDenDelay && psm.denDelayPtr) { *psm.denDelayPtr = modStep(st.epoch + 1, psm.maxDenDelay); }
+    }
+
+    // ---- ordered compaction: rank = spikes of the wave's earlier chunks + spikes of lower lanes in this chunk
+    uint32_t rank[NPL];
+    uint32_t waveCount = 0;
+    #pragma unroll
+    for(int j = 0; j < NPL; j++) {
+        const uint32_t i = first + j * WAVE;
+        const unsigned long long ballot = __ballot(spiked[j]);
+        rank[j] = waveCount + __popcll(ballot & ((1ull << lane) - 1ull));
+        waveCount += __popcll(ballot);
+        if(g.recordSpk && (lane & 31) == 0 && i < n) {
+            const uint32_t words = (n + 31) / 32;
+            g.recordSpk[((size_t)st.recT * gridDim.y + batch) * words + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
+        }
+    }
+    if(lane == 0) { shWaveCount[wave] = waveCount; }
+    __syncthreads();
+    uint32_t blockCount = 0, waveOffset = 0;
+    #pragma unroll
+    for(uint32_t w = 0; w < BLOCK / WAVE; w++) {
+        const uint32_t c = shWaveCount[w];
+        if(w < wave) { waveOffset += c; }
+        blockCount += c;
+    }
+    unsigned long long *groupAgg = agg + (size_t)totalNeuronBlocks * gridDim.y;
+    const uint32_t prefix = blockQueueOffset(blockCount, localBlock, G.numBlocks, (size_t)batch * totalNeuronBlocks + G.startBlock, agg, groupAgg,
+                                             (uint32_t)(st.epoch + 1), &shPrefix, errorFlag);
+    if(prefix == 0xFFFFFFFFu) { return; }
+    #pragma unroll
+    for(int j = 0; j < NPL; j++) {
+        if(spiked[j]) { g.spk[(size_t)batch * n + prefix + waveOffset + rank[j]] = first + j * WAVE; }
+    }
+    if(localBlock == G.numBlocks - 1 && threadIdx.x == 0) { g.spkCnt[batch] = prefix + blockCount; }
+}
+
+template<int NPL>
+__global__ __launch_bounds__(BLOCK)
+void neuronBulkKernel(const NeuronGroupDev * __restrict__ blocks, StepArgs args, float dt, unsigned long long *agg, uint32_t *errorFlag)
+{
+    neuronBulkBody<NPL>(blocks[blockIdx.x], blockIdx.x, gridDim.x, resolve(args, dt), dt, agg, errorFlag);
 }
 
 // One launch per timestep for networks whose projections all go through the dendritic-delay ring: the
@@ -1898,6 +2077,7 @@ struct gennmi_runner
     uint32_t resTiles = 0, resReplicaStride = 0; size_t resLdsBytes = 0;
     std::vector<u32x4*> resSegs;        // segment table of each presynaptic group, in push order
     std::vector<uint32_t> resSegTiles;  // tiles of its target population
+    uint32_t neuronsPerLane = 1;        // 2, 4 or 8: neuronBulkKernel instead of neuronUpdateKernel
     bool sourcesStale = false;          // startSpike / endSpike / spikeTimes of a spike source were written since nextSpikeTime was built
     bool resStale = false;              // connectivity or weights were written since the tables were built
     // graph
@@ -2465,10 +2645,33 @@ int gennmi_runner_finalise(gennmi_runner *r)
             }
         }
     }
+    // Large networks of plain groups take the several-neurons-per-lane kernel: what counts is the number of rounds of
+    // resident work-groups a launch needs (numCU x 8 work-groups of 256 lanes are resident at a time).
+    {
+        unsigned long long lanes = 0;
+        bool plain = r->post.empty();
+        for(const auto &n : r->neuron) {
+            const auto &g = n.g;
+            lanes += (unsigned long long)g.numNeurons * r->batch;
+            plain = plain && g.numPSM <= BULK_MAX_PSM && g.numCS <= BULK_MAX_CS && !g.preTrace && !g.postTrace && !g.sT && g.numExtraSpk == 0
+                    && g.numDelaySlots <= 1 && g.numSpkEvent == 0 && g.numPreOutput == 0;
+        }
+        // measured: four per lane from one round of work-groups up (10^6 Izhikevich neurons: 20.1 us with one, 18.0 with two,
+        // 16.4 with four), eight beyond five rounds (3.1 x 10^6 lanes of the batched convolution layer: 57 / 38 / 29 / 24 us
+        // with one / two / four / eight); GENNMI_NEURON_BULK = 0 (never), 2, 4 or 8 forces the choice
+        const unsigned long long round = 1ull * numCU * 8 * BLOCK;
+        uint32_t perLane = (lanes <= round) ? 1u : (2 * lanes <= 5 * round) ? 4u : 8u;
+        if(const char *envBulk = getenv("GENNMI_NEURON_BULK")) {
+            const int v = atoi(envBulk);
+            perLane = (v == 2 || v == 4 || v == 8) ? (uint32_t)v : (v == 1) ? 4u : 1u;
+        }
+        r->neuronsPerLane = plain ? perLane : 1u;
+    }
+    const uint32_t neuronsPerBlock = BLOCK * r->neuronsPerLane;
     uint32_t block = 0;
     for(auto &n : r->neuron) {
         n.startBlock = block;
-        n.numBlocks = (n.g.numNeurons + BLOCK - 1) / BLOCK;
+        n.numBlocks = (n.g.numNeurons + neuronsPerBlock - 1) / neuronsPerBlock;
         block += n.numBlocks;
     }
     r->neuronBlocks = block;
@@ -2657,7 +2860,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
     bool anyEvents = false;
     for(const auto &n : r->neuron) { anyEvents = anyEvents || n.g.numSpkEvent != 0; }
     const char *envFused = getenv("GENNMI_FUSED_STEP");
-    bool eligible = !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty() && r->dense.empty() && r->proc.empty() && !anyEvents;
+    bool eligible = !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty() && r->dense.empty() && r->proc.empty() && !anyEvents && r->neuronsPerLane == 1;
     for(const auto &p : r->pre) {
         eligible = eligible && p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY
                    && p.g.maxDenDelay >= 2 && p.g.numSrcDelaySlots <= 1;
@@ -2889,7 +3092,11 @@ static int launchNeurons(gennmi_runner *r, const StepArgs &a, bool timed)
 {
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if(timed) { const int rc = stamp(r, &e0); if(rc) { return rc; } }
-    neuronUpdateKernel<<<dim3(r->neuronBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dNeuron, a, r->dt, r->dAgg, r->dError);
+    const dim3 neuronGrid(r->neuronBlocks, r->batch);
+    if(r->neuronsPerLane == 2) { neuronBulkKernel<2><<<neuronGrid, dim3(BLOCK), 0, r->stream>>>(r->dNeuron, a, r->dt, r->dAgg, r->dError); }
+    else if(r->neuronsPerLane == 4) { neuronBulkKernel<4><<<neuronGrid, dim3(BLOCK), 0, r->stream>>>(r->dNeuron, a, r->dt, r->dAgg, r->dError); }
+    else if(r->neuronsPerLane == 8) { neuronBulkKernel<8><<<neuronGrid, dim3(BLOCK), 0, r->stream>>>(r->dNeuron, a, r->dt, r->dAgg, r->dError); }
+    else { neuronUpdateKernel<<<dim3(r->neuronBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dNeuron, a, r->dt, r->dAgg, r->dError); }
     if(timed) { const int rc = stamp(r, &e1); if(rc) { return rc; } r->pending.push_back({e0, e1, 2}); }
     HIP_TRY(hipGetLastError());
     return GENNMI_OK;
@@ -3065,7 +3272,7 @@ int gennmi_runner_get_info(gennmi_runner *r, uint32_t info[4])
 {
     if(!r || !info) { return fail(GENNMI_EINVAL, "runner_get_info: null argument"); }
     if(!r->finalised) { return fail(GENNMI_ESTATE, "runner_get_info: runner not finalised"); }
-    info[0] = (r->fusedStep ? 1u : 0u) | (r->resident ? 2u : 0u); info[1] = r->neuronBlocks; info[2] = r->preBlocks; info[3] = r->postBlocks;
+    info[0] = (r->fusedStep ? 1u : 0u) | (r->resident ? 2u : 0u) | (r->neuronsPerLane > 1 ? 4u : 0u); info[1] = r->neuronBlocks; info[2] = r->preBlocks; info[3] = r->postBlocks;
     return GENNMI_OK;
 }
 

@@ -931,7 +931,7 @@ class GeNNModel:
     def runner_info(self):
         info = (C.c_uint32 * 4)()
         _abi.check(_abi.load().gennmi_runner_get_info(self._runner, C.byref(info)))
-        return {"single_launch_step": bool(info[0] & 1), "resident_plan": bool(info[0] & 2), "neuron_blocks": info[1], "presyn_blocks": info[2], "postsyn_blocks": info[3]}
+        return {"single_launch_step": bool(info[0] & 1), "resident_plan": bool(info[0] & 2), "bulk_neuron_kernel": bool(info[0] & 4), "neuron_blocks": info[1], "presyn_blocks": info[2], "postsyn_blocks": info[3]}
 
     def set_timing(self, enabled):
         _abi.check(_abi.load().gennmi_runner_set_timing(self._runner, int(bool(enabled))))

@@ -344,7 +344,9 @@ int gennmi_runner_stream_elapsed(gennmi_runner *runner, double *seconds);
  * populations, all tiles of 256 neurons resident at once; GENNMI_RESIDENT=0 disables it); bit 0 if a whole timestep is one launch (all projections go
  * through a dendritic-delay ring; synapses with d % D == 0 are then delivered by the spiking neuron one launch
  * earlier, into the slot read in the next step — the visible difference is the content of that one ring slot
- * between steps; GENNMI_FUSED_STEP=0 in the environment keeps the reference's placement), info[1..3] = blocks of
+ * between steps; GENNMI_FUSED_STEP=0 in the environment keeps the reference's placement); bit 2 if the neuron update
+ * takes several neurons per lane (networks that need more than one round of resident work-groups and use only plain groups;
+ * GENNMI_NEURON_BULK=0 forbids it, 2 / 4 / 8 force that many), info[1..3] = blocks of
  * the neuron, presynaptic and postsynaptic kernels.  The reference logs the analogous choice of presynaptic
  * strategy (backendSIMT.cc:736). */
 int gennmi_runner_get_info(gennmi_runner *runner, uint32_t info[4]);
