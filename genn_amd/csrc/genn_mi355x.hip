@@ -2684,7 +2684,8 @@ int gennmi_runner_finalise(gennmi_runner *r)
     block = 0;
     const char *envBudget = getenv("GENNMI_PRESYN_BLOCKS_PER_CU");
     const uint32_t blocksPerCU = envBudget ? std::max(1, atoi(envBudget)) : 4u;
-    const uint64_t budget = (uint64_t)numCU * blocksPerCU;
+    // the launch has one grid row per batch, so the budget is per batch (at least one block per compute unit in all)
+    const uint64_t budget = std::max<uint64_t>((numCU + r->batch - 1) / r->batch, (uint64_t)numCU * blocksPerCU / r->batch);
     std::vector<uint64_t> wantBlocks;
     for(auto &p : r->pre) {
         const uint32_t rowLen = (p.g.matrix == GENNMI_MATRIX_SPARSE) ? p.g.rowStride : (uint32_t)(p.g.conv[0] * p.g.conv[1] * p.g.conv[7]);
@@ -2781,9 +2782,14 @@ int gennmi_runner_finalise(gennmi_runner *r)
                 const size_t fixedFloats = (size_t)c[0] * c[1] * c[4] * c[7] + CONV_TILE_SPIKES;      // kernel weights + staged spikes
                 const size_t budgetFloats = 60 * 1024 / sizeof(float);
                 if(fixedFloats + rowFloats <= budgetFloats) {
-                    // as many rows per block as fit in LDS, but enough blocks to cover the chip about twice
+                    // as many rows per block as fit in LDS, but enough blocks to cover the chip once
                     uint32_t rowsPerTile = (uint32_t)std::min<size_t>((budgetFloats - fixedFloats) / rowFloats, (size_t)c[5]);
-                    const uint32_t wantBlocks = std::max(1u, (2 * numCU) / r->batch);
+                    // measured on the batched 64x64 layer (us per launch of both presynaptic kernels): 119 / 75 / 61 with 4 / 2 / 1
+                    // blocks per compute unit — a spike concerns (rows + kh - 1) / rows tiles, so fewer, taller tiles do less
+                    // redundant work
+                    const char *envConvBlocks = getenv("GENNMI_CONV_TILE_BLOCKS_PER_CU");
+                    const uint32_t convBlocksPerCU = envConvBlocks ? (uint32_t)std::max(1, atoi(envConvBlocks)) : 1u;
+                    const uint32_t wantBlocks = std::max(1u, (convBlocksPerCU * numCU) / r->batch);
                     rowsPerTile = std::max(1u, std::min(rowsPerTile, ((uint32_t)c[5] + wantBlocks - 1) / wantBlocks));
                     ConvTileDev t{};
                     t.g = p.g; t.convBH = p.convBH; t.convBW = p.convBW; t.rowsPerTile = rowsPerTile;
