@@ -38,7 +38,7 @@ class Cs(C.Structure):
 
 
 class SpikeEvent(C.Structure):
-    _fields_ = [("spkCntEvent", p_u32), ("spkEvent", p_u32), ("threshold", C.c_float), ("pad_", C.c_uint32)]
+    _fields_ = [("spkCntEvent", p_u32), ("spkEvent", p_u32), ("recordSpkEvent", p_u32), ("threshold", C.c_float), ("pad_", C.c_uint32)]
 
 
 class NeuronUpdateGroup(C.Structure):

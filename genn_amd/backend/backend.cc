@@ -295,9 +295,8 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
                 if(arch.isSimRNGRequired()) { unsupported("random numbers in the update of population '" + arch.getName() + "'"); }
                 if(arch.isPrevSpikeTimeRequired()) { unsupported("previous spike times of population '" + arch.getName() + "'"); }
                 if(n.getMergedSpikeEventGroups().size() > GENNMI_MAX_SPK_EVENT) { unsupported("more than 2 spike-like event conditions on population '" + arch.getName() + "'"); }
-                if(!n.getMergedSpikeEventGroups().empty() && (arch.isDelayRequired() || arch.isSpikeEventTimeRequired() || arch.isPrevSpikeEventTimeRequired()
-                                                              || arch.isSpikeEventRecordingEnabled())) {
-                    unsupported("delay slots, event times or event recording with spike-like events on population '" + arch.getName() + "'");
+                if(!n.getMergedSpikeEventGroups().empty() && (arch.isDelayRequired() || arch.isSpikeEventTimeRequired() || arch.isPrevSpikeEventTimeRequired())) {
+                    unsupported("delay slots or event times with spike-like events on population '" + arch.getName() + "'");
                 }
                 if(n.getMergedOutSynPreOutputGroups().size() > GENNMI_MAX_PRE_OUTPUT) { unsupported("more than 2 presynaptic outputs into population '" + arch.getName() + "'"); }
 
@@ -503,6 +502,11 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
                     eenv.getStream() << "{ static const float v[] = " << table(thresholds, scalar) << "; d.spkEvent[" << k << "].spkCntEvent = gennmiDev("
                                      << eenv["_mi_spkCntEvent"] << "); d.spkEvent[" << k << "].spkEvent = gennmiDev(" << eenv["_mi_spkEvent"]
                                      << "); d.spkEvent[" << k << "].threshold = v[g]; }" << std::endl;
+                    if(arch.isSpikeEventRecordingEnabled()) {
+                        eenv.addField(Type::Uint32.createPointer(), "_mi_recordSpkEvent", "recordSpkEvent" + sfx,
+                                      [&n](const auto &runtime, const auto &g, size_t i) { return runtime.getFusedEventArray(n, i, g, "RecordSpkEvent"); });
+                        eenv.getStream() << "d.spkEvent[" << k << "].recordSpkEvent = gennmiDev(" << eenv["_mi_recordSpkEvent"] << ");" << std::endl;
+                    }
                 }
                 out << "d.numSpkEvent = " << events.size() << "u;" << std::endl;
                 // presynaptic output of outgoing projections ("OutSynPreOutput" children, neuronUpdateGroupMerged.cc:148-165)

@@ -902,13 +902,16 @@ __device__ __forceinline__ uint32_t blockQueueOffset(uint32_t blockCount, uint32
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ void appendOrdered(bool flag, uint32_t id, uint32_t localBlock, uint32_t numBlocks, size_t aggBase,
                                               unsigned long long *counts, unsigned long long *groupTotals, uint32_t tag,
-                                              uint32_t *queue, uint32_t *queueCount, uint32_t *errorFlag)
+                                              uint32_t *queue, uint32_t *queueCount, uint32_t *errorFlag,
+                                              uint32_t *recordWords = nullptr, bool inRange = false)
 {
     __shared__ uint32_t shCount[BLOCK / WAVE];
     __shared__ uint32_t shOffset;
     const uint32_t lane = threadIdx.x & (WAVE - 1);
     const uint32_t wave = threadIdx.x / WAVE;
     const unsigned long long ballot = __ballot(flag);
+    // recording: the ballot is the bitfield of this step's events (every word of the step is overwritten)
+    if(recordWords && (lane & 31) == 0 && inRange) { recordWords[id >> 5] = (uint32_t)(ballot >> (lane & 32)); }
     const uint32_t laneRank = __popcll(ballot & ((1ull << lane) - 1ull));
     if(lane == 0) { shCount[wave] = __popcll(ballot); }
     __syncthreads();
@@ -1081,7 +1084,8 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
             unsigned long long *counts = G.aggEvent + (size_t)e * 2 * perArea;
             appendOrdered(i < n && vEvent > g.spkEvent[e].threshold, i, localBlock, G.numBlocks, (size_t)batch * totalNeuronBlocks + G.startBlock,
                           counts, counts + perArea, (uint32_t)(st.epoch + 1), g.spkEvent[e].spkEvent + (size_t)batch * n,
-                          g.spkEvent[e].spkCntEvent + batch, errorFlag);
+                          g.spkEvent[e].spkCntEvent + batch, errorFlag,
+                          g.spkEvent[e].recordSpkEvent ? g.spkEvent[e].recordSpkEvent + ((size_t)st.recT * gridDim.y + batch) * ((n + 31) / 32) : nullptr, i < n);
         }
     }
 

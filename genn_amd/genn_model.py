@@ -215,6 +215,7 @@ class NeuronGroup:
         self.in_syn = []
         self.out_syn = []
         self.spike_recording_enabled = False
+        self.spike_event_recording_enabled = False
         self.fused_psm = []          # list of lists of SynapseGroup sharing one outPost
         self.pre_trace_owner = None
         self.post_trace_owner = None
@@ -338,6 +339,13 @@ class SynapseGroup:
     def get_sparse_post_inds(self):
         mask = np.arange(self.row_stride)[None, :] < self.row_length_host[:, None]
         return self.ind_host[mask]
+
+    @property
+    def pre_spike_event_recording_data(self):
+        """[(times, ids)] per batch of the presynaptic spike-like events this projection is driven by
+        (pygenn/genn_groups.py:397-406); needs spike_event_recording_enabled on the source population."""
+        e = self.src.event_thresholds.index(float(self.wu.params["Epre"]))
+        return self._model._decode_recording(self.src, f"recordSpkEvent{e}")
 
     @property
     def num_synapses(self):
@@ -529,6 +537,10 @@ class GeNNModel:
             for e in range(len(n.event_thresholds)):
                 n.vars[f"spkCntEvent{e}"] = self._alloc(B, np.uint32)
                 n.vars[f"spkEvent{e}"] = self._alloc(B * N, np.uint32)
+                if n.spike_event_recording_enabled:
+                    if not num_recording_timesteps:
+                        raise RuntimeError("Cannot use recording system without specifying number of recording timesteps")
+                    n.vars[f"recordSpkEvent{e}"] = self._alloc(((N + 31) // 32) * B * num_recording_timesteps, np.uint32)
             if n.spike_recording_enabled:
                 if not num_recording_timesteps:
                     raise RuntimeError("Cannot use recording system without specifying number of recording timesteps")
@@ -726,6 +738,8 @@ class GeNNModel:
                     d.numSpkEvent = len(n.event_thresholds)
                     d.spkEvent[e].spkCntEvent, d.spkEvent[e].spkEvent = n.vars[f"spkCntEvent{e}"].ptr, n.vars[f"spkEvent{e}"].ptr
                     d.spkEvent[e].threshold = thresholds[k]
+                    if f"recordSpkEvent{e}" in n.vars:
+                        d.spkEvent[e].recordSpkEvent = n.vars[f"recordSpkEvent{e}"].ptr
             # postsynaptic-model children
             num_psm = len(members[0].fused_psm)
             for m in range(num_psm):
@@ -894,12 +908,13 @@ class GeNNModel:
     def pull_recording_buffers_from_device(self):
         self.synchronize()
         for n in self.neuron_populations.values():
-            if "recordSpk" in n.vars:
-                n.vars["recordSpk"].pull_from_device()
+            for name, a in n.vars.items():
+                if name.startswith("recordSpk"):
+                    a.pull_from_device()
 
-    def _decode_recording(self, n):
+    def _decode_recording(self, n, var="recordSpk"):
         words = (n.num_neurons + 31) // 32
-        rec = n.vars["recordSpk"].view.reshape(self.num_recording_timesteps, self.batch_size, words)
+        rec = n.vars[var].view.reshape(self.num_recording_timesteps, self.batch_size, words)
         bits = np.unpackbits(rec.view(np.uint8), axis=2, bitorder="little")[:, :, :n.num_neurons]
         start = self.timestep - self.num_recording_timesteps if self.timestep >= self.num_recording_timesteps else 0
         out = []

@@ -133,6 +133,8 @@ typedef struct gennmi_cs_t {              /* one current source child (neuronUpd
 typedef struct gennmi_spike_event_t {
     uint32_t *spkCntEvent;                /* [batch] */
     uint32_t *spkEvent;                   /* [batch*numNeurons] */
+    uint32_t *recordSpkEvent;             /* [numRecordingTimesteps*batch*ceil(numNeurons/32)] or NULL: the events of every step as a
+                                           * bitfield, laid out like recordSpk (runtime.cc:307-311) */
     float threshold;                      /* StaticGraded: Epre */
     uint32_t pad_;
 } gennmi_spike_event_t;

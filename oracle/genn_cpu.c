@@ -53,6 +53,7 @@ enum { GC_CS_DC = 0, GC_CS_NOISE = 1 };
 typedef struct {
     float threshold;
     uint32_t *spkEvent, spkCntEvent;
+    uint32_t *recordSpkEvent;   /* [numRec * ceil(n/32)] or NULL (runtime.cc:307-311) */
 } gc_event;
 
 typedef struct {
@@ -232,6 +233,7 @@ void gc_set_static_graded(gc_net *net, int syn, float epre, float vslope)
     p->events[p->numEvents].threshold = epre;
     p->events[p->numEvents].spkEvent = (uint32_t*)calloc(p->n ? p->n : 1, sizeof(uint32_t));
     p->events[p->numEvents].spkCntEvent = 0;
+    p->events[p->numEvents].recordSpkEvent = net->numRec ? (uint32_t*)calloc(net->numRec * ((p->n + 31) / 32), sizeof(uint32_t)) : NULL;
     p->numEvents++;
 }
 
@@ -476,6 +478,10 @@ void gc_update_neurons(gc_net *net, float t, uint32_t recordingTimestep)
         const uint32_t numRecordingWords = (p->n + 31) / 32;
         uint32_t *rec = p->recordSpk ? &p->recordSpk[(size_t)recordingTimestep * numRecordingWords] : NULL;
         if(rec) { memset(rec, 0, numRecordingWords * sizeof(uint32_t)); }
+        /* spike-like event recording buffers are cleared the same way (backend.cc:309-318) */
+        for(int e = 0; e < p->numEvents; e++) {
+            if(p->events[e].recordSpkEvent) { memset(&p->events[e].recordSpkEvent[(size_t)recordingTimestep * numRecordingWords], 0, numRecordingWords * sizeof(uint32_t)); }
+        }
         for(uint32_t i = 0; i < p->n; i++) {
             int spiked;
             if(p->model == GC_SSA) {
@@ -548,7 +554,11 @@ void gc_update_neurons(gc_net *net, float t, uint32_t recordingTimestep)
             if(p->postTrace) { p->postTrace[i] *= p->postDecay; }
             /* spike-like event conditions: after the sim code, before the threshold test (neuronUpdateGroupMerged.cc:677-683) */
             for(int e = 0; e < p->numEvents; e++) {
-                if(l0 > p->events[e].threshold) { p->events[e].spkEvent[p->events[e].spkCntEvent++] = i; }
+                if(l0 > p->events[e].threshold) {
+                    p->events[e].spkEvent[p->events[e].spkCntEvent++] = i;
+                    /* backend.cc:360-380 */
+                    if(p->events[e].recordSpkEvent) { p->events[e].recordSpkEvent[(size_t)recordingTimestep * numRecordingWords + (i / 32)] |= (1u << (i % 32)); }
+                }
             }
             spiked = (p->model == GC_LIF) ? (l1 <= 0.0f && l0 >= p->p[4]) : (l0 >= 29.99f);
             if(spiked) {
@@ -598,6 +608,7 @@ uint32_t *gc_remap(gc_net *net, int syn) { return net->syns[syn].remap; }
 float *gc_out_pre(gc_net *net, int syn) { return net->pops[net->syns[syn].src].outPre[net->syns[syn].preOutput]; }
 uint32_t gc_event_count(const gc_net *net, int pop, int event) { return net->pops[pop].events[event].spkCntEvent; }
 const uint32_t *gc_events(const gc_net *net, int pop, int event) { return net->pops[pop].events[event].spkEvent; }
+uint32_t *gc_event_record(gc_net *net, int pop, int event) { return net->pops[pop].events[event].recordSpkEvent; }
 int gc_syn_event_queue(const gc_net *net, int syn) { return net->syns[syn].event; }
 uint64_t gc_syn_events(const gc_net *net, int syn) { return net->syns[syn].events; }
 uint64_t gc_timestep(const gc_net *net) { return net->timestep; }
@@ -611,7 +622,7 @@ void gc_destroy(gc_net *net)
         for(int m = 0; m < p->numPSM; m++) { free(p->psm[m].outPost); free(p->psm[m].denDelay); }
         free(p->preTrace); free(p->postTrace); free(p->sT); free(p->recordSpk);
         if(p->spkRing) { free(p->spkRing); free(p->spkCntRing); } else { free(p->spk); }
-        for(int e = 0; e < p->numEvents; e++) { free(p->events[e].spkEvent); }
+        for(int e = 0; e < p->numEvents; e++) { free(p->events[e].spkEvent); free(p->events[e].recordSpkEvent); }
         for(int q = 0; q < p->numPreOutput; q++) { free(p->outPre[q]); }
     }
     for(int k = 0; k < net->numSyns; k++) { free(net->syns[k].colLength); free(net->syns[k].remap); }

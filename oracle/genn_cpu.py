@@ -72,6 +72,7 @@ def lib():
         l.gc_out_pre.restype = vp; l.gc_out_pre.argtypes = [vp, i32]
         l.gc_event_count.restype = u32; l.gc_event_count.argtypes = [vp, i32, i32]
         l.gc_events.restype = vp; l.gc_events.argtypes = [vp, i32, i32]
+        l.gc_event_record.restype = vp; l.gc_event_record.argtypes = [vp, i32, i32]
         l.gc_syn_event_queue.restype = i32; l.gc_syn_event_queue.argtypes = [vp, i32]
         l.gc_timestep.restype = u64; l.gc_timestep.argtypes = [vp]
         l.gc_destroy.restype = None; l.gc_destroy.argtypes = [vp]
@@ -335,6 +336,13 @@ class OracleNet:
         s = self.net.syn(syn)
         pop, q = self.pop_id[s.src], self.l.gc_syn_event_queue(self.h, self.syn_id[syn])
         return self._arr(self.l.gc_events(self.h, pop, q), self.l.gc_event_count(self.h, pop, q), np.uint32).copy()
+
+    def event_record(self, syn, num_rec):
+        """Recorded spike-like events of the queue a graded projection reads: bitfield [num_rec, ceil(n/32)]."""
+        s = self.net.syn(syn)
+        pop, q = self.pop_id[s.src], self.l.gc_syn_event_queue(self.h, self.syn_id[syn])
+        n = self.net.pop(s.src).n
+        return self._arr(self.l.gc_event_record(self.h, pop, q), num_rec * ((n + 31) // 32), np.uint32)
 
     def events(self):
         return sum(self.l.gc_syn_events(self.h, i) for i in self.syn_id.values())

@@ -241,6 +241,8 @@ int main(int argc, char *argv[])
             p.ng->setSpikeRecordingEnabled(true);
             popByName[p.name] = &p;
         }
+        // populations that drive graded projections also record their spike-like events
+        for(auto &s : syns) { if(s.wum == "static_graded") { popByName.at(s.src)->ng->setSpikeEventRecordingEnabled(true); } }
         for(auto &c : css) {
             NeuronGroup *ng = popByName.at(c.pop)->ng;
             if(c.model == "dc") c.cs = model.addCurrentSource<CurrentSourceModels::DC>(c.name, ng, {{"amp", c.p.at(0)}}, {});
@@ -476,6 +478,18 @@ int main(int argc, char *argv[])
                 for(const auto &s : sorted) { pairs.push_back(s.first); pairs.push_back(s.second); }
                 appendFile(out + "/" + p.name + ".spikes" + (bi ? ".b" + std::to_string(bi) : std::string()) + ".u32", pairs.data(), pairs.size());
             }
+        }
+        // recorded spike-like events of the graded projections, as (step, presynaptic id) pairs of batch 0
+        for(auto &s : syns) {
+            if(s.wum != "static_graded") continue;
+            const auto ev = rt.getRecordedPreSpikeEvents(*s.sg);
+            std::vector<std::pair<uint32_t, uint32_t>> sorted;
+            const auto &times = ev.at(0).first; const auto &ids = ev.at(0).second;
+            for(size_t k = 0; k < times.size(); k++) { sorted.emplace_back((uint32_t)std::llround(times[k] / dt), ids[k]); }
+            std::sort(sorted.begin(), sorted.end());
+            std::vector<uint32_t> pairs;
+            for(const auto &e : sorted) { pairs.push_back(e.first); pairs.push_back(e.second); }
+            appendFile(out + "/" + s.name + ".events.u32", pairs.data(), pairs.size());
         }
         std::cout << "ref_driver: " << name << " ran " << steps << " steps" << std::endl;
     }

@@ -53,6 +53,9 @@ def make(name):
                     if var in ("g", "denDelay", "outPost", "preTrace", "postTrace"):
                         a = a.reshape(net.steps // snap, -1)[-1] if var in ("g", "denDelay") else a.reshape(net.steps // snap, -1)
                     data[f"{var}.{s.name}"] = a
+            f = os.path.join(out, f"{s.name}.events.u32")
+            if os.path.exists(f):
+                data[f"events.{s.name}"] = np.fromfile(f, np.uint32).reshape(-1, 2)
             f = os.path.join(out, f"{s.name}.colStride.txt")
             if os.path.exists(f):
                 data[f"colStride.{s.name}"] = np.array(int(open(f).read()))

@@ -73,6 +73,12 @@ def test_adapter_matches_reference_backend(case):
                     else:
                         _close(g, golden[key], key)
         assert spikes > 50
+        # recorded spike-like events, where the fixture holds them
+        for s in net.syns:
+            if f"events.{s.name}" in golden:
+                got = np.fromfile(os.path.join(out, f"{s.name}.events.u32"), np.uint32).reshape(-1, 2)
+                assert np.array_equal(got, golden[f"events.{s.name}"]), f"recorded events of {s.name} differ"
+
         for s in net.syns:
             for var in ("colLength", "remap"):
                 key = f"{var}.{s.name}"

@@ -148,3 +148,34 @@ def test_reverse_output_matches_the_oracle():
     1e-5 (a row's weights are summed in a different order)."""
     net = configs.reverse()
     _reverse_lock_step(net, 100, exact=False)
+
+
+def test_spike_event_recording():
+    """Recorded spike-like events (one bitfield per event queue, laid out like the spike recording) against the oracle,
+    through single steps and a replayed run, for every batch."""
+    net = configs.graded(steps=120)
+    B = 2
+    model = model_from_net(net, batch_size=B)
+    for p in model.neuron_populations.values():
+        p.spike_event_recording_enabled = True
+    model.load(num_recording_timesteps=120)
+    oracle = OracleNet(net, num_recording_timesteps=120)
+    for _ in range(20):
+        model.step_time()
+    model.run(100)
+    oracle.run(120)
+    model.pull_recording_buffers_from_device()
+    total = 0
+    for name in GRADED:
+        src = model.synapse_populations[name].src
+        words = (src.num_neurons + 31) // 32
+        e = src.event_thresholds.index(float(model.synapse_populations[name].wu.params["Epre"]))
+        got = src.vars[f"recordSpkEvent{e}"].view.reshape(120, B, words)
+        want = oracle.event_record(name, 120).reshape(120, words)
+        for b in range(B):
+            assert np.array_equal(got[:, b], want), f"recorded events of {name}, batch {b}"
+        times, ids = model.synapse_populations[name].pre_spike_event_recording_data[0]
+        assert len(ids) == int(np.unpackbits(want.view(np.uint8)).sum())
+        total += len(ids)
+    assert total > 5000
+    model.unload()

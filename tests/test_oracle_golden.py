@@ -32,7 +32,8 @@ def test_oracle_matches_reference_backend(case):
     assert net.input_digest() == str(gold["input_digest"]), "the input generator no longer reproduces the golden inputs"
     fuse = dict(item.split("=") for item in gold["fusemap"].tolist())
     col = {s.name: int(gold[f"colStride.{s.name}"]) for s in net.syns if f"colStride.{s.name}" in gold}
-    oracle = OracleNet(net, col_stride=col or None)
+    record_events = [s.name for s in net.syns if f"events.{s.name}" in gold]
+    oracle = OracleNet(net, num_recording_timesteps=net.steps if record_events else 0, col_stride=col or None)
     for s in net.syns:
         if s.name in col:
             col_length = gold[f"colLength.{s.name}"]
@@ -64,6 +65,12 @@ def test_oracle_matches_reference_backend(case):
             assert np.array_equal(oracle.syn_g(s.name), gold[f"g.{s.name}"])
         if fuse[s.name] == s.name and f"denDelay.{s.name}" in gold:
             assert np.array_equal(oracle.den_delay(s.name), gold[f"denDelay.{s.name}"])
+    for name in record_events:
+        n = net.pop(net.syn(name).src).n
+        bits = np.unpackbits(oracle.event_record(name, net.steps).reshape(net.steps, -1).view(np.uint8), axis=1, bitorder="little")[:, :n]
+        steps, ids = np.nonzero(bits)
+        assert np.array_equal(np.stack([steps, ids], axis=1).astype(np.uint32), gold[f"events.{name}"]), f"recorded events of {name}"
+        assert len(steps) > 100
     total = 0
     for p in net.pops:
         mine = np.concatenate(raster[p.name])
