@@ -571,7 +571,7 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
 
         modelMerged.genMergedPresynapticUpdateGroups(
             *this, memorySpaces,
-            [this, &funcEnv, batchSize, scalar](auto &s)
+            [this, &funcEnv, &model, batchSize, scalar](auto &s)
             {
                 const auto &arch = s.getArchetype();
                 const auto *wum = arch.getWUInitialiser().getSnippet();
@@ -591,8 +591,31 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                 const bool dense = (matrixType & SynapseMatrixConnectivity::DENSE) && (matrixType & SynapseMatrixWeight::INDIVIDUAL);
                 const bool bitmask = (matrixType & SynapseMatrixConnectivity::BITMASK) != 0;
                 const bool constantWeight = (wumKind == GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT);
-                if(!sparse && !toeplitz && !dense && !bitmask) {
-                    unsupported("matrix type of projection '" + arch.getName() + "' (SPARSE, DENSE, BITMASK or TOEPLITZ with kernel weights)");
+                // PROCEDURAL: connectivity and weights are regenerated per spike.  The snippets arrive as code for a backend
+                // to transpile; here they are recognised by identity with the built-in ones the device library implements.
+                const bool procedural = (matrixType & SynapseMatrixConnectivity::PROCEDURAL) && ((matrixType & SynapseMatrixWeight::PROCEDURAL) || constantWeight);
+                unsigned int procConnect = 0, procWeight = GENNMI_INIT_CONSTANT;
+                std::vector<std::string> procWeightParams;
+                if(procedural) {
+                    const auto *conn = arch.getSparseConnectivityInitialiser().getSnippet();
+                    if(conn == InitSparseConnectivitySnippet::FixedProbability::getInstance()) { procConnect = GENNMI_CONNECT_FIXED_PROBABILITY; }
+                    else if(conn == InitSparseConnectivitySnippet::FixedProbabilityNoAutapse::getInstance()) { procConnect = GENNMI_CONNECT_FIXED_PROBABILITY_NO_AUTAPSE; }
+                    else if(conn == InitSparseConnectivitySnippet::FixedNumberPostWithReplacement::getInstance()) { procConnect = GENNMI_CONNECT_FIXED_NUMBER_POST; }
+                    else { unsupported("connectivity snippet of PROCEDURAL projection '" + arch.getName() + "' (FixedProbability, FixedProbabilityNoAutapse, FixedNumberPostWithReplacement)"); }
+                    if(wumKind != GENNMI_WUM_STATIC_PULSE && !constantWeight) { unsupported("weight update model of PROCEDURAL projection '" + arch.getName() + "'"); }
+                    if(!constantWeight) {
+                        const auto *init = arch.getWUInitialiser().getVarInitialisers().at("g").getSnippet();
+                        if(init == InitVarSnippet::Constant::getInstance()) { procWeight = GENNMI_INIT_CONSTANT; procWeightParams = {"constant"}; }
+                        else if(init == InitVarSnippet::Uniform::getInstance()) { procWeight = GENNMI_INIT_UNIFORM; procWeightParams = {"min", "max"}; }
+                        else if(init == InitVarSnippet::Normal::getInstance()) { procWeight = GENNMI_INIT_NORMAL; procWeightParams = {"mean", "sd"}; }
+                        else if(init == InitVarSnippet::NormalClipped::getInstance()) { procWeight = GENNMI_INIT_NORMAL_CLIPPED; procWeightParams = {"mean", "sd", "min", "max"}; }
+                        else if(init == InitVarSnippet::Exponential::getInstance()) { procWeight = GENNMI_INIT_EXPONENTIAL; procWeightParams = {"lambda"}; }
+                        else { unsupported("weight initialisation snippet of PROCEDURAL projection '" + arch.getName() + "' (Constant, Uniform, Normal, NormalClipped, Exponential)"); }
+                    }
+                    if(srcDelay || arch.isDendriticOutputDelayRequired()) { unsupported("delays on PROCEDURAL projection '" + arch.getName() + "'"); }
+                }
+                if(!sparse && !toeplitz && !dense && !bitmask && !procedural) {
+                    unsupported("matrix type of projection '" + arch.getName() + "' (SPARSE, DENSE, BITMASK, PROCEDURAL or TOEPLITZ with kernel weights)");
                 }
                 if(graded && !sparse) { unsupported("graded synapses on a non-SPARSE projection ('" + arch.getName() + "')"); }
                 if(dense && wumKind != GENNMI_WUM_STATIC_PULSE && !constantWeight) { unsupported("weight update model of DENSE projection '" + arch.getName() + "'"); }
@@ -635,7 +658,7 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                 };
 
                 out << "gennmi_presynaptic_update_group_t d = {};" << std::endl;
-                out << "d.matrix = " << (sparse ? GENNMI_MATRIX_SPARSE : (dense ? GENNMI_MATRIX_DENSE : (bitmask ? GENNMI_MATRIX_BITMASK : GENNMI_MATRIX_TOEPLITZ_CONV2D)))
+                out << "d.matrix = " << (procedural ? GENNMI_MATRIX_PROCEDURAL : sparse ? GENNMI_MATRIX_SPARSE : (dense ? GENNMI_MATRIX_DENSE : (bitmask ? GENNMI_MATRIX_BITMASK : GENNMI_MATRIX_TOEPLITZ_CONV2D)))
                     << "u; d.wum = " << ((sparse && constantWeight) ? (unsigned int)GENNMI_WUM_STATIC_PULSE : wumKind) << "u;" << std::endl;
                 if(arch.getParallelismHint() == SynapseGroup::ParallelismHint::PRESYNAPTIC) {
                     out << "d.span = " << GENNMI_SPAN_PRE << "u; d.numThreadsPerSpike = " << arch.getNumThreadsPerSpike() << "u;" << std::endl;
@@ -680,8 +703,37 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                         out << "  GENNMI_CHECK(gennmi_fill_f32(w, d.constantWeight, count)); d.g = w; }" << std::endl;
                     }
                 }
-                else {
+                else if(!procedural) {
                     out << "d.g = " << wuVar("g", scalar) << ";" << std::endl;
+                }
+                if(procedural) {
+                    // one generator stream for the connectivity and one for the weights of every projection, numbered by
+                    // the projection's place in the model's (name-ordered) list, so that a model always regenerates the same
+                    // matrix: streams 2k + 1 and 2k + 2 of the model's seed
+                    auto place = [&model](const SynapseGroupInternal &g) -> uint64_t
+                    {
+                        return (uint64_t)std::distance(model.getSynapseGroups().cbegin(), model.getSynapseGroups().find(g.getName()));
+                    };
+                    out << "d.procedural.seed = " << model.getSeed() << "ull; d.procedural.connectivity = " << procConnect << "u; d.procedural.weightSnippet = "
+                        << procWeight << "u;" << std::endl;
+                    out << "{ static const uint32_t a[] = " << tableU32(counts([&place](const SynapseGroupInternal &g){ return 2 * place(g) + 1; }))
+                        << ", b[] = " << tableU32(counts([&place](const SynapseGroupInternal &g){ return 2 * place(g) + 2; }))
+                        << "; d.procedural.connectivityStream = a[g]; d.procedural.weightStream = b[g]; }" << std::endl;
+                    if(procConnect == GENNMI_CONNECT_FIXED_NUMBER_POST) {
+                        out << "{ static const uint32_t v[] = " << tableU32(counts([](const SynapseGroupInternal &g)
+                            { return (uint64_t)g.getSparseConnectivityInitialiser().getParams().at("num").template cast<unsigned int>(); }))
+                            << "; d.procedural.num = v[g]; }" << std::endl;
+                    }
+                    else {
+                        out << "{ static const double v[] = " << table(values([](const SynapseGroupInternal &g)
+                            { return g.getSparseConnectivityInitialiser().getParams().at("prob"); }), Type::Double) << "; d.procedural.prob = v[g]; }" << std::endl;
+                    }
+                    for(size_t k = 0; k < procWeightParams.size(); k++) {
+                        const std::string name = procWeightParams[k];
+                        out << "{ static const double v[] = " << table(values([name](const SynapseGroupInternal &g)
+                            { return g.getWUInitialiser().getVarInitialisers().at("g").getParams().at(name); }), Type::Double)
+                            << "; d.procedural.weightParams[" << k << "] = v[g]; }" << std::endl;
+                    }
                 }
                 if(sparse) {
                     out << "d.rowLength = gennmiDev(" << env["_row_length"] << "); d.ind = gennmiDev(" << env["_ind"] << ");" << std::endl;
@@ -1008,6 +1060,14 @@ size_t Backend::getSynapticMatrixRowStride(const SynapseGroupInternal &sg) const
     if(sg.getMatrixType() & SynapseMatrixConnectivity::SPARSE) {
         // rows padded to 4 entries start on 16-byte boundaries, which the row loads of the kernels exploit
         return padSize(sg.getMaxConnections(), 4);
+    }
+    else if(sg.getMatrixType() & SynapseMatrixConnectivity::PROCEDURAL) {
+        // The stride the same snippet would give a stored matrix (the reference only evaluates calcMaxRowLength for SPARSE
+        // groups, synapseGroup.cc:420-430): the regenerated weights are indexed by row * stride + position like stored ones.
+        const auto &init = sg.getSparseConnectivityInitialiser();
+        const auto calcMaxRowLength = init.getSnippet()->getCalcMaxRowLengthFunc();
+        return calcMaxRowLength ? calcMaxRowLength(sg.getSrcNeuronGroup()->getNumNeurons(), sg.getTrgNeuronGroup()->getNumNeurons(), init.getParams())
+                                : sg.getMaxConnections();
     }
     else if(sg.getMatrixType() & SynapseMatrixConnectivity::TOEPLITZ) {
         return sg.getMaxConnections();

@@ -292,6 +292,33 @@ def reverse(n_a=260, n_b=90, steps=200, seed=21, dt=1.0):
     return net
 
 
+def procedural(n_e=1600, n_i=400, steps=200, seed=31, dt=1.0, order_free=False):
+    """Recurrent LIF network whose four projections are PROCEDURAL: FixedProbability[NoAutapse] and
+    FixedNumberPostWithReplacement connectivity, constant, Uniform and Normal weights.  Nothing is stored: the matrices are a
+    function of the seed.  ``order_free``: one dyadic weight per projection into DeltaCurr inputs, so that every sum is exact
+    in any order and two executors that regenerate the same matrices stay identical for ever."""
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.56, TauRefrac=2.0)
+    net = Net(name="procedural", dt=dt, steps=steps, seed=seed)
+    net.pops.append(Pop("E", "lif", n_e, dict(lif), {"V": (-60.0 + 10.0 * rng.uniform(seed, 1, 0, n_e)).astype(np.float32), "RefracTime": np.zeros(n_e, np.float32)}))
+    net.pops.append(Pop("I", "lif", n_i, dict(lif), {"V": (-60.0 + 10.0 * rng.uniform(seed, 2, 0, n_i)).astype(np.float32), "RefracTime": np.zeros(n_i, np.float32)}))
+    net.syns.append(Syn("EE", "E", "E", matrix="procedural", wum="static", psm="expcurr", tau=5.0,
+                        connect=("FixedProbabilityNoAutapse", {"prob": 0.05}), g_init=("Uniform", {"min": 0.0, "max": 0.1})))
+    net.syns.append(Syn("EI", "E", "I", matrix="procedural", wum="static_const", wum_params={"g": 0.05}, psm="expcurr", tau=5.0,
+                        connect=("FixedNumberPostWithReplacement", {"num": 20})))
+    net.syns.append(Syn("IE", "I", "E", matrix="procedural", wum="static", psm="expcurr", tau=10.0,
+                        connect=("FixedProbability", {"prob": 0.05}), g_init=("Normal", {"mean": -0.3, "sd": 0.05})))
+    net.syns.append(Syn("II", "I", "I", matrix="procedural", wum="static", psm="expcurr", tau=10.0,
+                        connect=("FixedNumberPostWithReplacement", {"num": 300}), g_init=("Constant", {"constant": -0.3})))
+    if order_free:
+        for s, w in zip(net.syns, (0.015625, 0.03125, -0.0625, -0.0625)):
+            s.psm = "deltacurr"
+            if s.wum == "static_const":
+                s.wum_params = {"g": w}
+            else:
+                s.g_init = ("Constant", {"constant": w})
+    return net
+
+
 def dense_layer(n_in=8192, n_out=8192, rate_hz=50.0, steps=1000, seed=17, dt=1.0, w_sd=0.02):
     """A fully connected spiking layer: Poisson sources (rate_hz per source) into LIF neurons through a DENSE matrix
     with individual weights ~ N(0, w_sd); the shape of the dense layers of rate-coded classifiers."""

@@ -601,9 +601,10 @@ class GeNNModel:
             elif s.matrix_type == "PROCEDURAL":
                 # nothing is stored: the generator streams the stored matrix would have used are reserved in the same order
                 s.row_stride = max_row_length(s.conn.snippet, s.conn.params, s.src.num_neurons, s.trg.num_neurons)
-                s.procedural_streams = [self._next_stream(), 0]
-                if s.wu.snippet == "StaticPulse" and isinstance(s.wu.vars["g"], VarInit):
-                    s.procedural_streams[1] = self._next_stream()
+                if s.procedural_streams is None:        # (a caller that must reproduce another numbering sets them beforehand)
+                    s.procedural_streams = [self._next_stream(), 0]
+                    if s.wu.snippet == "StaticPulse" and isinstance(s.wu.vars["g"], VarInit):
+                        s.procedural_streams[1] = self._next_stream()
             elif s.matrix_type == "DENSE":
                 if s.wu.snippet == "StaticPulse":
                     count = s.src.num_neurons * s.trg.num_neurons
@@ -997,7 +998,14 @@ def model_from_net(net, batch_size=1, record=True, span=None, device=0):
             wu = init_weight_update("StaticPulseReverse", {}, {"g": 0.0})
         else:
             wu = init_weight_update("STDPTrace", s.wum_params, {"g": 0.0}, {"preTrace": 0.0}, {"postTrace": 0.0})
-        if s.matrix == "dense":
+        if s.matrix == "procedural":
+            if s.wum == "static":
+                wu = init_weight_update("StaticPulse", {}, {"g": init_var(*s.g_init)})
+            sg = m.add_synapse_population(s.name, "PROCEDURAL", pops[s.src], pops[s.trg], wu, ps, init_sparse_connectivity(*s.connect))
+            # the numbering a GeNN model gets from the backend adapter: streams 2k + 1 and 2k + 2 for the k-th projection by name
+            k = sorted(x.name for x in net.syns).index(s.name)
+            sg.procedural_streams = [2 * k + 1, 2 * k + 2]
+        elif s.matrix == "dense":
             sg = m.add_synapse_population(s.name, "DENSE", pops[s.src], pops[s.trg], wu, ps)
             if s.g is not None:
                 sg.set_var_ragged("g", s.g)
@@ -1024,5 +1032,6 @@ def model_from_net(net, batch_size=1, record=True, span=None, device=0):
             sg = m.add_synapse_population(s.name, "TOEPLITZ", pops[s.src], pops[s.trg], wu, ps,
                                           init_toeplitz_connectivity("Conv2D", s.conv))
             sg.set_var_ragged("g", s.g)
+    m.seed = net.seed
     m.build()
     return m

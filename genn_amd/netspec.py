@@ -64,11 +64,17 @@ class Syn:
     threads_per_spike: int = 1
     axonal_delay_steps: int = 0     # spikes reach the projection this many timesteps late (SynapseGroup::setAxonalDelaySteps)
     conv: Dict[str, int] = field(default_factory=dict)
+    # matrix == "procedural": connect = (snippet, params) of a built-in connectivity snippet, g_init = (snippet, params) of the
+    # weight initialisation snippet (or wum "static_const"); nothing is stored
+    connect: Optional[tuple] = None
+    g_init: Optional[tuple] = None
 
     @property
     def num_synapses(self):
         if self.matrix == "bitmask":
             return int(np.unpackbits(np.ascontiguousarray(self.gp).view(np.uint8)).sum())
+        if self.matrix == "procedural":
+            return 0
         if self.matrix == "dense":
             return int(self.g.size) if self.g is not None else 0
         return int(self.row_length.sum()) if self.row_length is not None else 0
@@ -133,6 +139,8 @@ def write_netspec(net: Net, path: str):
     lines.append(f"snap {snap}")
     if getattr(net, "batch_size", 1) != 1:
         lines.append(f"batch {int(net.batch_size)}")
+    if any(s.matrix == "procedural" for s in net.syns):
+        lines.append(f"seed {int(net.seed)}")        # procedural matrices are regenerated from the model's seed
     for p in net.pops:
         if p.model == "lif":
             ps = " ".join(repr(float(p.params[k])) for k in LIF_PARAMS)
@@ -159,14 +167,22 @@ def write_netspec(net: Net, path: str):
             np.ascontiguousarray(s.ind, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.ind.u32"))
         elif s.matrix == "dense":
             head = f"syn {s.name} dense {s.src} {s.trg}"
+        elif s.matrix == "procedural":
+            snippet, params = s.connect
+            value = params["num"] if snippet == "FixedNumberPostWithReplacement" else repr(float(params["prob"]))
+            head = f"syn {s.name} procedural {s.src} {s.trg} {snippet} {value}"
         elif s.matrix == "bitmask":
             head = f"syn {s.name} bitmask {s.src} {s.trg}"
             np.ascontiguousarray(s.gp, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.gp.u32"))
         else:
             head = f"syn {s.name} conv2d {s.src} {s.trg} " + " ".join(str(int(s.conv[k])) for k in CONV_PARAMS)
-        if s.wum != "static_const":
+        if s.wum != "static_const" and s.matrix != "procedural":
             np.ascontiguousarray(s.g, dtype=np.float32).tofile(os.path.join(path, f"{s.name}.g.f32"))
-        if s.wum in ("static", "static_reverse"):
+        if s.matrix == "procedural" and s.wum == "static":
+            snippet, params = s.g_init
+            order = {"Constant": ("constant",), "Uniform": ("min", "max"), "Normal": ("mean", "sd")}[snippet]
+            w = f"static_init {snippet} " + " ".join(repr(float(params[k])) for k in order)
+        elif s.wum in ("static", "static_reverse"):
             w = s.wum
         elif s.wum == "static_const":
             w = f"static_const {float(s.wum_params['g'])!r}"

@@ -144,7 +144,8 @@ struct PopSpec { std::string name, model; unsigned int n; std::vector<double> p;
 struct CSSpec { std::string name, model, pop; std::vector<double> p; CurrentSource *cs = nullptr; };
 struct SynSpec
 {
-    std::string name, matrix, src, trg, wum, psm;
+    std::string name, matrix, src, trg, wum, psm, connect, initSnippet;
+    double connectValue = 0.0;
     unsigned int rowStride = 0, maxDenDelay = 0, tps = 1, colStride = 0, axonalDelay = 0;
     bool hintPre = false;
     std::vector<double> conv, wumP, psmP;
@@ -174,7 +175,7 @@ int main(int argc, char *argv[])
         // ---- parse net.txt -----------------------------------------------------------------
         std::string name = "net";
         double dt = 1.0;
-        unsigned int steps = 1, snap = 0, fuse = 0, batch = 1;
+        unsigned int steps = 1, snap = 0, fuse = 0, batch = 1, seed = 0;
         std::vector<PopSpec> pops; std::vector<CSSpec> css; std::vector<SynSpec> syns;
         {
             std::ifstream f(in + "/net.txt");
@@ -189,19 +190,22 @@ int main(int argc, char *argv[])
                 else if(k == "snap") ls >> snap;
                 else if(k == "fuse_psm") ls >> fuse;
                 else if(k == "batch") ls >> batch;
+                else if(k == "seed") ls >> seed;
                 else if(k == "pop") { PopSpec p; ls >> p.name >> p.model >> p.n; double v; while(ls >> v) p.p.push_back(v); pops.push_back(p); }
                 else if(k == "cs") { CSSpec c; ls >> c.name >> c.model >> c.pop; double v; while(ls >> v) c.p.push_back(v); css.push_back(c); }
                 else if(k == "syn") {
                     SynSpec s; ls >> s.name >> s.matrix >> s.src >> s.trg;
                     if(s.matrix == "sparse") { ls >> s.rowStride; }
                     else if(s.matrix == "conv2d") { s.conv.resize(8); for(auto &c : s.conv) ls >> c; }
+                    else if(s.matrix == "procedural") { ls >> s.connect >> s.connectValue; }
                     else if(s.matrix != "dense" && s.matrix != "bitmask") throw std::runtime_error("matrix " + s.matrix);
                     ls >> s.wum;
+                    if(s.wum == "static_init") { ls >> s.initSnippet; const int np = (s.initSnippet == "Constant") ? 1 : 2; s.wumP.resize(np); for(auto &c : s.wumP) ls >> c; }
                     if(s.wum == "static_delay") { ls >> s.maxDenDelay; }
                     else if(s.wum == "stdp_trace" || s.wum == "stdp") { s.wumP.resize(6); for(auto &c : s.wumP) ls >> c; }
                     else if(s.wum == "static_const") { s.wumP.resize(1); ls >> s.wumP[0]; }
                     else if(s.wum == "static_graded") { s.wumP.resize(2); ls >> s.wumP[0] >> s.wumP[1]; }
-                    else if(s.wum != "static" && s.wum != "static_reverse") throw std::runtime_error("wum " + s.wum);
+                    else if(s.wum != "static" && s.wum != "static_reverse" && s.wum != "static_init") throw std::runtime_error("wum " + s.wum);
                     ls >> s.psm;
                     if(s.psm == "expcurr") { s.psmP.resize(1); ls >> s.psmP[0]; }
                     else if(s.psm != "deltacurr") throw std::runtime_error("psm " + s.psm);
@@ -218,6 +222,7 @@ int main(int argc, char *argv[])
         model.setName(name);
         model.setDT(dt);
         model.setBatchSize(batch);
+        if(seed) { model.setSeed(seed); }
         model.setPrecision(Type::Float);
         model.setFusePostsynapticModels(fuse != 0);
         std::map<std::string, PopSpec*> popByName;
@@ -282,7 +287,20 @@ int main(int argc, char *argv[])
                     {{"tauPlus", s.wumP[0]}, {"tauMinus", s.wumP[1]}, {"Aplus", s.wumP[2]}, {"Aminus", s.wumP[3]}, {"Wmin", s.wumP[4]}, {"Wmax", s.wumP[5]}},
                     {{"g", uninitialisedVar()}});
             }
-            if(s.matrix == "sparse") {
+            if(s.wum == "static_init") {
+                const auto init = (s.initSnippet == "Constant") ? initVar<InitVarSnippet::Constant>({{"constant", s.wumP[0]}})
+                                : (s.initSnippet == "Uniform") ? initVar<InitVarSnippet::Uniform>({{"min", s.wumP[0]}, {"max", s.wumP[1]}})
+                                : initVar<InitVarSnippet::Normal>({{"mean", s.wumP[0]}, {"sd", s.wumP[1]}});
+                wum = initWeightUpdate<WeightUpdateModels::StaticPulse>({}, {{"g", init}});
+            }
+            if(s.matrix == "procedural") {
+                const auto connect = (s.connect == "FixedNumberPostWithReplacement")
+                    ? initConnectivity<InitSparseConnectivitySnippet::FixedNumberPostWithReplacement>({{"num", (unsigned int)s.connectValue}})
+                    : (s.connect == "FixedProbabilityNoAutapse") ? initConnectivity<InitSparseConnectivitySnippet::FixedProbabilityNoAutapse>({{"prob", s.connectValue}})
+                    : initConnectivity<InitSparseConnectivitySnippet::FixedProbability>({{"prob", s.connectValue}});
+                s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::PROCEDURAL, src, trg, wum, psm, connect);
+            }
+            else if(s.matrix == "sparse") {
                 s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::SPARSE, src, trg, wum, psm);
                 s.sg->setMaxConnections(s.rowStride);
                 if(s.colStride) s.sg->setMaxSourceConnections(s.colStride);
@@ -378,7 +396,7 @@ int main(int argc, char *argv[])
             else if(s.matrix == "bitmask") {
                 load(rt.getArray(*s.sg, "gp"), s.name + ".gp.u32");
             }
-            else if(s.wum != "static_const") {
+            else if(s.wum != "static_const" && s.matrix != "procedural") {
                 load(rt.getArray(*s.sg, "g"), s.name + ".g.f32");
             }
             if(s.wum == "stdp_trace") {

@@ -70,3 +70,26 @@ def test_generated_runner_exports_reference_entry_points(case):
             assert "gennmi_build_remap" in init
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_procedural_projections_generate():
+    """PROCEDURAL matrices through the adapter: the built-in connectivity and weight snippets are recognised by identity and
+    become the descriptor's `procedural` block (seed, snippet, streams 2k + 1 / 2k + 2 by projection name, parameters)."""
+    from genn_amd import configs
+    net = configs.procedural()
+    net.snap = 50
+    tmp = tempfile.mkdtemp(prefix="adapter_proc_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(net, spec)
+        res = subprocess.run([DRIVER, spec, work, out, "--generate-only"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        assert res.returncode == 0, res.stdout[-3000:]
+        code = open(os.path.join(work, net.name + "_CODE", "synapseUpdate.cc")).read()
+        assert code.count("d.procedural.seed = 31ull") == 4
+        for streams in ("a[] = {1u}, b[] = {2u}", "a[] = {3u}, b[] = {4u}", "a[] = {5u}, b[] = {6u}", "a[] = {7u}, b[] = {8u}"):
+            assert streams in code
+        assert "d.rowLength" not in code and "d.ind" not in code           # nothing stored, nothing bound
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
