@@ -1,0 +1,172 @@
+// Part of libgenn_mi355x.so: included by genn_mi355x.hip only (one translation unit).
+#ifndef GENN_MI355X_DEVICE_H
+#define GENN_MI355X_DEVICE_H
+
+namespace
+{
+constexpr int BLOCK = 256;                  // 4 wave64 per work-group
+constexpr int WAVE = 64;
+constexpr int CONV_TILE_SPIKES = 2048;      // spikes staged in LDS at a time by the Conv2D tile kernel
+constexpr int CONV_TILE_THREADS = 512;      // work-group size of the Conv2D tile kernel (8 wave64 share one LDS tile)
+constexpr uint32_t SPIN_LIMIT = 1u << 22;   // default bound of every wait for another work-group (polls)
+constexpr uint32_t REMAP_SORT_MAX = 16384;  // longest column the LDS sort handles (64 KiB)
+
+thread_local std::string g_lastError;
+
+int fail(int code, const std::string &msg)
+{
+    g_lastError = msg;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                              \
+    do {                                                                                           \
+        hipError_t e_ = (expr);                                                                    \
+        if(e_ != hipSuccess) {                                                                     \
+            return fail(GENNMI_EHIP, std::string(#expr) + ": " + hipGetErrorString(e_));           \
+        }                                                                                          \
+    } while(0)
+
+// Polls a work-group spends waiting for another one before it raises the error flag and leaves.  Set from
+// GENNMI_SPIN_LIMIT when a runner is finalised; tests of the failure path set it to 0 so that the first missed poll expires.
+__constant__ uint32_t c_spinLimit = SPIN_LIMIT;
+
+// ------------------------------------------------------------------------------------------------
+// device-side tables
+// ------------------------------------------------------------------------------------------------
+struct StepState             // device-resident; lets a captured graph be replayed unchanged
+{
+    unsigned long long timestep;
+    unsigned long long epoch;           // number of completed steps since runner creation
+    unsigned long long numRecordingTimesteps;
+};
+
+struct StepArgs              // per-launch; either direct values or offsets from *base
+{
+    const StepState *base;
+    unsigned long long k;               // offset added to base->timestep / base->epoch
+    unsigned long long epoch;           // direct
+    float t;                            // direct
+    uint32_t recordingTimestep;         // direct
+};
+
+struct Resolved { float t; uint32_t recT; unsigned long long epoch; };
+
+// step counter modulo a 32-bit period: 64-bit division is a long software routine on this part, and the
+// counter fits 32 bits for the first 4e9 steps
+__device__ __forceinline__ uint32_t modStep(unsigned long long x, uint32_t d)
+{
+    return (x >> 32) ? (uint32_t)(x % d) : ((uint32_t)x % d);
+}
+
+__device__ __forceinline__ Resolved resolve(const StepArgs &a, float dt)
+{
+    Resolved r;
+    if(a.base) {
+        const unsigned long long ts = a.base->timestep + a.k;
+        // const float t = timestep * DT  (generateRunner.cc:283)
+        r.t = (float)ts * dt;
+        const unsigned long long nr = a.base->numRecordingTimesteps;
+        r.recT = nr ? (((ts | nr) >> 32) ? (uint32_t)(ts % nr) : ((uint32_t)ts % (uint32_t)nr)) : 0u;
+        r.epoch = a.base->epoch + a.k;
+    }
+    else {
+        r.t = a.t; r.recT = a.recordingTimestep; r.epoch = a.epoch;
+    }
+    return r;
+}
+
+// Synapses whose dendritic delay is a multiple of the ring depth land in the slot the target reads in
+// the very step that delivers them.  When a runner handles them in the neuron update (see
+// gennmi_runner_finalise), each population carries one of these per outgoing delayed projection:
+// the positions of such synapses within every row.
+struct ZeroDelayEntry
+{
+    float *ringElem;                    // &denDelay[ipost] of the target ring (slot 0, batch 0)
+    const float *weight;                // &g[idSyn]: read at delivery time, so pushed weights are honoured
+    uint32_t numTrgNeurons, maxDenDelay;
+};
+
+struct NeuronGroupDev
+{
+    gennmi_neuron_update_group_t g;
+    uint32_t startBlock, numBlocks;
+    const uint32_t *zeroStart;          // [N+1] CSR offsets into zeroEntries (all outgoing projections merged), or NULL
+    const ZeroDelayEntry *zeroEntries;
+    uint32_t *shadowSpk;                // [2][batch*N] engine-private double-buffered copy of the spike queue, or NULL
+    uint32_t *shadowCnt;                // [2][batch]
+    uint32_t *spikeBitmap;              // [ceil(N/32)] engine-private bitmap of this step's spikes (populations with learnPost), or NULL
+    unsigned long long *aggEvent;       // look-back area of the spike-like event queues (groups with events), or NULL
+    float *nextSpikeTime;               // spike sources: engine-private copy of spikeTimes[startSpike] per neuron (+inf: none left)
+    size_t spikeTimesBytes;             // spike sources: bytes from spikeTimes to the end of its allocation (host bookkeeping)
+};
+
+struct PreGroupDev
+{
+    gennmi_presynaptic_update_group_t g;
+    uint32_t startBlock, numBlocks;
+    uint32_t lanesPerSpike;             // power of two, 1..64
+    uint32_t vec4;                      // rows are 16-byte aligned and padded: dwordx4 loads
+    int32_t convBH, convBW;
+    uint32_t skipZeroDelay;             // synapses with d % D == 0 are delivered by the neuron update instead
+    uint32_t tileThreshold;             // != 0: leave the step to the tile kernel when numSpikes*workPerSpike reaches it
+    uint32_t workPerSpike, pad2_;       // rowStride (SPARSE) or kh*kw*oc (Toeplitz)
+    const uint32_t *shadowSpk;          // the source population's shadow queue (read instead of srcSpk when set)
+    const uint32_t *shadowCnt;
+};
+
+// Dense-activity path of a static SPARSE projection without delay: one block accumulates the events that
+// fall into one tile of postsynaptic neurons in LDS and flushes the tile with lane-consecutive atomics.
+struct TileGroupDev
+{
+    gennmi_presynaptic_update_group_t g;
+    const uint16_t *tileOff;            // [numSrc*(numTiles+1)] first position of every row whose target is >= tile*tileSize
+    uint32_t numTiles, tileSize;
+    uint32_t tile, split, numSplits;    // this block: which tile, which share of the spikes
+    uint32_t lanes;                     // lanes per (spike, tile) segment, power of two
+    uint32_t threshold, pad_;
+};
+
+// Dense-activity path of a Toeplitz Conv2D projection: a block owns rowsPerTile output rows (all columns and
+// channels) in LDS next to a copy of the kernel weights.
+struct ConvTileDev
+{
+    gennmi_presynaptic_update_group_t g;
+    int32_t convBH, convBW;
+    uint32_t rowsPerTile, tileRow0;
+    uint32_t threshold, pad_;
+};
+
+struct PostGroupDev
+{
+    gennmi_postsynaptic_update_group_t g;
+    uint32_t startBlock, numBlocks;
+    uint32_t lanesPerSpike;
+    uint32_t denseThreshold;            // != 0: steps with at least this many postsynaptic spikes walk the rows instead
+    const uint32_t *spikeBitmap;        // [ceil(numTrg/32)] this step's postsynaptic spikes, written by the neuron update
+};
+
+// Block -> group: groups occupy consecutive block ranges (the reference pads thread ranges to block
+// multiples for the same reason, backendSIMT.h:244-323).  Every block has its own copy of its group's
+// descriptor in a table indexed by blockIdx.x.
+
+// Pointers reach the kernels through descriptor tables, so the compiler cannot know their address
+// space; these casts let it emit global_load / global_atomic instead of flat instructions.
+#define GLOBAL_AS __attribute__((address_space(1)))
+template<typename T>
+__device__ __forceinline__ GLOBAL_AS T *asGlobal(T *p) { return (GLOBAL_AS T*)p; }
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint8_t u8x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4u __attribute__((ext_vector_type(4), aligned(4)));     // dword-aligned only: segments start anywhere in a row
+typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
+
+__device__ __forceinline__ void atomicAddF32(GLOBAL_AS float *addr, float v)
+{
+    // gfx950 has a native global_atomic_add_f32; the old value is not needed
+    __builtin_amdgcn_global_atomic_fadd_f32(addr, v);
+}
+
+}   // namespace
+
+#endif

@@ -1,0 +1,704 @@
+// Part of libgenn_mi355x.so: included by genn_mi355x.hip only (one translation unit).
+#ifndef GENN_MI355X_SYNAPSE_KERNELS_H
+#define GENN_MI355X_SYNAPSE_KERNELS_H
+
+namespace
+{
+// ------------------------------------------------------------------------------------------------
+// Presynaptic update.  The unit of work is (spike, chunk of its row): a sub-group of
+// `lanesPerSpike` lanes handles `span` consecutive synapses of one row, so a long row is spread
+// over many wavefronts instead of being walked serially, and every load of ind / g / d is one
+// contiguous segment (dwordx4 per lane when rows are padded to 4 entries and 16-byte aligned).
+// lanesPerSpike = 64 is the "post span" mapping (lanes span the row); small values are the
+// "pre span" mapping (few lanes per spike, many spikes per wavefront).  Work items are dealt
+// round-robin to the sub-groups of the synapse group's blocks, so the launch geometry is fixed
+// while the spike count lives on the device.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t blockInKernel, const Resolved &st, float dt,
+                                                unsigned long long *eventCounter)
+{
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const uint32_t W = G.lanesPerSpike;
+    const uint32_t localBlock = blockInKernel - G.startBlock;
+    const uint32_t lis = threadIdx.x & (W - 1);
+    const uint32_t subGroup = (localBlock * BLOCK + threadIdx.x) / W;
+    const uint32_t numSubGroups = (G.numBlocks * BLOCK) / W;
+    // spikes of the previous step: the population's own queue, or (when this launch may run next to the
+    // neuron update that refills that queue) the shadow copy written one step ago
+    const uint32_t parity = (uint32_t)((st.epoch + 1) & 1);
+    // axonal delay: the source's queue is a ring of slots; this projection reads the slot written axonalDelaySteps + 1
+    // updates ago, (spkQuePtr + slots - delay) % slots with spkQuePtr = epoch % slots (backendBase.cc:207-216)
+    const uint32_t slots = max(1u, g.numSrcDelaySlots);
+    const uint32_t readSlot = (slots > 1) ? modStep(st.epoch + slots - g.axonalDelaySteps, slots) : 0u;
+    GLOBAL_AS const uint32_t *cntPtr = G.shadowSpk ? asGlobal(G.shadowCnt) + (size_t)parity * gridDim.y + batch
+                                                   : asGlobal(g.srcSpkCnt) + ((size_t)batch * slots + readSlot);
+    GLOBAL_AS const uint32_t *spk = G.shadowSpk ? asGlobal(G.shadowSpk) + ((size_t)parity * gridDim.y + batch) * g.numSrcNeurons
+                                                : asGlobal(g.srcSpk) + ((size_t)batch * slots + readSlot) * g.numSrcNeurons;
+    // the first spike id this sub-group would handle is fetched together with the count, not after it (the
+    // queue always holds numSrcNeurons entries, so any index below that is readable)
+    const uint32_t sparseSpan = W * (G.vec4 ? 4u : 1u);
+    const uint32_t sparseChunksPerRow = (g.rowStride + sparseSpan - 1) / sparseSpan;
+    const uint32_t firstSpike = (g.matrix == GENNMI_MATRIX_SPARSE) ? spk[min(subGroup / max(sparseChunksPerRow, 1u), g.numSrcNeurons - 1)] : 0u;
+    const uint32_t numSpikes = cntPtr[0];
+    if(G.tileThreshold && (unsigned long long)numSpikes * G.workPerSpike >= G.tileThreshold) { return; }
+    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
+    unsigned long long events = 0;
+
+    if(g.matrix == GENNMI_MATRIX_TOEPLITZ_CONV2D) {
+        // initToeplitzConnectivitySnippet.h:116-137; lanes span the kh*kw*oc diagonals, so
+        // consecutive lanes hit consecutive output channels (consecutive outPost addresses)
+        const int kh = g.conv[0], kw = g.conv[1], iw = g.conv[3], ic = g.conv[4];
+        const int oh = g.conv[5], ow = g.conv[6], oc = g.conv[7];
+        const uint32_t numDiag = (uint32_t)(kh * kw * oc);
+        const uint32_t chunksPerRow = (numDiag + W - 1) / W;
+        GLOBAL_AS const float *kernel = asGlobal(g.g);
+        // item = subGroup + k*numSubGroups, split into (spike, chunk) incrementally: no division in the loop
+        const uint32_t stepSpike = numSubGroups / chunksPerRow, stepChunk = numSubGroups % chunksPerRow;
+        uint32_t chunk = subGroup % chunksPerRow;
+        for(unsigned long long s = subGroup / chunksPerRow; s < numSpikes; ) {
+            const uint32_t j = chunk * W + lis;
+            const uint32_t ipre = spk[s];
+            s += stepSpike; chunk += stepChunk;
+            if(chunk >= chunksPerRow) { chunk -= chunksPerRow; s++; }
+            if(j < numDiag) {
+                const int preRow = (int)(ipre / ic) / iw;
+                const int preCol = (int)(ipre / ic) % iw;
+                const int preChan = (int)(ipre % ic);
+                const int kernRow = (int)(j / oc) / kw;
+                const int kernCol = (int)(j / oc) % kw;
+                const int kernOutChan = (int)(j % oc);
+                const int postRow = preRow + kernRow - G.convBH;
+                const int postCol = preCol + kernCol - G.convBW;
+                if(postRow >= 0 && postCol >= 0 && postRow < oh && postCol < ow) {
+                    const int postInd = (postRow * ow * oc) + (postCol * oc) + kernOutChan;
+                    const int kernelInd = ((kh - kernRow - 1) * kw * ic * oc) + ((kw - kernCol - 1) * ic * oc) + (preChan * oc) + kernOutChan;
+                    atomicAddF32(&outPost[postInd], kernel[kernelInd]);
+                    events++;
+                }
+            }
+        }
+    }
+    else {
+        const uint32_t D = g.maxDenDelay;
+        // *denDelayPtr = (*denDelayPtr + 1) % D happens at the start of updateSynapses
+        // (synapseUpdateGroupMerged.cc:480-483); st.epoch counts completed steps, so the pointer
+        // in force during this step is (epoch + 1) % D.
+        const uint32_t denPtr = D ? modStep(st.epoch + 1, D) : 0;
+        GLOBAL_AS float *denDelay = D ? asGlobal(g.denDelay) + (size_t)batch * D * g.numTrgNeurons : nullptr;
+        GLOBAL_AS const uint32_t *rowLength = asGlobal(g.rowLength);
+        GLOBAL_AS const uint32_t *ind = asGlobal(g.ind);
+        GLOBAL_AS float *weight = asGlobal(g.g);
+        GLOBAL_AS const uint8_t *delay = asGlobal(g.d);
+        const uint32_t numTrg = g.numTrgNeurons;
+        const uint32_t perLane = G.vec4 ? 4u : 1u;
+        const uint32_t span = W * perLane;
+        const uint32_t chunksPerRow = (g.rowStride + span - 1) / span;
+        // Loads are issued ahead of the values that decide whether they are needed, so that the
+        // dependent chain per item is spike id -> {rowLength, row chunk} -> atomics: the spike id of
+        // the NEXT item is fetched while the current one is processed (spk always holds
+        // numSrcNeurons entries, so any index below that is readable), and the row chunk is read
+        // together with rowLength (rows are padded to rowStride, so any j < rowStride is readable).
+        const uint32_t lastSrc = g.numSrcNeurons - 1;
+        uint32_t idPreNext = firstSpike;
+        // item = subGroup + k*numSubGroups, split into (spike, chunk) incrementally: no division in the loop
+        const uint32_t stepSpike = numSubGroups / chunksPerRow, stepChunk = numSubGroups % chunksPerRow;
+        uint32_t chunkNext = subGroup % chunksPerRow;
+        for(unsigned long long sNext = subGroup / chunksPerRow; sNext < numSpikes; ) {
+            const uint32_t chunk = chunkNext;
+            const uint32_t idPre = idPreNext;
+            sNext += stepSpike; chunkNext += stepChunk;
+            if(chunkNext >= chunksPerRow) { chunkNext -= chunksPerRow; sNext++; }
+            idPreNext = spk[(uint32_t)min(sNext, (unsigned long long)lastSrc)];
+            const size_t rowBase = (size_t)idPre * g.rowStride;
+            const uint32_t j = chunk * span + lis * perLane;
+            const bool inRow = (j < g.rowStride);
+            const uint32_t npost = rowLength[idPre];
+            if(g.wum == GENNMI_WUM_STATIC_PULSE) {
+                if(G.vec4) {
+                    u32x4 ip = {0, 0, 0, 0}; f32x4 w = {0, 0, 0, 0};
+                    if(inRow) {
+                        ip = *reinterpret_cast<GLOBAL_AS const u32x4*>(ind + rowBase + j);
+                        w = *reinterpret_cast<GLOBAL_AS const f32x4*>(weight + rowBase + j);
+                    }
+                    if(j < npost) { atomicAddF32(&outPost[ip.x], w.x); }
+                    if(j + 1 < npost) { atomicAddF32(&outPost[ip.y], w.y); }
+                    if(j + 2 < npost) { atomicAddF32(&outPost[ip.z], w.z); }
+                    if(j + 3 < npost) { atomicAddF32(&outPost[ip.w], w.w); }
+                }
+                else {
+                    uint32_t ip = 0; float w = 0;
+                    if(inRow) { ip = ind[rowBase + j]; w = weight[rowBase + j]; }
+                    if(j < npost) { atomicAddF32(&outPost[ip], w); }
+                }
+            }
+            else if(g.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY) {
+                // addToPostDelay(g, d): denDelay[((ptr + d) % D) * numPost + idPost] += g  (synapseUpdateGroupMerged.cc:245-251)
+                if(G.vec4) {
+                    u32x4 ip = {0, 0, 0, 0}; f32x4 w = {0, 0, 0, 0}; u8x4 dl = {0, 0, 0, 0};
+                    if(inRow) {
+                        ip = *reinterpret_cast<GLOBAL_AS const u32x4*>(ind + rowBase + j);
+                        w = *reinterpret_cast<GLOBAL_AS const f32x4*>(weight + rowBase + j);
+                        dl = *reinterpret_cast<GLOBAL_AS const u8x4*>(delay + rowBase + j);
+                    }
+                    const uint32_t s0 = (denPtr + dl.x) % D, s1 = (denPtr + dl.y) % D, s2 = (denPtr + dl.z) % D, s3 = (denPtr + dl.w) % D;
+                    const bool skip = (G.skipZeroDelay != 0);       // slot == denPtr <=> d % D == 0
+                    if(j < npost && !(skip && s0 == denPtr)) { atomicAddF32(&denDelay[(size_t)s0 * numTrg + ip.x], w.x); }
+                    if(j + 1 < npost && !(skip && s1 == denPtr)) { atomicAddF32(&denDelay[(size_t)s1 * numTrg + ip.y], w.y); }
+                    if(j + 2 < npost && !(skip && s2 == denPtr)) { atomicAddF32(&denDelay[(size_t)s2 * numTrg + ip.z], w.z); }
+                    if(j + 3 < npost && !(skip && s3 == denPtr)) { atomicAddF32(&denDelay[(size_t)s3 * numTrg + ip.w], w.w); }
+                }
+                else {
+                    uint32_t ip = 0; float w = 0; uint32_t dl = 0;
+                    if(inRow) { ip = ind[rowBase + j]; w = weight[rowBase + j]; dl = delay[rowBase + j]; }
+                    const uint32_t slot = (denPtr + dl) % D;
+                    if(j < npost && !(G.skipZeroDelay && slot == denPtr)) { atomicAddF32(&denDelay[(size_t)slot * numTrg + ip], w); }
+                }
+            }
+            else if(g.wum == GENNMI_WUM_STATIC_PULSE_REVERSE) {
+                // addToPre(g): the weights of the row go to the spiking neuron itself; a lane sums its share, the lanes of the
+                // (spike, chunk) item combine theirs, one atomic per item
+                float sum = 0.0f;
+                for(uint32_t q = 0; q < perLane; q++) { if(inRow && j + q < npost) { sum += weight[rowBase + j + q]; } }
+                for(uint32_t off = W / 2; off > 0; off >>= 1) { sum += __shfl_xor(sum, off, WAVE); }
+                if(lis == 0 && sum != 0.0f) { atomicAddF32(asGlobal(g.outPre) + (size_t)batch * g.numSrcNeurons + idPre, sum); }
+            }
+            else if(g.wum == GENNMI_WUM_STATIC_GRADED) {
+                // event code of weightUpdateModels.h:318: addToPost(fmax(0.0, g * tanh((V_pre - Epre) / Vslope) * dt)).  The CPU
+                // backend's generated code evaluates tanh, the products and the maximum in double (only the double versions of
+                // tanh and fmax are in scope there); so does this, rounding once before the fp32 atomic.
+                const float vPre = asGlobal(g.srcV)[(size_t)batch * g.numSrcNeurons + idPre];
+                const double release = tanh((double)((vPre - g.gradedEpre) / g.gradedVslope));
+                for(uint32_t q = 0; q < perLane; q++) {
+                    if(inRow && j + q < npost) {
+                        atomicAddF32(&outPost[ind[rowBase + j + q]], (float)fmax(0.0, (double)weight[rowBase + j + q] * release * (double)dt));
+                    }
+                }
+            }
+            else if(j < npost) {
+                // trace STDP presynaptic-spike code (pygenn/genn_model.py:1456-1463); every synapse of
+                // the row is owned by exactly one lane, so the read-modify-write of g needs no atomic
+                const uint32_t idPost = ind[rowBase + j];
+                const float w = weight[rowBase + j];
+                const float stPost = dt + asGlobal(g.trgST)[idPost];   // st_post = DT*(backPropSteps+1) + trgST (synapseUpdateGroupMerged.cc:134-142)
+                atomicAddF32(&outPost[idPost], w);
+                const float dtSpike = st.t - stPost;
+                if(dtSpike > 0) {
+                    const float newWeight = w - (g.aMinus * asGlobal(g.postTrace)[idPost]);
+                    weight[rowBase + j] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
+                }
+            }
+            if(lis == 0 && chunk == 0) { events += npost; }
+        }
+    }
+
+    // one counter update per wave
+    for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
+    if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// ------------------------------------------------------------------------------------------------
+// DENSE and BITMASK projections (single_threaded_cpu/backend.cc:1985-2021 is the sequential definition).  One lane
+// per postsynaptic neuron walks the spike queue: weights of a spike's row are lane-consecutive (DENSE: g[idPre*numTrg
+// + idPost]) or one bit each (BITMASK, most significant bit first), so there is nothing to scatter and no atomic —
+// a lane that owns its outPost element alone continues the sum from the value that is there, in queue order, which is
+// the CPU backend's order bit for bit.  When several projections feed one outPost, or a step carries so many spikes
+// that the queue is shared between several blocks, the lane's partial sum is added with one (lane-consecutive) atomic.
+// ------------------------------------------------------------------------------------------------
+struct DenseGroupDev
+{
+    gennmi_presynaptic_update_group_t g;
+    uint32_t startBlock, numBlocks;     // numBlocks = column blocks x slices
+    uint32_t exclusive;                 // no other projection adds to this outPost
+    uint32_t slices;                    // blocks that may share the spike queue of one block of columns
+};
+
+constexpr uint32_t DENSE_SPIKES_PER_SLICE = 16;     // a step with fewer spikes than this per slice uses fewer slices
+
+__global__ __launch_bounds__(BLOCK)
+void presynapticDenseKernel(const DenseGroupDev * __restrict__ blocks, unsigned long long *eventCounter)
+{
+    const DenseGroupDev &G = blocks[blockIdx.x];
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const uint32_t local = blockIdx.x - G.startBlock;
+    const uint32_t slice = local % G.slices;
+    const uint32_t j = (local / G.slices) * BLOCK + threadIdx.x;
+    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
+    // The queue is cut into as many contiguous pieces as there are slices with at least 16 spikes each; with one
+    // piece the lane continues the sum from outPost itself (exact queue order), with more every piece adds its partial sum.
+    const uint32_t active = min(G.slices, max(1u, numSpikes / DENSE_SPIKES_PER_SLICE));
+    if(numSpikes == 0 || slice >= active) { return; }
+    const uint32_t perSlice = (numSpikes + active - 1) / active;
+    const uint32_t first = slice * perSlice, last = min(numSpikes, first + perSlice);
+    if(first >= numSpikes) { return; }          // rounding up perSlice can leave the last pieces empty
+    const bool continueSum = G.exclusive && active == 1;
+    GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
+    unsigned long long events = 0;
+    if(j < g.numTrgNeurons) {
+        float acc = continueSum ? outPost[j] : 0.0f;
+        if(g.matrix == GENNMI_MATRIX_DENSE) {
+            const bool constant = (g.wum == GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT);
+            GLOBAL_AS const float *weight = asGlobal(g.g);
+            // eight rows in flight; the additions keep queue order
+            uint32_t s = first;
+            for(; s + 8 <= last; s += 8) {
+                float w[8];
+                #pragma unroll
+                for(int u = 0; u < 8; u++) { w[u] = constant ? g.constantWeight : weight[(size_t)spk[s + u] * g.numTrgNeurons + j]; }
+                #pragma unroll
+                for(int u = 0; u < 8; u++) { acc += w[u]; }
+            }
+            for(; s < last; s++) { acc += constant ? g.constantWeight : weight[(size_t)spk[s] * g.numTrgNeurons + j]; }
+            if(j == 0) { events = (unsigned long long)(last - first) * g.numTrgNeurons; }
+        }
+        else {
+            GLOBAL_AS const uint32_t *gp = asGlobal(g.gp);
+            for(uint32_t s = first; s < last; s++) {
+                const unsigned long long gid = (unsigned long long)spk[s] * g.rowStride + j;
+                if(gp[gid >> 5] & (0x80000000u >> (gid & 31))) { acc += g.constantWeight; events++; }
+            }
+        }
+        if(continueSum) { outPost[j] = acc; }
+        else if(acc != 0.0f) { atomicAddF32(&outPost[j], acc); }
+    }
+    for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
+    if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// ------------------------------------------------------------------------------------------------
+// PROCEDURAL connectivity (the reference's PostSpan/PreSpan procedural strategies, presynapticUpdateStrategySIMT.cc:391-560,
+// re-run the connectivity snippet with a per-row generator state).  Here a wavefront regenerates the row of a spiking
+// neuron with exactly the code and draws the initialisation kernels use (genn_mi355x_rows.h), so a procedural projection
+// behaves synapse for synapse like the stored matrix the same seed would have produced — without reading a byte of
+// connectivity: the only memory traffic of an event is its atomic.
+// ------------------------------------------------------------------------------------------------
+struct ProcGroupDev
+{
+    gennmi_presynaptic_update_group_t g;
+    uint32_t startBlock, numBlocks;
+    gennmi_rows::Stream connectivity, weight;
+    gennmi_rows::VarInit weightInit;
+    float probLogRecip;
+    uint32_t pad_;
+};
+
+__global__ __launch_bounds__(BLOCK)
+void presynapticProceduralKernel(const ProcGroupDev * __restrict__ blocks, unsigned long long *eventCounter)
+{
+    using namespace gennmi_rows;
+    constexpr uint32_t MAX_ROUNDS = 64;                 // rows of up to 16,383 targets are shared between the block's waves
+    __shared__ double shRoundTotal[MAX_ROUNDS];
+    const ProcGroupDev &G = blocks[blockIdx.x];
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const uint32_t lane = threadIdx.x & (WAVE - 1);
+    const uint32_t wave = threadIdx.x / WAVE;
+    const uint32_t localBlock = blockIdx.x - G.startBlock;
+    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
+    GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
+    const uint32_t rowStride = g.rowStride;
+    unsigned long long events = 0;
+    if(g.procedural.connectivity == GENNMI_CONNECT_FIXED_NUMBER_POST) {
+        const uint32_t n = min(g.procedural.num, rowStride);
+        // a group of four synapses shares one generator call for its weights when the row starts on a multiple of four
+        const bool aligned = (rowStride & 3u) == 0;
+        auto deliver = [&](unsigned long long firstElement, uint32_t k, const uint32_t post[4]) {
+            float w[4];
+            if(aligned) { valuesAt4(G.weightInit, G.weight, firstElement + k, w); }
+            else { for(int i = 0; i < 4; i++) { w[i] = valueAt(G.weightInit, G.weight, firstElement + k + i); } }
+            for(int i = 0; i < 4 && k + i < n; i++) { atomicAddF32(&outPost[post[i]], w[i]); }
+        };
+        if(n / (4 * WAVE) + 1 > 1 && n / (4 * WAVE) + 1 <= MAX_ROUNDS) {
+            // long rows: one spike per block, the block's waves share the row's rounds of 256 draws
+            for(uint32_t s = localBlock; s < numSpikes; s += G.numBlocks) {
+                const uint32_t row = spk[s];
+                const unsigned long long firstElement = (unsigned long long)row * rowStride;
+                fixedNumberPostRowBlock<BLOCK / WAVE>(row, g.numTrgNeurons, n, G.connectivity, lane, wave, shRoundTotal, MAX_ROUNDS,
+                                                      [&](uint32_t k, const uint32_t post[4]) { deliver(firstElement, k, post); });
+                if(threadIdx.x == 0) { events += n; }
+            }
+        }
+        else {
+            const uint32_t numWaves = G.numBlocks * (BLOCK / WAVE);
+            for(uint32_t s = localBlock * (BLOCK / WAVE) + wave; s < numSpikes; s += numWaves) {
+                const uint32_t row = spk[s];
+                const unsigned long long firstElement = (unsigned long long)row * rowStride;
+                fixedNumberPostRow(row, g.numTrgNeurons, n, G.connectivity, lane, [&](uint32_t k, const uint32_t post[4]) { deliver(firstElement, k, post); });
+                if(lane == 0) { events += n; }
+            }
+        }
+    }
+    else {
+        const uint32_t numWaves = G.numBlocks * (BLOCK / WAVE);
+        for(uint32_t s = localBlock * (BLOCK / WAVE) + wave; s < numSpikes; s += numWaves) {
+            const uint32_t row = spk[s];
+            const unsigned long long firstElement = (unsigned long long)row * rowStride;
+            const uint32_t total = fixedProbabilityRow(row, g.numTrgNeurons, G.probLogRecip,
+                                                       g.procedural.connectivity == GENNMI_CONNECT_FIXED_PROBABILITY_NO_AUTAPSE, G.connectivity, lane,
+                                                       [&](uint32_t k, uint32_t post) {
+                if(k < rowStride) { atomicAddF32(&outPost[post], valueAt(G.weightInit, G.weight, firstElement + k)); }
+            });
+            if(lane == 0) { events += min(total, rowStride); }
+        }
+    }
+    for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
+    if(lane == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Tile kernel.  Scattered fp32 atomics cost one memory transaction each (≈20 G/s measured on this part,
+// whatever the array size), lane-consecutive ones ≈280 G/s.  When a step carries enough events
+// (numSpikes*rowStride >= numTrg), a block therefore owns a tile of postsynaptic neurons in LDS: it walks
+// its share of the spike list, reads only the segment of each row that falls into its tile (rows are
+// sorted by target; tileOff holds the segment boundaries), adds into LDS, and finally flushes the tile
+// with consecutive lanes on consecutive addresses.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024)
+void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs args, float dt, unsigned long long *eventCounter)
+{
+    extern __shared__ float shTile[];
+    const TileGroupDev &G = blocks[blockIdx.x];
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
+    if((unsigned long long)numSpikes * g.rowStride < G.threshold) { return; }      // the scatter kernel took this step
+    const uint32_t tileStart = G.tile * G.tileSize;
+    const uint32_t tileLen = min(G.tileSize, g.numTrgNeurons - tileStart);
+    for(uint32_t k = threadIdx.x; k < tileLen; k += blockDim.x) { shTile[k] = 0.0f; }
+    __syncthreads();
+
+    GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    GLOBAL_AS const uint16_t *off = asGlobal(G.tileOff);
+    GLOBAL_AS const uint32_t *ind = asGlobal(g.ind);
+    GLOBAL_AS float *weight = asGlobal(g.g);
+    // trace-STDP rows: besides delivering the (old) weight, every event applies the presynaptic-spike rule to its own
+    // synapse (pygenn/genn_model.py:1456-1463); a synapse belongs to exactly one tile, so g needs no atomic here either
+    const bool stdp = (g.wum == GENNMI_WUM_STDP_TRACE);
+    const float t = stdp ? resolve(args, dt).t : 0.0f;
+    GLOBAL_AS const float *trgST = asGlobal(g.trgST);
+    GLOBAL_AS const float *postTrace = asGlobal(g.postTrace);
+    auto depress = [&](uint32_t idPost, float w) -> float {
+        const float stPost = dt + trgST[idPost];
+        const float dtSpike = t - stPost;
+        if(dtSpike > 0) { return fminf(g.wMax, fmaxf(g.wMin, w - (g.aMinus * postTrace[idPost]))); }
+        return w;
+    };
+    const uint32_t L = G.lanes;
+    const uint32_t lis = threadIdx.x & (L - 1);
+    const uint32_t perBlock = blockDim.x / L;
+    const uint32_t stride = perBlock * G.numSplits;
+    const uint32_t lastSrc = g.numSrcNeurons - 1;
+    unsigned long long events = 0;
+    // software pipeline over this sub-group's spikes: the spike id is fetched two iterations ahead and the
+    // segment boundaries one iteration ahead (spk holds numSrcNeurons entries, so clamped indices are readable)
+    uint32_t s = G.split * perBlock + threadIdx.x / L;
+    uint32_t id0 = spk[min(s, lastSrc)], id1 = spk[min(s + stride, lastSrc)];
+    size_t o0 = (size_t)id0 * (G.numTiles + 1) + G.tile;
+    uint32_t a0 = off[o0], b0 = off[o0 + 1];
+    for(; s < numSpikes; s += stride) {
+        const uint32_t idPre = id0, a = a0, b = b0;
+        id0 = id1;
+        id1 = spk[min(s + 2 * stride, lastSrc)];
+        o0 = (size_t)id0 * (G.numTiles + 1) + G.tile;
+        a0 = off[o0]; b0 = off[o0 + 1];
+        const size_t rowBase = (size_t)idPre * g.rowStride;
+        for(uint32_t j = a + 4 * lis; j < b; j += 4 * L) {
+            if(j + 4 <= b) {
+                const u32x4u ip = *reinterpret_cast<GLOBAL_AS const u32x4u*>(ind + rowBase + j);
+                const f32x4u w = *reinterpret_cast<GLOBAL_AS const f32x4u*>(weight + rowBase + j);
+                if(stdp) {
+                    f32x4u nw;
+                    nw.x = depress(ip.x, w.x); nw.y = depress(ip.y, w.y); nw.z = depress(ip.z, w.z); nw.w = depress(ip.w, w.w);
+                    *reinterpret_cast<GLOBAL_AS f32x4u*>(weight + rowBase + j) = nw;
+                }
+                unsafeAtomicAdd(&shTile[ip.x - tileStart], w.x);
+                unsafeAtomicAdd(&shTile[ip.y - tileStart], w.y);
+                unsafeAtomicAdd(&shTile[ip.z - tileStart], w.z);
+                unsafeAtomicAdd(&shTile[ip.w - tileStart], w.w);
+            }
+            else {
+                for(uint32_t jj = j; jj < b; jj++) {
+                    const uint32_t idPost = ind[rowBase + jj];
+                    const float w = weight[rowBase + jj];
+                    if(stdp) { weight[rowBase + jj] = depress(idPost, w); }
+                    unsafeAtomicAdd(&shTile[idPost - tileStart], w);
+                }
+            }
+        }
+        if(lis == 0) { events += b - a; }
+    }
+    __syncthreads();
+    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons + tileStart;
+    for(uint32_t k = threadIdx.x; k < tileLen; k += blockDim.x) {
+        const float v = shTile[k];
+        if(v != 0.0f) { atomicAddF32(&outPost[k], v); }
+    }
+    for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
+    if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// Toeplitz Conv2D counterpart of the tile kernel: every block finds the run of spikes whose kernel footprint touches
+// its output rows and accumulates their contributions in an LDS tile, each wavefront in its own band of columns.  The block owns its rows exclusively, so the flush is a plain read-modify-write without atomics.
+__global__ __launch_bounds__(CONV_TILE_THREADS)
+void presynapticConvTileKernel(const ConvTileDev * __restrict__ blocks, unsigned long long *eventCounter)
+{
+    extern __shared__ float shConv[];
+    const ConvTileDev &G = blocks[blockIdx.x];
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const int kh = g.conv[0], kw = g.conv[1], iw = g.conv[3], ic = g.conv[4];
+    const int oh = g.conv[5], ow = g.conv[6], oc = g.conv[7];
+    const uint32_t numDiag = (uint32_t)(kh * kw * oc);
+    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
+    if((unsigned long long)numSpikes * numDiag < G.threshold) { return; }      // the scatter kernel took this step
+    const int row0 = (int)G.tileRow0;
+    const int rows = min((int)G.rowsPerTile, oh - row0);
+    const uint32_t tileLen = (uint32_t)(rows * ow * oc);
+    const uint32_t kernelLen = (uint32_t)(kh * kw * ic * oc);
+    float *tile = shConv;
+    float *kern = tile + G.rowsPerTile * ow * oc;
+    uint32_t *stage = reinterpret_cast<uint32_t*>(kern + kernelLen);
+    __shared__ uint32_t shLo, shHi;
+    if(threadIdx.x == 0) { shLo = 0u; shHi = 0u; }
+    for(uint32_t k = threadIdx.x; k < tileLen; k += blockDim.x) { tile[k] = 0.0f; }
+    for(uint32_t k = threadIdx.x; k < kernelLen; k += blockDim.x) { kern[k] = asGlobal(g.g)[k]; }
+    __syncthreads();
+
+    // The queue is in ascending neuron index, i.e. sorted by input row, so the spikes whose kernel footprint reaches
+    // this block's output rows — input rows [row0 + bh - kh + 1, row0 + rows + bh) — form one contiguous run
+    // [lo, hi): count the spikes in front of either bound.
+    GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+    const uint32_t lane = threadIdx.x & (WAVE - 1);
+    const uint32_t wave = threadIdx.x / WAVE, numWaves = blockDim.x / WAVE;
+    const int firstRow = row0 + G.convBH - kh + 1, endRow = row0 + rows + G.convBH;
+    uint32_t below = 0, upto = 0;
+    for(uint32_t s = threadIdx.x; s < numSpikes; s += blockDim.x) {
+        const int myRow = (int)(spk[s] / ic) / iw;
+        below += (myRow < firstRow) ? 1u : 0u;
+        upto += (myRow < endRow) ? 1u : 0u;
+    }
+    for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { below += __shfl_down(below, o2, WAVE); upto += __shfl_down(upto, o2, WAVE); }
+    if(lane == 0) { atomicAdd(&shLo, below); atomicAdd(&shHi, upto); }
+    __syncthreads();
+    const uint32_t lo = shLo, hi = shHi;
+    unsigned long long events = 0;
+    // The run is staged in LDS (decoded to row / column / channel) CONV_TILE_SPIKES at a time.  LDS float atomics
+    // retire about one lane per clock, so none are used: every wavefront owns a band of output columns, picks the
+    // staged spikes whose footprint touches its band (64 tested at a time), and adds their contributions to its own
+    // columns with plain read-modify-write.  Per output element the contributions arrive in queue order, the order of
+    // the CPU backend's loop.
+    const int colsPerWave = (ow + (int)numWaves - 1) / (int)numWaves;
+    const int col0 = (int)wave * colsPerWave, col1 = min(ow, col0 + colsPerWave);
+    for(uint32_t base = lo; base < hi; base += CONV_TILE_SPIKES) {
+        const uint32_t count = min((uint32_t)CONV_TILE_SPIKES, hi - base);
+        __syncthreads();
+        for(uint32_t k = threadIdx.x; k < count; k += blockDim.x) {
+            const uint32_t id = spk[base + k];
+            const uint32_t preRow = (id / ic) / iw, preCol = (id / ic) % iw, preChan = id % ic;
+            // a queue that is not sorted would put foreign spikes inside the run: they are marked and skipped
+            const bool relevant = ((int)preRow >= firstRow) && ((int)preRow < endRow);
+            stage[k] = relevant ? (preRow << 20 | preCol << 10 | preChan) : 0xFFFFFFFFu;
+        }
+        __syncthreads();
+        for(uint32_t sb = 0; sb < count && col0 < col1; sb += WAVE) {
+            const uint32_t mine = (sb + lane < count) ? stage[sb + lane] : 0xFFFFFFFFu;
+            const int myCol = (int)((mine >> 10) & 1023) - G.convBW;       // first output column this spike reaches
+            unsigned long long pending = __ballot(mine != 0xFFFFFFFFu && myCol + kw - 1 >= col0 && myCol < col1);
+            while(pending) {
+                const int src = __ffsll((long long)pending) - 1;
+                pending &= pending - 1;
+                // everything about the spike and the kernel position is wavefront-uniform (scalar registers, scalar
+                // branches); only the output channels are spread over the lanes
+                const uint32_t pre = __builtin_amdgcn_readlane(mine, src);
+                const int preRow = (int)(pre >> 20), preCol = (int)((pre >> 10) & 1023), preChan = (int)(pre & 1023);
+                for(int kernRow = 0; kernRow < kh; kernRow++) {
+                    const int postRow = preRow + kernRow - G.convBH;
+                    if(postRow < row0 || postRow >= row0 + rows) { continue; }
+                    for(int kernCol = 0; kernCol < kw; kernCol++) {
+                        const int postCol = preCol + kernCol - G.convBW;
+                        if(postCol < col0 || postCol >= col1) { continue; }
+                        const float *weights = kern + (((kh - kernRow - 1) * kw + (kw - kernCol - 1)) * ic + preChan) * oc;
+                        float *target = tile + ((postRow - row0) * ow + postCol) * oc;
+                        for(int ch = (int)lane; ch < oc; ch += WAVE) { target[ch] += weights[ch]; }
+                        if(lane == 0) { events += (unsigned long long)oc; }
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons + (size_t)row0 * ow * oc;
+    // the block owns these rows, so plain read-modify-write; loads of a batch of elements are issued together
+    for(uint32_t k0 = 0; k0 < tileLen; k0 += 8 * blockDim.x) {
+        float old[8];
+        #pragma unroll
+        for(int u = 0; u < 8; u++) { const uint32_t k = k0 + u * blockDim.x + threadIdx.x; old[u] = (k < tileLen) ? outPost[k] : 0.0f; }
+        #pragma unroll
+        for(int u = 0; u < 8; u++) {
+            const uint32_t k = k0 + u * blockDim.x + threadIdx.x;
+            if(k < tileLen) { const float v = tile[k]; if(v != 0.0f) { outPost[k] = old[u] + v; } }
+        }
+    }
+    for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
+    if(lane == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// Segment boundaries of every row for the tile kernel; also verifies that rows are sorted by target.
+__global__ void tileOffsetKernel(uint32_t numSrc, uint32_t rowStride, const uint32_t *rowLength, const uint32_t *ind,
+                                 uint32_t tileSize, uint32_t numTiles, uint16_t *off, uint32_t *unsorted)
+{
+    const uint32_t row = blockIdx.x * blockDim.x + threadIdx.x;
+    if(row >= numSrc) { return; }
+    const uint32_t len = rowLength[row];
+    const uint32_t *r = ind + (size_t)row * rowStride;
+    uint16_t *o = off + (size_t)row * (numTiles + 1);
+    uint32_t t = 0, prev = 0;
+    for(uint32_t j = 0; j < len; j++) {
+        const uint32_t p = r[j];
+        if(p < prev) { atomicOr(unsorted, 1u); }
+        prev = p;
+        while(t <= numTiles && (unsigned long long)t * tileSize <= p) { o[t++] = (uint16_t)j; }
+    }
+    while(t <= numTiles) { o[t++] = (uint16_t)len; }
+}
+
+__global__ __launch_bounds__(BLOCK)
+void presynapticUpdateKernel(const PreGroupDev * __restrict__ blocks, StepArgs args, float dt, unsigned long long *eventCounter)
+{
+    presynapticBody(blocks[blockIdx.x], blockIdx.x, resolve(args, dt), dt, eventCounter);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Postsynaptic update (learnPost): one sub-group per postsynaptic spike walks the column through
+// remap (coalesced), gathers g by synapse index.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(BLOCK)
+void postsynapticUpdateKernel(const PostGroupDev * __restrict__ blocks, StepArgs args, float dt)
+{
+    const Resolved st = resolve(args, dt);
+    const PostGroupDev &G = blocks[blockIdx.x];
+    const gennmi_postsynaptic_update_group_t &g = G.g;
+    const uint32_t W = G.lanesPerSpike;
+    const uint32_t localBlock = blockIdx.x - G.startBlock;
+    const uint32_t lis = threadIdx.x & (W - 1);
+    const uint32_t subGroup = (localBlock * BLOCK + threadIdx.x) / W;
+    const uint32_t numSubGroups = (G.numBlocks * BLOCK) / W;
+    const uint32_t numSpikes = g.trgSpkCnt[0];
+    if(G.denseThreshold && numSpikes >= G.denseThreshold) {
+        // A large share of the target population fired: nearly every row holds synapses to update, so walk the rows
+        // once (coalesced ind / g) and test each synapse's target against the spike bitmap, instead of one scattered
+        // read-modify-write per (spike, column entry).  Same arithmetic per synapse; every synapse is visited once.
+        extern __shared__ uint32_t shBits[];
+        const uint32_t words = (g.numTrgNeurons + 31) / 32;
+        for(uint32_t k = threadIdx.x; k < words; k += BLOCK) { shBits[k] = asGlobal(G.spikeBitmap)[k]; }
+        __syncthreads();
+        const uint32_t lane = threadIdx.x & (WAVE - 1);
+        const uint32_t numWaves = G.numBlocks * (BLOCK / WAVE);
+        GLOBAL_AS const uint32_t *ind = asGlobal(g.ind);
+        GLOBAL_AS float *weight = asGlobal(g.g);
+        // per-row scalars of the NEXT row are fetched while the current one is processed (indices clamped: readable)
+        const uint32_t lastRow = g.numSrcNeurons - 1;
+        uint32_t row = localBlock * (BLOCK / WAVE) + threadIdx.x / WAVE;
+        uint32_t lenNext = asGlobal(g.rowLength)[min(row, lastRow)];
+        float stNext = asGlobal(g.srcST)[min(row, lastRow)], traceNext = asGlobal(g.preTrace)[min(row, lastRow)];
+        for(; row < g.numSrcNeurons; row += numWaves) {
+            const uint32_t len = lenNext;
+            const float stPre = dt + stNext;
+            const float step = g.aPlus * traceNext;
+            const uint32_t nextRow = min(row + numWaves, lastRow);
+            lenNext = asGlobal(g.rowLength)[nextRow]; stNext = asGlobal(g.srcST)[nextRow]; traceNext = asGlobal(g.preTrace)[nextRow];
+            const float dtSpike = st.t - stPre;
+            if(!(dtSpike > 0) || len == 0) { continue; }
+            const size_t rowBase = (size_t)row * g.rowStride;
+            // up to four strides of the row in flight per lane
+            for(uint32_t j0 = lane; j0 < len; j0 += 4 * WAVE) {
+                uint32_t idPost[4]; float w[4];
+                #pragma unroll
+                for(int u = 0; u < 4; u++) {
+                    const uint32_t j = j0 + u * WAVE;
+                    idPost[u] = (j < len) ? ind[rowBase + j] : 0xFFFFFFFFu;
+                    w[u] = (j < len) ? weight[rowBase + j] : 0.0f;
+                }
+                #pragma unroll
+                for(int u = 0; u < 4; u++) {
+                    if(idPost[u] != 0xFFFFFFFFu && ((shBits[idPost[u] >> 5] >> (idPost[u] & 31)) & 1u)) {
+                        weight[rowBase + j0 + u * WAVE] = fminf(g.wMax, fmaxf(g.wMin, w[u] + step));
+                    }
+                }
+            }
+        }
+        return;
+    }
+    for(uint32_t s = subGroup; s < numSpikes; s += numSubGroups) {
+        const uint32_t spike = g.trgSpk[s];
+        const uint32_t npre = g.colLength[spike];
+        const size_t colBase = (size_t)spike * g.colStride;
+        for(uint32_t i = lis; i < npre; i += W) {
+            const uint32_t rowMajorIndex = g.remap[colBase + i];
+            const uint32_t idPre = rowMajorIndex / g.rowStride;
+            const float stPre = dt + g.srcST[idPre];
+            const float dtSpike = st.t - stPre;
+            if(dtSpike > 0) {
+                const float newWeight = g.g[rowMajorIndex] + (g.aPlus * g.preTrace[idPre]);
+                g.g[rowMajorIndex] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Remap build: scatter in arbitrary order, then sort every column ascending, which is the order
+// the CPU backend's row-major traversal produces (single_threaded_cpu/backend.cc:156-179).
+// ------------------------------------------------------------------------------------------------
+__global__ void remapCountKernel(uint32_t numSrc, uint32_t rowStride, const uint32_t *rowLength, const uint32_t *ind,
+                                 uint32_t colStride, uint32_t *colLength, uint32_t *remap, uint32_t *overflow)
+{
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t total = (size_t)numSrc * rowStride;
+    if(idx >= total) { return; }
+    const uint32_t row = (uint32_t)(idx / rowStride), j = (uint32_t)(idx % rowStride);
+    if(j >= rowLength[row]) { return; }
+    const uint32_t post = ind[idx];
+    const uint32_t pos = atomicAdd(&colLength[post], 1u);
+    if(remap) {
+        if(pos < colStride) { remap[(size_t)post * colStride + pos] = (uint32_t)idx; }
+        else { atomicMax(overflow, pos + 1); }
+    }
+}
+
+__global__ __launch_bounds__(BLOCK)
+void remapSortKernel(uint32_t colStride, const uint32_t *colLength, uint32_t *remap)
+{
+    extern __shared__ uint32_t shCol[];
+    const uint32_t col = blockIdx.x;
+    const uint32_t len = min(colLength[col], colStride);
+    if(len < 2) { return; }
+    uint32_t p2 = 1;
+    while(p2 < len) { p2 <<= 1; }
+    uint32_t *column = remap + (size_t)col * colStride;
+    for(uint32_t k = threadIdx.x; k < p2; k += BLOCK) { shCol[k] = (k < len) ? column[k] : 0xFFFFFFFFu; }
+    __syncthreads();
+    for(uint32_t size = 2; size <= p2; size <<= 1) {
+        for(uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+            for(uint32_t k = threadIdx.x; k < p2; k += BLOCK) {
+                const uint32_t partner = k ^ stride;
+                if(partner > k) {
+                    const bool up = ((k & size) == 0);
+                    const uint32_t a = shCol[k], b = shCol[partner];
+                    if((a > b) == up) { shCol[k] = b; shCol[partner] = a; }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    for(uint32_t k = threadIdx.x; k < len; k += BLOCK) { column[k] = shCol[k]; }
+}
+
+uint32_t pow2Floor(uint32_t v) { uint32_t p = 1; while(p * 2 <= v) { p *= 2; } return p; }
+uint32_t pow2Ceil(uint32_t v) { uint32_t p = 1; while(p < v) { p *= 2; } return p; }
+}   // namespace
+
+#endif
