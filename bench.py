@@ -40,6 +40,8 @@ def build_net(name, steps):
     from genn_amd import configs
     if name == "potjans":
         return configs.potjans(steps=steps), "C2 potjans_microcircuit 77169 neurons 298.6M synapses dt=0.1ms"
+    if name == "potjans_poisson":
+        return configs.potjans(steps=steps, poisson=True), "C2 potjans_microcircuit 77169 neurons 298.6M synapses dt=0.1ms, PoissonExp background (Philox)"
     if name == "potjans_small":
         return configs.potjans(neuron_scale=0.1, connectivity_scale=1.0, steps=steps), "potjans 10% neurons full in-degree"
     if name == "va":

@@ -14,7 +14,7 @@ MAX_PRE_OUTPUT = 2
 
 NEURON_LIF, NEURON_IZHIKEVICH, NEURON_SPIKE_SOURCE_ARRAY = 0, 1, 2
 PSM_EXPCURR, PSM_DELTACURR = 0, 1
-CS_DC, CS_ARRAY = 0, 1
+CS_DC, CS_ARRAY, CS_POISSON_EXP = 0, 1, 2
 WUM_STATIC_PULSE, WUM_STATIC_PULSE_DENDRITIC_DELAY, WUM_STDP_TRACE, WUM_STATIC_PULSE_CONSTANT_WEIGHT, WUM_STATIC_GRADED, WUM_STATIC_PULSE_REVERSE = 0, 1, 2, 3, 4, 5
 MATRIX_SPARSE, MATRIX_TOEPLITZ_CONV2D, MATRIX_DENSE, MATRIX_BITMASK, MATRIX_PROCEDURAL = 0, 1, 2, 3, 4
 CONNECT_SNIPPETS = {"FixedProbability": 0, "FixedProbabilityNoAutapse": 1, "FixedNumberPostWithReplacement": 2}
@@ -34,7 +34,9 @@ class Psm(C.Structure):
 
 
 class Cs(C.Structure):
-    _fields_ = [("array", p_f32), ("amp", C.c_float), ("kind", C.c_uint32), ("arraySteps", C.c_uint32), ("pad_", C.c_uint32)]
+    _fields_ = [("array", p_f32), ("amp", C.c_float), ("kind", C.c_uint32), ("arraySteps", C.c_uint32), ("stream", C.c_uint32),
+                ("current", p_f32), ("init", C.c_float), ("expDecay", C.c_float), ("expMinusLambda", C.c_float), ("pad_", C.c_uint32),
+                ("seed", C.c_uint64)]
 
 
 class SpikeEvent(C.Structure):

@@ -283,7 +283,7 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
         EnvironmentExternal funcEnv(libEnv);
         modelMerged.genMergedNeuronUpdateGroups(
             *this, memorySpaces,
-            [this, &funcEnv, &queue, batchSize, scalar](auto &n)
+            [this, &funcEnv, &queue, &model, batchSize, scalar](auto &n)
             {
                 const auto &arch = n.getArchetype();
                 const size_t numGroups = n.getGroups().size();
@@ -292,7 +292,12 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
                 if(arch.isDelayRequired() && (arch.isSpikeTimeRequired() || !n.getMergedOutSynWUMPreCodeGroups().empty() || !n.getMergedInSynWUMPostCodeGroups().empty())) {
                     unsupported("delay slots together with plasticity on population '" + arch.getName() + "'");
                 }
-                if(arch.isSimRNGRequired()) { unsupported("random numbers in the update of population '" + arch.getName() + "'"); }
+                // random numbers in the step: only the PoissonExp current source draws any (recognised below); the recognised
+                // neuron and postsynaptic models draw none
+                if(arch.isSimRNGRequired() && std::none_of(arch.getCurrentSources().cbegin(), arch.getCurrentSources().cend(),
+                                                           [](const CurrentSourceInternal *cs){ return Utils::isRNGRequired(cs->getInjectionCodeTokens()); })) {
+                    unsupported("random numbers in the update of population '" + arch.getName() + "'");
+                }
                 if(arch.isPrevSpikeTimeRequired()) { unsupported("previous spike times of population '" + arch.getName() + "'"); }
                 if(n.getMergedSpikeEventGroups().size() > GENNMI_MAX_SPK_EVENT) { unsupported("more than 2 spike-like event conditions on population '" + arch.getName() + "'"); }
                 if(!n.getMergedSpikeEventGroups().empty() && (arch.isDelayRequired() || arch.isSpikeEventTimeRequired() || arch.isPrevSpikeEventTimeRequired())) {
@@ -414,6 +419,24 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
                                       [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, "noise"); },
                                       "", GroupMergedFieldType::DYNAMIC);
                         cout << dst << ".kind = " << GENNMI_CS_ARRAY << "u; " << dst << ".arraySteps = 1u; " << dst << ".array = gennmiDev(" << cenv["_mi_noise"] << ");" << std::endl;
+                    }
+                    // PoissonExp: the uniforms of (neuron, step) are counter-based generator calls under the model's seed; one
+                    // stream per source, numbered by its place in the model's (name-ordered) list of current sources
+                    else if(same(cs.getModel()->getInjectionCode(), CurrentSourceModels::PoissonExp::getInstance()->getInjectionCode())) {
+                        cenv.addField(scalar.createPointer(), "_mi_current", "currentCS" + std::to_string(child.getIndex()),
+                                      [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, "current"); });
+                        cout << dst << ".kind = " << GENNMI_CS_POISSON_EXP << "u; " << dst << ".current = gennmiDev(" << cenv["_mi_current"] << "); "
+                             << dst << ".seed = " << model.getSeed() << "ull;" << std::endl;
+                        for(const auto &[field, param] : {std::pair<const char*, const char*>{"init", "Init"}, {"expDecay", "ExpDecay"}, {"expMinusLambda", "ExpMinusLambda"}}) {
+                            std::vector<Type::NumericValue> values;
+                            for(const auto &g : child.getGroups()) { values.push_back(g.get().getDerivedParams().at(param)); }
+                            cout << "{ static const float v[] = " << table(values, scalar) << "; " << dst << "." << field << " = v[g]; }" << std::endl;
+                        }
+                        std::vector<uint64_t> streams;
+                        for(const auto &g : child.getGroups()) {
+                            streams.push_back(1000 + (uint64_t)std::distance(model.getLocalCurrentSources().cbegin(), model.getLocalCurrentSources().find(g.get().getName())));
+                        }
+                        cout << "{ static const uint32_t v[] = " << tableU32(streams) << "; " << dst << ".stream = v[g]; }" << std::endl;
                     }
                     else {
                         unsupported("current source model of '" + cs.getName() + "'");

@@ -80,11 +80,13 @@ def pd_mean_weight(src, trg):
     return PD_G * PD_MEAN_W
 
 
-def potjans(neuron_scale=1.0, connectivity_scale=1.0, steps=10000, seed=4321, dt=0.1, pad=4):
+def potjans(neuron_scale=1.0, connectivity_scale=1.0, steps=10000, seed=4321, dt=0.1, pad=4, poisson=False):
     """Scaling rules are those of the reference script (userproject/potjans_microcircuit.py:105-147,
     193-200).  The Poisson background (PoissonExp, currentSourceModels.h:107-129) is replaced by a
-    DC source with the same stationary mean, w * tauSyn * rate[1/ms].  Rows are padded to
-    ``pad`` entries so that row starts are 16-byte aligned."""
+    DC source with the same stationary mean, w * tauSyn * rate[1/ms], unless ``poisson`` asks for the
+    script's own sources (weight, tauSyn 0.5 ms, rate as in potjans_microcircuit.py:193-200), which draw
+    from this build's counter-based generator.  Rows are padded to ``pad`` entries so that row starts
+    are 16-byte aligned."""
     pops = [l + p for l in PD_LAYERS for p in ("E", "I")]
     max_delay = {k: PD_MEAN_DELAY[k] + PD_DELAY_SD[k] * PD_NORM_Q9999 for k in ("E", "I")}
     slots = int(round(max(max_delay.values()) / dt))
@@ -102,7 +104,10 @@ def potjans(neuron_scale=1.0, connectivity_scale=1.0, steps=10000, seed=4321, dt
                             {"V": v0, "RefracTime": np.zeros(n, np.float32)}))
         ext_rate = PD_EXT[name] * connectivity_scale * PD_BG_RATE
         ext_w = PD_MEAN_W / math.sqrt(connectivity_scale)
-        net.css.append(CurrentSource(name + "_dc", "dc", name, amp=ext_w * 0.5 * ext_rate / 1000.0))
+        if poisson:
+            net.css.append(CurrentSource(name + "_poisson", "poisson_exp", name, params=dict(weight=ext_w, tauSyn=0.5, rate=ext_rate)))
+        else:
+            net.css.append(CurrentSource(name + "_dc", "dc", name, amp=ext_w * 0.5 * ext_rate / 1000.0))
     stream = 100
     fmax = float(np.finfo(np.float32).max)
     for trg in pops:

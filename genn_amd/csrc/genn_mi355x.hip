@@ -312,7 +312,8 @@ int gennmi_push_neuron_update_group(gennmi_runner *r, const gennmi_neuron_update
     }
     for(uint32_t c = 0; c < g->numCS; c++) {
         if(g->cs[c].kind == GENNMI_CS_ARRAY && (!g->cs[c].array || g->cs[c].arraySteps == 0)) { return fail(GENNMI_EINVAL, "push_neuron_update_group: current-source array missing"); }
-        if(g->cs[c].kind > GENNMI_CS_ARRAY) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: unknown current source"); }
+        if(g->cs[c].kind == GENNMI_CS_POISSON_EXP && !g->cs[c].current) { return fail(GENNMI_EINVAL, "push_neuron_update_group: PoissonExp state missing"); }
+        if(g->cs[c].kind > GENNMI_CS_POISSON_EXP) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: unknown current source"); }
     }
     if(g->numExtraSpk > GENNMI_MAX_EXTRA_SPK) { return fail(GENNMI_EUNSUPPORTED, "push_neuron_update_group: too many spike arrays"); }
     for(uint32_t q = 0; q < g->numExtraSpk; q++) {
@@ -454,7 +455,7 @@ int gennmi_push_postsynaptic_update_group(gennmi_runner *r, const gennmi_postsyn
 }
 
 // Resident plan (residentKernel): chosen when the whole network fits the chip — batch 1, static SPARSE projections
-// (with or without dendritic delay) with ascending rows between LIF / Izhikevich populations driven by DC sources, every
+// (with or without dendritic delay) with ascending rows between LIF / Izhikevich populations driven by DC or PoissonExp sources, every
 // tile of 256 neurons with its ring slices in LDS and all tiles resident at once.  GENNMI_RESIDENT=0 disables it.
 static int setupResident(gennmi_runner *r, uint32_t numCU)
 {
@@ -464,7 +465,7 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
     for(const auto &n : r->neuron) {
         const auto &g = n.g;
         if((g.model != GENNMI_NEURON_LIF && g.model != GENNMI_NEURON_IZHIKEVICH) || g.preTrace || g.postTrace || g.sT || g.numDelaySlots > 1 || g.numSpkEvent || g.numPreOutput) { return GENNMI_OK; }
-        for(uint32_t c = 0; c < g.numCS; c++) { if(g.cs[c].kind != GENNMI_CS_DC) { return GENNMI_OK; } }
+        for(uint32_t c = 0; c < g.numCS; c++) { if(g.cs[c].kind == GENNMI_CS_ARRAY) { return GENNMI_OK; } }
     }
     // tiles and their LDS layout
     std::vector<ResTile> tiles;
@@ -646,6 +647,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
         for(const auto &n : r->neuron) {
             const auto &g = n.g;
             lanes += (unsigned long long)g.numNeurons * r->batch;
+            for(uint32_t c = 0; c < g.numCS; c++) { plain = plain && g.cs[c].kind != GENNMI_CS_POISSON_EXP; }
             plain = plain && g.numPSM <= BULK_MAX_PSM && g.numCS <= BULK_MAX_CS && !g.preTrace && !g.postTrace && !g.sT && g.numExtraSpk == 0
                     && g.numDelaySlots <= 1 && g.numSpkEvent == 0 && g.numPreOutput == 0;
         }

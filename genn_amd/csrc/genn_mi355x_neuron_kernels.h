@@ -4,6 +4,44 @@
 
 namespace
 {
+// PoissonExp current source (currentSourceModels.h:100-129): the snippet's loop draws uniforms until their product falls to
+// ExpMinusLambda; here the draws of (neuron, step) are the words of counter-based generator calls, so the result does not
+// depend on the launch geometry or on which plan steps the network.
+__device__ __forceinline__ uint32_t poissonExpCount(const gennmi_cs_t &cs, size_t bi, unsigned long long epoch)
+{
+    const gennmi_rows::Stream s{(uint32_t)cs.seed, (uint32_t)(cs.seed >> 32), cs.stream};
+    float p = 1.0f;
+    uint32_t numSpikes = 0;
+    for(uint32_t call = 0; ; call++) {
+        const gennmi_rows::Words r = gennmi_rows::philox4x32((uint32_t)bi, (uint32_t)epoch, call, s.stream, s.k0, s.k1);
+        bool done = false;
+        #pragma unroll
+        for(int w = 0; w < 4 && !done; w++) {
+            numSpikes++;
+            p *= gennmi_rows::uniformHalfOpen(r.w[w]);
+            done = !(p > cs.expMinusLambda);
+        }
+        if(done) { break; }
+    }
+    return numSpikes - 1;
+}
+
+// one step of the source whose state the caller holds: returns the injected value, leaves the decayed one in `current`
+__device__ __forceinline__ float poissonExpStep(const gennmi_cs_t &cs, float &current, size_t bi, unsigned long long epoch)
+{
+    const float value = current + cs.init * (float)poissonExpCount(cs, bi, epoch);
+    current = value * cs.expDecay;
+    return value;
+}
+
+__device__ __forceinline__ float poissonExpInject(const gennmi_cs_t &cs, GLOBAL_AS float *current, size_t bi, unsigned long long epoch)
+{
+    float state = current[bi];
+    const float value = poissonExpStep(cs, state, bi, epoch);
+    current[bi] = state;
+    return value;
+}
+
 // ------------------------------------------------------------------------------------------------
 // Offset of a block's entries in its population's queue: the block publishes its count, then (wave 0) sums the counts of
 // the earlier blocks of its group of 64 and the published totals of the earlier groups.  Every thread of the block calls
@@ -153,7 +191,8 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
                 inj[c] = 0.0f;
                 if(c < numCS) {
                     inj[c] = (g.cs[c].kind == GENNMI_CS_DC) ? g.cs[c].amp
-                                                            : asGlobal(g.cs[c].array)[(size_t)modStep(st.epoch, g.cs[c].arraySteps) * n + i];
+                           : (g.cs[c].kind == GENNMI_CS_ARRAY) ? asGlobal(g.cs[c].array)[(size_t)modStep(st.epoch, g.cs[c].arraySteps) * n + i]
+                                                               : poissonExpInject(g.cs[c], asGlobal(g.cs[c].current), bi, st.epoch);
                 }
             }
             float Isyn = 0;

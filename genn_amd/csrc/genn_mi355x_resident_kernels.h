@@ -169,6 +169,12 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     // ---- state: neuron variables in registers, inSyn and ring slices in LDS
     float l0 = 0, l1 = 0;
     if(mine) { l0 = asGlobal(g.var0)[i]; l1 = asGlobal(g.var1)[i]; }
+    // state of the PoissonExp sources, in registers like the neuron's own
+    float csState[GENNMI_MAX_CS];
+    #pragma unroll
+    for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) {
+        csState[c] = (mine && c < numCS && g.cs[c].kind == GENNMI_CS_POISSON_EXP) ? asGlobal(g.cs[c].current)[i] : 0.0f;
+    }
     for(uint32_t m = 0; m < numPSM; m++) {
         lds[T.ldsIn[m] + tid] = mine ? asGlobal(g.psm[m].outPost)[i] : 0.0f;
         const uint32_t D = g.psm[m].maxDenDelay;
@@ -460,7 +466,9 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
                 }
             }
             #pragma unroll
-            for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) { if(c < numCS) { Isyn += g.cs[c].amp; } }
+            for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) {
+                if(c < numCS) { Isyn += (g.cs[c].kind == GENNMI_CS_DC) ? g.cs[c].amp : poissonExpStep(g.cs[c], csState[c], i, epoch); }
+            }
             if(g.model == GENNMI_NEURON_LIF) {
                 if(l1 <= 0.0f) {
                     const float alpha = ((Isyn + g.params[0]) * g.params[1]) + g.params[2];
@@ -517,7 +525,13 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     if(zeroDelaySplit) { deliverDue(numSteps + 1, PASS_DUE); }
     __syncthreads();
 
-    if(mine) { asGlobal(g.var0)[i] = l0; asGlobal(g.var1)[i] = l1; }
+    if(mine) {
+        asGlobal(g.var0)[i] = l0; asGlobal(g.var1)[i] = l1;
+        #pragma unroll
+        for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) {
+            if(c < numCS && g.cs[c].kind == GENNMI_CS_POISSON_EXP) { asGlobal(g.cs[c].current)[i] = csState[c]; }
+        }
+    }
     for(uint32_t m = 0; m < numPSM; m++) {
         if(mine) { asGlobal(g.psm[m].outPost)[i] = lds[T.ldsIn[m] + tid]; }
         const uint32_t D = g.psm[m].maxDenDelay;

@@ -256,6 +256,7 @@ class CurrentSource:
         self.params = dict(params)
         self.extra_global_params = {}
         self.vars = {}
+        self.stream = None          # PoissonExp: generator stream (the next free one of the model unless set)
 
     def set_extra_global_param(self, name, value):
         self.extra_global_params[name] = np.ascontiguousarray(value, dtype=np.float32)
@@ -391,7 +392,7 @@ class GeNNModel:
         return g
 
     def add_current_source(self, cs_name, current_source_model, pop, params=None, vars=None):
-        if current_source_model not in ("DC", "ArrayNoise"):
+        if current_source_model not in ("DC", "ArrayNoise", "PoissonExp"):
             raise NotImplementedError(f"current source {current_source_model}")
         cs = CurrentSource(cs_name, current_source_model, pop, params or {})
         pop.current_sources.append(cs)
@@ -559,6 +560,11 @@ class GeNNModel:
             if n.post_trace_owner is not None:
                 n.post_trace_owner.vars["postTrace"] = self._alloc(B * N, np.float32, fill=n.post_trace_owner.wu.post_vars.get("postTrace", 0.0))
             for cs in n.current_sources:
+                if cs.kind == "PoissonExp":
+                    cs.vars["current"] = self._alloc(B * N, np.float32)
+                    if cs.stream is None:
+                        # by place in the name-ordered list of the model's current sources, as the backend adapter numbers them
+                        cs.stream = 1000 + sorted(self.current_sources).index(cs.name)
                 if cs.kind == "ArrayNoise":
                     noise = np.ascontiguousarray(cs.extra_global_params["noise"], dtype=np.float32)
                     if noise.size % N:
@@ -768,8 +774,18 @@ class GeNNModel:
                 srcs = [n.current_sources[c] for n in members]
                 if srcs[0].kind == "DC":
                     amps = _merge_round([cs.params["amp"] for cs in srcs])
+                if srcs[0].kind == "PoissonExp":
+                    # the snippet's derived parameters (currentSourceModels.h:123-128)
+                    dt = self.dt
+                    decay = _merge_round([math.exp(-dt / cs.params["tauSyn"]) for cs in srcs])
+                    init = _merge_round([cs.params["weight"] * (1.0 - math.exp(-dt / cs.params["tauSyn"])) * (cs.params["tauSyn"] / dt) for cs in srcs])
+                    lam = _merge_round([math.exp(-(cs.params["rate"] / 1000.0) * dt) for cs in srcs])
                 for k, (d, cs, n) in enumerate(zip(descs, srcs, members)):
-                    if cs.kind == "DC":
+                    if cs.kind == "PoissonExp":
+                        d.cs[c].kind, d.cs[c].current = _abi.CS_POISSON_EXP, cs.vars["current"].ptr
+                        d.cs[c].init, d.cs[c].expDecay, d.cs[c].expMinusLambda = init[k], decay[k], lam[k]
+                        d.cs[c].seed, d.cs[c].stream = self.seed, cs.stream
+                    elif cs.kind == "DC":
                         d.cs[c].kind, d.cs[c].amp = _abi.CS_DC, amps[k]
                     else:
                         d.cs[c].kind, d.cs[c].array = _abi.CS_ARRAY, cs.vars["noise"].ptr
@@ -979,7 +995,9 @@ def model_from_net(net, batch_size=1, record=True, span=None, device=0):
         g.spike_recording_enabled = record
         pops[p.name] = g
     for c in net.css:
-        if c.model == "dc":
+        if c.model == "poisson_exp":
+            m.add_current_source(c.name, "PoissonExp", pops[c.pop], c.params)
+        elif c.model == "dc":
             m.add_current_source(c.name, "DC", pops[c.pop], {"amp": c.amp})
         else:
             cs = m.add_current_source(c.name, "ArrayNoise", pops[c.pop])

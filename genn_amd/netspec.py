@@ -34,9 +34,10 @@ class Pop:
 @dataclass
 class CurrentSource:
     name: str
-    model: str                      # "dc" | "noise"
+    model: str                      # "dc" | "noise" | "poisson_exp" (params weight [nA], tauSyn [ms], rate [Hz])
     pop: str
     amp: float = 0.0
+    params: Dict[str, float] = field(default_factory=dict)
     noise: Optional[np.ndarray] = None   # fp32 [steps, n] for "noise"
 
 
@@ -139,8 +140,8 @@ def write_netspec(net: Net, path: str):
     lines.append(f"snap {snap}")
     if getattr(net, "batch_size", 1) != 1:
         lines.append(f"batch {int(net.batch_size)}")
-    if any(s.matrix == "procedural" for s in net.syns):
-        lines.append(f"seed {int(net.seed)}")        # procedural matrices are regenerated from the model's seed
+    if any(s.matrix == "procedural" for s in net.syns) or any(c.model == "poisson_exp" for c in net.css):
+        lines.append(f"seed {int(net.seed)}")        # procedural matrices and Poisson sources draw from the model's seed
     for p in net.pops:
         if p.model == "lif":
             ps = " ".join(repr(float(p.params[k])) for k in LIF_PARAMS)
@@ -155,7 +156,9 @@ def write_netspec(net: Net, path: str):
         if p.spike_times is not None:
             np.ascontiguousarray(p.spike_times, dtype=np.float32).tofile(os.path.join(path, f"{p.name}.spikeTimes.f32"))
     for c in net.css:
-        if c.model == "dc":
+        if c.model == "poisson_exp":
+            lines.append(f"cs {c.name} poisson_exp {c.pop} {float(c.params['weight'])!r} {float(c.params['tauSyn'])!r} {float(c.params['rate'])!r}")
+        elif c.model == "dc":
             lines.append(f"cs {c.name} dc {c.pop} {float(c.amp)!r}")
         else:
             lines.append(f"cs {c.name} noise {c.pop}")

@@ -42,7 +42,7 @@ enum { GENNMI_NEURON_LIF = 0, GENNMI_NEURON_IZHIKEVICH = 1, GENNMI_NEURON_SPIKE_
 /* postsynaptic models: include/genn/genn/postsynapticModels.h:91-106 (ExpCurr), DeltaCurr */
 enum { GENNMI_PSM_EXPCURR = 0, GENNMI_PSM_DELTACURR = 1 };
 /* current sources: include/genn/genn/currentSourceModels.h:70-77 (DC); ARRAY injects noise[step*numNeurons+id] */
-enum { GENNMI_CS_DC = 0, GENNMI_CS_ARRAY = 1 };
+enum { GENNMI_CS_DC = 0, GENNMI_CS_ARRAY = 1, GENNMI_CS_POISSON_EXP = 2 };
 /* weight update models: include/genn/genn/weightUpdateModels.h:236-244, :279-287; trace STDP pygenn/genn_model.py:1448-1476 */
 enum { GENNMI_WUM_STATIC_PULSE = 0, GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY = 1, GENNMI_WUM_STDP_TRACE = 2,
        GENNMI_WUM_STATIC_PULSE_CONSTANT_WEIGHT = 3, /* weightUpdateModels.h:202-213: one weight for the whole projection */
@@ -121,7 +121,14 @@ typedef struct gennmi_cs_t {              /* one current source child (neuronUpd
     float amp;                            /* GENNMI_CS_DC */
     uint32_t kind;
     uint32_t arraySteps;
+    /* GENNMI_CS_POISSON_EXP (currentSourceModels.h:100-129): numSpikes ~ Poisson(rate*dt) by the snippet's product-of-uniforms
+     * loop, current += Init*numSpikes, injected, then current *= ExpDecay.  The uniforms of neuron i (batch-major index) in
+     * step k are the words of Philox4x32-10(counter = (i, k, call, stream), key = seed), call = 0, 1, ... as the loop needs them. */
+    uint32_t stream;
+    float *current;                       /* state variable [batch*numNeurons] */
+    float init, expDecay, expMinusLambda; /* the snippet's derived parameters, rounded to fp32 */
     uint32_t pad_;
+    uint64_t seed;
 } gennmi_cs_t;
 
 /* Spike-like events ("SynSpikeEvent" children, neuronUpdateGroupMerged.cc:189-330): after the neuron's sim code and

@@ -22,6 +22,8 @@
  *                        neuron loop + op order      backend.cc:187-398, neuronUpdateGroupMerged.cc:552-773 (PSM :66-137, CS :20-55,
  *                                                    WU pre/post :333-459), spike emission backend.cc:2119-2133
  *                        event conditions            neuronUpdateGroupMerged.cc:215-330, 677-683; emission backend.cc genEmitEvent
+ *                        PoissonExp source           include/genn/genn/currentSourceModels.h:100-129 (the generator behind gennrand_uniform is this
+ *                                                    build's own counter-based one: parity with the reference is statistical)
  *                        model arithmetic            include/genn/genn/neuronModels.h:163-186 (Izhikevich), :220-257 (LIF), :274-286
  *                                                    (SpikeSourceArray); postsynapticModels.h:91-106 (ExpCurr), DeltaCurr;
  *                                                    currentSourceModels.h:70-77 (DC); weightUpdateModels.h:236-287;
@@ -44,7 +46,7 @@ enum { GC_LIF = 0, GC_IZH = 1, GC_SSA = 2 };
 enum { GC_EXPCURR = 0, GC_DELTACURR = 1 };
 enum { GC_STATIC = 0, GC_STATIC_DELAY = 1, GC_STDP_TRACE = 2, GC_STATIC_GRADED = 3, GC_STATIC_REVERSE = 4 };
 enum { GC_SPARSE = 0, GC_CONV2D = 1, GC_DENSE = 2, GC_BITMASK = 3 };
-enum { GC_CS_DC = 0, GC_CS_NOISE = 1 };
+enum { GC_CS_DC = 0, GC_CS_NOISE = 1, GC_CS_POISSON_EXP = 2 };
 
 #define GC_MAX_CHILD 16
 #define GC_MAX_EVENT 4
@@ -70,6 +72,10 @@ typedef struct {
     float amp;
     const float *noise;     /* [noiseSteps * n]: row s % noiseSteps is what the host pushes before step s */
     uint64_t noiseSteps;
+    /* PoissonExp (currentSourceModels.h:100-129): state variable and derived parameters; the uniforms of neuron i in step k
+     * are the words of Philox4x32-10(counter = (indexOffset + i, k, call, stream), key = seed), call = 0, 1, ... */
+    float *current; float init, expDecay, expMinusLambda;
+    uint64_t seed; uint32_t stream, indexOffset;
 } gc_cs;
 
 typedef struct {
@@ -194,6 +200,33 @@ int gc_add_cs(gc_net *net, int pop, int kind, float amp, const float *noise, uin
     p->cs[p->numCS].noiseSteps = noiseSteps ? noiseSteps : 1;
     return p->numCS++;
 }
+
+/* Philox4x32-10 (Salmon et al., SC'11): the published round function and key schedule */
+void gc_philox4x32(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1, uint32_t out[4])
+{
+    for(int round = 0; round < 10; round++) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t hi0 = (uint32_t)(p0 >> 32), lo0 = (uint32_t)p0, hi1 = (uint32_t)(p1 >> 32), lo1 = (uint32_t)p1;
+        c0 = hi1 ^ c1 ^ k0; c1 = lo1; c2 = hi0 ^ c3 ^ k1; c3 = lo0;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+int gc_add_cs_poisson_exp(gc_net *net, int pop, float init, float expDecay, float expMinusLambda, uint64_t seed, uint32_t stream,
+                          uint32_t indexOffset, const float *current0)
+{
+    gc_pop *p = &net->pops[pop];
+    if(p->numCS == GC_MAX_CHILD) { return -1; }
+    gc_cs *c = &p->cs[p->numCS];
+    memset(c, 0, sizeof(*c));
+    c->kind = GC_CS_POISSON_EXP; c->init = init; c->expDecay = expDecay; c->expMinusLambda = expMinusLambda;
+    c->seed = seed; c->stream = stream; c->indexOffset = indexOffset; c->noiseSteps = 1;
+    c->current = (float*)gc_dup(current0, (size_t)p->n * sizeof(float));
+    return p->numCS++;
+}
+
+float *gc_cs_current(gc_net *net, int pop, int cs) { return net->pops[pop].cs[cs].current; }
 
 static gc_syn *gc_new_syn(gc_net *net)
 {
@@ -526,7 +559,28 @@ void gc_update_neurons(gc_net *net, float t, uint32_t recordingTimestep)
                 p->outPre[q][i] = 0.0f;
             }
             for(int c = 0; c < p->numCS; c++) {
-                Isyn += (p->cs[c].kind == GC_CS_DC) ? p->cs[c].amp : p->cs[c].noise[(size_t)(step % p->cs[c].noiseSteps) * p->n + i];
+                gc_cs *cs = &p->cs[c];
+                if(cs->kind == GC_CS_POISSON_EXP) {
+                    /* the snippet's loop (uniforms in [0, 1) with 24 significant bits, four per generator call) */
+                    float prod = 1.0f;
+                    uint32_t numSpikes = 0;
+                    int done = 0;
+                    for(uint32_t call = 0; !done; call++) {
+                        uint32_t r[4];
+                        gc_philox4x32(cs->indexOffset + i, (uint32_t)step, call, cs->stream, (uint32_t)cs->seed, (uint32_t)(cs->seed >> 32), r);
+                        for(int w = 0; w < 4 && !done; w++) {
+                            numSpikes++;
+                            prod *= (float)(r[w] >> 8) * (1.0f / 16777216.0f);
+                            done = !(prod > cs->expMinusLambda);
+                        }
+                    }
+                    cs->current[i] += cs->init * (float)(numSpikes - 1);
+                    Isyn += cs->current[i];
+                    cs->current[i] *= cs->expDecay;
+                }
+                else {
+                    Isyn += (cs->kind == GC_CS_DC) ? cs->amp : cs->noise[(size_t)(step % cs->noiseSteps) * p->n + i];
+                }
             }
             if(p->model == GC_LIF) {
                 /* p = {Ioffset, Rmembrane, Vrest, ExpTC, Vthresh, Vreset, TauRefrac} ; l0 = V, l1 = RefracTime */
@@ -621,6 +675,7 @@ void gc_destroy(gc_net *net)
         free(p->v0); free(p->v1); free(p->startSpike); free((void*)p->endSpike);
         for(int m = 0; m < p->numPSM; m++) { free(p->psm[m].outPost); free(p->psm[m].denDelay); }
         free(p->preTrace); free(p->postTrace); free(p->sT); free(p->recordSpk);
+        for(int c = 0; c < p->numCS; c++) { free(p->cs[c].current); }
         if(p->spkRing) { free(p->spkRing); free(p->spkCntRing); } else { free(p->spk); }
         for(int e = 0; e < p->numEvents; e++) { free(p->events[e].spkEvent); free(p->events[e].recordSpkEvent); }
         for(int q = 0; q < p->numPreOutput; q++) { free(p->outPre[q]); }

@@ -23,7 +23,7 @@ SRC = os.path.join(HERE, "genn_cpu.c")
 GC_LIF, GC_IZH, GC_SSA = 0, 1, 2
 GC_EXPCURR, GC_DELTACURR = 0, 1
 GC_STATIC, GC_STATIC_DELAY, GC_STDP_TRACE, GC_STATIC_GRADED, GC_STATIC_REVERSE = 0, 1, 2, 3, 4
-GC_CS_DC, GC_CS_NOISE = 0, 1
+GC_CS_DC, GC_CS_NOISE, GC_CS_POISSON_EXP = 0, 1, 2
 
 
 def build(force=False):
@@ -44,6 +44,9 @@ def lib():
         l.gc_add_pop.restype = i32; l.gc_add_pop.argtypes = [vp, i32, u32, vp, i32, vp, vp, vp]
         l.gc_add_psm.restype = i32; l.gc_add_psm.argtypes = [vp, i32, i32, f32, f32, u32]
         l.gc_add_cs.restype = i32; l.gc_add_cs.argtypes = [vp, i32, i32, f32, vp, u64]
+        l.gc_add_cs_poisson_exp.restype = i32; l.gc_add_cs_poisson_exp.argtypes = [vp, i32, f32, f32, f32, u64, u32, u32, vp]
+        l.gc_philox4x32.restype = None; l.gc_philox4x32.argtypes = [u32] * 6 + [vp]
+        l.gc_cs_current.restype = vp; l.gc_cs_current.argtypes = [vp, i32, i32]
         l.gc_add_syn_sparse.restype = i32; l.gc_add_syn_sparse.argtypes = [vp, i32, i32, i32, i32, u32, vp, vp, vp, vp, i32]
         l.gc_set_stdp_trace.restype = None; l.gc_set_stdp_trace.argtypes = [vp, i32, f32, f32, f32, f32, f32, f32, u32]
         l.gc_add_syn_conv2d.restype = i32; l.gc_add_syn_conv2d.argtypes = [vp, i32, i32, i32, vp, vp]
@@ -105,7 +108,7 @@ def _as(a, dtype):
 class OracleNet:
     """The oracle's view of a Net.  ``max_col`` maps projection name -> column stride."""
 
-    def __init__(self, net, num_recording_timesteps=0, col_stride=None):
+    def __init__(self, net, num_recording_timesteps=0, col_stride=None, batch_index=0):
         self.l = lib()
         self.net = net
         self.keep = []               # arrays the C side borrows
@@ -198,8 +201,22 @@ class OracleNet:
             for ci in range(len(css[0])):
                 if css[0][ci].model == "dc":
                     amps = _round_group([c[ci].amp for c in css])
+                if css[0][ci].model == "poisson_exp":
+                    # derived parameters of the snippet (currentSourceModels.h:123-128), rounded like any merged-group constant
+                    q = [c[ci].params for c in css]
+                    decay = _round_group([math.exp(-dt / x["tauSyn"]) for x in q])
+                    init = _round_group([x["weight"] * (1.0 - math.exp(-dt / x["tauSyn"])) * (x["tauSyn"] / dt) for x in q])
+                    lam = _round_group([math.exp(-(x["rate"] / 1000.0) * dt) for x in q])
                 for j, p in enumerate(members):
                     c = css[j][ci]
+                    if c.model == "poisson_exp":
+                        stream = 1000 + sorted(x.name for x in net.css).index(c.name)      # by place in the name-ordered list of the model's sources
+                        zero = np.zeros(p.n, np.float32)
+                        self.l.gc_add_cs_poisson_exp(self.h, self.pop_id[p.name], C.c_float(init[j]), C.c_float(decay[j]), C.c_float(lam[j]),
+                                                     net.seed, stream, batch_index * p.n, zero.ctypes.data)
+                        self.cs_id = getattr(self, "cs_id", {})
+                        self.cs_id[c.name] = (p.name, ci)
+                        continue
                     if c.model == "dc":
                         self.l.gc_add_cs(self.h, self.pop_id[p.name], GC_CS_DC, C.c_float(amps[j]), None, 0)
                     else:
@@ -330,6 +347,10 @@ class OracleNet:
     def out_pre(self, syn):
         s = self.net.syn(syn)
         return self._arr(self.l.gc_out_pre(self.h, self.syn_id[syn]), self.net.pop(s.src).n, np.float32)
+
+    def cs_current(self, name):
+        pop, ci = self.cs_id[name]
+        return self._arr(self.l.gc_cs_current(self.h, self.pop_id[pop], ci), self.net.pop(pop).n, np.float32)
 
     def spike_events(self, syn):
         """The spike-like event queue a graded projection read last / will read next (ids in ascending order)."""

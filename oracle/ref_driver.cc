@@ -252,6 +252,9 @@ int main(int argc, char *argv[])
             NeuronGroup *ng = popByName.at(c.pop)->ng;
             if(c.model == "dc") c.cs = model.addCurrentSource<CurrentSourceModels::DC>(c.name, ng, {{"amp", c.p.at(0)}}, {});
             else if(c.model == "noise") c.cs = model.addCurrentSource<ArrayNoise>(c.name, ng, {}, {});
+            else if(c.model == "poisson_exp") {
+                c.cs = model.addCurrentSource<CurrentSourceModels::PoissonExp>(c.name, ng, {{"weight", c.p.at(0)}, {"tauSyn", c.p.at(1)}, {"rate", c.p.at(2)}}, {{"current", 0.0}});
+            }
             else throw std::runtime_error("cs model " + c.model);
         }
         for(auto &s : syns) {

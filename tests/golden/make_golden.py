@@ -66,8 +66,37 @@ def make(name):
         shutil.rmtree(tmp, ignore_errors=True)
 
 
+def make_poisson_rates():
+    """potjans_poisson_rates.npz: spike counts per population of the scaled cortical microcircuit under its PoissonExp
+    background, run by the reference's CPU backend for 5 s of model time under two seeds.  The reference draws the
+    background from its host generator, which no other backend reproduces, so what these runs fix is the statistics:
+    the mean rates, and (from the two seeds) how far two correct runs differ."""
+    from cases import potjans_poisson_net
+    data = {}
+    for seed in (1234, 98765):
+        net = potjans_poisson_net()
+        net.seed = seed
+        net.snap = net.steps
+        tmp = tempfile.mkdtemp(prefix="golden_")
+        try:
+            spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+            for d in (work, out):
+                os.makedirs(d)
+            write_netspec(net, spec)
+            subprocess.check_call([DRIVER, spec, work, out], stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+            counts = [len(np.fromfile(os.path.join(out, f"{p.name}.spikes.u32"), np.uint32)) // 2 for p in net.pops]
+            data[f"counts.{seed}"] = np.array(counts, np.int64)
+            print(seed, {p.name: round(c / p.n / (net.steps * net.dt / 1000.0), 3) for p, c in zip(net.pops, counts)})
+        finally:
+            shutil.rmtree(tmp, ignore_errors=True)
+    data["input_digest"] = np.array(net.input_digest())
+    data["steps"] = np.array(net.steps)
+    data["sizes"] = np.array([p.n for p in net.pops], np.int64)
+    np.savez_compressed(os.path.join(HERE, "potjans_poisson_rates.npz"), **data)
+
+
 if __name__ == "__main__":
     if not os.path.exists(DRIVER):
         raise SystemExit("oracle/_ref/ref_driver is missing: run `make -f Makefile.ref` in oracle/ (needs /root/reference)")
-    for case in (sys.argv[1:] or list(CASES)):
-        make(case)
+    for case in (sys.argv[1:] or list(CASES) + ["potjans_poisson_rates"]):
+        make_poisson_rates() if case == "potjans_poisson_rates" else make(case)

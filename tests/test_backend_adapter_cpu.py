@@ -93,3 +93,28 @@ def test_procedural_projections_generate():
         assert "d.rowLength" not in code and "d.ind" not in code           # nothing stored, nothing bound
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_poisson_sources_generate():
+    """PoissonExp current sources through the adapter: recognised by their injection code (currentSourceModels.h:107-122), they
+    become descriptors with the model's seed, one generator stream per source (1000 + its place in the name-ordered list
+    of the model's current sources) and the snippet's derived parameters; the runner stays host code."""
+    from genn_amd import configs
+    net = configs.potjans(neuron_scale=0.02, connectivity_scale=0.2, steps=10, poisson=True)
+    net.snap = 10
+    tmp = tempfile.mkdtemp(prefix="adapter_poisson_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(net, spec)
+        res = subprocess.run([DRIVER, spec, work, out, "--generate-only"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        assert res.returncode == 0, res.stdout[-3000:]
+        code = open(os.path.join(work, net.name + "_CODE", "neuronUpdate.cc")).read()
+        assert f"d.cs[0].kind = 2u" in code and "d.cs[0].seed = 4321ull" in code
+        assert "{1000u, 1001u, 1002u, 1003u, 1004u, 1005u, 1006u, 1007u}; d.cs[0].stream = v[g]" in code
+        for field in ("init", "expDecay", "expMinusLambda", "current"):
+            assert f"d.cs[0].{field} = " in code
+        assert "gennrand" not in code and "__global__" not in code
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)

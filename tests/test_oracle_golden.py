@@ -325,3 +325,73 @@ def test_oracle_recording_bitfield():
     rec = o.record("S", 7).reshape(7, words)
     bits = np.unpackbits(rec.view(np.uint8), axis=1, bitorder="little")[:, :n]
     assert np.array_equal(bits, (fire_at[None, :] == np.arange(7)[:, None]).astype(np.uint8))
+
+
+# ---- PoissonExp current source ------------------------------------------------------------------------------------------
+def test_oracle_philox_known_answers():
+    """The generator under the oracle's PoissonExp source against the published Philox4x32-10 vectors."""
+    import ctypes as C
+    from oracle import genn_cpu
+    from philox_ref import KNOWN_ANSWERS
+    lib = genn_cpu.lib()
+    for counter, key, want in KNOWN_ANSWERS:
+        out = (C.c_uint32 * 4)()
+        lib.gc_philox4x32(*counter, *key, C.byref(out))
+        assert tuple(out) == want
+
+
+def _poisson_only(n, weight, tau, rate, dt=0.1, seed=77):
+    net = Net(name="poisson_only", dt=dt, steps=100, seed=seed)
+    net.pops.append(Pop("P", "lif", n, dict(C=0.25, TauM=10.0, Vrest=-65.0, Vreset=-65.0, Vthresh=1.0e6, Ioffset=0.0, TauRefrac=2.0),
+                        {"V": np.full(n, -65.0, np.float32), "RefracTime": np.zeros(n, np.float32)}))
+    net.css.append(CurrentSource("P_bg", "poisson_exp", "P", params=dict(weight=weight, tauSyn=tau, rate=rate)))
+    return net
+
+
+def test_oracle_poisson_exp_is_the_snippets_loop():
+    """The snippet (currentSourceModels.h:107-122) restated here in numpy from the same generator words: numSpikes is the
+    number of uniforms drawn until their running product is no longer above ExpMinusLambda; the state gains
+    Init * (numSpikes - 1), is injected, then decays.  One step from zero state leaves current = Init * k * ExpDecay, so
+    the counts can be read back from the oracle and compared draw for draw."""
+    from philox_ref import philox4x32
+    n, weight, tau, rate, dt, seed = 400, 0.0878, 0.5, 30000.0, 0.1, 77
+    net = _poisson_only(n, weight, tau, rate, dt, seed)
+    o = OracleNet(net)
+    o.step()
+    decay = np.float32(literal_f32(math.exp(-dt / tau)))
+    init = np.float32(literal_f32(weight * (1.0 - math.exp(-dt / tau)) * (tau / dt)))
+    lam = np.float32(literal_f32(math.exp(-(rate / 1000.0) * dt)))
+    counts = np.zeros(n, np.int64)
+    for i in range(n):
+        prod, k, call, done = np.float32(1.0), 0, 0, False
+        while not done:
+            words = philox4x32(i, 0, call, 1000, seed & 0xFFFFFFFF, seed >> 32)
+            for w in words:
+                k += 1
+                prod = np.float32(prod * (np.float32(int(w) >> 8) * np.float32(1.0 / 16777216.0)))
+                if not prod > lam:
+                    done = True
+                    break
+            call += 1
+        counts[i] = k - 1
+    want = (init * counts.astype(np.float32)) * decay
+    assert np.array_equal(o.cs_current("P_bg"), want)
+    assert counts.max() >= 8                     # some neurons needed a second generator call
+    # Poisson counts: mean and variance both lambda = 3
+    assert abs(counts.mean() - 3.0) < 5.0 * math.sqrt(3.0 / n) and abs(counts.var() - 3.0) < 1.0
+
+
+def test_oracle_poisson_exp_stationary_moments():
+    """Shot noise with kernel Init * a^k, a = exp(-dt / tau): the injected value has mean Init * lambda / (1 - a) (which is
+    weight * tau * rate, the mean the snippet's Init is chosen for) and variance Init^2 * lambda / (1 - a^2)."""
+    weight, tau, rate, dt, n = 0.0878, 0.5, 12800.0, 0.1, 40000
+    o = OracleNet(_poisson_only(n, weight, tau, rate, dt))
+    o.run(60)
+    a = math.exp(-dt / tau)
+    init = weight * (1.0 - a) * (tau / dt)
+    lam = rate / 1000.0 * dt
+    got = o.cs_current("P_bg").astype(np.float64) / a
+    mean, var = init * lam / (1.0 - a), init * init * lam / (1.0 - a * a)
+    assert abs(mean - weight * tau * rate / 1000.0) < 1e-12
+    assert abs(got.mean() - mean) < 5.0 * math.sqrt(var / n)
+    assert abs(got.var() - var) < 0.05 * var
