@@ -67,7 +67,7 @@ struct gennmi_runner
     bool resident = false;
     ResTile *dResTiles = nullptr; NeuronGroupDev *dResGroups = nullptr; uint8_t *dResTileGroup = nullptr;
     unsigned long long *dResTags = nullptr; uint32_t *dResSide = nullptr;
-    uint32_t resTiles = 0, resReplicaStride = 0; size_t resLdsBytes = 0;
+    uint32_t resTiles = 0, resReplicaStride = 0; size_t resLdsBytes = 0; bool resPoisson = false;
     std::vector<u32x4*> resSegs;        // segment table of each presynaptic group, in push order
     std::vector<uint32_t> resSegTiles;  // tiles of its target population
     uint32_t neuronsPerLane = 1;        // 2, 4 or 8: neuronBulkKernel instead of neuronUpdateKernel
@@ -495,11 +495,17 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
     if(tiles.empty() || tiles.size() > RES_MAX_TILES) { return GENNMI_OK; }
     const size_t ldsBytes = std::max<size_t>(ldsFloatsMax, 1) * sizeof(float);
     if(ldsBytes > 96 * 1024) { return GENNMI_OK; }
+    bool poisson = false;
+    for(const auto &n : r->neuron) {
+        for(uint32_t c = 0; c < n.g.numCS; c++) { poisson = poisson || n.g.cs[c].kind == GENNMI_CS_POISSON_EXP; }
+    }
+    const void *kernel = poisson ? reinterpret_cast<const void*>(residentKernel<true>) : reinterpret_cast<const void*>(residentKernel<false>);
     if(ldsBytes > 32 * 1024) {
-        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(residentKernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+        HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
     }
     int perCU = 0;
-    HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, residentKernel, BLOCK, ldsBytes));
+    if(poisson) { HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, residentKernel<true>, BLOCK, ldsBytes)); }
+    else { HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, residentKernel<false>, BLOCK, ldsBytes)); }
     if((size_t)perCU * numCU < tiles.size()) { return GENNMI_OK; }
 
     // projections: source group, target group and postsynaptic model, segment table
@@ -582,6 +588,7 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
     r->owned.push_back(r->dResSide);
     r->resTiles = (uint32_t)tiles.size();
     r->resLdsBytes = ldsBytes;
+    r->resPoisson = poisson;
     r->resident = true;
     return GENNMI_OK;
 }
@@ -610,7 +617,8 @@ static int launchResident(gennmi_runner *r, unsigned long long timestep, unsigne
     for(unsigned long long done = 0; done < numSteps; ) {
         const uint32_t chunk = (uint32_t)std::min(MAX_STEPS, numSteps - done);
         HIP_TRY(hipMemsetAsync(r->dResTags, 0, (size_t)RES_REPLICAS * r->resReplicaStride * sizeof(unsigned long long), r->stream));
-        residentKernel<<<dim3(r->resTiles), dim3(BLOCK), r->resLdsBytes, r->stream>>>(
+        auto launch = r->resPoisson ? residentKernel<true> : residentKernel<false>;
+        launch<<<dim3(r->resTiles), dim3(BLOCK), r->resLdsBytes, r->stream>>>(
             r->dResTiles, r->resTiles, r->dResGroups, r->dResTileGroup, r->dResTags, r->dResSide, timestep + done, r->epoch, numRecordingTimesteps,
             chunk, r->dt, r->fusedStep ? 1u : 0u, r->dError, r->dEvents, r->resReplicaStride);
         HIP_TRY(hipGetLastError());

@@ -112,6 +112,9 @@ __device__ __forceinline__ uint32_t waveInclusiveScanU32(uint32_t v, uint32_t la
     return v;
 }
 
+// POISSON: some population has a PoissonExp current source (its state then lives in a register per source and neuron);
+// the instantiation without it carries neither the registers nor the generator
+template<bool POISSON>
 __global__ __launch_bounds__(BLOCK)
 void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const NeuronGroupDev * __restrict__ groups,
                     const uint8_t * __restrict__ tileGroup, unsigned long long *tags, uint32_t *side,
@@ -173,7 +176,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     float csState[GENNMI_MAX_CS];
     #pragma unroll
     for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) {
-        csState[c] = (mine && c < numCS && g.cs[c].kind == GENNMI_CS_POISSON_EXP) ? asGlobal(g.cs[c].current)[i] : 0.0f;
+        csState[c] = (POISSON && mine && c < numCS && g.cs[c].kind == GENNMI_CS_POISSON_EXP) ? asGlobal(g.cs[c].current)[i] : 0.0f;
     }
     for(uint32_t m = 0; m < numPSM; m++) {
         lds[T.ldsIn[m] + tid] = mine ? asGlobal(g.psm[m].outPost)[i] : 0.0f;
@@ -467,7 +470,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             }
             #pragma unroll
             for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) {
-                if(c < numCS) { Isyn += (g.cs[c].kind == GENNMI_CS_DC) ? g.cs[c].amp : poissonExpStep(g.cs[c], csState[c], i, epoch); }
+                if(c < numCS) { Isyn += (!POISSON || g.cs[c].kind == GENNMI_CS_DC) ? g.cs[c].amp : poissonExpStep(g.cs[c], csState[c], i, epoch); }
             }
             if(g.model == GENNMI_NEURON_LIF) {
                 if(l1 <= 0.0f) {
@@ -529,7 +532,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         asGlobal(g.var0)[i] = l0; asGlobal(g.var1)[i] = l1;
         #pragma unroll
         for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) {
-            if(c < numCS && g.cs[c].kind == GENNMI_CS_POISSON_EXP) { asGlobal(g.cs[c].current)[i] = csState[c]; }
+            if(POISSON && c < numCS && g.cs[c].kind == GENNMI_CS_POISSON_EXP) { asGlobal(g.cs[c].current)[i] = csState[c]; }
         }
     }
     for(uint32_t m = 0; m < numPSM; m++) {
