@@ -108,7 +108,7 @@ def test_rates_against_the_reference_cpu_backend():
     0.4 % in the rate over all neurons.  This run is a third draw (and, the accumulation order of the atomics being free,
     not the same draw twice): it is held to 8 % of the reference's mean in every population — four times the spread seen
     between two correct runs; a wrong rate, weight or time constant of the background moves every rate by far more — and to
-    2.5 % in the rate over all neurons.
+    2.5 % in the rate over all neurons."""
     import os
     import sys
     here = os.path.dirname(os.path.abspath(__file__))
