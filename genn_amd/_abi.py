@@ -15,7 +15,7 @@ MAX_PRE_OUTPUT = 2
 NEURON_LIF, NEURON_IZHIKEVICH, NEURON_SPIKE_SOURCE_ARRAY = 0, 1, 2
 PSM_EXPCURR, PSM_DELTACURR = 0, 1
 CS_DC, CS_ARRAY, CS_POISSON_EXP = 0, 1, 2
-WUM_STATIC_PULSE, WUM_STATIC_PULSE_DENDRITIC_DELAY, WUM_STDP_TRACE, WUM_STATIC_PULSE_CONSTANT_WEIGHT, WUM_STATIC_GRADED, WUM_STATIC_PULSE_REVERSE = 0, 1, 2, 3, 4, 5
+WUM_STATIC_PULSE, WUM_STATIC_PULSE_DENDRITIC_DELAY, WUM_STDP_TRACE, WUM_STATIC_PULSE_CONSTANT_WEIGHT, WUM_STATIC_GRADED, WUM_STATIC_PULSE_REVERSE, WUM_STDP = 0, 1, 2, 3, 4, 5, 6
 MATRIX_SPARSE, MATRIX_TOEPLITZ_CONV2D, MATRIX_DENSE, MATRIX_BITMASK, MATRIX_PROCEDURAL = 0, 1, 2, 3, 4
 CONNECT_SNIPPETS = {"FixedProbability": 0, "FixedProbabilityNoAutapse": 1, "FixedNumberPostWithReplacement": 2}
 SPAN_AUTO, SPAN_POST, SPAN_PRE = 0, 1, 2
@@ -76,7 +76,7 @@ class PresynapticUpdateGroup(C.Structure):
                 ("aMinus", C.c_float), ("wMin", C.c_float), ("wMax", C.c_float),
                 ("conv", C.c_int32 * 8),
                 ("gp", p_u32), ("constantWeight", C.c_float), ("axonalDelaySteps", C.c_uint32),
-                ("numSrcDelaySlots", C.c_uint32), ("pad3_", C.c_uint32), ("procedural", Procedural),
+                ("numSrcDelaySlots", C.c_uint32), ("tauMinus", C.c_float), ("procedural", Procedural),
                 ("srcV", p_f32), ("gradedEpre", C.c_float), ("gradedVslope", C.c_float), ("outPre", p_f32)]
 
 
@@ -86,7 +86,7 @@ class PostsynapticUpdateGroup(C.Structure):
                 ("colLength", p_u32), ("remap", p_u32), ("g", p_f32),
                 ("trgSpkCnt", p_u32), ("trgSpk", p_u32),
                 ("srcST", p_f32), ("preTrace", p_f32),
-                ("aPlus", C.c_float), ("wMin", C.c_float), ("wMax", C.c_float), ("pad_", C.c_uint32),
+                ("aPlus", C.c_float), ("wMin", C.c_float), ("wMax", C.c_float), ("tauPlus", C.c_float),
                 ("rowLength", p_u32), ("ind", p_u32)]
 
 

@@ -169,9 +169,10 @@ def poisson_spike_source(seed, stream, n, rate_hz, steps, dt, rates=None):
 
 
 def plastic_stdp(n=100_000, n_src=1000, steps=10000, seed=99, dt=1.0, fan=500, src_fan=100, src_w=2.0,
-                 ioffset=0.45, w_ei=0.25, w_ie=-1.0, w_ii=-1.0):
+                 ioffset=0.45, w_ei=0.25, w_ie=-1.0, w_ii=-1.0, rule="stdp_trace"):
     """80 % excitatory neurons with plastic E->E (fanout ~``fan``, g0 ~ U[0,0.5], clipped to [0,1]); the
-    static E->I, I->E, I->I projections close a balanced loop; Poisson sources drive E."""
+    static E->I, I->E, I->I projections close a balanced loop; Poisson sources drive E.  ``rule``: "stdp_trace"
+    (pygenn/genn_model.py:1448-1476) or "stdp_additive" (the built-in nearest-neighbour rule, weightUpdateModels.h:345-367)."""
     n_e = (n * 4) // 5
     n_i = n - n_e
     net = Net(name="stdp", dt=dt, steps=steps, seed=seed)
@@ -184,7 +185,7 @@ def plastic_stdp(n=100_000, n_src=1000, steps=10000, seed=99, dt=1.0, fan=500, s
     p_conn = min(1.0, fan / n_e)
     rl, ind = netgen.fixed_probability(seed, 20, n_e, n_e, p_conn)
     g = netgen.rows_uniform(seed, 21, rl, ind.shape[1], n_e, 0.5, 0.0, 0.5, 0.0)
-    net.syns.append(Syn("EE", "E", "E", wum="stdp_trace",
+    net.syns.append(Syn("EE", "E", "E", wum=rule,
                         wum_params=dict(tauPlus=20.0, tauMinus=20.0, aPlus=0.01, aMinus=0.012, wMin=0.0, wMax=1.0),
                         psm="expcurr", tau=5.0, row_stride=ind.shape[1], row_length=rl, ind=ind, g=g))
     for name, src, trg, ns, nt, w, tau, st in (("EI", "E", "I", n_e, n_i, w_ei, 5.0, 22), ("IE", "I", "E", n_i, n_e, w_ie, 10.0, 23),

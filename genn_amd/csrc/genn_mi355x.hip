@@ -392,7 +392,7 @@ int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynap
     if(!g->g) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: required array missing"); }
     if(g->numSrcDelaySlots > 1) {
         if(g->axonalDelaySteps >= g->numSrcDelaySlots) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: axonal delay does not fit the source's delay slots"); }
-        if(g->wum == GENNMI_WUM_STDP_TRACE) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: axonal delay on a plastic projection"); }
+        if(g->wum == GENNMI_WUM_STDP_TRACE || g->wum == GENNMI_WUM_STDP) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: axonal delay on a plastic projection"); }
     }
     else if(g->axonalDelaySteps) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: axonal delay without delay slots"); }
     PreGroupDev d;
@@ -406,6 +406,10 @@ int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynap
         }
         else if(g->wum == GENNMI_WUM_STDP_TRACE) {
             if(!g->trgST || !g->postTrace) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: STDP arrays missing"); }
+            if(r->batch != 1) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: plastic weights need batch size 1"); }
+        }
+        else if(g->wum == GENNMI_WUM_STDP) {
+            if(!g->trgST || !(g->tauMinus > 0.0f)) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: STDP needs the target's spike times and tauMinus > 0"); }
             if(r->batch != 1) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: plastic weights need batch size 1"); }
         }
         else if(g->wum == GENNMI_WUM_STATIC_PULSE_REVERSE) {
@@ -440,7 +444,8 @@ int gennmi_push_postsynaptic_update_group(gennmi_runner *r, const gennmi_postsyn
 {
     if(!r || !g) { return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: null argument"); }
     if(r->finalised) { return fail(GENNMI_ESTATE, "push_postsynaptic_update_group: runner already finalised"); }
-    if(!g->colLength || !g->remap || !g->g || !g->trgSpk || !g->trgSpkCnt || !g->srcST || !g->preTrace) {
+    if(!(g->tauPlus >= 0.0f)) { return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: tauPlus must be 0 (trace rule) or positive"); }
+    if(!g->colLength || !g->remap || !g->g || !g->trgSpk || !g->trgSpkCnt || !g->srcST || (!g->preTrace && !(g->tauPlus > 0.0f))) {
         return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: required array missing");
     }
     if(g->rowStride == 0 || g->colStride == 0) { return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: zero stride"); }
@@ -697,7 +702,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
         else if(p.g.span == GENNMI_SPAN_POST) { W = WAVE; }
         else { W = std::min<uint32_t>(WAVE, std::max(4u, pow2Ceil((rowLen + 3) / 4))); }
         p.lanesPerSpike = W;
-        p.vec4 = (p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum != GENNMI_WUM_STDP_TRACE && (p.g.rowStride % 4) == 0
+        p.vec4 = (p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum != GENNMI_WUM_STDP_TRACE && p.g.wum != GENNMI_WUM_STDP && (p.g.rowStride % 4) == 0
                   && (reinterpret_cast<uintptr_t>(p.g.ind) % 16) == 0 && (reinterpret_cast<uintptr_t>(p.g.g) % 16) == 0
                   && (p.g.wum != GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY || (reinterpret_cast<uintptr_t>(p.g.d) % 4) == 0)
                   && W >= 16) ? 1u : 0u;
@@ -804,7 +809,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
                 continue;
             }
             if(tileFloats == 0 || p.g.matrix != GENNMI_MATRIX_SPARSE || p.g.rowStride > 65535
-               || (p.g.wum != GENNMI_WUM_STATIC_PULSE && p.g.wum != GENNMI_WUM_STDP_TRACE)) { continue; }
+               || (p.g.wum != GENNMI_WUM_STATIC_PULSE && p.g.wum != GENNMI_WUM_STDP_TRACE && p.g.wum != GENNMI_WUM_STDP)) { continue; }
             const uint32_t tileSize = std::min(tileFloats, p.g.numTrgNeurons);
             const uint32_t numTiles = (p.g.numTrgNeurons + tileSize - 1) / tileSize;
             uint16_t *dOff = nullptr; uint32_t *dFlag = nullptr;

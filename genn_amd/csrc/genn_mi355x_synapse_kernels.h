@@ -184,7 +184,10 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
                 atomicAddF32(&outPost[idPost], w);
                 const float dtSpike = st.t - stPost;
                 if(dtSpike > 0) {
-                    const float newWeight = w - (g.aMinus * asGlobal(g.postTrace)[idPost]);
+                    // trace rule: the target's trace; built-in additive rule (weightUpdateModels.h:352-359): the exponential
+                    // of the time since the target's last spike, evaluated in double and rounded once as the reference does
+                    const float factor = (g.wum == GENNMI_WUM_STDP) ? (float)exp((double)(-dtSpike / g.tauMinus)) : asGlobal(g.postTrace)[idPost];
+                    const float newWeight = w - (g.aMinus * factor);
                     weight[rowBase + j] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
                 }
             }
@@ -376,14 +379,18 @@ void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs ar
     GLOBAL_AS float *weight = asGlobal(g.g);
     // trace-STDP rows: besides delivering the (old) weight, every event applies the presynaptic-spike rule to its own
     // synapse (pygenn/genn_model.py:1456-1463); a synapse belongs to exactly one tile, so g needs no atomic here either
-    const bool stdp = (g.wum == GENNMI_WUM_STDP_TRACE);
+    const bool additive = (g.wum == GENNMI_WUM_STDP);
+    const bool stdp = (g.wum == GENNMI_WUM_STDP_TRACE) || additive;
     const float t = stdp ? resolve(args, dt).t : 0.0f;
     GLOBAL_AS const float *trgST = asGlobal(g.trgST);
     GLOBAL_AS const float *postTrace = asGlobal(g.postTrace);
     auto depress = [&](uint32_t idPost, float w) -> float {
         const float stPost = dt + trgST[idPost];
         const float dtSpike = t - stPost;
-        if(dtSpike > 0) { return fminf(g.wMax, fmaxf(g.wMin, w - (g.aMinus * postTrace[idPost]))); }
+        if(dtSpike > 0) {
+            const float factor = additive ? (float)exp((double)(-dtSpike / g.tauMinus)) : postTrace[idPost];
+            return fminf(g.wMax, fmaxf(g.wMin, w - (g.aMinus * factor)));
+        }
         return w;
     };
     const uint32_t L = G.lanes;
@@ -603,15 +610,18 @@ void postsynapticUpdateKernel(const PostGroupDev * __restrict__ blocks, StepArgs
         const uint32_t lastRow = g.numSrcNeurons - 1;
         uint32_t row = localBlock * (BLOCK / WAVE) + threadIdx.x / WAVE;
         uint32_t lenNext = asGlobal(g.rowLength)[min(row, lastRow)];
-        float stNext = asGlobal(g.srcST)[min(row, lastRow)], traceNext = asGlobal(g.preTrace)[min(row, lastRow)];
+        const bool additive = (g.tauPlus > 0.0f);          // built-in rule (weightUpdateModels.h:360-366): no trace array
+        float stNext = asGlobal(g.srcST)[min(row, lastRow)], traceNext = additive ? 0.0f : asGlobal(g.preTrace)[min(row, lastRow)];
         for(; row < g.numSrcNeurons; row += numWaves) {
             const uint32_t len = lenNext;
             const float stPre = dt + stNext;
-            const float step = g.aPlus * traceNext;
+            const float trace = traceNext;
             const uint32_t nextRow = min(row + numWaves, lastRow);
-            lenNext = asGlobal(g.rowLength)[nextRow]; stNext = asGlobal(g.srcST)[nextRow]; traceNext = asGlobal(g.preTrace)[nextRow];
+            lenNext = asGlobal(g.rowLength)[nextRow]; stNext = asGlobal(g.srcST)[nextRow];
+            if(!additive) { traceNext = asGlobal(g.preTrace)[nextRow]; }
             const float dtSpike = st.t - stPre;
             if(!(dtSpike > 0) || len == 0) { continue; }
+            const float step = g.aPlus * (additive ? (float)exp((double)(-dtSpike / g.tauPlus)) : trace);
             const size_t rowBase = (size_t)row * g.rowStride;
             // up to four strides of the row in flight per lane
             for(uint32_t j0 = lane; j0 < len; j0 += 4 * WAVE) {
@@ -642,7 +652,8 @@ void postsynapticUpdateKernel(const PostGroupDev * __restrict__ blocks, StepArgs
             const float stPre = dt + g.srcST[idPre];
             const float dtSpike = st.t - stPre;
             if(dtSpike > 0) {
-                const float newWeight = g.g[rowMajorIndex] + (g.aPlus * g.preTrace[idPre]);
+                const float factor = (g.tauPlus > 0.0f) ? (float)exp((double)(-dtSpike / g.tauPlus)) : g.preTrace[idPre];
+                const float newWeight = g.g[rowMajorIndex] + (g.aPlus * factor);
                 g.g[rowMajorIndex] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
             }
         }

@@ -75,7 +75,7 @@ def init_postsynaptic(snippet, params=None, vars=None):
 
 
 def init_weight_update(snippet, params=None, vars=None, pre_vars=None, post_vars=None):
-    if snippet not in ("StaticPulse", "StaticPulseConstantWeight", "StaticPulseDendriticDelay", "STDPTrace", "StaticGraded", "StaticPulseReverse"):
+    if snippet not in ("StaticPulse", "StaticPulseConstantWeight", "StaticPulseDendriticDelay", "STDPTrace", "STDP", "StaticGraded", "StaticPulseReverse"):
         raise NotImplementedError(f"weight update model {snippet}")
     return _Init(snippet, params, vars, pre_vars, post_vars)
 
@@ -460,6 +460,8 @@ class GeNNModel:
             post = [s for s in n.in_syn if s.wu.snippet == "STDPTrace"]
             if len(pre) > 1 or len(post) > 1:
                 raise NotImplementedError(f"{n.name}: more than one plastic projection per side")
+            # the built-in STDP (weightUpdateModels.h:345-367) keeps no traces: it reads both populations' spike times
+            additive = [s for s in n.out_syn + n.in_syn if s.wu.snippet == "STDP"]
             n.num_delay_slots = max([s.axonal_delay_steps for s in n.out_syn], default=0) + 1
             # projections whose event condition and parameters agree share one queue (neuronGroup.cc:505-517)
             n.event_thresholds = []
@@ -473,7 +475,7 @@ class GeNNModel:
                 raise NotImplementedError(f"{n.name}: more than {_abi.MAX_SPK_EVENT} spike-like event conditions")
             n.pre_trace_owner = pre[0] if pre else None
             n.post_trace_owner = post[0] if post else None
-            n.needs_spike_time = bool(pre or post)
+            n.needs_spike_time = bool(pre or post or additive)
         self._built = True
 
     @staticmethod
@@ -677,7 +679,7 @@ class GeNNModel:
         """initializeSparse(): column views for projections with postsynaptic-spike code."""
         lib = _abi.load()
         for s in self.synapse_populations.values():
-            if s.wu.snippet != "STDPTrace":
+            if s.wu.snippet not in ("STDPTrace", "STDP"):
                 continue
             n_pre, n_post = s.src.num_neurons, s.trg.num_neurons
             m = C.c_uint32()
@@ -810,8 +812,11 @@ class GeNNModel:
             syn_merged.setdefault((s.matrix_type, s.wu.snippet, self._den_delay(s) > 0), []).append(s)
         for members in syn_merged.values():
             stdp = members[0].wu.snippet == "STDPTrace"
+            additive = members[0].wu.snippet == "STDP"
             if stdp:
                 rounded = {q: _merge_round([s.wu.params[q] for s in members]) for q in ("aPlus", "aMinus", "wMin", "wMax")}
+            if additive:
+                rounded = {q: _merge_round([s.wu.params[q] for s in members]) for q in ("tauPlus", "tauMinus", "Aplus", "Aminus", "Wmin", "Wmax")}
             if members[0].wu.snippet == "StaticPulseConstantWeight":
                 consts = _merge_round([s.wu.params["g"] for s in members])
             if members[0].wu.snippet == "StaticGraded":
@@ -821,7 +826,7 @@ class GeNNModel:
                 d.matrix = {"SPARSE": _abi.MATRIX_SPARSE, "TOEPLITZ": _abi.MATRIX_TOEPLITZ_CONV2D, "DENSE": _abi.MATRIX_DENSE,
                             "BITMASK": _abi.MATRIX_BITMASK, "PROCEDURAL": _abi.MATRIX_PROCEDURAL}[s.matrix_type]
                 d.wum = {"StaticPulse": _abi.WUM_STATIC_PULSE, "StaticPulseDendriticDelay": _abi.WUM_STATIC_PULSE_DENDRITIC_DELAY,
-                         "STDPTrace": _abi.WUM_STDP_TRACE, "StaticPulseConstantWeight": _abi.WUM_STATIC_PULSE_CONSTANT_WEIGHT,
+                         "STDPTrace": _abi.WUM_STDP_TRACE, "STDP": _abi.WUM_STDP, "StaticPulseConstantWeight": _abi.WUM_STATIC_PULSE_CONSTANT_WEIGHT,
                          "StaticGraded": _abi.WUM_STATIC_GRADED, "StaticPulseReverse": _abi.WUM_STATIC_PULSE_REVERSE}[s.wu.snippet]
                 if s.wu.snippet == "StaticPulseConstantWeight":
                     d.constantWeight = consts[k]
@@ -880,7 +885,20 @@ class GeNNModel:
                 if stdp:
                     d.trgST, d.postTrace = s.trg.vars["sT"].ptr, s.vars["postTrace"].ptr
                     d.aMinus, d.wMin, d.wMax = rounded["aMinus"][k], rounded["wMin"][k], rounded["wMax"][k]
+                if additive:
+                    d.trgST, d.tauMinus = s.trg.vars["sT"].ptr, rounded["tauMinus"][k]
+                    d.aMinus, d.wMin, d.wMax = rounded["Aminus"][k], rounded["Wmin"][k], rounded["Wmax"][k]
                 _abi.check(lib.gennmi_push_presynaptic_update_group(self._runner, C.byref(d), None))
+                if additive:
+                    q = _abi.PostsynapticUpdateGroup()
+                    q.numSrcNeurons, q.numTrgNeurons = s.src.num_neurons, s.trg.num_neurons
+                    q.rowStride, q.colStride = s.row_stride, s.col_stride
+                    q.colLength, q.remap, q.g = s.vars["colLength"].ptr, s.vars["remap"].ptr, s.vars["g"].ptr
+                    q.trgSpkCnt, q.trgSpk = s.trg.vars["spkCnt"].ptr, s.trg.vars["spk"].ptr
+                    q.srcST, q.tauPlus = s.src.vars["sT"].ptr, rounded["tauPlus"][k]
+                    q.rowLength, q.ind = s.vars["rowLength"].ptr, s.vars["ind"].ptr
+                    q.aPlus, q.wMin, q.wMax = rounded["Aplus"][k], rounded["Wmin"][k], rounded["Wmax"][k]
+                    _abi.check(lib.gennmi_push_postsynaptic_update_group(self._runner, C.byref(q), None))
                 if stdp:
                     q = _abi.PostsynapticUpdateGroup()
                     q.numSrcNeurons, q.numTrgNeurons = s.src.num_neurons, s.trg.num_neurons
@@ -1016,6 +1034,10 @@ def model_from_net(net, batch_size=1, record=True, span=None, device=0):
             wu = init_weight_update("StaticPulseReverse", {}, {"g": 0.0})
         else:
             wu = init_weight_update("STDPTrace", s.wum_params, {"g": 0.0}, {"preTrace": 0.0}, {"postTrace": 0.0})
+        if s.wum == "stdp_additive":
+            q = s.wum_params
+            wu = init_weight_update("STDP", {"tauPlus": q["tauPlus"], "tauMinus": q["tauMinus"], "Aplus": q["aPlus"], "Aminus": q["aMinus"],
+                                             "Wmin": q["wMin"], "Wmax": q["wMax"]}, {"g": 0.0})
         if s.matrix == "procedural":
             if s.wum == "static":
                 wu = init_weight_update("StaticPulse", {}, {"g": init_var(*s.g_init)})

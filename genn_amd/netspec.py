@@ -47,7 +47,7 @@ class Syn:
     src: str
     trg: str
     matrix: str = "sparse"          # "sparse" | "conv2d" | "dense" | "bitmask"
-    wum: str = "static"             # "static" | "static_delay" | "stdp_trace" | "static_const" (one weight, wum_params["g"])
+    wum: str = "static"             # "static" | "static_delay" | "stdp_trace" | "stdp_additive" (built-in STDP) | "static_const" (one weight, wum_params["g"])
                                     # | "static_reverse" (addToPre(g): the row's weights go back to the spiking neuron)
                                     # | "static_graded" (spike-like events, wum_params["Epre"], ["Vslope"]; source must have a V)
     wum_params: Dict[str, float] = field(default_factory=dict)
@@ -192,8 +192,8 @@ def write_netspec(net: Net, path: str):
         elif s.wum == "static_delay":
             w = f"static_delay {s.max_den_delay}"
             np.ascontiguousarray(s.d, dtype=np.uint8).tofile(os.path.join(path, f"{s.name}.d.u8"))
-        elif s.wum == "stdp_trace":
-            w = "stdp_trace " + " ".join(repr(float(s.wum_params[k])) for k in STDP_PARAMS)
+        elif s.wum in ("stdp_trace", "stdp_additive"):
+            w = ("stdp" if s.wum == "stdp_additive" else s.wum) + " " + " ".join(repr(float(s.wum_params[k])) for k in STDP_PARAMS)
         elif s.wum == "static_graded":
             w = f"static_graded {float(s.wum_params['Epre'])!r} {float(s.wum_params['Vslope'])!r}"
         else:
@@ -202,7 +202,7 @@ def write_netspec(net: Net, path: str):
         opts = (" hint_pre" if s.hint_pre else "") + (f" tps {s.threads_per_spike}" if s.threads_per_spike > 1 else "")
         if s.axonal_delay_steps:
             opts += f" axonal_delay {int(s.axonal_delay_steps)}"
-        if s.wum == "stdp_trace":
+        if s.wum in ("stdp_trace", "stdp_additive"):
             mask = np.arange(s.row_stride)[None, :] < s.row_length[:, None]
             col = s.col_stride or int(np.bincount(s.ind[mask], minlength=net.pop(s.trg).n).max())
             opts += f" col_stride {max(1, col)}"

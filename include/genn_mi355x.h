@@ -51,7 +51,12 @@ enum { GENNMI_WUM_STATIC_PULSE = 0, GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY = 1,
        GENNMI_WUM_STATIC_GRADED = 4,
        /* presynaptic-spike code `addToPre(g);` (the static_pulse_reverse model of tests/features/test_event_propagation.py:584-590):
         * every synapse of a spiking neuron's row adds its weight to that neuron's own outPre (SPARSE only) */
-       GENNMI_WUM_STATIC_PULSE_REVERSE = 5 };
+       GENNMI_WUM_STATIC_PULSE_REVERSE = 5,
+       /* the built-in additive STDP with nearest-neighbour pairing (weightUpdateModels.h:345-367): a presynaptic spike
+        * delivers g, then g = clamp(g - Aminus * exp(-(t - st_post) / tauMinus)); a postsynaptic spike applies
+        * g = clamp(g + Aplus * exp(-(t - st_pre) / tauPlus)) down its column.  The exponential is the double one, rounded
+        * once, as in the code the reference generates for its CPU backend.  No trace arrays. */
+       GENNMI_WUM_STDP = 6 };
 /* connectivity: ragged SPARSE (runtime.cc:360-402) or TOEPLITZ Conv2D (initToeplitzConnectivitySnippet.h:105-150) */
 enum { GENNMI_MATRIX_SPARSE = 0, GENNMI_MATRIX_TOEPLITZ_CONV2D = 1,
        /* DENSE: g[numSrc*numTrg], idSyn = idPre*numTrg + idPost; BITMASK: one bit per pair, most significant bit first,
@@ -221,7 +226,8 @@ typedef struct gennmi_presynaptic_update_group_t { /* MergedPresynapticUpdateGro
      * numSrcDelaySlots (backendBase.cc:207-216), i.e. the spikes emitted axonalDelaySteps + 1 steps before the step that
      * delivers them.  numSrcDelaySlots must equal the source group's numDelaySlots (0 or 1: no ring). */
     uint32_t axonalDelaySteps;
-    uint32_t numSrcDelaySlots, pad3_;
+    uint32_t numSrcDelaySlots;
+    float tauMinus;                       /* GENNMI_WUM_STDP */
     gennmi_procedural_t procedural;       /* GENNMI_MATRIX_PROCEDURAL only (rowStride = the stride the stored matrix would have) */
     /* GENNMI_WUM_STATIC_GRADED (SPARSE only): srcSpk / srcSpkCnt are the source's event queue for threshold Epre; V_pre is
      * read when the event is delivered, i.e. after the update (and reset) that emitted it */
@@ -239,7 +245,7 @@ typedef struct gennmi_postsynaptic_update_group_t { /* MergedPostsynapticUpdateG
     const uint32_t *trgSpkCnt, *trgSpk;
     const float *srcST, *preTrace;
     float aPlus, wMin, wMax;
-    uint32_t pad_;
+    float tauPlus;                        /* > 0: the built-in additive rule (GENNMI_WUM_STDP), preTrace unused; 0: trace STDP */
     /* row view of the same matrix (optional, both or neither): lets a step in which a large share of the target
      * population fired walk the rows once, coalesced, instead of one gather per (spike, column entry) */
     const uint32_t *rowLength;            /* [numSrcNeurons] */

@@ -44,7 +44,7 @@
 
 enum { GC_LIF = 0, GC_IZH = 1, GC_SSA = 2 };
 enum { GC_EXPCURR = 0, GC_DELTACURR = 1 };
-enum { GC_STATIC = 0, GC_STATIC_DELAY = 1, GC_STDP_TRACE = 2, GC_STATIC_GRADED = 3, GC_STATIC_REVERSE = 4 };
+enum { GC_STATIC = 0, GC_STATIC_DELAY = 1, GC_STDP_TRACE = 2, GC_STATIC_GRADED = 3, GC_STATIC_REVERSE = 4, GC_STDP_ADDITIVE = 5 };
 enum { GC_SPARSE = 0, GC_CONV2D = 1, GC_DENSE = 2, GC_BITMASK = 3 };
 enum { GC_CS_DC = 0, GC_CS_NOISE = 1, GC_CS_POISSON_EXP = 2 };
 
@@ -108,6 +108,7 @@ typedef struct {
     const uint32_t *rowLength, *ind; float *g; const uint8_t *d;
     uint32_t *colLength, *remap;
     float aPlus, aMinus, wMin, wMax;
+    float tauPlus, tauMinus;   /* GC_STDP_ADDITIVE */
     int conv[8]; int conv_bh, conv_bw;
     uint32_t delaySteps;    /* axonal delay in timesteps: reads slot (spkQuePtr + slots - delaySteps) % slots of the source */
     const uint32_t *gp;     /* BITMASK connectivity words */
@@ -288,6 +289,19 @@ static void gc_need_st(gc_pop *p)
     }
 }
 
+/* built-in additive STDP with nearest-neighbour pairing (weightUpdateModels.h:345-367): no trace variables, spike times of
+ * both populations */
+void gc_set_stdp_additive(gc_net *net, int syn, float tauPlus, float tauMinus, float aPlus, float aMinus, float wMin, float wMax,
+                          uint32_t colStride)
+{
+    gc_syn *s = &net->syns[syn];
+    gc_pop *pre = &net->pops[s->src], *post = &net->pops[s->trg];
+    s->tauPlus = tauPlus; s->tauMinus = tauMinus; s->aPlus = aPlus; s->aMinus = aMinus; s->wMin = wMin; s->wMax = wMax; s->colStride = colStride;
+    gc_need_st(pre); gc_need_st(post);
+    s->colLength = (uint32_t*)calloc(post->n, sizeof(uint32_t));
+    s->remap = (uint32_t*)calloc((size_t)post->n * colStride, sizeof(uint32_t));
+}
+
 void gc_set_stdp_trace(gc_net *net, int syn, float aPlus, float aMinus, float wMin, float wMax,
                        float tauPlusDecay, float tauMinusDecay, uint32_t colStride)
 {
@@ -457,6 +471,18 @@ void gc_update_synapses(gc_net *net, float t)
                 else if(s->wum == GC_STATIC_DELAY) {
                     psm->denDelay[(size_t)((psm->denDelayPtr + s->d[idSyn]) % psm->maxDenDelay) * trg->n + idPost] += s->g[idSyn];
                 }
+                else if(s->wum == GC_STDP_ADDITIVE) {
+                    /* weightUpdateModels.h:352-359.  The generated code includes <cmath> only and calls exp unqualified, so
+                     * the exponential is the double one, rounded once on assignment to the scalar */
+                    const float stPost = net->dt + trg->sT[idPost];
+                    psm->outPost[idPost] += s->g[idSyn];
+                    const float dt = t - stPost;
+                    if(dt > 0) {
+                        const float timing = (float)exp((double)(-dt / s->tauMinus));
+                        const float newWeight = s->g[idSyn] - (s->aMinus * timing);
+                        s->g[idSyn] = fmaxf(s->wMin, fminf(s->wMax, newWeight));
+                    }
+                }
                 else {
                     const float stPost = net->dt + trg->sT[idPost];
                     psm->outPost[idPost] += s->g[idSyn];
@@ -472,7 +498,7 @@ void gc_update_synapses(gc_net *net, float t)
     /* postsynaptic updates (learnPost) through the column remap */
     for(int k = 0; k < net->numSyns; k++) {
         gc_syn *s = &net->syns[k];
-        if(s->wum != GC_STDP_TRACE) { continue; }
+        if(s->wum != GC_STDP_TRACE && s->wum != GC_STDP_ADDITIVE) { continue; }
         const gc_pop *src = &net->pops[s->src];
         const gc_pop *trg = &net->pops[s->trg];
         const uint32_t numSpikes = trg->spkCnt;
@@ -485,7 +511,13 @@ void gc_update_synapses(gc_net *net, float t)
                 const uint32_t idPre = rowMajorIndex / s->rowStride;
                 const float stPre = net->dt + src->sT[idPre];
                 const float dt = t - stPre;
-                if(dt > 0) {
+                if(dt > 0 && s->wum == GC_STDP_ADDITIVE) {
+                    /* weightUpdateModels.h:360-366 */
+                    const float timing = (float)exp((double)(-dt / s->tauPlus));
+                    const float newWeight = s->g[rowMajorIndex] + (s->aPlus * timing);
+                    s->g[rowMajorIndex] = fmaxf(s->wMin, fminf(s->wMax, newWeight));
+                }
+                else if(dt > 0) {
                     const float newWeight = s->g[rowMajorIndex] + (s->aPlus * src->preTrace[idPre]);
                     s->g[rowMajorIndex] = fminf(s->wMax, fmaxf(s->wMin, newWeight));
                 }

@@ -22,7 +22,7 @@ SRC = os.path.join(HERE, "genn_cpu.c")
 
 GC_LIF, GC_IZH, GC_SSA = 0, 1, 2
 GC_EXPCURR, GC_DELTACURR = 0, 1
-GC_STATIC, GC_STATIC_DELAY, GC_STDP_TRACE, GC_STATIC_GRADED, GC_STATIC_REVERSE = 0, 1, 2, 3, 4
+GC_STATIC, GC_STATIC_DELAY, GC_STDP_TRACE, GC_STATIC_GRADED, GC_STATIC_REVERSE, GC_STDP_ADDITIVE = 0, 1, 2, 3, 4, 5
 GC_CS_DC, GC_CS_NOISE, GC_CS_POISSON_EXP = 0, 1, 2
 
 
@@ -48,6 +48,7 @@ def lib():
         l.gc_philox4x32.restype = None; l.gc_philox4x32.argtypes = [u32] * 6 + [vp]
         l.gc_cs_current.restype = vp; l.gc_cs_current.argtypes = [vp, i32, i32]
         l.gc_add_syn_sparse.restype = i32; l.gc_add_syn_sparse.argtypes = [vp, i32, i32, i32, i32, u32, vp, vp, vp, vp, i32]
+        l.gc_set_stdp_additive.restype = None; l.gc_set_stdp_additive.argtypes = [vp, i32, f32, f32, f32, f32, f32, f32, u32]
         l.gc_set_stdp_trace.restype = None; l.gc_set_stdp_trace.argtypes = [vp, i32, f32, f32, f32, f32, f32, f32, u32]
         l.gc_add_syn_conv2d.restype = i32; l.gc_add_syn_conv2d.argtypes = [vp, i32, i32, i32, vp, vp]
         l.gc_set_delay_slots.restype = None; l.gc_set_delay_slots.argtypes = [vp, i32, u32]
@@ -234,9 +235,9 @@ class OracleNet:
                 d = _as(s.d, np.uint8) if s.d is not None else None
                 self.keep += [rl, ind, g, d]
                 wum = {"static": GC_STATIC, "static_const": GC_STATIC, "static_delay": GC_STATIC_DELAY, "stdp_trace": GC_STDP_TRACE,
-                       "static_graded": GC_STATIC_GRADED, "static_reverse": GC_STATIC_REVERSE}[s.wum]
+                       "static_graded": GC_STATIC_GRADED, "static_reverse": GC_STATIC_REVERSE, "stdp_additive": GC_STDP_ADDITIVE}[s.wum]
                 sid = self.l.gc_add_syn_sparse(self.h, src, trg, self.psm_id[s.name], wum, s.row_stride, rl.ctypes.data, ind.ctypes.data,
-                                               g.ctypes.data, d.ctypes.data if d is not None else None, int(s.wum == "stdp_trace"))
+                                               g.ctypes.data, d.ctypes.data if d is not None else None, int(s.wum in ("stdp_trace", "stdp_additive")))
                 if s.wum == "static_reverse":
                     self.l.gc_set_static_reverse(self.h, sid)
                 if s.wum == "static_graded":
@@ -245,12 +246,20 @@ class OracleNet:
                     k = graded.index(s)
                     self.l.gc_set_static_graded(self.h, sid, C.c_float(_round_group([x.wum_params["Epre"] for x in graded])[k]),
                                                 C.c_float(_round_group([x.wum_params["Vslope"] for x in graded])[k]))
-                if s.wum == "stdp_trace":
+                if s.wum in ("stdp_trace", "stdp_additive"):
                     q = s.wum_params
                     stride = (col_stride or {}).get(s.name)
                     if stride is None:
                         mask = np.arange(s.row_stride)[None, :] < rl[:, None]
                         stride = int(np.bincount(ind.reshape(len(rl), -1)[mask], minlength=net.pop(s.trg).n).max())
+                if s.wum == "stdp_additive":
+                    # the six parameters are literals in the generated code (one plastic projection per merged group)
+                    self.l.gc_set_stdp_additive(self.h, sid, *(C.c_float(literal_f32(q[k])) for k in ("tauPlus", "tauMinus", "aPlus", "aMinus", "wMin", "wMax")),
+                                                max(1, stride))
+                    self.l.gc_build_remap(self.h, sid)
+                    self.col_stride = getattr(self, "col_stride", {})
+                    self.col_stride[s.name] = max(1, stride)
+                if s.wum == "stdp_trace":
                     self.l.gc_set_stdp_trace(self.h, sid, C.c_float(literal_f32(q["aPlus"])), C.c_float(literal_f32(q["aMinus"])),
                                              C.c_float(literal_f32(q["wMin"])), C.c_float(literal_f32(q["wMax"])),
                                              C.c_float(literal_f32(math.exp(-dt / q["tauPlus"]))),

@@ -41,10 +41,14 @@ def reverse_small():
     return configs.reverse(), 25
 
 
+def stdp_additive_small():
+    return configs.plastic_stdp(n=500, n_src=50, steps=200, fan=60, src_fan=40, rule="stdp_additive"), 25
+
+
 def potjans_poisson_net():
     """10 % of the neurons at 20 % in-degree under the script's own Poisson background, 5 s of model time (rates fixture only)."""
     return configs.potjans(neuron_scale=0.1, connectivity_scale=0.2, steps=50000, poisson=True)
 
 
-CASES = {"reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+CASES = {"stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
          "stdp_small": stdp_small, "conv_small": conv_small}

@@ -31,7 +31,7 @@ def run_side_by_side(net, steps=None, check_every=1, exact=True, use_graph=False
     model = model_from_net(net, span=span)
     model.load(num_recording_timesteps=steps)
     oracle = OracleNet(net, num_recording_timesteps=steps,
-                       col_stride={s.name: model.synapse_populations[s.name].col_stride for s in net.syns if s.wum == "stdp_trace"} or None)
+                       col_stride={s.name: model.synapse_populations[s.name].col_stride for s in net.syns if s.wum in ("stdp_trace", "stdp_additive")} or None)
     counts = {p.name: 0 for p in net.pops}
     diverged = False
     for step in range(steps):
@@ -78,6 +78,8 @@ def compare_state(net, model, oracle, where, exact):
                     got.reshape(D, n)[nxt] = 0
                     want.reshape(D, n)[nxt] = 0
                 assert_close(got, want, f"{where}: denDelay of {s.name}", exact, accumulator=True)
+        if s.wum == "stdp_additive":
+            assert_close(sg.vars["g"].pull_from_device(), oracle.syn_g(s.name), f"{where}: g of {s.name}", exact)
         if s.wum == "stdp_trace":
             assert_close(sg.vars["g"].pull_from_device(), oracle.syn_g(s.name), f"{where}: g of {s.name}", exact)
             assert_close(sg.vars["preTrace"].pull_from_device(), oracle.pre_trace(s.src), f"{where}: preTrace of {s.name}", exact)

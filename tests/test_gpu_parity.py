@@ -87,9 +87,12 @@ def test_izhikevich_fanout_noise():
     model.unload()
 
 
-def test_plastic_stdp_learn_post():
-    """C4 shape: trace STDP on E->E with learnPost through the column remap, SpikeSourceArray drive."""
-    net = configs.plastic_stdp(n=5000, n_src=100, steps=200, fan=250, src_fan=50)
+@pytest.mark.parametrize("rule", ["stdp_trace", "stdp_additive"])
+def test_plastic_stdp_learn_post(rule):
+    """C4 shape: STDP on E->E with learnPost through the column remap, SpikeSourceArray drive — with the trace rule of the
+    benchmark script and with the built-in nearest-neighbour rule (weightUpdateModels.h:345-367), whose oracle restatement
+    the fixture stdp_additive_small pins to the reference's CPU backend."""
+    net = configs.plastic_stdp(n=5000, n_src=100, steps=200, fan=250, src_fan=50, rule=rule)
     model = model_from_net(net)
     model.load(num_recording_timesteps=net.steps)
     sg = model.synapse_populations["EE"]
@@ -118,14 +121,15 @@ def test_plastic_stdp_learn_post():
     model.unload()
 
 
+@pytest.mark.parametrize("rule", ["stdp_trace", "stdp_additive"])
 @pytest.mark.parametrize("divisor", ["1000000", "0"])
-def test_learn_post_row_walk_and_column_walk(divisor, monkeypatch):
+def test_learn_post_row_walk_and_column_walk(divisor, rule, monkeypatch):
     """learnPost has two device paths: columns of the spiking targets through the remap (few spikes) and a walk over
     all rows with a bitmap of the spiking targets (many spikes).  Forcing either for every step must leave the same
     weights as the oracle: each synapse gets the same single update, so g must agree to the last bit of the tolerance
     used everywhere else (and the two device paths with each other exactly)."""
     monkeypatch.setenv("GENNMI_POST_DENSE_DIVISOR", divisor)
-    net = configs.plastic_stdp(n=3000, n_src=100, steps=120, fan=150, src_fan=50)
+    net = configs.plastic_stdp(n=3000, n_src=100, steps=120, fan=150, src_fan=50, rule=rule)
     model = model_from_net(net)
     model.load(num_recording_timesteps=net.steps)
     sg = model.synapse_populations["EE"]

@@ -102,7 +102,7 @@ def test_unsupported_models_fail_loudly():
     with pytest.raises(NotImplementedError):
         m.add_neuron_population("p", 10, "TraubMiles", {}, {})
     with pytest.raises(NotImplementedError):
-        init_weight_update("STDP")
+        init_weight_update("PiecewiseSTDP")
     with pytest.raises(NotImplementedError):
         init_postsynaptic("ExpCond")
     with pytest.raises(NotImplementedError):

@@ -61,8 +61,9 @@ def test_oracle_matches_reference_backend(case):
                     assert np.array_equal(oracle.post_trace(s.trg), gold[f"postTrace.{s.name}"][k])
             k += 1
     for s in net.syns:
-        if s.wum == "stdp_trace":
+        if s.wum in ("stdp_trace", "stdp_additive"):
             assert np.array_equal(oracle.syn_g(s.name), gold[f"g.{s.name}"])
+            assert np.count_nonzero(gold[f"g.{s.name}"] != s.g.reshape(-1)) > 100, "the fixture's run changed no weight" 
         if fuse[s.name] == s.name and f"denDelay.{s.name}" in gold:
             assert np.array_equal(oracle.den_delay(s.name), gold[f"denDelay.{s.name}"])
     for name in record_events:
