@@ -170,6 +170,15 @@ bool isTraceSTDP(const WeightUpdateModels::Base *m)
         && same(m->getPreDynamicsCode(), "preTrace *= tauPlusDecay;") && same(m->getPostDynamicsCode(), "postTrace *= tauMinusDecay;")
         && m->getSynapseDynamicsCode().empty() && m->getPreEventSynCode().empty() && m->getPostEventSynCode().empty();
 }
+// the built-in additive STDP with nearest-neighbour pairing (weightUpdateModels.h:345-367)
+bool isAdditiveSTDP(const WeightUpdateModels::Base *m)
+{
+    const auto *builtin = WeightUpdateModels::STDP::getInstance();
+    return same(m->getPreSpikeSynCode(), builtin->getPreSpikeSynCode()) && same(m->getPostSpikeSynCode(), builtin->getPostSpikeSynCode())
+        && m->getPreSpikeCode().empty() && m->getPostSpikeCode().empty() && m->getPreDynamicsCode().empty() && m->getPostDynamicsCode().empty()
+        && m->getSynapseDynamicsCode().empty() && m->getPreEventSynCode().empty() && m->getPostEventSynCode().empty()
+        && m->getVars().size() == 1 && m->getVars()[0].name == "g" && m->getParams().size() == 6 && m->getPreVars().empty() && m->getPostVars().empty();
+}
 // StaticGraded (weightUpdateModels.h:308-319): spike-like events while V > Epre, each adding
 // fmax(0, g * tanh((V_pre - Epre) / Vslope) * dt).  The built-in's event code spells the presynaptic potential `V_pre`;
 // a model with the same code that spells it `V` — the name the 5.4.0 generator gives a presynaptic neuron variable
@@ -206,6 +215,7 @@ unsigned int recogniseWUM(const WeightUpdateModels::Base *m, const std::string &
         return GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY;
     }
     if(isTraceSTDP(m)) { return GENNMI_WUM_STDP_TRACE; }
+    if(isAdditiveSTDP(m)) { return GENNMI_WUM_STDP; }
     if(isStaticGraded(m)) { return GENNMI_WUM_STATIC_GRADED; }
     // presynaptic output: the static_pulse_reverse model of the reference's tests/features/test_event_propagation.py:584-590
     if(plain && same(m->getPreSpikeSynCode(), "addToPre(g);") && m->getVars().size() == 1 && m->getVars()[0].name == "g") { return GENNMI_WUM_STATIC_PULSE_REVERSE; }
@@ -600,13 +610,14 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                 const auto *wum = arch.getWUInitialiser().getSnippet();
                 const unsigned int wumKind = recogniseWUM(wum, arch.getName());
                 const bool srcDelay = arch.getSrcNeuronGroup()->isDelayRequired();
-                if(arch.getBackPropDelaySteps() != 0 || (wumKind == GENNMI_WUM_STDP_TRACE && (srcDelay || arch.getTrgNeuronGroup()->isDelayRequired()))) {
+                const bool plastic = (wumKind == GENNMI_WUM_STDP_TRACE || wumKind == GENNMI_WUM_STDP);
+                if(arch.getBackPropDelaySteps() != 0 || (plastic && (srcDelay || arch.getTrgNeuronGroup()->isDelayRequired()))) {
                     unsupported("back-propagation delay, or delay slots on a plastic projection ('" + arch.getName() + "')");
                 }
                 const bool graded = (wumKind == GENNMI_WUM_STATIC_GRADED);
                 if((arch.isPreSpikeEventRequired() && !graded) || arch.isPostSpikeEventRequired()) { unsupported("spike-like events on projection '" + arch.getName() + "'"); }
                 if(graded && srcDelay) { unsupported("delay slots on the source of graded projection '" + arch.getName() + "'"); }
-                if(wumKind == GENNMI_WUM_STDP_TRACE && batchSize != 1) { unsupported("plastic weights with a batch size above 1"); }
+                if(plastic && batchSize != 1) { unsupported("plastic weights with a batch size above 1"); }
 
                 const auto matrixType = arch.getMatrixType();
                 const bool sparse = (matrixType & SynapseMatrixConnectivity::SPARSE) && (matrixType & SynapseMatrixWeight::INDIVIDUAL);
@@ -776,6 +787,14 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                     out << "d.d = " << wuVar("d", Type::Uint8) << "; d.denDelay = gennmiDev(" << env["_den_delay"] << "); d.denDelayPtr = gennmiDev(" << env["_den_delay_ptr"] << ");" << std::endl;
                     out << "{ static const uint32_t v[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getMaxDendriticDelayTimesteps(); })) << "; d.maxDenDelay = v[g]; }" << std::endl;
                 }
+                if(wumKind == GENNMI_WUM_STDP) {
+                    out << "d.trgST = gennmiDev(" << env["_trg_st"] << ");" << std::endl;
+                    for(const auto &[field, p] : {std::pair<const char*, const char*>{"tauMinus", "tauMinus"}, {"aMinus", "Aminus"}, {"wMin", "Wmin"}, {"wMax", "Wmax"}}) {
+                        const std::string param = p;
+                        out << "{ static const float v[] = " << table(values([param](const SynapseGroupInternal &g){ return g.getWUInitialiser().getParams().at(param); }), scalar)
+                            << "; d." << field << " = v[g]; }" << std::endl;
+                    }
+                }
                 if(wumKind == GENNMI_WUM_STDP_TRACE) {
                     env.addField(scalar.createPointer(), "_mi_postTrace", "postTrace",
                                  [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g.getFusedWUPostTarget(), "postTrace"); });
@@ -793,7 +812,8 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
             [this, &funcEnv, batchSize, scalar](auto &s)
             {
                 const auto &arch = s.getArchetype();
-                if(!isTraceSTDP(arch.getWUInitialiser().getSnippet())) { unsupported("postsynaptic-spike code of projection '" + arch.getName() + "'"); }
+                const bool additive = isAdditiveSTDP(arch.getWUInitialiser().getSnippet());
+                if(!additive && !isTraceSTDP(arch.getWUInitialiser().getSnippet())) { unsupported("postsynaptic-spike code of projection '" + arch.getName() + "'"); }
                 if(!(arch.getMatrixType() & SynapseMatrixConnectivity::SPARSE)) { unsupported("postsynaptic learning on a non-SPARSE projection"); }
 
                 CodeStream::Scope b(funcEnv.getStream());
@@ -811,8 +831,10 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                     return v;
                 };
                 env.addField(scalar.createPointer(), "_mi_g", "g", [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, "g"); });
-                env.addField(scalar.createPointer(), "_mi_preTrace", "preTrace",
-                             [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g.getFusedWUPreTarget(), "preTrace"); });
+                if(!additive) {
+                    env.addField(scalar.createPointer(), "_mi_preTrace", "preTrace",
+                                 [](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g.getFusedWUPreTarget(), "preTrace"); });
+                }
                 out << "gennmi_postsynaptic_update_group_t d = {};" << std::endl;
                 out << "{ static const uint32_t a[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getSrcNeuronGroup()->getNumNeurons(); }))
                     << ", b[] = " << tableU32(counts([](const SynapseGroupInternal &g){ return g.getTrgNeuronGroup()->getNumNeurons(); }))
@@ -821,12 +843,16 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                     << "; d.numSrcNeurons = a[g]; d.numTrgNeurons = b[g]; d.rowStride = c[g]; d.colStride = e[g]; }" << std::endl;
                 out << "d.colLength = gennmiDev(" << env["_col_length"] << "); d.remap = gennmiDev(" << env["_remap"] << "); d.g = gennmiDev(" << env["_mi_g"] << ");" << std::endl;
                 out << "d.trgSpkCnt = gennmiDev(" << env["_trg_spk_cnt"] << "); d.trgSpk = gennmiDev(" << env["_trg_spk"] << ");" << std::endl;
-                out << "d.srcST = gennmiDev(" << env["_src_st"] << "); d.preTrace = gennmiDev(" << env["_mi_preTrace"] << ");" << std::endl;
+                out << "d.srcST = gennmiDev(" << env["_src_st"] << ");" << std::endl;
+                if(!additive) { out << "d.preTrace = gennmiDev(" << env["_mi_preTrace"] << ");" << std::endl; }
                 out << "d.rowLength = gennmiDev(" << env["_row_length"] << "); d.ind = gennmiDev(" << env["_ind"] << ");" << std::endl;
-                for(const char *p : {"aPlus", "wMin", "wMax"}) {
+                const std::vector<std::pair<std::string, std::string>> fields = additive
+                    ? std::vector<std::pair<std::string, std::string>>{{"tauPlus", "tauPlus"}, {"aPlus", "Aplus"}, {"wMin", "Wmin"}, {"wMax", "Wmax"}}
+                    : std::vector<std::pair<std::string, std::string>>{{"aPlus", "aPlus"}, {"wMin", "wMin"}, {"wMax", "wMax"}};
+                for(const auto &[field, p] : fields) {
                     std::vector<Type::NumericValue> v;
                     for(const auto &g : s.getGroups()) { v.push_back(g.get().getWUInitialiser().getParams().at(p)); }
-                    out << "{ static const float v[] = " << table(v, scalar) << "; d." << p << " = v[g]; }" << std::endl;
+                    out << "{ static const float v[] = " << table(v, scalar) << "; d." << field << " = v[g]; }" << std::endl;
                 }
                 out << "GENNMI_CHECK(gennmi_push_postsynaptic_update_group(gennmiRunner, &d, nullptr));" << std::endl;
             });

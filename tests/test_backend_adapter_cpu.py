@@ -40,7 +40,7 @@ def _exports(lib):
     return {line.split()[-1] for line in out.splitlines() if " T " in line}
 
 
-@pytest.mark.parametrize("case", ["stdp_small", "potjans_small", "conv_small", "dense_small", "va_delay_small", "graded_small", "reverse_small"])
+@pytest.mark.parametrize("case", ["stdp_small", "stdp_additive_small", "potjans_small", "conv_small", "dense_small", "va_delay_small", "graded_small", "reverse_small"])
 def test_generated_runner_exports_reference_entry_points(case):
     net, tmp, code = _generate(case)
     try:
@@ -50,9 +50,12 @@ def test_generated_runner_exports_reference_entry_points(case):
         pushes = {e for e in exports if e.startswith("pushMerged")}
         assert any(e.startswith("pushMergedNeuronUpdateGroup") for e in pushes)
         assert any(e.startswith("pushMergedPresynapticUpdateGroup") for e in pushes)
-        if case == "stdp_small":
+        if case in ("stdp_small", "stdp_additive_small"):
             assert any(e.startswith("pushMergedPostsynapticUpdateGroup") for e in pushes)
             assert "pushMergedNeuronUpdate0spikeTimesToDevice" in exports or any("spikeTimes" in e for e in pushes)
+        if case == "stdp_additive_small":
+            synapse_code = open(os.path.join(code, "synapseUpdate.cc")).read()
+            assert "d.wum = 6u" in synapse_code and "d.tauMinus = v[g]" in synapse_code and "d.tauPlus = v[g]" in synapse_code and "d.preTrace" not in synapse_code
         # the runner is host code: no device code object, only a link against the device library
         ldd = subprocess.run(["ldd", os.path.join(code, "librunner.so")], stdout=subprocess.PIPE, text=True).stdout
         assert "libgenn_mi355x.so" in ldd
@@ -66,7 +69,7 @@ def test_generated_runner_exports_reference_entry_points(case):
             assert "d.conv[7]" in synapse
         init = open(os.path.join(code, "init.cc")).read()
         assert "gennmi_push_mirrors" in init
-        if case == "stdp_small":
+        if case in ("stdp_small", "stdp_additive_small"):
             assert "gennmi_build_remap" in init
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
