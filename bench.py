@@ -27,12 +27,10 @@ BYTES_PER_EVENT = {"dense": 4,          # one weight read per (spike, target); o
                    "static": 16, "static_delay": 17, "stdp_trace": 28, "conv2d": 8}
 # HBM bytes per launch of the dominant kernel, from hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each
 # scaled by what the same counter reads for the library's 256 MiB copy kernel); recorded with the commands that
-# produced them in profiles/<kernel>_<workload>.md.  They are measurements of an earlier run of the same workload,
-# not of this one; workloads without an entry report null.
+# produced them in profiles/<kernel>_<workload>.md.  A counter run is a separate invocation of this script, so the figure
+# is only attached to a run of the very command line it was measured on (same workload, steps and warm-up: the network,
+# its seed and therefore its activity are then identical); any other run reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "potjans": {"bytes_per_launch": 5.76e6, "source": "profiles/stepFusedKernel_potjans_full.md (median launch: 3172.6 KiB read + 2447.8 KiB written)"},
-    "potjans_resident": {"bytes_per_step": 3.90e6, "source": "profiles/residentKernel_potjans_full.md (10,000-step launch: 38.05 GB read + 0.97 GB written)"},
-    "izh": {"bytes_per_launch": 2.43e8, "source": "profiles/presynapticTileKernel_izhikevich_1M_full.md (average launch of presynapticTileKernel + presynapticUpdateKernel over the first 500 steps)"},
 }
 
 
@@ -304,12 +302,10 @@ def main():
         for _ in range(5):
             b.copy_on_device(a)
         a.free(); b.free()
-    if roofline is not None and info["resident_plan"] and args.workload == "potjans":
-        roofline["traffic"] = MEASURED_TRAFFIC_BYTES["potjans_resident"]["bytes_per_step"] * args.steps
-        roofline["traffic_source"] = MEASURED_TRAFFIC_BYTES["potjans_resident"]["source"]
-    elif roofline is not None and args.workload in MEASURED_TRAFFIC_BYTES:
-        roofline["traffic"] = MEASURED_TRAFFIC_BYTES[args.workload]["bytes_per_launch"]
-        roofline["traffic_source"] = MEASURED_TRAFFIC_BYTES[args.workload]["source"]
+    measured = MEASURED_TRAFFIC_BYTES.get((args.workload, args.steps, args.warmup))
+    if roofline is not None and measured is not None and measured["plan"] == ("resident" if info["resident_plan"] else "stepped"):
+        roofline["traffic"] = measured["bytes_per_launch"]
+        roofline["traffic_source"] = measured["source"]
     model.unload()
 
     # ---- CPU baseline: the single-threaded oracle on the same network, bounded sample from t = 0
@@ -319,9 +315,10 @@ def main():
         # the reference's CPU backend (and the oracle) has no batch dimension: batch 0 is timed and the figure is per batch
         oracle = OracleNet(net.batch_nets[0] if batch > 1 else net)
         # activity is not stationary (silent start, bursts), so the sample is bounded by time, not sized from a probe:
-        # blocks of steps until ~12 s of CPU work or the GPU run's step count, whichever comes first
+        # blocks of steps until ~12 s of CPU work
+        # (the sample does not depend on --steps: a run of a few steps still gets a baseline worth the name)
         cpu_budget_s, block = 12.0, 10
-        limit = args.cpu_steps or (args.warmup + args.steps)
+        limit = args.cpu_steps or (1 << 62)
         cpu_steps, cpu_wall = 0, 0.0
         while cpu_steps < limit and (args.cpu_steps or cpu_wall < cpu_budget_s):
             n = min(block, limit - cpu_steps)
