@@ -123,6 +123,7 @@ SYMBOLS = {
     "gennmi_runner_finalise": (C.c_int, [C.c_void_p]),
     "gennmi_build_remap": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "gennmi_max_col_length": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]),
+    "gennmi_max_col_length_static": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "gennmi_init_var": (C.c_int, [C.c_void_p, C.c_uint32, C.c_size_t, C.c_uint32, C.POINTER(C.c_double * 4), C.c_uint64, C.c_uint32]),
     "gennmi_init_sparse_fixed_probability": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_double, C.c_int, C.c_uint64, C.c_uint32,
                                                        C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]),

@@ -120,6 +120,7 @@ namespace gennmi_detail
 // error reporting and write tracking for the library's other translation units
 int fail(int code, const std::string &msg) { return ::fail(code, msg); }
 void noteDeviceWrite(const void *dev, size_t bytes) { ::noteDeviceWrite(dev, bytes); }
+int prepareStaticScratch();             // looks up the current device's copy of the static counter array (defined with it)
 }
 
 extern "C" {
@@ -135,7 +136,7 @@ int gennmi_init(int device)
     hipDeviceProp_t prop;
     HIP_TRY(hipGetDeviceProperties(&prop, device));
     if(prop.warpSize != WAVE) { return fail(GENNMI_EUNSUPPORTED, "gennmi_init: kernels assume 64-wide wavefronts"); }
-    return GENNMI_OK;
+    return gennmi_detail::prepareStaticScratch();
 }
 
 int gennmi_device_name(char *buf, size_t len)
@@ -1313,6 +1314,84 @@ int gennmi_max_col_length(uint32_t numSrc, uint32_t numTrg, uint32_t rowStride, 
     uint32_t m = 0;
     for(uint32_t v : h) { m = std::max(m, v); }
     *maxColLength = m;
+    return GENNMI_OK;
+}
+
+// ---- the one entry point that allocates nothing: gennmi_max_col_length with its per-column counters in a file-scope
+// device array instead of a hipMalloc'd one.  Every device holds its own copy of the array at its own address; the
+// address is looked up once per device and that pointer — never the array's name, which in host code is only a
+// handle — is what the kernels receive.
+}   // extern "C"
+
+namespace
+{
+constexpr uint32_t STATIC_COUNTER_MAX = GENNMI_STATIC_MAX_TARGETS;       // 2^20 counters = 4 MiB per device
+static __device__ __align__(256) uint32_t scratch[STATIC_COUNTER_MAX];
+constexpr int STATIC_MAX_DEVICES = 64;
+std::mutex g_scratchMutex;
+uint32_t *g_scratchPtr[STATIC_MAX_DEVICES] = {};
+
+// clears the counters a call will use and its result word
+__global__ void staticClearKernel(uint32_t *counters, uint32_t count, uint32_t *result)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if(i < count) { counters[i] = 0u; }
+    if(i == 0) { *result = 0u; }
+}
+
+__global__ __launch_bounds__(BLOCK)
+void staticMaxKernel(const uint32_t *counters, uint32_t count, uint32_t *result)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    uint32_t v = (i < count) ? counters[i] : 0u;
+    for(int off = WAVE / 2; off > 0; off >>= 1) { v = max(v, (uint32_t)__shfl_down(v, off, WAVE)); }
+    if((threadIdx.x & (WAVE - 1)) == 0 && v) { atomicMax(result, v); }
+}
+
+// address of the current device's copy of `scratch` (looked up on first use, once per device)
+int staticScratch(uint32_t **ptr)
+{
+    int device = 0;
+    HIP_TRY(hipGetDevice(&device));
+    if(device < 0 || device >= STATIC_MAX_DEVICES) { return fail(GENNMI_EUNSUPPORTED, "static scratch: device index out of range"); }
+    std::lock_guard<std::mutex> lock(g_scratchMutex);
+    if(!g_scratchPtr[device]) {
+        uint32_t *p = nullptr;
+        HIP_TRY(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));
+        if(!p) { return fail(GENNMI_EHIP, "static scratch: hipGetSymbolAddress returned a null address"); }
+        g_scratchPtr[device] = p;
+    }
+    *ptr = g_scratchPtr[device];
+    return GENNMI_OK;
+}
+}   // namespace
+
+int gennmi_detail::prepareStaticScratch()
+{
+    uint32_t *unused = nullptr;
+    return staticScratch(&unused);
+}
+
+extern "C" {
+
+int gennmi_max_col_length_static(uint32_t numSrc, uint32_t numTrg, uint32_t rowStride, const uint32_t *rowLength, const uint32_t *ind,
+                                 uint32_t *maxColLengthDev)
+{
+    if(!rowLength || !ind || !maxColLengthDev || rowStride == 0 || numSrc == 0 || numTrg == 0) { return fail(GENNMI_EINVAL, "max_col_length_static: bad arguments"); }
+    if(numTrg > STATIC_COUNTER_MAX) {
+        return fail(GENNMI_EINVAL, "max_col_length_static: " + std::to_string(numTrg) + " postsynaptic neurons exceed the static counter array ("
+                                   + std::to_string(STATIC_COUNTER_MAX) + "); use gennmi_max_col_length");
+    }
+    const size_t total = (size_t)numSrc * rowStride;
+    if((total + BLOCK - 1) / BLOCK > 0x7FFFFFFFull) { return fail(GENNMI_EINVAL, "max_col_length_static: matrix too large for one launch"); }
+    uint32_t *counters = nullptr;
+    { const int rc = staticScratch(&counters); if(rc) { return rc; } }
+    // the array keeps the last call's counts: clear what this call uses (a kernel, not a memset, so that the sequence
+    // stays legal for callers that record it)
+    staticClearKernel<<<dim3((numTrg + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, 0>>>(counters, numTrg, maxColLengthDev);
+    remapCountKernel<<<dim3((unsigned int)((total + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, 0>>>(numSrc, rowStride, rowLength, ind, 0, counters, nullptr, nullptr);
+    staticMaxKernel<<<dim3((numTrg + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, 0>>>(counters, numTrg, maxColLengthDev);
+    HIP_TRY(hipGetLastError());
     return GENNMI_OK;
 }
 
