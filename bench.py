@@ -47,7 +47,10 @@ def build_net(name, steps):
     if name == "dense":
         return configs.dense_layer(steps=steps), "dense layer 8192 Poisson sources (50 Hz) -> 8192 LIF, DENSE individual weights, dt=1ms"
     if name == "izh":
-        return configs.izhikevich_fanout(steps=steps, noise_steps=64), "C3 izhikevich 1e6 neurons fanout 1000 dt=1ms (noise rows cycled)"
+        # the configuration's own noise array: one row of 10^6 values per step for 1 s simulated (4 GB); a run of more
+        # than 1000 steps starts over at its first row
+        return (configs.izhikevich_fanout(steps=steps, noise_steps=min(steps, 1000)),
+                "C3 izhikevich 1e6 neurons fanout 1000 dt=1ms, per-step noise array of min(steps, 1000) rows")
     if name == "izh_small":
         return configs.izhikevich_fanout(n=100_000, fanout=1000, steps=steps, noise_steps=64), "izhikevich 1e5 neurons fanout 1000"
     if name == "stdp":

@@ -315,6 +315,26 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
                 }
                 if(n.getMergedOutSynPreOutputGroups().size() > GENNMI_MAX_PRE_OUTPUT) { unsupported("more than 2 presynaptic outputs into population '" + arch.getName() + "'"); }
 
+                // Parameters reach the device as constants of the descriptors built once, before the first step.  A parameter the
+                // model marks dynamic (setParamDynamic: the reference gives it a DYNAMIC merged-struct field that
+                // setDynamicParamValue rewrites at run time, neuronGroup.h:135, currentSource.h:67, synapseGroup.h:187) would
+                // keep its first value for ever, so such a model is refused rather than run wrongly.
+                for(const auto &g : n.getGroups()) {
+                    for(const auto &p : g.get().getModel()->getParams()) {
+                        if(g.get().isParamDynamic(p.name)) { unsupported("dynamic parameter '" + p.name + "' of population '" + g.get().getName() + "'"); }
+                    }
+                    for(const auto *cs : g.get().getCurrentSources()) {
+                        for(const auto &p : cs->getModel()->getParams()) {
+                            if(cs->isParamDynamic(p.name)) { unsupported("dynamic parameter '" + p.name + "' of current source '" + cs->getName() + "'"); }
+                        }
+                    }
+                    for(const auto *sg : g.get().getFusedPSMInSyn()) {
+                        for(const auto &p : sg->getPSInitialiser().getSnippet()->getParams()) {
+                            if(sg->isPSParamDynamic(p.name)) { unsupported("dynamic postsynaptic-model parameter '" + p.name + "' of projection '" + sg->getName() + "'"); }
+                        }
+                    }
+                }
+
                 // values of one quantity across the groups of this merged group
                 auto perGroup = [&n](auto fn)
                 {
@@ -609,6 +629,12 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                 const auto &arch = s.getArchetype();
                 const auto *wum = arch.getWUInitialiser().getSnippet();
                 const unsigned int wumKind = recogniseWUM(wum, arch.getName());
+                // weight-update parameters become descriptor constants too: dynamic ones are refused (see the neuron groups)
+                for(const auto &g : s.getGroups()) {
+                    for(const auto &p : wum->getParams()) {
+                        if(g.get().isWUParamDynamic(p.name)) { unsupported("dynamic weight-update parameter '" + p.name + "' of projection '" + g.get().getName() + "'"); }
+                    }
+                }
                 const bool srcDelay = arch.getSrcNeuronGroup()->isDelayRequired();
                 const bool plastic = (wumKind == GENNMI_WUM_STDP_TRACE || wumKind == GENNMI_WUM_STDP);
                 if(arch.getBackPropDelaySteps() != 0 || (plastic && (srcDelay || arch.getTrgNeuronGroup()->isDelayRequired()))) {

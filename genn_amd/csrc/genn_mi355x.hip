@@ -42,6 +42,7 @@
 #include "genn_mi355x_synapse_kernels.h"
 #include "genn_mi355x_neuron_kernels.h"
 #include "genn_mi355x_resident_kernels.h"
+#include "genn_mi355x_ordered_kernels.h"
 
 struct gennmi_runner
 {
@@ -73,6 +74,18 @@ struct gennmi_runner
     uint32_t neuronsPerLane = 1;        // 2, 4 or 8: neuronBulkKernel instead of neuronUpdateKernel
     bool sourcesStale = false;          // startSpike / endSpike / spikeTimes of a spike source were written since nextSpikeTime was built
     bool resStale = false;              // connectivity or weights were written since the tables were built
+    bool tablesStale = false;           // rowLength / ind / d of a projection were written since the connectivity-derived tables were built
+    // connectivity-derived tables that are rebuilt when tablesStale: segment boundaries of the tile path ...
+    struct TileTable { size_t pre; uint16_t *off; uint32_t tileSize, numTiles; };
+    std::vector<TileTable> tileTables;
+    std::vector<void*> zeroOwned;       // ... the zero-delay lists of the single-launch step ...
+    // ... and the column views of ordered accumulation (validation mode: every element summed in the CPU backend's order)
+    bool ordered = false;
+    std::vector<OrderedGroupDev> orderedGroups; std::vector<size_t> orderedPre;
+    std::vector<OrderedSourceDev> orderedSources; OrderedSourceDev *dOrderedSources = nullptr; uint32_t orderedSourceBlocks = 0;
+    uint32_t *dOrderedBitmaps = nullptr; size_t orderedBitmapWords = 0;
+    std::vector<void*> orderedOwned;
+    bool scatterNeeded = true;          // some presynaptic group still goes through presynapticUpdateKernel
     // graph
     hipGraphExec_t graphExec = nullptr; unsigned long long graphSteps = 0;
     // timing
@@ -101,15 +114,22 @@ static void noteDeviceWrite(const void *dev, size_t bytes)
             const uintptr_t st = reinterpret_cast<uintptr_t>(n.g.startSpike), en = reinterpret_cast<uintptr_t>(n.g.endSpike);
             if((a < st + perNeuron && st < b) || (a < en + perNeuron && en < b) || (a < reinterpret_cast<uintptr_t>(n.g.spikeTimes) + n.spikeTimesBytes && reinterpret_cast<uintptr_t>(n.g.spikeTimes) < b)) { r->sourcesStale = true; }
         }
-        if(!r->resident || r->resStale) { continue; }
+        if(!r->finalised) { continue; }
         for(const auto &p : r->pre) {
+            if(p.g.matrix != GENNMI_MATRIX_SPARSE) { continue; }
             const size_t entries = (size_t)p.g.numSrcNeurons * p.g.rowStride;
-            const struct { const void *ptr; size_t size; } arrays[] = {
-                {p.g.g, entries * sizeof(float)}, {p.g.ind, entries * sizeof(uint32_t)}, {p.g.d, p.g.d ? entries : 0},
-                {p.g.rowLength, (size_t)p.g.numSrcNeurons * sizeof(uint32_t)}};
+            // connectivity (rowLength, ind, d) feeds the segment boundaries of the tile path, the zero-delay lists of the
+            // single-launch step, the column views of ordered accumulation and the resident plan's segment tables; weights
+            // are copied only into the latter
+            const struct { const void *ptr; size_t size; bool connectivity; } arrays[] = {
+                {p.g.g, entries * sizeof(float), false}, {p.g.ind, entries * sizeof(uint32_t), true}, {p.g.d, p.g.d ? entries : 0, true},
+                {p.g.rowLength, (size_t)p.g.numSrcNeurons * sizeof(uint32_t), true}};
             for(const auto &arr : arrays) {
                 const uintptr_t lo = reinterpret_cast<uintptr_t>(arr.ptr);
-                if(arr.size && a < lo + arr.size && lo < b) { r->resStale = true; }
+                if(arr.ptr && arr.size && a < lo + arr.size && lo < b) {
+                    if(r->resident) { r->resStale = true; }
+                    if(arr.connectivity) { r->tablesStale = true; }
+                }
             }
         }
     }
@@ -282,6 +302,9 @@ int gennmi_runner_destroy(gennmi_runner *r)
     for(hipEvent_t e : r->eventPool) { hipEventDestroy(e); }
     for(hipEvent_t e : r->marks) { if(e) { hipEventDestroy(e); } }
     for(void *q : r->owned) { hipFree(q); }
+    for(void *q : r->zeroOwned) { hipFree(q); }
+    for(void *q : r->orderedOwned) { hipFree(q); }
+    hipFree(r->dOrderedSources); hipFree(r->dOrderedBitmaps);
     hipFree(r->dTile); hipFree(r->dConvTile);
     hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dDense); hipFree(r->dProc); hipFree(r->dAgg); hipFree(r->dError); hipFree(r->dEvents); hipFree(r->dState);
     hipStreamDestroy(r->stream);
@@ -634,6 +657,254 @@ static int launchResident(gennmi_runner *r, unsigned long long timestep, unsigne
     return GENNMI_OK;
 }
 
+// Single-launch step: shadow spike queues and, per population, the list of outgoing synapses whose delay is a multiple of
+// the ring depth (delivered by the neuron update of the spiking neuron).  Called at finalise and again whenever the
+// connectivity has been rewritten; the caller then uploads the descriptor tables.
+static int buildZeroDelayLists(gennmi_runner *r)
+{
+    for(void *q : r->zeroOwned) { hipFree(q); }
+    r->zeroOwned.clear();
+    auto devAlloc = [](std::vector<void*> &owner, void **q, size_t bytes) -> hipError_t {
+        hipError_t e = hipMalloc(q, bytes ? bytes : 4);
+        if(e == hipSuccess) { owner.push_back(*q); e = hipMemset(*q, 0, bytes ? bytes : 4); }
+        return e;
+    };
+    for(auto &n : r->neuron) {
+        if(!n.shadowSpk) {
+            HIP_TRY(devAlloc(r->owned, (void**)&n.shadowSpk, 2 * (size_t)r->batch * n.g.numNeurons * sizeof(uint32_t)));
+            HIP_TRY(devAlloc(r->owned, (void**)&n.shadowCnt, 2 * (size_t)r->batch * sizeof(uint32_t)));
+        }
+        std::vector<PreGroupDev*> outs;
+        for(auto &p : r->pre) { if(p.g.srcSpk == n.g.spk) { outs.push_back(&p); } }
+        if(outs.empty()) { continue; }
+        const uint32_t N = n.g.numNeurons;
+        const dim3 grid((N + BLOCK - 1) / BLOCK);
+        uint32_t *dLen = nullptr;
+        HIP_TRY(devAlloc(r->zeroOwned, (void**)&dLen, (size_t)N * sizeof(uint32_t)));
+        std::vector<std::vector<uint32_t>> len(outs.size(), std::vector<uint32_t>(N));
+        for(size_t o = 0; o < outs.size(); o++) {
+            const auto &q = outs[o]->g;
+            zeroDelayScanKernel<<<grid, dim3(BLOCK), 0, 0>>>(N, q.rowStride, q.rowLength, q.d, q.maxDenDelay, q.ind, q.g, q.denDelay,
+                                                             q.numTrgNeurons, dLen, nullptr, nullptr);
+            HIP_TRY(hipGetLastError());
+            HIP_TRY(hipMemcpy(len[o].data(), dLen, (size_t)N * sizeof(uint32_t), hipMemcpyDeviceToHost));
+        }
+        std::vector<uint32_t> start(N + 1, 0);
+        for(uint32_t i = 0; i < N; i++) {
+            uint64_t sum = start[i];
+            for(size_t o = 0; o < outs.size(); o++) { sum += len[o][i]; }
+            if(sum > 0xFFFFFFFFull) { return fail(GENNMI_EUNSUPPORTED, "runner_finalise: too many zero-delay synapses"); }
+            start[i + 1] = (uint32_t)sum;
+        }
+        uint32_t *dStart = nullptr, *dOffset = nullptr; ZeroDelayEntry *dEntries = nullptr;
+        HIP_TRY(devAlloc(r->zeroOwned, (void**)&dStart, (size_t)(N + 1) * sizeof(uint32_t)));
+        HIP_TRY(hipMemcpy(dStart, start.data(), (size_t)(N + 1) * sizeof(uint32_t), hipMemcpyHostToDevice));
+        HIP_TRY(devAlloc(r->zeroOwned, (void**)&dOffset, (size_t)N * sizeof(uint32_t)));
+        HIP_TRY(devAlloc(r->zeroOwned, (void**)&dEntries, (size_t)std::max(1u, start[N]) * sizeof(ZeroDelayEntry)));
+        std::vector<uint32_t> offset(start.begin(), start.begin() + N);
+        for(size_t o = 0; o < outs.size(); o++) {
+            auto &q = outs[o]->g;
+            HIP_TRY(hipMemcpy(dOffset, offset.data(), (size_t)N * sizeof(uint32_t), hipMemcpyHostToDevice));
+            zeroDelayScanKernel<<<grid, dim3(BLOCK), 0, 0>>>(N, q.rowStride, q.rowLength, q.d, q.maxDenDelay, q.ind, q.g, q.denDelay,
+                                                             q.numTrgNeurons, nullptr, dOffset, dEntries);
+            HIP_TRY(hipGetLastError());
+            HIP_TRY(hipDeviceSynchronize());
+            for(uint32_t i = 0; i < N; i++) { offset[i] += len[o][i]; }
+            outs[o]->skipZeroDelay = 1; outs[o]->shadowSpk = n.shadowSpk; outs[o]->shadowCnt = n.shadowCnt;
+        }
+        n.zeroStart = dStart; n.zeroEntries = dEntries;
+    }
+    return GENNMI_OK;
+}
+
+// Single-launch step: where the zero-delay synapses of the last completed step's spikes have been delivered, keyed by
+// (weight address, batch) — one entry per synapse and batch
+static int pendingZeroDelay(gennmi_runner *r, std::map<std::pair<const float*, uint32_t>, float*> &out)
+{
+    if(r->epoch == 0) { return GENNMI_OK; }
+    const uint32_t parity = (uint32_t)((r->epoch + 1) & 1);         // the queue the coming step's presynaptic update reads
+    for(const auto &n : r->neuron) {
+        if(!n.zeroStart) { continue; }
+        const uint32_t N = n.g.numNeurons;
+        std::vector<uint32_t> start(N + 1);
+        HIP_TRY(hipMemcpy(start.data(), n.zeroStart, (size_t)(N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost));
+        for(uint32_t b = 0; b < r->batch; b++) {
+            uint32_t count = 0;
+            HIP_TRY(hipMemcpy(&count, n.shadowCnt + (size_t)parity * r->batch + b, sizeof(uint32_t), hipMemcpyDeviceToHost));
+            if(count == 0) { continue; }
+            std::vector<uint32_t> spikes(count);
+            HIP_TRY(hipMemcpy(spikes.data(), n.shadowSpk + ((size_t)parity * r->batch + b) * N, (size_t)count * sizeof(uint32_t), hipMemcpyDeviceToHost));
+            for(uint32_t i : spikes) {
+                const uint32_t len = start[i + 1] - start[i];
+                if(len == 0) { continue; }
+                std::vector<ZeroDelayEntry> entries(len);
+                HIP_TRY(hipMemcpy(entries.data(), n.zeroEntries + start[i], (size_t)len * sizeof(ZeroDelayEntry), hipMemcpyDeviceToHost));
+                for(const auto &e : entries) {
+                    const uint32_t slot = (uint32_t)((r->epoch + 1) % e.maxDenDelay);      // the slot the coming step reads
+                    out[{e.weight, b}] = e.ringElem + ((size_t)b * e.maxDenDelay + slot) * e.numTrgNeurons;
+                }
+            }
+        }
+    }
+    return GENNMI_OK;
+}
+
+// Segment boundaries of the tile path for one projection; rows that are not sorted by target are reported through *unsorted
+static int buildTileOffsets(const gennmi_presynaptic_update_group_t &g, uint16_t *dOff, uint32_t tileSize, uint32_t numTiles, uint32_t *unsorted)
+{
+    uint32_t *dFlag = nullptr;
+    HIP_TRY(hipMalloc(&dFlag, sizeof(uint32_t)));
+    HIP_TRY(hipMemset(dFlag, 0, sizeof(uint32_t)));
+    tileOffsetKernel<<<dim3((g.numSrcNeurons + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, 0>>>(
+        g.numSrcNeurons, g.rowStride, g.rowLength, g.ind, tileSize, numTiles, dOff, dFlag);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(unsorted, dFlag, sizeof(uint32_t), hipMemcpyDeviceToHost));
+    HIP_TRY(hipFree(dFlag));
+    return GENNMI_OK;
+}
+
+// Ordered accumulation: a column view of every SPARSE projection it covers (engine-private: the user's own colLength /
+// remap exist for plastic projections only) and one bitmap per distinct spike queue.  Called at finalise and again
+// whenever the connectivity has been rewritten.
+static int buildOrderedViews(gennmi_runner *r)
+{
+    for(void *q : r->orderedOwned) { hipFree(q); }
+    r->orderedOwned.clear();
+    r->orderedGroups.clear(); r->orderedPre.clear(); r->orderedSources.clear();
+    if(r->dOrderedSources) { HIP_TRY(hipFree(r->dOrderedSources)); r->dOrderedSources = nullptr; }
+    if(r->dOrderedBitmaps) { HIP_TRY(hipFree(r->dOrderedBitmaps)); r->dOrderedBitmaps = nullptr; }
+    std::vector<size_t> bitmapOffset;       // of every source, in words
+    size_t words = 0;
+    for(size_t k = 0; k < r->pre.size(); k++) {
+        auto &p = r->pre[k];
+        const auto &g = p.g;
+        const bool covered = g.matrix == GENNMI_MATRIX_SPARSE && (g.wum == GENNMI_WUM_STATIC_PULSE || g.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY
+                                                                  || g.wum == GENNMI_WUM_STDP_TRACE || g.wum == GENNMI_WUM_STDP);
+        p.ordered = covered ? 1u : 0u;
+        if(!covered) { continue; }
+        if(g.maxDenDelay > ORDERED_MAX_SLOT_REGS * WAVE) { return fail(GENNMI_EUNSUPPORTED, "ordered accumulation: dendritic-delay rings of more than 256 slots"); }
+        uint32_t maxLen = 0;
+        { const int rc = gennmi_max_col_length(g.numSrcNeurons, g.numTrgNeurons, g.rowStride, g.rowLength, g.ind, &maxLen); if(rc) { return rc; } }
+        OrderedGroupDev o{};
+        o.g = g;
+        o.colStride = std::max(1u, maxLen);
+        uint32_t *colLength = nullptr, *remap = nullptr;
+        HIP_TRY(hipMalloc(&colLength, (size_t)g.numTrgNeurons * sizeof(uint32_t)));
+        r->orderedOwned.push_back(colLength);
+        HIP_TRY(hipMalloc(&remap, (size_t)g.numTrgNeurons * o.colStride * sizeof(uint32_t)));
+        r->orderedOwned.push_back(remap);
+        { const int rc = gennmi_build_remap(g.numSrcNeurons, g.numTrgNeurons, g.rowStride, o.colStride, g.rowLength, g.ind, colLength, remap); if(rc) { return rc; } }
+        o.colLength = colLength; o.remap = remap;
+        // the queue this projection reads: shared with every other projection that reads the same slot of the same queue
+        size_t src = r->orderedSources.size();
+        for(size_t q = 0; q < r->orderedSources.size(); q++) {
+            const auto &c = r->orderedSources[q];
+            if(c.srcSpk == g.srcSpk && c.srcSpkCnt == g.srcSpkCnt && c.numSrcDelaySlots == g.numSrcDelaySlots && c.axonalDelaySteps == g.axonalDelaySteps) { src = q; }
+        }
+        if(src == r->orderedSources.size()) {
+            OrderedSourceDev c{};
+            c.srcSpk = g.srcSpk; c.srcSpkCnt = g.srcSpkCnt; c.numSrcNeurons = g.numSrcNeurons; c.words = (g.numSrcNeurons + 31) / 32;
+            c.numSrcDelaySlots = g.numSrcDelaySlots; c.axonalDelaySteps = g.axonalDelaySteps;
+            c.numBlocks = std::max(1u, std::min(64u, (g.numSrcNeurons + 16 * BLOCK - 1) / (16 * BLOCK)));
+            bitmapOffset.push_back(words);
+            words += (size_t)c.words * r->batch;
+            r->orderedSources.push_back(c);
+        }
+        o.words = r->orderedSources[src].words;
+        o.bitmap = reinterpret_cast<const uint32_t*>(bitmapOffset[src]);        // offset for now, pointer below
+        r->orderedGroups.push_back(o);
+        r->orderedPre.push_back(k);
+    }
+    r->scatterNeeded = false;
+    for(const auto &p : r->pre) { r->scatterNeeded = r->scatterNeeded || !p.ordered; }
+    if(r->orderedGroups.empty()) { return GENNMI_OK; }
+    HIP_TRY(hipMalloc(&r->dOrderedBitmaps, words * sizeof(uint32_t)));
+    HIP_TRY(hipMemset(r->dOrderedBitmaps, 0, words * sizeof(uint32_t)));
+    r->orderedBitmapWords = words;
+    for(auto &o : r->orderedGroups) { o.bitmap = r->dOrderedBitmaps + reinterpret_cast<uintptr_t>(o.bitmap); }
+    std::vector<OrderedSourceDev> table;
+    uint32_t block = 0;
+    for(size_t q = 0; q < r->orderedSources.size(); q++) {
+        auto &c = r->orderedSources[q];
+        c.bitmap = r->dOrderedBitmaps + bitmapOffset[q];
+        c.startBlock = block;
+        block += c.numBlocks;
+        for(uint32_t b = 0; b < c.numBlocks; b++) { table.push_back(c); }
+    }
+    r->orderedSourceBlocks = block;
+    HIP_TRY(hipMalloc(&r->dOrderedSources, table.size() * sizeof(OrderedSourceDev)));
+    HIP_TRY(hipMemcpy(r->dOrderedSources, table.data(), table.size() * sizeof(OrderedSourceDev), hipMemcpyHostToDevice));
+    return GENNMI_OK;
+}
+
+// Connectivity-derived tables follow the connectivity: when rowLength / ind / d of a projection have been written since
+// the tables were built (a connectivity push after load), they are rebuilt before the next launch.
+static int refreshTables(gennmi_runner *r)
+{
+    bool stale;
+    {
+        std::lock_guard<std::mutex> lock(g_runnersMutex);
+        stale = r->tablesStale;
+        r->tablesStale = false;
+    }
+    if(!stale) { return GENNMI_OK; }
+    HIP_TRY(hipStreamSynchronize(r->stream));
+    for(const auto &t : r->tileTables) {
+        uint32_t unsorted = 0;
+        { const int rc = buildTileOffsets(r->pre[t.pre].g, t.off, t.tileSize, t.numTiles, &unsorted); if(rc) { return rc; } }
+        if(unsorted) {
+            return fail(GENNMI_ESTATE, "connectivity written after load leaves the rows of a projection no longer sorted by target, which its launch plan relies on; "
+                                       "sort the rows or set GENNMI_TILE_FLOATS=0 before the runner is finalised");
+        }
+    }
+    if(r->fusedStep) {
+        // The spikes of the last completed step have already had their zero-delay synapses delivered — by the old lists —
+        // into the slot that is read next, and the coming step will skip every synapse that is zero-delay NOW.  Synapses of
+        // those spikes that changed sides are put right here: newly zero-delay ones are added to that slot (exact), ones that
+        // no longer are zero-delay are taken out again (a subtraction: the slot's sum is then right to rounding) and
+        // delivered by the coming step like any other.
+        std::map<std::pair<const float*, uint32_t>, float*> before, after;
+        { const int rc = pendingZeroDelay(r, before); if(rc) { return rc; } }
+        { const int rc = buildZeroDelayLists(r); if(rc) { return rc; } }
+        { const int rc = pendingZeroDelay(r, after); if(rc) { return rc; } }
+        std::vector<ZeroDelayCorrection> fix;
+        for(const auto &e : after) { if(!before.count(e.first)) { fix.push_back({e.second, e.first.first, 1.0f, 0u}); } }
+        for(const auto &e : before) { if(!after.count(e.first)) { fix.push_back({e.second, e.first.first, -1.0f, 0u}); } }
+        if(!fix.empty()) {
+            ZeroDelayCorrection *dFix = nullptr;
+            HIP_TRY(hipMalloc(&dFix, fix.size() * sizeof(ZeroDelayCorrection)));
+            HIP_TRY(hipMemcpy(dFix, fix.data(), fix.size() * sizeof(ZeroDelayCorrection), hipMemcpyHostToDevice));
+            zeroDelayCorrectionKernel<<<dim3((unsigned int)((fix.size() + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, 0>>>(dFix, (uint32_t)fix.size());
+            HIP_TRY(hipGetLastError());
+            HIP_TRY(hipDeviceSynchronize());
+            HIP_TRY(hipFree(dFix));
+        }
+        // the per-block descriptor tables carry the lists' addresses: same layout, new contents
+        std::vector<NeuronGroupDev> neuronTable;
+        for(const auto &g : r->neuron) { for(uint32_t b = 0; b < g.numBlocks; b++) { neuronTable.push_back(g); } }
+        HIP_TRY(hipMemcpy(r->dNeuron, neuronTable.data(), neuronTable.size() * sizeof(NeuronGroupDev), hipMemcpyHostToDevice));
+        std::vector<PreGroupDev> preTable;
+        for(const auto &g : r->pre) { for(uint32_t b = 0; b < g.numBlocks; b++) { preTable.push_back(g); } }
+        HIP_TRY(hipMemcpy(r->dPre, preTable.data(), preTable.size() * sizeof(PreGroupDev), hipMemcpyHostToDevice));
+    }
+    if(r->ordered) {
+        // the gather kernels receive their column views by value, so a captured step graph holds the addresses of the views
+        // just freed: it is captured again on the next replay
+        if(r->graphExec) { HIP_TRY(hipGraphExecDestroy(r->graphExec)); r->graphExec = nullptr; r->graphSteps = 0; }
+        const int rc = buildOrderedViews(r);
+        if(rc) { return rc; }
+    }
+    return GENNMI_OK;
+}
+
+int gennmi_runner_set_ordered(gennmi_runner *r, int enabled)
+{
+    if(!r) { return fail(GENNMI_EINVAL, "runner_set_ordered: null runner"); }
+    if(r->finalised) { return fail(GENNMI_ESTATE, "runner_set_ordered: the accumulation mode is fixed when the runner is finalised"); }
+    r->ordered = (enabled != 0);
+    return GENNMI_OK;
+}
+
 int gennmi_runner_finalise(gennmi_runner *r)
 {
     if(!r) { return fail(GENNMI_EINVAL, "runner_finalise: null runner"); }
@@ -645,6 +916,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
     HIP_TRY(hipGetDeviceProperties(&prop, device));
     const uint32_t numCU = (uint32_t)prop.multiProcessorCount;
 
+    if(const char *envOrdered = getenv("GENNMI_ORDERED")) { r->ordered = r->ordered || atoi(envOrdered) != 0; }
     // a projection's view of its source's delay slots must be the source's own
     for(const auto &p : r->pre) {
         for(const auto &n : r->neuron) {
@@ -775,7 +1047,8 @@ int gennmi_runner_finalise(gennmi_runner *r)
     // ---- tile path for delay-free SPARSE projections (static or trace-STDP weights) whose rows are sorted by target
     {
         const char *envTile = getenv("GENNMI_TILE_FLOATS");
-        const uint32_t tileFloats = envTile ? (uint32_t)std::max(0, atoi(envTile)) : 16384u;
+        // (ordered accumulation gathers SPARSE projections itself: no tile paths then)
+        const uint32_t tileFloats = r->ordered ? 0u : envTile ? (uint32_t)std::max(0, atoi(envTile)) : 16384u;
         const char *envThreads = getenv("GENNMI_TILE_THREADS");
         r->tileThreads = envThreads ? (uint32_t)std::min(1024, std::max(64, atoi(envThreads))) : (tileFloats > 16384 ? 1024u : (tileFloats > 8192 ? 512u : (uint32_t)BLOCK));
         std::vector<TileGroupDev> tiles, tileGroups;
@@ -813,19 +1086,14 @@ int gennmi_runner_finalise(gennmi_runner *r)
                || (p.g.wum != GENNMI_WUM_STATIC_PULSE && p.g.wum != GENNMI_WUM_STDP_TRACE && p.g.wum != GENNMI_WUM_STDP)) { continue; }
             const uint32_t tileSize = std::min(tileFloats, p.g.numTrgNeurons);
             const uint32_t numTiles = (p.g.numTrgNeurons + tileSize - 1) / tileSize;
-            uint16_t *dOff = nullptr; uint32_t *dFlag = nullptr;
+            uint16_t *dOff = nullptr;
             HIP_TRY(hipMalloc(&dOff, (size_t)p.g.numSrcNeurons * (numTiles + 1) * sizeof(uint16_t)));
             r->owned.push_back(dOff);
-            HIP_TRY(hipMalloc(&dFlag, sizeof(uint32_t)));
-            HIP_TRY(hipMemset(dFlag, 0, sizeof(uint32_t)));
-            tileOffsetKernel<<<dim3((p.g.numSrcNeurons + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, 0>>>(
-                p.g.numSrcNeurons, p.g.rowStride, p.g.rowLength, p.g.ind, tileSize, numTiles, dOff, dFlag);
-            HIP_TRY(hipGetLastError());
             uint32_t unsorted = 0;
-            HIP_TRY(hipMemcpy(&unsorted, dFlag, sizeof(uint32_t), hipMemcpyDeviceToHost));
-            HIP_TRY(hipFree(dFlag));
+            { const int rc = buildTileOffsets(p.g, dOff, tileSize, numTiles, &unsorted); if(rc) { return rc; } }
             if(unsorted) { continue; }          // rows not sorted by target: the scatter kernel handles every step
             p.tileThreshold = std::max(1u, p.g.numTrgNeurons);
+            r->tileTables.push_back({(size_t)(&p - r->pre.data()), dOff, tileSize, numTiles});
             const uint32_t avgSeg = std::max(1u, p.g.rowStride / numTiles);
             TileGroupDev t{};
             t.g = p.g; t.tileOff = dOff; t.numTiles = numTiles; t.tileSize = tileSize;
@@ -875,7 +1143,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
     bool anyEvents = false;
     for(const auto &n : r->neuron) { anyEvents = anyEvents || n.g.numSpkEvent != 0; }
     const char *envFused = getenv("GENNMI_FUSED_STEP");
-    bool eligible = !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty() && r->dense.empty() && r->proc.empty() && !anyEvents && r->neuronsPerLane == 1;
+    bool eligible = !r->ordered && !(envFused && atoi(envFused) == 0) && !r->pre.empty() && r->post.empty() && r->dense.empty() && r->proc.empty() && !anyEvents && r->neuronsPerLane == 1;
     for(const auto &p : r->pre) {
         eligible = eligible && p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY
                    && p.g.maxDenDelay >= 2 && p.g.numSrcDelaySlots <= 1;
@@ -884,54 +1152,8 @@ int gennmi_runner_finalise(gennmi_runner *r)
         eligible = eligible && found;
     }
     if(eligible) {
-        auto devAlloc = [r](void **q, size_t bytes) -> hipError_t {
-            hipError_t e = hipMalloc(q, bytes ? bytes : 4);
-            if(e == hipSuccess) { r->owned.push_back(*q); e = hipMemset(*q, 0, bytes ? bytes : 4); }
-            return e;
-        };
-        for(auto &n : r->neuron) {
-            HIP_TRY(devAlloc((void**)&n.shadowSpk, 2 * (size_t)r->batch * n.g.numNeurons * sizeof(uint32_t)));
-            HIP_TRY(devAlloc((void**)&n.shadowCnt, 2 * (size_t)r->batch * sizeof(uint32_t)));
-            std::vector<PreGroupDev*> outs;
-            for(auto &p : r->pre) { if(p.g.srcSpk == n.g.spk) { outs.push_back(&p); } }
-            if(outs.empty()) { continue; }
-            const uint32_t N = n.g.numNeurons;
-            const dim3 grid((N + BLOCK - 1) / BLOCK);
-            uint32_t *dLen = nullptr;
-            HIP_TRY(devAlloc((void**)&dLen, (size_t)N * sizeof(uint32_t)));
-            std::vector<std::vector<uint32_t>> len(outs.size(), std::vector<uint32_t>(N));
-            for(size_t o = 0; o < outs.size(); o++) {
-                const auto &q = outs[o]->g;
-                zeroDelayScanKernel<<<grid, dim3(BLOCK), 0, 0>>>(N, q.rowStride, q.rowLength, q.d, q.maxDenDelay, q.ind, q.g, q.denDelay,
-                                                                 q.numTrgNeurons, dLen, nullptr, nullptr);
-                HIP_TRY(hipGetLastError());
-                HIP_TRY(hipMemcpy(len[o].data(), dLen, (size_t)N * sizeof(uint32_t), hipMemcpyDeviceToHost));
-            }
-            std::vector<uint32_t> start(N + 1, 0);
-            for(uint32_t i = 0; i < N; i++) {
-                uint64_t sum = start[i];
-                for(size_t o = 0; o < outs.size(); o++) { sum += len[o][i]; }
-                if(sum > 0xFFFFFFFFull) { return fail(GENNMI_EUNSUPPORTED, "runner_finalise: too many zero-delay synapses"); }
-                start[i + 1] = (uint32_t)sum;
-            }
-            uint32_t *dStart = nullptr, *dOffset = nullptr; ZeroDelayEntry *dEntries = nullptr;
-            HIP_TRY(devAlloc((void**)&dStart, (size_t)(N + 1) * sizeof(uint32_t)));
-            HIP_TRY(hipMemcpy(dStart, start.data(), (size_t)(N + 1) * sizeof(uint32_t), hipMemcpyHostToDevice));
-            HIP_TRY(devAlloc((void**)&dOffset, (size_t)N * sizeof(uint32_t)));
-            HIP_TRY(devAlloc((void**)&dEntries, (size_t)std::max(1u, start[N]) * sizeof(ZeroDelayEntry)));
-            std::vector<uint32_t> offset(start.begin(), start.begin() + N);
-            for(size_t o = 0; o < outs.size(); o++) {
-                auto &q = outs[o]->g;
-                HIP_TRY(hipMemcpy(dOffset, offset.data(), (size_t)N * sizeof(uint32_t), hipMemcpyHostToDevice));
-                zeroDelayScanKernel<<<grid, dim3(BLOCK), 0, 0>>>(N, q.rowStride, q.rowLength, q.d, q.maxDenDelay, q.ind, q.g, q.denDelay,
-                                                                 q.numTrgNeurons, nullptr, dOffset, dEntries);
-                HIP_TRY(hipGetLastError());
-                HIP_TRY(hipDeviceSynchronize());
-                for(uint32_t i = 0; i < N; i++) { offset[i] += len[o][i]; }
-                outs[o]->skipZeroDelay = 1; outs[o]->shadowSpk = n.shadowSpk; outs[o]->shadowCnt = n.shadowCnt;
-            }
-            n.zeroStart = dStart; n.zeroEntries = dEntries;
-        }
+        const int rc = buildZeroDelayLists(r);
+        if(rc) { return rc; }
         r->fusedStep = true;
     }
     // ---- dense-activity path of learnPost: the neuron update of the target population keeps a bitmap of the step's
@@ -978,6 +1200,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
         HIP_TRY(hipMemset(area, 0, count * sizeof(unsigned long long)));
         for(auto &n : r->neuron) { n.aggEvent = area; }
     }
+    if(r->ordered) { const int rc = buildOrderedViews(r); if(rc) { return rc; } }
     HIP_TRY(uploadPerBlock(r->neuron, r->neuronBlocks, &r->dNeuron));
     HIP_TRY(uploadPerBlock(r->pre, r->preBlocks, &r->dPre));
     HIP_TRY(uploadPerBlock(r->post, r->postBlocks, &r->dPost));
@@ -986,7 +1209,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
     const size_t aggCount = 2 * (size_t)r->neuronBlocks * r->batch;       // per-block counts, then per-group totals
     HIP_TRY(hipMalloc(&r->dAgg, aggCount * sizeof(unsigned long long)));
     HIP_TRY(hipMemset(r->dAgg, 0, aggCount * sizeof(unsigned long long)));
-    { const int rc = setupResident(r, numCU); if(rc) { return rc; } }
+    if(!r->ordered) { const int rc = setupResident(r, numCU); if(rc) { return rc; } }
     if(const char *envSpin = getenv("GENNMI_SPIN_LIMIT")) {
         const uint32_t limit = (uint32_t)std::max(0ll, atoll(envSpin));
         HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(c_spinLimit), &limit, sizeof(limit)));
@@ -1063,7 +1286,16 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
         if(r->procBlocks) {
             presynapticProceduralKernel<<<dim3(r->procBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dProc, r->dEvents);
         }
-        if(r->preBlocks) {
+        if(r->ordered && !r->orderedGroups.empty()) {
+            // the step's spikes as bitmaps, then one gather per projection, in push order: projections that share a
+            // target add to it one after another, as the CPU backend's loop over its synapse groups does
+            orderedClearKernel<<<dim3((unsigned int)((r->orderedBitmapWords + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, r->stream>>>(r->dOrderedBitmaps, r->orderedBitmapWords);
+            orderedBitmapKernel<<<dim3(r->orderedSourceBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dOrderedSources, a, r->dt);
+            for(const auto &o : r->orderedGroups) {
+                presynapticOrderedKernel<<<dim3((o.g.numTrgNeurons + (BLOCK / WAVE) - 1) / (BLOCK / WAVE), r->batch), dim3(BLOCK), 0, r->stream>>>(o, a, r->dt, r->dEvents);
+            }
+        }
+        if(r->preBlocks && r->scatterNeeded) {
             presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dPre, a, r->dt, r->dEvents);
         }
         if(r->denseBlocks) {
@@ -1120,6 +1352,7 @@ static int launchNeurons(gennmi_runner *r, const StepArgs &a, bool timed)
 int gennmi_update_synapses(gennmi_runner *r, float t)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "update_synapses: runner not finalised"); }
+    { const int rc = refreshTables(r); if(rc) { return rc; } }
     StepArgs a{};
     a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = 0;
     const int rc = launchSynapses(r, a, r->timing);
@@ -1154,6 +1387,7 @@ int gennmi_step(gennmi_runner *r, float t, uint32_t recordingTimestep)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "step: runner not finalised"); }
     { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
+    { const int rc = refreshTables(r); if(rc) { return rc; } }
     if(r->fusedStep) {
         StepArgs a{};
         a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recordingTimestep;
@@ -1177,6 +1411,7 @@ int gennmi_run_steps(gennmi_runner *r, unsigned long long timestep, unsigned lon
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "run_steps: runner not finalised"); }
     { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
+    { const int rc = refreshTables(r); if(rc) { return rc; } }
     constexpr unsigned long long CHUNK = 100;
     const StepState hs{timestep, r->epoch, numRecordingTimesteps};
     HIP_TRY(hipMemcpyAsync(r->dState, &hs, sizeof(hs), hipMemcpyHostToDevice, r->stream));
@@ -1287,7 +1522,7 @@ int gennmi_runner_get_info(gennmi_runner *r, uint32_t info[4])
 {
     if(!r || !info) { return fail(GENNMI_EINVAL, "runner_get_info: null argument"); }
     if(!r->finalised) { return fail(GENNMI_ESTATE, "runner_get_info: runner not finalised"); }
-    info[0] = (r->fusedStep ? 1u : 0u) | (r->resident ? 2u : 0u) | (r->neuronsPerLane > 1 ? 4u : 0u); info[1] = r->neuronBlocks; info[2] = r->preBlocks; info[3] = r->postBlocks;
+    info[0] = (r->fusedStep ? 1u : 0u) | (r->resident ? 2u : 0u) | (r->neuronsPerLane > 1 ? 4u : 0u) | (r->ordered ? 8u : 0u); info[1] = r->neuronBlocks; info[2] = r->preBlocks; info[3] = r->postBlocks;
     return GENNMI_OK;
 }
 

@@ -110,7 +110,8 @@ struct PreGroupDev
     int32_t convBH, convBW;
     uint32_t skipZeroDelay;             // synapses with d % D == 0 are delivered by the neuron update instead
     uint32_t tileThreshold;             // != 0: leave the step to the tile kernel when numSpikes*workPerSpike reaches it
-    uint32_t workPerSpike, pad2_;       // rowStride (SPARSE) or kh*kw*oc (Toeplitz)
+    uint32_t workPerSpike;              // rowStride (SPARSE) or kh*kw*oc (Toeplitz)
+    uint32_t ordered;                   // != 0: the projection is gathered by presynapticOrderedKernel, the scatter kernel leaves it alone
     const uint32_t *shadowSpk;          // the source population's shadow queue (read instead of srcSpk when set)
     const uint32_t *shadowCnt;
 };

@@ -638,6 +638,14 @@ __global__ void advanceStepKernel(StepState *state, unsigned long long steps)
 }
 
 // four floats per lane; dwordx4 when both pointers are 16-byte aligned (hipMalloc'd arrays are), else scalar
+// early deliveries of zero-delay synapses that have to be added or taken back after the connectivity was rewritten
+struct ZeroDelayCorrection { float *target; const float *weight; float sign; uint32_t pad_; };
+__global__ void zeroDelayCorrectionKernel(const ZeroDelayCorrection *fix, uint32_t count)
+{
+    const uint32_t k = blockIdx.x * blockDim.x + threadIdx.x;
+    if(k < count) { atomicAddF32(asGlobal(fix[k].target), fix[k].sign * fix[k].weight[0]); }
+}
+
 __global__ void copyKernel(float *dst, const float *src, size_t n)
 {
     const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;

@@ -18,6 +18,7 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
                                                 unsigned long long *eventCounter)
 {
     const gennmi_presynaptic_update_group_t &g = G.g;
+    if(G.ordered) { return; }
     const uint32_t batch = blockIdx.y;
     const uint32_t W = G.lanesPerSpike;
     const uint32_t localBlock = blockInKernel - G.startBlock;

@@ -368,6 +368,9 @@ class GeNNModel:
         self.dt = float(dt)
         self.fuse_postsynaptic_models = False
         self.timing_enabled = False
+        # validation mode: synaptic input is summed per postsynaptic neuron in the order of the reference's CPU backend
+        # (no atomics; bit-identical accumulators, slow).  Read when the model is loaded.
+        self.ordered_accumulation = False
         self.neuron_populations = {}
         self.synapse_populations = {}
         self.current_sources = {}
@@ -641,6 +644,8 @@ class GeNNModel:
 
         self._initialize_sparse()
         self._push_merged_groups()
+        if self.ordered_accumulation:
+            _abi.check(lib.gennmi_runner_set_ordered(self._runner, 1))
         _abi.check(lib.gennmi_runner_finalise(self._runner))
         if self.timing_enabled:
             _abi.check(lib.gennmi_runner_set_timing(self._runner, 1))
@@ -807,7 +812,11 @@ class GeNNModel:
                 _abi.check(lib.gennmi_push_neuron_update_group(self._runner, C.byref(d), None))
 
         # presynaptic / postsynaptic update groups; merged by weight-update code and matrix type
+        # (descriptors are pushed in the order the projections were added to the model, whatever their merged group: projections
+        # that share a target are then added to it in that order under ordered accumulation, as the oracle's loop does)
         syn_merged = {}
+        creation = {id(s): k for k, s in enumerate(self.synapse_populations.values())}
+        pushes = []
         for s in self.synapse_populations.values():
             syn_merged.setdefault((s.matrix_type, s.wu.snippet, self._den_delay(s) > 0), []).append(s)
         for members in syn_merged.values():
@@ -888,7 +897,7 @@ class GeNNModel:
                 if additive:
                     d.trgST, d.tauMinus = s.trg.vars["sT"].ptr, rounded["tauMinus"][k]
                     d.aMinus, d.wMin, d.wMax = rounded["Aminus"][k], rounded["Wmin"][k], rounded["Wmax"][k]
-                _abi.check(lib.gennmi_push_presynaptic_update_group(self._runner, C.byref(d), None))
+                pushes.append((creation[id(s)], 0, d))
                 if additive:
                     q = _abi.PostsynapticUpdateGroup()
                     q.numSrcNeurons, q.numTrgNeurons = s.src.num_neurons, s.trg.num_neurons
@@ -898,7 +907,7 @@ class GeNNModel:
                     q.srcST, q.tauPlus = s.src.vars["sT"].ptr, rounded["tauPlus"][k]
                     q.rowLength, q.ind = s.vars["rowLength"].ptr, s.vars["ind"].ptr
                     q.aPlus, q.wMin, q.wMax = rounded["Aplus"][k], rounded["Wmin"][k], rounded["Wmax"][k]
-                    _abi.check(lib.gennmi_push_postsynaptic_update_group(self._runner, C.byref(q), None))
+                    pushes.append((creation[id(s)], 1, q))
                 if stdp:
                     q = _abi.PostsynapticUpdateGroup()
                     q.numSrcNeurons, q.numTrgNeurons = s.src.num_neurons, s.trg.num_neurons
@@ -908,7 +917,12 @@ class GeNNModel:
                     q.srcST, q.preTrace = s.src.vars["sT"].ptr, s.vars["preTrace"].ptr
                     q.rowLength, q.ind = s.vars["rowLength"].ptr, s.vars["ind"].ptr
                     q.aPlus, q.wMin, q.wMax = rounded["aPlus"][k], rounded["wMin"][k], rounded["wMax"][k]
-                    _abi.check(lib.gennmi_push_postsynaptic_update_group(self._runner, C.byref(q), None))
+                    pushes.append((creation[id(s)], 1, q))
+        for _, post, desc in sorted(pushes, key=lambda e: (e[0], e[1])):
+            if post:
+                _abi.check(lib.gennmi_push_postsynaptic_update_group(self._runner, C.byref(desc), None))
+            else:
+                _abi.check(lib.gennmi_push_presynaptic_update_group(self._runner, C.byref(desc), None))
 
     # ------------------------------------------------------------------ stepping
     @property
@@ -981,7 +995,7 @@ class GeNNModel:
     def runner_info(self):
         info = (C.c_uint32 * 4)()
         _abi.check(_abi.load().gennmi_runner_get_info(self._runner, C.byref(info)))
-        return {"single_launch_step": bool(info[0] & 1), "resident_plan": bool(info[0] & 2), "bulk_neuron_kernel": bool(info[0] & 4), "neuron_blocks": info[1], "presyn_blocks": info[2], "postsyn_blocks": info[3]}
+        return {"single_launch_step": bool(info[0] & 1), "resident_plan": bool(info[0] & 2), "bulk_neuron_kernel": bool(info[0] & 4), "ordered_accumulation": bool(info[0] & 8), "neuron_blocks": info[1], "presyn_blocks": info[2], "postsyn_blocks": info[3]}
 
     def set_timing(self, enabled):
         _abi.check(_abi.load().gennmi_runner_set_timing(self._runner, int(bool(enabled))))
@@ -997,9 +1011,10 @@ class GeNNModel:
 
 
 # --------------------------------------------------------------------------------------------
-def model_from_net(net, batch_size=1, record=True, span=None, device=0):
+def model_from_net(net, batch_size=1, record=True, span=None, device=0, ordered=False):
     """Build a GeNNModel from a :class:`genn_amd.netspec.Net` (arrays are loaded, never generated here)."""
     m = GeNNModel("float", net.name, batch_size=batch_size, dt=net.dt, device=device)
+    m.ordered_accumulation = bool(ordered)
     m.fuse_postsynaptic_models = net.fuse_psm
     pops = {}
     for p in net.pops:

@@ -268,6 +268,16 @@ int gennmi_push_neuron_update_group(gennmi_runner *runner, const gennmi_neuron_u
 int gennmi_push_presynaptic_update_group(gennmi_runner *runner, const gennmi_presynaptic_update_group_t *group, uint32_t *idx);
 int gennmi_push_postsynaptic_update_group(gennmi_runner *runner, const gennmi_postsynaptic_update_group_t *group, uint32_t *idx);
 
+/* Ordered accumulation, a validation mode (no counterpart in the reference's GPU backends, whose sums are in atomic
+ * order like this library's default): every SPARSE projection with StaticPulse, StaticPulseDendriticDelay or an STDP rule is
+ * gathered per postsynaptic neuron through a column view of its matrix, spikes in queue order and synapses in ascending
+ * index, projections one after another in push order — the order of the SingleThreadedCPU backend's loops
+ * (src/genn/backends/single_threaded_cpu/backend.cc:1884-1929) — so outPost, the dendritic-delay rings and everything
+ * downstream are bit-identical to that backend's, not merely within reassociation error.  No atomics, no tile,
+ * single-launch or resident plan; it reads every column every step, so it is slow.  Call before gennmi_runner_finalise;
+ * GENNMI_ORDERED=1 in the environment selects it for every runner.  Bit 3 of info[0] (gennmi_runner_get_info) reports it. */
+int gennmi_runner_set_ordered(gennmi_runner *runner, int enabled);
+
 /* Validates descriptors against the kernels' assumptions, uploads the descriptor tables, fixes
  * the launch geometry.  Corresponds to the end of Runtime::allocate (runtime.cc:497-661). */
 int gennmi_runner_finalise(gennmi_runner *runner);

@@ -159,10 +159,14 @@ int main(int argc, char *argv[])
         const std::string in = argv[1], work = argv[2], out = argv[3];
         bool generateOnly = false;
         std::string userCxxFlags;
+        std::vector<std::string> dynamicParams;
         for(int a = 4; a < argc; a++) {
             const std::string opt = argv[a];
             if(opt == "--generate-only") { generateOnly = true; }
             else if(opt.rfind("--cxxflags=", 0) == 0) { userCxxFlags = opt.substr(11); }      // e.g. -O3: same results as the default build, faster
+            // --dynamic=neuron:<population>.<param> | cs:<source>.<param> | wu:<projection>.<param> | ps:<projection>.<param>: marks a
+            // parameter dynamic (setParamDynamic and friends), as a model that calls setDynamicParamValue at run time would
+            else if(opt.rfind("--dynamic=", 0) == 0) { dynamicParams.push_back(opt.substr(10)); }
             else { std::cerr << "unknown option " << opt << std::endl; return 1; }
         }
 
@@ -324,6 +328,17 @@ int main(int argc, char *argv[])
             if(s.axonalDelay) s.sg->setAxonalDelaySteps(s.axonalDelay);
             if(s.hintPre) s.sg->setParallelismHint(SynapseGroup::ParallelismHint::PRESYNAPTIC);
             if(s.tps > 1) s.sg->setNumThreadsPerSpike(s.tps);
+        }
+        for(const auto &spec : dynamicParams) {
+            const size_t colon = spec.find(':'), dot = spec.rfind('.');
+            if(colon == std::string::npos || dot == std::string::npos || dot < colon) { throw std::runtime_error("--dynamic=" + spec); }
+            const std::string kind = spec.substr(0, colon), group = spec.substr(colon + 1, dot - colon - 1), param = spec.substr(dot + 1);
+            bool found = false;
+            if(kind == "neuron") { for(auto &p : pops) { if(p.name == group) { p.ng->setParamDynamic(param); found = true; } } }
+            else if(kind == "cs") { for(auto &c : css) { if(c.name == group) { c.cs->setParamDynamic(param); found = true; } } }
+            else if(kind == "wu") { for(auto &q : syns) { if(q.name == group) { q.sg->setWUParamDynamic(param); found = true; } } }
+            else if(kind == "ps") { for(auto &q : syns) { if(q.name == group) { q.sg->setPSParamDynamic(param); found = true; } } }
+            if(!found) { throw std::runtime_error("--dynamic=" + spec + ": no such group"); }
         }
         model.finalise();
 

@@ -121,3 +121,24 @@ def test_poisson_sources_generate():
         assert "gennrand" not in code and "__global__" not in code
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+
+
+@pytest.mark.parametrize("dynamic, case", [("neuron:E.Ioffset", "va_small"), ("ps:EE.tau", "va_small"), ("cs:23E_dc.amp", "potjans_small"),
+                                           ("wu:EE.aPlus", "stdp_small")])
+def test_dynamic_parameters_are_refused(dynamic, case):
+    """Parameters are baked into the descriptors built before the first step, so a model that marks one dynamic
+    (setParamDynamic; the reference gives it a DYNAMIC merged-struct field, neuronGroup.h:135, currentSource.h:67,
+    synapseGroup.h:187-190) must be refused at generation time instead of running with the value frozen."""
+    net, snap = CASES[case]()
+    net.snap = snap
+    tmp = tempfile.mkdtemp(prefix="adapter_dyn_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(net, spec)
+        res = subprocess.run([DRIVER, spec, work, out, "--generate-only", "--dynamic=" + dynamic], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        assert res.returncode != 0
+        assert "dynamic" in res.stdout and dynamic.split(".")[-1] in res.stdout and "not among the models" in res.stdout, res.stdout[-2000:]
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)

@@ -111,7 +111,7 @@ def test_izhikevich_full_size_first_100ms():
     within 1e-5 of the array's peak; the engine's sums are then copied into the oracle, and from those identical
     inputs the neuron update must produce identical spike queues and V, U within 1e-5 (then copied likewise).  Every
     step of the full-size run is checked this way, and the event counters must agree exactly at the end."""
-    net = configs.izhikevich_fanout(steps=100, noise_steps=64)
+    net = configs.izhikevich_fanout(steps=100)            # one row of the noise array per step, as the configuration states
     n = net.pops[0].n
     assert n == 1_000_000 and int(net.syns[0].row_length.sum()) == 1_000_000_000
     model = model_from_net(net)
@@ -146,6 +146,33 @@ def test_izhikevich_full_size_first_100ms():
             w[:] = g
     assert dense_steps >= 10 and sparse_steps >= 10, (dense_steps, sparse_steps)
     assert model.synaptic_event_count == oracle.events() == events
+    model.unload()
+
+
+def test_izhikevich_full_size_free_run_ordered():
+    """The same 10^6-neuron, 10^9-synapse network FREE-RUNNING for its first 100 ms under ordered accumulation (every input
+    sum in the CPU backend's order, no atomics): the raster of all 100 steps, V, U and the input sums must be identical
+    to the oracle's bit for bit.  In the default mode the free-running rasters part at the first population burst (step 66:
+    one neuron of 123,688, after hundreds of differently-valued weights per neuron have been added in atomic order); that
+    this mode has no such step is the proof that the order of the additions is all that separated them."""
+    steps = 100
+    net = configs.izhikevich_fanout(steps=steps)
+    assert net.css[0].noise.shape == (steps, 1_000_000)
+    model = model_from_net(net, ordered=True)
+    model.load(num_recording_timesteps=steps)
+    assert model.runner_info()["ordered_accumulation"]
+    oracle = OracleNet(net, num_recording_timesteps=steps)
+    model.run(steps)
+    oracle.run(steps)
+    model.pull_recording_buffers_from_device()
+    got, want = model.neuron_populations["N"].vars["recordSpk"].view, oracle.record("N", steps)
+    if not np.array_equal(got, want):
+        g, w = _raster_bits(got, 1_000_000, steps), _raster_bits(want, 1_000_000, steps)
+        raise AssertionError(f"raster differs first at step {int(np.nonzero((g != w).any(axis=1))[0][0])}")
+    per_step = _raster_bits(want, 1_000_000, steps).sum(axis=1)
+    assert per_step.max() > 100_000 and (per_step[:-1] * 1000 >= 1_000_000).sum() >= 10, "the run must include the population burst"
+    compare_state(net, model, oracle, "after 100 free-running steps", exact=True)
+    assert model.synaptic_event_count == oracle.events()
     model.unload()
 
 
