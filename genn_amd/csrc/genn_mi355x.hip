@@ -78,6 +78,11 @@ struct gennmi_runner
     // connectivity-derived tables that are rebuilt when tablesStale: segment boundaries of the tile path ...
     struct TileTable { size_t pre; uint16_t *off; uint32_t tileSize, numTiles; };
     std::vector<TileTable> tileTables;
+    // segment records of the tile path (copies of static weights and targets, one aligned record per (row, tile)): rebuilt
+    // when the projection's connectivity or weights have been written
+    struct RecordTable { size_t pre; uint8_t *records; const uint16_t *off; uint32_t lanes, tileSize, numTiles; };
+    std::vector<RecordTable> recordTables;
+    bool recordsStale = false;
     std::vector<void*> zeroOwned;       // ... the zero-delay lists of the single-launch step ...
     // ... and the column views of ordered accumulation (validation mode: every element summed in the CPU backend's order)
     bool ordered = false;
@@ -129,6 +134,7 @@ static void noteDeviceWrite(const void *dev, size_t bytes)
                 if(arr.ptr && arr.size && a < lo + arr.size && lo < b) {
                     if(r->resident) { r->resStale = true; }
                     if(arr.connectivity) { r->tablesStale = true; }
+                    if(!r->recordTables.empty()) { r->recordsStale = true; }
                 }
             }
         }
@@ -837,18 +843,35 @@ static int buildOrderedViews(gennmi_runner *r)
     return GENNMI_OK;
 }
 
+static int buildTileRecords(const gennmi_runner *r, const gennmi_runner::RecordTable &t)
+{
+    const auto &g = r->pre[t.pre].g;
+    const size_t count = (size_t)g.numSrcNeurons * t.numTiles;
+    const dim3 grid((unsigned int)((count + BLOCK - 1) / BLOCK));
+    if(t.lanes == 5) { tileRecordBuildKernel<5><<<grid, dim3(BLOCK), 0, 0>>>(g.numSrcNeurons, g.rowStride, g.ind, g.g, t.off, t.tileSize, t.numTiles, t.records); }
+    else { tileRecordBuildKernel<10><<<grid, dim3(BLOCK), 0, 0>>>(g.numSrcNeurons, g.rowStride, g.ind, g.g, t.off, t.tileSize, t.numTiles, t.records); }
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipDeviceSynchronize());
+    return GENNMI_OK;
+}
+
 // Connectivity-derived tables follow the connectivity: when rowLength / ind / d of a projection have been written since
 // the tables were built (a connectivity push after load), they are rebuilt before the next launch.
 static int refreshTables(gennmi_runner *r)
 {
-    bool stale;
+    bool stale, recordsStale;
     {
         std::lock_guard<std::mutex> lock(g_runnersMutex);
-        stale = r->tablesStale;
-        r->tablesStale = false;
+        stale = r->tablesStale; recordsStale = r->recordsStale;
+        r->tablesStale = false; r->recordsStale = false;
     }
-    if(!stale) { return GENNMI_OK; }
+    if(!stale && !recordsStale) { return GENNMI_OK; }
     HIP_TRY(hipStreamSynchronize(r->stream));
+    if(!stale) {
+        // only weights were written: the records hold copies of them
+        for(const auto &t : r->recordTables) { const int rc = buildTileRecords(r, t); if(rc) { return rc; } }
+        return GENNMI_OK;
+    }
     for(const auto &t : r->tileTables) {
         uint32_t unsorted = 0;
         { const int rc = buildTileOffsets(r->pre[t.pre].g, t.off, t.tileSize, t.numTiles, &unsorted); if(rc) { return rc; } }
@@ -857,6 +880,7 @@ static int refreshTables(gennmi_runner *r)
                                        "sort the rows or set GENNMI_TILE_FLOATS=0 before the runner is finalised");
         }
     }
+    for(const auto &t : r->recordTables) { const int rc = buildTileRecords(r, t); if(rc) { return rc; } }
     if(r->fusedStep) {
         // The spikes of the last completed step have already had their zero-delay synapses delivered — by the old lists —
         // into the slot that is read next, and the coming step will skip every synapse that is zero-delay NOW.  Synapses of
@@ -1100,6 +1124,26 @@ int gennmi_runner_finalise(gennmi_runner *r)
             const char *envLanes = getenv("GENNMI_TILE_LANES");
             t.lanes = envLanes ? std::min<uint32_t>(WAVE, pow2Ceil((uint32_t)std::max(1, atoi(envLanes)))) : std::min<uint32_t>(WAVE, pow2Ceil((avgSeg + 7) / 8));
             t.threshold = p.tileThreshold;
+            // Short segments (a row spread over many tiles) are what the plain tile path reads worst: two short reads at
+            // arbitrary offsets plus the boundary look-up per (spike, tile).  Static projections whose segments fit a
+            // record of 20 or 40 synapses get the record copy; GENNMI_TILE_RECORDS=0 keeps the rows only.
+            const char *envRecords = getenv("GENNMI_TILE_RECORDS");
+            const uint32_t segLen = (p.g.rowStride + numTiles - 1) / numTiles;
+            if(!(envRecords && atoi(envRecords) == 0) && p.g.wum == GENNMI_WUM_STATIC_PULSE && segLen >= 6 && segLen <= 34 && tileSize <= 65536) {
+                const uint32_t lanes = (segLen <= 17) ? 5u : 10u;
+                const size_t bytes = (size_t)numTiles * p.g.numSrcNeurons * recordBytes(lanes);
+                size_t freeBytes = 0, totalBytes = 0;
+                HIP_TRY(hipMemGetInfo(&freeBytes, &totalBytes));
+                if(bytes + (size_t(2) << 30) < freeBytes) {
+                    uint8_t *records = nullptr;
+                    HIP_TRY(hipMalloc(&records, bytes));
+                    r->owned.push_back(records);
+                    const gennmi_runner::RecordTable table{(size_t)(&p - r->pre.data()), records, dOff, lanes, tileSize, numTiles};
+                    { const int rc = buildTileRecords(r, table); if(rc) { return rc; } }
+                    r->recordTables.push_back(table);
+                    t.records = records; t.recLanes = lanes;
+                }
+            }
             tileGroups.push_back(t);
             r->tileFloats = std::max(r->tileFloats, tileSize);
         }

@@ -125,8 +125,20 @@ struct TileGroupDev
     uint32_t numTiles, tileSize;
     uint32_t tile, split, numSplits;    // this block: which tile, which share of the spikes
     uint32_t lanes;                     // lanes per (spike, tile) segment, power of two
-    uint32_t threshold, pad_;
+    uint32_t threshold;
+    uint32_t recLanes;                  // != 0: the projection has segment records (below), read by this many lanes each (5 or 10)
+    const uint8_t *records;             // [numTiles][numSrc] records of 24 * recLanes + 8 bytes (128 or 256), or NULL
 };
+
+// Segment records: an engine-private copy of a static SPARSE projection in which the synapses of one (row, tile) segment
+// form one record that starts on a cache-line boundary:
+//     float    weight[4 * recLanes]        zero-filled beyond the segment
+//     uint16_t target[4 * recLanes]        tile-local postsynaptic index
+//     uint16_t count, first                synapses in the segment; position of the first one within its row
+//     uint32_t spare
+// A spike then costs each tile exactly one aligned line of 128 (256) bytes instead of two short reads at arbitrary offsets
+// plus a look-up of the segment's boundaries.  Segments longer than a record keep their tail in the row itself.
+__host__ __device__ constexpr uint32_t recordBytes(uint32_t recLanes) { return 24u * recLanes + 8u; }
 
 // Dense-activity path of a Toeplitz Conv2D projection: a block owns rowsPerTile output rows (all columns and
 // channels) in LDS next to a copy of the kernel weights.
@@ -159,6 +171,7 @@ __device__ __forceinline__ GLOBAL_AS T *asGlobal(T *p) { return (GLOBAL_AS T*)p;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint8_t u8x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4u __attribute__((ext_vector_type(4), aligned(4)));     // dword-aligned only: segments start anywhere in a row
 typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
 
@@ -166,6 +179,41 @@ __device__ __forceinline__ void atomicAddF32(GLOBAL_AS float *addr, float v)
 {
     // gfx950 has a native global_atomic_add_f32; the old value is not needed
     __builtin_amdgcn_global_atomic_fadd_f32(addr, v);
+}
+
+// fp32 add into LDS.  The native LDS float atomic of this part (ds_add_f32) retires one lane every three clocks per
+// compute unit — 204 G adds/s for the whole chip, measured, whatever the addresses — while the integer path of the same
+// banks sustains over 3,000 G/s; a compare-and-swap loop on that path adds floats at 1,450 to 1,600 G/s.  The sum is the
+// same single fp32 addition either way.
+__device__ __forceinline__ void ldsAddF32(float *addr, float v)
+{
+    uint32_t *p = reinterpret_cast<uint32_t*>(addr);
+    uint32_t old = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP), assumed;
+    do {
+        assumed = old;
+        old = atomicCAS(p, assumed, __float_as_uint(__uint_as_float(assumed) + v));
+    } while(old != assumed);
+}
+
+// four adds of one lane with their LDS round trips overlapped: all reads, then all swaps, then whatever lost a race
+// (including two of the four that name the same element) one by one
+__device__ __forceinline__ void ldsAddF32x4(float *a0, float v0, bool p0, float *a1, float v1, bool p1, float *a2, float v2, bool p2, float *a3, float v3, bool p3)
+{
+    uint32_t *q0 = reinterpret_cast<uint32_t*>(a0), *q1 = reinterpret_cast<uint32_t*>(a1), *q2 = reinterpret_cast<uint32_t*>(a2), *q3 = reinterpret_cast<uint32_t*>(a3);
+    uint32_t o0 = 0, o1 = 0, o2 = 0, o3 = 0;
+    if(p0) { o0 = __hip_atomic_load(q0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+    if(p1) { o1 = __hip_atomic_load(q1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+    if(p2) { o2 = __hip_atomic_load(q2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+    if(p3) { o3 = __hip_atomic_load(q3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+    uint32_t r0 = o0, r1 = o1, r2 = o2, r3 = o3;
+    if(p0) { r0 = atomicCAS(q0, o0, __float_as_uint(__uint_as_float(o0) + v0)); }
+    if(p1) { r1 = atomicCAS(q1, o1, __float_as_uint(__uint_as_float(o1) + v1)); }
+    if(p2) { r2 = atomicCAS(q2, o2, __float_as_uint(__uint_as_float(o2) + v2)); }
+    if(p3) { r3 = atomicCAS(q3, o3, __float_as_uint(__uint_as_float(o3) + v3)); }
+    if(p0 && r0 != o0) { ldsAddF32(a0, v0); }
+    if(p1 && r1 != o1) { ldsAddF32(a1, v1); }
+    if(p2 && r2 != o2) { ldsAddF32(a2, v2); }
+    if(p3 && r3 != o3) { ldsAddF32(a3, v3); }
 }
 
 }   // namespace

@@ -360,6 +360,61 @@ void presynapticProceduralKernel(const ProcGroupDev * __restrict__ blocks, unsig
 // sorted by target; tileOff holds the segment boundaries), adds into LDS, and finally flushes the tile
 // with consecutive lanes on consecutive addresses.
 // ------------------------------------------------------------------------------------------------
+// Record variant of the tile kernel's main loop (static weights): L lanes read one (spike, tile) record — four weights
+// (16 bytes) and four tile-local targets (8 bytes) each, plus the record's count word — so a wavefront takes 64 / L records
+// per pass, every one a single aligned line.  The block's share of the spike queue is dealt so that one pass of the block
+// covers consecutive queue entries: the queue ascends, so the block walks its tile's record array front to back.
+template<uint32_t L>
+__device__ __forceinline__ unsigned long long tileRecordLoop(const TileGroupDev &G, GLOBAL_AS const uint32_t *spk, uint32_t numSpikes, uint32_t activeSplits,
+                                                             float *shTile, uint32_t tileStart)
+{
+    constexpr uint32_t C = 4 * L, REC = recordBytes(L), GROUPS = WAVE / L;
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    const uint32_t lane = threadIdx.x & (WAVE - 1);
+    const uint32_t group = lane / L, k = lane % L;
+    const bool live = group < GROUPS;
+    const uint32_t perBlock = (blockDim.x / WAVE) * GROUPS;
+    const uint32_t stride = perBlock * activeSplits;
+    const uint32_t lastSrc = g.numSrcNeurons - 1;
+    GLOBAL_AS const uint8_t *records = asGlobal(G.records) + (size_t)G.tile * g.numSrcNeurons * REC;
+    unsigned long long events = 0;
+    struct Rec { f32x4 w; uint32_t t01, t23, meta; };
+    auto fetch = [&](uint32_t id) -> Rec {
+        GLOBAL_AS const uint8_t *rec = records + (size_t)id * REC;
+        Rec r;
+        r.w = *reinterpret_cast<GLOBAL_AS const f32x4*>(rec + 16 * k);
+        const u32x2 t = *reinterpret_cast<GLOBAL_AS const u32x2*>(rec + 16 * L + 8 * k);
+        r.t01 = t.x; r.t23 = t.y;
+        r.meta = *reinterpret_cast<GLOBAL_AS const uint32_t*>(rec + 24 * L);
+        return r;
+    };
+    // two records in flight per lane group: the spike id is fetched two passes ahead, the record one pass ahead
+    uint32_t s = G.split * perBlock + (threadIdx.x / WAVE) * GROUPS + min(group, GROUPS - 1);
+    uint32_t id0 = spk[min(s, lastSrc)], id1 = spk[min(s + stride, lastSrc)];
+    Rec next = fetch(id0);
+    for(; s < numSpikes; s += stride) {
+        const Rec cur = next;
+        const uint32_t idPre = id0;
+        id0 = id1;
+        id1 = spk[min(s + 2 * stride, lastSrc)];
+        next = fetch(id0);
+        if(!live) { continue; }
+        const uint32_t n = cur.meta & 0xFFFFu;
+        const uint32_t j = 4 * k;
+        ldsAddF32x4(&shTile[cur.t01 & 0xFFFFu], cur.w.x, j < n, &shTile[cur.t01 >> 16], cur.w.y, j + 1 < n,
+                    &shTile[cur.t23 & 0xFFFFu], cur.w.z, j + 2 < n, &shTile[cur.t23 >> 16], cur.w.w, j + 3 < n);
+        if(n > C) {
+            // the tail of a segment longer than a record is read from the row itself
+            const size_t base = (size_t)idPre * g.rowStride + (cur.meta >> 16);
+            for(uint32_t jj = C + k; jj < n; jj += L) {
+                ldsAddF32(&shTile[asGlobal(g.ind)[base + jj] - tileStart], asGlobal(g.g)[base + jj]);
+            }
+        }
+        if(k == 0) { events += n; }
+    }
+    return events;
+}
+
 __global__ __launch_bounds__(1024)
 void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs args, float dt, unsigned long long *eventCounter)
 {
@@ -369,6 +424,28 @@ void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs ar
     const uint32_t batch = blockIdx.y;
     const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
     if((unsigned long long)numSpikes * g.rowStride < G.threshold) { return; }      // the scatter kernel took this step
+    if(G.recLanes) {
+        // a step with few spikes is shared between fewer blocks per tile (every block zeroes and flushes a whole tile)
+        const uint32_t perBlock = (blockDim.x / WAVE) * (WAVE / G.recLanes);
+        const uint32_t activeSplits = min(G.numSplits, max(1u, numSpikes / (2 * perBlock)));
+        if(G.split >= activeSplits) { return; }
+        const uint32_t tileStart = G.tile * G.tileSize;
+        const uint32_t tileLen = min(G.tileSize, g.numTrgNeurons - tileStart);
+        for(uint32_t k = threadIdx.x; k < tileLen; k += blockDim.x) { shTile[k] = 0.0f; }
+        __syncthreads();
+        GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
+        unsigned long long events = (G.recLanes == 5) ? tileRecordLoop<5>(G, spk, numSpikes, activeSplits, shTile, tileStart)
+                                                      : tileRecordLoop<10>(G, spk, numSpikes, activeSplits, shTile, tileStart);
+        __syncthreads();
+        GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons + tileStart;
+        for(uint32_t k = threadIdx.x; k < tileLen; k += blockDim.x) {
+            const float v = shTile[k];
+            if(v != 0.0f) { atomicAddF32(&outPost[k], v); }
+        }
+        for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
+        if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+        return;
+    }
     const uint32_t tileStart = G.tile * G.tileSize;
     const uint32_t tileLen = min(G.tileSize, g.numTrgNeurons - tileStart);
     for(uint32_t k = threadIdx.x; k < tileLen; k += blockDim.x) { shTile[k] = 0.0f; }
@@ -422,17 +499,15 @@ void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs ar
                     nw.x = depress(ip.x, w.x); nw.y = depress(ip.y, w.y); nw.z = depress(ip.z, w.z); nw.w = depress(ip.w, w.w);
                     *reinterpret_cast<GLOBAL_AS f32x4u*>(weight + rowBase + j) = nw;
                 }
-                unsafeAtomicAdd(&shTile[ip.x - tileStart], w.x);
-                unsafeAtomicAdd(&shTile[ip.y - tileStart], w.y);
-                unsafeAtomicAdd(&shTile[ip.z - tileStart], w.z);
-                unsafeAtomicAdd(&shTile[ip.w - tileStart], w.w);
+                ldsAddF32x4(&shTile[ip.x - tileStart], w.x, true, &shTile[ip.y - tileStart], w.y, true,
+                            &shTile[ip.z - tileStart], w.z, true, &shTile[ip.w - tileStart], w.w, true);
             }
             else {
                 for(uint32_t jj = j; jj < b; jj++) {
                     const uint32_t idPost = ind[rowBase + jj];
                     const float w = weight[rowBase + jj];
                     if(stdp) { weight[rowBase + jj] = depress(idPost, w); }
-                    unsafeAtomicAdd(&shTile[idPost - tileStart], w);
+                    ldsAddF32(&shTile[idPost - tileStart], w);
                 }
             }
         }
@@ -571,6 +646,35 @@ __global__ void tileOffsetKernel(uint32_t numSrc, uint32_t rowStride, const uint
         while(t <= numTiles && (unsigned long long)t * tileSize <= p) { o[t++] = (uint16_t)j; }
     }
     while(t <= numTiles) { o[t++] = (uint16_t)len; }
+}
+
+// Builds the segment records of one projection from its rows and the segment boundaries: one thread per (tile, row).
+template<uint32_t L>
+__global__ __launch_bounds__(BLOCK)
+void tileRecordBuildKernel(uint32_t numSrc, uint32_t rowStride, const uint32_t *ind, const float *weight, const uint16_t *off,
+                           uint32_t tileSize, uint32_t numTiles, uint8_t *records)
+{
+    constexpr uint32_t C = 4 * L, REC = recordBytes(L);
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if(idx >= (size_t)numSrc * numTiles) { return; }
+    const uint32_t tile = (uint32_t)(idx / numSrc), row = (uint32_t)(idx % numSrc);
+    const uint32_t a = off[(size_t)row * (numTiles + 1) + tile], b = off[(size_t)row * (numTiles + 1) + tile + 1];
+    const uint32_t n = b - a, tileStart = tile * tileSize;
+    uint8_t *rec = records + idx * REC;
+    const size_t base = (size_t)row * rowStride + a;
+    for(uint32_t q = 0; q < L; q++) {
+        f32x4 w; uint32_t t[4];
+        for(uint32_t e = 0; e < 4; e++) {
+            const uint32_t j = 4 * q + e;
+            const bool valid = j < n;           // j < C always
+            ((float*)&w)[e] = valid ? weight[base + j] : 0.0f;
+            t[e] = valid ? (ind[base + j] - tileStart) : 0u;
+        }
+        *reinterpret_cast<f32x4*>(rec + 16 * q) = w;
+        *reinterpret_cast<u32x2*>(rec + 16 * L + 8 * q) = u32x2{t[0] | (t[1] << 16), t[2] | (t[3] << 16)};
+    }
+    *reinterpret_cast<u32x2*>(rec + 24 * L) = u32x2{n | (a << 16), 0u};
+    (void)C;
 }
 
 __global__ __launch_bounds__(BLOCK)

@@ -59,6 +59,30 @@ def test_rewritten_rows_on_the_tile_path(ordered):
     model.unload()
 
 
+def test_rewritten_weights_reach_the_segment_records(monkeypatch):
+    """The tile path's segment records hold copies of the weights: a weight push in the middle of a run must reach them."""
+    monkeypatch.setenv("GENNMI_TILE_FLOATS", "600")
+    net = _exact_net()                      # 1111 targets in tiles of 600, 40 synapses per row: records of 40
+    syn = net.syns[0]
+    model = model_from_net(net)
+    model.load(num_recording_timesteps=net.steps)
+    oracle = OracleNet(net, num_recording_timesteps=net.steps)
+    for phase in range(2):
+        for _ in range(30):
+            model.step_time()
+            oracle.step()
+            for p in net.pops:
+                assert np.array_equal(model.neuron_populations[p.name].current_spikes[0], oracle.spikes(p.name)), f"step {model.timestep}: {p.name}"
+        if phase == 0:
+            syn.g[:] = (syn.g * 0.5 + 0.25).astype(np.float32)          # still multiples of 1/8: sums stay exact
+            sg = model.synapse_populations["AB"]
+            sg.vars["g"].view[:] = syn.g.reshape(-1)
+            sg.vars["g"].push_to_device()
+    compare_state(net, model, oracle, "after the weight push", exact=True)
+    assert model.synaptic_event_count == oracle.events()
+    model.unload()
+
+
 @pytest.mark.parametrize("ordered", [False, True])
 def test_rewritten_delays(ordered):
     """Delays of six projections are set to zero for half of their rows in the middle of a run.  Default mode: the network is

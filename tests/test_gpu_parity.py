@@ -78,6 +78,34 @@ def test_dense_activity_tile_path(tile_floats, monkeypatch):
     model.unload()
 
 
+@pytest.mark.parametrize("m, fan, tile_floats, records", [(4000, 100, "600", "1"), (4000, 100, "600", "0"), (1111, 40, "600", "1"), (6000, 230, "1024", "1")])
+def test_tile_path_segment_records(m, fan, tile_floats, records, monkeypatch):
+    """Static projections whose (row, tile) segments are short are read through segment records: one aligned record of 20
+    (or 40) synapses per (row, tile), the tail of a longer segment from the row itself.  4000 targets in tiles of 600 with
+    100 synapses per row: ~15 per segment, so records of 20 with overflowing segments; 1111 targets, 40 per row: ~20 per
+    segment, records of 40; 6000 targets in tiles of 1024, 230 per row: ~38 per segment, records of 40 that overflow often.
+    Exact sums (integer-valued weights into DeltaCurr), so everything must be bit-identical to the oracle, with and without
+    the records."""
+    from genn_amd.netspec import Net, Pop, Syn
+    from genn_amd import netgen
+    monkeypatch.setenv("GENNMI_TILE_FLOATS", tile_floats)
+    monkeypatch.setenv("GENNMI_TILE_RECORDS", records)
+    n = 3000
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.7, TauRefrac=2.0)
+    net = Net(name="records", dt=1.0, steps=60)
+    v0 = (-60.0 + 10.0 * np.linspace(0, 1, n)).astype(np.float32)
+    net.pops.append(Pop("A", "lif", n, dict(lif), {"V": v0, "RefracTime": np.zeros(n, np.float32)}))
+    net.pops.append(Pop("B", "lif", m, dict(lif, Ioffset=0.0), {"V": np.full(m, -60.0, np.float32), "RefracTime": np.zeros(m, np.float32)}))
+    rl, ind = netgen.fixed_number_post(11, 3, n, m, fan)
+    rl[::7] = (rl[::7] * 2) // 3            # ragged rows: the last segments of those rows are short or empty
+    g = np.round(netgen.rows_uniform(11, 4, rl, fan, n, 3.0, 0.0, 3.0, 0.0)).astype(np.float32) * 0.125
+    net.syns.append(Syn("AB", "A", "B", wum="static", psm="deltacurr", row_stride=fan, row_length=rl, ind=ind, g=g))
+    model, oracle, counts = run_side_by_side(net, check_every=10, exact=True)
+    assert counts["A"] > 2 * n
+    assert model.synaptic_event_count == oracle.events()
+    model.unload()
+
+
 def test_izhikevich_fanout_noise():
     """C3 shape: Izhikevich neurons, fixed fanout with replacement (multapses), DeltaCurr input,
     per-step noise current from a pregenerated array.  dt = 1 ms, first 100 ms = 100 steps."""
