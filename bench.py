@@ -244,6 +244,7 @@ def main():
     wall = time.perf_counter() - t0
     region_s = model.stream_elapsed()          # HIP events on the runner's stream around the timed region
     events = model.synaptic_event_count - ev0
+    events_with_warmup = events + ev0
 
     model.pull_recording_buffers_from_device()
     rates = {}
@@ -381,7 +382,7 @@ def main():
         "gsop_per_s": round(events / wall / 1e9, 4),
         "neuron_updates_per_s": round(num_neurons * batch * args.steps / wall, 1),
         "wall_s_per_sim_s": round(wall / sim_s, 4),
-        "events_per_step": round(events / args.steps, 1),
+        "events_per_step": round(events / args.steps, 1), "events_including_warmup": events_with_warmup,
         "algorithmic_gb_per_s_wallclock": round(events * (bytes_per_event or 16) / wall / 1e9, 3),
         "firing_rates_hz": rates,
         "setup_s": {"generate": round(gen_s, 1), "load": round(load_s, 1)},

@@ -80,7 +80,7 @@ struct gennmi_runner
     std::vector<TileTable> tileTables;
     // segment records of the tile path (copies of static weights and targets, one aligned record per (row, tile)): rebuilt
     // when the projection's connectivity or weights have been written
-    struct RecordTable { size_t pre; uint8_t *records; const uint16_t *off; uint32_t lanes, tileSize, numTiles; };
+    struct RecordTable { size_t pre; uint8_t *records; uint8_t *overflow; const uint16_t *off; uint32_t lanes, tileSize, numTiles; };
     std::vector<RecordTable> recordTables;
     bool recordsStale = false;
     std::vector<void*> zeroOwned;       // ... the zero-delay lists of the single-launch step ...
@@ -848,8 +848,8 @@ static int buildTileRecords(const gennmi_runner *r, const gennmi_runner::RecordT
     const auto &g = r->pre[t.pre].g;
     const size_t count = (size_t)g.numSrcNeurons * t.numTiles;
     const dim3 grid((unsigned int)((count + BLOCK - 1) / BLOCK));
-    if(t.lanes == 5) { tileRecordBuildKernel<5><<<grid, dim3(BLOCK), 0, 0>>>(g.numSrcNeurons, g.rowStride, g.ind, g.g, t.off, t.tileSize, t.numTiles, t.records); }
-    else { tileRecordBuildKernel<10><<<grid, dim3(BLOCK), 0, 0>>>(g.numSrcNeurons, g.rowStride, g.ind, g.g, t.off, t.tileSize, t.numTiles, t.records); }
+    if(t.lanes == 5) { tileRecordBuildKernel<5><<<grid, dim3(BLOCK), 0, 0>>>(g.numSrcNeurons, g.rowStride, g.ind, g.g, t.off, t.tileSize, t.numTiles, t.records, t.overflow); }
+    else { tileRecordBuildKernel<10><<<grid, dim3(BLOCK), 0, 0>>>(g.numSrcNeurons, g.rowStride, g.ind, g.g, t.off, t.tileSize, t.numTiles, t.records, t.overflow); }
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipDeviceSynchronize());
     return GENNMI_OK;
@@ -1138,10 +1138,18 @@ int gennmi_runner_finalise(gennmi_runner *r)
                     uint8_t *records = nullptr;
                     HIP_TRY(hipMalloc(&records, bytes));
                     r->owned.push_back(records);
-                    const gennmi_runner::RecordTable table{(size_t)(&p - r->pre.data()), records, dOff, lanes, tileSize, numTiles};
+                    // overflow records where memory allows: segments are Poisson-like around rowStride / numTiles, so a
+                    // sixth or so of them exceed a record sized for the mean
+                    uint8_t *overflow = nullptr;
+                    const size_t overflowBytes = (size_t)numTiles * p.g.numSrcNeurons * 64;
+                    if(bytes + overflowBytes + (size_t(2) << 30) < freeBytes) {
+                        HIP_TRY(hipMalloc(&overflow, overflowBytes));
+                        r->owned.push_back(overflow);
+                    }
+                    const gennmi_runner::RecordTable table{(size_t)(&p - r->pre.data()), records, overflow, dOff, lanes, tileSize, numTiles};
                     { const int rc = buildTileRecords(r, table); if(rc) { return rc; } }
                     r->recordTables.push_back(table);
-                    t.records = records; t.recLanes = lanes;
+                    t.records = records; t.recLanes = lanes; t.overflow = overflow;
                 }
             }
             tileGroups.push_back(t);

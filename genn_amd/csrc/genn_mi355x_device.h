@@ -128,7 +128,9 @@ struct TileGroupDev
     uint32_t threshold;
     uint32_t recLanes;                  // != 0: the projection has segment records (below), read by this many lanes each (5 or 10)
     const uint8_t *records;             // [numTiles][numSrc] records of 24 * recLanes + 8 bytes (128 or 256), or NULL
+    const uint8_t *overflow;            // [numTiles][numSrc] 64-byte records of the 8 synapses that follow a full record, or NULL
 };
+constexpr uint32_t REC_OVERFLOW = 8;    // synapses per overflow record: float weight[8], uint16_t target[8], 16 spare bytes
 
 // Segment records: an engine-private copy of a static SPARSE projection in which the synapses of one (row, tile) segment
 // form one record that starts on a cache-line boundary:
@@ -137,7 +139,9 @@ struct TileGroupDev
 //     uint16_t count, first                synapses in the segment; position of the first one within its row
 //     uint32_t spare
 // A spike then costs each tile exactly one aligned line of 128 (256) bytes instead of two short reads at arbitrary offsets
-// plus a look-up of the segment's boundaries.  Segments longer than a record keep their tail in the row itself.
+// plus a look-up of the segment's boundaries.  The next 8 synapses of a segment longer than a record sit in a second,
+// 64-byte record (read only by those segments: one more aligned read instead of two unaligned ones into the row); what
+// exceeds both is read from the row itself.
 __host__ __device__ constexpr uint32_t recordBytes(uint32_t recLanes) { return 24u * recLanes + 8u; }
 
 // Dense-activity path of a Toeplitz Conv2D projection: a block owns rowsPerTile output rows (all columns and

@@ -377,6 +377,7 @@ __device__ __forceinline__ unsigned long long tileRecordLoop(const TileGroupDev 
     const uint32_t stride = perBlock * activeSplits;
     const uint32_t lastSrc = g.numSrcNeurons - 1;
     GLOBAL_AS const uint8_t *records = asGlobal(G.records) + (size_t)G.tile * g.numSrcNeurons * REC;
+    GLOBAL_AS const uint8_t *overflow = G.overflow ? asGlobal(G.overflow) + (size_t)G.tile * g.numSrcNeurons * 64 : nullptr;
     unsigned long long events = 0;
     struct Rec { f32x4 w; uint32_t t01, t23, meta; };
     auto fetch = [&](uint32_t id) -> Rec {
@@ -388,29 +389,47 @@ __device__ __forceinline__ unsigned long long tileRecordLoop(const TileGroupDev 
         r.meta = *reinterpret_cast<GLOBAL_AS const uint32_t*>(rec + 24 * L);
         return r;
     };
-    // two records in flight per lane group: the spike id is fetched two passes ahead, the record one pass ahead
+    // DEPTH records in flight per lane group (a pass of the block is one dependent chain spike id -> record -> adds, and a
+    // step of a few thousand spikes is only a handful of passes per block): ids are fetched DEPTH passes ahead of their
+    // records, records DEPTH passes ahead of their adds
+    constexpr uint32_t DEPTH = 4;
     uint32_t s = G.split * perBlock + (threadIdx.x / WAVE) * GROUPS + min(group, GROUPS - 1);
-    uint32_t id0 = spk[min(s, lastSrc)], id1 = spk[min(s + stride, lastSrc)];
-    Rec next = fetch(id0);
-    for(; s < numSpikes; s += stride) {
-        const Rec cur = next;
-        const uint32_t idPre = id0;
-        id0 = id1;
-        id1 = spk[min(s + 2 * stride, lastSrc)];
-        next = fetch(id0);
-        if(!live) { continue; }
-        const uint32_t n = cur.meta & 0xFFFFu;
-        const uint32_t j = 4 * k;
-        ldsAddF32x4(&shTile[cur.t01 & 0xFFFFu], cur.w.x, j < n, &shTile[cur.t01 >> 16], cur.w.y, j + 1 < n,
-                    &shTile[cur.t23 & 0xFFFFu], cur.w.z, j + 2 < n, &shTile[cur.t23 >> 16], cur.w.w, j + 3 < n);
-        if(n > C) {
-            // the tail of a segment longer than a record is read from the row itself
-            const size_t base = (size_t)idPre * g.rowStride + (cur.meta >> 16);
-            for(uint32_t jj = C + k; jj < n; jj += L) {
-                ldsAddF32(&shTile[asGlobal(g.ind)[base + jj] - tileStart], asGlobal(g.g)[base + jj]);
+    uint32_t ids[2 * DEPTH];
+    Rec recs[DEPTH];
+    #pragma unroll
+    for(uint32_t u = 0; u < 2 * DEPTH; u++) { ids[u] = spk[min(s + u * stride, lastSrc)]; }
+    #pragma unroll
+    for(uint32_t u = 0; u < DEPTH; u++) { recs[u] = fetch(ids[u]); }
+    for(; s < numSpikes; s += DEPTH * stride) {
+        #pragma unroll
+        for(uint32_t u = 0; u < DEPTH; u++) {
+            const Rec cur = recs[u];
+            const uint32_t idPre = ids[u];
+            ids[u] = ids[u + DEPTH];
+            ids[u + DEPTH] = spk[min(s + (u + 2 * DEPTH) * stride, lastSrc)];
+            recs[u] = fetch(ids[u]);
+            if(!live || s + u * stride >= numSpikes) { continue; }
+            const uint32_t n = cur.meta & 0xFFFFu;
+            const uint32_t j = 4 * k;
+            ldsAddF32x4(&shTile[cur.t01 & 0xFFFFu], cur.w.x, j < n, &shTile[cur.t01 >> 16], cur.w.y, j + 1 < n,
+                        &shTile[cur.t23 & 0xFFFFu], cur.w.z, j + 2 < n, &shTile[cur.t23 >> 16], cur.w.w, j + 3 < n);
+            if(n > C) {
+                // a segment longer than a record: the next 8 synapses from its overflow record, the rest from the row itself
+                uint32_t done = C;
+                if(overflow) {
+                    GLOBAL_AS const uint8_t *ovf = overflow + (size_t)idPre * 64;
+                    for(uint32_t jj = k; jj < min(n - C, REC_OVERFLOW); jj += L) {
+                        ldsAddF32(&shTile[reinterpret_cast<GLOBAL_AS const uint16_t*>(ovf + 32)[jj]], reinterpret_cast<GLOBAL_AS const float*>(ovf)[jj]);
+                    }
+                    done = C + REC_OVERFLOW;
+                }
+                const size_t base = (size_t)idPre * g.rowStride + (cur.meta >> 16);
+                for(uint32_t jj = done + k; jj < n; jj += L) {
+                    ldsAddF32(&shTile[asGlobal(g.ind)[base + jj] - tileStart], asGlobal(g.g)[base + jj]);
+                }
             }
+            if(k == 0) { events += n; }
         }
-        if(k == 0) { events += n; }
     }
     return events;
 }
@@ -425,9 +444,11 @@ void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs ar
     const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
     if((unsigned long long)numSpikes * g.rowStride < G.threshold) { return; }      // the scatter kernel took this step
     if(G.recLanes) {
-        // a step with few spikes is shared between fewer blocks per tile (every block zeroes and flushes a whole tile)
-        const uint32_t perBlock = (blockDim.x / WAVE) * (WAVE / G.recLanes);
-        const uint32_t activeSplits = min(G.numSplits, max(1u, numSpikes / (2 * perBlock)));
+        // A step with few spikes is shared between fewer blocks per tile: every block zeroes a whole tile and flushes what it
+        // touched with global atomics, which costs more than the adds themselves while a block's share of the tile is
+        // sparsely filled.  Measured on 10^6 rows x 1000 synapses (us per step with 2 / 4 / 8 / 16 blocks per tile): 3 x 10^3
+        // spikes 49 / 54 / 73 / 102, 2 x 10^4 spikes 171 / 114 / 111 / 159, 3 x 10^5 spikes 2281 / 1190 / 754 / 766.
+        const uint32_t activeSplits = min(G.numSplits, max(2u, numSpikes / 4096u));
         if(G.split >= activeSplits) { return; }
         const uint32_t tileStart = G.tile * G.tileSize;
         const uint32_t tileLen = min(G.tileSize, g.numTrgNeurons - tileStart);
@@ -652,7 +673,7 @@ __global__ void tileOffsetKernel(uint32_t numSrc, uint32_t rowStride, const uint
 template<uint32_t L>
 __global__ __launch_bounds__(BLOCK)
 void tileRecordBuildKernel(uint32_t numSrc, uint32_t rowStride, const uint32_t *ind, const float *weight, const uint16_t *off,
-                           uint32_t tileSize, uint32_t numTiles, uint8_t *records)
+                           uint32_t tileSize, uint32_t numTiles, uint8_t *records, uint8_t *overflow)
 {
     constexpr uint32_t C = 4 * L, REC = recordBytes(L);
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -674,7 +695,14 @@ void tileRecordBuildKernel(uint32_t numSrc, uint32_t rowStride, const uint32_t *
         *reinterpret_cast<u32x2*>(rec + 16 * L + 8 * q) = u32x2{t[0] | (t[1] << 16), t[2] | (t[3] << 16)};
     }
     *reinterpret_cast<u32x2*>(rec + 24 * L) = u32x2{n | (a << 16), 0u};
-    (void)C;
+    if(overflow && n > C) {
+        uint8_t *ovf = overflow + idx * 64;
+        for(uint32_t e = 0; e < REC_OVERFLOW; e++) {
+            const bool valid = C + e < n;
+            reinterpret_cast<float*>(ovf)[e] = valid ? weight[base + C + e] : 0.0f;
+            reinterpret_cast<uint16_t*>(ovf + 32)[e] = valid ? (uint16_t)(ind[base + C + e] - tileStart) : (uint16_t)0;
+        }
+    }
 }
 
 __global__ __launch_bounds__(BLOCK)
