@@ -295,3 +295,28 @@ def test_adapter_poisson_background_matches_host_layer():
         model.unload()
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_genn_buildmodel_flow_matches_the_reference_backend():
+    """The reference's own generator driver (src/genn/generator/generator.cc, built by oracle/Makefile.ref with
+    -DBACKEND_NAMESPACE=MI355X as genn_amd/backend/MakefileMI355X sets it) on the example model file
+    genn_amd/backend/example/model.cc: generate, compile, construct the Runtime, and run the model file's simulate() — 3000
+    steps of the balanced network, connectivity and initial state from GeNN's seeded built-in snippets.  Spike counts and
+    raster checksums must equal what the same driver built for the SingleThreadedCPU backend printed
+    (tests/golden/selection_example.json, written by tests/golden/make_selection_golden.py)."""
+    import json
+    import re
+    generator = os.path.join(ROOT, "oracle", "_ref", "mi355x_generator")
+    if not os.path.exists(generator):
+        pytest.skip("oracle/_ref/mi355x_generator is not built")
+    golden = json.load(open(os.path.join(HERE, "golden", "selection_example.json")))
+    tmp = tempfile.mkdtemp(prefix="buildmodel_")
+    try:
+        res = subprocess.run([generator, ROOT, tmp, "1"], cwd=tmp, env=dict(os.environ, GENN_EXAMPLE_STEPS=str(golden["steps"])),
+                             stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        assert res.returncode == 0, res.stdout[-3000:]
+        got = {m.group(1): {"spikes": int(m.group(2)), "checksum": m.group(3)}
+               for m in re.finditer(r"example: population (\w+) spikes (\d+) checksum (\d+)", res.stdout)}
+        assert got == golden["populations"], (got, golden["populations"])
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
