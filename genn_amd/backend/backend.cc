@@ -934,9 +934,18 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
         emit();
     };
 
+    // initTime / initSparseTime (generateRunner.cc:161-162): initialisation runs on the host and ends with an upload, so the
+    // counters are wall-clock time of the whole function, taken when the model enables timing as the reference's are
+    const bool timing = model.isTimingEnabled();
+    const std::string timerStart = "const auto gennmiInitStart = std::chrono::steady_clock::now();";
+    auto timerStop = [](const std::string &counter)
+    {
+        return counter + " += std::chrono::duration<double>(std::chrono::steady_clock::now() - gennmiInitStart).count();";
+    };
     body << "void initialize()";
     {
         CodeStream::Scope b(body);
+        if(timing) { body << timerStart << std::endl; }
         EnvironmentExternal funcEnv(initEnv);
         funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
 
@@ -1017,6 +1026,7 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                 });
             });
         funcEnv.getStream() << "GENNMI_CHECK(gennmi_push_mirrors());" << std::endl;
+        if(timing) { funcEnv.getStream() << timerStop("initTime") << std::endl; }
     }
     body << std::endl;
 
@@ -1025,6 +1035,7 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
     body << "void initializeSparse()";
     {
         CodeStream::Scope b(body);
+        if(timing) { body << timerStart << std::endl; }
         EnvironmentExternal funcEnv(initEnv);
         funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
 
@@ -1058,6 +1069,7 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
             });
         funcEnv.getStream() << "GENNMI_CHECK(gennmi_push_mirrors());" << std::endl;
         funcEnv.getStream() << remapStream.str();
+        if(timing) { funcEnv.getStream() << "GENNMI_CHECK(gennmi_synchronize());" << std::endl << timerStop("initSparseTime") << std::endl; }
     }
 
     modelMerged.genMergedNeuronInitGroupStructs(os, *this);
@@ -1158,7 +1170,7 @@ size_t Backend::getSynapticMatrixRowStride(const SynapseGroupInternal &sg) const
 void Backend::genDefinitionsPreamble(CodeStream &os, const ModelSpecMerged&) const
 {
     os << "// Standard C++ includes" << std::endl;
-    for(const char *h : {"algorithm", "cassert", "cmath", "cstdint", "cstring", "iostream", "random", "stdexcept", "string", "vector"}) {
+    for(const char *h : {"algorithm", "cassert", "chrono", "cmath", "cstdint", "cstring", "iostream", "random", "stdexcept", "string", "vector"}) {
         os << "#include <" << h << ">" << std::endl;
     }
     os << std::endl;

@@ -1535,7 +1535,9 @@ int gennmi_runner_get_times(gennmi_runner *r, double *neuronUpdateTime, double *
 {
     if(!r) { return fail(GENNMI_EINVAL, "runner_get_times: null runner"); }
     { const int rc = drainTimers(r); if(rc) { return rc; } }
-    if(neuronUpdateTime) { *neuronUpdateTime = r->neuronTime; }
+    // a single-launch step is one kernel that holds the neuron update and, in blocks of its own, the presynaptic update of the
+    // previous step's spikes: its whole duration counts as neuron update time (the reference has no such kernel)
+    if(neuronUpdateTime) { *neuronUpdateTime = r->neuronTime + r->stepTime; }
     if(presynapticUpdateTime) { *presynapticUpdateTime = r->preTime; }
     if(postsynapticUpdateTime) { *postsynapticUpdateTime = r->postTime; }
     return GENNMI_OK;

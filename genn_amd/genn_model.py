@@ -10,6 +10,7 @@ simulation on the host.
 """
 import ctypes as C
 import math
+import time
 from fractions import Fraction
 
 import numpy as np
@@ -368,6 +369,8 @@ class GeNNModel:
         self.dt = float(dt)
         self.fuse_postsynaptic_models = False
         self.timing_enabled = False
+        self._init_time = 0.0
+        self._init_sparse_time = 0.0
         # validation mode: synaptic input is summed per postsynaptic neuron in the order of the reference's CPU backend
         # (no atomics; bit-identical accumulators, slow).  Read when the model is loaded.
         self.ordered_accumulation = False
@@ -505,6 +508,7 @@ class GeNNModel:
             raise RuntimeError("build() must be called before load()")
         lib = _abi.load()
         _abi.check(lib.gennmi_init(self._device))
+        load_start = time.perf_counter()
         B = self.batch_size
         self.num_recording_timesteps = num_recording_timesteps
         dt32 = lit32(self.dt)
@@ -642,7 +646,12 @@ class GeNNModel:
                 a.push_to_device()
                 s.vars["g"] = a
 
+        _abi.check(lib.gennmi_synchronize())
+        self._init_time += time.perf_counter() - load_start
+        sparse_start = time.perf_counter()
         self._initialize_sparse()
+        _abi.check(lib.gennmi_synchronize())
+        self._init_sparse_time += time.perf_counter() - sparse_start
         self._push_merged_groups()
         if self.ordered_accumulation:
             _abi.check(lib.gennmi_runner_set_ordered(self._runner, 1))
@@ -996,6 +1005,38 @@ class GeNNModel:
         info = (C.c_uint32 * 4)()
         _abi.check(_abi.load().gennmi_runner_get_info(self._runner, C.byref(info)))
         return {"single_launch_step": bool(info[0] & 1), "resident_plan": bool(info[0] & 2), "bulk_neuron_kernel": bool(info[0] & 4), "ordered_accumulation": bool(info[0] & 8), "neuron_blocks": info[1], "presyn_blocks": info[2], "postsyn_blocks": info[3]}
+
+    # timing counters under PyGeNN's names (pygenn/genn_model.py:292-326), in seconds, accumulated while `timing_enabled`
+    def _times(self):
+        n, pre, post = C.c_double(), C.c_double(), C.c_double()
+        _abi.check(_abi.load().gennmi_runner_get_times(self._runner, C.byref(n), C.byref(pre), C.byref(post)))
+        return n.value, pre.value, post.value
+
+    @property
+    def neuron_update_time(self):
+        return self._times()[0]
+
+    @property
+    def presynaptic_update_time(self):
+        return self._times()[1]
+
+    @property
+    def postsynaptic_update_time(self):
+        return self._times()[2]
+
+    @property
+    def init_time(self):
+        """Wall-clock seconds load() spent allocating and initialising arrays (on the host or by the initialisation kernels)."""
+        return self._init_time
+
+    @property
+    def init_sparse_time(self):
+        """Wall-clock seconds load() spent on connectivity-dependent initialisation (column views of plastic projections)."""
+        return self._init_sparse_time
+
+    @property
+    def synapse_dynamics_time(self):
+        return 0.0          # no model of the supported set has synapse dynamics code
 
     def set_timing(self, enabled):
         _abi.check(_abi.load().gennmi_runner_set_timing(self._runner, int(bool(enabled))))

@@ -361,7 +361,11 @@ int gennmi_run_steps(gennmi_runner *runner, unsigned long long timestep, unsigne
 int gennmi_runner_synchronize(gennmi_runner *runner);
 
 /* Timers: neuronUpdateTime / presynapticUpdateTime / postsynapticUpdateTime of generateRunner.cc:161-174,
- * in seconds, accumulated with HIP events while enabled (backendCUDAHIP.cc:36-76, 1479-1504). */
+ * in seconds, accumulated with HIP events while enabled (backendCUDAHIP.cc:36-76, 1479-1504).  While timing is enabled
+ * every step is launched on its own, kernel by kernel (gennmi_run_steps included: no resident launch, no graph replay),
+ * so that each kernel has an event pair around it.  A single-launch step (see gennmi_runner_get_info) is one kernel that
+ * holds the neuron update and the presynaptic update of the previous step's spikes: its duration is reported as
+ * neuronUpdateTime and presynapticUpdateTime stays 0 for such a runner. */
 int gennmi_runner_set_timing(gennmi_runner *runner, int enabled);
 int gennmi_runner_get_times(gennmi_runner *runner, double *neuronUpdateTime, double *presynapticUpdateTime,
                             double *postsynapticUpdateTime);

@@ -160,6 +160,7 @@ int main(int argc, char *argv[])
         bool generateOnly = false;
         std::string userCxxFlags;
         std::vector<std::string> dynamicParams;
+        bool timing = false;
         for(int a = 4; a < argc; a++) {
             const std::string opt = argv[a];
             if(opt == "--generate-only") { generateOnly = true; }
@@ -167,6 +168,7 @@ int main(int argc, char *argv[])
             // --dynamic=neuron:<population>.<param> | cs:<source>.<param> | wu:<projection>.<param> | ps:<projection>.<param>: marks a
             // parameter dynamic (setParamDynamic and friends), as a model that calls setDynamicParamValue at run time would
             else if(opt.rfind("--dynamic=", 0) == 0) { dynamicParams.push_back(opt.substr(10)); }
+            else if(opt == "--timing") { timing = true; }       // ModelSpec::setTimingEnabled; the Runtime's counters are printed after the run
             else { std::cerr << "unknown option " << opt << std::endl; return 1; }
         }
 
@@ -229,6 +231,7 @@ int main(int argc, char *argv[])
         if(seed) { model.setSeed(seed); }
         model.setPrecision(Type::Float);
         model.setFusePostsynapticModels(fuse != 0);
+        model.setTimingEnabled(timing);
         std::map<std::string, PopSpec*> popByName;
         for(auto &p : pops) {
             if(p.model == "lif") {
@@ -526,6 +529,10 @@ int main(int argc, char *argv[])
             std::vector<uint32_t> pairs;
             for(const auto &e : sorted) { pairs.push_back(e.first); pairs.push_back(e.second); }
             appendFile(out + "/" + s.name + ".events.u32", pairs.data(), pairs.size());
+        }
+        if(timing) {
+            std::cout << "ref_driver: timers init " << rt.getInitTime() << " initSparse " << rt.getInitSparseTime() << " neuronUpdate " << rt.getNeuronUpdateTime()
+                      << " presynapticUpdate " << rt.getPresynapticUpdateTime() << " postsynapticUpdate " << rt.getPostsynapticUpdateTime() << std::endl;
         }
         std::cout << "ref_driver: " << name << " ran " << steps << " steps" << std::endl;
     }
