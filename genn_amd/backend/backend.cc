@@ -261,8 +261,8 @@ std::string tableU32(const std::vector<uint64_t> &values)
 //--------------------------------------------------------------------------
 namespace GeNN::CodeGenerator::MI355X
 {
-Backend::Backend(const Preferences &preferences)
-:   BackendBase(preferences)
+Backend::Backend(const Preferences &preferences, bool generatedKernels)
+:   BackendBase(preferences), m_GeneratedKernels(generatedKernels)
 {
 }
 //--------------------------------------------------------------------------
@@ -272,6 +272,10 @@ Backend::Backend(const Preferences &preferences)
 void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelMerged,
                               BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const
 {
+    if(m_GeneratedKernels) {
+        genNeuronUpdateGenerated(os, modelMerged, memorySpaces, preambleHandler);
+        return;
+    }
     const ModelSpecInternal &model = modelMerged.getModel();
     const unsigned int batchSize = model.getBatchSize();
     const auto scalar = model.getPrecision();
@@ -605,6 +609,10 @@ void Backend::genNeuronUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
 void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelMerged,
                                BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const
 {
+    if(m_GeneratedKernels) {
+        genSynapseUpdateGenerated(os, modelMerged, memorySpaces, preambleHandler);
+        return;
+    }
     const ModelSpecInternal &model = modelMerged.getModel();
     const unsigned int batchSize = model.getBatchSize();
     const auto scalar = model.getPrecision();
@@ -1176,6 +1184,14 @@ void Backend::genDefinitionsPreamble(CodeStream &os, const ModelSpecMerged&) con
     os << std::endl;
     os << "// MI355X device library" << std::endl;
     os << "#include \"genn_mi355x.h\"" << std::endl;
+    if(m_GeneratedKernels) {
+        os << "// building blocks of the generated kernels (every module is compiled with hipcc)" << std::endl;
+        os << "#include \"genn_mi355x_kernel_support.h\"" << std::endl;
+        os << "extern bool gennmiStructsDirty;" << std::endl;
+        os << "void gennmiUploadNeuronGroups();" << std::endl;
+        os << "void gennmiUploadSynapseGroups();" << std::endl;
+        os << "void gennmiCheckNeuronKernels();" << std::endl;
+    }
     os << "#define GENNMI_CHECK(call) do { if((call) != GENNMI_OK) { throw std::runtime_error(std::string(__FILE__) + \": \" + std::to_string(__LINE__) + \": \" + gennmi_last_error()); } } while(0)" << std::endl;
     os << std::endl;
     os << "extern gennmi_runner *gennmiRunner;" << std::endl;
@@ -1210,6 +1226,24 @@ void Backend::genRunnerPreamble(CodeStream &os, const ModelSpecMerged&) const
         os << "gennmiScratchBuffers.push_back(p);" << std::endl;
         os << "return (uint32_t*)p;" << std::endl;
     }
+    if(m_GeneratedKernels) {
+        os << "// device copies of the merged-group struct arrays: uploaded before the first step and after every push of a dynamic field" << std::endl;
+        os << "bool gennmiStructsDirty = true;" << std::endl;
+        os << "void gennmiBuildNeuronGroups() {}" << std::endl;
+        os << "void gennmiBuildSynapseGroups() {}" << std::endl;
+        os << "void gennmiEnsureFinalised()";
+        {
+            CodeStream::Scope b(os);
+            os << "if(!gennmiStructsDirty) { return; }" << std::endl;
+            os << "GENNMI_CHECK(gennmi_synchronize());" << std::endl;
+            os << "gennmiUploadNeuronGroups();" << std::endl;
+            os << "gennmiUploadSynapseGroups();" << std::endl;
+            os << "gennmiStructsDirty = false;" << std::endl;
+            os << "gennmiFinalised = true;" << std::endl;
+        }
+        os << std::endl;
+        return;
+    }
     os << "// every merged update group becomes descriptors of the device library, once, before the first step" << std::endl;
     os << "void gennmiEnsureFinalised()";
     {
@@ -1217,6 +1251,9 @@ void Backend::genRunnerPreamble(CodeStream &os, const ModelSpecMerged&) const
         os << "if(gennmiFinalised) { return; }" << std::endl;
         os << "gennmiBuildNeuronGroups();" << std::endl;
         os << "gennmiBuildSynapseGroups();" << std::endl;
+        if(getPreferences<Preferences>().orderedAccumulation) {
+            os << "GENNMI_CHECK(gennmi_runner_set_ordered(gennmiRunner, 1));" << std::endl;
+        }
         os << "GENNMI_CHECK(gennmi_runner_finalise(gennmiRunner));" << std::endl;
         os << "gennmiFinalised = true;" << std::endl;
     }
@@ -1227,6 +1264,10 @@ void Backend::genAllocateMemPreamble(CodeStream &os, const ModelSpecMerged &mode
 {
     const ModelSpecInternal &model = modelMerged.getModel();
     os << "GENNMI_CHECK(gennmi_init(" << getPreferences<Preferences>().deviceID << "));" << std::endl;
+    if(m_GeneratedKernels) {
+        os << "gennmiStructsDirty = true;" << std::endl;
+        return;
+    }
     os << "GENNMI_CHECK(gennmi_runner_create(&gennmiRunner, " << Type::writeNumeric(model.getDT(), model.getTimePrecision()) << ", " << model.getBatchSize() << "u));" << std::endl;
     if(model.isTimingEnabled()) {
         os << "GENNMI_CHECK(gennmi_runner_set_timing(gennmiRunner, 1));" << std::endl;
@@ -1243,6 +1284,14 @@ void Backend::genFreeMemPreamble(CodeStream &os, const ModelSpecMerged&) const
 //--------------------------------------------------------------------------
 void Backend::genStepTimeFinalisePreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const
 {
+    if(m_GeneratedKernels) {
+        // (kernel timers are not generated: the counters of such a runner stay 0)
+        if(modelMerged.getModel().isTimingEnabled()) {
+            os << "GENNMI_CHECK(gennmi_synchronize());" << std::endl;
+            os << "gennmiCheckNeuronKernels();" << std::endl;
+        }
+        return;
+    }
     // the reference's device backends synchronise here too when timing (backendCUDAHIP.cc:1400-1411)
     if(modelMerged.getModel().isTimingEnabled()) {
         os << "GENNMI_CHECK(gennmi_runner_synchronize(gennmiRunner));" << std::endl;
@@ -1283,6 +1332,7 @@ void Backend::genMergedDynamicVariablePush(CodeStream &os, const std::string &su
                                            const std::string &egpName) const
 {
     os << "merged" << suffix << "Group" << mergedGroupIdx << "[" << groupIdx << "]." << fieldName << " = " << egpName << ";" << std::endl;
+    if(m_GeneratedKernels) { os << "gennmiStructsDirty = true;" << std::endl; }
 }
 //--------------------------------------------------------------------------
 std::string Backend::getAtomicOperation(const std::string &lhsPointer, const std::string &rhsValue,
@@ -1321,8 +1371,14 @@ void Backend::genMakefilePreamble(std::ostream &os) const
     }
     std::string cxxFlags = "-c -fPIC -std=c++17 -MMD -MP -I\"" + root + "/include\" " + getPreferences().userCxxFlagsGNU;
     cxxFlags += getPreferences().debugCode ? " -O0 -g" : " -O2";
+    if(m_GeneratedKernels) {
+        // every module holds or calls device code: hipcc for gfx950, fp32 operations neither contracted nor packed so that
+        // results match the SingleThreadedCPU backend's operation for operation
+        os << "CXX := " << (std::getenv("HIP_PATH") ? std::string(std::getenv("HIP_PATH")) + "/bin/hipcc" : std::string("hipcc")) << std::endl;
+        cxxFlags += " -x hip --offload-arch=gfx950 -ffp-contract=off -Xclang -target-feature -Xclang -packed-fp32-ops -Wno-unused-value";
+    }
     os << "CXXFLAGS := " << cxxFlags << std::endl;
-    os << "LINKFLAGS := -shared" << std::endl;
+    os << "LINKFLAGS := -shared" << (m_GeneratedKernels ? " --offload-arch=gfx950 -fPIC" : "") << std::endl;
     os << "LINKLIBS := -L\"" << root << "/genn_amd/lib\" -lgenn_mi355x -Wl,-rpath,\"" << root << "/genn_amd/lib\"" << std::endl;
     os << std::endl;
 }
@@ -1370,7 +1426,7 @@ boost::uuids::detail::sha1::digest_type Backend::getHashDigest() const
 //--------------------------------------------------------------------------
 namespace Optimiser
 {
-Backend createBackend(const ModelSpecInternal&, const filesystem::path&, plog::Severity backendLevel,
+Backend createBackend(const ModelSpecInternal &model, const filesystem::path&, plog::Severity backendLevel,
                       plog::IAppender *backendAppender, const Preferences &preferences)
 {
     if(plog::get<Logging::CHANNEL_BACKEND>() == nullptr) {
@@ -1379,7 +1435,45 @@ Backend createBackend(const ModelSpecInternal&, const filesystem::path&, plog::S
     else {
         plog::get<Logging::CHANNEL_BACKEND>()->setMaxSeverity(backendLevel);
     }
-    return Backend(preferences);
+    bool generated = (preferences.kernelSource == Preferences::KernelSource::GENERATED);
+    if(preferences.kernelSource == Preferences::KernelSource::AUTO) {
+        // generated kernels when some snippet of the model is not one the device library implements ...
+        auto recognised = [](auto fn) { try { fn(); return true; } catch(const std::runtime_error&) { return false; } };
+        for(const auto &n : model.getNeuronGroups()) {
+            generated = generated || !recognised([&]{ recogniseNeuron(n.second.getModel(), n.first); });
+            for(const auto *cs : n.second.getCurrentSources()) {
+                const std::string code = cs->getModel()->getInjectionCode();
+                const bool known = same(code, CurrentSourceModels::DC::getInstance()->getInjectionCode()) || same(code, CurrentSourceModels::PoissonExp::getInstance()->getInjectionCode())
+                                   || (same(code, "injectCurrent(noise[id]);") && cs->getModel()->getExtraGlobalParams().size() == 1);
+                generated = generated || !known;
+            }
+        }
+        for(const auto &s : model.getSynapseGroups()) {
+            generated = generated || !recognised([&]{ recognisePSM(s.second.getPSInitialiser().getSnippet(), s.first); });
+            generated = generated || !recognised([&]{ recogniseWUM(s.second.getWUInitialiser().getSnippet(), s.first); });
+        }
+        // ... or when a parameter is dynamic: the library's descriptors hold parameters as constants, generated kernels read
+        // them from the merged structs that setDynamicParamValue rewrites
+        auto anyDynamic = [](const auto &params, auto isDynamic)
+        {
+            return std::any_of(params.cbegin(), params.cend(), [&](const auto &p) { return isDynamic(p.name); });
+        };
+        for(const auto &n : model.getNeuronGroups()) {
+            generated = generated || anyDynamic(n.second.getModel()->getParams(), [&](const std::string &p) { return n.second.isParamDynamic(p); });
+            for(const auto *cs : n.second.getCurrentSources()) {
+                generated = generated || anyDynamic(cs->getModel()->getParams(), [&](const std::string &p) { return cs->isParamDynamic(p); });
+            }
+        }
+        for(const auto &s : model.getSynapseGroups()) {
+            generated = generated || anyDynamic(s.second.getPSInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isPSParamDynamic(p); });
+            generated = generated || anyDynamic(s.second.getWUInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isWUParamDynamic(p); });
+        }
+        if(generated) { LOGI_BACKEND << "The model uses snippets the device library does not implement, or dynamic parameters: the step's kernels are generated from the model's code"; }
+    }
+    if(generated && preferences.orderedAccumulation) {
+        throw std::runtime_error("MI355X backend: ordered accumulation is a mode of the device library's kernels, not of generated ones");
+    }
+    return Backend(preferences, generated);
 }
 }   // namespace Optimiser
 }   // namespace GeNN::CodeGenerator::MI355X

@@ -30,10 +30,23 @@ struct Preferences : public PreferencesBase
     //! (empty: the GENN_MI355X_ROOT environment variable at code-generation time)
     std::string installRoot;
 
+    //! Where the step's device code comes from.  LIBRARY: every neuron, postsynaptic, current-source and weight-update model
+    //! must be one the device library implements (anything else is refused); the runner is host code.  GENERATED: kernels
+    //! are generated from the model's own code strings for every group and compiled with hipcc into the runner.  AUTO:
+    //! LIBRARY when every snippet of the model is recognised, GENERATED otherwise.
+    enum class KernelSource { AUTO, LIBRARY, GENERATED };
+    KernelSource kernelSource = KernelSource::AUTO;
+
+    //! Validation mode of the device library: synaptic input is summed per postsynaptic neuron in the order of the
+    //! SingleThreadedCPU backend, without atomics (gennmi_runner_set_ordered); LIBRARY kernels only
+    bool orderedAccumulation = false;
+
     void updateHash(boost::uuids::detail::sha1 &hash) const
     {
         PreferencesBase::updateHash(hash);
         Utils::updateHash(deviceID, hash);
+        Utils::updateHash(static_cast<int>(kernelSource), hash);
+        Utils::updateHash(orderedAccumulation, hash);
     }
 };
 
@@ -44,7 +57,10 @@ class State : public Runtime::StateBase
 class BACKEND_EXPORT Backend : public BackendBase
 {
 public:
-    Backend(const Preferences &preferences);
+    //! `generatedKernels`: the step's kernels are generated from the model's code (see Preferences::kernelSource)
+    Backend(const Preferences &preferences, bool generatedKernels = false);
+
+    bool areKernelsGenerated() const { return m_GeneratedKernels; }
 
     //--------------------------------------------------------------------------
     // BackendBase virtuals
@@ -124,5 +140,12 @@ public:
     virtual size_t getDeviceMemoryBytes() const final;
     virtual MemorySpaces getMergedGroupMemorySpaces(const ModelSpecMerged &modelMerged) const final { return {}; }
     virtual boost::uuids::detail::sha1::digest_type getHashDigest() const final;
+
+private:
+    // generated.cc: kernels printed from the model's own code into this backend's skeletons
+    void genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMerged, BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const;
+    void genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMerged, BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const;
+
+    const bool m_GeneratedKernels;
 };
 }   // namespace GeNN::CodeGenerator::MI355X

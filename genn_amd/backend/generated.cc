@@ -1,0 +1,512 @@
+// GeNN::CodeGenerator::MI355X::Backend — generated kernels.
+//
+// For models whose snippets the device library does not implement, the step's device code is generated: the model's own
+// code strings — sim / threshold / reset code, postsynaptic and current-source code, weight-update code with its pre and
+// post variables — are printed by GeNN's environments and pretty-printer (the transpiler stays in libgenn:
+// NeuronUpdateGroupMerged::generateNeuronUpdate, PresynapticUpdateGroupMerged::generateSpikeUpdate, ...) into the
+// skeletons emitted here, and the resulting translation unit is compiled for gfx950 with hipcc as part of the runner.
+//
+// Skeletons (what the reference's SIMT backends generate in src/genn/genn/code_generator/backendSIMT.cc:405-803, designed
+// anew for 64-wide wavefronts):
+//   neuron update        one lane per neuron; the model's code sets a flag where the reference appends to a shared-memory
+//                        list; the flags are compacted in ascending neuron index by wave ballot, LDS scan and a tagged
+//                        look-back across work-groups (include/genn_mi355x_kernel_support.h), once per population, and
+//                        every spike queue of the population is written from the same positions; the ballot is the
+//                        recording bitfield.  No spike-queue reset kernel: the population's last work-group stores the count.
+//   presynaptic update   (spike, 64-synapse chunk of its row) items dealt round-robin to the wavefronts of a group's
+//                        work-groups: a lane owns one synapse, loads of ind and the synapse variables are coalesced, a long
+//                        row is shared by many wavefronts.  addToPost / addToPostDelay / addToPre are fp32 atomics.
+//   postsynaptic update  (postsynaptic spike, 64-entry chunk of its column) items through the column view (remap).
+//   dendritic delay      one thread per group advances the ring pointer.
+// Merged-group structs are GeNN's own (same fields, same push functions); a device copy of every struct array, with host
+// pointers replaced by the device buffers registered behind them, is uploaded before the first step and again whenever a
+// dynamic field is pushed.  Initialisation is unchanged (the reference's generic host code, then an upload).
+#include "backend.h"
+
+#include <algorithm>
+#include <sstream>
+#include <stdexcept>
+
+#include "code_generator/codeStream.h"
+#include "code_generator/modelSpecMerged.h"
+#include "code_generator/standardLibrary.h"
+
+using namespace GeNN;
+using namespace GeNN::CodeGenerator;
+
+namespace
+{
+[[noreturn]] void notGenerated(const std::string &what)
+{
+    throw std::runtime_error("MI355X backend: generated kernels do not cover " + what);
+}
+
+// block table of one kernel: {group, first id, block in group, blocks in group} per work-group, merged groups back to back
+struct BlockTable
+{
+    std::ostringstream entries;
+    size_t numBlocks = 0;
+    void add(size_t group, size_t firstId, size_t blockInGroup, size_t blocksInGroup)
+    {
+        entries << "{" << group << "u, " << firstId << "u, " << blockInGroup << "u, " << blocksInGroup << "u}, ";
+        if((++numBlocks % 4) == 0) { entries << std::endl; }
+    }
+};
+
+// device copy of a merged group's struct array: declaration, and the statements that translate and upload it
+template<typename G>
+void genDeviceStructArray(CodeStream &decl, CodeStream &upload, const BackendBase &backend, const G &g, const std::string &name)
+{
+    const std::string type = "Merged" + name + "Group" + std::to_string(g.getIndex());
+    const std::string host = "merged" + name + "Group" + std::to_string(g.getIndex());
+    const std::string dev = "d_" + host;
+    const size_t count = g.getGroups().size();
+    decl << "static " << type << " *" << dev << " = nullptr;" << std::endl;
+    upload << "// " << host << std::endl;
+    {
+        CodeStream::Scope b(upload);
+        upload << "static " << type << " staging[" << count << "];" << std::endl;
+        upload << "for(unsigned int g = 0; g < " << count << "; g++)";
+        {
+            CodeStream::Scope b2(upload);
+            upload << "staging[g] = " << host << "[g];" << std::endl;
+            for(const auto &f : g.getSortedFields(backend)) {
+                if(f.type.isPointer()) {
+                    upload << "staging[g]." << f.name << " = gennmiDev(staging[g]." << f.name << ");" << std::endl;
+                }
+            }
+        }
+        upload << "if(!" << dev << ") { void *p = nullptr; GENNMI_CHECK(gennmi_malloc(&p, sizeof(staging))); " << dev << " = (" << type << "*)p; }" << std::endl;
+        upload << "GENNMI_CHECK(gennmi_memcpy_to_device(" << dev << ", staging, sizeof(staging)));" << std::endl;
+    }
+}
+}   // anonymous namespace
+
+namespace GeNN::CodeGenerator::MI355X
+{
+//--------------------------------------------------------------------------
+void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMerged, BackendBase::MemorySpaces &memorySpaces,
+                                       HostHandler preambleHandler) const
+{
+    const ModelSpecInternal &model = modelMerged.getModel();
+    if(model.getBatchSize() != 1) { notGenerated("batch sizes above 1"); }
+    if(model.getPrecision() != Type::Float || model.getTimePrecision() != Type::Float) { notGenerated("double precision"); }
+    const bool recording = model.isRecordingInUse();
+
+    std::ostringstream kernelStream, declStream, uploadStream, argStream, paramStream;
+    CodeStream kernel(kernelStream), decl(declStream), upload(uploadStream);
+    BlockTable table;
+
+    EnvironmentLibrary kernelEnv(kernel, StandardLibrary::getMathsFunctions());
+    {   // (environments write what they hold when they go out of scope: the kernel's text is complete after this block)
+    EnvironmentExternal funcEnv(kernelEnv);
+    funcEnv.add(model.getTimePrecision().addConst(), "t", "t");
+    funcEnv.add(Type::Uint32.addConst(), "batch", "0");
+    funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
+
+    modelMerged.genMergedNeuronUpdateGroups(
+        *this, memorySpaces,
+        [&](auto &n)
+        {
+            const auto &arch = n.getArchetype();
+            if(arch.isDelayRequired()) { notGenerated("axonal delay slots (population '" + arch.getName() + "')"); }
+            if(arch.isSimRNGRequired()) { notGenerated("random numbers in the update of population '" + arch.getName() + "'"); }
+            if(arch.isPrevSpikeTimeRequired() || arch.isSpikeEventTimeRequired() || arch.isPrevSpikeEventTimeRequired()) {
+                notGenerated("previous spike times and spike-like event times (population '" + arch.getName() + "')");
+            }
+            if(!n.getMergedSpikeEventGroups().empty()) { notGenerated("spike-like events (population '" + arch.getName() + "')"); }
+
+            const size_t firstBlock = table.numBlocks;
+            for(size_t g = 0; g < n.getGroups().size(); g++) {
+                const size_t num = n.getGroups()[g].get().getNumNeurons();
+                const size_t blocks = (num + 255) / 256;
+                for(size_t b = 0; b < blocks; b++) { table.add(g, b * 256, b, blocks); }
+            }
+            const std::string structArray = "mergedNeuronUpdateGroup" + std::to_string(n.getIndex());
+            argStream << ", d_" << structArray;
+            paramStream << ", const MergedNeuronUpdateGroup" << n.getIndex() << " *" << structArray;
+
+            funcEnv.getStream() << "// merged neuron update group " << n.getIndex() << std::endl;
+            funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << table.numBlocks << "u)";
+            CodeStream::Scope b(funcEnv.getStream());
+            funcEnv.getStream() << "const gennmi_kernel::BlockEntry entry = gennmiNeuronBlocks[blockIdx.x];" << std::endl;
+            funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
+            funcEnv.getStream() << "const unsigned int id = entry.firstId + threadIdx.x;" << std::endl;
+            funcEnv.getStream() << "bool gennmiSpiked = false;" << std::endl;
+
+            EnvironmentGroupMergedField<NeuronUpdateGroupMerged> groupEnv(funcEnv, n);
+            buildStandardEnvironment(groupEnv, 1);
+            groupEnv.add(Type::Uint32.addConst(), "id", "id");
+            if(arch.isSpikeRecordingEnabled()) {
+                groupEnv.printLine("const unsigned int numRecordingWords = ($(num_neurons) + 31) / 32;");
+            }
+            groupEnv.print("if($(id) < $(num_neurons))");
+            {
+                CodeStream::Scope b2(groupEnv.getStream());
+                n.generateNeuronUpdate(
+                    groupEnv, 1,
+                    // a true spike: weight-update pre / post spike code, spike time; the queue is written after the
+                    // population's flags have been compacted (below), the recording word comes from the ballot
+                    [&n, &arch](EnvironmentExternalBase &env)
+                    {
+                        n.generateWUVarUpdate(env, 1);
+                        if(arch.isSpikeTimeRequired()) { env.printLine("$(_st)[$(id)] = $(t);"); }
+                        env.getStream() << "gennmiSpiked = true;" << std::endl;
+                    },
+                    [](EnvironmentExternalBase&, NeuronUpdateGroupMerged::SynSpikeEvent&) {});
+            }
+            groupEnv.printLine("const gennmi_kernel::QueueSlot slot = gennmi_kernel::orderedSlot(gennmiSpiked, entry.blockInGroup, entry.blocksInGroup, "
+                               "blockIdx.x - entry.blockInGroup, gennmiAgg, gennmiAgg + gridDim.x, gennmiTag, gennmiError);");
+            if(arch.isSpikeRecordingEnabled()) {
+                groupEnv.printLine("gennmi_kernel::recordBallot(&$(_record_spk)[recordingTimestep * numRecordingWords], $(id), $(id) < $(num_neurons), slot.ballot);");
+            }
+            // every spike queue of the population (one per fused outgoing / incoming spike target) from the same positions
+            n.generateSpikes(
+                groupEnv,
+                [](EnvironmentExternalBase &env)
+                {
+                    env.print("if(slot.ok)");
+                    CodeStream::Scope b3(env.getStream());
+                    env.printLine("if(gennmiSpiked) { $(_spk)[slot.position] = $(id); }");
+                    env.printLine("if(slot.writeTotal) { $(_spk_cnt)[0] = slot.total; }");
+                });
+        });
+    }
+
+    // struct definitions, host arrays and their push functions are GeNN's own
+    modelMerged.genMergedNeuronUpdateGroupStructs(os, *this);
+    modelMerged.genMergedNeuronUpdateGroupHostStructArrayPush(os, *this);
+    preambleHandler(os);
+    for(const auto &n : modelMerged.getMergedNeuronUpdateGroups()) {
+        genDeviceStructArray(decl, upload, *this, n, "NeuronUpdate");
+    }
+
+    os << declStream.str();
+    os << "static unsigned long long *gennmiNeuronAgg = nullptr;" << std::endl;
+    os << "static uint32_t *gennmiNeuronError = nullptr;" << std::endl;
+    os << "static unsigned int gennmiNeuronLaunches = 0;" << std::endl;
+    os << "__device__ const gennmi_kernel::BlockEntry gennmiNeuronBlocks[] = {" << std::endl << table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+    os << std::endl;
+    os << "void gennmiUploadNeuronGroups()";
+    {
+        CodeStream::Scope b(os);
+        os << uploadStream.str();
+        os << "if(!gennmiNeuronAgg)";
+        {
+            CodeStream::Scope b2(os);
+            os << "void *p = nullptr;" << std::endl;
+            os << "GENNMI_CHECK(gennmi_malloc(&p, " << 2 * std::max<size_t>(1, table.numBlocks) << " * sizeof(unsigned long long)));" << std::endl;
+            os << "GENNMI_CHECK(gennmi_memset(p, 0, " << 2 * std::max<size_t>(1, table.numBlocks) << " * sizeof(unsigned long long)));" << std::endl;
+            os << "gennmiNeuronAgg = (unsigned long long*)p;" << std::endl;
+            os << "GENNMI_CHECK(gennmi_malloc(&p, sizeof(uint32_t)));" << std::endl;
+            os << "GENNMI_CHECK(gennmi_memset(p, 0, sizeof(uint32_t)));" << std::endl;
+            os << "gennmiNeuronError = (uint32_t*)p;" << std::endl;
+        }
+    }
+    os << std::endl;
+    os << "__global__ __launch_bounds__(256) void gennmiNeuronUpdateKernel(float t, unsigned int recordingTimestep, uint32_t gennmiTag, "
+          "unsigned long long *gennmiAgg, uint32_t *gennmiError" << paramStream.str() << ")";
+    {
+        CodeStream::Scope b(os);
+        os << kernelStream.str();
+    }
+    os << std::endl;
+    os << "void updateNeurons(" << model.getTimePrecision().getName() << " t";
+    if(recording) { os << ", unsigned int recordingTimestep"; }
+    os << ")";
+    {
+        CodeStream::Scope b(os);
+        os << "gennmiEnsureFinalised();" << std::endl;
+        if(table.numBlocks > 0) {
+            // the tag of a launch: differs from one launch to the next, never 0 (the look-back words start out zero)
+            os << "gennmiNeuronLaunches = (gennmiNeuronLaunches == 0xFFFFFFFFu) ? 1u : gennmiNeuronLaunches + 1u;" << std::endl;
+            os << "gennmiNeuronUpdateKernel<<<dim3(" << table.numBlocks << "), dim3(256), 0, 0>>>(t, " << (recording ? "recordingTimestep" : "0u")
+               << ", gennmiNeuronLaunches, gennmiNeuronAgg, gennmiNeuronError" << argStream.str() << ");" << std::endl;
+            os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateNeurons: kernel launch failed\"); }" << std::endl;
+        }
+    }
+    os << std::endl;
+    // bounded waits of the compaction that expired are reported where the reference's backends check for launch errors
+    os << "void gennmiCheckNeuronKernels()";
+    {
+        CodeStream::Scope b(os);
+        os << "if(!gennmiNeuronError) { return; }" << std::endl;
+        os << "uint32_t flag = 0;" << std::endl;
+        os << "GENNMI_CHECK(gennmi_memcpy_from_device(&flag, gennmiNeuronError, sizeof(flag)));" << std::endl;
+        os << "if(flag) { throw std::runtime_error(\"updateNeurons: a work-group's bounded wait for spike-queue offsets expired\"); }" << std::endl;
+    }
+}
+//--------------------------------------------------------------------------
+void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMerged, BackendBase::MemorySpaces &memorySpaces,
+                                        HostHandler preambleHandler) const
+{
+    const ModelSpecInternal &model = modelMerged.getModel();
+    const double dt = model.getDT();
+
+    std::ostringstream declStream, uploadStream;
+    CodeStream decl(declStream), upload(uploadStream);
+
+    // every kernel's body, arguments and block table
+    struct KernelText
+    {
+        std::ostringstream body, args, params;
+        BlockTable table;
+    };
+    KernelText delay, pre, post;
+    auto makeEnv = [&model](CodeStream &stream, EnvironmentLibrary &lib, auto use)
+    {
+        EnvironmentExternal funcEnv(lib);
+        funcEnv.add(model.getTimePrecision().addConst(), "t", "t");
+        funcEnv.add(Type::Uint32.addConst(), "batch", "0");
+        funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
+        (void)stream;
+        use(funcEnv);
+    };
+
+    modelMerged.genMergedSynapseDynamicsGroups(
+        *this, memorySpaces,
+        [](auto &s) { notGenerated("synapse dynamics code (projection '" + s.getArchetype().getName() + "')"); });
+
+    // ---- dendritic delay pointers: one thread per group
+    {
+        CodeStream stream(delay.body);
+        EnvironmentLibrary lib(stream, StandardLibrary::getMathsFunctions());
+        makeEnv(stream, lib, [&](EnvironmentExternal &funcEnv)
+        {
+            modelMerged.genMergedSynapseDendriticDelayUpdateGroups(
+                *this, memorySpaces,
+                [&](auto &sg)
+                {
+                    const std::string structArray = "mergedSynapseDendriticDelayUpdateGroup" + std::to_string(sg.getIndex());
+                    delay.table.numBlocks++;
+                    delay.args << ", d_" << structArray;
+                    delay.params << ", const MergedSynapseDendriticDelayUpdateGroup" << sg.getIndex() << " *" << structArray;
+                    funcEnv.getStream() << "for(unsigned int g = threadIdx.x; g < " << sg.getGroups().size() << "u; g += blockDim.x)";
+                    CodeStream::Scope b(funcEnv.getStream());
+                    funcEnv.getStream() << "const auto *group = &" << structArray << "[g];" << std::endl;
+                    EnvironmentGroupMergedField<SynapseDendriticDelayUpdateGroupMerged> groupEnv(funcEnv, sg);
+                    buildStandardEnvironment(groupEnv, 1);
+                    sg.generateSynapseUpdate(groupEnv);
+                });
+        });
+    }
+
+    // ---- presynaptic update
+    {
+        CodeStream stream(pre.body);
+        EnvironmentLibrary lib(stream, StandardLibrary::getMathsFunctions());
+        makeEnv(stream, lib, [&](EnvironmentExternal &funcEnv)
+        {
+            modelMerged.genMergedPresynapticUpdateGroups(
+                *this, memorySpaces,
+                [&](auto &s)
+                {
+                    const auto &arch = s.getArchetype();
+                    const auto matrix = arch.getMatrixType();
+                    const bool sparse = (matrix & SynapseMatrixConnectivity::SPARSE);
+                    const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
+                    if(!sparse && !dense) { notGenerated("connectivity other than SPARSE and DENSE (projection '" + arch.getName() + "')"); }
+                    if(arch.isPreSpikeEventRequired()) { notGenerated("spike-like events (projection '" + arch.getName() + "')"); }
+                    if(arch.getSrcNeuronGroup()->isDelayRequired() || arch.getTrgNeuronGroup()->isDelayRequired() || arch.getBackPropDelaySteps() != 0) {
+                        notGenerated("axonal or back-propagation delay (projection '" + arch.getName() + "')");
+                    }
+                    if(!arch.isPreSpikeRequired()) { return; }
+
+                    const size_t firstBlock = pre.table.numBlocks;
+                    for(size_t g = 0; g < s.getGroups().size(); g++) {
+                        const auto &sg = s.getGroups()[g].get();
+                        const size_t rowLen = sparse ? getSynapticMatrixRowStride(sg) : sg.getTrgNeuronGroup()->getNumNeurons();
+                        const size_t chunks = (rowLen + 63) / 64;
+                        // enough wavefronts for ~1.5 % of the source population firing in one step, at most 128 work-groups
+                        const size_t blocks = std::clamp<size_t>((sg.getSrcNeuronGroup()->getNumNeurons() * chunks + 255) / 256, 1, 128);
+                        for(size_t b = 0; b < blocks; b++) { pre.table.add(g, 0, b, blocks); }
+                    }
+                    const std::string structArray = "mergedPresynapticUpdateGroup" + std::to_string(s.getIndex());
+                    pre.args << ", d_" << structArray;
+                    pre.params << ", const MergedPresynapticUpdateGroup" << s.getIndex() << " *" << structArray;
+
+                    funcEnv.getStream() << "// merged presynaptic update group " << s.getIndex() << std::endl;
+                    funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << pre.table.numBlocks << "u)";
+                    CodeStream::Scope b(funcEnv.getStream());
+                    funcEnv.getStream() << "const gennmi_kernel::BlockEntry entry = gennmiPresynapticBlocks[blockIdx.x];" << std::endl;
+                    funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
+                    EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> groupEnv(funcEnv, s);
+                    buildStandardEnvironment(groupEnv, 1);
+                    groupEnv.printLine("const unsigned int numSpikes = $(_src_spk_cnt)[0];");
+                    groupEnv.printLine(std::string("const unsigned int rowSpan = ") + (sparse ? "$(_row_stride)" : "$(num_post)") + ";");
+                    groupEnv.getStream() << "const unsigned int chunksPerRow = (rowSpan + 63u) / 64u;" << std::endl;
+                    groupEnv.getStream() << "const unsigned int numWaves = entry.blocksInGroup * 4u;" << std::endl;
+                    groupEnv.getStream() << "const unsigned long long numItems = (unsigned long long)numSpikes * chunksPerRow;" << std::endl;
+                    groupEnv.getStream() << "for(unsigned long long item = entry.blockInGroup * 4u + (threadIdx.x / 64u); item < numItems; item += numWaves)";
+                    {
+                        CodeStream::Scope b2(groupEnv.getStream());
+                        EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> synEnv(groupEnv, s);
+                        synEnv.getStream() << "const unsigned int spike = (unsigned int)(item / chunksPerRow);" << std::endl;
+                        synEnv.getStream() << "const unsigned int j = (unsigned int)(item % chunksPerRow) * 64u + (threadIdx.x & 63u);" << std::endl;
+                        synEnv.printLine("const unsigned int idPre = $(_src_spk)[spike];");
+                        synEnv.add(Type::Uint32.addConst(), "id_pre", "idPre");
+                        const auto indexType = getSynapseIndexType(s);
+                        const std::string indexTypeName = indexType.getName();
+                        if(sparse) {
+                            synEnv.print("if(j < $(_row_length)[idPre])");
+                        }
+                        else {
+                            synEnv.print("if(j < $(num_post))");
+                        }
+                        {
+                            CodeStream::Scope b3(synEnv.getStream());
+                            EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> codeEnv(synEnv, s);
+                            if(sparse) {
+                                codeEnv.add(indexType.addConst(), "id_syn", "idSyn",
+                                            {codeEnv.addInitialiser("const " + indexTypeName + " idSyn = ((" + indexTypeName + ")idPre * $(_row_stride)) + j;")});
+                                codeEnv.add(Type::Uint32.addConst(), "id_post", "idPost",
+                                            {codeEnv.addInitialiser("const unsigned int idPost = $(_ind)[$(id_syn)];")});
+                            }
+                            else {
+                                codeEnv.add(Type::Uint32.addConst(), "id_post", "j");
+                                codeEnv.add(indexType.addConst(), "id_syn", "idSyn",
+                                            {codeEnv.addInitialiser("const " + indexTypeName + " idSyn = ((" + indexTypeName + ")idPre * $(num_post)) + j;")});
+                            }
+                            codeEnv.add(Type::getAddToPrePostDelay(s.getScalarType()), "addToPostDelay",
+                                        "gennmi_kernel::addScalar(&$(_den_delay)[" + s.getPostDenDelayIndex(1, "$(id_post)", "$(1)") + "], $(0))");
+                            codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPost",
+                                        "gennmi_kernel::addScalar(&$(_out_post)[" + s.getPostISynIndex(1, "$(id_post)") + "], $(0))");
+                            codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
+                                        "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(1, "$(id_pre)") + "], $(0))");
+                            s.generateSpikeUpdate(*this, codeEnv, 1, dt);
+                        }
+                    }
+                });
+        });
+    }
+
+    // ---- postsynaptic update (learnPost) through the column view
+    {
+        CodeStream stream(post.body);
+        EnvironmentLibrary lib(stream, StandardLibrary::getMathsFunctions());
+        makeEnv(stream, lib, [&](EnvironmentExternal &funcEnv)
+        {
+            modelMerged.genMergedPostsynapticUpdateGroups(
+                *this, memorySpaces,
+                [&](auto &s)
+                {
+                    const auto &arch = s.getArchetype();
+                    const auto matrix = arch.getMatrixType();
+                    const bool sparse = (matrix & SynapseMatrixConnectivity::SPARSE);
+                    const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
+                    if(!sparse && !dense) { notGenerated("connectivity other than SPARSE and DENSE (projection '" + arch.getName() + "')"); }
+                    if(arch.isPostSpikeEventRequired()) { notGenerated("spike-like events (projection '" + arch.getName() + "')"); }
+                    if(!arch.isPostSpikeRequired()) { return; }
+
+                    const size_t firstBlock = post.table.numBlocks;
+                    for(size_t g = 0; g < s.getGroups().size(); g++) {
+                        const auto &sg = s.getGroups()[g].get();
+                        const size_t colLen = sparse ? sg.getMaxSourceConnections() : sg.getSrcNeuronGroup()->getNumNeurons();
+                        const size_t chunks = (colLen + 63) / 64;
+                        const size_t blocks = std::clamp<size_t>((sg.getTrgNeuronGroup()->getNumNeurons() * chunks + 255) / 256, 1, 128);
+                        for(size_t b = 0; b < blocks; b++) { post.table.add(g, 0, b, blocks); }
+                    }
+                    const std::string structArray = "mergedPostsynapticUpdateGroup" + std::to_string(s.getIndex());
+                    post.args << ", d_" << structArray;
+                    post.params << ", const MergedPostsynapticUpdateGroup" << s.getIndex() << " *" << structArray;
+
+                    funcEnv.getStream() << "// merged postsynaptic update group " << s.getIndex() << std::endl;
+                    funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << post.table.numBlocks << "u)";
+                    CodeStream::Scope b(funcEnv.getStream());
+                    funcEnv.getStream() << "const gennmi_kernel::BlockEntry entry = gennmiPostsynapticBlocks[blockIdx.x];" << std::endl;
+                    funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
+                    EnvironmentGroupMergedField<PostsynapticUpdateGroupMerged> groupEnv(funcEnv, s);
+                    buildStandardEnvironment(groupEnv, 1);
+                    groupEnv.printLine("const unsigned int numSpikes = $(_trg_spk_cnt)[0];");
+                    groupEnv.printLine(std::string("const unsigned int colSpan = ") + (sparse ? "$(_col_stride)" : "$(num_pre)") + ";");
+                    groupEnv.getStream() << "const unsigned int chunksPerCol = (colSpan + 63u) / 64u;" << std::endl;
+                    groupEnv.getStream() << "const unsigned int numWaves = entry.blocksInGroup * 4u;" << std::endl;
+                    groupEnv.getStream() << "const unsigned long long numItems = (unsigned long long)numSpikes * chunksPerCol;" << std::endl;
+                    groupEnv.getStream() << "for(unsigned long long item = entry.blockInGroup * 4u + (threadIdx.x / 64u); item < numItems; item += numWaves)";
+                    {
+                        CodeStream::Scope b2(groupEnv.getStream());
+                        EnvironmentGroupMergedField<PostsynapticUpdateGroupMerged> synEnv(groupEnv, s);
+                        synEnv.printLine("const unsigned int spike = $(_trg_spk)[(unsigned int)(item / chunksPerCol)];");
+                        synEnv.getStream() << "const unsigned int i = (unsigned int)(item % chunksPerCol) * 64u + (threadIdx.x & 63u);" << std::endl;
+                        if(sparse) {
+                            synEnv.print("if(i < $(_col_length)[spike])");
+                        }
+                        else {
+                            synEnv.print("if(i < $(num_pre))");
+                        }
+                        {
+                            CodeStream::Scope b3(synEnv.getStream());
+                            EnvironmentGroupMergedField<PostsynapticUpdateGroupMerged> codeEnv(synEnv, s);
+                            if(sparse) {
+                                const size_t colMajor = codeEnv.addInitialiser("const unsigned int colMajorIndex = (spike * $(_col_stride)) + i;");
+                                const size_t rowMajor = codeEnv.addInitialiser("const unsigned int rowMajorIndex = $(_remap)[colMajorIndex];");
+                                const size_t idPre = codeEnv.addInitialiser("const unsigned int idPre = rowMajorIndex / $(_row_stride);");
+                                codeEnv.add(Type::Uint32.addConst(), "id_pre", "idPre", {colMajor, rowMajor, idPre});
+                                codeEnv.add(Type::Uint32.addConst(), "id_syn", "rowMajorIndex", {colMajor, rowMajor});
+                            }
+                            else {
+                                codeEnv.add(Type::Uint32.addConst(), "id_pre", "i");
+                                codeEnv.add(Type::Uint32.addConst(), "id_syn", "idSyn",
+                                            {codeEnv.addInitialiser("const unsigned int idSyn = (i * $(num_post)) + spike;")});
+                            }
+                            codeEnv.add(Type::Uint32.addConst(), "id_post", "spike");
+                            codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
+                                        "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(1, "$(id_pre)") + "], $(0))");
+                            s.generateSpikeUpdate(*this, codeEnv, 1, dt);
+                        }
+                    }
+                });
+        });
+    }
+
+    // struct definitions, host arrays and push functions (GeNN's own), then the device copies
+    modelMerged.genMergedSynapseDendriticDelayUpdateStructs(os, *this);
+    modelMerged.genMergedPresynapticUpdateGroupStructs(os, *this);
+    modelMerged.genMergedPostsynapticUpdateGroupStructs(os, *this);
+    modelMerged.genMergedSynapseDendriticDelayUpdateHostStructArrayPush(os, *this);
+    modelMerged.genMergedPresynapticUpdateGroupHostStructArrayPush(os, *this);
+    modelMerged.genMergedPostsynapticUpdateGroupHostStructArrayPush(os, *this);
+    preambleHandler(os);
+    for(const auto &g : modelMerged.getMergedSynapseDendriticDelayUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "SynapseDendriticDelayUpdate"); }
+    for(const auto &g : modelMerged.getMergedPresynapticUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "PresynapticUpdate"); }
+    for(const auto &g : modelMerged.getMergedPostsynapticUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "PostsynapticUpdate"); }
+
+    os << declStream.str();
+    os << "__device__ const gennmi_kernel::BlockEntry gennmiPresynapticBlocks[] = {" << std::endl << pre.table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+    os << "__device__ const gennmi_kernel::BlockEntry gennmiPostsynapticBlocks[] = {" << std::endl << post.table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+    os << std::endl;
+    os << "void gennmiUploadSynapseGroups()";
+    {
+        CodeStream::Scope b(os);
+        os << uploadStream.str();
+    }
+    os << std::endl;
+    const bool anyDelay = delay.table.numBlocks > 0, anyPre = pre.table.numBlocks > 0, anyPost = post.table.numBlocks > 0;
+    if(anyDelay) {
+        os << "__global__ void gennmiDendriticDelayUpdateKernel(float t" << delay.params.str() << ")";
+        CodeStream::Scope b(os);
+        os << delay.body.str();
+    }
+    if(anyPre) {
+        os << "__global__ __launch_bounds__(256) void gennmiPresynapticUpdateKernel(float t" << pre.params.str() << ")";
+        CodeStream::Scope b(os);
+        os << pre.body.str();
+    }
+    if(anyPost) {
+        os << "__global__ __launch_bounds__(256) void gennmiPostsynapticUpdateKernel(float t" << post.params.str() << ")";
+        CodeStream::Scope b(os);
+        os << post.body.str();
+    }
+    os << std::endl;
+    os << "void updateSynapses(" << model.getTimePrecision().getName() << " t)";
+    {
+        CodeStream::Scope b(os);
+        os << "gennmiEnsureFinalised();" << std::endl;
+        // order of the reference's updateSynapses (backendCUDAHIP.cc:548-589): ring pointers, presynaptic, postsynaptic
+        if(anyDelay) { os << "gennmiDendriticDelayUpdateKernel<<<dim3(1), dim3(64), 0, 0>>>(t" << delay.args.str() << ");" << std::endl; }
+        if(anyPre) { os << "gennmiPresynapticUpdateKernel<<<dim3(" << pre.table.numBlocks << "), dim3(256), 0, 0>>>(t" << pre.args.str() << ");" << std::endl; }
+        if(anyPost) { os << "gennmiPostsynapticUpdateKernel<<<dim3(" << post.table.numBlocks << "), dim3(256), 0, 0>>>(t" << post.args.str() << ");" << std::endl; }
+        os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateSynapses: kernel launch failed\"); }" << std::endl;
+    }
+}
+}   // namespace GeNN::CodeGenerator::MI355X

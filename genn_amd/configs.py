@@ -336,3 +336,30 @@ def dense_layer(n_in=8192, n_out=8192, rate_hz=50.0, steps=1000, seed=17, dt=1.0
     g = netgen.normal_f32(seed, 2, 0, n_in * n_out, 0.0, w_sd).reshape(n_in, n_out)
     net.syns.append(Syn("InOut", "In", "Out", matrix="dense", wum="static", psm="expcurr", tau=5.0, g=g))
     return net
+
+
+def custom_models(n_a=300, n_b=200, steps=300, seed=41, dt=1.0):
+    """A network of models that are NOT built into GeNN or into the device library — what a user writes with the model
+    API: LIF neurons with a spike-triggered adaptation variable ("lifa": the built-in LIF plus A, which decays every step,
+    is subtracted from the input and grows by dA at each spike), and a weight update model with a presynaptic and a
+    postsynaptic variable after tests/features/test_wu_vars.py ("timing_copy": each neuron's variable holds the time of
+    its last spike; a presynaptic spike delivers g and copies the target's variable into the row's synapses, a
+    postsynaptic spike copies the source's variable into its column).  Their code exists only as strings of the test
+    driver's model classes, so on the MI355X backend this network runs through generated kernels."""
+    lifa = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.9, TauRefrac=2.0, TauA=50.0, dA=0.12)
+    net = Net(name="custom", dt=dt, steps=steps, seed=seed)
+    for k, (name, n, ioff) in enumerate((("A", n_a, 0.9), ("B", n_b, 0.45))):
+        net.pops.append(Pop(name, "lifa", n, dict(lifa, Ioffset=ioff),
+                            {"V": (-60.0 + 9.5 * rng.uniform(seed, 1 + k, 0, n)).astype(np.float32), "RefracTime": np.zeros(n, np.float32),
+                             "A": (0.1 * rng.uniform(seed, 5 + k, 0, n)).astype(np.float32)}))
+
+    def sparse(name, src, trg, n_src, n_trg, stride, stream, lo, hi, wum, tau):
+        ind = np.sort(rng.randint(seed, stream, 0, n_src * stride, n_trg).reshape(n_src, stride), axis=1).astype(np.uint32)
+        row_length = (stride - rng.randint(seed, stream + 1, 0, n_src, stride // 3)).astype(np.uint32)
+        g = (lo + (hi - lo) * rng.uniform(seed, stream + 2, 0, n_src * stride)).astype(np.float32).reshape(n_src, stride)
+        return Syn(name, src, trg, psm="expcurr", tau=tau, row_stride=stride, row_length=row_length, ind=ind, g=g, wum=wum)
+
+    net.syns.append(sparse("AB_timing", "A", "B", n_a, n_b, 30, 10, 0.0, 0.12, "timing_copy", 5.0))
+    net.syns.append(sparse("BA_inhibit", "B", "A", n_b, n_a, 24, 20, -0.5, -0.1, "static", 10.0))
+    net.syns.append(sparse("AA_timing", "A", "A", n_a, n_a, 70, 30, 0.0, 0.02, "timing_copy", 5.0))
+    return net

@@ -91,6 +91,9 @@ class Net:
     syns: List[Syn] = field(default_factory=list)
     fuse_psm: bool = False
     seed: int = 0
+    # parameters changed while the model runs (setParamDynamic + Runtime::setDynamicParamValue):
+    # (kind, group, parameter, step, value) with kind in neuron | cs | wu | ps; the value holds from `step` on
+    dynamic: List[tuple] = field(default_factory=list)
 
     def pop(self, name):
         return next(p for p in self.pops if p.name == name)
@@ -113,6 +116,8 @@ class Net:
             for a in (s.row_length, s.ind, s.g, s.d, s.gp):
                 if a is not None:
                     h.update(np.ascontiguousarray(a).tobytes())
+        for d in self.dynamic:
+            h.update(repr(tuple(d)).encode())
         return h.hexdigest()
 
 
@@ -142,9 +147,13 @@ def write_netspec(net: Net, path: str):
         lines.append(f"batch {int(net.batch_size)}")
     if any(s.matrix == "procedural" for s in net.syns) or any(c.model == "poisson_exp" for c in net.css):
         lines.append(f"seed {int(net.seed)}")        # procedural matrices and Poisson sources draw from the model's seed
+    for kind, group, param, step, value in net.dynamic:
+        lines.append(f"dynamic {kind} {group} {param} {int(step)} {float(value)!r}")
     for p in net.pops:
         if p.model == "lif":
             ps = " ".join(repr(float(p.params[k])) for k in LIF_PARAMS)
+        elif p.model == "lifa":       # LIF with an adaptation variable: a model of the test driver, not a built-in one
+            ps = " ".join(repr(float(p.params[k])) for k in LIF_PARAMS + ("TauA", "dA"))
         elif p.model == "izh":
             ps = " ".join(repr(float(p.params[k])) for k in IZH_PARAMS)
         else:
@@ -185,7 +194,7 @@ def write_netspec(net: Net, path: str):
             snippet, params = s.g_init
             order = {"Constant": ("constant",), "Uniform": ("min", "max"), "Normal": ("mean", "sd")}[snippet]
             w = f"static_init {snippet} " + " ".join(repr(float(params[k])) for k in order)
-        elif s.wum in ("static", "static_reverse"):
+        elif s.wum in ("static", "static_reverse", "timing_copy"):
             w = s.wum
         elif s.wum == "static_const":
             w = f"static_const {float(s.wum_params['g'])!r}"
@@ -202,7 +211,7 @@ def write_netspec(net: Net, path: str):
         opts = (" hint_pre" if s.hint_pre else "") + (f" tps {s.threads_per_spike}" if s.threads_per_spike > 1 else "")
         if s.axonal_delay_steps:
             opts += f" axonal_delay {int(s.axonal_delay_steps)}"
-        if s.wum in ("stdp_trace", "stdp_additive"):
+        if s.wum in ("stdp_trace", "stdp_additive", "timing_copy"):
             mask = np.arange(s.row_stride)[None, :] < s.row_length[:, None]
             col = s.col_stride or int(np.bincount(s.ind[mask], minlength=net.pop(s.trg).n).max())
             opts += f" col_stride {max(1, col)}"

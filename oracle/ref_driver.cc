@@ -106,6 +106,57 @@ public:
 };
 IMPLEMENT_SNIPPET(StaticPulseReverse);
 
+// Models no backend has built in (what a user of the API writes): they reach the MI355X backend's generated kernels.
+// LIF with a spike-triggered adaptation current: the built-in LIF (neuronModels.h:220-257) plus one state variable that
+// decays every step, is subtracted from the input and grows at every spike.
+class LIFAdapt : public NeuronModels::Base
+{
+public:
+    DECLARE_SNIPPET(LIFAdapt);
+    SET_SIM_CODE(
+        "if (RefracTime <= 0.0) {\n"
+        "  scalar alpha = ((Isyn + Ioffset - A) * Rmembrane) + Vrest;\n"
+        "  V = alpha - (ExpTC * (alpha - V));\n"
+        "}\n"
+        "else {\n"
+        "  RefracTime -= dt;\n"
+        "}\n"
+        "A *= ExpA;\n");
+    SET_THRESHOLD_CONDITION_CODE("RefracTime <= 0.0 && V >= Vthresh");
+    SET_RESET_CODE(
+        "V = Vreset;\n"
+        "RefracTime = TauRefrac;\n"
+        "A += dA;\n");
+    SET_PARAMS({"C", "TauM", "Vrest", "Vreset", "Vthresh", "Ioffset", "TauRefrac", "TauA", "dA"});
+    SET_DERIVED_PARAMS({
+        {"ExpTC", [](const ParamValues &pars, double dt){ return std::exp(-dt / pars.at("TauM").cast<double>()); }},
+        {"Rmembrane", [](const ParamValues &pars, double){ return pars.at("TauM").cast<double>() / pars.at("C").cast<double>(); }},
+        {"ExpA", [](const ParamValues &pars, double dt){ return std::exp(-dt / pars.at("TauA").cast<double>()); }}});
+    SET_VARS({{"V", "scalar"}, {"RefracTime", "scalar"}, {"A", "scalar"}});
+    SET_NEEDS_AUTO_REFRACTORY(false);
+};
+IMPLEMENT_SNIPPET(LIFAdapt);
+
+// Weight update model with presynaptic and postsynaptic variables, after the models of tests/features/test_wu_vars.py:
+// each neuron's variable takes the time of its last spike (pre / post spike code, run in the neuron update); a
+// presynaptic spike delivers g and copies the target's variable into its synapses, a postsynaptic spike copies the
+// source's variable into its column (learnPost).
+class TimingCopy : public WeightUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(TimingCopy);
+    SET_VARS({{"g", "scalar", VarAccess::READ_ONLY}, {"wPre", "scalar"}, {"wPost", "scalar"}});
+    SET_PRE_VARS({{"sPre", "scalar"}});
+    SET_POST_VARS({{"sPost", "scalar"}});
+    SET_PRE_SPIKE_CODE("sPre = t;\n");
+    SET_POST_SPIKE_CODE("sPost = t;\n");
+    SET_PRE_SPIKE_SYN_CODE(
+        "addToPost(g);\n"
+        "wPost = sPost;\n");
+    SET_POST_SPIKE_SYN_CODE("wPre = sPre;\n");
+};
+IMPLEMENT_SNIPPET(TimingCopy);
+
 // Current source fed from a host-pregenerated array; the driver rewrites the N-element
 // window before every step, so the injected value at step s is noise[s*N + id].
 class ArrayNoise : public CurrentSourceModels::Base
@@ -142,6 +193,7 @@ static void appendFile(const std::string &path, const T *data, size_t n)
 
 struct PopSpec { std::string name, model; unsigned int n; std::vector<double> p; NeuronGroup *ng = nullptr; };
 struct CSSpec { std::string name, model, pop; std::vector<double> p; CurrentSource *cs = nullptr; };
+struct DynamicSpec { std::string kind, group, param; unsigned int step; double value; };     // a parameter set while the model runs
 struct SynSpec
 {
     std::string name, matrix, src, trg, wum, psm, connect, initSnippet;
@@ -160,7 +212,8 @@ int main(int argc, char *argv[])
         bool generateOnly = false;
         std::string userCxxFlags;
         std::vector<std::string> dynamicParams;
-        bool timing = false;
+        bool timing = false, ordered = false;
+        std::string kernels = "auto";
         for(int a = 4; a < argc; a++) {
             const std::string opt = argv[a];
             if(opt == "--generate-only") { generateOnly = true; }
@@ -168,6 +221,8 @@ int main(int argc, char *argv[])
             // --dynamic=neuron:<population>.<param> | cs:<source>.<param> | wu:<projection>.<param> | ps:<projection>.<param>: marks a
             // parameter dynamic (setParamDynamic and friends), as a model that calls setDynamicParamValue at run time would
             else if(opt.rfind("--dynamic=", 0) == 0) { dynamicParams.push_back(opt.substr(10)); }
+            else if(opt.rfind("--kernels=", 0) == 0) { kernels = opt.substr(10); }    // MI355X backend: library | generated | auto (Preferences::kernelSource)
+            else if(opt == "--ordered") { ordered = true; }                          // MI355X backend: Preferences::orderedAccumulation
             else if(opt == "--timing") { timing = true; }       // ModelSpec::setTimingEnabled; the Runtime's counters are printed after the run
             else { std::cerr << "unknown option " << opt << std::endl; return 1; }
         }
@@ -175,6 +230,12 @@ int main(int argc, char *argv[])
         plog::ConsoleAppender<plog::TxtFormatter> app;
         Preferences prefs;
         prefs.userCxxFlagsGNU = userCxxFlags;
+#ifdef DRIVER_BACKEND_MI355X
+        prefs.kernelSource = (kernels == "generated") ? Preferences::KernelSource::GENERATED : (kernels == "library") ? Preferences::KernelSource::LIBRARY : Preferences::KernelSource::AUTO;
+        prefs.orderedAccumulation = ordered;
+#else
+        (void)ordered;
+#endif
         Logging::init(prefs.gennLogLevel, prefs.codeGeneratorLogLevel, prefs.transpilerLogLevel,
                       prefs.runtimeLogLevel, &app, &app, &app, &app);
 
@@ -182,7 +243,7 @@ int main(int argc, char *argv[])
         std::string name = "net";
         double dt = 1.0;
         unsigned int steps = 1, snap = 0, fuse = 0, batch = 1, seed = 0;
-        std::vector<PopSpec> pops; std::vector<CSSpec> css; std::vector<SynSpec> syns;
+        std::vector<PopSpec> pops; std::vector<CSSpec> css; std::vector<SynSpec> syns; std::vector<DynamicSpec> dynamics;
         {
             std::ifstream f(in + "/net.txt");
             if(!f) { throw std::runtime_error("no net.txt in " + in); }
@@ -197,6 +258,7 @@ int main(int argc, char *argv[])
                 else if(k == "fuse_psm") ls >> fuse;
                 else if(k == "batch") ls >> batch;
                 else if(k == "seed") ls >> seed;
+                else if(k == "dynamic") { DynamicSpec d; ls >> d.kind >> d.group >> d.param >> d.step >> d.value; dynamics.push_back(d); dynamicParams.push_back(d.kind + ":" + d.group + "." + d.param); }
                 else if(k == "pop") { PopSpec p; ls >> p.name >> p.model >> p.n; double v; while(ls >> v) p.p.push_back(v); pops.push_back(p); }
                 else if(k == "cs") { CSSpec c; ls >> c.name >> c.model >> c.pop; double v; while(ls >> v) c.p.push_back(v); css.push_back(c); }
                 else if(k == "syn") {
@@ -211,7 +273,7 @@ int main(int argc, char *argv[])
                     else if(s.wum == "stdp_trace" || s.wum == "stdp") { s.wumP.resize(6); for(auto &c : s.wumP) ls >> c; }
                     else if(s.wum == "static_const") { s.wumP.resize(1); ls >> s.wumP[0]; }
                     else if(s.wum == "static_graded") { s.wumP.resize(2); ls >> s.wumP[0] >> s.wumP[1]; }
-                    else if(s.wum != "static" && s.wum != "static_reverse" && s.wum != "static_init") throw std::runtime_error("wum " + s.wum);
+                    else if(s.wum != "static" && s.wum != "static_reverse" && s.wum != "static_init" && s.wum != "timing_copy") throw std::runtime_error("wum " + s.wum);
                     ls >> s.psm;
                     if(s.psm == "expcurr") { s.psmP.resize(1); ls >> s.psmP[0]; }
                     else if(s.psm != "deltacurr") throw std::runtime_error("psm " + s.psm);
@@ -239,6 +301,12 @@ int main(int argc, char *argv[])
                     {{"C", p.p.at(0)}, {"TauM", p.p.at(1)}, {"Vrest", p.p.at(2)}, {"Vreset", p.p.at(3)},
                      {"Vthresh", p.p.at(4)}, {"Ioffset", p.p.at(5)}, {"TauRefrac", p.p.at(6)}},
                     {{"V", uninitialisedVar()}, {"RefracTime", uninitialisedVar()}});
+            }
+            else if(p.model == "lifa") {
+                p.ng = model.addNeuronPopulation<LIFAdapt>(p.name, p.n,
+                    {{"C", p.p.at(0)}, {"TauM", p.p.at(1)}, {"Vrest", p.p.at(2)}, {"Vreset", p.p.at(3)},
+                     {"Vthresh", p.p.at(4)}, {"Ioffset", p.p.at(5)}, {"TauRefrac", p.p.at(6)}, {"TauA", p.p.at(7)}, {"dA", p.p.at(8)}},
+                    {{"V", uninitialisedVar()}, {"RefracTime", uninitialisedVar()}, {"A", uninitialisedVar()}});
             }
             else if(p.model == "izh") {
                 p.ng = model.addNeuronPopulation<NeuronModels::Izhikevich>(p.name, p.n,
@@ -274,6 +342,9 @@ int main(int argc, char *argv[])
             }
             else if(s.wum == "static_reverse") {
                 wum = initWeightUpdate<StaticPulseReverse>({}, {{"g", uninitialisedVar()}});
+            }
+            else if(s.wum == "timing_copy") {
+                wum = initWeightUpdate<TimingCopy>({}, {{"g", uninitialisedVar()}, {"wPre", 0.0}, {"wPost", 0.0}}, {{"sPre", 0.0}}, {{"sPost", 0.0}});
             }
             else if(s.wum == "static_graded") {
 #ifdef DRIVER_BACKEND_MI355X
@@ -379,6 +450,9 @@ int main(int argc, char *argv[])
         };
         for(auto &p : pops) {
             if(p.model == "lif") { load(rt.getArray(*p.ng, "V"), p.name + ".V.f32"); load(rt.getArray(*p.ng, "RefracTime"), p.name + ".RefracTime.f32"); }
+            else if(p.model == "lifa") {
+                load(rt.getArray(*p.ng, "V"), p.name + ".V.f32"); load(rt.getArray(*p.ng, "RefracTime"), p.name + ".RefracTime.f32"); load(rt.getArray(*p.ng, "A"), p.name + ".A.f32");
+            }
             else if(p.model == "izh") { load(rt.getArray(*p.ng, "V"), p.name + ".V.f32"); load(rt.getArray(*p.ng, "U"), p.name + ".U.f32"); }
             else if(p.model == "ssa") {
                 load(rt.getArray(*p.ng, "startSpike"), p.name + ".startSpike.u32");
@@ -433,7 +507,7 @@ int main(int argc, char *argv[])
             for(auto &s : syns) {
                 const auto *sgi = static_cast<const SynapseGroupInternal*>(s.sg);
                 fm << s.name << " " << sgi->getFusedPSTarget().getName() << std::endl;
-                if(s.wum == "stdp_trace" || s.wum == "stdp") {
+                if(s.wum == "stdp_trace" || s.wum == "stdp" || s.wum == "timing_copy") {
                     auto *cl = rt.getArray(*s.sg, "colLength"); auto *rm = rt.getArray(*s.sg, "remap");
                     cl->pullFromDevice(); rm->pullFromDevice();
                     appendFile(out + "/" + s.name + ".colLength.u32", cl->getHostPointer<uint32_t>(), cl->getCount());
@@ -452,9 +526,10 @@ int main(int argc, char *argv[])
             for(auto &p : pops) {
                 if(p.model == "ssa") continue;
                 pulled(rt.getArray(*p.ng, "V"));
-                pulled(rt.getArray(*p.ng, p.model == "lif" ? "RefracTime" : "U"));
+                pulled(rt.getArray(*p.ng, (p.model == "lif" || p.model == "lifa") ? "RefracTime" : "U"));
                 appendFile(out + "/" + p.name + ".V.f32", rt.getArray(*p.ng, "V")->getHostPointer<float>(), (size_t)p.n * batch);
-                if(p.model == "lif") appendFile(out + "/" + p.name + ".RefracTime.f32", rt.getArray(*p.ng, "RefracTime")->getHostPointer<float>(), (size_t)p.n * batch);
+                if(p.model == "lif" || p.model == "lifa") appendFile(out + "/" + p.name + ".RefracTime.f32", rt.getArray(*p.ng, "RefracTime")->getHostPointer<float>(), (size_t)p.n * batch);
+                if(p.model == "lifa") { auto *a = pulled(rt.getArray(*p.ng, "A")); appendFile(out + "/" + p.name + ".A.f32", a->getHostPointer<float>(), (size_t)p.n * batch); }
                 if(p.model == "izh") appendFile(out + "/" + p.name + ".U.f32", rt.getArray(*p.ng, "U")->getHostPointer<float>(), (size_t)p.n * batch);
             }
             for(auto &s : syns) {
@@ -471,6 +546,17 @@ int main(int argc, char *argv[])
                     auto *a = pulled(rt.getArray(*s.sg, "g"));
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
                     for(size_t i = 0; i < numPre; i++) { appendFile(out + "/" + s.name + ".g.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
+                }
+                if(s.wum == "timing_copy") {
+                    const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
+                    for(const char *var : {"wPre", "wPost"}) {
+                        auto *a = pulled(rt.getArray(*s.sg, var));
+                        for(size_t i = 0; i < numPre; i++) { appendFile(out + "/" + s.name + "." + var + ".f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
+                    }
+                    for(const char *var : {"sPre", "sPost"}) {
+                        auto *a = pulled(rt.getArray(*s.sg, var));
+                        appendFile(out + "/" + s.name + "." + var + ".f32", a->getHostPointer<float>(), a->getCount());
+                    }
                 }
                 if(s.wum == "stdp_trace") {
                     auto *a = pulled(rt.getArray(*s.sg, "preTrace")); auto *b = pulled(rt.getArray(*s.sg, "postTrace"));
@@ -489,6 +575,14 @@ int main(int argc, char *argv[])
                     std::copy_n(noise[c.name].begin() + (size_t)i * n, n, a->getHostPointer<float>());
                     a->pushToDevice();
                 }
+            }
+            // scheduled parameter changes (Runtime::setDynamicParamValue, runtime.cc:945-976): in force from step d.step on
+            for(const auto &d : dynamics) {
+                if(d.step != i) { continue; }
+                const Type::NumericValue value(d.value);
+                if(d.kind == "neuron") { rt.setDynamicParamValue(*popByName.at(d.group)->ng, d.param, value); }
+                else if(d.kind == "cs") { for(auto &c : css) { if(c.name == d.group) { rt.setDynamicParamValue(*c.cs, d.param, value); } } }
+                else { for(auto &q : syns) { if(q.name == d.group) { rt.setDynamicParamValue(*q.sg, d.param, value); } } }
             }
             rt.stepTime();
             if(snap && ((i + 1) % snap) == 0) snapshot();

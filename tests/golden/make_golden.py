@@ -40,17 +40,18 @@ def make(name):
         data["fusemap"] = np.array([f"{k}={v}" for k, v in fuse.items()])
         for p in net.pops:
             data[f"spikes.{p.name}"] = np.fromfile(os.path.join(out, f"{p.name}.spikes.u32"), np.uint32).reshape(-1, 2)
-            for var in ("V", "RefracTime", "U"):
+            for var in ("V", "RefracTime", "U", "A"):
                 f = os.path.join(out, f"{p.name}.{var}.f32")
                 if os.path.exists(f):
                     data[f"{var}.{p.name}"] = np.fromfile(f, np.float32).reshape(-1, p.n)
         for s in net.syns:
             for var, dtype in (("outPost", np.float32), ("denDelay", np.float32), ("g", np.float32), ("preTrace", np.float32),
-                               ("postTrace", np.float32), ("colLength", np.uint32), ("remap", np.uint32)):
+                               ("postTrace", np.float32), ("colLength", np.uint32), ("remap", np.uint32),
+                               ("wPre", np.float32), ("wPost", np.float32), ("sPre", np.float32), ("sPost", np.float32)):
                 f = os.path.join(out, f"{s.name}.{var}.{'u32' if dtype == np.uint32 else 'f32'}")
                 if os.path.exists(f):
                     a = np.fromfile(f, dtype)
-                    if var in ("g", "denDelay", "outPost", "preTrace", "postTrace"):
+                    if var in ("g", "denDelay", "outPost", "preTrace", "postTrace", "wPre", "wPost", "sPre", "sPost"):
                         a = a.reshape(net.steps // snap, -1)[-1] if var in ("g", "denDelay") else a.reshape(net.steps // snap, -1)
                     data[f"{var}.{s.name}"] = a
             f = os.path.join(out, f"{s.name}.events.u32")

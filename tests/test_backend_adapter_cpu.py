@@ -126,9 +126,10 @@ def test_poisson_sources_generate():
 @pytest.mark.parametrize("dynamic, case", [("neuron:E.Ioffset", "va_small"), ("ps:EE.tau", "va_small"), ("cs:23E_dc.amp", "potjans_small"),
                                            ("wu:EE.aPlus", "stdp_small")])
 def test_dynamic_parameters_are_refused(dynamic, case):
-    """Parameters are baked into the descriptors built before the first step, so a model that marks one dynamic
-    (setParamDynamic; the reference gives it a DYNAMIC merged-struct field, neuronGroup.h:135, currentSource.h:67,
-    synapseGroup.h:187-190) must be refused at generation time instead of running with the value frozen."""
+    """The device library's descriptors hold parameters as constants built before the first step, so with the library's
+    kernels asked for explicitly a model that marks a parameter dynamic (setParamDynamic; the reference gives it a DYNAMIC
+    merged-struct field, neuronGroup.h:135, currentSource.h:67, synapseGroup.h:187-190) must be refused at generation
+    time instead of running with the value frozen.  (Left to choose, the backend generates kernels for such a model.)"""
     net, snap = CASES[case]()
     net.snap = snap
     tmp = tempfile.mkdtemp(prefix="adapter_dyn_")
@@ -137,8 +138,63 @@ def test_dynamic_parameters_are_refused(dynamic, case):
         for d in (work, out):
             os.makedirs(d)
         write_netspec(net, spec)
-        res = subprocess.run([DRIVER, spec, work, out, "--generate-only", "--dynamic=" + dynamic], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        res = subprocess.run([DRIVER, spec, work, out, "--generate-only", "--kernels=library", "--dynamic=" + dynamic], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
         assert res.returncode != 0
         assert "dynamic" in res.stdout and dynamic.split(".")[-1] in res.stdout and "not among the models" in res.stdout, res.stdout[-2000:]
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
+def _generate_with(case, *options):
+    net, snap = CASES[case]()
+    net.snap = snap
+    tmp = tempfile.mkdtemp(prefix="adapter_genk_")
+    spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+    for d in (work, out):
+        os.makedirs(d)
+    write_netspec(net, spec)
+    res = subprocess.run([DRIVER, spec, work, out, "--generate-only", *options], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    return net, tmp, os.path.join(work, net.name + "_CODE"), res
+
+
+@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("stdp_small", ("--kernels=generated",)),
+                                           ("va_small", ("--dynamic=neuron:E.Ioffset",))])
+def test_generated_kernels_are_chosen_and_build(case, options):
+    """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the runner then holds device
+    code (the model's snippets inside this backend's kernel skeletons), built for gfx950 by the runner's own Makefile, with
+    the reference's entry points around it."""
+    net, tmp, code, res = _generate_with(case, *options)
+    try:
+        assert res.returncode == 0, res.stdout[-3000:]
+        neuron = open(os.path.join(code, "neuronUpdate.cc")).read()
+        synapse = open(os.path.join(code, "synapseUpdate.cc")).read()
+        assert "__global__" in neuron and "gennmi_kernel::orderedSlot" in neuron and "gennmi_kernel::recordBallot" in neuron
+        assert "__global__" in synapse and "gennmi_kernel::addScalar" in synapse
+        assert "gennmi_runner_create" not in open(os.path.join(code, "runner.cc")).read()
+        makefile = open(os.path.join(code, "Makefile")).read()
+        assert "hipcc" in makefile and "--offload-arch=gfx950" in makefile and "-packed-fp32-ops" in makefile and "-ffp-contract=off" in makefile
+        exports = _exports(os.path.join(code, "librunner.so"))
+        for name in ("allocateMem", "freeMem", "initialize", "initializeSparse", "stepTime", "updateNeurons", "updateSynapses"):
+            assert name in exports
+        if case == "custom_small":
+            # the extra state variable and the weight-update variables are in the kernels under the reference's names
+            assert "group->A[id]" in neuron and "sPreOutSynWUMPre" in neuron and "sPostInSynWUMPost" in neuron
+            assert "group->wPost[idSyn] = group->sPost[idPost]" in synapse and "group->wPre[rowMajorIndex] = group->sPre[idPre]" in synapse
+        if case in ("dynamic_small", "va_small"):
+            # the dynamic parameter is a struct field the kernel reads, with a push function that marks the device copy stale
+            assert "group->Ioffset" in neuron
+            assert any(e.startswith("pushMergedNeuronUpdate") and e.endswith("IoffsetToDevice") for e in exports)
+            assert "gennmiStructsDirty = true" in open(os.path.join(code, "runner.cc")).read()
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
+@pytest.mark.parametrize("case, what", [("va_delay_small", "delay"), ("conv_small", "connectivity"), ("graded_small", "spike-like")])
+def test_generated_kernels_say_what_they_do_not_cover(case, what):
+    """Asked to generate kernels for a feature only the device library implements, the backend names the feature."""
+    net, tmp, code, res = _generate_with(case, "--kernels=generated")
+    try:
+        assert res.returncode != 0
+        assert "generated kernels do not cover" in res.stdout and what in res.stdout, res.stdout[-2000:]
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
