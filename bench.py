@@ -31,6 +31,9 @@ BYTES_PER_EVENT = {"dense": 4,          # one weight read per (spike, target); o
 # is only attached to a run of the very command line it was measured on (same workload, steps and warm-up: the network,
 # its seed and therefore its activity are then identical); any other run reports null.
 MEASURED_TRAFFIC_BYTES = {
+    ("potjans", 20, 5): {"plan": "resident", "bytes_per_launch": 212421734,
+                         "source": "rocprofv3 --pmc FETCH_SIZE (95626.44 x 2 KiB) + WRITE_SIZE (16190.22 x 1 KiB) of the timed 20-step "
+                                   "launch, profiles/residentKernel_potjans_full.md"},
 }
 
 
@@ -267,8 +270,8 @@ def main():
         bpe = bytes_per_event or max(BYTES_PER_EVENT[k] for k in kinds)
         neuron_bytes = sum(p.n * (0 if p.model == "ssa" else 32) for p in net.pops)     # 32 B per LIF/Izhikevich update (state + one PSM)
         if info["resident_plan"]:
-            # the timed region is ONE launch of residentKernel that performs all K steps (preceded by an 8-byte-per-tile
-            # memset), so HIP events around the region give that launch's duration; a launch moves K steps' worth of
+            # the timed region is ONE launch of residentKernel that performs all K steps and nothing else, so HIP events
+            # around the region give that launch's duration; a launch moves K steps' worth of
             # algorithmic bytes
             achieved = (events * bpe + neuron_bytes * args.steps) / region_s / 1e9
             roofline = {"bound": "hbm", "kernel": "residentKernel (all timesteps of the timed region in one launch)",

@@ -68,7 +68,7 @@ struct gennmi_runner
     bool resident = false;
     ResTile *dResTiles = nullptr; NeuronGroupDev *dResGroups = nullptr; uint8_t *dResTileGroup = nullptr;
     unsigned long long *dResTags = nullptr; uint32_t *dResSide = nullptr;
-    uint32_t resTiles = 0, resReplicaStride = 0; size_t resLdsBytes = 0; bool resPoisson = false;
+    uint32_t resTiles = 0, resReplicaStride = 0, resSeq = 0; size_t resLdsBytes = 0; bool resPoisson = false;
     std::vector<u32x4*> resSegs;        // segment table of each presynaptic group, in push order
     std::vector<uint32_t> resSegTiles;  // tiles of its target population
     uint32_t neuronsPerLane = 1;        // 2, 4 or 8: neuronBulkKernel instead of neuronUpdateKernel
@@ -619,6 +619,9 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
     r->resReplicaStride = (uint32_t)((2 * tiles.size() + 511) / 512 * 512);          // in words: copies start 4 KiB-aligned
     HIP_TRY(hipMalloc(&r->dResTags, (size_t)RES_REPLICAS * r->resReplicaStride * sizeof(unsigned long long)));
     r->owned.push_back(r->dResTags);
+    // cleared once: sequence number 0 is the one no work-group ever waits for before it has come round again
+    HIP_TRY(hipMemset(r->dResTags, 0, (size_t)RES_REPLICAS * r->resReplicaStride * sizeof(unsigned long long)));
+    r->resSeq = 0;
     HIP_TRY(hipMalloc(&r->dResSide, 2 * tiles.size() * RES_T * sizeof(uint32_t)));
     r->owned.push_back(r->dResSide);
     r->resTiles = (uint32_t)tiles.size();
@@ -651,12 +654,12 @@ static int launchResident(gennmi_runner *r, unsigned long long timestep, unsigne
     }
     for(unsigned long long done = 0; done < numSteps; ) {
         const uint32_t chunk = (uint32_t)std::min(MAX_STEPS, numSteps - done);
-        HIP_TRY(hipMemsetAsync(r->dResTags, 0, (size_t)RES_REPLICAS * r->resReplicaStride * sizeof(unsigned long long), r->stream));
         auto launch = r->resPoisson ? residentKernel<true> : residentKernel<false>;
         launch<<<dim3(r->resTiles), dim3(BLOCK), r->resLdsBytes, r->stream>>>(
             r->dResTiles, r->resTiles, r->dResGroups, r->dResTileGroup, r->dResTags, r->dResSide, timestep + done, r->epoch, numRecordingTimesteps,
-            chunk, r->dt, r->fusedStep ? 1u : 0u, r->dError, r->dEvents, r->resReplicaStride);
+            chunk, r->dt, r->fusedStep ? 1u : 0u, r->dError, r->dEvents, r->resReplicaStride, r->resSeq);
         HIP_TRY(hipGetLastError());
+        r->resSeq = (r->resSeq + chunk + 1u) & RES_SEQ_MASK;       // the launch used sequence numbers resSeq + 1 ... resSeq + chunk + 1
         done += chunk;
         r->epoch += chunk;
     }

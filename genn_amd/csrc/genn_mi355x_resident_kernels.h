@@ -32,6 +32,7 @@ constexpr uint32_t RES_FRONT_MAX = 4;        // front-slot synapses held inline 
 constexpr uint32_t RES_SEG_OVERFLOW = 1u << 24, RES_SEG_NO_DELAY = 1u << 25;
 constexpr uint32_t RES_PAIR_GROUP = 16;      // pairs a wavefront expands at a time
 constexpr int RES_SEQ_SHIFT = 41;            // word = seq << 41 | count << 32 | up to four tile-local neuron indices, 8 bits each
+constexpr uint32_t RES_SEQ_MASK = (1u << (64 - RES_SEQ_SHIFT)) - 1u;    // sequence numbers run on from launch to launch, modulo 2^23
 constexpr uint32_t RES_WORD_IDS = 4;         // spikes of a tile and step that travel inside its word (more: side buffer)
 constexpr uint32_t RES_REPLICAS = 8;         // copies of the word array, one per XCD, so that polling spreads over memory channels
 
@@ -119,7 +120,8 @@ __global__ __launch_bounds__(BLOCK)
 void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const NeuronGroupDev * __restrict__ groups,
                     const uint8_t * __restrict__ tileGroup, unsigned long long *tags, uint32_t *side,
                     unsigned long long timestep0, unsigned long long epoch0, unsigned long long numRecordingTimesteps, uint32_t numSteps,
-                    float dt, uint32_t zeroDelaySplit, uint32_t *errorFlag, unsigned long long *eventCounter, uint32_t replicaStride)
+                    float dt, uint32_t zeroDelaySplit, uint32_t *errorFlag, unsigned long long *eventCounter, uint32_t replicaStride,
+                    uint32_t seqBase)
 {
     extern __shared__ float lds[];                       // inSyn rows and ring slices of this tile
     __shared__ unsigned long long shTag[RES_MAX_TILES];
@@ -155,16 +157,19 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
 
     // ---- tables into LDS
     for(uint32_t k = tid; k < numTiles; k += BLOCK) { shTileGroup[k] = tileGroup[k]; }
-    if(tid < T.numProj) { shProj[tid] = T.proj[tid]; }
+    const uint32_t numProj = T.numProj;
+    if(tid < numProj) { shProj[tid] = T.proj[tid]; }
+    __syncthreads();
     if(tid == 0) {
-        // projections grouped by source group (counting sort; a handful of entries)
+        // projections grouped by source group (counting sort; a handful of entries, read from the LDS copy: one thread
+        // chasing them through global memory costs tens of microseconds per launch)
         for(uint32_t s = 0; s <= RES_MAX_GROUPS; s++) { shProjStart[s] = 0; }
-        for(uint32_t p = 0; p < T.numProj; p++) { shProjStart[T.proj[p].srcGroup + 1]++; }
+        for(uint32_t p = 0; p < numProj; p++) { shProjStart[shProj[p].srcGroup + 1]++; }
         for(uint32_t s = 0; s < RES_MAX_GROUPS; s++) { shProjStart[s + 1] += shProjStart[s]; }
-        for(uint32_t p = 0; p < T.numProj; p++) {
-            const uint32_t s = T.proj[p].srcGroup;
+        for(uint32_t p = 0; p < numProj; p++) {
+            const uint32_t s = shProj[p].srcGroup;
             uint32_t before = 0;
-            for(uint32_t q = 0; q < p; q++) { before += (T.proj[q].srcGroup == s) ? 1u : 0u; }
+            for(uint32_t q = 0; q < p; q++) { before += (shProj[q].srcGroup == s) ? 1u : 0u; }
             shProjIdx[shProjStart[s] + before] = (uint8_t)p;
         }
     }
@@ -210,7 +215,11 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     uint32_t ownCount = shScalar[1];
 
     // (callers synchronise the work-group after filling shOwn)
-    auto publish = [&](uint32_t seq, uint32_t count) {
+    // A word slot is rewritten every second sequence number, and a launch continues the numbering of the one before
+    // (seqBase), so a slot never holds the number a reader waits for before its writer has stored it: nothing is cleared
+    // between launches.
+    auto publish = [&](uint32_t step, uint32_t count) {
+        const uint32_t seq = (seqBase + step) & RES_SEQ_MASK;
         const uint32_t parity = seq & 1u;
         if(count > RES_WORD_IDS) {
             for(uint32_t r = tid; r < count; r += BLOCK) {
@@ -243,7 +252,8 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     // Waits for every tile's word of sequence number seq (false when the bounded wait expired somewhere) and stages the
     // (spike, projection) pairs that concern this tile in shPair; shScalar[0] receives their number, which may exceed
     // RES_PAIR_CAP (then only the claims that fitted were written and the caller takes the chunked path).
-    auto poll = [&](uint32_t seq, unsigned long long epoch) -> bool {
+    auto poll = [&](uint32_t step, unsigned long long epoch) -> bool {
+        const uint32_t seq = (seqBase + step) & RES_SEQ_MASK;
         const uint32_t parity = seq & 1u;
         bool ok = true;
         unsigned long long word[WATCH];
@@ -276,7 +286,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             return false;
         }
         // front slot of every projection's ring in the step this exchange feeds
-        if(tid < T.numProj) { shProjPtr[tid] = shProj[tid].D ? modStep(epoch + 1, shProj[tid].D) : 0u; }
+        if(tid < numProj) { shProjPtr[tid] = shProj[tid].D ? modStep(epoch + 1, shProj[tid].D) : 0u; }
         #pragma unroll
         for(uint32_t q = 0; q < WATCH; q++) {
             const uint32_t c = (uint32_t)(word[q] >> 32) & 0x1FFu, np = watchNumProj[q];
@@ -373,8 +383,8 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     };
 
     // the pairs of a step that holds more of them than shPair does: staged and walked RES_PAIR_CAP at a time, in full
-    auto processChunked = [&](uint32_t seq, uint32_t total, uint32_t pass, bool count) {
-        const uint32_t parity = seq & 1u;
+    auto processChunked = [&](uint32_t step, uint32_t total, uint32_t pass, bool count) {
+        const uint32_t parity = (seqBase + step) & 1u;
         uint32_t want = 0;
         for(uint32_t k = tid; k < numTiles; k += BLOCK) {
             const uint32_t c = (uint32_t)(shTag[k] >> 32) & 0x1FFu;
