@@ -122,6 +122,7 @@ SYMBOLS = {
     "gennmi_push_postsynaptic_update_group": (C.c_int, [C.c_void_p, C.POINTER(PostsynapticUpdateGroup), C.POINTER(C.c_uint32)]),
     "gennmi_runner_finalise": (C.c_int, [C.c_void_p]),
     "gennmi_runner_set_ordered": (C.c_int, [C.c_void_p, C.c_int]),
+    "gennmi_runner_set_step_queue": (C.c_int, [C.c_void_p, C.c_uint32]),
     "gennmi_build_remap": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "gennmi_max_col_length": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]),
     "gennmi_max_col_length_static": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p]),

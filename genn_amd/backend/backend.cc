@@ -1255,6 +1255,9 @@ void Backend::genRunnerPreamble(CodeStream &os, const ModelSpecMerged&) const
             os << "GENNMI_CHECK(gennmi_runner_set_ordered(gennmiRunner, 1));" << std::endl;
         }
         os << "GENNMI_CHECK(gennmi_runner_finalise(gennmiRunner));" << std::endl;
+        if(getPreferences<Preferences>().stepQueueLength > 0) {
+            os << "GENNMI_CHECK(gennmi_runner_set_step_queue(gennmiRunner, " << getPreferences<Preferences>().stepQueueLength << "u));" << std::endl;
+        }
         os << "gennmiFinalised = true;" << std::endl;
     }
     os << std::endl;

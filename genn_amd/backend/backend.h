@@ -41,12 +41,19 @@ struct Preferences : public PreferencesBase
     //! SingleThreadedCPU backend, without atomics (gennmi_runner_set_ordered); LIBRARY kernels only
     bool orderedAccumulation = false;
 
+    //! Steps the generated stepTime() may leave queued in the device library before they are launched
+    //! (gennmi_runner_set_step_queue): Runtime::stepTime() asks for one step at a time, and a model whose runner is on the
+    //! resident plan runs a whole queue in one launch.  Every pull, push and synchronisation executes the queue first, so
+    //! results do not depend on it; 0 launches every step when it is asked for.
+    unsigned int stepQueueLength = 256;
+
     void updateHash(boost::uuids::detail::sha1 &hash) const
     {
         PreferencesBase::updateHash(hash);
         Utils::updateHash(deviceID, hash);
         Utils::updateHash(static_cast<int>(kernelSource), hash);
         Utils::updateHash(orderedAccumulation, hash);
+        Utils::updateHash(stepQueueLength, hash);
     }
 };
 

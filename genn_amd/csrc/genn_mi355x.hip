@@ -25,6 +25,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -101,6 +102,10 @@ struct gennmi_runner
     struct Pending { hipEvent_t a, b; int kind; };          // kind: 0 presynaptic, 1 postsynaptic, 2 neuron, 3 single-launch step
     std::vector<hipEvent_t> eventPool; size_t eventNext = 0; std::vector<Pending> pending;
     hipEvent_t marks[2] = {nullptr, nullptr};               // gennmi_runner_stream_mark
+    // step queue (gennmi_runner_set_step_queue): steps asked for one at a time and not yet launched
+    struct QueuedStep { float t; uint32_t recordingTimestep; };
+    uint32_t stepQueueLimit = 0;
+    std::vector<QueuedStep> queued;
 };
 
 // Runners whose resident plan holds copies of weights (inline in the segment tables): a write to device memory that
@@ -141,11 +146,35 @@ static void noteDeviceWrite(const void *dev, size_t bytes)
     }
 }
 
+// Step queue.  A caller that advances the model one gennmi_step() at a time (the reference's Runtime::stepTime does) would
+// pay a launch per step; a runner on the resident plan can do many steps in one launch.  With a queue enabled, gennmi_step()
+// only notes the step; the noted steps run, as one launch where they can, before anything could observe the difference:
+// every entry point of the library that reads, writes or frees device memory, synchronises, reads counters or steps by another
+// route first executes what is queued (flushQueuedSteps), and so does the queue reaching its limit.
+static std::atomic<int> g_queuedRunners{0};
+static int flushRunner(gennmi_runner *r);
+static int flushQueuedSteps()
+{
+    if(g_queuedRunners.load(std::memory_order_relaxed) == 0) { return GENNMI_OK; }
+    std::vector<gennmi_runner*> runners;
+    {
+        std::lock_guard<std::mutex> lock(g_runnersMutex);
+        runners = g_runners;
+    }
+    for(gennmi_runner *r : runners) {
+        const int rc = flushRunner(r);
+        if(rc) { return rc; }
+    }
+    return GENNMI_OK;
+}
+#define FLUSH_QUEUED() do { const int rcFlush_ = flushQueuedSteps(); if(rcFlush_) { return rcFlush_; } } while(0)
+
 namespace gennmi_detail
 {
 // error reporting and write tracking for the library's other translation units
 int fail(int code, const std::string &msg) { return ::fail(code, msg); }
 void noteDeviceWrite(const void *dev, size_t bytes) { ::noteDeviceWrite(dev, bytes); }
+int flushQueuedSteps() { return ::flushQueuedSteps(); }
 int prepareStaticScratch();             // looks up the current device's copy of the static counter array (defined with it)
 }
 
@@ -180,22 +209,25 @@ int gennmi_malloc(void **devPtr, size_t bytes)
     HIP_TRY(hipMalloc(devPtr, bytes ? bytes : 4));
     return GENNMI_OK;
 }
-int gennmi_free(void *devPtr) { HIP_TRY(hipFree(devPtr)); return GENNMI_OK; }
+int gennmi_free(void *devPtr) { FLUSH_QUEUED(); HIP_TRY(hipFree(devPtr)); return GENNMI_OK; }
 int gennmi_memcpy_to_device(void *dev, const void *host, size_t bytes)
 {
+    FLUSH_QUEUED();
     HIP_TRY(hipMemcpy(dev, host, bytes, hipMemcpyHostToDevice));
     noteDeviceWrite(dev, bytes);
     return GENNMI_OK;
 }
-int gennmi_memcpy_from_device(void *host, const void *dev, size_t bytes) { HIP_TRY(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost)); return GENNMI_OK; }
+int gennmi_memcpy_from_device(void *host, const void *dev, size_t bytes) { FLUSH_QUEUED(); HIP_TRY(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost)); return GENNMI_OK; }
 int gennmi_memset(void *dev, int value, size_t bytes)
 {
+    FLUSH_QUEUED();
     HIP_TRY(hipMemset(dev, value, bytes));
     noteDeviceWrite(dev, bytes);
     return GENNMI_OK;
 }
 int gennmi_fill_f32(float *dev, float value, size_t count)
 {
+    FLUSH_QUEUED();
     if(count) {
         fillKernel<<<dim3((unsigned int)((count + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, 0>>>(dev, value, count);
         HIP_TRY(hipGetLastError());
@@ -206,6 +238,7 @@ int gennmi_fill_f32(float *dev, float value, size_t count)
 }
 int gennmi_copy_f32(float *dst, const float *src, size_t count)
 {
+    FLUSH_QUEUED();
     if(count) {
         if(!dst || !src) { return fail(GENNMI_EINVAL, "copy_f32: null pointer"); }
         const size_t lanes = (count + 3) / 4;
@@ -216,7 +249,7 @@ int gennmi_copy_f32(float *dst, const float *src, size_t count)
     }
     return GENNMI_OK;
 }
-int gennmi_synchronize(void) { HIP_TRY(hipDeviceSynchronize()); return GENNMI_OK; }
+int gennmi_synchronize(void) { FLUSH_QUEUED(); HIP_TRY(hipDeviceSynchronize()); return GENNMI_OK; }
 
 // ---- host mirrors: host buffer <-> device buffer pairs, for callers whose generated code only knows host pointers
 namespace
@@ -254,6 +287,7 @@ int gennmi_mirror_device_pointer(const void *host, void **dev)
 }
 int gennmi_push_mirrors(void)
 {
+    FLUSH_QUEUED();
     std::lock_guard<std::mutex> lock(g_mirrorMutex);
     for(const auto &m : g_mirrors) {
         HIP_TRY(hipMemcpy(m.second.dev, reinterpret_cast<const void*>(m.first), m.second.bytes, hipMemcpyHostToDevice));
@@ -299,6 +333,7 @@ int gennmi_runner_create(gennmi_runner **runner, float dt, uint32_t batchSize)
 int gennmi_runner_destroy(gennmi_runner *r)
 {
     if(!r) { return GENNMI_OK; }
+    if(!r->queued.empty()) { r->queued.clear(); g_queuedRunners--; }      // nothing can observe these steps any more
     {
         std::lock_guard<std::mutex> lock(g_runnersMutex);
         g_runners.erase(std::remove(g_runners.begin(), g_runners.end(), r), g_runners.end());
@@ -1407,6 +1442,7 @@ static int launchNeurons(gennmi_runner *r, const StepArgs &a, bool timed)
 int gennmi_update_synapses(gennmi_runner *r, float t)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "update_synapses: runner not finalised"); }
+    FLUSH_QUEUED();
     { const int rc = refreshTables(r); if(rc) { return rc; } }
     StepArgs a{};
     a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = 0;
@@ -1419,6 +1455,7 @@ int gennmi_update_synapses(gennmi_runner *r, float t)
 int gennmi_update_neurons(gennmi_runner *r, float t, uint32_t recordingTimestep)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "update_neurons: runner not finalised"); }
+    FLUSH_QUEUED();
     { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
     StepArgs a{};
     a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recordingTimestep;
@@ -1438,11 +1475,9 @@ int gennmi_step_time(gennmi_runner *r, unsigned long long timestep, unsigned lon
     return gennmi_step(r, t, recT);
 }
 
-int gennmi_step(gennmi_runner *r, float t, uint32_t recordingTimestep)
+// one step, launched now
+static int stepNow(gennmi_runner *r, float t, uint32_t recordingTimestep)
 {
-    if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "step: runner not finalised"); }
-    { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
-    { const int rc = refreshTables(r); if(rc) { return rc; } }
     if(r->fusedStep) {
         StepArgs a{};
         a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recordingTimestep;
@@ -1462,9 +1497,64 @@ int gennmi_step(gennmi_runner *r, float t, uint32_t recordingTimestep)
     return gennmi_update_neurons(r, t, recordingTimestep);
 }
 
+// Executes the steps a runner has queued: runs of steps whose recording rows follow one another (or that all record into row
+// 0: no recording, or a one-row buffer) go to the resident kernel in one launch, anything shorter than it accepts step by step.
+static int flushRunner(gennmi_runner *r)
+{
+    if(r->queued.empty()) { return GENNMI_OK; }
+    std::vector<gennmi_runner::QueuedStep> steps;
+    steps.swap(r->queued);
+    g_queuedRunners--;
+    { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
+    { const int rc = refreshTables(r); if(rc) { return rc; } }
+    size_t first = 0;
+    while(first < steps.size()) {
+        size_t end = first + 1;
+        const bool flat = (end < steps.size() && steps[first].recordingTimestep == 0 && steps[end].recordingTimestep == 0);
+        while(end < steps.size() && steps[end].recordingTimestep == (flat ? 0u : steps[end - 1].recordingTimestep + 1u)) { end++; }
+        const size_t count = end - first;
+        if(r->resident && !r->timing && count >= 4) {
+            // the kernel records step k of the launch into row (timestep + k) % numRecordingTimesteps
+            const int rc = flat ? launchResident(r, 0, count, 1) : launchResident(r, steps[first].recordingTimestep, count, 1ull << 32);
+            if(rc) { return rc; }
+        }
+        else {
+            for(size_t k = first; k < end; k++) {
+                const int rc = stepNow(r, steps[k].t, steps[k].recordingTimestep);
+                if(rc) { return rc; }
+            }
+        }
+        first = end;
+    }
+    return GENNMI_OK;
+}
+
+int gennmi_runner_set_step_queue(gennmi_runner *r, uint32_t maxSteps)
+{
+    if(!r) { return fail(GENNMI_EINVAL, "runner_set_step_queue: null runner"); }
+    { const int rc = flushRunner(r); if(rc) { return rc; } }
+    r->stepQueueLimit = maxSteps;
+    return GENNMI_OK;
+}
+
+int gennmi_step(gennmi_runner *r, float t, uint32_t recordingTimestep)
+{
+    if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "step: runner not finalised"); }
+    if(r->stepQueueLimit && r->resident && !r->timing) {
+        if(r->queued.empty()) { g_queuedRunners++; }
+        r->queued.push_back({t, recordingTimestep});
+        return (r->queued.size() >= r->stepQueueLimit) ? flushRunner(r) : GENNMI_OK;
+    }
+    FLUSH_QUEUED();
+    { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
+    { const int rc = refreshTables(r); if(rc) { return rc; } }
+    return stepNow(r, t, recordingTimestep);
+}
+
 int gennmi_run_steps(gennmi_runner *r, unsigned long long timestep, unsigned long long numSteps, unsigned long long numRecordingTimesteps)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "run_steps: runner not finalised"); }
+    FLUSH_QUEUED();
     { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
     { const int rc = refreshTables(r); if(rc) { return rc; } }
     constexpr unsigned long long CHUNK = 100;
@@ -1519,6 +1609,7 @@ int gennmi_run_steps(gennmi_runner *r, unsigned long long timestep, unsigned lon
 int gennmi_runner_synchronize(gennmi_runner *r)
 {
     if(!r) { return fail(GENNMI_EINVAL, "runner_synchronize: null runner"); }
+    FLUSH_QUEUED();
     HIP_TRY(hipStreamSynchronize(r->stream));
     uint32_t err = 0;
     HIP_TRY(hipMemcpy(&err, r->dError, sizeof(err), hipMemcpyDeviceToHost));
@@ -1529,6 +1620,7 @@ int gennmi_runner_synchronize(gennmi_runner *r)
 int gennmi_runner_set_timing(gennmi_runner *r, int enabled)
 {
     if(!r) { return fail(GENNMI_EINVAL, "runner_set_timing: null runner"); }
+    FLUSH_QUEUED();
     if(!enabled) { const int rc = drainTimers(r); if(rc) { return rc; } }
     r->timing = (enabled != 0);
     return GENNMI_OK;
@@ -1537,6 +1629,7 @@ int gennmi_runner_set_timing(gennmi_runner *r, int enabled)
 int gennmi_runner_get_times(gennmi_runner *r, double *neuronUpdateTime, double *presynapticUpdateTime, double *postsynapticUpdateTime)
 {
     if(!r) { return fail(GENNMI_EINVAL, "runner_get_times: null runner"); }
+    FLUSH_QUEUED();
     { const int rc = drainTimers(r); if(rc) { return rc; } }
     // a single-launch step is one kernel that holds the neuron update and, in blocks of its own, the presynaptic update of the
     // previous step's spikes: its whole duration counts as neuron update time (the reference has no such kernel)
@@ -1549,6 +1642,7 @@ int gennmi_runner_get_times(gennmi_runner *r, double *neuronUpdateTime, double *
 int gennmi_runner_kernel_stats(gennmi_runner *r, double stats[8])
 {
     if(!r || !stats) { return fail(GENNMI_EINVAL, "runner_kernel_stats: null argument"); }
+    FLUSH_QUEUED();
     { const int rc = drainTimers(r); if(rc) { return rc; } }
     stats[0] = (double)r->preLaunches; stats[1] = r->preTime;
     stats[2] = (double)r->neuronLaunches; stats[3] = r->neuronTime;
@@ -1560,6 +1654,7 @@ int gennmi_runner_kernel_stats(gennmi_runner *r, double stats[8])
 int gennmi_runner_stream_mark(gennmi_runner *r, int which)
 {
     if(!r || which < 0 || which > 1) { return fail(GENNMI_EINVAL, "runner_stream_mark: bad arguments"); }
+    FLUSH_QUEUED();
     if(!r->marks[which]) { HIP_TRY(hipEventCreate(&r->marks[which])); }
     HIP_TRY(hipEventRecord(r->marks[which], r->stream));
     return GENNMI_OK;
@@ -1586,6 +1681,7 @@ int gennmi_runner_get_info(gennmi_runner *r, uint32_t info[4])
 int gennmi_runner_event_count(gennmi_runner *r, unsigned long long *events)
 {
     if(!r || !events) { return fail(GENNMI_EINVAL, "runner_event_count: null argument"); }
+    FLUSH_QUEUED();
     HIP_TRY(hipStreamSynchronize(r->stream));
     HIP_TRY(hipMemcpy(events, r->dEvents, sizeof(*events), hipMemcpyDeviceToHost));
     return GENNMI_OK;
@@ -1594,6 +1690,7 @@ int gennmi_runner_event_count(gennmi_runner *r, unsigned long long *events)
 int gennmi_max_col_length(uint32_t numSrc, uint32_t numTrg, uint32_t rowStride, const uint32_t *rowLength, const uint32_t *ind, uint32_t *maxColLength)
 {
     if(!rowLength || !ind || !maxColLength || rowStride == 0) { return fail(GENNMI_EINVAL, "max_col_length: bad arguments"); }
+    FLUSH_QUEUED();
     uint32_t *dCount = nullptr;
     HIP_TRY(hipMalloc(&dCount, (size_t)numTrg * sizeof(uint32_t)));
     HIP_TRY(hipMemset(dCount, 0, (size_t)numTrg * sizeof(uint32_t)));
@@ -1691,6 +1788,7 @@ int gennmi_build_remap(uint32_t numSrc, uint32_t numTrg, uint32_t rowStride, uin
                        const uint32_t *rowLength, const uint32_t *ind, uint32_t *colLength, uint32_t *remap)
 {
     if(!rowLength || !ind || !colLength || !remap || rowStride == 0 || colStride == 0) { return fail(GENNMI_EINVAL, "build_remap: bad arguments"); }
+    FLUSH_QUEUED();
     if(colStride > REMAP_SORT_MAX) { return fail(GENNMI_EUNSUPPORTED, "build_remap: column stride above 16384 is not supported"); }
     uint32_t *dOverflow = nullptr;
     HIP_TRY(hipMalloc(&dOverflow, sizeof(uint32_t)));

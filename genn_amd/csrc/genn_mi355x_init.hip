@@ -31,6 +31,7 @@ namespace gennmi_detail
 {
 int fail(int code, const std::string &msg);
 void noteDeviceWrite(const void *dev, size_t bytes);     // lets runners that hold copies of weights refresh them
+int flushQueuedSteps();                                  // steps a runner has queued run before this library writes device memory
 }
 
 namespace
@@ -253,6 +254,7 @@ int gennmi_philox4x32(const uint32_t counter[4], const uint32_t key[2], uint32_t
 
 int gennmi_init_random_words(uint32_t *dev, size_t count, uint64_t seed, uint32_t stream)
 {
+    { const int rcFlush = gennmi_detail::flushQueuedSteps(); if(rcFlush) { return rcFlush; } }
     if(count == 0) { return GENNMI_OK; }
     const unsigned long long groups = (count + 3) / 4;
     const unsigned int blocks = (unsigned int)std::min<unsigned long long>((groups + BLOCK - 1) / BLOCK, 256ull * 32ull);
@@ -263,6 +265,7 @@ int gennmi_init_random_words(uint32_t *dev, size_t count, uint64_t seed, uint32_
 
 int gennmi_init_var(void *dev, uint32_t elementType, size_t count, uint32_t snippet, const double params[4], uint64_t seed, uint32_t stream)
 {
+    { const int rcFlush = gennmi_detail::flushQueuedSteps(); if(rcFlush) { return rcFlush; } }
     if(count == 0) { return GENNMI_OK; }
     if(snippet > GENNMI_INIT_BINOMIAL) { return gennmi_detail::fail(GENNMI_EUNSUPPORTED, "unknown value-initialisation snippet"); }
     if((uintptr_t)dev % 16) { return gennmi_detail::fail(GENNMI_EINVAL, "array to initialise is not 16-byte aligned"); }
@@ -293,6 +296,7 @@ int gennmi_init_var(void *dev, uint32_t elementType, size_t count, uint32_t snip
 int gennmi_init_sparse_fixed_probability(uint32_t numPre, uint32_t numPost, uint32_t rowStride, double prob, int noAutapse,
                                          uint64_t seed, uint32_t stream, uint32_t *rowLength, uint32_t *ind, uint32_t *overflowRows)
 {
+    { const int rcFlush = gennmi_detail::flushQueuedSteps(); if(rcFlush) { return rcFlush; } }
     if(!(prob >= 0.0 && prob <= 1.0)) { return gennmi_detail::fail(GENNMI_EINVAL, "connection probability outside [0, 1]"); }
     if(numPre == 0 || numPost == 0 || rowStride == 0) { return gennmi_detail::fail(GENNMI_EINVAL, "empty matrix"); }
     if(numPost > 0x7fffffffu || rowStride > 0x7fffffffu) { return gennmi_detail::fail(GENNMI_EINVAL, "more than 2^31-1 postsynaptic neurons or row entries"); }
@@ -309,6 +313,7 @@ int gennmi_init_sparse_fixed_probability(uint32_t numPre, uint32_t numPost, uint
 int gennmi_init_sparse_fixed_number_post(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t num, const uint32_t *rowLengthIn,
                                          uint64_t seed, uint32_t stream, uint32_t *rowLength, uint32_t *ind, uint32_t *overflowRows)
 {
+    { const int rcFlush = gennmi_detail::flushQueuedSteps(); if(rcFlush) { return rcFlush; } }
     if(numPre == 0 || numPost == 0 || rowStride == 0) { return gennmi_detail::fail(GENNMI_EINVAL, "empty matrix"); }
     if(!rowLengthIn && num > rowStride) { return gennmi_detail::fail(GENNMI_EINVAL, "num exceeds rowStride"); }
     if(rowStride > 0x7fffffffu) { return gennmi_detail::fail(GENNMI_EINVAL, "more than 2^31-1 row entries"); }
@@ -321,6 +326,7 @@ int gennmi_init_sparse_fixed_number_post(uint32_t numPre, uint32_t numPost, uint
 
 int gennmi_init_sparse_one_to_one(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t *rowLength, uint32_t *ind)
 {
+    { const int rcFlush = gennmi_detail::flushQueuedSteps(); if(rcFlush) { return rcFlush; } }
     if(numPre == 0 || numPost == 0 || rowStride == 0) { return gennmi_detail::fail(GENNMI_EINVAL, "empty matrix"); }
     hipLaunchKernelGGL(oneToOneKernel, dim3((numPre + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, 0, numPre, numPost, rowStride, rowLength, ind);
     HIP_TRY(hipGetLastError());

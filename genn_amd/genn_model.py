@@ -1041,6 +1041,11 @@ class GeNNModel:
     def set_timing(self, enabled):
         _abi.check(_abi.load().gennmi_runner_set_timing(self._runner, int(bool(enabled))))
 
+    def set_step_queue(self, max_steps):
+        """Let step_time() leave up to max_steps steps queued in the library (a runner on the resident plan executes a
+        queue in one launch); every pull, push, synchronisation and counter read executes the queue first.  0: off."""
+        _abi.check(_abi.load().gennmi_runner_set_step_queue(self._runner, int(max_steps)))
+
     def unload(self):
         if self._runner:
             _abi.load().gennmi_runner_destroy(self._runner)

@@ -356,6 +356,15 @@ int gennmi_step_time(gennmi_runner *runner, unsigned long long timestep, unsigne
  * of 100 steps.  Either way the arrays are left as numSteps calls of gennmi_step_time would leave them. */
 int gennmi_run_steps(gennmi_runner *runner, unsigned long long timestep, unsigned long long numSteps,
                      unsigned long long numRecordingTimesteps);
+/* Step queue (no counterpart in the reference).  A caller that advances the model one gennmi_step() at a time -- the
+ * reference's Runtime::stepTime() does, runtime.cc:686-697 -- pays one launch per step, while a runner on the resident
+ * plan can take many steps in one launch.  With maxSteps > 0, gennmi_step() on such a runner only notes the step;
+ * the noted steps are executed, as one launch where the plan allows it, before anything can observe the difference:
+ * by every entry point of this library that reads, writes or frees device memory, synchronises, reads counters or
+ * steps by another route, and when maxSteps steps are waiting.  Results are those of unqueued stepping; errors of a
+ * queued step are reported by the call that executes it.  Runners on other plans, and runners with timing enabled,
+ * step at once as before.  maxSteps = 0 (the default) switches the queue off after executing what it holds. */
+int gennmi_runner_set_step_queue(gennmi_runner *runner, uint32_t maxSteps);
 /* stepTimeFinalise: blocks until everything queued has finished and reports device-side
  * failures (backendCUDAHIP.cc:1400-1411). */
 int gennmi_runner_synchronize(gennmi_runner *runner);

@@ -213,6 +213,7 @@ int main(int argc, char *argv[])
         std::string userCxxFlags;
         std::vector<std::string> dynamicParams;
         bool timing = false, ordered = false;
+        int stepQueue = -1;
         std::string kernels = "auto";
         for(int a = 4; a < argc; a++) {
             const std::string opt = argv[a];
@@ -222,6 +223,7 @@ int main(int argc, char *argv[])
             // parameter dynamic (setParamDynamic and friends), as a model that calls setDynamicParamValue at run time would
             else if(opt.rfind("--dynamic=", 0) == 0) { dynamicParams.push_back(opt.substr(10)); }
             else if(opt.rfind("--kernels=", 0) == 0) { kernels = opt.substr(10); }    // MI355X backend: library | generated | auto (Preferences::kernelSource)
+            else if(opt.rfind("--step-queue=", 0) == 0) { stepQueue = std::stoi(opt.substr(13)); }      // MI355X backend: Preferences::stepQueueLength
             else if(opt == "--ordered") { ordered = true; }                          // MI355X backend: Preferences::orderedAccumulation
             else if(opt == "--timing") { timing = true; }       // ModelSpec::setTimingEnabled; the Runtime's counters are printed after the run
             else { std::cerr << "unknown option " << opt << std::endl; return 1; }
@@ -233,8 +235,9 @@ int main(int argc, char *argv[])
 #ifdef DRIVER_BACKEND_MI355X
         prefs.kernelSource = (kernels == "generated") ? Preferences::KernelSource::GENERATED : (kernels == "library") ? Preferences::KernelSource::LIBRARY : Preferences::KernelSource::AUTO;
         prefs.orderedAccumulation = ordered;
+        if(stepQueue >= 0) { prefs.stepQueueLength = (unsigned int)stepQueue; }
 #else
-        (void)ordered;
+        (void)ordered; (void)stepQueue;
 #endif
         Logging::init(prefs.gennLogLevel, prefs.codeGeneratorLogLevel, prefs.transpilerLogLevel,
                       prefs.runtimeLogLevel, &app, &app, &app, &app);
@@ -567,6 +570,7 @@ int main(int argc, char *argv[])
         };
 
         const auto loopStart = std::chrono::steady_clock::now();
+        double firstSeconds = 0.0;
         for(unsigned int i = 0; i < steps; i++) {
             for(auto &c : css) {
                 if(c.model == "noise") {
@@ -586,12 +590,15 @@ int main(int argc, char *argv[])
             }
             rt.stepTime();
             if(snap && ((i + 1) % snap) == 0) snapshot();
+            // the first call also builds whatever the backend prepares lazily (the MI355X backend: its device tables)
+            if(i == 0) { firstSeconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - loopStart).count(); }
         }
         // a blocking pull drains whatever the backend still has queued, so the loop time below is complete
         if(!pops.empty() && pops.front().model != "ssa") { rt.getArray(*pops.front().ng, "V")->pullFromDevice(); }
         const double loopSeconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - loopStart).count();
         std::cout << "ref_driver: stepping loop " << loopSeconds << " s for " << steps << " steps ("
-                  << loopSeconds / steps * 1e6 << " us per Runtime::stepTime, snapshots included)" << std::endl;
+                  << loopSeconds / steps * 1e6 << " us per Runtime::stepTime, snapshots included; first call " << firstSeconds * 1e3
+                  << " ms, the others " << (steps > 1 ? (loopSeconds - firstSeconds) / (steps - 1) * 1e6 : 0.0) << " us each)" << std::endl;
         if(!snap || (steps % snap) != 0) snapshot();
 
         // spike rasters as (step, id) pairs; the reference reports times in ms = step*dt

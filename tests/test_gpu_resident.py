@@ -139,6 +139,49 @@ def test_pushed_weights_reach_the_inline_copies(monkeypatch):
     model.unload()
 
 
+@pytest.mark.parametrize("limit, rows", [(64, 230), (1000, 230), (7, 230), (64, 50), (64, 0)])
+def test_queued_single_steps_take_the_resident_launch(limit, rows):
+    """step_time() one call at a time with the step queue on (what the reference's Runtime::stepTime amounts to): the steps
+    run as resident launches of up to `limit` steps, cut wherever something looks at the device -- state pulls, a push
+    of membrane potentials, the event counter, a recording buffer of `rows` rows that wraps -- and everything is as unqueued stepping leaves it."""
+    n_a, n_b, depth = 700, 300, 7
+    net = Net(name="resident_queue", dt=1.0, steps=230)
+    net.pops.append(_pop("A", n_a, 0.62, -60.0 + 9.5 * rng.uniform(5, 1, 0, n_a)))
+    net.pops.append(_pop("B", n_b, 0.45, -60.0 + 9.5 * rng.uniform(5, 2, 0, n_b)))
+    net.syns.append(_projection("AB", "A", "B", n_a, n_b, 40, 0.11, 11, depth, 0.3))
+    net.syns.append(_projection("BA", "B", "A", n_b, n_a, 64, -0.07, 12, depth, 0.3))
+    model = model_from_net(net, record=bool(rows))
+    model.load(num_recording_timesteps=rows or None)
+    assert model.runner_info()["resident_plan"]
+    model.set_step_queue(limit)
+    oracle = OracleNet(net, num_recording_timesteps=rows)
+    done = 0
+    for chunk in (1, 2, 3, 40, 9, 100, 75):
+        for _ in range(chunk):
+            model.step_time()
+        oracle.run(chunk)
+        done += chunk
+        if done == 55:
+            # a push lands between the steps it was issued between (the steps queued before it have run by then)
+            v = model.neuron_populations["B"].vars["V"]
+            v.pull_from_device()
+            v.view[::3] = np.float32(-50.5)
+            v.push_to_device()
+            oracle.var("B", 0)[::3] = np.float32(-50.5)
+        elif done == 155:
+            assert model.synaptic_event_count == oracle.events()
+        else:
+            compare_state(net, model, oracle, f"after {done} queued steps", exact=True)      # pulls, no synchronize() first
+    assert done == net.steps
+    if rows:
+        model.pull_recording_buffers_from_device()
+        for p in net.pops:
+            assert np.array_equal(model.neuron_populations[p.name].vars["recordSpk"].view, oracle.record(p.name, rows)), f"recording of {p.name} differs"
+    assert model.synaptic_event_count == oracle.events() and oracle.events() > 50000
+    model.set_step_queue(0)
+    model.unload()
+
+
 def test_plan_can_be_switched_off(monkeypatch):
     monkeypatch.setenv("GENNMI_RESIDENT", "0")
     n, depth = 600, 4
