@@ -651,7 +651,9 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
                 const bool graded = (wumKind == GENNMI_WUM_STATIC_GRADED);
                 if((arch.isPreSpikeEventRequired() && !graded) || arch.isPostSpikeEventRequired()) { unsupported("spike-like events on projection '" + arch.getName() + "'"); }
                 if(graded && srcDelay) { unsupported("delay slots on the source of graded projection '" + arch.getName() + "'"); }
-                if(plastic && batchSize != 1) { unsupported("plastic weights with a batch size above 1"); }
+                // (plastic weights, traces and spike times with a batch size above 1: one copy per batch, batch-major, which is
+                // how the Runtime lays out variables with the batch dimension and how the device library indexes them)
+                if(plastic && batchSize != 1 && getPreferences<Preferences>().orderedAccumulation) { unsupported("ordered accumulation of plastic weights with a batch size above 1"); }
 
                 const auto matrixType = arch.getMatrixType();
                 const bool sparse = (matrixType & SynapseMatrixConnectivity::SPARSE) && (matrixType & SynapseMatrixWeight::INDIVIDUAL);

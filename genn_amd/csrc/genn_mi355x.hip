@@ -63,6 +63,8 @@ struct gennmi_runner
     bool fusedStep = false;             // zero-delay synapses are delivered by the neuron update; one launch per step
     TileGroupDev *dTile = nullptr; uint32_t tileBlocks = 0, tileFloats = 0, tileThreads = BLOCK;
     uint32_t postLdsBytes = 0;
+    // one launch for the scatter path, the tile path and the paired postsynaptic passes of a step (synapseCombinedKernel)
+    bool combineSynapses = false, combinePost = false; uint32_t synapseThreads = BLOCK; size_t combinedLdsBytes = 0;
     ConvTileDev *dConvTile = nullptr; uint32_t convTileBlocks = 0; size_t convTileBytes = 0;
     std::vector<void*> owned;           // engine-private device allocations (shadow queues, zero-delay lists)
     // resident plan (many steps per launch)
@@ -471,11 +473,9 @@ int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynap
         }
         else if(g->wum == GENNMI_WUM_STDP_TRACE) {
             if(!g->trgST || !g->postTrace) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: STDP arrays missing"); }
-            if(r->batch != 1) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: plastic weights need batch size 1"); }
         }
         else if(g->wum == GENNMI_WUM_STDP) {
             if(!g->trgST || !(g->tauMinus > 0.0f)) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: STDP needs the target's spike times and tauMinus > 0"); }
-            if(r->batch != 1) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: plastic weights need batch size 1"); }
         }
         else if(g->wum == GENNMI_WUM_STATIC_PULSE_REVERSE) {
             if(!g->outPre) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: outPre missing"); }
@@ -514,7 +514,6 @@ int gennmi_push_postsynaptic_update_group(gennmi_runner *r, const gennmi_postsyn
         return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: required array missing");
     }
     if(g->rowStride == 0 || g->colStride == 0) { return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: zero stride"); }
-    if(r->batch != 1) { return fail(GENNMI_EUNSUPPORTED, "push_postsynaptic_update_group: plastic weights need batch size 1"); }
     if((g->rowLength == nullptr) != (g->ind == nullptr)) { return fail(GENNMI_EINVAL, "push_postsynaptic_update_group: rowLength and ind go together"); }
     PostGroupDev d;
     memset(&d, 0, sizeof(d));
@@ -987,6 +986,47 @@ int gennmi_runner_finalise(gennmi_runner *r)
             }
         }
     }
+    // ---- plastic projections: pair the postsynaptic pass of each with its presynaptic half (LearnPostDev), so that every
+    // synapse has one writer per step and the passes can share a launch.  Needs the spikes of the last neuron update of both
+    // populations as bitmaps, which their neuron updates keep.  GENNMI_PAIRED_LEARN=0 leaves the passes as two launches in a row.
+    {
+        const char *envPaired = getenv("GENNMI_PAIRED_LEARN");
+        const bool pairing = !r->ordered && !(envPaired && atoi(envPaired) == 0);
+        auto populationOf = [r](const uint32_t *queue, uint32_t numNeurons) -> NeuronGroupDev*
+        {
+            for(auto &n : r->neuron) {
+                bool feeds = (n.g.spk == queue);
+                for(uint32_t q = 0; q < n.g.numExtraSpk; q++) { feeds = feeds || (n.g.extraSpk[q] == queue); }
+                if(feeds && n.g.numNeurons == numNeurons) { return &n; }
+            }
+            return nullptr;
+        };
+        auto bitmapOf = [r](NeuronGroupDev *n) -> hipError_t
+        {
+            if(n->spikeBitmap) { return hipSuccess; }
+            const size_t bytes = (size_t)r->batch * ((n->g.numNeurons + 31) / 32) * sizeof(uint32_t);
+            hipError_t e = hipMalloc((void**)&n->spikeBitmap, bytes);
+            if(e != hipSuccess) { return e; }
+            r->owned.push_back(n->spikeBitmap);
+            return hipMemset(n->spikeBitmap, 0, bytes);
+        };
+        r->combinePost = pairing && !r->post.empty();
+        for(auto &p : r->post) {
+            PreGroupDev *partner = nullptr;
+            for(auto &q : r->pre) {
+                if(q.g.g == p.g.g && (q.g.wum == GENNMI_WUM_STDP_TRACE || q.g.wum == GENNMI_WUM_STDP) && q.g.matrix == GENNMI_MATRIX_SPARSE
+                   && q.g.numSrcDelaySlots <= 1 && q.g.numSrcNeurons == p.g.numSrcNeurons && q.g.numTrgNeurons == p.g.numTrgNeurons) { partner = &q; }
+            }
+            NeuronGroupDev *src = partner ? populationOf(partner->g.srcSpk, p.g.numSrcNeurons) : nullptr;
+            NeuronGroupDev *trg = populationOf(p.g.trgSpk, p.g.numTrgNeurons);
+            if(!pairing || !partner || !src || !trg || std::max(1u, src->g.numDelaySlots) > 1 || std::max(1u, trg->g.numDelaySlots) > 1) { r->combinePost = false; continue; }
+            HIP_TRY(bitmapOf(src));
+            HIP_TRY(bitmapOf(trg));
+            partner->learn.srcST = p.g.srcST; partner->learn.preTrace = p.g.preTrace; partner->learn.trgBitmap = trg->spikeBitmap;
+            partner->learn.aPlus = p.g.aPlus; partner->learn.tauPlus = p.g.tauPlus; partner->learn.enabled = 1;
+            p.srcBitmap = src->spikeBitmap;
+        }
+    }
     // Large networks of plain groups take the several-neurons-per-lane kernel: what counts is the number of rounds of
     // resident work-groups a launch needs (numCU x 8 work-groups of 256 lanes are resident at a time).
     {
@@ -1019,54 +1059,6 @@ int gennmi_runner_finalise(gennmi_runner *r)
     }
     r->neuronBlocks = block;
 
-    // Presynaptic launch geometry.  The number of spikes is only known on the device, so every
-    // group gets a fixed number of blocks and deals its (spike, chunk) work items round-robin to their
-    // sub-groups.  A group wants enough sub-groups for ~1.5 % of its source population firing in one step; when
-    // the groups together want more than the budget, it is shared in proportion (work per step scales with
-    // source size x row length, whatever the rates turn out to be).
-    block = 0;
-    const char *envBudget = getenv("GENNMI_PRESYN_BLOCKS_PER_CU");
-    const uint32_t blocksPerCU = envBudget ? std::max(1, atoi(envBudget)) : 4u;
-    // the launch has one grid row per batch, so the budget is per batch (at least one block per compute unit in all)
-    const uint64_t budget = std::max<uint64_t>((numCU + r->batch - 1) / r->batch, (uint64_t)numCU * blocksPerCU / r->batch);
-    std::vector<uint64_t> wantBlocks;
-    for(auto &p : r->pre) {
-        const uint32_t rowLen = (p.g.matrix == GENNMI_MATRIX_SPARSE) ? p.g.rowStride : (uint32_t)(p.g.conv[0] * p.g.conv[1] * p.g.conv[7]);
-        uint32_t W;
-        if(p.g.span == GENNMI_SPAN_PRE) { W = std::min(64u, pow2Ceil(std::max(1u, p.g.numThreadsPerSpike))); }
-        else if(p.g.span == GENNMI_SPAN_POST) { W = WAVE; }
-        else { W = std::min<uint32_t>(WAVE, std::max(4u, pow2Ceil((rowLen + 3) / 4))); }
-        p.lanesPerSpike = W;
-        p.vec4 = (p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum != GENNMI_WUM_STDP_TRACE && p.g.wum != GENNMI_WUM_STDP && (p.g.rowStride % 4) == 0
-                  && (reinterpret_cast<uintptr_t>(p.g.ind) % 16) == 0 && (reinterpret_cast<uintptr_t>(p.g.g) % 16) == 0
-                  && (p.g.wum != GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY || (reinterpret_cast<uintptr_t>(p.g.d) % 4) == 0)
-                  && W >= 16) ? 1u : 0u;
-        const uint32_t span = W * (p.vec4 ? 4u : 1u);
-        const uint64_t chunksPerRow = (rowLen + span - 1) / span;
-        const uint64_t wantSubGroups = std::max<uint64_t>(8, ((uint64_t)p.g.numSrcNeurons * chunksPerRow) / 64);
-        wantBlocks.push_back(std::min<uint64_t>((wantSubGroups * W + BLOCK - 1) / BLOCK, budget));
-    }
-    uint64_t wantTotal = 0;
-    for(uint64_t w : wantBlocks) { wantTotal += w; }
-    for(size_t k = 0; k < r->pre.size(); k++) {
-        auto &p = r->pre[k];
-        const uint64_t blocks = (wantTotal <= budget) ? wantBlocks[k] : (wantBlocks[k] * budget + wantTotal - 1) / wantTotal;
-        p.startBlock = block;
-        p.numBlocks = (uint32_t)std::max<uint64_t>(1, blocks);
-        block += p.numBlocks;
-    }
-    r->preBlocks = block;
-
-    block = 0;
-    for(auto &p : r->post) {
-        p.lanesPerSpike = std::min<uint32_t>(WAVE, std::max(4u, pow2Ceil((p.g.colStride + 3) / 4)));
-        const uint64_t wantSubGroups = std::max<uint64_t>(8, p.g.numTrgNeurons / 16);
-        const uint32_t cap = std::max(1u, (numCU * 16u) / (uint32_t)r->post.size());
-        p.startBlock = block;
-        p.numBlocks = std::max(1u, (uint32_t)std::min<uint64_t>((wantSubGroups * p.lanesPerSpike + BLOCK - 1) / BLOCK, cap));
-        block += p.numBlocks;
-    }
-    r->postBlocks = block;
 
     // DENSE / BITMASK projections: one lane per postsynaptic neuron; a group owns its outPost unless another dense or
     // bitmask group adds to the same one (sparse groups have finished by the time this kernel starts)
@@ -1158,7 +1150,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
             r->tileTables.push_back({(size_t)(&p - r->pre.data()), dOff, tileSize, numTiles});
             const uint32_t avgSeg = std::max(1u, p.g.rowStride / numTiles);
             TileGroupDev t{};
-            t.g = p.g; t.tileOff = dOff; t.numTiles = numTiles; t.tileSize = tileSize;
+            t.g = p.g; t.learn = p.learn; t.tileOff = dOff; t.numTiles = numTiles; t.tileSize = tileSize;
             const char *envLanes = getenv("GENNMI_TILE_LANES");
             t.lanes = envLanes ? std::min<uint32_t>(WAVE, pow2Ceil((uint32_t)std::max(1, atoi(envLanes)))) : std::min<uint32_t>(WAVE, pow2Ceil((avgSeg + 7) / 8));
             t.threshold = p.tileThreshold;
@@ -1200,8 +1192,14 @@ int gennmi_runner_finalise(gennmi_runner *r)
             const char *envSplit = getenv("GENNMI_TILE_BLOCKS_PER_CU");
             const uint32_t blocksPerCUTile = envSplit ? (uint32_t)std::max(1, atoi(envSplit)) : 4u;
             const uint32_t budget = blocksPerCUTile * numCU * BLOCK / r->tileThreads;
+            // ... several groups share two such rounds in proportion to their synapse counts: a launch's floor is the
+            // dispatch of its blocks, and the quiet steps of a network with many projections should not pay for a round each
+            double totalWeight = 0.0;
+            for(const auto &t : tileGroups) { totalWeight += (double)t.g.numSrcNeurons * t.g.rowStride; }
             for(auto &t : tileGroups) {
-                const uint32_t numSplits = std::max(1u, std::min(256u, budget / t.numTiles));
+                const double share = (tileGroups.size() == 1) ? 1.0 : 2.0 * ((double)t.g.numSrcNeurons * t.g.rowStride) / totalWeight;
+                const uint32_t groupBudget = std::max(t.numTiles, (uint32_t)(share * budget));
+                const uint32_t numSplits = std::max(1u, std::min(256u, groupBudget / t.numTiles));
                 t.numSplits = numSplits;
                 for(uint32_t tile = 0; tile < t.numTiles; tile++) {
                     for(uint32_t split = 0; split < numSplits; split++) { t.tile = tile; t.split = split; tiles.push_back(t); }
@@ -1227,6 +1225,59 @@ int gennmi_runner_finalise(gennmi_runner *r)
             }
         }
     }
+
+    // Presynaptic launch geometry.  The number of spikes is only known on the device, so every
+    // group gets a fixed number of blocks and deals its (spike, chunk) work items round-robin to their
+    // sub-groups.  A group wants enough sub-groups for ~1.5 % of its source population firing in one step; when
+    // the groups together want more than the budget, it is shared in proportion (work per step scales with
+    // source size x row length, whatever the rates turn out to be).
+    // Scatter, tile and postsynaptic blocks may share a launch (synapseCombinedKernel), so all three use the tile path's
+    // block size where there is one; budgets are in blocks of 256 threads and converted.
+    block = 0;
+    const uint32_t synThreads = r->tileBlocks ? r->tileThreads : (uint32_t)BLOCK;
+    r->synapseThreads = synThreads;
+    const char *envBudget = getenv("GENNMI_PRESYN_BLOCKS_PER_CU");
+    const uint32_t blocksPerCU = envBudget ? std::max(1, atoi(envBudget)) : 4u;
+    // the launch has one grid row per batch, so the budget is per batch (at least one block per compute unit in all)
+    const uint64_t budget = std::max<uint64_t>((numCU + r->batch - 1) / r->batch, (uint64_t)numCU * blocksPerCU * BLOCK / synThreads / r->batch);
+    std::vector<uint64_t> wantBlocks;
+    for(auto &p : r->pre) {
+        const uint32_t rowLen = (p.g.matrix == GENNMI_MATRIX_SPARSE) ? p.g.rowStride : (uint32_t)(p.g.conv[0] * p.g.conv[1] * p.g.conv[7]);
+        uint32_t W;
+        if(p.g.span == GENNMI_SPAN_PRE) { W = std::min(64u, pow2Ceil(std::max(1u, p.g.numThreadsPerSpike))); }
+        else if(p.g.span == GENNMI_SPAN_POST) { W = WAVE; }
+        else { W = std::min<uint32_t>(WAVE, std::max(4u, pow2Ceil((rowLen + 3) / 4))); }
+        p.lanesPerSpike = W;
+        p.vec4 = (p.g.matrix == GENNMI_MATRIX_SPARSE && p.g.wum != GENNMI_WUM_STDP_TRACE && p.g.wum != GENNMI_WUM_STDP && (p.g.rowStride % 4) == 0
+                  && (reinterpret_cast<uintptr_t>(p.g.ind) % 16) == 0 && (reinterpret_cast<uintptr_t>(p.g.g) % 16) == 0
+                  && (p.g.wum != GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY || (reinterpret_cast<uintptr_t>(p.g.d) % 4) == 0)
+                  && W >= 16) ? 1u : 0u;
+        const uint32_t span = W * (p.vec4 ? 4u : 1u);
+        const uint64_t chunksPerRow = (rowLen + span - 1) / span;
+        const uint64_t wantSubGroups = std::max<uint64_t>(8, ((uint64_t)p.g.numSrcNeurons * chunksPerRow) / 64);
+        wantBlocks.push_back(std::min<uint64_t>((wantSubGroups * W + synThreads - 1) / synThreads, budget));
+    }
+    uint64_t wantTotal = 0;
+    for(uint64_t w : wantBlocks) { wantTotal += w; }
+    for(size_t k = 0; k < r->pre.size(); k++) {
+        auto &p = r->pre[k];
+        const uint64_t blocks = (wantTotal <= budget) ? wantBlocks[k] : (wantBlocks[k] * budget + wantTotal - 1) / wantTotal;
+        p.startBlock = block;
+        p.numBlocks = (uint32_t)std::max<uint64_t>(1, blocks);
+        block += p.numBlocks;
+    }
+    r->preBlocks = block;
+
+    block = 0;
+    for(auto &p : r->post) {
+        p.lanesPerSpike = std::min<uint32_t>(WAVE, std::max(4u, pow2Ceil((p.g.colStride + 3) / 4)));
+        const uint64_t wantSubGroups = std::max<uint64_t>(8, p.g.numTrgNeurons / 16);
+        const uint32_t cap = std::max(1u, (numCU * 4u * BLOCK / synThreads) / (uint32_t)r->post.size());
+        p.startBlock = block;
+        p.numBlocks = std::max(1u, (uint32_t)std::min<uint64_t>((wantSubGroups * p.lanesPerSpike + synThreads - 1) / synThreads, cap));
+        block += p.numBlocks;
+    }
+    r->postBlocks = block;
 
     // ---- single-launch step: possible when every projection is a SPARSE dendritic-delay one with ring depth >= 2
     // and nothing is plastic
@@ -1256,8 +1307,8 @@ int gennmi_runner_finalise(gennmi_runner *r)
             for(uint32_t q = 0; q < n.g.numExtraSpk; q++) { feeds = feeds || (n.g.extraSpk[q] == p.g.trgSpk); }
             if(!feeds || n.g.numNeurons != p.g.numTrgNeurons) { continue; }
             if(!n.spikeBitmap) {
-                HIP_TRY(hipMalloc((void**)&n.spikeBitmap, words * sizeof(uint32_t)));
-                HIP_TRY(hipMemset(n.spikeBitmap, 0, words * sizeof(uint32_t)));
+                HIP_TRY(hipMalloc((void**)&n.spikeBitmap, (size_t)r->batch * words * sizeof(uint32_t)));
+                HIP_TRY(hipMemset(n.spikeBitmap, 0, (size_t)r->batch * words * sizeof(uint32_t)));
                 r->owned.push_back(n.spikeBitmap);
             }
             p.spikeBitmap = n.spikeBitmap;
@@ -1270,6 +1321,16 @@ int gennmi_runner_finalise(gennmi_runner *r)
     if(r->postLdsBytes > 48 * 1024) {
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(postsynapticUpdateKernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)r->postLdsBytes));
     }
+    // ---- one launch for scatter path, tile path and paired postsynaptic passes (GENNMI_COMBINED=0: a launch each)
+    {
+        const char *envCombined = getenv("GENNMI_COMBINED");
+        r->combineSynapses = !r->ordered && !(envCombined && atoi(envCombined) == 0) && (r->tileBlocks != 0 || r->combinePost);
+        r->combinedLdsBytes = std::max<size_t>(r->tileBlocks ? (size_t)r->tileFloats * sizeof(float) : 0, r->combinePost ? r->postLdsBytes : 0);
+        if(r->combineSynapses && r->combinedLdsBytes > 48 * 1024) {
+            HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(synapseCombinedKernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)r->combinedLdsBytes));
+        }
+    }
+    if(r->ordered && r->batch != 1 && !r->post.empty()) { return fail(GENNMI_EUNSUPPORTED, "runner_finalise: ordered accumulation of plastic projections needs batch size 1"); }
     // spike sources: per-neuron copy of the next spike time, built before the first step and again after writes to the arrays
     for(auto &n : r->neuron) {
         if(n.g.model != GENNMI_NEURON_SPIKE_SOURCE_ARRAY) { continue; }
@@ -1368,6 +1429,7 @@ static int refreshSpikeSources(gennmi_runner *r)
 static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
 {
     hipEvent_t e0 = nullptr, e1 = nullptr, e2 = nullptr;
+    bool postInCombined = false;
     if(timed) {
         if(r->pending.size() >= 2048) { const int rc = drainTimers(r); if(rc) { return rc; } }
         const int rc = stamp(r, &e0); if(rc) { return rc; }
@@ -1385,13 +1447,22 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
                 presynapticOrderedKernel<<<dim3((o.g.numTrgNeurons + (BLOCK / WAVE) - 1) / (BLOCK / WAVE), r->batch), dim3(BLOCK), 0, r->stream>>>(o, a, r->dt, r->dEvents);
             }
         }
-        if(r->preBlocks && r->scatterNeeded) {
-            presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dPre, a, r->dt, r->dEvents);
+        // (timed runs keep a launch per kernel, so that presynaptic and postsynaptic time stay apart as the reference reports them)
+        const bool combined = r->combineSynapses && !timed;
+        if(combined) {
+            const uint32_t scatterBlocks = (r->preBlocks && r->scatterNeeded) ? r->preBlocks : 0u;
+            const uint32_t postBlocks = r->combinePost ? r->postBlocks : 0u;
+            postInCombined = (postBlocks != 0);
+            synapseCombinedKernel<<<dim3(scatterBlocks + r->tileBlocks + postBlocks, r->batch), dim3(r->synapseThreads), r->combinedLdsBytes, r->stream>>>(
+                r->dPre, scatterBlocks, r->dTile, r->tileBlocks, r->dPost, a, r->dt, r->dEvents);
+        }
+        else if(r->preBlocks && r->scatterNeeded) {
+            presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(r->synapseThreads), 0, r->stream>>>(r->dPre, a, r->dt, r->dEvents);
         }
         if(r->denseBlocks) {
             presynapticDenseKernel<<<dim3(r->denseBlocks, r->batch), dim3(BLOCK), 0, r->stream>>>(r->dDense, r->dEvents);
         }
-        if(r->tileBlocks) {
+        if(r->tileBlocks && !combined) {
             presynapticTileKernel<<<dim3(r->tileBlocks, r->batch), dim3(r->tileThreads), r->tileFloats * sizeof(float), r->stream>>>(r->dTile, a, r->dt, r->dEvents);
         }
         if(r->convTileBlocks) {
@@ -1399,8 +1470,8 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
         }
         if(timed) { const int rc = stamp(r, &e1); if(rc) { return rc; } r->pending.push_back({e0, e1, 0}); }
     }
-    if(!r->post.empty()) {
-        postsynapticUpdateKernel<<<dim3(r->postBlocks), dim3(BLOCK), r->postLdsBytes, r->stream>>>(r->dPost, a, r->dt);
+    if(!r->post.empty() && !postInCombined) {
+        postsynapticUpdateKernel<<<dim3(r->postBlocks, r->batch), dim3(r->synapseThreads), r->postLdsBytes, r->stream>>>(r->dPost, a, r->dt);
         if(timed) { const int rc = stamp(r, &e2); if(rc) { return rc; } r->pending.push_back({e1 ? e1 : e0, e2, 1}); }
     }
     HIP_TRY(hipGetLastError());
@@ -1674,7 +1745,8 @@ int gennmi_runner_get_info(gennmi_runner *r, uint32_t info[4])
 {
     if(!r || !info) { return fail(GENNMI_EINVAL, "runner_get_info: null argument"); }
     if(!r->finalised) { return fail(GENNMI_ESTATE, "runner_get_info: runner not finalised"); }
-    info[0] = (r->fusedStep ? 1u : 0u) | (r->resident ? 2u : 0u) | (r->neuronsPerLane > 1 ? 4u : 0u) | (r->ordered ? 8u : 0u); info[1] = r->neuronBlocks; info[2] = r->preBlocks; info[3] = r->postBlocks;
+    info[0] = (r->fusedStep ? 1u : 0u) | (r->resident ? 2u : 0u) | (r->neuronsPerLane > 1 ? 4u : 0u) | (r->ordered ? 8u : 0u)
+              | (r->combineSynapses ? 16u : 0u) | ((r->combineSynapses && r->combinePost) ? 32u : 0u); info[1] = r->neuronBlocks; info[2] = r->preBlocks; info[3] = r->postBlocks;
     return GENNMI_OK;
 }
 

@@ -95,15 +95,31 @@ struct NeuronGroupDev
     const ZeroDelayEntry *zeroEntries;
     uint32_t *shadowSpk;                // [2][batch*N] engine-private double-buffered copy of the spike queue, or NULL
     uint32_t *shadowCnt;                // [2][batch]
-    uint32_t *spikeBitmap;              // [ceil(N/32)] engine-private bitmap of this step's spikes (populations with learnPost), or NULL
+    uint32_t *spikeBitmap;              // [batch][ceil(N/32)] engine-private bitmap of this step's spikes (populations at either end of a plastic projection), or NULL
     unsigned long long *aggEvent;       // look-back area of the spike-like event queues (groups with events), or NULL
     float *nextSpikeTime;               // spike sources: engine-private copy of spikeTimes[startSpike] per neuron (+inf: none left)
     size_t spikeTimesBytes;             // spike sources: bytes from spikeTimes to the end of its allocation (host bookkeeping)
 };
 
+// The learnPost half of a plastic projection, as its presynaptic half needs it.  The reference runs the presynaptic update of
+// every projection, then the postsynaptic one (backendSIMT.cc genPresynapticUpdateKernel / genPostsynapticUpdateKernel,
+// launched one after the other): a synapse whose two ends both fired in the last neuron update gets the presynaptic-spike
+// rule first and the postsynaptic-spike rule second.  Here the thread that applies the first rule to such a synapse also
+// applies the second, and the postsynaptic pass leaves every synapse of a row whose neuron fired to it — each synapse has
+// one writer per step, the order on it is the reference's, and the two passes need not wait for each other.
+struct LearnPostDev
+{
+    const float *srcST, *preTrace;      // [batch][numSrc] the postsynaptic-spike rule's view of the source neurons
+    const uint32_t *trgBitmap;          // [batch][ceil(numTrg/32)] the target population's spikes of the last neuron update
+    float aPlus, tauPlus;
+    uint32_t enabled;                   // 0: the projection has no such partner, its presynaptic half is all there is
+    uint32_t pad_;
+};
+
 struct PreGroupDev
 {
     gennmi_presynaptic_update_group_t g;
+    LearnPostDev learn;
     uint32_t startBlock, numBlocks;
     uint32_t lanesPerSpike;             // power of two, 1..64
     uint32_t vec4;                      // rows are 16-byte aligned and padded: dwordx4 loads
@@ -121,6 +137,7 @@ struct PreGroupDev
 struct TileGroupDev
 {
     gennmi_presynaptic_update_group_t g;
+    LearnPostDev learn;
     const uint16_t *tileOff;            // [numSrc*(numTiles+1)] first position of every row whose target is >= tile*tileSize
     uint32_t numTiles, tileSize;
     uint32_t tile, split, numSplits;    // this block: which tile, which share of the spikes
@@ -160,7 +177,8 @@ struct PostGroupDev
     uint32_t startBlock, numBlocks;
     uint32_t lanesPerSpike;
     uint32_t denseThreshold;            // != 0: steps with at least this many postsynaptic spikes walk the rows instead
-    const uint32_t *spikeBitmap;        // [ceil(numTrg/32)] this step's postsynaptic spikes, written by the neuron update
+    const uint32_t *spikeBitmap;        // [batch][ceil(numTrg/32)] this step's postsynaptic spikes, written by the neuron update
+    const uint32_t *srcBitmap;          // [batch][ceil(numSrc/32)] != NULL: rows of neurons that fired are left to the presynaptic pass (LearnPostDev)
 };
 
 // Block -> group: groups occupy consecutive block ranges (the reference pads thread ranges to block

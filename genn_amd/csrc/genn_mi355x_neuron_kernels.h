@@ -301,7 +301,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
         const uint32_t words = (n + 31) / 32;
         g.recordSpk[((size_t)st.recT * gridDim.y + batch) * words + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
     }
-    if(G.spikeBitmap && (lane & 31) == 0 && i < n) { G.spikeBitmap[i >> 5] = (uint32_t)(ballot >> (lane & 32)); }
+    if(G.spikeBitmap && (lane & 31) == 0 && i < n) { G.spikeBitmap[(size_t)batch * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballot >> (lane & 32)); }
     __syncthreads();
 
     uint32_t blockCount = 0, waveOffset = 0;

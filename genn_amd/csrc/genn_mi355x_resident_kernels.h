@@ -293,6 +293,9 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             if(c == 0 || np == 0) { continue; }
             uint32_t pos = atomicAdd(&shScalar[0], c * np);
             if(pos + c * np > RES_PAIR_CAP) { continue; }
+            // ids beyond those inside the word were stored before a release fence and the word after it (publish): the
+            // reads below must not be served ahead of the word's load
+            if(c > RES_WORD_IDS) { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
             for(uint32_t e = 0; e < c; e++) {
                 const uint32_t id = (c <= RES_WORD_IDS) ? watchFirst[q] + (((uint32_t)word[q] >> (8 * e)) & 0xFFu)
                                                         : __hip_atomic_load(&side[((size_t)parity * numTiles + tid + q * BLOCK) * RES_T + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -406,6 +409,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
                 const uint32_t p0 = shProjStart[s], np = shProjStart[s + 1] - p0;
                 if(c == 0 || np == 0) { continue; }
                 if(pos + c * np <= chunk0 || pos >= chunk0 + RES_PAIR_CAP) { pos += c * np; continue; }
+                if(c > RES_WORD_IDS) { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }     // as in poll()
                 for(uint32_t q = 0; q < c; q++) {
                     const uint32_t id = (c <= RES_WORD_IDS) ? tiles[k].first + (((uint32_t)tag >> (8 * q)) & 0xFFu)
                                                             : __hip_atomic_load(&side[((size_t)parity * numTiles + k) * RES_T + q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -4,6 +4,24 @@
 
 namespace
 {
+// The postsynaptic-spike rule on one synapse (pygenn/genn_model.py:1464-1471 for the trace rule, weightUpdateModels.h:360-366
+// for the built-in additive one), with the arithmetic of postsynapticUpdateKernel: used by the presynaptic passes for synapses
+// whose target fired in the last neuron update as well (see LearnPostDev).
+__device__ __forceinline__ float learnPostOnSynapse(const LearnPostDev &L, const gennmi_presynaptic_update_group_t &g, uint32_t batch,
+                                                    uint32_t idPre, float w, float t, float dt, bool &changed)
+{
+    const size_t pre = (size_t)batch * g.numSrcNeurons + idPre;
+    const float stPre = dt + asGlobal(L.srcST)[pre];
+    const float dtSpike = t - stPre;
+    if(dtSpike > 0) {
+        const float factor = (L.tauPlus > 0.0f) ? (float)exp((double)(-dtSpike / L.tauPlus)) : asGlobal(L.preTrace)[pre];
+        changed = true;
+        return fminf(g.wMax, fmaxf(g.wMin, w + (L.aPlus * factor)));
+    }
+    return w;
+}
+__device__ __forceinline__ bool bitmapTest(GLOBAL_AS const uint32_t *bitmap, uint32_t i) { return (bitmap[i >> 5] >> (i & 31)) & 1u; }
+
 // ------------------------------------------------------------------------------------------------
 // Presynaptic update.  The unit of work is (spike, chunk of its row): a sub-group of
 // `lanesPerSpike` lanes handles `span` consecutive synapses of one row, so a long row is spread
@@ -23,8 +41,8 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
     const uint32_t W = G.lanesPerSpike;
     const uint32_t localBlock = blockInKernel - G.startBlock;
     const uint32_t lis = threadIdx.x & (W - 1);
-    const uint32_t subGroup = (localBlock * BLOCK + threadIdx.x) / W;
-    const uint32_t numSubGroups = (G.numBlocks * BLOCK) / W;
+    const uint32_t subGroup = (localBlock * blockDim.x + threadIdx.x) / W;      // (any multiple of the wavefront size will do as block size)
+    const uint32_t numSubGroups = (G.numBlocks * blockDim.x) / W;
     // spikes of the previous step: the population's own queue, or (when this launch may run next to the
     // neuron update that refills that queue) the shadow copy written one step ago
     const uint32_t parity = (uint32_t)((st.epoch + 1) & 1);
@@ -179,18 +197,27 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
             else if(j < npost) {
                 // trace STDP presynaptic-spike code (pygenn/genn_model.py:1456-1463); every synapse of
                 // the row is owned by exactly one lane, so the read-modify-write of g needs no atomic
+                // (plastic weights, spike times and traces are per batch: VarAccess::READ_WRITE variables are duplicated)
                 const uint32_t idPost = ind[rowBase + j];
-                const float w = weight[rowBase + j];
-                const float stPost = dt + asGlobal(g.trgST)[idPost];   // st_post = DT*(backPropSteps+1) + trgST (synapseUpdateGroupMerged.cc:134-142)
+                GLOBAL_AS float *wPtr = weight + (size_t)batch * g.numSrcNeurons * g.rowStride + rowBase + j;
+                const float w = *wPtr;
+                const size_t post = (size_t)batch * numTrg + idPost;
+                const float stPost = dt + asGlobal(g.trgST)[post];   // st_post = DT*(backPropSteps+1) + trgST (synapseUpdateGroupMerged.cc:134-142)
                 atomicAddF32(&outPost[idPost], w);
                 const float dtSpike = st.t - stPost;
+                float newWeight = w;
+                bool changed = false;
                 if(dtSpike > 0) {
                     // trace rule: the target's trace; built-in additive rule (weightUpdateModels.h:352-359): the exponential
                     // of the time since the target's last spike, evaluated in double and rounded once as the reference does
-                    const float factor = (g.wum == GENNMI_WUM_STDP) ? (float)exp((double)(-dtSpike / g.tauMinus)) : asGlobal(g.postTrace)[idPost];
-                    const float newWeight = w - (g.aMinus * factor);
-                    weight[rowBase + j] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
+                    const float factor = (g.wum == GENNMI_WUM_STDP) ? (float)exp((double)(-dtSpike / g.tauMinus)) : asGlobal(g.postTrace)[post];
+                    newWeight = fminf(g.wMax, fmaxf(g.wMin, w - (g.aMinus * factor)));
+                    changed = true;
                 }
+                if(G.learn.enabled && bitmapTest(asGlobal(G.learn.trgBitmap) + (size_t)batch * ((numTrg + 31) / 32), idPost)) {
+                    newWeight = learnPostOnSynapse(G.learn, g, batch, idPre, newWeight, st.t, dt, changed);
+                }
+                if(changed) { *wPtr = newWeight; }
             }
             if(lis == 0 && chunk == 0) { events += npost; }
         }
@@ -434,11 +461,8 @@ __device__ __forceinline__ unsigned long long tileRecordLoop(const TileGroupDev 
     return events;
 }
 
-__global__ __launch_bounds__(1024)
-void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs args, float dt, unsigned long long *eventCounter)
+__device__ __forceinline__ void presynapticTileBody(const TileGroupDev &G, float *shTile, const StepArgs &args, float dt, unsigned long long *eventCounter)
 {
-    extern __shared__ float shTile[];
-    const TileGroupDev &G = blocks[blockIdx.x];
     const gennmi_presynaptic_update_group_t &g = G.g;
     const uint32_t batch = blockIdx.y;
     const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
@@ -475,22 +499,28 @@ void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs ar
     GLOBAL_AS const uint32_t *spk = asGlobal(g.srcSpk) + (size_t)batch * g.numSrcNeurons;
     GLOBAL_AS const uint16_t *off = asGlobal(G.tileOff);
     GLOBAL_AS const uint32_t *ind = asGlobal(g.ind);
-    GLOBAL_AS float *weight = asGlobal(g.g);
     // trace-STDP rows: besides delivering the (old) weight, every event applies the presynaptic-spike rule to its own
-    // synapse (pygenn/genn_model.py:1456-1463); a synapse belongs to exactly one tile, so g needs no atomic here either
+    // synapse (pygenn/genn_model.py:1456-1463); a synapse belongs to exactly one tile, so g needs no atomic here either.
+    // Plastic weights, spike times and traces are per batch.
     const bool additive = (g.wum == GENNMI_WUM_STDP);
     const bool stdp = (g.wum == GENNMI_WUM_STDP_TRACE) || additive;
+    GLOBAL_AS float *weight = asGlobal(g.g) + (stdp ? (size_t)batch * g.numSrcNeurons * g.rowStride : (size_t)0);
     const float t = stdp ? resolve(args, dt).t : 0.0f;
-    GLOBAL_AS const float *trgST = asGlobal(g.trgST);
-    GLOBAL_AS const float *postTrace = asGlobal(g.postTrace);
-    auto depress = [&](uint32_t idPost, float w) -> float {
+    GLOBAL_AS const float *trgST = asGlobal(g.trgST) + (size_t)batch * g.numTrgNeurons;
+    GLOBAL_AS const float *postTrace = asGlobal(g.postTrace) + (size_t)batch * g.numTrgNeurons;
+    GLOBAL_AS const uint32_t *trgBitmap = asGlobal(G.learn.trgBitmap) + (size_t)batch * ((g.numTrgNeurons + 31) / 32);
+    const bool paired = (G.learn.enabled != 0);
+    auto depress = [&](uint32_t idPre, uint32_t idPost, float w) -> float {
         const float stPost = dt + trgST[idPost];
         const float dtSpike = t - stPost;
+        float nw = w;
         if(dtSpike > 0) {
             const float factor = additive ? (float)exp((double)(-dtSpike / g.tauMinus)) : postTrace[idPost];
-            return fminf(g.wMax, fmaxf(g.wMin, w - (g.aMinus * factor)));
+            nw = fminf(g.wMax, fmaxf(g.wMin, w - (g.aMinus * factor)));
         }
-        return w;
+        // the target fired in the last update too: its postsynaptic-spike rule follows here (see LearnPostDev)
+        if(paired && bitmapTest(trgBitmap, idPost)) { bool changed = false; nw = learnPostOnSynapse(G.learn, g, batch, idPre, nw, t, dt, changed); }
+        return nw;
     };
     const uint32_t L = G.lanes;
     const uint32_t lis = threadIdx.x & (L - 1);
@@ -517,7 +547,7 @@ void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs ar
                 const f32x4u w = *reinterpret_cast<GLOBAL_AS const f32x4u*>(weight + rowBase + j);
                 if(stdp) {
                     f32x4u nw;
-                    nw.x = depress(ip.x, w.x); nw.y = depress(ip.y, w.y); nw.z = depress(ip.z, w.z); nw.w = depress(ip.w, w.w);
+                    nw.x = depress(idPre, ip.x, w.x); nw.y = depress(idPre, ip.y, w.y); nw.z = depress(idPre, ip.z, w.z); nw.w = depress(idPre, ip.w, w.w);
                     *reinterpret_cast<GLOBAL_AS f32x4u*>(weight + rowBase + j) = nw;
                 }
                 ldsAddF32x4(&shTile[ip.x - tileStart], w.x, true, &shTile[ip.y - tileStart], w.y, true,
@@ -527,7 +557,7 @@ void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs ar
                 for(uint32_t jj = j; jj < b; jj++) {
                     const uint32_t idPost = ind[rowBase + jj];
                     const float w = weight[rowBase + jj];
-                    if(stdp) { weight[rowBase + jj] = depress(idPost, w); }
+                    if(stdp) { weight[rowBase + jj] = depress(idPre, idPost, w); }
                     ldsAddF32(&shTile[idPost - tileStart], w);
                 }
             }
@@ -542,6 +572,13 @@ void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs ar
     }
     for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
     if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+__global__ __launch_bounds__(1024)
+void presynapticTileKernel(const TileGroupDev * __restrict__ blocks, StepArgs args, float dt, unsigned long long *eventCounter)
+{
+    extern __shared__ float shTile[];
+    presynapticTileBody(blocks[blockIdx.x], shTile, args, dt, eventCounter);
 }
 
 // Toeplitz Conv2D counterpart of the tile kernel: every block finds the run of spikes whose kernel footprint touches
@@ -705,7 +742,7 @@ void tileRecordBuildKernel(uint32_t numSrc, uint32_t rowStride, const uint32_t *
     }
 }
 
-__global__ __launch_bounds__(BLOCK)
+__global__ __launch_bounds__(1024)
 void presynapticUpdateKernel(const PreGroupDev * __restrict__ blocks, StepArgs args, float dt, unsigned long long *eventCounter)
 {
     presynapticBody(blocks[blockIdx.x], blockIdx.x, resolve(args, dt), dt, eventCounter);
@@ -715,45 +752,50 @@ void presynapticUpdateKernel(const PreGroupDev * __restrict__ blocks, StepArgs a
 // Postsynaptic update (learnPost): one sub-group per postsynaptic spike walks the column through
 // remap (coalesced), gathers g by synapse index.
 // ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(BLOCK)
-void postsynapticUpdateKernel(const PostGroupDev * __restrict__ blocks, StepArgs args, float dt)
+__device__ __forceinline__ void postsynapticBody(const PostGroupDev &G, uint32_t blockInKernel, uint32_t *shBits, const Resolved &st, float dt)
 {
-    const Resolved st = resolve(args, dt);
-    const PostGroupDev &G = blocks[blockIdx.x];
     const gennmi_postsynaptic_update_group_t &g = G.g;
+    const uint32_t batch = blockIdx.y;
+    const uint32_t BS = blockDim.x;
     const uint32_t W = G.lanesPerSpike;
-    const uint32_t localBlock = blockIdx.x - G.startBlock;
+    const uint32_t localBlock = blockInKernel - G.startBlock;
     const uint32_t lis = threadIdx.x & (W - 1);
-    const uint32_t subGroup = (localBlock * BLOCK + threadIdx.x) / W;
-    const uint32_t numSubGroups = (G.numBlocks * BLOCK) / W;
-    const uint32_t numSpikes = g.trgSpkCnt[0];
+    const uint32_t subGroup = (localBlock * BS + threadIdx.x) / W;
+    const uint32_t numSubGroups = (G.numBlocks * BS) / W;
+    // plastic weights, spike times and traces are per batch (VarAccess::READ_WRITE variables are duplicated); connectivity is shared
+    const uint32_t numSpikes = g.trgSpkCnt[batch];
+    GLOBAL_AS const uint32_t *trgSpk = asGlobal(g.trgSpk) + (size_t)batch * g.numTrgNeurons;
+    GLOBAL_AS float *weight = asGlobal(g.g) + (size_t)batch * g.numSrcNeurons * g.rowStride;
+    GLOBAL_AS const float *srcST = asGlobal(g.srcST) + (size_t)batch * g.numSrcNeurons;
+    GLOBAL_AS const float *preTrace = asGlobal(g.preTrace) + (size_t)batch * g.numSrcNeurons;
+    // rows of neurons that fired in the last update are left to the presynaptic pass, which applies this rule after its own
+    GLOBAL_AS const uint32_t *srcBitmap = asGlobal(G.srcBitmap) + (size_t)batch * ((g.numSrcNeurons + 31) / 32);
+    const bool paired = (G.srcBitmap != nullptr);
+    const bool additive = (g.tauPlus > 0.0f);          // built-in rule (weightUpdateModels.h:360-366): no trace array
     if(G.denseThreshold && numSpikes >= G.denseThreshold) {
         // A large share of the target population fired: nearly every row holds synapses to update, so walk the rows
         // once (coalesced ind / g) and test each synapse's target against the spike bitmap, instead of one scattered
         // read-modify-write per (spike, column entry).  Same arithmetic per synapse; every synapse is visited once.
-        extern __shared__ uint32_t shBits[];
         const uint32_t words = (g.numTrgNeurons + 31) / 32;
-        for(uint32_t k = threadIdx.x; k < words; k += BLOCK) { shBits[k] = asGlobal(G.spikeBitmap)[k]; }
+        for(uint32_t k = threadIdx.x; k < words; k += BS) { shBits[k] = asGlobal(G.spikeBitmap)[(size_t)batch * words + k]; }
         __syncthreads();
         const uint32_t lane = threadIdx.x & (WAVE - 1);
-        const uint32_t numWaves = G.numBlocks * (BLOCK / WAVE);
+        const uint32_t numWaves = G.numBlocks * (BS / WAVE);
         GLOBAL_AS const uint32_t *ind = asGlobal(g.ind);
-        GLOBAL_AS float *weight = asGlobal(g.g);
         // per-row scalars of the NEXT row are fetched while the current one is processed (indices clamped: readable)
         const uint32_t lastRow = g.numSrcNeurons - 1;
-        uint32_t row = localBlock * (BLOCK / WAVE) + threadIdx.x / WAVE;
+        uint32_t row = localBlock * (BS / WAVE) + threadIdx.x / WAVE;
         uint32_t lenNext = asGlobal(g.rowLength)[min(row, lastRow)];
-        const bool additive = (g.tauPlus > 0.0f);          // built-in rule (weightUpdateModels.h:360-366): no trace array
-        float stNext = asGlobal(g.srcST)[min(row, lastRow)], traceNext = additive ? 0.0f : asGlobal(g.preTrace)[min(row, lastRow)];
+        float stNext = srcST[min(row, lastRow)], traceNext = additive ? 0.0f : preTrace[min(row, lastRow)];
         for(; row < g.numSrcNeurons; row += numWaves) {
             const uint32_t len = lenNext;
             const float stPre = dt + stNext;
             const float trace = traceNext;
             const uint32_t nextRow = min(row + numWaves, lastRow);
-            lenNext = asGlobal(g.rowLength)[nextRow]; stNext = asGlobal(g.srcST)[nextRow];
-            if(!additive) { traceNext = asGlobal(g.preTrace)[nextRow]; }
+            lenNext = asGlobal(g.rowLength)[nextRow]; stNext = srcST[nextRow];
+            if(!additive) { traceNext = preTrace[nextRow]; }
             const float dtSpike = st.t - stPre;
-            if(!(dtSpike > 0) || len == 0) { continue; }
+            if(!(dtSpike > 0) || len == 0 || (paired && bitmapTest(srcBitmap, row))) { continue; }
             const float step = g.aPlus * (additive ? (float)exp((double)(-dtSpike / g.tauPlus)) : trace);
             const size_t rowBase = (size_t)row * g.rowStride;
             // up to four strides of the row in flight per lane
@@ -776,20 +818,49 @@ void postsynapticUpdateKernel(const PostGroupDev * __restrict__ blocks, StepArgs
         return;
     }
     for(uint32_t s = subGroup; s < numSpikes; s += numSubGroups) {
-        const uint32_t spike = g.trgSpk[s];
+        const uint32_t spike = trgSpk[s];
         const uint32_t npre = g.colLength[spike];
         const size_t colBase = (size_t)spike * g.colStride;
         for(uint32_t i = lis; i < npre; i += W) {
             const uint32_t rowMajorIndex = g.remap[colBase + i];
             const uint32_t idPre = rowMajorIndex / g.rowStride;
-            const float stPre = dt + g.srcST[idPre];
+            if(paired && bitmapTest(srcBitmap, idPre)) { continue; }
+            const float stPre = dt + srcST[idPre];
             const float dtSpike = st.t - stPre;
             if(dtSpike > 0) {
-                const float factor = (g.tauPlus > 0.0f) ? (float)exp((double)(-dtSpike / g.tauPlus)) : g.preTrace[idPre];
-                const float newWeight = g.g[rowMajorIndex] + (g.aPlus * factor);
-                g.g[rowMajorIndex] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
+                const float factor = additive ? (float)exp((double)(-dtSpike / g.tauPlus)) : preTrace[idPre];
+                const float newWeight = weight[rowMajorIndex] + (g.aPlus * factor);
+                weight[rowMajorIndex] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
             }
         }
+    }
+}
+
+__global__ __launch_bounds__(1024)
+void postsynapticUpdateKernel(const PostGroupDev * __restrict__ blocks, StepArgs args, float dt)
+{
+    extern __shared__ uint32_t shBits[];
+    postsynapticBody(blocks[blockIdx.x], blockIdx.x, shBits, resolve(args, dt), dt);
+}
+
+// All synaptic work of a step that can share a launch: the scatter path of every projection, the tile path of those that
+// have one (a projection's step is taken by one or the other, decided on the device from its spike count) and the
+// postsynaptic passes whose projections are paired with their presynaptic halves (LearnPostDev: no synapse is written by
+// both, so nothing orders the passes).  Block ranges [0, preBlocks), [preBlocks, preBlocks + tileBlocks), then the rest.
+__global__ __launch_bounds__(1024)
+void synapseCombinedKernel(const PreGroupDev * __restrict__ pre, uint32_t preBlocks, const TileGroupDev * __restrict__ tiles, uint32_t tileBlocks,
+                           const PostGroupDev * __restrict__ post, StepArgs args, float dt, unsigned long long *eventCounter)
+{
+    extern __shared__ float shDynamic[];
+    if(blockIdx.x < preBlocks) {
+        presynapticBody(pre[blockIdx.x], blockIdx.x, resolve(args, dt), dt, eventCounter);
+    }
+    else if(blockIdx.x < preBlocks + tileBlocks) {
+        presynapticTileBody(tiles[blockIdx.x - preBlocks], shDynamic, args, dt, eventCounter);
+    }
+    else {
+        const uint32_t b = blockIdx.x - preBlocks - tileBlocks;
+        postsynapticBody(post[b], b, reinterpret_cast<uint32_t*>(shDynamic), resolve(args, dt), dt);
     }
 }
 

@@ -601,14 +601,19 @@ class GeNNModel:
                     # the sparse kernels read a weight per synapse: the one weight is written out
                     s.vars["g"] = self._alloc(n_pre * s.row_stride, np.float32, fill=np.float32(lit32(s.wu.params["g"])))
                 names = [] if s.wu.snippet == "StaticPulseConstantWeight" else ["g"] + (["d"] if s.wu.snippet == "StaticPulseDendriticDelay" else [])
+                # weights a learning rule writes are READ_WRITE variables: one copy per batch (models.h VarAccess::READ_WRITE has
+                # the batch dimension), every copy starting from the same initial values
+                copies = B if s.wu.snippet in ("STDPTrace", "STDP") else 1
                 for name in names:
                     dtype = np.uint8 if name == "d" else np.float32
                     if name not in s.var_host and isinstance(s.wu.vars[name], VarInit):
+                        if copies != 1:
+                            raise NotImplementedError(f"{s.name}: device-side initialisation of plastic weights with batch size > 1")
                         s.vars[name] = self._alloc_device_init(n_pre * s.row_stride, dtype, s.wu.vars[name])
                         continue
-                    a = self._alloc(n_pre * s.row_stride, dtype)
+                    a = self._alloc(copies * n_pre * s.row_stride, dtype)
                     if name in s.var_host:
-                        a.view[:] = np.asarray(s.var_host[name], dtype=dtype).reshape(-1)
+                        a.view[:] = np.tile(np.asarray(s.var_host[name], dtype=dtype).reshape(-1), copies)
                     else:
                         a.view[:] = dtype(s.wu.vars[name])
                     a.push_to_device()
@@ -1004,7 +1009,8 @@ class GeNNModel:
     def runner_info(self):
         info = (C.c_uint32 * 4)()
         _abi.check(_abi.load().gennmi_runner_get_info(self._runner, C.byref(info)))
-        return {"single_launch_step": bool(info[0] & 1), "resident_plan": bool(info[0] & 2), "bulk_neuron_kernel": bool(info[0] & 4), "ordered_accumulation": bool(info[0] & 8), "neuron_blocks": info[1], "presyn_blocks": info[2], "postsyn_blocks": info[3]}
+        return {"single_launch_step": bool(info[0] & 1), "resident_plan": bool(info[0] & 2), "bulk_neuron_kernel": bool(info[0] & 4), "ordered_accumulation": bool(info[0] & 8),
+                "combined_synapse_launch": bool(info[0] & 16), "postsynaptic_in_combined_launch": bool(info[0] & 32), "neuron_blocks": info[1], "presyn_blocks": info[2], "postsyn_blocks": info[3]}
 
     # timing counters under PyGeNN's names (pygenn/genn_model.py:292-326), in seconds, accumulated while `timing_enabled`
     def _times(self):

@@ -395,7 +395,11 @@ int gennmi_runner_stream_elapsed(gennmi_runner *runner, double *seconds);
  * earlier, into the slot read in the next step — the visible difference is the content of that one ring slot
  * between steps; GENNMI_FUSED_STEP=0 in the environment keeps the reference's placement); bit 2 if the neuron update
  * takes several neurons per lane (networks that need more than one round of resident work-groups and use only plain groups;
- * GENNMI_NEURON_BULK=0 forbids it, 2 / 4 / 8 force that many), info[1..3] = blocks of
+ * GENNMI_NEURON_BULK=0 forbids it, 2 / 4 / 8 force that many); bit 3: ordered accumulation; bit 4 if the scatter path, the
+ * tile path and (bit 5) the postsynaptic passes of a step share one launch (projections with a tile path, or plastic ones
+ * whose postsynaptic pass is paired with the presynaptic one: a synapse both of whose ends fired gets both rules from the
+ * thread of the presynaptic pass, in the reference's order, and the postsynaptic pass leaves that row alone;
+ * GENNMI_COMBINED=0 keeps a launch per kernel, GENNMI_PAIRED_LEARN=0 the reference's two passes); info[1..3] = blocks of
  * the neuron, presynaptic and postsynaptic kernels.  The reference logs the analogous choice of presynaptic
  * strategy (backendSIMT.cc:736). */
 int gennmi_runner_get_info(gennmi_runner *runner, uint32_t info[4]);

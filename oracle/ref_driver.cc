@@ -482,7 +482,11 @@ int main(int argc, char *argv[])
             const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
             const auto rows = readFile<T>(in + "/" + file, numPre * s.rowStride);
             auto *dst = a->getHostPointer<T>();
-            for(size_t i = 0; i < numPre; i++) { std::copy_n(rows.begin() + i * s.rowStride, s.rowStride, dst + i * stride); }
+            // (variables a learning rule writes have one copy per batch: every copy starts from the file's values)
+            const size_t copies = a->getCount() / (numPre * stride);
+            for(size_t c = 0; c < copies; c++) {
+                for(size_t i = 0; i < numPre; i++) { std::copy_n(rows.begin() + i * s.rowStride, s.rowStride, dst + (c * numPre + i) * stride); }
+            }
         };
         for(auto &s : syns) {
             if(s.matrix == "sparse") {
@@ -548,7 +552,7 @@ int main(int argc, char *argv[])
                 if(s.wum == "stdp_trace" || s.wum == "stdp") {
                     auto *a = pulled(rt.getArray(*s.sg, "g"));
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
-                    for(size_t i = 0; i < numPre; i++) { appendFile(out + "/" + s.name + ".g.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
+                    for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + ".g.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
                 }
                 if(s.wum == "timing_copy") {
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);

@@ -226,6 +226,63 @@ def test_adapter_batched_toeplitz_layer():
         shutil.rmtree(tmp, ignore_errors=True)
 
 
+def test_adapter_batched_plastic_network():
+    """Batch size 2 with trace STDP through the adapter: the Runtime duplicates the weights (VarAccess::READ_WRITE), the traces
+    and the spike times per batch; the batches differ in initial membrane potentials and Poisson spike trains, and batch b
+    must equal a batch-1 oracle run on batch b's inputs, final weights included."""
+    import copy
+    from genn_amd import configs, rng
+    from genn_amd.configs import poisson_spike_source
+    from oracle.genn_cpu import OracleNet
+    B, steps = 2, 100
+    nets = []
+    for b in range(B):
+        net = configs.plastic_stdp(n=1500, n_src=100, steps=steps, fan=80, src_fan=60)
+        if b:
+            for k, name in enumerate(("E", "I")):
+                p = net.pop(name)
+                p.vars["V"] = (-60.0 + 10.0 * rng.uniform(4321 + b, 1 + k, 0, p.n)).astype(np.float32)
+            start, end, times = poisson_spike_source(net.seed, 70 + b, 100, 10.0, steps, net.dt)
+            net.pop("P").vars = {"startSpike": start, "endSpike": end}
+            net.pop("P").spike_times = times
+        nets.append(net)
+    batched = copy.deepcopy(nets[0])
+    for name in ("E", "I"):
+        batched.pop(name).vars = {"V": np.stack([n.pop(name).vars["V"] for n in nets]), "RefracTime": np.zeros((B, nets[0].pop(name).n), np.float32)}
+    offs = np.cumsum([0] + [len(n.pop("P").spike_times) for n in nets])
+    batched.pop("P").vars = {"startSpike": np.stack([n.pop("P").vars["startSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32),
+                             "endSpike": np.stack([n.pop("P").vars["endSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32)}
+    batched.pop("P").spike_times = np.concatenate([n.pop("P").spike_times for n in nets])
+    batched.batch_size = B
+    batched.snap = 0
+    tmp = tempfile.mkdtemp(prefix="adapter_batch_stdp_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(batched, spec)
+        print(f"adapter batched plastic network: running {DRIVER}", flush=True)
+        res = subprocess.run([DRIVER, spec, work, out], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+        assert res.returncode == 0, res.stdout[-3000:]
+        total = 0
+        g = np.fromfile(os.path.join(out, "EE.g.f32"), np.float32).reshape(B, -1)
+        for b, net in enumerate(nets):
+            oracle = OracleNet(net, num_recording_timesteps=net.steps)
+            oracle.run(net.steps)
+            for p in net.pops:
+                got = np.fromfile(os.path.join(out, f"{p.name}.spikes{'.b%d' % b if b else ''}.u32"), np.uint32).reshape(-1, 2)
+                words = (p.n + 31) // 32
+                bits = np.unpackbits(oracle.record(p.name, net.steps).view(np.uint8).reshape(net.steps, words * 4), axis=1, bitorder="little")[:, :p.n]
+                steps_, ids = np.nonzero(bits)
+                assert np.array_equal(got, np.stack([steps_, ids], axis=1).astype(np.uint32)), f"batch {b}: raster of {p.name} differs"
+                total += len(ids)
+            assert np.array_equal(g[b], oracle.syn_g("EE").reshape(-1)), f"batch {b}: weights differ"
+            oracle.close()
+        assert total > 1000 and not np.array_equal(g[0], g[1])
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
 def _procedural_pair(net, steps, snap):
     """Runs `net` through GeNN's generator and Runtime on the adapter and through the Python host layer with the adapter's
     stream numbering; returns (driver output directory, temporary directory, host-layer model after `steps` steps,

@@ -222,6 +222,62 @@ def test_toeplitz_batches_are_independent():
     model.unload()
 
 
+@pytest.mark.parametrize("rule, combined", [("stdp_trace", "1"), ("stdp_additive", "1"), ("stdp_trace", "0")])
+def test_plastic_batches_are_independent(rule, combined, monkeypatch):
+    """Batch b of a batched plastic network equals a batch-1 run of the oracle on batch b's inputs: weights a learning rule
+    writes, traces and spike times are per batch (models.h: VarAccess::READ_WRITE has the batch dimension), connectivity is
+    shared.  The batches differ in their initial membrane potentials and in their Poisson spike trains.  Run with the
+    scatter / tile / learnPost passes sharing one launch and with a launch each."""
+    monkeypatch.setenv("GENNMI_COMBINED", combined)
+    import copy
+    from genn_amd import rng
+    from genn_amd.configs import poisson_spike_source
+    B, steps = 3, 120
+    nets = []
+    for b in range(B):
+        net = configs.plastic_stdp(n=1500, n_src=100, steps=steps, fan=80, src_fan=60, rule=rule)
+        if b:
+            for k, name in enumerate(("E", "I")):
+                p = net.pop(name)
+                p.vars["V"] = (-60.0 + 10.0 * rng.uniform(1234 + b, 1 + k, 0, p.n)).astype(np.float32)
+            start, end, times = poisson_spike_source(net.seed, 50 + b, 100, 10.0, steps, net.dt)
+            src = net.pop("P")
+            src.vars = {"startSpike": start, "endSpike": end}
+            src.spike_times = times
+        nets.append(net)
+    batched = copy.deepcopy(nets[0])
+    for name in ("E", "I"):
+        batched.pop(name).vars = {"V": np.stack([n.pop(name).vars["V"] for n in nets]), "RefracTime": np.zeros((B, nets[0].pop(name).n), np.float32)}
+    offs = np.cumsum([0] + [len(n.pop("P").spike_times) for n in nets])
+    batched.pop("P").vars = {"startSpike": np.stack([n.pop("P").vars["startSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32),
+                             "endSpike": np.stack([n.pop("P").vars["endSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32)}
+    batched.pop("P").spike_times = np.concatenate([n.pop("P").spike_times for n in nets])
+    model = model_from_net(batched, batch_size=B)
+    model.load(num_recording_timesteps=steps)
+    info = model.runner_info()
+    assert info["combined_synapse_launch"] == (combined == "1") and info["postsynaptic_in_combined_launch"] == (combined == "1")
+    oracles = [OracleNet(n) for n in nets]
+    total = 0
+    for step in range(steps):
+        model.step_time()
+        got = {p.name: model.neuron_populations[p.name].current_spikes for p in batched.pops}
+        for b, o in enumerate(oracles):
+            o.step()
+            for p in batched.pops:
+                assert np.array_equal(got[p.name][b], o.spikes(p.name)), f"step {step} batch {b}: {p.name} spikes differ"
+                total += len(o.spikes(p.name))
+    assert total > 1500
+    g = model.synapse_populations["EE"].vars["g"].pull_from_device().reshape(B, -1)
+    v = model.neuron_populations["E"].vars["V"].pull_from_device().reshape(B, -1)
+    for b, o in enumerate(oracles):
+        # every weight has one writer per step and the rules are evaluated as the oracle evaluates them: identical
+        assert np.array_equal(g[b], o.syn_g("EE").reshape(-1)), f"batch {b}: weights differ"
+        np.testing.assert_allclose(v[b], o.var("E", 0), rtol=1e-5, atol=1e-5)
+        assert np.count_nonzero(g[b] != nets[b].syn("EE").g.reshape(-1)) > 500
+    assert not np.array_equal(g[0], g[1])
+    model.unload()
+
+
 @pytest.mark.parametrize("span", ["POSTSYNAPTIC", "PRESYNAPTIC"])
 def test_axonal_delays(span):
     """Balanced LIF network with axonal delays of 3, 1, 0 and 5 timesteps: the spike queue of a population is a ring of
