@@ -66,6 +66,8 @@ struct gennmi_runner
     // one launch for the scatter path, the tile path and the paired postsynaptic passes of a step (synapseCombinedKernel)
     bool combineSynapses = false, combinePost = false; uint32_t synapseThreads = BLOCK; size_t combinedLdsBytes = 0;
     ConvTileDev *dConvTile = nullptr; uint32_t convTileBlocks = 0; size_t convTileBytes = 0;
+    ConvMfmaDev *dConvMfma = nullptr; uint32_t convMfmaBlocks = 0; size_t convMfmaBytes = 0;      // Conv2D on the matrix cores (instead of dConvTile)
+    bool bitmapsStale = false;          // a spike queue was written by the caller: the bitmaps kept beside the queues are rebuilt before the next step
     std::vector<void*> owned;           // engine-private device allocations (shadow queues, zero-delay lists)
     // resident plan (many steps per launch)
     bool resident = false;
@@ -121,6 +123,11 @@ static void noteDeviceWrite(const void *dev, size_t bytes)
     const uintptr_t a = reinterpret_cast<uintptr_t>(dev), b = a + bytes;
     for(gennmi_runner *r : g_runners) {
         for(const auto &n : r->neuron) {
+            if(n.spikeBitmap && !r->bitmapsStale) {
+                const uintptr_t q = reinterpret_cast<uintptr_t>(n.g.spk), c = reinterpret_cast<uintptr_t>(n.g.spkCnt);
+                const size_t slots = std::max(1u, n.g.numDelaySlots);
+                if((a < q + (size_t)r->batch * slots * n.g.numNeurons * sizeof(uint32_t) && q < b) || (a < c + (size_t)r->batch * slots * sizeof(uint32_t) && c < b)) { r->bitmapsStale = true; }
+            }
             if(n.g.model != GENNMI_NEURON_SPIKE_SOURCE_ARRAY || r->sourcesStale) { continue; }
             const size_t perNeuron = (size_t)r->batch * n.g.numNeurons * sizeof(uint32_t);
             const uintptr_t st = reinterpret_cast<uintptr_t>(n.g.startSpike), en = reinterpret_cast<uintptr_t>(n.g.endSpike);
@@ -1114,6 +1121,54 @@ int gennmi_runner_finalise(gennmi_runner *r)
                && p.g.conv[0] < 1024 && p.g.conv[1] < 1024 && p.g.conv[7] < 1024
                && p.g.conv[2] < 1024 && p.g.conv[3] < 1024 && p.g.conv[4] < 1024) {        // rows, columns and channels are packed 10 bits each
                 const int32_t *c = p.g.conv;
+                // the matrix cores take the layer when its source's neuron update can keep a spike bitmap and a block's patch
+                // and the kernel fit in LDS (GENNMI_CONV_MFMA=0: the event-driven tile kernel below)
+                {
+                    const char *envMfma = getenv("GENNMI_CONV_MFMA");
+                    NeuronGroupDev *src = nullptr;
+                    for(auto &n : r->neuron) { if(n.g.spk == p.g.srcSpk && n.g.numNeurons == p.g.numSrcNeurons) { src = &n; } }
+                    if(!(envMfma && atoi(envMfma) == 0) && src) {
+                        ConvMfmaDev m{};
+                        m.g = p.g; m.convBH = p.convBH; m.convBW = p.convBW;
+                        const uint32_t K = (uint32_t)(c[0] * c[1] * c[4]);
+                        m.kernPitch = ((uint32_t)c[7] + 31) / 32 * 32;
+                        if(m.kernPitch % 64 == 0) { m.kernPitch += 32; }         // the two halves of a wavefront read consecutive rows
+                        m.patchPitch = ((uint32_t)c[6] + 31) / 32 * 32 + (uint32_t)c[1] - 1;
+                        const size_t kernFloats = (size_t)2 * (((K + 1) / 2 + CONV_MFMA_STEPS - 1) / CONV_MFMA_STEPS) * CONV_MFMA_STEPS * m.kernPitch;       // whole chunks of steps
+                        // as many output rows per block as give every compute unit one block, fewer if LDS says so
+                        uint32_t rowsPerBlock = std::max(1u, std::min<uint32_t>((uint32_t)c[5], ((uint32_t)c[5] * r->batch) / numCU));
+                        size_t bytes = 0;
+                        for(;; rowsPerBlock--) {
+                            m.patchRows = rowsPerBlock + (uint32_t)c[0] - 1;
+                            m.planePitch = (m.patchRows * m.patchPitch + 63) / 64 * 64 + 32;
+                            bytes = ((size_t)c[4] * m.planePitch + kernFloats) * sizeof(float);
+                            if(bytes <= 64 * 1024 || rowsPerBlock == 1) { break; }
+                        }
+                        if(bytes <= 64 * 1024) {
+                            if(!src->spikeBitmap) {
+                                const size_t bitmapBytes = (size_t)r->batch * ((src->g.numNeurons + 31) / 32) * sizeof(uint32_t);
+                                HIP_TRY(hipMalloc((void**)&src->spikeBitmap, bitmapBytes));
+                                r->owned.push_back(src->spikeBitmap);
+                                HIP_TRY(hipMemset(src->spikeBitmap, 0, bitmapBytes));
+                                r->bitmapsStale = true;          // the queue may already hold spikes
+                            }
+                            m.srcBitmap = src->spikeBitmap;
+                            m.rowsPerBlock = rowsPerBlock;
+                            m.numBatches = r->batch;
+                            p.tileThreshold = std::max(1u, p.g.numTrgNeurons / 4);
+                            m.threshold = p.tileThreshold;
+                            HIP_TRY(hipMalloc(&r->dConvMfma, sizeof(ConvMfmaDev)));
+                            HIP_TRY(hipMemcpy(r->dConvMfma, &m, sizeof(ConvMfmaDev), hipMemcpyHostToDevice));
+                            r->owned.push_back(r->dConvMfma);
+                            r->convMfmaBlocks = ((uint32_t)c[5] + rowsPerBlock - 1) / rowsPerBlock;
+                            r->convMfmaBytes = bytes;
+                            if(bytes > 48 * 1024) {
+                                HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(presynapticConvMfmaKernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+                            }
+                            continue;
+                        }
+                    }
+                }
                 const size_t rowFloats = (size_t)c[6] * c[7];
                 const size_t fixedFloats = (size_t)c[0] * c[1] * c[4] * c[7] + CONV_TILE_SPIKES;      // kernel weights + staged spikes
                 const size_t budgetFloats = 60 * 1024 / sizeof(float);
@@ -1409,11 +1464,23 @@ static int stamp(gennmi_runner *r, hipEvent_t *out)
 // spike sources: bring the per-neuron copies of the next spike time up to date with arrays written since they were built
 static int refreshSpikeSources(gennmi_runner *r)
 {
-    bool stale;
+    bool stale, bitmaps;
     {
         std::lock_guard<std::mutex> lock(g_runnersMutex);
         stale = r->sourcesStale;
         r->sourcesStale = false;
+        bitmaps = r->bitmapsStale;
+        r->bitmapsStale = false;
+    }
+    if(bitmaps) {
+        // a spike queue was written from outside (or held spikes before its bitmap existed): the bitmap follows the queue
+        for(const auto &n : r->neuron) {
+            if(!n.spikeBitmap || n.g.numDelaySlots > 1) { continue; }
+            const uint32_t words = (n.g.numNeurons + 31) / 32;
+            spikeBitmapFromQueueKernel<<<dim3((words + BLOCK - 1) / BLOCK, r->batch), dim3(BLOCK), 0, r->stream>>>(n.g.spkCnt, n.g.spk, n.spikeBitmap, n.g.numNeurons, 1u);
+            spikeBitmapFromQueueKernel<<<dim3((n.g.numNeurons + BLOCK - 1) / BLOCK, r->batch), dim3(BLOCK), 0, r->stream>>>(n.g.spkCnt, n.g.spk, n.spikeBitmap, n.g.numNeurons, 0u);
+            HIP_TRY(hipGetLastError());
+        }
     }
     if(!stale) { return GENNMI_OK; }
     for(const auto &n : r->neuron) {
@@ -1456,7 +1523,7 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
             synapseCombinedKernel<<<dim3(scatterBlocks + r->tileBlocks + postBlocks, r->batch), dim3(r->synapseThreads), r->combinedLdsBytes, r->stream>>>(
                 r->dPre, scatterBlocks, r->dTile, r->tileBlocks, r->dPost, a, r->dt, r->dEvents);
         }
-        else if(r->preBlocks && r->scatterNeeded) {
+        else if(r->preBlocks && r->scatterNeeded && !(r->convMfmaBlocks && !timed)) {
             presynapticUpdateKernel<<<dim3(r->preBlocks, r->batch), dim3(r->synapseThreads), 0, r->stream>>>(r->dPre, a, r->dt, r->dEvents);
         }
         if(r->denseBlocks) {
@@ -1464,6 +1531,12 @@ static int launchSynapses(gennmi_runner *r, const StepArgs &a, bool timed)
         }
         if(r->tileBlocks && !combined) {
             presynapticTileKernel<<<dim3(r->tileBlocks, r->batch), dim3(r->tileThreads), r->tileFloats * sizeof(float), r->stream>>>(r->dTile, a, r->dt, r->dEvents);
+        }
+        if(r->convMfmaBlocks) {
+            // (the scatter blocks of the projection ride along unless the run is timed)
+            const uint32_t scatterBlocks = (r->preBlocks && r->scatterNeeded && !timed) ? r->preBlocks : 0u;
+            presynapticConvMfmaKernel<<<dim3((r->convMfmaBlocks + scatterBlocks) * r->batch), dim3(CONV_MFMA_THREADS), r->convMfmaBytes, r->stream>>>(
+                r->dConvMfma, r->convMfmaBlocks * r->batch, r->dPre, a, r->dt, r->dEvents);
         }
         if(r->convTileBlocks) {
             presynapticConvTileKernel<<<dim3(r->convTileBlocks, r->batch), dim3(CONV_TILE_THREADS), r->convTileBytes, r->stream>>>(r->dConvTile, r->dEvents);
@@ -1746,7 +1819,7 @@ int gennmi_runner_get_info(gennmi_runner *r, uint32_t info[4])
     if(!r || !info) { return fail(GENNMI_EINVAL, "runner_get_info: null argument"); }
     if(!r->finalised) { return fail(GENNMI_ESTATE, "runner_get_info: runner not finalised"); }
     info[0] = (r->fusedStep ? 1u : 0u) | (r->resident ? 2u : 0u) | (r->neuronsPerLane > 1 ? 4u : 0u) | (r->ordered ? 8u : 0u)
-              | (r->combineSynapses ? 16u : 0u) | ((r->combineSynapses && r->combinePost) ? 32u : 0u); info[1] = r->neuronBlocks; info[2] = r->preBlocks; info[3] = r->postBlocks;
+              | (r->combineSynapses ? 16u : 0u) | ((r->combineSynapses && r->combinePost) ? 32u : 0u) | (r->convMfmaBlocks ? 64u : 0u); info[1] = r->neuronBlocks; info[2] = r->preBlocks; info[3] = r->postBlocks;
     return GENNMI_OK;
 }
 

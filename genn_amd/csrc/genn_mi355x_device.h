@@ -171,6 +171,23 @@ struct ConvTileDev
     uint32_t threshold, pad_;
 };
 
+// Dense path of a Toeplitz Conv2D projection on the matrix cores: at the activity that sends a step to a tile kernel, the
+// layer is a small GEMM per batch — output pixels x (kh*kw*ic) x output channels — whose left operand is the source
+// population's spike bitmap expanded to 0 / 1.
+struct ConvMfmaDev
+{
+    gennmi_presynaptic_update_group_t g;
+    const uint32_t *srcBitmap;          // [batch][ceil(numSrc/32)] the source population's spikes of the last neuron update
+    int32_t convBH, convBW;
+    uint32_t rowsPerBlock;              // output rows of a block
+    uint32_t patchRows, patchPitch;     // the input patch of a block in LDS: [ic][patchRows][patchPitch] floats
+    uint32_t planePitch;                // patchRows * patchPitch, padded
+    uint32_t kernPitch;                 // the kernel in LDS: [kh*kw*ic, rounded up to whole chunks of steps][kernPitch] floats
+    uint32_t threshold;
+    uint32_t numBatches;                // the grid is one-dimensional: block = rowGroup * numBatches + batch
+    uint32_t pad_;
+};
+
 struct PostGroupDev
 {
     gennmi_postsynaptic_update_group_t g;
@@ -194,6 +211,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint8_t u8x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4u __attribute__((ext_vector_type(4), aligned(4)));     // dword-aligned only: segments start anywhere in a row
 typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
 

@@ -556,6 +556,7 @@ __device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t
             const uint32_t words = (n + 31) / 32;
             g.recordSpk[((size_t)st.recT * gridDim.y + batch) * words + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
         }
+        if(G.spikeBitmap && (lane & 31) == 0 && i < n) { G.spikeBitmap[(size_t)batch * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballot >> (lane & 32)); }
     }
     if(lane == 0) { shWaveCount[wave] = waveCount; }
     __syncthreads();
@@ -600,7 +601,7 @@ void stepFusedKernel(const NeuronGroupDev * __restrict__ neuronBlocks, uint32_t 
         __builtin_amdgcn_s_setprio(3);
         neuronBody(neuronBlocks[blockIdx.x], blockIdx.x, numNeuronBlocks, st, dt, agg, errorFlag);
     }
-    else { presynapticBody(preBlocks[blockIdx.x - numNeuronBlocks], blockIdx.x - numNeuronBlocks, st, dt, eventCounter); }
+    else { presynapticBody(preBlocks[blockIdx.x - numNeuronBlocks], blockIdx.x - numNeuronBlocks, blockIdx.y, gridDim.y, st, dt, eventCounter); }
 }
 
 // Per row: count the synapses with d % D == 0 and, when `entries` is given, append them at offset[row].

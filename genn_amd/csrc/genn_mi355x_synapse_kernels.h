@@ -32,12 +32,11 @@ __device__ __forceinline__ bool bitmapTest(GLOBAL_AS const uint32_t *bitmap, uin
 // round-robin to the sub-groups of the synapse group's blocks, so the launch geometry is fixed
 // while the spike count lives on the device.
 // ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t blockInKernel, const Resolved &st, float dt,
-                                                unsigned long long *eventCounter)
+__device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t blockInKernel, uint32_t batch, uint32_t numBatches,
+                                                const Resolved &st, float dt, unsigned long long *eventCounter)
 {
     const gennmi_presynaptic_update_group_t &g = G.g;
     if(G.ordered) { return; }
-    const uint32_t batch = blockIdx.y;
     const uint32_t W = G.lanesPerSpike;
     const uint32_t localBlock = blockInKernel - G.startBlock;
     const uint32_t lis = threadIdx.x & (W - 1);
@@ -50,9 +49,9 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
     // updates ago, (spkQuePtr + slots - delay) % slots with spkQuePtr = epoch % slots (backendBase.cc:207-216)
     const uint32_t slots = max(1u, g.numSrcDelaySlots);
     const uint32_t readSlot = (slots > 1) ? modStep(st.epoch + slots - g.axonalDelaySteps, slots) : 0u;
-    GLOBAL_AS const uint32_t *cntPtr = G.shadowSpk ? asGlobal(G.shadowCnt) + (size_t)parity * gridDim.y + batch
+    GLOBAL_AS const uint32_t *cntPtr = G.shadowSpk ? asGlobal(G.shadowCnt) + (size_t)parity * numBatches + batch
                                                    : asGlobal(g.srcSpkCnt) + ((size_t)batch * slots + readSlot);
-    GLOBAL_AS const uint32_t *spk = G.shadowSpk ? asGlobal(G.shadowSpk) + ((size_t)parity * gridDim.y + batch) * g.numSrcNeurons
+    GLOBAL_AS const uint32_t *spk = G.shadowSpk ? asGlobal(G.shadowSpk) + ((size_t)parity * numBatches + batch) * g.numSrcNeurons
                                                 : asGlobal(g.srcSpk) + ((size_t)batch * slots + readSlot) * g.numSrcNeurons;
     // the first spike id this sub-group would handle is fetched together with the count, not after it (the
     // queue always holds numSrcNeurons entries, so any index below that is readable)
@@ -742,10 +741,207 @@ void tileRecordBuildKernel(uint32_t numSrc, uint32_t rowStride, const uint32_t *
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Toeplitz Conv2D on the matrix cores (fp32 MFMA: products of a 0 / 1 spike indicator and an fp32 weight are exact, the
+// sums are fp32 like every other path's; only their order differs from the CPU backend's queue order).
+//
+//   outPost[y][x][o] += sum over (a, b, ch) of S[y + a - PH][x + b - PW][ch] * kernel[a][b][ch][o],
+//   PH = kh - 1 - convBH, PW = kw - 1 - convBW
+// is the gather form of initToeplitzConnectivitySnippet.h:116-137 (a, b are the kernel taps counted from the far corner).
+// A block owns `rowsPerBlock` output rows of one batch.  It expands the bits of the input rows those reach into a planar
+// patch in LDS ([channel][row][column], so that the 32 pixels of an MFMA tile read consecutive words), copies the kernel
+// next to it, and every wavefront then computes tiles of 32 pixels x 32 output channels with v_mfma_f32_32x32x2_f32, two
+// steps of the (tap, channel) sum per instruction, and adds its tile to outPost (the block owns these rows).
+// ------------------------------------------------------------------------------------------------
+constexpr int CONV_MFMA_THREADS = 512;       // eight wavefronts: a compute unit then holds one block, whose wavefronts start together
+constexpr int CONV_MFMA_STEPS = 72;         // steps of the (tap, channel) sum per unrolled chunk of the inner loop
+constexpr int CONV_MFMA_AHEAD = 6;          // steps whose operands are fetched ahead of the matrix instructions (divides the above)
+
+__global__ __launch_bounds__(CONV_MFMA_THREADS)
+void presynapticConvMfmaKernel(const ConvMfmaDev * __restrict__ blocks, uint32_t mfmaBlocks, const PreGroupDev * __restrict__ scatter,
+                               StepArgs args, float dt, unsigned long long *eventCounter)
+{
+    extern __shared__ float shConvM[];
+    const ConvMfmaDev &G = blocks[0];
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    // Blocks are numbered batch-first (block = index * numBatches + batch), so that consecutive work-groups, which go to
+    // consecutive XCDs, differ in batch.  Behind the blocks of the dense path come those of the scatter path, which takes
+    // the steps too quiet for it: one launch, and the device decides which of the two does the work.
+    const uint32_t numBatches = G.numBatches;
+    const uint32_t batch = blockIdx.x % numBatches;
+    if(blockIdx.x >= mfmaBlocks) {
+        const uint32_t b = (blockIdx.x - mfmaBlocks) / numBatches;
+        presynapticBody(scatter[b], b, batch, numBatches, resolve(args, dt), dt, eventCounter);
+        return;
+    }
+    const uint32_t rowGroup = blockIdx.x / numBatches;
+    const int kh = g.conv[0], kw = g.conv[1], ih = g.conv[2], iw = g.conv[3], ic = g.conv[4];
+    const int oh = g.conv[5], ow = g.conv[6], oc = g.conv[7];
+    const uint32_t numDiag = (uint32_t)(kh * kw * oc);
+    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
+    if((unsigned long long)numSpikes * numDiag < G.threshold) { return; }      // the scatter kernel took this step
+    const uint32_t planePitch = G.planePitch, patchPitch = G.patchPitch, kernPitch = G.kernPitch;
+    const int y0 = (int)(rowGroup * G.rowsPerBlock);
+    const int rows = min((int)G.rowsPerBlock, oh - y0);
+    const int PH = kh - 1 - G.convBH, PW = kw - 1 - G.convBW;
+    const uint32_t K = (uint32_t)(kh * kw * ic), steps = (K + 1) / 2;
+    // kernel rows in LDS: whole chunks of steps, so that the unrolled loop needs no guard (rows beyond K are zero)
+    const uint32_t kernRows = 2 * ((steps + CONV_MFMA_STEPS - 1) / CONV_MFMA_STEPS) * CONV_MFMA_STEPS;
+    float *patch = shConvM;
+    float *kern = patch + (size_t)ic * planePitch;
+    const uint32_t lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const uint32_t half = lane >> 5, col = lane & 31;
+    GLOBAL_AS const uint32_t *bitmap = asGlobal(G.srcBitmap) + (size_t)batch * ((g.numSrcNeurons + 31) / 32);
+    GLOBAL_AS const float *kernel = asGlobal(g.g);
+    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
+    const uint32_t xTiles = ((uint32_t)ow + 31) / 32, oTiles = ((uint32_t)oc + 31) / 32;
+    const uint32_t numTiles = (uint32_t)rows * xTiles * oTiles;
+
+    // ---- requested before anything is waited for: this thread's first words of the bitmap, the kernel
+    const int patchRows = rows + kh - 1;
+    const uint32_t patchElems = (uint32_t)patchRows * patchPitch;
+    auto pixelOf = [&](uint32_t e, int &inRow, int &inCol) -> bool {
+        const int r = (int)(e / patchPitch), c = (int)(e - (uint32_t)r * patchPitch);
+        inRow = y0 - PH + r; inCol = c - PW;
+        return (e < patchElems && inRow >= 0 && inRow < ih && inCol >= 0 && inCol < iw);
+    };
+    // (a thread's first two pixels: all there is to do for patches of up to 512 elements)
+    int inRow0, inCol0, inRow1, inCol1;
+    const bool inside0 = pixelOf(threadIdx.x, inRow0, inCol0), inside1 = pixelOf(threadIdx.x + CONV_MFMA_THREADS, inRow1, inCol1);
+    const uint32_t first0 = inside0 ? (uint32_t)((inRow0 * iw + inCol0) * ic) : 0u, first1 = inside1 ? (uint32_t)((inRow1 * iw + inCol1) * ic) : 0u;
+    const uint32_t word0 = bitmap[first0 >> 5], word1 = bitmap[first1 >> 5];
+
+    // ---- kernel weights [k][o] into LDS, rows padded to kernPitch
+    if(kernPitch == (uint32_t)oc && (oc & 3) == 0 && (reinterpret_cast<uintptr_t>(g.g) & 15) == 0) {
+        // rows are contiguous on both sides: 16 bytes per load, up to eight loads in flight per thread
+        const uint32_t quads = K * (uint32_t)oc / 4, allQuads = kernRows * kernPitch / 4;
+        GLOBAL_AS const f32x4 *src = reinterpret_cast<GLOBAL_AS const f32x4*>(kernel);
+        f32x4 *dst = reinterpret_cast<f32x4*>(kern);
+        for(uint32_t q0 = 0; q0 < allQuads; q0 += 8 * CONV_MFMA_THREADS) {
+            f32x4 w[8];
+            #pragma unroll
+            for(int u = 0; u < 8; u++) { const uint32_t q = q0 + u * CONV_MFMA_THREADS + threadIdx.x; w[u] = src[min(q, quads - 1)]; }
+            #pragma unroll
+            for(int u = 0; u < 8; u++) {
+                const uint32_t q = q0 + u * CONV_MFMA_THREADS + threadIdx.x;
+                const f32x4 zero = {0, 0, 0, 0};
+                if(q < allQuads) { dst[q] = (q < quads) ? w[u] : zero; }
+            }
+        }
+    }
+    else {
+        for(uint32_t e0 = 0; e0 < kernRows * kernPitch; e0 += 8 * CONV_MFMA_THREADS) {
+            float w[8];
+            #pragma unroll
+            for(int u = 0; u < 8; u++) {
+                const uint32_t e = e0 + u * CONV_MFMA_THREADS + threadIdx.x;
+                const uint32_t k = e / kernPitch, o = e - k * kernPitch;
+                w[u] = kernel[(size_t)min(k, K - 1) * oc + min(o, (uint32_t)oc - 1)] * ((k < K && o < (uint32_t)oc) ? 1.0f : 0.0f);
+            }
+            #pragma unroll
+            for(int u = 0; u < 8; u++) {
+                const uint32_t e = e0 + u * CONV_MFMA_THREADS + threadIdx.x;
+                if(e < kernRows * kernPitch) { kern[e] = w[u]; }
+            }
+        }
+    }
+
+    // ---- input patch: bit (row * iw + col) * ic + ch of the source's bitmap -> patch[ch][r][c].  A pixel's spikes are
+    // counted as events by the block whose output rows include the pixel's row (the last block takes the rows below):
+    // every spike reaches kh * kw * oc targets less what falls outside the output.
+    unsigned long long events = 0;
+    const bool lastBlock = (y0 + rows >= oh);
+    for(uint32_t e = threadIdx.x; e < patchElems; e += CONV_MFMA_THREADS) {
+        int inRow, inCol;
+        const bool inside = pixelOf(e, inRow, inCol);
+        const uint32_t id0 = inside ? (uint32_t)((inRow * iw + inCol) * ic) : 0u;
+        uint32_t wordIdx = id0 >> 5, word = (e == threadIdx.x) ? word0 : (e == threadIdx.x + CONV_MFMA_THREADS) ? word1 : bitmap[wordIdx], fired = 0;
+        for(int ch = 0; ch < ic; ch++) {
+            const uint32_t id = id0 + (uint32_t)ch;
+            if(inside && (id >> 5) != wordIdx) { wordIdx = id >> 5; word = bitmap[wordIdx]; }
+            const bool bit = inside && ((word >> (id & 31)) & 1u);
+            patch[(size_t)ch * planePitch + e] = bit ? 1.0f : 0.0f;
+            fired += bit ? 1u : 0u;
+        }
+        if(fired && inRow >= y0 && (inRow < y0 + rows || lastBlock)) {
+            int rowTaps = 0, colTaps = 0;
+            for(int kr = 0; kr < kh; kr++) { const int pr = inRow + kr - G.convBH; rowTaps += (pr >= 0 && pr < oh) ? 1 : 0; }
+            for(int kc = 0; kc < kw; kc++) { const int pc = inCol + kc - G.convBW; colTaps += (pc >= 0 && pc < ow) ? 1 : 0; }
+            events += (unsigned long long)fired * (unsigned long long)(rowTaps * colTaps * oc);
+        }
+    }
+    __syncthreads();
+
+    // A[i][k]: pixel x0 + i, k = (a * kw + b) * ic + ch -> patch[ch][r + a][x0 + i + b];  B[k][j] = kern[k][n0 + j]; the
+    // two halves of the wavefront take k = 2 s and 2 s + 1.  Where step s starts in the patch is worked out once per chunk
+    // of steps, lane L keeping the offsets of steps L and L + 64 for either half; the loop fetches them with readlane, so
+    // it holds no division and no branch and its LDS reads can all be in flight ahead of the matrix instructions.
+    auto patchOffsetOf = [&](uint32_t k) -> uint32_t {
+        const uint32_t kk = min(k, K - 1);                          // (beyond K: any valid place, B is zero there)
+        const uint32_t tap = kk / (uint32_t)ic, ch = kk - tap * (uint32_t)ic;
+        const uint32_t ta = tap / (uint32_t)kw;
+        return ch * planePitch + ta * patchPitch + (tap - ta * (uint32_t)kw);
+    };
+    for(uint32_t tile = wave; tile < numTiles; tile += CONV_MFMA_THREADS / WAVE) {
+        const uint32_t r = tile / (xTiles * oTiles), x0 = ((tile / oTiles) % xTiles) * 32, n0 = (tile % oTiles) * 32;
+        const uint32_t y = (uint32_t)y0 + r, o = n0 + col;
+        f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        const float *aBase = patch + r * patchPitch + x0 + col;
+        for(uint32_t s0 = 0; s0 < steps; s0 += CONV_MFMA_STEPS) {
+            const int evenLo = (int)patchOffsetOf(2 * (s0 + lane)), oddLo = (int)patchOffsetOf(2 * (s0 + lane) + 1);
+            const int evenHi = (int)patchOffsetOf(2 * (s0 + lane + WAVE)), oddHi = (int)patchOffsetOf(2 * (s0 + lane + WAVE) + 1);
+            const float *bBase = kern + (size_t)(2 * s0 + half) * kernPitch + n0 + col;
+            // software pipeline: the operands of the next CONV_MFMA_AHEAD steps are read from LDS while the matrix
+            // instructions of the current ones run (the scheduling barriers keep the reads where they are written: left to itself
+            // the compiler sinks every read to just before its use)
+            constexpr int AHEAD = CONV_MFMA_AHEAD;
+            float av[2][AHEAD], bv[2][AHEAD];
+            auto fetch = [&](int buffer, int first) {
+                #pragma unroll
+                for(int u = 0; u < AHEAD; u++) {
+                    const int s = first + u;
+                    const int even = __builtin_amdgcn_readlane((s < WAVE) ? evenLo : evenHi, s & (WAVE - 1));
+                    const int odd = __builtin_amdgcn_readlane((s < WAVE) ? oddLo : oddHi, s & (WAVE - 1));
+                    av[buffer][u] = aBase[half ? odd : even];
+                    bv[buffer][u] = bBase[(size_t)2 * s * kernPitch];
+                }
+            };
+            fetch(0, 0);
+            #pragma unroll
+            for(int c = 0; c < CONV_MFMA_STEPS / AHEAD; c++) {
+                __builtin_amdgcn_sched_barrier(0);
+                if(c + 1 < CONV_MFMA_STEPS / AHEAD) { fetch((c + 1) & 1, (c + 1) * AHEAD); }
+                __builtin_amdgcn_sched_barrier(0);
+                #pragma unroll
+                for(int u = 0; u < AHEAD; u++) { acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[c & 1][u], bv[c & 1][u], acc, 0, 0, 0); }
+            }
+        }
+        // register v of lane (half, col) holds D[i][j] with i = 8 * (v / 4) + 4 * half + v % 4, j = col: the 32 lanes of a
+        // half add to the 32 consecutive channels of one pixel (one atomic without return per element and step, so the
+        // result does not depend on their order; a read-modify-write by the owning lane measured no faster)
+        #pragma unroll
+        for(int v = 0; v < 16; v++) {
+            const uint32_t x = x0 + 8 * (v / 4) + 4 * half + (v % 4);
+            if(x < (uint32_t)ow && o < (uint32_t)oc && acc[v] != 0.0f) { atomicAddF32(&outPost[((size_t)y * ow + x) * oc + o], acc[v]); }
+        }
+    }
+    for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
+    if(lane == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+// bitmap of a population's spike queue, for callers that wrote the queue themselves (the neuron update keeps it otherwise)
+__global__ void spikeBitmapFromQueueKernel(const uint32_t *spkCnt, const uint32_t *spk, uint32_t *bitmap, uint32_t numNeurons, uint32_t clear)
+{
+    const uint32_t batch = blockIdx.y, words = (numNeurons + 31) / 32;
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if(clear) { if(i < words) { bitmap[(size_t)batch * words + i] = 0u; } return; }
+    if(i < spkCnt[batch]) { const uint32_t id = spk[(size_t)batch * numNeurons + i]; atomicOr(&bitmap[(size_t)batch * words + (id >> 5)], 1u << (id & 31)); }
+}
+
 __global__ __launch_bounds__(1024)
 void presynapticUpdateKernel(const PreGroupDev * __restrict__ blocks, StepArgs args, float dt, unsigned long long *eventCounter)
 {
-    presynapticBody(blocks[blockIdx.x], blockIdx.x, resolve(args, dt), dt, eventCounter);
+    presynapticBody(blocks[blockIdx.x], blockIdx.x, blockIdx.y, gridDim.y, resolve(args, dt), dt, eventCounter);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -853,7 +1049,7 @@ void synapseCombinedKernel(const PreGroupDev * __restrict__ pre, uint32_t preBlo
 {
     extern __shared__ float shDynamic[];
     if(blockIdx.x < preBlocks) {
-        presynapticBody(pre[blockIdx.x], blockIdx.x, resolve(args, dt), dt, eventCounter);
+        presynapticBody(pre[blockIdx.x], blockIdx.x, blockIdx.y, gridDim.y, resolve(args, dt), dt, eventCounter);
     }
     else if(blockIdx.x < preBlocks + tileBlocks) {
         presynapticTileBody(tiles[blockIdx.x - preBlocks], shDynamic, args, dt, eventCounter);

@@ -399,7 +399,9 @@ int gennmi_runner_stream_elapsed(gennmi_runner *runner, double *seconds);
  * tile path and (bit 5) the postsynaptic passes of a step share one launch (projections with a tile path, or plastic ones
  * whose postsynaptic pass is paired with the presynaptic one: a synapse both of whose ends fired gets both rules from the
  * thread of the presynaptic pass, in the reference's order, and the postsynaptic pass leaves that row alone;
- * GENNMI_COMBINED=0 keeps a launch per kernel, GENNMI_PAIRED_LEARN=0 the reference's two passes); info[1..3] = blocks of
+ * GENNMI_COMBINED=0 keeps a launch per kernel, GENNMI_PAIRED_LEARN=0 the reference's two passes); bit 6 if the busy steps
+ * of a Toeplitz Conv2D projection run on the matrix cores (the layer as a GEMM over the source's spike bitmap in fp32 MFMA:
+ * same products, sums in another order than the event-driven kernels'; GENNMI_CONV_MFMA=0 keeps those); info[1..3] = blocks of
  * the neuron, presynaptic and postsynaptic kernels.  The reference logs the analogous choice of presynaptic
  * strategy (backendSIMT.cc:736). */
 int gennmi_runner_get_info(gennmi_runner *runner, uint32_t info[4]);

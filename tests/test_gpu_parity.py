@@ -187,6 +187,32 @@ def test_toeplitz_conv_layer():
     model.unload()
 
 
+@pytest.mark.parametrize("h, w, ic, oc, k", [(10, 12, 3, 5, 3), (8, 40, 4, 40, 5), (6, 33, 8, 32, 5), (9, 9, 1, 3, 3)])
+def test_toeplitz_conv_on_matrix_cores(h, w, ic, oc, k, monkeypatch):
+    """The dense path of a Conv2D projection (fp32 MFMA over the spike bitmap) on shapes that exercise its edges: an odd
+    number of input channels (a pair of sum steps straddles two kernel taps) and an odd K (zero padding row), output
+    channels and widths that are no multiple of the 32 x 32 tile or need several tiles, and 5 x 5 kernels whose sum is
+    longer than one unrolled chunk of steps.  Activity is high enough that every step takes the dense path; rasters must be
+    the oracle's, state within 1e-5, and the event count exact."""
+    net = configs.conv_toeplitz(h=h, w=w, ic=ic, oc=oc, k=k, steps=60, w_sd=0.5 / k, max_rate=400.0, ioffset=0.3)
+    model, oracle, counts = run_side_by_side(net, check_every=20, exact=False, exact_steps=60)
+    assert counts["Out"] > 50 and counts["In"] > 5 * h * w * ic
+    assert model.synaptic_event_count == oracle.events()
+    assert model.runner_info()["conv_on_matrix_cores"]
+    # the event-driven kernels on the same network: same rasters, same event count
+    monkeypatch.setenv("GENNMI_CONV_MFMA", "0")
+    other = model_from_net(net)
+    other.load(num_recording_timesteps=60)
+    assert not other.runner_info()["conv_on_matrix_cores"]
+    other.run(60)
+    other.synchronize()
+    assert other.synaptic_event_count == model.synaptic_event_count
+    for p in net.pops:
+        assert np.array_equal(other.neuron_populations[p.name].current_spikes[0], model.neuron_populations[p.name].current_spikes[0])
+    other.unload()
+    model.unload()
+
+
 def test_toeplitz_batches_are_independent():
     """Batch b of a batched run equals a batch-1 run of the oracle fed batch b's spike trains."""
     B = 3
