@@ -357,7 +357,9 @@ def main():
             try:
                 spec, work, out_dir = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
                 os.makedirs(work); os.makedirs(out_dir)
-                old_steps, net.steps, net.snap = net.steps, args.reference_steps, 0
+                # (a per-step noise array holds as many rows as it holds: the driver reads one per step)
+                rows = [c.noise.size // net.pop(c.pop).n for c in net.css if getattr(c, "noise", None) is not None]
+                old_steps, net.steps, net.snap = net.steps, min([args.reference_steps] + rows), 0
                 write_netspec(net, spec)
                 net.steps = old_steps
                 res = subprocess.run([driver, spec, work, out_dir, "--cxxflags=-O3"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
@@ -381,7 +383,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": label, "neurons": num_neurons, "synapses": num_synapses, "dt_ms": net.dt, "seed": net.seed,
                    "stepping": ("resident plan: one launch for all timed steps, state in registers/LDS" if info["resident_plan"] else
-                                "hipGraph replay, 100 steps per graph, " + ("1 launch per step" if info["single_launch_step"] else "2-3 launches per step"))},
+                                "hipGraph replay, 100 steps per graph, " + ("1 launch per step" if info["single_launch_step"] else
+                                                                           "2 launches per step (synaptic kernels combined)" if (info["combined_synapse_launch"] or info["conv_on_matrix_cores"]) else
+                                                                           "2-3 launches per step"))},
         "gsop_per_s": round(events / wall / 1e9, 4),
         "neuron_updates_per_s": round(num_neurons * batch * args.steps / wall, 1),
         "wall_s_per_sim_s": round(wall / sim_s, 4),
