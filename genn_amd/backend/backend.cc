@@ -922,11 +922,38 @@ void Backend::genCustomUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
 // the arrays' host buffers (merged init groups carry host pointers), followed by an upload of every buffer.
 // initializeSparse() additionally builds the column view of plastic projections on the device.
 //--------------------------------------------------------------------------
+namespace
+{
+// value snippets the device library draws itself: snippet id and parameter names in the order gennmi_init_var takes them
+bool deviceVarSnippet(const InitVarSnippet::Base *snippet, unsigned int &id, std::vector<std::string> &params)
+{
+    if(snippet == InitVarSnippet::Constant::getInstance()) { id = GENNMI_INIT_CONSTANT; params = {"constant"}; }
+    else if(snippet == InitVarSnippet::Uniform::getInstance()) { id = GENNMI_INIT_UNIFORM; params = {"min", "max"}; }
+    else if(snippet == InitVarSnippet::Normal::getInstance()) { id = GENNMI_INIT_NORMAL; params = {"mean", "sd"}; }
+    else if(snippet == InitVarSnippet::NormalClipped::getInstance()) { id = GENNMI_INIT_NORMAL_CLIPPED; params = {"mean", "sd", "min", "max"}; }
+    else if(snippet == InitVarSnippet::Exponential::getInstance()) { id = GENNMI_INIT_EXPONENTIAL; params = {"lambda"}; }
+    else if(snippet == InitVarSnippet::Gamma::getInstance()) { id = GENNMI_INIT_GAMMA; params = {"a", "b"}; }
+    else { return false; }
+    return true;
+}
+}
+
 void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelMerged,
                       BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const
 {
     const ModelSpecInternal &model = modelMerged.getModel();
     const unsigned int batchSize = model.getBatchSize();
+    const bool deviceInit = getPreferences<Preferences>().deviceInitialisation;
+    // generator streams of device-side initialisation: 2k + 1 for the connectivity of the k-th projection by name (the numbering
+    // PROCEDURAL projections use for the same purpose), 2k + 2 + 2 * (number of projections) * v for its v-th variable by name
+    auto place = [&model](const SynapseGroupInternal &g) -> uint64_t
+    {
+        return (uint64_t)std::distance(model.getSynapseGroups().cbegin(), model.getSynapseGroups().find(g.getName()));
+    };
+    const uint64_t numProjections = model.getSynapseGroups().size();
+    // the model's seed, or one drawn when the runner is loaded (ModelSpec: seed 0 = a different one every run)
+    const std::string seedExpr = (model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull")
+                                                        : std::string("gennmiRandomSeed()");
 
     std::ostringstream bodyStream;
     CodeStream body(bodyStream);
@@ -991,6 +1018,51 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                     unsupported("connectivity initialisation of projection '" + arch.getName() + "' (SPARSE without kernel only)");
                 }
                 const bool byRow = !Utils::areTokensEmpty(connect.getRowBuildCodeTokens());
+                // built-in snippets the device library generates itself (Preferences::deviceInitialisation)
+                const auto *snippet = connect.getSnippet();
+                const int deviceSnippet = !deviceInit ? -1
+                    : (snippet == InitSparseConnectivitySnippet::FixedProbability::getInstance()) ? 0
+                    : (snippet == InitSparseConnectivitySnippet::FixedProbabilityNoAutapse::getInstance()) ? 1
+                    : (snippet == InitSparseConnectivitySnippet::FixedNumberPostWithReplacement::getInstance()) ? 2
+                    : (snippet == InitSparseConnectivitySnippet::OneToOne::getInstance()) ? 3 : -1;
+                if(deviceSnippet >= 0) {
+                    forEachGroup(funcEnv, "SynapseConnectivityInitGroup", s.getIndex(), s.getGroups().size(), [&]
+                    {
+                        EnvironmentGroupMergedField<SynapseConnectivityInitGroupMerged> env(funcEnv, s);
+                        buildStandardEnvironment(env, batchSize);
+                        std::vector<uint64_t> streams;
+                        std::vector<Type::NumericValue> values;
+                        for(const auto &g : s.getGroups()) {
+                            streams.push_back(2 * place(g.get()) + 1);
+                            const auto &params = g.get().getSparseConnectivityInitialiser().getParams();
+                            if(deviceSnippet <= 1) { values.push_back(params.at("prob")); }
+                            else if(deviceSnippet == 2) { values.push_back(params.at("num")); }
+                        }
+                        CodeStream::Scope scope(env.getStream());
+                        env.getStream() << "static const uint32_t stream[] = " << tableU32(streams) << ";" << std::endl;
+                        if(deviceSnippet <= 2) { env.getStream() << "static const double value[] = " << table(values, Type::Double) << ";" << std::endl; }
+                        env.getStream() << "uint32_t overflowRows = 0;" << std::endl;
+                        const std::string arrays = "gennmiDev(" + env["_row_length"] + "), gennmiDev(" + env["_ind"] + ")";
+                        const std::string shape = env["num_pre"] + ", " + env["num_post"] + ", " + env["_row_stride"];
+                        if(deviceSnippet <= 1) {
+                            env.getStream() << "GENNMI_CHECK(gennmi_init_sparse_fixed_probability(" << shape << ", value[g], " << deviceSnippet << ", " << seedExpr
+                                            << ", stream[g], " << arrays << ", &overflowRows));" << std::endl;
+                        }
+                        else if(deviceSnippet == 2) {
+                            env.getStream() << "GENNMI_CHECK(gennmi_init_sparse_fixed_number_post(" << shape << ", (uint32_t)value[g], nullptr, " << seedExpr
+                                            << ", stream[g], " << arrays << ", &overflowRows));" << std::endl;
+                        }
+                        else {
+                            env.getStream() << "(void)stream; GENNMI_CHECK(gennmi_init_sparse_one_to_one(" << shape << ", " << arrays << "));" << std::endl;
+                        }
+                        // the host mirrors follow: per-row initialisation code, pulls and the upload that ends initialize() read them
+                        env.getStream() << "GENNMI_CHECK(gennmi_memcpy_from_device(" << env["_row_length"] << ", gennmiDev(" << env["_row_length"] << "), (size_t)"
+                                        << env["num_pre"] << " * sizeof(uint32_t)));" << std::endl;
+                        env.getStream() << "GENNMI_CHECK(gennmi_memcpy_from_device(" << env["_ind"] << ", gennmiDev(" << env["_ind"] << "), (size_t)"
+                                        << env["num_pre"] << " * " << env["_row_stride"] << " * sizeof(uint32_t)));" << std::endl;
+                    });
+                    return;
+                }
                 forEachGroup(funcEnv, "SynapseConnectivityInitGroup", s.getIndex(), s.getGroups().size(), [&]
                 {
                     EnvironmentGroupMergedField<SynapseConnectivityInitGroupMerged> env(funcEnv, s);
@@ -1060,7 +1132,49 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                 {
                     EnvironmentGroupMergedField<SynapseSparseInitGroupMerged> env(funcEnv, s);
                     buildStandardEnvironment(env, batchSize);
-                    if(s.getArchetype().isWUVarInitRequired()) {
+                    // per-synapse variables whose initialisers are all snippets the device library draws itself
+                    // (Preferences::deviceInitialisation): filled over the whole numPre * rowStride range, padding is never read
+                    bool varsOnDevice = deviceInit && s.getArchetype().isWUVarInitRequired() && (batchSize == 1);
+                    struct DeviceVar { std::string name; unsigned int snippet; std::vector<std::string> params; };
+                    std::vector<DeviceVar> deviceVars;
+                    if(varsOnDevice) {
+                        for(const auto &var : s.getArchetype().getWUInitialiser().getSnippet()->getVars()) {
+                            const auto &init = s.getArchetype().getWUInitialiser().getVarInitialisers().at(var.name);
+                            if(Utils::areTokensEmpty(init.getCodeTokens())) { continue; }           // left uninitialised: nothing to do
+                            DeviceVar d{var.name, 0, {}};
+                            varsOnDevice = varsOnDevice && var.type.resolve(model.getTypeContext()) == Type::Float
+                                           && deviceVarSnippet(init.getSnippet(), d.snippet, d.params);
+                            for(const auto &g : s.getGroups()) {
+                                varsOnDevice = varsOnDevice && (g.get().getWUInitialiser().getVarInitialisers().at(var.name).getSnippet() == init.getSnippet());
+                            }
+                            deviceVars.push_back(d);
+                        }
+                    }
+                    if(varsOnDevice) {
+                        size_t varIndex = 0;
+                        for(const auto &d : deviceVars) {
+                            const std::string name = d.name;
+                            env.addField(Type::Float.createPointer(), "_mi_init_" + name, name,
+                                         [name](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, name); });
+                            std::vector<uint64_t> streams;
+                            for(const auto &g : s.getGroups()) { streams.push_back(2 * place(g.get()) + 2 + 2 * numProjections * varIndex); }
+                            CodeStream::Scope scope(env.getStream());
+                            env.getStream() << "static const uint32_t stream[] = " << tableU32(streams) << ";" << std::endl;
+                            env.getStream() << "double params[4] = {0.0, 0.0, 0.0, 0.0};" << std::endl;
+                            for(size_t k = 0; k < d.params.size(); k++) {
+                                std::vector<Type::NumericValue> values;
+                                for(const auto &g : s.getGroups()) { values.push_back(g.get().getWUInitialiser().getVarInitialisers().at(name).getParams().at(d.params[k])); }
+                                env.getStream() << "{ static const double v[] = " << table(values, Type::Double) << "; params[" << k << "] = v[g]; }" << std::endl;
+                            }
+                            const std::string count = "(size_t)" + env["num_pre"] + " * " + env["_row_stride"];
+                            env.getStream() << "GENNMI_CHECK(gennmi_init_var(gennmiDev(" << env["_mi_init_" + name] << "), " << GENNMI_TYPE_F32 << "u, " << count << ", "
+                                            << d.snippet << "u, params, " << seedExpr << ", stream[g]));" << std::endl;
+                            env.getStream() << "GENNMI_CHECK(gennmi_memcpy_from_device(" << env["_mi_init_" + name] << ", gennmiDev(" << env["_mi_init_" + name] << "), "
+                                            << count << " * sizeof(float)));" << std::endl;
+                            varIndex++;
+                        }
+                    }
+                    else if(s.getArchetype().isWUVarInitRequired()) {
                         env.print("for(unsigned int i = 0; i < $(num_pre); i++)");
                         CodeStream::Scope loop(env.getStream());
                         env.add(Type::Uint32.addConst(), "id_pre", "i");
@@ -1211,6 +1325,8 @@ void Backend::genDefinitionsPreamble(CodeStream &os, const ModelSpecMerged&) con
     }
     os << "using std::min;" << std::endl;
     os << "using std::max;" << std::endl;
+    os << "// seed of device-side initialisation for models that leave theirs at 0 (a different one every run, ModelSpec::setSeed)" << std::endl;
+    os << "inline uint64_t gennmiRandomSeed() { static const uint64_t seed = [] { std::random_device rd; return ((uint64_t)rd() << 32) | rd(); }(); return seed; }" << std::endl;
     os << std::endl;
 }
 //--------------------------------------------------------------------------

@@ -47,6 +47,15 @@ struct Preferences : public PreferencesBase
     //! results do not depend on it; 0 launches every step when it is asked for.
     unsigned int stepQueueLength = 256;
 
+    //! initialize() / initializeSparse() run the reference's generic initialisation code on the host (which is what makes
+    //! a model start from exactly the state the SingleThreadedCPU backend gives it).  With this switch, SPARSE connectivity
+    //! built by FixedProbability, FixedProbabilityNoAutapse, FixedNumberPostWithReplacement or OneToOne and per-synapse
+    //! variables initialised by Constant, Uniform, Normal, NormalClipped, Exponential or Gamma are generated on the device
+    //! instead (gennmi_init_sparse_*, gennmi_init_var: counter-based Philox draws from the model's seed, one stream per
+    //! array) and copied back into the host mirrors: same distributions, other numbers -- as between the reference's own
+    //! CPU and GPU backends.  Everything else is initialised on the host as before.
+    bool deviceInitialisation = false;
+
     void updateHash(boost::uuids::detail::sha1 &hash) const
     {
         PreferencesBase::updateHash(hash);
@@ -54,6 +63,7 @@ struct Preferences : public PreferencesBase
         Utils::updateHash(static_cast<int>(kernelSource), hash);
         Utils::updateHash(orderedAccumulation, hash);
         Utils::updateHash(stepQueueLength, hash);
+        Utils::updateHash(deviceInitialisation, hash);
     }
 };
 

@@ -325,6 +325,16 @@ def procedural(n_e=1600, n_i=400, steps=200, seed=31, dt=1.0, order_free=False):
     return net
 
 
+def snippet_initialised(n_e=1600, n_i=400, steps=200, seed=31, dt=1.0):
+    """The network of :func:`procedural` with its four projections stored: SPARSE matrices whose connectivity and weights are
+    built by the same snippets at initialisation time."""
+    net = procedural(n_e=n_e, n_i=n_i, steps=steps, seed=seed, dt=dt)
+    net.name = "snippet_initialised"
+    for s in net.syns:
+        s.matrix = "sparse_init"
+    return net
+
+
 def dense_layer(n_in=8192, n_out=8192, rate_hz=50.0, steps=1000, seed=17, dt=1.0, w_sd=0.02):
     """A fully connected spiking layer: Poisson sources (rate_hz per source) into LIF neurons through a DENSE matrix
     with individual weights ~ N(0, w_sd); the shape of the dense layers of rate-coded classifiers."""

@@ -493,9 +493,9 @@ class GeNNModel:
         self._arrays.append(a)
         return a
 
-    def _alloc_device_init(self, count, dtype, init):
+    def _alloc_device_init(self, count, dtype, init, stream=None):
         a = self._alloc(count, dtype, device_only=True)
-        a.init_on_device(init, self.seed, self._next_stream(), self.dt)
+        a.init_on_device(init, self.seed, self._next_stream() if stream is None else stream, self.dt)
         return a
 
     def _next_stream(self):
@@ -609,7 +609,8 @@ class GeNNModel:
                     if name not in s.var_host and isinstance(s.wu.vars[name], VarInit):
                         if copies != 1:
                             raise NotImplementedError(f"{s.name}: device-side initialisation of plastic weights with batch size > 1")
-                        s.vars[name] = self._alloc_device_init(n_pre * s.row_stride, dtype, s.wu.vars[name])
+                        streams = getattr(s, "init_streams", None)
+                        s.vars[name] = self._alloc_device_init(n_pre * s.row_stride, dtype, s.wu.vars[name], streams[1] if streams and name == "g" else None)
                         continue
                     a = self._alloc(copies * n_pre * s.row_stride, dtype)
                     if name in s.var_host:
@@ -671,11 +672,13 @@ class GeNNModel:
         lib = _abi.load()
         n_pre, n_post = s.src.num_neurons, s.trg.num_neurons
         snippet, params = s.conn.snippet, s.conn.params
-        s.row_stride = max_row_length(snippet, params, n_pre, n_post)
+        multiple = getattr(s, "row_stride_multiple", 1)         # (the GeNN backend pads rows to 4 entries)
+        s.row_stride = (max_row_length(snippet, params, n_pre, n_post) + multiple - 1) // multiple * multiple
         s.vars["rowLength"] = self._alloc(n_pre, np.uint32, device_only=True)
         s.vars["ind"] = self._alloc(n_pre * s.row_stride, np.uint32, device_only=True)
         row_length, ind = s.vars["rowLength"].ptr, s.vars["ind"].ptr
-        stream = self._next_stream()
+        # (a caller that must reproduce another numbering of the generator streams sets init_streams beforehand)
+        stream = s.init_streams[0] if getattr(s, "init_streams", None) else self._next_stream()
         if snippet == "OneToOne":
             _abi.check(lib.gennmi_init_sparse_one_to_one(n_pre, n_post, s.row_stride, row_length, ind))
         elif snippet in ("FixedProbability", "FixedProbabilityNoAutapse"):
@@ -1106,13 +1109,18 @@ def model_from_net(net, batch_size=1, record=True, span=None, device=0, ordered=
             q = s.wum_params
             wu = init_weight_update("STDP", {"tauPlus": q["tauPlus"], "tauMinus": q["tauMinus"], "Aplus": q["aPlus"], "Aminus": q["aMinus"],
                                              "Wmin": q["wMin"], "Wmax": q["wMax"]}, {"g": 0.0})
-        if s.matrix == "procedural":
+        if s.matrix in ("procedural", "sparse_init"):
             if s.wum == "static":
                 wu = init_weight_update("StaticPulse", {}, {"g": init_var(*s.g_init)})
-            sg = m.add_synapse_population(s.name, "PROCEDURAL", pops[s.src], pops[s.trg], wu, ps, init_sparse_connectivity(*s.connect))
+            sg = m.add_synapse_population(s.name, "PROCEDURAL" if s.matrix == "procedural" else "SPARSE", pops[s.src], pops[s.trg], wu, ps,
+                                          init_sparse_connectivity(*s.connect))
             # the numbering a GeNN model gets from the backend adapter: streams 2k + 1 and 2k + 2 for the k-th projection by name
             k = sorted(x.name for x in net.syns).index(s.name)
-            sg.procedural_streams = [2 * k + 1, 2 * k + 2]
+            if s.matrix == "procedural":
+                sg.procedural_streams = [2 * k + 1, 2 * k + 2]
+            else:
+                sg.init_streams = [2 * k + 1, 2 * k + 2]
+                sg.row_stride_multiple = 4
         elif s.matrix == "dense":
             sg = m.add_synapse_population(s.name, "DENSE", pops[s.src], pops[s.trg], wu, ps)
             if s.g is not None:

@@ -66,7 +66,8 @@ class Syn:
     axonal_delay_steps: int = 0     # spikes reach the projection this many timesteps late (SynapseGroup::setAxonalDelaySteps)
     conv: Dict[str, int] = field(default_factory=dict)
     # matrix == "procedural": connect = (snippet, params) of a built-in connectivity snippet, g_init = (snippet, params) of the
-    # weight initialisation snippet (or wum "static_const"); nothing is stored
+    # weight initialisation snippet (or wum "static_const"); nothing is stored.  matrix == "sparse_init": the same two
+    # snippets initialise a stored SPARSE matrix (on the host, or on the device where the executor is asked to)
     connect: Optional[tuple] = None
     g_init: Optional[tuple] = None
 
@@ -74,7 +75,7 @@ class Syn:
     def num_synapses(self):
         if self.matrix == "bitmask":
             return int(np.unpackbits(np.ascontiguousarray(self.gp).view(np.uint8)).sum())
-        if self.matrix == "procedural":
+        if self.matrix in ("procedural", "sparse_init"):
             return 0
         if self.matrix == "dense":
             return int(self.g.size) if self.g is not None else 0
@@ -145,7 +146,7 @@ def write_netspec(net: Net, path: str):
     lines.append(f"snap {snap}")
     if getattr(net, "batch_size", 1) != 1:
         lines.append(f"batch {int(net.batch_size)}")
-    if any(s.matrix == "procedural" for s in net.syns) or any(c.model == "poisson_exp" for c in net.css):
+    if any(s.matrix in ("procedural", "sparse_init") for s in net.syns) or any(c.model == "poisson_exp" for c in net.css):
         lines.append(f"seed {int(net.seed)}")        # procedural matrices and Poisson sources draw from the model's seed
     for kind, group, param, step, value in net.dynamic:
         lines.append(f"dynamic {kind} {group} {param} {int(step)} {float(value)!r}")
@@ -179,18 +180,18 @@ def write_netspec(net: Net, path: str):
             np.ascontiguousarray(s.ind, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.ind.u32"))
         elif s.matrix == "dense":
             head = f"syn {s.name} dense {s.src} {s.trg}"
-        elif s.matrix == "procedural":
+        elif s.matrix in ("procedural", "sparse_init"):
             snippet, params = s.connect
             value = params["num"] if snippet == "FixedNumberPostWithReplacement" else repr(float(params["prob"]))
-            head = f"syn {s.name} procedural {s.src} {s.trg} {snippet} {value}"
+            head = f"syn {s.name} {s.matrix} {s.src} {s.trg} {snippet} {value}"
         elif s.matrix == "bitmask":
             head = f"syn {s.name} bitmask {s.src} {s.trg}"
             np.ascontiguousarray(s.gp, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.gp.u32"))
         else:
             head = f"syn {s.name} conv2d {s.src} {s.trg} " + " ".join(str(int(s.conv[k])) for k in CONV_PARAMS)
-        if s.wum != "static_const" and s.matrix != "procedural":
+        if s.wum != "static_const" and s.matrix not in ("procedural", "sparse_init"):
             np.ascontiguousarray(s.g, dtype=np.float32).tofile(os.path.join(path, f"{s.name}.g.f32"))
-        if s.matrix == "procedural" and s.wum == "static":
+        if s.matrix in ("procedural", "sparse_init") and s.wum == "static":
             snippet, params = s.g_init
             order = {"Constant": ("constant",), "Uniform": ("min", "max"), "Normal": ("mean", "sd")}[snippet]
             w = f"static_init {snippet} " + " ".join(repr(float(params[k])) for k in order)

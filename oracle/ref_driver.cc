@@ -212,7 +212,7 @@ int main(int argc, char *argv[])
         bool generateOnly = false;
         std::string userCxxFlags;
         std::vector<std::string> dynamicParams;
-        bool timing = false, ordered = false;
+        bool timing = false, ordered = false, deviceInit = false;
         int stepQueue = -1;
         std::string kernels = "auto";
         for(int a = 4; a < argc; a++) {
@@ -224,6 +224,7 @@ int main(int argc, char *argv[])
             else if(opt.rfind("--dynamic=", 0) == 0) { dynamicParams.push_back(opt.substr(10)); }
             else if(opt.rfind("--kernels=", 0) == 0) { kernels = opt.substr(10); }    // MI355X backend: library | generated | auto (Preferences::kernelSource)
             else if(opt.rfind("--step-queue=", 0) == 0) { stepQueue = std::stoi(opt.substr(13)); }      // MI355X backend: Preferences::stepQueueLength
+            else if(opt == "--device-init") { deviceInit = true; }                  // MI355X backend: Preferences::deviceInitialisation
             else if(opt == "--ordered") { ordered = true; }                          // MI355X backend: Preferences::orderedAccumulation
             else if(opt == "--timing") { timing = true; }       // ModelSpec::setTimingEnabled; the Runtime's counters are printed after the run
             else { std::cerr << "unknown option " << opt << std::endl; return 1; }
@@ -236,8 +237,9 @@ int main(int argc, char *argv[])
         prefs.kernelSource = (kernels == "generated") ? Preferences::KernelSource::GENERATED : (kernels == "library") ? Preferences::KernelSource::LIBRARY : Preferences::KernelSource::AUTO;
         prefs.orderedAccumulation = ordered;
         if(stepQueue >= 0) { prefs.stepQueueLength = (unsigned int)stepQueue; }
+        prefs.deviceInitialisation = deviceInit;
 #else
-        (void)ordered; (void)stepQueue;
+        (void)ordered; (void)stepQueue; (void)deviceInit;
 #endif
         Logging::init(prefs.gennLogLevel, prefs.codeGeneratorLogLevel, prefs.transpilerLogLevel,
                       prefs.runtimeLogLevel, &app, &app, &app, &app);
@@ -268,7 +270,7 @@ int main(int argc, char *argv[])
                     SynSpec s; ls >> s.name >> s.matrix >> s.src >> s.trg;
                     if(s.matrix == "sparse") { ls >> s.rowStride; }
                     else if(s.matrix == "conv2d") { s.conv.resize(8); for(auto &c : s.conv) ls >> c; }
-                    else if(s.matrix == "procedural") { ls >> s.connect >> s.connectValue; }
+                    else if(s.matrix == "procedural" || s.matrix == "sparse_init") { ls >> s.connect >> s.connectValue; }
                     else if(s.matrix != "dense" && s.matrix != "bitmask") throw std::runtime_error("matrix " + s.matrix);
                     ls >> s.wum;
                     if(s.wum == "static_init") { ls >> s.initSnippet; const int np = (s.initSnippet == "Constant") ? 1 : 2; s.wumP.resize(np); for(auto &c : s.wumP) ls >> c; }
@@ -377,12 +379,13 @@ int main(int argc, char *argv[])
                                 : initVar<InitVarSnippet::Normal>({{"mean", s.wumP[0]}, {"sd", s.wumP[1]}});
                 wum = initWeightUpdate<WeightUpdateModels::StaticPulse>({}, {{"g", init}});
             }
-            if(s.matrix == "procedural") {
+            if(s.matrix == "procedural" || s.matrix == "sparse_init") {
                 const auto connect = (s.connect == "FixedNumberPostWithReplacement")
                     ? initConnectivity<InitSparseConnectivitySnippet::FixedNumberPostWithReplacement>({{"num", (unsigned int)s.connectValue}})
                     : (s.connect == "FixedProbabilityNoAutapse") ? initConnectivity<InitSparseConnectivitySnippet::FixedProbabilityNoAutapse>({{"prob", s.connectValue}})
                     : initConnectivity<InitSparseConnectivitySnippet::FixedProbability>({{"prob", s.connectValue}});
-                s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::PROCEDURAL, src, trg, wum, psm, connect);
+                // ("sparse_init": the same snippets initialise a stored SPARSE matrix)
+                s.sg = model.addSynapsePopulation(s.name, (s.matrix == "procedural") ? SynapseMatrixType::PROCEDURAL : SynapseMatrixType::SPARSE, src, trg, wum, psm, connect);
             }
             else if(s.matrix == "sparse") {
                 s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::SPARSE, src, trg, wum, psm);
@@ -498,7 +501,7 @@ int main(int argc, char *argv[])
             else if(s.matrix == "bitmask") {
                 load(rt.getArray(*s.sg, "gp"), s.name + ".gp.u32");
             }
-            else if(s.wum != "static_const" && s.matrix != "procedural") {
+            else if(s.wum != "static_const" && s.matrix != "procedural" && s.matrix != "sparse_init") {
                 load(rt.getArray(*s.sg, "g"), s.name + ".g.f32");
             }
             if(s.wum == "stdp_trace") {
@@ -507,6 +510,20 @@ int main(int argc, char *argv[])
             }
         }
         rt.initializeSparse();
+        // matrices initialised by snippets: what the initialisation produced, with the backend's row stride
+        for(auto &s : syns) {
+            if(s.matrix != "sparse_init") { continue; }
+            const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
+            std::ofstream(out + "/" + s.name + ".rowStride.txt") << stride << std::endl;
+            auto *rl = rt.getArray(*s.sg, "rowLength"); rl->pullFromDevice();
+            auto *ind = rt.getArray(*s.sg, "ind"); ind->pullFromDevice();
+            appendFile(out + "/" + s.name + ".rowLength.u32", rl->getHostPointer<uint32_t>(), numPre);
+            appendFile(out + "/" + s.name + ".ind.u32", ind->getHostPointer<uint32_t>(), numPre * stride);
+            if(s.wum != "static_const") {
+                auto *g = rt.getArray(*s.sg, "g"); g->pullFromDevice();
+                appendFile(out + "/" + s.name + ".g.f32", g->getHostPointer<float>(), numPre * stride);
+            }
+        }
 
         // fuse map + remap dump
         {

@@ -198,3 +198,32 @@ def test_generated_kernels_say_what_they_do_not_cover(case, what):
         assert "generated kernels do not cover" in res.stdout and what in res.stdout, res.stdout[-2000:]
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_device_initialisation_is_generated_on_request():
+    """Preferences::deviceInitialisation: built-in connectivity and per-synapse variable snippets of SPARSE projections become
+    calls of the device library's generators (with the model's seed and one stream per array) followed by a copy into the host
+    mirrors; without the switch the reference's generic initialisation code runs on the host as before."""
+    from genn_amd import configs
+    net = configs.snippet_initialised(n_e=200, n_i=50, steps=10)
+    net.snap = 0
+    tmp = tempfile.mkdtemp(prefix="adapter_devinit_")
+    try:
+        spec = os.path.join(tmp, "spec")
+        write_netspec(net, spec)
+        for flag in (True, False):
+            work, out = os.path.join(tmp, f"work{int(flag)}"), os.path.join(tmp, f"out{int(flag)}")
+            os.makedirs(work); os.makedirs(out)
+            res = subprocess.run([DRIVER, spec, work, out, "--generate-only"] + (["--device-init"] if flag else []),
+                                 stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+            assert res.returncode == 0, res.stdout[-3000:]
+            init = open(os.path.join(work, net.name + "_CODE", "init.cc")).read()
+            assert ("gennmi_init_sparse_fixed_probability(" in init) == flag
+            assert ("gennmi_init_sparse_fixed_number_post(" in init) == flag
+            assert ("gennmi_init_var(" in init) == flag
+            if flag:
+                assert f"{net.seed}ull" in init and "gennmi_memcpy_from_device(" in init
+                # EI has a constant weight (no variable), so three weight arrays are drawn; four matrices are generated
+                assert init.count("gennmi_init_var(") == 3 or init.count("gennmi_init_var(") == 2
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)

@@ -283,6 +283,63 @@ def test_adapter_batched_plastic_network():
         shutil.rmtree(tmp, ignore_errors=True)
 
 
+def test_adapter_device_initialisation_matches_host_layer():
+    """Preferences::deviceInitialisation through GeNN's generator and Runtime: SPARSE matrices built by FixedProbability
+    (with and without autapses) and FixedNumberPostWithReplacement with Uniform, Normal, Constant and constant-parameter
+    weights.  The adapter numbers the generator streams by projection name, so the Python host layer given the same numbering
+    must produce the very same matrices (row lengths, targets, weights) and then the same rasters; with the switch off the
+    reference's host code draws from mt19937, which gives other matrices of the same distribution."""
+    from genn_amd import configs
+    from genn_amd.genn_model import model_from_net
+    net = configs.snippet_initialised(n_e=1600, n_i=400, steps=150)
+    net.snap = 0
+    tmp = tempfile.mkdtemp(prefix="adapter_devinit_")
+    try:
+        spec = os.path.join(tmp, "spec")
+        write_netspec(net, spec)
+        outs = {}
+        for flag in (True, False):
+            work, out = os.path.join(tmp, f"work{int(flag)}"), os.path.join(tmp, f"out{int(flag)}")
+            os.makedirs(work); os.makedirs(out)
+            print(f"adapter device initialisation ({flag}): running {DRIVER}", flush=True)
+            res = subprocess.run([DRIVER, spec, work, out] + (["--device-init"] if flag else []), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+            assert res.returncode == 0, res.stdout[-3000:]
+            outs[flag] = out
+        model = model_from_net(net)
+        model.load(num_recording_timesteps=net.steps)
+        for s in net.syns:
+            sg = model.synapse_populations[s.name]
+            n_pre = net.pop(s.src).n
+            stride = int(open(os.path.join(outs[True], f"{s.name}.rowStride.txt")).read())
+            assert stride == sg.row_stride
+            got_len = np.fromfile(os.path.join(outs[True], f"{s.name}.rowLength.u32"), np.uint32)
+            got_ind = np.fromfile(os.path.join(outs[True], f"{s.name}.ind.u32"), np.uint32).reshape(n_pre, stride)
+            want_len = sg.vars["rowLength"].pull_from_device()
+            want_ind = sg.vars["ind"].pull_from_device().reshape(n_pre, stride)
+            mask = np.arange(stride)[None, :] < want_len[:, None]
+            assert np.array_equal(got_len, want_len), f"{s.name}: row lengths differ"
+            assert np.array_equal(got_ind[mask], want_ind[mask]), f"{s.name}: targets differ"
+            if s.wum != "static_const":
+                got_g = np.fromfile(os.path.join(outs[True], f"{s.name}.g.f32"), np.float32).reshape(n_pre, stride)
+                assert np.array_equal(got_g[mask], sg.vars["g"].pull_from_device().reshape(n_pre, stride)[mask]), f"{s.name}: weights differ"
+            # host initialisation: another draw of the same distribution
+            host_len = np.fromfile(os.path.join(outs[False], f"{s.name}.rowLength.u32"), np.uint32)
+            assert not np.array_equal(host_len, got_len) or s.connect[0] == "FixedNumberPostWithReplacement"
+            assert abs(host_len.mean() - got_len.mean()) <= 0.05 * got_len.mean() + 1e-9
+        model.run(net.steps)
+        model.pull_recording_buffers_from_device()
+        total = 0
+        for p in net.pops:
+            got = np.fromfile(os.path.join(outs[True], f"{p.name}.spikes.u32"), np.uint32).reshape(-1, 2)
+            want = _raster(model, net, p.name)
+            assert np.array_equal(got, want), f"raster of {p.name} differs ({len(got)} vs {len(want)} spikes)"
+            total += len(want)
+        assert total > 1000
+        model.unload()
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
 def _procedural_pair(net, steps, snap):
     """Runs `net` through GeNN's generator and Runtime on the adapter and through the Python host layer with the adapter's
     stream numbering; returns (driver output directory, temporary directory, host-layer model after `steps` steps,
