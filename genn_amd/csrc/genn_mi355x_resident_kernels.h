@@ -186,8 +186,14 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     for(uint32_t m = 0; m < numPSM; m++) {
         lds[T.ldsIn[m] + tid] = mine ? asGlobal(g.psm[m].outPost)[i] : 0.0f;
         const uint32_t D = g.psm[m].maxDenDelay;
-        for(uint32_t slot = 0; slot < D; slot++) {
-            lds[T.ldsRing[m] + slot * RES_T + tid] = mine ? asGlobal(g.psm[m].denDelay)[(size_t)slot * n + i] : 0.0f;
+        // (sixteen slots' loads in flight at a time: one at a time, a ring of 43 slots is 43 memory round trips per launch)
+        GLOBAL_AS const float *ring = asGlobal(g.psm[m].denDelay) + (mine ? i : 0u);
+        for(uint32_t slot0 = 0; slot0 < D; slot0 += 16) {
+            float v[16];
+            #pragma unroll
+            for(uint32_t u = 0; u < 16; u++) { v[u] = (mine && slot0 + u < D) ? ring[(size_t)min(slot0 + u, D - 1) * n] : 0.0f; }
+            #pragma unroll
+            for(uint32_t u = 0; u < 16; u++) { if(slot0 + u < D) { lds[T.ldsRing[m] + (slot0 + u) * RES_T + tid] = v[u]; } }
         }
     }
 
