@@ -76,6 +76,7 @@ struct gennmi_runner
     uint32_t resTiles = 0, resReplicaStride = 0, resSeq = 0; size_t resLdsBytes = 0; bool resPoisson = false;
     std::vector<u32x4*> resSegs;        // segment table of each presynaptic group, in push order
     std::vector<uint32_t> resSegTiles;  // tiles of its target population
+    std::vector<u32x2*> resPacked;      // its synapses as the resident kernel reads them
     uint32_t neuronsPerLane = 1;        // 2, 4 or 8: neuronBulkKernel instead of neuronUpdateKernel
     bool sourcesStale = false;          // startSpike / endSpike / spikeTimes of a spike source were written since nextSpikeTime was built
     bool resStale = false;              // connectivity or weights were written since the tables were built
@@ -638,9 +639,22 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
         r->resSegs.push_back(dSeg);
         r->resSegTiles.push_back(tilesInGroup);
         HIP_TRY(hipGetLastError());
+        const size_t padded = (size_t)q.numSrcNeurons * q.rowStride;
+        u32x2 *dPacked = nullptr;
+        if(hipMalloc(&dPacked, std::max<size_t>(padded, 1) * sizeof(u32x2)) != hipSuccess) {
+            (void)hipGetLastError();            // no room for the second copy of the synapses: the network steps with the other plans
+            return GENNMI_OK;
+        }
+        r->owned.push_back(dPacked);
+        if(padded) {
+            residentPackKernel<<<dim3((unsigned int)((padded + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, 0>>>(padded, q.ind, q.g, depth ? q.d : nullptr, dPacked);
+            HIP_TRY(hipGetLastError());
+        }
+        r->resPacked.push_back(dPacked);
         ResProj proj{};
-        proj.ind = q.ind; proj.g = q.g; proj.d = q.d; proj.seg = dSeg;
+        proj.packed = dPacked; proj.seg = dSeg;
         proj.D = (q.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY) ? q.maxDenDelay : 0u;
+        proj.magic = proj.D ? (uint32_t)(0x100000000ull / proj.D) + 1u : 0u;
         proj.srcGroup = (uint32_t)l.src;
         for(uint32_t t = firstTile[l.trg]; t < firstTile[l.trg] + tilesInGroup; t++) {
             proj.lds = proj.D ? tiles[t].ldsRing[l.psm] : tiles[t].ldsIn[l.psm];
@@ -690,6 +704,10 @@ static int launchResident(gennmi_runner *r, unsigned long long timestep, unsigne
             const uint32_t depth = (q.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY) ? q.maxDenDelay : 0u;
             residentSegKernel<<<dim3((unsigned int)((entries + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, r->stream>>>(
                 q.numSrcNeurons, q.rowStride, q.rowLength, q.ind, q.g, q.d, depth, r->resSegTiles[k], r->resSegs[k]);
+            const size_t padded = (size_t)q.numSrcNeurons * q.rowStride;
+            if(padded) {
+                residentPackKernel<<<dim3((unsigned int)((padded + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, r->stream>>>(padded, q.ind, q.g, depth ? q.d : nullptr, r->resPacked[k]);
+            }
         }
         HIP_TRY(hipGetLastError());
     }

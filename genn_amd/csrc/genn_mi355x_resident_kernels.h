@@ -38,11 +38,12 @@ constexpr uint32_t RES_REPLICAS = 8;         // copies of the word array, one pe
 
 struct ResProj
 {
-    const uint32_t *ind; const float *g; const uint8_t *d;
+    const u32x2 *packed;                // one record per (padded) synapse, see residentPackKernel
     const u32x4 *seg;                   // [numSrc * tilesInGroup][2]: the row's part inside a tile, see residentSegKernel
     uint32_t D;                         // ring depth; 0 = no dendritic delay, events add to inSyn
     uint32_t lds;                       // float offset of the ring (D x RES_T, slot-major) or inSyn row in the tile's LDS
-    uint32_t srcGroup, pad_;
+    uint32_t srcGroup;
+    uint32_t magic;                     // floor(2^32 / D) + 1: x % D for x < 2^16 is x - mulhi(x, magic) * D
 };
 
 struct ResTile
@@ -92,6 +93,18 @@ __global__ void residentSegKernel(uint32_t numSrc, uint32_t rowStride, const uin
     hi4.x = w[2]; hi4.y = w[3]; hi4.z = locals; hi4.w = 0;
     seg[2 * id] = lo4;
     seg[2 * id + 1] = hi4;
+}
+
+// The synapses as the row walk reads them: target inside its tile | dendritic delay << 8, and the weight's bits — one
+// 8-byte load per synapse instead of three loads from three arrays (three pages, three cache lines per row part).
+// Same index as the arrays it is made from; padding beyond a row's length is copied as it is and never read.
+__global__ void residentPackKernel(size_t numSynapses, const uint32_t *ind, const float *weight, const uint8_t *delay, u32x2 *packed)
+{
+    const size_t id = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if(id >= numSynapses) { return; }
+    u32x2 rec;
+    rec.x = (ind[id] & (RES_T - 1)) | (delay ? (uint32_t)delay[id] << 8 : 0u); rec.y = __float_as_uint(weight[id]);
+    packed[id] = rec;
 }
 
 // rows must ascend for the segments to be contiguous
@@ -338,54 +351,47 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         }
     };
 
-    // Walks the row segments of the staged pairs, 16 pairs per wavefront at a time, all lanes sharing their synapses.
+    // Walks the row segments of the staged pairs: a group of lanes per pair, a lane taking every n-th synapse of its
+    // pair's segment, eight of them per trip to memory.  Sixteen lanes per pair when the pairs are few (a quiet step: one
+    // trip covers 128 synapses of each of a wavefront's four pairs), four when they are many (a synchronous burst).
+    // (Segments of a tile are short — a row's share of 256 targets — so lanes idle in the longest segment's last trip
+    // cost less than finding, for every lane, its place in a list of all the segments' synapses would.)
     // A synapse is "due" when it lands in the slot read this step (delay a multiple of the ring depth, or no ring).
     // PASS_ALL adds every synapse, PASS_LATER those not due, PASS_DUE the due ones; `flaggedOnly` restricts the walk to
     // segments whose due synapses are not all inline in their entry.
     auto process = [&](uint32_t numPairs, uint32_t pass, bool flaggedOnly) {
-        for(uint32_t q0 = wave * RES_PAIR_GROUP; q0 < numPairs; q0 += (BLOCK / WAVE) * RES_PAIR_GROUP) {
+        constexpr uint32_t TRIP = 8;
+        const uint32_t shift = (numPairs <= 4 * (BLOCK / WAVE)) ? 4u : (numPairs <= 8 * (BLOCK / WAVE)) ? 3u : 2u;
+        const uint32_t lanesPerPair = 1u << shift, pairsPerGroup = WAVE >> shift;
+        for(uint32_t q0 = wave * pairsPerGroup; q0 < numPairs; q0 += (BLOCK / WAVE) * pairsPerGroup) {
+            const uint32_t q = q0 + (lane >> shift);
             uint32_t len = 0, start = 0, proj = 0;
-            if(lane < RES_PAIR_GROUP && q0 + lane < numPairs) {
-                const uint2 sg = shSeg[q0 + lane];
-                proj = shPair[q0 + lane].y;
+            if(q < numPairs) {
+                const uint2 sg = shSeg[q];
+                proj = shPair[q].y;
                 const bool flagged = (sg.y & (RES_SEG_OVERFLOW | RES_SEG_NO_DELAY)) != 0;
                 const bool skip = (flaggedOnly && !flagged) || (pass == PASS_LATER && (sg.y & RES_SEG_NO_DELAY));
                 start = sg.x; len = skip ? 0u : (sg.y & 0xFFFFu);
             }
-            const uint32_t incl = waveInclusiveScanU32(len, lane);
-            const uint32_t sum = __shfl(incl, WAVE - 1, WAVE);
-            for(uint32_t f0 = 0; f0 < sum; f0 += 4 * WAVE) {
-                uint32_t post[4], slotPtr[4], ldsBase[4], depth[4], dly[4]; float w[4]; bool valid[4];
+            const ResProj &P = shProj[proj];
+            const uint32_t depth = P.D, front = shProjPtr[proj], ldsBase = P.lds, magic = P.magic;
+            GLOBAL_AS const u32x2 *packed = asGlobal(P.packed) + start;
+            for(uint32_t i0 = lane & (lanesPerPair - 1); __any(i0 < len); i0 += TRIP * lanesPerPair) {
+                u32x2 rec[TRIP];
                 #pragma unroll
-                for(int u = 0; u < 4; u++) {
-                    const uint32_t f = f0 + u * WAVE + lane;
-                    valid[u] = f < sum;
-                    uint32_t j = 0;
-                    #pragma unroll
-                    for(uint32_t step = RES_PAIR_GROUP / 2; step > 0; step >>= 1) {
-                        const uint32_t v = __shfl(incl, j + step - 1, WAVE);
-                        if(v <= f) { j += step; }
-                    }
-                    const uint32_t lenJ = __shfl(len, j, WAVE), startJ = __shfl(start, j, WAVE), projJ = __shfl(proj, j, WAVE);
-                    const uint32_t inclJ = __shfl(incl, j, WAVE);
-                    post[u] = 0; w[u] = 0.0f; dly[u] = 0; depth[u] = 0; ldsBase[u] = 0; slotPtr[u] = 0;
-                    if(valid[u]) {
-                        const ResProj &P = shProj[projJ];
-                        const uint32_t syn = startJ + (f - (inclJ - lenJ));
-                        post[u] = asGlobal(P.ind)[syn];
-                        w[u] = asGlobal(P.g)[syn];
-                        depth[u] = P.D; ldsBase[u] = P.lds; slotPtr[u] = shProjPtr[projJ];
-                        if(P.D) { dly[u] = asGlobal(P.d)[syn]; }
-                    }
+                for(uint32_t u = 0; u < TRIP; u++) {
+                    const uint32_t i = i0 + u * lanesPerPair;
+                    rec[u].x = 0x80000000u; rec[u].y = 0u;               // (no synapse)
+                    if(i < len) { rec[u] = packed[i]; }
                 }
                 #pragma unroll
-                for(int u = 0; u < 4; u++) {
-                    const uint32_t local = post[u] - T.first;
-                    if(!valid[u] || local >= RES_T) { continue; }
-                    const uint32_t slot = depth[u] ? (slotPtr[u] + dly[u]) % depth[u] : 0u;
-                    const bool due = !depth[u] || (slot == slotPtr[u]);
+                for(uint32_t u = 0; u < TRIP; u++) {
+                    if(rec[u].x >> 31) { continue; }
+                    const uint32_t x = front + (rec[u].x >> 8);              // far below 2^16: the ring fits the LDS, a delay is a byte
+                    const uint32_t slot = depth ? x - __umulhi(x, magic) * depth : 0u;
+                    const bool due = !depth || (slot == front);
                     if((pass == PASS_LATER && due) || (pass == PASS_DUE && !due)) { continue; }
-                    unsafeAtomicAdd(&lds[ldsBase[u] + slot * RES_T + local], w[u]);
+                    unsafeAtomicAdd(&lds[ldsBase + slot * RES_T + (rec[u].x & 0xFFu)], __uint_as_float(rec[u].y));
                 }
             }
         }
