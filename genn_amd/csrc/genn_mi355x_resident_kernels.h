@@ -459,6 +459,24 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         if(numPairs) { process(numPairs, PASS_LATER, false); }
     };
 
+    // What the update reads of its group and tile, once: through the references every step would load it again (the
+    // compiler cannot tell that nobody writes those structures while the kernel runs).
+    float psmInit[GENNMI_MAX_PSM], psmDecay[GENNMI_MAX_PSM], csAmp[GENNMI_MAX_CS], par[8];
+    uint32_t psmKind[GENNMI_MAX_PSM], psmDepth[GENNMI_MAX_PSM], psmIn[GENNMI_MAX_PSM], psmRing[GENNMI_MAX_PSM], csKind[GENNMI_MAX_CS];
+    #pragma unroll
+    for(uint32_t m = 0; m < GENNMI_MAX_PSM; m++) {
+        const bool on = m < numPSM;
+        psmInit[m] = on ? g.psm[m].init : 0.0f; psmDecay[m] = on ? g.psm[m].expDecay : 0.0f;
+        psmKind[m] = on ? g.psm[m].kind : 0u; psmDepth[m] = on ? g.psm[m].maxDenDelay : 0u;
+        psmIn[m] = on ? T.ldsIn[m] : 0u; psmRing[m] = on ? T.ldsRing[m] : 0u;
+    }
+    #pragma unroll
+    for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) { csAmp[c] = (c < numCS) ? g.cs[c].amp : 0.0f; csKind[c] = (c < numCS) ? g.cs[c].kind : 0u; }
+    #pragma unroll
+    for(uint32_t q = 0; q < 8; q++) { par[q] = g.params[q]; }
+    const uint32_t neuronModel = g.model;
+    uint32_t * const recordSpk = g.recordSpk;
+
     // ---- exchange the spikes that precede the first step, then step
     publish(1u, ownCount);
     bool ok = true;
@@ -476,47 +494,47 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             #pragma unroll
             for(uint32_t m = 0; m < GENNMI_MAX_PSM; m++) {
                 if(m < numPSM) {
-                    float linSyn = lds[T.ldsIn[m] + tid];
-                    const uint32_t D = g.psm[m].maxDenDelay;
+                    float linSyn = lds[psmIn[m] + tid];
+                    const uint32_t D = psmDepth[m];
                     if(D) {
-                        const uint32_t front = T.ldsRing[m] + modStep(epoch + 1, D) * RES_T + tid;
+                        const uint32_t front = psmRing[m] + modStep(epoch + 1, D) * RES_T + tid;
                         linSyn += lds[front];
                         lds[front] = 0.0f;
                     }
-                    if(g.psm[m].kind == GENNMI_PSM_EXPCURR) {
-                        Isyn += g.psm[m].init * linSyn;
-                        linSyn *= g.psm[m].expDecay;
+                    if(psmKind[m] == GENNMI_PSM_EXPCURR) {
+                        Isyn += psmInit[m] * linSyn;
+                        linSyn *= psmDecay[m];
                     }
                     else {
                         Isyn += linSyn;
                         linSyn = 0.0f;
                     }
-                    lds[T.ldsIn[m] + tid] = linSyn;
+                    lds[psmIn[m] + tid] = linSyn;
                 }
             }
             #pragma unroll
             for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) {
-                if(c < numCS) { Isyn += (!POISSON || g.cs[c].kind == GENNMI_CS_DC) ? g.cs[c].amp : poissonExpStep(g.cs[c], csState[c], i, epoch); }
+                if(c < numCS) { Isyn += (!POISSON || csKind[c] == GENNMI_CS_DC) ? csAmp[c] : poissonExpStep(g.cs[c], csState[c], i, epoch); }
             }
-            if(g.model == GENNMI_NEURON_LIF) {
+            if(neuronModel == GENNMI_NEURON_LIF) {
                 if(l1 <= 0.0f) {
-                    const float alpha = ((Isyn + g.params[0]) * g.params[1]) + g.params[2];
-                    l0 = alpha - (g.params[3] * (alpha - l0));
+                    const float alpha = ((Isyn + par[0]) * par[1]) + par[2];
+                    l0 = alpha - (par[3] * (alpha - l0));
                 }
                 else {
                     l1 -= dt;
                 }
-                spiked = (l1 <= 0.0f && l0 >= g.params[4]);
-                if(spiked) { l0 = g.params[5]; l1 = g.params[6]; }
+                spiked = (l1 <= 0.0f && l0 >= par[4]);
+                if(spiked) { l0 = par[5]; l1 = par[6]; }
             }
             else {
                 if(l0 >= 30.0f) {
-                    l0 = g.params[2];
-                    l1 += g.params[3];
+                    l0 = par[2];
+                    l1 += par[3];
                 }
                 l0 += 0.5f * (0.04f * l0 * l0 + 5.0f * l0 + 140.0f - l1 + Isyn) * dt;
                 l0 += 0.5f * (0.04f * l0 * l0 + 5.0f * l0 + 140.0f - l1 + Isyn) * dt;
-                l1 += g.params[0] * (g.params[1] * l0 - l1) * dt;
+                l1 += par[0] * (par[1] * l0 - l1) * dt;
                 if(l0 > 30.0f) { l0 = 30.0f; }
                 spiked = (l0 >= 29.99f);
             }
@@ -524,11 +542,11 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         const unsigned long long ballot = __ballot(spiked);
         const uint32_t laneRank = __popcll(ballot & ((1ull << lane) - 1ull));
         if(lane == 0) { shWave[wave] = __popcll(ballot); }
-        if(g.recordSpk && (lane & 31) == 0 && mine) {
+        if(recordSpk && (lane & 31) == 0 && mine) {
             const unsigned long long ts = timestep0 + k;
             const uint32_t recT = numRecordingTimesteps ? (((ts | numRecordingTimesteps) >> 32) ? (uint32_t)(ts % numRecordingTimesteps)
                                                                                                 : ((uint32_t)ts % (uint32_t)numRecordingTimesteps)) : 0u;
-            g.recordSpk[(size_t)recT * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
+            recordSpk[(size_t)recT * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
         }
         __syncthreads();
         uint32_t waveOffset = 0;
