@@ -111,6 +111,27 @@ def test_more_pairs_than_a_tile_stages(depth):
     model.unload()
 
 
+@pytest.mark.parametrize("n_a, ioffset", [(400, 1.0), (24, 0.62), (12, 0.62)])
+def test_long_row_parts_take_several_trips(n_a, ioffset):
+    """Rows of 120 targets inside one tile of 200 neurons: a pair's part is longer than what its group of lanes reads in
+    one trip to memory when many pairs are staged (400 sources crossing threshold together: 4 lanes per pair, 32 synapses
+    per trip), and fits one trip when few are (24 or 12 sources firing now and then: 8 or 16 lanes per pair)."""
+    n_b, depth = 200, 6
+    net = Net(name="resident_long_parts", dt=1.0, steps=0)
+    v0 = np.full(n_a, -50.4) if n_a == 400 else -60.0 + 9.5 * rng.uniform(41, 1, 0, n_a)
+    net.pops.append(_pop("A", n_a, ioffset, v0))
+    net.pops.append(_pop("B", n_b, 0.3, np.full(n_b, -58.0)))
+    net.syns.append(_projection("AB", "A", "B", n_a, n_b, 120, 0.004 if n_a == 400 else 0.05, 42, depth, 0.1))
+    net.steps = 90
+
+    def check(model, oracle):
+        compare_state(net, model, oracle, f"after {model.timestep} steps", exact=True)
+
+    model, oracle, spikes = _run_chunks(net, (30, 60), check)
+    assert spikes > (n_a if n_a == 400 else 20)
+    model.unload()
+
+
 def test_pushed_weights_reach_the_inline_copies(monkeypatch):
     """The segment tables hold copies of the weights of due synapses; a push of `g` between launches must refresh them.
     (With the one-launch-per-step plan the due synapses of the last step's spikes are already in the ring when the push
