@@ -72,8 +72,8 @@ struct gennmi_runner
     // resident plan (many steps per launch)
     bool resident = false;
     ResTile *dResTiles = nullptr; NeuronGroupDev *dResGroups = nullptr; uint8_t *dResTileGroup = nullptr;
-    unsigned long long *dResTags = nullptr; uint32_t *dResSide = nullptr;
-    uint32_t resTiles = 0, resReplicaStride = 0, resSeq = 0; size_t resLdsBytes = 0; bool resPoisson = false;
+    unsigned long long *dResTags = nullptr, *dResSide = nullptr;
+    uint32_t resTiles = 0, resReplicaStride = 0; unsigned long long resSeq = 0; size_t resLdsBytes = 0; bool resPoisson = false;
     std::vector<u32x4*> resSegs;        // segment table of each presynaptic group, in push order
     std::vector<uint32_t> resSegTiles;  // tiles of its target population
     std::vector<u32x2*> resPacked;      // its synapses as the resident kernel reads them
@@ -677,8 +677,10 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
     // cleared once: sequence number 0 is the one no work-group ever waits for before it has come round again
     HIP_TRY(hipMemset(r->dResTags, 0, (size_t)RES_REPLICAS * r->resReplicaStride * sizeof(unsigned long long)));
     r->resSeq = 0;
-    HIP_TRY(hipMalloc(&r->dResSide, 2 * tiles.size() * RES_T * sizeof(uint32_t)));
+    HIP_TRY(hipMalloc(&r->dResSide, 2 * tiles.size() * RES_T * sizeof(unsigned long long)));
     r->owned.push_back(r->dResSide);
+    // (cleared once as well: its entries name their exchange by the unwrapped sequence number, which starts at 1)
+    HIP_TRY(hipMemset(r->dResSide, 0, 2 * tiles.size() * RES_T * sizeof(unsigned long long)));
     r->resTiles = (uint32_t)tiles.size();
     r->resLdsBytes = ldsBytes;
     r->resPoisson = poisson;
@@ -718,7 +720,7 @@ static int launchResident(gennmi_runner *r, unsigned long long timestep, unsigne
             r->dResTiles, r->resTiles, r->dResGroups, r->dResTileGroup, r->dResTags, r->dResSide, timestep + done, r->epoch, numRecordingTimesteps,
             chunk, r->dt, r->fusedStep ? 1u : 0u, r->dError, r->dEvents, r->resReplicaStride, r->resSeq);
         HIP_TRY(hipGetLastError());
-        r->resSeq = (r->resSeq + chunk + 1u) & RES_SEQ_MASK;       // the launch used sequence numbers resSeq + 1 ... resSeq + chunk + 1
+        r->resSeq += chunk + 1u;                                   // the launch used sequence numbers resSeq + 1 ... resSeq + chunk + 1 (words hold them modulo 2^23)
         done += chunk;
         r->epoch += chunk;
     }

@@ -131,10 +131,10 @@ __device__ __forceinline__ uint32_t waveInclusiveScanU32(uint32_t v, uint32_t la
 template<bool POISSON>
 __global__ __launch_bounds__(BLOCK)
 void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const NeuronGroupDev * __restrict__ groups,
-                    const uint8_t * __restrict__ tileGroup, unsigned long long *tags, uint32_t *side,
+                    const uint8_t * __restrict__ tileGroup, unsigned long long *tags, unsigned long long *side,
                     unsigned long long timestep0, unsigned long long epoch0, unsigned long long numRecordingTimesteps, uint32_t numSteps,
                     float dt, uint32_t zeroDelaySplit, uint32_t *errorFlag, unsigned long long *eventCounter, uint32_t replicaStride,
-                    uint32_t seqBase)
+                    unsigned long long seqBase)
 {
     extern __shared__ float lds[];                       // inSyn rows and ring slices of this tile
     __shared__ unsigned long long shTag[RES_MAX_TILES];
@@ -236,17 +236,17 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     // (callers synchronise the work-group after filling shOwn)
     // A word slot is rewritten every second sequence number, and a launch continues the numbering of the one before
     // (seqBase), so a slot never holds the number a reader waits for before its writer has stored it: nothing is cleared
-    // between launches.
+    // between launches.  A tile's spikes beyond those its word holds go through the side buffer, one 64-bit entry each that
+    // says which exchange it belongs to (the unwrapped sequence number, 56 bits, above the tile-local index): entries and
+    // word are stored in any order without a fence, and a reader that finds the word first waits for the entries.
     auto publish = [&](uint32_t step, uint32_t count) {
-        const uint32_t seq = (seqBase + step) & RES_SEQ_MASK;
+        const uint32_t seq = (uint32_t)((seqBase + step) & RES_SEQ_MASK);
         const uint32_t parity = seq & 1u;
         if(count > RES_WORD_IDS) {
             for(uint32_t r = tid; r < count; r += BLOCK) {
-                __hip_atomic_store(&side[((size_t)parity * numTiles + blockIdx.x) * RES_T + r], shOwn[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&side[((size_t)parity * numTiles + blockIdx.x) * RES_T + r], ((seqBase + step) << 8) | (shOwn[r] - T.first),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            // the ids must have reached memory before the word that announces them
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            __syncthreads();
         }
         if(tid < RES_REPLICAS) {
             uint32_t locals = 0;
@@ -271,8 +271,26 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     // Waits for every tile's word of sequence number seq (false when the bounded wait expired somewhere) and stages the
     // (spike, projection) pairs that concern this tile in shPair; shScalar[0] receives their number, which may exceed
     // RES_PAIR_CAP (then only the claims that fitted were written and the caller takes the chunked path).
+    // Entries e0 .. e0 + 7 (below c) of a tile's side list of the exchange `full`: waits, bounded, until each says so
+    auto sideIds = [&](uint32_t tile, uint32_t e0, uint32_t c, unsigned long long full, uint32_t parity, uint32_t (&local)[8]) -> bool {
+        const unsigned long long *base = side + ((size_t)parity * numTiles + tile) * RES_T + e0;
+        const unsigned long long want = full & 0x00FFFFFFFFFFFFFFull;
+        uint32_t need = (c - e0 >= 8) ? 0xFFu : (1u << (c - e0)) - 1u, spins = 0;
+        unsigned long long v[8];
+        while(true) {
+            #pragma unroll
+            for(uint32_t u = 0; u < 8; u++) { v[u] = 0; if(need & (1u << u)) { v[u] = __hip_atomic_load(base + u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); } }
+            #pragma unroll
+            for(uint32_t u = 0; u < 8; u++) {
+                if((need & (1u << u)) && (v[u] >> 8) == want) { local[u] = (uint32_t)v[u] & 0xFFu; need &= ~(1u << u); }
+            }
+            if(!need) { return true; }
+            if(++spins > c_spinLimit) { return false; }
+            __builtin_amdgcn_s_sleep(1);
+        }
+    };
     auto poll = [&](uint32_t step, unsigned long long epoch) -> bool {
-        const uint32_t seq = (seqBase + step) & RES_SEQ_MASK;
+        const uint32_t seq = (uint32_t)((seqBase + step) & RES_SEQ_MASK);
         const uint32_t parity = seq & 1u;
         bool ok = true;
         unsigned long long word[WATCH];
@@ -299,8 +317,9 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         }
         #pragma unroll
         for(uint32_t q = 0; q < WATCH; q++) { if(tid + q * BLOCK < numTiles) { shTag[tid + q * BLOCK] = word[q]; } }
-        const bool allOk = __syncthreads_and(ok ? 1 : 0) != 0;
-        if(!allOk) {
+        if(!ok) { shScalar[3] = 1u; }                  // (zero since the launch began: a launch that finds the error flag raised has left)
+        __syncthreads();
+        if(shScalar[3]) {
             if(tid == 0) { atomicOr(errorFlag, 1u); }
             return false;
         }
@@ -311,17 +330,32 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
             const uint32_t c = (uint32_t)(word[q] >> 32) & 0x1FFu, np = watchNumProj[q];
             if(c == 0 || np == 0) { continue; }
             uint32_t pos = atomicAdd(&shScalar[0], c * np);
-            if(pos + c * np > RES_PAIR_CAP) { continue; }
-            // ids beyond those inside the word were stored before a release fence and the word after it (publish): the
-            // reads below must not be served ahead of the word's load
-            if(c > RES_WORD_IDS) { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
-            for(uint32_t e = 0; e < c; e++) {
-                const uint32_t id = (c <= RES_WORD_IDS) ? watchFirst[q] + (((uint32_t)word[q] >> (8 * e)) & 0xFFu)
-                                                        : __hip_atomic_load(&side[((size_t)parity * numTiles + tid + q * BLOCK) * RES_T + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                for(uint32_t j = 0; j < np; j++) { shPair[pos++] = make_uint2(id, shProjIdx[watchProj0[q] + j]); }
+            const bool fits = pos + c * np <= RES_PAIR_CAP;
+            if(c <= RES_WORD_IDS) {
+                for(uint32_t e = 0; fits && e < c; e++) {
+                    const uint32_t id = watchFirst[q] + (((uint32_t)word[q] >> (8 * e)) & 0xFFu);
+                    for(uint32_t j = 0; j < np; j++) { shPair[pos++] = make_uint2(id, shProjIdx[watchProj0[q] + j]); }
+                }
+                continue;
+            }
+            // a longer list: its entries, eight loads at a time (also when the pairs do not fit and the chunked walk will
+            // read the list again: once seen here, an entry is there for every later read of this work-group)
+            for(uint32_t e0 = 0; e0 < c && ok; e0 += 8) {
+                uint32_t local[8];
+                if(!sideIds(tid + q * BLOCK, e0, c, seqBase + step, parity, local)) { ok = false; break; }
+                #pragma unroll
+                for(uint32_t u = 0; u < 8; u++) {
+                    if(!fits || e0 + u >= c) { continue; }
+                    for(uint32_t j = 0; j < np; j++) { shPair[pos++] = make_uint2(watchFirst[q] + local[u], shProjIdx[watchProj0[q] + j]); }
+                }
             }
         }
+        if(!ok) { shScalar[3] = 1u; }
         __syncthreads();
+        if(shScalar[3]) {
+            if(tid == 0) { atomicOr(errorFlag, 1u); }
+            return false;
+        }
         return true;
     };
 
@@ -421,10 +455,9 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
                 const uint32_t p0 = shProjStart[s], np = shProjStart[s + 1] - p0;
                 if(c == 0 || np == 0) { continue; }
                 if(pos + c * np <= chunk0 || pos >= chunk0 + RES_PAIR_CAP) { pos += c * np; continue; }
-                if(c > RES_WORD_IDS) { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }     // as in poll()
                 for(uint32_t q = 0; q < c; q++) {
                     const uint32_t id = (c <= RES_WORD_IDS) ? tiles[k].first + (((uint32_t)tag >> (8 * q)) & 0xFFu)
-                                                            : __hip_atomic_load(&side[((size_t)parity * numTiles + k) * RES_T + q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                                            : tiles[k].first + ((uint32_t)__hip_atomic_load(&side[((size_t)parity * numTiles + k) * RES_T + q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xFFu);
                     for(uint32_t j = 0; j < np; j++, pos++) {
                         if(pos >= chunk0 && pos < chunk0 + RES_PAIR_CAP) { shPair[pos - chunk0] = make_uint2(id, shProjIdx[p0 + j]); }
                     }
@@ -451,7 +484,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         }
         readSegments(total, convention == PASS_LATER, convention != PASS_DUE);
         __syncthreads();
-        if(convention != PASS_LATER && shFlagged) { process(total, PASS_DUE, true); }
+        if(convention != PASS_LATER && shFlagged) { process(total, PASS_DUE, true); __syncthreads(); }
         return (convention == PASS_DUE) ? 0u : total;
     };
     // the rest of those pairs' synapses: none of them is read before the next step
@@ -484,8 +517,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     for(; k < numSteps; k++) {
         const unsigned long long epoch = epoch0 + k;
         if(!poll(k + 1, epoch)) { ok = false; break; }
-        const uint32_t later = deliverDue(k + 1, (zeroDelaySplit && k == 0) ? PASS_LATER : PASS_ALL);
-        __syncthreads();
+        const uint32_t later = deliverDue(k + 1, (zeroDelaySplit && k == 0) ? PASS_LATER : PASS_ALL);     // (ends with a barrier)
 
         // neuron update: same operations in the same order as neuronBody
         bool spiked = false;
