@@ -31,8 +31,8 @@ BYTES_PER_EVENT = {"dense": 4,          # one weight read per (spike, target); o
 # is only attached to a run of the very command line it was measured on (same workload, steps and warm-up: the network,
 # its seed and therefore its activity are then identical); any other run reports null.
 MEASURED_TRAFFIC_BYTES = {
-    ("potjans", 20, 5): {"plan": "resident", "bytes_per_launch": 155344224,
-                         "source": "rocprofv3 --pmc FETCH_SIZE (67756.38 x 2 KiB) + WRITE_SIZE (16190.59 x 1 KiB) of the timed 20-step "
+    ("potjans", 20, 5): {"plan": "resident", "bytes_per_launch": 155544259,
+                         "source": "rocprofv3 --pmc FETCH_SIZE (67852.50 x 2 KiB) + WRITE_SIZE (16193.69 x 1 KiB) of the timed 20-step "
                                    "launch, profiles/residentKernel_potjans_full.md"},
 }
 
