@@ -390,7 +390,9 @@ int gennmi_runner_stream_mark(gennmi_runner *runner, int which);
 int gennmi_runner_stream_elapsed(gennmi_runner *runner, double *seconds);
 /* Launch plan chosen by gennmi_runner_finalise: bit 1 of info[0] is set if gennmi_run_steps keeps the network resident on
  * the chip (many steps per launch: batch 1, static SPARSE projections with ascending rows between LIF / Izhikevich
- * populations, all tiles of 256 neurons resident at once; GENNMI_RESIDENT=0 disables it); bit 0 if a whole timestep is one launch (all projections go
+ * populations, all tiles of 256 neurons resident at once, and room in device memory for a per-(row, tile) table of 32 bytes
+ * per entry and a second, 8-byte-per-synapse copy of the projections, both kept up to date with writes made through this
+ * library; GENNMI_RESIDENT=0 disables it); bit 0 if a whole timestep is one launch (all projections go
  * through a dendritic-delay ring; synapses with d % D == 0 are then delivered by the spiking neuron one launch
  * earlier, into the slot read in the next step — the visible difference is the content of that one ring slot
  * between steps; GENNMI_FUSED_STEP=0 in the environment keeps the reference's placement); bit 2 if the neuron update
