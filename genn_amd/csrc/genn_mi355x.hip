@@ -475,7 +475,12 @@ int gennmi_push_presynaptic_update_group(gennmi_runner *r, const gennmi_presynap
     d.g = *g;
     if(g->matrix == GENNMI_MATRIX_SPARSE) {
         if(!g->rowLength || !g->ind || g->rowStride == 0) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: sparse arrays missing"); }
-        if((uint64_t)g->numSrcNeurons * g->rowStride > 0xFFFFFFFFull) { return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: synapse index exceeds 32 bits"); }
+        // Synapse ids beyond 32 bits (backendBase.cc:503-522 switches the index type at numPre * rowStride > 2^32 - 1): the scatter
+        // and tile paths of a static projection index rows in 64 bits throughout; the views other rules need (column remap,
+        // zero-delay lists, segment tables of the resident plan) hold 32-bit ids
+        if((uint64_t)g->numSrcNeurons * g->rowStride > 0xFFFFFFFFull && g->wum != GENNMI_WUM_STATIC_PULSE) {
+            return fail(GENNMI_EUNSUPPORTED, "push_presynaptic_update_group: synapse index exceeds 32 bits (supported for static projections without delay only)");
+        }
         if(g->wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY) {
             if(!g->d || !g->denDelay || g->maxDenDelay == 0) { return fail(GENNMI_EINVAL, "push_presynaptic_update_group: dendritic delay arrays missing"); }
         }
@@ -853,6 +858,7 @@ static int buildOrderedViews(gennmi_runner *r)
         p.ordered = covered ? 1u : 0u;
         if(!covered) { continue; }
         if(g.maxDenDelay > ORDERED_MAX_SLOT_REGS * WAVE) { return fail(GENNMI_EUNSUPPORTED, "ordered accumulation: dendritic-delay rings of more than 256 slots"); }
+        if((uint64_t)g.numSrcNeurons * g.rowStride > 0xFFFFFFFFull) { return fail(GENNMI_EUNSUPPORTED, "ordered accumulation: synapse index exceeds 32 bits (the column view holds 32-bit ids)"); }
         uint32_t maxLen = 0;
         { const int rc = gennmi_max_col_length(g.numSrcNeurons, g.numTrgNeurons, g.rowStride, g.rowLength, g.ind, &maxLen); if(rc) { return rc; } }
         OrderedGroupDev o{};

@@ -184,6 +184,16 @@ class Array:
             _abi.check(_abi.load().gennmi_memcpy_from_device(self.view.ctypes.data_as(C.c_void_p), self._dev, self.view.nbytes))
         return self.view
 
+    def pull_slice(self, first, count):
+        """Elements first .. first + count - 1 from the device, as a new array (for arrays too large to mirror on the host)."""
+        first, count = int(first), int(count)
+        if first < 0 or count < 0 or first + count > self.count:
+            raise IndexError("slice outside the array")
+        out = np.empty(count, dtype=self.dtype)
+        if count:
+            _abi.check(_abi.load().gennmi_memcpy_from_device(out.ctypes.data_as(C.c_void_p), C.c_void_p(self._dev.value + first * self.dtype.itemsize), out.nbytes))
+        return out
+
     def init_on_device(self, init, seed, stream, dt):
         """Fill from a value snippet (gennmi_init_var); the host copy is not touched."""
         params = (C.c_double * 4)(*init.values(dt))
