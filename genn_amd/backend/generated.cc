@@ -89,7 +89,8 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                                        HostHandler preambleHandler) const
 {
     const ModelSpecInternal &model = modelMerged.getModel();
-    if(model.getBatchSize() != 1) { notGenerated("batch sizes above 1"); }
+    // batches: the grid's second dimension (backendCUDAHIP.cc:332-338 does the same); every batch compacts its own queue
+    const unsigned int batchSize = model.getBatchSize();
     if(model.getPrecision() != Type::Float || model.getTimePrecision() != Type::Float) { notGenerated("double precision"); }
     const bool recording = model.isRecordingInUse();
 
@@ -101,7 +102,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     {   // (environments write what they hold when they go out of scope: the kernel's text is complete after this block)
     EnvironmentExternal funcEnv(kernelEnv);
     funcEnv.add(model.getTimePrecision().addConst(), "t", "t");
-    funcEnv.add(Type::Uint32.addConst(), "batch", "0");
+    funcEnv.add(Type::Uint32.addConst(), "batch", (batchSize > 1) ? "blockIdx.y" : "0");
     funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
 
     modelMerged.genMergedNeuronUpdateGroups(
@@ -135,8 +136,10 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             funcEnv.getStream() << "bool gennmiSpiked = false;" << std::endl;
 
             EnvironmentGroupMergedField<NeuronUpdateGroupMerged> groupEnv(funcEnv, n);
-            buildStandardEnvironment(groupEnv, 1);
+            buildStandardEnvironment(groupEnv, batchSize);
             groupEnv.add(Type::Uint32.addConst(), "id", "id");
+            // where a batch's entries of a per-neuron array (spike queue, spike times) begin
+            const std::string queueOffset = n.getWriteVarIndex(false, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "");
             if(arch.isSpikeRecordingEnabled()) {
                 groupEnv.printLine("const unsigned int numRecordingWords = ($(num_neurons) + 31) / 32;");
             }
@@ -144,31 +147,33 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             {
                 CodeStream::Scope b2(groupEnv.getStream());
                 n.generateNeuronUpdate(
-                    groupEnv, 1,
+                    groupEnv, batchSize,
                     // a true spike: weight-update pre / post spike code, spike time; the queue is written after the
                     // population's flags have been compacted (below), the recording word comes from the ballot
-                    [&n, &arch](EnvironmentExternalBase &env)
+                    [&n, &arch, &queueOffset, batchSize](EnvironmentExternalBase &env)
                     {
-                        n.generateWUVarUpdate(env, 1);
-                        if(arch.isSpikeTimeRequired()) { env.printLine("$(_st)[$(id)] = $(t);"); }
+                        n.generateWUVarUpdate(env, batchSize);
+                        if(arch.isSpikeTimeRequired()) { env.printLine("$(_st)[" + queueOffset + "$(id)] = $(t);"); }
                         env.getStream() << "gennmiSpiked = true;" << std::endl;
                     },
                     [](EnvironmentExternalBase&, NeuronUpdateGroupMerged::SynSpikeEvent&) {});
             }
             groupEnv.printLine("const gennmi_kernel::QueueSlot slot = gennmi_kernel::orderedSlot(gennmiSpiked, entry.blockInGroup, entry.blocksInGroup, "
-                               "blockIdx.x - entry.blockInGroup, gennmiAgg, gennmiAgg + gridDim.x, gennmiTag, gennmiError);");
+                               "blockIdx.x - entry.blockInGroup, gennmiAgg + (size_t)2 * gridDim.x * blockIdx.y, gennmiAgg + (size_t)2 * gridDim.x * blockIdx.y + gridDim.x, "
+                               "gennmiTag, gennmiError);");
             if(arch.isSpikeRecordingEnabled()) {
-                groupEnv.printLine("gennmi_kernel::recordBallot(&$(_record_spk)[recordingTimestep * numRecordingWords], $(id), $(id) < $(num_neurons), slot.ballot);");
+                groupEnv.printLine("gennmi_kernel::recordBallot(&$(_record_spk)[((size_t)recordingTimestep * " + std::to_string(batchSize) + "u + $(batch)) * numRecordingWords], "
+                                   "$(id), $(id) < $(num_neurons), slot.ballot);");
             }
             // every spike queue of the population (one per fused outgoing / incoming spike target) from the same positions
             n.generateSpikes(
                 groupEnv,
-                [](EnvironmentExternalBase &env)
+                [&queueOffset](EnvironmentExternalBase &env)
                 {
                     env.print("if(slot.ok)");
                     CodeStream::Scope b3(env.getStream());
-                    env.printLine("if(gennmiSpiked) { $(_spk)[slot.position] = $(id); }");
-                    env.printLine("if(slot.writeTotal) { $(_spk_cnt)[0] = slot.total; }");
+                    env.printLine("if(gennmiSpiked) { $(_spk)[" + queueOffset + "slot.position] = $(id); }");
+                    env.printLine("if(slot.writeTotal) { $(_spk_cnt)[$(batch)] = slot.total; }");
                 });
         });
     }
@@ -195,8 +200,8 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         {
             CodeStream::Scope b2(os);
             os << "void *p = nullptr;" << std::endl;
-            os << "GENNMI_CHECK(gennmi_malloc(&p, " << 2 * std::max<size_t>(1, table.numBlocks) << " * sizeof(unsigned long long)));" << std::endl;
-            os << "GENNMI_CHECK(gennmi_memset(p, 0, " << 2 * std::max<size_t>(1, table.numBlocks) << " * sizeof(unsigned long long)));" << std::endl;
+            os << "GENNMI_CHECK(gennmi_malloc(&p, " << 2 * std::max<size_t>(1, table.numBlocks) * batchSize << " * sizeof(unsigned long long)));" << std::endl;
+            os << "GENNMI_CHECK(gennmi_memset(p, 0, " << 2 * std::max<size_t>(1, table.numBlocks) * batchSize << " * sizeof(unsigned long long)));" << std::endl;
             os << "gennmiNeuronAgg = (unsigned long long*)p;" << std::endl;
             os << "GENNMI_CHECK(gennmi_malloc(&p, sizeof(uint32_t)));" << std::endl;
             os << "GENNMI_CHECK(gennmi_memset(p, 0, sizeof(uint32_t)));" << std::endl;
@@ -220,7 +225,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         if(table.numBlocks > 0) {
             // the tag of a launch: differs from one launch to the next, never 0 (the look-back words start out zero)
             os << "gennmiNeuronLaunches = (gennmiNeuronLaunches == 0xFFFFFFFFu) ? 1u : gennmiNeuronLaunches + 1u;" << std::endl;
-            os << "gennmiNeuronUpdateKernel<<<dim3(" << table.numBlocks << "), dim3(256), 0, 0>>>(t, " << (recording ? "recordingTimestep" : "0u")
+            os << "gennmiNeuronUpdateKernel<<<dim3(" << table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t, " << (recording ? "recordingTimestep" : "0u")
                << ", gennmiNeuronLaunches, gennmiNeuronAgg, gennmiNeuronError" << argStream.str() << ");" << std::endl;
             os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateNeurons: kernel launch failed\"); }" << std::endl;
         }
@@ -242,6 +247,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
 {
     const ModelSpecInternal &model = modelMerged.getModel();
     const double dt = model.getDT();
+    const unsigned int batchSize = model.getBatchSize();
 
     std::ostringstream declStream, uploadStream;
     CodeStream decl(declStream), upload(uploadStream);
@@ -257,7 +263,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
     {
         EnvironmentExternal funcEnv(lib);
         funcEnv.add(model.getTimePrecision().addConst(), "t", "t");
-        funcEnv.add(Type::Uint32.addConst(), "batch", "0");
+        funcEnv.add(Type::Uint32.addConst(), "batch", (model.getBatchSize() > 1) ? "blockIdx.y" : "0");
         funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
         (void)stream;
         use(funcEnv);
@@ -331,8 +337,9 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     funcEnv.getStream() << "const gennmi_kernel::BlockEntry entry = gennmiPresynapticBlocks[blockIdx.x];" << std::endl;
                     funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
                     EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> groupEnv(funcEnv, s);
-                    buildStandardEnvironment(groupEnv, 1);
-                    groupEnv.printLine("const unsigned int numSpikes = $(_src_spk_cnt)[0];");
+                    buildStandardEnvironment(groupEnv, batchSize);
+                    const std::string preOffset = (batchSize > 1) ? "$(_pre_batch_offset) + " : "";
+                    groupEnv.printLine("const unsigned int numSpikes = $(_src_spk_cnt)[$(batch)];");
                     groupEnv.printLine(std::string("const unsigned int rowSpan = ") + (sparse ? "$(_row_stride)" : "$(num_post)") + ";");
                     groupEnv.getStream() << "const unsigned int chunksPerRow = (rowSpan + 63u) / 64u;" << std::endl;
                     groupEnv.getStream() << "const unsigned int numWaves = entry.blocksInGroup * 4u;" << std::endl;
@@ -343,7 +350,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> synEnv(groupEnv, s);
                         synEnv.getStream() << "const unsigned int spike = (unsigned int)(item / chunksPerRow);" << std::endl;
                         synEnv.getStream() << "const unsigned int j = (unsigned int)(item % chunksPerRow) * 64u + (threadIdx.x & 63u);" << std::endl;
-                        synEnv.printLine("const unsigned int idPre = $(_src_spk)[spike];");
+                        synEnv.printLine("const unsigned int idPre = $(_src_spk)[" + preOffset + "spike];");
                         synEnv.add(Type::Uint32.addConst(), "id_pre", "idPre");
                         const auto indexType = getSynapseIndexType(s);
                         const std::string indexTypeName = indexType.getName();
@@ -368,12 +375,12 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                                             {codeEnv.addInitialiser("const " + indexTypeName + " idSyn = ((" + indexTypeName + ")idPre * $(num_post)) + j;")});
                             }
                             codeEnv.add(Type::getAddToPrePostDelay(s.getScalarType()), "addToPostDelay",
-                                        "gennmi_kernel::addScalar(&$(_den_delay)[" + s.getPostDenDelayIndex(1, "$(id_post)", "$(1)") + "], $(0))");
+                                        "gennmi_kernel::addScalar(&$(_den_delay)[" + s.getPostDenDelayIndex(batchSize, "$(id_post)", "$(1)") + "], $(0))");
                             codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPost",
-                                        "gennmi_kernel::addScalar(&$(_out_post)[" + s.getPostISynIndex(1, "$(id_post)") + "], $(0))");
+                                        "gennmi_kernel::addScalar(&$(_out_post)[" + s.getPostISynIndex(batchSize, "$(id_post)") + "], $(0))");
                             codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
-                                        "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(1, "$(id_pre)") + "], $(0))");
-                            s.generateSpikeUpdate(*this, codeEnv, 1, dt);
+                                        "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(batchSize, "$(id_pre)") + "], $(0))");
+                            s.generateSpikeUpdate(*this, codeEnv, batchSize, dt);
                         }
                     }
                 });
@@ -416,8 +423,9 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     funcEnv.getStream() << "const gennmi_kernel::BlockEntry entry = gennmiPostsynapticBlocks[blockIdx.x];" << std::endl;
                     funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
                     EnvironmentGroupMergedField<PostsynapticUpdateGroupMerged> groupEnv(funcEnv, s);
-                    buildStandardEnvironment(groupEnv, 1);
-                    groupEnv.printLine("const unsigned int numSpikes = $(_trg_spk_cnt)[0];");
+                    buildStandardEnvironment(groupEnv, batchSize);
+                    const std::string postOffset = (batchSize > 1) ? "$(_post_batch_offset) + " : "";
+                    groupEnv.printLine("const unsigned int numSpikes = $(_trg_spk_cnt)[$(batch)];");
                     groupEnv.printLine(std::string("const unsigned int colSpan = ") + (sparse ? "$(_col_stride)" : "$(num_pre)") + ";");
                     groupEnv.getStream() << "const unsigned int chunksPerCol = (colSpan + 63u) / 64u;" << std::endl;
                     groupEnv.getStream() << "const unsigned int numWaves = entry.blocksInGroup * 4u;" << std::endl;
@@ -426,7 +434,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     {
                         CodeStream::Scope b2(groupEnv.getStream());
                         EnvironmentGroupMergedField<PostsynapticUpdateGroupMerged> synEnv(groupEnv, s);
-                        synEnv.printLine("const unsigned int spike = $(_trg_spk)[(unsigned int)(item / chunksPerCol)];");
+                        synEnv.printLine("const unsigned int spike = $(_trg_spk)[" + postOffset + "(unsigned int)(item / chunksPerCol)];");
                         synEnv.getStream() << "const unsigned int i = (unsigned int)(item % chunksPerCol) * 64u + (threadIdx.x & 63u);" << std::endl;
                         if(sparse) {
                             synEnv.print("if(i < $(_col_length)[spike])");
@@ -451,8 +459,8 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                             }
                             codeEnv.add(Type::Uint32.addConst(), "id_post", "spike");
                             codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
-                                        "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(1, "$(id_pre)") + "], $(0))");
-                            s.generateSpikeUpdate(*this, codeEnv, 1, dt);
+                                        "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(batchSize, "$(id_pre)") + "], $(0))");
+                            s.generateSpikeUpdate(*this, codeEnv, batchSize, dt);
                         }
                     }
                 });
@@ -504,8 +512,8 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         os << "gennmiEnsureFinalised();" << std::endl;
         // order of the reference's updateSynapses (backendCUDAHIP.cc:548-589): ring pointers, presynaptic, postsynaptic
         if(anyDelay) { os << "gennmiDendriticDelayUpdateKernel<<<dim3(1), dim3(64), 0, 0>>>(t" << delay.args.str() << ");" << std::endl; }
-        if(anyPre) { os << "gennmiPresynapticUpdateKernel<<<dim3(" << pre.table.numBlocks << "), dim3(256), 0, 0>>>(t" << pre.args.str() << ");" << std::endl; }
-        if(anyPost) { os << "gennmiPostsynapticUpdateKernel<<<dim3(" << post.table.numBlocks << "), dim3(256), 0, 0>>>(t" << post.args.str() << ");" << std::endl; }
+        if(anyPre) { os << "gennmiPresynapticUpdateKernel<<<dim3(" << pre.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << pre.args.str() << ");" << std::endl; }
+        if(anyPost) { os << "gennmiPostsynapticUpdateKernel<<<dim3(" << post.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << post.args.str() << ");" << std::endl; }
         os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateSynapses: kernel launch failed\"); }" << std::endl;
     }
 }

@@ -575,7 +575,7 @@ int main(int argc, char *argv[])
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
                     for(const char *var : {"wPre", "wPost"}) {
                         auto *a = pulled(rt.getArray(*s.sg, var));
-                        for(size_t i = 0; i < numPre; i++) { appendFile(out + "/" + s.name + "." + var + ".f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
+                        for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + "." + var + ".f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
                     }
                     for(const char *var : {"sPre", "sPost"}) {
                         auto *a = pulled(rt.getArray(*s.sg, var));

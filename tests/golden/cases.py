@@ -51,6 +51,19 @@ def custom_small():
     return configs.custom_models(), 25
 
 
+def custom_batch1_small():
+    # custom_small from other initial values (same matrices): what the second batch of a batched run of custom_small
+    # starts from.  The reference's CPU backend has no batches, so every batch of that run is pinned by a run of its own.
+    import numpy as np
+    from genn_amd import rng
+    net, snap = custom_small()
+    net.name = "custom_batch1"
+    for k, p in enumerate(net.pops):
+        p.vars["V"] = (-60.0 + 9.5 * rng.uniform(net.seed, 61 + k, 0, p.n)).astype(np.float32)
+        p.vars["A"] = (0.1 * rng.uniform(net.seed, 65 + k, 0, p.n)).astype(np.float32)
+    return net, snap
+
+
 def dynamic_small():
     # parameters changed while the model runs (setParamDynamic + Runtime::setDynamicParamValue): the drive of the
     # excitatory population twice, the threshold of the inhibitory one, and the time constant of a postsynaptic model, whose
@@ -70,7 +83,7 @@ def potjans_poisson_net():
 
 # cases the reference's CPU backend pins directly (fixtures) and that the oracle, a restatement of the built-in models
 # with fixed parameters, does not cover
-REFERENCE_ONLY = {"custom_small", "dynamic_small"}
+REFERENCE_ONLY = {"custom_small", "custom_batch1_small", "dynamic_small"}
 
-CASES = {"custom_small": custom_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+CASES = {"custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
          "stdp_small": stdp_small, "conv_small": conv_small}

@@ -189,6 +189,34 @@ def test_generated_kernels_are_chosen_and_build(case, options):
         shutil.rmtree(tmp, ignore_errors=True)
 
 
+def test_generated_kernels_take_the_batch_from_the_grid():
+    """A batched model on generated kernels: the launches have the batch as the grid's second dimension and the kernels
+    index neuron variables, spike queues, recording words and per-synapse variables by it (GeNN's own index helpers)."""
+    import numpy as np
+    net, snap = CASES["custom_small"]()
+    net.snap = snap
+    net.batch_size = 2
+    for p in net.pops:
+        p.vars = {v: np.stack([a, a]) for v, a in p.vars.items()}
+    tmp = tempfile.mkdtemp(prefix="adapter_genk_batch_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(net, spec)
+        res = subprocess.run([DRIVER, spec, work, out, "--generate-only"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        assert res.returncode == 0, res.stdout[-3000:]
+        code = os.path.join(work, net.name + "_CODE")
+        neuron = open(os.path.join(code, "neuronUpdate.cc")).read()
+        synapse = open(os.path.join(code, "synapseUpdate.cc")).read()
+        assert "<<<dim3(" in neuron and ", 2), dim3(256)" in neuron and ", 2), dim3(256)" in synapse
+        assert "group->A[batchOffset + id]" in neuron and "[blockIdx.y] = slot.total" in neuron
+        assert "(size_t)recordingTimestep * 2u + blockIdx.y" in neuron
+        assert "group->srcSpk[preBatchOffset + spike]" in synapse and "group->wPost[synBatchOffset + idSyn]" in synapse
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
 @pytest.mark.parametrize("case, what", [("va_delay_small", "delay"), ("conv_small", "connectivity"), ("graded_small", "spike-like")])
 def test_generated_kernels_say_what_they_do_not_cover(case, what):
     """Asked to generate kernels for a feature only the device library implements, the backend names the feature."""

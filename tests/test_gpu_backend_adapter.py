@@ -283,6 +283,61 @@ def test_adapter_batched_plastic_network():
         shutil.rmtree(tmp, ignore_errors=True)
 
 
+def test_generated_kernels_with_batches():
+    """Batch size 2 for models only the generated kernels cover (`custom_small`: a neuron with an extra state variable, a
+    weight-update model with presynaptic, postsynaptic and per-synapse variables): the batch is the grid's second
+    dimension, every batch compacts its own spike queue, and GeNN's own index helpers place variables by their batch
+    dimension.  The reference's CPU backend has no batches, so batch b is pinned by that backend's run from batch b's
+    initial values (fixtures `custom_small` and `custom_batch1_small`): rasters identical, spike times copied through the
+    weight-update variables exact, state within 1e-5."""
+    import copy
+    B = 2
+    cases = ("custom_small", "custom_batch1_small")
+    nets, snap = [], None
+    for case in cases:
+        net, snap = CASES[case]()
+        nets.append(net)
+    batched = copy.deepcopy(nets[0])
+    for p in batched.pops:
+        p.vars = {v: np.stack([n.pop(p.name).vars[v] for n in nets]) for v in p.vars}
+    batched.batch_size = B
+    batched.snap = snap
+    tmp = tempfile.mkdtemp(prefix="adapter_batch_generated_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(batched, spec)
+        print(f"adapter batched generated kernels: running {DRIVER}", flush=True)
+        res = subprocess.run([DRIVER, spec, work, out], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+        assert res.returncode == 0, res.stdout[-3000:]
+        assert "__global__" in open(os.path.join(work, batched.name + "_CODE", "neuronUpdate.cc")).read()
+        snaps = batched.steps // snap
+        for b, case in enumerate(cases):
+            golden = np.load(os.path.join(HERE, "golden", case + ".npz"))
+            assert str(golden["input_digest"]) == nets[b].input_digest(), "generator output changed since the fixture was made"
+            spikes = 0
+            for p in batched.pops:
+                got = np.fromfile(os.path.join(out, f"{p.name}.spikes{'.b%d' % b if b else ''}.u32"), np.uint32).reshape(-1, 2)
+                want = golden[f"spikes.{p.name}"]
+                assert np.array_equal(got, want), f"batch {b}: raster of {p.name} differs ({len(got)} vs {len(want)} spikes)"
+                spikes += len(want)
+                for var in ("V", "RefracTime", "A"):
+                    g = np.fromfile(os.path.join(out, f"{p.name}.{var}.f32"), np.float32).reshape(snaps, B, p.n)[:, b]
+                    _close(g, golden[f"{var}.{p.name}"], f"batch {b}: {var}.{p.name}")
+            assert spikes > 500
+            for s in batched.syns:
+                for var in ("sPre", "sPost", "wPre", "wPost"):
+                    key = f"{var}.{s.name}"
+                    if key in golden:
+                        got = np.fromfile(os.path.join(out, f"{s.name}.{var}.f32"), np.float32).reshape(snaps, B, -1)[:, b]
+                        assert np.array_equal(got, golden[key]), f"batch {b}: {key}"
+                got = np.fromfile(os.path.join(out, f"{s.name}.outPost.f32"), np.float32).reshape(snaps, B, -1)[:, b]
+                _close(got, golden[f"outPost.{s.name}"], f"batch {b}: outPost.{s.name}", accumulator=True)
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
 def test_adapter_device_initialisation_matches_host_layer():
     """Preferences::deviceInitialisation through GeNN's generator and Runtime: SPARSE matrices built by FixedProbability
     (with and without autapses) and FixedNumberPostWithReplacement with Uniform, Normal, Constant and constant-parameter
