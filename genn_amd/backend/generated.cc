@@ -80,6 +80,16 @@ void genDeviceStructArray(CodeStream &decl, CodeStream &upload, const BackendBas
         upload << "GENNMI_CHECK(gennmi_memcpy_to_device(" << dev << ", staging, sizeof(staging)));" << std::endl;
     }
 }
+// gennrand_* as the reference's backends declare them (cuda/backend.cc:35-43), over gennmi_kernel::Rng
+const EnvironmentLibrary::Library simRNGFunctions = {
+    {"gennrand", {Type::ResolvedType::createFunction(Type::Uint32, {}), "gennmi_kernel::rngWord($(_rng))"}},
+    {"gennrand_uniform", {Type::ResolvedType::createFunction(Type::Float, {}), "gennmi_kernel::rngUniform($(_rng))"}},
+    {"gennrand_normal", {Type::ResolvedType::createFunction(Type::Float, {}), "gennmi_kernel::rngNormal($(_rng))"}},
+    {"gennrand_exponential", {Type::ResolvedType::createFunction(Type::Float, {}), "gennmi_kernel::rngExponential($(_rng))"}},
+    {"gennrand_log_normal", {Type::ResolvedType::createFunction(Type::Float, {Type::Float, Type::Float}), "gennmi_kernel::rngLogNormal($(_rng), $(0), $(1))"}},
+    {"gennrand_gamma", {Type::ResolvedType::createFunction(Type::Float, {Type::Float}), "gennmi_kernel::rngGamma($(_rng), $(0))"}},
+    {"gennrand_binomial", {Type::ResolvedType::createFunction(Type::Uint32, {Type::Uint32, Type::Float}), "gennmi_kernel::rngBinomial($(_rng), $(0), $(1))"}},
+};
 }   // anonymous namespace
 
 namespace GeNN::CodeGenerator::MI355X
@@ -99,8 +109,12 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     BlockTable table;
 
     EnvironmentLibrary kernelEnv(kernel, StandardLibrary::getMathsFunctions());
+    bool anyRNG = false;
     {   // (environments write what they hold when they go out of scope: the kernel's text is complete after this block)
-    EnvironmentExternal funcEnv(kernelEnv);
+    // gennrand_* of simulation code: words of a counter-based generator, see gennmi_kernel::Rng (`_rng` exists in the
+    // populations that need it)
+    EnvironmentLibrary rngEnv(kernelEnv, simRNGFunctions);
+    EnvironmentExternal funcEnv(rngEnv);
     funcEnv.add(model.getTimePrecision().addConst(), "t", "t");
     funcEnv.add(Type::Uint32.addConst(), "batch", (batchSize > 1) ? "blockIdx.y" : "0");
     funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
@@ -111,7 +125,6 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         {
             const auto &arch = n.getArchetype();
             if(arch.isDelayRequired()) { notGenerated("axonal delay slots (population '" + arch.getName() + "')"); }
-            if(arch.isSimRNGRequired()) { notGenerated("random numbers in the update of population '" + arch.getName() + "'"); }
             if(arch.isPrevSpikeTimeRequired() || arch.isSpikeEventTimeRequired() || arch.isPrevSpikeEventTimeRequired()) {
                 notGenerated("previous spike times and spike-like event times (population '" + arch.getName() + "')");
             }
@@ -140,6 +153,18 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             groupEnv.add(Type::Uint32.addConst(), "id", "id");
             // where a batch's entries of a per-neuron array (spike queue, spike times) begin
             const std::string queueOffset = n.getWriteVarIndex(false, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "");
+            if(arch.isSimRNGRequired()) {
+                // one generator stream per population: 2000 + its place in the model's name-ordered list of populations
+                anyRNG = true;
+                groupEnv.addField(Type::Uint32.addConst(), "_rng_stream", Type::Uint32, "rngStream",
+                                  [&model](const NeuronGroupInternal &g, size_t)
+                                  {
+                                      return Type::NumericValue((uint64_t)(2000 + std::distance(model.getNeuronGroups().cbegin(), model.getNeuronGroups().find(g.getName()))));
+                                  });
+                groupEnv.add(Type::Uint32, "_rng", "gennmiRng",
+                             {groupEnv.addInitialiser("gennmi_kernel::Rng gennmiRng = gennmi_kernel::rngBegin(gennmiSeed, $(_rng_stream), "
+                                                      + n.getVarIndex(batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "$(id)") + ", gennmiStep);")});
+            }
             if(arch.isSpikeRecordingEnabled()) {
                 groupEnv.printLine("const unsigned int numRecordingWords = ($(num_neurons) + 31) / 32;");
             }
@@ -210,7 +235,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     }
     os << std::endl;
     os << "__global__ __launch_bounds__(256) void gennmiNeuronUpdateKernel(float t, unsigned int recordingTimestep, uint32_t gennmiTag, "
-          "unsigned long long *gennmiAgg, uint32_t *gennmiError" << paramStream.str() << ")";
+          "unsigned long long *gennmiAgg, uint32_t *gennmiError, unsigned long long gennmiSeed, unsigned long long gennmiStep" << paramStream.str() << ")";
     {
         CodeStream::Scope b(os);
         os << kernelStream.str();
@@ -225,8 +250,12 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         if(table.numBlocks > 0) {
             // the tag of a launch: differs from one launch to the next, never 0 (the look-back words start out zero)
             os << "gennmiNeuronLaunches = (gennmiNeuronLaunches == 0xFFFFFFFFu) ? 1u : gennmiNeuronLaunches + 1u;" << std::endl;
+            // (the generator's step counter: calls of updateNeurons so far; the seed: the model's, or one drawn at load time)
+            os << "static unsigned long long gennmiNeuronStep = 0;" << std::endl;
             os << "gennmiNeuronUpdateKernel<<<dim3(" << table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t, " << (recording ? "recordingTimestep" : "0u")
-               << ", gennmiNeuronLaunches, gennmiNeuronAgg, gennmiNeuronError" << argStream.str() << ");" << std::endl;
+               << ", gennmiNeuronLaunches, gennmiNeuronAgg, gennmiNeuronError, "
+               << (anyRNG ? ((model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull") : std::string("gennmiRandomSeed()")) : std::string("0ull"))
+               << ", gennmiNeuronStep++" << argStream.str() << ");" << std::endl;
             os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateNeurons: kernel launch failed\"); }" << std::endl;
         }
     }
@@ -313,6 +342,9 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
                     if(!sparse && !dense) { notGenerated("connectivity other than SPARSE and DENSE (projection '" + arch.getName() + "')"); }
                     if(arch.isPreSpikeEventRequired()) { notGenerated("spike-like events (projection '" + arch.getName() + "')"); }
+                    if(Utils::isRNGRequired(arch.getWUInitialiser().getPreSpikeSynCodeTokens()) || Utils::isRNGRequired(arch.getWUInitialiser().getPostSpikeSynCodeTokens())) {
+                        notGenerated("random numbers in weight-update code (projection '" + arch.getName() + "')");
+                    }
                     if(arch.getSrcNeuronGroup()->isDelayRequired() || arch.getTrgNeuronGroup()->isDelayRequired() || arch.getBackPropDelaySteps() != 0) {
                         notGenerated("axonal or back-propagation delay (projection '" + arch.getName() + "')");
                     }

@@ -348,6 +348,24 @@ def dense_layer(n_in=8192, n_out=8192, rate_hz=50.0, steps=1000, seed=17, dt=1.0
     return net
 
 
+def poisson_input(n_in=1500, n_out=400, rate=20.0, steps=1000, seed=53, dt=1.0):
+    """A population of the built-in Poisson neuron (neuronModels.h:307-325: a countdown to the next spike, refilled with
+    isi * gennrand_exponential()) driving LIF neurons through a static SPARSE projection.  The model draws random numbers
+    while it runs, from whatever generator its backend has — no two backends of the reference produce the same spikes —
+    so what can be compared is statistics.  On the MI355X backend the neuron's code reaches the generated kernels."""
+    net = Net(name="poisson_input", dt=dt, steps=steps, seed=seed)
+    net.pops.append(Pop("In", "poisson", n_in, {"rate": rate}, {"timeStepToSpike": np.zeros(n_in, np.float32)}))
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.0, TauRefrac=2.0)
+    net.pops.append(Pop("Out", "lif", n_out, lif, {"V": (-60.0 + 9.0 * rng.uniform(seed, 1, 0, n_out)).astype(np.float32),
+                                                      "RefracTime": np.zeros(n_out, np.float32)}))
+    stride = 40
+    ind = np.sort(rng.randint(seed, 2, 0, n_in * stride, n_out).reshape(n_in, stride), axis=1).astype(np.uint32)
+    g = (0.02 + 0.06 * rng.uniform(seed, 3, 0, n_in * stride)).astype(np.float32).reshape(n_in, stride)
+    net.syns.append(Syn("InOut", "In", "Out", psm="expcurr", tau=5.0, row_stride=stride, row_length=np.full(n_in, stride, np.uint32),
+                        ind=ind, g=g, wum="static"))
+    return net
+
+
 def custom_models(n_a=300, n_b=200, steps=300, seed=41, dt=1.0):
     """A network of models that are NOT built into GeNN or into the device library — what a user writes with the model
     API: LIF neurons with a spike-triggered adaptation variable ("lifa": the built-in LIF plus A, which decays every step,

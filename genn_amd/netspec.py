@@ -146,7 +146,7 @@ def write_netspec(net: Net, path: str):
     lines.append(f"snap {snap}")
     if getattr(net, "batch_size", 1) != 1:
         lines.append(f"batch {int(net.batch_size)}")
-    if any(s.matrix in ("procedural", "sparse_init") for s in net.syns) or any(c.model == "poisson_exp" for c in net.css):
+    if any(s.matrix in ("procedural", "sparse_init") for s in net.syns) or any(c.model == "poisson_exp" for c in net.css) or any(p.model == "poisson" for p in net.pops):
         lines.append(f"seed {int(net.seed)}")        # procedural matrices and Poisson sources draw from the model's seed
     for kind, group, param, step, value in net.dynamic:
         lines.append(f"dynamic {kind} {group} {param} {int(step)} {float(value)!r}")
@@ -157,6 +157,8 @@ def write_netspec(net: Net, path: str):
             ps = " ".join(repr(float(p.params[k])) for k in LIF_PARAMS + ("TauA", "dA"))
         elif p.model == "izh":
             ps = " ".join(repr(float(p.params[k])) for k in IZH_PARAMS)
+        elif p.model == "poisson":    # the built-in Poisson neuron (neuronModels.h:307-325): draws random numbers while it runs
+            ps = repr(float(p.params["rate"]))
         else:
             ps = ""
         lines.append(f"pop {p.name} {p.model} {p.n} {ps}".rstrip())

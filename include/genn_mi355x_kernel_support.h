@@ -122,6 +122,111 @@ __device__ inline void recordBallot(uint32_t *recordWords, uint32_t id, bool inR
     if((lane & 31) == 0 && inRange) { recordWords[id >> 5] = (uint32_t)(ballot >> (lane & 32)); }
 }
 
+// ---- random numbers of simulation code (gennrand_* in neuron, current-source and postsynaptic snippets).
+// The reference keeps a generator state per neuron in memory (XORWOW on its SIMT backends, one host mt19937 on the CPU
+// backend: no two of its backends draw the same numbers, so there is nothing bit-exact to match).  Here a draw is a word of
+// Philox4x32-10 (Salmon, Moraes, Dror, Shaw, SC'11) under key = the model's seed with counter = (batch * neurons + neuron,
+// timestep, number of the call within the step, one stream per population): no state in memory, the same numbers whatever
+// the launch geometry.
+struct Rng
+{
+    uint32_t k0, k1, element, stepLow, stepHighAndCall, stream;
+    uint32_t w0, w1, w2, w3, left;
+};
+
+__device__ inline void philox4x32(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1, uint32_t &o0, uint32_t &o1, uint32_t &o2, uint32_t &o3)
+{
+    #pragma unroll
+    for(int round = 0; round < 10; round++) {
+        const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+        c0 = hi1 ^ c1 ^ k0;
+        c1 = lo1;
+        c2 = hi0 ^ c3 ^ k1;
+        c3 = lo0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    o0 = c0; o1 = c1; o2 = c2; o3 = c3;
+}
+
+__device__ inline Rng rngBegin(unsigned long long seed, uint32_t stream, uint32_t element, unsigned long long step)
+{
+    Rng r;
+    r.k0 = (uint32_t)seed; r.k1 = (uint32_t)(seed >> 32);
+    r.element = element; r.stepLow = (uint32_t)step; r.stepHighAndCall = (uint32_t)(step >> 32) << 16; r.stream = stream;
+    r.w0 = r.w1 = r.w2 = r.w3 = 0; r.left = 0;
+    return r;
+}
+
+// next 32-bit word of the neuron's sequence for this step (four per generator call; at most 65,536 calls per neuron and step)
+__device__ inline uint32_t rngWord(Rng &r)
+{
+    if(r.left == 0) {
+        philox4x32(r.element, r.stepLow, r.stepHighAndCall, r.stream, r.k0, r.k1, r.w0, r.w1, r.w2, r.w3);
+        r.stepHighAndCall = (r.stepHighAndCall & 0xFFFF0000u) | ((r.stepHighAndCall + 1u) & 0xFFFFu);
+        r.left = 4;
+    }
+    const uint32_t word = r.w0;
+    r.w0 = r.w1; r.w1 = r.w2; r.w2 = r.w3;
+    r.left--;
+    return word;
+}
+
+__device__ inline float rngUniform(Rng &r) { return ((float)(rngWord(r) >> 8) + 0.5f) * (1.0f / 16777216.0f); }          // (0, 1)
+__device__ inline float rngExponential(Rng &r) { return -logf(rngUniform(r)); }
+__device__ inline float rngNormal(Rng &r)
+{
+    // Box-Muller; the sine branch is not kept (a neuron that wants two normals pays two pairs of words)
+    const float radius = sqrtf(-2.0f * logf(rngUniform(r)));
+    return radius * cospif(2.0f * ((float)(rngWord(r) >> 8) * (1.0f / 16777216.0f)));
+}
+__device__ inline float rngLogNormal(Rng &r, float mean, float sd) { return expf(mean + sd * rngNormal(r)); }
+// Marsaglia & Tsang (2000) for shape >= 1; shape < 1 through gamma(a + 1) * u^(1/a)
+__device__ inline float rngGamma(Rng &r, float a)
+{
+    const float boost = (a < 1.0f) ? 1.0f : 0.0f;
+    const float d = (a + boost) - (1.0f / 3.0f);
+    const float c = 1.0f / sqrtf(9.0f * d);
+    while(true) {
+        const float x = rngNormal(r);
+        float v = 1.0f + c * x;
+        if(v <= 0.0f) { continue; }
+        v = v * v * v;
+        const float u = rngUniform(r);
+        if(u < 1.0f - 0.0331f * (x * x) * (x * x) || logf(u) < 0.5f * x * x + d * (1.0f - v + logf(v))) {
+            return (boost != 0.0f) ? d * v * powf(rngUniform(r), 1.0f / a) : d * v;
+        }
+    }
+}
+// Binomial(n, p) by inversion of the CDF from k = 0, in slices of n short enough that (1 - p)^slice stays a normal double
+__device__ inline uint32_t rngBinomial(Rng &r, uint32_t n, float p)
+{
+    if(!(p > 0.0f) || n == 0) { return 0; }
+    if(p >= 1.0f) { return n; }
+    const bool flip = p > 0.5f;
+    const double pp = flip ? 1.0 - (double)p : (double)p;
+    const double logQ = log1p(-pp);
+    const uint32_t maxSlice = (uint32_t)fmin(4.0e9, fmax(1.0, floor(-600.0 / logQ)));
+    const double ratio = pp / (1.0 - pp);
+    uint32_t total = 0, done = 0;
+    while(done < n) {
+        const uint32_t m = min(maxSlice, n - done);
+        const uint32_t hi = rngWord(r), lo = rngWord(r);
+        double u = ((double)hi * 4294967296.0 + (double)lo + 0.5) * (1.0 / 18446744073709551616.0);
+        double pmf = exp((double)m * logQ);
+        uint32_t k = 0;
+        while(u > pmf && k < m) {
+            u -= pmf;
+            k++;
+            pmf *= ratio * (double)(m - k + 1) / (double)k;
+        }
+        total += k;
+        done += m;
+    }
+    return flip ? n - total : total;
+}
+
 __device__ inline void addScalar(float *address, float value) { unsafeAtomicAdd(address, value); }
 __device__ inline void addScalar(double *address, double value) { unsafeAtomicAdd(address, value); }
 }   // namespace gennmi_kernel

@@ -318,6 +318,9 @@ int main(int argc, char *argv[])
                     {{"a", p.p.at(0)}, {"b", p.p.at(1)}, {"c", p.p.at(2)}, {"d", p.p.at(3)}},
                     {{"V", uninitialisedVar()}, {"U", uninitialisedVar()}});
             }
+            else if(p.model == "poisson") {
+                p.ng = model.addNeuronPopulation<NeuronModels::Poisson>(p.name, p.n, {{"rate", p.p.at(0)}}, {{"timeStepToSpike", uninitialisedVar()}});
+            }
             else if(p.model == "ssa") {
                 p.ng = model.addNeuronPopulation<NeuronModels::SpikeSourceArray>(p.name, p.n, {},
                     {{"startSpike", uninitialisedVar()}, {"endSpike", uninitialisedVar()}});
@@ -460,6 +463,7 @@ int main(int argc, char *argv[])
                 load(rt.getArray(*p.ng, "V"), p.name + ".V.f32"); load(rt.getArray(*p.ng, "RefracTime"), p.name + ".RefracTime.f32"); load(rt.getArray(*p.ng, "A"), p.name + ".A.f32");
             }
             else if(p.model == "izh") { load(rt.getArray(*p.ng, "V"), p.name + ".V.f32"); load(rt.getArray(*p.ng, "U"), p.name + ".U.f32"); }
+            else if(p.model == "poisson") { load(rt.getArray(*p.ng, "timeStepToSpike"), p.name + ".timeStepToSpike.f32"); }
             else if(p.model == "ssa") {
                 load(rt.getArray(*p.ng, "startSpike"), p.name + ".startSpike.u32");
                 load(rt.getArray(*p.ng, "endSpike"), p.name + ".endSpike.u32");
@@ -548,7 +552,7 @@ int main(int argc, char *argv[])
         auto pulled = [](Runtime::ArrayBase *a) { a->pullFromDevice(); return a; };
         auto snapshot = [&]() {
             for(auto &p : pops) {
-                if(p.model == "ssa") continue;
+                if(p.model == "ssa" || p.model == "poisson") continue;
                 pulled(rt.getArray(*p.ng, "V"));
                 pulled(rt.getArray(*p.ng, (p.model == "lif" || p.model == "lifa") ? "RefracTime" : "U"));
                 appendFile(out + "/" + p.name + ".V.f32", rt.getArray(*p.ng, "V")->getHostPointer<float>(), (size_t)p.n * batch);
@@ -615,7 +619,7 @@ int main(int argc, char *argv[])
             if(i == 0) { firstSeconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - loopStart).count(); }
         }
         // a blocking pull drains whatever the backend still has queued, so the loop time below is complete
-        if(!pops.empty() && pops.front().model != "ssa") { rt.getArray(*pops.front().ng, "V")->pullFromDevice(); }
+        for(auto &p : pops) { if(p.model != "ssa" && p.model != "poisson") { rt.getArray(*p.ng, "V")->pullFromDevice(); break; } }
         const double loopSeconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - loopStart).count();
         std::cout << "ref_driver: stepping loop " << loopSeconds << " s for " << steps << " steps ("
                   << loopSeconds / steps * 1e6 << " us per Runtime::stepTime, snapshots included; first call " << firstSeconds * 1e3

@@ -64,6 +64,12 @@ def custom_batch1_small():
     return net, snap
 
 
+def poisson_input_small():
+    # the built-in Poisson neuron (random numbers in simulation code): the fixture holds the reference CPU backend's rasters,
+    # of which only the statistics carry over to another generator
+    return configs.poisson_input(), 250
+
+
 def dynamic_small():
     # parameters changed while the model runs (setParamDynamic + Runtime::setDynamicParamValue): the drive of the
     # excitatory population twice, the threshold of the inhibitory one, and the time constant of a postsynaptic model, whose
@@ -83,7 +89,7 @@ def potjans_poisson_net():
 
 # cases the reference's CPU backend pins directly (fixtures) and that the oracle, a restatement of the built-in models
 # with fixed parameters, does not cover
-REFERENCE_ONLY = {"custom_small", "custom_batch1_small", "dynamic_small"}
+REFERENCE_ONLY = {"custom_small", "custom_batch1_small", "dynamic_small", "poisson_input_small"}
 
-CASES = {"custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+CASES = {"poisson_input_small": poisson_input_small, "custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
          "stdp_small": stdp_small, "conv_small": conv_small}

@@ -157,7 +157,7 @@ def _generate_with(case, *options):
     return net, tmp, os.path.join(work, net.name + "_CODE"), res
 
 
-@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("stdp_small", ("--kernels=generated",)),
+@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("stdp_small", ("--kernels=generated",)),
                                            ("va_small", ("--dynamic=neuron:E.Ioffset",))])
 def test_generated_kernels_are_chosen_and_build(case, options):
     """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the runner then holds device
@@ -180,6 +180,11 @@ def test_generated_kernels_are_chosen_and_build(case, options):
             # the extra state variable and the weight-update variables are in the kernels under the reference's names
             assert "group->A[id]" in neuron and "sPreOutSynWUMPre" in neuron and "sPostInSynWUMPost" in neuron
             assert "group->wPost[idSyn] = group->sPost[idPost]" in synapse and "group->wPre[rowMajorIndex] = group->sPre[idPre]" in synapse
+        if case == "poisson_input_small":
+            # gennrand_exponential() of the built-in Poisson neuron: a counter-based generator keyed by the model's seed, one
+            # stream per population, the step counted by the launcher
+            assert "gennmi_kernel::rngBegin(gennmiSeed, (2000u), id, gennmiStep)" in neuron and "gennmi_kernel::rngExponential(gennmiRng)" in neuron
+            assert f"{net.seed}ull, gennmiNeuronStep++" in neuron
         if case in ("dynamic_small", "va_small"):
             # the dynamic parameter is a struct field the kernel reads, with a push function that marks the device copy stale
             assert "group->Ioffset" in neuron

@@ -338,6 +338,54 @@ def test_generated_kernels_with_batches():
         shutil.rmtree(tmp, ignore_errors=True)
 
 
+def test_generated_kernels_with_simulation_random_numbers():
+    """Random numbers in simulation code (the built-in Poisson neuron, neuronModels.h:307-325: `gennrand_exponential()` refills a
+    countdown): the generated kernels draw them from a counter-based generator keyed by the model's seed.  Every backend of
+    the reference draws from a generator of its own, so its CPU backend's fixture pins statistics, not spikes: the input
+    population's spike count and that of the LIF population it drives agree with the fixture's within sampling error, the
+    inter-spike intervals are exponential with the configured mean, neurons are independent, and the same seed gives the same
+    raster again."""
+    golden = np.load(os.path.join(HERE, "golden", "poisson_input_small.npz"))
+    rasters = []
+    for attempt in range(2):
+        net, snap, tmp, out = _run("poisson_input_small")
+        try:
+            assert net.generated_kernels
+            assert str(golden["input_digest"]) == net.input_digest()
+            rasters.append({p.name: np.fromfile(os.path.join(out, f"{p.name}.spikes.u32"), np.uint32).reshape(-1, 2) for p in net.pops})
+        finally:
+            shutil.rmtree(tmp, ignore_errors=True)
+    for name in ("In", "Out"):
+        assert np.array_equal(rasters[0][name], rasters[1][name]), f"{name}: the same seed gave another raster"
+    got, n_in, steps = rasters[0]["In"], net.pop("In").n, net.steps
+    rate_per_step = net.pop("In").params["rate"] * net.dt / 1000.0
+    expected = n_in * steps * rate_per_step
+    # counts: against the expectation and against the reference backend's draw of the same process (5 sigma of a difference)
+    assert abs(len(got) - expected) <= 5.0 * np.sqrt(expected), f"{len(got)} input spikes, expected about {expected:.0f}"
+    assert abs(len(got) - len(golden["spikes.In"])) <= 5.0 * np.sqrt(2.0 * expected)
+    assert not np.array_equal(got, golden["spikes.In"])                      # (another generator: other spikes)
+    # neurons: counts of a renewal process with exponential intervals have variance ~ mean
+    counts = np.bincount(got[:, 1], minlength=n_in)
+    assert 0.8 <= counts.var() / counts.mean() <= 1.2, f"Fano factor {counts.var() / counts.mean():.3f}"
+    # intervals: exponential, so coefficient of variation 1; their mean inside a window of 1,000 steps falls short of
+    # 1 / rate = 50 steps (long intervals do not fit), by how much the reference's own raster says
+    def intervals(raster):
+        order = np.lexsort((raster[:, 0], raster[:, 1]))
+        t, i = raster[order, 0].astype(np.float64), raster[order, 1]
+        return t, i, np.diff(t)[np.diff(i) == 0]
+    t, i, isi = intervals(got)
+    ref_isi = intervals(golden["spikes.In"])[2]
+    assert 0.9 / rate_per_step <= ref_isi.mean() <= 1.0 / rate_per_step
+    assert abs(isi.mean() - ref_isi.mean()) <= 0.02 * ref_isi.mean(), f"mean interval {isi.mean():.2f} steps, the reference's {ref_isi.mean():.2f}"
+    assert abs(isi.std() / isi.mean() - 1.0) <= 0.05, f"CV of the intervals {isi.std() / isi.mean():.3f}"
+    # no two neurons share a train (streams are per neuron)
+    trains = {tuple(t[i == k][:5]) for k in range(0, n_in, 7)}
+    assert len(trains) >= 0.99 * len(range(0, n_in, 7))
+    # the driven population: same input statistics, same connectivity, so the same output rate up to sampling error
+    out_got, out_ref = len(rasters[0]["Out"]), len(golden["spikes.Out"])
+    assert out_ref > 2000 and abs(out_got - out_ref) <= 0.05 * out_ref, f"{out_got} output spikes against {out_ref}"
+
+
 def test_adapter_device_initialisation_matches_host_layer():
     """Preferences::deviceInitialisation through GeNN's generator and Runtime: SPARSE matrices built by FixedProbability
     (with and without autapses) and FixedNumberPostWithReplacement with Uniform, Normal, Constant and constant-parameter
