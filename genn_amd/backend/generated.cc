@@ -287,7 +287,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         std::ostringstream body, args, params;
         BlockTable table;
     };
-    KernelText delay, pre, post;
+    KernelText delay, dynamics, pre, post;
     auto makeEnv = [&model](CodeStream &stream, EnvironmentLibrary &lib, auto use)
     {
         EnvironmentExternal funcEnv(lib);
@@ -298,9 +298,85 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         use(funcEnv);
     };
 
-    modelMerged.genMergedSynapseDynamicsGroups(
-        *this, memorySpaces,
-        [](auto &s) { notGenerated("synapse dynamics code (projection '" + s.getArchetype().getName() + "')"); });
+    // ---- synapse dynamics: every (padded) synapse every step, a grid-stride walk per group (backendSIMT.cc:805-863 gives each
+    // synapse a thread)
+    {
+        CodeStream stream(dynamics.body);
+        EnvironmentLibrary lib(stream, StandardLibrary::getMathsFunctions());
+        makeEnv(stream, lib, [&](EnvironmentExternal &funcEnv)
+        {
+            modelMerged.genMergedSynapseDynamicsGroups(
+                *this, memorySpaces,
+                [&](auto &s)
+                {
+                    const auto &arch = s.getArchetype();
+                    const auto matrix = arch.getMatrixType();
+                    const bool sparse = (matrix & SynapseMatrixConnectivity::SPARSE);
+                    const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
+                    if(!sparse && !dense) { notGenerated("connectivity other than SPARSE and DENSE (projection '" + arch.getName() + "')"); }
+                    if(arch.getSrcNeuronGroup()->isDelayRequired() || arch.getTrgNeuronGroup()->isDelayRequired() || arch.getBackPropDelaySteps() != 0) {
+                        notGenerated("axonal or back-propagation delay (projection '" + arch.getName() + "')");
+                    }
+                    if(Utils::isRNGRequired(arch.getWUInitialiser().getSynapseDynamicsCodeTokens())) {
+                        notGenerated("random numbers in weight-update code (projection '" + arch.getName() + "')");
+                    }
+                    const size_t firstBlock = dynamics.table.numBlocks;
+                    for(size_t g = 0; g < s.getGroups().size(); g++) {
+                        const auto &sg = s.getGroups()[g].get();
+                        const size_t rowLen = sparse ? getSynapticMatrixRowStride(sg) : sg.getTrgNeuronGroup()->getNumNeurons();
+                        const size_t blocks = std::clamp<size_t>((sg.getSrcNeuronGroup()->getNumNeurons() * rowLen + 255) / 256, 1, 1024);
+                        for(size_t b = 0; b < blocks; b++) { dynamics.table.add(g, 0, b, blocks); }
+                    }
+                    const std::string structArray = "mergedSynapseDynamicsGroup" + std::to_string(s.getIndex());
+                    dynamics.args << ", d_" << structArray;
+                    dynamics.params << ", const MergedSynapseDynamicsGroup" << s.getIndex() << " *" << structArray;
+
+                    funcEnv.getStream() << "// merged synapse dynamics group " << s.getIndex() << std::endl;
+                    funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << dynamics.table.numBlocks << "u)";
+                    CodeStream::Scope b(funcEnv.getStream());
+                    funcEnv.getStream() << "const gennmi_kernel::BlockEntry entry = gennmiSynapseDynamicsBlocks[blockIdx.x];" << std::endl;
+                    funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
+                    EnvironmentGroupMergedField<SynapseDynamicsGroupMerged> groupEnv(funcEnv, s);
+                    buildStandardEnvironment(groupEnv, batchSize);
+                    const auto indexType = getSynapseIndexType(s);
+                    const std::string indexTypeName = indexType.getName();
+                    groupEnv.printLine(std::string("const unsigned int rowSpan = ") + (sparse ? "$(_row_stride)" : "$(num_post)") + ";");
+                    groupEnv.printLine("const unsigned long long numSynapses = (unsigned long long)$(num_pre) * rowSpan;");
+                    groupEnv.getStream() << "for(unsigned long long item = (unsigned long long)entry.blockInGroup * 256u + threadIdx.x; item < numSynapses; "
+                                            "item += (unsigned long long)entry.blocksInGroup * 256u)";
+                    {
+                        CodeStream::Scope b2(groupEnv.getStream());
+                        EnvironmentGroupMergedField<SynapseDynamicsGroupMerged> synEnv(groupEnv, s);
+                        synEnv.getStream() << "const unsigned int row = (unsigned int)(item / rowSpan);" << std::endl;
+                        synEnv.getStream() << "const unsigned int col = (unsigned int)(item % rowSpan);" << std::endl;
+                        if(sparse) {
+                            synEnv.print("if(col < $(_row_length)[row])");
+                        }
+                        {
+                            CodeStream::Scope b3(synEnv.getStream());
+                            EnvironmentGroupMergedField<SynapseDynamicsGroupMerged> codeEnv(synEnv, s);
+                            codeEnv.add(Type::Uint32.addConst(), "id_pre", "row");
+                            codeEnv.add(indexType.addConst(), "id_syn", "idSyn",
+                                        {codeEnv.addInitialiser("const " + indexTypeName + " idSyn = (" + indexTypeName + ")item;")});
+                            if(sparse) {
+                                codeEnv.add(Type::Uint32.addConst(), "id_post", "idPost",
+                                            {codeEnv.addInitialiser("const unsigned int idPost = $(_ind)[item];")});
+                            }
+                            else {
+                                codeEnv.add(Type::Uint32.addConst(), "id_post", "col");
+                            }
+                            codeEnv.add(Type::getAddToPrePostDelay(s.getScalarType()), "addToPostDelay",
+                                        "gennmi_kernel::addScalar(&$(_den_delay)[" + s.getPostDenDelayIndex(batchSize, "$(id_post)", "$(1)") + "], $(0))");
+                            codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPost",
+                                        "gennmi_kernel::addScalar(&$(_out_post)[" + s.getPostISynIndex(batchSize, "$(id_post)") + "], $(0))");
+                            codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
+                                        "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(batchSize, "$(id_pre)") + "], $(0))");
+                            s.generateSynapseUpdate(*this, codeEnv, batchSize, dt);
+                        }
+                    }
+                });
+        });
+    }
 
     // ---- dendritic delay pointers: one thread per group
     {
@@ -503,17 +579,21 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
     modelMerged.genMergedSynapseDendriticDelayUpdateStructs(os, *this);
     modelMerged.genMergedPresynapticUpdateGroupStructs(os, *this);
     modelMerged.genMergedPostsynapticUpdateGroupStructs(os, *this);
+    modelMerged.genMergedSynapseDynamicsGroupStructs(os, *this);
     modelMerged.genMergedSynapseDendriticDelayUpdateHostStructArrayPush(os, *this);
     modelMerged.genMergedPresynapticUpdateGroupHostStructArrayPush(os, *this);
     modelMerged.genMergedPostsynapticUpdateGroupHostStructArrayPush(os, *this);
+    modelMerged.genMergedSynapseDynamicsGroupHostStructArrayPush(os, *this);
     preambleHandler(os);
     for(const auto &g : modelMerged.getMergedSynapseDendriticDelayUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "SynapseDendriticDelayUpdate"); }
     for(const auto &g : modelMerged.getMergedPresynapticUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "PresynapticUpdate"); }
     for(const auto &g : modelMerged.getMergedPostsynapticUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "PostsynapticUpdate"); }
+    for(const auto &g : modelMerged.getMergedSynapseDynamicsGroups()) { genDeviceStructArray(decl, upload, *this, g, "SynapseDynamics"); }
 
     os << declStream.str();
     os << "__device__ const gennmi_kernel::BlockEntry gennmiPresynapticBlocks[] = {" << std::endl << pre.table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
     os << "__device__ const gennmi_kernel::BlockEntry gennmiPostsynapticBlocks[] = {" << std::endl << post.table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+    os << "__device__ const gennmi_kernel::BlockEntry gennmiSynapseDynamicsBlocks[] = {" << std::endl << dynamics.table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
     os << std::endl;
     os << "void gennmiUploadSynapseGroups()";
     {
@@ -521,7 +601,12 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         os << uploadStream.str();
     }
     os << std::endl;
-    const bool anyDelay = delay.table.numBlocks > 0, anyPre = pre.table.numBlocks > 0, anyPost = post.table.numBlocks > 0;
+    const bool anyDelay = delay.table.numBlocks > 0, anyPre = pre.table.numBlocks > 0, anyPost = post.table.numBlocks > 0, anyDynamics = dynamics.table.numBlocks > 0;
+    if(anyDynamics) {
+        os << "__global__ __launch_bounds__(256) void gennmiSynapseDynamicsKernel(float t" << dynamics.params.str() << ")";
+        CodeStream::Scope b(os);
+        os << dynamics.body.str();
+    }
     if(anyDelay) {
         os << "__global__ void gennmiDendriticDelayUpdateKernel(float t" << delay.params.str() << ")";
         CodeStream::Scope b(os);
@@ -542,8 +627,9 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
     {
         CodeStream::Scope b(os);
         os << "gennmiEnsureFinalised();" << std::endl;
-        // order of the reference's updateSynapses (backendCUDAHIP.cc:548-589): ring pointers, presynaptic, postsynaptic
+        // order of the reference's updateSynapses (backendCUDAHIP.cc:548-589): ring pointers, synapse dynamics, presynaptic, postsynaptic
         if(anyDelay) { os << "gennmiDendriticDelayUpdateKernel<<<dim3(1), dim3(64), 0, 0>>>(t" << delay.args.str() << ");" << std::endl; }
+        if(anyDynamics) { os << "gennmiSynapseDynamicsKernel<<<dim3(" << dynamics.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << dynamics.args.str() << ");" << std::endl; }
         if(anyPre) { os << "gennmiPresynapticUpdateKernel<<<dim3(" << pre.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << pre.args.str() << ");" << std::endl; }
         if(anyPost) { os << "gennmiPostsynapticUpdateKernel<<<dim3(" << post.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << post.args.str() << ");" << std::endl; }
         os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateSynapses: kernel launch failed\"); }" << std::endl;

@@ -366,6 +366,28 @@ def poisson_input(n_in=1500, n_out=400, rate=20.0, steps=1000, seed=53, dt=1.0):
     return net
 
 
+def synapse_dynamics(n_a=240, n_b=160, steps=300, seed=67, dt=1.0):
+    """Weight-update code that runs for every synapse every step ("leaky_graded", a model of the test driver: each synapse keeps
+    a decaying trace of how far its source's membrane potential is above a midpoint and delivers g times the trace, spike or
+    no spike) between two LIF populations, beside an ordinary static inhibitory projection.  Exists only as code strings of
+    the driver's model class, so on the MI355X backend it runs through generated kernels."""
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.55, TauRefrac=2.0)
+    net = Net(name="synapse_dynamics", dt=dt, steps=steps, seed=seed)
+    net.pops.append(Pop("A", "lif", n_a, lif, {"V": (-60.0 + 9.5 * rng.uniform(seed, 1, 0, n_a)).astype(np.float32), "RefracTime": np.zeros(n_a, np.float32)}))
+    net.pops.append(Pop("B", "lif", n_b, dict(lif, Ioffset=0.2), {"V": (-60.0 + 9.5 * rng.uniform(seed, 2, 0, n_b)).astype(np.float32),
+                                                                    "RefracTime": np.zeros(n_b, np.float32)}))
+
+    def sparse(name, src, trg, n_src, n_trg, stride, stream, lo, hi, wum, tau, params=None):
+        ind = np.sort(rng.randint(seed, stream, 0, n_src * stride, n_trg).reshape(n_src, stride), axis=1).astype(np.uint32)
+        row_length = (stride - rng.randint(seed, stream + 1, 0, n_src, stride // 3)).astype(np.uint32)
+        g = (lo + (hi - lo) * rng.uniform(seed, stream + 2, 0, n_src * stride)).astype(np.float32).reshape(n_src, stride)
+        return Syn(name, src, trg, psm="expcurr", tau=tau, row_stride=stride, row_length=row_length, ind=ind, g=g, wum=wum, wum_params=params or {})
+
+    net.syns.append(sparse("AB_graded", "A", "B", n_a, n_b, 24, 10, 0.0, 0.004, "leaky_graded", 5.0, {"Vmid": -56.0, "decay": 0.8}))
+    net.syns.append(sparse("BA_inhibit", "B", "A", n_b, n_a, 20, 20, -0.4, -0.1, "static", 10.0))
+    return net
+
+
 def custom_models(n_a=300, n_b=200, steps=300, seed=41, dt=1.0):
     """A network of models that are NOT built into GeNN or into the device library — what a user writes with the model
     API: LIF neurons with a spike-triggered adaptation variable ("lifa": the built-in LIF plus A, which decays every step,

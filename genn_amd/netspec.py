@@ -208,6 +208,8 @@ def write_netspec(net: Net, path: str):
             w = ("stdp" if s.wum == "stdp_additive" else s.wum) + " " + " ".join(repr(float(s.wum_params[k])) for k in STDP_PARAMS)
         elif s.wum == "static_graded":
             w = f"static_graded {float(s.wum_params['Epre'])!r} {float(s.wum_params['Vslope'])!r}"
+        elif s.wum == "leaky_graded":      # a model of the test driver with synapse dynamics code (runs for every synapse every step)
+            w = f"leaky_graded {float(s.wum_params['Vmid'])!r} {float(s.wum_params['decay'])!r}"
         else:
             raise ValueError(s.wum)
         psm = f"expcurr {float(s.tau)!r}" if s.psm == "expcurr" else "deltacurr"

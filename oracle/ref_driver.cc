@@ -157,6 +157,22 @@ public:
 };
 IMPLEMENT_SNIPPET(TimingCopy);
 
+// Weight update model that runs EVERY step for EVERY synapse (synapse dynamics code), after the continuous models of
+// tests/features/test_synapse_dynamics*.py: each synapse low-pass filters how far its source's membrane potential is above a
+// midpoint and delivers g times that trace, spike or no spike.
+class LeakyGraded : public WeightUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(LeakyGraded);
+    SET_PARAMS({"Vmid", "decay"});
+    SET_VARS({{"g", "scalar", VarAccess::READ_ONLY}, {"x", "scalar"}});
+    SET_PRE_NEURON_VAR_REFS({{"Vpre", "scalar", VarAccessMode::READ_ONLY}});
+    SET_SYNAPSE_DYNAMICS_CODE(
+        "x = (x * decay) + fmax(0.0, Vpre - Vmid);\n"
+        "addToPost(g * x);\n");
+};
+IMPLEMENT_SNIPPET(LeakyGraded);
+
 // Current source fed from a host-pregenerated array; the driver rewrites the N-element
 // window before every step, so the injected value at step s is noise[s*N + id].
 class ArrayNoise : public CurrentSourceModels::Base
@@ -277,7 +293,7 @@ int main(int argc, char *argv[])
                     if(s.wum == "static_delay") { ls >> s.maxDenDelay; }
                     else if(s.wum == "stdp_trace" || s.wum == "stdp") { s.wumP.resize(6); for(auto &c : s.wumP) ls >> c; }
                     else if(s.wum == "static_const") { s.wumP.resize(1); ls >> s.wumP[0]; }
-                    else if(s.wum == "static_graded") { s.wumP.resize(2); ls >> s.wumP[0] >> s.wumP[1]; }
+                    else if(s.wum == "static_graded" || s.wum == "leaky_graded") { s.wumP.resize(2); ls >> s.wumP[0] >> s.wumP[1]; }
                     else if(s.wum != "static" && s.wum != "static_reverse" && s.wum != "static_init" && s.wum != "timing_copy") throw std::runtime_error("wum " + s.wum);
                     ls >> s.psm;
                     if(s.psm == "expcurr") { s.psmP.resize(1); ls >> s.psmP[0]; }
@@ -350,6 +366,10 @@ int main(int argc, char *argv[])
             }
             else if(s.wum == "static_reverse") {
                 wum = initWeightUpdate<StaticPulseReverse>({}, {{"g", uninitialisedVar()}});
+            }
+            else if(s.wum == "leaky_graded") {
+                wum = initWeightUpdate<LeakyGraded>({{"Vmid", s.wumP.at(0)}, {"decay", s.wumP.at(1)}}, {{"g", uninitialisedVar()}, {"x", 0.0}}, {}, {},
+                                                    {{"Vpre", createVarRef(popByName.at(s.src)->ng, "V")}}, {});
             }
             else if(s.wum == "timing_copy") {
                 wum = initWeightUpdate<TimingCopy>({}, {{"g", uninitialisedVar()}, {"wPre", 0.0}, {"wPost", 0.0}}, {{"sPre", 0.0}}, {{"sPost", 0.0}});
@@ -574,6 +594,11 @@ int main(int argc, char *argv[])
                     auto *a = pulled(rt.getArray(*s.sg, "g"));
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
                     for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + ".g.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
+                }
+                if(s.wum == "leaky_graded") {
+                    const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
+                    auto *a = pulled(rt.getArray(*s.sg, "x"));
+                    for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + ".x.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
                 }
                 if(s.wum == "timing_copy") {
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);

@@ -70,6 +70,11 @@ def poisson_input_small():
     return configs.poisson_input(), 250
 
 
+def synapse_dynamics_small():
+    # weight-update code that runs for every synapse every step (a model of the test driver): generated kernels only
+    return configs.synapse_dynamics(), 25
+
+
 def dynamic_small():
     # parameters changed while the model runs (setParamDynamic + Runtime::setDynamicParamValue): the drive of the
     # excitatory population twice, the threshold of the inhibitory one, and the time constant of a postsynaptic model, whose
@@ -89,7 +94,7 @@ def potjans_poisson_net():
 
 # cases the reference's CPU backend pins directly (fixtures) and that the oracle, a restatement of the built-in models
 # with fixed parameters, does not cover
-REFERENCE_ONLY = {"custom_small", "custom_batch1_small", "dynamic_small", "poisson_input_small"}
+REFERENCE_ONLY = {"custom_small", "custom_batch1_small", "dynamic_small", "poisson_input_small", "synapse_dynamics_small"}
 
-CASES = {"poisson_input_small": poisson_input_small, "custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+CASES = {"synapse_dynamics_small": synapse_dynamics_small, "poisson_input_small": poisson_input_small, "custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
          "stdp_small": stdp_small, "conv_small": conv_small}

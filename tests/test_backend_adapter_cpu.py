@@ -157,7 +157,7 @@ def _generate_with(case, *options):
     return net, tmp, os.path.join(work, net.name + "_CODE"), res
 
 
-@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("stdp_small", ("--kernels=generated",)),
+@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("stdp_small", ("--kernels=generated",)),
                                            ("va_small", ("--dynamic=neuron:E.Ioffset",))])
 def test_generated_kernels_are_chosen_and_build(case, options):
     """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the runner then holds device
@@ -180,6 +180,10 @@ def test_generated_kernels_are_chosen_and_build(case, options):
             # the extra state variable and the weight-update variables are in the kernels under the reference's names
             assert "group->A[id]" in neuron and "sPreOutSynWUMPre" in neuron and "sPostInSynWUMPost" in neuron
             assert "group->wPost[idSyn] = group->sPost[idPost]" in synapse and "group->wPre[rowMajorIndex] = group->sPre[idPre]" in synapse
+        if case == "synapse_dynamics_small":
+            # code that runs for every synapse every step: a kernel of its own, launched before the presynaptic update
+            assert "gennmiSynapseDynamicsKernel<<<" in synapse and synapse.index("gennmiSynapseDynamicsKernel<<<") < synapse.index("gennmiPresynapticUpdateKernel<<<")
+            assert "group->x[idSyn]" in synapse and "group->Vpre[row]" in synapse
         if case == "poisson_input_small":
             # gennrand_exponential() of the built-in Poisson neuron: a counter-based generator keyed by the model's seed, one
             # stream per population, the step counted by the launcher

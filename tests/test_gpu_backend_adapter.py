@@ -58,7 +58,7 @@ def _run(case, *options):
 LIBRARY_CASES = sorted(set(CASES) - REFERENCE_ONLY)
 # what the generated kernels cover: SPARSE / DENSE matrices, any neuron, postsynaptic, current-source and weight-update code
 # without delay slots, spike-like events or random numbers
-GENERATED_CASES = ["custom_small", "dynamic_small", "va_small", "potjans_small", "izhikevich_small", "stdp_small", "stdp_additive_small", "reverse_small"]
+GENERATED_CASES = ["custom_small", "dynamic_small", "synapse_dynamics_small", "va_small", "potjans_small", "izhikevich_small", "stdp_small", "stdp_additive_small", "reverse_small"]
 
 
 @pytest.mark.parametrize("case", LIBRARY_CASES)
@@ -125,7 +125,7 @@ def _compare_with_fixture(case, *options):
                 if key in golden:
                     got = np.fromfile(os.path.join(out, f"{s.name}.{var}.f32"), np.float32).reshape(net.steps // snap, -1)
                     assert np.array_equal(got, golden[key]), key
-            for var in ("g", "preTrace", "postTrace", "outPost"):
+            for var in ("g", "preTrace", "postTrace", "outPost", "x"):
                 key = f"{var}.{s.name}"
                 if key in golden:
                     got = np.fromfile(os.path.join(out, f"{s.name}.{var}.f32"), np.float32).reshape(net.steps // snap, -1)
