@@ -1572,6 +1572,14 @@ Backend createBackend(const ModelSpecInternal &model, const filesystem::path&, p
         for(const auto &s : model.getSynapseGroups()) {
             generated = generated || !recognised([&]{ recognisePSM(s.second.getPSInitialiser().getSnippet(), s.first); });
             generated = generated || !recognised([&]{ recogniseWUM(s.second.getWUInitialiser().getSnippet(), s.first); });
+            // ... or when a learning rule meets delay slots (spike times, traces and weight-update variables per slot): the
+            // library's plastic kernels read populations without a ring, GeNN's generic code in generated kernels handles it
+            const auto *wum = s.second.getWUInitialiser().getSnippet();
+            const bool learns = !wum->getPostSpikeSynCode().empty() || !wum->getPreSpikeCode().empty() || !wum->getPostSpikeCode().empty()
+                                || !wum->getPreVars().empty() || !wum->getPostVars().empty();
+            const bool delayed = s.second.getSrcNeuronGroup()->isDelayRequired() || s.second.getTrgNeuronGroup()->isDelayRequired()
+                                 || s.second.getBackPropDelaySteps() != 0;
+            generated = generated || (learns && delayed);
         }
         // ... or when a parameter is dynamic: the library's descriptors hold parameters as constants, generated kernels read
         // them from the merged structs that setDynamicParamValue rewrites
@@ -1589,7 +1597,7 @@ Backend createBackend(const ModelSpecInternal &model, const filesystem::path&, p
             generated = generated || anyDynamic(s.second.getPSInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isPSParamDynamic(p); });
             generated = generated || anyDynamic(s.second.getWUInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isWUParamDynamic(p); });
         }
-        if(generated) { LOGI_BACKEND << "The model uses snippets the device library does not implement, or dynamic parameters: the step's kernels are generated from the model's code"; }
+        if(generated) { LOGI_BACKEND << "The model uses snippets or combinations the device library does not implement, or dynamic parameters: the step's kernels are generated from the model's code"; }
     }
     if(generated && preferences.orderedAccumulation) {
         throw std::runtime_error("MI355X backend: ordered accumulation is a mode of the device library's kernels, not of generated ones");

@@ -124,7 +124,6 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         [&](auto &n)
         {
             const auto &arch = n.getArchetype();
-            if(arch.isDelayRequired()) { notGenerated("axonal delay slots (population '" + arch.getName() + "')"); }
             if(arch.isPrevSpikeTimeRequired() || arch.isSpikeEventTimeRequired() || arch.isPrevSpikeEventTimeRequired()) {
                 notGenerated("previous spike times and spike-like event times (population '" + arch.getName() + "')");
             }
@@ -152,7 +151,11 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             buildStandardEnvironment(groupEnv, batchSize);
             groupEnv.add(Type::Uint32.addConst(), "id", "id");
             // where a batch's entries of a per-neuron array (spike queue, spike times) begin
-            const std::string queueOffset = n.getWriteVarIndex(false, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "");
+            // (with axonal delay: in the slot of the population's ring that this step writes, the one *spk_que_ptr names after
+            // the queue-update kernel has advanced it; GeNN's generic code copies delayed variables of neurons that did not
+            // spike from the slot read to the slot written, neuronUpdateGroupMerged.cc:714-770)
+            const std::string queueOffset = n.getWriteVarIndex(arch.isSpikeDelayRequired(), batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "");
+            const std::string countIndex = arch.isSpikeDelayRequired() ? ((batchSize > 1) ? "$(_write_batch_delay_slot)" : "$(_write_delay_slot)") : "$(batch)";
             if(arch.isSimRNGRequired()) {
                 // one generator stream per population: 2000 + its place in the model's name-ordered list of populations
                 anyRNG = true;
@@ -193,22 +196,54 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             // every spike queue of the population (one per fused outgoing / incoming spike target) from the same positions
             n.generateSpikes(
                 groupEnv,
-                [&queueOffset](EnvironmentExternalBase &env)
+                [&queueOffset, &countIndex](EnvironmentExternalBase &env)
                 {
                     env.print("if(slot.ok)");
                     CodeStream::Scope b3(env.getStream());
                     env.printLine("if(gennmiSpiked) { $(_spk)[" + queueOffset + "slot.position] = $(id); }");
-                    env.printLine("if(slot.writeTotal) { $(_spk_cnt)[$(batch)] = slot.total; }");
+                    env.printLine("if(slot.writeTotal) { $(_spk_cnt)[" + countIndex + "] = slot.total; }");
                 });
         });
+    }
+
+    // Populations with delay slots: their ring pointer moves on before the update (backendSIMT.cc:372-401; one thread per group).
+    // Without delay slots that kernel would only clear counts that the compaction overwrites anyway, and is left out.
+    const bool anyDelaySlots = std::any_of(model.getNeuronGroups().cbegin(), model.getNeuronGroups().cend(),
+                                           [](const auto &n) { return n.second.isDelayRequired(); });
+    std::ostringstream queueStream, queueArgs, queueParams;
+    if(anyDelaySlots) {
+        CodeStream queue(queueStream);
+        EnvironmentLibrary queueLib(queue, StandardLibrary::getMathsFunctions());
+        EnvironmentExternal queueEnv(queueLib);
+        modelMerged.genMergedNeuronSpikeQueueUpdateGroups(
+            *this, memorySpaces,
+            [&](auto &n)
+            {
+                const std::string structArray = "mergedNeuronSpikeQueueUpdateGroup" + std::to_string(n.getIndex());
+                queueArgs << (queueArgs.str().empty() ? "" : ", ") << "d_" << structArray;
+                queueParams << (queueParams.str().empty() ? "" : ", ") << "MergedNeuronSpikeQueueUpdateGroup" << n.getIndex() << " *" << structArray;
+                queueEnv.getStream() << "for(unsigned int g = threadIdx.x; g < " << n.getGroups().size() << "u; g += blockDim.x)";
+                CodeStream::Scope b(queueEnv.getStream());
+                queueEnv.getStream() << "auto *group = &" << structArray << "[g];" << std::endl;
+                EnvironmentGroupMergedField<NeuronSpikeQueueUpdateGroupMerged> groupEnv(queueEnv, n);
+                buildStandardEnvironment(groupEnv, batchSize);
+                n.genSpikeQueueUpdate(groupEnv, batchSize);
+            });
     }
 
     // struct definitions, host arrays and their push functions are GeNN's own
     modelMerged.genMergedNeuronUpdateGroupStructs(os, *this);
     modelMerged.genMergedNeuronUpdateGroupHostStructArrayPush(os, *this);
+    if(anyDelaySlots) {
+        modelMerged.genMergedNeuronSpikeQueueUpdateStructs(os, *this);
+        modelMerged.genMergedNeuronSpikeQueueUpdateHostStructArrayPush(os, *this);
+    }
     preambleHandler(os);
     for(const auto &n : modelMerged.getMergedNeuronUpdateGroups()) {
         genDeviceStructArray(decl, upload, *this, n, "NeuronUpdate");
+    }
+    if(anyDelaySlots) {
+        for(const auto &n : modelMerged.getMergedNeuronSpikeQueueUpdateGroups()) { genDeviceStructArray(decl, upload, *this, n, "NeuronSpikeQueueUpdate"); }
     }
 
     os << declStream.str();
@@ -234,6 +269,12 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         }
     }
     os << std::endl;
+    if(anyDelaySlots) {
+        os << "__global__ void gennmiSpikeQueueUpdateKernel(" << queueParams.str() << ")";
+        CodeStream::Scope b(os);
+        os << queueStream.str();
+    }
+    os << std::endl;
     os << "__global__ __launch_bounds__(256) void gennmiNeuronUpdateKernel(float t, unsigned int recordingTimestep, uint32_t gennmiTag, "
           "unsigned long long *gennmiAgg, uint32_t *gennmiError, unsigned long long gennmiSeed, unsigned long long gennmiStep" << paramStream.str() << ")";
     {
@@ -247,6 +288,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     {
         CodeStream::Scope b(os);
         os << "gennmiEnsureFinalised();" << std::endl;
+        if(anyDelaySlots) { os << "gennmiSpikeQueueUpdateKernel<<<dim3(1), dim3(64), 0, 0>>>(" << queueArgs.str() << ");" << std::endl; }
         if(table.numBlocks > 0) {
             // the tag of a launch: differs from one launch to the next, never 0 (the look-back words start out zero)
             os << "gennmiNeuronLaunches = (gennmiNeuronLaunches == 0xFFFFFFFFu) ? 1u : gennmiNeuronLaunches + 1u;" << std::endl;
@@ -314,9 +356,6 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const bool sparse = (matrix & SynapseMatrixConnectivity::SPARSE);
                     const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
                     if(!sparse && !dense) { notGenerated("connectivity other than SPARSE and DENSE (projection '" + arch.getName() + "')"); }
-                    if(arch.getSrcNeuronGroup()->isDelayRequired() || arch.getTrgNeuronGroup()->isDelayRequired() || arch.getBackPropDelaySteps() != 0) {
-                        notGenerated("axonal or back-propagation delay (projection '" + arch.getName() + "')");
-                    }
                     if(Utils::isRNGRequired(arch.getWUInitialiser().getSynapseDynamicsCodeTokens())) {
                         notGenerated("random numbers in weight-update code (projection '" + arch.getName() + "')");
                     }
@@ -421,9 +460,6 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     if(Utils::isRNGRequired(arch.getWUInitialiser().getPreSpikeSynCodeTokens()) || Utils::isRNGRequired(arch.getWUInitialiser().getPostSpikeSynCodeTokens())) {
                         notGenerated("random numbers in weight-update code (projection '" + arch.getName() + "')");
                     }
-                    if(arch.getSrcNeuronGroup()->isDelayRequired() || arch.getTrgNeuronGroup()->isDelayRequired() || arch.getBackPropDelaySteps() != 0) {
-                        notGenerated("axonal or back-propagation delay (projection '" + arch.getName() + "')");
-                    }
                     if(!arch.isPreSpikeRequired()) { return; }
 
                     const size_t firstBlock = pre.table.numBlocks;
@@ -446,8 +482,9 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
                     EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> groupEnv(funcEnv, s);
                     buildStandardEnvironment(groupEnv, batchSize);
-                    const std::string preOffset = (batchSize > 1) ? "$(_pre_batch_offset) + " : "";
-                    groupEnv.printLine("const unsigned int numSpikes = $(_src_spk_cnt)[$(batch)];");
+                    // (axonal delay: the slot of the source's ring written `delay` steps ago, presynapticUpdateStrategySIMT.cc:224-247)
+                    const bool preDelay = arch.getSrcNeuronGroup()->isSpikeQueueRequired() && arch.getSrcNeuronGroup()->isDelayRequired();
+                    groupEnv.printLine("const unsigned int numSpikes = $(_src_spk_cnt)[" + s.getPreSlot(preDelay, batchSize) + "];");
                     groupEnv.printLine(std::string("const unsigned int rowSpan = ") + (sparse ? "$(_row_stride)" : "$(num_post)") + ";");
                     groupEnv.getStream() << "const unsigned int chunksPerRow = (rowSpan + 63u) / 64u;" << std::endl;
                     groupEnv.getStream() << "const unsigned int numWaves = entry.blocksInGroup * 4u;" << std::endl;
@@ -458,7 +495,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> synEnv(groupEnv, s);
                         synEnv.getStream() << "const unsigned int spike = (unsigned int)(item / chunksPerRow);" << std::endl;
                         synEnv.getStream() << "const unsigned int j = (unsigned int)(item % chunksPerRow) * 64u + (threadIdx.x & 63u);" << std::endl;
-                        synEnv.printLine("const unsigned int idPre = $(_src_spk)[" + preOffset + "spike];");
+                        synEnv.printLine("const unsigned int idPre = $(_src_spk)[" + s.getPreVarIndex(preDelay, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "spike") + "];");
                         synEnv.add(Type::Uint32.addConst(), "id_pre", "idPre");
                         const auto indexType = getSynapseIndexType(s);
                         const std::string indexTypeName = indexType.getName();
@@ -532,8 +569,9 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
                     EnvironmentGroupMergedField<PostsynapticUpdateGroupMerged> groupEnv(funcEnv, s);
                     buildStandardEnvironment(groupEnv, batchSize);
-                    const std::string postOffset = (batchSize > 1) ? "$(_post_batch_offset) + " : "";
-                    groupEnv.printLine("const unsigned int numSpikes = $(_trg_spk_cnt)[$(batch)];");
+                    // (back-propagation delay: the slot of the target's ring written `delay` steps ago, backendSIMT.cc:1822-1835)
+                    const bool postDelay = arch.getTrgNeuronGroup()->isSpikeQueueRequired() && arch.getTrgNeuronGroup()->isDelayRequired();
+                    groupEnv.printLine("const unsigned int numSpikes = $(_trg_spk_cnt)[" + s.getPostSlot(postDelay, batchSize) + "];");
                     groupEnv.printLine(std::string("const unsigned int colSpan = ") + (sparse ? "$(_col_stride)" : "$(num_pre)") + ";");
                     groupEnv.getStream() << "const unsigned int chunksPerCol = (colSpan + 63u) / 64u;" << std::endl;
                     groupEnv.getStream() << "const unsigned int numWaves = entry.blocksInGroup * 4u;" << std::endl;
@@ -542,7 +580,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     {
                         CodeStream::Scope b2(groupEnv.getStream());
                         EnvironmentGroupMergedField<PostsynapticUpdateGroupMerged> synEnv(groupEnv, s);
-                        synEnv.printLine("const unsigned int spike = $(_trg_spk)[" + postOffset + "(unsigned int)(item / chunksPerCol)];");
+                        synEnv.printLine("const unsigned int spike = $(_trg_spk)[" + s.getPostVarIndex(postDelay, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "(unsigned int)(item / chunksPerCol)") + "];");
                         synEnv.getStream() << "const unsigned int i = (unsigned int)(item % chunksPerCol) * 64u + (threadIdx.x & 63u);" << std::endl;
                         if(sparse) {
                             synEnv.print("if(i < $(_col_length)[spike])");

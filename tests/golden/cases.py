@@ -51,6 +51,17 @@ def custom_small():
     return configs.custom_models(), 25
 
 
+def stdp_delay_small():
+    # trace STDP over a projection with an axonal delay (spike times, traces and the weight-update variables then live in
+    # the populations' delay slots, neuronUpdateGroupMerged.cc:714-770 copies them from slot to slot) beside a delayed static one:
+    # the device library refuses that combination, so on the MI355X backend the model takes generated kernels
+    net, snap = stdp_small()
+    net.name = "stdp_delay"
+    net.syn("EE").axonal_delay_steps = 3
+    net.syn("EI").axonal_delay_steps = 1
+    return net, snap
+
+
 def custom_batch1_small():
     # custom_small from other initial values (same matrices): what the second batch of a batched run of custom_small
     # starts from.  The reference's CPU backend has no batches, so every batch of that run is pinned by a run of its own.
@@ -94,7 +105,7 @@ def potjans_poisson_net():
 
 # cases the reference's CPU backend pins directly (fixtures) and that the oracle, a restatement of the built-in models
 # with fixed parameters, does not cover
-REFERENCE_ONLY = {"custom_small", "custom_batch1_small", "dynamic_small", "poisson_input_small", "synapse_dynamics_small"}
+REFERENCE_ONLY = {"stdp_delay_small", "custom_small", "custom_batch1_small", "dynamic_small", "poisson_input_small", "synapse_dynamics_small"}
 
-CASES = {"synapse_dynamics_small": synapse_dynamics_small, "poisson_input_small": poisson_input_small, "custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+CASES = {"stdp_delay_small": stdp_delay_small, "synapse_dynamics_small": synapse_dynamics_small, "poisson_input_small": poisson_input_small, "custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
          "stdp_small": stdp_small, "conv_small": conv_small}
