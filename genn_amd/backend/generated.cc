@@ -110,6 +110,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
 
     EnvironmentLibrary kernelEnv(kernel, StandardLibrary::getMathsFunctions());
     bool anyRNG = false;
+    size_t maxEventGroups = 0;      // spike-like event conditions of one population: each compacts a queue of its own
     {   // (environments write what they hold when they go out of scope: the kernel's text is complete after this block)
     // gennrand_* of simulation code: words of a counter-based generator, see gennmi_kernel::Rng (`_rng` exists in the
     // populations that need it)
@@ -127,7 +128,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             if(arch.isPrevSpikeTimeRequired() || arch.isSpikeEventTimeRequired() || arch.isPrevSpikeEventTimeRequired()) {
                 notGenerated("previous spike times and spike-like event times (population '" + arch.getName() + "')");
             }
-            if(!n.getMergedSpikeEventGroups().empty()) { notGenerated("spike-like events (population '" + arch.getName() + "')"); }
+            maxEventGroups = std::max(maxEventGroups, n.getMergedSpikeEventGroups().size());
 
             const size_t firstBlock = table.numBlocks;
             for(size_t g = 0; g < n.getGroups().size(); g++) {
@@ -146,6 +147,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
             funcEnv.getStream() << "const unsigned int id = entry.firstId + threadIdx.x;" << std::endl;
             funcEnv.getStream() << "bool gennmiSpiked = false;" << std::endl;
+            for(const auto &e : n.getMergedSpikeEventGroups()) { funcEnv.getStream() << "bool gennmiEvent" << e.getIndex() << " = false;" << std::endl; }
 
             EnvironmentGroupMergedField<NeuronUpdateGroupMerged> groupEnv(funcEnv, n);
             buildStandardEnvironment(groupEnv, batchSize);
@@ -184,7 +186,11 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                         if(arch.isSpikeTimeRequired()) { env.printLine("$(_st)[" + queueOffset + "$(id)] = $(t);"); }
                         env.getStream() << "gennmiSpiked = true;" << std::endl;
                     },
-                    [](EnvironmentExternalBase&, NeuronUpdateGroupMerged::SynSpikeEvent&) {});
+                    // a spike-like event of one of the population's conditions: flagged here, queued below like the true spikes
+                    [](EnvironmentExternalBase &env, NeuronUpdateGroupMerged::SynSpikeEvent &e)
+                    {
+                        env.getStream() << "gennmiEvent" << e.getIndex() << " = true;" << std::endl;
+                    });
             }
             groupEnv.printLine("const gennmi_kernel::QueueSlot slot = gennmi_kernel::orderedSlot(gennmiSpiked, entry.blockInGroup, entry.blocksInGroup, "
                                "blockIdx.x - entry.blockInGroup, gennmiAgg + (size_t)2 * gridDim.x * blockIdx.y, gennmiAgg + (size_t)2 * gridDim.x * blockIdx.y + gridDim.x, "
@@ -192,6 +198,32 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             if(arch.isSpikeRecordingEnabled()) {
                 groupEnv.printLine("gennmi_kernel::recordBallot(&$(_record_spk)[((size_t)recordingTimestep * " + std::to_string(batchSize) + "u + $(batch)) * numRecordingWords], "
                                    "$(id), $(id) < $(num_neurons), slot.ballot);");
+            }
+            // spike-like events: one ordered compaction per condition (its own look-back words), the ballot as recording bitfield
+            if(!n.getMergedSpikeEventGroups().empty()) {
+                const std::string eventOffset = n.getWriteVarIndex(arch.isSpikeEventDelayRequired(), batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "");
+                const std::string eventCountIndex = arch.isSpikeEventDelayRequired() ? ((batchSize > 1) ? "$(_write_batch_delay_slot)" : "$(_write_delay_slot)") : "$(batch)";
+                const bool recordEvents = arch.isSpikeEventRecordingEnabled();
+                if(recordEvents && !arch.isSpikeRecordingEnabled()) {
+                    groupEnv.printLine("const unsigned int numRecordingWords = ($(num_neurons) + 31) / 32;");
+                }
+                n.generateSpikeEvents(
+                    groupEnv,
+                    [&eventOffset, &eventCountIndex, recordEvents, batchSize](EnvironmentExternalBase &env, NeuronUpdateGroupMerged::SynSpikeEvent &e)
+                    {
+                        const std::string k = std::to_string(e.getIndex());
+                        const std::string region = "gennmiAgg + (size_t)2 * gridDim.x * (gridDim.y * " + std::to_string(e.getIndex() + 1) + "u + blockIdx.y)";
+                        env.printLine("const gennmi_kernel::QueueSlot eventSlot" + k + " = gennmi_kernel::orderedSlot(gennmiEvent" + k + ", entry.blockInGroup, entry.blocksInGroup, "
+                                      "blockIdx.x - entry.blockInGroup, " + region + ", " + region + " + gridDim.x, gennmiTag, gennmiError);");
+                        if(recordEvents) {
+                            env.printLine("gennmi_kernel::recordBallot(&$(_record_spk_event)[((size_t)recordingTimestep * " + std::to_string(batchSize) + "u + $(batch)) * numRecordingWords], "
+                                          "$(id), $(id) < $(num_neurons), eventSlot" + k + ".ballot);");
+                        }
+                        env.print("if(eventSlot" + k + ".ok)");
+                        CodeStream::Scope b3(env.getStream());
+                        env.printLine("if(gennmiEvent" + k + ") { $(_spk_event)[" + eventOffset + "eventSlot" + k + ".position] = $(id); }");
+                        env.printLine("if(eventSlot" + k + ".writeTotal) { $(_spk_cnt_event)[" + eventCountIndex + "] = eventSlot" + k + ".total; }");
+                    });
             }
             // every spike queue of the population (one per fused outgoing / incoming spike target) from the same positions
             n.generateSpikes(
@@ -260,8 +292,8 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         {
             CodeStream::Scope b2(os);
             os << "void *p = nullptr;" << std::endl;
-            os << "GENNMI_CHECK(gennmi_malloc(&p, " << 2 * std::max<size_t>(1, table.numBlocks) * batchSize << " * sizeof(unsigned long long)));" << std::endl;
-            os << "GENNMI_CHECK(gennmi_memset(p, 0, " << 2 * std::max<size_t>(1, table.numBlocks) * batchSize << " * sizeof(unsigned long long)));" << std::endl;
+            os << "GENNMI_CHECK(gennmi_malloc(&p, " << 2 * std::max<size_t>(1, table.numBlocks) * batchSize * (1 + maxEventGroups) << " * sizeof(unsigned long long)));" << std::endl;
+            os << "GENNMI_CHECK(gennmi_memset(p, 0, " << 2 * std::max<size_t>(1, table.numBlocks) * batchSize * (1 + maxEventGroups) << " * sizeof(unsigned long long)));" << std::endl;
             os << "gennmiNeuronAgg = (unsigned long long*)p;" << std::endl;
             os << "GENNMI_CHECK(gennmi_malloc(&p, sizeof(uint32_t)));" << std::endl;
             os << "GENNMI_CHECK(gennmi_memset(p, 0, sizeof(uint32_t)));" << std::endl;
@@ -456,11 +488,11 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const bool sparse = (matrix & SynapseMatrixConnectivity::SPARSE);
                     const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
                     if(!sparse && !dense) { notGenerated("connectivity other than SPARSE and DENSE (projection '" + arch.getName() + "')"); }
-                    if(arch.isPreSpikeEventRequired()) { notGenerated("spike-like events (projection '" + arch.getName() + "')"); }
-                    if(Utils::isRNGRequired(arch.getWUInitialiser().getPreSpikeSynCodeTokens()) || Utils::isRNGRequired(arch.getWUInitialiser().getPostSpikeSynCodeTokens())) {
+                    if(Utils::isRNGRequired(arch.getWUInitialiser().getPreSpikeSynCodeTokens()) || Utils::isRNGRequired(arch.getWUInitialiser().getPostSpikeSynCodeTokens())
+                       || Utils::isRNGRequired(arch.getWUInitialiser().getPreEventSynCodeTokens())) {
                         notGenerated("random numbers in weight-update code (projection '" + arch.getName() + "')");
                     }
-                    if(!arch.isPreSpikeRequired()) { return; }
+                    if(!arch.isPreSpikeRequired() && !arch.isPreSpikeEventRequired()) { return; }
 
                     const size_t firstBlock = pre.table.numBlocks;
                     for(size_t g = 0; g < s.getGroups().size(); g++) {
@@ -482,20 +514,26 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
                     EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> groupEnv(funcEnv, s);
                     buildStandardEnvironment(groupEnv, batchSize);
-                    // (axonal delay: the slot of the source's ring written `delay` steps ago, presynapticUpdateStrategySIMT.cc:224-247)
-                    const bool preDelay = arch.getSrcNeuronGroup()->isSpikeQueueRequired() && arch.getSrcNeuronGroup()->isDelayRequired();
-                    groupEnv.printLine("const unsigned int numSpikes = $(_src_spk_cnt)[" + s.getPreSlot(preDelay, batchSize) + "];");
                     groupEnv.printLine(std::string("const unsigned int rowSpan = ") + (sparse ? "$(_row_stride)" : "$(num_post)") + ";");
                     groupEnv.getStream() << "const unsigned int chunksPerRow = (rowSpan + 63u) / 64u;" << std::endl;
                     groupEnv.getStream() << "const unsigned int numWaves = entry.blocksInGroup * 4u;" << std::endl;
-                    groupEnv.getStream() << "const unsigned long long numItems = (unsigned long long)numSpikes * chunksPerRow;" << std::endl;
-                    groupEnv.getStream() << "for(unsigned long long item = entry.blockInGroup * 4u + (threadIdx.x / 64u); item < numItems; item += numWaves)";
+                    // the queue of spike-like events first, then the true spikes (the reference's order, backendSIMT.cc:745-760);
+                    // either is a walk over (entry of the queue, 64-synapse chunk of its row) items
+                    auto walk = [&](bool trueSpike)
                     {
+                        const std::string suffix = trueSpike ? "" : "_event";
+                        const auto *src = arch.getSrcNeuronGroup();
+                        // (axonal delay: the slot of the source's ring written `delay` steps ago, presynapticUpdateStrategySIMT.cc:224-247)
+                        const bool preDelay = src->isDelayRequired() && (trueSpike ? src->isSpikeQueueRequired() : src->isSpikeEventQueueRequired());
+                        CodeStream::Scope b1(groupEnv.getStream());
+                        groupEnv.printLine("const unsigned int numSpikes = $(_src_spk_cnt" + suffix + ")[" + s.getPreSlot(preDelay, batchSize) + "];");
+                        groupEnv.getStream() << "const unsigned long long numItems = (unsigned long long)numSpikes * chunksPerRow;" << std::endl;
+                        groupEnv.getStream() << "for(unsigned long long item = entry.blockInGroup * 4u + (threadIdx.x / 64u); item < numItems; item += numWaves)";
                         CodeStream::Scope b2(groupEnv.getStream());
                         EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> synEnv(groupEnv, s);
                         synEnv.getStream() << "const unsigned int spike = (unsigned int)(item / chunksPerRow);" << std::endl;
                         synEnv.getStream() << "const unsigned int j = (unsigned int)(item % chunksPerRow) * 64u + (threadIdx.x & 63u);" << std::endl;
-                        synEnv.printLine("const unsigned int idPre = $(_src_spk)[" + s.getPreVarIndex(preDelay, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "spike") + "];");
+                        synEnv.printLine("const unsigned int idPre = $(_src_spk" + suffix + ")[" + s.getPreVarIndex(preDelay, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "spike") + "];");
                         synEnv.add(Type::Uint32.addConst(), "id_pre", "idPre");
                         const auto indexType = getSynapseIndexType(s);
                         const std::string indexTypeName = indexType.getName();
@@ -505,29 +543,34 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         else {
                             synEnv.print("if(j < $(num_post))");
                         }
-                        {
-                            CodeStream::Scope b3(synEnv.getStream());
-                            EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> codeEnv(synEnv, s);
-                            if(sparse) {
-                                codeEnv.add(indexType.addConst(), "id_syn", "idSyn",
-                                            {codeEnv.addInitialiser("const " + indexTypeName + " idSyn = ((" + indexTypeName + ")idPre * $(_row_stride)) + j;")});
-                                codeEnv.add(Type::Uint32.addConst(), "id_post", "idPost",
-                                            {codeEnv.addInitialiser("const unsigned int idPost = $(_ind)[$(id_syn)];")});
-                            }
-                            else {
-                                codeEnv.add(Type::Uint32.addConst(), "id_post", "j");
-                                codeEnv.add(indexType.addConst(), "id_syn", "idSyn",
-                                            {codeEnv.addInitialiser("const " + indexTypeName + " idSyn = ((" + indexTypeName + ")idPre * $(num_post)) + j;")});
-                            }
-                            codeEnv.add(Type::getAddToPrePostDelay(s.getScalarType()), "addToPostDelay",
-                                        "gennmi_kernel::addScalar(&$(_den_delay)[" + s.getPostDenDelayIndex(batchSize, "$(id_post)", "$(1)") + "], $(0))");
-                            codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPost",
-                                        "gennmi_kernel::addScalar(&$(_out_post)[" + s.getPostISynIndex(batchSize, "$(id_post)") + "], $(0))");
-                            codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
-                                        "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(batchSize, "$(id_pre)") + "], $(0))");
+                        CodeStream::Scope b3(synEnv.getStream());
+                        EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> codeEnv(synEnv, s);
+                        if(sparse) {
+                            codeEnv.add(indexType.addConst(), "id_syn", "idSyn",
+                                        {codeEnv.addInitialiser("const " + indexTypeName + " idSyn = ((" + indexTypeName + ")idPre * $(_row_stride)) + j;")});
+                            codeEnv.add(Type::Uint32.addConst(), "id_post", "idPost",
+                                        {codeEnv.addInitialiser("const unsigned int idPost = $(_ind)[$(id_syn)];")});
+                        }
+                        else {
+                            codeEnv.add(Type::Uint32.addConst(), "id_post", "j");
+                            codeEnv.add(indexType.addConst(), "id_syn", "idSyn",
+                                        {codeEnv.addInitialiser("const " + indexTypeName + " idSyn = ((" + indexTypeName + ")idPre * $(num_post)) + j;")});
+                        }
+                        codeEnv.add(Type::getAddToPrePostDelay(s.getScalarType()), "addToPostDelay",
+                                    "gennmi_kernel::addScalar(&$(_den_delay)[" + s.getPostDenDelayIndex(batchSize, "$(id_post)", "$(1)") + "], $(0))");
+                        codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPost",
+                                    "gennmi_kernel::addScalar(&$(_out_post)[" + s.getPostISynIndex(batchSize, "$(id_post)") + "], $(0))");
+                        codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
+                                    "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(batchSize, "$(id_pre)") + "], $(0))");
+                        if(trueSpike) {
                             s.generateSpikeUpdate(*this, codeEnv, batchSize, dt);
                         }
-                    }
+                        else {
+                            s.generateSpikeEventUpdate(*this, codeEnv, batchSize, dt);
+                        }
+                    };
+                    if(arch.isPreSpikeEventRequired()) { walk(false); }
+                    if(arch.isPreSpikeRequired()) { walk(true); }
                 });
         });
     }
@@ -547,7 +590,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const bool sparse = (matrix & SynapseMatrixConnectivity::SPARSE);
                     const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
                     if(!sparse && !dense) { notGenerated("connectivity other than SPARSE and DENSE (projection '" + arch.getName() + "')"); }
-                    if(arch.isPostSpikeEventRequired()) { notGenerated("spike-like events (projection '" + arch.getName() + "')"); }
+                    if(arch.isPostSpikeEventRequired()) { notGenerated("postsynaptic spike-like events (projection '" + arch.getName() + "')"); }
                     if(!arch.isPostSpikeRequired()) { return; }
 
                     const size_t firstBlock = post.table.numBlocks;

@@ -375,13 +375,15 @@ int main(int argc, char *argv[])
                 wum = initWeightUpdate<TimingCopy>({}, {{"g", uninitialisedVar()}, {"wPre", 0.0}, {"wPost", 0.0}}, {{"sPre", 0.0}}, {{"sPost", 0.0}});
             }
             else if(s.wum == "static_graded") {
+                const ParamValues gradedParams{{"Epre", s.wumP[0]}, {"Vslope", s.wumP[1]}};
+                const VarValues gradedVars{{"g", uninitialisedVar()}};
 #ifdef DRIVER_BACKEND_MI355X
-                // the adapter recognises the built-in as it stands (it never transpiles the event code)
-                wum = initWeightUpdate<WeightUpdateModels::StaticGraded>(
-#else
-                wum = initWeightUpdate<GradedSynapse>(
+                // the adapter recognises the built-in as it stands (its library path never transpiles the event code); kernels
+                // generated from the code need the variant that transpiles
+                if(kernels != "generated") { wum = initWeightUpdate<WeightUpdateModels::StaticGraded>(gradedParams, gradedVars, {}, {}, {{"V", std::string("V")}}); }
+                else
 #endif
-                    {{"Epre", s.wumP[0]}, {"Vslope", s.wumP[1]}}, {{"g", uninitialisedVar()}}, {}, {}, {{"V", std::string("V")}});
+                { wum = initWeightUpdate<GradedSynapse>(gradedParams, gradedVars, {}, {}, {{"V", std::string("V")}}); }
             }
             else if(s.wum == "static_delay") {
                 wum = initWeightUpdate<WeightUpdateModels::StaticPulseDendriticDelay>({}, {{"g", uninitialisedVar()}, {"d", uninitialisedVar()}});

@@ -157,7 +157,7 @@ def _generate_with(case, *options):
     return net, tmp, os.path.join(work, net.name + "_CODE"), res
 
 
-@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("stdp_delay_small", ()), ("stdp_small", ("--kernels=generated",)),
+@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
                                            ("va_small", ("--dynamic=neuron:E.Ioffset",))])
 def test_generated_kernels_are_chosen_and_build(case, options):
     """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the runner then holds device
@@ -180,6 +180,10 @@ def test_generated_kernels_are_chosen_and_build(case, options):
             # the extra state variable and the weight-update variables are in the kernels under the reference's names
             assert "group->A[id]" in neuron and "sPreOutSynWUMPre" in neuron and "sPostInSynWUMPost" in neuron
             assert "group->wPost[idSyn] = group->sPost[idPost]" in synapse and "group->wPre[rowMajorIndex] = group->sPre[idPre]" in synapse
+        if case == "graded_small":
+            # spike-like events: a queue per condition, compacted in order like the true spikes and recorded from the ballot
+            assert "gennmiEvent0 = true" in neuron and "eventSlot0 = gennmi_kernel::orderedSlot(gennmiEvent0" in neuron and "recordSpkEvent" in neuron
+            assert "srcSpkCntEvent" in synapse or "srcSpkCntEvent".lower() in synapse.lower()
         if case == "stdp_delay_small":
             # a learning rule over delay slots: chosen for generated kernels by itself; the populations' ring pointers move on
             # in a kernel of their own before the update, and the queues are read through GeNN's delay-slot helpers
@@ -231,7 +235,7 @@ def test_generated_kernels_take_the_batch_from_the_grid():
         shutil.rmtree(tmp, ignore_errors=True)
 
 
-@pytest.mark.parametrize("case, what", [("conv_small", "connectivity"), ("graded_small", "spike-like")])
+@pytest.mark.parametrize("case, what", [("conv_small", "connectivity")])
 def test_generated_kernels_say_what_they_do_not_cover(case, what):
     """Asked to generate kernels for a feature only the device library implements, the backend names the feature."""
     net, tmp, code, res = _generate_with(case, "--kernels=generated")
