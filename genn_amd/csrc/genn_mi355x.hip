@@ -228,6 +228,13 @@ int gennmi_memcpy_to_device(void *dev, const void *host, size_t bytes)
     return GENNMI_OK;
 }
 int gennmi_memcpy_from_device(void *host, const void *dev, size_t bytes) { FLUSH_QUEUED(); HIP_TRY(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost)); return GENNMI_OK; }
+int gennmi_note_device_write(const void *dev, size_t bytes)
+{
+    FLUSH_QUEUED();
+    if(!dev) { return fail(GENNMI_EINVAL, "note_device_write: null pointer"); }
+    noteDeviceWrite(dev, bytes);
+    return GENNMI_OK;
+}
 int gennmi_memset(void *dev, int value, size_t bytes)
 {
     FLUSH_QUEUED();

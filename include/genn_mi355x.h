@@ -89,6 +89,13 @@ int gennmi_fill_f32(float *dev, float value, size_t count);     /* e.g. sT = -TI
  * exactly 8*count bytes). */
 int gennmi_copy_f32(float *dst, const float *src, size_t count);
 int gennmi_synchronize(void);
+/* No counterpart in the reference.  Arrays handed to a runner stay the caller's: it may write them by its own means (a
+ * hipMemcpy of its own, a kernel of its own) instead of through the calls above.  The library keeps copies derived from
+ * some of them — the resident plan's segment tables and packed synapse records (weights, targets, delays), the tile path's
+ * segment boundaries and records, the zero-delay lists of the single-launch step, column views, spike bitmaps — and
+ * refreshes them before the next step when it knows the array was written; the calls above tell it, this call is for
+ * writes it cannot see.  Cheap; naming a range that feeds no copy does nothing. */
+int gennmi_note_device_write(const void *dev, size_t bytes);
 /* Host mirrors.  GeNN's Runtime serialises HOST pointers into merged-group structs for backends that report
  * isArrayDeviceObjectRequired() == false (runtime.cc:700-720, 1027-1044) — which lets the generated initialize() /
  * initializeSparse() run the reference's own host-side initialisation code on those pointers.  An Array

@@ -160,6 +160,40 @@ def test_pushed_weights_reach_the_inline_copies(monkeypatch):
     model.unload()
 
 
+def test_weights_written_behind_the_library_are_reported(monkeypatch):
+    """A caller that overwrites `g` by its own means (here: a device-to-device copy the runner is not told about) and then
+    names the range with gennmi_note_device_write gets the same refresh of the inline copies and packed records as a push."""
+    import ctypes as C
+    from genn_amd import _abi
+    monkeypatch.setenv("GENNMI_FUSED_STEP", "0")
+    n, depth = 600, 4
+    net = Net(name="resident_note", dt=1.0, steps=0)
+    net.pops.append(_pop("A", n, 0.6, -60.0 + 9.5 * rng.uniform(7, 1, 0, n)))
+    net.syns.append(_projection("AA", "A", "A", n, n, 48, 0.04, 31, depth, 0.4))
+    net.steps = 120
+    state = {"written": False}
+
+    def check(model, oracle):
+        compare_state(net, model, oracle, f"after {model.timestep} steps", exact=True)
+        if not state["written"]:
+            g = model.synapse_populations["AA"].vars["g"]
+            lib = _abi.load()
+            staging = C.c_void_p()
+            _abi.check(lib.gennmi_malloc(C.byref(staging), g.view.nbytes))
+            new = np.full(g.count, -0.03, np.float32)
+            _abi.check(lib.gennmi_memcpy_to_device(staging, new.ctypes.data_as(C.c_void_p), new.nbytes))
+            hip = C.CDLL("libamdhip64.so")
+            assert hip.hipMemcpy(C.c_void_p(g.ptr), staging, C.c_size_t(new.nbytes), C.c_int(3)) == 0      # hipMemcpyDeviceToDevice
+            _abi.check(lib.gennmi_note_device_write(C.c_void_p(g.ptr), new.nbytes))
+            lib.gennmi_free(staging)
+            oracle.syn_g("AA")[:] = np.float32(-0.03)
+            state["written"] = True
+
+    model, oracle, spikes = _run_chunks(net, (60, 60), check)
+    assert spikes > 500
+    model.unload()
+
+
 @pytest.mark.parametrize("limit, rows", [(64, 230), (1000, 230), (7, 230), (64, 50), (64, 0)])
 def test_queued_single_steps_take_the_resident_launch(limit, rows):
     """step_time() one call at a time with the step queue on (what the reference's Runtime::stepTime amounts to): the steps
