@@ -364,12 +364,33 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
     KernelText delay, dynamics, pre, post;
     auto makeEnv = [&model](CodeStream &stream, EnvironmentLibrary &lib, auto use)
     {
-        EnvironmentExternal funcEnv(lib);
+        EnvironmentLibrary rngLib(lib, simRNGFunctions);        // (gennrand_* of weight-update code: `_rng` exists where it is used)
+        EnvironmentExternal funcEnv(rngLib);
         funcEnv.add(model.getTimePrecision().addConst(), "t", "t");
         funcEnv.add(Type::Uint32.addConst(), "batch", (model.getBatchSize() > 1) ? "blockIdx.y" : "0");
         funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
         (void)stream;
         use(funcEnv);
+    };
+
+    // Random numbers in weight-update code: a generator per synapse and step — counter (synapse id of the batch, step, call),
+    // stream 3000 + 4 x the projection's place in the model's name-ordered list + the kind of code (0 spike, 1 spike-like
+    // event, 2 postsynaptic spike, 3 synapse dynamics), key = the model's seed.  (The reference skips ahead in one Philox
+    // sequence per thread, backendCUDAHIP.cc:497, so there as here no two backends draw the same numbers.)
+    bool anySynapseRNG = false;
+    auto addSynapseRng = [&model, &anySynapseRNG, batchSize](auto &codeEnv, const SynapseGroupInternal &, const auto &tokens, unsigned int kind)
+    {
+        if(!Utils::isRNGRequired(tokens)) { return; }
+        anySynapseRNG = true;
+        const std::string k = std::to_string(kind);
+        codeEnv.addField(Type::Uint32.addConst(), "_rng_stream" + k, Type::Uint32, "rngStream" + k,
+                         [&model, kind](const SynapseGroupInternal &g, size_t)
+                         {
+                             return Type::NumericValue((uint64_t)(3000 + 4 * std::distance(model.getSynapseGroups().cbegin(), model.getSynapseGroups().find(g.getName())) + kind));
+                         });
+        const std::string element = (batchSize > 1) ? "(unsigned long long)$(_syn_batch_offset) + $(id_syn)" : "(unsigned long long)$(id_syn)";
+        codeEnv.add(Type::Uint32, "_rng", "gennmiRng",
+                    {codeEnv.addInitialiser("gennmi_kernel::Rng gennmiRng = gennmi_kernel::rngBegin(gennmiSeed, $(_rng_stream" + k + "), " + element + ", gennmiStep);")});
     };
 
     // ---- synapse dynamics: every (padded) synapse every step, a grid-stride walk per group (backendSIMT.cc:805-863 gives each
@@ -388,9 +409,6 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const bool sparse = (matrix & SynapseMatrixConnectivity::SPARSE);
                     const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
                     if(!sparse && !dense) { notGenerated("connectivity other than SPARSE and DENSE (projection '" + arch.getName() + "')"); }
-                    if(Utils::isRNGRequired(arch.getWUInitialiser().getSynapseDynamicsCodeTokens())) {
-                        notGenerated("random numbers in weight-update code (projection '" + arch.getName() + "')");
-                    }
                     const size_t firstBlock = dynamics.table.numBlocks;
                     for(size_t g = 0; g < s.getGroups().size(); g++) {
                         const auto &sg = s.getGroups()[g].get();
@@ -442,6 +460,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                                         "gennmi_kernel::addScalar(&$(_out_post)[" + s.getPostISynIndex(batchSize, "$(id_post)") + "], $(0))");
                             codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
                                         "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(batchSize, "$(id_pre)") + "], $(0))");
+                            addSynapseRng(codeEnv, arch, arch.getWUInitialiser().getSynapseDynamicsCodeTokens(), 3);
                             s.generateSynapseUpdate(*this, codeEnv, batchSize, dt);
                         }
                     }
@@ -488,10 +507,6 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const bool sparse = (matrix & SynapseMatrixConnectivity::SPARSE);
                     const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
                     if(!sparse && !dense) { notGenerated("connectivity other than SPARSE and DENSE (projection '" + arch.getName() + "')"); }
-                    if(Utils::isRNGRequired(arch.getWUInitialiser().getPreSpikeSynCodeTokens()) || Utils::isRNGRequired(arch.getWUInitialiser().getPostSpikeSynCodeTokens())
-                       || Utils::isRNGRequired(arch.getWUInitialiser().getPreEventSynCodeTokens())) {
-                        notGenerated("random numbers in weight-update code (projection '" + arch.getName() + "')");
-                    }
                     if(!arch.isPreSpikeRequired() && !arch.isPreSpikeEventRequired()) { return; }
 
                     const size_t firstBlock = pre.table.numBlocks;
@@ -563,9 +578,11 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
                                     "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(batchSize, "$(id_pre)") + "], $(0))");
                         if(trueSpike) {
+                            addSynapseRng(codeEnv, arch, arch.getWUInitialiser().getPreSpikeSynCodeTokens(), 0);
                             s.generateSpikeUpdate(*this, codeEnv, batchSize, dt);
                         }
                         else {
+                            addSynapseRng(codeEnv, arch, arch.getWUInitialiser().getPreEventSynCodeTokens(), 1);
                             s.generateSpikeEventUpdate(*this, codeEnv, batchSize, dt);
                         }
                     };
@@ -649,6 +666,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                             codeEnv.add(Type::Uint32.addConst(), "id_post", "spike");
                             codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
                                         "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(batchSize, "$(id_pre)") + "], $(0))");
+                            addSynapseRng(codeEnv, arch, arch.getWUInitialiser().getPostSpikeSynCodeTokens(), 2);
                             s.generateSpikeUpdate(*this, codeEnv, batchSize, dt);
                         }
                     }
@@ -684,7 +702,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
     os << std::endl;
     const bool anyDelay = delay.table.numBlocks > 0, anyPre = pre.table.numBlocks > 0, anyPost = post.table.numBlocks > 0, anyDynamics = dynamics.table.numBlocks > 0;
     if(anyDynamics) {
-        os << "__global__ __launch_bounds__(256) void gennmiSynapseDynamicsKernel(float t" << dynamics.params.str() << ")";
+        os << "__global__ __launch_bounds__(256) void gennmiSynapseDynamicsKernel(float t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << dynamics.params.str() << ")";
         CodeStream::Scope b(os);
         os << dynamics.body.str();
     }
@@ -694,12 +712,12 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         os << delay.body.str();
     }
     if(anyPre) {
-        os << "__global__ __launch_bounds__(256) void gennmiPresynapticUpdateKernel(float t" << pre.params.str() << ")";
+        os << "__global__ __launch_bounds__(256) void gennmiPresynapticUpdateKernel(float t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << pre.params.str() << ")";
         CodeStream::Scope b(os);
         os << pre.body.str();
     }
     if(anyPost) {
-        os << "__global__ __launch_bounds__(256) void gennmiPostsynapticUpdateKernel(float t" << post.params.str() << ")";
+        os << "__global__ __launch_bounds__(256) void gennmiPostsynapticUpdateKernel(float t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << post.params.str() << ")";
         CodeStream::Scope b(os);
         os << post.body.str();
     }
@@ -710,9 +728,14 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         os << "gennmiEnsureFinalised();" << std::endl;
         // order of the reference's updateSynapses (backendCUDAHIP.cc:548-589): ring pointers, synapse dynamics, presynaptic, postsynaptic
         if(anyDelay) { os << "gennmiDendriticDelayUpdateKernel<<<dim3(1), dim3(64), 0, 0>>>(t" << delay.args.str() << ");" << std::endl; }
-        if(anyDynamics) { os << "gennmiSynapseDynamicsKernel<<<dim3(" << dynamics.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << dynamics.args.str() << ");" << std::endl; }
-        if(anyPre) { os << "gennmiPresynapticUpdateKernel<<<dim3(" << pre.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << pre.args.str() << ");" << std::endl; }
-        if(anyPost) { os << "gennmiPostsynapticUpdateKernel<<<dim3(" << post.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << post.args.str() << ");" << std::endl; }
+        // (the generators' step counter: calls of updateSynapses so far; the seed: the model's, or one drawn at load time)
+        const std::string seedAndStep = std::string(", ") + (anySynapseRNG ? ((model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull") : std::string("gennmiRandomSeed()")) : std::string("0ull"))
+                                        + ", gennmiSynapseStep";
+        os << "static unsigned long long gennmiSynapseStep = 0;" << std::endl;
+        if(anyDynamics) { os << "gennmiSynapseDynamicsKernel<<<dim3(" << dynamics.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << seedAndStep << dynamics.args.str() << ");" << std::endl; }
+        if(anyPre) { os << "gennmiPresynapticUpdateKernel<<<dim3(" << pre.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << seedAndStep << pre.args.str() << ");" << std::endl; }
+        if(anyPost) { os << "gennmiPostsynapticUpdateKernel<<<dim3(" << post.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << seedAndStep << post.args.str() << ");" << std::endl; }
+        os << "gennmiSynapseStep++;" << std::endl;
         os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateSynapses: kernel launch failed\"); }" << std::endl;
     }
 }

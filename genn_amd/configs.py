@@ -388,6 +388,31 @@ def synapse_dynamics(n_a=240, n_b=160, steps=300, seed=67, dt=1.0):
     return net
 
 
+def stochastic_synapses(n_a=400, n_b=300, steps=600, seed=71, dt=1.0, twin=False):
+    """Synapses that transmit with a probability ("stochastic", a model of the test driver: `if(gennrand_uniform() < pRelease)
+    addToPost(g)`): a driven LIF population A onto B, whose threshold is out of reach so that its membrane potential is a
+    linear functional of its input, through synapses that release 40 % of the time, and onto spiking C through synapses that
+    always release.  `twin`: the same network with static synapses — weights times 0.4 onto B (the expectation of the
+    stochastic input), unchanged onto C (the same input exactly)."""
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.0, TauRefrac=2.0)
+    net = Net(name="stochastic_twin" if twin else "stochastic", dt=dt, steps=steps, seed=seed)
+    net.pops.append(Pop("A", "lif", n_a, dict(lif, Ioffset=0.75), {"V": (-60.0 + 9.5 * rng.uniform(seed, 1, 0, n_a)).astype(np.float32),
+                                                                   "RefracTime": np.zeros(n_a, np.float32)}))
+    net.pops.append(Pop("B", "lif", n_b, dict(lif, Vthresh=1.0e9), {"V": np.full(n_b, -60.0, np.float32), "RefracTime": np.zeros(n_b, np.float32)}))
+    net.pops.append(Pop("C", "lif", n_b, lif, {"V": np.full(n_b, -60.0, np.float32), "RefracTime": np.zeros(n_b, np.float32)}))
+    stride = 60
+    ind = np.sort(rng.randint(seed, 2, 0, n_a * stride, n_b).reshape(n_a, stride), axis=1).astype(np.uint32)
+    g = (0.05 + 0.1 * rng.uniform(seed, 3, 0, n_a * stride)).astype(np.float32).reshape(n_a, stride)
+    common = dict(psm="expcurr", tau=5.0, row_stride=stride, row_length=np.full(n_a, stride, np.uint32), ind=ind)
+    if twin:
+        net.syns.append(Syn("AB", "A", "B", g=(g * np.float32(0.4)).astype(np.float32), wum="static", **common))
+        net.syns.append(Syn("AC", "A", "C", g=g, wum="static", **common))
+    else:
+        net.syns.append(Syn("AB", "A", "B", g=g, wum="stochastic", wum_params={"pRelease": 0.4}, **common))
+        net.syns.append(Syn("AC", "A", "C", g=g, wum="stochastic", wum_params={"pRelease": 1.0}, **common))
+    return net
+
+
 def custom_models(n_a=300, n_b=200, steps=300, seed=41, dt=1.0):
     """A network of models that are NOT built into GeNN or into the device library — what a user writes with the model
     API: LIF neurons with a spike-triggered adaptation variable ("lifa": the built-in LIF plus A, which decays every step,

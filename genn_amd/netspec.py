@@ -146,7 +146,8 @@ def write_netspec(net: Net, path: str):
     lines.append(f"snap {snap}")
     if getattr(net, "batch_size", 1) != 1:
         lines.append(f"batch {int(net.batch_size)}")
-    if any(s.matrix in ("procedural", "sparse_init") for s in net.syns) or any(c.model == "poisson_exp" for c in net.css) or any(p.model == "poisson" for p in net.pops):
+    if any(s.matrix in ("procedural", "sparse_init") for s in net.syns) or any(c.model == "poisson_exp" for c in net.css) or any(p.model == "poisson" for p in net.pops) \
+            or any(s.wum == "stochastic" for s in net.syns):
         lines.append(f"seed {int(net.seed)}")        # procedural matrices and Poisson sources draw from the model's seed
     for kind, group, param, step, value in net.dynamic:
         lines.append(f"dynamic {kind} {group} {param} {int(step)} {float(value)!r}")
@@ -208,6 +209,8 @@ def write_netspec(net: Net, path: str):
             w = ("stdp" if s.wum == "stdp_additive" else s.wum) + " " + " ".join(repr(float(s.wum_params[k])) for k in STDP_PARAMS)
         elif s.wum == "static_graded":
             w = f"static_graded {float(s.wum_params['Epre'])!r} {float(s.wum_params['Vslope'])!r}"
+        elif s.wum == "stochastic":        # a model of the test driver that draws a random number per synaptic event
+            w = f"stochastic {float(s.wum_params['pRelease'])!r}"
         elif s.wum == "leaky_graded":      # a model of the test driver with synapse dynamics code (runs for every synapse every step)
             w = f"leaky_graded {float(s.wum_params['Vmid'])!r} {float(s.wum_params['decay'])!r}"
         else:

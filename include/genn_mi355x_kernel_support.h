@@ -150,11 +150,13 @@ __device__ inline void philox4x32(uint32_t c0, uint32_t c1, uint32_t c2, uint32_
     o0 = c0; o1 = c1; o2 = c2; o3 = c3;
 }
 
-__device__ inline Rng rngBegin(unsigned long long seed, uint32_t stream, uint32_t element, unsigned long long step)
+// (element: a neuron of a batch, or a synapse of a batch — up to 2^44 of them; its high bits travel above the stream number)
+__device__ inline Rng rngBegin(unsigned long long seed, uint32_t stream, unsigned long long element, unsigned long long step)
 {
     Rng r;
     r.k0 = (uint32_t)seed; r.k1 = (uint32_t)(seed >> 32);
-    r.element = element; r.stepLow = (uint32_t)step; r.stepHighAndCall = (uint32_t)(step >> 32) << 16; r.stream = stream;
+    r.element = (uint32_t)element; r.stepLow = (uint32_t)step; r.stepHighAndCall = (uint32_t)(step >> 32) << 16;
+    r.stream = stream | ((uint32_t)(element >> 32) << 20);
     r.w0 = r.w1 = r.w2 = r.w3 = 0; r.left = 0;
     return r;
 }

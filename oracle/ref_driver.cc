@@ -173,6 +173,21 @@ public:
 };
 IMPLEMENT_SNIPPET(LeakyGraded);
 
+// Synapses that release with a probability: random numbers in weight-update code (what a user writes for stochastic
+// transmission; cf. tests/features/test_rng.py, which draws in neuron code).
+class StochasticPulse : public WeightUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(StochasticPulse);
+    SET_PARAMS({"pRelease"});
+    SET_VARS({{"g", "scalar", VarAccess::READ_ONLY}});
+    SET_PRE_SPIKE_SYN_CODE(
+        "if(gennrand_uniform() < pRelease) {\n"
+        "    addToPost(g);\n"
+        "}\n");
+};
+IMPLEMENT_SNIPPET(StochasticPulse);
+
 // Current source fed from a host-pregenerated array; the driver rewrites the N-element
 // window before every step, so the injected value at step s is noise[s*N + id].
 class ArrayNoise : public CurrentSourceModels::Base
@@ -292,7 +307,7 @@ int main(int argc, char *argv[])
                     if(s.wum == "static_init") { ls >> s.initSnippet; const int np = (s.initSnippet == "Constant") ? 1 : 2; s.wumP.resize(np); for(auto &c : s.wumP) ls >> c; }
                     if(s.wum == "static_delay") { ls >> s.maxDenDelay; }
                     else if(s.wum == "stdp_trace" || s.wum == "stdp") { s.wumP.resize(6); for(auto &c : s.wumP) ls >> c; }
-                    else if(s.wum == "static_const") { s.wumP.resize(1); ls >> s.wumP[0]; }
+                    else if(s.wum == "static_const" || s.wum == "stochastic") { s.wumP.resize(1); ls >> s.wumP[0]; }
                     else if(s.wum == "static_graded" || s.wum == "leaky_graded") { s.wumP.resize(2); ls >> s.wumP[0] >> s.wumP[1]; }
                     else if(s.wum != "static" && s.wum != "static_reverse" && s.wum != "static_init" && s.wum != "timing_copy") throw std::runtime_error("wum " + s.wum);
                     ls >> s.psm;
@@ -366,6 +381,9 @@ int main(int argc, char *argv[])
             }
             else if(s.wum == "static_reverse") {
                 wum = initWeightUpdate<StaticPulseReverse>({}, {{"g", uninitialisedVar()}});
+            }
+            else if(s.wum == "stochastic") {
+                wum = initWeightUpdate<StochasticPulse>({{"pRelease", s.wumP.at(0)}}, {{"g", uninitialisedVar()}});
             }
             else if(s.wum == "leaky_graded") {
                 wum = initWeightUpdate<LeakyGraded>({{"Vmid", s.wumP.at(0)}, {"decay", s.wumP.at(1)}}, {{"g", uninitialisedVar()}, {"x", 0.0}}, {}, {},

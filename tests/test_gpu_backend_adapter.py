@@ -386,6 +386,48 @@ def test_generated_kernels_with_simulation_random_numbers():
     assert out_ref > 2000 and abs(out_got - out_ref) <= 0.05 * out_ref, f"{out_got} output spikes against {out_ref}"
 
 
+def test_generated_kernels_with_random_numbers_in_weight_update_code():
+    """`gennrand_uniform()` in presynaptic spike code (synapses that release with probability 0.4).  No backend of the reference
+    pins this — its CPU backend refuses the model ("Undefined identifier" for gennrand_* in weight-update code), its SIMT backends
+    each draw from generators of their own — so the check is against what the mathematics fixes: a population whose threshold is
+    out of reach integrates its input linearly, so its mean potential must equal that of a twin network with static synapses of
+    0.4 times the weight (the expectation); synapses with release probability 1 must reproduce the twin's static projection
+    spike for spike; neuron by neuron the stochastic input must differ from its expectation; and the same seed must give
+    the same result again."""
+    from genn_amd import configs
+    results = []
+    for twin, repeat in ((False, 0), (False, 1), (True, 0)):
+        net = configs.stochastic_synapses(twin=twin)
+        net.snap = 100
+        tmp = tempfile.mkdtemp(prefix="adapter_stochastic_")
+        try:
+            spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+            for d in (work, out):
+                os.makedirs(d)
+            write_netspec(net, spec)
+            print(f"adapter stochastic synapses (twin={twin}): running {DRIVER}", flush=True)
+            res = subprocess.run([DRIVER, spec, work, out] + (["--kernels=generated"] if twin else []), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+            assert res.returncode == 0, res.stdout[-3000:]
+            code = open(os.path.join(work, net.name + "_CODE", "synapseUpdate.cc")).read()
+            assert "__global__" in code and (("gennmi_kernel::rngUniform(gennmiRng)" in code) != twin)
+            results.append({"C": np.fromfile(os.path.join(out, "C.spikes.u32"), np.uint32).reshape(-1, 2),
+                            "A": np.fromfile(os.path.join(out, "A.spikes.u32"), np.uint32).reshape(-1, 2),
+                            "V": np.fromfile(os.path.join(out, "B.V.f32"), np.float32).reshape(net.steps // net.snap, -1)})
+        finally:
+            shutil.rmtree(tmp, ignore_errors=True)
+    first, again, twin = results
+    # (the same draws, added up in whatever order the atomics came: equal up to the rounding of reordered sums)
+    assert np.allclose(first["V"], again["V"], rtol=1e-5, atol=0.0) and np.array_equal(first["C"], again["C"]), "the same seed gave another result"
+    assert len(first["A"]) > 5000 and np.array_equal(first["A"], twin["A"])
+    assert len(twin["C"]) > 500 and np.array_equal(first["C"], twin["C"]), "release probability 1 must behave like a static synapse"
+    rest = -60.0
+    for k in range(first["V"].shape[0]):
+        got, want = first["V"][k].astype(np.float64) - rest, twin["V"][k].astype(np.float64) - rest
+        assert want.mean() > 0.5
+        assert abs(got.mean() - want.mean()) <= 0.02 * want.mean(), f"snapshot {k}: mean depolarisation {got.mean():.4f} against {want.mean():.4f}"
+        assert np.abs(got - want).std() > 0.01 * want.mean(), "the stochastic input equals its expectation neuron by neuron"
+
+
 def test_adapter_device_initialisation_matches_host_layer():
     """Preferences::deviceInitialisation through GeNN's generator and Runtime: SPARSE matrices built by FixedProbability
     (with and without autapses) and FixedNumberPostWithReplacement with Uniform, Normal, Constant and constant-parameter
