@@ -125,9 +125,6 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         [&](auto &n)
         {
             const auto &arch = n.getArchetype();
-            if(arch.isPrevSpikeTimeRequired() || arch.isSpikeEventTimeRequired() || arch.isPrevSpikeEventTimeRequired()) {
-                notGenerated("previous spike times and spike-like event times (population '" + arch.getName() + "')");
-            }
             maxEventGroups = std::max(maxEventGroups, n.getMergedSpikeEventGroups().size());
 
             const size_t firstBlock = table.numBlocks;
@@ -209,7 +206,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                 }
                 n.generateSpikeEvents(
                     groupEnv,
-                    [&eventOffset, &eventCountIndex, recordEvents, batchSize](EnvironmentExternalBase &env, NeuronUpdateGroupMerged::SynSpikeEvent &e)
+                    [&eventOffset, &eventCountIndex, &arch, recordEvents, batchSize](EnvironmentExternalBase &env, NeuronUpdateGroupMerged::SynSpikeEvent &e)
                     {
                         const std::string k = std::to_string(e.getIndex());
                         const std::string region = "gennmiAgg + (size_t)2 * gridDim.x * (gridDim.y * " + std::to_string(e.getIndex() + 1) + "u + blockIdx.y)";
@@ -219,6 +216,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                             env.printLine("gennmi_kernel::recordBallot(&$(_record_spk_event)[((size_t)recordingTimestep * " + std::to_string(batchSize) + "u + $(batch)) * numRecordingWords], "
                                           "$(id), $(id) < $(num_neurons), eventSlot" + k + ".ballot);");
                         }
+                        if(arch.isSpikeEventTimeRequired()) { env.printLine("if(gennmiEvent" + k + ") { $(_set)[" + eventOffset + "$(id)] = $(t); }"); }
                         env.print("if(eventSlot" + k + ".ok)");
                         CodeStream::Scope b3(env.getStream());
                         env.printLine("if(gennmiEvent" + k + ") { $(_spk_event)[" + eventOffset + "eventSlot" + k + ".position] = $(id); }");
@@ -237,6 +235,59 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                 });
         });
     }
+
+    // Previous spike (and event) times: every neuron in last step's queue gets prev_st = t - dt, in a kernel that runs before
+    // the ring pointers move on (backendSIMT.cc:320-368, 1897-1925)
+    std::ostringstream prevStream, prevArgs, prevParams;
+    BlockTable prevTable;
+    if(!modelMerged.getMergedNeuronPrevSpikeTimeUpdateGroups().empty()) {
+        CodeStream prev(prevStream);
+        EnvironmentLibrary prevLib(prev, StandardLibrary::getMathsFunctions());
+        EnvironmentExternal prevEnv(prevLib);
+        prevEnv.add(model.getTimePrecision().addConst(), "t", "t");
+        prevEnv.add(Type::Uint32.addConst(), "batch", (batchSize > 1) ? "blockIdx.y" : "0");
+        prevEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
+        modelMerged.genMergedNeuronPrevSpikeTimeUpdateGroups(
+            *this, memorySpaces,
+            [&](auto &n)
+            {
+                const auto &arch = n.getArchetype();
+                const size_t firstBlock = prevTable.numBlocks;
+                for(size_t g = 0; g < n.getGroups().size(); g++) {
+                    const size_t blocks = (n.getGroups()[g].get().getNumNeurons() + 255) / 256;
+                    for(size_t b = 0; b < blocks; b++) { prevTable.add(g, b * 256, b, blocks); }
+                }
+                const std::string structArray = "mergedNeuronPrevSpikeTimeUpdateGroup" + std::to_string(n.getIndex());
+                prevArgs << ", d_" << structArray;
+                prevParams << ", const MergedNeuronPrevSpikeTimeUpdateGroup" << n.getIndex() << " *" << structArray;
+                prevEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << prevTable.numBlocks << "u)";
+                CodeStream::Scope b(prevEnv.getStream());
+                prevEnv.getStream() << "const gennmi_kernel::BlockEntry entry = gennmiPrevSpikeTimeBlocks[blockIdx.x];" << std::endl;
+                prevEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
+                prevEnv.getStream() << "const unsigned int id = entry.firstId + threadIdx.x;" << std::endl;
+                EnvironmentGroupMergedField<NeuronPrevSpikeTimeUpdateGroupMerged> groupEnv(prevEnv, n);
+                buildStandardEnvironment(groupEnv, batchSize);
+                groupEnv.add(Type::Uint32.addConst(), "id", "id");
+                if(arch.isDelayRequired()) {
+                    groupEnv.printLine("const unsigned int lastSlot = *$(_spk_que_ptr)" + ((batchSize > 1) ? " + ($(batch) * " + std::to_string(arch.getNumDelaySlots()) + "u)" : std::string("")) + ";");
+                    groupEnv.printLine("const unsigned int lastOffset = lastSlot * $(num_neurons);");
+                }
+                auto stamp = [&arch, batchSize](EnvironmentExternalBase &env, bool trueSpike)
+                {
+                    const std::string suffix = trueSpike ? "" : "_event", time = trueSpike ? "st" : "set";
+                    if(trueSpike ? arch.isSpikeDelayRequired() : arch.isSpikeEventDelayRequired()) {
+                        env.printLine("if($(id) < $(_spk_cnt" + suffix + ")[lastSlot]) { $(_prev_" + time + ")[lastOffset + $(_spk" + suffix + ")[lastOffset + $(id)]] = $(t) - $(dt); }");
+                    }
+                    else {
+                        const std::string offset = (batchSize > 1) ? "$(_batch_offset) + " : "";
+                        env.printLine("if($(id) < $(_spk_cnt" + suffix + ")[$(batch)]) { $(_prev_" + time + ")[" + offset + "$(_spk" + suffix + ")[" + offset + "$(id)]] = $(t) - $(dt); }");
+                    }
+                };
+                if(arch.isPrevSpikeTimeRequired()) { n.generateSpikes(groupEnv, [&stamp](EnvironmentExternalBase &env) { stamp(env, true); }); }
+                if(arch.isPrevSpikeEventTimeRequired()) { n.generateSpikeEvents(groupEnv, [&stamp](EnvironmentExternalBase &env) { stamp(env, false); }); }
+            });
+    }
+    const bool anyPrevTimes = prevTable.numBlocks > 0;
 
     // Populations with delay slots: their ring pointer moves on before the update (backendSIMT.cc:372-401; one thread per group).
     // Without delay slots that kernel would only clear counts that the compaction overwrites anyway, and is left out.
@@ -270,12 +321,19 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         modelMerged.genMergedNeuronSpikeQueueUpdateStructs(os, *this);
         modelMerged.genMergedNeuronSpikeQueueUpdateHostStructArrayPush(os, *this);
     }
+    if(anyPrevTimes) {
+        modelMerged.genMergedNeuronPrevSpikeTimeUpdateStructs(os, *this);
+        modelMerged.genMergedNeuronPrevSpikeTimeUpdateHostStructArrayPush(os, *this);
+    }
     preambleHandler(os);
     for(const auto &n : modelMerged.getMergedNeuronUpdateGroups()) {
         genDeviceStructArray(decl, upload, *this, n, "NeuronUpdate");
     }
     if(anyDelaySlots) {
         for(const auto &n : modelMerged.getMergedNeuronSpikeQueueUpdateGroups()) { genDeviceStructArray(decl, upload, *this, n, "NeuronSpikeQueueUpdate"); }
+    }
+    if(anyPrevTimes) {
+        for(const auto &n : modelMerged.getMergedNeuronPrevSpikeTimeUpdateGroups()) { genDeviceStructArray(decl, upload, *this, n, "NeuronPrevSpikeTimeUpdate"); }
     }
 
     os << declStream.str();
@@ -301,6 +359,12 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         }
     }
     os << std::endl;
+    if(anyPrevTimes) {
+        os << "__device__ const gennmi_kernel::BlockEntry gennmiPrevSpikeTimeBlocks[] = {" << std::endl << prevTable.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+        os << "__global__ __launch_bounds__(256) void gennmiPrevSpikeTimeKernel(float t" << prevParams.str() << ")";
+        CodeStream::Scope b(os);
+        os << prevStream.str();
+    }
     if(anyDelaySlots) {
         os << "__global__ void gennmiSpikeQueueUpdateKernel(" << queueParams.str() << ")";
         CodeStream::Scope b(os);
@@ -320,6 +384,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     {
         CodeStream::Scope b(os);
         os << "gennmiEnsureFinalised();" << std::endl;
+        if(anyPrevTimes) { os << "gennmiPrevSpikeTimeKernel<<<dim3(" << prevTable.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << prevArgs.str() << ");" << std::endl; }
         if(anyDelaySlots) { os << "gennmiSpikeQueueUpdateKernel<<<dim3(1), dim3(64), 0, 0>>>(" << queueArgs.str() << ");" << std::endl; }
         if(table.numBlocks > 0) {
             // the tag of a launch: differs from one launch to the next, never 0 (the look-back words start out zero)

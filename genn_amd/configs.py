@@ -413,7 +413,7 @@ def stochastic_synapses(n_a=400, n_b=300, steps=600, seed=71, dt=1.0, twin=False
     return net
 
 
-def custom_models(n_a=300, n_b=200, steps=300, seed=41, dt=1.0):
+def custom_models(n_a=300, n_b=200, steps=300, seed=41, dt=1.0, timing="timing_copy"):
     """A network of models that are NOT built into GeNN or into the device library — what a user writes with the model
     API: LIF neurons with a spike-triggered adaptation variable ("lifa": the built-in LIF plus A, which decays every step,
     is subtracted from the input and grows by dA at each spike), and a weight update model with a presynaptic and a
@@ -434,7 +434,7 @@ def custom_models(n_a=300, n_b=200, steps=300, seed=41, dt=1.0):
         g = (lo + (hi - lo) * rng.uniform(seed, stream + 2, 0, n_src * stride)).astype(np.float32).reshape(n_src, stride)
         return Syn(name, src, trg, psm="expcurr", tau=tau, row_stride=stride, row_length=row_length, ind=ind, g=g, wum=wum)
 
-    net.syns.append(sparse("AB_timing", "A", "B", n_a, n_b, 30, 10, 0.0, 0.12, "timing_copy", 5.0))
+    net.syns.append(sparse("AB_timing", "A", "B", n_a, n_b, 30, 10, 0.0, 0.12, timing, 5.0))
     net.syns.append(sparse("BA_inhibit", "B", "A", n_b, n_a, 24, 20, -0.5, -0.1, "static", 10.0))
-    net.syns.append(sparse("AA_timing", "A", "A", n_a, n_a, 70, 30, 0.0, 0.02, "timing_copy", 5.0))
+    net.syns.append(sparse("AA_timing", "A", "A", n_a, n_a, 70, 30, 0.0, 0.02, timing, 5.0))
     return net

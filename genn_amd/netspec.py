@@ -198,7 +198,7 @@ def write_netspec(net: Net, path: str):
             snippet, params = s.g_init
             order = {"Constant": ("constant",), "Uniform": ("min", "max"), "Normal": ("mean", "sd")}[snippet]
             w = f"static_init {snippet} " + " ".join(repr(float(params[k])) for k in order)
-        elif s.wum in ("static", "static_reverse", "timing_copy"):
+        elif s.wum in ("static", "static_reverse", "timing_copy", "prev_timing"):
             w = s.wum
         elif s.wum == "static_const":
             w = f"static_const {float(s.wum_params['g'])!r}"
@@ -219,7 +219,7 @@ def write_netspec(net: Net, path: str):
         opts = (" hint_pre" if s.hint_pre else "") + (f" tps {s.threads_per_spike}" if s.threads_per_spike > 1 else "")
         if s.axonal_delay_steps:
             opts += f" axonal_delay {int(s.axonal_delay_steps)}"
-        if s.wum in ("stdp_trace", "stdp_additive", "timing_copy"):
+        if s.wum in ("stdp_trace", "stdp_additive", "timing_copy", "prev_timing"):
             mask = np.arange(s.row_stride)[None, :] < s.row_length[:, None]
             col = s.col_stride or int(np.bincount(s.ind[mask], minlength=net.pop(s.trg).n).max())
             opts += f" col_stride {max(1, col)}"

@@ -157,6 +157,21 @@ public:
 };
 IMPLEMENT_SNIPPET(TimingCopy);
 
+// The same idea with the times GeNN keeps itself: a presynaptic spike delivers g and writes the time of the target's spike
+// BEFORE its latest one into the row's synapses, a postsynaptic spike writes the source's into its column (prev_st_post /
+// prev_st_pre: both populations then keep previous spike times, updated by a kernel of their own on the SIMT backends).
+class PrevTiming : public WeightUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(PrevTiming);
+    SET_VARS({{"g", "scalar", VarAccess::READ_ONLY}, {"wPre", "scalar"}, {"wPost", "scalar"}});
+    SET_PRE_SPIKE_SYN_CODE(
+        "addToPost(g);\n"
+        "wPost = prev_st_post;\n");
+    SET_POST_SPIKE_SYN_CODE("wPre = prev_st_pre;\n");
+};
+IMPLEMENT_SNIPPET(PrevTiming);
+
 // Weight update model that runs EVERY step for EVERY synapse (synapse dynamics code), after the continuous models of
 // tests/features/test_synapse_dynamics*.py: each synapse low-pass filters how far its source's membrane potential is above a
 // midpoint and delivers g times that trace, spike or no spike.
@@ -309,7 +324,7 @@ int main(int argc, char *argv[])
                     else if(s.wum == "stdp_trace" || s.wum == "stdp") { s.wumP.resize(6); for(auto &c : s.wumP) ls >> c; }
                     else if(s.wum == "static_const" || s.wum == "stochastic") { s.wumP.resize(1); ls >> s.wumP[0]; }
                     else if(s.wum == "static_graded" || s.wum == "leaky_graded") { s.wumP.resize(2); ls >> s.wumP[0] >> s.wumP[1]; }
-                    else if(s.wum != "static" && s.wum != "static_reverse" && s.wum != "static_init" && s.wum != "timing_copy") throw std::runtime_error("wum " + s.wum);
+                    else if(s.wum != "static" && s.wum != "static_reverse" && s.wum != "static_init" && s.wum != "timing_copy" && s.wum != "prev_timing") throw std::runtime_error("wum " + s.wum);
                     ls >> s.psm;
                     if(s.psm == "expcurr") { s.psmP.resize(1); ls >> s.psmP[0]; }
                     else if(s.psm != "deltacurr") throw std::runtime_error("psm " + s.psm);
@@ -388,6 +403,9 @@ int main(int argc, char *argv[])
             else if(s.wum == "leaky_graded") {
                 wum = initWeightUpdate<LeakyGraded>({{"Vmid", s.wumP.at(0)}, {"decay", s.wumP.at(1)}}, {{"g", uninitialisedVar()}, {"x", 0.0}}, {}, {},
                                                     {{"Vpre", createVarRef(popByName.at(s.src)->ng, "V")}}, {});
+            }
+            else if(s.wum == "prev_timing") {
+                wum = initWeightUpdate<PrevTiming>({}, {{"g", uninitialisedVar()}, {"wPre", -1.0}, {"wPost", -1.0}});
             }
             else if(s.wum == "timing_copy") {
                 wum = initWeightUpdate<TimingCopy>({}, {{"g", uninitialisedVar()}, {"wPre", 0.0}, {"wPost", 0.0}}, {{"sPre", 0.0}}, {{"sPost", 0.0}});
@@ -575,7 +593,7 @@ int main(int argc, char *argv[])
             for(auto &s : syns) {
                 const auto *sgi = static_cast<const SynapseGroupInternal*>(s.sg);
                 fm << s.name << " " << sgi->getFusedPSTarget().getName() << std::endl;
-                if(s.wum == "stdp_trace" || s.wum == "stdp" || s.wum == "timing_copy") {
+                if(s.wum == "stdp_trace" || s.wum == "stdp" || s.wum == "timing_copy" || s.wum == "prev_timing") {
                     auto *cl = rt.getArray(*s.sg, "colLength"); auto *rm = rt.getArray(*s.sg, "remap");
                     cl->pullFromDevice(); rm->pullFromDevice();
                     appendFile(out + "/" + s.name + ".colLength.u32", cl->getHostPointer<uint32_t>(), cl->getCount());
@@ -620,12 +638,14 @@ int main(int argc, char *argv[])
                     auto *a = pulled(rt.getArray(*s.sg, "x"));
                     for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + ".x.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
                 }
-                if(s.wum == "timing_copy") {
+                if(s.wum == "timing_copy" || s.wum == "prev_timing") {
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
                     for(const char *var : {"wPre", "wPost"}) {
                         auto *a = pulled(rt.getArray(*s.sg, var));
                         for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + "." + var + ".f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
                     }
+                }
+                if(s.wum == "timing_copy") {
                     for(const char *var : {"sPre", "sPost"}) {
                         auto *a = pulled(rt.getArray(*s.sg, var));
                         appendFile(out + "/" + s.name + "." + var + ".f32", a->getHostPointer<float>(), a->getCount());

@@ -86,6 +86,14 @@ def synapse_dynamics_small():
     return configs.synapse_dynamics(), 25
 
 
+def prev_times_small():
+    # weight-update code that reads the PREVIOUS spike times of both ends (prev_st_pre, prev_st_post): populations then keep
+    # them, updated before each step from the last step's spike queue
+    net = configs.custom_models(timing="prev_timing")
+    net.name = "prev_times"
+    return net, 25
+
+
 def dynamic_small():
     # parameters changed while the model runs (setParamDynamic + Runtime::setDynamicParamValue): the drive of the
     # excitatory population twice, the threshold of the inhibitory one, and the time constant of a postsynaptic model, whose
@@ -105,7 +113,7 @@ def potjans_poisson_net():
 
 # cases the reference's CPU backend pins directly (fixtures) and that the oracle, a restatement of the built-in models
 # with fixed parameters, does not cover
-REFERENCE_ONLY = {"stdp_delay_small", "custom_small", "custom_batch1_small", "dynamic_small", "poisson_input_small", "synapse_dynamics_small"}
+REFERENCE_ONLY = {"stdp_delay_small", "custom_small", "custom_batch1_small", "dynamic_small", "poisson_input_small", "synapse_dynamics_small", "prev_times_small"}
 
-CASES = {"stdp_delay_small": stdp_delay_small, "synapse_dynamics_small": synapse_dynamics_small, "poisson_input_small": poisson_input_small, "custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+CASES = {"prev_times_small": prev_times_small, "stdp_delay_small": stdp_delay_small, "synapse_dynamics_small": synapse_dynamics_small, "poisson_input_small": poisson_input_small, "custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
          "stdp_small": stdp_small, "conv_small": conv_small}

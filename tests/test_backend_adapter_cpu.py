@@ -157,7 +157,7 @@ def _generate_with(case, *options):
     return net, tmp, os.path.join(work, net.name + "_CODE"), res
 
 
-@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
+@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
                                            ("va_small", ("--dynamic=neuron:E.Ioffset",))])
 def test_generated_kernels_are_chosen_and_build(case, options):
     """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the runner then holds device
@@ -180,6 +180,10 @@ def test_generated_kernels_are_chosen_and_build(case, options):
             # the extra state variable and the weight-update variables are in the kernels under the reference's names
             assert "group->A[id]" in neuron and "sPreOutSynWUMPre" in neuron and "sPostInSynWUMPost" in neuron
             assert "group->wPost[idSyn] = group->sPost[idPost]" in synapse and "group->wPre[rowMajorIndex] = group->sPre[idPre]" in synapse
+        if case == "prev_times_small":
+            # previous spike times: a kernel of its own stamps last step's spikes before the update
+            assert "gennmiPrevSpikeTimeKernel<<<" in neuron and neuron.index("gennmiPrevSpikeTimeKernel<<<") < neuron.index("gennmiNeuronUpdateKernel<<<")
+            assert "group->prevST[" in neuron
         if case == "graded_small":
             # spike-like events: a queue per condition, compacted in order like the true spikes and recorded from the ballot
             assert "gennmiEvent0 = true" in neuron and "eventSlot0 = gennmi_kernel::orderedSlot(gennmiEvent0" in neuron and "recordSpkEvent" in neuron
