@@ -571,13 +571,14 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const auto matrix = arch.getMatrixType();
                     const bool sparse = (matrix & SynapseMatrixConnectivity::SPARSE);
                     const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
-                    if(!sparse && !dense) { notGenerated("connectivity other than SPARSE and DENSE (projection '" + arch.getName() + "')"); }
+                    const bool toeplitz = (matrix & SynapseMatrixConnectivity::TOEPLITZ);
+                    if(!sparse && !dense && !toeplitz) { notGenerated("connectivity other than SPARSE, DENSE and TOEPLITZ (projection '" + arch.getName() + "')"); }
                     if(!arch.isPreSpikeRequired() && !arch.isPreSpikeEventRequired()) { return; }
 
                     const size_t firstBlock = pre.table.numBlocks;
                     for(size_t g = 0; g < s.getGroups().size(); g++) {
                         const auto &sg = s.getGroups()[g].get();
-                        const size_t rowLen = sparse ? getSynapticMatrixRowStride(sg) : sg.getTrgNeuronGroup()->getNumNeurons();
+                        const size_t rowLen = (sparse || toeplitz) ? getSynapticMatrixRowStride(sg) : sg.getTrgNeuronGroup()->getNumNeurons();
                         const size_t chunks = (rowLen + 63) / 64;
                         // enough wavefronts for ~1.5 % of the source population firing in one step, at most 128 work-groups
                         const size_t blocks = std::clamp<size_t>((sg.getSrcNeuronGroup()->getNumNeurons() * chunks + 255) / 256, 1, 128);
@@ -594,7 +595,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
                     EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> groupEnv(funcEnv, s);
                     buildStandardEnvironment(groupEnv, batchSize);
-                    groupEnv.printLine(std::string("const unsigned int rowSpan = ") + (sparse ? "$(_row_stride)" : "$(num_post)") + ";");
+                    groupEnv.printLine(std::string("const unsigned int rowSpan = ") + ((sparse || toeplitz) ? "$(_row_stride)" : "$(num_post)") + ";");
                     groupEnv.getStream() << "const unsigned int chunksPerRow = (rowSpan + 63u) / 64u;" << std::endl;
                     groupEnv.getStream() << "const unsigned int numWaves = entry.blocksInGroup * 4u;" << std::endl;
                     // the queue of spike-like events first, then the true spikes (the reference's order, backendSIMT.cc:745-760);
@@ -615,6 +616,51 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         synEnv.getStream() << "const unsigned int j = (unsigned int)(item % chunksPerRow) * 64u + (threadIdx.x & 63u);" << std::endl;
                         synEnv.printLine("const unsigned int idPre = $(_src_spk" + suffix + ")[" + s.getPreVarIndex(preDelay, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "spike") + "];");
                         synEnv.add(Type::Uint32.addConst(), "id_pre", "idPre");
+                        if(toeplitz) {
+                            // A row of a Toeplitz matrix is the connectivity snippet's diagonal build code run for (presynaptic
+                            // neuron, diagonal): lane j of an item takes diagonal j, and the snippet's addSynapse(idPost, kernel
+                            // indices...) becomes the weight-update code with those values (presynapticUpdateStrategySIMT.cc:784-917)
+                            std::ostringstream updateStream;
+                            CodeStream update(updateStream);
+                            {
+                                CodeStream::Scope bu(update);
+                                EnvironmentExternal updateEnv(synEnv, update);
+                                updateEnv.add(Type::Uint32.addConst(), "id_post", "idPost", {updateEnv.addInitialiser("const unsigned int idPost = $(0);")});
+                                for(size_t i = 0; i < arch.getKernelSize().size(); i++) {
+                                    const std::string iStr = std::to_string(i);
+                                    updateEnv.add(Type::Uint32.addConst(), "id_kernel_" + iStr, "idKernel" + iStr,
+                                                  {updateEnv.addInitialiser("const unsigned int idKernel" + iStr + " = $(" + std::to_string(i + 1) + ");")});
+                                }
+                                updateEnv.add(Type::getAddToPrePostDelay(s.getScalarType()), "addToPostDelay",
+                                              "gennmi_kernel::addScalar(&$(_den_delay)[" + s.getPostDenDelayIndex(batchSize, "$(id_post)", "$(1)") + "], $(0))");
+                                updateEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPost",
+                                              "gennmi_kernel::addScalar(&$(_out_post)[" + s.getPostISynIndex(batchSize, "$(id_post)") + "], $(0))");
+                                updateEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
+                                              "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(batchSize, "$(id_pre)") + "], $(0))");
+                                if(trueSpike) { s.generateSpikeUpdate(*this, updateEnv, batchSize, dt); }
+                                else { s.generateSpikeEventUpdate(*this, updateEnv, batchSize, dt); }
+                            }
+                            synEnv.print("if(j < $(_row_stride))");
+                            CodeStream::Scope bt(synEnv.getStream());
+                            EnvironmentExternal diagEnv(synEnv);
+                            diagEnv.add(Type::Uint32.addConst(), "id_diag", "j");
+                            const auto addSynapseType = Type::ResolvedType::createFunction(
+                                Type::Void, std::vector<Type::ResolvedType>{1ull + arch.getKernelSize().size(), Type::Uint32});
+                            s.generateToeplitzConnectivity(
+                                diagEnv,
+                                [addSynapseType](auto &env, auto &errorHandler)
+                                {
+                                    env.define(Transpiler::Token{Transpiler::Token::Type::IDENTIFIER, "addSynapse", 0}, addSynapseType, errorHandler);
+                                    env.define(Transpiler::Token{Transpiler::Token::Type::IDENTIFIER, "id_pre", 0}, Type::Uint32.addConst(), errorHandler);
+                                },
+                                [addSynapseType, &updateStream](auto &env, auto generateBody)
+                                {
+                                    EnvironmentExternal bodyEnv(env);
+                                    bodyEnv.add(addSynapseType, "addSynapse", updateStream.str());
+                                    generateBody(bodyEnv);
+                                });
+                            return;
+                        }
                         const auto indexType = getSynapseIndexType(s);
                         const std::string indexTypeName = indexType.getName();
                         if(sparse) {

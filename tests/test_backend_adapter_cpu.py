@@ -157,7 +157,7 @@ def _generate_with(case, *options):
     return net, tmp, os.path.join(work, net.name + "_CODE"), res
 
 
-@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
+@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("conv_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
                                            ("va_small", ("--dynamic=neuron:E.Ioffset",))])
 def test_generated_kernels_are_chosen_and_build(case, options):
     """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the runner then holds device
@@ -180,6 +180,9 @@ def test_generated_kernels_are_chosen_and_build(case, options):
             # the extra state variable and the weight-update variables are in the kernels under the reference's names
             assert "group->A[id]" in neuron and "sPreOutSynWUMPre" in neuron and "sPostInSynWUMPost" in neuron
             assert "group->wPost[idSyn] = group->sPost[idPost]" in synapse and "group->wPre[rowMajorIndex] = group->sPre[idPre]" in synapse
+        if case == "conv_small":
+            # TOEPLITZ connectivity: the snippet's diagonal build code inside the presynaptic walk, its addSynapse become the update
+            assert "const unsigned int idPost = " in synapse and "idKernel0" in synapse and "idKernel3" in synapse
         if case == "prev_times_small":
             # previous spike times: a kernel of its own stamps last step's spikes before the update
             assert "gennmiPrevSpikeTimeKernel<<<" in neuron and neuron.index("gennmiPrevSpikeTimeKernel<<<") < neuron.index("gennmiNeuronUpdateKernel<<<")
@@ -239,7 +242,7 @@ def test_generated_kernels_take_the_batch_from_the_grid():
         shutil.rmtree(tmp, ignore_errors=True)
 
 
-@pytest.mark.parametrize("case, what", [("conv_small", "connectivity")])
+@pytest.mark.parametrize("case, what", [("dense_small", "connectivity")])
 def test_generated_kernels_say_what_they_do_not_cover(case, what):
     """Asked to generate kernels for a feature only the device library implements, the backend names the feature."""
     net, tmp, code, res = _generate_with(case, "--kernels=generated")
