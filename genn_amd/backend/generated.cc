@@ -570,15 +570,17 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const auto &arch = s.getArchetype();
                     const auto matrix = arch.getMatrixType();
                     const bool sparse = (matrix & SynapseMatrixConnectivity::SPARSE);
-                    const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
+                    const bool dense = (matrix & SynapseMatrixConnectivity::DENSE);
                     const bool toeplitz = (matrix & SynapseMatrixConnectivity::TOEPLITZ);
-                    if(!sparse && !dense && !toeplitz) { notGenerated("connectivity other than SPARSE, DENSE and TOEPLITZ (projection '" + arch.getName() + "')"); }
+                    const bool bitmask = (matrix & SynapseMatrixConnectivity::BITMASK);
+                    if(!sparse && !dense && !toeplitz && !bitmask) { notGenerated("PROCEDURAL connectivity (projection '" + arch.getName() + "')"); }
+                    if(matrix & SynapseMatrixWeight::PROCEDURAL) { notGenerated("weights regenerated from their initialisation snippet (projection '" + arch.getName() + "')"); }
                     if(!arch.isPreSpikeRequired() && !arch.isPreSpikeEventRequired()) { return; }
 
                     const size_t firstBlock = pre.table.numBlocks;
                     for(size_t g = 0; g < s.getGroups().size(); g++) {
                         const auto &sg = s.getGroups()[g].get();
-                        const size_t rowLen = (sparse || toeplitz) ? getSynapticMatrixRowStride(sg) : sg.getTrgNeuronGroup()->getNumNeurons();
+                        const size_t rowLen = (sparse || toeplitz || bitmask) ? getSynapticMatrixRowStride(sg) : sg.getTrgNeuronGroup()->getNumNeurons();
                         const size_t chunks = (rowLen + 63) / 64;
                         // enough wavefronts for ~1.5 % of the source population firing in one step, at most 128 work-groups
                         const size_t blocks = std::clamp<size_t>((sg.getSrcNeuronGroup()->getNumNeurons() * chunks + 255) / 256, 1, 128);
@@ -595,7 +597,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
                     EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> groupEnv(funcEnv, s);
                     buildStandardEnvironment(groupEnv, batchSize);
-                    groupEnv.printLine(std::string("const unsigned int rowSpan = ") + ((sparse || toeplitz) ? "$(_row_stride)" : "$(num_post)") + ";");
+                    groupEnv.printLine(std::string("const unsigned int rowSpan = ") + ((sparse || toeplitz || bitmask) ? "$(_row_stride)" : "$(num_post)") + ";");
                     groupEnv.getStream() << "const unsigned int chunksPerRow = (rowSpan + 63u) / 64u;" << std::endl;
                     groupEnv.getStream() << "const unsigned int numWaves = entry.blocksInGroup * 4u;" << std::endl;
                     // the queue of spike-like events first, then the true spikes (the reference's order, backendSIMT.cc:745-760);
@@ -666,6 +668,12 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         if(sparse) {
                             synEnv.print("if(j < $(_row_length)[idPre])");
                         }
+                        else if(bitmask) {
+                            // a bit per (source, target), rows padded to whole words, most significant bit of a word first
+                            // (presynapticUpdateStrategySIMT.cc:276-281)
+                            synEnv.getStream() << "const " << indexTypeName << " bit = ((" << indexTypeName << ")idPre * rowSpan) + j;" << std::endl;
+                            synEnv.print("if(j < $(num_post) && ($(_gp)[bit / 32] & (0x80000000u >> (bit & 31))))");
+                        }
                         else {
                             synEnv.print("if(j < $(num_post))");
                         }
@@ -680,7 +688,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         else {
                             codeEnv.add(Type::Uint32.addConst(), "id_post", "j");
                             codeEnv.add(indexType.addConst(), "id_syn", "idSyn",
-                                        {codeEnv.addInitialiser("const " + indexTypeName + " idSyn = ((" + indexTypeName + ")idPre * $(num_post)) + j;")});
+                                        {codeEnv.addInitialiser("const " + indexTypeName + " idSyn = ((" + indexTypeName + ")idPre * " + (bitmask ? "rowSpan" : "$(num_post)") + ") + j;")});
                         }
                         codeEnv.add(Type::getAddToPrePostDelay(s.getScalarType()), "addToPostDelay",
                                     "gennmi_kernel::addScalar(&$(_den_delay)[" + s.getPostDenDelayIndex(batchSize, "$(id_post)", "$(1)") + "], $(0))");

@@ -58,7 +58,7 @@ def _run(case, *options):
 LIBRARY_CASES = sorted(set(CASES) - REFERENCE_ONLY)
 # what the generated kernels cover: SPARSE / DENSE matrices, any neuron, postsynaptic, current-source and weight-update code
 # without delay slots, spike-like events or random numbers
-GENERATED_CASES = ["custom_small", "dynamic_small", "synapse_dynamics_small", "prev_times_small", "stdp_delay_small", "va_delay_small", "graded_small", "conv_small", "va_small", "potjans_small", "izhikevich_small", "stdp_small", "stdp_additive_small", "reverse_small"]
+GENERATED_CASES = ["custom_small", "dynamic_small", "synapse_dynamics_small", "prev_times_small", "stdp_delay_small", "va_delay_small", "graded_small", "conv_small", "dense_small", "va_small", "potjans_small", "izhikevich_small", "stdp_small", "stdp_additive_small", "reverse_small"]
 
 
 @pytest.mark.parametrize("case", LIBRARY_CASES)
