@@ -909,11 +909,17 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
 }
 //--------------------------------------------------------------------------
 void Backend::genCustomUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelMerged,
-                              BackendBase::MemorySpaces&, HostHandler preambleHandler) const
+                              BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const
 {
+    if(m_GeneratedKernels) {
+        genCustomUpdateGenerated(os, modelMerged, memorySpaces, preambleHandler);
+        return;
+    }
+    // custom update code is arbitrary model code: its kernels are generated, and a model that has any takes generated
+    // kernels for its step as well (Optimiser::createBackend)
     const ModelSpecInternal &model = modelMerged.getModel();
     if(!model.getCustomUpdates().empty() || !model.getCustomWUUpdates().empty() || !model.getCustomConnectivityUpdates().empty()) {
-        unsupported("custom updates");
+        unsupported("custom updates next to the device library's own kernels (Preferences::kernelSource LIBRARY); AUTO and GENERATED generate them");
     }
     preambleHandler(os);
 }
@@ -1006,6 +1012,29 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                     EnvironmentGroupMergedField<SynapseInitGroupMerged> env(funcEnv, s);
                     buildStandardEnvironment(env, batchSize);
                     s.generateInit(*this, env, batchSize);
+                });
+            });
+        // variables of custom updates (per neuron, and per synapse of DENSE and KERNEL matrices)
+        modelMerged.genMergedCustomUpdateInitGroups(
+            *this, memorySpaces,
+            [&](auto &c)
+            {
+                forEachGroup(funcEnv, "CustomUpdateInitGroup", c.getIndex(), c.getGroups().size(), [&]
+                {
+                    EnvironmentGroupMergedField<CustomUpdateInitGroupMerged> env(funcEnv, c);
+                    buildStandardEnvironment(env, batchSize);
+                    c.generateInit(*this, env, batchSize);
+                });
+            });
+        modelMerged.genMergedCustomWUUpdateInitGroups(
+            *this, memorySpaces,
+            [&](auto &c)
+            {
+                forEachGroup(funcEnv, "CustomWUUpdateInitGroup", c.getIndex(), c.getGroups().size(), [&]
+                {
+                    EnvironmentGroupMergedField<CustomWUUpdateInitGroupMerged> env(funcEnv, c);
+                    buildStandardEnvironment(env, batchSize);
+                    c.generateInit(*this, env, batchSize);
                 });
             });
         modelMerged.genMergedSynapseConnectivityInitGroups(
@@ -1191,6 +1220,22 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                     }
                 });
             });
+        // per-synapse variables of custom updates over SPARSE matrices: row by row, like the projection's own
+        modelMerged.genMergedCustomWUUpdateSparseInitGroups(
+            *this, memorySpaces,
+            [&](auto &c)
+            {
+                forEachGroup(funcEnv, "CustomWUUpdateSparseInitGroup", c.getIndex(), c.getGroups().size(), [&]
+                {
+                    EnvironmentGroupMergedField<CustomWUUpdateSparseInitGroupMerged> env(funcEnv, c);
+                    buildStandardEnvironment(env, batchSize);
+                    env.print("for(unsigned int i = 0; i < $(num_pre); i++)");
+                    CodeStream::Scope loop(env.getStream());
+                    env.add(Type::Uint32.addConst(), "id_pre", "i");
+                    env.add(Type::Uint32.addConst(), "row_len", "$(_row_length)[i]");
+                    c.generateInit(*this, env, batchSize);
+                });
+            });
         funcEnv.getStream() << "GENNMI_CHECK(gennmi_push_mirrors());" << std::endl;
         funcEnv.getStream() << remapStream.str();
         if(timing) { funcEnv.getStream() << "GENNMI_CHECK(gennmi_synchronize());" << std::endl << timerStop("initSparseTime") << std::endl; }
@@ -1200,10 +1245,16 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
     modelMerged.genMergedSynapseInitGroupStructs(os, *this);
     modelMerged.genMergedSynapseConnectivityInitGroupStructs(os, *this);
     modelMerged.genMergedSynapseSparseInitGroupStructs(os, *this);
+    modelMerged.genMergedCustomUpdateInitGroupStructs(os, *this);
+    modelMerged.genMergedCustomWUUpdateInitGroupStructs(os, *this);
+    modelMerged.genMergedCustomWUUpdateSparseInitGroupStructs(os, *this);
     modelMerged.genMergedNeuronInitGroupHostStructArrayPush(os, *this);
     modelMerged.genMergedSynapseInitGroupHostStructArrayPush(os, *this);
     modelMerged.genMergedSynapseConnectivityInitGroupHostStructArrayPush(os, *this);
     modelMerged.genMergedSynapseSparseInitGroupHostStructArrayPush(os, *this);
+    modelMerged.genMergedCustomUpdateInitGroupHostStructArrayPush(os, *this);
+    modelMerged.genMergedCustomWUUpdateInitGroupHostStructArrayPush(os, *this);
+    modelMerged.genMergedCustomWUUpdateSparseInitGroupHostStructArrayPush(os, *this);
     preambleHandler(os);
     os << bodyStream.str();
 }
@@ -1261,9 +1312,26 @@ void Backend::genKernelSynapseVariableInit(EnvironmentExternalBase &env, Synapse
         loopEnv.getStream() << CodeStream::CB(500 + d - 1);
     }
 }
-void Backend::genKernelCustomUpdateVariableInit(EnvironmentExternalBase&, CustomWUUpdateInitGroupMerged&, HandlerEnv) const
+void Backend::genKernelCustomUpdateVariableInit(EnvironmentExternalBase &env, CustomWUUpdateInitGroupMerged &cu, HandlerEnv handler) const
 {
-    unsupported("custom updates");
+    // the same nest of loops over the kernel's dimensions as for a projection's own kernel variables
+    EnvironmentExternal loopEnv(env);
+    const size_t numDims = cu.getArchetype().getSynapseGroup()->getKernelSize().size();
+    std::string index;
+    for(size_t d = 0; d < numDims; d++) {
+        const std::string v = "k" + std::to_string(d);
+        loopEnv.getStream() << "for(unsigned int " << v << " = 0; " << v << " < " << getKernelSize(cu, d) << "; " << v << "++)" << CodeStream::OB(600 + d);
+        loopEnv.add(Type::Uint32.addConst(), "id_kernel_" + std::to_string(d), v);
+        index = index.empty() ? v : ("(" + index + ") * " + getKernelSize(cu, d) + " + " + v);
+    }
+    {
+        EnvironmentExternal varEnv(static_cast<EnvironmentExternalBase&>(loopEnv));
+        varEnv.add(Type::Uint32.addConst(), "id_syn", "idSyn", {varEnv.addInitialiser("const unsigned int idSyn = " + index + ";")});
+        handler(varEnv);
+    }
+    for(size_t d = numDims; d > 0; d--) {
+        loopEnv.getStream() << CodeStream::CB(600 + d - 1);
+    }
 }
 //--------------------------------------------------------------------------
 size_t Backend::getSynapticMatrixRowStride(const SynapseGroupInternal &sg) const
@@ -1306,6 +1374,7 @@ void Backend::genDefinitionsPreamble(CodeStream &os, const ModelSpecMerged&) con
         os << "extern bool gennmiStructsDirty;" << std::endl;
         os << "void gennmiUploadNeuronGroups();" << std::endl;
         os << "void gennmiUploadSynapseGroups();" << std::endl;
+        os << "void gennmiUploadCustomUpdateGroups();" << std::endl;
         os << "void gennmiCheckNeuronKernels();" << std::endl;
     }
     os << "#define GENNMI_CHECK(call) do { if((call) != GENNMI_OK) { throw std::runtime_error(std::string(__FILE__) + \": \" + std::to_string(__LINE__) + \": \" + gennmi_last_error()); } } while(0)" << std::endl;
@@ -1356,6 +1425,7 @@ void Backend::genRunnerPreamble(CodeStream &os, const ModelSpecMerged&) const
             os << "GENNMI_CHECK(gennmi_synchronize());" << std::endl;
             os << "gennmiUploadNeuronGroups();" << std::endl;
             os << "gennmiUploadSynapseGroups();" << std::endl;
+            os << "gennmiUploadCustomUpdateGroups();" << std::endl;
             os << "gennmiStructsDirty = false;" << std::endl;
             os << "gennmiFinalised = true;" << std::endl;
         }
@@ -1528,7 +1598,9 @@ bool Backend::isGlobalHostRNGRequired(const ModelSpecInternal &model) const
     const auto &sgs = model.getSynapseGroups();
     return std::any_of(ngs.cbegin(), ngs.cend(), [](const auto &n){ return n.second.isInitRNGRequired(); })
         || std::any_of(sgs.cbegin(), sgs.cend(), [](const auto &s){ return s.second.isWUInitRNGRequired() || s.second.getSparseConnectivityInitialiser().isRNGRequired()
-                                                                          || s.second.getSparseConnectivityInitialiser().isHostRNGRequired(); });
+                                                                          || s.second.getSparseConnectivityInitialiser().isHostRNGRequired(); })
+        || std::any_of(model.getCustomUpdates().cbegin(), model.getCustomUpdates().cend(), [](const auto &c){ return c.second.isInitRNGRequired(); })
+        || std::any_of(model.getCustomWUUpdates().cbegin(), model.getCustomWUUpdates().cend(), [](const auto &c){ return c.second.isInitRNGRequired(); });
 }
 size_t Backend::getDeviceMemoryBytes() const
 {
@@ -1597,6 +1669,9 @@ Backend createBackend(const ModelSpecInternal &model, const filesystem::path&, p
             generated = generated || anyDynamic(s.second.getPSInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isPSParamDynamic(p); });
             generated = generated || anyDynamic(s.second.getWUInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isWUParamDynamic(p); });
         }
+        // ... or when it has custom updates: their code is arbitrary model code, and the arrays they write are the ones the
+        // step's kernels read
+        generated = generated || !model.getCustomUpdates().empty() || !model.getCustomWUUpdates().empty() || !model.getCustomConnectivityUpdates().empty();
         if(generated) { LOGI_BACKEND << "The model uses snippets or combinations the device library does not implement, or dynamic parameters: the step's kernels are generated from the model's code"; }
     }
     if(generated && preferences.orderedAccumulation) {

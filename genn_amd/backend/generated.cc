@@ -24,6 +24,7 @@
 #include "backend.h"
 
 #include <algorithm>
+#include <set>
 #include <sstream>
 #include <stdexcept>
 
@@ -857,5 +858,365 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         os << "gennmiSynapseStep++;" << std::endl;
         os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateSynapses: kernel launch failed\"); }" << std::endl;
     }
+}
+//--------------------------------------------------------------------------
+// Custom updates: update<Group>(timestep), one function per update-group name (Runtime::customUpdate looks them up by that
+// name, runtime.cc:114-118), launching up to three kernels of the group's merged custom updates:
+//   per neuron      one lane per element (the batch is the grid's second dimension); a reduction over batches loops over them
+//                   in the lane that owns the element; a reduction over neurons takes one work-group per batch — lanes stride
+//                   over the population, partial results meet through wave shuffles and LDS
+//   per synapse     one lane per entry of the padded matrix (SPARSE: those beyond the row's length idle), of the dense matrix
+//                   or of the kernel; work-groups find their group by bisection, not through a table entry each
+//   transpose       64 x 64 tiles of a DENSE matrix through LDS: rows are read and written 256 bytes at a time
+// (what backendSIMT.cc:868-1270 does with 32-wide tiles and one warp per reduction).  The update code itself, its variable
+// and variable-reference indexing (delay slots, batches, shared dimensions) are GeNN's: generateCustomUpdate.
+//--------------------------------------------------------------------------
+void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMerged, BackendBase::MemorySpaces &memorySpaces,
+                                       HostHandler preambleHandler) const
+{
+    const ModelSpecInternal &model = modelMerged.getModel();
+    const unsigned int batchSize = model.getBatchSize();
+    if(!model.getCustomConnectivityUpdates().empty()) { notGenerated("custom connectivity updates"); }
+
+    std::set<std::string> groupNames;
+    for(const auto &c : model.getCustomUpdates()) { groupNames.insert(c.second.getUpdateGroupName()); }
+    for(const auto &c : model.getCustomWUUpdates()) { groupNames.insert(c.second.getUpdateGroupName()); }
+    auto refuseRNG = [](const auto &arch)
+    {
+        if(Utils::isRNGRequired(arch.getUpdateCodeTokens())) { notGenerated("random numbers in custom update code (custom update '" + arch.getName() + "')"); }
+    };
+
+    std::ostringstream declStream, uploadStream, deviceStream, hostStream;
+    CodeStream decl(declStream), upload(uploadStream), device(deviceStream), host(hostStream);
+    const std::string timeType = model.getTimePrecision().getName();
+    auto reduceOps = [this](auto &env, const std::vector<ReductionTarget> &targets)
+    {
+        for(const auto &r : targets) { env.printLine(getReductionOperation("_lr" + r.name, "$(" + r.name + ")", r.access, r.type) + ";"); }
+    };
+
+    for(const std::string &name : groupNames) {
+        // ---- per-neuron custom updates
+        std::ostringstream neuronBody, neuronArgs, neuronParams;
+        BlockTable neuronTable;
+        {
+            CodeStream body(neuronBody);
+            EnvironmentLibrary lib(body, StandardLibrary::getMathsFunctions());
+            EnvironmentExternal funcEnv(lib);
+            funcEnv.add(model.getTimePrecision().addConst(), "t", "t");
+            funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
+            modelMerged.genMergedCustomUpdateGroups(
+                *this, memorySpaces, name,
+                [&](auto &c)
+                {
+                    const auto &arch = c.getArchetype();
+                    refuseRNG(arch);
+                    const bool perElement = (arch.getDims() & VarAccessDim::ELEMENT);
+                    const bool batched = (arch.getDims() & VarAccessDim::BATCH) && (batchSize > 1);
+                    const bool oneBlock = arch.isNeuronReduction() || !perElement;
+                    const size_t firstBlock = neuronTable.numBlocks;
+                    for(size_t g = 0; g < c.getGroups().size(); g++) {
+                        const size_t blocks = oneBlock ? 1 : ((size_t)c.getGroups()[g].get().getNumNeurons() + 255) / 256;
+                        for(size_t b = 0; b < blocks; b++) { neuronTable.add(g, b * 256, b, blocks); }
+                    }
+                    const std::string structArray = "mergedCustomUpdateGroup" + std::to_string(c.getIndex());
+                    neuronArgs << ", d_" << structArray;
+                    neuronParams << ", const MergedCustomUpdateGroup" << c.getIndex() << " *" << structArray;
+
+                    funcEnv.getStream() << "// merged custom update group " << c.getIndex() << std::endl;
+                    funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << neuronTable.numBlocks << "u)";
+                    CodeStream::Scope b(funcEnv.getStream());
+                    funcEnv.getStream() << "const gennmi_kernel::BlockEntry entry = gennmiCustomUpdate" << name << "Blocks[blockIdx.x];" << std::endl;
+                    funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
+                    // (updates that are not batched run in the first of the grid's batch rows only)
+                    const std::string firstRowOnly = (batchSize > 1) ? "blockIdx.y == 0u && " : "";
+
+                    EnvironmentGroupMergedField<CustomUpdateGroupMerged> groupEnv(funcEnv, c);
+                    buildSizeEnvironment(groupEnv);
+                    if(arch.isBatchReduction()) {
+                        groupEnv.getStream() << "const unsigned int id = entry.firstId + threadIdx.x;" << std::endl;
+                        groupEnv.add(Type::Uint32.addConst(), "id", "id");
+                        groupEnv.print("if(" + firstRowOnly + "$(id) < $(num_neurons))");
+                        CodeStream::Scope b2(groupEnv.getStream());
+                        const auto targets = genInitReductionTargets(groupEnv.getStream(), c, batchSize, groupEnv["id"]);
+                        groupEnv.getStream() << "for(unsigned int batch = 0; batch < " << batchSize << "u; batch++)";
+                        {
+                            CodeStream::Scope b3(groupEnv.getStream());
+                            EnvironmentGroupMergedField<CustomUpdateGroupMerged> batchEnv(groupEnv, c);
+                            batchEnv.add(Type::Uint32.addConst(), "batch", "batch");
+                            buildStandardEnvironment(batchEnv, batchSize);
+                            c.generateCustomUpdate(batchEnv, batchSize, [&](auto &env, const auto&) { reduceOps(env, targets); });
+                        }
+                        for(const auto &r : targets) { groupEnv.printLine("group->" + r.name + "[" + r.index + "] = _lr" + r.name + ";"); }
+                    }
+                    else if(arch.isNeuronReduction()) {
+                        groupEnv.add(Type::Uint32.addConst(), "batch", batched ? "blockIdx.y" : "0");
+                        groupEnv.getStream() << "if(" << (batched ? "true" : ((batchSize > 1) ? "blockIdx.y == 0u" : "true")) << ")";
+                        CodeStream::Scope b2(groupEnv.getStream());
+                        EnvironmentGroupMergedField<CustomUpdateGroupMerged> batchEnv(groupEnv, c);
+                        buildStandardEnvironment(batchEnv, batchSize);
+                        const auto targets = genInitReductionTargets(batchEnv.getStream(), c, batchSize);
+                        batchEnv.print("for(unsigned int idx = threadIdx.x; idx < $(num_neurons); idx += 256u)");
+                        {
+                            CodeStream::Scope b3(batchEnv.getStream());
+                            EnvironmentGroupMergedField<CustomUpdateGroupMerged> loopEnv(batchEnv, c);
+                            loopEnv.add(Type::Uint32.addConst(), "id", "idx");
+                            c.generateCustomUpdate(loopEnv, batchSize, [&](auto &env, const auto&) { reduceOps(env, targets); });
+                        }
+                        for(const auto &r : targets) {
+                            batchEnv.getStream() << "_lr" << r.name << " = gennmi_kernel::blockReduce" << ((r.access & VarAccessModeAttribute::SUM) ? "Sum" : "Max")
+                                                 << "(_lr" << r.name << ");" << std::endl;
+                        }
+                        batchEnv.getStream() << "if(threadIdx.x == 0u)";
+                        {
+                            CodeStream::Scope b3(batchEnv.getStream());
+                            for(const auto &r : targets) { batchEnv.printLine("group->" + r.name + "[" + r.index + "] = _lr" + r.name + ";"); }
+                        }
+                    }
+                    else if(perElement) {
+                        groupEnv.getStream() << "const unsigned int id = entry.firstId + threadIdx.x;" << std::endl;
+                        groupEnv.add(Type::Uint32.addConst(), "id", "id");
+                        groupEnv.add(Type::Uint32.addConst(), "batch", batched ? "blockIdx.y" : "0");
+                        EnvironmentGroupMergedField<CustomUpdateGroupMerged> batchEnv(groupEnv, c);
+                        buildStandardEnvironment(batchEnv, batchSize);
+                        batchEnv.print("if(" + (batched ? std::string() : firstRowOnly) + "$(id) < $(num_neurons))");
+                        CodeStream::Scope b2(batchEnv.getStream());
+                        c.generateCustomUpdate(batchEnv, batchSize, [](auto&, auto&) {});
+                    }
+                    else {
+                        // variables shared between the neurons of a population: one lane per batch
+                        groupEnv.add(Type::Uint32.addConst(), "id", "0");
+                        groupEnv.add(Type::Uint32.addConst(), "batch", batched ? "blockIdx.y" : "0");
+                        groupEnv.getStream() << "if(" << (batched ? std::string() : firstRowOnly) << "threadIdx.x == 0u)";
+                        CodeStream::Scope b2(groupEnv.getStream());
+                        EnvironmentGroupMergedField<CustomUpdateGroupMerged> batchEnv(groupEnv, c);
+                        buildStandardEnvironment(batchEnv, batchSize);
+                        c.generateCustomUpdate(batchEnv, batchSize, [](auto&, auto&) {});
+                    }
+                });
+        }
+
+        // ---- per-synapse custom updates
+        std::ostringstream wuBody, wuArgs, wuParams, wuTables;
+        size_t wuBlocks = 0;
+        {
+            CodeStream body(wuBody);
+            EnvironmentLibrary lib(body, StandardLibrary::getMathsFunctions());
+            EnvironmentExternal funcEnv(lib);
+            funcEnv.add(model.getTimePrecision().addConst(), "t", "t");
+            funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
+            modelMerged.genMergedCustomUpdateWUGroups(
+                *this, memorySpaces, name,
+                [&](auto &c)
+                {
+                    const auto &arch = c.getArchetype();
+                    refuseRNG(arch);
+                    const SynapseGroupInternal *sg = arch.getSynapseGroup();
+                    const bool kernel = (sg->getMatrixType() & SynapseMatrixWeight::KERNEL);
+                    const bool sparse = (sg->getMatrixType() & SynapseMatrixConnectivity::SPARSE);
+                    if(!kernel && !sparse && !(sg->getMatrixType() & SynapseMatrixConnectivity::DENSE)) {
+                        notGenerated("custom updates of matrices that are neither SPARSE, DENSE nor KERNEL (custom update '" + arch.getName() + "')");
+                    }
+                    const bool batched = (arch.getDims() & VarAccessDim::BATCH) && (batchSize > 1);
+                    const bool batchReduction = arch.isBatchReduction();
+                    const size_t firstBlock = wuBlocks;
+                    const std::string starts = "gennmiCustomUpdateWU" + name + "Starts" + std::to_string(c.getIndex());
+                    wuTables << "__device__ const uint32_t " << starts << "[] = {";
+                    for(const auto &g : c.getGroups()) {
+                        const SynapseGroupInternal *gsg = g.get().getSynapseGroup();
+                        size_t size = 1;
+                        if(kernel) { for(unsigned int k : gsg->getKernelSize()) { size *= k; } }
+                        else { size = (size_t)gsg->getSrcNeuronGroup()->getNumNeurons() * getSynapticMatrixRowStride(*gsg); }
+                        wuTables << wuBlocks << "u, ";
+                        wuBlocks += (size + 255) / 256;
+                        if(wuBlocks > 0x7FFFFFFFull) { notGenerated("custom updates over this many synapses in one update group"); }
+                    }
+                    wuTables << wuBlocks << "u};" << std::endl;
+                    const std::string structArray = "mergedCustomUpdateWUGroup" + std::to_string(c.getIndex());
+                    wuArgs << ", d_" << structArray;
+                    wuParams << ", const MergedCustomUpdateWUGroup" << c.getIndex() << " *" << structArray;
+                    const std::string idType = getSynapseIndexType(c).getName();
+
+                    funcEnv.getStream() << "// merged custom WU update group " << c.getIndex() << std::endl;
+                    funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << wuBlocks << "u)";
+                    CodeStream::Scope b(funcEnv.getStream());
+                    funcEnv.getStream() << "const unsigned int gennmiGroup = gennmi_kernel::groupOfBlock(" << starts << ", " << c.getGroups().size() << "u, blockIdx.x);" << std::endl;
+                    funcEnv.getStream() << "const auto *group = &" << structArray << "[gennmiGroup];" << std::endl;
+                    funcEnv.getStream() << "const " << idType << " id = (" << idType << ")(blockIdx.x - " << starts << "[gennmiGroup]) * 256u + threadIdx.x;" << std::endl;
+
+                    EnvironmentGroupMergedField<CustomUpdateWUGroupMerged> groupEnv(funcEnv, c);
+                    buildSizeEnvironment(groupEnv);
+                    groupEnv.add(getSynapseIndexType(c).addConst(), "id", "id");
+                    if(!batchReduction) { groupEnv.add(Type::Uint32.addConst(), "batch", batched ? "blockIdx.y" : "0"); }
+                    groupEnv.print("if(" + std::string((batched && !batchReduction) || batchSize == 1 ? "" : "blockIdx.y == 0u && ") + "$(id) < $(_size))");
+                    CodeStream::Scope b2(groupEnv.getStream());
+                    EnvironmentGroupMergedField<CustomUpdateWUGroupMerged> synEnv(groupEnv, c);
+                    if(kernel) {
+                        synEnv.add(Type::Uint32.addConst(), "id_kernel", "$(id)");
+                    }
+                    else if(sparse) {
+                        synEnv.printLine("const unsigned int row = (unsigned int)($(id) / $(_row_stride));");
+                        synEnv.printLine("const unsigned int col = (unsigned int)($(id) % $(_row_stride));");
+                        synEnv.add(Type::Uint32.addConst(), "id_pre", "row");
+                        synEnv.add(Type::Uint32.addConst(), "id_post", "$(_ind)[$(id)]");
+                        synEnv.print("if(col < $(_row_length)[row])");
+                        synEnv.getStream() << CodeStream::OB(2);
+                    }
+                    else {
+                        synEnv.add(Type::Uint32.addConst(), "id_pre", "idPre", {synEnv.addInitialiser("const unsigned int idPre = (unsigned int)($(id) / $(_row_stride));")});
+                        synEnv.add(Type::Uint32.addConst(), "id_post", "idPost", {synEnv.addInitialiser("const unsigned int idPost = (unsigned int)($(id) % $(_row_stride));")});
+                    }
+                    synEnv.add(getSynapseIndexType(c).addConst(), "id_syn", "$(id)");
+                    const auto targets = genInitReductionTargets(synEnv.getStream(), c, batchSize, synEnv["id_syn"]);
+                    if(batchReduction) {
+                        synEnv.getStream() << "for(unsigned int batch = 0; batch < " << batchSize << "u; batch++)";
+                        synEnv.getStream() << CodeStream::OB(1);
+                        synEnv.add(Type::Uint32.addConst(), "batch", "batch");
+                    }
+                    {
+                        EnvironmentGroupMergedField<CustomUpdateWUGroupMerged> batchEnv(synEnv, c);
+                        buildStandardEnvironment(batchEnv, batchSize);
+                        c.generateCustomUpdate(batchEnv, batchSize, [&](auto &env, auto&) { if(batchReduction) { reduceOps(env, targets); } });
+                    }
+                    if(batchReduction) {
+                        synEnv.getStream() << CodeStream::CB(1);
+                        for(const auto &r : targets) { synEnv.printLine("group->" + r.name + "[" + r.index + "] = _lr" + r.name + ";"); }
+                    }
+                    if(sparse && !kernel) { synEnv.getStream() << CodeStream::CB(2); }
+                });
+        }
+
+        // ---- per-synapse custom updates that also write the transpose of one variable (DENSE only, customUpdate.cc checks)
+        std::ostringstream trBody, trArgs, trParams, trTables;
+        size_t trBlocks = 0;
+        {
+            CodeStream body(trBody);
+            EnvironmentLibrary lib(body, StandardLibrary::getMathsFunctions());
+            EnvironmentExternal funcEnv(lib);
+            funcEnv.add(model.getTimePrecision().addConst(), "t", "t");
+            funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
+            modelMerged.genMergedCustomUpdateTransposeWUGroups(
+                *this, memorySpaces, name,
+                [&](auto &c)
+                {
+                    const auto &arch = c.getArchetype();
+                    refuseRNG(arch);
+                    const bool batched = (arch.getDims() & VarAccessDim::BATCH) && (batchSize > 1);
+                    const size_t firstBlock = trBlocks;
+                    const std::string starts = "gennmiCustomUpdateTranspose" + name + "Starts" + std::to_string(c.getIndex());
+                    trTables << "__device__ const uint32_t " << starts << "[] = {";
+                    for(const auto &g : c.getGroups()) {
+                        const SynapseGroupInternal *gsg = g.get().getSynapseGroup();
+                        trTables << trBlocks << "u, ";
+                        trBlocks += (((size_t)gsg->getSrcNeuronGroup()->getNumNeurons() + 63) / 64) * (((size_t)gsg->getTrgNeuronGroup()->getNumNeurons() + 63) / 64);
+                    }
+                    trTables << trBlocks << "u};" << std::endl;
+                    const std::string structArray = "mergedCustomUpdateTransposeWUGroup" + std::to_string(c.getIndex());
+                    trArgs << ", d_" << structArray;
+                    trParams << ", const MergedCustomUpdateTransposeWUGroup" << c.getIndex() << " *" << structArray;
+
+                    funcEnv.getStream() << "// merged custom WU transpose update group " << c.getIndex() << std::endl;
+                    funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << trBlocks << "u)";
+                    CodeStream::Scope b(funcEnv.getStream());
+                    funcEnv.getStream() << "const unsigned int gennmiGroup = gennmi_kernel::groupOfBlock(" << starts << ", " << c.getGroups().size() << "u, blockIdx.x);" << std::endl;
+                    funcEnv.getStream() << "const auto *group = &" << structArray << "[gennmiGroup];" << std::endl;
+                    funcEnv.getStream() << "const unsigned int block = blockIdx.x - " << starts << "[gennmiGroup];" << std::endl;
+                    funcEnv.getStream() << "const unsigned int tx = threadIdx.x & 63u, ty = threadIdx.x >> 6;" << std::endl;
+                    // (an update that is not batched runs in the first of the grid's batch rows only; the condition is uniform
+                    // over a work-group, as the barrier below needs)
+                    funcEnv.getStream() << "if(" << ((batched || batchSize == 1) ? "true" : "blockIdx.y == 0u") << ")";
+                    CodeStream::Scope b2(funcEnv.getStream());
+
+                    EnvironmentGroupMergedField<CustomUpdateTransposeWUGroupMerged> groupEnv(funcEnv, c);
+                    buildSizeEnvironment(groupEnv);
+                    groupEnv.add(Type::Uint32.addConst(), "batch", batched ? "blockIdx.y" : "0");
+                    EnvironmentGroupMergedField<CustomUpdateTransposeWUGroupMerged> batchEnv(groupEnv, c);
+                    buildStandardEnvironment(batchEnv, batchSize);
+                    const std::string transposeVar = c.addTransposeField(batchEnv);
+                    batchEnv.printLine("const unsigned int numXBlocks = ($(num_post) + 63u) / 64u;");
+                    batchEnv.printLine("const unsigned int blockX = block % numXBlocks, blockY = block / numXBlocks;");
+                    {
+                        CodeStream::Scope b3(batchEnv.getStream());
+                        batchEnv.getStream() << "const unsigned int x = blockX * 64u + tx, y = blockY * 64u + ty;" << std::endl;
+                        batchEnv.print("if(x < $(num_post))");
+                        CodeStream::Scope b4(batchEnv.getStream());
+                        batchEnv.print("for(unsigned int j = 0; j < 64u && (y + j) < $(num_pre); j += 4u)");
+                        CodeStream::Scope b5(batchEnv.getStream());
+                        EnvironmentGroupMergedField<CustomUpdateTransposeWUGroupMerged> synEnv(batchEnv, c);
+                        synEnv.add(Type::Uint32.addConst(), "id_pre", "(y + j)");
+                        synEnv.add(Type::Uint32.addConst(), "id_post", "x");
+                        synEnv.add(Type::Uint32.addConst(), "id_syn", "idSyn", {synEnv.addInitialiser("const unsigned int idSyn = ((y + j) * $(num_post)) + x;")});
+                        c.generateCustomUpdate(synEnv, batchSize,
+                                               [&transposeVar](auto &env, const auto&) { env.printLine("gennmiTile[ty + j][tx] = $(" + transposeVar + ");"); });
+                    }
+                    batchEnv.getStream() << "__syncthreads();" << std::endl;
+                    {
+                        CodeStream::Scope b3(batchEnv.getStream());
+                        batchEnv.getStream() << "const unsigned int x = blockY * 64u + tx, y = blockX * 64u + ty;" << std::endl;
+                        batchEnv.print("if(x < $(num_pre))");
+                        CodeStream::Scope b4(batchEnv.getStream());
+                        batchEnv.print("for(unsigned int j = 0; j < 64u && (y + j) < $(num_post); j += 4u)");
+                        CodeStream::Scope b5(batchEnv.getStream());
+                        batchEnv.printLine("$(" + transposeVar + "_transpose)[" + (batched ? "$(_batch_offset) + " : "") + "((y + j) * $(num_pre)) + x] = gennmiTile[tx][ty + j];");
+                    }
+                });
+        }
+
+        // ---- kernels and the host function of this update group
+        const std::string signature = "(" + timeType + " t";
+        if(neuronTable.numBlocks > 0) {
+            device << "__device__ const gennmi_kernel::BlockEntry gennmiCustomUpdate" << name << "Blocks[] = {" << std::endl << neuronTable.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+            device << "__global__ __launch_bounds__(256) void gennmiCustomUpdate" << name << "Kernel" << signature << neuronParams.str() << ")";
+            CodeStream::Scope b(device);
+            device << neuronBody.str();
+        }
+        if(wuBlocks > 0) {
+            device << wuTables.str();
+            device << "__global__ __launch_bounds__(256) void gennmiCustomUpdateWU" << name << "Kernel" << signature << wuParams.str() << ")";
+            CodeStream::Scope b(device);
+            device << wuBody.str();
+        }
+        if(trBlocks > 0) {
+            device << trTables.str();
+            device << "__global__ __launch_bounds__(256) void gennmiCustomUpdateTranspose" << name << "Kernel" << signature << trParams.str() << ")";
+            CodeStream::Scope b(device);
+            device << "__shared__ " << model.getPrecision().getName() << " gennmiTile[64][65];" << std::endl;
+            device << trBody.str();
+        }
+        host << "void update" << name << "(unsigned long long timestep)";
+        {
+            CodeStream::Scope b(host);
+            host << "gennmiEnsureFinalised();" << std::endl;
+            host << "const " << timeType << " t = timestep * " << Type::writeNumeric(model.getDT(), model.getTimePrecision()) << ";" << std::endl;
+            const std::string grid = ", " + std::to_string(batchSize) + "), dim3(256), 0, 0>>>(t";
+            if(neuronTable.numBlocks > 0) { host << "gennmiCustomUpdate" << name << "Kernel<<<dim3(" << neuronTable.numBlocks << grid << neuronArgs.str() << ");" << std::endl; }
+            if(wuBlocks > 0) { host << "gennmiCustomUpdateWU" << name << "Kernel<<<dim3(" << wuBlocks << grid << wuArgs.str() << ");" << std::endl; }
+            if(trBlocks > 0) { host << "gennmiCustomUpdateTranspose" << name << "Kernel<<<dim3(" << trBlocks << grid << trArgs.str() << ");" << std::endl; }
+            host << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"update" << name << ": kernel launch failed\"); }" << std::endl;
+        }
+        host << std::endl;
+    }
+
+    // struct definitions, host arrays and push functions (GeNN's own), then the device copies
+    modelMerged.genMergedCustomUpdateStructs(os, *this);
+    modelMerged.genMergedCustomUpdateWUStructs(os, *this);
+    modelMerged.genMergedCustomUpdateTransposeWUStructs(os, *this);
+    modelMerged.genMergedCustomUpdateHostStructArrayPush(os, *this);
+    modelMerged.genMergedCustomUpdateWUHostStructArrayPush(os, *this);
+    modelMerged.genMergedCustomUpdateTransposeWUHostStructArrayPush(os, *this);
+    preambleHandler(os);
+    for(const auto &g : modelMerged.getMergedCustomUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "CustomUpdate"); }
+    for(const auto &g : modelMerged.getMergedCustomUpdateWUGroups()) { genDeviceStructArray(decl, upload, *this, g, "CustomUpdateWU"); }
+    for(const auto &g : modelMerged.getMergedCustomUpdateTransposeWUGroups()) { genDeviceStructArray(decl, upload, *this, g, "CustomUpdateTransposeWU"); }
+    os << declStream.str();
+    os << std::endl;
+    os << "void gennmiUploadCustomUpdateGroups()";
+    {
+        CodeStream::Scope b(os);
+        os << uploadStream.str();
+    }
+    os << std::endl;
+    os << deviceStream.str();
+    os << std::endl;
+    os << hostStream.str();
 }
 }   // namespace GeNN::CodeGenerator::MI355X

@@ -11,7 +11,7 @@ import math
 import numpy as np
 
 from . import netgen, rng
-from .netspec import Net, Pop, CurrentSource, Syn
+from .netspec import Net, Pop, CurrentSource, Syn, Custom
 
 
 def _const_rows(row_length, stride, value):
@@ -437,4 +437,44 @@ def custom_models(n_a=300, n_b=200, steps=300, seed=41, dt=1.0, timing="timing_c
     net.syns.append(sparse("AB_timing", "A", "B", n_a, n_b, 30, 10, 0.0, 0.12, timing, 5.0))
     net.syns.append(sparse("BA_inhibit", "B", "A", n_b, n_a, 24, 20, -0.5, -0.1, "static", 10.0))
     net.syns.append(sparse("AA_timing", "A", "A", n_a, n_a, 70, 30, 0.0, 0.02, timing, 5.0))
+    return net
+
+
+def custom_updates(n_a=200, n_b=90, steps=200, seed=57, dt=1.0):
+    """A network with custom updates — functions of the model that the user calls between steps (Runtime::customUpdate),
+    after tests/features/test_custom_update.py: every 20 steps population B's membrane potentials are pulled towards rest
+    and population A's are summed and maximised over the population; every 30 steps the plastic A -> B weights and the
+    dense A -> B weights decay (each update accumulating into a variable of its own) and the decayed dense matrix is
+    transposed into the dense B -> A projection's weights; every 50 steps the plastic weights are reduced over batches."""
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.7, TauRefrac=2.0)
+    net = Net(name="custom_update", dt=dt, steps=steps, seed=seed)
+    net.pops.append(Pop("A", "lif", n_a, dict(lif), {"V": (-60.0 + 9.5 * rng.uniform(seed, 1, 0, n_a)).astype(np.float32),
+                                                     "RefracTime": np.zeros(n_a, np.float32)}))
+    net.pops.append(Pop("B", "lif", n_b, dict(lif, Ioffset=0.4), {"V": (-60.0 + 9.5 * rng.uniform(seed, 2, 0, n_b)).astype(np.float32),
+                                                                  "RefracTime": np.zeros(n_b, np.float32)}))
+    stride = 24
+    ind = np.sort(rng.randint(seed, 10, 0, n_a * stride, n_b).reshape(n_a, stride), axis=1).astype(np.uint32)
+    # (a target at most once per row: the plastic rule and the decay both own their synapse)
+    row_length = np.zeros(n_a, np.uint32)
+    for i in range(n_a):
+        row = np.unique(ind[i])
+        row_length[i] = len(row)
+        ind[i, :len(row)] = row
+        ind[i, len(row):] = 0
+    g = (0.05 + 0.25 * rng.uniform(seed, 11, 0, n_a * stride)).astype(np.float32).reshape(n_a, stride)
+    net.syns.append(Syn("AB_plastic", "A", "B", wum="stdp_trace",
+                        wum_params=dict(tauPlus=20.0, tauMinus=20.0, aPlus=0.01, aMinus=0.012, wMin=0.0, wMax=1.0),
+                        psm="expcurr", tau=5.0, row_stride=stride, row_length=row_length, ind=ind, g=g))
+    g_ab = (0.004 * rng.uniform(seed, 12, 0, n_a * n_b)).astype(np.float32).reshape(n_a, n_b)
+    net.syns.append(Syn("AB_dense", "A", "B", matrix="dense", wum="static", psm="expcurr", tau=5.0, g=g_ab))
+    # (its weights are overwritten by the transpose: until the first call it carries these)
+    g_ba = (-0.002 * rng.uniform(seed, 13, 0, n_b * n_a)).astype(np.float32).reshape(n_b, n_a)
+    net.syns.append(Syn("BA_dense", "B", "A", matrix="dense", wum="static", psm="expcurr", tau=10.0, g=g_ba))
+    net.customs.append(Custom("BDecay", "Homeostasis", "decay", "B", params=dict(rest=-60.0, factor=0.5)))
+    net.customs.append(Custom("ASum", "Homeostasis", "neuron_reduce", "A"))
+    net.customs.append(Custom("PlasticDecay", "Decay", "wu_decay", "AB_plastic", params=dict(factor=0.9)))
+    net.customs.append(Custom("DenseDecay", "Decay", "wu_decay", "AB_dense", params=dict(factor=0.75)))
+    net.customs.append(Custom("Feedback", "Decay", "transpose", "AB_dense", "BA_dense"))
+    net.customs.append(Custom("PlasticReduce", "Reduce", "batch_reduce", "AB_plastic"))
+    net.custom_calls += [("Homeostasis", 20), ("Decay", 30), ("Reduce", 50)]
     return net

@@ -83,6 +83,21 @@ class Syn:
 
 
 @dataclass
+class Custom:
+    """A custom update (a function of the model called between steps, Runtime::customUpdate) of the test driver:
+    kind "decay" (per neuron: V of population `target` towards params rest by params factor, counts its calls),
+    "neuron_reduce" (sum and maximum of V over the population, per batch), "wu_decay" (per synapse of projection `target`:
+    g *= factor, accumulated), "batch_reduce" (sum and maximum of g over batches), "transpose" (g of DENSE projection
+    `target` transposed into g of DENSE projection `target2`)."""
+    name: str
+    group: str                      # update group: everything in a group runs in one call
+    kind: str
+    target: str
+    target2: str = ""
+    params: Dict[str, float] = field(default_factory=dict)
+
+
+@dataclass
 class Net:
     name: str
     dt: float
@@ -95,6 +110,8 @@ class Net:
     # parameters changed while the model runs (setParamDynamic + Runtime::setDynamicParamValue):
     # (kind, group, parameter, step, value) with kind in neuron | cs | wu | ps; the value holds from `step` on
     dynamic: List[tuple] = field(default_factory=list)
+    customs: List[Custom] = field(default_factory=list)
+    custom_calls: List[tuple] = field(default_factory=list)     # (update group, every n steps): called after steps n, 2n, ...
 
     def pop(self, name):
         return next(p for p in self.pops if p.name == name)
@@ -119,6 +136,10 @@ class Net:
                     h.update(np.ascontiguousarray(a).tobytes())
         for d in self.dynamic:
             h.update(repr(tuple(d)).encode())
+        for c in self.customs:
+            h.update(repr((c.name, c.group, c.kind, c.target, c.target2, sorted(c.params.items()))).encode())
+        for c in self.custom_calls:
+            h.update(repr(tuple(c)).encode())
         return h.hexdigest()
 
 
@@ -224,5 +245,11 @@ def write_netspec(net: Net, path: str):
             col = s.col_stride or int(np.bincount(s.ind[mask], minlength=net.pop(s.trg).n).max())
             opts += f" col_stride {max(1, col)}"
         lines.append(f"{head} {w} {psm}{opts}")
+    for c in net.customs:
+        order = {"decay": ("rest", "factor"), "wu_decay": ("factor",)}.get(c.kind, ())
+        lines.append(" ".join([f"custom {c.name} {c.group} {c.kind} {c.target}"] + ([c.target2] if c.kind == "transpose" else [])
+                              + [repr(float(c.params[k])) for k in order]))
+    for group, every in net.custom_calls:
+        lines.append(f"custom_call {group} {int(every)}")
     with open(os.path.join(path, "net.txt"), "w") as f:
         f.write("\n".join(lines) + "\n")

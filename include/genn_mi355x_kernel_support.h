@@ -231,6 +231,40 @@ __device__ inline uint32_t rngBinomial(Rng &r, uint32_t n, float p)
 
 __device__ inline void addScalar(float *address, float value) { unsafeAtomicAdd(address, value); }
 __device__ inline void addScalar(double *address, double value) { unsafeAtomicAdd(address, value); }
+
+// ---- custom updates ---------------------------------------------------------------------------------------------------
+// Per-synapse custom updates can span millions of work-groups, so their kernels do not carry a table entry per
+// work-group: `starts` holds, per group of a merged group, the first work-group of the group (count + 1 entries,
+// ascending); the group of a work-group is found by bisection (backendSIMT.h:244-323 does the same over thread ids).
+__device__ inline uint32_t groupOfBlock(const uint32_t *starts, uint32_t count, uint32_t block)
+{
+    uint32_t lo = 0, hi = count;
+    while(hi - lo > 1) {
+        const uint32_t mid = (lo + hi) / 2;
+        if(block >= starts[mid]) { lo = mid; } else { hi = mid; }
+    }
+    return lo;
+}
+
+// Reductions over the neurons of a population (custom update variables with REDUCE_NEURON_* access): every thread of the
+// work-group brings its partial result, every thread leaves with the work-group's.  Wave shuffles, then one LDS word per
+// wave.  A sum's order differs from the CPU backend's index order, so fp32 sums agree to rounding, not bit for bit.
+template<typename T, typename Op>
+__device__ inline T blockReduce(T value, Op op)
+{
+    __shared__ T shWave[BLOCK / WAVE];
+    for(int o = WAVE / 2; o > 0; o >>= 1) { value = op(value, __shfl_xor(value, o, WAVE)); }
+    __syncthreads();                                    // (the words may still be read from an earlier reduction)
+    if((threadIdx.x & (WAVE - 1)) == 0) { shWave[threadIdx.x / WAVE] = value; }
+    __syncthreads();
+    T result = shWave[0];
+    for(int w = 1; w < BLOCK / WAVE; w++) { result = op(result, shWave[w]); }
+    return result;
+}
+template<typename T> __device__ inline T blockReduceSum(T value) { return blockReduce(value, [](T a, T b) { return a + b; }); }
+template<typename T> __device__ inline T blockReduceMax(T value) { return blockReduce(value, [](T a, T b) { return (a > b) ? a : b; }); }
+__device__ inline float blockReduceMax(float value) { return blockReduce(value, [](float a, float b) { return fmaxf(a, b); }); }
+__device__ inline double blockReduceMax(double value) { return blockReduce(value, [](double a, double b) { return fmax(a, b); }); }
 }   // namespace gennmi_kernel
 
 #endif

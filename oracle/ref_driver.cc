@@ -214,6 +214,63 @@ public:
 };
 IMPLEMENT_SNIPPET(ArrayNoise);
 
+// Custom updates (functions a user calls between steps, Runtime::customUpdate), after tests/features/test_custom_update.py:
+// a per-neuron one that pulls a referenced variable towards a rest value and counts its calls in a variable of its own;
+class DecayToRest : public CustomUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(DecayToRest);
+    SET_PARAMS({"rest", "factor"});
+    SET_CUSTOM_UPDATE_VARS({{"applied", "scalar", CustomUpdateVarAccess::READ_WRITE}});
+    SET_VAR_REFS({{"v", "scalar", VarAccessMode::READ_WRITE}});
+    SET_UPDATE_CODE(
+        "v = rest + ((v - rest) * factor);\n"
+        "applied += 1.0;\n");
+};
+IMPLEMENT_SNIPPET(DecayToRest);
+
+// a reduction over the neurons of a population: sum and maximum of a referenced variable, one value each per batch;
+class NeuronSumMax : public CustomUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(NeuronSumMax);
+    SET_CUSTOM_UPDATE_VARS({{"sum", "scalar", CustomUpdateVarAccess::REDUCE_NEURON_SUM}, {"peak", "scalar", CustomUpdateVarAccess::REDUCE_NEURON_MAX}});
+    SET_VAR_REFS({{"v", "scalar", VarAccessMode::READ_ONLY}});
+    SET_UPDATE_CODE(
+        "sum = v;\n"
+        "peak = v;\n");
+};
+IMPLEMENT_SNIPPET(NeuronSumMax);
+
+// a per-synapse one: weight decay with the decayed weight accumulated in a variable of its own, every `t`-dependence
+// included so that the time the function is handed shows (the time of the step the model has reached);
+class WeightDecay : public CustomUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(WeightDecay);
+    SET_PARAMS({"factor"});
+    SET_CUSTOM_UPDATE_VARS({{"total", "scalar", CustomUpdateVarAccess::READ_WRITE}, {"when", "scalar", CustomUpdateVarAccess::READ_WRITE}});
+    SET_VAR_REFS({{"w", "scalar", VarAccessMode::READ_WRITE}});
+    SET_UPDATE_CODE(
+        "w *= factor;\n"
+        "total += w;\n"
+        "when = t + (0.001 * id_pre) + (1000.0 * id_post);\n");
+};
+IMPLEMENT_SNIPPET(WeightDecay);
+
+// a reduction over batches: the sum and the maximum of a per-batch synaptic variable (what gradient accumulation does)
+class BatchSumMax : public CustomUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(BatchSumMax);
+    SET_CUSTOM_UPDATE_VARS({{"sum", "scalar", CustomUpdateVarAccess::REDUCE_BATCH_SUM}, {"peak", "scalar", CustomUpdateVarAccess::REDUCE_BATCH_MAX}});
+    SET_VAR_REFS({{"w", "scalar", VarAccessMode::READ_ONLY}});
+    SET_UPDATE_CODE(
+        "sum = w;\n"
+        "peak = w;\n");
+};
+IMPLEMENT_SNIPPET(BatchSumMax);
+
 // ---------------------------------------------------------------------------------------------
 template<typename T>
 static std::vector<T> readFile(const std::string &path, size_t expect = 0)
@@ -249,6 +306,16 @@ struct SynSpec
     std::vector<double> conv, wumP, psmP;
     SynapseGroup *sg = nullptr;
 };
+
+// custom <name> <update group> <kind> <target> [<second target>] [<params>]; custom_call <update group> <every n steps>
+struct CustomSpec
+{
+    std::string name, group, kind, target, target2;
+    std::vector<double> p;
+    CustomUpdate *cu = nullptr;
+    CustomUpdateWU *cuWU = nullptr;
+};
+struct CustomCallSpec { std::string group; unsigned int every; };
 
 int main(int argc, char *argv[])
 {
@@ -295,6 +362,7 @@ int main(int argc, char *argv[])
         double dt = 1.0;
         unsigned int steps = 1, snap = 0, fuse = 0, batch = 1, seed = 0;
         std::vector<PopSpec> pops; std::vector<CSSpec> css; std::vector<SynSpec> syns; std::vector<DynamicSpec> dynamics;
+        std::vector<CustomSpec> customs; std::vector<CustomCallSpec> customCalls;
         {
             std::ifstream f(in + "/net.txt");
             if(!f) { throw std::runtime_error("no net.txt in " + in); }
@@ -332,6 +400,13 @@ int main(int argc, char *argv[])
                     while(ls >> o) { if(o == "hint_pre") s.hintPre = true; else if(o == "tps") ls >> s.tps; else if(o == "col_stride") ls >> s.colStride; else if(o == "axonal_delay") ls >> s.axonalDelay; else throw std::runtime_error("opt " + o); }
                     syns.push_back(s);
                 }
+                else if(k == "custom") {
+                    CustomSpec c; ls >> c.name >> c.group >> c.kind >> c.target;
+                    if(c.kind == "transpose") { ls >> c.target2; }
+                    double v; while(ls >> v) c.p.push_back(v);
+                    customs.push_back(c);
+                }
+                else if(k == "custom_call") { CustomCallSpec c; ls >> c.group >> c.every; customCalls.push_back(c); }
                 else throw std::runtime_error("unknown key " + k);
             }
         }
@@ -480,6 +555,31 @@ int main(int argc, char *argv[])
             else if(kind == "wu") { for(auto &q : syns) { if(q.name == group) { q.sg->setWUParamDynamic(param); found = true; } } }
             else if(kind == "ps") { for(auto &q : syns) { if(q.name == group) { q.sg->setPSParamDynamic(param); found = true; } } }
             if(!found) { throw std::runtime_error("--dynamic=" + spec + ": no such group"); }
+        }
+        std::map<std::string, SynSpec*> synByName;
+        for(auto &q : syns) { synByName[q.name] = &q; }
+        for(auto &c : customs) {
+            if(c.kind == "decay") {
+                c.cu = model.addCustomUpdate<DecayToRest>(c.name, c.group, {{"rest", c.p.at(0)}, {"factor", c.p.at(1)}}, {{"applied", 0.0}},
+                                                          {{"v", createVarRef(popByName.at(c.target)->ng, "V")}});
+            }
+            else if(c.kind == "neuron_reduce") {
+                c.cu = model.addCustomUpdate<NeuronSumMax>(c.name, c.group, {}, {{"sum", 0.0}, {"peak", 0.0}},
+                                                           {{"v", createVarRef(popByName.at(c.target)->ng, "V")}});
+            }
+            else if(c.kind == "wu_decay") {
+                c.cuWU = model.addCustomUpdate<WeightDecay>(c.name, c.group, {{"factor", c.p.at(0)}}, {{"total", 0.0}, {"when", -1.0}},
+                                                            WUVarReferences{{"w", createWUVarRef(synByName.at(c.target)->sg, "g")}});
+            }
+            else if(c.kind == "batch_reduce") {
+                c.cuWU = model.addCustomUpdate<BatchSumMax>(c.name, c.group, {}, {{"sum", 0.0}, {"peak", 0.0}},
+                                                            WUVarReferences{{"w", createWUVarRef(synByName.at(c.target)->sg, "g")}});
+            }
+            else if(c.kind == "transpose") {
+                c.cuWU = model.addCustomUpdate<CustomUpdateModels::Transpose>(c.name, c.group, {}, {},
+                    WUVarReferences{{"variable", createWUVarRef(synByName.at(c.target)->sg, "g", synByName.at(c.target2)->sg, "g")}});
+            }
+            else throw std::runtime_error("custom update kind " + c.kind);
         }
         model.finalise();
 
@@ -659,6 +759,48 @@ int main(int argc, char *argv[])
             }
         };
 
+        // variables of the custom updates, and what they write in the projections they refer to (per-synapse arrays row by
+        // row in terms of the netspec's stride, like the projections' own)
+        auto dumpRows = [&](Runtime::ArrayBase *a, const std::string &file, const SynSpec &q) {
+            a->pullFromDevice();
+            if(q.matrix == "sparse") {
+                const size_t numPre = popByName.at(q.src)->n, stride = backendStride(q), copies = a->getCount() / (numPre * stride);
+                for(size_t i = 0; i < numPre * copies; i++) { appendFile(out + "/" + file, a->getHostPointer<float>() + i * stride, q.rowStride); }
+            }
+            else {
+                appendFile(out + "/" + file, a->getHostPointer<float>(), a->getCount());
+            }
+        };
+        auto customSnapshot = [&]() {
+            for(auto &c : customs) {
+                if(c.kind == "decay") {
+                    auto *a = pulled(rt.getArray(*c.cu, "applied"));
+                    appendFile(out + "/" + c.name + ".applied.f32", a->getHostPointer<float>(), a->getCount());
+                }
+                else if(c.kind == "neuron_reduce") {
+                    for(const char *var : {"sum", "peak"}) {
+                        auto *a = pulled(rt.getArray(*c.cu, var));
+                        appendFile(out + "/" + c.name + "." + var + ".f32", a->getHostPointer<float>(), a->getCount());
+                    }
+                }
+                else if(c.kind == "wu_decay") {
+                    const SynSpec &q = *synByName.at(c.target);
+                    dumpRows(rt.getArray(*c.cuWU, "total"), c.name + ".total.f32", q);
+                    dumpRows(rt.getArray(*c.cuWU, "when"), c.name + ".when.f32", q);
+                    dumpRows(rt.getArray(*q.sg, "g"), c.name + ".w.f32", q);
+                }
+                else if(c.kind == "batch_reduce") {
+                    const SynSpec &q = *synByName.at(c.target);
+                    dumpRows(rt.getArray(*c.cuWU, "sum"), c.name + ".sum.f32", q);
+                    dumpRows(rt.getArray(*c.cuWU, "peak"), c.name + ".peak.f32", q);
+                    dumpRows(rt.getArray(*q.sg, "g"), c.name + ".w.f32", q);
+                }
+                else if(c.kind == "transpose") {
+                    dumpRows(rt.getArray(*synByName.at(c.target2)->sg, "g"), c.name + ".transposed.f32", *synByName.at(c.target2));
+                }
+            }
+        };
+
         const auto loopStart = std::chrono::steady_clock::now();
         double firstSeconds = 0.0;
         for(unsigned int i = 0; i < steps; i++) {
@@ -679,7 +821,8 @@ int main(int argc, char *argv[])
                 else { for(auto &q : syns) { if(q.name == d.group) { rt.setDynamicParamValue(*q.sg, d.param, value); } } }
             }
             rt.stepTime();
-            if(snap && ((i + 1) % snap) == 0) snapshot();
+            for(const auto &c : customCalls) { if(((i + 1) % c.every) == 0) { rt.customUpdate(c.group); } }
+            if(snap && ((i + 1) % snap) == 0) { snapshot(); customSnapshot(); }
             // the first call also builds whatever the backend prepares lazily (the MI355X backend: its device tables)
             if(i == 0) { firstSeconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - loopStart).count(); }
         }
@@ -689,7 +832,7 @@ int main(int argc, char *argv[])
         std::cout << "ref_driver: stepping loop " << loopSeconds << " s for " << steps << " steps ("
                   << loopSeconds / steps * 1e6 << " us per Runtime::stepTime, snapshots included; first call " << firstSeconds * 1e3
                   << " ms, the others " << (steps > 1 ? (loopSeconds - firstSeconds) / (steps - 1) * 1e6 : 0.0) << " us each)" << std::endl;
-        if(!snap || (steps % snap) != 0) snapshot();
+        if(!snap || (steps % snap) != 0) { snapshot(); customSnapshot(); }
 
         // spike rasters as (step, id) pairs; the reference reports times in ms = step*dt
         rt.pullRecordingBuffersFromDevice();

@@ -106,6 +106,12 @@ def dynamic_small():
     return net, snap
 
 
+def custom_update_small():
+    # custom updates (Runtime::customUpdate): per-neuron, reductions over neurons and batches, per-synapse over SPARSE and
+    # DENSE matrices, transpose; kernels generated from the update code on the MI355X backend
+    return configs.custom_updates(), 50
+
+
 def potjans_poisson_net():
     """10 % of the neurons at 20 % in-degree under the script's own Poisson background, 5 s of model time (rates fixture only)."""
     return configs.potjans(neuron_scale=0.1, connectivity_scale=0.2, steps=50000, poisson=True)
@@ -113,7 +119,7 @@ def potjans_poisson_net():
 
 # cases the reference's CPU backend pins directly (fixtures) and that the oracle, a restatement of the built-in models
 # with fixed parameters, does not cover
-REFERENCE_ONLY = {"stdp_delay_small", "custom_small", "custom_batch1_small", "dynamic_small", "poisson_input_small", "synapse_dynamics_small", "prev_times_small"}
+REFERENCE_ONLY = {"custom_update_small", "stdp_delay_small", "custom_small", "custom_batch1_small", "dynamic_small", "poisson_input_small", "synapse_dynamics_small", "prev_times_small"}
 
-CASES = {"prev_times_small": prev_times_small, "stdp_delay_small": stdp_delay_small, "synapse_dynamics_small": synapse_dynamics_small, "poisson_input_small": poisson_input_small, "custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+CASES = {"custom_update_small": custom_update_small, "prev_times_small": prev_times_small, "stdp_delay_small": stdp_delay_small, "synapse_dynamics_small": synapse_dynamics_small, "poisson_input_small": poisson_input_small, "custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
          "stdp_small": stdp_small, "conv_small": conv_small}

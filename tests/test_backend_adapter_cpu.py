@@ -157,7 +157,7 @@ def _generate_with(case, *options):
     return net, tmp, os.path.join(work, net.name + "_CODE"), res
 
 
-@pytest.mark.parametrize("case, options", [("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("conv_small", ("--kernels=generated",)), ("dense_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
+@pytest.mark.parametrize("case, options", [("custom_update_small", ()), ("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("conv_small", ("--kernels=generated",)), ("dense_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
                                            ("va_small", ("--dynamic=neuron:E.Ioffset",))])
 def test_generated_kernels_are_chosen_and_build(case, options):
     """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the runner then holds device
@@ -176,6 +176,20 @@ def test_generated_kernels_are_chosen_and_build(case, options):
         exports = _exports(os.path.join(code, "librunner.so"))
         for name in ("allocateMem", "freeMem", "initialize", "initializeSparse", "stepTime", "updateNeurons", "updateSynapses"):
             assert name in exports
+        if case == "custom_update_small":
+            # custom updates: a model that has any takes generated kernels by itself; one entry point per update group under
+            # the reference's name, its kernels generated from the update code
+            custom = open(os.path.join(code, "customUpdate.cc")).read()
+            for group in ("Homeostasis", "Decay", "Reduce"):
+                assert "update" + group in exports
+            assert "gennmiCustomUpdateHomeostasisKernel<<<" in custom and "gennmiCustomUpdateWUDecayKernel<<<" in custom
+            # (order within a group as in the reference: per-neuron, per-synapse, transpose)
+            assert custom.index("gennmiCustomUpdateWUDecayKernel<<<") < custom.index("gennmiCustomUpdateTransposeDecayKernel<<<")
+            assert "gennmi_kernel::blockReduceSum(_lrsum)" in custom and "gennmi_kernel::blockReduceMax(_lrpeak)" in custom
+            assert "gennmi_kernel::groupOfBlock(gennmiCustomUpdateWUDecayStarts" in custom
+            assert "group->variableTranspose[" in custom and "gennmiTile[tx][ty + j]" in custom
+            assert "if(col < group->rowLength[row])" in custom
+            assert "gennmiUploadCustomUpdateGroups();" in open(os.path.join(code, "runner.cc")).read()
         if case == "custom_small":
             # the extra state variable and the weight-update variables are in the kernels under the reference's names
             assert "group->A[id]" in neuron and "sPreOutSynWUMPre" in neuron and "sPostInSynWUMPost" in neuron
@@ -238,6 +252,33 @@ def test_generated_kernels_take_the_batch_from_the_grid():
         assert "group->A[batchOffset + id]" in neuron and "[blockIdx.y] = slot.total" in neuron
         assert "(size_t)recordingTimestep * 2u + blockIdx.y" in neuron
         assert "group->srcSpk[preBatchOffset + spike]" in synapse and "group->wPost[synBatchOffset + idSyn]" in synapse
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_custom_updates_take_the_batch_from_the_grid_and_reduce_over_it():
+    """Custom updates of a batched model: per-batch updates read the batch from the grid's second dimension, a reduction over
+    batches loops over them in the lane that owns the element, and the device library's own kernels refuse a model with custom
+    updates by name (their kernels are generated)."""
+    net, snap = CASES["custom_update_small"]()
+    net.snap = snap
+    net.batch_size = 3
+    tmp = tempfile.mkdtemp(prefix="adapter_custom_batch_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(net, spec)
+        res = subprocess.run([DRIVER, spec, work, out, "--generate-only"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        assert res.returncode == 0, res.stdout[-3000:]
+        custom = open(os.path.join(work, net.name + "_CODE", "customUpdate.cc")).read()
+        assert "Kernel<<<dim3(" in custom and ", 3), dim3(256)" in custom
+        assert "for(unsigned int batch = 0; batch < 3u; batch++)" in custom
+        # the per-neuron update and the reduction over neurons run once per batch, the static dense weights once
+        assert "group->applied[batchOffset + id]" in custom and "group->sum[blockIdx.y] = _lrsum" in custom
+        assert "if(blockIdx.y == 0u && id < size)" in custom
+        res = subprocess.run([DRIVER, spec, work, out, "--generate-only", "--kernels=library"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        assert res.returncode != 0 and "custom updates" in res.stdout, res.stdout[-2000:]
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
 

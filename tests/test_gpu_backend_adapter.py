@@ -131,6 +131,16 @@ def _compare_with_fixture(case, *options):
                     got = np.fromfile(os.path.join(out, f"{s.name}.{var}.f32"), np.float32).reshape(net.steps // snap, -1)
                     want = golden[key]
                     _close(got[-1] if want.ndim == 1 else got, want, key, accumulator=(var == "outPost"))
+        # variables of custom updates and what the updates wrote into the arrays they refer to, snapshot by snapshot
+        for key in golden.files:
+            if key.startswith("custom."):
+                _, name, var = key.split(".")
+                got = np.fromfile(os.path.join(out, f"{name}.{var}.f32"), np.float32).reshape(net.steps // snap, -1)
+                if var in ("applied", "when"):
+                    # call counts and the time handed to the update: nothing is summed
+                    assert np.array_equal(got, golden[key]), key
+                _close(got, golden[key], key)
+        for s in net.syns:
             key = f"denDelay.{s.name}"
             if key in golden:
                 D, n = s.max_den_delay, net.pop(s.trg).n
@@ -334,6 +344,77 @@ def test_generated_kernels_with_batches():
                         assert np.array_equal(got, golden[key]), f"batch {b}: {key}"
                 got = np.fromfile(os.path.join(out, f"{s.name}.outPost.f32"), np.float32).reshape(snaps, B, -1)[:, b]
                 _close(got, golden[f"outPost.{s.name}"], f"batch {b}: outPost.{s.name}", accumulator=True)
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_custom_updates_match_reference_backend():
+    """Custom updates (Runtime::customUpdate, after tests/features/test_custom_update.py): update groups called every 20, 30
+    and 50 steps while the network runs — a per-neuron update of the membrane potentials with a variable of its own, sum and
+    maximum over a population, weight decay over a plastic SPARSE and a static DENSE matrix with per-synapse variables,
+    the decayed dense matrix transposed into another projection's weights, and a reduction over batches.  A model with custom
+    updates takes generated kernels by itself; rasters identical to the reference CPU backend's, call counts and the time
+    handed to the update code exact, everything else within 1e-5."""
+    _compare_with_fixture("custom_update_small")
+
+
+def test_custom_updates_with_batches():
+    """The same network with batch size 3.  The reference's CPU backend has no batches, so batch 0 (same initial values) is
+    pinned by its fixture, and what batches add by closed forms: the reduction over neurons gives every batch the sum and
+    maximum of ITS membrane potentials, the reduction over batches the sum and maximum of the per-batch plastic weights,
+    the static dense weights (shared between batches) decay once per call, not once per batch."""
+    import copy
+    B = 3
+    net, snap = CASES["custom_update_small"]()
+    golden = np.load(os.path.join(HERE, "golden", "custom_update_small.npz"))
+    assert str(golden["input_digest"]) == net.input_digest(), "generator output changed since the fixture was made"
+    batched = copy.deepcopy(net)
+    from genn_amd import rng
+    for k, p in enumerate(batched.pops):
+        other = [(-60.0 + 9.5 * rng.uniform(net.seed, 71 + 2 * k + b, 0, p.n)).astype(np.float32) for b in range(B - 1)]
+        p.vars = {"V": np.stack([p.vars["V"]] + other), "RefracTime": np.zeros((B, p.n), np.float32)}
+    batched.batch_size = B
+    batched.snap = snap
+    tmp = tempfile.mkdtemp(prefix="adapter_custom_batched_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(batched, spec)
+        print(f"adapter batched custom updates: running {DRIVER}", flush=True)
+        res = subprocess.run([DRIVER, spec, work, out], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+        assert res.returncode == 0, res.stdout[-3000:]
+        snaps = batched.steps // snap
+        load = lambda name: np.fromfile(os.path.join(out, name), np.float32)        # noqa: E731
+        # batch 0 against the fixture
+        for p in batched.pops:
+            got = np.fromfile(os.path.join(out, f"{p.name}.spikes.u32"), np.uint32).reshape(-1, 2)
+            assert np.array_equal(got, golden[f"spikes.{p.name}"]), f"batch 0: raster of {p.name} differs"
+            other = np.fromfile(os.path.join(out, f"{p.name}.spikes.b1.u32"), np.uint32).reshape(-1, 2)
+            assert len(other) > 100 and not np.array_equal(other, got)
+            _close(load(f"{p.name}.V.f32").reshape(snaps, B, p.n)[:, 0], golden[f"V.{p.name}"], f"batch 0: V.{p.name}")
+        assert np.array_equal(load("BDecay.applied.f32").reshape(snaps, B, -1)[:, 0], golden["custom.BDecay.applied"])
+        assert np.array_equal(load("BDecay.applied.f32").reshape(snaps, B, -1)[:, 2], golden["custom.BDecay.applied"])
+        _close(load("PlasticDecay.w.f32").reshape(snaps, B, -1)[:, 0], golden["custom.PlasticDecay.w"], "batch 0: plastic weights")
+        _close(load("PlasticDecay.total.f32").reshape(snaps, B, -1)[:, 0], golden["custom.PlasticDecay.total"], "batch 0: PlasticDecay.total")
+        # shared between batches: one copy, decayed once per call
+        for var in ("w", "total", "when"):
+            _close(load(f"DenseDecay.{var}.f32").reshape(snaps, -1), golden[f"custom.DenseDecay.{var}"], f"DenseDecay.{var}")
+        _close(load("Feedback.transposed.f32").reshape(snaps, -1), golden["custom.Feedback.transposed"], "Feedback.transposed")
+        # reduction over neurons, per batch: the calls after steps 100 and 200 coincide with snapshots, and nothing writes A's V
+        # between the call and the snapshot
+        V = load("A.V.f32").reshape(snaps, B, -1).astype(np.float64)
+        total, peak = load("ASum.sum.f32").reshape(snaps, B), load("ASum.peak.f32").reshape(snaps, B)
+        for k in (1, 3):
+            assert np.allclose(total[k], V[k].sum(axis=1), rtol=2e-6) and np.array_equal(peak[k], V[k].max(axis=1).astype(np.float32))
+        assert len(set(total[3].tolist())) == B
+        # reduction over batches: every snapshot follows a call (both every 50 steps)
+        w = load("PlasticReduce.w.f32").reshape(snaps, B, -1)
+        mask = (np.arange(net.syn("AB_plastic").row_stride)[None, :] < net.syn("AB_plastic").row_length[:, None]).reshape(-1)
+        assert np.abs(w[-1, 0] - w[-1, 1])[mask].max() > 1e-3           # the batches' weights have diverged
+        got_sum, got_peak = load("PlasticReduce.sum.f32").reshape(snaps, -1), load("PlasticReduce.peak.f32").reshape(snaps, -1)
+        assert np.allclose(got_sum[:, mask], w.astype(np.float64).sum(axis=1)[:, mask], rtol=1e-6, atol=1e-7)
+        assert np.array_equal(got_peak[:, mask], w.max(axis=1)[:, mask])
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
 
