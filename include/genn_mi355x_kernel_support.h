@@ -10,7 +10,8 @@
  *     -> position in the population's queue.  Queues come out in ascending neuron index, the order of the reference's
  *     SingleThreadedCPU backend (single_threaded_cpu/backend.cc:321, 2119-2133); its SIMT backends append with a
  *     shared-memory atomicAdd in arbitrary order (backendSIMT.cc:1931-1956);
- *   - the fp32 scatter-add of addToPost / addToPostDelay / addToPre (backendSIMT.cc getAtomic).
+ *   - the fp32 scatter-add of addToPost / addToPostDelay / addToPre (backendSIMT.cc getAtomic);
+ *   - for custom updates: the group of a work-group by bisection, and work-group-wide sum / maximum.
  * gfx950 only: 64-wide wavefronts, work-groups of 256 threads.
  */
 #ifndef GENN_MI355X_KERNEL_SUPPORT_H
