@@ -1476,7 +1476,7 @@ void Backend::genFreeMemPreamble(CodeStream &os, const ModelSpecMerged&) const
 void Backend::genStepTimeFinalisePreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const
 {
     if(m_GeneratedKernels) {
-        // (kernel timers are not generated: the counters of such a runner stay 0)
+        // (the timers' events are read right after this: genTimer)
         if(modelMerged.getModel().isTimingEnabled()) {
             os << "GENNMI_CHECK(gennmi_synchronize());" << std::endl;
             os << "gennmiCheckNeuronKernels();" << std::endl;
@@ -1536,9 +1536,26 @@ void Backend::genGlobalDeviceRNG(CodeStream&, CodeStream&, CodeStream&, CodeStre
 {
     unsupported("a device random number generator");
 }
-void Backend::genTimer(CodeStream&, CodeStream&, CodeStream&, CodeStream&, CodeStream&, const std::string&, bool) const
+void Backend::genTimer(CodeStream &definitions, CodeStream &runner, CodeStream &allocations, CodeStream &free,
+                       CodeStream &stepTimeFinalise, const std::string &name, bool updateInStepTime) const
 {
-    // kernel durations are accumulated inside the device library (gennmi_runner_set_timing / get_times)
+    // library kernels: durations are accumulated inside the device library (gennmi_runner_set_timing / get_times);
+    // initialisation: wall-clock time of the host functions (genInit)
+    if(!m_GeneratedKernels || name == "init" || name == "initSparse") { return; }
+    // generated kernels: a pair of events around each update's launches, as the reference's device backends do
+    // (backendCUDAHIP.cc:1479-1504); read after the step has been synchronised (genStepTimeFinalisePreamble)
+    definitions << "extern hipEvent_t " << name << "Start;" << std::endl;
+    definitions << "extern hipEvent_t " << name << "Stop;" << std::endl;
+    runner << "hipEvent_t " << name << "Start;" << std::endl;
+    runner << "hipEvent_t " << name << "Stop;" << std::endl;
+    allocations << "if(hipEventCreate(&" << name << "Start) != hipSuccess || hipEventCreate(&" << name << "Stop) != hipSuccess) { throw std::runtime_error(\"" << name << ": no timer events\"); }" << std::endl;
+    free << "hipEventDestroy(" << name << "Start);" << std::endl;
+    free << "hipEventDestroy(" << name << "Stop);" << std::endl;
+    if(updateInStepTime) {
+        CodeStream::Scope b(stepTimeFinalise);
+        stepTimeFinalise << "float tmp = 0.0f;" << std::endl;
+        stepTimeFinalise << "if(hipEventElapsedTime(&tmp, " << name << "Start, " << name << "Stop) == hipSuccess) { " << name << "Time += tmp / 1000.0; }" << std::endl;
+    }
 }
 void Backend::genReturnFreeDeviceMemoryBytes(CodeStream &os) const
 {

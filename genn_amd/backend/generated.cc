@@ -387,6 +387,8 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         os << "gennmiEnsureFinalised();" << std::endl;
         if(anyPrevTimes) { os << "gennmiPrevSpikeTimeKernel<<<dim3(" << prevTable.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << prevArgs.str() << ");" << std::endl; }
         if(anyDelaySlots) { os << "gennmiSpikeQueueUpdateKernel<<<dim3(1), dim3(64), 0, 0>>>(" << queueArgs.str() << ");" << std::endl; }
+        const bool timing = model.isTimingEnabled();
+        if(timing) { os << "hipEventRecord(neuronUpdateStart, 0);" << std::endl; }
         if(table.numBlocks > 0) {
             // the tag of a launch: differs from one launch to the next, never 0 (the look-back words start out zero)
             os << "gennmiNeuronLaunches = (gennmiNeuronLaunches == 0xFFFFFFFFu) ? 1u : gennmiNeuronLaunches + 1u;" << std::endl;
@@ -398,6 +400,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                << ", gennmiNeuronStep++" << argStream.str() << ");" << std::endl;
             os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateNeurons: kernel launch failed\"); }" << std::endl;
         }
+        if(timing) { os << "hipEventRecord(neuronUpdateStop, 0);" << std::endl; }
     }
     os << std::endl;
     // bounded waits of the compaction that expired are reported where the reference's backends check for launch errors
@@ -852,9 +855,18 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         const std::string seedAndStep = std::string(", ") + (anySynapseRNG ? ((model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull") : std::string("gennmiRandomSeed()")) : std::string("0ull"))
                                         + ", gennmiSynapseStep";
         os << "static unsigned long long gennmiSynapseStep = 0;" << std::endl;
+        // (timers exist for the kinds of update the model has merged groups of, generateRunner.cc:177-199)
+        const bool timing = model.isTimingEnabled();
+        auto timer = [&](bool exists, const char *name, const char *edge) { if(timing && exists) { os << "hipEventRecord(" << name << edge << ", 0);" << std::endl; } };
+        timer(!modelMerged.getMergedSynapseDynamicsGroups().empty(), "synapseDynamics", "Start");
         if(anyDynamics) { os << "gennmiSynapseDynamicsKernel<<<dim3(" << dynamics.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << seedAndStep << dynamics.args.str() << ");" << std::endl; }
+        timer(!modelMerged.getMergedSynapseDynamicsGroups().empty(), "synapseDynamics", "Stop");
+        timer(!modelMerged.getMergedPresynapticUpdateGroups().empty(), "presynapticUpdate", "Start");
         if(anyPre) { os << "gennmiPresynapticUpdateKernel<<<dim3(" << pre.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << seedAndStep << pre.args.str() << ");" << std::endl; }
+        timer(!modelMerged.getMergedPresynapticUpdateGroups().empty(), "presynapticUpdate", "Stop");
+        timer(!modelMerged.getMergedPostsynapticUpdateGroups().empty(), "postsynapticUpdate", "Start");
         if(anyPost) { os << "gennmiPostsynapticUpdateKernel<<<dim3(" << post.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << seedAndStep << post.args.str() << ");" << std::endl; }
+        timer(!modelMerged.getMergedPostsynapticUpdateGroups().empty(), "postsynapticUpdate", "Stop");
         os << "gennmiSynapseStep++;" << std::endl;
         os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateSynapses: kernel launch failed\"); }" << std::endl;
     }
@@ -1188,10 +1200,21 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             host << "gennmiEnsureFinalised();" << std::endl;
             host << "const " << timeType << " t = timestep * " << Type::writeNumeric(model.getDT(), model.getTimePrecision()) << ";" << std::endl;
             const std::string grid = ", " + std::to_string(batchSize) + "), dim3(256), 0, 0>>>(t";
+            const bool timing = model.isTimingEnabled();
+            if(timing) { host << "hipEventRecord(customUpdate" << name << "Start, 0);" << std::endl; }
             if(neuronTable.numBlocks > 0) { host << "gennmiCustomUpdate" << name << "Kernel<<<dim3(" << neuronTable.numBlocks << grid << neuronArgs.str() << ");" << std::endl; }
             if(wuBlocks > 0) { host << "gennmiCustomUpdateWU" << name << "Kernel<<<dim3(" << wuBlocks << grid << wuArgs.str() << ");" << std::endl; }
+            if(timing) { host << "hipEventRecord(customUpdate" << name << "Stop, 0);" << std::endl << "hipEventRecord(customUpdate" << name << "TransposeStart, 0);" << std::endl; }
             if(trBlocks > 0) { host << "gennmiCustomUpdateTranspose" << name << "Kernel<<<dim3(" << trBlocks << grid << trArgs.str() << ");" << std::endl; }
+            if(timing) { host << "hipEventRecord(customUpdate" << name << "TransposeStop, 0);" << std::endl; }
             host << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"update" << name << ": kernel launch failed\"); }" << std::endl;
+            if(timing) {
+                // (these counters are not part of stepTime: read here, after the group's kernels have finished, backendCUDAHIP.cc:826-856)
+                host << "GENNMI_CHECK(gennmi_synchronize());" << std::endl;
+                host << "float tmp = 0.0f;" << std::endl;
+                host << "if(hipEventElapsedTime(&tmp, customUpdate" << name << "Start, customUpdate" << name << "Stop) == hipSuccess) { customUpdate" << name << "Time += tmp / 1000.0; }" << std::endl;
+                host << "if(hipEventElapsedTime(&tmp, customUpdate" << name << "TransposeStart, customUpdate" << name << "TransposeStop) == hipSuccess) { customUpdate" << name << "TransposeTime += tmp / 1000.0; }" << std::endl;
+            }
         }
         host << std::endl;
     }

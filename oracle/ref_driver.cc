@@ -867,6 +867,9 @@ int main(int argc, char *argv[])
         if(timing) {
             std::cout << "ref_driver: timers init " << rt.getInitTime() << " initSparse " << rt.getInitSparseTime() << " neuronUpdate " << rt.getNeuronUpdateTime()
                       << " presynapticUpdate " << rt.getPresynapticUpdateTime() << " postsynapticUpdate " << rt.getPostsynapticUpdateTime() << std::endl;
+            for(const auto &c : customCalls) {
+                std::cout << "ref_driver: timers customUpdate " << c.group << " " << rt.getCustomUpdateTime(c.group) << " transpose " << rt.getCustomUpdateTransposeTime(c.group) << std::endl;
+            }
         }
         std::cout << "ref_driver: " << name << " ran " << steps << " steps" << std::endl;
     }

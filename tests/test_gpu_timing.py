@@ -98,3 +98,40 @@ def test_counters_through_the_reference_runtime():
         assert neuron + pre + post < 1.0
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_counters_of_generated_kernels_through_the_reference_runtime():
+    """The same counters when the step's kernels are generated from model code: events around each update's launches, read
+    in stepTime after the step has been synchronised (as the reference's device backends do), and per custom update group
+    inside its update function."""
+    driver = os.path.join(ROOT, "oracle", "_ref", "mi355x_driver")
+    if not os.path.exists(driver):
+        pytest.skip("oracle/_ref/mi355x_driver is not built")
+    from cases import CASES
+    net, snap = CASES["custom_update_small"]()
+    net.snap = snap
+    tmp = tempfile.mkdtemp(prefix="adapter_timing_generated_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(net, spec)
+        res = subprocess.run([driver, spec, work, out, "--timing"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        assert res.returncode == 0, res.stdout[-3000:]
+        m = re.search(r"timers init (\S+) initSparse (\S+) neuronUpdate (\S+) presynapticUpdate (\S+) postsynapticUpdate (\S+)", res.stdout)
+        assert m, res.stdout[-2000:]
+        init, sparse, neuron, pre, post = (float(x) for x in m.groups())
+        assert init > 0 and sparse > 0 and neuron > 0 and pre > 0 and post > 0
+        # 200 steps of three kernels of a few microseconds each
+        assert 200 * 1e-6 < neuron < 0.5 and 200 * 1e-6 < pre < 0.5 and 200 * 1e-6 < post < 0.5
+        custom = {g: (float(a), float(b)) for g, a, b in re.findall(r"timers customUpdate (\S+) (\S+) transpose (\S+)", res.stdout)}
+        assert set(custom) == {"Homeostasis", "Decay", "Reduce"}
+        assert all(1e-6 < t < 0.5 for t, _ in custom.values())
+        assert custom["Decay"][1] > 1e-6 and custom["Reduce"][1] < 1e-4        # only Decay transposes
+        # the rasters are those of the untimed run
+        golden = np.load(os.path.join(HERE, "golden", "custom_update_small.npz"))
+        for p in net.pops:
+            got = np.fromfile(os.path.join(out, f"{p.name}.spikes.u32"), np.uint32).reshape(-1, 2)
+            assert np.array_equal(got, golden[f"spikes.{p.name}"])
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
