@@ -114,6 +114,8 @@ SYMBOLS = {
     "gennmi_step": (C.c_int, [C.c_void_p, C.c_float, C.c_uint32]),
     "gennmi_synchronize": (C.c_int, []),
     "gennmi_note_device_write": (C.c_int, [C.c_void_p, C.c_size_t]),
+    "gennmi_flush": (C.c_int, []),
+    "gennmi_note_mirror_write": (C.c_int, [C.c_void_p]),
     "gennmi_free_device_memory_bytes": (C.c_int, [C.POINTER(C.c_size_t)]),
     "gennmi_abi_struct_sizes": (C.c_int, [C.POINTER(C.c_size_t * 5)]),
     "gennmi_runner_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_float, C.c_uint32]),

@@ -261,8 +261,8 @@ std::string tableU32(const std::vector<uint64_t> &values)
 //--------------------------------------------------------------------------
 namespace GeNN::CodeGenerator::MI355X
 {
-Backend::Backend(const Preferences &preferences, bool generatedKernels)
-:   BackendBase(preferences), m_GeneratedKernels(generatedKernels)
+Backend::Backend(const Preferences &preferences, bool generatedKernels, bool customUpdateKernels)
+:   BackendBase(preferences), m_GeneratedKernels(generatedKernels), m_CustomUpdateKernels(customUpdateKernels && !generatedKernels)
 {
 }
 //--------------------------------------------------------------------------
@@ -911,15 +911,15 @@ void Backend::genSynapseUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerge
 void Backend::genCustomUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelMerged,
                               BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const
 {
-    if(m_GeneratedKernels) {
+    // custom update code is arbitrary model code: its kernels are generated, whichever kernels the step runs on
+    // (Optimiser::createBackend tells the backend that the model has any)
+    if(hasDeviceModules()) {
         genCustomUpdateGenerated(os, modelMerged, memorySpaces, preambleHandler);
         return;
     }
-    // custom update code is arbitrary model code: its kernels are generated, and a model that has any takes generated
-    // kernels for its step as well (Optimiser::createBackend)
     const ModelSpecInternal &model = modelMerged.getModel();
     if(!model.getCustomUpdates().empty() || !model.getCustomWUUpdates().empty() || !model.getCustomConnectivityUpdates().empty()) {
-        unsupported("custom updates next to the device library's own kernels (Preferences::kernelSource LIBRARY); AUTO and GENERATED generate them");
+        unsupported("custom updates with a backend object that was not told of them (create it with Optimiser::createBackend)");
     }
     preambleHandler(os);
 }
@@ -1368,13 +1368,15 @@ void Backend::genDefinitionsPreamble(CodeStream &os, const ModelSpecMerged&) con
     os << std::endl;
     os << "// MI355X device library" << std::endl;
     os << "#include \"genn_mi355x.h\"" << std::endl;
-    if(m_GeneratedKernels) {
+    if(hasDeviceModules()) {
         os << "// building blocks of the generated kernels (every module is compiled with hipcc)" << std::endl;
         os << "#include \"genn_mi355x_kernel_support.h\"" << std::endl;
         os << "extern bool gennmiStructsDirty;" << std::endl;
+        os << "void gennmiUploadCustomUpdateGroups();" << std::endl;
+    }
+    if(m_GeneratedKernels) {
         os << "void gennmiUploadNeuronGroups();" << std::endl;
         os << "void gennmiUploadSynapseGroups();" << std::endl;
-        os << "void gennmiUploadCustomUpdateGroups();" << std::endl;
         os << "void gennmiCheckNeuronKernels();" << std::endl;
     }
     os << "#define GENNMI_CHECK(call) do { if((call) != GENNMI_OK) { throw std::runtime_error(std::string(__FILE__) + \": \" + std::to_string(__LINE__) + \": \" + gennmi_last_error()); } } while(0)" << std::endl;
@@ -1432,10 +1434,17 @@ void Backend::genRunnerPreamble(CodeStream &os, const ModelSpecMerged&) const
         os << std::endl;
         return;
     }
+    if(m_CustomUpdateKernels) {
+        os << "// device copies of the custom updates' merged-group struct arrays: uploaded before the first use and after every push of a dynamic field" << std::endl;
+        os << "bool gennmiStructsDirty = true;" << std::endl;
+    }
     os << "// every merged update group becomes descriptors of the device library, once, before the first step" << std::endl;
     os << "void gennmiEnsureFinalised()";
     {
         CodeStream::Scope b(os);
+        if(m_CustomUpdateKernels) {
+            os << "if(gennmiStructsDirty) { GENNMI_CHECK(gennmi_synchronize()); gennmiUploadCustomUpdateGroups(); gennmiStructsDirty = false; }" << std::endl;
+        }
         os << "if(gennmiFinalised) { return; }" << std::endl;
         os << "gennmiBuildNeuronGroups();" << std::endl;
         os << "gennmiBuildSynapseGroups();" << std::endl;
@@ -1455,10 +1464,8 @@ void Backend::genAllocateMemPreamble(CodeStream &os, const ModelSpecMerged &mode
 {
     const ModelSpecInternal &model = modelMerged.getModel();
     os << "GENNMI_CHECK(gennmi_init(" << getPreferences<Preferences>().deviceID << "));" << std::endl;
-    if(m_GeneratedKernels) {
-        os << "gennmiStructsDirty = true;" << std::endl;
-        return;
-    }
+    if(hasDeviceModules()) { os << "gennmiStructsDirty = true;" << std::endl; }
+    if(m_GeneratedKernels) { return; }
     os << "GENNMI_CHECK(gennmi_runner_create(&gennmiRunner, " << Type::writeNumeric(model.getDT(), model.getTimePrecision()) << ", " << model.getBatchSize() << "u));" << std::endl;
     if(model.isTimingEnabled()) {
         os << "GENNMI_CHECK(gennmi_runner_set_timing(gennmiRunner, 1));" << std::endl;
@@ -1523,7 +1530,7 @@ void Backend::genMergedDynamicVariablePush(CodeStream &os, const std::string &su
                                            const std::string &egpName) const
 {
     os << "merged" << suffix << "Group" << mergedGroupIdx << "[" << groupIdx << "]." << fieldName << " = " << egpName << ";" << std::endl;
-    if(m_GeneratedKernels) { os << "gennmiStructsDirty = true;" << std::endl; }
+    if(hasDeviceModules()) { os << "gennmiStructsDirty = true;" << std::endl; }
 }
 //--------------------------------------------------------------------------
 std::string Backend::getAtomicOperation(const std::string &lhsPointer, const std::string &rhsValue,
@@ -1541,7 +1548,8 @@ void Backend::genTimer(CodeStream &definitions, CodeStream &runner, CodeStream &
 {
     // library kernels: durations are accumulated inside the device library (gennmi_runner_set_timing / get_times);
     // initialisation: wall-clock time of the host functions (genInit)
-    if(!m_GeneratedKernels || name == "init" || name == "initSparse") { return; }
+    // (beside library kernels only the custom updates' kernels are generated, and timed this way)
+    if(!hasDeviceModules() || name == "init" || name == "initSparse" || (!m_GeneratedKernels && name.rfind("customUpdate", 0) != 0)) { return; }
     // generated kernels: a pair of events around each update's launches, as the reference's device backends do
     // (backendCUDAHIP.cc:1479-1504); read after the step has been synchronised (genStepTimeFinalisePreamble)
     definitions << "extern hipEvent_t " << name << "Start;" << std::endl;
@@ -1579,14 +1587,14 @@ void Backend::genMakefilePreamble(std::ostream &os) const
     }
     std::string cxxFlags = "-c -fPIC -std=c++17 -MMD -MP -I\"" + root + "/include\" " + getPreferences().userCxxFlagsGNU;
     cxxFlags += getPreferences().debugCode ? " -O0 -g" : " -O2";
-    if(m_GeneratedKernels) {
+    if(hasDeviceModules()) {
         // every module holds or calls device code: hipcc for gfx950, fp32 operations neither contracted nor packed so that
         // results match the SingleThreadedCPU backend's operation for operation
         os << "CXX := " << (std::getenv("HIP_PATH") ? std::string(std::getenv("HIP_PATH")) + "/bin/hipcc" : std::string("hipcc")) << std::endl;
         cxxFlags += " -x hip --offload-arch=gfx950 -ffp-contract=off -Xclang -target-feature -Xclang -packed-fp32-ops -Wno-unused-value";
     }
     os << "CXXFLAGS := " << cxxFlags << std::endl;
-    os << "LINKFLAGS := -shared" << (m_GeneratedKernels ? " --offload-arch=gfx950 -fPIC" : "") << std::endl;
+    os << "LINKFLAGS := -shared" << (hasDeviceModules() ? " --offload-arch=gfx950 -fPIC" : "") << std::endl;
     os << "LINKLIBS := -L\"" << root << "/genn_amd/lib\" -lgenn_mi355x -Wl,-rpath,\"" << root << "/genn_amd/lib\"" << std::endl;
     os << std::endl;
 }
@@ -1686,15 +1694,14 @@ Backend createBackend(const ModelSpecInternal &model, const filesystem::path&, p
             generated = generated || anyDynamic(s.second.getPSInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isPSParamDynamic(p); });
             generated = generated || anyDynamic(s.second.getWUInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isWUParamDynamic(p); });
         }
-        // ... or when it has custom updates: their code is arbitrary model code, and the arrays they write are the ones the
-        // step's kernels read
-        generated = generated || !model.getCustomUpdates().empty() || !model.getCustomWUUpdates().empty() || !model.getCustomConnectivityUpdates().empty();
         if(generated) { LOGI_BACKEND << "The model uses snippets or combinations the device library does not implement, or dynamic parameters: the step's kernels are generated from the model's code"; }
     }
     if(generated && preferences.orderedAccumulation) {
         throw std::runtime_error("MI355X backend: ordered accumulation is a mode of the device library's kernels, not of generated ones");
     }
-    return Backend(preferences, generated);
+    // custom updates are arbitrary model code: their kernels are generated whichever kernels the step runs on
+    const bool customUpdates = !model.getCustomUpdates().empty() || !model.getCustomWUUpdates().empty() || !model.getCustomConnectivityUpdates().empty();
+    return Backend(preferences, generated, customUpdates);
 }
 }   // namespace Optimiser
 }   // namespace GeNN::CodeGenerator::MI355X

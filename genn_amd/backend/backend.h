@@ -74,10 +74,13 @@ class State : public Runtime::StateBase
 class BACKEND_EXPORT Backend : public BackendBase
 {
 public:
-    //! `generatedKernels`: the step's kernels are generated from the model's code (see Preferences::kernelSource)
-    Backend(const Preferences &preferences, bool generatedKernels = false);
+    //! `generatedKernels`: the step's kernels are generated from the model's code (see Preferences::kernelSource);
+    //! `customUpdateKernels`: the step runs on the device library's kernels and the model's custom updates on generated ones
+    Backend(const Preferences &preferences, bool generatedKernels = false, bool customUpdateKernels = false);
 
     bool areKernelsGenerated() const { return m_GeneratedKernels; }
+    //! the runner's modules hold device code and are compiled with hipcc
+    bool hasDeviceModules() const { return m_GeneratedKernels || m_CustomUpdateKernels; }
 
     //--------------------------------------------------------------------------
     // BackendBase virtuals
@@ -165,5 +168,6 @@ private:
     void genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMerged, BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const;
 
     const bool m_GeneratedKernels;
+    const bool m_CustomUpdateKernels;
 };
 }   // namespace GeNN::CodeGenerator::MI355X

@@ -906,7 +906,26 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         for(const auto &r : targets) { env.printLine(getReductionOperation("_lr" + r.name, "$(" + r.name + ")", r.access, r.type) + ";"); }
     };
 
+    // beside the device library's kernels: the arrays a custom update may have written (variable references that are not
+    // read-only, the transpose target) are named to the library afterwards, which refreshes what it derives from them
+    auto noteWrites = [this](std::ostringstream &notes, const auto &c, const std::string &structName, const std::vector<std::string> &extra)
+    {
+        if(m_GeneratedKernels) { return; }
+        std::vector<std::string> written(extra);
+        for(const auto &v : c.getArchetype().getModel()->getVarRefs()) {
+            if(v.access != VarAccessMode::READ_ONLY) { written.push_back(v.name); }
+        }
+        const auto fields = c.getSortedFields(*this);
+        for(const auto &w : written) {
+            if(std::any_of(fields.cbegin(), fields.cend(), [&w](const auto &f) { return f.name == w; })) {
+                notes << "for(unsigned int g = 0; g < " << c.getGroups().size() << "u; g++) { GENNMI_CHECK(gennmi_note_mirror_write(merged" << structName
+                      << "Group" << c.getIndex() << "[g]." << w << ")); }" << std::endl;
+            }
+        }
+    };
+
     for(const std::string &name : groupNames) {
+        std::ostringstream notes;
         // ---- per-neuron custom updates
         std::ostringstream neuronBody, neuronArgs, neuronParams;
         BlockTable neuronTable;
@@ -1004,6 +1023,7 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                         buildStandardEnvironment(batchEnv, batchSize);
                         c.generateCustomUpdate(batchEnv, batchSize, [](auto&, auto&) {});
                     }
+                    noteWrites(notes, c, "CustomUpdate", {});
                 });
         }
 
@@ -1094,6 +1114,7 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                         for(const auto &r : targets) { synEnv.printLine("group->" + r.name + "[" + r.index + "] = _lr" + r.name + ";"); }
                     }
                     if(sparse && !kernel) { synEnv.getStream() << CodeStream::CB(2); }
+                    noteWrites(notes, c, "CustomUpdateWU", {});
                 });
         }
 
@@ -1170,6 +1191,7 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                         CodeStream::Scope b5(batchEnv.getStream());
                         batchEnv.printLine("$(" + transposeVar + "_transpose)[" + (batched ? "$(_batch_offset) + " : "") + "((y + j) * $(num_pre)) + x] = gennmiTile[tx][ty + j];");
                     }
+                    noteWrites(notes, c, "CustomUpdateTransposeWU", {transposeVar + "Transpose"});
                 });
         }
 
@@ -1198,6 +1220,9 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         {
             CodeStream::Scope b(host);
             host << "gennmiEnsureFinalised();" << std::endl;
+            // (beside the library's kernels: steps still queued run first; the launches below go to the null stream, which is
+            // ordered against the runner's stream in both directions)
+            if(!m_GeneratedKernels) { host << "GENNMI_CHECK(gennmi_flush());" << std::endl; }
             host << "const " << timeType << " t = timestep * " << Type::writeNumeric(model.getDT(), model.getTimePrecision()) << ";" << std::endl;
             const std::string grid = ", " + std::to_string(batchSize) + "), dim3(256), 0, 0>>>(t";
             const bool timing = model.isTimingEnabled();
@@ -1208,6 +1233,7 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             if(trBlocks > 0) { host << "gennmiCustomUpdateTranspose" << name << "Kernel<<<dim3(" << trBlocks << grid << trArgs.str() << ");" << std::endl; }
             if(timing) { host << "hipEventRecord(customUpdate" << name << "TransposeStop, 0);" << std::endl; }
             host << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"update" << name << ": kernel launch failed\"); }" << std::endl;
+            host << notes.str();
             if(timing) {
                 // (these counters are not part of stepTime: read here, after the group's kernels have finished, backendCUDAHIP.cc:826-856)
                 host << "GENNMI_CHECK(gennmi_synchronize());" << std::endl;

@@ -267,6 +267,7 @@ int gennmi_copy_f32(float *dst, const float *src, size_t count)
     return GENNMI_OK;
 }
 int gennmi_synchronize(void) { FLUSH_QUEUED(); HIP_TRY(hipDeviceSynchronize()); return GENNMI_OK; }
+int gennmi_flush(void) { FLUSH_QUEUED(); return GENNMI_OK; }
 
 // ---- host mirrors: host buffer <-> device buffer pairs, for callers whose generated code only knows host pointers
 namespace
@@ -300,6 +301,23 @@ int gennmi_mirror_device_pointer(const void *host, void **dev)
     --it;
     if(h - it->first >= it->second.bytes) { return fail(GENNMI_EINVAL, "mirror_device_pointer: host pointer is not inside a registered buffer"); }
     *dev = static_cast<char*>(it->second.dev) + (h - it->first);
+    return GENNMI_OK;
+}
+int gennmi_note_mirror_write(const void *host)
+{
+    FLUSH_QUEUED();
+    if(!host) { return GENNMI_OK; }         // absent arrays stay absent
+    Mirror m{nullptr, 0};
+    {
+        std::lock_guard<std::mutex> lock(g_mirrorMutex);
+        const uintptr_t h = reinterpret_cast<uintptr_t>(host);
+        auto it = g_mirrors.upper_bound(h);
+        if(it == g_mirrors.begin()) { return fail(GENNMI_EINVAL, "note_mirror_write: host pointer is not inside a registered buffer"); }
+        --it;
+        if(h - it->first >= it->second.bytes) { return fail(GENNMI_EINVAL, "note_mirror_write: host pointer is not inside a registered buffer"); }
+        m = it->second;
+    }
+    noteDeviceWrite(m.dev, m.bytes);
     return GENNMI_OK;
 }
 int gennmi_push_mirrors(void)

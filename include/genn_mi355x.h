@@ -96,6 +96,13 @@ int gennmi_synchronize(void);
  * refreshes them before the next step when it knows the array was written; the calls above tell it, this call is for
  * writes it cannot see.  Cheap; naming a range that feeds no copy does nothing. */
 int gennmi_note_device_write(const void *dev, size_t bytes);
+/* No counterpart in the reference.  For callers that launch kernels of their own between steps (the custom updates the
+ * GeNN backend generates beside the library's step kernels): gennmi_flush runs whatever gennmi_step() calls are still
+ * queued (see gennmi_runner_set_step_queue), so that work launched next on the null stream sees their results — the
+ * runners' streams are blocking streams, ordered against the null stream in both directions.  gennmi_note_mirror_write is
+ * gennmi_note_device_write for the whole device buffer registered behind the host buffer `host` points into. */
+int gennmi_flush(void);
+int gennmi_note_mirror_write(const void *host);
 /* Host mirrors.  GeNN's Runtime serialises HOST pointers into merged-group structs for backends that report
  * isArrayDeviceObjectRequired() == false (runtime.cc:700-720, 1027-1044) — which lets the generated initialize() /
  * initializeSparse() run the reference's own host-side initialisation code on those pointers.  An Array

@@ -112,6 +112,19 @@ def custom_update_small():
     return configs.custom_updates(), 50
 
 
+def custom_update_static_small():
+    # custom updates over a network the device library steps on its resident plan (static weights, no delays, steps queued
+    # through Runtime::stepTime): the weights of a static projection decay every 40 steps, one population's potentials are
+    # pulled to rest every 25 — the library has to run its queued steps first and rebuild its packed copies of the weights after
+    from genn_amd.netspec import Custom
+    net, _ = va_small()
+    net.name = "custom_update_static"
+    net.customs.append(Custom("EEDecay", "Decay", "wu_decay", "EE", params=dict(factor=0.8)))
+    net.customs.append(Custom("IRest", "Homeostasis", "decay", "I", params=dict(rest=-60.0, factor=0.25)))
+    net.custom_calls += [("Decay", 40), ("Homeostasis", 25)]
+    return net, 100
+
+
 def potjans_poisson_net():
     """10 % of the neurons at 20 % in-degree under the script's own Poisson background, 5 s of model time (rates fixture only)."""
     return configs.potjans(neuron_scale=0.1, connectivity_scale=0.2, steps=50000, poisson=True)
@@ -119,7 +132,7 @@ def potjans_poisson_net():
 
 # cases the reference's CPU backend pins directly (fixtures) and that the oracle, a restatement of the built-in models
 # with fixed parameters, does not cover
-REFERENCE_ONLY = {"custom_update_small", "stdp_delay_small", "custom_small", "custom_batch1_small", "dynamic_small", "poisson_input_small", "synapse_dynamics_small", "prev_times_small"}
+REFERENCE_ONLY = {"custom_update_small", "custom_update_static_small", "stdp_delay_small", "custom_small", "custom_batch1_small", "dynamic_small", "poisson_input_small", "synapse_dynamics_small", "prev_times_small"}
 
-CASES = {"custom_update_small": custom_update_small, "prev_times_small": prev_times_small, "stdp_delay_small": stdp_delay_small, "synapse_dynamics_small": synapse_dynamics_small, "poisson_input_small": poisson_input_small, "custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
+CASES = {"custom_update_small": custom_update_small, "custom_update_static_small": custom_update_static_small, "prev_times_small": prev_times_small, "stdp_delay_small": stdp_delay_small, "synapse_dynamics_small": synapse_dynamics_small, "poisson_input_small": poisson_input_small, "custom_small": custom_small, "custom_batch1_small": custom_batch1_small, "dynamic_small": dynamic_small, "stdp_additive_small": stdp_additive_small, "reverse_small": reverse_small, "graded_small": graded_small, "va_delay_small": va_delay_small, "dense_small": dense_small, "va_small": va_small, "potjans_small": potjans_small, "izhikevich_small": izhikevich_small,
          "stdp_small": stdp_small, "conv_small": conv_small}

@@ -157,7 +157,7 @@ def _generate_with(case, *options):
     return net, tmp, os.path.join(work, net.name + "_CODE"), res
 
 
-@pytest.mark.parametrize("case, options", [("custom_update_small", ()), ("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("conv_small", ("--kernels=generated",)), ("dense_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
+@pytest.mark.parametrize("case, options", [("custom_update_small", ("--kernels=generated",)), ("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("conv_small", ("--kernels=generated",)), ("dense_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
                                            ("va_small", ("--dynamic=neuron:E.Ioffset",))])
 def test_generated_kernels_are_chosen_and_build(case, options):
     """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the runner then holds device
@@ -177,8 +177,8 @@ def test_generated_kernels_are_chosen_and_build(case, options):
         for name in ("allocateMem", "freeMem", "initialize", "initializeSparse", "stepTime", "updateNeurons", "updateSynapses"):
             assert name in exports
         if case == "custom_update_small":
-            # custom updates: a model that has any takes generated kernels by itself; one entry point per update group under
-            # the reference's name, its kernels generated from the update code
+            # custom updates: one entry point per update group under the reference's name, its kernels generated from the
+            # update code
             custom = open(os.path.join(code, "customUpdate.cc")).read()
             for group in ("Homeostasis", "Decay", "Reduce"):
                 assert "update" + group in exports
@@ -277,8 +277,33 @@ def test_custom_updates_take_the_batch_from_the_grid_and_reduce_over_it():
         # the per-neuron update and the reduction over neurons run once per batch, the static dense weights once
         assert "group->applied[batchOffset + id]" in custom and "group->sum[blockIdx.y] = _lrsum" in custom
         assert "if(blockIdx.y == 0u && id < size)" in custom
-        res = subprocess.run([DRIVER, spec, work, out, "--generate-only", "--kernels=library"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
-        assert res.returncode != 0 and "custom updates" in res.stdout, res.stdout[-2000:]
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_custom_updates_beside_library_kernels():
+    """A model of built-in snippets with custom updates keeps the device library's kernels for its step (descriptors, no
+    device code in neuronUpdate.cc) and gets generated kernels for the custom updates only: queued steps are flushed before
+    they launch, and the arrays they may have written are named to the library, which refreshes what it derives from them."""
+    net, tmp, code, res = _generate_with("custom_update_small")
+    try:
+        assert res.returncode == 0, res.stdout[-3000:]
+        neuron = open(os.path.join(code, "neuronUpdate.cc")).read()
+        custom = open(os.path.join(code, "customUpdate.cc")).read()
+        runner = open(os.path.join(code, "runner.cc")).read()
+        assert "__global__" not in neuron and "gennmi_push_neuron_update_group" in neuron and "gennmi_runner_create" in runner
+        assert "__global__" in custom and "gennmiCustomUpdateWUDecayKernel<<<" in custom
+        body = custom[custom.index("void updateDecay("):]
+        assert body.index("gennmi_flush()") < body.index("Kernel<<<") < body.index("gennmi_note_mirror_write(")
+        # written: the weights both decays refer to and the transpose target; the read-only reference of the reduction is not
+        assert "gennmi_note_mirror_write(mergedCustomUpdateTransposeWUGroup0[g].variableTranspose)" in custom
+        reduce = custom[custom.index("void updateReduce("):]
+        assert "gennmi_note_mirror_write" not in reduce[:reduce.index("\n}")]
+        assert "gennmiUploadCustomUpdateGroups();" in runner
+        assert "hipcc" in open(os.path.join(code, "Makefile")).read()
+        exports = _exports(os.path.join(code, "librunner.so"))
+        for name in ("updateHomeostasis", "updateDecay", "updateReduce", "stepTime"):
+            assert name in exports
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
 

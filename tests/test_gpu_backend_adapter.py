@@ -83,7 +83,8 @@ def _compare_with_fixture(case, *options):
     golden = np.load(os.path.join(HERE, "golden", case + ".npz"))
     net, snap, tmp, out = _run(case, *options)
     try:
-        assert net.generated_kernels == (bool(options) or case in REFERENCE_ONLY)
+        # (custom_update_*: built-in snippets, so the step keeps the library's kernels; only its custom updates are generated)
+        assert net.generated_kernels == ("--kernels=generated" in options or (case in REFERENCE_ONLY and not case.startswith("custom_update_")))
         assert str(golden["input_digest"]) == net.input_digest(), "generator output changed since the fixture was made"
         exact = (case == "va_small")
         spikes = 0
@@ -352,14 +353,32 @@ def test_custom_updates_match_reference_backend():
     """Custom updates (Runtime::customUpdate, after tests/features/test_custom_update.py): update groups called every 20, 30
     and 50 steps while the network runs — a per-neuron update of the membrane potentials with a variable of its own, sum and
     maximum over a population, weight decay over a plastic SPARSE and a static DENSE matrix with per-synapse variables,
-    the decayed dense matrix transposed into another projection's weights, and a reduction over batches.  A model with custom
-    updates takes generated kernels by itself; rasters identical to the reference CPU backend's, call counts and the time
-    handed to the update code exact, everything else within 1e-5."""
+    the decayed dense matrix transposed into another projection's weights, and a reduction over batches.  The custom
+    updates' kernels are generated from their code; the step runs on the device library's kernels (the model's snippets are
+    built-in ones), which are told what the updates wrote.  Rasters identical to the reference CPU backend's, call counts
+    and the time handed to the update code exact, everything else within 1e-5."""
     _compare_with_fixture("custom_update_small")
 
 
-def test_custom_updates_with_batches():
-    """The same network with batch size 3.  The reference's CPU backend has no batches, so batch 0 (same initial values) is
+@pytest.mark.parametrize("options", [(), ("--step-queue=0",), ("--kernels=generated",)], ids=["queued_steps", "step_by_step", "generated_step"])
+def test_custom_updates_between_queued_resident_steps(options):
+    """Custom updates over a static network without delays, which the device library steps on its resident plan with
+    Runtime::stepTime calls queued: every 40 steps the weights of a static projection decay (the library keeps packed
+    copies of them), every 25 one population's potentials are pulled towards rest (the resident kernel keeps them in
+    registers while it runs).  The queued steps must have run before an update launches and the copies must be rebuilt
+    after it: rasters identical to the reference CPU backend's, with the queue, with every step launched when asked
+    for, and on generated kernels."""
+    _compare_with_fixture("custom_update_static_small", *options)
+
+
+def test_custom_updates_match_reference_backend_on_generated_kernels():
+    """The same with the step's kernels generated too (what a model of the user's own snippets gets)."""
+    _compare_with_fixture("custom_update_small", "--kernels=generated")
+
+
+@pytest.mark.parametrize("options", [(), ("--kernels=generated",)], ids=["library_step", "generated_step"])
+def test_custom_updates_with_batches(options):
+    """The same network with batch size 3, the step on the library's kernels or on generated ones.  The reference's CPU backend has no batches, so batch 0 (same initial values) is
     pinned by its fixture, and what batches add by closed forms: the reduction over neurons gives every batch the sum and
     maximum of ITS membrane potentials, the reduction over batches the sum and maximum of the per-batch plastic weights,
     the static dense weights (shared between batches) decay once per call, not once per batch."""
@@ -381,8 +400,8 @@ def test_custom_updates_with_batches():
         for d in (work, out):
             os.makedirs(d)
         write_netspec(batched, spec)
-        print(f"adapter batched custom updates: running {DRIVER}", flush=True)
-        res = subprocess.run([DRIVER, spec, work, out], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+        print(f"adapter batched custom updates: running {DRIVER} {' '.join(options)}", flush=True)
+        res = subprocess.run([DRIVER, spec, work, out, *options], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
         assert res.returncode == 0, res.stdout[-3000:]
         snaps = batched.steps // snap
         load = lambda name: np.fromfile(os.path.join(out, name), np.float32)        # noqa: E731
