@@ -577,14 +577,20 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const bool dense = (matrix & SynapseMatrixConnectivity::DENSE);
                     const bool toeplitz = (matrix & SynapseMatrixConnectivity::TOEPLITZ);
                     const bool bitmask = (matrix & SynapseMatrixConnectivity::BITMASK);
-                    if(!sparse && !dense && !toeplitz && !bitmask) { notGenerated("PROCEDURAL connectivity (projection '" + arch.getName() + "')"); }
-                    if(matrix & SynapseMatrixWeight::PROCEDURAL) { notGenerated("weights regenerated from their initialisation snippet (projection '" + arch.getName() + "')"); }
+                    const bool procedural = (matrix & SynapseMatrixConnectivity::PROCEDURAL);
+                    if(!sparse && !dense && !toeplitz && !bitmask && !procedural) { notGenerated("this matrix type (projection '" + arch.getName() + "')"); }
+                    if((matrix & SynapseMatrixWeight::PROCEDURAL) && !procedural) {
+                        notGenerated("weights regenerated from their initialisation snippet on stored connectivity (projection '" + arch.getName() + "')");
+                    }
                     if(!arch.isPreSpikeRequired() && !arch.isPreSpikeEventRequired()) { return; }
+                    // PROCEDURAL: a row is the connectivity snippet's row build code, run by `threadsPerSpike` lanes that share the
+                    // target range between them (SynapseGroup::setNumThreadsPerSpike)
+                    const size_t threadsPerSpike = procedural ? arch.getNumThreadsPerSpike() : 1;
 
                     const size_t firstBlock = pre.table.numBlocks;
                     for(size_t g = 0; g < s.getGroups().size(); g++) {
                         const auto &sg = s.getGroups()[g].get();
-                        const size_t rowLen = (sparse || toeplitz || bitmask) ? getSynapticMatrixRowStride(sg) : sg.getTrgNeuronGroup()->getNumNeurons();
+                        const size_t rowLen = procedural ? threadsPerSpike : (sparse || toeplitz || bitmask) ? getSynapticMatrixRowStride(sg) : sg.getTrgNeuronGroup()->getNumNeurons();
                         const size_t chunks = (rowLen + 63) / 64;
                         // enough wavefronts for ~1.5 % of the source population firing in one step, at most 128 work-groups
                         const size_t blocks = std::clamp<size_t>((sg.getSrcNeuronGroup()->getNumNeurons() * chunks + 255) / 256, 1, 128);
@@ -601,7 +607,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
                     EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> groupEnv(funcEnv, s);
                     buildStandardEnvironment(groupEnv, batchSize);
-                    groupEnv.printLine(std::string("const unsigned int rowSpan = ") + ((sparse || toeplitz || bitmask) ? "$(_row_stride)" : "$(num_post)") + ";");
+                    groupEnv.printLine(std::string("const unsigned int rowSpan = ") + (procedural ? (std::to_string(threadsPerSpike) + "u") : (sparse || toeplitz || bitmask) ? "$(_row_stride)" : "$(num_post)") + ";");
                     groupEnv.getStream() << "const unsigned int chunksPerRow = (rowSpan + 63u) / 64u;" << std::endl;
                     groupEnv.getStream() << "const unsigned int numWaves = entry.blocksInGroup * 4u;" << std::endl;
                     // the queue of spike-like events first, then the true spikes (the reference's order, backendSIMT.cc:745-760);
@@ -622,6 +628,72 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         synEnv.getStream() << "const unsigned int j = (unsigned int)(item % chunksPerRow) * 64u + (threadIdx.x & 63u);" << std::endl;
                         synEnv.printLine("const unsigned int idPre = $(_src_spk" + suffix + ")[" + s.getPreVarIndex(preDelay, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "spike") + "];");
                         synEnv.add(Type::Uint32.addConst(), "id_pre", "idPre");
+                        if(procedural) {
+                            // A row of a PROCEDURAL matrix is the connectivity snippet's row build code, run afresh for every spike:
+                            // lane j of an item takes the j-th share of the target range, and the snippet's addSynapse(idPost,
+                            // kernel indices...) becomes the weight-update code (presynapticUpdateStrategySIMT.cc:425-565).  Random
+                            // numbers of the row build code and of weights regenerated from their initialisation snippet come from
+                            // one counter-based generator per (row, lane): key = the model's seed, stream 2k + 1 for the k-th
+                            // projection by name, counter = the lane's number, step 0 — so a row is the same every time it is built
+                            // (the reference skips ahead in one Philox sequence to the same end).
+                            EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> rowEnv(synEnv, s);
+                            const std::string tps = std::to_string(threadsPerSpike);
+                            // (the population's size under another name: `num_post` itself becomes a lane's share below)
+                            rowEnv.add(Type::Uint32.addConst(), "_num_post", "$(num_post)");
+                            if(Utils::isRNGRequired(arch.getSparseConnectivityInitialiser().getRowBuildCodeTokens())
+                               || ((matrix & SynapseMatrixWeight::PROCEDURAL) && Utils::isRNGRequired(arch.getWUInitialiser().getVarInitialisers())))
+                            {
+                                anySynapseRNG = true;
+                                rowEnv.addField(Type::Uint32.addConst(), "_rng_stream_row", Type::Uint32, "rngStreamRow",
+                                                [&model](const SynapseGroupInternal &g, size_t)
+                                                {
+                                                    return Type::NumericValue((uint64_t)(2 * std::distance(model.getSynapseGroups().cbegin(), model.getSynapseGroups().find(g.getName())) + 1));
+                                                });
+                                rowEnv.add(Type::Uint32, "_rng", "gennmiRng",
+                                           {rowEnv.addInitialiser("gennmi_kernel::Rng gennmiRng = gennmi_kernel::rngBegin(gennmiSeed, $(_rng_stream_row), (unsigned long long)idPre * " + tps + "u + j, 0ull);")});
+                            }
+                            std::ostringstream updateStream;
+                            CodeStream update(updateStream);
+                            {
+                                CodeStream::Scope bu(update);
+                                EnvironmentExternal updateEnv(rowEnv, update);
+                                updateEnv.add(Type::Uint32.addConst(), "id_post", "idPost", {updateEnv.addInitialiser("const unsigned int idPost = $(0);")});
+                                for(size_t i = 0; i < arch.getKernelSize().size(); i++) {
+                                    const std::string iStr = std::to_string(i);
+                                    updateEnv.add(Type::Uint32.addConst(), "id_kernel_" + iStr, "idKernel" + iStr,
+                                                  {updateEnv.addInitialiser("const unsigned int idKernel" + iStr + " = $(" + std::to_string(i + 1) + ");")});
+                                }
+                                updateEnv.add(Type::getAddToPrePostDelay(s.getScalarType()), "addToPostDelay",
+                                              "gennmi_kernel::addScalar(&$(_den_delay)[" + s.getPostDenDelayIndex(batchSize, "$(id_post)", "$(1)") + "], $(0))");
+                                updateEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPost",
+                                              "gennmi_kernel::addScalar(&$(_out_post)[" + s.getPostISynIndex(batchSize, "$(id_post)") + "], $(0))");
+                                updateEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
+                                              "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(batchSize, "$(id_pre)") + "], $(0))");
+                                if(trueSpike) { s.generateSpikeUpdate(*this, updateEnv, batchSize, dt); }
+                                else { s.generateSpikeEventUpdate(*this, updateEnv, batchSize, dt); }
+                            }
+                            rowEnv.getStream() << "if(j < " << tps << "u)";
+                            CodeStream::Scope bt(rowEnv.getStream());
+                            EnvironmentExternal connEnv(rowEnv);
+                            connEnv.add(Type::Uint32.addConst(), "num_threads", tps);
+                            connEnv.add(Type::Uint32.addConst(), "id_thread", "j");
+                            if(threadsPerSpike > 1) {
+                                const size_t perThread = connEnv.addInitialiser("const unsigned int numPostPerThread = ($(_num_post) + " + tps + "u - 1u) / " + tps + "u;");
+                                connEnv.add(Type::Uint32.addConst(), "id_post_begin", "idPostBegin",
+                                            {perThread, connEnv.addInitialiser("const unsigned int idPostBegin = j * numPostPerThread;")});
+                                // (the last lanes' shares end with the population)
+                                connEnv.add(Type::Uint32.addConst(), "num_post", "numPostOfThread",
+                                            {perThread, connEnv.addInitialiser("const unsigned int numPostOfThread = (j * numPostPerThread >= $(_num_post)) ? 0u : min(numPostPerThread, $(_num_post) - j * numPostPerThread);")});
+                            }
+                            else {
+                                connEnv.add(Type::Uint32.addConst(), "id_post_begin", "0");
+                            }
+                            const auto addSynapseType = Type::ResolvedType::createFunction(
+                                Type::Void, std::vector<Type::ResolvedType>{1ull + arch.getKernelSize().size(), Type::Uint32});
+                            connEnv.add(addSynapseType, "addSynapse", updateStream.str());
+                            s.generateProceduralConnectivity(connEnv);
+                            return;
+                        }
                         if(toeplitz) {
                             // A row of a Toeplitz matrix is the connectivity snippet's diagonal build code run for (presynaptic
                             // neuron, diagonal): lane j of an item takes diagonal j, and the snippet's addSynapse(idPost, kernel

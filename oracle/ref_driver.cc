@@ -325,7 +325,7 @@ int main(int argc, char *argv[])
         bool generateOnly = false;
         std::string userCxxFlags;
         std::vector<std::string> dynamicParams;
-        bool timing = false, ordered = false, deviceInit = false;
+        bool timing = false, ordered = false, deviceInit = false, doublePrecision = false;
         int stepQueue = -1;
         std::string kernels = "auto";
         for(int a = 4; a < argc; a++) {
@@ -339,6 +339,7 @@ int main(int argc, char *argv[])
             else if(opt.rfind("--step-queue=", 0) == 0) { stepQueue = std::stoi(opt.substr(13)); }      // MI355X backend: Preferences::stepQueueLength
             else if(opt == "--device-init") { deviceInit = true; }                  // MI355X backend: Preferences::deviceInitialisation
             else if(opt == "--ordered") { ordered = true; }                          // MI355X backend: Preferences::orderedAccumulation
+            else if(opt == "--precision=double") { doublePrecision = true; }        // ModelSpec::setPrecision(Type::Double); for --generate-only runs (the netspec's arrays are fp32)
             else if(opt == "--timing") { timing = true; }       // ModelSpec::setTimingEnabled; the Runtime's counters are printed after the run
             else { std::cerr << "unknown option " << opt << std::endl; return 1; }
         }
@@ -417,7 +418,7 @@ int main(int argc, char *argv[])
         model.setDT(dt);
         model.setBatchSize(batch);
         if(seed) { model.setSeed(seed); }
-        model.setPrecision(Type::Float);
+        model.setPrecision(doublePrecision ? Type::Double : Type::Float);
         model.setFusePostsynapticModels(fuse != 0);
         model.setTimingEnabled(timing);
         std::map<std::string, PopSpec*> popByName;

@@ -146,7 +146,11 @@ def test_dynamic_parameters_are_refused(dynamic, case):
 
 
 def _generate_with(case, *options):
-    net, snap = CASES[case]()
+    if case == "procedural":        # (no fixture: nothing in the reference's CPU backend regenerates matrices)
+        from genn_amd import configs
+        net, snap = configs.procedural(), 50
+    else:
+        net, snap = CASES[case]()
     net.snap = snap
     tmp = tempfile.mkdtemp(prefix="adapter_genk_")
     spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
@@ -157,7 +161,7 @@ def _generate_with(case, *options):
     return net, tmp, os.path.join(work, net.name + "_CODE"), res
 
 
-@pytest.mark.parametrize("case, options", [("custom_update_small", ("--kernels=generated",)), ("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("conv_small", ("--kernels=generated",)), ("dense_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
+@pytest.mark.parametrize("case, options", [("custom_update_small", ("--kernels=generated",)), ("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("conv_small", ("--kernels=generated",)), ("procedural", ("--kernels=generated",)), ("dense_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
                                            ("va_small", ("--dynamic=neuron:E.Ioffset",))])
 def test_generated_kernels_are_chosen_and_build(case, options):
     """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the runner then holds device
@@ -194,6 +198,12 @@ def test_generated_kernels_are_chosen_and_build(case, options):
             # the extra state variable and the weight-update variables are in the kernels under the reference's names
             assert "group->A[id]" in neuron and "sPreOutSynWUMPre" in neuron and "sPostInSynWUMPost" in neuron
             assert "group->wPost[idSyn] = group->sPost[idPost]" in synapse and "group->wPre[rowMajorIndex] = group->sPre[idPre]" in synapse
+        if case == "procedural":
+            # PROCEDURAL connectivity and weights: the snippets' own code inside the presynaptic walk, drawing from a generator
+            # keyed by (seed, projection, row, lane) at step 0
+            assert "gennmi_kernel::rngBegin(gennmiSeed, (1u), (unsigned long long)idPre * 1u + j, 0ull)" in synapse
+            assert "gennmi_kernel::rngUniform(gennmiRng)" in synapse and "gennmi_kernel::rngNormal(gennmiRng)" in synapse
+            assert "const unsigned int idPost = " in synapse and "_prevJ" in synapse
         if case == "conv_small":
             # TOEPLITZ connectivity: the snippet's diagonal build code inside the presynaptic walk, its addSynapse become the update
             assert "const unsigned int idPost = " in synapse and "idKernel0" in synapse and "idKernel3" in synapse
@@ -309,19 +319,18 @@ def test_custom_updates_beside_library_kernels():
 
 
 def test_generated_kernels_say_what_they_do_not_cover():
-    """Asked to generate kernels for a feature only the device library implements, the backend names the feature."""
-    from genn_amd import configs
-    net = configs.procedural()
-    net.snap = 50
+    """Asked to generate kernels for something they do not cover, the backend names it."""
+    net, snap = CASES["va_small"]()
+    net.snap = snap
     tmp = tempfile.mkdtemp(prefix="adapter_genk_refuse_")
     try:
         spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
         for d in (work, out):
             os.makedirs(d)
         write_netspec(net, spec)
-        res = subprocess.run([DRIVER, spec, work, out, "--generate-only", "--kernels=generated"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        res = subprocess.run([DRIVER, spec, work, out, "--generate-only", "--kernels=generated", "--precision=double"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
         assert res.returncode != 0
-        assert "generated kernels do not cover" in res.stdout and "PROCEDURAL" in res.stdout, res.stdout[-2000:]
+        assert "generated kernels do not cover" in res.stdout and "double precision" in res.stdout, res.stdout[-2000:]
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
 

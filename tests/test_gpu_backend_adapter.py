@@ -438,6 +438,84 @@ def test_custom_updates_with_batches(options):
         shutil.rmtree(tmp, ignore_errors=True)
 
 
+def test_generated_kernels_on_procedural_matrices():
+    """PROCEDURAL connectivity on generated kernels: a row is the connectivity snippet's own row build code, run afresh for
+    every spike with random numbers from a counter-based generator keyed by (seed, projection, row, lane).  No backend of the
+    reference draws the same numbers (its CPU backend has no procedural matrices at all), so this is **parity unpinned**
+    against the reference and held to what the construction fixes instead.  Eight sources fire together twice, ten steps
+    apart, through FixedProbability(0.1) with a dyadic weight into a DeltaCurr input of 1000 silent LIF neurons, four lanes
+    per row: every target must receive exactly the same number of inputs both times (the matrix is a function of the seed,
+    not of the step), the number of synapses must be Binomial(8000, 0.1), and no target outside a lane's share may be hit
+    twice by one row.  Then the recurrent procedural network of the library tests (all four snippets, dyadic weights):
+    identical rasters from two runs, population rates within 15 % of the device library's own procedural path."""
+    from genn_amd import configs
+    from genn_amd.netspec import Net, Pop, Syn
+    n_src, n_trg, p_conn, g = 8, 1000, 0.1, 0.25
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=1e9, Ioffset=0.0, TauRefrac=2.0)
+    net = Net(name="procedural_rows", dt=1.0, steps=14, seed=4242)
+    net.pops.append(Pop("S", "ssa", n_src, {}, {"startSpike": (2 * np.arange(n_src)).astype(np.uint32), "endSpike": (2 * np.arange(n_src) + 2).astype(np.uint32)},
+                        spike_times=np.tile(np.array([1.0, 11.0], np.float32), n_src)))
+    net.pops.append(Pop("T", "lif", n_trg, lif, {"V": np.full(n_trg, -60.0, np.float32), "RefracTime": np.zeros(n_trg, np.float32)}))
+    net.syns.append(Syn("ST", "S", "T", matrix="procedural", wum="static_const", wum_params={"g": g}, psm="deltacurr",
+                        connect=("FixedProbability", {"prob": p_conn}), threads_per_spike=4))
+    net.snap = 1
+
+    def run(network, *options):
+        tmp = tempfile.mkdtemp(prefix="adapter_proc_generated_")
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(network, spec)
+        print(f"adapter procedural on generated kernels: running {DRIVER} {' '.join(options)}", flush=True)
+        res = subprocess.run([DRIVER, spec, work, out, *options], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+        assert res.returncode == 0, res.stdout[-3000:]
+        generated = "__global__" in open(os.path.join(work, network.name + "_CODE", "neuronUpdate.cc")).read()
+        return tmp, out, generated
+
+    tmp, out, generated = run(net, "--kernels=generated")
+    try:
+        assert generated
+        V = np.fromfile(os.path.join(out, "T.V.f32"), np.float32).reshape(net.steps, n_trg).astype(np.float64)
+        rest, decay = -60.0, np.exp(-1.0 / 20.0)
+        quantum = (1.0 - decay) * 20.0 * g                  # what one input adds to V (Rmembrane = TauM / C)
+        moved = [k for k in range(net.steps) if np.any(V[k] != rest)]
+        first = moved[0]
+        hits1 = (V[first] - rest) / quantum
+        hits2 = (V[first + 10] - rest - decay * (V[first + 9] - rest)) / quantum
+        assert np.abs(hits1 - np.rint(hits1)).max() < 1e-3 and np.abs(hits2 - np.rint(hits2)).max() < 1e-3
+        hits1, hits2 = np.rint(hits1).astype(int), np.rint(hits2).astype(int)
+        assert np.array_equal(hits1, hits2), "the rows differ between the two times they were built"
+        total = hits1.sum()
+        sd = np.sqrt(n_src * n_trg * p_conn * (1 - p_conn))
+        assert abs(total - n_src * n_trg * p_conn) < 4 * sd, f"{total} synapses in {n_src} rows of {n_trg} at p = {p_conn}"
+        assert hits1.max() <= n_src and (hits1 > 0).sum() > 400
+        # every lane's share of the target range got its part
+        for lane in range(4):
+            share = hits1[lane * 250:(lane + 1) * 250].sum()
+            assert abs(share - total / 4) < 4 * sd / 2 + 1, f"lane {lane}: {share} of {total} synapses"
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+    recurrent = configs.procedural(order_free=True)
+    recurrent.steps, recurrent.snap = 100, 100
+    counts = {}
+    rasters = {}
+    for label, options in (("generated", ("--kernels=generated",)), ("again", ("--kernels=generated",)), ("library", ())):
+        tmp, out, generated = run(recurrent, *options)
+        try:
+            assert generated == (label != "library")
+            rasters[label] = {p.name: np.fromfile(os.path.join(out, f"{p.name}.spikes.u32"), np.uint32).reshape(-1, 2) for p in recurrent.pops}
+            counts[label] = {name: len(r) for name, r in rasters[label].items()}
+        finally:
+            shutil.rmtree(tmp, ignore_errors=True)
+    print("spike counts:", counts, flush=True)
+    for p in recurrent.pops:
+        assert np.array_equal(rasters["generated"][p.name], rasters["again"][p.name]), f"{p.name}: two runs from one seed differ"
+        assert not np.array_equal(rasters["generated"][p.name], rasters["library"][p.name])        # another generator, another matrix
+        assert counts["library"][p.name] > 200, counts
+        assert abs(counts["generated"][p.name] - counts["library"][p.name]) <= 0.15 * counts["library"][p.name], (p.name, counts)
+
+
 def test_generated_kernels_with_simulation_random_numbers():
     """Random numbers in simulation code (the built-in Poisson neuron, neuronModels.h:307-325: `gennrand_exponential()` refills a
     countdown): the generated kernels draw them from a counter-based generator keyed by the model's seed.  Every backend of
