@@ -914,6 +914,9 @@ void Backend::genCustomUpdate(CodeStream &os, FileStreamCreator, ModelSpecMerged
     // custom update code is arbitrary model code: its kernels are generated, whichever kernels the step runs on
     // (Optimiser::createBackend tells the backend that the model has any)
     if(hasDeviceModules()) {
+        if(!m_GeneratedKernels && !modelMerged.getModel().getCustomConnectivityUpdates().empty()) {
+            unsupported("custom connectivity updates beside the device library's step kernels, whose launch plans rely on rows sorted by target (Preferences::kernelSource AUTO or GENERATED generates the step's kernels)");
+        }
         genCustomUpdateGenerated(os, modelMerged, memorySpaces, preambleHandler);
         return;
     }
@@ -1034,6 +1037,29 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                 {
                     EnvironmentGroupMergedField<CustomWUUpdateInitGroupMerged> env(funcEnv, c);
                     buildStandardEnvironment(env, batchSize);
+                    c.generateInit(*this, env, batchSize);
+                });
+            });
+        // presynaptic and postsynaptic variables of custom connectivity updates
+        modelMerged.genMergedCustomConnectivityUpdatePreInitGroups(
+            *this, memorySpaces,
+            [&](auto &c)
+            {
+                forEachGroup(funcEnv, "CustomConnectivityUpdatePreInitGroup", c.getIndex(), c.getGroups().size(), [&]
+                {
+                    EnvironmentGroupMergedField<CustomConnectivityUpdatePreInitGroupMerged> env(funcEnv, c);
+                    buildStandardEnvironment(env);
+                    c.generateInit(*this, env, batchSize);
+                });
+            });
+        modelMerged.genMergedCustomConnectivityUpdatePostInitGroups(
+            *this, memorySpaces,
+            [&](auto &c)
+            {
+                forEachGroup(funcEnv, "CustomConnectivityUpdatePostInitGroup", c.getIndex(), c.getGroups().size(), [&]
+                {
+                    EnvironmentGroupMergedField<CustomConnectivityUpdatePostInitGroupMerged> env(funcEnv, c);
+                    buildStandardEnvironment(env);
                     c.generateInit(*this, env, batchSize);
                 });
             });
@@ -1236,6 +1262,22 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                     c.generateInit(*this, env, batchSize);
                 });
             });
+        // per-synapse variables of custom connectivity updates
+        modelMerged.genMergedCustomConnectivityUpdateSparseInitGroups(
+            *this, memorySpaces,
+            [&](auto &c)
+            {
+                forEachGroup(funcEnv, "CustomConnectivityUpdateSparseInitGroup", c.getIndex(), c.getGroups().size(), [&]
+                {
+                    EnvironmentGroupMergedField<CustomConnectivityUpdateSparseInitGroupMerged> env(funcEnv, c);
+                    buildStandardEnvironment(env);
+                    env.print("for(unsigned int i = 0; i < $(num_pre); i++)");
+                    CodeStream::Scope loop(env.getStream());
+                    env.add(Type::Uint32.addConst(), "id_pre", "i");
+                    env.add(Type::Uint32.addConst(), "row_len", "$(_row_length)[i]");
+                    c.generateInit(*this, env, batchSize);
+                });
+            });
         funcEnv.getStream() << "GENNMI_CHECK(gennmi_push_mirrors());" << std::endl;
         funcEnv.getStream() << remapStream.str();
         if(timing) { funcEnv.getStream() << "GENNMI_CHECK(gennmi_synchronize());" << std::endl << timerStop("initSparseTime") << std::endl; }
@@ -1248,6 +1290,9 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
     modelMerged.genMergedCustomUpdateInitGroupStructs(os, *this);
     modelMerged.genMergedCustomWUUpdateInitGroupStructs(os, *this);
     modelMerged.genMergedCustomWUUpdateSparseInitGroupStructs(os, *this);
+    modelMerged.genMergedCustomConnectivityUpdatePreInitStructs(os, *this);
+    modelMerged.genMergedCustomConnectivityUpdatePostInitStructs(os, *this);
+    modelMerged.genMergedCustomConnectivityUpdateSparseInitStructs(os, *this);
     modelMerged.genMergedNeuronInitGroupHostStructArrayPush(os, *this);
     modelMerged.genMergedSynapseInitGroupHostStructArrayPush(os, *this);
     modelMerged.genMergedSynapseConnectivityInitGroupHostStructArrayPush(os, *this);
@@ -1255,6 +1300,9 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
     modelMerged.genMergedCustomUpdateInitGroupHostStructArrayPush(os, *this);
     modelMerged.genMergedCustomWUUpdateInitGroupHostStructArrayPush(os, *this);
     modelMerged.genMergedCustomWUUpdateSparseInitGroupHostStructArrayPush(os, *this);
+    modelMerged.genMergedCustomConnectivityUpdatePreInitHostStructArrayPush(os, *this);
+    modelMerged.genMergedCustomConnectivityUpdatePostInitHostStructArrayPush(os, *this);
+    modelMerged.genMergedCustomConnectivityUpdateSparseInitHostStructArrayPush(os, *this);
     preambleHandler(os);
     os << bodyStream.str();
 }
@@ -1694,6 +1742,9 @@ Backend createBackend(const ModelSpecInternal &model, const filesystem::path&, p
             generated = generated || anyDynamic(s.second.getPSInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isPSParamDynamic(p); });
             generated = generated || anyDynamic(s.second.getWUInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isWUParamDynamic(p); });
         }
+        // ... or when custom connectivity updates rewire a projection: the library's launch plans rely on rows sorted by target,
+        // which removing and adding synapses does not keep
+        generated = generated || !model.getCustomConnectivityUpdates().empty();
         if(generated) { LOGI_BACKEND << "The model uses snippets or combinations the device library does not implement, or dynamic parameters: the step's kernels are generated from the model's code"; }
     }
     if(generated && preferences.orderedAccumulation) {

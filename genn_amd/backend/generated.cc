@@ -945,13 +945,15 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
 }
 //--------------------------------------------------------------------------
 // Custom updates: update<Group>(timestep), one function per update-group name (Runtime::customUpdate looks them up by that
-// name, runtime.cc:114-118), launching up to three kernels of the group's merged custom updates:
+// name, runtime.cc:114-118), launching up to four kernels of the group's merged custom updates:
 //   per neuron      one lane per element (the batch is the grid's second dimension); a reduction over batches loops over them
 //                   in the lane that owns the element; a reduction over neurons takes one work-group per batch — lanes stride
 //                   over the population, partial results meet through wave shuffles and LDS
 //   per synapse     one lane per entry of the padded matrix (SPARSE: those beyond the row's length idle), of the dense matrix
 //                   or of the kernel; work-groups find their group by bisection, not through a table entry each
 //   transpose       64 x 64 tiles of a DENSE matrix through LDS: rows are read and written 256 bytes at a time
+//   connectivity    (custom connectivity updates, which run first) a lane per row of a SPARSE matrix runs the row update code;
+//                   the column views of projections that learn from postsynaptic spikes are rebuilt afterwards
 // (what backendSIMT.cc:868-1270 does with 32-wide tiles and one warp per reduction).  The update code itself, its variable
 // and variable-reference indexing (delay slots, batches, shared dimensions) are GeNN's: generateCustomUpdate.
 //--------------------------------------------------------------------------
@@ -960,11 +962,11 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
 {
     const ModelSpecInternal &model = modelMerged.getModel();
     const unsigned int batchSize = model.getBatchSize();
-    if(!model.getCustomConnectivityUpdates().empty()) { notGenerated("custom connectivity updates"); }
-
     std::set<std::string> groupNames;
     for(const auto &c : model.getCustomUpdates()) { groupNames.insert(c.second.getUpdateGroupName()); }
     for(const auto &c : model.getCustomWUUpdates()) { groupNames.insert(c.second.getUpdateGroupName()); }
+    for(const auto &c : model.getCustomConnectivityUpdates()) { groupNames.insert(c.second.getUpdateGroupName()); }
+    if(!modelMerged.getMergedCustomConnectivityHostUpdateGroups().empty()) { notGenerated("host update code of custom connectivity updates"); }
     auto refuseRNG = [](const auto &arch)
     {
         if(Utils::isRNGRequired(arch.getUpdateCodeTokens())) { notGenerated("random numbers in custom update code (custom update '" + arch.getName() + "')"); }
@@ -1267,6 +1269,76 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                 });
         }
 
+        // ---- custom connectivity updates: a lane per row runs the row update code; add_synapse / remove_synapse and the
+        // bookkeeping of every variable that lives on the synapses are GeNN's (generateUpdate).  Random numbers: a
+        // counter-based generator per row and call (key = the model's seed, stream 6000 + the update's place in the model's
+        // name-ordered list; the reference keeps a generator state per row in memory, backendSIMT.cc:1273-1305)
+        std::ostringstream ccBody, ccArgs, ccParams, ccRemap;
+        BlockTable ccTable;
+        {
+            CodeStream body(ccBody);
+            EnvironmentLibrary lib(body, StandardLibrary::getMathsFunctions());
+            EnvironmentLibrary rngLib(lib, simRNGFunctions);
+            EnvironmentExternal funcEnv(rngLib);
+            funcEnv.add(model.getTimePrecision().addConst(), "t", "t");
+            funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
+            modelMerged.genMergedCustomConnectivityUpdateGroups(
+                *this, memorySpaces, name,
+                [&](auto &c)
+                {
+                    const auto &arch = c.getArchetype();
+                    const size_t firstBlock = ccTable.numBlocks;
+                    for(size_t g = 0; g < c.getGroups().size(); g++) {
+                        const size_t blocks = ((size_t)c.getGroups()[g].get().getSynapseGroup()->getSrcNeuronGroup()->getNumNeurons() + 255) / 256;
+                        for(size_t b = 0; b < blocks; b++) { ccTable.add(g, b * 256, b, blocks); }
+                    }
+                    const std::string structArray = "mergedCustomConnectivityUpdateGroup" + std::to_string(c.getIndex());
+                    ccArgs << ", d_" << structArray;
+                    ccParams << ", const MergedCustomConnectivityUpdateGroup" << c.getIndex() << " *" << structArray;
+                    funcEnv.getStream() << "// merged custom connectivity update group " << c.getIndex() << std::endl;
+                    funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << ccTable.numBlocks << "u)";
+                    CodeStream::Scope b(funcEnv.getStream());
+                    funcEnv.getStream() << "const gennmi_kernel::BlockEntry entry = gennmiCustomConnectivityUpdate" << name << "Blocks[blockIdx.x];" << std::endl;
+                    funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
+                    funcEnv.getStream() << "const unsigned int id = entry.firstId + threadIdx.x;" << std::endl;
+                    EnvironmentGroupMergedField<CustomConnectivityUpdateGroupMerged> groupEnv(funcEnv, c);
+                    buildStandardEnvironment(groupEnv);
+                    groupEnv.print("if(id < $(num_pre))");
+                    CodeStream::Scope b2(groupEnv.getStream());
+                    EnvironmentGroupMergedField<CustomConnectivityUpdateGroupMerged> rowEnv(groupEnv, c);
+                    rowEnv.add(Type::Uint32.addConst(), "id_pre", "id");
+                    if(Utils::isRNGRequired(arch.getRowUpdateCodeTokens())) {
+                        rowEnv.addField(Type::Uint32.addConst(), "_rng_stream", Type::Uint32, "rngStream",
+                                        [&model](const CustomConnectivityUpdateInternal &g, size_t)
+                                        {
+                                            return Type::NumericValue((uint64_t)(6000 + std::distance(model.getCustomConnectivityUpdates().cbegin(), model.getCustomConnectivityUpdates().find(g.getName()))));
+                                        });
+                        rowEnv.add(Type::Uint32, "_rng", "gennmiRng",
+                                   {rowEnv.addInitialiser("gennmi_kernel::Rng gennmiRng = gennmi_kernel::rngBegin(gennmiSeed, $(_rng_stream), (unsigned long long)id, gennmiStep);")});
+                    }
+                    c.generateUpdate(*this, rowEnv, batchSize);
+                });
+        }
+        // ... after which the column views of projections that learn from postsynaptic spikes are rebuilt by the device library
+        // (deterministic order, as at initialisation; the reference has a kernel of its own for this, backendSIMT.cc:1307-1400)
+        {
+            CodeStream remap(ccRemap);
+            EnvironmentLibrary lib(remap, StandardLibrary::getMathsFunctions());
+            EnvironmentExternal funcEnv(lib);
+            modelMerged.genMergedCustomConnectivityRemapUpdateGroups(
+                *this, memorySpaces, name,
+                [&](auto &c)
+                {
+                    funcEnv.getStream() << "for(unsigned int g = 0; g < " << c.getGroups().size() << "u; g++)";
+                    CodeStream::Scope b(funcEnv.getStream());
+                    funcEnv.getStream() << "const auto *group = &mergedCustomConnectivityRemapUpdateGroup" << c.getIndex() << "[g];" << std::endl;
+                    EnvironmentGroupMergedField<CustomConnectivityRemapUpdateGroupMerged> env(funcEnv, c);
+                    buildStandardEnvironment(env);
+                    env.printLine("GENNMI_CHECK(gennmi_build_remap($(num_pre), $(num_post), $(_row_stride), $(_col_stride), gennmiDev($(_row_length)), gennmiDev($(_ind)), "
+                                  "gennmiDev($(_col_length)), gennmiDev($(_remap))));");
+                });
+        }
+
         // ---- kernels and the host function of this update group
         const std::string signature = "(" + timeType + " t";
         if(neuronTable.numBlocks > 0) {
@@ -1280,6 +1352,12 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             device << "__global__ __launch_bounds__(256) void gennmiCustomUpdateWU" << name << "Kernel" << signature << wuParams.str() << ")";
             CodeStream::Scope b(device);
             device << wuBody.str();
+        }
+        if(ccTable.numBlocks > 0) {
+            device << "__device__ const gennmi_kernel::BlockEntry gennmiCustomConnectivityUpdate" << name << "Blocks[] = {" << std::endl << ccTable.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+            device << "__global__ __launch_bounds__(256) void gennmiCustomConnectivityUpdate" << name << "Kernel" << signature << ", unsigned long long gennmiSeed, unsigned long long gennmiStep" << ccParams.str() << ")";
+            CodeStream::Scope b(device);
+            device << ccBody.str();
         }
         if(trBlocks > 0) {
             device << trTables.str();
@@ -1299,6 +1377,13 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             const std::string grid = ", " + std::to_string(batchSize) + "), dim3(256), 0, 0>>>(t";
             const bool timing = model.isTimingEnabled();
             if(timing) { host << "hipEventRecord(customUpdate" << name << "Start, 0);" << std::endl; }
+            if(ccTable.numBlocks > 0) {
+                // (connectivity first, like the reference: single_threaded_cpu/backend.cc:824-860; the generator's step counts this group's calls)
+                host << "static unsigned long long gennmiCalls = 0;" << std::endl;
+                host << "gennmiCustomConnectivityUpdate" << name << "Kernel<<<dim3(" << ccTable.numBlocks << ", 1), dim3(256), 0, 0>>>(t, "
+                     << ((model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull") : std::string("gennmiRandomSeed()")) << ", gennmiCalls++" << ccArgs.str() << ");" << std::endl;
+                host << ccRemap.str();
+            }
             if(neuronTable.numBlocks > 0) { host << "gennmiCustomUpdate" << name << "Kernel<<<dim3(" << neuronTable.numBlocks << grid << neuronArgs.str() << ");" << std::endl; }
             if(wuBlocks > 0) { host << "gennmiCustomUpdateWU" << name << "Kernel<<<dim3(" << wuBlocks << grid << wuArgs.str() << ");" << std::endl; }
             if(timing) { host << "hipEventRecord(customUpdate" << name << "Stop, 0);" << std::endl << "hipEventRecord(customUpdate" << name << "TransposeStart, 0);" << std::endl; }
@@ -1321,6 +1406,10 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     modelMerged.genMergedCustomUpdateStructs(os, *this);
     modelMerged.genMergedCustomUpdateWUStructs(os, *this);
     modelMerged.genMergedCustomUpdateTransposeWUStructs(os, *this);
+    modelMerged.genMergedCustomConnectivityUpdateStructs(os, *this);
+    modelMerged.genMergedCustomConnectivityRemapUpdateStructs(os, *this);
+    modelMerged.genMergedCustomConnectivityUpdateHostStructArrayPush(os, *this);
+    modelMerged.genMergedCustomConnectivityRemapUpdateHostStructArrayPush(os, *this);
     modelMerged.genMergedCustomUpdateHostStructArrayPush(os, *this);
     modelMerged.genMergedCustomUpdateWUHostStructArrayPush(os, *this);
     modelMerged.genMergedCustomUpdateTransposeWUHostStructArrayPush(os, *this);
@@ -1328,6 +1417,7 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     for(const auto &g : modelMerged.getMergedCustomUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "CustomUpdate"); }
     for(const auto &g : modelMerged.getMergedCustomUpdateWUGroups()) { genDeviceStructArray(decl, upload, *this, g, "CustomUpdateWU"); }
     for(const auto &g : modelMerged.getMergedCustomUpdateTransposeWUGroups()) { genDeviceStructArray(decl, upload, *this, g, "CustomUpdateTransposeWU"); }
+    for(const auto &g : modelMerged.getMergedCustomConnectivityUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "CustomConnectivityUpdate"); }
     os << declStream.str();
     os << std::endl;
     os << "void gennmiUploadCustomUpdateGroups()";

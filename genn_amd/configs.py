@@ -478,3 +478,19 @@ def custom_updates(n_a=200, n_b=90, steps=200, seed=57, dt=1.0):
     net.customs.append(Custom("PlasticReduce", "Reduce", "batch_reduce", "AB_plastic"))
     net.custom_calls += [("Homeostasis", 20), ("Decay", 30), ("Reduce", 50)]
     return net
+
+
+def rewiring(steps=200):
+    """The plastic network of :func:`custom_updates` with custom CONNECTIVITY updates (structural plasticity): every 40
+    steps synapses of the plastic projection whose weight has fallen below a threshold are removed (the row's last synapse
+    moves into the gap, with every variable that lives on the synapses), every 25 steps each row that has room sprouts a
+    synapse onto a target that moves on from call to call; in between the weights keep learning and decaying.  The
+    projection learns from postsynaptic spikes, so its column view is rebuilt after every change."""
+    net = custom_updates(steps=steps)
+    net.name = "rewiring"
+    net.customs = [c for c in net.customs if c.name == "PlasticDecay"]
+    net.syn("AB_plastic").col_stride = 128          # room for the columns to grow
+    net.customs.append(Custom("Prune", "Prune", "prune", "AB_plastic", params=dict(threshold=0.12)))
+    net.customs.append(Custom("Sprout", "Sprout", "sprout", "AB_plastic", params=dict(weight=0.2)))
+    net.custom_calls = [("Decay", 30), ("Prune", 40), ("Sprout", 25)]
+    return net

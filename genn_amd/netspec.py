@@ -88,7 +88,9 @@ class Custom:
     kind "decay" (per neuron: V of population `target` towards params rest by params factor, counts its calls),
     "neuron_reduce" (sum and maximum of V over the population, per batch), "wu_decay" (per synapse of projection `target`:
     g *= factor, accumulated), "batch_reduce" (sum and maximum of g over batches), "transpose" (g of DENSE projection
-    `target` transposed into g of DENSE projection `target2`)."""
+    `target` transposed into g of DENSE projection `target2`); custom connectivity updates of SPARSE projection `target`:
+    "prune" (removes synapses with g < params threshold, counting per row) and "sprout" (adds one synapse per row and call
+    where there is room, weight params weight)."""
     name: str
     group: str                      # update group: everything in a group runs in one call
     kind: str
@@ -246,7 +248,7 @@ def write_netspec(net: Net, path: str):
             opts += f" col_stride {max(1, col)}"
         lines.append(f"{head} {w} {psm}{opts}")
     for c in net.customs:
-        order = {"decay": ("rest", "factor"), "wu_decay": ("factor",)}.get(c.kind, ())
+        order = {"decay": ("rest", "factor"), "wu_decay": ("factor",), "prune": ("threshold",), "sprout": ("weight",)}.get(c.kind, ())
         lines.append(" ".join([f"custom {c.name} {c.group} {c.kind} {c.target}"] + ([c.target2] if c.kind == "transpose" else [])
                               + [repr(float(c.params[k])) for k in order]))
     for group, every in net.custom_calls:

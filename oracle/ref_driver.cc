@@ -271,6 +271,53 @@ public:
 };
 IMPLEMENT_SNIPPET(BatchSumMax);
 
+// Custom connectivity updates (structural plasticity: a function of the model that rewires a SPARSE projection between steps),
+// after tests/features/test_custom_connectivity_update.py: one that removes every synapse whose weight has fallen below a
+// threshold and counts the removals of its row in a presynaptic variable of its own;
+class PruneWeak : public CustomConnectivityUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(PruneWeak);
+    SET_PARAMS({"threshold"});
+    SET_PRE_VARS({{"removed", "scalar"}});
+    SET_VAR_REFS({{"w", "scalar", VarAccessMode::READ_ONLY}});
+    SET_ROW_UPDATE_CODE(
+        "for_each_synapse {\n"
+        "    if(w < threshold) {\n"
+        "        remove_synapse();\n"
+        "        removed += 1.0;\n"
+        "    }\n"
+        "}\n");
+};
+IMPLEMENT_SNIPPET(PruneWeak);
+
+// and one that gives every row that has room a new synapse onto a target that moves on with every call (rows start apart, so
+// that columns fill evenly), with a weight the
+// call fixes and a per-synapse variable of its own that records when the synapse was made (older synapses keep theirs)
+class Sprout : public CustomConnectivityUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(Sprout);
+    SET_PARAMS({"weight"});
+    SET_VARS({{"born", "scalar"}});
+    SET_PRE_VARS({{"next", "unsigned int"}});
+    SET_VAR_REFS({{"w", "scalar", VarAccessMode::READ_WRITE}});
+    SET_ROW_UPDATE_CODE(
+        "const unsigned int target = (next + (3 * id_pre)) % num_post;\n"
+        "bool present = false;\n"
+        "for_each_synapse {\n"
+        "    if(id_post == target) {\n"
+        "        present = true;\n"
+        "        break;\n"
+        "    }\n"
+        "}\n"
+        "if(!present && row_length < row_stride) {\n"
+        "    add_synapse(target, t, weight);\n"
+        "}\n"
+        "next = (next + 7) % num_post;\n");
+};
+IMPLEMENT_SNIPPET(Sprout);
+
 // ---------------------------------------------------------------------------------------------
 template<typename T>
 static std::vector<T> readFile(const std::string &path, size_t expect = 0)
@@ -314,6 +361,7 @@ struct CustomSpec
     std::vector<double> p;
     CustomUpdate *cu = nullptr;
     CustomUpdateWU *cuWU = nullptr;
+    CustomConnectivityUpdate *ccu = nullptr;
 };
 struct CustomCallSpec { std::string group; unsigned int every; };
 
@@ -580,6 +628,14 @@ int main(int argc, char *argv[])
                 c.cuWU = model.addCustomUpdate<CustomUpdateModels::Transpose>(c.name, c.group, {}, {},
                     WUVarReferences{{"variable", createWUVarRef(synByName.at(c.target)->sg, "g", synByName.at(c.target2)->sg, "g")}});
             }
+            else if(c.kind == "prune") {
+                c.ccu = model.addCustomConnectivityUpdate<PruneWeak>(c.name, c.group, synByName.at(c.target)->sg, {{"threshold", c.p.at(0)}}, {}, {{"removed", 0.0}}, {},
+                                                                    WUVarReferences{{"w", createWUVarRef(synByName.at(c.target)->sg, "g")}}, {}, {});
+            }
+            else if(c.kind == "sprout") {
+                c.ccu = model.addCustomConnectivityUpdate<Sprout>(c.name, c.group, synByName.at(c.target)->sg, {{"weight", c.p.at(0)}}, {{"born", -1.0}}, {{"next", 0.0}}, {},
+                                                                 WUVarReferences{{"w", createWUVarRef(synByName.at(c.target)->sg, "g")}}, {}, {});
+            }
             else throw std::runtime_error("custom update kind " + c.kind);
         }
         model.finalise();
@@ -798,6 +854,24 @@ int main(int argc, char *argv[])
                 }
                 else if(c.kind == "transpose") {
                     dumpRows(rt.getArray(*synByName.at(c.target2)->sg, "g"), c.name + ".transposed.f32", *synByName.at(c.target2));
+                }
+                else if(c.kind == "prune" || c.kind == "sprout") {
+                    // the rewired matrix: row lengths, and targets and weights row by row in terms of the netspec's stride
+                    const SynSpec &q = *synByName.at(c.target);
+                    const size_t numPre = popByName.at(q.src)->n, stride = backendStride(q);
+                    auto *rl = pulled(rt.getArray(*q.sg, "rowLength")); auto *ind = pulled(rt.getArray(*q.sg, "ind"));
+                    appendFile(out + "/" + c.name + ".rowLength.u32", rl->getHostPointer<uint32_t>(), numPre);
+                    for(size_t i = 0; i < numPre; i++) { appendFile(out + "/" + c.name + ".ind.u32", ind->getHostPointer<uint32_t>() + i * stride, q.rowStride); }
+                    dumpRows(rt.getArray(*q.sg, "g"), c.name + ".w.f32", q);
+                    if(c.kind == "prune") {
+                        auto *a = pulled(rt.getArray(*c.ccu, "removed"));
+                        appendFile(out + "/" + c.name + ".removed.f32", a->getHostPointer<float>(), a->getCount());
+                    }
+                    else {
+                        dumpRows(rt.getArray(*c.ccu, "born"), c.name + ".born.f32", q);
+                        auto *a = pulled(rt.getArray(*c.ccu, "next"));
+                        appendFile(out + "/" + c.name + ".next.u32", a->getHostPointer<uint32_t>(), a->getCount());
+                    }
                 }
             }
         };

@@ -62,10 +62,14 @@ def make(name):
                 data[f"colStride.{s.name}"] = np.array(int(open(f).read()))
         # variables of custom updates and what they wrote into the projections they refer to: one row per snapshot
         for c in net.customs:
-            for var in ("applied", "sum", "peak", "total", "when", "w", "transposed"):
+            for var in ("applied", "sum", "peak", "total", "when", "w", "transposed", "removed", "born"):
                 f = os.path.join(out, f"{c.name}.{var}.f32")
                 if os.path.exists(f):
                     data[f"custom.{c.name}.{var}"] = np.fromfile(f, np.float32).reshape(net.steps // snap, -1)
+            for var in ("rowLength", "ind", "next"):
+                f = os.path.join(out, f"{c.name}.{var}.u32")
+                if os.path.exists(f):
+                    data[f"custom.{c.name}.{var}"] = np.fromfile(f, np.uint32).reshape(net.steps // snap, -1)
         np.savez_compressed(os.path.join(HERE, name + ".npz"), **data)
         total = sum(len(data[f"spikes.{p.name}"]) for p in net.pops)
         print(f"{name}: {total} spikes, {os.path.getsize(os.path.join(HERE, name + '.npz')) / 1024:.0f} KiB")

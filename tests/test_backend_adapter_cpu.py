@@ -318,6 +318,33 @@ def test_custom_updates_beside_library_kernels():
         shutil.rmtree(tmp, ignore_errors=True)
 
 
+def test_custom_connectivity_updates_generate_and_build():
+    """Custom connectivity updates: a lane per row runs the row update code (add_synapse / remove_synapse and the bookkeeping
+    of every variable on the synapses are GeNN's), the column view of a projection that learns from postsynaptic spikes is
+    rebuilt by the device library afterwards, and the model takes generated kernels by itself; asked for the library's step
+    kernels, the backend says why not."""
+    net, tmp, code, res = _generate_with("rewiring_small")
+    try:
+        assert res.returncode == 0, res.stdout[-3000:]
+        assert "__global__" in open(os.path.join(code, "neuronUpdate.cc")).read()
+        custom = open(os.path.join(code, "customUpdate.cc")).read()
+        assert "gennmiCustomConnectivityUpdatePruneKernel<<<" in custom and "gennmiCustomConnectivityUpdateSproutKernel<<<" in custom
+        prune = custom[custom.index("void updatePrune("):]
+        assert prune.index("gennmiCustomConnectivityUpdatePruneKernel<<<") < prune.index("gennmi_build_remap(")
+        # the removed synapse's slot takes the row's last one, with the weight and the other custom updates' variables
+        assert "group->ind[idx] = group->ind[lastIdx];" in custom and "group->dependentVar0[idx] = group->dependentVar0[lastIdx];" in custom
+        assert "group->rowLength[id]--;" in custom and "group->rowLength[id]++;" in custom
+        exports = _exports(os.path.join(code, "librunner.so"))
+        assert "updatePrune" in exports and "updateSprout" in exports and "updateDecay" in exports
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    net, tmp, code, res = _generate_with("rewiring_small", "--kernels=library")
+    try:
+        assert res.returncode != 0 and "custom connectivity updates beside the device library's step kernels" in res.stdout, res.stdout[-2000:]
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
 def test_generated_kernels_say_what_they_do_not_cover():
     """Asked to generate kernels for something they do not cover, the backend names it."""
     net, snap = CASES["va_small"]()
