@@ -443,8 +443,8 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
     };
 
     // Random numbers in weight-update code: a generator per synapse and step — counter (synapse id of the batch, step, call),
-    // stream 3000 + 4 x the projection's place in the model's name-ordered list + the kind of code (0 spike, 1 spike-like
-    // event, 2 postsynaptic spike, 3 synapse dynamics), key = the model's seed.  (The reference skips ahead in one Philox
+    // stream 3000 + 8 x the projection's place in the model's name-ordered list + the kind of code (0 spike, 1 spike-like
+    // event, 2 postsynaptic spike, 3 synapse dynamics, 4 postsynaptic spike-like event), key = the model's seed.  (The reference skips ahead in one Philox
     // sequence per thread, backendCUDAHIP.cc:497, so there as here no two backends draw the same numbers.)
     bool anySynapseRNG = false;
     auto addSynapseRng = [&model, &anySynapseRNG, batchSize](auto &codeEnv, const SynapseGroupInternal &, const auto &tokens, unsigned int kind)
@@ -455,7 +455,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         codeEnv.addField(Type::Uint32.addConst(), "_rng_stream" + k, Type::Uint32, "rngStream" + k,
                          [&model, kind](const SynapseGroupInternal &g, size_t)
                          {
-                             return Type::NumericValue((uint64_t)(3000 + 4 * std::distance(model.getSynapseGroups().cbegin(), model.getSynapseGroups().find(g.getName())) + kind));
+                             return Type::NumericValue((uint64_t)(3000 + 8 * std::distance(model.getSynapseGroups().cbegin(), model.getSynapseGroups().find(g.getName())) + kind));
                          });
         const std::string element = (batchSize > 1) ? "(unsigned long long)$(_syn_batch_offset) + $(id_syn)" : "(unsigned long long)$(id_syn)";
         codeEnv.add(Type::Uint32, "_rng", "gennmiRng",
@@ -802,8 +802,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const bool sparse = (matrix & SynapseMatrixConnectivity::SPARSE);
                     const bool dense = (matrix & SynapseMatrixConnectivity::DENSE) && (matrix & SynapseMatrixWeight::INDIVIDUAL);
                     if(!sparse && !dense) { notGenerated("connectivity other than SPARSE and DENSE (projection '" + arch.getName() + "')"); }
-                    if(arch.isPostSpikeEventRequired()) { notGenerated("postsynaptic spike-like events (projection '" + arch.getName() + "')"); }
-                    if(!arch.isPostSpikeRequired()) { return; }
+                    if(!arch.isPostSpikeRequired() && !arch.isPostSpikeEventRequired()) { return; }
 
                     const size_t firstBlock = post.table.numBlocks;
                     for(size_t g = 0; g < s.getGroups().size(); g++) {
@@ -824,18 +823,24 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     funcEnv.getStream() << "const auto *group = &" << structArray << "[entry.group];" << std::endl;
                     EnvironmentGroupMergedField<PostsynapticUpdateGroupMerged> groupEnv(funcEnv, s);
                     buildStandardEnvironment(groupEnv, batchSize);
-                    // (back-propagation delay: the slot of the target's ring written `delay` steps ago, backendSIMT.cc:1822-1835)
-                    const bool postDelay = arch.getTrgNeuronGroup()->isSpikeQueueRequired() && arch.getTrgNeuronGroup()->isDelayRequired();
-                    groupEnv.printLine("const unsigned int numSpikes = $(_trg_spk_cnt)[" + s.getPostSlot(postDelay, batchSize) + "];");
                     groupEnv.printLine(std::string("const unsigned int colSpan = ") + (sparse ? "$(_col_stride)" : "$(num_pre)") + ";");
                     groupEnv.getStream() << "const unsigned int chunksPerCol = (colSpan + 63u) / 64u;" << std::endl;
                     groupEnv.getStream() << "const unsigned int numWaves = entry.blocksInGroup * 4u;" << std::endl;
+                    // the queue of postsynaptic spike-like events first, then the true spikes (single_threaded_cpu/backend.cc:573-580)
+                    auto walk = [&](bool trueSpike)
+                    {
+                    const std::string suffix = trueSpike ? "" : "_event";
+                    const auto *trg = arch.getTrgNeuronGroup();
+                    // (back-propagation delay: the slot of the target's ring written `delay` steps ago, backendSIMT.cc:1822-1835)
+                    const bool postDelay = trg->isDelayRequired() && (trueSpike ? trg->isSpikeQueueRequired() : trg->isSpikeEventQueueRequired());
+                    CodeStream::Scope b1(groupEnv.getStream());
+                    groupEnv.printLine("const unsigned int numSpikes = $(_trg_spk_cnt" + suffix + ")[" + s.getPostSlot(postDelay, batchSize) + "];");
                     groupEnv.getStream() << "const unsigned long long numItems = (unsigned long long)numSpikes * chunksPerCol;" << std::endl;
                     groupEnv.getStream() << "for(unsigned long long item = entry.blockInGroup * 4u + (threadIdx.x / 64u); item < numItems; item += numWaves)";
                     {
                         CodeStream::Scope b2(groupEnv.getStream());
                         EnvironmentGroupMergedField<PostsynapticUpdateGroupMerged> synEnv(groupEnv, s);
-                        synEnv.printLine("const unsigned int spike = $(_trg_spk)[" + s.getPostVarIndex(postDelay, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "(unsigned int)(item / chunksPerCol)") + "];");
+                        synEnv.printLine("const unsigned int spike = $(_trg_spk" + suffix + ")[" + s.getPostVarIndex(postDelay, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "(unsigned int)(item / chunksPerCol)") + "];");
                         synEnv.getStream() << "const unsigned int i = (unsigned int)(item % chunksPerCol) * 64u + (threadIdx.x & 63u);" << std::endl;
                         if(sparse) {
                             synEnv.print("if(i < $(_col_length)[spike])");
@@ -861,10 +866,19 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                             codeEnv.add(Type::Uint32.addConst(), "id_post", "spike");
                             codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPre",
                                         "gennmi_kernel::addScalar(&$(_out_pre)[" + s.getPreISynIndex(batchSize, "$(id_pre)") + "], $(0))");
-                            addSynapseRng(codeEnv, arch, arch.getWUInitialiser().getPostSpikeSynCodeTokens(), 2);
-                            s.generateSpikeUpdate(*this, codeEnv, batchSize, dt);
+                            if(trueSpike) {
+                                addSynapseRng(codeEnv, arch, arch.getWUInitialiser().getPostSpikeSynCodeTokens(), 2);
+                                s.generateSpikeUpdate(*this, codeEnv, batchSize, dt);
+                            }
+                            else {
+                                addSynapseRng(codeEnv, arch, arch.getWUInitialiser().getPostEventSynCodeTokens(), 4);
+                                s.generateSpikeEventUpdate(*this, codeEnv, batchSize, dt);
+                            }
                         }
                     }
+                    };
+                    if(arch.isPostSpikeEventRequired()) { walk(false); }
+                    if(arch.isPostSpikeRequired()) { walk(true); }
                 });
         });
     }

@@ -494,3 +494,25 @@ def rewiring(steps=200):
     net.customs.append(Custom("Sprout", "Sprout", "sprout", "AB_plastic", params=dict(weight=0.2)))
     net.custom_calls = [("Decay", 30), ("Prune", 40), ("Sprout", 25)]
     return net
+
+
+def post_events(n_a=300, n_b=130, steps=200, seed=23, dt=1.0):
+    """Postsynaptic spike-like events: a projection whose synapses, while their TARGET's membrane potential is above a midpoint,
+    count the step and send a fraction of their weight back to their source (a model of the test driver after
+    tests/features/test_event_propagation.py), beside a plain inhibitory projection back."""
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.55, TauRefrac=2.0)
+    net = Net(name="post_events", dt=dt, steps=steps, seed=seed)
+    net.pops.append(Pop("A", "lif", n_a, dict(lif), {"V": (-60.0 + 9.5 * rng.uniform(seed, 1, 0, n_a)).astype(np.float32),
+                                                     "RefracTime": np.zeros(n_a, np.float32)}))
+    net.pops.append(Pop("B", "lif", n_b, dict(lif, Ioffset=0.45), {"V": (-60.0 + 9.5 * rng.uniform(seed, 2, 0, n_b)).astype(np.float32),
+                                                                   "RefracTime": np.zeros(n_b, np.float32)}))
+
+    def sparse(name, src, trg, n_src, n_trg, stride, stream, lo, hi, **kw):
+        ind = np.sort(rng.randint(seed, stream, 0, n_src * stride, n_trg).reshape(n_src, stride), axis=1).astype(np.uint32)
+        row_length = (stride - rng.randint(seed, stream + 1, 0, n_src, stride // 3)).astype(np.uint32)
+        g = (lo + (hi - lo) * rng.uniform(seed, stream + 2, 0, n_src * stride)).astype(np.float32).reshape(n_src, stride)
+        return Syn(name, src, trg, psm="expcurr", tau=5.0, row_stride=stride, row_length=row_length, ind=ind, g=g, **kw)
+
+    net.syns.append(sparse("AB_feedback", "A", "B", n_a, n_b, 20, 10, 0.0, 0.1, wum="post_event", wum_params=dict(Vmid=-53.0, back=0.002)))
+    net.syns.append(sparse("BA_inhibit", "B", "A", n_b, n_a, 30, 20, -0.3, -0.05, wum="static"))
+    return net

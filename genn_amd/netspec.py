@@ -234,6 +234,8 @@ def write_netspec(net: Net, path: str):
             w = f"static_graded {float(s.wum_params['Epre'])!r} {float(s.wum_params['Vslope'])!r}"
         elif s.wum == "stochastic":        # a model of the test driver that draws a random number per synaptic event
             w = f"stochastic {float(s.wum_params['pRelease'])!r}"
+        elif s.wum == "post_event":        # a model of the test driver with postsynaptic spike-like events (condition on the target's V)
+            w = f"post_event {float(s.wum_params['Vmid'])!r} {float(s.wum_params['back'])!r}"
         elif s.wum == "leaky_graded":      # a model of the test driver with synapse dynamics code (runs for every synapse every step)
             w = f"leaky_graded {float(s.wum_params['Vmid'])!r} {float(s.wum_params['decay'])!r}"
         else:
@@ -242,7 +244,7 @@ def write_netspec(net: Net, path: str):
         opts = (" hint_pre" if s.hint_pre else "") + (f" tps {s.threads_per_spike}" if s.threads_per_spike > 1 else "")
         if s.axonal_delay_steps:
             opts += f" axonal_delay {int(s.axonal_delay_steps)}"
-        if s.wum in ("stdp_trace", "stdp_additive", "timing_copy", "prev_timing"):
+        if s.wum in ("stdp_trace", "stdp_additive", "timing_copy", "prev_timing", "post_event"):
             mask = np.arange(s.row_stride)[None, :] < s.row_length[:, None]
             col = s.col_stride or int(np.bincount(s.ind[mask], minlength=net.pop(s.trg).n).max())
             opts += f" col_stride {max(1, col)}"

@@ -188,6 +188,24 @@ public:
 };
 IMPLEMENT_SNIPPET(LeakyGraded);
 
+// Postsynaptic spike-like events (after tests/features/test_event_propagation.py): while a target's membrane potential is above
+// a midpoint, every synapse onto it counts the step in a variable of its own and sends a fraction of its weight back to its
+// source (addToPre), next to ordinary forward transmission.
+class PostEventFeedback : public WeightUpdateModels::Base
+{
+public:
+    DECLARE_SNIPPET(PostEventFeedback);
+    SET_PARAMS({"Vmid", "back"});
+    SET_VARS({{"g", "scalar", VarAccess::READ_ONLY}, {"hits", "scalar"}});
+    SET_POST_NEURON_VAR_REFS({{"Vpost", "scalar", VarAccessMode::READ_ONLY}});
+    SET_PRE_SPIKE_SYN_CODE("addToPost(g);\n");
+    SET_POST_EVENT_THRESHOLD_CONDITION_CODE("Vpost > Vmid");
+    SET_POST_EVENT_SYN_CODE(
+        "hits += 1.0;\n"
+        "addToPre(back * g);\n");
+};
+IMPLEMENT_SNIPPET(PostEventFeedback);
+
 // Synapses that release with a probability: random numbers in weight-update code (what a user writes for stochastic
 // transmission; cf. tests/features/test_rng.py, which draws in neuron code).
 class StochasticPulse : public WeightUpdateModels::Base
@@ -440,7 +458,7 @@ int main(int argc, char *argv[])
                     if(s.wum == "static_delay") { ls >> s.maxDenDelay; }
                     else if(s.wum == "stdp_trace" || s.wum == "stdp") { s.wumP.resize(6); for(auto &c : s.wumP) ls >> c; }
                     else if(s.wum == "static_const" || s.wum == "stochastic") { s.wumP.resize(1); ls >> s.wumP[0]; }
-                    else if(s.wum == "static_graded" || s.wum == "leaky_graded") { s.wumP.resize(2); ls >> s.wumP[0] >> s.wumP[1]; }
+                    else if(s.wum == "static_graded" || s.wum == "leaky_graded" || s.wum == "post_event") { s.wumP.resize(2); ls >> s.wumP[0] >> s.wumP[1]; }
                     else if(s.wum != "static" && s.wum != "static_reverse" && s.wum != "static_init" && s.wum != "timing_copy" && s.wum != "prev_timing") throw std::runtime_error("wum " + s.wum);
                     ls >> s.psm;
                     if(s.psm == "expcurr") { s.psmP.resize(1); ls >> s.psmP[0]; }
@@ -527,6 +545,10 @@ int main(int argc, char *argv[])
             else if(s.wum == "leaky_graded") {
                 wum = initWeightUpdate<LeakyGraded>({{"Vmid", s.wumP.at(0)}, {"decay", s.wumP.at(1)}}, {{"g", uninitialisedVar()}, {"x", 0.0}}, {}, {},
                                                     {{"Vpre", createVarRef(popByName.at(s.src)->ng, "V")}}, {});
+            }
+            else if(s.wum == "post_event") {
+                wum = initWeightUpdate<PostEventFeedback>({{"Vmid", s.wumP.at(0)}, {"back", s.wumP.at(1)}}, {{"g", uninitialisedVar()}, {"hits", 0.0}}, {}, {},
+                                                          {}, {{"Vpost", createVarRef(popByName.at(s.trg)->ng, "V")}});
             }
             else if(s.wum == "prev_timing") {
                 wum = initWeightUpdate<PrevTiming>({}, {{"g", uninitialisedVar()}, {"wPre", -1.0}, {"wPost", -1.0}});
@@ -750,7 +772,7 @@ int main(int argc, char *argv[])
             for(auto &s : syns) {
                 const auto *sgi = static_cast<const SynapseGroupInternal*>(s.sg);
                 fm << s.name << " " << sgi->getFusedPSTarget().getName() << std::endl;
-                if(s.wum == "stdp_trace" || s.wum == "stdp" || s.wum == "timing_copy" || s.wum == "prev_timing") {
+                if(s.wum == "stdp_trace" || s.wum == "stdp" || s.wum == "timing_copy" || s.wum == "prev_timing" || s.wum == "post_event") {
                     auto *cl = rt.getArray(*s.sg, "colLength"); auto *rm = rt.getArray(*s.sg, "remap");
                     cl->pullFromDevice(); rm->pullFromDevice();
                     appendFile(out + "/" + s.name + ".colLength.u32", cl->getHostPointer<uint32_t>(), cl->getCount());
@@ -789,6 +811,11 @@ int main(int argc, char *argv[])
                     auto *a = pulled(rt.getArray(*s.sg, "g"));
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
                     for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + ".g.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
+                }
+                if(s.wum == "post_event") {
+                    const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
+                    auto *a = pulled(rt.getArray(*s.sg, "hits"));
+                    for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + ".hits.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
                 }
                 if(s.wum == "leaky_graded") {
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);

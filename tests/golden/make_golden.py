@@ -47,11 +47,11 @@ def make(name):
         for s in net.syns:
             for var, dtype in (("outPost", np.float32), ("denDelay", np.float32), ("g", np.float32), ("preTrace", np.float32),
                                ("postTrace", np.float32), ("colLength", np.uint32), ("remap", np.uint32),
-                               ("wPre", np.float32), ("wPost", np.float32), ("sPre", np.float32), ("sPost", np.float32), ("x", np.float32)):
+                               ("wPre", np.float32), ("wPost", np.float32), ("sPre", np.float32), ("sPost", np.float32), ("x", np.float32), ("hits", np.float32)):
                 f = os.path.join(out, f"{s.name}.{var}.{'u32' if dtype == np.uint32 else 'f32'}")
                 if os.path.exists(f):
                     a = np.fromfile(f, dtype)
-                    if var in ("g", "denDelay", "outPost", "preTrace", "postTrace", "wPre", "wPost", "sPre", "sPost", "x"):
+                    if var in ("g", "denDelay", "outPost", "preTrace", "postTrace", "wPre", "wPost", "sPre", "sPost", "x", "hits"):
                         a = a.reshape(net.steps // snap, -1)[-1] if var in ("g", "denDelay") else a.reshape(net.steps // snap, -1)
                     data[f"{var}.{s.name}"] = a
             f = os.path.join(out, f"{s.name}.events.u32")

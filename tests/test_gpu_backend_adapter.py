@@ -58,7 +58,7 @@ def _run(case, *options):
 LIBRARY_CASES = sorted(set(CASES) - REFERENCE_ONLY)
 # what the generated kernels cover: SPARSE / DENSE matrices, any neuron, postsynaptic, current-source and weight-update code
 # without delay slots, spike-like events or random numbers
-GENERATED_CASES = ["custom_small", "dynamic_small", "synapse_dynamics_small", "prev_times_small", "stdp_delay_small", "va_delay_small", "graded_small", "conv_small", "dense_small", "va_small", "potjans_small", "izhikevich_small", "stdp_small", "stdp_additive_small", "reverse_small"]
+GENERATED_CASES = ["post_events_small", "custom_small", "dynamic_small", "synapse_dynamics_small", "prev_times_small", "stdp_delay_small", "va_delay_small", "graded_small", "conv_small", "dense_small", "va_small", "potjans_small", "izhikevich_small", "stdp_small", "stdp_additive_small", "reverse_small"]
 
 
 @pytest.mark.parametrize("case", LIBRARY_CASES)
@@ -130,6 +130,12 @@ def _compare_with_fixture(case, *options):
                 if key in golden:
                     got = np.fromfile(os.path.join(out, f"{s.name}.{var}.f32"), np.float32).reshape(net.steps // snap, -1)
                     assert np.array_equal(got, golden[key]), key
+            if f"hits.{s.name}" in golden:
+                # steps counted per synapse by postsynaptic spike-like events (within the rows: their padding is never initialised)
+                valid = (np.arange(s.row_stride)[None, :] < s.row_length[:, None]).reshape(-1)
+                got = np.fromfile(os.path.join(out, f"{s.name}.hits.f32"), np.float32).reshape(net.steps // snap, -1)
+                assert np.array_equal(got[:, valid], golden[f"hits.{s.name}"][:, valid]), f"hits.{s.name}"
+                assert got[-1, valid].sum() > 1000
             for var in ("g", "preTrace", "postTrace", "outPost", "x"):
                 key = f"{var}.{s.name}"
                 if key in golden:
