@@ -1742,6 +1742,8 @@ Backend createBackend(const ModelSpecInternal &model, const filesystem::path&, p
             generated = generated || anyDynamic(s.second.getPSInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isPSParamDynamic(p); });
             generated = generated || anyDynamic(s.second.getWUInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isWUParamDynamic(p); });
         }
+        // ... or when the model is not single precision: the library's kernels are fp32
+        generated = generated || model.getPrecision() != Type::Float || model.getTimePrecision() != Type::Float;
         // ... or when custom connectivity updates rewire a projection: the library's launch plans rely on rows sorted by target,
         // which removing and adding synapses does not keep
         generated = generated || !model.getCustomConnectivityUpdates().empty();

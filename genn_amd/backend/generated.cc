@@ -81,16 +81,21 @@ void genDeviceStructArray(CodeStream &decl, CodeStream &upload, const BackendBas
         upload << "GENNMI_CHECK(gennmi_memcpy_to_device(" << dev << ", staging, sizeof(staging)));" << std::endl;
     }
 }
-// gennrand_* as the reference's backends declare them (cuda/backend.cc:35-43), over gennmi_kernel::Rng
-const EnvironmentLibrary::Library simRNGFunctions = {
-    {"gennrand", {Type::ResolvedType::createFunction(Type::Uint32, {}), "gennmi_kernel::rngWord($(_rng))"}},
-    {"gennrand_uniform", {Type::ResolvedType::createFunction(Type::Float, {}), "gennmi_kernel::rngUniform($(_rng))"}},
-    {"gennrand_normal", {Type::ResolvedType::createFunction(Type::Float, {}), "gennmi_kernel::rngNormal($(_rng))"}},
-    {"gennrand_exponential", {Type::ResolvedType::createFunction(Type::Float, {}), "gennmi_kernel::rngExponential($(_rng))"}},
-    {"gennrand_log_normal", {Type::ResolvedType::createFunction(Type::Float, {Type::Float, Type::Float}), "gennmi_kernel::rngLogNormal($(_rng), $(0), $(1))"}},
-    {"gennrand_gamma", {Type::ResolvedType::createFunction(Type::Float, {Type::Float}), "gennmi_kernel::rngGamma($(_rng), $(0))"}},
-    {"gennrand_binomial", {Type::ResolvedType::createFunction(Type::Uint32, {Type::Uint32, Type::Float}), "gennmi_kernel::rngBinomial($(_rng), $(0), $(1))"}},
-};
+// gennrand_* as the reference's backends declare them (cuda/backend.cc:35-43), over gennmi_kernel::Rng.  The draws have fp32
+// resolution whatever the model's precision (a double-precision model gets them converted).
+EnvironmentLibrary::Library simRNGLibrary(const Type::ResolvedType &scalar)
+{
+    const std::string cast = (scalar == Type::Float) ? "" : ("(" + scalar.getName() + ")");
+    return {
+        {"gennrand", {Type::ResolvedType::createFunction(Type::Uint32, {}), "gennmi_kernel::rngWord($(_rng))"}},
+        {"gennrand_uniform", {Type::ResolvedType::createFunction(scalar, {}), cast + "gennmi_kernel::rngUniform($(_rng))"}},
+        {"gennrand_normal", {Type::ResolvedType::createFunction(scalar, {}), cast + "gennmi_kernel::rngNormal($(_rng))"}},
+        {"gennrand_exponential", {Type::ResolvedType::createFunction(scalar, {}), cast + "gennmi_kernel::rngExponential($(_rng))"}},
+        {"gennrand_log_normal", {Type::ResolvedType::createFunction(scalar, {scalar, scalar}), cast + "gennmi_kernel::rngLogNormal($(_rng), (float)($(0)), (float)($(1)))"}},
+        {"gennrand_gamma", {Type::ResolvedType::createFunction(scalar, {scalar}), cast + "gennmi_kernel::rngGamma($(_rng), (float)($(0)))"}},
+        {"gennrand_binomial", {Type::ResolvedType::createFunction(Type::Uint32, {Type::Uint32, scalar}), "gennmi_kernel::rngBinomial($(_rng), $(0), (float)($(1)))"}},
+    };
+}
 }   // anonymous namespace
 
 namespace GeNN::CodeGenerator::MI355X
@@ -102,7 +107,8 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     const ModelSpecInternal &model = modelMerged.getModel();
     // batches: the grid's second dimension (backendCUDAHIP.cc:332-338 does the same); every batch compacts its own queue
     const unsigned int batchSize = model.getBatchSize();
-    if(model.getPrecision() != Type::Float || model.getTimePrecision() != Type::Float) { notGenerated("double precision"); }
+    const std::string timeType = model.getTimePrecision().getName();
+    const EnvironmentLibrary::Library simRNGFunctions = simRNGLibrary(model.getPrecision());
     const bool recording = model.isRecordingInUse();
 
     std::ostringstream kernelStream, declStream, uploadStream, argStream, paramStream;
@@ -362,7 +368,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     os << std::endl;
     if(anyPrevTimes) {
         os << "__device__ const gennmi_kernel::BlockEntry gennmiPrevSpikeTimeBlocks[] = {" << std::endl << prevTable.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
-        os << "__global__ __launch_bounds__(256) void gennmiPrevSpikeTimeKernel(float t" << prevParams.str() << ")";
+        os << "__global__ __launch_bounds__(256) void gennmiPrevSpikeTimeKernel(" << timeType << " t" << prevParams.str() << ")";
         CodeStream::Scope b(os);
         os << prevStream.str();
     }
@@ -372,7 +378,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         os << queueStream.str();
     }
     os << std::endl;
-    os << "__global__ __launch_bounds__(256) void gennmiNeuronUpdateKernel(float t, unsigned int recordingTimestep, uint32_t gennmiTag, "
+    os << "__global__ __launch_bounds__(256) void gennmiNeuronUpdateKernel(" << timeType << " t, unsigned int recordingTimestep, uint32_t gennmiTag, "
           "unsigned long long *gennmiAgg, uint32_t *gennmiError, unsigned long long gennmiSeed, unsigned long long gennmiStep" << paramStream.str() << ")";
     {
         CodeStream::Scope b(os);
@@ -421,6 +427,9 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
     const double dt = model.getDT();
     const unsigned int batchSize = model.getBatchSize();
 
+    const std::string timeType = model.getTimePrecision().getName();
+    const EnvironmentLibrary::Library simRNGFunctions = simRNGLibrary(model.getPrecision());
+
     std::ostringstream declStream, uploadStream;
     CodeStream decl(declStream), upload(uploadStream);
 
@@ -431,7 +440,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         BlockTable table;
     };
     KernelText delay, dynamics, pre, post;
-    auto makeEnv = [&model](CodeStream &stream, EnvironmentLibrary &lib, auto use)
+    auto makeEnv = [&model, &simRNGFunctions](CodeStream &stream, EnvironmentLibrary &lib, auto use)
     {
         EnvironmentLibrary rngLib(lib, simRNGFunctions);        // (gennrand_* of weight-update code: `_rng` exists where it is used)
         EnvironmentExternal funcEnv(rngLib);
@@ -911,22 +920,22 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
     os << std::endl;
     const bool anyDelay = delay.table.numBlocks > 0, anyPre = pre.table.numBlocks > 0, anyPost = post.table.numBlocks > 0, anyDynamics = dynamics.table.numBlocks > 0;
     if(anyDynamics) {
-        os << "__global__ __launch_bounds__(256) void gennmiSynapseDynamicsKernel(float t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << dynamics.params.str() << ")";
+        os << "__global__ __launch_bounds__(256) void gennmiSynapseDynamicsKernel(" << timeType << " t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << dynamics.params.str() << ")";
         CodeStream::Scope b(os);
         os << dynamics.body.str();
     }
     if(anyDelay) {
-        os << "__global__ void gennmiDendriticDelayUpdateKernel(float t" << delay.params.str() << ")";
+        os << "__global__ void gennmiDendriticDelayUpdateKernel(" << timeType << " t" << delay.params.str() << ")";
         CodeStream::Scope b(os);
         os << delay.body.str();
     }
     if(anyPre) {
-        os << "__global__ __launch_bounds__(256) void gennmiPresynapticUpdateKernel(float t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << pre.params.str() << ")";
+        os << "__global__ __launch_bounds__(256) void gennmiPresynapticUpdateKernel(" << timeType << " t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << pre.params.str() << ")";
         CodeStream::Scope b(os);
         os << pre.body.str();
     }
     if(anyPost) {
-        os << "__global__ __launch_bounds__(256) void gennmiPostsynapticUpdateKernel(float t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << post.params.str() << ")";
+        os << "__global__ __launch_bounds__(256) void gennmiPostsynapticUpdateKernel(" << timeType << " t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << post.params.str() << ")";
         CodeStream::Scope b(os);
         os << post.body.str();
     }
@@ -989,6 +998,7 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     std::ostringstream declStream, uploadStream, deviceStream, hostStream;
     CodeStream decl(declStream), upload(uploadStream), device(deviceStream), host(hostStream);
     const std::string timeType = model.getTimePrecision().getName();
+    const EnvironmentLibrary::Library simRNGFunctions = simRNGLibrary(model.getPrecision());
     auto reduceOps = [this](auto &env, const std::vector<ReductionTarget> &targets)
     {
         for(const auto &r : targets) { env.printLine(getReductionOperation("_lr" + r.name, "$(" + r.name + ")", r.access, r.type) + ";"); }

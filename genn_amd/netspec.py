@@ -112,6 +112,7 @@ class Net:
     # parameters changed while the model runs (setParamDynamic + Runtime::setDynamicParamValue):
     # (kind, group, parameter, step, value) with kind in neuron | cs | wu | ps; the value holds from `step` on
     dynamic: List[tuple] = field(default_factory=list)
+    precision: str = "float"        # "double": ModelSpec::setPrecision(Type::Double); the netspec's arrays and the dumps stay fp32
     customs: List[Custom] = field(default_factory=list)
     custom_calls: List[tuple] = field(default_factory=list)     # (update group, every n steps): called after steps n, 2n, ...
 
@@ -138,6 +139,8 @@ class Net:
                     h.update(np.ascontiguousarray(a).tobytes())
         for d in self.dynamic:
             h.update(repr(tuple(d)).encode())
+        if self.precision != "float":
+            h.update(self.precision.encode())
         for c in self.customs:
             h.update(repr((c.name, c.group, c.kind, c.target, c.target2, sorted(c.params.items()))).encode())
         for c in self.custom_calls:
@@ -169,6 +172,8 @@ def write_netspec(net: Net, path: str):
     lines.append(f"snap {snap}")
     if getattr(net, "batch_size", 1) != 1:
         lines.append(f"batch {int(net.batch_size)}")
+    if net.precision != "float":
+        lines.append(f"precision {net.precision}")
     if any(s.matrix in ("procedural", "sparse_init") for s in net.syns) or any(c.model == "poisson_exp" for c in net.css) or any(p.model == "poisson" for p in net.pops) \
             or any(s.wum == "stochastic" for s in net.syns):
         lines.append(f"seed {int(net.seed)}")        # procedural matrices and Poisson sources draw from the model's seed

@@ -24,6 +24,7 @@
 #include <map>
 #include <sstream>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include <plog/Appenders/ConsoleAppender.h>
@@ -372,6 +373,24 @@ struct SynSpec
     SynapseGroup *sg = nullptr;
 };
 
+// Arrays of the model's scalar type hold float or double (--precision=double); the netspec's files and the dumps are fp32 either way
+static void appendScalars(const std::string &path, Runtime::ArrayBase *a, size_t first, size_t count)
+{
+    if(a->getType() == Type::Double) {
+        const double *src = a->getHostPointer<double>() + first;
+        std::vector<float> narrow(src, src + count);
+        appendFile(path, narrow.data(), count);
+    }
+    else {
+        appendFile(path, a->getHostPointer<float>() + first, count);
+    }
+}
+static void storeScalars(Runtime::ArrayBase *a, size_t first, const float *src, size_t count)
+{
+    if(a->getType() == Type::Double) { std::copy_n(src, count, a->getHostPointer<double>() + first); }
+    else { std::copy_n(src, count, a->getHostPointer<float>() + first); }
+}
+
 // custom <name> <update group> <kind> <target> [<second target>] [<params>]; custom_call <update group> <every n steps>
 struct CustomSpec
 {
@@ -444,6 +463,7 @@ int main(int argc, char *argv[])
                 else if(k == "fuse_psm") ls >> fuse;
                 else if(k == "batch") ls >> batch;
                 else if(k == "seed") ls >> seed;
+                else if(k == "precision") { std::string v; ls >> v; doublePrecision = (v == "double"); }      // ModelSpec::setPrecision
                 else if(k == "dynamic") { DynamicSpec d; ls >> d.kind >> d.group >> d.param >> d.step >> d.value; dynamics.push_back(d); dynamicParams.push_back(d.kind + ":" + d.group + "." + d.param); }
                 else if(k == "pop") { PopSpec p; ls >> p.name >> p.model >> p.n; double v; while(ls >> v) p.p.push_back(v); pops.push_back(p); }
                 else if(k == "cs") { CSSpec c; ls >> c.name >> c.model >> c.pop; double v; while(ls >> v) c.p.push_back(v); css.push_back(c); }
@@ -686,6 +706,12 @@ int main(int argc, char *argv[])
         rt.initialize();
         // a file holds either the whole array or one batch's worth, which is then replicated
         auto load = [&](Runtime::ArrayBase *a, const std::string &file) {
+            if(a->getType() == Type::Double && file.size() > 4 && file.compare(file.size() - 4, 4, ".f32") == 0) {
+                const auto values = readFile<float>(in + "/" + file);
+                if(values.empty() || (a->getCount() % values.size()) != 0) { throw std::runtime_error(file + ": does not tile the array"); }
+                for(size_t o = 0; o < a->getCount(); o += values.size()) { storeScalars(a, o, values.data(), values.size()); }
+                return;
+            }
             const auto bytes = readFile<char>(in + "/" + file);
             if(bytes.empty() || (a->getSizeBytes() % bytes.size()) != 0) {
                 throw std::runtime_error(file + ": " + std::to_string(bytes.size()) + " bytes do not tile an array of " + std::to_string(a->getSizeBytes()));
@@ -707,7 +733,7 @@ int main(int argc, char *argv[])
                 const auto st = readFile<float>(in + "/" + p.name + ".spikeTimes.f32");
                 rt.allocateArray(*p.ng, "spikeTimes", st.size());
                 auto *a = rt.getArray(*p.ng, "spikeTimes");
-                std::copy(st.begin(), st.end(), a->getHostPointer<float>());
+                storeScalars(a, 0, st.data(), st.size());
                 a->pushToDevice();
             }
         }
@@ -725,11 +751,18 @@ int main(int argc, char *argv[])
             using T = decltype(zero);
             const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
             const auto rows = readFile<T>(in + "/" + file, numPre * s.rowStride);
-            auto *dst = a->getHostPointer<T>();
             // (variables a learning rule writes have one copy per batch: every copy starts from the file's values)
             const size_t copies = a->getCount() / (numPre * stride);
-            for(size_t c = 0; c < copies; c++) {
-                for(size_t i = 0; i < numPre; i++) { std::copy_n(rows.begin() + i * s.rowStride, s.rowStride, dst + (c * numPre + i) * stride); }
+            if constexpr(std::is_same_v<T, float>) {
+                for(size_t c = 0; c < copies; c++) {
+                    for(size_t i = 0; i < numPre; i++) { storeScalars(a, (c * numPre + i) * stride, rows.data() + i * s.rowStride, s.rowStride); }
+                }
+            }
+            else {
+                auto *dst = a->getHostPointer<T>();
+                for(size_t c = 0; c < copies; c++) {
+                    for(size_t i = 0; i < numPre; i++) { std::copy_n(rows.begin() + i * s.rowStride, s.rowStride, dst + (c * numPre + i) * stride); }
+                }
             }
         };
         for(auto &s : syns) {
@@ -762,7 +795,7 @@ int main(int argc, char *argv[])
             appendFile(out + "/" + s.name + ".ind.u32", ind->getHostPointer<uint32_t>(), numPre * stride);
             if(s.wum != "static_const") {
                 auto *g = rt.getArray(*s.sg, "g"); g->pullFromDevice();
-                appendFile(out + "/" + s.name + ".g.f32", g->getHostPointer<float>(), numPre * stride);
+                appendScalars(out + "/" + s.name + ".g.f32", g, 0, numPre * stride);
             }
         }
 
@@ -792,53 +825,53 @@ int main(int argc, char *argv[])
                 if(p.model == "ssa" || p.model == "poisson") continue;
                 pulled(rt.getArray(*p.ng, "V"));
                 pulled(rt.getArray(*p.ng, (p.model == "lif" || p.model == "lifa") ? "RefracTime" : "U"));
-                appendFile(out + "/" + p.name + ".V.f32", rt.getArray(*p.ng, "V")->getHostPointer<float>(), (size_t)p.n * batch);
-                if(p.model == "lif" || p.model == "lifa") appendFile(out + "/" + p.name + ".RefracTime.f32", rt.getArray(*p.ng, "RefracTime")->getHostPointer<float>(), (size_t)p.n * batch);
-                if(p.model == "lifa") { auto *a = pulled(rt.getArray(*p.ng, "A")); appendFile(out + "/" + p.name + ".A.f32", a->getHostPointer<float>(), (size_t)p.n * batch); }
-                if(p.model == "izh") appendFile(out + "/" + p.name + ".U.f32", rt.getArray(*p.ng, "U")->getHostPointer<float>(), (size_t)p.n * batch);
+                appendScalars(out + "/" + p.name + ".V.f32", rt.getArray(*p.ng, "V"), 0, (size_t)p.n * batch);
+                if(p.model == "lif" || p.model == "lifa") appendScalars(out + "/" + p.name + ".RefracTime.f32", rt.getArray(*p.ng, "RefracTime"), 0, (size_t)p.n * batch);
+                if(p.model == "lifa") { auto *a = pulled(rt.getArray(*p.ng, "A")); appendScalars(out + "/" + p.name + ".A.f32", a, 0, (size_t)p.n * batch); }
+                if(p.model == "izh") appendScalars(out + "/" + p.name + ".U.f32", rt.getArray(*p.ng, "U"), 0, (size_t)p.n * batch);
             }
             for(auto &s : syns) {
                 const auto *sgi = static_cast<const SynapseGroupInternal*>(s.sg);
                 if(&sgi->getFusedPSTarget() == sgi) {
                     auto *a = pulled(rt.getArray(*s.sg, "outPost"));
-                    appendFile(out + "/" + s.name + ".outPost.f32", a->getHostPointer<float>(), a->getCount());
+                    appendScalars(out + "/" + s.name + ".outPost.f32", a, 0, a->getCount());
                     if(sgi->isDendriticOutputDelayRequired()) {
                         auto *d = pulled(rt.getArray(*s.sg, "denDelay"));
-                        appendFile(out + "/" + s.name + ".denDelay.f32", d->getHostPointer<float>(), d->getCount());
+                        appendScalars(out + "/" + s.name + ".denDelay.f32", d, 0, d->getCount());
                     }
                 }
                 if(s.wum == "stdp_trace" || s.wum == "stdp") {
                     auto *a = pulled(rt.getArray(*s.sg, "g"));
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
-                    for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + ".g.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
+                    for(size_t i = 0; i < numPre * batch; i++) { appendScalars(out + "/" + s.name + ".g.f32", a, i * stride, s.rowStride); }
                 }
                 if(s.wum == "post_event") {
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
                     auto *a = pulled(rt.getArray(*s.sg, "hits"));
-                    for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + ".hits.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
+                    for(size_t i = 0; i < numPre * batch; i++) { appendScalars(out + "/" + s.name + ".hits.f32", a, i * stride, s.rowStride); }
                 }
                 if(s.wum == "leaky_graded") {
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
                     auto *a = pulled(rt.getArray(*s.sg, "x"));
-                    for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + ".x.f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
+                    for(size_t i = 0; i < numPre * batch; i++) { appendScalars(out + "/" + s.name + ".x.f32", a, i * stride, s.rowStride); }
                 }
                 if(s.wum == "timing_copy" || s.wum == "prev_timing") {
                     const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
                     for(const char *var : {"wPre", "wPost"}) {
                         auto *a = pulled(rt.getArray(*s.sg, var));
-                        for(size_t i = 0; i < numPre * batch; i++) { appendFile(out + "/" + s.name + "." + var + ".f32", a->getHostPointer<float>() + i * stride, s.rowStride); }
+                        for(size_t i = 0; i < numPre * batch; i++) { appendScalars(out + "/" + s.name + "." + var + ".f32", a, i * stride, s.rowStride); }
                     }
                 }
                 if(s.wum == "timing_copy") {
                     for(const char *var : {"sPre", "sPost"}) {
                         auto *a = pulled(rt.getArray(*s.sg, var));
-                        appendFile(out + "/" + s.name + "." + var + ".f32", a->getHostPointer<float>(), a->getCount());
+                        appendScalars(out + "/" + s.name + "." + var + ".f32", a, 0, a->getCount());
                     }
                 }
                 if(s.wum == "stdp_trace") {
                     auto *a = pulled(rt.getArray(*s.sg, "preTrace")); auto *b = pulled(rt.getArray(*s.sg, "postTrace"));
-                    appendFile(out + "/" + s.name + ".preTrace.f32", a->getHostPointer<float>(), a->getCount());
-                    appendFile(out + "/" + s.name + ".postTrace.f32", b->getHostPointer<float>(), b->getCount());
+                    appendScalars(out + "/" + s.name + ".preTrace.f32", a, 0, a->getCount());
+                    appendScalars(out + "/" + s.name + ".postTrace.f32", b, 0, b->getCount());
                 }
             }
         };
@@ -849,22 +882,22 @@ int main(int argc, char *argv[])
             a->pullFromDevice();
             if(q.matrix == "sparse") {
                 const size_t numPre = popByName.at(q.src)->n, stride = backendStride(q), copies = a->getCount() / (numPre * stride);
-                for(size_t i = 0; i < numPre * copies; i++) { appendFile(out + "/" + file, a->getHostPointer<float>() + i * stride, q.rowStride); }
+                for(size_t i = 0; i < numPre * copies; i++) { appendScalars(out + "/" + file, a, i * stride, q.rowStride); }
             }
             else {
-                appendFile(out + "/" + file, a->getHostPointer<float>(), a->getCount());
+                appendScalars(out + "/" + file, a, 0, a->getCount());
             }
         };
         auto customSnapshot = [&]() {
             for(auto &c : customs) {
                 if(c.kind == "decay") {
                     auto *a = pulled(rt.getArray(*c.cu, "applied"));
-                    appendFile(out + "/" + c.name + ".applied.f32", a->getHostPointer<float>(), a->getCount());
+                    appendScalars(out + "/" + c.name + ".applied.f32", a, 0, a->getCount());
                 }
                 else if(c.kind == "neuron_reduce") {
                     for(const char *var : {"sum", "peak"}) {
                         auto *a = pulled(rt.getArray(*c.cu, var));
-                        appendFile(out + "/" + c.name + "." + var + ".f32", a->getHostPointer<float>(), a->getCount());
+                        appendScalars(out + "/" + c.name + "." + var + ".f32", a, 0, a->getCount());
                     }
                 }
                 else if(c.kind == "wu_decay") {
@@ -892,7 +925,7 @@ int main(int argc, char *argv[])
                     dumpRows(rt.getArray(*q.sg, "g"), c.name + ".w.f32", q);
                     if(c.kind == "prune") {
                         auto *a = pulled(rt.getArray(*c.ccu, "removed"));
-                        appendFile(out + "/" + c.name + ".removed.f32", a->getHostPointer<float>(), a->getCount());
+                        appendScalars(out + "/" + c.name + ".removed.f32", a, 0, a->getCount());
                     }
                     else {
                         dumpRows(rt.getArray(*c.ccu, "born"), c.name + ".born.f32", q);
@@ -910,7 +943,7 @@ int main(int argc, char *argv[])
                 if(c.model == "noise") {
                     const unsigned int n = popByName.at(c.pop)->n;
                     auto *a = rt.getArray(*c.cs, "noise");
-                    std::copy_n(noise[c.name].begin() + (size_t)i * n, n, a->getHostPointer<float>());
+                    storeScalars(a, 0, noise[c.name].data() + (size_t)i * n, n);
                     a->pushToDevice();
                 }
             }

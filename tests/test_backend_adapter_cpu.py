@@ -161,7 +161,7 @@ def _generate_with(case, *options):
     return net, tmp, os.path.join(work, net.name + "_CODE"), res
 
 
-@pytest.mark.parametrize("case, options", [("custom_update_small", ("--kernels=generated",)), ("post_events_small", ()), ("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("conv_small", ("--kernels=generated",)), ("procedural", ("--kernels=generated",)), ("dense_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
+@pytest.mark.parametrize("case, options", [("custom_update_small", ("--kernels=generated",)), ("va_double_small", ()), ("post_events_small", ()), ("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("conv_small", ("--kernels=generated",)), ("procedural", ("--kernels=generated",)), ("dense_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
                                            ("va_small", ("--dynamic=neuron:E.Ioffset",))])
 def test_generated_kernels_are_chosen_and_build(case, options):
     """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the runner then holds device
@@ -198,6 +198,10 @@ def test_generated_kernels_are_chosen_and_build(case, options):
             # the extra state variable and the weight-update variables are in the kernels under the reference's names
             assert "group->A[id]" in neuron and "sPreOutSynWUMPre" in neuron and "sPostInSynWUMPost" in neuron
             assert "group->wPost[idSyn] = group->sPost[idPost]" in synapse and "group->wPre[rowMajorIndex] = group->sPre[idPre]" in synapse
+        if case == "va_double_small":
+            # a double-precision model takes generated kernels by itself (the library's are fp32): state and accumulators are fp64
+            assert "double* __restrict__ V" in neuron.replace("double * ", "double* ") and "gennmi_kernel::addScalar(&group->outPost" in synapse
+            assert "double t" in neuron or "float t" in neuron
         if case == "post_events_small":
             # spike-like events of the postsynaptic population: queued by the neuron update like presynaptic ones, walked through
             # the column view before the true spikes
@@ -350,8 +354,9 @@ def test_custom_connectivity_updates_generate_and_build():
         shutil.rmtree(tmp, ignore_errors=True)
 
 
-def test_generated_kernels_say_what_they_do_not_cover():
-    """Asked to generate kernels for something they do not cover, the backend names it."""
+def test_library_kernels_say_what_they_do_not_cover():
+    """Asked for the device library's own kernels for something they do not cover (a double-precision model: they are fp32), the
+    backend says so."""
     net, snap = CASES["va_small"]()
     net.snap = snap
     tmp = tempfile.mkdtemp(prefix="adapter_genk_refuse_")
@@ -360,9 +365,9 @@ def test_generated_kernels_say_what_they_do_not_cover():
         for d in (work, out):
             os.makedirs(d)
         write_netspec(net, spec)
-        res = subprocess.run([DRIVER, spec, work, out, "--generate-only", "--kernels=generated", "--precision=double"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+        res = subprocess.run([DRIVER, spec, work, out, "--generate-only", "--kernels=library", "--precision=double"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
         assert res.returncode != 0
-        assert "generated kernels do not cover" in res.stdout and "double precision" in res.stdout, res.stdout[-2000:]
+        assert "single-precision" in res.stdout, res.stdout[-2000:]
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
 
