@@ -588,8 +588,8 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const bool bitmask = (matrix & SynapseMatrixConnectivity::BITMASK);
                     const bool procedural = (matrix & SynapseMatrixConnectivity::PROCEDURAL);
                     if(!sparse && !dense && !toeplitz && !bitmask && !procedural) { notGenerated("this matrix type (projection '" + arch.getName() + "')"); }
-                    if((matrix & SynapseMatrixWeight::PROCEDURAL) && !procedural) {
-                        notGenerated("weights regenerated from their initialisation snippet on stored connectivity (projection '" + arch.getName() + "')");
+                    if((matrix & SynapseMatrixWeight::PROCEDURAL) && !procedural && !dense) {
+                        notGenerated("weights regenerated from their initialisation snippet on connectivity other than DENSE and PROCEDURAL (projection '" + arch.getName() + "')");
                     }
                     if(!arch.isPreSpikeRequired() && !arch.isPreSpikeEventRequired()) { return; }
                     // PROCEDURAL: a row is the connectivity snippet's row build code, run by `threadsPerSpike` lanes that share the
@@ -775,6 +775,8 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                             codeEnv.add(indexType.addConst(), "id_syn", "idSyn",
                                         {codeEnv.addInitialiser("const " + indexTypeName + " idSyn = ((" + indexTypeName + ")idPre * " + (bitmask ? "rowSpan" : "$(num_post)") + ") + j;")});
                         }
+                        // (DENSE with weights regenerated from their initialisation snippet at every event: GeNN allows such snippets no
+                        // random numbers — synapseGroup.cc — so the snippet's code is evaluated as it stands, generateSpikeUpdate does it)
                         codeEnv.add(Type::getAddToPrePostDelay(s.getScalarType()), "addToPostDelay",
                                     "gennmi_kernel::addScalar(&$(_den_delay)[" + s.getPostDenDelayIndex(batchSize, "$(id_post)", "$(1)") + "], $(0))");
                         codeEnv.add(Type::getAddToPrePost(s.getScalarType()), "addToPost",

@@ -220,9 +220,10 @@ def write_netspec(net: Net, path: str):
             np.ascontiguousarray(s.gp, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.gp.u32"))
         else:
             head = f"syn {s.name} conv2d {s.src} {s.trg} " + " ".join(str(int(s.conv[k])) for k in CONV_PARAMS)
-        if s.wum != "static_const" and s.matrix not in ("procedural", "sparse_init"):
+        regenerated = (s.matrix == "dense" and s.wum == "static" and s.g_init is not None)     # DENSE with weights from a snippet, never stored
+        if s.wum != "static_const" and s.matrix not in ("procedural", "sparse_init") and not regenerated:
             np.ascontiguousarray(s.g, dtype=np.float32).tofile(os.path.join(path, f"{s.name}.g.f32"))
-        if s.matrix in ("procedural", "sparse_init") and s.wum == "static":
+        if (s.matrix in ("procedural", "sparse_init") or regenerated) and s.wum == "static":
             snippet, params = s.g_init
             order = {"Constant": ("constant",), "Uniform": ("min", "max"), "Normal": ("mean", "sd")}[snippet]
             w = f"static_init {snippet} " + " ".join(repr(float(params[k])) for k in order)

@@ -620,7 +620,8 @@ int main(int argc, char *argv[])
                 if(s.colStride) s.sg->setMaxSourceConnections(s.colStride);
             }
             else if(s.matrix == "dense") {
-                s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::DENSE, src, trg, wum, psm);
+                // (weights given by an initialisation snippet are regenerated at every event, never stored: DENSE_PROCEDURALG)
+                s.sg = model.addSynapsePopulation(s.name, (s.wum == "static_init") ? SynapseMatrixType::DENSE_PROCEDURALG : SynapseMatrixType::DENSE, src, trg, wum, psm);
             }
             else if(s.matrix == "bitmask") {
                 s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::BITMASK, src, trg, wum, psm);
@@ -775,7 +776,7 @@ int main(int argc, char *argv[])
             else if(s.matrix == "bitmask") {
                 load(rt.getArray(*s.sg, "gp"), s.name + ".gp.u32");
             }
-            else if(s.wum != "static_const" && s.matrix != "procedural" && s.matrix != "sparse_init") {
+            else if(s.wum != "static_const" && s.wum != "static_init" && s.matrix != "procedural" && s.matrix != "sparse_init") {
                 load(rt.getArray(*s.sg, "g"), s.name + ".g.f32");
             }
             if(s.wum == "stdp_trace") {

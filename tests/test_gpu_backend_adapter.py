@@ -559,6 +559,42 @@ def test_generated_kernels_on_procedural_matrices():
         assert abs(counts["generated"][p.name] - counts["library"][p.name]) <= 0.15 * counts["library"][p.name], (p.name, counts)
 
 
+def test_generated_kernels_regenerate_dense_weights():
+    """DENSE connectivity whose weights are never stored but regenerated from their initialisation snippet at every event
+    (DENSE_PROCEDURALG; GeNN allows such snippets no random numbers).  Eight sources fire together twice into 500 silent LIF
+    neurons through Constant(0.375) weights and a DeltaCurr input: potentials identical, step by step, to the same network with
+    StaticPulseConstantWeight."""
+    from genn_amd.netspec import Net, Pop, Syn
+    n_src, n_trg = 8, 500
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=1e9, Ioffset=0.0, TauRefrac=2.0)
+
+    def potentials(name, **syn):
+        net = Net(name=name, dt=1.0, steps=14, seed=777)
+        net.pops.append(Pop("S", "ssa", n_src, {}, {"startSpike": (2 * np.arange(n_src)).astype(np.uint32), "endSpike": (2 * np.arange(n_src) + 2).astype(np.uint32)},
+                            spike_times=np.tile(np.array([1.0, 11.0], np.float32), n_src)))
+        net.pops.append(Pop("T", "lif", n_trg, lif, {"V": np.full(n_trg, -60.0, np.float32), "RefracTime": np.zeros(n_trg, np.float32)}))
+        net.syns.append(Syn("ST", "S", "T", matrix="dense", psm="deltacurr", **syn))
+        net.snap = 1
+        tmp = tempfile.mkdtemp(prefix="adapter_dense_regenerated_")
+        try:
+            spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+            for d in (work, out):
+                os.makedirs(d)
+            write_netspec(net, spec)
+            print(f"adapter regenerated dense weights ({net.name}): running {DRIVER}", flush=True)
+            res = subprocess.run([DRIVER, spec, work, out, "--kernels=generated"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+            assert res.returncode == 0, res.stdout[-3000:]
+            return np.fromfile(os.path.join(out, "T.V.f32"), np.float32).reshape(net.steps, n_trg)
+        finally:
+            shutil.rmtree(tmp, ignore_errors=True)
+
+    constant = potentials("dense_constant", wum="static", g_init=("Constant", {"constant": 0.375}))
+    twin = potentials("dense_twin", wum="static_const", wum_params={"g": 0.375})
+    assert np.array_equal(constant, twin)
+    moved = [k for k in range(len(constant)) if np.any(constant[k] != np.float32(-60.0))]
+    assert moved and np.allclose(constant[moved[0]], -60.0 + (1.0 - np.exp(-1.0 / 20.0)) * 20.0 * n_src * 0.375, rtol=1e-6)
+
+
 def test_generated_kernels_with_simulation_random_numbers():
     """Random numbers in simulation code (the built-in Poisson neuron, neuronModels.h:307-325: `gennrand_exponential()` refills a
     countdown): the generated kernels draw them from a counter-based generator keyed by the model's seed.  Every backend of
