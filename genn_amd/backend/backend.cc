@@ -1567,11 +1567,17 @@ void Backend::genLazyVariableDynamicAllocation(CodeStream &os, const Type::Resol
     const auto &valueType = type.isPointer() ? *type.getPointer().valueType : type;
     os << (type.isPointer() ? "*" : "") << "$(_" << name << ") = new " << valueType.getValue().name << "[" << countVarName << "];" << std::endl;
 }
-void Backend::genLazyVariableDynamicPush(CodeStream&, const Type::ResolvedType&, const std::string&, VarLocation, const std::string&) const
+// (pointer-typed: an extra global parameter of host initialisation code, a plain host array — nothing to copy.  Otherwise: an
+// array of a custom connectivity update's host update code, whose host buffer has a device buffer registered behind it)
+void Backend::genLazyVariableDynamicPush(CodeStream &os, const Type::ResolvedType &type, const std::string &name, VarLocation, const std::string &countVarName) const
 {
+    if(type.isPointer()) { return; }
+    os << "GENNMI_CHECK(gennmi_memcpy_to_device(gennmiDev($(_" << name << ")), $(_" << name << "), (size_t)(" << countVarName << ") * sizeof(" << type.getName() << ")));" << std::endl;
 }
-void Backend::genLazyVariableDynamicPull(CodeStream&, const Type::ResolvedType&, const std::string&, VarLocation, const std::string&) const
+void Backend::genLazyVariableDynamicPull(CodeStream &os, const Type::ResolvedType &type, const std::string &name, VarLocation, const std::string &countVarName) const
 {
+    if(type.isPointer()) { return; }
+    os << "GENNMI_CHECK(gennmi_memcpy_from_device($(_" << name << "), gennmiDev($(_" << name << ")), (size_t)(" << countVarName << ") * sizeof(" << type.getName() << ")));" << std::endl;
 }
 void Backend::genMergedDynamicVariablePush(CodeStream &os, const std::string &suffix, size_t mergedGroupIdx,
                                            const std::string &groupIdx, const std::string &fieldName,
@@ -1673,7 +1679,10 @@ bool Backend::isGlobalHostRNGRequired(const ModelSpecInternal &model) const
         || std::any_of(sgs.cbegin(), sgs.cend(), [](const auto &s){ return s.second.isWUInitRNGRequired() || s.second.getSparseConnectivityInitialiser().isRNGRequired()
                                                                           || s.second.getSparseConnectivityInitialiser().isHostRNGRequired(); })
         || std::any_of(model.getCustomUpdates().cbegin(), model.getCustomUpdates().cend(), [](const auto &c){ return c.second.isInitRNGRequired(); })
-        || std::any_of(model.getCustomWUUpdates().cbegin(), model.getCustomWUUpdates().cend(), [](const auto &c){ return c.second.isInitRNGRequired(); });
+        || std::any_of(model.getCustomWUUpdates().cbegin(), model.getCustomWUUpdates().cend(), [](const auto &c){ return c.second.isInitRNGRequired(); })
+        || std::any_of(model.getCustomConnectivityUpdates().cbegin(), model.getCustomConnectivityUpdates().cend(),
+                       [](const auto &c){ return Utils::isRNGRequired(c.second.getVarInitialisers()) || Utils::isRNGRequired(c.second.getPreVarInitialisers())
+                                                 || Utils::isRNGRequired(c.second.getPostVarInitialisers()) || Utils::isRNGRequired(c.second.getHostUpdateCodeTokens()); });
 }
 size_t Backend::getDeviceMemoryBytes() const
 {

@@ -991,7 +991,6 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     for(const auto &c : model.getCustomUpdates()) { groupNames.insert(c.second.getUpdateGroupName()); }
     for(const auto &c : model.getCustomWUUpdates()) { groupNames.insert(c.second.getUpdateGroupName()); }
     for(const auto &c : model.getCustomConnectivityUpdates()) { groupNames.insert(c.second.getUpdateGroupName()); }
-    if(!modelMerged.getMergedCustomConnectivityHostUpdateGroups().empty()) { notGenerated("host update code of custom connectivity updates"); }
     auto refuseRNG = [](const auto &arch)
     {
         if(Utils::isRNGRequired(arch.getUpdateCodeTokens())) { notGenerated("random numbers in custom update code (custom update '" + arch.getName() + "')"); }
@@ -1365,6 +1364,19 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                 });
         }
 
+        // ---- host update code of custom connectivity updates: plain host code over the arrays' host buffers, run before the
+        // group's kernels; its pushXToDevice / pullXFromDevice are copies between a host buffer and the device buffer behind it
+        std::ostringstream ccHost;
+        {
+            CodeStream hostCode(ccHost);
+            EnvironmentLibrary lib(hostCode, StandardLibrary::getMathsFunctions());
+            EnvironmentExternal funcEnv(lib);
+            funcEnv.add(model.getTimePrecision().addConst(), "t", "t");
+            funcEnv.add(Type::Uint32.addConst(), "batch", "0");
+            funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
+            modelMerged.genMergedCustomConnectivityHostUpdateGroups(*this, memorySpaces, name, [&](auto &c) { c.generateUpdate(*this, funcEnv); });
+        }
+
         // ---- kernels and the host function of this update group
         const std::string signature = "(" + timeType + " t";
         if(neuronTable.numBlocks > 0) {
@@ -1403,6 +1415,7 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             const std::string grid = ", " + std::to_string(batchSize) + "), dim3(256), 0, 0>>>(t";
             const bool timing = model.isTimingEnabled();
             if(timing) { host << "hipEventRecord(customUpdate" << name << "Start, 0);" << std::endl; }
+            host << ccHost.str();
             if(ccTable.numBlocks > 0) {
                 // (connectivity first, like the reference: single_threaded_cpu/backend.cc:824-860; the generator's step counts this group's calls)
                 host << "static unsigned long long gennmiCalls = 0;" << std::endl;
@@ -1434,6 +1447,8 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     modelMerged.genMergedCustomUpdateTransposeWUStructs(os, *this);
     modelMerged.genMergedCustomConnectivityUpdateStructs(os, *this);
     modelMerged.genMergedCustomConnectivityRemapUpdateStructs(os, *this);
+    modelMerged.genMergedCustomConnectivityHostUpdateStructs(os, *this);
+    modelMerged.genMergedCustomConnectivityHostUpdateStructArrayPush(os, *this);
     modelMerged.genMergedCustomConnectivityUpdateHostStructArrayPush(os, *this);
     modelMerged.genMergedCustomConnectivityRemapUpdateHostStructArrayPush(os, *this);
     modelMerged.genMergedCustomUpdateHostStructArrayPush(os, *this);

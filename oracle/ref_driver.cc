@@ -292,17 +292,23 @@ IMPLEMENT_SNIPPET(BatchSumMax);
 
 // Custom connectivity updates (structural plasticity: a function of the model that rewires a SPARSE projection between steps),
 // after tests/features/test_custom_connectivity_update.py: one that removes every synapse whose weight has fallen below a
-// threshold and counts the removals of its row in a presynaptic variable of its own;
+// threshold (set per row by host update code) and counts the removals of its row in a presynaptic variable of its own;
 class PruneWeak : public CustomConnectivityUpdateModels::Base
 {
 public:
     DECLARE_SNIPPET(PruneWeak);
     SET_PARAMS({"threshold"});
-    SET_PRE_VARS({{"removed", "scalar"}});
+    SET_PRE_VARS({{"removed", "scalar"}, {"limit", "scalar"}});
     SET_VAR_REFS({{"w", "scalar", VarAccessMode::READ_ONLY}});
+    // (the threshold of a row is set by host code that runs before the rows are walked, and rises with the row and the time)
+    SET_HOST_UPDATE_CODE(
+        "for(unsigned int i = 0; i < num_pre; i++) {\n"
+        "    limit[i] = threshold + (0.0001 * i) + (0.00005 * t);\n"
+        "}\n"
+        "pushlimitToDevice();\n");
     SET_ROW_UPDATE_CODE(
         "for_each_synapse {\n"
-        "    if(w < threshold) {\n"
+        "    if(w < limit) {\n"
         "        remove_synapse();\n"
         "        removed += 1.0;\n"
         "    }\n"
@@ -672,7 +678,7 @@ int main(int argc, char *argv[])
                     WUVarReferences{{"variable", createWUVarRef(synByName.at(c.target)->sg, "g", synByName.at(c.target2)->sg, "g")}});
             }
             else if(c.kind == "prune") {
-                c.ccu = model.addCustomConnectivityUpdate<PruneWeak>(c.name, c.group, synByName.at(c.target)->sg, {{"threshold", c.p.at(0)}}, {}, {{"removed", 0.0}}, {},
+                c.ccu = model.addCustomConnectivityUpdate<PruneWeak>(c.name, c.group, synByName.at(c.target)->sg, {{"threshold", c.p.at(0)}}, {}, {{"removed", 0.0}, {"limit", 0.0}}, {},
                                                                     WUVarReferences{{"w", createWUVarRef(synByName.at(c.target)->sg, "g")}}, {}, {});
             }
             else if(c.kind == "sprout") {

@@ -340,6 +340,8 @@ def test_custom_connectivity_updates_generate_and_build():
         assert "gennmiCustomConnectivityUpdatePruneKernel<<<" in custom and "gennmiCustomConnectivityUpdateSproutKernel<<<" in custom
         prune = custom[custom.index("void updatePrune("):]
         assert prune.index("gennmiCustomConnectivityUpdatePruneKernel<<<") < prune.index("gennmi_build_remap(")
+        # host update code first: plain host code over the host buffers, pushed to the device buffers behind them
+        assert "group->limit[_i] = " in prune and prune.index("gennmi_memcpy_to_device(gennmiDev(group->limit), group->limit") < prune.index("Kernel<<<")
         # the removed synapse's slot takes the row's last one, with the weight and the other custom updates' variables
         assert "group->ind[idx] = group->ind[lastIdx];" in custom and "group->dependentVar0[idx] = group->dependentVar0[lastIdx];" in custom
         assert "group->rowLength[id]--;" in custom and "group->rowLength[id]++;" in custom
