@@ -79,7 +79,8 @@ struct gennmi_runner
     std::vector<u32x2*> resPacked;      // its synapses as the resident kernel reads them
     uint32_t neuronsPerLane = 1;        // 2, 4 or 8: neuronBulkKernel instead of neuronUpdateKernel
     bool sourcesStale = false;          // startSpike / endSpike / spikeTimes of a spike source were written since nextSpikeTime was built
-    bool resStale = false;              // connectivity or weights were written since the tables were built
+    bool resStale = false;              // connectivity or weights were written since the tables were built ...
+    std::vector<uint8_t> resStaleProj;  // ... of these projections (index into pre)
     bool tablesStale = false;           // rowLength / ind / d of a projection were written since the connectivity-derived tables were built
     // connectivity-derived tables that are rebuilt when tablesStale: segment boundaries of the tile path ...
     struct TileTable { size_t pre; uint16_t *off; uint32_t tileSize, numTiles; };
@@ -135,7 +136,8 @@ static void noteDeviceWrite(const void *dev, size_t bytes)
             if((a < st + perNeuron && st < b) || (a < en + perNeuron && en < b) || (a < reinterpret_cast<uintptr_t>(n.g.spikeTimes) + n.spikeTimesBytes && reinterpret_cast<uintptr_t>(n.g.spikeTimes) < b)) { r->sourcesStale = true; }
         }
         if(!r->finalised) { continue; }
-        for(const auto &p : r->pre) {
+        for(size_t k = 0; k < r->pre.size(); k++) {
+            const auto &p = r->pre[k];
             if(p.g.matrix != GENNMI_MATRIX_SPARSE) { continue; }
             const size_t entries = (size_t)p.g.numSrcNeurons * p.g.rowStride;
             // connectivity (rowLength, ind, d) feeds the segment boundaries of the tile path, the zero-delay lists of the
@@ -147,7 +149,7 @@ static void noteDeviceWrite(const void *dev, size_t bytes)
             for(const auto &arr : arrays) {
                 const uintptr_t lo = reinterpret_cast<uintptr_t>(arr.ptr);
                 if(arr.ptr && arr.size && a < lo + arr.size && lo < b) {
-                    if(r->resident) { r->resStale = true; }
+                    if(r->resident) { r->resStale = true; r->resStaleProj.resize(r->pre.size(), 0); r->resStaleProj[k] = 1; }
                     if(arr.connectivity) { r->tablesStale = true; }
                     if(!r->recordTables.empty()) { r->recordsStale = true; }
                 }
@@ -723,14 +725,17 @@ static int launchResident(gennmi_runner *r, unsigned long long timestep, unsigne
 {
     constexpr unsigned long long MAX_STEPS = 1ull << 20;
     bool stale;
+    std::vector<uint8_t> staleProj;
     {
         std::lock_guard<std::mutex> lock(g_runnersMutex);
         stale = r->resStale;
         r->resStale = false;
+        staleProj.swap(r->resStaleProj);
     }
     if(stale) {
-        // weights or connectivity were written since the segment tables were built: the inline synapses may be out of date
+        // weights or connectivity of these projections were written since their segment tables and packed records were built
         for(size_t k = 0; k < r->pre.size(); k++) {
+            if(k >= staleProj.size() || !staleProj[k]) { continue; }
             const auto &q = r->pre[k].g;
             const size_t entries = (size_t)q.numSrcNeurons * r->resSegTiles[k];
             const uint32_t depth = (q.wum == GENNMI_WUM_STATIC_PULSE_DENDRITIC_DELAY) ? q.maxDenDelay : 0u;
