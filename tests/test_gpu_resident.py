@@ -194,6 +194,50 @@ def test_weights_written_behind_the_library_are_reported(monkeypatch):
     model.unload()
 
 
+def test_writes_named_through_a_registered_host_buffer(monkeypatch):
+    """The same for callers that only know host pointers (generated custom update code beside the library's kernels): the
+    device buffer is registered behind a host buffer, gennmi_flush runs queued steps before the caller's own device work, and
+    gennmi_note_mirror_write names the whole device buffer through any pointer into the host one.  One of two projections is
+    rewritten: only its copies are rebuilt, and the other one's stay valid."""
+    import ctypes as C
+    from genn_amd import _abi
+    monkeypatch.setenv("GENNMI_FUSED_STEP", "0")
+    n, depth = 600, 4
+    net = Net(name="resident_mirror", dt=1.0, steps=0)
+    net.pops.append(_pop("A", n, 0.6, -60.0 + 9.5 * rng.uniform(17, 1, 0, n)))
+    net.syns.append(_projection("AA", "A", "A", n, n, 48, 0.04, 31, depth, 0.4))
+    net.syns.append(_projection("AA2", "A", "A", n, n, 24, -0.02, 41, depth, 0.3))
+    net.steps = 120
+    state = {"written": False, "host": None}
+
+    def check(model, oracle):
+        compare_state(net, model, oracle, f"after {model.timestep} steps", exact=True)
+        if not state["written"]:
+            g = model.synapse_populations["AA"].vars["g"]
+            lib = _abi.load()
+            host = np.zeros(g.count, np.float32)                       # the caller's host buffer (never copied from here)
+            state["host"] = host
+            _abi.check(lib.gennmi_register_mirror(host.ctypes.data_as(C.c_void_p), C.c_void_p(g.ptr), host.nbytes))
+            _abi.check(lib.gennmi_flush())
+            staging = C.c_void_p()
+            _abi.check(lib.gennmi_malloc(C.byref(staging), host.nbytes))
+            new = np.full(g.count, -0.03, np.float32)
+            _abi.check(lib.gennmi_memcpy_to_device(staging, new.ctypes.data_as(C.c_void_p), new.nbytes))
+            hip = C.CDLL("libamdhip64.so")
+            assert hip.hipMemcpy(C.c_void_p(g.ptr), staging, C.c_size_t(new.nbytes), C.c_int(3)) == 0      # hipMemcpyDeviceToDevice
+            _abi.check(lib.gennmi_note_mirror_write(C.c_void_p(host.ctypes.data + 4 * 100)))               # a pointer INTO the host buffer
+            lib.gennmi_free(staging)
+            assert lib.gennmi_note_mirror_write(C.c_void_p(new.ctypes.data)) != 0                           # not a registered buffer
+            _abi.check(lib.gennmi_unregister_mirror(host.ctypes.data_as(C.c_void_p)))
+            oracle.syn_g("AA")[:] = np.float32(-0.03)
+            state["written"] = True
+
+    model, oracle, spikes = _run_chunks(net, (60, 60), check)
+    assert model.runner_info()["resident_plan"]
+    assert spikes > 500
+    model.unload()
+
+
 @pytest.mark.parametrize("limit, rows", [(64, 230), (1000, 230), (7, 230), (64, 50), (64, 0)])
 def test_queued_single_steps_take_the_resident_launch(limit, rows):
     """step_time() one call at a time with the step queue on (what the reference's Runtime::stepTime amounts to): the steps
