@@ -1236,6 +1236,9 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                         env.add(Type::Uint32.addConst(), "row_len", "$(_row_length)[i]");
                         s.generateInit(*this, env, batchSize);
                     }
+                    if(learnPost && s.getArchetype().getSparseIndType() != Type::Uint32) {
+                        unsupported("the column view of projection '" + s.getArchetype().getName() + "' over a narrow sparse index type");
+                    }
                     if(learnPost) {
                         // evaluated here so the fields exist; executed after the upload below
                         remap << "for(unsigned int g = 0; g < " << s.getGroups().size() << "; g++)";
@@ -1750,6 +1753,11 @@ Backend createBackend(const ModelSpecInternal &model, const filesystem::path&, p
         for(const auto &s : model.getSynapseGroups()) {
             generated = generated || anyDynamic(s.second.getPSInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isPSParamDynamic(p); });
             generated = generated || anyDynamic(s.second.getWUInitialiser().getSnippet()->getParams(), [&](const std::string &p) { return s.second.isWUParamDynamic(p); });
+        }
+        // ... or when a SPARSE projection stores its targets in a narrow type (ModelSpec::setDefaultNarrowSparseIndEnabled): the library
+        // reads 32-bit ones, generated code takes the type from the merged struct
+        for(const auto &s : model.getSynapseGroups()) {
+            generated = generated || ((s.second.getMatrixType() & SynapseMatrixConnectivity::SPARSE) && s.second.getSparseIndType() != Type::Uint32);
         }
         // ... or when the model is not single precision: the library's kernels are fp32
         generated = generated || model.getPrecision() != Type::Float || model.getTimePrecision() != Type::Float;

@@ -416,7 +416,7 @@ int main(int argc, char *argv[])
         bool generateOnly = false;
         std::string userCxxFlags;
         std::vector<std::string> dynamicParams;
-        bool timing = false, ordered = false, deviceInit = false, doublePrecision = false;
+        bool timing = false, ordered = false, deviceInit = false, doublePrecision = false, narrowInd = false;
         int stepQueue = -1;
         std::string kernels = "auto";
         for(int a = 4; a < argc; a++) {
@@ -430,6 +430,7 @@ int main(int argc, char *argv[])
             else if(opt.rfind("--step-queue=", 0) == 0) { stepQueue = std::stoi(opt.substr(13)); }      // MI355X backend: Preferences::stepQueueLength
             else if(opt == "--device-init") { deviceInit = true; }                  // MI355X backend: Preferences::deviceInitialisation
             else if(opt == "--ordered") { ordered = true; }                          // MI355X backend: Preferences::orderedAccumulation
+            else if(opt == "--narrow-ind") { narrowInd = true; }     // ModelSpec::setDefaultNarrowSparseIndEnabled; for --generate-only runs (the netspec's targets are 32-bit)
             else if(opt == "--precision=double") { doublePrecision = true; }        // ModelSpec::setPrecision(Type::Double); for --generate-only runs (the netspec's arrays are fp32)
             else if(opt == "--timing") { timing = true; }       // ModelSpec::setTimingEnabled; the Runtime's counters are printed after the run
             else { std::cerr << "unknown option " << opt << std::endl; return 1; }
@@ -512,6 +513,7 @@ int main(int argc, char *argv[])
         if(seed) { model.setSeed(seed); }
         model.setPrecision(doublePrecision ? Type::Double : Type::Float);
         model.setFusePostsynapticModels(fuse != 0);
+        model.setDefaultNarrowSparseIndEnabled(narrowInd);
         model.setTimingEnabled(timing);
         std::map<std::string, PopSpec*> popByName;
         for(auto &p : pops) {

@@ -356,6 +356,18 @@ def test_custom_connectivity_updates_generate_and_build():
         shutil.rmtree(tmp, ignore_errors=True)
 
 
+def test_narrow_sparse_indices_take_generated_kernels():
+    """ModelSpec::setDefaultNarrowSparseIndEnabled stores the targets of SPARSE rows in the narrowest type that holds them; the device
+    library reads 32-bit targets, so such a model takes generated kernels, whose code takes the type from the merged struct."""
+    net, tmp, code, res = _generate_with("va_small", "--narrow-ind")
+    try:
+        assert res.returncode == 0, res.stdout[-3000:]
+        synapse = open(os.path.join(code, "synapseUpdate.cc")).read()
+        assert "__global__" in synapse and "uint16_t* __restrict__ ind" in synapse.replace("uint16_t * ", "uint16_t* ")
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
 def test_library_kernels_say_what_they_do_not_cover():
     """Asked for the device library's own kernels for something they do not cover (a double-precision model: they are fp32), the
     backend says so."""
