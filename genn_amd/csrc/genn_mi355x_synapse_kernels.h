@@ -1013,20 +1013,41 @@ __device__ __forceinline__ void postsynapticBody(const PostGroupDev &G, uint32_t
         }
         return;
     }
+    // A column entry is a chain of dependent memory round trips (remap -> spike time, trace and weight of that synapse ->
+    // store), and a sub-group walks its column alone: four entries per lane are in flight at a time.  Every synapse is still
+    // visited once, with the same arithmetic.
+    constexpr int INFLIGHT = 4;
+    GLOBAL_AS const uint32_t *remap = asGlobal(g.remap);
     for(uint32_t s = subGroup; s < numSpikes; s += numSubGroups) {
         const uint32_t spike = trgSpk[s];
-        const uint32_t npre = g.colLength[spike];
+        const uint32_t npre = asGlobal(g.colLength)[spike];
         const size_t colBase = (size_t)spike * g.colStride;
-        for(uint32_t i = lis; i < npre; i += W) {
-            const uint32_t rowMajorIndex = g.remap[colBase + i];
-            const uint32_t idPre = rowMajorIndex / g.rowStride;
-            if(paired && bitmapTest(srcBitmap, idPre)) { continue; }
-            const float stPre = dt + srcST[idPre];
-            const float dtSpike = st.t - stPre;
-            if(dtSpike > 0) {
-                const float factor = additive ? (float)exp((double)(-dtSpike / g.tauPlus)) : preTrace[idPre];
-                const float newWeight = weight[rowMajorIndex] + (g.aPlus * factor);
-                weight[rowMajorIndex] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
+        for(uint32_t i0 = lis; i0 < npre; i0 += INFLIGHT * W) {
+            uint32_t rowMajorIndex[INFLIGHT];
+            bool live[INFLIGHT];
+            #pragma unroll
+            for(int u = 0; u < INFLIGHT; u++) {
+                const uint32_t i = i0 + u * W;
+                live[u] = (i < npre);
+                rowMajorIndex[u] = live[u] ? remap[colBase + i] : 0u;
+            }
+            float stPre[INFLIGHT], trace[INFLIGHT], w[INFLIGHT];
+            #pragma unroll
+            for(int u = 0; u < INFLIGHT; u++) {
+                const uint32_t idPre = rowMajorIndex[u] / g.rowStride;
+                live[u] = live[u] && !(paired && bitmapTest(srcBitmap, idPre));
+                stPre[u] = live[u] ? srcST[idPre] : 0.0f;
+                trace[u] = (live[u] && !additive) ? preTrace[idPre] : 0.0f;
+                w[u] = live[u] ? weight[rowMajorIndex[u]] : 0.0f;
+            }
+            #pragma unroll
+            for(int u = 0; u < INFLIGHT; u++) {
+                const float dtSpike = st.t - (dt + stPre[u]);
+                if(live[u] && dtSpike > 0) {
+                    const float factor = additive ? (float)exp((double)(-dtSpike / g.tauPlus)) : trace[u];
+                    const float newWeight = w[u] + (g.aPlus * factor);
+                    weight[rowMajorIndex[u]] = fminf(g.wMax, fmaxf(g.wMin, newWeight));
+                }
             }
         }
     }
