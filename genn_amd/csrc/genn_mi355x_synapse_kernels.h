@@ -956,7 +956,10 @@ __device__ __forceinline__ void postsynapticBody(const PostGroupDev &G, uint32_t
     const uint32_t W = G.lanesPerSpike;
     const uint32_t localBlock = blockInKernel - G.startBlock;
     const uint32_t lis = threadIdx.x & (W - 1);
-    const uint32_t subGroup = (localBlock * BS + threadIdx.x) / W;
+    // Sub-groups are numbered across the blocks first (sub-group k of block b is number k * numBlocks + b): a column walk is
+    // a stream of scattered accesses, which a compute unit issues at one lane per clock, so the first spikes of the queue
+    // should each find a compute unit of their own rather than share the first block's.
+    const uint32_t subGroup = (threadIdx.x / W) * G.numBlocks + localBlock;
     const uint32_t numSubGroups = (G.numBlocks * BS) / W;
     // plastic weights, spike times and traces are per batch (VarAccess::READ_WRITE variables are duplicated); connectivity is shared
     const uint32_t numSpikes = g.trgSpkCnt[batch];
