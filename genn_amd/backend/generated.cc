@@ -847,7 +847,9 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     CodeStream::Scope b1(groupEnv.getStream());
                     groupEnv.printLine("const unsigned int numSpikes = $(_trg_spk_cnt" + suffix + ")[" + s.getPostSlot(postDelay, batchSize) + "];");
                     groupEnv.getStream() << "const unsigned long long numItems = (unsigned long long)numSpikes * chunksPerCol;" << std::endl;
-                    groupEnv.getStream() << "for(unsigned long long item = entry.blockInGroup * 4u + (threadIdx.x / 64u); item < numItems; item += numWaves)";
+                    // (items are dealt to the work-groups first, then to their wavefronts: a column walk is a stream of scattered accesses,
+                    // which a compute unit issues at about one lane per clock, so the first items should each find a compute unit of their own)
+                    groupEnv.getStream() << "for(unsigned long long item = (threadIdx.x / 64u) * entry.blocksInGroup + entry.blockInGroup; item < numItems; item += numWaves)";
                     {
                         CodeStream::Scope b2(groupEnv.getStream());
                         EnvironmentGroupMergedField<PostsynapticUpdateGroupMerged> synEnv(groupEnv, s);
