@@ -57,6 +57,7 @@ struct gennmi_runner
     NeuronGroupDev *dNeuron = nullptr; PreGroupDev *dPre = nullptr; PostGroupDev *dPost = nullptr;
     uint32_t neuronBlocks = 0, preBlocks = 0, postBlocks = 0;
     unsigned long long *dAgg = nullptr; uint32_t *dError = nullptr; unsigned long long *dEvents = nullptr;
+    uint32_t *hError = nullptr;     // pinned host word that the error flag is copied into on the runner's stream, ahead of a wait
     StepState *dState = nullptr;
     unsigned long long epoch = 0;       // completed steps (host mirror)
     bool synapsesDone = false;          // updateSynapses ran for the current step
@@ -355,6 +356,8 @@ int gennmi_runner_create(gennmi_runner **runner, float dt, uint32_t batchSize)
     HIP_TRY(hipStreamCreate(&r->stream));       // blocking stream: ordered against null-stream copies
     HIP_TRY(hipMalloc(&r->dError, sizeof(uint32_t)));
     HIP_TRY(hipMemset(r->dError, 0, sizeof(uint32_t)));
+    HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&r->hError), sizeof(uint32_t), hipHostMallocDefault));
+    *r->hError = 0;
     HIP_TRY(hipMalloc(&r->dEvents, sizeof(unsigned long long)));
     HIP_TRY(hipMemset(r->dEvents, 0, sizeof(unsigned long long)));
     HIP_TRY(hipMalloc(&r->dState, sizeof(StepState)));
@@ -384,7 +387,7 @@ int gennmi_runner_destroy(gennmi_runner *r)
     for(void *q : r->orderedOwned) { hipFree(q); }
     hipFree(r->dOrderedSources); hipFree(r->dOrderedBitmaps);
     hipFree(r->dTile); hipFree(r->dConvTile);
-    hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dDense); hipFree(r->dProc); hipFree(r->dAgg); hipFree(r->dError); hipFree(r->dEvents); hipFree(r->dState);
+    hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dDense); hipFree(r->dProc); hipFree(r->dAgg); hipFree(r->dError); if(r->hError) { hipHostFree(r->hError); } hipFree(r->dEvents); hipFree(r->dState);
     hipStreamDestroy(r->stream);
     delete r;
     return GENNMI_OK;
@@ -1810,9 +1813,11 @@ int gennmi_runner_synchronize(gennmi_runner *r)
 {
     if(!r) { return fail(GENNMI_EINVAL, "runner_synchronize: null runner"); }
     FLUSH_QUEUED();
+    // (the flag travels on the stream behind the queued work, so that one wait covers both: a blocking copy after the wait
+    // would cost a second round trip, as long as several steps of a small model)
+    HIP_TRY(hipMemcpyAsync(r->hError, r->dError, sizeof(uint32_t), hipMemcpyDeviceToHost, r->stream));
     HIP_TRY(hipStreamSynchronize(r->stream));
-    uint32_t err = 0;
-    HIP_TRY(hipMemcpy(&err, r->dError, sizeof(err), hipMemcpyDeviceToHost));
+    const uint32_t err = *r->hError;
     if(err) { return fail(GENNMI_EDEVICE, "a kernel's bounded wait for other work-groups expired (spike offsets or spike exchange); state is undefined"); }
     return GENNMI_OK;
 }
