@@ -33,6 +33,7 @@
 #include <type_traits>
 #include <map>
 #include <mutex>
+#include <chrono>
 #include <vector>
 
 #include "genn_mi355x.h"
@@ -1816,6 +1817,15 @@ int gennmi_runner_synchronize(gennmi_runner *r)
     // (the flag travels on the stream behind the queued work, so that one wait covers both: a blocking copy after the wait
     // would cost a second round trip, as long as several steps of a small model)
     HIP_TRY(hipMemcpyAsync(r->hError, r->dError, sizeof(uint32_t), hipMemcpyDeviceToHost, r->stream));
+    // (short waits are polled: a blocking wait wakes up some tens of microseconds after the work has ended; GENNMI_POLL_US=0 blocks at once)
+    static const long pollMicroseconds = [] { const char *e = getenv("GENNMI_POLL_US"); return e ? atol(e) : 500l; }();
+    if(pollMicroseconds > 0) {
+        const auto begin = std::chrono::steady_clock::now();
+        hipError_t state = hipStreamQuery(r->stream);
+        while(state == hipErrorNotReady && std::chrono::steady_clock::now() - begin < std::chrono::microseconds(pollMicroseconds)) { state = hipStreamQuery(r->stream); }
+        (void)hipGetLastError();    // "not ready" is an answer, not a failure to keep
+        if(state != hipSuccess && state != hipErrorNotReady) { HIP_TRY(state); }
+    }
     HIP_TRY(hipStreamSynchronize(r->stream));
     const uint32_t err = *r->hError;
     if(err) { return fail(GENNMI_EDEVICE, "a kernel's bounded wait for other work-groups expired (spike offsets or spike exchange); state is undefined"); }
