@@ -1420,15 +1420,22 @@ void Backend::genDefinitionsPreamble(CodeStream &os, const ModelSpecMerged&) con
     os << "// MI355X device library" << std::endl;
     os << "#include \"genn_mi355x.h\"" << std::endl;
     if(hasDeviceModules()) {
-        os << "// building blocks of the generated kernels (every module is compiled with hipcc)" << std::endl;
+        os << "// building blocks of the generated kernels: seen by the device pass of a module only (hipcc --genco); the host" << std::endl;
+        os << "// pass (the host compiler) sees structs and host functions, which reach the device through the C ABI above" << std::endl;
+        os << "#ifdef __HIPCC__" << std::endl;
         os << "#include \"genn_mi355x_kernel_support.h\"" << std::endl;
+        os << "#endif" << std::endl;
         os << "extern bool gennmiStructsDirty;" << std::endl;
+        os << "extern gennmi_program *gennmiProgram;" << std::endl;
+        os << "extern uint32_t *gennmiProgramError;" << std::endl;
         os << "void gennmiUploadCustomUpdateGroups();" << std::endl;
+        os << "void gennmiFreeCustomUpdateGroups();" << std::endl;
     }
     if(m_GeneratedKernels) {
         os << "void gennmiUploadNeuronGroups();" << std::endl;
         os << "void gennmiUploadSynapseGroups();" << std::endl;
-        os << "void gennmiCheckNeuronKernels();" << std::endl;
+        os << "void gennmiFreeNeuronGroups();" << std::endl;
+        os << "void gennmiFreeSynapseGroups();" << std::endl;
     }
     os << "#define GENNMI_CHECK(call) do { if((call) != GENNMI_OK) { throw std::runtime_error(std::string(__FILE__) + \": \" + std::to_string(__LINE__) + \": \" + gennmi_last_error()); } } while(0)" << std::endl;
     os << std::endl;
@@ -1455,6 +1462,11 @@ void Backend::genDefinitionsPreamble(CodeStream &os, const ModelSpecMerged&) con
 void Backend::genRunnerPreamble(CodeStream &os, const ModelSpecMerged&) const
 {
     os << "gennmi_runner *gennmiRunner = nullptr;" << std::endl;
+    if(hasDeviceModules()) {
+        os << "// the model's generated device code: code objects, launch sequences, stream, timers and error flag live in the device library" << std::endl;
+        os << "gennmi_program *gennmiProgram = nullptr;" << std::endl;
+        os << "uint32_t *gennmiProgramError = nullptr;" << std::endl;
+    }
     os << "static bool gennmiFinalised = false;" << std::endl;
     os << "static std::vector<void*> gennmiScratchBuffers;" << std::endl;
     os << "uint32_t *gennmiScratch(size_t count)";
@@ -1516,15 +1528,30 @@ void Backend::genAllocateMemPreamble(CodeStream &os, const ModelSpecMerged &mode
     const ModelSpecInternal &model = modelMerged.getModel();
     os << "GENNMI_CHECK(gennmi_init(" << getPreferences<Preferences>().deviceID << "));" << std::endl;
     if(hasDeviceModules()) { os << "gennmiStructsDirty = true;" << std::endl; }
-    if(m_GeneratedKernels) { return; }
-    os << "GENNMI_CHECK(gennmi_runner_create(&gennmiRunner, " << Type::writeNumeric(model.getDT(), model.getTimePrecision()) << ", " << model.getBatchSize() << "u));" << std::endl;
-    if(model.isTimingEnabled()) {
-        os << "GENNMI_CHECK(gennmi_runner_set_timing(gennmiRunner, 1));" << std::endl;
+    if(!m_GeneratedKernels) {
+        os << "GENNMI_CHECK(gennmi_runner_create(&gennmiRunner, " << Type::writeNumeric(model.getDT(), model.getTimePrecision()) << ", " << model.getBatchSize() << "u));" << std::endl;
+        if(model.isTimingEnabled()) {
+            os << "GENNMI_CHECK(gennmi_runner_set_timing(gennmiRunner, 1));" << std::endl;
+        }
+    }
+    if(hasDeviceModules()) {
+        // (generated step kernels: updateSynapses / updateNeurons calls are noted and replayed from a captured graph of
+        // stepQueueLength steps; custom updates beside library kernels are launched when called, on the runner's stream)
+        os << "GENNMI_CHECK(gennmi_program_create(&gennmiProgram, gennmiRunner, " << (m_GeneratedKernels ? getPreferences<Preferences>().stepQueueLength : 0u) << "u));" << std::endl;
+        os << "GENNMI_CHECK(gennmi_program_error_flag(gennmiProgram, &gennmiProgramError));" << std::endl;
+        if(model.isTimingEnabled()) {
+            os << "GENNMI_CHECK(gennmi_program_set_timing(gennmiProgram, 1));" << std::endl;
+        }
     }
 }
 //--------------------------------------------------------------------------
 void Backend::genFreeMemPreamble(CodeStream &os, const ModelSpecMerged&) const
 {
+    if(hasDeviceModules()) {
+        os << "if(gennmiProgram) { GENNMI_CHECK(gennmi_program_destroy(gennmiProgram)); gennmiProgram = nullptr; gennmiProgramError = nullptr; }" << std::endl;
+        os << "gennmiFreeCustomUpdateGroups();" << std::endl;
+        if(m_GeneratedKernels) { os << "gennmiFreeNeuronGroups();" << std::endl << "gennmiFreeSynapseGroups();" << std::endl; }
+    }
     os << "if(gennmiRunner) { GENNMI_CHECK(gennmi_runner_destroy(gennmiRunner)); gennmiRunner = nullptr; }" << std::endl;
     os << "for(void *p : gennmiScratchBuffers) { gennmi_free(p); }" << std::endl;
     os << "gennmiScratchBuffers.clear();" << std::endl;
@@ -1534,10 +1561,10 @@ void Backend::genFreeMemPreamble(CodeStream &os, const ModelSpecMerged&) const
 void Backend::genStepTimeFinalisePreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const
 {
     if(m_GeneratedKernels) {
-        // (the timers' events are read right after this: genTimer)
+        // (the timers are read right after this: genTimer.  A bounded wait that expired in a kernel is reported by this call, and —
+        // whatever the timing setting — by every later call of the library that waits for the device: pulls, synchronisation)
         if(modelMerged.getModel().isTimingEnabled()) {
-            os << "GENNMI_CHECK(gennmi_synchronize());" << std::endl;
-            os << "gennmiCheckNeuronKernels();" << std::endl;
+            os << "GENNMI_CHECK(gennmi_program_synchronize(gennmiProgram));" << std::endl;
         }
         return;
     }
@@ -1607,20 +1634,23 @@ void Backend::genTimer(CodeStream &definitions, CodeStream &runner, CodeStream &
     // initialisation: wall-clock time of the host functions (genInit)
     // (beside library kernels only the custom updates' kernels are generated, and timed this way)
     if(!hasDeviceModules() || name == "init" || name == "initSparse" || (!m_GeneratedKernels && name.rfind("customUpdate", 0) != 0)) { return; }
-    // generated kernels: a pair of events around each update's launches, as the reference's device backends do
-    // (backendCUDAHIP.cc:1479-1504); read after the step has been synchronised (genStepTimeFinalisePreamble)
-    definitions << "extern hipEvent_t " << name << "Start;" << std::endl;
-    definitions << "extern hipEvent_t " << name << "Stop;" << std::endl;
-    runner << "hipEvent_t " << name << "Start;" << std::endl;
-    runner << "hipEvent_t " << name << "Stop;" << std::endl;
-    allocations << "if(hipEventCreate(&" << name << "Start) != hipSuccess || hipEventCreate(&" << name << "Stop) != hipSuccess) { throw std::runtime_error(\"" << name << ": no timer events\"); }" << std::endl;
-    free << "hipEventDestroy(" << name << "Start);" << std::endl;
-    free << "hipEventDestroy(" << name << "Stop);" << std::endl;
+    // generated kernels: the device library records a pair of events around each launch of the update's kind, as the
+    // reference's device backends do inline (backendCUDAHIP.cc:1479-1504), and accumulates their durations per timer
+    (void)definitions; (void)runner; (void)allocations; (void)free;
     if(updateInStepTime) {
-        CodeStream::Scope b(stepTimeFinalise);
-        stepTimeFinalise << "float tmp = 0.0f;" << std::endl;
-        stepTimeFinalise << "if(hipEventElapsedTime(&tmp, " << name << "Start, " << name << "Stop) == hipSuccess) { " << name << "Time += tmp / 1000.0; }" << std::endl;
+        stepTimeFinalise << "GENNMI_CHECK(gennmi_program_get_time(gennmiProgram, " << timerId(name) << ", &" << name << "Time));" << std::endl;
     }
+}
+// which of the program's timers accumulates an update's launches (asked for by the modules that register the launches and by
+// the runner that reads the time)
+int Backend::timerId(const std::string &name) const
+{
+    const auto it = m_TimerIds.find(name);
+    if(it != m_TimerIds.cend()) { return it->second; }
+    if(m_TimerIds.size() >= GENNMI_MAX_TIMERS) { unsupported("this many timed update groups"); }
+    const int id = (int)m_TimerIds.size();
+    m_TimerIds.emplace(name, id);
+    return id;
 }
 void Backend::genReturnFreeDeviceMemoryBytes(CodeStream &os) const
 {
@@ -1644,14 +1674,15 @@ void Backend::genMakefilePreamble(std::ostream &os) const
     }
     std::string cxxFlags = "-c -fPIC -std=c++17 -MMD -MP -I\"" + root + "/include\" " + getPreferences().userCxxFlagsGNU;
     cxxFlags += getPreferences().debugCode ? " -O0 -g" : " -O2";
-    if(hasDeviceModules()) {
-        // every module holds or calls device code: hipcc for gfx950, fp32 operations neither contracted nor packed so that
-        // results match the SingleThreadedCPU backend's operation for operation
-        os << "CXX := " << (std::getenv("HIP_PATH") ? std::string(std::getenv("HIP_PATH")) + "/bin/hipcc" : std::string("hipcc")) << std::endl;
-        cxxFlags += " -x hip --offload-arch=gfx950 -ffp-contract=off -Xclang -target-feature -Xclang -packed-fp32-ops -Wno-unused-value";
-    }
     os << "CXXFLAGS := " << cxxFlags << std::endl;
-    os << "LINKFLAGS := -shared" << (hasDeviceModules() ? " --offload-arch=gfx950 -fPIC" : "") << std::endl;
+    if(hasDeviceModules()) {
+        // modules that hold device code are compiled a second time, device side only, into a gfx950 code object: fp32 operations
+        // neither contracted nor packed so that results match the SingleThreadedCPU backend's operation for operation
+        os << "HIPCC := " << (std::getenv("HIP_PATH") ? std::string(std::getenv("HIP_PATH")) + "/bin/hipcc" : std::string("hipcc")) << std::endl;
+        os << "HIPCCFLAGS := --genco --offload-arch=gfx950 -std=c++17 -x hip -I\"" << root << "/include\" " << (getPreferences().debugCode ? "-O0 -g" : "-O2")
+           << " -ffp-contract=off -Xclang -target-feature -Xclang -packed-fp32-ops -Wno-unused-value" << std::endl;
+    }
+    os << "LINKFLAGS := -shared" << std::endl;
     os << "LINKLIBS := -L\"" << root << "/genn_amd/lib\" -lgenn_mi355x -Wl,-rpath,\"" << root << "/genn_amd/lib\"" << std::endl;
     os << std::endl;
 }
@@ -1662,7 +1693,18 @@ void Backend::genMakefileLinkRule(std::ostream &os) const
 void Backend::genMakefileCompileRule(std::ostream &os) const
 {
     os << "%.o: %.cc %.d" << std::endl;
-    os << "\t@$(CXX) $(CXXFLAGS) -o $@ $<" << std::endl;
+    if(!hasDeviceModules()) {
+        os << "\t@$(CXX) $(CXXFLAGS) -o $@ $<" << std::endl;
+        return;
+    }
+    // host pass into <module>.host.o; for a module that says GENNMI_DEVICE_MODULE, device pass into <module>.hsaco, which is
+    // wrapped into an object (symbols gennmi_<module>_image / _image_end) and joined with the host object into <module>.o
+    os << "\t@$(CXX) $(CXXFLAGS) -MF $*.d -MT $@ -o $*.host.o $<" << std::endl;
+    os << "\t@if grep -q '^#define GENNMI_DEVICE_MODULE' $<; then \\" << std::endl;
+    os << "\t    $(HIPCC) $(HIPCCFLAGS) -o $*.hsaco $< && \\" << std::endl;
+    os << "\t    printf '.section .rodata\\n.balign 4096\\n.global gennmi_$*_image\\ngennmi_$*_image:\\n.incbin \"$*.hsaco\"\\n.global gennmi_$*_image_end\\ngennmi_$*_image_end:\\n.section .note.GNU-stack,\"\",@progbits\\n' > $*.image.s && \\" << std::endl;
+    os << "\t    $(CXX) -c -o $*.image.o $*.image.s && $(LD) -r -o $@ $*.host.o $*.image.o; \\" << std::endl;
+    os << "\telse cp $*.host.o $@; fi" << std::endl;
 }
 void Backend::genNMakefilePreamble(std::ostream&) const { unsupported("NMake"); }
 void Backend::genNMakefileLinkRule(std::ostream&) const { unsupported("NMake"); }

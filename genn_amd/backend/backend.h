@@ -11,6 +11,7 @@
 //    one of the models the device library implements and translated, once, into a descriptor
 //    (gennmi_*_update_group_t); anything else is rejected at code-generation time with std::runtime_error.
 #include <memory>
+#include <map>
 #include <string>
 
 #include "backendExport.h"
@@ -79,7 +80,7 @@ public:
     Backend(const Preferences &preferences, bool generatedKernels = false, bool customUpdateKernels = false);
 
     bool areKernelsGenerated() const { return m_GeneratedKernels; }
-    //! the runner's modules hold device code and are compiled with hipcc
+    //! some of the runner's modules hold device code: the Makefile builds a gfx950 code object from each of them beside the host object
     bool hasDeviceModules() const { return m_GeneratedKernels || m_CustomUpdateKernels; }
 
     //--------------------------------------------------------------------------
@@ -167,7 +168,11 @@ private:
     void genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMerged, BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const;
     void genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMerged, BackendBase::MemorySpaces &memorySpaces, HostHandler preambleHandler) const;
 
+    //! the timer of the runner's program (gennmi_program_get_time) that accumulates the launches of an update kind
+    int timerId(const std::string &name) const;
+
     const bool m_GeneratedKernels;
     const bool m_CustomUpdateKernels;
+    mutable std::map<std::string, int> m_TimerIds;
 };
 }   // namespace GeNN::CodeGenerator::MI355X

@@ -4,7 +4,11 @@
 // code strings — sim / threshold / reset code, postsynaptic and current-source code, weight-update code with its pre and
 // post variables — are printed by GeNN's environments and pretty-printer (the transpiler stays in libgenn:
 // NeuronUpdateGroupMerged::generateNeuronUpdate, PresynapticUpdateGroupMerged::generateSpikeUpdate, ...) into the
-// skeletons emitted here, and the resulting translation unit is compiled for gfx950 with hipcc as part of the runner.
+// skeletons emitted here.  Every module that holds device code is compiled twice by the runner's Makefile: by the host
+// compiler, which sees the merged-group structs, the host arrays and the host functions (the kernels are hidden from it), and
+// by `hipcc --genco`, which turns the kernels into a gfx950 code object that is embedded in the module's object file.  The host
+// functions load and launch that code object through the device library's C ABI (gennmi_program_*, include/genn_mi355x.h): the
+// runner contains no launch syntax and no HIP call, and a model's steps can be noted and replayed from a captured graph.
 //
 // Skeletons (what the reference's SIMT backends generate in src/genn/genn/code_generator/backendSIMT.cc:405-803, designed
 // anew for 64-wide wavefronts):
@@ -54,15 +58,70 @@ struct BlockTable
     }
 };
 
+// Arguments of one generated kernel beyond the launch header: a struct that both passes of the module see.  Every kernel
+// gets the look-back area and error flag of ordered compactions, the seed of counter-based random numbers, and a pointer to
+// the device copy of each merged group's struct array it walks.
+struct KernelArgs
+{
+    explicit KernelArgs(const std::string &kernelName) : name(kernelName) {}
+    std::string name;
+    std::ostringstream members, unpack, fill;
+    void add(const std::string &type, const std::string &structArray)
+    {
+        members << "    const " << type << " *" << structArray << ";" << std::endl;
+        unpack << "const " << type << " *" << structArray << " = gennmiArgs." << structArray << ";" << std::endl;
+        fill << "a." << structArray << " = d_" << structArray << "; ";
+    }
+    std::string type() const { return "G" + name.substr(1) + "Args"; }      // gennmiXKernel -> GennmiXKernelArgs
+    void define(CodeStream &os) const
+    {
+        os << "struct " << type() << std::endl << "{" << std::endl;
+        os << "    unsigned long long *agg;" << std::endl << "    uint32_t *error;" << std::endl << "    unsigned long long seed;" << std::endl;
+        os << members.str() << "};" << std::endl;
+    }
+    // device pass: signature and the statements that give the kernel's body the names it was written with
+    void open(CodeStream &os, const std::string &timeType, const std::string &attributes = "__launch_bounds__(256) ") const
+    {
+        os << "extern \"C\" __global__ " << attributes << "void " << name << "(gennmi_launch_header_t gennmiLaunch, " << type() << " gennmiArgs)";
+        os << CodeStream::OB(9000);
+        os << "const gennmi_step_entry_t gennmiEntry = gennmi_kernel::stepEntry(gennmiLaunch);" << std::endl;
+        os << "const " << timeType << " t = (" << timeType << ")gennmiEntry.t;" << std::endl;
+        os << "const unsigned int recordingTimestep = gennmiEntry.recordingTimestep;" << std::endl;
+        os << "const uint32_t gennmiTag = gennmiEntry.tag;" << std::endl;
+        os << "const unsigned long long gennmiStep = gennmiEntry.step;" << std::endl;
+        os << "unsigned long long *gennmiAgg = gennmiArgs.agg;" << std::endl;
+        os << "uint32_t *gennmiError = gennmiArgs.error;" << std::endl;
+        os << "const unsigned long long gennmiSeed = gennmiArgs.seed;" << std::endl;
+        os << unpack.str();
+    }
+    void close(CodeStream &os) const { os << CodeStream::CB(9000); }
+    // host pass: the statements that fill an argument block `a` (agg / seed as given)
+    std::string fillBlock(const std::string &agg, const std::string &seed) const
+    {
+        return type() + " a{}; a.agg = " + agg + "; a.error = gennmiProgramError; a.seed = " + seed + "; " + fill.str();
+    }
+    // host pass: looks the kernel up in `module` and appends it to a phase of the program
+    void addToPhase(CodeStream &os, const std::string &phase, size_t gridX, size_t gridY, unsigned int block, int timer,
+                    const std::string &agg, const std::string &seed) const
+    {
+        CodeStream::Scope b(os);
+        os << "uint32_t k = 0;" << std::endl;
+        os << "GENNMI_CHECK(gennmi_program_get_kernel(gennmiProgram, module, \"" << name << "\", &k));" << std::endl;
+        os << fillBlock(agg, seed) << std::endl;
+        os << "GENNMI_CHECK(gennmi_program_add_launch(gennmiProgram, " << phase << ", k, " << gridX << "u, " << gridY << "u, " << block << "u, &a, sizeof(a), " << timer << "));" << std::endl;
+    }
+};
+
 // device copy of a merged group's struct array: declaration, and the statements that translate and upload it
 template<typename G>
-void genDeviceStructArray(CodeStream &decl, CodeStream &upload, const BackendBase &backend, const G &g, const std::string &name)
+void genDeviceStructArray(CodeStream &decl, CodeStream &upload, CodeStream &release, const BackendBase &backend, const G &g, const std::string &name)
 {
     const std::string type = "Merged" + name + "Group" + std::to_string(g.getIndex());
     const std::string host = "merged" + name + "Group" + std::to_string(g.getIndex());
     const std::string dev = "d_" + host;
     const size_t count = g.getGroups().size();
     decl << "static " << type << " *" << dev << " = nullptr;" << std::endl;
+    release << "if(" << dev << ") { gennmi_free(" << dev << "); " << dev << " = nullptr; }" << std::endl;
     upload << "// " << host << std::endl;
     {
         CodeStream::Scope b(upload);
@@ -111,9 +170,10 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     const EnvironmentLibrary::Library simRNGFunctions = simRNGLibrary(model.getPrecision());
     const bool recording = model.isRecordingInUse();
 
-    std::ostringstream kernelStream, declStream, uploadStream, argStream, paramStream;
-    CodeStream kernel(kernelStream), decl(declStream), upload(uploadStream);
+    std::ostringstream kernelStream, declStream, uploadStream, releaseStream;
+    CodeStream kernel(kernelStream), decl(declStream), upload(uploadStream), release(releaseStream);
     BlockTable table;
+    KernelArgs neuronKernel("gennmiNeuronUpdateKernel"), prevKernel("gennmiPrevSpikeTimeKernel"), queueKernel("gennmiSpikeQueueUpdateKernel");
 
     EnvironmentLibrary kernelEnv(kernel, StandardLibrary::getMathsFunctions());
     bool anyRNG = false;
@@ -141,8 +201,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                 for(size_t b = 0; b < blocks; b++) { table.add(g, b * 256, b, blocks); }
             }
             const std::string structArray = "mergedNeuronUpdateGroup" + std::to_string(n.getIndex());
-            argStream << ", d_" << structArray;
-            paramStream << ", const MergedNeuronUpdateGroup" << n.getIndex() << " *" << structArray;
+            neuronKernel.add("MergedNeuronUpdateGroup" + std::to_string(n.getIndex()), structArray);
 
             funcEnv.getStream() << "// merged neuron update group " << n.getIndex() << std::endl;
             funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << table.numBlocks << "u)";
@@ -198,7 +257,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             }
             groupEnv.printLine("const gennmi_kernel::QueueSlot slot = gennmi_kernel::orderedSlot(gennmiSpiked, entry.blockInGroup, entry.blocksInGroup, "
                                "blockIdx.x - entry.blockInGroup, gennmiAgg + (size_t)2 * gridDim.x * blockIdx.y, gennmiAgg + (size_t)2 * gridDim.x * blockIdx.y + gridDim.x, "
-                               "gennmiTag, gennmiError);");
+                               "gennmiTag, gennmiError, gennmiLaunch.spinLimit);");
             if(arch.isSpikeRecordingEnabled()) {
                 groupEnv.printLine("gennmi_kernel::recordBallot(&$(_record_spk)[((size_t)recordingTimestep * " + std::to_string(batchSize) + "u + $(batch)) * numRecordingWords], "
                                    "$(id), $(id) < $(num_neurons), slot.ballot);");
@@ -218,7 +277,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                         const std::string k = std::to_string(e.getIndex());
                         const std::string region = "gennmiAgg + (size_t)2 * gridDim.x * (gridDim.y * " + std::to_string(e.getIndex() + 1) + "u + blockIdx.y)";
                         env.printLine("const gennmi_kernel::QueueSlot eventSlot" + k + " = gennmi_kernel::orderedSlot(gennmiEvent" + k + ", entry.blockInGroup, entry.blocksInGroup, "
-                                      "blockIdx.x - entry.blockInGroup, " + region + ", " + region + " + gridDim.x, gennmiTag, gennmiError);");
+                                      "blockIdx.x - entry.blockInGroup, " + region + ", " + region + " + gridDim.x, gennmiTag, gennmiError, gennmiLaunch.spinLimit);");
                         if(recordEvents) {
                             env.printLine("gennmi_kernel::recordBallot(&$(_record_spk_event)[((size_t)recordingTimestep * " + std::to_string(batchSize) + "u + $(batch)) * numRecordingWords], "
                                           "$(id), $(id) < $(num_neurons), eventSlot" + k + ".ballot);");
@@ -245,7 +304,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
 
     // Previous spike (and event) times: every neuron in last step's queue gets prev_st = t - dt, in a kernel that runs before
     // the ring pointers move on (backendSIMT.cc:320-368, 1897-1925)
-    std::ostringstream prevStream, prevArgs, prevParams;
+    std::ostringstream prevStream;
     BlockTable prevTable;
     if(!modelMerged.getMergedNeuronPrevSpikeTimeUpdateGroups().empty()) {
         CodeStream prev(prevStream);
@@ -265,8 +324,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                     for(size_t b = 0; b < blocks; b++) { prevTable.add(g, b * 256, b, blocks); }
                 }
                 const std::string structArray = "mergedNeuronPrevSpikeTimeUpdateGroup" + std::to_string(n.getIndex());
-                prevArgs << ", d_" << structArray;
-                prevParams << ", const MergedNeuronPrevSpikeTimeUpdateGroup" << n.getIndex() << " *" << structArray;
+                prevKernel.add("MergedNeuronPrevSpikeTimeUpdateGroup" + std::to_string(n.getIndex()), structArray);
                 prevEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << prevTable.numBlocks << "u)";
                 CodeStream::Scope b(prevEnv.getStream());
                 prevEnv.getStream() << "const gennmi_kernel::BlockEntry entry = gennmiPrevSpikeTimeBlocks[blockIdx.x];" << std::endl;
@@ -300,7 +358,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     // Without delay slots that kernel would only clear counts that the compaction overwrites anyway, and is left out.
     const bool anyDelaySlots = std::any_of(model.getNeuronGroups().cbegin(), model.getNeuronGroups().cend(),
                                            [](const auto &n) { return n.second.isDelayRequired(); });
-    std::ostringstream queueStream, queueArgs, queueParams;
+    std::ostringstream queueStream;
     if(anyDelaySlots) {
         CodeStream queue(queueStream);
         EnvironmentLibrary queueLib(queue, StandardLibrary::getMathsFunctions());
@@ -310,49 +368,74 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             [&](auto &n)
             {
                 const std::string structArray = "mergedNeuronSpikeQueueUpdateGroup" + std::to_string(n.getIndex());
-                queueArgs << (queueArgs.str().empty() ? "" : ", ") << "d_" << structArray;
-                queueParams << (queueParams.str().empty() ? "" : ", ") << "MergedNeuronSpikeQueueUpdateGroup" << n.getIndex() << " *" << structArray;
+                queueKernel.add("MergedNeuronSpikeQueueUpdateGroup" + std::to_string(n.getIndex()), structArray);
                 queueEnv.getStream() << "for(unsigned int g = threadIdx.x; g < " << n.getGroups().size() << "u; g += blockDim.x)";
                 CodeStream::Scope b(queueEnv.getStream());
-                queueEnv.getStream() << "auto *group = &" << structArray << "[g];" << std::endl;
+                queueEnv.getStream() << "const auto *group = &" << structArray << "[g];" << std::endl;
                 EnvironmentGroupMergedField<NeuronSpikeQueueUpdateGroupMerged> groupEnv(queueEnv, n);
                 buildStandardEnvironment(groupEnv, batchSize);
                 n.genSpikeQueueUpdate(groupEnv, batchSize);
             });
     }
 
-    // struct definitions, host arrays and their push functions are GeNN's own
+    // struct definitions (both passes), then the host arrays and their push functions (GeNN's own) for the host pass
+    const bool timing = model.isTimingEnabled();
+    const std::string seed = anyRNG ? ((model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull") : std::string("gennmiRandomSeed()")) : std::string("0ull");
+    os << "#define GENNMI_DEVICE_MODULE 1      // the Makefile builds a gfx950 code object from this file as well" << std::endl;
     modelMerged.genMergedNeuronUpdateGroupStructs(os, *this);
-    modelMerged.genMergedNeuronUpdateGroupHostStructArrayPush(os, *this);
-    if(anyDelaySlots) {
-        modelMerged.genMergedNeuronSpikeQueueUpdateStructs(os, *this);
-        modelMerged.genMergedNeuronSpikeQueueUpdateHostStructArrayPush(os, *this);
-    }
+    if(anyDelaySlots) { modelMerged.genMergedNeuronSpikeQueueUpdateStructs(os, *this); }
+    if(anyPrevTimes) { modelMerged.genMergedNeuronPrevSpikeTimeUpdateStructs(os, *this); }
+    neuronKernel.define(os);
+    if(anyDelaySlots) { queueKernel.define(os); }
+    if(anyPrevTimes) { prevKernel.define(os); }
+    os << std::endl;
+
+    // ---- device pass
+    os << "#ifdef __HIPCC__" << std::endl;
+    os << "__device__ const gennmi_kernel::BlockEntry gennmiNeuronBlocks[] = {" << std::endl << table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
     if(anyPrevTimes) {
-        modelMerged.genMergedNeuronPrevSpikeTimeUpdateStructs(os, *this);
-        modelMerged.genMergedNeuronPrevSpikeTimeUpdateHostStructArrayPush(os, *this);
+        os << "__device__ const gennmi_kernel::BlockEntry gennmiPrevSpikeTimeBlocks[] = {" << std::endl << prevTable.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+        prevKernel.open(os, timeType);
+        os << prevStream.str();
+        prevKernel.close(os);
     }
+    if(anyDelaySlots) {
+        queueKernel.open(os, timeType, "");
+        os << queueStream.str();
+        queueKernel.close(os);
+    }
+    os << std::endl;
+    neuronKernel.open(os, timeType);
+    os << kernelStream.str();
+    neuronKernel.close(os);
+    os << std::endl;
+
+    // ---- host pass
+    os << "#else" << std::endl;
+    modelMerged.genMergedNeuronUpdateGroupHostStructArrayPush(os, *this);
+    if(anyDelaySlots) { modelMerged.genMergedNeuronSpikeQueueUpdateHostStructArrayPush(os, *this); }
+    if(anyPrevTimes) { modelMerged.genMergedNeuronPrevSpikeTimeUpdateHostStructArrayPush(os, *this); }
     preambleHandler(os);
     for(const auto &n : modelMerged.getMergedNeuronUpdateGroups()) {
-        genDeviceStructArray(decl, upload, *this, n, "NeuronUpdate");
+        genDeviceStructArray(decl, upload, release, *this, n, "NeuronUpdate");
     }
     if(anyDelaySlots) {
-        for(const auto &n : modelMerged.getMergedNeuronSpikeQueueUpdateGroups()) { genDeviceStructArray(decl, upload, *this, n, "NeuronSpikeQueueUpdate"); }
+        for(const auto &n : modelMerged.getMergedNeuronSpikeQueueUpdateGroups()) { genDeviceStructArray(decl, upload, release, *this, n, "NeuronSpikeQueueUpdate"); }
     }
     if(anyPrevTimes) {
-        for(const auto &n : modelMerged.getMergedNeuronPrevSpikeTimeUpdateGroups()) { genDeviceStructArray(decl, upload, *this, n, "NeuronPrevSpikeTimeUpdate"); }
+        for(const auto &n : modelMerged.getMergedNeuronPrevSpikeTimeUpdateGroups()) { genDeviceStructArray(decl, upload, release, *this, n, "NeuronPrevSpikeTimeUpdate"); }
     }
-
     os << declStream.str();
     os << "static unsigned long long *gennmiNeuronAgg = nullptr;" << std::endl;
-    os << "static uint32_t *gennmiNeuronError = nullptr;" << std::endl;
-    os << "static unsigned int gennmiNeuronLaunches = 0;" << std::endl;
-    os << "__device__ const gennmi_kernel::BlockEntry gennmiNeuronBlocks[] = {" << std::endl << table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+    os << "extern \"C\" const unsigned char gennmi_neuronUpdate_image[];" << std::endl;
+    os << "extern \"C\" const unsigned char gennmi_neuronUpdate_image_end[];" << std::endl;
     os << std::endl;
     os << "void gennmiUploadNeuronGroups()";
     {
         CodeStream::Scope b(os);
         os << uploadStream.str();
+        // (the first time: the look-back words of the ordered compactions, then the launches of updateNeurons(), in the order of
+        // the reference's function, backendCUDAHIP.cc:386-420: previous spike times, ring pointers of the spike queues, the update)
         os << "if(!gennmiNeuronAgg)";
         {
             CodeStream::Scope b2(os);
@@ -360,64 +443,33 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             os << "GENNMI_CHECK(gennmi_malloc(&p, " << 2 * std::max<size_t>(1, table.numBlocks) * batchSize * (1 + maxEventGroups) << " * sizeof(unsigned long long)));" << std::endl;
             os << "GENNMI_CHECK(gennmi_memset(p, 0, " << 2 * std::max<size_t>(1, table.numBlocks) * batchSize * (1 + maxEventGroups) << " * sizeof(unsigned long long)));" << std::endl;
             os << "gennmiNeuronAgg = (unsigned long long*)p;" << std::endl;
-            os << "GENNMI_CHECK(gennmi_malloc(&p, sizeof(uint32_t)));" << std::endl;
-            os << "GENNMI_CHECK(gennmi_memset(p, 0, sizeof(uint32_t)));" << std::endl;
-            os << "gennmiNeuronError = (uint32_t*)p;" << std::endl;
+            os << "uint32_t module = 0;" << std::endl;
+            os << "GENNMI_CHECK(gennmi_program_load_module(gennmiProgram, gennmi_neuronUpdate_image, (size_t)(gennmi_neuronUpdate_image_end - gennmi_neuronUpdate_image), &module));" << std::endl;
+            if(anyPrevTimes) { prevKernel.addToPhase(os, "GENNMI_PHASE_NEURONS", prevTable.numBlocks, batchSize, 256, -1, "nullptr", "0ull"); }
+            if(anyDelaySlots) { queueKernel.addToPhase(os, "GENNMI_PHASE_NEURONS", 1, 1, 64, -1, "nullptr", "0ull"); }
+            if(table.numBlocks > 0) { neuronKernel.addToPhase(os, "GENNMI_PHASE_NEURONS", table.numBlocks, batchSize, 256, timing ? timerId("neuronUpdate") : -1, "gennmiNeuronAgg", seed); }
         }
     }
     os << std::endl;
-    if(anyPrevTimes) {
-        os << "__device__ const gennmi_kernel::BlockEntry gennmiPrevSpikeTimeBlocks[] = {" << std::endl << prevTable.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
-        os << "__global__ __launch_bounds__(256) void gennmiPrevSpikeTimeKernel(" << timeType << " t" << prevParams.str() << ")";
-        CodeStream::Scope b(os);
-        os << prevStream.str();
-    }
-    if(anyDelaySlots) {
-        os << "__global__ void gennmiSpikeQueueUpdateKernel(" << queueParams.str() << ")";
-        CodeStream::Scope b(os);
-        os << queueStream.str();
-    }
-    os << std::endl;
-    os << "__global__ __launch_bounds__(256) void gennmiNeuronUpdateKernel(" << timeType << " t, unsigned int recordingTimestep, uint32_t gennmiTag, "
-          "unsigned long long *gennmiAgg, uint32_t *gennmiError, unsigned long long gennmiSeed, unsigned long long gennmiStep" << paramStream.str() << ")";
+    os << "void gennmiFreeNeuronGroups()";
     {
         CodeStream::Scope b(os);
-        os << kernelStream.str();
+        os << "if(gennmiNeuronAgg) { gennmi_free(gennmiNeuronAgg); gennmiNeuronAgg = nullptr; }" << std::endl;
+        os << releaseStream.str();
     }
     os << std::endl;
+    // the time, the recording row, the generator's step (calls of updateNeurons so far) and the look-back tag of the call travel
+    // in the launch header; a bounded wait of the compaction that expires raises the program's error flag, which the library
+    // reports from the next call that waits for the device (whatever the timing setting)
     os << "void updateNeurons(" << model.getTimePrecision().getName() << " t";
     if(recording) { os << ", unsigned int recordingTimestep"; }
     os << ")";
     {
         CodeStream::Scope b(os);
         os << "gennmiEnsureFinalised();" << std::endl;
-        if(anyPrevTimes) { os << "gennmiPrevSpikeTimeKernel<<<dim3(" << prevTable.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << prevArgs.str() << ");" << std::endl; }
-        if(anyDelaySlots) { os << "gennmiSpikeQueueUpdateKernel<<<dim3(1), dim3(64), 0, 0>>>(" << queueArgs.str() << ");" << std::endl; }
-        const bool timing = model.isTimingEnabled();
-        if(timing) { os << "hipEventRecord(neuronUpdateStart, 0);" << std::endl; }
-        if(table.numBlocks > 0) {
-            // the tag of a launch: differs from one launch to the next, never 0 (the look-back words start out zero)
-            os << "gennmiNeuronLaunches = (gennmiNeuronLaunches == 0xFFFFFFFFu) ? 1u : gennmiNeuronLaunches + 1u;" << std::endl;
-            // (the generator's step counter: calls of updateNeurons so far; the seed: the model's, or one drawn at load time)
-            os << "static unsigned long long gennmiNeuronStep = 0;" << std::endl;
-            os << "gennmiNeuronUpdateKernel<<<dim3(" << table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t, " << (recording ? "recordingTimestep" : "0u")
-               << ", gennmiNeuronLaunches, gennmiNeuronAgg, gennmiNeuronError, "
-               << (anyRNG ? ((model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull") : std::string("gennmiRandomSeed()")) : std::string("0ull"))
-               << ", gennmiNeuronStep++" << argStream.str() << ");" << std::endl;
-            os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateNeurons: kernel launch failed\"); }" << std::endl;
-        }
-        if(timing) { os << "hipEventRecord(neuronUpdateStop, 0);" << std::endl; }
+        os << "GENNMI_CHECK(gennmi_program_update(gennmiProgram, GENNMI_PHASE_NEURONS, (double)t, " << (recording ? "recordingTimestep" : "0u") << "));" << std::endl;
     }
-    os << std::endl;
-    // bounded waits of the compaction that expired are reported where the reference's backends check for launch errors
-    os << "void gennmiCheckNeuronKernels()";
-    {
-        CodeStream::Scope b(os);
-        os << "if(!gennmiNeuronError) { return; }" << std::endl;
-        os << "uint32_t flag = 0;" << std::endl;
-        os << "GENNMI_CHECK(gennmi_memcpy_from_device(&flag, gennmiNeuronError, sizeof(flag)));" << std::endl;
-        os << "if(flag) { throw std::runtime_error(\"updateNeurons: a work-group's bounded wait for spike-queue offsets expired\"); }" << std::endl;
-    }
+    os << "#endif" << std::endl;
 }
 //--------------------------------------------------------------------------
 void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMerged, BackendBase::MemorySpaces &memorySpaces,
@@ -430,16 +482,18 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
     const std::string timeType = model.getTimePrecision().getName();
     const EnvironmentLibrary::Library simRNGFunctions = simRNGLibrary(model.getPrecision());
 
-    std::ostringstream declStream, uploadStream;
-    CodeStream decl(declStream), upload(uploadStream);
+    std::ostringstream declStream, uploadStream, releaseStream;
+    CodeStream decl(declStream), upload(uploadStream), release(releaseStream);
 
     // every kernel's body, arguments and block table
     struct KernelText
     {
-        std::ostringstream body, args, params;
+        explicit KernelText(const std::string &name) : args(name) {}
+        std::ostringstream body;
+        KernelArgs args;
         BlockTable table;
     };
-    KernelText delay, dynamics, pre, post;
+    KernelText delay("gennmiDendriticDelayUpdateKernel"), dynamics("gennmiSynapseDynamicsKernel"), pre("gennmiPresynapticUpdateKernel"), post("gennmiPostsynapticUpdateKernel");
     auto makeEnv = [&model, &simRNGFunctions](CodeStream &stream, EnvironmentLibrary &lib, auto use)
     {
         EnvironmentLibrary rngLib(lib, simRNGFunctions);        // (gennrand_* of weight-update code: `_rng` exists where it is used)
@@ -495,8 +549,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         for(size_t b = 0; b < blocks; b++) { dynamics.table.add(g, 0, b, blocks); }
                     }
                     const std::string structArray = "mergedSynapseDynamicsGroup" + std::to_string(s.getIndex());
-                    dynamics.args << ", d_" << structArray;
-                    dynamics.params << ", const MergedSynapseDynamicsGroup" << s.getIndex() << " *" << structArray;
+                    dynamics.args.add("MergedSynapseDynamicsGroup" + std::to_string(s.getIndex()), structArray);
 
                     funcEnv.getStream() << "// merged synapse dynamics group " << s.getIndex() << std::endl;
                     funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << dynamics.table.numBlocks << "u)";
@@ -558,8 +611,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                 {
                     const std::string structArray = "mergedSynapseDendriticDelayUpdateGroup" + std::to_string(sg.getIndex());
                     delay.table.numBlocks++;
-                    delay.args << ", d_" << structArray;
-                    delay.params << ", const MergedSynapseDendriticDelayUpdateGroup" << sg.getIndex() << " *" << structArray;
+                    delay.args.add("MergedSynapseDendriticDelayUpdateGroup" + std::to_string(sg.getIndex()), structArray);
                     funcEnv.getStream() << "for(unsigned int g = threadIdx.x; g < " << sg.getGroups().size() << "u; g += blockDim.x)";
                     CodeStream::Scope b(funcEnv.getStream());
                     funcEnv.getStream() << "const auto *group = &" << structArray << "[g];" << std::endl;
@@ -606,8 +658,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         for(size_t b = 0; b < blocks; b++) { pre.table.add(g, 0, b, blocks); }
                     }
                     const std::string structArray = "mergedPresynapticUpdateGroup" + std::to_string(s.getIndex());
-                    pre.args << ", d_" << structArray;
-                    pre.params << ", const MergedPresynapticUpdateGroup" << s.getIndex() << " *" << structArray;
+                    pre.args.add("MergedPresynapticUpdateGroup" + std::to_string(s.getIndex()), structArray);
 
                     funcEnv.getStream() << "// merged presynaptic update group " << s.getIndex() << std::endl;
                     funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << pre.table.numBlocks << "u)";
@@ -824,8 +875,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         for(size_t b = 0; b < blocks; b++) { post.table.add(g, 0, b, blocks); }
                     }
                     const std::string structArray = "mergedPostsynapticUpdateGroup" + std::to_string(s.getIndex());
-                    post.args << ", d_" << structArray;
-                    post.params << ", const MergedPostsynapticUpdateGroup" << s.getIndex() << " *" << structArray;
+                    post.args.add("MergedPostsynapticUpdateGroup" + std::to_string(s.getIndex()), structArray);
 
                     funcEnv.getStream() << "// merged postsynaptic update group " << s.getIndex() << std::endl;
                     funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << post.table.numBlocks << "u)";
@@ -896,79 +946,85 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         });
     }
 
-    // struct definitions, host arrays and push functions (GeNN's own), then the device copies
+    // struct definitions (both passes), then the kernels (device pass) or the host arrays, push functions and updateSynapses() (host pass)
+    const bool anyDelay = delay.table.numBlocks > 0, anyPre = pre.table.numBlocks > 0, anyPost = post.table.numBlocks > 0, anyDynamics = dynamics.table.numBlocks > 0;
+    const bool timing = model.isTimingEnabled();
+    const std::string seed = anySynapseRNG ? ((model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull") : std::string("gennmiRandomSeed()")) : std::string("0ull");
+    if(anyDelay || anyDynamics || anyPre || anyPost) { os << "#define GENNMI_DEVICE_MODULE 1      // the Makefile builds a gfx950 code object from this file as well" << std::endl; }
     modelMerged.genMergedSynapseDendriticDelayUpdateStructs(os, *this);
     modelMerged.genMergedPresynapticUpdateGroupStructs(os, *this);
     modelMerged.genMergedPostsynapticUpdateGroupStructs(os, *this);
     modelMerged.genMergedSynapseDynamicsGroupStructs(os, *this);
+    for(const auto *k : {&delay, &dynamics, &pre, &post}) {
+        if(k->table.numBlocks > 0) { k->args.define(os); }
+    }
+    os << std::endl;
+
+    // ---- device pass
+    os << "#ifdef __HIPCC__" << std::endl;
+    os << "__device__ const gennmi_kernel::BlockEntry gennmiPresynapticBlocks[] = {" << std::endl << pre.table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+    os << "__device__ const gennmi_kernel::BlockEntry gennmiPostsynapticBlocks[] = {" << std::endl << post.table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+    os << "__device__ const gennmi_kernel::BlockEntry gennmiSynapseDynamicsBlocks[] = {" << std::endl << dynamics.table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+    os << std::endl;
+    if(anyDynamics) { dynamics.args.open(os, timeType); os << dynamics.body.str(); dynamics.args.close(os); }
+    if(anyDelay) { delay.args.open(os, timeType, ""); os << delay.body.str(); delay.args.close(os); }
+    if(anyPre) { pre.args.open(os, timeType); os << pre.body.str(); pre.args.close(os); }
+    if(anyPost) { post.args.open(os, timeType); os << post.body.str(); post.args.close(os); }
+    os << std::endl;
+
+    // ---- host pass
+    os << "#else" << std::endl;
     modelMerged.genMergedSynapseDendriticDelayUpdateHostStructArrayPush(os, *this);
     modelMerged.genMergedPresynapticUpdateGroupHostStructArrayPush(os, *this);
     modelMerged.genMergedPostsynapticUpdateGroupHostStructArrayPush(os, *this);
     modelMerged.genMergedSynapseDynamicsGroupHostStructArrayPush(os, *this);
     preambleHandler(os);
-    for(const auto &g : modelMerged.getMergedSynapseDendriticDelayUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "SynapseDendriticDelayUpdate"); }
-    for(const auto &g : modelMerged.getMergedPresynapticUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "PresynapticUpdate"); }
-    for(const auto &g : modelMerged.getMergedPostsynapticUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "PostsynapticUpdate"); }
-    for(const auto &g : modelMerged.getMergedSynapseDynamicsGroups()) { genDeviceStructArray(decl, upload, *this, g, "SynapseDynamics"); }
-
+    for(const auto &g : modelMerged.getMergedSynapseDendriticDelayUpdateGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "SynapseDendriticDelayUpdate"); }
+    for(const auto &g : modelMerged.getMergedPresynapticUpdateGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "PresynapticUpdate"); }
+    for(const auto &g : modelMerged.getMergedPostsynapticUpdateGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "PostsynapticUpdate"); }
+    for(const auto &g : modelMerged.getMergedSynapseDynamicsGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "SynapseDynamics"); }
     os << declStream.str();
-    os << "__device__ const gennmi_kernel::BlockEntry gennmiPresynapticBlocks[] = {" << std::endl << pre.table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
-    os << "__device__ const gennmi_kernel::BlockEntry gennmiPostsynapticBlocks[] = {" << std::endl << post.table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
-    os << "__device__ const gennmi_kernel::BlockEntry gennmiSynapseDynamicsBlocks[] = {" << std::endl << dynamics.table.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
+    os << "static bool gennmiSynapseLaunchesRegistered = false;" << std::endl;
+    os << "extern \"C\" const unsigned char gennmi_synapseUpdate_image[];" << std::endl;
+    os << "extern \"C\" const unsigned char gennmi_synapseUpdate_image_end[];" << std::endl;
     os << std::endl;
     os << "void gennmiUploadSynapseGroups()";
     {
         CodeStream::Scope b(os);
         os << uploadStream.str();
+        // the first time: the launches of updateSynapses() in the order of the reference's function (backendCUDAHIP.cc:548-589):
+        // ring pointers, synapse dynamics, presynaptic, postsynaptic; timers exist for the kinds of update the model has merged
+        // groups of (generateRunner.cc:177-199)
+        os << "if(!gennmiSynapseLaunchesRegistered)";
+        {
+            CodeStream::Scope b2(os);
+            if(anyDelay || anyDynamics || anyPre || anyPost) {
+                os << "uint32_t module = 0;" << std::endl;
+                os << "GENNMI_CHECK(gennmi_program_load_module(gennmiProgram, gennmi_synapseUpdate_image, (size_t)(gennmi_synapseUpdate_image_end - gennmi_synapseUpdate_image), &module));" << std::endl;
+            }
+            if(anyDelay) { delay.args.addToPhase(os, "GENNMI_PHASE_SYNAPSES", 1, 1, 64, -1, "nullptr", "0ull"); }
+            if(anyDynamics) { dynamics.args.addToPhase(os, "GENNMI_PHASE_SYNAPSES", dynamics.table.numBlocks, batchSize, 256, timing ? timerId("synapseDynamics") : -1, "nullptr", seed); }
+            if(anyPre) { pre.args.addToPhase(os, "GENNMI_PHASE_SYNAPSES", pre.table.numBlocks, batchSize, 256, timing ? timerId("presynapticUpdate") : -1, "nullptr", seed); }
+            if(anyPost) { post.args.addToPhase(os, "GENNMI_PHASE_SYNAPSES", post.table.numBlocks, batchSize, 256, timing ? timerId("postsynapticUpdate") : -1, "nullptr", seed); }
+            os << "gennmiSynapseLaunchesRegistered = true;" << std::endl;
+        }
     }
     os << std::endl;
-    const bool anyDelay = delay.table.numBlocks > 0, anyPre = pre.table.numBlocks > 0, anyPost = post.table.numBlocks > 0, anyDynamics = dynamics.table.numBlocks > 0;
-    if(anyDynamics) {
-        os << "__global__ __launch_bounds__(256) void gennmiSynapseDynamicsKernel(" << timeType << " t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << dynamics.params.str() << ")";
+    os << "void gennmiFreeSynapseGroups()";
+    {
         CodeStream::Scope b(os);
-        os << dynamics.body.str();
-    }
-    if(anyDelay) {
-        os << "__global__ void gennmiDendriticDelayUpdateKernel(" << timeType << " t" << delay.params.str() << ")";
-        CodeStream::Scope b(os);
-        os << delay.body.str();
-    }
-    if(anyPre) {
-        os << "__global__ __launch_bounds__(256) void gennmiPresynapticUpdateKernel(" << timeType << " t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << pre.params.str() << ")";
-        CodeStream::Scope b(os);
-        os << pre.body.str();
-    }
-    if(anyPost) {
-        os << "__global__ __launch_bounds__(256) void gennmiPostsynapticUpdateKernel(" << timeType << " t, unsigned long long gennmiSeed, unsigned long long gennmiStep" << post.params.str() << ")";
-        CodeStream::Scope b(os);
-        os << post.body.str();
+        os << "gennmiSynapseLaunchesRegistered = false;" << std::endl;
+        os << releaseStream.str();
     }
     os << std::endl;
+    // (the generators' step counter — calls of updateSynapses so far — travels in the launch header)
     os << "void updateSynapses(" << model.getTimePrecision().getName() << " t)";
     {
         CodeStream::Scope b(os);
         os << "gennmiEnsureFinalised();" << std::endl;
-        // order of the reference's updateSynapses (backendCUDAHIP.cc:548-589): ring pointers, synapse dynamics, presynaptic, postsynaptic
-        if(anyDelay) { os << "gennmiDendriticDelayUpdateKernel<<<dim3(1), dim3(64), 0, 0>>>(t" << delay.args.str() << ");" << std::endl; }
-        // (the generators' step counter: calls of updateSynapses so far; the seed: the model's, or one drawn at load time)
-        const std::string seedAndStep = std::string(", ") + (anySynapseRNG ? ((model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull") : std::string("gennmiRandomSeed()")) : std::string("0ull"))
-                                        + ", gennmiSynapseStep";
-        os << "static unsigned long long gennmiSynapseStep = 0;" << std::endl;
-        // (timers exist for the kinds of update the model has merged groups of, generateRunner.cc:177-199)
-        const bool timing = model.isTimingEnabled();
-        auto timer = [&](bool exists, const char *name, const char *edge) { if(timing && exists) { os << "hipEventRecord(" << name << edge << ", 0);" << std::endl; } };
-        timer(!modelMerged.getMergedSynapseDynamicsGroups().empty(), "synapseDynamics", "Start");
-        if(anyDynamics) { os << "gennmiSynapseDynamicsKernel<<<dim3(" << dynamics.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << seedAndStep << dynamics.args.str() << ");" << std::endl; }
-        timer(!modelMerged.getMergedSynapseDynamicsGroups().empty(), "synapseDynamics", "Stop");
-        timer(!modelMerged.getMergedPresynapticUpdateGroups().empty(), "presynapticUpdate", "Start");
-        if(anyPre) { os << "gennmiPresynapticUpdateKernel<<<dim3(" << pre.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << seedAndStep << pre.args.str() << ");" << std::endl; }
-        timer(!modelMerged.getMergedPresynapticUpdateGroups().empty(), "presynapticUpdate", "Stop");
-        timer(!modelMerged.getMergedPostsynapticUpdateGroups().empty(), "postsynapticUpdate", "Start");
-        if(anyPost) { os << "gennmiPostsynapticUpdateKernel<<<dim3(" << post.table.numBlocks << ", " << batchSize << "), dim3(256), 0, 0>>>(t" << seedAndStep << post.args.str() << ");" << std::endl; }
-        timer(!modelMerged.getMergedPostsynapticUpdateGroups().empty(), "postsynapticUpdate", "Stop");
-        os << "gennmiSynapseStep++;" << std::endl;
-        os << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"updateSynapses: kernel launch failed\"); }" << std::endl;
+        os << "GENNMI_CHECK(gennmi_program_update(gennmiProgram, GENNMI_PHASE_SYNAPSES, (double)t, 0u));" << std::endl;
     }
+    os << "#endif" << std::endl;
 }
 //--------------------------------------------------------------------------
 // Custom updates: update<Group>(timestep), one function per update-group name (Runtime::customUpdate looks them up by that
@@ -998,8 +1054,8 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         if(Utils::isRNGRequired(arch.getUpdateCodeTokens())) { notGenerated("random numbers in custom update code (custom update '" + arch.getName() + "')"); }
     };
 
-    std::ostringstream declStream, uploadStream, deviceStream, hostStream;
-    CodeStream decl(declStream), upload(uploadStream), device(deviceStream), host(hostStream);
+    std::ostringstream declStream, uploadStream, releaseStream, deviceStream, hostStream, argsStream, lookupStream, kernelIdStream;
+    CodeStream decl(declStream), upload(uploadStream), release(releaseStream), device(deviceStream), host(hostStream), argsDefs(argsStream), lookup(lookupStream);
     const std::string timeType = model.getTimePrecision().getName();
     const EnvironmentLibrary::Library simRNGFunctions = simRNGLibrary(model.getPrecision());
     auto reduceOps = [this](auto &env, const std::vector<ReductionTarget> &targets)
@@ -1028,7 +1084,8 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     for(const std::string &name : groupNames) {
         std::ostringstream notes;
         // ---- per-neuron custom updates
-        std::ostringstream neuronBody, neuronArgs, neuronParams;
+        std::ostringstream neuronBody;
+        KernelArgs neuronArgs("gennmiCustomUpdate" + name + "Kernel");
         BlockTable neuronTable;
         {
             CodeStream body(neuronBody);
@@ -1051,8 +1108,7 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                         for(size_t b = 0; b < blocks; b++) { neuronTable.add(g, b * 256, b, blocks); }
                     }
                     const std::string structArray = "mergedCustomUpdateGroup" + std::to_string(c.getIndex());
-                    neuronArgs << ", d_" << structArray;
-                    neuronParams << ", const MergedCustomUpdateGroup" << c.getIndex() << " *" << structArray;
+                    neuronArgs.add("MergedCustomUpdateGroup" + std::to_string(c.getIndex()), structArray);
 
                     funcEnv.getStream() << "// merged custom update group " << c.getIndex() << std::endl;
                     funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << neuronTable.numBlocks << "u)";
@@ -1129,7 +1185,8 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         }
 
         // ---- per-synapse custom updates
-        std::ostringstream wuBody, wuArgs, wuParams, wuTables;
+        std::ostringstream wuBody, wuTables;
+        KernelArgs wuArgs("gennmiCustomUpdateWU" + name + "Kernel");
         size_t wuBlocks = 0;
         {
             CodeStream body(wuBody);
@@ -1165,8 +1222,7 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                     }
                     wuTables << wuBlocks << "u};" << std::endl;
                     const std::string structArray = "mergedCustomUpdateWUGroup" + std::to_string(c.getIndex());
-                    wuArgs << ", d_" << structArray;
-                    wuParams << ", const MergedCustomUpdateWUGroup" << c.getIndex() << " *" << structArray;
+                    wuArgs.add("MergedCustomUpdateWUGroup" + std::to_string(c.getIndex()), structArray);
                     const std::string idType = getSynapseIndexType(c).getName();
 
                     funcEnv.getStream() << "// merged custom WU update group " << c.getIndex() << std::endl;
@@ -1220,7 +1276,8 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         }
 
         // ---- per-synapse custom updates that also write the transpose of one variable (DENSE only, customUpdate.cc checks)
-        std::ostringstream trBody, trArgs, trParams, trTables;
+        std::ostringstream trBody, trTables;
+        KernelArgs trArgs("gennmiCustomUpdateTranspose" + name + "Kernel");
         size_t trBlocks = 0;
         {
             CodeStream body(trBody);
@@ -1245,8 +1302,7 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                     }
                     trTables << trBlocks << "u};" << std::endl;
                     const std::string structArray = "mergedCustomUpdateTransposeWUGroup" + std::to_string(c.getIndex());
-                    trArgs << ", d_" << structArray;
-                    trParams << ", const MergedCustomUpdateTransposeWUGroup" << c.getIndex() << " *" << structArray;
+                    trArgs.add("MergedCustomUpdateTransposeWUGroup" + std::to_string(c.getIndex()), structArray);
 
                     funcEnv.getStream() << "// merged custom WU transpose update group " << c.getIndex() << std::endl;
                     funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << trBlocks << "u)";
@@ -1300,7 +1356,8 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         // bookkeeping of every variable that lives on the synapses are GeNN's (generateUpdate).  Random numbers: a
         // counter-based generator per row and call (key = the model's seed, stream 6000 + the update's place in the model's
         // name-ordered list; the reference keeps a generator state per row in memory, backendSIMT.cc:1273-1305)
-        std::ostringstream ccBody, ccArgs, ccParams, ccRemap;
+        std::ostringstream ccBody, ccRemap;
+        KernelArgs ccArgs("gennmiCustomConnectivityUpdate" + name + "Kernel");
         BlockTable ccTable;
         {
             CodeStream body(ccBody);
@@ -1320,8 +1377,7 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
                         for(size_t b = 0; b < blocks; b++) { ccTable.add(g, b * 256, b, blocks); }
                     }
                     const std::string structArray = "mergedCustomConnectivityUpdateGroup" + std::to_string(c.getIndex());
-                    ccArgs << ", d_" << structArray;
-                    ccParams << ", const MergedCustomConnectivityUpdateGroup" << c.getIndex() << " *" << structArray;
+                    ccArgs.add("MergedCustomConnectivityUpdateGroup" + std::to_string(c.getIndex()), structArray);
                     funcEnv.getStream() << "// merged custom connectivity update group " << c.getIndex() << std::endl;
                     funcEnv.getStream() << (firstBlock == 0 ? "if" : "else if") << "(blockIdx.x < " << ccTable.numBlocks << "u)";
                     CodeStream::Scope b(funcEnv.getStream());
@@ -1380,76 +1436,91 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         }
 
         // ---- kernels and the host function of this update group
-        const std::string signature = "(" + timeType + " t";
+        const std::string seed = (model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull") : std::string("gennmiRandomSeed()");
+        // (a kernel's place in the program is looked up once, when the device copies of the struct arrays are first uploaded)
+        auto declare = [&](const KernelArgs &k)
+        {
+            k.define(argsDefs);
+            kernelIdStream << "static uint32_t " << k.name << "Id = 0;" << std::endl;
+            lookup << "GENNMI_CHECK(gennmi_program_get_kernel(gennmiProgram, module, \"" << k.name << "\", &" << k.name << "Id));" << std::endl;
+        };
+        auto launch = [&](const KernelArgs &k, size_t gridX, size_t gridY, const std::string &seedExpr, const std::string &step, int timer)
+        {
+            CodeStream::Scope b(host);
+            host << k.fillBlock("nullptr", seedExpr) << std::endl;
+            host << "GENNMI_CHECK(gennmi_program_launch(gennmiProgram, " << k.name << "Id, " << gridX << "u, " << gridY << "u, 256u, &a, sizeof(a), (double)t, " << step << ", " << timer << "));" << std::endl;
+        };
         if(neuronTable.numBlocks > 0) {
+            declare(neuronArgs);
             device << "__device__ const gennmi_kernel::BlockEntry gennmiCustomUpdate" << name << "Blocks[] = {" << std::endl << neuronTable.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
-            device << "__global__ __launch_bounds__(256) void gennmiCustomUpdate" << name << "Kernel" << signature << neuronParams.str() << ")";
-            CodeStream::Scope b(device);
+            neuronArgs.open(device, timeType);
             device << neuronBody.str();
+            neuronArgs.close(device);
         }
         if(wuBlocks > 0) {
+            declare(wuArgs);
             device << wuTables.str();
-            device << "__global__ __launch_bounds__(256) void gennmiCustomUpdateWU" << name << "Kernel" << signature << wuParams.str() << ")";
-            CodeStream::Scope b(device);
+            wuArgs.open(device, timeType);
             device << wuBody.str();
+            wuArgs.close(device);
         }
         if(ccTable.numBlocks > 0) {
+            declare(ccArgs);
             device << "__device__ const gennmi_kernel::BlockEntry gennmiCustomConnectivityUpdate" << name << "Blocks[] = {" << std::endl << ccTable.entries.str() << "{0u, 0u, 0u, 0u}};" << std::endl;
-            device << "__global__ __launch_bounds__(256) void gennmiCustomConnectivityUpdate" << name << "Kernel" << signature << ", unsigned long long gennmiSeed, unsigned long long gennmiStep" << ccParams.str() << ")";
-            CodeStream::Scope b(device);
+            ccArgs.open(device, timeType);
             device << ccBody.str();
+            ccArgs.close(device);
         }
         if(trBlocks > 0) {
+            declare(trArgs);
             device << trTables.str();
-            device << "__global__ __launch_bounds__(256) void gennmiCustomUpdateTranspose" << name << "Kernel" << signature << trParams.str() << ")";
-            CodeStream::Scope b(device);
+            trArgs.open(device, timeType);
             device << "__shared__ " << model.getPrecision().getName() << " gennmiTile[64][65];" << std::endl;
             device << trBody.str();
+            trArgs.close(device);
         }
         host << "void update" << name << "(unsigned long long timestep)";
         {
             CodeStream::Scope b(host);
             host << "gennmiEnsureFinalised();" << std::endl;
-            // (beside the library's kernels: steps still queued run first; the launches below go to the null stream, which is
-            // ordered against the runner's stream in both directions)
-            if(!m_GeneratedKernels) { host << "GENNMI_CHECK(gennmi_flush());" << std::endl; }
+            // (every launch below first runs the steps still noted — the library's queue and the program's — and goes to the
+            // stream the step's kernels use)
             host << "const " << timeType << " t = timestep * " << Type::writeNumeric(model.getDT(), model.getTimePrecision()) << ";" << std::endl;
-            const std::string grid = ", " + std::to_string(batchSize) + "), dim3(256), 0, 0>>>(t";
             const bool timing = model.isTimingEnabled();
-            if(timing) { host << "hipEventRecord(customUpdate" << name << "Start, 0);" << std::endl; }
+            const int timer = timing ? timerId("customUpdate" + name) : -1, transposeTimer = timing ? timerId("customUpdate" + name + "Transpose") : -1;
             host << ccHost.str();
             if(ccTable.numBlocks > 0) {
                 // (connectivity first, like the reference: single_threaded_cpu/backend.cc:824-860; the generator's step counts this group's calls)
                 host << "static unsigned long long gennmiCalls = 0;" << std::endl;
-                host << "gennmiCustomConnectivityUpdate" << name << "Kernel<<<dim3(" << ccTable.numBlocks << ", 1), dim3(256), 0, 0>>>(t, "
-                     << ((model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull") : std::string("gennmiRandomSeed()")) << ", gennmiCalls++" << ccArgs.str() << ");" << std::endl;
+                launch(ccArgs, ccTable.numBlocks, 1, seed, "gennmiCalls++", timer);
                 host << ccRemap.str();
             }
-            if(neuronTable.numBlocks > 0) { host << "gennmiCustomUpdate" << name << "Kernel<<<dim3(" << neuronTable.numBlocks << grid << neuronArgs.str() << ");" << std::endl; }
-            if(wuBlocks > 0) { host << "gennmiCustomUpdateWU" << name << "Kernel<<<dim3(" << wuBlocks << grid << wuArgs.str() << ");" << std::endl; }
-            if(timing) { host << "hipEventRecord(customUpdate" << name << "Stop, 0);" << std::endl << "hipEventRecord(customUpdate" << name << "TransposeStart, 0);" << std::endl; }
-            if(trBlocks > 0) { host << "gennmiCustomUpdateTranspose" << name << "Kernel<<<dim3(" << trBlocks << grid << trArgs.str() << ");" << std::endl; }
-            if(timing) { host << "hipEventRecord(customUpdate" << name << "TransposeStop, 0);" << std::endl; }
-            host << "if(hipGetLastError() != hipSuccess) { throw std::runtime_error(\"update" << name << ": kernel launch failed\"); }" << std::endl;
+            if(neuronTable.numBlocks > 0) { launch(neuronArgs, neuronTable.numBlocks, batchSize, "0ull", "0ull", timer); }
+            if(wuBlocks > 0) { launch(wuArgs, wuBlocks, batchSize, "0ull", "0ull", timer); }
+            if(trBlocks > 0) { launch(trArgs, trBlocks, batchSize, "0ull", "0ull", transposeTimer); }
             host << notes.str();
             if(timing) {
                 // (these counters are not part of stepTime: read here, after the group's kernels have finished, backendCUDAHIP.cc:826-856)
-                host << "GENNMI_CHECK(gennmi_synchronize());" << std::endl;
-                host << "float tmp = 0.0f;" << std::endl;
-                host << "if(hipEventElapsedTime(&tmp, customUpdate" << name << "Start, customUpdate" << name << "Stop) == hipSuccess) { customUpdate" << name << "Time += tmp / 1000.0; }" << std::endl;
-                host << "if(hipEventElapsedTime(&tmp, customUpdate" << name << "TransposeStart, customUpdate" << name << "TransposeStop) == hipSuccess) { customUpdate" << name << "TransposeTime += tmp / 1000.0; }" << std::endl;
+                host << "GENNMI_CHECK(gennmi_program_get_time(gennmiProgram, " << timer << ", &customUpdate" << name << "Time));" << std::endl;
+                host << "GENNMI_CHECK(gennmi_program_get_time(gennmiProgram, " << transposeTimer << ", &customUpdate" << name << "TransposeTime));" << std::endl;
             }
         }
         host << std::endl;
     }
 
-    // struct definitions, host arrays and push functions (GeNN's own), then the device copies
+    // struct definitions (both passes), then the kernels (device pass) or the host arrays, push functions and update functions (host pass)
+    if(!deviceStream.str().empty()) { os << "#define GENNMI_DEVICE_MODULE 1      // the Makefile builds a gfx950 code object from this file as well" << std::endl; }
     modelMerged.genMergedCustomUpdateStructs(os, *this);
     modelMerged.genMergedCustomUpdateWUStructs(os, *this);
     modelMerged.genMergedCustomUpdateTransposeWUStructs(os, *this);
     modelMerged.genMergedCustomConnectivityUpdateStructs(os, *this);
     modelMerged.genMergedCustomConnectivityRemapUpdateStructs(os, *this);
     modelMerged.genMergedCustomConnectivityHostUpdateStructs(os, *this);
+    os << argsStream.str();
+    os << std::endl;
+    os << "#ifdef __HIPCC__" << std::endl;
+    os << deviceStream.str();
+    os << "#else" << std::endl;
     modelMerged.genMergedCustomConnectivityHostUpdateStructArrayPush(os, *this);
     modelMerged.genMergedCustomConnectivityUpdateHostStructArrayPush(os, *this);
     modelMerged.genMergedCustomConnectivityRemapUpdateHostStructArrayPush(os, *this);
@@ -1457,20 +1528,38 @@ void Backend::genCustomUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     modelMerged.genMergedCustomUpdateWUHostStructArrayPush(os, *this);
     modelMerged.genMergedCustomUpdateTransposeWUHostStructArrayPush(os, *this);
     preambleHandler(os);
-    for(const auto &g : modelMerged.getMergedCustomUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "CustomUpdate"); }
-    for(const auto &g : modelMerged.getMergedCustomUpdateWUGroups()) { genDeviceStructArray(decl, upload, *this, g, "CustomUpdateWU"); }
-    for(const auto &g : modelMerged.getMergedCustomUpdateTransposeWUGroups()) { genDeviceStructArray(decl, upload, *this, g, "CustomUpdateTransposeWU"); }
-    for(const auto &g : modelMerged.getMergedCustomConnectivityUpdateGroups()) { genDeviceStructArray(decl, upload, *this, g, "CustomConnectivityUpdate"); }
+    for(const auto &g : modelMerged.getMergedCustomUpdateGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "CustomUpdate"); }
+    for(const auto &g : modelMerged.getMergedCustomUpdateWUGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "CustomUpdateWU"); }
+    for(const auto &g : modelMerged.getMergedCustomUpdateTransposeWUGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "CustomUpdateTransposeWU"); }
+    for(const auto &g : modelMerged.getMergedCustomConnectivityUpdateGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "CustomConnectivityUpdate"); }
     os << declStream.str();
+    os << kernelIdStream.str();
+    os << "static bool gennmiCustomUpdateKernelsLoaded = false;" << std::endl;
+    os << "extern \"C\" const unsigned char gennmi_customUpdate_image[];" << std::endl;
+    os << "extern \"C\" const unsigned char gennmi_customUpdate_image_end[];" << std::endl;
     os << std::endl;
     os << "void gennmiUploadCustomUpdateGroups()";
     {
         CodeStream::Scope b(os);
         os << uploadStream.str();
+        if(!lookupStream.str().empty()) {
+            os << "if(!gennmiCustomUpdateKernelsLoaded)";
+            CodeStream::Scope b2(os);
+            os << "uint32_t module = 0;" << std::endl;
+            os << "GENNMI_CHECK(gennmi_program_load_module(gennmiProgram, gennmi_customUpdate_image, (size_t)(gennmi_customUpdate_image_end - gennmi_customUpdate_image), &module));" << std::endl;
+            os << lookupStream.str();
+            os << "gennmiCustomUpdateKernelsLoaded = true;" << std::endl;
+        }
     }
     os << std::endl;
-    os << deviceStream.str();
+    os << "void gennmiFreeCustomUpdateGroups()";
+    {
+        CodeStream::Scope b(os);
+        os << "gennmiCustomUpdateKernelsLoaded = false;" << std::endl;
+        os << releaseStream.str();
+    }
     os << std::endl;
     os << hostStream.str();
+    os << "#endif" << std::endl;
 }
 }   // namespace GeNN::CodeGenerator::MI355X

@@ -167,8 +167,11 @@ static void noteDeviceWrite(const void *dev, size_t bytes)
 // route first executes what is queued (flushQueuedSteps), and so does the queue reaching its limit.
 static std::atomic<int> g_queuedRunners{0};
 static int flushRunner(gennmi_runner *r);
+static int flushPrograms();             // the noted calls of programs (generated kernels), genn_mi355x_program.h
+static int checkPrograms();
 static int flushQueuedSteps()
 {
+    { const int rc = flushPrograms(); if(rc) { return rc; } }
     if(g_queuedRunners.load(std::memory_order_relaxed) == 0) { return GENNMI_OK; }
     std::vector<gennmi_runner*> runners;
     {
@@ -231,7 +234,12 @@ int gennmi_memcpy_to_device(void *dev, const void *host, size_t bytes)
     noteDeviceWrite(dev, bytes);
     return GENNMI_OK;
 }
-int gennmi_memcpy_from_device(void *host, const void *dev, size_t bytes) { FLUSH_QUEUED(); HIP_TRY(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost)); return GENNMI_OK; }
+int gennmi_memcpy_from_device(void *host, const void *dev, size_t bytes)
+{
+    FLUSH_QUEUED();
+    HIP_TRY(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost));
+    return checkPrograms();         // (the copy waited for every program's stream: their error flags are in host memory)
+}
 int gennmi_note_device_write(const void *dev, size_t bytes)
 {
     FLUSH_QUEUED();
@@ -270,7 +278,7 @@ int gennmi_copy_f32(float *dst, const float *src, size_t count)
     }
     return GENNMI_OK;
 }
-int gennmi_synchronize(void) { FLUSH_QUEUED(); HIP_TRY(hipDeviceSynchronize()); return GENNMI_OK; }
+int gennmi_synchronize(void) { FLUSH_QUEUED(); HIP_TRY(hipDeviceSynchronize()); return checkPrograms(); }
 int gennmi_flush(void) { FLUSH_QUEUED(); return GENNMI_OK; }
 
 // ---- host mirrors: host buffer <-> device buffer pairs, for callers whose generated code only knows host pointers
@@ -2028,3 +2036,6 @@ int gennmi_build_remap(uint32_t numSrc, uint32_t numTrg, uint32_t rowStride, uin
 }
 
 }   // extern "C"
+
+// generated code objects behind the C ABI: gennmi_program_*
+#include "genn_mi355x_program.h"

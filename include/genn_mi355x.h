@@ -424,6 +424,78 @@ int gennmi_runner_get_info(gennmi_runner *runner, uint32_t info[4]);
 /* Synaptic events processed so far, summed over presynaptic groups (device counter). */
 int gennmi_runner_event_count(gennmi_runner *runner, unsigned long long *events);
 
+
+/* ---------------------------------------------------------------------------------------------
+ * Generated kernels behind this boundary.  For model code the device library does not implement, the backend
+ * generates gfx950 device code (one code object per module of the runner, built with `hipcc --genco` and embedded in
+ * the module's object file); the runner itself stays host C++ and loads and launches that code through the calls
+ * below.  This is what inline `kernel<<<grid, block, 0, stream>>>(...)` launches, hipEventRecord pairs and
+ * hipGetLastError checks are in the reference's generated runner (src/genn/genn/code_generator/backendCUDAHIP.cc:386-420
+ * genNeuronUpdate, :548-589 genSynapseUpdate, :750-856 genCustomUpdate, :1479-1504 genTimer).
+ *
+ * A program owns a stream (the runner's, when it is created beside one), the code objects, a device error flag that
+ * its kernels raise when a bounded wait expires, timers, and the sequence of launches that makes up each phase of a
+ * timestep (GENNMI_PHASE_SYNAPSES = updateSynapses, GENNMI_PHASE_NEURONS = updateNeurons).  Every kernel takes a
+ * gennmi_launch_header_t as its first argument and the launch's own argument block as its second; the header tells it
+ * where the values of its step are: in `inlineEntry` (steps[] == NULL: a launch made when it was asked for) or in
+ * steps[k] (device memory: a launch replayed from a captured HIP graph, whose arguments cannot change from replay to
+ * replay).  With stepQueueLength > 0 gennmi_program_update() only notes the call; noted calls run, from a graph of the
+ * whole queue when it is full and the phases came in the order the graph was captured for, before anything can observe
+ * the difference (every entry point of this library that reads, writes or frees device memory, synchronises or
+ * launches by another route executes them first).
+ * ------------------------------------------------------------------------------------------- */
+typedef struct gennmi_program gennmi_program;
+typedef struct gennmi_step_entry
+{
+    double t;                       /* simulation time of the step (converted to the model's time type in the kernel) */
+    unsigned long long step;        /* calls of this phase so far: the step counter of counter-based random numbers */
+    uint32_t recordingTimestep;     /* row of the recording buffers */
+    uint32_t tag;                   /* differs from one call of a phase to the next and is never 0 (tagged look-back words) */
+} gennmi_step_entry_t;
+typedef struct gennmi_launch_header
+{
+    const gennmi_step_entry_t *steps;   /* device table of the queued calls, or NULL */
+    uint32_t k;                         /* index into steps */
+    uint32_t spinLimit;                 /* polls a work-group waits for another one before it raises the error flag */
+    gennmi_step_entry_t inlineEntry;    /* used when steps == NULL */
+} gennmi_launch_header_t;
+enum { GENNMI_PHASE_SYNAPSES = 0, GENNMI_PHASE_NEURONS = 1, GENNMI_NUM_PHASES = 2 };
+#define GENNMI_MAX_LAUNCH_ARG_BYTES 3072u
+#define GENNMI_MAX_TIMERS 64
+
+/* `runner` may be NULL (a model whose step runs on generated kernels only); otherwise the program shares the runner's
+ * stream, so that its launches are ordered against the runner's.  stepQueueLength = 0: every call launches at once. */
+int gennmi_program_create(gennmi_program **program, gennmi_runner *runner, uint32_t stepQueueLength);
+int gennmi_program_destroy(gennmi_program *program);
+/* hipModuleLoadData / hipModuleGetFunction: `image` is a gfx950 code object in host memory (it is copied) */
+int gennmi_program_load_module(gennmi_program *program, const void *image, size_t bytes, uint32_t *module);
+int gennmi_program_get_kernel(gennmi_program *program, uint32_t module, const char *name, uint32_t *kernel);
+/* the device word the program's kernels raise (atomicOr) when a bounded wait expires; reported as GENNMI_EDEVICE by
+ * gennmi_program_synchronize and by the next gennmi_synchronize / gennmi_memcpy_from_device that follows the launches */
+int gennmi_program_error_flag(gennmi_program *program, uint32_t **deviceFlag);
+/* Appends a launch to a phase's sequence: kernel<<<dim3(gridX, gridY), dim3(blockX), 0, stream>>>(header, args).
+ * `args` (argBytes <= GENNMI_MAX_LAUNCH_ARG_BYTES, 8-byte aligned layout) is copied.  `timer` (0 ..
+ * GENNMI_MAX_TIMERS-1, or -1) names the timer that accumulates the launch's duration while timing is enabled.
+ * gennmi_program_clear_phases forgets every sequence (and the captured graph). */
+int gennmi_program_add_launch(gennmi_program *program, int phase, uint32_t kernel, uint32_t gridX, uint32_t gridY, uint32_t blockX,
+                              const void *args, size_t argBytes, int timer);
+int gennmi_program_clear_phases(gennmi_program *program);
+/* updateSynapses(t) / updateNeurons(t, recordingTimestep) of a runner on generated kernels: runs (or notes) the
+ * phase's launches.  Replaces the launch sequences of backendCUDAHIP.cc:386-420 and :548-589. */
+int gennmi_program_update(gennmi_program *program, int phase, double t, uint32_t recordingTimestep);
+/* One launch now, after everything noted has run (custom updates: update<Group>(), backendCUDAHIP.cc:750-856).
+ * `step`: the counter handed to the kernel in its header's inlineEntry. */
+int gennmi_program_launch(gennmi_program *program, uint32_t kernel, uint32_t gridX, uint32_t gridY, uint32_t blockX,
+                          const void *args, size_t argBytes, double t, unsigned long long step, int timer);
+/* blocks until the program's stream is idle; GENNMI_EDEVICE if a kernel raised the error flag */
+int gennmi_program_synchronize(gennmi_program *program);
+/* Timers (genTimer, backendCUDAHIP.cc:1479-1504): while enabled, nothing is queued or replayed from a graph and every
+ * launch has a HIP event pair around it; get_time returns the seconds accumulated by a timer since creation. */
+int gennmi_program_set_timing(gennmi_program *program, int enabled);
+int gennmi_program_get_time(gennmi_program *program, int timer, double *seconds);
+/* info = {calls of gennmi_program_update executed so far, of which replayed from a captured graph, launches made, graphs captured} */
+int gennmi_program_get_info(gennmi_program *program, unsigned long long info[4]);
+
 #ifdef __cplusplus
 }
 #endif

@@ -20,11 +20,19 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "genn_mi355x.h"        // gennmi_launch_header_t: the first argument of every generated kernel
+
 namespace gennmi_kernel
 {
 constexpr int BLOCK = 256;
 constexpr int WAVE = 64;
-constexpr uint32_t SPIN_LIMIT = 1u << 22;       // polls a work-group waits for another one before it gives up
+
+// the values of the step a launch belongs to: by value in the header (a launch made when it was asked for) or in a device
+// table (a launch replayed from a captured graph, whose arguments are the same at every replay)
+__device__ inline gennmi_step_entry_t stepEntry(const gennmi_launch_header_t &header)
+{
+    return header.steps ? header.steps[header.k] : header.inlineEntry;
+}
 
 struct BlockEntry
 {
@@ -45,9 +53,11 @@ struct QueueSlot
 
 // Position of every firing lane in its population's queue.  All threads of the work-group call this, once per launch
 // and population; `counts` / `groupTotals` hold one 64-bit word per work-group of the launch, tagged with `tag` (a value
-// that differs from launch to launch and is never 0), so nothing is ever cleared.
+// that differs from launch to launch and is never 0), so nothing is ever cleared.  A work-group polls another one's word at
+// most `spinLimit` times; then it raises the error flag and leaves (slot.ok == false) instead of hanging.
 __device__ inline QueueSlot orderedSlot(bool flag, uint32_t localBlock, uint32_t numBlocks, size_t aggBase,
-                                        unsigned long long *counts, unsigned long long *groupTotals, uint32_t tag, uint32_t *errorFlag)
+                                        unsigned long long *counts, unsigned long long *groupTotals, uint32_t tag, uint32_t *errorFlag,
+                                        uint32_t spinLimit)
 {
     __shared__ uint32_t shCount[BLOCK / WAVE];
     __shared__ uint32_t shOffset;
@@ -81,7 +91,7 @@ __device__ inline QueueSlot orderedSlot(bool flag, uint32_t localBlock, uint32_t
             while(true) {
                 const unsigned long long a = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if((uint32_t)(a >> 32) == tag) { return (uint32_t)a; }
-                if(++spins > SPIN_LIMIT) { ok = false; return 0u; }
+                if(++spins > spinLimit) { ok = false; return 0u; }
                 __builtin_amdgcn_s_sleep(1);
             }
         };

@@ -145,6 +145,25 @@ def test_dynamic_parameters_are_refused(dynamic, case):
         shutil.rmtree(tmp, ignore_errors=True)
 
 
+def _assert_host_passes_hold_no_hip(code):
+    """What the host compiler sees of a generated runner — every module outside its `#ifdef __HIPCC__` section — holds no
+    launch syntax, no HIP call and no HIP header: device code is reached through the device library's C ABI only.  The
+    objects were in fact built that way: the host pass is $(CXX), the device pass `hipcc --genco`."""
+    import re
+    for name in sorted(os.listdir(code)):
+        if not name.endswith((".cc", ".h")):
+            continue
+        text = open(os.path.join(code, name)).read()
+        host = re.sub(r"#ifdef __HIPCC__.*?(#else|#endif)", "", text, flags=re.S)
+        assert "<<<" not in host, name
+        assert not re.search(r"\bhip[A-Z]\w*\s*\(", host), (name, re.search(r"\bhip[A-Z]\w*\s*\(", host))
+        assert "hip_runtime" not in host, name
+    makefile = open(os.path.join(code, "Makefile")).read()
+    assert "$(CXX) $(CXXFLAGS) -MF" in makefile and "$(HIPCC) $(HIPCCFLAGS)" in makefile and "CXX :=" not in makefile
+    undefined = subprocess.run(["nm", "-D", "--undefined-only", os.path.join(code, "librunner.so")], stdout=subprocess.PIPE, text=True, check=True).stdout
+    assert "gennmi_program_update" in undefined and not re.search(r"\bhip[A-Z]", undefined), undefined
+
+
 def _generate_with(case, *options):
     if case == "procedural":        # (no fixture: nothing in the reference's CPU backend regenerates matrices)
         from genn_amd import configs
@@ -164,9 +183,10 @@ def _generate_with(case, *options):
 @pytest.mark.parametrize("case, options", [("custom_update_small", ("--kernels=generated",)), ("va_double_small", ()), ("post_events_small", ()), ("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("conv_small", ("--kernels=generated",)), ("procedural", ("--kernels=generated",)), ("dense_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
                                            ("va_small", ("--dynamic=neuron:E.Ioffset",))])
 def test_generated_kernels_are_chosen_and_build(case, options):
-    """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the runner then holds device
-    code (the model's snippets inside this backend's kernel skeletons), built for gfx950 by the runner's own Makefile, with
-    the reference's entry points around it."""
+    """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the modules then hold device
+    code (the model's snippets inside this backend's kernel skeletons), built into gfx950 code objects by the runner's own
+    Makefile and embedded in the modules' objects; the runner itself is host C++ that launches them through the device
+    library's C ABI, with the reference's entry points around it."""
     net, tmp, code, res = _generate_with(case, *options)
     try:
         assert res.returncode == 0, res.stdout[-3000:]
@@ -176,7 +196,12 @@ def test_generated_kernels_are_chosen_and_build(case, options):
         assert "__global__" in synapse and "gennmi_kernel::addScalar" in synapse
         assert "gennmi_runner_create" not in open(os.path.join(code, "runner.cc")).read()
         makefile = open(os.path.join(code, "Makefile")).read()
-        assert "hipcc" in makefile and "--offload-arch=gfx950" in makefile and "-packed-fp32-ops" in makefile and "-ffp-contract=off" in makefile
+        assert "hipcc" in makefile and "--genco" in makefile and "--offload-arch=gfx950" in makefile and "-packed-fp32-ops" in makefile and "-ffp-contract=off" in makefile
+        _assert_host_passes_hold_no_hip(code)
+        # a bounded wait of the spike compaction that expires raises the program's error flag, whatever the timing setting:
+        # the kernels get the flag from the library, which reports it from the next call that waits for the device
+        assert "a.error = gennmiProgramError" in neuron and "gennmi_program_error_flag(gennmiProgram, &gennmiProgramError)" in open(os.path.join(code, "runner.cc")).read()
+        assert "gennmiError, gennmiLaunch.spinLimit)" in neuron
         exports = _exports(os.path.join(code, "librunner.so"))
         for name in ("allocateMem", "freeMem", "initialize", "initializeSparse", "stepTime", "updateNeurons", "updateSynapses"):
             assert name in exports
@@ -186,9 +211,9 @@ def test_generated_kernels_are_chosen_and_build(case, options):
             custom = open(os.path.join(code, "customUpdate.cc")).read()
             for group in ("Homeostasis", "Decay", "Reduce"):
                 assert "update" + group in exports
-            assert "gennmiCustomUpdateHomeostasisKernel<<<" in custom and "gennmiCustomUpdateWUDecayKernel<<<" in custom
+            assert "gennmi_program_launch(gennmiProgram, gennmiCustomUpdateHomeostasisKernelId" in custom and "gennmi_program_launch(gennmiProgram, gennmiCustomUpdateWUDecayKernelId" in custom
             # (order within a group as in the reference: per-neuron, per-synapse, transpose)
-            assert custom.index("gennmiCustomUpdateWUDecayKernel<<<") < custom.index("gennmiCustomUpdateTransposeDecayKernel<<<")
+            assert custom.index("gennmi_program_launch(gennmiProgram, gennmiCustomUpdateWUDecayKernelId") < custom.index("gennmi_program_launch(gennmiProgram, gennmiCustomUpdateTransposeDecayKernelId")
             assert "gennmi_kernel::blockReduceSum(_lrsum)" in custom and "gennmi_kernel::blockReduceMax(_lrpeak)" in custom
             assert "gennmi_kernel::groupOfBlock(gennmiCustomUpdateWUDecayStarts" in custom
             assert "group->variableTranspose[" in custom and "gennmiTile[tx][ty + j]" in custom
@@ -218,7 +243,7 @@ def test_generated_kernels_are_chosen_and_build(case, options):
             assert "const unsigned int idPost = " in synapse and "idKernel0" in synapse and "idKernel3" in synapse
         if case == "prev_times_small":
             # previous spike times: a kernel of its own stamps last step's spikes before the update
-            assert "gennmiPrevSpikeTimeKernel<<<" in neuron and neuron.index("gennmiPrevSpikeTimeKernel<<<") < neuron.index("gennmiNeuronUpdateKernel<<<")
+            assert neuron.index('gennmiProgram, module, "gennmiPrevSpikeTimeKernel"') < neuron.index('gennmiProgram, module, "gennmiNeuronUpdateKernel"')
             assert "group->prevST[" in neuron
         if case == "graded_small":
             # spike-like events: a queue per condition, compacted in order like the true spikes and recorded from the ballot
@@ -227,17 +252,17 @@ def test_generated_kernels_are_chosen_and_build(case, options):
         if case == "stdp_delay_small":
             # a learning rule over delay slots: chosen for generated kernels by itself; the populations' ring pointers move on
             # in a kernel of their own before the update, and the queues are read through GeNN's delay-slot helpers
-            assert "gennmiSpikeQueueUpdateKernel<<<" in neuron and neuron.index("gennmiSpikeQueueUpdateKernel<<<") < neuron.index("gennmiNeuronUpdateKernel<<<")
+            assert neuron.index('gennmiProgram, module, "gennmiSpikeQueueUpdateKernel"') < neuron.index('gennmiProgram, module, "gennmiNeuronUpdateKernel"')
             assert "writeDelaySlot" in neuron and "preDelaySlot" in synapse
         if case == "synapse_dynamics_small":
             # code that runs for every synapse every step: a kernel of its own, launched before the presynaptic update
-            assert "gennmiSynapseDynamicsKernel<<<" in synapse and synapse.index("gennmiSynapseDynamicsKernel<<<") < synapse.index("gennmiPresynapticUpdateKernel<<<")
+            assert synapse.index('gennmiProgram, module, "gennmiSynapseDynamicsKernel"') < synapse.index('gennmiProgram, module, "gennmiPresynapticUpdateKernel"')
             assert "group->x[idSyn]" in synapse and "group->Vpre[row]" in synapse
         if case == "poisson_input_small":
             # gennrand_exponential() of the built-in Poisson neuron: a counter-based generator keyed by the model's seed, one
             # stream per population, the step counted by the launcher
             assert "gennmi_kernel::rngBegin(gennmiSeed, (2000u), id, gennmiStep)" in neuron and "gennmi_kernel::rngExponential(gennmiRng)" in neuron
-            assert f"{net.seed}ull, gennmiNeuronStep++" in neuron
+            assert f"a.seed = {net.seed}ull;" in neuron and "const unsigned long long gennmiStep = gennmiEntry.step;" in neuron
         if case in ("dynamic_small", "va_small"):
             # the dynamic parameter is a struct field the kernel reads, with a push function that marks the device copy stale
             assert "group->Ioffset" in neuron
@@ -267,7 +292,7 @@ def test_generated_kernels_take_the_batch_from_the_grid():
         code = os.path.join(work, net.name + "_CODE")
         neuron = open(os.path.join(code, "neuronUpdate.cc")).read()
         synapse = open(os.path.join(code, "synapseUpdate.cc")).read()
-        assert "<<<dim3(" in neuron and ", 2), dim3(256)" in neuron and ", 2), dim3(256)" in synapse
+        assert "u, 2u, 256u, &a, sizeof(a)" in neuron and "u, 2u, 256u, &a, sizeof(a)" in synapse
         assert "group->A[batchOffset + id]" in neuron and "[blockIdx.y] = slot.total" in neuron
         assert "(size_t)recordingTimestep * 2u + blockIdx.y" in neuron
         assert "group->srcSpk[preBatchOffset + spike]" in synapse and "group->wPost[synBatchOffset + idSyn]" in synapse
@@ -291,7 +316,7 @@ def test_custom_updates_take_the_batch_from_the_grid_and_reduce_over_it():
         res = subprocess.run([DRIVER, spec, work, out, "--generate-only"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
         assert res.returncode == 0, res.stdout[-3000:]
         custom = open(os.path.join(work, net.name + "_CODE", "customUpdate.cc")).read()
-        assert "Kernel<<<dim3(" in custom and ", 3), dim3(256)" in custom
+        assert "gennmi_program_launch(gennmiProgram, " in custom and "u, 3u, 256u, &a, sizeof(a)" in custom
         assert "for(unsigned int batch = 0; batch < 3u; batch++)" in custom
         # the per-neuron update and the reduction over neurons run once per batch, the static dense weights once
         assert "group->applied[batchOffset + id]" in custom and "group->sum[blockIdx.y] = _lrsum" in custom
@@ -311,9 +336,9 @@ def test_custom_updates_beside_library_kernels():
         custom = open(os.path.join(code, "customUpdate.cc")).read()
         runner = open(os.path.join(code, "runner.cc")).read()
         assert "__global__" not in neuron and "gennmi_push_neuron_update_group" in neuron and "gennmi_runner_create" in runner
-        assert "__global__" in custom and "gennmiCustomUpdateWUDecayKernel<<<" in custom
+        assert "__global__" in custom and "gennmi_program_launch(gennmiProgram, gennmiCustomUpdateWUDecayKernelId" in custom
         body = custom[custom.index("void updateDecay("):]
-        assert body.index("gennmi_flush()") < body.index("Kernel<<<") < body.index("gennmi_note_mirror_write(")
+        assert body.index("gennmi_program_launch(") < body.index("gennmi_note_mirror_write(")
         # written: the weights both decays refer to and the transpose target; the read-only reference of the reduction is not
         assert "gennmi_note_mirror_write(mergedCustomUpdateTransposeWUGroup0[g].variableTranspose)" in custom
         reduce = custom[custom.index("void updateReduce("):]
@@ -337,11 +362,11 @@ def test_custom_connectivity_updates_generate_and_build():
         assert res.returncode == 0, res.stdout[-3000:]
         assert "__global__" in open(os.path.join(code, "neuronUpdate.cc")).read()
         custom = open(os.path.join(code, "customUpdate.cc")).read()
-        assert "gennmiCustomConnectivityUpdatePruneKernel<<<" in custom and "gennmiCustomConnectivityUpdateSproutKernel<<<" in custom
+        assert "gennmi_program_launch(gennmiProgram, gennmiCustomConnectivityUpdatePruneKernelId" in custom and "gennmi_program_launch(gennmiProgram, gennmiCustomConnectivityUpdateSproutKernelId" in custom
         prune = custom[custom.index("void updatePrune("):]
-        assert prune.index("gennmiCustomConnectivityUpdatePruneKernel<<<") < prune.index("gennmi_build_remap(")
+        assert prune.index("gennmi_program_launch(gennmiProgram, gennmiCustomConnectivityUpdatePruneKernelId") < prune.index("gennmi_build_remap(")
         # host update code first: plain host code over the host buffers, pushed to the device buffers behind them
-        assert "group->limit[_i] = " in prune and prune.index("gennmi_memcpy_to_device(gennmiDev(group->limit), group->limit") < prune.index("Kernel<<<")
+        assert "group->limit[_i] = " in prune and prune.index("gennmi_memcpy_to_device(gennmiDev(group->limit), group->limit") < prune.index("gennmi_program_launch(")
         # the removed synapse's slot takes the row's last one, with the weight and the other custom updates' variables
         assert "group->ind[idx] = group->ind[lastIdx];" in custom and "group->dependentVar0[idx] = group->dependentVar0[lastIdx];" in custom
         assert "group->rowLength[id]--;" in custom and "group->rowLength[id]++;" in custom

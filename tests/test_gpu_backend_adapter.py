@@ -46,11 +46,22 @@ def _run(case, *options):
         os.makedirs(d)
     write_netspec(net, spec)
     print(f"adapter case {case}: running {DRIVER}", flush=True)
-    res = subprocess.run([DRIVER, spec, work, out, *options], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+    res = subprocess.run([DRIVER, spec, work, out, *options], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240,
+                         env=dict(os.environ, GENNMI_PROGRAM_STATS="1"))
     assert res.returncode == 0, res.stdout[-3000:]
     code = os.path.join(work, net.name + "_CODE")
     net.generated_kernels = "__global__" in open(os.path.join(code, "neuronUpdate.cc")).read()
+    net.driver_output = res.stdout
     return net, snap, tmp, out
+
+
+def _program_stats(output):
+    """calls of updateSynapses / updateNeurons executed by the runner's program, how many of them replayed from a captured
+    graph, launches made, graphs captured (printed by the device library when the program is destroyed)"""
+    import re
+    m = re.search(r"gennmi_program: calls (\d+), replayed (\d+), launches (\d+), graphs (\d+)", output)
+    assert m, output[-2000:]
+    return tuple(int(g) for g in m.groups())
 
 
 # cases whose models the device library implements; the others (models of the test driver's own, parameters set while the
@@ -77,6 +88,48 @@ def test_generated_kernels_match_reference_backend(case):
     reference's CPU backend produced for a covered feature (dendritic delay, trace and built-in STDP with learnPost,
     presynaptic output, an array-fed current source) also pins the generated kernels."""
     _compare_with_fixture(case, "--kernels=generated")
+
+
+@pytest.mark.parametrize("case", ["potjans_small", "stdp_small", "custom_small", "stdp_delay_small", "dynamic_small"])
+@pytest.mark.parametrize("queue", [8, 0])
+def test_generated_kernels_replayed_from_a_graph_match_reference_backend(case, queue):
+    """Runtime::stepTime asks for one step at a time; the runner's program notes the calls of updateSynapses / updateNeurons
+    and replays a full queue from a captured graph whose kernels read their step's time, recording row, random-number step and
+    look-back tag from a device table.  With a queue of 8 steps most of a run is replayed (what is left when the driver takes
+    a snapshot is launched call by call); with no queue every call is launched when made.  Either way the fixtures of the
+    reference's CPU backend must be met exactly as with the default queue, replay after replay."""
+    net = _compare_with_fixture(case, "--kernels=generated", f"--step-queue={queue}")
+    calls, replayed, launches, graphs = _program_stats(net.driver_output)
+    assert calls == 2 * net.steps, (calls, net.steps)
+    if queue:
+        assert graphs >= 1 and replayed >= calls // 2 and replayed % (2 * queue) == 0, (calls, replayed, graphs)
+    else:
+        assert graphs == 0 and replayed == 0
+
+
+def test_generated_kernels_report_an_expired_wait():
+    """Failure path of the generated spike compaction, forced from the host (a wait bound of zero polls): the work-group that
+    finds another one's count not yet published raises the program's error flag and leaves, every kernel ends normally, and
+    the next call that waits for the device — here the driver's first pull — reports it, whatever the model's timing setting
+    (timing is off here).  The run must fail with that message instead of going on with undefined spike queues."""
+    from genn_amd import configs
+    net = configs.potjans(neuron_scale=0.05, connectivity_scale=0.2, steps=200)
+    net.snap = 100
+    tmp = tempfile.mkdtemp(prefix="adapter_expired_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(net, spec)
+        print("adapter: generated kernels with a wait bound of zero", flush=True)
+        res = subprocess.run([DRIVER, spec, work, out, "--kernels=generated"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240,
+                             env=dict(os.environ, GENNMI_SPIN_LIMIT="0"))
+        assert res.returncode != 0 and "bounded wait" in res.stdout, res.stdout[-3000:]
+        print("adapter: the same run with the default bound", flush=True)
+        res = subprocess.run([DRIVER, spec, work, out, "--kernels=generated"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+        assert res.returncode == 0, res.stdout[-3000:]
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
 
 
 def _compare_with_fixture(case, *options):
@@ -187,6 +240,7 @@ def _compare_with_fixture(case, *options):
                 _close(got, want, key, accumulator=True)
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+    return net
 
 
 def test_adapter_full_size_microcircuit_first_100ms():

@@ -1,0 +1,179 @@
+"""GPU parity over the FULL run of every benchmark configuration at its published size.
+
+Beyond the first 100 ms a free-running network may part from the CPU oracle once the order of fp32 atomic additions
+flips a threshold crossing, so the bar over the whole run is statistical (the configuration's own statement): every
+population's firing rate within 2 % of the oracle's, the number of synaptic events delivered within 2 %, and — for the
+plastic network — the distribution of the learnt weights (mean, variance, fraction at either clipping bound) within
+the tolerances written below.  Each test also reports up to which step the rasters were identical.
+(The microcircuit's full run is in test_gpu_full_size.py.)
+"""
+import copy
+
+import numpy as np
+import pytest
+
+from genn_amd import configs
+from genn_amd.genn_model import model_from_net
+from oracle.genn_cpu import OracleNet
+
+pytestmark = pytest.mark.gpu
+
+RATE_TOL = 0.02         # relative, per population, over the full run
+EVENT_TOL = 0.02        # relative, synaptic events delivered over the full run
+
+
+def _bits(words, n, steps):
+    w = (n + 31) // 32
+    return np.unpackbits(np.ascontiguousarray(words).view(np.uint8).reshape(steps, w * 4), axis=1, bitorder="little")[:, :n]
+
+
+def _compare_rates(net, model, oracle, steps, min_spikes_per_neuron=0.05):
+    """Returns the first step at which any raster differs (``steps`` if none does)."""
+    identical_until = steps
+    for p in net.pops:
+        got = _bits(model.neuron_populations[p.name].vars["recordSpk"].view, p.n, steps)
+        want = _bits(oracle.record(p.name, steps), p.n, steps)
+        diff = np.nonzero((got != want).any(axis=1))[0]
+        if len(diff):
+            identical_until = min(identical_until, int(diff[0]))
+        rate_got, rate_want = got.sum() / p.n, want.sum() / p.n          # spikes per neuron over the run
+        assert rate_want > min_spikes_per_neuron, f"{p.name} is (nearly) silent in the oracle: {rate_want:.4f} spikes per neuron"
+        assert abs(rate_got - rate_want) <= RATE_TOL * rate_want, f"{p.name}: {rate_got:.4f} vs {rate_want:.4f} spikes per neuron"
+    return identical_until
+
+
+def _full_run(net, steps, col_stride_of=()):
+    model = model_from_net(net)
+    model.load(num_recording_timesteps=steps)
+    col_stride = {name: model.synapse_populations[name].col_stride for name in col_stride_of} or None
+    oracle = OracleNet(net, num_recording_timesteps=steps, col_stride=col_stride)
+    model.run(steps)
+    oracle.run(steps)
+    model.pull_recording_buffers_from_device()
+    return model, oracle
+
+
+def test_balanced_lif_full_run():
+    """Config 1: 4,000 LIF neurons, dt 0.1 ms, 10,000 steps (1 s simulated)."""
+    steps = 10000
+    net = configs.vogels_abbott(steps=steps)
+    assert sum(p.n for p in net.pops) == 4000
+    model, oracle = _full_run(net, steps)
+    identical_until = _compare_rates(net, model, oracle, steps)
+    assert identical_until >= 1000, f"rasters differ from step {identical_until}"
+    assert abs(model.synaptic_event_count - oracle.events()) <= EVENT_TOL * oracle.events()
+    print(f"config 1: rasters identical for the first {identical_until} of {steps} steps")
+    model.unload()
+
+
+def test_izhikevich_full_run():
+    """Config 3: 10^6 Izhikevich neurons, 10^9 synapses, dt 1 ms, 1,000 steps (1 s simulated), one row of the noise array
+    per step.  Activity is a sequence of population bursts; excitatory and inhibitory rows are rated separately."""
+    steps = 1000
+    net = configs.izhikevich_fanout(steps=steps)
+    n = net.pops[0].n
+    assert n == 1_000_000 and int(net.syns[0].row_length.sum()) == 1_000_000_000 and net.css[0].noise.shape[0] == steps
+    model, oracle = _full_run(net, steps)
+    got = _bits(model.neuron_populations["N"].vars["recordSpk"].view, n, steps)
+    want = _bits(oracle.record("N", steps), n, steps)
+    diff = np.nonzero((got != want).any(axis=1))[0]
+    identical_until = int(diff[0]) if len(diff) else steps
+    assert identical_until >= 50, f"rasters differ from step {identical_until}"
+    n_e = (n * 4) // 5
+    for name, sl in (("excitatory", slice(0, n_e)), ("inhibitory", slice(n_e, n))):
+        rate_got, rate_want = got[:, sl].sum() / (sl.stop - sl.start), want[:, sl].sum() / (sl.stop - sl.start)
+        assert rate_want > 1.0, f"{name} neurons are silent in the oracle"
+        assert abs(rate_got - rate_want) <= RATE_TOL * rate_want, f"{name}: {rate_got:.3f} Hz vs {rate_want:.3f} Hz"
+    assert abs(model.synaptic_event_count - oracle.events()) <= EVENT_TOL * oracle.events()
+    print(f"config 3: rasters identical for the first {identical_until} of {steps} steps; "
+          f"{got.sum() / n:.3f} Hz vs {want.sum() / n:.3f} Hz")
+    model.unload()
+
+
+def test_plastic_stdp_full_run():
+    """Config 4: 100,000 LIF neurons, trace STDP on 80k -> 80k, dt 1 ms, 10,000 steps (10 s simulated): rates and events as
+    everywhere, and the learnt weights after ten seconds — mean within 1 %, variance within 3 %, fraction of synapses at
+    each clipping bound within 0.01 of the oracle's (absolute; the fraction at a bound is a tail of the distribution and moves
+    with the burst times once the free-running rasters have parted: 0.0394 against 0.0456 at the lower bound when measured)."""
+    steps = 10000
+    net = configs.plastic_stdp(steps=steps)
+    assert sum(p.n for p in net.pops if p.model != "ssa") == 100_000
+    model, oracle = _full_run(net, steps, col_stride_of=("EE",))
+    identical_until = _compare_rates(net, model, oracle, steps)
+    assert identical_until >= 100, f"rasters differ from step {identical_until}"
+    assert abs(model.synaptic_event_count - oracle.events()) <= EVENT_TOL * oracle.events()
+    sg = model.synapse_populations["EE"]
+    syn = net.syn("EE") if hasattr(net, "syn") else [s for s in net.syns if s.name == "EE"][0]
+    mask = (np.arange(syn.row_stride)[None, :] < syn.row_length[:, None]).ravel()
+    got = sg.vars["g"].pull_from_device().ravel()[mask].astype(np.float64)
+    want = oracle.syn_g("EE").ravel()[mask].astype(np.float64)
+    g0 = np.asarray(syn.g).ravel()[mask].astype(np.float64)
+    assert np.abs(want - g0).mean() > 1e-3, "the oracle's weights did not learn"
+    print(f"config 4: rasters identical for the first {identical_until} of {steps} steps; mean {got.mean():.6f} / {want.mean():.6f}, "
+          f"variance {got.var():.6f} / {want.var():.6f}, at 0: {(got == 0).mean():.5f} / {(want == 0).mean():.5f}, "
+          f"at 1: {(got == 1).mean():.5f} / {(want == 1).mean():.5f}", flush=True)
+    assert abs(got.mean() - want.mean()) <= 0.01 * abs(want.mean()), f"mean weight {got.mean():.6f} vs {want.mean():.6f}"
+    assert abs(got.var() - want.var()) <= 0.03 * want.var(), f"weight variance {got.var():.6f} vs {want.var():.6f}"
+    for bound in (0.0, 1.0):
+        f_got, f_want = float((got == bound).mean()), float((want == bound).mean())
+        assert abs(f_got - f_want) <= 0.01, f"fraction of weights at {bound}: {f_got:.5f} vs {f_want:.5f}"
+    model.unload()
+
+
+def test_toeplitz_conv_full_run_batch16(monkeypatch):
+    """Config 5: 64x64x16 sources -> 64x64x32 LIF through Conv2D 3x3, batch 16, dt 1 ms, 500 steps: every batch against a
+    batch-1 oracle run fed that batch's input spike trains (the CPU backend has no batches).
+
+    The layer is run twice.  On the event-driven kernels every output element receives its contributions in queue order,
+    the CPU backend's order, so the rasters of all 500 steps must be identical bit for bit.  On the matrix cores (the
+    default for busy steps) the same products are summed in another order, so a neuron whose potential lands within
+    rounding of the threshold may fire a step apart (measured: the first such neuron at step 78 of one batch): rasters
+    identical over the first 50 steps, then every batch's rate within 2 % and the event total within 2 %."""
+    B, steps = 16, 500
+    nets = [configs.conv_toeplitz(steps=steps, batch_index=b) for b in range(B)]
+    times = np.concatenate([n.pop("In").spike_times for n in nets])
+    offs = np.cumsum([0] + [len(n.pop("In").spike_times) for n in nets])
+    start = np.stack([n.pop("In").vars["startSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32)
+    end = np.stack([n.pop("In").vars["endSpike"] + offs[b] for b, n in enumerate(nets)]).astype(np.uint32)
+    batched = copy.deepcopy(nets[0])
+    batched.pop("In").vars = {"startSpike": start, "endSpike": end}
+    batched.pop("In").spike_times = times
+    runs = {}
+    for mode in ("matrix cores", "event-driven"):
+        if mode == "event-driven":
+            monkeypatch.setenv("GENNMI_CONV_MFMA", "0")         # (read when the runner is finalised)
+        model = model_from_net(batched, batch_size=B)
+        model.load(num_recording_timesteps=steps)
+        assert model.runner_info()["conv_on_matrix_cores"] == (mode == "matrix cores")
+        model.run(steps)
+        model.pull_recording_buffers_from_device()
+        runs[mode] = ({name: model.neuron_populations[name].vars["recordSpk"].view.copy() for name in ("In", "Out")}, model.synaptic_event_count)
+        model.unload()
+    identical_until = {mode: steps for mode in runs}
+    flipped = {mode: 0 for mode in runs}
+    events = 0
+    for b, net in enumerate(nets):
+        oracle = OracleNet(net, num_recording_timesteps=steps)
+        oracle.run(steps)
+        events += oracle.events()
+        for name in ("In", "Out"):
+            n = net.pop(name).n
+            words = (n + 31) // 32
+            want = _bits(oracle.record(name, steps), n, steps)
+            rate_want = want.sum() / n
+            assert rate_want > 0.05, f"batch {b}: {name} is silent in the oracle"
+            for mode, (records, _) in runs.items():
+                got = _bits(np.ascontiguousarray(records[name].reshape(steps, B, words)[:, b, :]), n, steps)
+                diff = np.nonzero((got != want).any(axis=1))[0]
+                if len(diff):
+                    identical_until[mode] = min(identical_until[mode], int(diff[0]))
+                    flipped[mode] += int((got != want).sum())
+                rate_got = got.sum() / n
+                assert abs(rate_got - rate_want) <= RATE_TOL * rate_want, f"{mode}, batch {b}, {name}: {rate_got:.4f} vs {rate_want:.4f} spikes per neuron"
+        oracle.close()
+    print(f"config 5: rasters of all {B} batches identical for the first {identical_until['event-driven']} (event-driven kernels) / "
+          f"{identical_until['matrix cores']} (matrix cores, {flipped['matrix cores']} raster bits differ in all) of {steps} steps", flush=True)
+    assert identical_until["event-driven"] == steps, f"event-driven kernels: rasters differ from step {identical_until['event-driven']}"
+    assert identical_until["matrix cores"] >= 50, f"matrix cores: rasters differ from step {identical_until['matrix cores']}"
+    for mode, (_, count) in runs.items():
+        assert abs(count - events) <= EVENT_TOL * events, mode
