@@ -1488,8 +1488,8 @@ void Backend::genRunnerPreamble(CodeStream &os, const ModelSpecMerged&) const
             CodeStream::Scope b(os);
             os << "if(!gennmiStructsDirty) { return; }" << std::endl;
             os << "GENNMI_CHECK(gennmi_synchronize());" << std::endl;
+            os << "gennmiUploadSynapseGroups();" << std::endl;     // (first: the neuron update walks the ring-pointer groups this uploads)
             os << "gennmiUploadNeuronGroups();" << std::endl;
-            os << "gennmiUploadSynapseGroups();" << std::endl;
             os << "gennmiUploadCustomUpdateGroups();" << std::endl;
             os << "gennmiStructsDirty = false;" << std::endl;
             os << "gennmiFinalised = true;" << std::endl;

@@ -72,6 +72,11 @@ struct KernelArgs
         unpack << "const " << type << " *" << structArray << " = gennmiArgs." << structArray << ";" << std::endl;
         fill << "a." << structArray << " = d_" << structArray << "; ";
     }
+    void addWord(const std::string &member, const std::string &hostValue)     // a device word of the launch's own
+    {
+        members << "    uint32_t *" << member << ";" << std::endl;
+        fill << "a." << member << " = " << hostValue << "; ";
+    }
     std::string type() const { return "G" + name.substr(1) + "Args"; }      // gennmiXKernel -> GennmiXKernelArgs
     void define(CodeStream &os) const
     {
@@ -114,13 +119,14 @@ struct KernelArgs
 
 // device copy of a merged group's struct array: declaration, and the statements that translate and upload it
 template<typename G>
-void genDeviceStructArray(CodeStream &decl, CodeStream &upload, CodeStream &release, const BackendBase &backend, const G &g, const std::string &name)
+void genDeviceStructArray(CodeStream &decl, CodeStream &upload, CodeStream &release, const BackendBase &backend, const G &g, const std::string &name,
+                          bool shared = false)
 {
     const std::string type = "Merged" + name + "Group" + std::to_string(g.getIndex());
     const std::string host = "merged" + name + "Group" + std::to_string(g.getIndex());
     const std::string dev = "d_" + host;
     const size_t count = g.getGroups().size();
-    decl << "static " << type << " *" << dev << " = nullptr;" << std::endl;
+    decl << (shared ? "" : "static ") << type << " *" << dev << " = nullptr;" << std::endl;     // (shared: another module's kernel walks the array too)
     release << "if(" << dev << ") { gennmi_free(" << dev << "); " << dev << " = nullptr; }" << std::endl;
     upload << "// " << host << std::endl;
     {
@@ -378,6 +384,32 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             });
     }
 
+    // Dendritic-delay ring pointers: moved on for the next step by the last work-group of this kernel to finish (the reference
+    // launches a one-thread-per-group kernel at the start of updateSynapses, synapseUpdateGroupMerged.cc:480-483; every read of a
+    // pointer in this step lies before its work-group's arrival at the counter, and the next kernel starts after this one ends)
+    std::ostringstream delayStream;
+    bool anyDenDelay = false;
+    {
+        CodeStream delayCode(delayStream);
+        EnvironmentLibrary delayLib(delayCode, StandardLibrary::getMathsFunctions());
+        EnvironmentExternal delayEnv(delayLib);
+        modelMerged.genMergedSynapseDendriticDelayUpdateGroups(
+            *this, memorySpaces,
+            [&](auto &sg)
+            {
+                anyDenDelay = true;
+                const std::string structArray = "mergedSynapseDendriticDelayUpdateGroup" + std::to_string(sg.getIndex());
+                neuronKernel.add("MergedSynapseDendriticDelayUpdateGroup" + std::to_string(sg.getIndex()), structArray);
+                delayEnv.getStream() << "for(unsigned int g = threadIdx.x; g < " << sg.getGroups().size() << "u; g += blockDim.x)";
+                CodeStream::Scope b(delayEnv.getStream());
+                delayEnv.getStream() << "const auto *group = &" << structArray << "[g];" << std::endl;
+                EnvironmentGroupMergedField<SynapseDendriticDelayUpdateGroupMerged> groupEnv(delayEnv, sg);
+                buildStandardEnvironment(groupEnv, 1);
+                sg.generateSynapseUpdate(groupEnv);
+            });
+    }
+    if(anyDenDelay && table.numBlocks > 0) { neuronKernel.addWord("finished", "gennmiNeuronFinished"); }
+
     // struct definitions (both passes), then the host arrays and their push functions (GeNN's own) for the host pass
     const bool timing = model.isTimingEnabled();
     const std::string seed = anyRNG ? ((model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull") : std::string("gennmiRandomSeed()")) : std::string("0ull");
@@ -385,6 +417,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     modelMerged.genMergedNeuronUpdateGroupStructs(os, *this);
     if(anyDelaySlots) { modelMerged.genMergedNeuronSpikeQueueUpdateStructs(os, *this); }
     if(anyPrevTimes) { modelMerged.genMergedNeuronPrevSpikeTimeUpdateStructs(os, *this); }
+    if(anyDenDelay) { modelMerged.genMergedSynapseDendriticDelayUpdateStructs(os, *this); }
     neuronKernel.define(os);
     if(anyDelaySlots) { queueKernel.define(os); }
     if(anyPrevTimes) { prevKernel.define(os); }
@@ -407,6 +440,24 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     os << std::endl;
     neuronKernel.open(os, timeType);
     os << kernelStream.str();
+    if(anyDenDelay && table.numBlocks > 0) {
+        os << "// the last work-group to get here moves the dendritic-delay ring pointers on for the next step" << std::endl;
+        os << "__shared__ bool gennmiLastToFinish;" << std::endl;
+        os << "__syncthreads();" << std::endl;
+        os << "if(threadIdx.x == 0u)";
+        {
+            CodeStream::Scope b(os);
+            os << "const unsigned int arrived = __hip_atomic_fetch_add(gennmiArgs.finished, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);" << std::endl;
+            os << "gennmiLastToFinish = (arrived == gridDim.x * gridDim.y - 1u);" << std::endl;
+            os << "if(gennmiLastToFinish) { __hip_atomic_store(gennmiArgs.finished, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }" << std::endl;
+        }
+        os << "__syncthreads();" << std::endl;
+        os << "if(gennmiLastToFinish)";
+        {
+            CodeStream::Scope b(os);
+            os << delayStream.str();
+        }
+    }
     neuronKernel.close(os);
     os << std::endl;
 
@@ -427,6 +478,12 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     }
     os << declStream.str();
     os << "static unsigned long long *gennmiNeuronAgg = nullptr;" << std::endl;
+    if(anyDenDelay) {
+        os << "static uint32_t *gennmiNeuronFinished = nullptr;     // work-groups of the running neuron update that have finished" << std::endl;
+        for(const auto &g : modelMerged.getMergedSynapseDendriticDelayUpdateGroups()) {
+            os << "extern MergedSynapseDendriticDelayUpdateGroup" << g.getIndex() << " *d_mergedSynapseDendriticDelayUpdateGroup" << g.getIndex() << ";      // (uploaded by the synapse module)" << std::endl;
+        }
+    }
     os << "extern \"C\" const unsigned char gennmi_neuronUpdate_image[];" << std::endl;
     os << "extern \"C\" const unsigned char gennmi_neuronUpdate_image_end[];" << std::endl;
     os << std::endl;
@@ -443,6 +500,11 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             os << "GENNMI_CHECK(gennmi_malloc(&p, " << 2 * std::max<size_t>(1, table.numBlocks) * batchSize * (1 + maxEventGroups) << " * sizeof(unsigned long long)));" << std::endl;
             os << "GENNMI_CHECK(gennmi_memset(p, 0, " << 2 * std::max<size_t>(1, table.numBlocks) * batchSize * (1 + maxEventGroups) << " * sizeof(unsigned long long)));" << std::endl;
             os << "gennmiNeuronAgg = (unsigned long long*)p;" << std::endl;
+            if(anyDenDelay) {
+                os << "GENNMI_CHECK(gennmi_malloc(&p, sizeof(uint32_t)));" << std::endl;
+                os << "GENNMI_CHECK(gennmi_memset(p, 0, sizeof(uint32_t)));" << std::endl;
+                os << "gennmiNeuronFinished = (uint32_t*)p;" << std::endl;
+            }
             os << "uint32_t module = 0;" << std::endl;
             os << "GENNMI_CHECK(gennmi_program_load_module(gennmiProgram, gennmi_neuronUpdate_image, (size_t)(gennmi_neuronUpdate_image_end - gennmi_neuronUpdate_image), &module));" << std::endl;
             if(anyPrevTimes) { prevKernel.addToPhase(os, "GENNMI_PHASE_NEURONS", prevTable.numBlocks, batchSize, 256, -1, "nullptr", "0ull"); }
@@ -455,6 +517,7 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
     {
         CodeStream::Scope b(os);
         os << "if(gennmiNeuronAgg) { gennmi_free(gennmiNeuronAgg); gennmiNeuronAgg = nullptr; }" << std::endl;
+        if(anyDenDelay) { os << "if(gennmiNeuronFinished) { gennmi_free(gennmiNeuronFinished); gennmiNeuronFinished = nullptr; }" << std::endl; }
         os << releaseStream.str();
     }
     os << std::endl;
@@ -623,6 +686,22 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
     }
 
     // ---- presynaptic update
+    auto presynapticBlocks = [this](const SynapseGroupInternal &sg) -> size_t
+    {
+        const auto matrix = sg.getMatrixType();
+        const size_t rowLen = (matrix & SynapseMatrixConnectivity::PROCEDURAL) ? sg.getNumThreadsPerSpike()
+                              : (matrix & SynapseMatrixConnectivity::DENSE) ? sg.getTrgNeuronGroup()->getNumNeurons() : getSynapticMatrixRowStride(sg);
+        return std::clamp<size_t>((sg.getSrcNeuronGroup()->getNumNeurons() * ((rowLen + 63) / 64) + 255) / 256, 1, 128);
+    };
+    double presynapticScale = 1.0;
+    {
+        size_t wanted = 0;
+        for(const auto &sg : model.getSynapseGroups()) {
+            if(sg.second.isPreSpikeRequired() || sg.second.isPreSpikeEventRequired()) { wanted += presynapticBlocks(sg.second); }
+        }
+        constexpr size_t oneRound = 256 * 8;        // work-groups of 256 threads the chip holds at once
+        if(wanted > oneRound) { presynapticScale = (double)oneRound / (double)wanted; }
+    }
     {
         CodeStream stream(pre.body);
         EnvironmentLibrary lib(stream, StandardLibrary::getMathsFunctions());
@@ -651,10 +730,10 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                     const size_t firstBlock = pre.table.numBlocks;
                     for(size_t g = 0; g < s.getGroups().size(); g++) {
                         const auto &sg = s.getGroups()[g].get();
-                        const size_t rowLen = procedural ? threadsPerSpike : (sparse || toeplitz || bitmask) ? getSynapticMatrixRowStride(sg) : sg.getTrgNeuronGroup()->getNumNeurons();
-                        const size_t chunks = (rowLen + 63) / 64;
-                        // enough wavefronts for ~1.5 % of the source population firing in one step, at most 128 work-groups
-                        const size_t blocks = std::clamp<size_t>((sg.getSrcNeuronGroup()->getNumNeurons() * chunks + 255) / 256, 1, 128);
+                        // enough wavefronts for ~1.5 % of the source population firing in one step, at most 128 work-groups; a model of
+                        // many projections shares one round of the chip between them in that proportion (a work-group that finds no
+                        // spike leaves at once, but thousands of them still take microseconds to come and go)
+                        const size_t blocks = std::max<size_t>(1, (size_t)((double)presynapticBlocks(sg) * presynapticScale));
                         for(size_t b = 0; b < blocks; b++) { pre.table.add(g, 0, b, blocks); }
                     }
                     const std::string structArray = "mergedPresynapticUpdateGroup" + std::to_string(s.getIndex());
@@ -979,7 +1058,7 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
     modelMerged.genMergedPostsynapticUpdateGroupHostStructArrayPush(os, *this);
     modelMerged.genMergedSynapseDynamicsGroupHostStructArrayPush(os, *this);
     preambleHandler(os);
-    for(const auto &g : modelMerged.getMergedSynapseDendriticDelayUpdateGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "SynapseDendriticDelayUpdate"); }
+    for(const auto &g : modelMerged.getMergedSynapseDendriticDelayUpdateGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "SynapseDendriticDelayUpdate", true); }
     for(const auto &g : modelMerged.getMergedPresynapticUpdateGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "PresynapticUpdate"); }
     for(const auto &g : modelMerged.getMergedPostsynapticUpdateGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "PostsynapticUpdate"); }
     for(const auto &g : modelMerged.getMergedSynapseDynamicsGroups()) { genDeviceStructArray(decl, upload, release, *this, g, "SynapseDynamics"); }
@@ -1002,7 +1081,16 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                 os << "uint32_t module = 0;" << std::endl;
                 os << "GENNMI_CHECK(gennmi_program_load_module(gennmiProgram, gennmi_synapseUpdate_image, (size_t)(gennmi_synapseUpdate_image_end - gennmi_synapseUpdate_image), &module));" << std::endl;
             }
-            if(anyDelay) { delay.args.addToPhase(os, "GENNMI_PHASE_SYNAPSES", 1, 1, 64, -1, "nullptr", "0ull"); }
+            if(anyDelay) {
+                // The reference moves the ring pointers on at the start of every updateSynapses (backendCUDAHIP.cc:560-566), a launch
+                // of one thread per group.  Here the last work-group of the neuron update to finish does it for the step that
+                // follows (nothing reads the pointers in between), so the kernel below runs once, before the first step.
+                CodeStream::Scope b3(os);
+                os << "uint32_t k = 0;" << std::endl;
+                os << "GENNMI_CHECK(gennmi_program_get_kernel(gennmiProgram, module, \"" << delay.args.name << "\", &k));" << std::endl;
+                os << delay.args.fillBlock("nullptr", "0ull") << std::endl;
+                os << "GENNMI_CHECK(gennmi_program_launch(gennmiProgram, k, 1u, 1u, 64u, &a, sizeof(a), 0.0, 0ull, -1));" << std::endl;
+            }
             if(anyDynamics) { dynamics.args.addToPhase(os, "GENNMI_PHASE_SYNAPSES", dynamics.table.numBlocks, batchSize, 256, timing ? timerId("synapseDynamics") : -1, "nullptr", seed); }
             if(anyPre) { pre.args.addToPhase(os, "GENNMI_PHASE_SYNAPSES", pre.table.numBlocks, batchSize, 256, timing ? timerId("presynapticUpdate") : -1, "nullptr", seed); }
             if(anyPost) { post.args.addToPhase(os, "GENNMI_PHASE_SYNAPSES", post.table.numBlocks, batchSize, 256, timing ? timerId("postsynapticUpdate") : -1, "nullptr", seed); }
