@@ -8,9 +8,15 @@ Workload (default): the full-scale cortical microcircuit — 77,169 LIF neurons 
 resident in HBM when the timed region starts.
 
 Prints ONE JSON line: whole-job synaptic events per second, plus
-  roofline      the presynaptic-update kernel against the HBM roofline (algorithmic bytes per event
+  roofline      the dominant kernel against the HBM roofline (algorithmic bytes per event
                 x events per launch / average launch duration from HIP events on the kernel's stream)
   cpu_baseline  the single-threaded CPU oracle timed on this host on a bounded sample of the same network
+  steady_state  (short runs only) the same network stepped on in the same process — 2,000 untimed steps, then 10,000
+                timed ones — with its own roofline: a run of a few steps from t = 0 times the launch's start-up and the
+                synchronous burst every cold start of the network goes through, not the running network
+  secondary     (default workload only) the bandwidth-bound case beside the latency-bound headline: configuration 3 —
+                10^6 Izhikevich neurons, 10^9 synapses, its own noise array — for 1,000 steps (1 s simulated), with the
+                presynaptic kernels' fraction of the HBM roofline
 """
 import argparse
 import json
@@ -30,11 +36,20 @@ BYTES_PER_EVENT = {"dense": 4,          # one weight read per (spike, target); o
 # produced them in profiles/<kernel>_<workload>.md.  A counter run is a separate invocation of this script, so the figure
 # is only attached to a run of the very command line it was measured on (same workload, steps and warm-up: the network,
 # its seed and therefore its activity are then identical); any other run reports null.
+# The kernel's source is named with a digest: a figure measured on another version of the kernel is not attached.
 MEASURED_TRAFFIC_BYTES = {
     ("potjans", 20, 5): {"plan": "resident", "bytes_per_launch": 155544259,
+                         "kernel_source": ("genn_amd/csrc/genn_mi355x_resident_kernels.h", "6e38adb29614848d"),
                          "source": "rocprofv3 --pmc FETCH_SIZE (67852.50 x 2 KiB) + WRITE_SIZE (16193.69 x 1 KiB) of the timed 20-step "
                                    "launch, profiles/residentKernel_potjans_full.md"},
 }
+FP32_MFMA_PEAK_TFLOPS = 157.3
+
+
+def source_digest(path):
+    import hashlib
+    with open(os.path.join(ROOT, path), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
 
 
 def build_net(name, steps):
@@ -122,8 +137,8 @@ def bench_init(args):
     print(json.dumps(out))
 
 
-def bench_procedural(args, stored):
-    """--workload izh_procedural / izh_stored: the 10^6-neuron, 10^9-synapse Izhikevich network with its connectivity and
+def bench_procedural(args, stored, steps=None, warmup=None, profile_steps=None):
+    """--workload izh_procedural / izh_stored (the latter is also the default run's `secondary` block): the 10^6-neuron, 10^9-synapse Izhikevich network with its connectivity and
     weights regenerated for every spike (PROCEDURAL: nothing stored), or its stored twin built on the device from the same
     seed (SPARSE).  800,000 excitatory and 200,000 inhibitory neurons; every neuron has 800 + 200 targets
     (FixedNumberPostWithReplacement per target population), weights U[0, 0.5) from excitatory and U[-1, 0) from inhibitory
@@ -148,25 +163,28 @@ def bench_procedural(args, stored):
             model.add_synapse_population(src + trg, matrix, pops[src], pops[trg],
                                          init_weight_update("StaticPulse", {}, {"g": init_var("Uniform", {"min": lo, "max": hi})}),
                                          init_postsynaptic("DeltaCurr"), init_sparse_connectivity("FixedNumberPostWithReplacement", {"num": num}))
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
+    profile_steps = args.profile_steps if profile_steps is None else profile_steps
     model.build()
-    model.load(num_recording_timesteps=args.warmup + args.steps)
+    model.load(num_recording_timesteps=warmup + steps)
     model.synchronize()
     load_s = time.time() - t0
-    model.run(args.warmup)
+    model.run(warmup)
     model.synchronize()
     ev0 = model.synaptic_event_count
     t0 = time.perf_counter()
-    model.run(args.steps)
+    model.run(steps)
     model.synchronize()
     wall = time.perf_counter() - t0
     events = model.synaptic_event_count - ev0
     model.pull_recording_buffers_from_device()
-    rates = {name: round(len(p.spike_recording_data[0][1]) / p.num_neurons / ((args.warmup + args.steps) / 1000.0), 3) for name, p in pops.items()}
+    rates = {name: round(len(p.spike_recording_data[0][1]) / p.num_neurons / ((warmup + steps) / 1000.0), 3) for name, p in pops.items()}
     roofline = None
-    if args.profile_steps > 0:
+    if profile_steps > 0:
         model.set_timing(True)
         evp0 = model.synaptic_event_count
-        model.run(args.profile_steps)
+        model.run(profile_steps)
         model.synchronize()
         st = model.kernel_stats()
         evp = model.synaptic_event_count - evp0
@@ -174,54 +192,32 @@ def bench_procedural(args, stored):
         # algorithmic bytes per event: the fp32 read-modify-write of outPost, plus the stored index and weight if there are any
         bpe = 16 if stored else 8
         achieved = evp / max(1, st["presyn_launches"]) * bpe / avg_s / 1e9
-        roofline = {"bound": "hbm", "kernel": "presynapticUpdateKernel (+ presynapticTileKernel)" if stored else "presynapticProceduralKernel",
+        roofline = {"bound": "hbm", "kernel": "presynapticUpdateKernel + presynapticTileKernel (every step launches both; one of them takes the step)" if stored else "presynapticProceduralKernel",
                     "achieved": round(achieved, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6), "traffic": None,
                     "bytes_per_event": bpe, "events_per_launch": round(evp / max(1, st["presyn_launches"]), 1), "avg_launch_us": round(avg_s * 1e6, 3),
                     "events_per_s_in_kernel": round(evp / st["presyn_seconds"], 1) if st["presyn_seconds"] else None,
                     "neuron_kernel_avg_us": round(st["neuron_seconds"] / max(1, st["neuron_launches"]) * 1e6, 3)}
     model.unload()
-    print(json.dumps({
-        "metric": "synaptic_events_per_s", "value": round(events / wall, 1), "unit": "events/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(wall / args.steps * 1e3, 6), "higher_is_better": True, "scaling": "weak",
+    return {
+        "metric": "synaptic_events_per_s", "value": round(events / wall, 1), "unit": "events/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": round(wall / steps * 1e3, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "10^6 Izhikevich neurons, 10^9 synapses, " + ("stored on the device (SPARSE, built there)" if stored else "PROCEDURAL (regenerated per spike)"),
                    "neurons": n_e + n_i, "synapses": (n_e + n_i) * 1000, "dt_ms": 1.0, "seed": 777},
-        "gsop_per_s": round(events / wall / 1e9, 4), "wall_s_per_sim_s": round(wall / (args.steps / 1000.0), 4),
-        "events_per_step": round(events / args.steps, 1), "firing_rates_hz": rates, "setup_s": {"build_and_load": round(load_s, 2)},
-        "roofline": roofline, "cpu_baseline": None}))
+        "gsop_per_s": round(events / wall / 1e9, 4), "wall_s_per_sim_s": round(wall / (steps / 1000.0), 4),
+        "events_per_step": round(events / steps, 1), "firing_rates_hz": rates, "setup_s": {"build_and_load": round(load_s, 2)},
+        "roofline": roofline, "cpu_baseline": None}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10000)
-    ap.add_argument("--warmup", type=int, default=2000)
-    ap.add_argument("--workload", default="potjans")
-    ap.add_argument("--cpu-steps", type=int, default=None, help="steps of the CPU baseline sample (default: sized for ~10-20 s)")
-    ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--reference-steps", type=int, default=2000,
-                    help="steps of the extra CPU leg on the reference's own SingleThreadedCPU backend (oracle/_ref/ref_driver, "
-                         "only where that prebuilt driver exists; 0 disables)")
-    ap.add_argument("--profile-steps", type=int, default=2000, help="extra steps replayed with HIP event nodes around every kernel (multiple of 100)")
-    ap.add_argument("--yardstick-mib", type=int, default=0,
-                    help="also run the library's plain copy kernel on this many MiB (5 launches, 2x this traffic each), so a "
-                         "hardware-counter run has a kernel of known HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        raise SystemExit("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
-                         "(the hot path is single-GPU: sharded by postsynaptic neuron it would exchange only the spike lists each step)")
-
-    if args.workload == "init_izhikevich":
-        return bench_init(args)
-    if args.workload in ("izh_procedural", "izh_stored"):
-        return bench_procedural(args, stored=(args.workload == "izh_stored"))
-
+def run_net_workload(args, workload, steps, warmup, profile_steps, with_cpu, with_steady):
+    """One host-generated network: load, warm-up, timed region, per-kernel pass, (running-network block), (CPU baseline).
+    Returns the record of the run."""
     import numpy as np
     from genn_amd.genn_model import model_from_net
 
-    total_steps = args.warmup + args.steps + args.profile_steps
+    total_steps = warmup + steps + profile_steps
     t0 = time.time()
-    net, label = build_net(args.workload, total_steps)
+    net, label = build_net(workload, total_steps)
     gen_s = time.time() - t0
     num_neurons = sum(p.n for p in net.pops)
     num_synapses = sum(s.num_synapses for s in net.syns)
@@ -231,17 +227,17 @@ def main():
     t0 = time.time()
     batch = getattr(net, "batch_size", 1)
     model = model_from_net(net, batch_size=batch, record=True)
-    model.load(num_recording_timesteps=args.warmup + args.steps)
+    model.load(num_recording_timesteps=warmup + steps)
     model.synchronize()
     load_s = time.time() - t0
 
     # ---- warm-up (also captures the step graph), then the timed region
-    model.run(args.warmup)
+    model.run(warmup)
     model.synchronize()
     ev0 = model.synaptic_event_count
     t0 = time.perf_counter()
     model.stream_mark(0)
-    model.run(args.steps)
+    model.run(steps)
     model.stream_mark(1)
     model.synchronize()
     wall = time.perf_counter() - t0
@@ -253,38 +249,38 @@ def main():
     rates = {}
     for p in net.pops:
         data = model.neuron_populations[p.name].spike_recording_data
-        rates[p.name] = round(sum(len(ids) for _, ids in data) / batch / p.n / ((args.warmup + args.steps) * net.dt / 1000.0), 3)
+        rates[p.name] = round(sum(len(ids) for _, ids in data) / batch / p.n / ((warmup + steps) * net.dt / 1000.0), 3)
 
     # ---- per-kernel durations: the same graph replay with HIP event nodes between the kernels of every step
     # (events on the runner's stream; durations are those of back-to-back execution)
     roofline = None
     info = model.runner_info()
-    if args.profile_steps > 0:
+    if profile_steps > 0:
         model.set_timing(True)
         evp0 = model.synaptic_event_count
-        model.run(args.profile_steps)
+        model.run(profile_steps)
         model.synchronize()
         st = model.kernel_stats()
         evp = model.synaptic_event_count - evp0
         model.set_timing(False)
         bpe = bytes_per_event or max(BYTES_PER_EVENT[k] for k in kinds)
-        neuron_bytes = sum(p.n * (0 if p.model == "ssa" else 32) for p in net.pops)     # 32 B per LIF/Izhikevich update (state + one PSM)
+        neuron_bytes = batch * sum(p.n * (0 if p.model == "ssa" else 32) for p in net.pops)     # 32 B per LIF/Izhikevich update (state + one PSM), every batch
         if info["resident_plan"]:
             # the timed region is ONE launch of residentKernel that performs all K steps and nothing else, so HIP events
             # around the region give that launch's duration; a launch moves K steps' worth of
             # algorithmic bytes
-            achieved = (events * bpe + neuron_bytes * args.steps) / region_s / 1e9
+            achieved = (events * bpe + neuron_bytes * steps) / region_s / 1e9
             roofline = {"bound": "hbm", "kernel": "residentKernel (all timesteps of the timed region in one launch)",
                         "achieved": round(achieved, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6),
-                        "traffic": None, "bytes_per_event": bpe, "events_per_launch": events, "steps_per_launch": args.steps,
-                        "neuron_bytes_per_launch": neuron_bytes * args.steps, "avg_launch_us": round(region_s * 1e6, 3),
-                        "us_per_step": round(region_s / args.steps * 1e6, 3),
+                        "traffic": None, "bytes_per_event": bpe, "events_per_launch": events, "steps_per_launch": steps,
+                        "neuron_bytes_per_launch": neuron_bytes * steps, "avg_launch_us": round(region_s * 1e6, 3),
+                        "us_per_step": round(region_s / steps * 1e6, 3),
                         "avg_launch_us_one_step_per_launch": round(st["step_seconds"] / max(1, st["step_launches"]) * 1e6, 3) if st["step_launches"] else None}
         elif info["single_launch_step"]:
             # the timed region consists of this kernel only (one launch per step, back to back inside the replayed
             # graphs, plus one 1-thread node per 100 steps), so HIP events around the region give its average duration
-            avg_s = region_s / args.steps
-            ev_per_launch = events / args.steps
+            avg_s = region_s / steps
+            ev_per_launch = events / steps
             achieved = (ev_per_launch * bpe + neuron_bytes) / avg_s / 1e9
             roofline = {"bound": "hbm", "kernel": "stepFusedKernel (presynaptic + neuron update of one timestep)",
                         "achieved": round(achieved, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6),
@@ -296,12 +292,30 @@ def main():
             ev_per_launch = evp / st["presyn_launches"]
             achieved = ev_per_launch * bpe / avg_s / 1e9
             navg = st["neuron_seconds"] / max(1, st["neuron_launches"])
-            roofline = {"bound": "hbm", "kernel": "presynapticDenseKernel" if kinds == {"dense"} else "presynapticUpdateKernel (+ presynapticTileKernel)", "achieved": round(achieved, 3),
+            # (the timed pass launches every kernel on its own so that each has an event pair; the untimed region combines the
+            # synaptic kernels of a step into one launch where the runner's plan says so)
+            if kinds == {"dense"}:
+                kernel = "presynapticDenseKernel"
+            elif info["conv_on_matrix_cores"]:
+                kernel = "presynapticConvMfmaKernel (busy steps) + presynapticUpdateKernel (quiet steps)"
+            elif info["combined_synapse_launch"]:
+                kernel = ("presynapticUpdateKernel + presynapticTileKernel, launched separately in this timed pass; the untimed region runs them"
+                          + (" and the postsynaptic pass" if info["postsynaptic_in_combined_launch"] else "") + " as one synapseCombinedKernel launch per step")
+            else:
+                kernel = "presynapticUpdateKernel"
+            roofline = {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 3),
                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6), "traffic": None,
                         "bytes_per_event": bpe, "events_per_launch": round(ev_per_launch, 1), "avg_launch_us": round(avg_s * 1e6, 3),
                         "neuron_kernel_avg_us": round(navg * 1e6, 3), "neuron_kernel_gbs": round(neuron_bytes / navg / 1e9, 3)}
             if st["postsyn_launches"]:
                 roofline["postsyn_kernel_avg_us"] = round(st["postsyn_seconds"] / st["postsyn_launches"] * 1e6, 3)
+            if info["conv_on_matrix_cores"]:
+                # the layer as a GEMM per batch and step: (output pixels) x (kh kw ic) x (output channels), fp32 MFMA; every
+                # step of this workload is a busy one, so the presynaptic time is the matrix-core kernel's
+                c = [s_ for s_ in net.syns if s_.matrix == "conv2d"][0].conv
+                flops = 2.0 * batch * c["conv_oh"] * c["conv_ow"] * c["conv_kh"] * c["conv_kw"] * c["conv_ic"] * c["conv_oc"]
+                roofline["mfma"] = {"bound": "mfma", "kernel": "presynapticConvMfmaKernel", "achieved": round(flops / avg_s / 1e12, 3), "peak": FP32_MFMA_PEAK_TFLOPS,
+                                    "unit": "TFLOP/s", "frac": round(flops / avg_s / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4), "flops_per_launch": flops}
     if args.yardstick_mib > 0:
         from genn_amd.genn_model import Array
         count = args.yardstick_mib * (1 << 20) // 4
@@ -309,15 +323,45 @@ def main():
         for _ in range(5):
             b.copy_on_device(a)
         a.free(); b.free()
-    measured = MEASURED_TRAFFIC_BYTES.get((args.workload, args.steps, args.warmup))
+    measured = MEASURED_TRAFFIC_BYTES.get((workload, steps, warmup))
     if roofline is not None and measured is not None and measured["plan"] == ("resident" if info["resident_plan"] else "stepped"):
-        roofline["traffic"] = measured["bytes_per_launch"]
-        roofline["traffic_source"] = measured["source"]
+        if source_digest(measured["kernel_source"][0]) == measured["kernel_source"][1]:
+            roofline["traffic"] = measured["bytes_per_launch"]
+            roofline["traffic_source"] = measured["source"]
+        else:
+            roofline["traffic_source"] = "not attached: " + measured["kernel_source"][0] + " has changed since the counters were read"
+
+    # ---- the running network: short runs only (see the module docstring)
+    steady = None
+    if with_steady and args.steady_steps > 0 and steps < 1000:
+        model.run(args.steady_warmup)
+        model.synchronize()
+        ev0s = model.synaptic_event_count
+        t0 = time.perf_counter()
+        model.stream_mark(0)
+        model.run(args.steady_steps)
+        model.stream_mark(1)
+        model.synchronize()
+        wall_s = time.perf_counter() - t0
+        region = model.stream_elapsed()
+        ev_s = model.synaptic_event_count - ev0s
+        bpe = bytes_per_event or max(BYTES_PER_EVENT[k] for k in kinds)
+        nbytes = batch * sum(p.n * (0 if p.model == "ssa" else 32) for p in net.pops)
+        achieved = (ev_s * bpe + nbytes * args.steady_steps) / region / 1e9
+        steady = {"steps": args.steady_steps, "warmup": args.steady_warmup, "us_per_step": round(wall_s / args.steady_steps * 1e6, 3),
+                  "events_per_s": round(ev_s / wall_s, 1), "gsop_per_s": round(ev_s / wall_s / 1e9, 4),
+                  "events_per_step": round(ev_s / args.steady_steps, 1),
+                  "wall_s_per_sim_s": round(wall_s / (args.steady_steps * net.dt / 1000.0), 4),
+                  "roofline": {"bound": "hbm", "kernel": ("residentKernel (one launch for all steps of the block)" if info["resident_plan"] else
+                                                          "all kernels of the block's steps (hipGraph replay)"),
+                               "achieved": round(achieved, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6),
+                               "avg_launch_us": round(region * 1e6, 3), "us_per_step": round(region / args.steady_steps * 1e6, 3),
+                               "bytes_per_event": bpe, "events_per_launch": ev_s, "neuron_bytes_per_launch": nbytes * args.steady_steps, "traffic": None}}
     model.unload()
 
     # ---- CPU baseline: the single-threaded oracle on the same network, bounded sample from t = 0
     cpu = None
-    if not args.no_cpu:
+    if with_cpu:
         from oracle.genn_cpu import OracleNet
         # the reference's CPU backend (and the oracle) has no batch dimension: batch 0 is timed and the figure is per batch
         oracle = OracleNet(net.batch_nets[0] if batch > 1 else net)
@@ -376,10 +420,10 @@ def main():
             finally:
                 shutil.rmtree(tmp, ignore_errors=True)
 
-    sim_s = args.steps * net.dt / 1000.0
+    sim_s = steps * net.dt / 1000.0
     out = {
         "metric": "synaptic_events_per_s", "value": round(events / wall, 1), "unit": "events/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall / args.steps * 1e3, 6),
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(wall / steps * 1e3, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": label, "neurons": num_neurons, "synapses": num_synapses, "dt_ms": net.dt, "seed": net.seed,
                    "stepping": ("resident plan: one launch for all timed steps, state in registers/LDS" if info["resident_plan"] else
@@ -387,14 +431,59 @@ def main():
                                                                            "2 launches per step (synaptic kernels combined)" if (info["combined_synapse_launch"] or info["conv_on_matrix_cores"]) else
                                                                            "2-3 launches per step"))},
         "gsop_per_s": round(events / wall / 1e9, 4),
-        "neuron_updates_per_s": round(num_neurons * batch * args.steps / wall, 1),
+        "neuron_updates_per_s": round(num_neurons * batch * steps / wall, 1),
         "wall_s_per_sim_s": round(wall / sim_s, 4),
-        "events_per_step": round(events / args.steps, 1), "events_including_warmup": events_with_warmup,
+        "events_per_step": round(events / steps, 1), "events_including_warmup": events_with_warmup,
         "algorithmic_gb_per_s_wallclock": round(events * (bytes_per_event or 16) / wall / 1e9, 3),
         "firing_rates_hz": rates,
         "setup_s": {"generate": round(gen_s, 1), "load": round(load_s, 1)},
         "roofline": roofline, "cpu_baseline": cpu,
     }
+    if steady is not None:
+        out["steady_state"] = steady
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10000)
+    ap.add_argument("--warmup", type=int, default=2000)
+    ap.add_argument("--workload", default="potjans")
+    ap.add_argument("--cpu-steps", type=int, default=None, help="steps of the CPU baseline sample (default: sized for ~10-20 s)")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--reference-steps", type=int, default=2000,
+                    help="steps of the extra CPU leg on the reference's own SingleThreadedCPU backend (oracle/_ref/ref_driver, "
+                         "only where that prebuilt driver exists; 0 disables)")
+    ap.add_argument("--profile-steps", type=int, default=2000, help="extra steps replayed with HIP event nodes around every kernel (multiple of 100)")
+    ap.add_argument("--steady-steps", type=int, default=10000,
+                    help="runs of fewer than 1000 timed steps: steps of the `steady_state` block that follows in the same process (0 disables)")
+    ap.add_argument("--steady-warmup", type=int, default=2000, help="untimed steps before the `steady_state` block")
+    ap.add_argument("--secondary-steps", type=int, default=1000,
+                    help="default workload only: timed steps of the `secondary` block (configuration 3: 10^6 Izhikevich neurons, 10^9 synapses; 0 disables)")
+    ap.add_argument("--yardstick-mib", type=int, default=0,
+                    help="also run the library's plain copy kernel on this many MiB (5 launches, 2x this traffic each), so a "
+                         "hardware-counter run has a kernel of known HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
+                         "(the hot path is single-GPU: sharded by postsynaptic neuron it would exchange only the spike lists each step)")
+
+    if args.workload == "init_izhikevich":
+        return bench_init(args)
+    if args.workload in ("izh_procedural", "izh_stored"):
+        print(json.dumps(bench_procedural(args, stored=(args.workload == "izh_stored"))))
+        return
+
+    out = run_net_workload(args, args.workload, args.steps, args.warmup, args.profile_steps, with_cpu=not args.no_cpu, with_steady=True)
+    if args.workload == "potjans" and args.secondary_steps > 0:
+        # configuration 3 as it stands (the bandwidth-bound case), generated on the host and uploaded like the headline network
+        try:
+            sec = run_net_workload(args, "izh", args.secondary_steps, 100, min(args.secondary_steps, 1000), with_cpu=False, with_steady=False)
+            out["secondary"] = {k: sec[k] for k in ("metric", "value", "unit", "steps", "warmup", "ms_per_step", "dtype", "data", "config", "gsop_per_s",
+                                                    "neuron_updates_per_s", "wall_s_per_sim_s", "events_per_step", "firing_rates_hz", "setup_s", "roofline")}
+        except Exception as e:          # a reported extra: never let it take the bench line down
+            out["secondary"] = {"error": repr(e)}
     print(json.dumps(out))
 
 
