@@ -1575,6 +1575,22 @@ void Backend::genStepTimeFinalisePreamble(CodeStream &os, const ModelSpecMerged 
     }
 }
 //--------------------------------------------------------------------------
+std::string State::getDeviceName() const
+{
+    char name[256] = {0};
+    if(gennmi_device_name(name, sizeof(name)) != GENNMI_OK) { throw std::runtime_error(gennmi_last_error()); }
+    return name;
+}
+size_t State::getFreeDeviceMemBytes() const
+{
+    size_t bytes = 0;
+    if(gennmi_free_device_memory_bytes(&bytes) != GENNMI_OK) { throw std::runtime_error(gennmi_last_error()); }
+    return bytes;
+}
+void State::synchronize() const
+{
+    if(gennmi_synchronize() != GENNMI_OK) { throw std::runtime_error(gennmi_last_error()); }
+}
 std::unique_ptr<GeNN::Runtime::StateBase> Backend::createState(const Runtime::Runtime&) const
 {
     return std::make_unique<State>();

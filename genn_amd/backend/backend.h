@@ -68,8 +68,18 @@ struct Preferences : public PreferencesBase
     }
 };
 
-class State : public Runtime::StateBase
+//! Backend state of a loaded model (Runtime::getState; PyGeNN exposes it as `_Runtime`): what the device library can say about
+//! the device the model runs on.  The reference's HIP backend keeps its NCCL communicator here (hip/backend.h:150-175); this
+//! backend is single-GPU.
+class BACKEND_EXPORT State : public Runtime::StateBase
 {
+public:
+    //! name, architecture and compute-unit count of the current device
+    std::string getDeviceName() const;
+    //! device memory still free, in bytes
+    size_t getFreeDeviceMemBytes() const;
+    //! runs everything the device library has noted and waits for the device; throws if a kernel raised an error flag
+    void synchronize() const;
 };
 
 class BACKEND_EXPORT Backend : public BackendBase

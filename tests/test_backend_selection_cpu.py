@@ -33,6 +33,31 @@ def test_generator_configuration_names_the_backend():
     assert "mi355x_backend" in open(os.path.join(BACKEND_DIR, "pygenn_module.cc")).read()
 
 
+def test_pygenn_module_exposes_every_preference_and_the_backend_state():
+    """PyGeNN sets backend preferences by attribute (pygenn/genn_model.py:673-681: every keyword of GeNNModel that is not a
+    model option becomes `setattr(preferences, name, value)`), so every member of the backend's Preferences struct must be
+    bound, under its snake_case name, and the backend state must be there under the name PyGeNN looks up (`_Runtime`,
+    pygenn/src/hipBackend.cc:57-67).  `pygenn._genn` is not built here, so the module cannot be imported: the check is
+    of the source against the struct, plus the module having been compiled (its init symbol)."""
+    import re
+    header = open(os.path.join(BACKEND_DIR, "backend.h")).read()
+    struct = header[header.index("struct Preferences"):header.index("void updateHash")]
+    members = re.findall(r"^\s+(?:int|bool|unsigned int|std::string|KernelSource)\s+(\w+)\s*(?:=[^;]*)?;", struct, flags=re.M)
+    assert set(members) == {"deviceID", "installRoot", "kernelSource", "orderedAccumulation", "stepQueueLength", "deviceInitialisation"}, members
+    module = open(os.path.join(BACKEND_DIR, "pygenn_module.cc")).read()
+    for member in members:
+        snake = re.sub(r"(?<=[a-z])([A-Z])", lambda m: "_" + m.group(1).lower(), member).replace("_i_d", "_id").lower()
+        assert f'.def_readwrite("{snake}", &Preferences::{member})' in module, (member, snake)
+    for value in ("AUTO", "LIBRARY", "GENERATED"):
+        assert f'.value("{value}", Preferences::KernelSource::{value})' in module
+    assert 'pybind11::class_<State, Runtime::StateBase>(m, "_Runtime")' in module
+    assert '"_Backend"' in module and '"_create_backend"' in module
+    import sysconfig
+    built = os.path.join(ROOT, "genn_amd", "lib", "mi355x_backend" + sysconfig.get_config_var("EXT_SUFFIX"))
+    if os.path.exists(built):
+        assert "PyInit_mi355x_backend" in _exports(built)
+
+
 @pytest.mark.skipif(not os.path.exists(GENERATOR), reason="oracle/_ref/mi355x_generator is not built (needs the reference tree at build time)")
 def test_reference_generator_selects_the_backend_and_builds_a_runner():
     """generator.cc as genn-buildmodel runs it: <genn dir> <target dir> <force rebuild>.  It creates the backend through
