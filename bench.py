@@ -287,6 +287,22 @@ def run_net_workload(args, workload, steps, warmup, profile_steps, with_cpu, wit
                         "traffic": None, "bytes_per_event": bpe, "events_per_launch": round(ev_per_launch, 1),
                         "neuron_bytes_per_launch": neuron_bytes, "avg_launch_us": round(avg_s * 1e6, 3),
                         "avg_launch_us_individually_launched": round(st["step_seconds"] / max(1, st["step_launches"]) * 1e6, 3)}
+        elif info["conv_step_in_one_launch"]:
+            # the timed region consists of this kernel only (the layer on the matrix cores, the postsynaptic and neuron model on its
+            # accumulators, the source population's update in blocks of the same launch), so HIP events around the region give
+            # its average duration; bytes by the event accounting (8 B per event: the target's read-modify-write) plus the state
+            avg_s = region_s / steps
+            ev_per_launch = events / steps
+            achieved = (ev_per_launch * bpe + neuron_bytes) / avg_s / 1e9
+            c = [s_ for s_ in net.syns if s_.matrix == "conv2d"][0].conv
+            flops = 2.0 * batch * c["conv_oh"] * c["conv_ow"] * c["conv_kh"] * c["conv_kw"] * c["conv_ic"] * c["conv_oc"]
+            roofline = {"bound": "hbm", "kernel": "convStepKernel (Conv2D on the matrix cores + neuron update of one timestep)",
+                        "achieved": round(achieved, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 6),
+                        "traffic": None, "bytes_per_event": bpe, "events_per_launch": round(ev_per_launch, 1),
+                        "neuron_bytes_per_launch": neuron_bytes, "avg_launch_us": round(avg_s * 1e6, 3),
+                        "avg_launch_us_individually_launched": round(st["step_seconds"] / max(1, st["step_launches"]) * 1e6, 3),
+                        "mfma": {"bound": "mfma", "achieved": round(flops / avg_s / 1e12, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                 "frac": round(flops / avg_s / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4), "flops_per_launch": flops}}
         elif st["presyn_launches"]:
             avg_s = st["presyn_seconds"] / st["presyn_launches"]
             ev_per_launch = evp / st["presyn_launches"]
@@ -427,7 +443,7 @@ def run_net_workload(args, workload, steps, warmup, profile_steps, with_cpu, wit
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": label, "neurons": num_neurons, "synapses": num_synapses, "dt_ms": net.dt, "seed": net.seed,
                    "stepping": ("resident plan: one launch for all timed steps, state in registers/LDS" if info["resident_plan"] else
-                                "hipGraph replay, 100 steps per graph, " + ("1 launch per step" if info["single_launch_step"] else
+                                "hipGraph replay, 100 steps per graph, " + ("1 launch per step" if (info["single_launch_step"] or info["conv_step_in_one_launch"]) else
                                                                            "2 launches per step (synaptic kernels combined)" if (info["combined_synapse_launch"] or info["conv_on_matrix_cores"]) else
                                                                            "2-3 launches per step"))},
         "gsop_per_s": round(events / wall / 1e9, 4),

@@ -45,6 +45,7 @@
 #include "genn_mi355x_neuron_kernels.h"
 #include "genn_mi355x_resident_kernels.h"
 #include "genn_mi355x_ordered_kernels.h"
+#include "genn_mi355x_conv_step_kernels.h"
 
 struct gennmi_runner
 {
@@ -69,6 +70,11 @@ struct gennmi_runner
     bool combineSynapses = false, combinePost = false; uint32_t synapseThreads = BLOCK; size_t combinedLdsBytes = 0;
     ConvTileDev *dConvTile = nullptr; uint32_t convTileBlocks = 0; size_t convTileBytes = 0;
     ConvMfmaDev *dConvMfma = nullptr; uint32_t convMfmaBlocks = 0; size_t convMfmaBytes = 0;      // Conv2D on the matrix cores (instead of dConvTile)
+    ConvMfmaDev convMfma{}; size_t convSource = 0;      // host copy of its descriptor; index of its source population in `neuron`
+    // a convolutional layer's whole step in one launch (convStepKernel): the layer's target population is updated on the accumulators
+    bool convStep = false;
+    NeuronGroupDev *dConvTarget = nullptr, *dConvRest = nullptr; uint32_t convRestBlocks = 0; size_t convStepBytes = 0;
+    unsigned long long *dConvAgg = nullptr, *dConvRestAgg = nullptr;
     bool bitmapsStale = false;          // a spike queue was written by the caller: the bitmaps kept beside the queues are rebuilt before the next step
     std::vector<void*> owned;           // engine-private device allocations (shadow queues, zero-delay lists)
     // resident plan (many steps per launch)
@@ -80,6 +86,7 @@ struct gennmi_runner
     std::vector<uint32_t> resSegTiles;  // tiles of its target population
     std::vector<u32x2*> resPacked;      // its synapses as the resident kernel reads them
     uint32_t neuronsPerLane = 1;        // 2, 4 or 8: neuronBulkKernel instead of neuronUpdateKernel
+    bool plainGroups = false;           // every group is one the several-neurons-per-lane neuron update covers
     bool sourcesStale = false;          // startSpike / endSpike / spikeTimes of a spike source were written since nextSpikeTime was built
     bool resStale = false;              // connectivity or weights were written since the tables were built ...
     std::vector<uint8_t> resStaleProj;  // ... of these projections (index into pre)
@@ -1124,6 +1131,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
             perLane = (v == 2 || v == 4 || v == 8) ? (uint32_t)v : (v == 1) ? 4u : 1u;
         }
         r->neuronsPerLane = plain ? perLane : 1u;
+        r->plainGroups = plain;
     }
     const uint32_t neuronsPerBlock = BLOCK * r->neuronsPerLane;
     uint32_t block = 0;
@@ -1205,6 +1213,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
                         const size_t kernFloats = (size_t)2 * (((K + 1) / 2 + CONV_MFMA_STEPS - 1) / CONV_MFMA_STEPS) * CONV_MFMA_STEPS * m.kernPitch;       // whole chunks of steps
                         // as many output rows per block as give every compute unit one block, fewer if LDS says so
                         uint32_t rowsPerBlock = std::max(1u, std::min<uint32_t>((uint32_t)c[5], ((uint32_t)c[5] * r->batch) / numCU));
+                        if(const char *envRows = getenv("GENNMI_CONV_ROWS")) { rowsPerBlock = std::max(1u, std::min<uint32_t>((uint32_t)c[5], (uint32_t)atoi(envRows))); }
                         size_t bytes = 0;
                         for(;; rowsPerBlock--) {
                             m.patchRows = rowsPerBlock + (uint32_t)c[0] - 1;
@@ -1221,10 +1230,12 @@ int gennmi_runner_finalise(gennmi_runner *r)
                                 r->bitmapsStale = true;          // the queue may already hold spikes
                             }
                             m.srcBitmap = src->spikeBitmap;
+                            r->convSource = (size_t)(src - r->neuron.data());
                             m.rowsPerBlock = rowsPerBlock;
                             m.numBatches = r->batch;
                             p.tileThreshold = std::max(1u, p.g.numTrgNeurons / 4);
                             m.threshold = p.tileThreshold;
+                            r->convMfma = m;
                             HIP_TRY(hipMalloc(&r->dConvMfma, sizeof(ConvMfmaDev)));
                             HIP_TRY(hipMemcpy(r->dConvMfma, &m, sizeof(ConvMfmaDev), hipMemcpyHostToDevice));
                             r->owned.push_back(r->dConvMfma);
@@ -1475,6 +1486,66 @@ int gennmi_runner_finalise(gennmi_runner *r)
         for(auto &n : r->neuron) { n.aggEvent = area; }
     }
     if(r->ordered) { const int rc = buildOrderedViews(r); if(rc) { return rc; } }
+    // ---- a convolutional layer's whole step in one launch: the layer on the matrix cores is the model's only projection and its
+    // target is a plain population whose only input it is (GENNMI_CONV_STEP=0: the layer's kernel, then the neuron kernel)
+    if(r->convMfmaBlocks && !r->ordered) {
+        const char *envStep = getenv("GENNMI_CONV_STEP");
+        ConvMfmaDev &m = r->convMfma;
+        const uint32_t ow = (uint32_t)m.g.conv[6], oc = (uint32_t)m.g.conv[7];
+        NeuronGroupDev *target = nullptr;
+        for(auto &n : r->neuron) {
+            if(n.g.numPSM == 1 && n.g.psm[0].outPost == m.g.outPost && n.g.numNeurons == m.g.numTrgNeurons) { target = &n; }
+        }
+        NeuronGroupDev *src = &r->neuron[r->convSource];
+        m.spikeWords = (m.rowsPerBlock * ow * oc + 31) / 32 + 1;
+        const size_t bytes = r->convMfmaBytes + (size_t)m.spikeWords * sizeof(uint32_t);
+        bool eligible = !(envStep && atoi(envStep) == 0) && r->plainGroups && target && target != src && bytes <= 64 * 1024 && (m.rowsPerBlock * ow * oc) % 32 == 0;
+        if(eligible) {
+            const auto &g = target->g;
+            eligible = (g.model == GENNMI_NEURON_LIF || g.model == GENNMI_NEURON_IZHIKEVICH) && g.psm[0].maxDenDelay == 0
+                       && (g.psm[0].kind == GENNMI_PSM_EXPCURR || g.psm[0].kind == GENNMI_PSM_DELTACURR)
+                       && (g.numCS == 0 || (g.numCS == 1 && g.cs[0].kind == GENNMI_CS_DC)) && !g.preTrace && !g.postTrace && !g.sT && g.numExtraSpk == 0
+                       && g.numDelaySlots <= 1 && g.numSpkEvent == 0 && g.numPreOutput == 0 && !target->spikeBitmap && !target->shadowSpk;
+        }
+        if(eligible) {
+            // the source's spike bitmap twice: the layer reads last step's copy while the source's blocks of the same launch write this step's
+            const size_t words = (size_t)r->batch * ((src->g.numNeurons + 31) / 32);
+            uint32_t *both = nullptr;
+            HIP_TRY(hipMalloc((void**)&both, 2 * words * sizeof(uint32_t)));
+            r->owned.push_back(both);
+            HIP_TRY(hipMemset(both, 0, 2 * words * sizeof(uint32_t)));
+            src->spikeBitmap = both; src->bitmapStride = words;
+            r->bitmapsStale = true;
+            m.srcBitmap = both; m.bitmapStride = words;
+            // the other populations' blocks, numbered from 0
+            std::vector<NeuronGroupDev> rest;
+            uint32_t block = 0;
+            for(const auto &n : r->neuron) {
+                if(&n == target) { continue; }
+                rest.push_back(n);
+                rest.back().startBlock = block;
+                rest.back().numBlocks = (n.g.numNeurons + CONV_STEP_THREADS * r->neuronsPerLane - 1) / (CONV_STEP_THREADS * r->neuronsPerLane);
+                block += rest.back().numBlocks;
+            }
+            r->convRestBlocks = block;
+            m.restBlocks = block; m.restNeuronsPerLane = r->neuronsPerLane;
+            HIP_TRY(hipMemcpy(r->dConvMfma, &m, sizeof(ConvMfmaDev), hipMemcpyHostToDevice));
+            HIP_TRY(uploadPerBlock(rest, r->convRestBlocks, &r->dConvRest));
+            HIP_TRY(hipMalloc(&r->dConvTarget, sizeof(NeuronGroupDev)));
+            HIP_TRY(hipMemcpy(r->dConvTarget, target, sizeof(NeuronGroupDev), hipMemcpyHostToDevice));
+            const size_t aggCount = 2 * (size_t)r->convMfmaBlocks * r->batch, restCount = 2 * (size_t)std::max(1u, r->convRestBlocks) * r->batch;
+            HIP_TRY(hipMalloc(&r->dConvAgg, aggCount * sizeof(unsigned long long)));
+            HIP_TRY(hipMemset(r->dConvAgg, 0, aggCount * sizeof(unsigned long long)));
+            HIP_TRY(hipMalloc(&r->dConvRestAgg, restCount * sizeof(unsigned long long)));
+            HIP_TRY(hipMemset(r->dConvRestAgg, 0, restCount * sizeof(unsigned long long)));
+            for(void *q : {(void*)r->dConvRest, (void*)r->dConvTarget, (void*)r->dConvAgg, (void*)r->dConvRestAgg}) { if(q) { r->owned.push_back(q); } }
+            r->convStepBytes = bytes;
+            if(bytes > 48 * 1024) {
+                HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(convStepKernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+            }
+            r->convStep = true;
+        }
+    }
     HIP_TRY(uploadPerBlock(r->neuron, r->neuronBlocks, &r->dNeuron));
     HIP_TRY(uploadPerBlock(r->pre, r->preBlocks, &r->dPre));
     HIP_TRY(uploadPerBlock(r->post, r->postBlocks, &r->dPost));
@@ -1545,8 +1616,10 @@ static int refreshSpikeSources(gennmi_runner *r)
         for(const auto &n : r->neuron) {
             if(!n.spikeBitmap || n.g.numDelaySlots > 1) { continue; }
             const uint32_t words = (n.g.numNeurons + 31) / 32;
-            spikeBitmapFromQueueKernel<<<dim3((words + BLOCK - 1) / BLOCK, r->batch), dim3(BLOCK), 0, r->stream>>>(n.g.spkCnt, n.g.spk, n.spikeBitmap, n.g.numNeurons, 1u);
-            spikeBitmapFromQueueKernel<<<dim3((n.g.numNeurons + BLOCK - 1) / BLOCK, r->batch), dim3(BLOCK), 0, r->stream>>>(n.g.spkCnt, n.g.spk, n.spikeBitmap, n.g.numNeurons, 0u);
+            // (of two copies, the one the coming step reads: the update after k completed steps writes copy (k + 1) & 1)
+            uint32_t *bitmap = n.spikeBitmap + (r->epoch & 1) * n.bitmapStride;
+            spikeBitmapFromQueueKernel<<<dim3((words + BLOCK - 1) / BLOCK, r->batch), dim3(BLOCK), 0, r->stream>>>(n.g.spkCnt, n.g.spk, bitmap, n.g.numNeurons, 1u);
+            spikeBitmapFromQueueKernel<<<dim3((n.g.numNeurons + BLOCK - 1) / BLOCK, r->batch), dim3(BLOCK), 0, r->stream>>>(n.g.spkCnt, n.g.spk, bitmap, n.g.numNeurons, 0u);
             HIP_TRY(hipGetLastError());
         }
     }
@@ -1629,10 +1702,19 @@ static int launchFusedStep(gennmi_runner *r, const StepArgs &a)
     return GENNMI_OK;
 }
 
+static int launchConvStep(gennmi_runner *r, const StepArgs &a)
+{
+    convStepKernel<<<dim3((r->convMfmaBlocks + r->convRestBlocks) * r->batch), dim3(CONV_STEP_THREADS), r->convStepBytes, r->stream>>>(
+        r->dConvMfma, r->dConvTarget, r->dConvRest, r->batch, a, r->dt, r->dConvAgg, r->dConvRestAgg, r->dError, r->dEvents);
+    HIP_TRY(hipGetLastError());
+    return GENNMI_OK;
+}
+
 // one whole timestep: a single launch where the runner allows it, else synapse kernels then the neuron kernel
 static int launchStep(gennmi_runner *r, const StepArgs &a)
 {
     if(r->fusedStep) { return launchFusedStep(r, a); }
+    if(r->convStep) { return launchConvStep(r, a); }
     const int rc = launchSynapses(r, a, false);
     return rc ? rc : launchNeurons(r, a, false);
 }
@@ -1690,7 +1772,7 @@ int gennmi_step_time(gennmi_runner *r, unsigned long long timestep, unsigned lon
 // one step, launched now
 static int stepNow(gennmi_runner *r, float t, uint32_t recordingTimestep)
 {
-    if(r->fusedStep) {
+    if(r->fusedStep || r->convStep) {
         StepArgs a{};
         a.base = nullptr; a.epoch = r->epoch; a.t = t; a.recordingTimestep = recordingTimestep;
         hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -1698,7 +1780,7 @@ static int stepNow(gennmi_runner *r, float t, uint32_t recordingTimestep)
             if(r->pending.size() >= 2048) { const int rc = drainTimers(r); if(rc) { return rc; } }
             const int rc = stamp(r, &e0); if(rc) { return rc; }
         }
-        const int rc = launchFusedStep(r, a);
+        const int rc = r->fusedStep ? launchFusedStep(r, a) : launchConvStep(r, a);
         if(rc) { return rc; }
         if(r->timing) { const int rc2 = stamp(r, &e1); if(rc2) { return rc2; } r->pending.push_back({e0, e1, 3}); }
         r->epoch++;
@@ -1898,7 +1980,7 @@ int gennmi_runner_get_info(gennmi_runner *r, uint32_t info[4])
     if(!r || !info) { return fail(GENNMI_EINVAL, "runner_get_info: null argument"); }
     if(!r->finalised) { return fail(GENNMI_ESTATE, "runner_get_info: runner not finalised"); }
     info[0] = (r->fusedStep ? 1u : 0u) | (r->resident ? 2u : 0u) | (r->neuronsPerLane > 1 ? 4u : 0u) | (r->ordered ? 8u : 0u)
-              | (r->combineSynapses ? 16u : 0u) | ((r->combineSynapses && r->combinePost) ? 32u : 0u) | (r->convMfmaBlocks ? 64u : 0u); info[1] = r->neuronBlocks; info[2] = r->preBlocks; info[3] = r->postBlocks;
+              | (r->combineSynapses ? 16u : 0u) | ((r->combineSynapses && r->combinePost) ? 32u : 0u) | (r->convMfmaBlocks ? 64u : 0u) | (r->convStep ? 128u : 0u); info[1] = r->neuronBlocks; info[2] = r->preBlocks; info[3] = r->postBlocks;
     return GENNMI_OK;
 }
 

@@ -96,6 +96,8 @@ struct NeuronGroupDev
     uint32_t *shadowSpk;                // [2][batch*N] engine-private double-buffered copy of the spike queue, or NULL
     uint32_t *shadowCnt;                // [2][batch]
     uint32_t *spikeBitmap;              // [batch][ceil(N/32)] engine-private bitmap of this step's spikes (populations at either end of a plastic projection), or NULL
+    size_t bitmapStride;                // != 0: two bitmaps this many words apart; the update after k completed steps writes copy (k + 1) & 1, so that a
+                                        //       kernel of the same launch can still read the spikes of the step before (copy k & 1)
     unsigned long long *aggEvent;       // look-back area of the spike-like event queues (groups with events), or NULL
     float *nextSpikeTime;               // spike sources: engine-private copy of spikeTimes[startSpike] per neuron (+inf: none left)
     size_t spikeTimesBytes;             // spike sources: bytes from spikeTimes to the end of its allocation (host bookkeeping)
@@ -185,7 +187,10 @@ struct ConvMfmaDev
     uint32_t kernPitch;                 // the kernel in LDS: [kh*kw*ic, rounded up to whole chunks of steps][kernPitch] floats
     uint32_t threshold;
     uint32_t numBatches;                // the grid is one-dimensional: block = rowGroup * numBatches + batch
-    uint32_t pad_;
+    uint32_t spikeWords;                // conv + neuron update in one kernel: words of a block's spike bitmap in LDS (behind patch and kernel)
+    uint32_t restBlocks;                // ... and blocks of the other populations' updates, shared out between the layer's work-groups
+    uint32_t restNeuronsPerLane, pad2_;
+    size_t bitmapStride;                // see NeuronGroupDev::bitmapStride: after k completed steps the layer reads copy k & 1 of srcBitmap
 };
 
 struct PostGroupDev

@@ -301,7 +301,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
         const uint32_t words = (n + 31) / 32;
         g.recordSpk[((size_t)st.recT * gridDim.y + batch) * words + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
     }
-    if(G.spikeBitmap && (lane & 31) == 0 && i < n) { G.spikeBitmap[(size_t)batch * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballot >> (lane & 32)); }
+    if(G.spikeBitmap && (lane & 31) == 0 && i < n) { G.spikeBitmap[((st.epoch + 1) & 1) * G.bitmapStride + (size_t)batch * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballot >> (lane & 32)); }
     __syncthreads();
 
     uint32_t blockCount = 0, waveOffset = 0;
@@ -430,21 +430,90 @@ void neuronUpdateKernel(const NeuronGroupDev * __restrict__ blocks, StepArgs arg
 // ------------------------------------------------------------------------------------------------
 constexpr uint32_t BULK_MAX_PSM = 2, BULK_MAX_CS = 1;
 
-template<int NPL>
-__device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t blockInKernel, uint32_t totalNeuronBlocks,
-                                               const Resolved &st, float dt, unsigned long long *agg, uint32_t *errorFlag)
+// What the update of a plain neuron needs of its group, read once into registers: the descriptor lives in global memory, and
+// behind every store the compiler would read its fields again (a store may alias anything), ten dependent scalar loads per neuron.
+struct PlainNeuron
 {
-    __shared__ uint32_t shWaveCount[BLOCK / WAVE];
+    uint32_t model;
+    float p[7];
+};
+__device__ __forceinline__ PlainNeuron plainNeuronOf(const gennmi_neuron_update_group_t &g)
+{
+    PlainNeuron c;
+    c.model = g.model;
+    #pragma unroll
+    for(int k = 0; k < 7; k++) { c.p[k] = g.params[k]; }
+    return c;
+}
+// sim code, threshold and reset of a LIF (neuronModels.h:220-257) or Izhikevich (:163-186) neuron from its summed input:
+// operations and their order as in neuronBody
+__device__ __forceinline__ bool plainNeuronStep(const PlainNeuron &c, float Isyn, float dt, float &v0, float &v1)
+{
+    bool spiked;
+    if(c.model == GENNMI_NEURON_LIF) {
+        if(v1 <= 0.0f) {
+            const float alpha = ((Isyn + c.p[0]) * c.p[1]) + c.p[2];
+            v0 = alpha - (c.p[3] * (alpha - v0));
+        }
+        else {
+            v1 -= dt;
+        }
+        spiked = (v1 <= 0.0f && v0 >= c.p[4]);
+        if(spiked) { v0 = c.p[5]; v1 = c.p[6]; }
+    }
+    else {
+        if(v0 >= 30.0f) {
+            v0 = c.p[2];
+            v1 += c.p[3];
+        }
+        v0 += 0.5f * (0.04f * v0 * v0 + 5.0f * v0 + 140.0f - v1 + Isyn) * dt;
+        v0 += 0.5f * (0.04f * v0 * v0 + 5.0f * v0 + 140.0f - v1 + Isyn) * dt;
+        v1 += c.p[0] * (c.p[1] * v0 - v1) * dt;
+        if(v0 > 30.0f) { v0 = 30.0f; }
+        spiked = (v0 >= 29.99f);
+    }
+    return spiked;
+}
+
+// (THREADS: threads of the calling work-group, all of which call; batch / numBatches: the grid's second dimension in the neuron kernels)
+template<int NPL, int THREADS = BLOCK>
+__device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t blockInKernel, uint32_t totalNeuronBlocks,
+                                               const Resolved &st, float dt, unsigned long long *agg, uint32_t *errorFlag,
+                                               uint32_t batch, uint32_t numBatches)
+{
+    __shared__ uint32_t shWaveCount[THREADS / WAVE];
     __shared__ uint32_t shPrefix;
     const gennmi_neuron_update_group_t &g = G.g;
-    const uint32_t batch = blockIdx.y;
     const uint32_t localBlock = blockInKernel - G.startBlock;
     const uint32_t n = g.numNeurons;
     const uint32_t lane = threadIdx.x & (WAVE - 1);
     const uint32_t wave = threadIdx.x / WAVE;
     const float t = st.t;
-    const uint32_t first = (localBlock * (BLOCK / WAVE) + wave) * (WAVE * NPL) + lane;      // this lane's neuron in chunk 0
+    const uint32_t first = (localBlock * (THREADS / WAVE) + wave) * (WAVE * NPL) + lane;      // this lane's neuron in chunk 0
     const uint32_t numPSM = g.numPSM, numCS = g.numCS;
+    // the group's constants and array addresses, read once (see PlainNeuron)
+    const PlainNeuron constants = plainNeuronOf(g);
+    const bool source = (constants.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY);
+    GLOBAL_AS float *var0 = asGlobal(g.var0), *var1 = asGlobal(g.var1);
+    GLOBAL_AS float *psmOut[BULK_MAX_PSM], *psmRing[BULK_MAX_PSM];
+    uint32_t psmD[BULK_MAX_PSM], psmKind[BULK_MAX_PSM];
+    float psmInit[BULK_MAX_PSM], psmDecay[BULK_MAX_PSM];
+    #pragma unroll
+    for(uint32_t m = 0; m < BULK_MAX_PSM; m++) {
+        const bool have = (m < numPSM);
+        psmOut[m] = have ? asGlobal(g.psm[m].outPost) : nullptr; psmRing[m] = have ? asGlobal(g.psm[m].denDelay) : nullptr;
+        psmD[m] = have ? g.psm[m].maxDenDelay : 0u; psmKind[m] = have ? g.psm[m].kind : 0u;
+        psmInit[m] = have ? g.psm[m].init : 0.0f; psmDecay[m] = have ? g.psm[m].expDecay : 0.0f;
+    }
+    const uint32_t csKind = numCS ? g.cs[0].kind : 0u, csSteps = numCS ? g.cs[0].arraySteps : 1u;
+    const float csAmp = numCS ? g.cs[0].amp : 0.0f;
+    GLOBAL_AS const float *csArray = numCS ? asGlobal(g.cs[0].array) : nullptr;
+    uint32_t *recordSpk = g.recordSpk, *spikeBitmap = G.spikeBitmap;
+    uint32_t *startSpikeArr = g.startSpike; const uint32_t *endSpikeArr = g.endSpike; const float *spikeTimesArr = g.spikeTimes;
+    float *nextSpikeTime = G.nextSpikeTime;
+    const size_t bitmapStride = G.bitmapStride;
+    uint32_t *spkQueue = g.spk, *spkCount = g.spkCnt;
+    const uint32_t groupBlocks = G.numBlocks, groupStart = G.startBlock;
 
     float l0[NPL], l1[NPL], lin[NPL][BULK_MAX_PSM], front[NPL][BULK_MAX_PSM], inj[NPL];
     bool spiked[NPL];
@@ -458,22 +527,21 @@ __device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t
         for(uint32_t m = 0; m < BULK_MAX_PSM; m++) { lin[j][m] = front[j][m] = 0.0f; }
         spiked[j] = false;
         if(i < n) {
-            if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
-                l0[j] = asGlobal(G.nextSpikeTime)[bi];
+            if(source) {
+                l0[j] = asGlobal(nextSpikeTime)[bi];
             }
             else {
-                l0[j] = asGlobal(g.var0)[bi]; l1[j] = asGlobal(g.var1)[bi];
+                l0[j] = var0[bi]; l1[j] = var1[bi];
                 #pragma unroll
                 for(uint32_t m = 0; m < BULK_MAX_PSM; m++) {
                     if(m < numPSM) {
-                        lin[j][m] = asGlobal(g.psm[m].outPost)[bi];
-                        const uint32_t D = g.psm[m].maxDenDelay;
-                        if(D) { front[j][m] = asGlobal(g.psm[m].denDelay)[((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i]; }
+                        lin[j][m] = psmOut[m][bi];
+                        const uint32_t D = psmD[m];
+                        if(D) { front[j][m] = psmRing[m][((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i]; }
                     }
                 }
                 if(numCS) {
-                    inj[j] = (g.cs[0].kind == GENNMI_CS_DC) ? g.cs[0].amp
-                                                            : asGlobal(g.cs[0].array)[(size_t)modStep(st.epoch, g.cs[0].arraySteps) * n + i];
+                    inj[j] = (csKind == GENNMI_CS_DC) ? csAmp : csArray[(size_t)modStep(st.epoch, csSteps) * n + i];
                 }
             }
         }
@@ -484,12 +552,12 @@ __device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t
         const uint32_t i = first + j * WAVE;
         const size_t bi = (size_t)batch * n + i;
         if(i >= n) { continue; }
-        if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
+        if(source) {
             spiked[j] = (t >= l0[j]);
             if(spiked[j]) {
-                const uint32_t startSpike = g.startSpike[bi] + 1;
-                g.startSpike[bi] = startSpike;
-                G.nextSpikeTime[bi] = (startSpike != g.endSpike[bi]) ? g.spikeTimes[startSpike] : INFINITY;
+                const uint32_t startSpike = startSpikeArr[bi] + 1;
+                startSpikeArr[bi] = startSpike;
+                nextSpikeTime[bi] = (startSpike != endSpikeArr[bi]) ? spikeTimesArr[startSpike] : INFINITY;
             }
             continue;
         }
@@ -498,45 +566,24 @@ __device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t
         for(uint32_t m = 0; m < BULK_MAX_PSM; m++) {
             if(m < numPSM) {
                 float linSyn = lin[j][m];
-                const uint32_t D = g.psm[m].maxDenDelay;
+                const uint32_t D = psmD[m];
                 if(D) { linSyn += front[j][m]; }
-                if(g.psm[m].kind == GENNMI_PSM_EXPCURR) {
-                    Isyn += g.psm[m].init * linSyn;
-                    linSyn *= g.psm[m].expDecay;
+                if(psmKind[m] == GENNMI_PSM_EXPCURR) {
+                    Isyn += psmInit[m] * linSyn;
+                    linSyn *= psmDecay[m];
                 }
                 else {
                     Isyn += linSyn;
                     linSyn = 0.0f;
                 }
-                if(D) { asGlobal(g.psm[m].denDelay)[((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i] = 0.0f; }
-                asGlobal(g.psm[m].outPost)[bi] = linSyn;
+                if(D) { psmRing[m][((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i] = 0.0f; }
+                psmOut[m][bi] = linSyn;
             }
         }
         if(numCS) { Isyn += inj[j]; }
         float v0 = l0[j], v1 = l1[j];
-        if(g.model == GENNMI_NEURON_LIF) {
-            if(v1 <= 0.0f) {
-                const float alpha = ((Isyn + g.params[0]) * g.params[1]) + g.params[2];
-                v0 = alpha - (g.params[3] * (alpha - v0));
-            }
-            else {
-                v1 -= dt;
-            }
-            spiked[j] = (v1 <= 0.0f && v0 >= g.params[4]);
-            if(spiked[j]) { v0 = g.params[5]; v1 = g.params[6]; }
-        }
-        else {
-            if(v0 >= 30.0f) {
-                v0 = g.params[2];
-                v1 += g.params[3];
-            }
-            v0 += 0.5f * (0.04f * v0 * v0 + 5.0f * v0 + 140.0f - v1 + Isyn) * dt;
-            v0 += 0.5f * (0.04f * v0 * v0 + 5.0f * v0 + 140.0f - v1 + Isyn) * dt;
-            v1 += g.params[0] * (g.params[1] * v0 - v1) * dt;
-            if(v0 > 30.0f) { v0 = 30.0f; }
-            spiked[j] = (v0 >= 29.99f);
-        }
-        g.var0[bi] = v0; g.var1[bi] = v1;
+        spiked[j] = plainNeuronStep(constants, Isyn, dt, v0, v1);
+        var0[bi] = v0; var1[bi] = v1;
     }
     if(localBlock == 0 && batch == 0 && threadIdx.x < g.numPSM) {
         const gennmi_psm_t &psm = g.psm[threadIdx.x];
@@ -552,37 +599,37 @@ __device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t
         const unsigned long long ballot = __ballot(spiked[j]);
         rank[j] = waveCount + __popcll(ballot & ((1ull << lane) - 1ull));
         waveCount += __popcll(ballot);
-        if(g.recordSpk && (lane & 31) == 0 && i < n) {
+        if(recordSpk && (lane & 31) == 0 && i < n) {
             const uint32_t words = (n + 31) / 32;
-            g.recordSpk[((size_t)st.recT * gridDim.y + batch) * words + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
+            recordSpk[((size_t)st.recT * numBatches + batch) * words + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
         }
-        if(G.spikeBitmap && (lane & 31) == 0 && i < n) { G.spikeBitmap[(size_t)batch * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballot >> (lane & 32)); }
+        if(spikeBitmap && (lane & 31) == 0 && i < n) { spikeBitmap[((st.epoch + 1) & 1) * bitmapStride + (size_t)batch * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballot >> (lane & 32)); }
     }
     if(lane == 0) { shWaveCount[wave] = waveCount; }
     __syncthreads();
     uint32_t blockCount = 0, waveOffset = 0;
     #pragma unroll
-    for(uint32_t w = 0; w < BLOCK / WAVE; w++) {
+    for(uint32_t w = 0; w < THREADS / WAVE; w++) {
         const uint32_t c = shWaveCount[w];
         if(w < wave) { waveOffset += c; }
         blockCount += c;
     }
-    unsigned long long *groupAgg = agg + (size_t)totalNeuronBlocks * gridDim.y;
-    const uint32_t prefix = blockQueueOffset(blockCount, localBlock, G.numBlocks, (size_t)batch * totalNeuronBlocks + G.startBlock, agg, groupAgg,
+    unsigned long long *groupAgg = agg + (size_t)totalNeuronBlocks * numBatches;
+    const uint32_t prefix = blockQueueOffset(blockCount, localBlock, groupBlocks, (size_t)batch * totalNeuronBlocks + groupStart, agg, groupAgg,
                                              (uint32_t)(st.epoch + 1), &shPrefix, errorFlag);
     if(prefix == 0xFFFFFFFFu) { return; }
     #pragma unroll
     for(int j = 0; j < NPL; j++) {
-        if(spiked[j]) { g.spk[(size_t)batch * n + prefix + waveOffset + rank[j]] = first + j * WAVE; }
+        if(spiked[j]) { spkQueue[(size_t)batch * n + prefix + waveOffset + rank[j]] = first + j * WAVE; }
     }
-    if(localBlock == G.numBlocks - 1 && threadIdx.x == 0) { g.spkCnt[batch] = prefix + blockCount; }
+    if(localBlock == groupBlocks - 1 && threadIdx.x == 0) { spkCount[batch] = prefix + blockCount; }
 }
 
 template<int NPL>
 __global__ __launch_bounds__(BLOCK)
 void neuronBulkKernel(const NeuronGroupDev * __restrict__ blocks, StepArgs args, float dt, unsigned long long *agg, uint32_t *errorFlag)
 {
-    neuronBulkBody<NPL>(blocks[blockIdx.x], blockIdx.x, gridDim.x, resolve(args, dt), dt, agg, errorFlag);
+    neuronBulkBody<NPL>(blocks[blockIdx.x], blockIdx.x, gridDim.x, resolve(args, dt), dt, agg, errorFlag, blockIdx.y, gridDim.y);
 }
 
 // One launch per timestep for networks whose projections all go through the dendritic-delay ring: the

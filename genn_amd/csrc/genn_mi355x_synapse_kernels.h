@@ -757,29 +757,39 @@ constexpr int CONV_MFMA_THREADS = 512;       // eight wavefronts: a compute unit
 constexpr int CONV_MFMA_STEPS = 72;         // steps of the (tap, channel) sum per unrolled chunk of the inner loop
 constexpr int CONV_MFMA_AHEAD = 6;          // steps whose operands are fetched ahead of the matrix instructions (divides the above)
 
-__global__ __launch_bounds__(CONV_MFMA_THREADS)
-void presynapticConvMfmaKernel(const ConvMfmaDev * __restrict__ blocks, uint32_t mfmaBlocks, const PreGroupDev * __restrict__ scatter,
-                               StepArgs args, float dt, unsigned long long *eventCounter)
+// what a block does with a finished tile of 32 pixels x 32 output channels: here, add it to outPost
+struct ConvAddToOutPost
 {
-    extern __shared__ float shConvM[];
-    const ConvMfmaDev &G = blocks[0];
-    const gennmi_presynaptic_update_group_t &g = G.g;
-    // Blocks are numbered batch-first (block = index * numBatches + batch), so that consecutive work-groups, which go to
-    // consecutive XCDs, differ in batch.  Behind the blocks of the dense path come those of the scatter path, which takes
-    // the steps too quiet for it: one launch, and the device decides which of the two does the work.
-    const uint32_t numBatches = G.numBatches;
-    const uint32_t batch = blockIdx.x % numBatches;
-    if(blockIdx.x >= mfmaBlocks) {
-        const uint32_t b = (blockIdx.x - mfmaBlocks) / numBatches;
-        presynapticBody(scatter[b], b, batch, numBatches, resolve(args, dt), dt, eventCounter);
-        return;
+    GLOBAL_AS float *outPost;           // of this batch
+    uint32_t ow, oc;
+    __device__ __forceinline__ void prefetch(uint32_t, uint32_t, uint32_t, uint32_t, uint32_t) {}
+    __device__ __forceinline__ void finish(const f32x16 &acc, uint32_t, uint32_t y, uint32_t x0, uint32_t o, uint32_t half)
+    {
+        // one atomic without return per element and step, so the result does not depend on their order (a read-modify-write
+        // by the owning lane measured no faster)
+        #pragma unroll
+        for(int v = 0; v < 16; v++) {
+            const uint32_t x = x0 + 8 * (v / 4) + 4 * half + (v % 4);
+            if(x < ow && o < oc && acc[v] != 0.0f) { atomicAddF32(&outPost[((size_t)y * ow + x) * oc + o], acc[v]); }
+        }
     }
-    const uint32_t rowGroup = blockIdx.x / numBatches;
+};
+
+// floats of LDS that a block's input patch and its copy of the kernel take (what follows them belongs to the caller)
+__device__ __forceinline__ uint32_t convMfmaLdsFloats(const ConvMfmaDev &G)
+{
+    const uint32_t K = (uint32_t)(G.g.conv[0] * G.g.conv[1] * G.g.conv[4]), steps = (K + 1) / 2;
+    return (uint32_t)G.g.conv[4] * G.planePitch + 2 * ((steps + CONV_MFMA_STEPS - 1) / CONV_MFMA_STEPS) * CONV_MFMA_STEPS * G.kernPitch;
+}
+
+// the output rows [rowGroup * rowsPerBlock, ...) of one batch, by all THREADS threads of a block; `epoch`: completed steps
+template<int THREADS, typename Epilogue>
+__device__ __forceinline__ void convMfmaBlock(const ConvMfmaDev &G, uint32_t rowGroup, uint32_t batch, unsigned long long epoch, float *lds,
+                                              Epilogue &epilogue, unsigned long long *eventCounter)
+{
+    const gennmi_presynaptic_update_group_t &g = G.g;
     const int kh = g.conv[0], kw = g.conv[1], ih = g.conv[2], iw = g.conv[3], ic = g.conv[4];
     const int oh = g.conv[5], ow = g.conv[6], oc = g.conv[7];
-    const uint32_t numDiag = (uint32_t)(kh * kw * oc);
-    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
-    if((unsigned long long)numSpikes * numDiag < G.threshold) { return; }      // the scatter kernel took this step
     const uint32_t planePitch = G.planePitch, patchPitch = G.patchPitch, kernPitch = G.kernPitch;
     const int y0 = (int)(rowGroup * G.rowsPerBlock);
     const int rows = min((int)G.rowsPerBlock, oh - y0);
@@ -787,17 +797,21 @@ void presynapticConvMfmaKernel(const ConvMfmaDev * __restrict__ blocks, uint32_t
     const uint32_t K = (uint32_t)(kh * kw * ic), steps = (K + 1) / 2;
     // kernel rows in LDS: whole chunks of steps, so that the unrolled loop needs no guard (rows beyond K are zero)
     const uint32_t kernRows = 2 * ((steps + CONV_MFMA_STEPS - 1) / CONV_MFMA_STEPS) * CONV_MFMA_STEPS;
-    float *patch = shConvM;
+    float *patch = lds;
     float *kern = patch + (size_t)ic * planePitch;
     const uint32_t lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const uint32_t half = lane >> 5, col = lane & 31;
-    GLOBAL_AS const uint32_t *bitmap = asGlobal(G.srcBitmap) + (size_t)batch * ((g.numSrcNeurons + 31) / 32);
+    GLOBAL_AS const uint32_t *bitmap = asGlobal(G.srcBitmap) + (epoch & 1) * G.bitmapStride + (size_t)batch * ((g.numSrcNeurons + 31) / 32);
     GLOBAL_AS const float *kernel = asGlobal(g.g);
-    GLOBAL_AS float *outPost = asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons;
     const uint32_t xTiles = ((uint32_t)ow + 31) / 32, oTiles = ((uint32_t)oc + 31) / 32;
     const uint32_t numTiles = (uint32_t)rows * xTiles * oTiles;
 
-    // ---- requested before anything is waited for: this thread's first words of the bitmap, the kernel
+    // ---- requested before anything is waited for: what the epilogue wants of the wavefront's first tile, this thread's first
+    // words of the bitmap, the kernel
+    if(wave < numTiles) {
+        const uint32_t r = wave / (xTiles * oTiles), x0 = ((wave / oTiles) % xTiles) * 32, n0 = (wave % oTiles) * 32;
+        epilogue.prefetch(r, (uint32_t)y0 + r, x0, n0 + col, half);
+    }
     const int patchRows = rows + kh - 1;
     const uint32_t patchElems = (uint32_t)patchRows * patchPitch;
     auto pixelOf = [&](uint32_t e, int &inRow, int &inCol) -> bool {
@@ -805,9 +819,9 @@ void presynapticConvMfmaKernel(const ConvMfmaDev * __restrict__ blocks, uint32_t
         inRow = y0 - PH + r; inCol = c - PW;
         return (e < patchElems && inRow >= 0 && inRow < ih && inCol >= 0 && inCol < iw);
     };
-    // (a thread's first two pixels: all there is to do for patches of up to 512 elements)
+    // (a thread's first two pixels: all there is to do for patches of up to 2 x THREADS elements)
     int inRow0, inCol0, inRow1, inCol1;
-    const bool inside0 = pixelOf(threadIdx.x, inRow0, inCol0), inside1 = pixelOf(threadIdx.x + CONV_MFMA_THREADS, inRow1, inCol1);
+    const bool inside0 = pixelOf(threadIdx.x, inRow0, inCol0), inside1 = pixelOf(threadIdx.x + THREADS, inRow1, inCol1);
     const uint32_t first0 = inside0 ? (uint32_t)((inRow0 * iw + inCol0) * ic) : 0u, first1 = inside1 ? (uint32_t)((inRow1 * iw + inCol1) * ic) : 0u;
     const uint32_t word0 = bitmap[first0 >> 5], word1 = bitmap[first1 >> 5];
 
@@ -817,45 +831,44 @@ void presynapticConvMfmaKernel(const ConvMfmaDev * __restrict__ blocks, uint32_t
         const uint32_t quads = K * (uint32_t)oc / 4, allQuads = kernRows * kernPitch / 4;
         GLOBAL_AS const f32x4 *src = reinterpret_cast<GLOBAL_AS const f32x4*>(kernel);
         f32x4 *dst = reinterpret_cast<f32x4*>(kern);
-        for(uint32_t q0 = 0; q0 < allQuads; q0 += 8 * CONV_MFMA_THREADS) {
+        for(uint32_t q0 = 0; q0 < allQuads; q0 += 8 * THREADS) {
             f32x4 w[8];
             #pragma unroll
-            for(int u = 0; u < 8; u++) { const uint32_t q = q0 + u * CONV_MFMA_THREADS + threadIdx.x; w[u] = src[min(q, quads - 1)]; }
+            for(int u = 0; u < 8; u++) { const uint32_t q = q0 + u * THREADS + threadIdx.x; w[u] = src[min(q, quads - 1)]; }
             #pragma unroll
             for(int u = 0; u < 8; u++) {
-                const uint32_t q = q0 + u * CONV_MFMA_THREADS + threadIdx.x;
+                const uint32_t q = q0 + u * THREADS + threadIdx.x;
                 const f32x4 zero = {0, 0, 0, 0};
                 if(q < allQuads) { dst[q] = (q < quads) ? w[u] : zero; }
             }
         }
     }
     else {
-        for(uint32_t e0 = 0; e0 < kernRows * kernPitch; e0 += 8 * CONV_MFMA_THREADS) {
+        for(uint32_t e0 = 0; e0 < kernRows * kernPitch; e0 += 8 * THREADS) {
             float w[8];
             #pragma unroll
             for(int u = 0; u < 8; u++) {
-                const uint32_t e = e0 + u * CONV_MFMA_THREADS + threadIdx.x;
+                const uint32_t e = e0 + u * THREADS + threadIdx.x;
                 const uint32_t k = e / kernPitch, o = e - k * kernPitch;
                 w[u] = kernel[(size_t)min(k, K - 1) * oc + min(o, (uint32_t)oc - 1)] * ((k < K && o < (uint32_t)oc) ? 1.0f : 0.0f);
             }
             #pragma unroll
             for(int u = 0; u < 8; u++) {
-                const uint32_t e = e0 + u * CONV_MFMA_THREADS + threadIdx.x;
+                const uint32_t e = e0 + u * THREADS + threadIdx.x;
                 if(e < kernRows * kernPitch) { kern[e] = w[u]; }
             }
         }
     }
-
     // ---- input patch: bit (row * iw + col) * ic + ch of the source's bitmap -> patch[ch][r][c].  A pixel's spikes are
     // counted as events by the block whose output rows include the pixel's row (the last block takes the rows below):
     // every spike reaches kh * kw * oc targets less what falls outside the output.
     unsigned long long events = 0;
     const bool lastBlock = (y0 + rows >= oh);
-    for(uint32_t e = threadIdx.x; e < patchElems; e += CONV_MFMA_THREADS) {
+    for(uint32_t e = threadIdx.x; e < patchElems; e += THREADS) {
         int inRow, inCol;
         const bool inside = pixelOf(e, inRow, inCol);
         const uint32_t id0 = inside ? (uint32_t)((inRow * iw + inCol) * ic) : 0u;
-        uint32_t wordIdx = id0 >> 5, word = (e == threadIdx.x) ? word0 : (e == threadIdx.x + CONV_MFMA_THREADS) ? word1 : bitmap[wordIdx], fired = 0;
+        uint32_t wordIdx = id0 >> 5, word = (e == threadIdx.x) ? word0 : (e == threadIdx.x + THREADS) ? word1 : bitmap[wordIdx], fired = 0;
         for(int ch = 0; ch < ic; ch++) {
             const uint32_t id = id0 + (uint32_t)ch;
             if(inside && (id >> 5) != wordIdx) { wordIdx = id >> 5; word = bitmap[wordIdx]; }
@@ -882,10 +895,11 @@ void presynapticConvMfmaKernel(const ConvMfmaDev * __restrict__ blocks, uint32_t
         const uint32_t ta = tap / (uint32_t)kw;
         return ch * planePitch + ta * patchPitch + (tap - ta * (uint32_t)kw);
     };
-    for(uint32_t tile = wave; tile < numTiles; tile += CONV_MFMA_THREADS / WAVE) {
+    for(uint32_t tile = wave; tile < numTiles; tile += THREADS / WAVE) {
         const uint32_t r = tile / (xTiles * oTiles), x0 = ((tile / oTiles) % xTiles) * 32, n0 = (tile % oTiles) * 32;
         const uint32_t y = (uint32_t)y0 + r, o = n0 + col;
         f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        if(tile != wave) { epilogue.prefetch(r, y, x0, o, half); }
         const float *aBase = patch + r * patchPitch + x0 + col;
         for(uint32_t s0 = 0; s0 < steps; s0 += CONV_MFMA_STEPS) {
             const int evenLo = (int)patchOffsetOf(2 * (s0 + lane)), oddLo = (int)patchOffsetOf(2 * (s0 + lane) + 1);
@@ -917,16 +931,36 @@ void presynapticConvMfmaKernel(const ConvMfmaDev * __restrict__ blocks, uint32_t
             }
         }
         // register v of lane (half, col) holds D[i][j] with i = 8 * (v / 4) + 4 * half + v % 4, j = col: the 32 lanes of a
-        // half add to the 32 consecutive channels of one pixel (one atomic without return per element and step, so the
-        // result does not depend on their order; a read-modify-write by the owning lane measured no faster)
-        #pragma unroll
-        for(int v = 0; v < 16; v++) {
-            const uint32_t x = x0 + 8 * (v / 4) + 4 * half + (v % 4);
-            if(x < (uint32_t)ow && o < (uint32_t)oc && acc[v] != 0.0f) { atomicAddF32(&outPost[((size_t)y * ow + x) * oc + o], acc[v]); }
-        }
+        // half hold the 32 consecutive channels of one pixel
+        epilogue.finish(acc, r, y, x0, o, half);
     }
     for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
     if(lane == 0 && events) { atomicAdd(eventCounter, events); }
+}
+
+__global__ __launch_bounds__(CONV_MFMA_THREADS)
+void presynapticConvMfmaKernel(const ConvMfmaDev * __restrict__ blocks, uint32_t mfmaBlocks, const PreGroupDev * __restrict__ scatter,
+                               StepArgs args, float dt, unsigned long long *eventCounter)
+{
+    extern __shared__ float shConvM[];
+    const ConvMfmaDev &G = blocks[0];
+    const gennmi_presynaptic_update_group_t &g = G.g;
+    // Blocks are numbered batch-first (block = index * numBatches + batch), so that consecutive work-groups, which go to
+    // consecutive XCDs, differ in batch.  Behind the blocks of the dense path come those of the scatter path, which takes
+    // the steps too quiet for it: one launch, and the device decides which of the two does the work.
+    const uint32_t numBatches = G.numBatches;
+    const uint32_t batch = blockIdx.x % numBatches;
+    const Resolved st = resolve(args, dt);
+    if(blockIdx.x >= mfmaBlocks) {
+        const uint32_t b = (blockIdx.x - mfmaBlocks) / numBatches;
+        presynapticBody(scatter[b], b, batch, numBatches, st, dt, eventCounter);
+        return;
+    }
+    const uint32_t numDiag = (uint32_t)(g.conv[0] * g.conv[1] * g.conv[7]);
+    const uint32_t numSpikes = asGlobal(g.srcSpkCnt)[batch];
+    if((unsigned long long)numSpikes * numDiag < G.threshold) { return; }      // the scatter kernel took this step
+    ConvAddToOutPost epilogue{asGlobal(g.outPost) + (size_t)batch * g.numTrgNeurons, (uint32_t)g.conv[6], (uint32_t)g.conv[7]};
+    convMfmaBlock<CONV_MFMA_THREADS>(G, blockIdx.x / numBatches, batch, st.epoch, shConvM, epilogue, eventCounter);
 }
 
 // bitmap of a population's spike queue, for callers that wrote the queue themselves (the neuron update keeps it otherwise)

@@ -1024,7 +1024,7 @@ class GeNNModel:
         _abi.check(_abi.load().gennmi_runner_get_info(self._runner, C.byref(info)))
         return {"single_launch_step": bool(info[0] & 1), "resident_plan": bool(info[0] & 2), "bulk_neuron_kernel": bool(info[0] & 4), "ordered_accumulation": bool(info[0] & 8),
                 "combined_synapse_launch": bool(info[0] & 16), "postsynaptic_in_combined_launch": bool(info[0] & 32),
-                "conv_on_matrix_cores": bool(info[0] & 64), "neuron_blocks": info[1], "presyn_blocks": info[2], "postsyn_blocks": info[3]}
+                "conv_on_matrix_cores": bool(info[0] & 64), "conv_step_in_one_launch": bool(info[0] & 128), "neuron_blocks": info[1], "presyn_blocks": info[2], "postsyn_blocks": info[3]}
 
     # timing counters under PyGeNN's names (pygenn/genn_model.py:292-326), in seconds, accumulated while `timing_enabled`
     def _times(self):

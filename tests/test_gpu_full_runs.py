@@ -124,11 +124,13 @@ def test_toeplitz_conv_full_run_batch16(monkeypatch):
     """Config 5: 64x64x16 sources -> 64x64x32 LIF through Conv2D 3x3, batch 16, dt 1 ms, 500 steps: every batch against a
     batch-1 oracle run fed that batch's input spike trains (the CPU backend has no batches).
 
-    The layer is run twice.  On the event-driven kernels every output element receives its contributions in queue order,
-    the CPU backend's order, so the rasters of all 500 steps must be identical bit for bit.  On the matrix cores (the
-    default for busy steps) the same products are summed in another order, so a neuron whose potential lands within
-    rounding of the threshold may fire a step apart (measured: the first such neuron at step 78 of one batch): rasters
-    identical over the first 50 steps, then every batch's rate within 2 % and the event total within 2 %."""
+    The layer is run three times: on the matrix cores with the whole step in one launch (the default: the neuron model
+    applied to the layer's accumulators), on the matrix cores with the layer's kernel followed by the neuron kernel, and on
+    the event-driven kernels.  Every one of them sums a neuron's inputs in another order than the CPU backend (matrix
+    instructions, or atomics in quiet steps), so a neuron whose potential lands within rounding of the threshold may fire a
+    step apart (measured: the first such neuron at step 78 of one batch, on all three): rasters identical over the first
+    50 steps, then every batch's rate within 2 % and the event total within 2 %.  The two matrix-core plans compute the
+    same sums and must agree with each other bit for bit."""
     B, steps = 16, 500
     nets = [configs.conv_toeplitz(steps=steps, batch_index=b) for b in range(B)]
     times = np.concatenate([n.pop("In").spike_times for n in nets])
@@ -139,12 +141,15 @@ def test_toeplitz_conv_full_run_batch16(monkeypatch):
     batched.pop("In").vars = {"startSpike": start, "endSpike": end}
     batched.pop("In").spike_times = times
     runs = {}
-    for mode in ("matrix cores", "event-driven"):
+    for mode in ("matrix cores", "matrix cores, two launches", "event-driven"):
+        if mode == "matrix cores, two launches":
+            monkeypatch.setenv("GENNMI_CONV_STEP", "0")         # (read when the runner is finalised)
         if mode == "event-driven":
-            monkeypatch.setenv("GENNMI_CONV_MFMA", "0")         # (read when the runner is finalised)
+            monkeypatch.setenv("GENNMI_CONV_MFMA", "0")
         model = model_from_net(batched, batch_size=B)
         model.load(num_recording_timesteps=steps)
-        assert model.runner_info()["conv_on_matrix_cores"] == (mode == "matrix cores")
+        assert model.runner_info()["conv_on_matrix_cores"] == (mode != "event-driven")
+        assert model.runner_info()["conv_step_in_one_launch"] == (mode == "matrix cores")
         model.run(steps)
         model.pull_recording_buffers_from_device()
         runs[mode] = ({name: model.neuron_populations[name].vars["recordSpk"].view.copy() for name in ("In", "Out")}, model.synaptic_event_count)
@@ -171,9 +176,11 @@ def test_toeplitz_conv_full_run_batch16(monkeypatch):
                 rate_got = got.sum() / n
                 assert abs(rate_got - rate_want) <= RATE_TOL * rate_want, f"{mode}, batch {b}, {name}: {rate_got:.4f} vs {rate_want:.4f} spikes per neuron"
         oracle.close()
-    print(f"config 5: rasters of all {B} batches identical for the first {identical_until['event-driven']} (event-driven kernels) / "
-          f"{identical_until['matrix cores']} (matrix cores, {flipped['matrix cores']} raster bits differ in all) of {steps} steps", flush=True)
-    assert identical_until["event-driven"] == steps, f"event-driven kernels: rasters differ from step {identical_until['event-driven']}"
-    assert identical_until["matrix cores"] >= 50, f"matrix cores: rasters differ from step {identical_until['matrix cores']}"
+    print("config 5: rasters of all %d batches identical to the oracle's for the first " % B
+          + ", ".join(f"{identical_until[m]} ({m}: {flipped[m]} raster bits differ in all)" for m in runs) + f" of {steps} steps", flush=True)
+    for mode in runs:
+        assert identical_until[mode] >= 50, f"{mode}: rasters differ from step {identical_until[mode]}"
+    for name in ("In", "Out"):
+        assert np.array_equal(runs["matrix cores"][0][name], runs["matrix cores, two launches"][0][name]), f"the two matrix-core plans differ in {name}"
     for mode, (_, count) in runs.items():
         assert abs(count - events) <= EVENT_TOL * events, mode

@@ -209,6 +209,7 @@ def test_toeplitz_conv_full_size_batch16():
     batched.pop("In").spike_times = times
     model = model_from_net(batched, batch_size=B)
     model.load(num_recording_timesteps=steps)
+    assert model.runner_info()["conv_step_in_one_launch"]
     model.run(steps)
     model.pull_recording_buffers_from_device()
     v = model.neuron_populations["Out"].vars["V"].pull_from_device().reshape(B, -1)

@@ -199,17 +199,27 @@ def test_toeplitz_conv_on_matrix_cores(h, w, ic, oc, k, monkeypatch):
     assert counts["Out"] > 50 and counts["In"] > 5 * h * w * ic
     assert model.synaptic_event_count == oracle.events()
     assert model.runner_info()["conv_on_matrix_cores"]
-    # the event-driven kernels on the same network: same rasters, same event count
-    monkeypatch.setenv("GENNMI_CONV_MFMA", "0")
-    other = model_from_net(net)
-    other.load(num_recording_timesteps=60)
-    assert not other.runner_info()["conv_on_matrix_cores"]
-    other.run(60)
-    other.synchronize()
-    assert other.synaptic_event_count == model.synaptic_event_count
-    for p in net.pops:
-        assert np.array_equal(other.neuron_populations[p.name].current_spikes[0], model.neuron_populations[p.name].current_spikes[0])
-    other.unload()
+    # The whole step is one launch (postsynaptic and neuron model applied to the layer's accumulators) where a work-group's
+    # neurons start on a word of the recording bitmap: two of the four shapes, one of them with 40 output channels, so that
+    # a pixel's channels straddle the words of the work-group's spike bitmap.
+    one_launch = model.runner_info()["conv_step_in_one_launch"]
+    assert one_launch == ((w * oc) % 32 == 0)
+    # the same network with the layer's kernel and the neuron kernel launched one after the other, and on the event-driven
+    # kernels: same rasters, same event count
+    for switch, flag in (("GENNMI_CONV_STEP", "conv_step_in_one_launch"), ("GENNMI_CONV_MFMA", "conv_on_matrix_cores")):
+        monkeypatch.setenv(switch, "0")
+        other = model_from_net(net)
+        other.load(num_recording_timesteps=60)
+        assert not other.runner_info()[flag]
+        other.run(60)
+        other.synchronize()
+        assert other.synaptic_event_count == model.synaptic_event_count
+        for p in net.pops:
+            assert np.array_equal(other.neuron_populations[p.name].current_spikes[0], model.neuron_populations[p.name].current_spikes[0])
+        model.pull_recording_buffers_from_device(); other.pull_recording_buffers_from_device()
+        for p in net.pops:
+            assert np.array_equal(other.neuron_populations[p.name].vars["recordSpk"].view, model.neuron_populations[p.name].vars["recordSpk"].view), p.name
+        other.unload()
     model.unload()
 
 
