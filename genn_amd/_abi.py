@@ -111,6 +111,10 @@ SYMBOLS = {
     "gennmi_unregister_mirror": (C.c_int, [C.c_void_p]),
     "gennmi_mirror_device_pointer": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
     "gennmi_push_mirrors": (C.c_int, []),
+    "gennmi_register_device_array": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "gennmi_mirrors_begin_initialisation": (C.c_int, []),
+    "gennmi_mirror_device_initialised": (C.c_int, [C.c_void_p]),
+    "gennmi_mirror_ensure_host": (C.c_int, [C.c_void_p]),
     "gennmi_step": (C.c_int, [C.c_void_p, C.c_float, C.c_uint32]),
     "gennmi_synchronize": (C.c_int, []),
     "gennmi_note_device_write": (C.c_int, [C.c_void_p, C.c_size_t]),
@@ -129,11 +133,30 @@ SYMBOLS = {
     "gennmi_build_remap": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "gennmi_max_col_length": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]),
     "gennmi_max_col_length_static": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p]),
+    # generated code objects behind the C ABI (bound by generated C++ host code; listed so that the table and the header agree)
+    "gennmi_program_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_void_p, C.c_uint32]),
+    "gennmi_program_destroy": (C.c_int, [C.c_void_p]),
+    "gennmi_program_load_module": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_uint32)]),
+    "gennmi_program_get_kernel": (C.c_int, [C.c_void_p, C.c_uint32, C.c_char_p, C.POINTER(C.c_uint32)]),
+    "gennmi_program_error_flag": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "gennmi_program_add_launch": (C.c_int, [C.c_void_p, C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_size_t, C.c_int]),
+    "gennmi_program_clear_phases": (C.c_int, [C.c_void_p]),
+    "gennmi_program_update": (C.c_int, [C.c_void_p, C.c_int, C.c_double, C.c_uint32]),
+    "gennmi_program_launch": (C.c_int, [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_size_t, C.c_double,
+                                        C.c_ulonglong, C.c_int]),
+    "gennmi_program_synchronize": (C.c_int, [C.c_void_p]),
+    "gennmi_program_set_timing": (C.c_int, [C.c_void_p, C.c_int]),
+    "gennmi_program_get_time": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_double)]),
+    "gennmi_program_get_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_ulonglong * 4)]),
     "gennmi_init_var": (C.c_int, [C.c_void_p, C.c_uint32, C.c_size_t, C.c_uint32, C.POINTER(C.c_double * 4), C.c_uint64, C.c_uint32]),
     "gennmi_init_sparse_fixed_probability": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_double, C.c_int, C.c_uint64, C.c_uint32,
                                                        C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]),
     "gennmi_init_sparse_fixed_number_post": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_uint64, C.c_uint32,
                                                        C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]),
+    "gennmi_init_sparse_fixed_number_pre": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint32,
+                                                      C.c_void_p, C.c_void_p, C.POINTER(C.c_uint32)]),
+    "gennmi_init_sparse_conv2d": (C.c_int, [C.POINTER(C.c_int32), C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                            C.POINTER(C.c_uint32)]),
     "gennmi_init_sparse_one_to_one": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]),
     "gennmi_philox4x32": (C.c_int, [C.POINTER(C.c_uint32 * 4), C.POINTER(C.c_uint32 * 2), C.POINTER(C.c_uint32 * 4)]),
     "gennmi_init_random_words": (C.c_int, [C.c_void_p, C.c_size_t, C.c_uint64, C.c_uint32]),

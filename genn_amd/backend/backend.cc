@@ -2,6 +2,7 @@
 #include "backend.h"
 #include "optimiser.h"
 
+#include <sys/mman.h>
 #include <algorithm>
 #include <cctype>
 #include <cstdio>
@@ -44,9 +45,12 @@ void check(int rc, const char *what)
 }
 
 //--------------------------------------------------------------------------
-// Array: a host buffer (always present: generated initialisation code and merged groups work on host pointers)
-// mirrored by a device buffer; the pair is registered with the device library so generated code can translate
-// pointers.  Counterpart of the Array classes of the reference's backends (hip/backend.cc:61-236).
+// Array: a host buffer (generated initialisation code and merged groups work on host pointers) mirrored by a device
+// buffer; the pair is registered with the device library so generated code can translate pointers.  Counterpart of the
+// Array classes of the reference's backends (hip/backend.cc:61-236).  An array the model places on the device only
+// (VarLocation::DEVICE) gets no host memory there; here it gets address space that is committed only where host code
+// touches it and given back after every upload (gennmi_register_device_array), so a 4 GB index array that the device
+// generates never exists on the host.
 //--------------------------------------------------------------------------
 class Array : public Runtime::ArrayBase
 {
@@ -68,18 +72,29 @@ public:
     virtual void allocate(size_t count) final
     {
         setCount(count);
-        auto *host = static_cast<std::byte*>(std::calloc(getSizeBytes(), 1));
-        if(!host) { throw std::bad_alloc(); }
+        m_Reserved = !(getLocation() & VarLocationAttribute::HOST);
+        std::byte *host = nullptr;
+        if(m_Reserved) {
+            void *space = mmap(nullptr, getSizeBytes(), PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+            if(space == MAP_FAILED) { throw std::bad_alloc(); }
+            host = static_cast<std::byte*>(space);
+        }
+        else {
+            host = static_cast<std::byte*>(std::calloc(getSizeBytes(), 1));
+            if(!host) { throw std::bad_alloc(); }
+        }
         setHostPointer(host);
         check(gennmi_malloc(&m_Device, getSizeBytes()), "array allocation");
         check(gennmi_memset(m_Device, 0, getSizeBytes()), "array clear");
-        check(gennmi_register_mirror(host, m_Device, getSizeBytes()), "array registration");
+        check(m_Reserved ? gennmi_register_device_array(host, m_Device, getSizeBytes())
+                         : gennmi_register_mirror(host, m_Device, getSizeBytes()), "array registration");
     }
     virtual void free() final
     {
         check(gennmi_unregister_mirror(getHostPointer()), "array deregistration");
         check(gennmi_free(m_Device), "array release");
-        std::free(getHostPointer());
+        if(m_Reserved) { munmap(getHostPointer(), getSizeBytes()); }
+        else { std::free(getHostPointer()); }
         m_Device = nullptr;
         setHostPointer(nullptr);
         setCount(0);
@@ -128,6 +143,7 @@ private:
     }
 
     void *m_Device;
+    bool m_Reserved = false;    // the host side is address space without memory behind it (device-only array)
 };
 
 //--------------------------------------------------------------------------
@@ -992,6 +1008,7 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
     {
         CodeStream::Scope b(body);
         if(timing) { body << timerStart << std::endl; }
+        body << "GENNMI_CHECK(gennmi_mirrors_begin_initialisation());" << std::endl;
         EnvironmentExternal funcEnv(initEnv);
         funcEnv.add(model.getTimePrecision().addConst(), "dt", Type::writeNumeric(model.getDT(), model.getTimePrecision()));
 
@@ -1069,17 +1086,33 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
             {
                 const auto &arch = s.getArchetype();
                 const auto &connect = arch.getSparseConnectivityInitialiser();
-                if(!(arch.getMatrixType() & SynapseMatrixConnectivity::SPARSE) || !arch.getKernelSize().empty()) {
-                    unsupported("connectivity initialisation of projection '" + arch.getName() + "' (SPARSE without kernel only)");
+                if(!(arch.getMatrixType() & SynapseMatrixConnectivity::SPARSE)) {
+                    unsupported("connectivity initialisation of projection '" + arch.getName() + "' (SPARSE only)");
                 }
                 const bool byRow = !Utils::areTokensEmpty(connect.getRowBuildCodeTokens());
                 // built-in snippets the device library generates itself (Preferences::deviceInitialisation)
                 const auto *snippet = connect.getSnippet();
-                const int deviceSnippet = !deviceInit ? -1
+                int deviceSnippet = !deviceInit ? -1
                     : (snippet == InitSparseConnectivitySnippet::FixedProbability::getInstance()) ? 0
                     : (snippet == InitSparseConnectivitySnippet::FixedProbabilityNoAutapse::getInstance()) ? 1
                     : (snippet == InitSparseConnectivitySnippet::FixedNumberPostWithReplacement::getInstance()) ? 2
-                    : (snippet == InitSparseConnectivitySnippet::OneToOne::getInstance()) ? 3 : -1;
+                    : (snippet == InitSparseConnectivitySnippet::OneToOne::getInstance()) ? 3
+                    : (snippet == InitSparseConnectivitySnippet::FixedNumberPreWithReplacement::getInstance()) ? 4
+                    : (snippet == InitSparseConnectivitySnippet::Conv2D::getInstance()) ? 5 : -1;
+                // per-synapse variables initialised from a kernel (the synapse's position in it is only known while its row is
+                // built): on the device when each is a float copy of a kernel entry (InitVarSnippet::Kernel)
+                std::vector<std::string> kernelVars;
+                for(const auto &var : arch.getWUInitialiser().getSnippet()->getVars()) {
+                    const auto &init = arch.getWUInitialiser().getVarInitialisers().at(var.name);
+                    if(Utils::areTokensEmpty(init.getCodeTokens()) || !init.isKernelRequired()) { continue; }
+                    kernelVars.push_back(var.name);
+                    bool eligible = (deviceSnippet == 5) && (batchSize == 1) && var.type.resolve(model.getTypeContext()) == Type::Float;
+                    for(const auto &g : s.getGroups()) {
+                        eligible = eligible && (g.get().getWUInitialiser().getVarInitialisers().at(var.name).getSnippet() == InitVarSnippet::Kernel::getInstance());
+                    }
+                    if(!eligible) { deviceSnippet = -1; }
+                }
+                if(deviceSnippet != 5 && !kernelVars.empty() && deviceSnippet >= 0) { deviceSnippet = -1; }
                 if(deviceSnippet >= 0) {
                     forEachGroup(funcEnv, "SynapseConnectivityInitGroup", s.getIndex(), s.getGroups().size(), [&]
                     {
@@ -1091,11 +1124,17 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                             streams.push_back(2 * place(g.get()) + 1);
                             const auto &params = g.get().getSparseConnectivityInitialiser().getParams();
                             if(deviceSnippet <= 1) { values.push_back(params.at("prob")); }
-                            else if(deviceSnippet == 2) { values.push_back(params.at("num")); }
+                            else if(deviceSnippet == 2 || deviceSnippet == 4) { values.push_back(params.at("num")); }
+                            else if(deviceSnippet == 5) {
+                                for(const char *name : {"conv_kh", "conv_kw", "conv_sh", "conv_sw", "conv_padh", "conv_padw", "conv_ih", "conv_iw", "conv_ic",
+                                                        "conv_oh", "conv_ow", "conv_oc"}) {
+                                    values.push_back(params.at(name));
+                                }
+                            }
                         }
                         CodeStream::Scope scope(env.getStream());
                         env.getStream() << "static const uint32_t stream[] = " << tableU32(streams) << ";" << std::endl;
-                        if(deviceSnippet <= 2) { env.getStream() << "static const double value[] = " << table(values, Type::Double) << ";" << std::endl; }
+                        if(deviceSnippet != 3) { env.getStream() << "static const double value[] = " << table(values, Type::Double) << ";" << std::endl; }
                         env.getStream() << "uint32_t overflowRows = 0;" << std::endl;
                         const std::string arrays = "gennmiDev(" + env["_row_length"] + "), gennmiDev(" + env["_ind"] + ")";
                         const std::string shape = env["num_pre"] + ", " + env["num_post"] + ", " + env["_row_stride"];
@@ -1107,14 +1146,33 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                             env.getStream() << "GENNMI_CHECK(gennmi_init_sparse_fixed_number_post(" << shape << ", (uint32_t)value[g], nullptr, " << seedExpr
                                             << ", stream[g], " << arrays << ", &overflowRows));" << std::endl;
                         }
-                        else {
+                        else if(deviceSnippet == 3) {
                             env.getStream() << "(void)stream; GENNMI_CHECK(gennmi_init_sparse_one_to_one(" << shape << ", " << arrays << "));" << std::endl;
                         }
-                        // the host mirrors follow: per-row initialisation code, pulls and the upload that ends initialize() read them
-                        env.getStream() << "GENNMI_CHECK(gennmi_memcpy_from_device(" << env["_row_length"] << ", gennmiDev(" << env["_row_length"] << "), (size_t)"
-                                        << env["num_pre"] << " * sizeof(uint32_t)));" << std::endl;
-                        env.getStream() << "GENNMI_CHECK(gennmi_memcpy_from_device(" << env["_ind"] << ", gennmiDev(" << env["_ind"] << "), (size_t)"
-                                        << env["num_pre"] << " * " << env["_row_stride"] << " * sizeof(uint32_t)));" << std::endl;
+                        else if(deviceSnippet == 4) {
+                            env.getStream() << "GENNMI_CHECK(gennmi_init_sparse_fixed_number_pre(" << shape << ", (uint32_t)value[g], " << seedExpr
+                                            << ", stream[g], " << arrays << ", &overflowRows));" << std::endl;
+                        }
+                        else {
+                            env.getStream() << "(void)stream; int32_t conv[12]; for(int k = 0; k < 12; k++) { conv[k] = (int32_t)value[12 * g + k]; }" << std::endl;
+                            env.getStream() << "if((unsigned long long)conv[6] * conv[7] * conv[8] != " << env["num_pre"] << " || (unsigned long long)conv[9] * conv[10] * conv[11] != "
+                                            << env["num_post"] << ") { throw std::runtime_error(\"Conv2D connectivity: shapes do not match the populations' sizes\"); }" << std::endl;
+                            env.getStream() << "GENNMI_CHECK(gennmi_init_sparse_conv2d(conv, " << env["_row_stride"] << ", " << arrays << ", nullptr, nullptr, &overflowRows));" << std::endl;
+                            // weights that are kernel entries are written beside the connectivity (the row build is repeated per variable)
+                            for(const auto &name : kernelVars) {
+                                EnvironmentGroupMergedField<SynapseConnectivityInitGroupMerged> varEnv(env, s);
+                                varEnv.addExtraGlobalParams(InitVarSnippet::Kernel::getInstance()->getExtraGlobalParams(), name);
+                                varEnv.addField(Type::Float.createPointer(), "_mi_kernel_var", name,
+                                                [name](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, name); });
+                                varEnv.getStream() << "GENNMI_CHECK(gennmi_init_sparse_conv2d(conv, " << env["_row_stride"] << ", " << arrays << ", gennmiDev(" << varEnv["kernel"]
+                                                   << "), gennmiDev(" << varEnv["_mi_kernel_var"] << "), &overflowRows));" << std::endl;
+                                varEnv.getStream() << "GENNMI_CHECK(gennmi_mirror_device_initialised(" << varEnv["_mi_kernel_var"] << "));" << std::endl;
+                            }
+                        }
+                        // the device holds the matrix: the upload that ends initialize() leaves it alone, and host code that reads
+                        // rows (per-row initialisation code) asks for the copy first
+                        env.getStream() << "GENNMI_CHECK(gennmi_mirror_device_initialised(" << env["_row_length"] << "));" << std::endl;
+                        env.getStream() << "GENNMI_CHECK(gennmi_mirror_device_initialised(" << env["_ind"] << "));" << std::endl;
                     });
                     return;
                 }
@@ -1150,10 +1208,24 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                         else {
                             addEnv.add(Type::Uint32.addConst(), "id_pre", "idPre", {addEnv.addInitialiser("const unsigned int idPre = $(0);")});
                         }
-                        addEnv.printLine("$(_ind)[($(id_pre) * $(_row_stride)) + $(_row_length)[$(id_pre)]] = $(id_post);");
+                        addEnv.add(Type::Uint32.addConst(), "id_syn", "idSyn",
+                                   {addEnv.addInitialiser("const unsigned int idSyn = ($(id_pre) * $(_row_stride)) + $(_row_length)[$(id_pre)];")});
+                        if(!arch.getKernelSize().empty()) {
+                            // variables that are functions of the synapse's position in the kernel: addSynapse's further arguments
+                            // name it (single_threaded_cpu/backend.cc:1200-1215)
+                            EnvironmentGroupMergedField<SynapseConnectivityInitGroupMerged> kernelEnv(addEnv, s);
+                            for(size_t k = 0; k < arch.getKernelSize().size(); k++) {
+                                const std::string index = std::to_string(k);
+                                kernelEnv.add(Type::Uint32.addConst(), "id_kernel_" + index, "idKernel" + index,
+                                              {kernelEnv.addInitialiser("const unsigned int idKernel" + index + " = $(" + std::to_string(k + 1) + ");")});
+                            }
+                            s.generateKernelInit(kernelEnv, batchSize);
+                        }
+                        addEnv.printLine("$(_ind)[$(id_syn)] = $(id_post);");
                         addEnv.printLine("$(_row_length)[$(id_pre)]++;");
                     }
-                    env.add(Type::ResolvedType::createFunction(Type::Void, {Type::Uint32}), "addSynapse", addStream.str());
+                    env.add(Type::ResolvedType::createFunction(Type::Void, std::vector<Type::ResolvedType>(1 + arch.getKernelSize().size(), Type::Uint32)),
+                            "addSynapse", addStream.str());
                     if(byRow) {
                         s.generateSparseRowInit(env);
                     }
@@ -1192,10 +1264,16 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                     bool varsOnDevice = deviceInit && s.getArchetype().isWUVarInitRequired() && (batchSize == 1);
                     struct DeviceVar { std::string name; unsigned int snippet; std::vector<std::string> params; };
                     std::vector<DeviceVar> deviceVars;
+                    // (variables initialised from a kernel were written while the rows were built)
+                    bool anyRowVar = false;
+                    for(const auto &var : s.getArchetype().getWUInitialiser().getSnippet()->getVars()) {
+                        const auto &init = s.getArchetype().getWUInitialiser().getVarInitialisers().at(var.name);
+                        anyRowVar = anyRowVar || (!Utils::areTokensEmpty(init.getCodeTokens()) && !init.isKernelRequired());
+                    }
                     if(varsOnDevice) {
                         for(const auto &var : s.getArchetype().getWUInitialiser().getSnippet()->getVars()) {
                             const auto &init = s.getArchetype().getWUInitialiser().getVarInitialisers().at(var.name);
-                            if(Utils::areTokensEmpty(init.getCodeTokens())) { continue; }           // left uninitialised: nothing to do
+                            if(Utils::areTokensEmpty(init.getCodeTokens()) || init.isKernelRequired()) { continue; }    // nothing to do here
                             DeviceVar d{var.name, 0, {}};
                             varsOnDevice = varsOnDevice && var.type.resolve(model.getTypeContext()) == Type::Float
                                            && deviceVarSnippet(init.getSnippet(), d.snippet, d.params);
@@ -1224,12 +1302,13 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                             const std::string count = "(size_t)" + env["num_pre"] + " * " + env["_row_stride"];
                             env.getStream() << "GENNMI_CHECK(gennmi_init_var(gennmiDev(" << env["_mi_init_" + name] << "), " << GENNMI_TYPE_F32 << "u, " << count << ", "
                                             << d.snippet << "u, params, " << seedExpr << ", stream[g]));" << std::endl;
-                            env.getStream() << "GENNMI_CHECK(gennmi_memcpy_from_device(" << env["_mi_init_" + name] << ", gennmiDev(" << env["_mi_init_" + name] << "), "
-                                            << count << " * sizeof(float)));" << std::endl;
+                            env.getStream() << "GENNMI_CHECK(gennmi_mirror_device_initialised(" << env["_mi_init_" + name] << "));" << std::endl;
                             varIndex++;
                         }
                     }
-                    else if(s.getArchetype().isWUVarInitRequired()) {
+                    else if(s.getArchetype().isWUVarInitRequired() && anyRowVar) {
+                        // (rows the device generated are fetched first)
+                        env.printLine("GENNMI_CHECK(gennmi_mirror_ensure_host($(_row_length))); GENNMI_CHECK(gennmi_mirror_ensure_host($(_ind)));");
                         env.print("for(unsigned int i = 0; i < $(num_pre); i++)");
                         CodeStream::Scope loop(env.getStream());
                         env.add(Type::Uint32.addConst(), "id_pre", "i");
@@ -1258,6 +1337,7 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                 {
                     EnvironmentGroupMergedField<CustomWUUpdateSparseInitGroupMerged> env(funcEnv, c);
                     buildStandardEnvironment(env, batchSize);
+                    env.printLine("GENNMI_CHECK(gennmi_mirror_ensure_host($(_row_length))); GENNMI_CHECK(gennmi_mirror_ensure_host($(_ind)));");
                     env.print("for(unsigned int i = 0; i < $(num_pre); i++)");
                     CodeStream::Scope loop(env.getStream());
                     env.add(Type::Uint32.addConst(), "id_pre", "i");
@@ -1274,6 +1354,7 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                 {
                     EnvironmentGroupMergedField<CustomConnectivityUpdateSparseInitGroupMerged> env(funcEnv, c);
                     buildStandardEnvironment(env);
+                    env.printLine("GENNMI_CHECK(gennmi_mirror_ensure_host($(_row_length))); GENNMI_CHECK(gennmi_mirror_ensure_host($(_ind)));");
                     env.print("for(unsigned int i = 0; i < $(num_pre); i++)");
                     CodeStream::Scope loop(env.getStream());
                     env.add(Type::Uint32.addConst(), "id_pre", "i");

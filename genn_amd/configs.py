@@ -151,6 +151,24 @@ def izhikevich_fanout(n=1_000_000, fanout=1000, steps=1000, seed=777, dt=1.0, no
     return net
 
 
+def izhikevich_fanout_snippets(n=1_000_000, fanout=1000, steps=20, seed=777, dt=1.0):
+    """The network of :func:`izhikevich_fanout` described by snippets instead of arrays, as a GeNN model would state it:
+    excitatory and inhibitory neurons are populations of their own, every population pair a SPARSE projection built by
+    FixedNumberPostWithReplacement (the fan-out of 1,000 split 80/20 like the targets) with Uniform weights ([0, 0.5) from
+    excitatory, [-1, 0) from inhibitory sources).  Nothing of the matrices exists on the host."""
+    n_e = (n * 4) // 5
+    net = Net(name="izh_snippets", dt=dt, steps=steps, seed=seed)
+    for name, count, stream in (("E", n_e, 12), ("I", n - n_e, 13)):
+        v0 = np.full(count, -65.0, np.float32)
+        net.pops.append(Pop(name, "izh", count, dict(a=0.02, b=0.2, c=-65.0, d=8.0), {"V": v0, "U": (np.float32(0.2) * v0).astype(np.float32)}))
+        net.css.append(CurrentSource(name + "_noise", "noise", name, noise=netgen.uniform_f32(seed, stream, 0, steps * count, 5.0, 0.0).reshape(steps, count)))
+    for src, lo, hi in (("E", 0.0, 0.5), ("I", -1.0, 0.0)):
+        for trg, share in (("E", (fanout * 4) // 5), ("I", fanout - (fanout * 4) // 5)):
+            net.syns.append(Syn(src + trg, src, trg, matrix="sparse_init", wum="static", psm="deltacurr",
+                                connect=("FixedNumberPostWithReplacement", {"num": share}), g_init=("Uniform", {"min": lo, "max": hi})))
+    return net
+
+
 # --------------------------------------------------------------------------------------------
 # C4: plastic sparse network with trace STDP (pygenn/genn_model.py:1448-1476)
 # --------------------------------------------------------------------------------------------
@@ -332,6 +350,29 @@ def snippet_initialised(n_e=1600, n_i=400, steps=200, seed=31, dt=1.0):
     net.name = "snippet_initialised"
     for s in net.syns:
         s.matrix = "sparse_init"
+    return net
+
+
+def snippet_initialised_layers(steps=200, seed=37, dt=1.0):
+    """A small feed-forward network whose stored SPARSE matrices are built by the remaining built-in snippets: Poisson
+    sources on an 8 x 8 x 2 grid drive an 8 x 8 x 4 layer through Conv2D connectivity with kernel-initialised weights
+    (3 x 3, stride 1, padding 1), the layer drives a read-out population through FixedNumberPreWithReplacement with Uniform
+    weights, and the read-out inhibits the layer through FixedNumberPreWithReplacement with one weight."""
+    net = Net(name="snippet_initialised_layers", dt=dt, steps=steps, seed=seed)
+    shape = dict(conv_kh=3, conv_kw=3, conv_sh=1, conv_sw=1, conv_padh=1, conv_padw=1, conv_ih=8, conv_iw=8, conv_ic=2, conv_oh=8, conv_ow=8, conv_oc=4)
+    n_in, n_mid, n_out = 8 * 8 * 2, 8 * 8 * 4, 200
+    start, end, times = poisson_spike_source(seed, 1, n_in, 80.0, steps, dt)
+    net.pops.append(Pop("In", "ssa", n_in, {}, {"startSpike": start, "endSpike": end}, spike_times=times))
+    lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.35, TauRefrac=2.0)
+    net.pops.append(Pop("Mid", "lif", n_mid, dict(lif), {"V": (-60.0 + 9.0 * rng.uniform(seed, 2, 0, n_mid)).astype(np.float32), "RefracTime": np.zeros(n_mid, np.float32)}))
+    net.pops.append(Pop("Out", "lif", n_out, dict(lif, Ioffset=0.2), {"V": (-60.0 + 9.0 * rng.uniform(seed, 3, 0, n_out)).astype(np.float32), "RefracTime": np.zeros(n_out, np.float32)}))
+    kernel = (0.05 + 0.25 * rng.uniform(seed, 4, 0, 3 * 3 * 2 * 4)).astype(np.float32).reshape(3, 3, 2, 4)
+    net.syns.append(Syn("InMid", "In", "Mid", matrix="sparse_init", wum="static", psm="expcurr", tau=5.0,
+                        connect=("Conv2D", shape), g_init=("Kernel", {"kernel": kernel})))
+    net.syns.append(Syn("MidOut", "Mid", "Out", matrix="sparse_init", wum="static", psm="expcurr", tau=5.0,
+                        connect=("FixedNumberPreWithReplacement", {"num": 30}), g_init=("Uniform", {"min": 0.0, "max": 0.08})))
+    net.syns.append(Syn("OutMid", "Out", "Mid", matrix="sparse_init", wum="static_const", wum_params={"g": -0.05}, psm="expcurr", tau=10.0,
+                        connect=("FixedNumberPreWithReplacement", {"num": 10})))
     return net
 
 

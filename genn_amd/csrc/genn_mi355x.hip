@@ -22,6 +22,7 @@
 // Arithmetic contract: fp32, one rounding per operation, same operation order as the code the
 // reference's SingleThreadedCPU backend generates (build with -ffp-contract=off).  The only
 // permitted divergence is the order of fp32 atomic adds into outPost / denDelay.
+#include <sys/mman.h>
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -291,15 +292,66 @@ int gennmi_flush(void) { FLUSH_QUEUED(); return GENNMI_OK; }
 // ---- host mirrors: host buffer <-> device buffer pairs, for callers whose generated code only knows host pointers
 namespace
 {
-struct Mirror { void *dev; size_t bytes; };
+// deviceInitialised: a device generator filled the buffer since initialisation began, so the host copy is not the one to
+// upload; hostStale: ... and has not been copied back since.  releaseHost: the host side is lazily committed address space
+// (an array the model places on the device only) whose pages are given back after every upload.
+struct Mirror { void *dev; size_t bytes; bool deviceInitialised = false, hostStale = false, releaseHost = false; };
 std::map<uintptr_t, Mirror> g_mirrors;      // keyed by host base address
 std::mutex g_mirrorMutex;
+// the registered buffer `host` points into (g_mirrorMutex held)
+Mirror *findMirror(const void *host, uintptr_t *base = nullptr)
+{
+    const uintptr_t h = reinterpret_cast<uintptr_t>(host);
+    auto it = g_mirrors.upper_bound(h);
+    if(it == g_mirrors.begin()) { return nullptr; }
+    --it;
+    if(h - it->first >= it->second.bytes) { return nullptr; }
+    if(base) { *base = it->first; }
+    return &it->second;
+}
 }
 int gennmi_register_mirror(const void *host, void *dev, size_t bytes)
 {
     if(!host || !dev || bytes == 0) { return fail(GENNMI_EINVAL, "register_mirror: null pointer or empty buffer"); }
     std::lock_guard<std::mutex> lock(g_mirrorMutex);
     g_mirrors[reinterpret_cast<uintptr_t>(host)] = Mirror{dev, bytes};
+    return GENNMI_OK;
+}
+int gennmi_register_device_array(const void *host, void *dev, size_t bytes)
+{
+    if(int rc = gennmi_register_mirror(host, dev, bytes)) { return rc; }
+    if(reinterpret_cast<uintptr_t>(host) % 4096 != 0) { return fail(GENNMI_EINVAL, "register_device_array: the host range must start on a page boundary"); }
+    std::lock_guard<std::mutex> lock(g_mirrorMutex);
+    g_mirrors[reinterpret_cast<uintptr_t>(host)].releaseHost = true;
+    return GENNMI_OK;
+}
+int gennmi_mirrors_begin_initialisation(void)
+{
+    std::lock_guard<std::mutex> lock(g_mirrorMutex);
+    for(auto &m : g_mirrors) { m.second.deviceInitialised = m.second.hostStale = false; }
+    return GENNMI_OK;
+}
+int gennmi_mirror_device_initialised(const void *host)
+{
+    if(!host) { return GENNMI_OK; }
+    std::lock_guard<std::mutex> lock(g_mirrorMutex);
+    Mirror *m = findMirror(host);
+    if(!m) { return fail(GENNMI_EINVAL, "mirror_device_initialised: host pointer is not inside a registered buffer"); }
+    m->deviceInitialised = m->hostStale = true;
+    return GENNMI_OK;
+}
+int gennmi_mirror_ensure_host(const void *host)
+{
+    if(!host) { return GENNMI_OK; }
+    FLUSH_QUEUED();
+    std::lock_guard<std::mutex> lock(g_mirrorMutex);
+    uintptr_t base = 0;
+    Mirror *m = findMirror(host, &base);
+    if(!m) { return fail(GENNMI_EINVAL, "mirror_ensure_host: host pointer is not inside a registered buffer"); }
+    if(m->hostStale) {
+        HIP_TRY(hipMemcpy(reinterpret_cast<void*>(base), m->dev, m->bytes, hipMemcpyDeviceToHost));
+        m->hostStale = false;
+    }
     return GENNMI_OK;
 }
 int gennmi_unregister_mirror(const void *host)
@@ -344,8 +396,15 @@ int gennmi_push_mirrors(void)
     FLUSH_QUEUED();
     std::lock_guard<std::mutex> lock(g_mirrorMutex);
     for(const auto &m : g_mirrors) {
-        HIP_TRY(hipMemcpy(m.second.dev, reinterpret_cast<const void*>(m.first), m.second.bytes, hipMemcpyHostToDevice));
-        noteDeviceWrite(m.second.dev, m.second.bytes);
+        if(!m.second.deviceInitialised) {
+            HIP_TRY(hipMemcpy(m.second.dev, reinterpret_cast<const void*>(m.first), m.second.bytes, hipMemcpyHostToDevice));
+            noteDeviceWrite(m.second.dev, m.second.bytes);
+        }
+        if(m.second.releaseHost) {
+            // the pages come back as zeros when next touched; what the model keeps is on the device
+            const size_t whole = m.second.bytes / 4096 * 4096;
+            if(whole && madvise(reinterpret_cast<void*>(m.first), whole, MADV_DONTNEED) != 0) { return fail(GENNMI_EINVAL, "push_mirrors: madvise failed"); }
+        }
     }
     return GENNMI_OK;
 }

@@ -211,6 +211,92 @@ __global__ void oneToOneKernel(uint32_t numPre, uint32_t numPost, uint32_t rowSt
     }
 }
 
+// FixedNumberPreWithReplacement (initSparseConnectivitySnippet.h:380-410): every postsynaptic neuron draws `num` sources,
+// idPre = gennrand() % num_pre, and each draw appends the neuron to its source's row.  A thread makes four draws of one
+// column (one generator call); rows are appended to through an atomic counter, in arbitrary order ...
+__global__ __launch_bounds__(BLOCK)
+void fixedNumberPreScatterKernel(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t num, Stream s, uint32_t *rowLength, uint32_t *ind)
+{
+    const uint32_t groupsPerColumn = (num + 3) / 4;
+    const unsigned long long item = (unsigned long long)blockIdx.x * BLOCK + threadIdx.x;
+    if(item >= (unsigned long long)numPost * groupsPerColumn) { return; }
+    const uint32_t column = (uint32_t)(item / groupsPerColumn), group = (uint32_t)(item - (unsigned long long)column * groupsPerColumn);
+    const Words r = s.at(item, 0);
+    #pragma unroll
+    for(int k = 0; k < 4; k++) {
+        if(group * 4 + k >= num) { break; }
+        const uint32_t idPre = r.w[k] % numPre;
+        const uint32_t position = atomicAdd(&rowLength[idPre], 1u);
+        if(position < rowStride) { ind[(size_t)idPre * rowStride + position] = column; }
+        else if(position == rowStride) { atomicAdd(&g_rowOverflow, 1u); }
+    }
+}
+// ... and then sorted (one work-group per row, bitonic network in LDS over the next power of two), so that rows come out
+// ascending like those of every other generator here, whatever order the appends happened in
+__global__ __launch_bounds__(BLOCK)
+void rowSortKernel(uint32_t rowStride, uint32_t *rowLength, uint32_t *ind, uint32_t capacity)
+{
+    extern __shared__ uint32_t shRow[];
+    const uint32_t row = blockIdx.x;
+    const uint32_t length = min(rowLength[row], rowStride);
+    if(threadIdx.x == 0) { rowLength[row] = length; }
+    if(length < 2) { return; }
+    uint32_t n = 2;
+    while(n < length) { n <<= 1; }
+    (void)capacity;
+    uint32_t *entries = ind + (size_t)row * rowStride;
+    for(uint32_t i = threadIdx.x; i < n; i += BLOCK) { shRow[i] = (i < length) ? entries[i] : 0xFFFFFFFFu; }
+    __syncthreads();
+    for(uint32_t k = 2; k <= n; k <<= 1) {
+        for(uint32_t j = k >> 1; j > 0; j >>= 1) {
+            for(uint32_t i = threadIdx.x; i < n; i += BLOCK) {
+                const uint32_t partner = i ^ j;
+                if(partner > i) {
+                    const uint32_t a = shRow[i], b = shRow[partner];
+                    const bool ascending = ((i & k) == 0);
+                    if((a > b) == ascending) { shRow[i] = b; shRow[partner] = a; }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    for(uint32_t i = threadIdx.x; i < length; i += BLOCK) { entries[i] = shRow[i]; }
+}
+
+// Conv2D as SPARSE connectivity (initSparseConnectivitySnippet.h:438-497): the snippet's row build code, one thread per
+// presynaptic neuron; targets come out ascending (output row, column, channel).  With `kernel` and `g`, every synapse's weight
+// is the kernel entry its (kernel row, kernel column, input channel, output channel) names — InitVarSnippet::Kernel
+// (initVarSnippet.h:100-108) over the snippet's kernel size {kh, kw, ic, oc}.
+struct Conv2DParams { int kh, kw, sh, sw, padh, padw, ih, iw, ic, oh, ow, oc; };
+__global__ __launch_bounds__(BLOCK)
+void conv2dSparseKernel(Conv2DParams c, uint32_t rowStride, uint32_t *rowLength, uint32_t *ind, const float *kernel, float *g)
+{
+    const uint32_t idPre = blockIdx.x * BLOCK + threadIdx.x;
+    if(idPre >= (uint32_t)(c.ih * c.iw * c.ic)) { return; }
+    const int inRow = ((int)idPre / c.ic) / c.iw, inCol = ((int)idPre / c.ic) % c.iw, inChan = (int)idPre % c.ic;
+    const int maxOutRow = min(c.oh, max(0, 1 + ((inRow + c.padh) / c.sh)));
+    const int minOutCol = min(c.ow, max(0, 1 + (int)floorf((float)(inCol + c.padw - c.kw) / (float)c.sw)));
+    const int maxOutCol = min(c.ow, max(0, 1 + ((inCol + c.padw) / c.sw)));
+    int outRow = min(c.oh, max(0, 1 + (int)floorf((float)(inRow + c.padh - c.kh) / (float)c.sh)));
+    uint32_t length = 0;
+    for(; outRow < maxOutRow; outRow++) {
+        const int kernRow = inRow - ((outRow * c.sh) - c.padh);
+        for(int outCol = minOutCol; outCol < maxOutCol; outCol++) {
+            const int kernCol = inCol - ((outCol * c.sw) - c.padw);
+            for(int outChan = 0; outChan < c.oc; outChan++) {
+                if(length < rowStride) {
+                    const size_t idSyn = (size_t)idPre * rowStride + length;
+                    ind[idSyn] = (uint32_t)((outRow * c.ow * c.oc) + (outCol * c.oc) + outChan);
+                    if(g) { g[idSyn] = kernel[((size_t)(kernRow * c.kw + kernCol) * c.ic + inChan) * c.oc + outChan]; }
+                }
+                length++;
+            }
+        }
+    }
+    if(length > rowStride) { atomicAdd(&g_rowOverflow, 1u); length = rowStride; }
+    rowLength[idPre] = length;
+}
+
 Stream makeStream(uint64_t seed, uint32_t stream) { return Stream{(uint32_t)seed, (uint32_t)(seed >> 32), stream}; }
 
 int finishConnectivity(uint32_t *overflowRows)
@@ -321,6 +407,46 @@ int gennmi_init_sparse_fixed_number_post(uint32_t numPre, uint32_t numPost, uint
     const unsigned int blocks = (numPre + (BLOCK / WAVE) - 1) / (BLOCK / WAVE);
     hipLaunchKernelGGL(fixedNumberPostKernel, dim3(blocks), dim3(BLOCK), 0, 0, numPre, numPost, rowStride, num, rowLengthIn,
                        makeStream(seed, stream), rowLength, ind);
+    return finishConnectivity(overflowRows);
+}
+
+int gennmi_init_sparse_fixed_number_pre(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t num,
+                                        uint64_t seed, uint32_t stream, uint32_t *rowLength, uint32_t *ind, uint32_t *overflowRows)
+{
+    { const int rcFlush = gennmi_detail::flushQueuedSteps(); if(rcFlush) { return rcFlush; } }
+    if(numPre == 0 || numPost == 0 || rowStride == 0) { return gennmi_detail::fail(GENNMI_EINVAL, "empty matrix"); }
+    if(rowStride > 16384) { return gennmi_detail::fail(GENNMI_EUNSUPPORTED, "rows of more than 16384 entries are not sorted on the device"); }
+    if(int rc = clearOverflow()) { return rc; }
+    HIP_TRY(hipMemset(rowLength, 0, (size_t)numPre * sizeof(uint32_t)));
+    const unsigned long long items = (unsigned long long)numPost * ((num + 3) / 4);
+    if(items > 0x7fffffffull * BLOCK) { return gennmi_detail::fail(GENNMI_EINVAL, "too many draws for one launch"); }
+    if(items) {
+        hipLaunchKernelGGL(fixedNumberPreScatterKernel, dim3((unsigned int)((items + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, 0, numPre, numPost, rowStride, num,
+                           makeStream(seed, stream), rowLength, ind);
+    }
+    uint32_t capacity = 2;
+    while(capacity < rowStride) { capacity <<= 1; }
+    hipLaunchKernelGGL(rowSortKernel, dim3(numPre), dim3(BLOCK), capacity * sizeof(uint32_t), 0, rowStride, rowLength, ind, capacity);
+    return finishConnectivity(overflowRows);
+}
+
+int gennmi_init_sparse_conv2d(const int32_t conv[12], uint32_t rowStride, uint32_t *rowLength, uint32_t *ind, const float *kernel, float *g,
+                              uint32_t *overflowRows)
+{
+    { const int rcFlush = gennmi_detail::flushQueuedSteps(); if(rcFlush) { return rcFlush; } }
+    if(!conv || !rowLength || !ind || rowStride == 0 || ((kernel == nullptr) != (g == nullptr))) { return gennmi_detail::fail(GENNMI_EINVAL, "init_sparse_conv2d: bad arguments"); }
+    const Conv2DParams c{conv[0], conv[1], conv[2], conv[3], conv[4], conv[5], conv[6], conv[7], conv[8], conv[9], conv[10], conv[11]};
+    if(c.kh <= 0 || c.kw <= 0 || c.sh <= 0 || c.sw <= 0 || c.padh < 0 || c.padw < 0 || c.ih <= 0 || c.iw <= 0 || c.ic <= 0 || c.oh <= 0 || c.ow <= 0 || c.oc <= 0) {
+        return gennmi_detail::fail(GENNMI_EINVAL, "init_sparse_conv2d: sizes and strides must be positive, padding non-negative");
+    }
+    if((unsigned long long)c.ih * c.iw * c.ic > 0xffffffffull || (unsigned long long)c.oh * c.ow * c.oc > 0xffffffffull) {
+        return gennmi_detail::fail(GENNMI_EINVAL, "init_sparse_conv2d: more than 2^32-1 neurons");
+    }
+    if(int rc = clearOverflow()) { return rc; }
+    const uint32_t numPre = (uint32_t)(c.ih * c.iw * c.ic);
+    hipLaunchKernelGGL(conv2dSparseKernel, dim3((numPre + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, 0, c, rowStride, rowLength, ind, kernel, g);
+    gennmi_detail::noteDeviceWrite(ind, (size_t)numPre * rowStride * sizeof(uint32_t));
+    if(g) { gennmi_detail::noteDeviceWrite(g, (size_t)numPre * rowStride * sizeof(float)); }
     return finishConnectivity(overflowRows);
 }
 

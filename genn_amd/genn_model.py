@@ -89,7 +89,9 @@ def init_toeplitz_connectivity(snippet, params=None):
 
 # initSparseConnectivitySnippet.h:107-370; maximum row length as each snippet's SET_CALC_MAX_ROW_LENGTH_FUNC
 _SPARSE_SNIPPETS = ("OneToOne", "FixedProbability", "FixedProbabilityNoAutapse", "FixedNumberPostWithReplacement",
-                    "FixedNumberTotalWithReplacement")
+                    "FixedNumberTotalWithReplacement", "FixedNumberPreWithReplacement", "Conv2D")
+_CONV2D_PARAMS = ("conv_kh", "conv_kw", "conv_sh", "conv_sw", "conv_padh", "conv_padw", "conv_ih", "conv_iw", "conv_ic",
+                  "conv_oh", "conv_ow", "conv_oc")
 
 
 def init_sparse_connectivity(snippet, params=None):
@@ -117,6 +119,13 @@ def max_row_length(snippet, params, num_pre, num_post):
     if snippet == "FixedNumberTotalWithReplacement":
         # :372-381: rows are binomial(num, 1/numPre)
         return max(1, binomial_inverse_cdf(0.9999 ** (1.0 / num_pre), int(params["num"]), 1.0 / num_pre))
+    if snippet == "FixedNumberPreWithReplacement":
+        # :391-400: a row receives each of the num * numPost draws with probability 1 / numPre
+        return max(1, binomial_inverse_cdf(0.9999 ** (1.0 / num_pre), int(params["num"]) * num_post, 1.0 / num_pre))
+    if snippet == "Conv2D":
+        # :485-491
+        kh, kw, sh, sw, oc = (int(params[k]) for k in ("conv_kh", "conv_kw", "conv_sh", "conv_sw", "conv_oc"))
+        return -(-kh // sh) * -(-kw // sw) * oc
     raise NotImplementedError(snippet)
 
 
@@ -124,7 +133,10 @@ class VarInit:
     """Value snippet evaluated on the device at load() (pygenn.init_var; initVarSnippet.h:87-262)."""
     _PARAMS = {"Constant": ("constant",), "Uniform": ("min", "max"), "Normal": ("mean", "sd"),
                "NormalClipped": ("mean", "sd", "min", "max"), "NormalClippedDelay": ("mean", "sd", "min", "max"),
-               "Exponential": ("lambda",), "Gamma": ("a", "b"), "Binomial": ("n", "p")}
+               "Exponential": ("lambda",), "Gamma": ("a", "b"), "Binomial": ("n", "p"),
+               # initVarSnippet.h:100-108: the value is an entry of the `kernel` array (an extra global parameter in the
+               # reference), which one names the connectivity snippet; only behind Conv2D connectivity here
+               "Kernel": ("kernel",)}
 
     def __init__(self, snippet, params):
         if snippet not in self._PARAMS:
@@ -136,6 +148,8 @@ class VarInit:
         self.params = dict(params)
 
     def values(self, dt):
+        if self.snippet == "Kernel":
+            raise NotImplementedError("Kernel variable initialisation is only available behind Conv2D sparse connectivity")
         v = [float(self.params[k]) for k in self._PARAMS[self.snippet]]
         if self.snippet == "NormalClippedDelay":
             v = [x / dt for x in v]          # the snippet's derived parameters (initVarSnippet.h:204-208)
@@ -616,6 +630,8 @@ class GeNNModel:
                 copies = B if s.wu.snippet in ("STDPTrace", "STDP") else 1
                 for name in names:
                     dtype = np.uint8 if name == "d" else np.float32
+                    if name in s.vars:          # (written together with the connectivity)
+                        continue
                     if name not in s.var_host and isinstance(s.wu.vars[name], VarInit):
                         if copies != 1:
                             raise NotImplementedError(f"{s.name}: device-side initialisation of plastic weights with batch size > 1")
@@ -697,6 +713,26 @@ class GeNNModel:
         elif snippet == "FixedNumberPostWithReplacement":
             _abi.check(lib.gennmi_init_sparse_fixed_number_post(n_pre, n_post, s.row_stride, int(params["num"]), None,
                                                                 self.seed, stream, row_length, ind, None))
+        elif snippet == "FixedNumberPreWithReplacement":
+            _abi.check(lib.gennmi_init_sparse_fixed_number_pre(n_pre, n_post, s.row_stride, int(params["num"]),
+                                                               self.seed, stream, row_length, ind, None))
+        elif snippet == "Conv2D":
+            conv = (C.c_int32 * 12)(*(int(params[k]) for k in _CONV2D_PARAMS))
+            if conv[6] * conv[7] * conv[8] != n_pre or conv[9] * conv[10] * conv[11] != n_post:
+                raise ValueError(f"{s.name}: Conv2D shapes do not match the populations' sizes")
+            kernel = g = None
+            init = s.wu.vars.get("g")
+            if isinstance(init, VarInit) and init.snippet == "Kernel" and "g" not in s.var_host:
+                values = np.ascontiguousarray(init.params["kernel"], dtype=np.float32).reshape(-1)
+                if values.size != conv[0] * conv[1] * conv[8] * conv[11]:
+                    raise ValueError(f"{s.name}: the kernel must hold conv_kh * conv_kw * conv_ic * conv_oc values")
+                k = self._alloc(values.size, np.float32)
+                k.view[:] = values
+                k.push_to_device()
+                s.vars["kernel"] = k
+                s.vars["g"] = self._alloc(n_pre * s.row_stride, np.float32, device_only=True)
+                kernel, g = k.ptr, s.vars["g"].ptr
+            _abi.check(lib.gennmi_init_sparse_conv2d(conv, s.row_stride, row_length, ind, kernel, g, None))
         else:
             # FixedNumberTotalWithReplacement: the row lengths are one multinomial draw, made on the host as the
             # snippet's host init code does (initSparseConnectivitySnippet.h:312-358), then handed to the device

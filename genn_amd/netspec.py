@@ -19,6 +19,9 @@ LIF_PARAMS = ("C", "TauM", "Vrest", "Vreset", "Vthresh", "Ioffset", "TauRefrac")
 IZH_PARAMS = ("a", "b", "c", "d")
 STDP_PARAMS = ("tauPlus", "tauMinus", "aPlus", "aMinus", "wMin", "wMax")
 CONV_PARAMS = ("conv_kh", "conv_kw", "conv_ih", "conv_iw", "conv_ic", "conv_oh", "conv_ow", "conv_oc")
+# Conv2D as SPARSE connectivity (initSparseConnectivitySnippet.h:438-497): strides and padding as well
+CONV_SPARSE_PARAMS = ("conv_kh", "conv_kw", "conv_sh", "conv_sw", "conv_padh", "conv_padw", "conv_ih", "conv_iw", "conv_ic",
+                      "conv_oh", "conv_ow", "conv_oc")
 
 
 @dataclass
@@ -211,9 +214,11 @@ def write_netspec(net: Net, path: str):
             np.ascontiguousarray(s.ind, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.ind.u32"))
         elif s.matrix == "dense":
             head = f"syn {s.name} dense {s.src} {s.trg}"
+        elif s.matrix == "sparse_init" and s.connect[0] == "Conv2D":
+            head = f"syn {s.name} conv2d_sparse {s.src} {s.trg} " + " ".join(str(int(s.connect[1][k])) for k in CONV_SPARSE_PARAMS)
         elif s.matrix in ("procedural", "sparse_init"):
             snippet, params = s.connect
-            value = params["num"] if snippet == "FixedNumberPostWithReplacement" else repr(float(params["prob"]))
+            value = params["num"] if snippet in ("FixedNumberPostWithReplacement", "FixedNumberPreWithReplacement") else repr(float(params["prob"]))
             head = f"syn {s.name} {s.matrix} {s.src} {s.trg} {snippet} {value}"
         elif s.matrix == "bitmask":
             head = f"syn {s.name} bitmask {s.src} {s.trg}"
@@ -223,7 +228,11 @@ def write_netspec(net: Net, path: str):
         regenerated = (s.matrix == "dense" and s.wum == "static" and s.g_init is not None)     # DENSE with weights from a snippet, never stored
         if s.wum != "static_const" and s.matrix not in ("procedural", "sparse_init") and not regenerated:
             np.ascontiguousarray(s.g, dtype=np.float32).tofile(os.path.join(path, f"{s.name}.g.f32"))
-        if (s.matrix in ("procedural", "sparse_init") or regenerated) and s.wum == "static":
+        if s.matrix == "sparse_init" and s.wum == "static" and s.g_init[0] == "Kernel":
+            # every weight is an entry of the kernel ([kh][kw][ic][oc]), named by the synapse's position in it
+            np.ascontiguousarray(s.g_init[1]["kernel"], dtype=np.float32).tofile(os.path.join(path, f"{s.name}.kernel.f32"))
+            w = "static_kernel"
+        elif (s.matrix in ("procedural", "sparse_init") or regenerated) and s.wum == "static":
             snippet, params = s.g_init
             order = {"Constant": ("constant",), "Uniform": ("min", "max"), "Normal": ("mean", "sd")}[snippet]
             w = f"static_init {snippet} " + " ".join(repr(float(params[k])) for k in order)

@@ -113,6 +113,22 @@ int gennmi_register_mirror(const void *host, void *dev, size_t bytes);
 int gennmi_unregister_mirror(const void *host);
 int gennmi_mirror_device_pointer(const void *host, void **dev);   /* NULL host -> NULL device, no error */
 int gennmi_push_mirrors(void);
+/* Arrays a device generator fills, and arrays without a host copy (VarLocation::DEVICE, varLocation.h:20-27; the reference's
+ * Array allocates no host memory for them, hip/backend.cc:75-90).  No counterparts in the reference, whose GPU backends
+ * initialise in kernels and never upload afterwards.
+ *  - gennmi_mirrors_begin_initialisation(): first statement of initialize(): forgets which buffers were device-initialised.
+ *  - gennmi_mirror_device_initialised(host): a gennmi_init_* call has just filled the device buffer behind `host`:
+ *    gennmi_push_mirrors() leaves it alone from now on, and the host copy counts as stale.
+ *  - gennmi_mirror_ensure_host(host): called before host code READS such a buffer (per-row initialisation code that walks
+ *    rowLength / ind): copies it back if it is stale.
+ *  - gennmi_register_device_array: gennmi_register_mirror for an array the model keeps on the device only: `host` is
+ *    page-aligned, lazily committed address space (mmap with MAP_NORESERVE) that serves as the array's key in merged
+ *    groups and as staging for host-side initialisation code; gennmi_push_mirrors() returns its pages to the system
+ *    after uploading, so that such an array holds no host memory once initialisation is over. */
+int gennmi_register_device_array(const void *host, void *dev, size_t bytes);
+int gennmi_mirrors_begin_initialisation(void);
+int gennmi_mirror_device_initialised(const void *host);
+int gennmi_mirror_ensure_host(const void *host);
 int gennmi_free_device_memory_bytes(size_t *bytes);             /* genReturnFreeDeviceMemoryBytes, backendCUDAHIP.cc */
 /* sizeof() of the five descriptor structs below, in declaration order (psm, cs, neuron update, presynaptic
  * update, postsynaptic update), so that a binding in another language can verify its struct layout.  Needs
@@ -331,6 +347,19 @@ int gennmi_init_sparse_fixed_probability(uint32_t numPre, uint32_t numPost, uint
  * the reference too draws on the host (its host init code) and hands to the device.  rowLengthIn may alias rowLength. */
 int gennmi_init_sparse_fixed_number_post(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t num, const uint32_t *rowLengthIn,
                                          uint64_t seed, uint32_t stream, uint32_t *rowLength, uint32_t *ind, uint32_t *overflowRows);
+/* FixedNumberPreWithReplacement (:380-410): every postsynaptic neuron draws `num` sources with replacement (idPre =
+ * gennrand() % numPre, the snippet's own arithmetic); a column therefore holds exactly `num` entries, multiplicities counted.
+ * Rows are appended to in arbitrary order and then sorted, so they come out ascending like every other generator's;
+ * rowStride <= 16384.  Row lengths are Binomial(num * numPost, 1 / numPre): the reference sizes rowStride for the 0.9999
+ * quantile (:391-400); rows beyond it are truncated and counted as for the other generators. */
+int gennmi_init_sparse_fixed_number_pre(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t num,
+                                        uint64_t seed, uint32_t stream, uint32_t *rowLength, uint32_t *ind, uint32_t *overflowRows);
+/* Conv2D as SPARSE connectivity (:438-497): conv = {kh, kw, sh, sw, padh, padw, ih, iw, ic, oh, ow, oc}, the snippet's row
+ * build code per presynaptic neuron, targets ascending; rowStride >= ceil(kh / sh) * ceil(kw / sw) * oc (:485-491).  With
+ * `kernel` (device array [kh][kw][ic][oc]) and `g`, every synapse's weight is the kernel entry named by its (kernel row,
+ * kernel column, input channel, output channel): InitVarSnippet::Kernel (initVarSnippet.h:100-108).  Both NULL: connectivity only. */
+int gennmi_init_sparse_conv2d(const int32_t conv[12], uint32_t rowStride, uint32_t *rowLength, uint32_t *ind, const float *kernel, float *g,
+                              uint32_t *overflowRows);
 /* OneToOne (:107-118) */
 int gennmi_init_sparse_one_to_one(uint32_t numPre, uint32_t numPost, uint32_t rowStride, uint32_t *rowLength, uint32_t *ind);
 /* The generator itself, for known-answer tests: one Philox4x32-10 block on the host, and the raw words of a stream

@@ -13,6 +13,7 @@
 // initialisation snippets is used, because their draw order cannot be reproduced elsewhere.
 //
 // usage: ref_driver <netspec dir> <work dir> <out dir>
+#include <sys/resource.h>
 #include <algorithm>
 #include <chrono>
 #include <cmath>
@@ -416,7 +417,7 @@ int main(int argc, char *argv[])
         bool generateOnly = false;
         std::string userCxxFlags;
         std::vector<std::string> dynamicParams;
-        bool timing = false, ordered = false, deviceInit = false, doublePrecision = false, narrowInd = false;
+        bool timing = false, ordered = false, deviceInit = false, doublePrecision = false, narrowInd = false, deviceArrays = false;
         int stepQueue = -1;
         std::string kernels = "auto";
         for(int a = 4; a < argc; a++) {
@@ -429,6 +430,8 @@ int main(int argc, char *argv[])
             else if(opt.rfind("--kernels=", 0) == 0) { kernels = opt.substr(10); }    // MI355X backend: library | generated | auto (Preferences::kernelSource)
             else if(opt.rfind("--step-queue=", 0) == 0) { stepQueue = std::stoi(opt.substr(13)); }      // MI355X backend: Preferences::stepQueueLength
             else if(opt == "--device-init") { deviceInit = true; }                  // MI355X backend: Preferences::deviceInitialisation
+            // matrices built by snippets are placed on the device only (VarLocation::DEVICE) and not written to the out directory
+            else if(opt == "--device-arrays") { deviceArrays = true; }
             else if(opt == "--ordered") { ordered = true; }                          // MI355X backend: Preferences::orderedAccumulation
             else if(opt == "--narrow-ind") { narrowInd = true; }     // ModelSpec::setDefaultNarrowSparseIndEnabled; for --generate-only runs (the netspec's targets are 32-bit)
             else if(opt == "--precision=double") { doublePrecision = true; }        // ModelSpec::setPrecision(Type::Double); for --generate-only runs (the netspec's arrays are fp32)
@@ -478,6 +481,8 @@ int main(int argc, char *argv[])
                     SynSpec s; ls >> s.name >> s.matrix >> s.src >> s.trg;
                     if(s.matrix == "sparse") { ls >> s.rowStride; }
                     else if(s.matrix == "conv2d") { s.conv.resize(8); for(auto &c : s.conv) ls >> c; }
+                    // Conv2D as SPARSE connectivity: kh kw sh sw padh padw ih iw ic oh ow oc (initSparseConnectivitySnippet.h:438-497)
+                    else if(s.matrix == "conv2d_sparse") { s.conv.resize(12); for(auto &c : s.conv) ls >> c; }
                     else if(s.matrix == "procedural" || s.matrix == "sparse_init") { ls >> s.connect >> s.connectValue; }
                     else if(s.matrix != "dense" && s.matrix != "bitmask") throw std::runtime_error("matrix " + s.matrix);
                     ls >> s.wum;
@@ -486,7 +491,7 @@ int main(int argc, char *argv[])
                     else if(s.wum == "stdp_trace" || s.wum == "stdp") { s.wumP.resize(6); for(auto &c : s.wumP) ls >> c; }
                     else if(s.wum == "static_const" || s.wum == "stochastic") { s.wumP.resize(1); ls >> s.wumP[0]; }
                     else if(s.wum == "static_graded" || s.wum == "leaky_graded" || s.wum == "post_event") { s.wumP.resize(2); ls >> s.wumP[0] >> s.wumP[1]; }
-                    else if(s.wum != "static" && s.wum != "static_reverse" && s.wum != "static_init" && s.wum != "timing_copy" && s.wum != "prev_timing") throw std::runtime_error("wum " + s.wum);
+                    else if(s.wum != "static" && s.wum != "static_reverse" && s.wum != "static_init" && s.wum != "static_kernel" && s.wum != "timing_copy" && s.wum != "prev_timing") throw std::runtime_error("wum " + s.wum);
                     ls >> s.psm;
                     if(s.psm == "expcurr") { s.psmP.resize(1); ls >> s.psmP[0]; }
                     else if(s.psm != "deltacurr") throw std::runtime_error("psm " + s.psm);
@@ -614,9 +619,22 @@ int main(int argc, char *argv[])
                                 : initVar<InitVarSnippet::Normal>({{"mean", s.wumP[0]}, {"sd", s.wumP[1]}});
                 wum = initWeightUpdate<WeightUpdateModels::StaticPulse>({}, {{"g", init}});
             }
-            if(s.matrix == "procedural" || s.matrix == "sparse_init") {
+            if(s.wum == "static_kernel") {
+                // every weight is the entry of <name>.kernel.f32 that the synapse's position in the kernel names
+                wum = initWeightUpdate<WeightUpdateModels::StaticPulse>({}, {{"g", initVar<InitVarSnippet::Kernel>()}});
+            }
+            if(s.matrix == "conv2d_sparse") {
+                s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::SPARSE, src, trg, wum, psm,
+                    initConnectivity<InitSparseConnectivitySnippet::Conv2D>(
+                        {{"conv_kh", (int)s.conv[0]}, {"conv_kw", (int)s.conv[1]}, {"conv_sh", (int)s.conv[2]}, {"conv_sw", (int)s.conv[3]},
+                         {"conv_padh", (int)s.conv[4]}, {"conv_padw", (int)s.conv[5]}, {"conv_ih", (int)s.conv[6]}, {"conv_iw", (int)s.conv[7]},
+                         {"conv_ic", (int)s.conv[8]}, {"conv_oh", (int)s.conv[9]}, {"conv_ow", (int)s.conv[10]}, {"conv_oc", (int)s.conv[11]}}));
+            }
+            else if(s.matrix == "procedural" || s.matrix == "sparse_init") {
                 const auto connect = (s.connect == "FixedNumberPostWithReplacement")
                     ? initConnectivity<InitSparseConnectivitySnippet::FixedNumberPostWithReplacement>({{"num", (unsigned int)s.connectValue}})
+                    : (s.connect == "FixedNumberPreWithReplacement")
+                    ? initConnectivity<InitSparseConnectivitySnippet::FixedNumberPreWithReplacement>({{"num", (unsigned int)s.connectValue}})
                     : (s.connect == "FixedProbabilityNoAutapse") ? initConnectivity<InitSparseConnectivitySnippet::FixedProbabilityNoAutapse>({{"prob", s.connectValue}})
                     : initConnectivity<InitSparseConnectivitySnippet::FixedProbability>({{"prob", s.connectValue}});
                 // ("sparse_init": the same snippets initialise a stored SPARSE matrix)
@@ -639,6 +657,10 @@ int main(int argc, char *argv[])
                     initToeplitzConnectivity<InitToeplitzConnectivitySnippet::Conv2D>(
                         {{"conv_kh", (int)s.conv[0]}, {"conv_kw", (int)s.conv[1]}, {"conv_ih", (int)s.conv[2]}, {"conv_iw", (int)s.conv[3]},
                          {"conv_ic", (int)s.conv[4]}, {"conv_oh", (int)s.conv[5]}, {"conv_ow", (int)s.conv[6]}, {"conv_oc", (int)s.conv[7]}}));
+            }
+            if(deviceArrays && (s.matrix == "sparse_init" || s.matrix == "conv2d_sparse")) {
+                s.sg->setSparseConnectivityLocation(VarLocation::DEVICE);
+                if(s.wum != "static_const") { s.sg->setWUVarLocation("g", VarLocation::DEVICE); }
             }
             if(s.maxDenDelay) s.sg->setMaxDendriticDelayTimesteps(s.maxDenDelay);
             if(s.axonalDelay) s.sg->setAxonalDelaySteps(s.axonalDelay);
@@ -710,9 +732,22 @@ int main(int argc, char *argv[])
         }
 
         // ---- run ---------------------------------------------------------------------------
+        const auto startOfRun = std::chrono::steady_clock::now();
+        auto sinceStart = [&startOfRun]() { return std::chrono::duration<double>(std::chrono::steady_clock::now() - startOfRun).count(); };
         Runtime::Runtime rt(targetPath, modelMerged, backend);
         rt.allocate(steps);
+        const double allocated = sinceStart();
+        // kernels that weights are initialised from are extra global parameters of the variable's initialiser: present before initialize()
+        for(auto &s : syns) {
+            if(s.wum != "static_kernel") { continue; }
+            const auto kernel = readFile<float>(in + "/" + s.name + ".kernel.f32");
+            rt.allocateArray(*s.sg, "kernelg", kernel.size());
+            auto *a = rt.getArray(*s.sg, "kernelg");
+            storeScalars(a, 0, kernel.data(), kernel.size());
+            a->pushToDevice();
+        }
         rt.initialize();
+        const double initialised = sinceStart();
         // a file holds either the whole array or one batch's worth, which is then replicated
         auto load = [&](Runtime::ArrayBase *a, const std::string &file) {
             if(a->getType() == Type::Double && file.size() > 4 && file.compare(file.size() - 4, 4, ".f32") == 0) {
@@ -784,7 +819,7 @@ int main(int argc, char *argv[])
             else if(s.matrix == "bitmask") {
                 load(rt.getArray(*s.sg, "gp"), s.name + ".gp.u32");
             }
-            else if(s.wum != "static_const" && s.wum != "static_init" && s.matrix != "procedural" && s.matrix != "sparse_init") {
+            else if(s.wum != "static_const" && s.wum != "static_init" && s.wum != "static_kernel" && s.matrix != "procedural" && s.matrix != "sparse_init") {
                 load(rt.getArray(*s.sg, "g"), s.name + ".g.f32");
             }
             if(s.wum == "stdp_trace") {
@@ -793,9 +828,16 @@ int main(int argc, char *argv[])
             }
         }
         rt.initializeSparse();
+        // (how long a model takes from loading its code to its first step: allocation, initialize(), initializeSparse())
+        {
+            struct rusage usage;
+            getrusage(RUSAGE_SELF, &usage);
+            std::cout << "ref_driver: ready after " << sinceStart() << " s (allocate " << allocated << ", initialize " << (initialised - allocated)
+                      << "), peak resident host memory " << usage.ru_maxrss / 1024 << " MiB" << std::endl;
+        }
         // matrices initialised by snippets: what the initialisation produced, with the backend's row stride
         for(auto &s : syns) {
-            if(s.matrix != "sparse_init") { continue; }
+            if((s.matrix != "sparse_init" && s.matrix != "conv2d_sparse") || deviceArrays) { continue; }
             const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
             std::ofstream(out + "/" + s.name + ".rowStride.txt") << stride << std::endl;
             auto *rl = rt.getArray(*s.sg, "rowLength"); rl->pullFromDevice();

@@ -413,11 +413,14 @@ def test_library_kernels_say_what_they_do_not_cover():
 
 def test_device_initialisation_is_generated_on_request():
     """Preferences::deviceInitialisation: built-in connectivity and per-synapse variable snippets of SPARSE projections become
-    calls of the device library's generators (with the model's seed and one stream per array) followed by a copy into the host
-    mirrors; without the switch the reference's generic initialisation code runs on the host as before."""
+    calls of the device library's generators (with the model's seed and one stream per array), each followed by a note that
+    the device now holds the array (so that the upload which ends initialize() leaves it alone); host code that walks rows asks
+    for the copy first; without the switch the reference's generic initialisation code runs on the host as before."""
     from genn_amd import configs
     net = configs.snippet_initialised(n_e=200, n_i=50, steps=10)
     net.snap = 0
+    layers = configs.snippet_initialised_layers(steps=10)
+    layers.snap = 0
     tmp = tempfile.mkdtemp(prefix="adapter_devinit_")
     try:
         spec = os.path.join(tmp, "spec")
@@ -432,9 +435,26 @@ def test_device_initialisation_is_generated_on_request():
             assert ("gennmi_init_sparse_fixed_probability(" in init) == flag
             assert ("gennmi_init_sparse_fixed_number_post(" in init) == flag
             assert ("gennmi_init_var(" in init) == flag
+            assert "gennmi_mirrors_begin_initialisation()" in init
             if flag:
-                assert f"{net.seed}ull" in init and "gennmi_memcpy_from_device(" in init
+                assert f"{net.seed}ull" in init and "gennmi_memcpy_from_device(" not in init
+                assert init.count("gennmi_mirror_device_initialised(") >= 8 and "gennmi_mirror_ensure_host(" not in init
                 # EI has a constant weight (no variable), so three weight arrays are drawn; four matrices are generated
                 assert init.count("gennmi_init_var(") == 3 or init.count("gennmi_init_var(") == 2
+        # Conv2D with kernel-initialised weights and FixedNumberPreWithReplacement
+        spec = os.path.join(tmp, "spec_layers")
+        write_netspec(layers, spec)
+        for flag in (True, False):
+            work, out = os.path.join(tmp, f"work_layers{int(flag)}"), os.path.join(tmp, f"out_layers{int(flag)}")
+            os.makedirs(work); os.makedirs(out)
+            res = subprocess.run([DRIVER, spec, work, out, "--generate-only"] + (["--device-init", "--device-arrays"] if flag else []),
+                                 stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+            assert res.returncode == 0, res.stdout[-3000:]
+            init = open(os.path.join(work, layers.name + "_CODE", "init.cc")).read()
+            assert ("gennmi_init_sparse_fixed_number_pre(" in init) == flag
+            # (connectivity, then once more per kernel-initialised variable)
+            assert init.count("gennmi_init_sparse_conv2d(") == (2 if flag else 0)
+            if not flag:
+                assert "idKernel0" in init and "idKernel3" in init
     finally:
         shutil.rmtree(tmp, ignore_errors=True)

@@ -9,6 +9,7 @@ column remap bit-exact.
 Needs the prebuilt driver (built where the reference tree is mounted) and g++/make for the generated runner.
 """
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -739,15 +740,20 @@ def test_generated_kernels_with_random_numbers_in_weight_update_code():
         assert np.abs(got - want).std() > 0.01 * want.mean(), "the stochastic input equals its expectation neuron by neuron"
 
 
-def test_adapter_device_initialisation_matches_host_layer():
+@pytest.mark.parametrize("config", ["snippet_initialised", "snippet_initialised_layers"])
+def test_adapter_device_initialisation_matches_host_layer(config):
     """Preferences::deviceInitialisation through GeNN's generator and Runtime: SPARSE matrices built by FixedProbability
     (with and without autapses) and FixedNumberPostWithReplacement with Uniform, Normal, Constant and constant-parameter
-    weights.  The adapter numbers the generator streams by projection name, so the Python host layer given the same numbering
-    must produce the very same matrices (row lengths, targets, weights) and then the same rasters; with the switch off the
-    reference's host code draws from mt19937, which gives other matrices of the same distribution."""
+    weights; in the second network by Conv2D with kernel-initialised weights and FixedNumberPreWithReplacement.  The adapter
+    numbers the generator streams by projection name, so the Python host layer given the same numbering must produce the very
+    same matrices (row lengths, targets, weights) and then the same rasters; with the switch off the reference's host code
+    draws from mt19937, which gives other matrices of the same distribution — and, for Conv2D, where nothing is drawn, the
+    very same matrix: the reference's own row build code and kernel indexing, run on the host, against the device generator.
+    Further runs place the matrices on the device only (VarLocation::DEVICE: nothing is copied back, the rasters must not
+    change) and take the step's kernels from generated code."""
     from genn_amd import configs
     from genn_amd.genn_model import model_from_net
-    net = configs.snippet_initialised(n_e=1600, n_i=400, steps=150)
+    net = configs.snippet_initialised(n_e=1600, n_i=400, steps=150) if config == "snippet_initialised" else configs.snippet_initialised_layers(steps=150)
     net.snap = 0
     tmp = tempfile.mkdtemp(prefix="adapter_devinit_")
     try:
@@ -761,6 +767,20 @@ def test_adapter_device_initialisation_matches_host_layer():
             res = subprocess.run([DRIVER, spec, work, out] + (["--device-init"] if flag else []), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
             assert res.returncode == 0, res.stdout[-3000:]
             outs[flag] = out
+        # (generated kernels only for the first network: the reference's own generic update code cannot print a merged group
+        # whose archetype has a kernel size while another member has none — getKernelIndex, codeGenUtils.h:131-151, reads
+        # every member's kernel size — and the second network's Conv2D projection merges with a plain SPARSE one)
+        variants = [("device arrays", ["--device-init", "--device-arrays"])]
+        if config == "snippet_initialised":
+            variants.append(("generated", ["--device-init", "--device-arrays", "--kernels=generated"]))
+        for label, options in variants:
+            work, out = os.path.join(tmp, f"work_{label[:6]}"), os.path.join(tmp, f"out_{label[:6]}")
+            os.makedirs(work); os.makedirs(out)
+            print(f"adapter device initialisation ({label}): running {DRIVER}", flush=True)
+            res = subprocess.run([DRIVER, spec, work, out] + options, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+            assert res.returncode == 0, res.stdout[-3000:]
+            assert re.search(r"ready after \S+ s", res.stdout)
+            outs[label] = out
         model = model_from_net(net)
         model.load(num_recording_timesteps=net.steps)
         for s in net.syns:
@@ -780,8 +800,16 @@ def test_adapter_device_initialisation_matches_host_layer():
                 assert np.array_equal(got_g[mask], sg.vars["g"].pull_from_device().reshape(n_pre, stride)[mask]), f"{s.name}: weights differ"
             # host initialisation: another draw of the same distribution
             host_len = np.fromfile(os.path.join(outs[False], f"{s.name}.rowLength.u32"), np.uint32)
-            assert not np.array_equal(host_len, got_len) or s.connect[0] == "FixedNumberPostWithReplacement"
+            assert not np.array_equal(host_len, got_len) or s.connect[0] in ("FixedNumberPostWithReplacement", "Conv2D")
             assert abs(host_len.mean() - got_len.mean()) <= 0.05 * got_len.mean() + 1e-9
+            if s.connect[0] == "Conv2D":
+                host_ind = np.fromfile(os.path.join(outs[False], f"{s.name}.ind.u32"), np.uint32).reshape(n_pre, stride)
+                host_g = np.fromfile(os.path.join(outs[False], f"{s.name}.g.f32"), np.float32).reshape(n_pre, stride)
+                assert np.array_equal(host_len, got_len) and np.array_equal(host_ind[mask], got_ind[mask]) and np.array_equal(host_g[mask], got_g[mask])
+            if s.connect[0] == "FixedNumberPreWithReplacement":
+                for lengths, ind in ((got_len, got_ind), (host_len, np.fromfile(os.path.join(outs[False], f"{s.name}.ind.u32"), np.uint32).reshape(n_pre, stride))):
+                    valid = np.arange(stride)[None, :] < lengths[:, None]
+                    assert np.all(np.bincount(ind[valid], minlength=net.pop(s.trg).n) == s.connect[1]["num"])
         model.run(net.steps)
         model.pull_recording_buffers_from_device()
         total = 0
@@ -789,6 +817,14 @@ def test_adapter_device_initialisation_matches_host_layer():
             got = np.fromfile(os.path.join(outs[True], f"{p.name}.spikes.u32"), np.uint32).reshape(-1, 2)
             want = _raster(model, net, p.name)
             assert np.array_equal(got, want), f"raster of {p.name} differs ({len(got)} vs {len(want)} spikes)"
+            for label, _ in variants:
+                other = np.fromfile(os.path.join(outs[label], f"{p.name}.spikes.u32"), np.uint32).reshape(-1, 2)
+                # (generated kernels add a step's inputs in another order: the rasters agree until rounding separates them)
+                if label == "generated":
+                    first = _first_difference(other, want)
+                    assert first is None or first >= 50, f"{label}: raster of {p.name} differs at step {first}"
+                else:
+                    assert np.array_equal(other, want), f"{label}: raster of {p.name} differs"
             total += len(want)
         assert total > 1000
         model.unload()
@@ -821,6 +857,16 @@ def _procedural_pair(net, steps, snap):
                          if "outPost" in model.synapse_populations[s.name].vars}})
     model.pull_recording_buffers_from_device()
     return out, tmp, model, state
+
+
+def _first_difference(a, b):
+    """First timestep at which two rasters ((step, neuron) pairs in ascending order) differ, or None."""
+    if np.array_equal(a, b):
+        return None
+    n = min(len(a), len(b))
+    diff = np.nonzero(np.any(a[:n] != b[:n], axis=1))[0]
+    k = int(diff[0]) if len(diff) else n
+    return int(min(a[k, 0] if k < len(a) else 1 << 30, b[k, 0] if k < len(b) else 1 << 30))
 
 
 def _raster(model, net, name):

@@ -230,3 +230,42 @@ def test_toeplitz_conv_full_size_batch16():
         oracle.close()
     assert total > 100000
     model.unload()
+
+
+def test_izhikevich_full_size_through_the_reference_runtime_is_ready_within_a_second():
+    """The 10^6-neuron, 10^9-synapse network stated with snippets, through GeNN's generator and Runtime on the MI355X
+    backend with Preferences::deviceInitialisation and every matrix at VarLocation::DEVICE: connectivity and weights are
+    generated where they live, so that from loading the compiled model to the first step (allocation, initialize(),
+    initializeSparse()) takes under a second and the 8 GB of matrices never exist on the host (the process's peak resident
+    memory stays far below them).  The model then steps: within 30 steps the noise current has brought the first
+    thousands of neurons to threshold."""
+    import os
+    import re
+    import shutil
+    import subprocess
+    import tempfile
+    from genn_amd.netspec import write_netspec
+    driver = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "_ref", "mi355x_driver")
+    if not os.path.exists(driver):
+        pytest.skip("oracle/_ref/mi355x_driver is not built")
+    net = configs.izhikevich_fanout_snippets(steps=30)
+    net.snap = 0
+    tmp = tempfile.mkdtemp(prefix="adapter_izh_full_")
+    try:
+        spec, work, out = (os.path.join(tmp, d) for d in ("spec", "work", "out"))
+        for d in (work, out):
+            os.makedirs(d)
+        write_netspec(net, spec)
+        print(f"full-size izhikevich network through {driver}", flush=True)
+        res = subprocess.run([driver, spec, work, out, "--device-init", "--device-arrays"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=400)
+        assert res.returncode == 0, res.stdout[-3000:]
+        m = re.search(r"ready after (\S+) s \(allocate (\S+), initialize (\S+)\), peak resident host memory (\d+) MiB", res.stdout)
+        assert m, res.stdout[-2000:]
+        ready, peak = float(m.group(1)), int(m.group(4))
+        print(res.stdout[-600:], flush=True)
+        assert ready < 1.0, f"ready after {ready} s"
+        assert peak < 2048, f"peak resident host memory {peak} MiB"
+        spikes = sum(len(np.fromfile(os.path.join(out, f"{p.name}.spikes.u32"), np.uint32)) // 2 for p in net.pops)
+        assert spikes > 5000, spikes
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)

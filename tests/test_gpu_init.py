@@ -141,17 +141,21 @@ def test_connect_init():
                                          init_sparse_connectivity("FixedNumberTotalWithReplacement", {"num": 1000}))
     fixed_post = model.add_synapse_population("FixedNumberPost", "SPARSE", pre, post, _static(), init_postsynaptic("DeltaCurr"),
                                               init_sparse_connectivity("FixedNumberPostWithReplacement", {"num": 10}))
+    fixed_pre = model.add_synapse_population("FixedNumberPre", "SPARSE", pre, post, _static(), init_postsynaptic("DeltaCurr"),
+                                             init_sparse_connectivity("FixedNumberPreWithReplacement", {"num": 10}))
     one = model.add_synapse_population("OneToOne", "SPARSE", pre, post, _static(), init_postsynaptic("DeltaCurr"),
                                        init_sparse_connectivity("OneToOne"))
     model.build()
     model.load()
-    for s in (total, fixed_post, one):
+    for s in (total, fixed_post, fixed_pre, one):
         s.pull_connectivity_from_device()
         assert s.get_sparse_post_inds().max() < 100
         for r in range(100):
             row = s.ind_host[r, :s.row_length_host[r]]
             assert np.all(np.diff(row.astype(np.int64)) >= 0), f"{s.name}: row {r} is not ascending"
     assert np.all(np.bincount(fixed_post.get_sparse_pre_inds()) == 10)
+    assert np.all(np.bincount(fixed_pre.get_sparse_post_inds()) == 10)
+    assert stats.chisquare(np.bincount(fixed_pre.get_sparse_pre_inds(), minlength=100)).pvalue > P_CONNECT
     assert len(total.get_sparse_pre_inds()) == 1000
     assert np.array_equal(one.get_sparse_pre_inds(), one.get_sparse_post_inds())
     assert stats.chisquare(np.bincount(fixed_post.get_sparse_post_inds(), minlength=100)).pvalue > P_CONNECT
@@ -203,6 +207,98 @@ def test_fixed_number_post_long_rows():
         p = stats.kstest(x[:, k - 1], stats.beta(k, n + 1 - k).cdf).pvalue
         assert p > P_CONNECT, f"order statistic {k} of {n} fails the KS test (p={p})"
     assert stats.chisquare(np.bincount(ind.reshape(-1) // 1000, minlength=100)).pvalue > P_CONNECT
+
+
+@pytest.mark.parametrize("num_pre,num_post,num", [(1000, 20000, 50), (37, 5000, 3), (20000, 300, 1000), (1, 100, 7)])
+def test_fixed_number_pre(num_pre, num_post, num):
+    """FixedNumberPreWithReplacement (initSparseConnectivitySnippet.h:380-410): every column holds exactly `num` entries
+    (tests/features/test_connect_init.py:55), the sources of one column are independent uniform draws (so the pooled
+    sources are uniform, row lengths are Binomial(num * numPost, 1 / numPre) and the number of DISTINCT sources of a column
+    follows the occupancy law), rows come out ascending and nothing overflows at the reference's row stride."""
+    row_length, ind = _connectivity("FixedNumberPreWithReplacement", {"num": num}, num_pre, num_post)
+    assert ind.shape[0] == num_pre and row_length.sum() == num * num_post
+    valid = np.arange(ind.shape[1])[None, :] < row_length[:, None]
+    post = ind[valid]
+    pre = np.repeat(np.arange(num_pre), row_length)
+    assert post.max() < num_post
+    assert np.all(np.bincount(post, minlength=num_post) == num)
+    for r in range(0, num_pre, max(1, num_pre // 200)):
+        assert np.all(np.diff(ind[r, :row_length[r]].astype(np.int64)) >= 0), f"row {r} is not ascending"
+    if num_pre > 1:
+        assert stats.chisquare(row_length.astype(np.float64)).pvalue > P_CONNECT
+        # distinct sources per column: E = numPre (1 - (1 - 1/numPre)^num); a generator that reused one word for several
+        # draws of a column, or one column's draws for the next, would collapse this
+        distinct = np.zeros(num_post, dtype=np.int64)
+        pairs = np.unique(post.astype(np.int64) * num_pre + pre)
+        np.add.at(distinct, pairs // num_pre, 1)
+        expected = num_pre * (1.0 - (1.0 - 1.0 / num_pre) ** num)
+        spread = np.sqrt(max(1e-12, num_pre * (1 - 1 / num_pre) ** num * (1 - (1 - 1 / num_pre) ** num)) / num_post)
+        assert abs(distinct.mean() - expected) < 5.0 * spread + 1e-9, (distinct.mean(), expected, spread)
+        # two columns never share their whole draw
+        if num >= 3 and num_pre >= 1000:
+            order = np.lexsort((pre, post))
+            columns = pre[order].reshape(num_post, num)
+            assert len(np.unique(columns, axis=0)) == num_post
+
+
+def _conv2d_rows(p):
+    """Brute force over (pre, post) pairs: a synapse exists where the kernel covers the input pixel, the definition that
+    the snippet's row build code (initSparseConnectivitySnippet.h:438-483) enumerates."""
+    rows, kernel_index = [], []
+    for pre in range(p["conv_ih"] * p["conv_iw"] * p["conv_ic"]):
+        in_row, in_col, in_chan = (pre // p["conv_ic"]) // p["conv_iw"], (pre // p["conv_ic"]) % p["conv_iw"], pre % p["conv_ic"]
+        row, kern = [], []
+        for out_row in range(p["conv_oh"]):
+            kr = in_row - (out_row * p["conv_sh"] - p["conv_padh"])
+            if not 0 <= kr < p["conv_kh"]:
+                continue
+            for out_col in range(p["conv_ow"]):
+                kc = in_col - (out_col * p["conv_sw"] - p["conv_padw"])
+                if not 0 <= kc < p["conv_kw"]:
+                    continue
+                for out_chan in range(p["conv_oc"]):
+                    row.append((out_row * p["conv_ow"] + out_col) * p["conv_oc"] + out_chan)
+                    kern.append(((kr * p["conv_kw"] + kc) * p["conv_ic"] + in_chan) * p["conv_oc"] + out_chan)
+        rows.append(row)
+        kernel_index.append(kern)
+    return rows, kernel_index
+
+
+@pytest.mark.parametrize("shape", [
+    dict(conv_kh=3, conv_kw=3, conv_sh=1, conv_sw=1, conv_padh=1, conv_padw=1, conv_ih=8, conv_iw=8, conv_ic=2, conv_oh=8, conv_ow=8, conv_oc=3),
+    dict(conv_kh=3, conv_kw=3, conv_sh=1, conv_sw=1, conv_padh=0, conv_padw=0, conv_ih=10, conv_iw=7, conv_ic=1, conv_oh=8, conv_ow=5, conv_oc=4),
+    dict(conv_kh=5, conv_kw=3, conv_sh=2, conv_sw=2, conv_padh=2, conv_padw=1, conv_ih=11, conv_iw=9, conv_ic=3, conv_oh=6, conv_ow=5, conv_oc=2),
+    dict(conv_kh=2, conv_kw=4, conv_sh=3, conv_sw=2, conv_padh=0, conv_padw=1, conv_ih=9, conv_iw=12, conv_ic=1, conv_oh=3, conv_ow=6, conv_oc=5),
+    dict(conv_kh=1, conv_kw=1, conv_sh=1, conv_sw=1, conv_padh=0, conv_padw=0, conv_ih=4, conv_iw=4, conv_ic=3, conv_oh=4, conv_ow=4, conv_oc=3),
+])
+def test_conv2d_as_sparse_connectivity(shape):
+    """Conv2D as SPARSE connectivity with Kernel-initialised weights (initSparseConnectivitySnippet.h:438-497,
+    initVarSnippet.h:100-108) against a brute force over every (pre, post) pair: same targets in the same (ascending)
+    order, every weight the kernel entry of its (kernel row, kernel column, input channel, output channel); strides above
+    one (where some kernel rows have no output row), no padding, and kernels wider than the stride are covered."""
+    rng = np.random.default_rng(3)
+    kernel = rng.normal(size=(shape["conv_kh"], shape["conv_kw"], shape["conv_ic"], shape["conv_oc"])).astype(np.float32)
+    model = _empty_model(1)
+    n_pre, n_post = shape["conv_ih"] * shape["conv_iw"] * shape["conv_ic"], shape["conv_oh"] * shape["conv_ow"] * shape["conv_oc"]
+    pre = model.add_neuron_population("Pre", n_pre, "LIF", _LIF, {"V": 0.0, "RefracTime": 0.0})
+    post = model.add_neuron_population("Post", n_post, "LIF", _LIF, {"V": 0.0, "RefracTime": 0.0})
+    s = model.add_synapse_population("S", "SPARSE", pre, post, init_weight_update("StaticPulse", {}, {"g": init_var("Kernel", {"kernel": kernel})}),
+                                     init_postsynaptic("DeltaCurr"), init_sparse_connectivity("Conv2D", shape))
+    model.build()
+    model.load()
+    s.pull_connectivity_from_device()
+    s.vars["g"].pull_from_device()
+    g = s.vars["g"].view.reshape(n_pre, s.row_stride).copy()
+    row_length, ind = s.row_length_host.copy(), s.ind_host.copy()
+    model.unload()
+    rows, kernel_index = _conv2d_rows(shape)
+    flat = kernel.reshape(-1)
+    assert s.row_stride == -(-shape["conv_kh"] // shape["conv_sh"]) * -(-shape["conv_kw"] // shape["conv_sw"]) * shape["conv_oc"]
+    assert max(len(r) for r in rows) <= s.row_stride
+    for i, (row, kern) in enumerate(zip(rows, kernel_index)):
+        assert row_length[i] == len(row), f"row {i}"
+        assert np.array_equal(ind[i, :len(row)], np.asarray(row, dtype=np.uint32)), f"row {i}"
+        assert np.array_equal(g[i, :len(row)], flat[kern]), f"row {i}: weights"
 
 
 @pytest.mark.parametrize("num_post", [1000, 37, 5000])
