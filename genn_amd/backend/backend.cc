@@ -980,6 +980,48 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
     const std::string seedExpr = (model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull")
                                                         : std::string("gennmiRandomSeed()");
 
+    // Per-synapse variables whose initialisers are all value snippets the device library draws itself
+    // (Preferences::deviceInitialisation), of every projection of merged group `s`: one gennmi_init_var per variable over
+    // `count` elements (padding of sparse rows included: it is never read), and a note that the device now holds the array.
+    // False, and nothing emitted, when some variable needs the reference's host code.
+    auto emitDeviceVars = [&](auto &s, auto &env, const std::string &count) -> bool
+    {
+        if(!deviceInit || !s.getArchetype().isWUVarInitRequired() || batchSize != 1) { return false; }
+        struct DeviceVar { std::string name; unsigned int snippet; std::vector<std::string> params; };
+        std::vector<DeviceVar> deviceVars;
+        for(const auto &var : s.getArchetype().getWUInitialiser().getSnippet()->getVars()) {
+            const auto &init = s.getArchetype().getWUInitialiser().getVarInitialisers().at(var.name);
+            if(Utils::areTokensEmpty(init.getCodeTokens()) || init.isKernelRequired()) { continue; }    // nothing to do here
+            DeviceVar d{var.name, 0, {}};
+            if(var.type.resolve(model.getTypeContext()) != Type::Float || !deviceVarSnippet(init.getSnippet(), d.snippet, d.params)) { return false; }
+            for(const auto &g : s.getGroups()) {
+                if(g.get().getWUInitialiser().getVarInitialisers().at(var.name).getSnippet() != init.getSnippet()) { return false; }
+            }
+            deviceVars.push_back(d);
+        }
+        size_t varIndex = 0;
+        for(const auto &d : deviceVars) {
+            const std::string name = d.name;
+            env.addField(Type::Float.createPointer(), "_mi_init_" + name, name,
+                         [name](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, name); });
+            std::vector<uint64_t> streams;
+            for(const auto &g : s.getGroups()) { streams.push_back(2 * place(g.get()) + 2 + 2 * numProjections * varIndex); }
+            CodeStream::Scope scope(env.getStream());
+            env.getStream() << "static const uint32_t stream[] = " << tableU32(streams) << ";" << std::endl;
+            env.getStream() << "double params[4] = {0.0, 0.0, 0.0, 0.0};" << std::endl;
+            for(size_t k = 0; k < d.params.size(); k++) {
+                std::vector<Type::NumericValue> values;
+                for(const auto &g : s.getGroups()) { values.push_back(g.get().getWUInitialiser().getVarInitialisers().at(name).getParams().at(d.params[k])); }
+                env.getStream() << "{ static const double v[] = " << table(values, Type::Double) << "; params[" << k << "] = v[g]; }" << std::endl;
+            }
+            env.getStream() << "GENNMI_CHECK(gennmi_init_var(gennmiDev(" << env["_mi_init_" + name] << "), " << GENNMI_TYPE_F32 << "u, " << count << ", "
+                            << d.snippet << "u, params, " << seedExpr << ", stream[g]));" << std::endl;
+            env.getStream() << "GENNMI_CHECK(gennmi_mirror_device_initialised(" << env["_mi_init_" + name] << "));" << std::endl;
+            varIndex++;
+        }
+        return true;
+    };
+
     std::ostringstream bodyStream;
     CodeStream body(bodyStream);
     EnvironmentLibrary rngEnv(body, StandardLibrary::getHostRNGFunctions(model.getPrecision()));
@@ -1031,7 +1073,12 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                 {
                     EnvironmentGroupMergedField<SynapseInitGroupMerged> env(funcEnv, s);
                     buildStandardEnvironment(env, batchSize);
-                    s.generateInit(*this, env, batchSize);
+                    // variables of DENSE matrices and of kernels (initGroupMerged.cc:563-593): drawn on the device where every
+                    // one of them can be, else the reference's loops on the host
+                    const bool kernel = (s.getArchetype().getMatrixType() & SynapseMatrixWeight::KERNEL);
+                    if(!emitDeviceVars(s, env, kernel ? ("(size_t)" + env["_kernel_size"]) : ("(size_t)" + env["num_pre"] + " * " + env["_row_stride"]))) {
+                        s.generateInit(*this, env, batchSize);
+                    }
                 });
             });
         // variables of custom updates (per neuron, and per synapse of DENSE and KERNEL matrices)
@@ -1259,52 +1306,14 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                 {
                     EnvironmentGroupMergedField<SynapseSparseInitGroupMerged> env(funcEnv, s);
                     buildStandardEnvironment(env, batchSize);
-                    // per-synapse variables whose initialisers are all snippets the device library draws itself
-                    // (Preferences::deviceInitialisation): filled over the whole numPre * rowStride range, padding is never read
-                    bool varsOnDevice = deviceInit && s.getArchetype().isWUVarInitRequired() && (batchSize == 1);
-                    struct DeviceVar { std::string name; unsigned int snippet; std::vector<std::string> params; };
-                    std::vector<DeviceVar> deviceVars;
                     // (variables initialised from a kernel were written while the rows were built)
                     bool anyRowVar = false;
                     for(const auto &var : s.getArchetype().getWUInitialiser().getSnippet()->getVars()) {
                         const auto &init = s.getArchetype().getWUInitialiser().getVarInitialisers().at(var.name);
                         anyRowVar = anyRowVar || (!Utils::areTokensEmpty(init.getCodeTokens()) && !init.isKernelRequired());
                     }
-                    if(varsOnDevice) {
-                        for(const auto &var : s.getArchetype().getWUInitialiser().getSnippet()->getVars()) {
-                            const auto &init = s.getArchetype().getWUInitialiser().getVarInitialisers().at(var.name);
-                            if(Utils::areTokensEmpty(init.getCodeTokens()) || init.isKernelRequired()) { continue; }    // nothing to do here
-                            DeviceVar d{var.name, 0, {}};
-                            varsOnDevice = varsOnDevice && var.type.resolve(model.getTypeContext()) == Type::Float
-                                           && deviceVarSnippet(init.getSnippet(), d.snippet, d.params);
-                            for(const auto &g : s.getGroups()) {
-                                varsOnDevice = varsOnDevice && (g.get().getWUInitialiser().getVarInitialisers().at(var.name).getSnippet() == init.getSnippet());
-                            }
-                            deviceVars.push_back(d);
-                        }
-                    }
-                    if(varsOnDevice) {
-                        size_t varIndex = 0;
-                        for(const auto &d : deviceVars) {
-                            const std::string name = d.name;
-                            env.addField(Type::Float.createPointer(), "_mi_init_" + name, name,
-                                         [name](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, name); });
-                            std::vector<uint64_t> streams;
-                            for(const auto &g : s.getGroups()) { streams.push_back(2 * place(g.get()) + 2 + 2 * numProjections * varIndex); }
-                            CodeStream::Scope scope(env.getStream());
-                            env.getStream() << "static const uint32_t stream[] = " << tableU32(streams) << ";" << std::endl;
-                            env.getStream() << "double params[4] = {0.0, 0.0, 0.0, 0.0};" << std::endl;
-                            for(size_t k = 0; k < d.params.size(); k++) {
-                                std::vector<Type::NumericValue> values;
-                                for(const auto &g : s.getGroups()) { values.push_back(g.get().getWUInitialiser().getVarInitialisers().at(name).getParams().at(d.params[k])); }
-                                env.getStream() << "{ static const double v[] = " << table(values, Type::Double) << "; params[" << k << "] = v[g]; }" << std::endl;
-                            }
-                            const std::string count = "(size_t)" + env["num_pre"] + " * " + env["_row_stride"];
-                            env.getStream() << "GENNMI_CHECK(gennmi_init_var(gennmiDev(" << env["_mi_init_" + name] << "), " << GENNMI_TYPE_F32 << "u, " << count << ", "
-                                            << d.snippet << "u, params, " << seedExpr << ", stream[g]));" << std::endl;
-                            env.getStream() << "GENNMI_CHECK(gennmi_mirror_device_initialised(" << env["_mi_init_" + name] << "));" << std::endl;
-                            varIndex++;
-                        }
+                    if(emitDeviceVars(s, env, "(size_t)" + env["num_pre"] + " * " + env["_row_stride"])) {
+                        // (drawn on the device)
                     }
                     else if(s.getArchetype().isWUVarInitRequired() && anyRowVar) {
                         // (rows the device generated are fetched first)

@@ -177,7 +177,7 @@ def write_netspec(net: Net, path: str):
         lines.append(f"batch {int(net.batch_size)}")
     if net.precision != "float":
         lines.append(f"precision {net.precision}")
-    if any(s.matrix in ("procedural", "sparse_init") for s in net.syns) or any(c.model == "poisson_exp" for c in net.css) or any(p.model == "poisson" for p in net.pops) \
+    if any(s.matrix in ("procedural", "sparse_init") or s.g_init is not None for s in net.syns) or any(c.model == "poisson_exp" for c in net.css) or any(p.model == "poisson" for p in net.pops) \
             or any(s.wum == "stochastic" for s in net.syns):
         lines.append(f"seed {int(net.seed)}")        # procedural matrices and Poisson sources draw from the model's seed
     for kind, group, param, step, value in net.dynamic:
@@ -212,8 +212,8 @@ def write_netspec(net: Net, path: str):
             head = f"syn {s.name} sparse {s.src} {s.trg} {s.row_stride}"
             np.ascontiguousarray(s.row_length, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.rowLength.u32"))
             np.ascontiguousarray(s.ind, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.ind.u32"))
-        elif s.matrix == "dense":
-            head = f"syn {s.name} dense {s.src} {s.trg}"
+        elif s.matrix in ("dense", "dense_init"):
+            head = f"syn {s.name} {s.matrix} {s.src} {s.trg}"
         elif s.matrix == "sparse_init" and s.connect[0] == "Conv2D":
             head = f"syn {s.name} conv2d_sparse {s.src} {s.trg} " + " ".join(str(int(s.connect[1][k])) for k in CONV_SPARSE_PARAMS)
         elif s.matrix in ("procedural", "sparse_init"):
@@ -225,7 +225,8 @@ def write_netspec(net: Net, path: str):
             np.ascontiguousarray(s.gp, dtype=np.uint32).tofile(os.path.join(path, f"{s.name}.gp.u32"))
         else:
             head = f"syn {s.name} conv2d {s.src} {s.trg} " + " ".join(str(int(s.conv[k])) for k in CONV_PARAMS)
-        regenerated = (s.matrix == "dense" and s.wum == "static" and s.g_init is not None)     # DENSE with weights from a snippet, never stored
+        # DENSE with weights from a snippet, never stored; "dense_init": stored, and a kernel whose entries a snippet draws
+        regenerated = (s.matrix in ("dense", "dense_init", "conv2d") and s.wum == "static" and s.g_init is not None)
         if s.wum != "static_const" and s.matrix not in ("procedural", "sparse_init") and not regenerated:
             np.ascontiguousarray(s.g, dtype=np.float32).tofile(os.path.join(path, f"{s.name}.g.f32"))
         if s.matrix == "sparse_init" and s.wum == "static" and s.g_init[0] == "Kernel":

@@ -484,7 +484,8 @@ int main(int argc, char *argv[])
                     // Conv2D as SPARSE connectivity: kh kw sh sw padh padw ih iw ic oh ow oc (initSparseConnectivitySnippet.h:438-497)
                     else if(s.matrix == "conv2d_sparse") { s.conv.resize(12); for(auto &c : s.conv) ls >> c; }
                     else if(s.matrix == "procedural" || s.matrix == "sparse_init") { ls >> s.connect >> s.connectValue; }
-                    else if(s.matrix != "dense" && s.matrix != "bitmask") throw std::runtime_error("matrix " + s.matrix);
+                    // ("dense_init": a stored DENSE matrix whose weights an initialisation snippet draws, wum static_init)
+                    else if(s.matrix != "dense" && s.matrix != "dense_init" && s.matrix != "bitmask") throw std::runtime_error("matrix " + s.matrix);
                     ls >> s.wum;
                     if(s.wum == "static_init") { ls >> s.initSnippet; const int np = (s.initSnippet == "Constant") ? 1 : 2; s.wumP.resize(np); for(auto &c : s.wumP) ls >> c; }
                     if(s.wum == "static_delay") { ls >> s.maxDenDelay; }
@@ -644,6 +645,9 @@ int main(int argc, char *argv[])
                 s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::SPARSE, src, trg, wum, psm);
                 s.sg->setMaxConnections(s.rowStride);
                 if(s.colStride) s.sg->setMaxSourceConnections(s.colStride);
+            }
+            else if(s.matrix == "dense_init") {
+                s.sg = model.addSynapsePopulation(s.name, SynapseMatrixType::DENSE, src, trg, wum, psm);
             }
             else if(s.matrix == "dense") {
                 // (weights given by an initialisation snippet are regenerated at every event, never stored: DENSE_PROCEDURALG)
@@ -837,6 +841,11 @@ int main(int argc, char *argv[])
         }
         // matrices initialised by snippets: what the initialisation produced, with the backend's row stride
         for(auto &s : syns) {
+            if(s.matrix == "dense_init" || (s.matrix == "conv2d" && s.wum == "static_init")) {
+                auto *g = rt.getArray(*s.sg, "g"); g->pullFromDevice();
+                appendScalars(out + "/" + s.name + ".g.f32", g, 0, g->getCount());
+                continue;
+            }
             if((s.matrix != "sparse_init" && s.matrix != "conv2d_sparse") || deviceArrays) { continue; }
             const size_t numPre = popByName.at(s.src)->n, stride = backendStride(s);
             std::ofstream(out + "/" + s.name + ".rowStride.txt") << stride << std::endl;
