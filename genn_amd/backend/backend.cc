@@ -976,6 +976,20 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
         return (uint64_t)std::distance(model.getSynapseGroups().cbegin(), model.getSynapseGroups().find(g.getName()));
     };
     const uint64_t numProjections = model.getSynapseGroups().size();
+    // Generator streams are numbered in ranges per consumer under one key (the model's seed): initialisation arrays from 1
+    // (2k + 1, 2k + 2 + 2 P v), current sources from 1000, neuron code from 2000, weight-update code from 3000 (eight per
+    // projection), custom connectivity updates from 6000.  A model large enough for two ranges to meet would draw the same
+    // words in two places, so it is refused here rather than simulated with correlated noise.
+    {
+        size_t maxVars = 0;
+        for(const auto &g : model.getSynapseGroups()) { maxVars = std::max(maxVars, g.second.getWUInitialiser().getSnippet()->getVars().size()); }
+        size_t numCurrentSources = 0;
+        for(const auto &n : model.getNeuronGroups()) { numCurrentSources += n.second.getCurrentSources().size(); }
+        if(2 * numProjections * (maxVars + 1) + 2 >= 1000 || numCurrentSources >= 1000 || model.getNeuronGroups().size() >= 1000 || numProjections >= 375) {
+            unsupported("a model of this many groups (the counter-based generator's stream ranges of initialisation arrays, current sources, "
+                        "neuron code and weight-update code would overlap)");
+        }
+    }
     // the model's seed, or one drawn when the runner is loaded (ModelSpec: seed 0 = a different one every run)
     const std::string seedExpr = (model.getSeed() != 0) ? (std::to_string(model.getSeed()) + "ull")
                                                         : std::string("gennmiRandomSeed()");

@@ -89,6 +89,7 @@ struct gennmi_runner
     uint32_t neuronsPerLane = 1;        // 2, 4 or 8: neuronBulkKernel instead of neuronUpdateKernel
     bool plainGroups = false;           // every group is one the several-neurons-per-lane neuron update covers
     bool sourcesStale = false;          // startSpike / endSpike / spikeTimes of a spike source were written since nextSpikeTime was built
+    bool failed = false;                // a queued step failed part-way: what was queued behind it is lost, the runner refuses to go on
     bool resStale = false;              // connectivity or weights were written since the tables were built ...
     std::vector<uint8_t> resStaleProj;  // ... of these projections (index into pre)
     bool tablesStale = false;           // rowLength / ind / d of a projection were written since the connectivity-derived tables were built
@@ -1795,6 +1796,7 @@ static int launchNeurons(gennmi_runner *r, const StepArgs &a, bool timed)
 int gennmi_update_synapses(gennmi_runner *r, float t)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "update_synapses: runner not finalised"); }
+    if(r->failed) { return fail(GENNMI_ESTATE, "update_synapses: an earlier queued step of this runner failed, the runner cannot continue"); }
     FLUSH_QUEUED();
     { const int rc = refreshTables(r); if(rc) { return rc; } }
     StepArgs a{};
@@ -1808,6 +1810,7 @@ int gennmi_update_synapses(gennmi_runner *r, float t)
 int gennmi_update_neurons(gennmi_runner *r, float t, uint32_t recordingTimestep)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "update_neurons: runner not finalised"); }
+    if(r->failed) { return fail(GENNMI_ESTATE, "update_neurons: an earlier queued step of this runner failed, the runner cannot continue"); }
     FLUSH_QUEUED();
     { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
     StepArgs a{};
@@ -1852,12 +1855,21 @@ static int stepNow(gennmi_runner *r, float t, uint32_t recordingTimestep)
 
 // Executes the steps a runner has queued: runs of steps whose recording rows follow one another (or that all record into row
 // 0: no recording, or a one-row buffer) go to the resident kernel in one launch, anything shorter than it accepts step by step.
+static int flushRunnerSteps(gennmi_runner *r, const std::vector<gennmi_runner::QueuedStep> &steps);
+// (The queue belongs to the thread that steps the runner: one host thread per runner.)
 static int flushRunner(gennmi_runner *r)
 {
     if(r->queued.empty()) { return GENNMI_OK; }
     std::vector<gennmi_runner::QueuedStep> steps;
     steps.swap(r->queued);
     g_queuedRunners--;
+    const int rc = flushRunnerSteps(r, steps);
+    // steps behind a failed one cannot be run later (the network's state is that of a step half done): say so from now on
+    if(rc) { r->failed = true; }
+    return rc;
+}
+static int flushRunnerSteps(gennmi_runner *r, const std::vector<gennmi_runner::QueuedStep> &steps)
+{
     { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
     { const int rc = refreshTables(r); if(rc) { return rc; } }
     size_t first = 0;
@@ -1893,6 +1905,7 @@ int gennmi_runner_set_step_queue(gennmi_runner *r, uint32_t maxSteps)
 int gennmi_step(gennmi_runner *r, float t, uint32_t recordingTimestep)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "step: runner not finalised"); }
+    if(r->failed) { return fail(GENNMI_ESTATE, "step: an earlier queued step of this runner failed, the runner cannot continue"); }
     if(r->stepQueueLimit && r->resident && !r->timing) {
         if(r->queued.empty()) { g_queuedRunners++; }
         r->queued.push_back({t, recordingTimestep});
@@ -1907,6 +1920,7 @@ int gennmi_step(gennmi_runner *r, float t, uint32_t recordingTimestep)
 int gennmi_run_steps(gennmi_runner *r, unsigned long long timestep, unsigned long long numSteps, unsigned long long numRecordingTimesteps)
 {
     if(!r || !r->finalised) { return fail(GENNMI_ESTATE, "run_steps: runner not finalised"); }
+    if(r->failed) { return fail(GENNMI_ESTATE, "run_steps: an earlier queued step of this runner failed, the runner cannot continue"); }
     FLUSH_QUEUED();
     { const int rc = refreshSpikeSources(r); if(rc) { return rc; } }
     { const int rc = refreshTables(r); if(rc) { return rc; } }
@@ -2140,8 +2154,7 @@ int gennmi_max_col_length_static(uint32_t numSrc, uint32_t numTrg, uint32_t rowS
     if((total + BLOCK - 1) / BLOCK > 0x7FFFFFFFull) { return fail(GENNMI_EINVAL, "max_col_length_static: matrix too large for one launch"); }
     uint32_t *counters = nullptr;
     { const int rc = staticScratch(&counters); if(rc) { return rc; } }
-    // the array keeps the last call's counts: clear what this call uses (a kernel, not a memset, so that the sequence
-    // stays legal for callers that record it)
+    // the array keeps the last call's counts: clear what this call uses
     staticClearKernel<<<dim3((numTrg + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, 0>>>(counters, numTrg, maxColLengthDev);
     remapCountKernel<<<dim3((unsigned int)((total + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, 0>>>(numSrc, rowStride, rowLength, ind, 0, counters, nullptr, nullptr);
     staticMaxKernel<<<dim3((numTrg + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, 0>>>(counters, numTrg, maxColLengthDev);

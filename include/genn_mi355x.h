@@ -371,12 +371,14 @@ int gennmi_init_random_words(uint32_t *dev, size_t count, uint64_t seed, uint32_
 int gennmi_max_col_length(uint32_t numSrcNeurons, uint32_t numTrgNeurons, uint32_t rowStride,
                           const uint32_t *rowLength, const uint32_t *ind, uint32_t *maxColLength);
 
-/* gennmi_max_col_length for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The per-column counters live in an array
+/* gennmi_max_col_length for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc).  It has no counterpart in the reference.  The per-column counters live in an array
  * that is part of the library's device image (GENNMI_STATIC_MAX_TARGETS counters = 4 MiB on every GPU the library runs
  * on, held until the process ends), so the call allocates and frees nothing; numTrgNeurons above that limit is rejected
  * with GENNMI_EINVAL.  The result is written to DEVICE memory (*maxColLengthDev, one uint32 the caller owns); the
- * kernels are queued on the null stream and the call returns without waiting for them.  All calls on one GPU share
+ * kernels are queued on the null stream (so the call is ordered against every blocking stream, and cannot itself be recorded
+ * into a graph) and the call returns without waiting for them; steps still queued in a runner are not run first (gennmi_flush
+ * does that).  All calls on one GPU share
  * the array: calls that overlap on one GPU (from several threads or streams) race. */
 #define GENNMI_STATIC_MAX_TARGETS (1u << 20)
 int gennmi_max_col_length_static(uint32_t numSrcNeurons, uint32_t numTrgNeurons, uint32_t rowStride,

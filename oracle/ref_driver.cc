@@ -13,7 +13,6 @@
 // initialisation snippets is used, because their draw order cannot be reproduced elsewhere.
 //
 // usage: ref_driver <netspec dir> <work dir> <out dir>
-#include <sys/resource.h>
 #include <algorithm>
 #include <chrono>
 #include <cmath>
@@ -834,10 +833,14 @@ int main(int argc, char *argv[])
         rt.initializeSparse();
         // (how long a model takes from loading its code to its first step: allocation, initialize(), initializeSparse())
         {
-            struct rusage usage;
-            getrusage(RUSAGE_SELF, &usage);
+            // (VmHWM of this process image: getrusage's ru_maxrss also carries the peak of the process that started this one)
+            long peakKiB = 0;
+            std::ifstream status("/proc/self/status");
+            for(std::string line; std::getline(status, line); ) {
+                if(line.rfind("VmHWM:", 0) == 0) { peakKiB = std::stol(line.substr(6)); }
+            }
             std::cout << "ref_driver: ready after " << sinceStart() << " s (allocate " << allocated << ", initialize " << (initialised - allocated)
-                      << "), peak resident host memory " << usage.ru_maxrss / 1024 << " MiB" << std::endl;
+                      << "), peak resident host memory " << peakKiB / 1024 << " MiB" << std::endl;
         }
         // matrices initialised by snippets: what the initialisation produced, with the backend's row stride
         for(auto &s : syns) {

@@ -66,27 +66,48 @@ def test_balanced_lif_full_run():
     model.unload()
 
 
+def _spikes_per_step(words, steps, words_per_step, first_word, last_word):
+    """Spikes per step of the neurons whose recording words are [first_word, last_word), from the packed bitfield."""
+    rows = np.ascontiguousarray(words).reshape(steps, words_per_step)[:, first_word:last_word]
+    counts = np.zeros(steps, dtype=np.int64)
+    for s0 in range(0, steps, 200):         # (unpacked 200 steps at a time: a byte per neuron and step otherwise)
+        chunk = np.ascontiguousarray(rows[s0:s0 + 200]).view(np.uint8)
+        counts[s0:s0 + 200] = np.unpackbits(chunk, axis=1).sum(axis=1)
+    return counts
+
+
 def test_izhikevich_full_run():
-    """Config 3: 10^6 Izhikevich neurons, 10^9 synapses, dt 1 ms, 1,000 steps (1 s simulated), one row of the noise array
-    per step.  Activity is a sequence of population bursts; excitatory and inhibitory rows are rated separately."""
-    steps = 1000
-    net = configs.izhikevich_fanout(steps=steps)
+    """Config 3: 10^6 Izhikevich neurons, 10^9 synapses, dt 1 ms, the noise array's 1,000 rows cycled.  Excitatory and
+    inhibitory rows are rated separately.
+
+    This network fires in population bursts, about one spike per neuron each and a dozen per second, and parts from the
+    oracle at the first of them (step 66: a threshold crossing flipped by the order of fp32 atomic additions).  Whether the
+    window's last burst falls inside it then moves the rate over the configuration's one simulated second by a few
+    per cent from run to run of the very same kernels (two runs: 0.45 % and 3.1 % from the oracle), so one second cannot
+    carry a 2 % gate; four seconds (some fifty bursts) can.  The first second is held to 8 %, one burst's worth."""
+    steps, second = 4000, 1000
+    net = configs.izhikevich_fanout(steps=steps, noise_steps=1000)
     n = net.pops[0].n
-    assert n == 1_000_000 and int(net.syns[0].row_length.sum()) == 1_000_000_000 and net.css[0].noise.shape[0] == steps
+    assert n == 1_000_000 and int(net.syns[0].row_length.sum()) == 1_000_000_000 and net.css[0].noise.shape[0] == 1000
     model, oracle = _full_run(net, steps)
-    got = _bits(model.neuron_populations["N"].vars["recordSpk"].view, n, steps)
-    want = _bits(oracle.record("N", steps), n, steps)
+    words = (n + 31) // 32
+    got = np.ascontiguousarray(model.neuron_populations["N"].vars["recordSpk"].view).reshape(steps, words)
+    want = np.ascontiguousarray(oracle.record("N", steps)).reshape(steps, words)
     diff = np.nonzero((got != want).any(axis=1))[0]
     identical_until = int(diff[0]) if len(diff) else steps
     assert identical_until >= 50, f"rasters differ from step {identical_until}"
     n_e = (n * 4) // 5
-    for name, sl in (("excitatory", slice(0, n_e)), ("inhibitory", slice(n_e, n))):
-        rate_got, rate_want = got[:, sl].sum() / (sl.stop - sl.start), want[:, sl].sum() / (sl.stop - sl.start)
-        assert rate_want > 1.0, f"{name} neurons are silent in the oracle"
-        assert abs(rate_got - rate_want) <= RATE_TOL * rate_want, f"{name}: {rate_got:.3f} Hz vs {rate_want:.3f} Hz"
+    assert n_e % 32 == 0
+    report = []
+    for name, first, last, count in (("excitatory", 0, n_e // 32, n_e), ("inhibitory", n_e // 32, words, n - n_e)):
+        per_step_got, per_step_want = _spikes_per_step(got, steps, words, first, last), _spikes_per_step(want, steps, words, first, last)
+        for label, upto, tol in (("first second", second, 0.08), ("four seconds", steps, RATE_TOL)):
+            rate_got, rate_want = per_step_got[:upto].sum() / count / (upto / 1000.0), per_step_want[:upto].sum() / count / (upto / 1000.0)
+            report.append(f"{name} {label}: {rate_got:.3f} / {rate_want:.3f} Hz")
+            assert rate_want > 1.0, f"{name} neurons are silent in the oracle"
+            assert abs(rate_got - rate_want) <= tol * rate_want, f"{name}, {label}: {rate_got:.3f} Hz vs {rate_want:.3f} Hz"
     assert abs(model.synaptic_event_count - oracle.events()) <= EVENT_TOL * oracle.events()
-    print(f"config 3: rasters identical for the first {identical_until} of {steps} steps; "
-          f"{got.sum() / n:.3f} Hz vs {want.sum() / n:.3f} Hz")
+    print(f"config 3: rasters identical for the first {identical_until} of {steps} steps; " + "; ".join(report), flush=True)
     model.unload()
 
 
