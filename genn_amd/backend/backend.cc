@@ -1699,6 +1699,18 @@ std::unique_ptr<GeNN::Runtime::StateBase> Backend::createState(const Runtime::Ru
 {
     return std::make_unique<State>();
 }
+void Backend::genPushProfilerRange(CodeStream &os, const std::string &name) const
+{
+    if(getPreferences<Preferences>().profilerRanges) {
+        os << "gennmi_profiler_range_push(\"" << name << "\");" << std::endl;
+    }
+}
+void Backend::genPopProfilerRange(CodeStream &os) const
+{
+    if(getPreferences<Preferences>().profilerRanges) {
+        os << "gennmi_profiler_range_pop();" << std::endl;
+    }
+}
 std::unique_ptr<Runtime::ArrayBase> Backend::createArray(const Type::ResolvedType &type, size_t count,
                                                          VarLocation location, bool uninitialized) const
 {

@@ -53,9 +53,15 @@ struct Preferences : public PreferencesBase
     //! built by FixedProbability, FixedProbabilityNoAutapse, FixedNumberPostWithReplacement or OneToOne and per-synapse
     //! variables initialised by Constant, Uniform, Normal, NormalClipped, Exponential or Gamma are generated on the device
     //! instead (gennmi_init_sparse_*, gennmi_init_var: counter-based Philox draws from the model's seed, one stream per
-    //! array) and copied back into the host mirrors: same distributions, other numbers -- as between the reference's own
-    //! CPU and GPU backends.  Everything else is initialised on the host as before.
+    //! array): same distributions, other numbers -- as between the reference's own CPU and GPU backends.  So are the
+    //! remaining built-in connectivity snippets (FixedNumberPreWithReplacement, Conv2D with kernel-initialised weights) and
+    //! the variables of DENSE and kernel matrices.  Everything else is initialised on the host as before.
     bool deviceInitialisation = false;
+
+    //! Named ranges around stepTime, updateSynapses and updateNeurons for profilers (the CUDA backend's enableNVTX,
+    //! cuda/backend.h:77-78): roctx ranges through gennmi_profiler_range_push / _pop.  With a step queue the ranges bracket
+    //! the noting of a step, the launches happen where the queue is flushed.
+    bool profilerRanges = false;
 
     void updateHash(boost::uuids::detail::sha1 &hash) const
     {
@@ -65,6 +71,7 @@ struct Preferences : public PreferencesBase
         Utils::updateHash(orderedAccumulation, hash);
         Utils::updateHash(stepQueueLength, hash);
         Utils::updateHash(deviceInitialisation, hash);
+        Utils::updateHash(profilerRanges, hash);
     }
 };
 
@@ -110,6 +117,9 @@ public:
     virtual void genDefinitionsPreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const final;
     virtual void genRunnerPreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const final;
     virtual void genAllocateMemPreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const final;
+    //! backendBase.h:345-349, cuda/backend.cc:741-752
+    virtual void genPushProfilerRange(CodeStream &os, const std::string &name) const final;
+    virtual void genPopProfilerRange(CodeStream &os) const final;
     virtual void genFreeMemPreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const final;
     virtual void genStepTimeFinalisePreamble(CodeStream &os, const ModelSpecMerged &modelMerged) const final;
 

@@ -44,7 +44,8 @@ PYBIND11_MODULE(mi355x_backend, m)
         .def_readwrite("kernel_source", &Preferences::kernelSource)
         .def_readwrite("ordered_accumulation", &Preferences::orderedAccumulation)
         .def_readwrite("step_queue_length", &Preferences::stepQueueLength)
-        .def_readwrite("device_initialisation", &Preferences::deviceInitialisation);
+        .def_readwrite("device_initialisation", &Preferences::deviceInitialisation)
+        .def_readwrite("profiler_ranges", &Preferences::profilerRanges);
 
     pybind11::class_<State, Runtime::StateBase>(m, "_Runtime")
         .def_property_readonly("device_name", &State::getDeviceName)

@@ -22,6 +22,7 @@
 // Arithmetic contract: fp32, one rounding per operation, same operation order as the code the
 // reference's SingleThreadedCPU backend generates (build with -ffp-contract=off).  The only
 // permitted divergence is the order of fp32 atomic adds into outPost / denDelay.
+#include <dlfcn.h>
 #include <sys/mman.h>
 #include <hip/hip_runtime.h>
 
@@ -407,6 +408,39 @@ int gennmi_push_mirrors(void)
             if(whole && madvise(reinterpret_cast<void*>(m.first), whole, MADV_DONTNEED) != 0) { return fail(GENNMI_EINVAL, "push_mirrors: madvise failed"); }
         }
     }
+    return GENNMI_OK;
+}
+extern "C++" {
+namespace
+{
+// roctx, if the process can load it (profilers bring it; nothing links against it)
+struct Roctx { int (*push)(const char*) = nullptr; int (*pop)() = nullptr; };
+const Roctx &roctx()
+{
+    static const Roctx r = [] {
+        Roctx x;
+        for(const char *name : {"libroctx64.so.4", "libroctx64.so", "librocprofiler-sdk-roctx.so.1"}) {
+            if(void *lib = dlopen(name, RTLD_NOW | RTLD_GLOBAL)) {
+                x.push = reinterpret_cast<int(*)(const char*)>(dlsym(lib, "roctxRangePushA"));
+                x.pop = reinterpret_cast<int(*)()>(dlsym(lib, "roctxRangePop"));
+                if(x.push && x.pop) { break; }
+                x = Roctx{};
+            }
+        }
+        return x;
+    }();
+    return r;
+}
+}
+}   // extern "C++"
+int gennmi_profiler_range_push(const char *name)
+{
+    if(name && roctx().push) { roctx().push(name); }
+    return GENNMI_OK;
+}
+int gennmi_profiler_range_pop(void)
+{
+    if(roctx().pop) { roctx().pop(); }
     return GENNMI_OK;
 }
 int gennmi_free_device_memory_bytes(size_t *bytes)

@@ -129,7 +129,13 @@ int gennmi_register_device_array(const void *host, void *dev, size_t bytes);
 int gennmi_mirrors_begin_initialisation(void);
 int gennmi_mirror_device_initialised(const void *host);
 int gennmi_mirror_ensure_host(const void *host);
-int gennmi_free_device_memory_bytes(size_t *bytes);             /* genReturnFreeDeviceMemoryBytes, backendCUDAHIP.cc */
+int gennmi_free_device_memory_bytes(size_t *bytes);
+/* Named ranges for profilers around stepTime / updateSynapses / updateNeurons (BackendBase::genPushProfilerRange /
+ * genPopProfilerRange, backendBase.h:345-349; nvtxRangePushA / nvtxRangePop in cuda/backend.cc:741-752): roctxRangePushA /
+ * roctxRangePop of libroctx64, looked up when first called; without that library the calls do nothing.  Both return
+ * GENNMI_OK. */
+int gennmi_profiler_range_push(const char *name);
+int gennmi_profiler_range_pop(void);             /* genReturnFreeDeviceMemoryBytes, backendCUDAHIP.cc */
 /* sizeof() of the five descriptor structs below, in declaration order (psm, cs, neuron update, presynaptic
  * update, postsynaptic update), so that a binding in another language can verify its struct layout.  Needs
  * no device.  The reference gets the same guarantee from generating both sides of every push call from one

@@ -458,3 +458,28 @@ def test_device_initialisation_is_generated_on_request():
                 assert "idKernel0" in init and "idKernel3" in init
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_profiler_ranges_are_generated_on_request():
+    """Preferences::profilerRanges (the CUDA backend's enableNVTX, cuda/backend.cc:741-752): stepTime, updateSynapses and
+    updateNeurons are bracketed by gennmi_profiler_range_push / _pop in the generated runner (generateRunner.cc:275-297), and
+    not otherwise."""
+    from cases import CASES
+    net, snap = CASES["va_small"]()
+    net.snap = snap
+    tmp = tempfile.mkdtemp(prefix="adapter_ranges_")
+    try:
+        spec = os.path.join(tmp, "spec")
+        write_netspec(net, spec)
+        for flag in (True, False):
+            work, out = os.path.join(tmp, f"work{int(flag)}"), os.path.join(tmp, f"out{int(flag)}")
+            os.makedirs(work); os.makedirs(out)
+            res = subprocess.run([DRIVER, spec, work, out, "--generate-only"] + (["--profiler-ranges"] if flag else []),
+                                 stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+            assert res.returncode == 0, res.stdout[-3000:]
+            runner = open(os.path.join(work, net.name + "_CODE", "runner.cc")).read()
+            for name in ("stepTime", "updateSynapses", "updateNeurons"):
+                assert (f'gennmi_profiler_range_push("{name}");' in runner) == flag
+            assert runner.count("gennmi_profiler_range_pop();") == (3 if flag else 0)
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)

@@ -43,7 +43,7 @@ def test_pygenn_module_exposes_every_preference_and_the_backend_state():
     header = open(os.path.join(BACKEND_DIR, "backend.h")).read()
     struct = header[header.index("struct Preferences"):header.index("void updateHash")]
     members = re.findall(r"^\s+(?:int|bool|unsigned int|std::string|KernelSource)\s+(\w+)\s*(?:=[^;]*)?;", struct, flags=re.M)
-    assert set(members) == {"deviceID", "installRoot", "kernelSource", "orderedAccumulation", "stepQueueLength", "deviceInitialisation"}, members
+    assert set(members) == {"deviceID", "installRoot", "kernelSource", "orderedAccumulation", "stepQueueLength", "deviceInitialisation", "profilerRanges"}, members
     module = open(os.path.join(BACKEND_DIR, "pygenn_module.cc")).read()
     for member in members:
         snake = re.sub(r"(?<=[a-z])([A-Z])", lambda m: "_" + m.group(1).lower(), member).replace("_i_d", "_id").lower()

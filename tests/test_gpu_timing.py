@@ -135,3 +135,14 @@ def test_counters_of_generated_kernels_through_the_reference_runtime():
             assert np.array_equal(got, golden[f"spikes.{p.name}"])
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_profiler_ranges_nest_and_cost_nothing_without_a_profiler():
+    """gennmi_profiler_range_push / _pop (roctx ranges when libroctx64 can be loaded, nothing otherwise): always GENNMI_OK,
+    nesting as generateRunner.cc:275-297 nests them."""
+    from genn_amd import _abi
+    lib = _abi.load()
+    for name in (b"stepTime", b"updateSynapses"):
+        assert lib.gennmi_profiler_range_push(name) == 0
+    assert lib.gennmi_profiler_range_pop() == 0 and lib.gennmi_profiler_range_pop() == 0
+    assert lib.gennmi_profiler_range_push(None) == 0
