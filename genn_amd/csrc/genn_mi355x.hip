@@ -2201,7 +2201,6 @@ int gennmi_build_remap(uint32_t numSrc, uint32_t numTrg, uint32_t rowStride, uin
 {
     if(!rowLength || !ind || !colLength || !remap || rowStride == 0 || colStride == 0) { return fail(GENNMI_EINVAL, "build_remap: bad arguments"); }
     FLUSH_QUEUED();
-    if(colStride > REMAP_SORT_MAX) { return fail(GENNMI_EUNSUPPORTED, "build_remap: column stride above 16384 is not supported"); }
     uint32_t *dOverflow = nullptr;
     HIP_TRY(hipMalloc(&dOverflow, sizeof(uint32_t)));
     HIP_TRY(hipMemset(dOverflow, 0, sizeof(uint32_t)));
@@ -2213,11 +2212,13 @@ int gennmi_build_remap(uint32_t numSrc, uint32_t numTrg, uint32_t rowStride, uin
     HIP_TRY(hipMemcpy(&overflow, dOverflow, sizeof(uint32_t), hipMemcpyDeviceToHost));
     HIP_TRY(hipFree(dOverflow));
     if(overflow) { return fail(GENNMI_EINVAL, "build_remap: a column holds " + std::to_string(overflow) + " synapses, more than colStride"); }
-    const size_t lds = (size_t)pow2Ceil(colStride) * sizeof(uint32_t);
+    const size_t lds = (size_t)pow2Ceil(std::min(colStride, REMAP_SORT_MAX)) * sizeof(uint32_t);
     if(lds > 48 * 1024) {
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(remapSortKernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     }
     remapSortKernel<<<dim3(numTrg), dim3(BLOCK), lds, 0>>>(colStride, colLength, remap);
+    // columns beyond what the LDS holds, in place in global memory
+    if(colStride > REMAP_SORT_MAX) { remapSortLongKernel<<<dim3(numTrg), dim3(BLOCK), 0, 0>>>(colStride, colLength, remap); }
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipDeviceSynchronize());
     return GENNMI_OK;

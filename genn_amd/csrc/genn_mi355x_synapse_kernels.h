@@ -1144,7 +1144,7 @@ void remapSortKernel(uint32_t colStride, const uint32_t *colLength, uint32_t *re
     extern __shared__ uint32_t shCol[];
     const uint32_t col = blockIdx.x;
     const uint32_t len = min(colLength[col], colStride);
-    if(len < 2) { return; }
+    if(len < 2 || len > REMAP_SORT_MAX) { return; }         // (longer columns: remapSortLongKernel)
     uint32_t p2 = 1;
     while(p2 < len) { p2 <<= 1; }
     uint32_t *column = remap + (size_t)col * colStride;
@@ -1164,6 +1164,37 @@ void remapSortKernel(uint32_t colStride, const uint32_t *colLength, uint32_t *re
         }
     }
     for(uint32_t k = threadIdx.x; k < len; k += BLOCK) { column[k] = shCol[k]; }
+}
+
+// Columns too long for the LDS: the same kind of network in place, in global memory (a column of 10^5 entries stays in the
+// L2), one work-group per column.  Every comparator of this form of the bitonic network puts the smaller entry at the
+// lower index (a merge's first step pairs k with its mirror image in the block, k ^ (size - 1), the following ones k with
+// k ^ stride), so positions beyond the column's length behave like entries of infinite value without being stored:
+// a comparator that reaches beyond the length never exchanges.  (The reference's remap build has no limit on the column
+// length, backendSIMT.cc:1977-1991.)
+__global__ __launch_bounds__(BLOCK)
+void remapSortLongKernel(uint32_t colStride, const uint32_t *colLength, uint32_t *remap)
+{
+    const uint32_t col = blockIdx.x;
+    const uint32_t len = min(colLength[col], colStride);
+    if(len <= REMAP_SORT_MAX) { return; }
+    uint32_t p2 = 1;
+    while(p2 < len) { p2 <<= 1; }
+    uint32_t *column = remap + (size_t)col * colStride;
+    for(uint32_t size = 2; size <= p2; size <<= 1) {
+        for(uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+            const uint32_t mask = (stride == (size >> 1)) ? size - 1u : stride;
+            for(uint32_t k = threadIdx.x; k < len; k += BLOCK) {
+                const uint32_t partner = k ^ mask;
+                if(partner > k && partner < len) {
+                    const uint32_t a = column[k], b = column[partner];
+                    if(a > b) { column[k] = b; column[partner] = a; }
+                }
+            }
+            __threadfence_block();
+            __syncthreads();
+        }
+    }
 }
 
 uint32_t pow2Floor(uint32_t v) { uint32_t p = 1; while(p * 2 <= v) { p *= 2; } return p; }

@@ -259,3 +259,53 @@ def test_spike_source_arrays_rewritten_between_steps(replay):
     assert np.array_equal(got, expected(0) | expected(30))
     assert got.sum() == 2 * per.sum() and per.sum() > 300
     model.unload()
+
+
+def test_column_view_of_columns_longer_than_the_lds_sort():
+    """gennmi_build_remap with columns beyond 16,384 entries (the reference's remap build has no limit on the column length,
+    backendSIMT.cc:1977-1991): two long columns (40,000 and 20,001 entries) among short and empty ones; every column of the
+    view must list its synapses in ascending idSyn — the order of the CPU backend's row-major build
+    (single_threaded_cpu/backend.cc:156-179) — and the lengths must be the counts."""
+    import ctypes as C
+    from genn_amd import _abi
+    from genn_amd.genn_model import Array
+    lib = _abi.load()
+    _abi.check(lib.gennmi_init(0))
+    num_src, num_trg, row_stride = 40000, 7, 4
+    rng = np.random.default_rng(5)
+    ind = np.zeros((num_src, row_stride), np.uint32)
+    row_length = np.zeros(num_src, np.uint32)
+    for i in range(num_src):
+        targets = [0]                                   # every row reaches column 0
+        if i % 2 == 0 or i == 1:
+            targets.append(3)                           # 20,001 rows reach column 3
+        if i % 97 == 0:
+            targets.append(5)
+        if i == 12345:
+            targets.append(6)
+        targets.sort()
+        row_length[i] = len(targets)
+        ind[i, :len(targets)] = targets
+        ind[i, len(targets):] = rng.integers(0, num_trg, row_stride - len(targets))       # padding: never read
+    want = [[] for _ in range(num_trg)]
+    for i in range(num_src):
+        for j in range(row_length[i]):
+            want[ind[i, j]].append(i * row_stride + j)
+    col_stride = max(len(c) for c in want)
+    assert col_stride == 40000 and len(want[3]) == 20001 and not want[1]
+    arrays = {}
+    for name, host in (("rowLength", row_length), ("ind", ind.reshape(-1))):
+        a = Array(host.size, np.uint32)
+        a.view[:] = host
+        a.push_to_device()
+        arrays[name] = a
+    col_length = Array(num_trg, np.uint32, device_only=True)
+    remap = Array(num_trg * col_stride, np.uint32, device_only=True)
+    _abi.check(lib.gennmi_build_remap(num_src, num_trg, row_stride, col_stride, arrays["rowLength"].ptr, arrays["ind"].ptr, col_length.ptr, remap.ptr))
+    got_length = col_length.pull_from_device().copy()
+    got = remap.pull_from_device().reshape(num_trg, col_stride).copy()
+    for a in (*arrays.values(), col_length, remap):
+        a.free()
+    assert np.array_equal(got_length, [len(c) for c in want])
+    for j in range(num_trg):
+        assert np.array_equal(got[j, :len(want[j])], np.asarray(want[j], dtype=np.uint32)), f"column {j}"
