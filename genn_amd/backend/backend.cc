@@ -978,7 +978,8 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
     const uint64_t numProjections = model.getSynapseGroups().size();
     // Generator streams are numbered in ranges per consumer under one key (the model's seed): initialisation arrays from 1
     // (2k + 1, 2k + 2 + 2 P v), current sources from 1000, neuron code from 2000, weight-update code from 3000 (eight per
-    // projection), custom connectivity updates from 6000.  A model large enough for two ranges to meet would draw the same
+    // projection), custom connectivity updates from 6000, neuron variable initialisation from 8000 (sixteen per population).
+    // A model large enough for two ranges to meet would draw the same
     // words in two places, so it is refused here rather than simulated with correlated noise.
     {
         size_t maxVars = 0;
@@ -1076,7 +1077,48 @@ void Backend::genInit(CodeStream &os, FileStreamCreator, ModelSpecMerged &modelM
                 {
                     EnvironmentGroupMergedField<NeuronInitGroupMerged> env(funcEnv, n);
                     buildStandardEnvironment(env, batchSize);
+                    // neuron variables whose initialiser is a value snippet the device draws (Preferences::deviceInitialisation):
+                    // one gennmi_init_var each; genVariableInit then leaves their host loops out of the generic code below.
+                    // Streams 8000 + 16 * (the population's place by name) + the variable's place in the model.
+                    m_DeviceInitialisedVars.clear();
+                    if(deviceInit && batchSize == 1) {
+                        const auto &arch = n.getArchetype();
+                        const auto vars = arch.getModel()->getVars();
+                        for(size_t v = 0; v < vars.size() && v < 16; v++) {
+                            const auto &var = vars[v];
+                            const auto &init = arch.getVarInitialisers().at(var.name);
+                            unsigned int snippet = 0;
+                            std::vector<std::string> paramNames;
+                            bool eligible = !Utils::areTokensEmpty(init.getCodeTokens()) && var.type.resolve(model.getTypeContext()) == Type::Float
+                                            && (getVarAccessDim(var.access) & VarAccessDim::ELEMENT) && !arch.isVarQueueRequired(var.name)
+                                            && deviceVarSnippet(init.getSnippet(), snippet, paramNames);
+                            for(const auto &g : n.getGroups()) {
+                                eligible = eligible && (g.get().getVarInitialisers().at(var.name).getSnippet() == init.getSnippet()) && !g.get().isVarQueueRequired(var.name);
+                            }
+                            if(!eligible) { continue; }
+                            const std::string name = var.name;
+                            env.addField(Type::Float.createPointer(), "_mi_init_" + name, name,
+                                         [name](const auto &runtime, const auto &g, size_t) { return runtime.getArray(g, name); });
+                            std::vector<uint64_t> streams;
+                            for(const auto &g : n.getGroups()) {
+                                streams.push_back(8000 + 16 * (uint64_t)std::distance(model.getNeuronGroups().cbegin(), model.getNeuronGroups().find(g.get().getName())) + v);
+                            }
+                            CodeStream::Scope scope(env.getStream());
+                            env.getStream() << "static const uint32_t stream[] = " << tableU32(streams) << ";" << std::endl;
+                            env.getStream() << "double params[4] = {0.0, 0.0, 0.0, 0.0};" << std::endl;
+                            for(size_t k = 0; k < paramNames.size(); k++) {
+                                std::vector<Type::NumericValue> values;
+                                for(const auto &g : n.getGroups()) { values.push_back(g.get().getVarInitialisers().at(name).getParams().at(paramNames[k])); }
+                                env.getStream() << "{ static const double v[] = " << table(values, Type::Double) << "; params[" << k << "] = v[g]; }" << std::endl;
+                            }
+                            env.getStream() << "GENNMI_CHECK(gennmi_init_var(gennmiDev(" << env["_mi_init_" + name] << "), " << GENNMI_TYPE_F32 << "u, (size_t)" << env["num_neurons"]
+                                            << ", " << snippet << "u, params, " << seedExpr << ", stream[g]));" << std::endl;
+                            env.getStream() << "GENNMI_CHECK(gennmi_mirror_device_initialised(" << env["_mi_init_" + name] << "));" << std::endl;
+                            m_DeviceInitialisedVars.insert(name);
+                        }
+                    }
                     n.generateInit(*this, env, batchSize);
+                    m_DeviceInitialisedVars.clear();
                 });
             });
         modelMerged.genMergedSynapseInitGroups(
@@ -1422,6 +1464,13 @@ void Backend::genPopVariableInit(EnvironmentExternalBase &env, HandlerEnv handle
 }
 void Backend::genVariableInit(EnvironmentExternalBase &env, const std::string &count, const std::string &indexVarName, HandlerEnv handler) const
 {
+    // a neuron variable the device has just drawn (genInit): its host loop is left out
+    if(!m_DeviceInitialisedVars.empty()) {
+        std::string target;
+        try { target = env["_value"]; } catch(const std::exception&) {}     // (loops that initialise no variable have no such name)
+        const size_t arrow = target.rfind("->");
+        if(arrow != std::string::npos && m_DeviceInitialisedVars.count(target.substr(arrow + 2))) { return; }
+    }
     env.getStream() << "for(unsigned int k = 0; k < (" << env[count] << "); k++)";
     CodeStream::Scope b(env.getStream());
     EnvironmentExternal varEnv(env);

@@ -12,6 +12,7 @@
 //    (gennmi_*_update_group_t); anything else is rejected at code-generation time with std::runtime_error.
 #include <memory>
 #include <map>
+#include <set>
 #include <string>
 
 #include "backendExport.h"
@@ -55,7 +56,8 @@ struct Preferences : public PreferencesBase
     //! instead (gennmi_init_sparse_*, gennmi_init_var: counter-based Philox draws from the model's seed, one stream per
     //! array): same distributions, other numbers -- as between the reference's own CPU and GPU backends.  So are the
     //! remaining built-in connectivity snippets (FixedNumberPreWithReplacement, Conv2D with kernel-initialised weights) and
-    //! the variables of DENSE and kernel matrices.  Everything else is initialised on the host as before.
+    //! the variables of DENSE and kernel matrices, and unbatched, undelayed float variables of neuron populations.
+    //! Everything else is initialised on the host as before.
     bool deviceInitialisation = false;
 
     //! Named ranges around stepTime, updateSynapses and updateNeurons for profilers (the CUDA backend's enableNVTX,
@@ -194,5 +196,7 @@ private:
     const bool m_GeneratedKernels;
     const bool m_CustomUpdateKernels;
     mutable std::map<std::string, int> m_TimerIds;
+    //! neuron variables of the merged init group being printed that a device generator fills (their host loops are left out)
+    mutable std::set<std::string> m_DeviceInitialisedVars;
 };
 }   // namespace GeNN::CodeGenerator::MI355X

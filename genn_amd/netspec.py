@@ -185,6 +185,8 @@ def write_netspec(net: Net, path: str):
     for p in net.pops:
         if p.model == "lif":
             ps = " ".join(repr(float(p.params[k])) for k in LIF_PARAMS)
+        elif p.model == "lif_init":   # LIF whose V is drawn by an initialisation snippet (Uniform[Vmin, Vmax)), RefracTime constant 0
+            ps = " ".join(repr(float(p.params[k])) for k in LIF_PARAMS + ("Vmin", "Vmax"))
         elif p.model == "lifa":       # LIF with an adaptation variable: a model of the test driver, not a built-in one
             ps = " ".join(repr(float(p.params[k])) for k in LIF_PARAMS + ("TauA", "dA"))
         elif p.model == "izh":

@@ -530,6 +530,13 @@ int main(int argc, char *argv[])
                      {"Vthresh", p.p.at(4)}, {"Ioffset", p.p.at(5)}, {"TauRefrac", p.p.at(6)}},
                     {{"V", uninitialisedVar()}, {"RefracTime", uninitialisedVar()}});
             }
+            else if(p.model == "lif_init") {
+                // the membrane potential by an initialisation snippet instead of a file
+                p.ng = model.addNeuronPopulation<NeuronModels::LIF>(p.name, p.n,
+                    {{"C", p.p.at(0)}, {"TauM", p.p.at(1)}, {"Vrest", p.p.at(2)}, {"Vreset", p.p.at(3)},
+                     {"Vthresh", p.p.at(4)}, {"Ioffset", p.p.at(5)}, {"TauRefrac", p.p.at(6)}},
+                    {{"V", initVar<InitVarSnippet::Uniform>({{"min", p.p.at(7)}, {"max", p.p.at(8)}})}, {"RefracTime", 0.0}});
+            }
             else if(p.model == "lifa") {
                 p.ng = model.addNeuronPopulation<LIFAdapt>(p.name, p.n,
                     {{"C", p.p.at(0)}, {"TauM", p.p.at(1)}, {"Vrest", p.p.at(2)}, {"Vreset", p.p.at(3)},
@@ -833,6 +840,11 @@ int main(int argc, char *argv[])
             }
         }
         rt.initializeSparse();
+        for(auto &p : pops) {
+            if(p.model != "lif_init") { continue; }
+            auto *v = rt.getArray(*p.ng, "V"); v->pullFromDevice();
+            appendScalars(out + "/" + p.name + ".V0.f32", v, 0, (size_t)p.n * batch);
+        }
         // (how long a model takes from loading its code to its first step: allocation, initialize(), initializeSparse())
         {
             // (VmHWM of this process image: getrusage's ru_maxrss also carries the peak of the process that started this one)
@@ -889,9 +901,9 @@ int main(int argc, char *argv[])
             for(auto &p : pops) {
                 if(p.model == "ssa" || p.model == "poisson") continue;
                 pulled(rt.getArray(*p.ng, "V"));
-                pulled(rt.getArray(*p.ng, (p.model == "lif" || p.model == "lifa") ? "RefracTime" : "U"));
+                pulled(rt.getArray(*p.ng, (p.model == "lif" || p.model == "lifa" || p.model == "lif_init") ? "RefracTime" : "U"));
                 appendScalars(out + "/" + p.name + ".V.f32", rt.getArray(*p.ng, "V"), 0, (size_t)p.n * batch);
-                if(p.model == "lif" || p.model == "lifa") appendScalars(out + "/" + p.name + ".RefracTime.f32", rt.getArray(*p.ng, "RefracTime"), 0, (size_t)p.n * batch);
+                if(p.model == "lif" || p.model == "lifa" || p.model == "lif_init") appendScalars(out + "/" + p.name + ".RefracTime.f32", rt.getArray(*p.ng, "RefracTime"), 0, (size_t)p.n * batch);
                 if(p.model == "lifa") { auto *a = pulled(rt.getArray(*p.ng, "A")); appendScalars(out + "/" + p.name + ".A.f32", a, 0, (size_t)p.n * batch); }
                 if(p.model == "izh") appendScalars(out + "/" + p.name + ".U.f32", rt.getArray(*p.ng, "U"), 0, (size_t)p.n * batch);
             }

@@ -859,11 +859,13 @@ def _procedural_pair(net, steps, snap):
     return out, tmp, model, state
 
 
-def test_adapter_dense_and_kernel_variables_initialised_on_the_device():
-    """Preferences::deviceInitialisation for the variables of a stored DENSE matrix and of a TOEPLITZ projection's kernel
-    (initGroupMerged.cc:563-593): with the switch the dumped weights are exactly what gennmi_init_var draws for the model's
-    seed and the array's stream (2k + 2 for the k-th projection by name); without it the reference's host loops draw other
-    values of the same distribution (Uniform and Normal, Kolmogorov-Smirnov).  Both runs step the model afterwards."""
+def test_adapter_dense_kernel_and_neuron_variables_initialised_on_the_device():
+    """Preferences::deviceInitialisation for the variables of a stored DENSE matrix, of a TOEPLITZ projection's kernel
+    (initGroupMerged.cc:563-593) and of a neuron population (:126-196): with the switch the dumped values are exactly what
+    gennmi_init_var draws for the model's seed and the array's stream (2k + 2 for the k-th projection by name, 8000 + 16 p + v
+    for variable v of the p-th population by name), and the host loops of those variables are not generated; without it the
+    reference's host loops draw other values of the same distribution (Uniform and Normal, Kolmogorov-Smirnov).  Both runs step
+    the model afterwards."""
     import ctypes as C
     from scipy import stats
     from genn_amd import _abi, configs, rng
@@ -874,8 +876,8 @@ def test_adapter_dense_and_kernel_variables_initialised_on_the_device():
     start, end, times = configs.poisson_spike_source(seed, 1, 8 * 8 * 2, 60.0, steps, 1.0)
     net.pops.append(Pop("In", "ssa", 8 * 8 * 2, {}, {"startSpike": start, "endSpike": end}, spike_times=times))
     lif = dict(C=1.0, TauM=20.0, Vrest=-60.0, Vreset=-60.0, Vthresh=-50.0, Ioffset=0.4, TauRefrac=2.0)
-    for name, n, stream in (("Mid", 8 * 8 * 4, 2), ("Out", 700, 3)):
-        net.pops.append(Pop(name, "lif", n, dict(lif), {"V": (-60.0 + 9.0 * rng.uniform(seed, stream, 0, n)).astype(np.float32), "RefracTime": np.zeros(n, np.float32)}))
+    net.pops.append(Pop("Mid", "lif", 8 * 8 * 4, dict(lif), {"V": (-60.0 + 9.0 * rng.uniform(seed, 2, 0, 8 * 8 * 4)).astype(np.float32), "RefracTime": np.zeros(8 * 8 * 4, np.float32)}))
+    net.pops.append(Pop("Out", "lif_init", 700, dict(lif, Vmin=-60.0, Vmax=-51.0), {}))
     net.syns.append(Syn("InMid", "In", "Mid", matrix="conv2d", wum="static", psm="expcurr", tau=5.0, g_init=("Normal", {"mean": 0.1, "sd": 0.05}),
                         conv=dict(conv_kh=3, conv_kw=3, conv_ih=8, conv_iw=8, conv_ic=2, conv_oh=8, conv_ow=8, conv_oc=4)))
     net.syns.append(Syn("MidOut", "Mid", "Out", matrix="dense_init", wum="static", psm="expcurr", tau=5.0, g_init=("Uniform", {"min": -0.01, "max": 0.03})))
@@ -892,25 +894,27 @@ def test_adapter_dense_and_kernel_variables_initialised_on_the_device():
             res = subprocess.run([DRIVER, spec, work, out] + (["--device-init"] if flag else []), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
             assert res.returncode == 0, res.stdout[-3000:]
             init = open(os.path.join(work, net.name + "_CODE", "init.cc")).read()
-            assert init.count("gennmi_init_var(") == (2 if flag else 0)
+            assert init.count("gennmi_init_var(") == (4 if flag else 0)          # two matrices, V and RefracTime (a constant is a snippet too)
             weights[flag] = {s.name: np.fromfile(os.path.join(out, f"{s.name}.g.f32"), np.float32) for s in net.syns}
+            weights[flag]["Out.V"] = np.fromfile(os.path.join(out, "Out.V0.f32"), np.float32)
             assert sum(len(np.fromfile(os.path.join(out, f"{p.name}.spikes.u32"), np.uint32)) // 2 for p in net.pops[1:]) > 100
         lib = _abi.load()
         _abi.check(lib.gennmi_init(0))
-        for k, (s, count, snippet, params, law) in enumerate((
-                (net.syns[0], 3 * 3 * 2 * 4, "Normal", (0.1, 0.05), stats.norm(0.1, 0.05)),
-                (net.syns[1], 256 * 700, "Uniform", (-0.01, 0.03), stats.uniform(-0.01, 0.04)))):
-            assert sorted(x.name for x in net.syns).index(s.name) == k
+        place = sorted(p.name for p in net.pops).index("Out")
+        for name, stream, count, snippet, params, law in (
+                ("InMid", 2, 3 * 3 * 2 * 4, "Normal", (0.1, 0.05), stats.norm(0.1, 0.05)),
+                ("MidOut", 4, 256 * 700, "Uniform", (-0.01, 0.03), stats.uniform(-0.01, 0.04)),
+                ("Out.V", 8000 + 16 * place, 700, "Uniform", (-60.0, -51.0), stats.uniform(-60.0, 9.0))):
             a = Array(count, np.float32, device_only=True)
             p = (C.c_double * 4)(*(list(params) + [0.0, 0.0]))
-            _abi.check(lib.gennmi_init_var(a.ptr, _abi.ELEMENT_TYPES["float32"], count, _abi.INIT_SNIPPETS[snippet], C.byref(p), seed, 2 * k + 2))
+            _abi.check(lib.gennmi_init_var(a.ptr, _abi.ELEMENT_TYPES["float32"], count, _abi.INIT_SNIPPETS[snippet], C.byref(p), seed, stream))
             want = a.pull_from_device().copy()
             a.free()
-            assert weights[True][s.name].shape == want.shape
-            assert np.array_equal(weights[True][s.name], want), f"{s.name}: weights are not the device generator's"
-            assert not np.array_equal(weights[False][s.name], want)
-            for values in (weights[True][s.name], weights[False][s.name]):
-                assert stats.kstest(values.astype(np.float64), law.cdf).pvalue > 0.00034, s.name
+            assert weights[True][name].shape == want.shape
+            assert np.array_equal(weights[True][name], want), f"{name}: values are not the device generator's"
+            assert not np.array_equal(weights[False][name], want)
+            for values in (weights[True][name], weights[False][name]):
+                assert stats.kstest(values.astype(np.float64), law.cdf).pvalue > 0.00034, name
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
 
