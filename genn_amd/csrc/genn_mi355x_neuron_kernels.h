@@ -46,13 +46,20 @@ __device__ __forceinline__ float poissonExpInject(const gennmi_cs_t &cs, GLOBAL_
 // Offset of a block's entries in its population's queue: the block publishes its count, then (wave 0) sums the counts of
 // the earlier blocks of its group of 64 and the published totals of the earlier groups.  Every thread of the block calls
 // this between two barriers of its own; returns 0xFFFFFFFF after a bounded wait expired (error flag raised).
+// (`published`: the caller has stored the block's count itself, earlier — see publishBlockCount)
+__device__ __forceinline__ void publishBlockCount(uint32_t blockCount, uint32_t localBlock, size_t aggBase, unsigned long long *counts, uint32_t tag)
+{
+    if(threadIdx.x == 0) {
+        __hip_atomic_store(&counts[aggBase + localBlock], ((unsigned long long)tag << 32) | blockCount, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
 __device__ __forceinline__ uint32_t blockQueueOffset(uint32_t blockCount, uint32_t localBlock, uint32_t numBlocks, size_t aggBase,
                                                     unsigned long long *counts, unsigned long long *groupTotals, uint32_t tag,
-                                                    uint32_t *shOffset, uint32_t *errorFlag)
+                                                    uint32_t *shOffset, uint32_t *errorFlag, bool published = false)
 {
     const uint32_t lane = threadIdx.x & (WAVE - 1);
     const uint32_t wave = threadIdx.x / WAVE;
-    if(threadIdx.x == 0) {
+    if(threadIdx.x == 0 && !published) {
         __hip_atomic_store(&counts[aggBase + localBlock], ((unsigned long long)tag << 32) | blockCount, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     const bool last = (localBlock == numBlocks - 1);
@@ -546,19 +553,22 @@ __device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t
             }
         }
     }
-    // ---- update and store, chunk by chunk (operations and their order as in neuronBody)
+    // ---- update, chunk by chunk (operations and their order as in neuronBody); results stay in registers until the block's
+    // spike count is on its way: work-groups behind this one wait for that count, and a wavefront that has to queue
+    // behind the store traffic of the whole chip before it can vote would keep them waiting
+    float outLin[NPL][BULK_MAX_PSM];
+    uint32_t newStart[NPL];
     #pragma unroll
     for(int j = 0; j < NPL; j++) {
         const uint32_t i = first + j * WAVE;
         const size_t bi = (size_t)batch * n + i;
+        newStart[j] = 0;
+        #pragma unroll
+        for(uint32_t m = 0; m < BULK_MAX_PSM; m++) { outLin[j][m] = 0.0f; }
         if(i >= n) { continue; }
         if(source) {
             spiked[j] = (t >= l0[j]);
-            if(spiked[j]) {
-                const uint32_t startSpike = startSpikeArr[bi] + 1;
-                startSpikeArr[bi] = startSpike;
-                nextSpikeTime[bi] = (startSpike != endSpikeArr[bi]) ? spikeTimesArr[startSpike] : INFINITY;
-            }
+            if(spiked[j]) { newStart[j] = startSpikeArr[bi] + 1; }
             continue;
         }
         float Isyn = 0;
@@ -576,34 +586,22 @@ __device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t
                     Isyn += linSyn;
                     linSyn = 0.0f;
                 }
-                if(D) { psmRing[m][((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i] = 0.0f; }
-                psmOut[m][bi] = linSyn;
+                outLin[j][m] = linSyn;
             }
         }
         if(numCS) { Isyn += inj[j]; }
-        float v0 = l0[j], v1 = l1[j];
-        spiked[j] = plainNeuronStep(constants, Isyn, dt, v0, v1);
-        var0[bi] = v0; var1[bi] = v1;
-    }
-    if(localBlock == 0 && batch == 0 && threadIdx.x < g.numPSM) {
-        const gennmi_psm_t &psm = g.psm[threadIdx.x];
-        if(psm.maxDenDelay && psm.denDelayPtr) { *psm.denDelayPtr = modStep(st.epoch + 1, psm.maxDenDelay); }
+        spiked[j] = plainNeuronStep(constants, Isyn, dt, l0[j], l1[j]);
     }
 
     // ---- ordered compaction: rank = spikes of the wave's earlier chunks + spikes of lower lanes in this chunk
     uint32_t rank[NPL];
+    unsigned long long ballots[NPL];
     uint32_t waveCount = 0;
     #pragma unroll
     for(int j = 0; j < NPL; j++) {
-        const uint32_t i = first + j * WAVE;
-        const unsigned long long ballot = __ballot(spiked[j]);
-        rank[j] = waveCount + __popcll(ballot & ((1ull << lane) - 1ull));
-        waveCount += __popcll(ballot);
-        if(recordSpk && (lane & 31) == 0 && i < n) {
-            const uint32_t words = (n + 31) / 32;
-            recordSpk[((size_t)st.recT * numBatches + batch) * words + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
-        }
-        if(spikeBitmap && (lane & 31) == 0 && i < n) { spikeBitmap[((st.epoch + 1) & 1) * bitmapStride + (size_t)batch * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballot >> (lane & 32)); }
+        ballots[j] = __ballot(spiked[j]);
+        rank[j] = waveCount + __popcll(ballots[j] & ((1ull << lane) - 1ull));
+        waveCount += __popcll(ballots[j]);
     }
     if(lane == 0) { shWaveCount[wave] = waveCount; }
     __syncthreads();
@@ -615,8 +613,44 @@ __device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t
         blockCount += c;
     }
     unsigned long long *groupAgg = agg + (size_t)totalNeuronBlocks * numBatches;
-    const uint32_t prefix = blockQueueOffset(blockCount, localBlock, groupBlocks, (size_t)batch * totalNeuronBlocks + groupStart, agg, groupAgg,
-                                             (uint32_t)(st.epoch + 1), &shPrefix, errorFlag);
+    const size_t aggBase = (size_t)batch * totalNeuronBlocks + groupStart;
+    publishBlockCount(blockCount, localBlock, aggBase, agg, (uint32_t)(st.epoch + 1));
+
+    // ---- state, recording words and bitmap
+    #pragma unroll
+    for(int j = 0; j < NPL; j++) {
+        const uint32_t i = first + j * WAVE;
+        const size_t bi = (size_t)batch * n + i;
+        if(i >= n) { continue; }
+        if(recordSpk && (lane & 31) == 0) {
+            const uint32_t words = (n + 31) / 32;
+            recordSpk[((size_t)st.recT * numBatches + batch) * words + (i >> 5)] = (uint32_t)(ballots[j] >> (lane & 32));
+        }
+        if(spikeBitmap && (lane & 31) == 0) { spikeBitmap[((st.epoch + 1) & 1) * bitmapStride + (size_t)batch * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballots[j] >> (lane & 32)); }
+        if(source) {
+            if(spiked[j]) {
+                startSpikeArr[bi] = newStart[j];
+                nextSpikeTime[bi] = (newStart[j] != endSpikeArr[bi]) ? spikeTimesArr[newStart[j]] : INFINITY;
+            }
+            continue;
+        }
+        #pragma unroll
+        for(uint32_t m = 0; m < BULK_MAX_PSM; m++) {
+            if(m < numPSM) {
+                const uint32_t D = psmD[m];
+                if(D) { psmRing[m][((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i] = 0.0f; }
+                psmOut[m][bi] = outLin[j][m];
+            }
+        }
+        var0[bi] = l0[j]; var1[bi] = l1[j];
+    }
+    if(localBlock == 0 && batch == 0 && threadIdx.x < g.numPSM) {
+        const gennmi_psm_t &psm = g.psm[threadIdx.x];
+        if(psm.maxDenDelay && psm.denDelayPtr) { *psm.denDelayPtr = modStep(st.epoch + 1, psm.maxDenDelay); }
+    }
+
+    const uint32_t prefix = blockQueueOffset(blockCount, localBlock, groupBlocks, aggBase, agg, groupAgg,
+                                             (uint32_t)(st.epoch + 1), &shPrefix, errorFlag, true);
     if(prefix == 0xFFFFFFFFu) { return; }
     #pragma unroll
     for(int j = 0; j < NPL; j++) {
