@@ -163,11 +163,14 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
     float vEvent = 0.0f;
     uint32_t z0 = 0, z1 = 0;
     if(G.zeroStart && i < n) { z0 = asGlobal(G.zeroStart)[i]; z1 = asGlobal(G.zeroStart)[i + 1]; }
+    // what the update leaves to be stored (see storeState below)
+    float l0 = 0, l1 = 0, preTrace = 0, postTrace = 0;
+    float lin[GENNMI_MAX_PSM];
+    #pragma unroll
+    for(uint32_t m = 0; m < GENNMI_MAX_PSM; m++) { lin[m] = 0.0f; }
     if(i < n) {
         // order of operations: neuronUpdateGroupMerged.cc:552-773 — PSMs, current sources, sim code,
         // WU pre/post dynamics, threshold, then (on a spike) WU pre/post spike code, sT, reset
-        float l0 = 0, l1 = 0;
-        uint32_t startSpike = 0;
         float nextTime = 0.0f;
         if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
             // one coalesced read instead of startSpike, endSpike and a gather from spikeTimes: the time of the neuron's next
@@ -179,7 +182,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
             // descriptor in memory, so a store in between would force the compiler to re-read the descriptor
             // and would serialise the loads, and each dependent access costs about a microsecond at the start of
             // a launch (nothing is cached yet).  Sums keep the reference's order (PSMs, then current sources).
-            float lin[GENNMI_MAX_PSM], front[GENNMI_MAX_PSM], inj[GENNMI_MAX_CS], rev[GENNMI_MAX_PRE_OUTPUT];
+            float front[GENNMI_MAX_PSM], inj[GENNMI_MAX_CS], rev[GENNMI_MAX_PRE_OUTPUT];
             const uint32_t numPSM = g.numPSM, numCS = g.numCS, numRev = g.numPreOutput;
             #pragma unroll
             for(uint32_t q = 0; q < GENNMI_MAX_PRE_OUTPUT; q++) { rev[q] = (q < numRev) ? asGlobal(g.outPre[q])[bi] : 0.0f; }
@@ -226,16 +229,6 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
             for(uint32_t q = 0; q < GENNMI_MAX_PRE_OUTPUT; q++) { if(q < numRev) { Isyn += rev[q]; } }
             #pragma unroll
             for(uint32_t c = 0; c < GENNMI_MAX_CS; c++) { if(c < numCS) { Isyn += inj[c]; } }
-            #pragma unroll
-            for(uint32_t q = 0; q < GENNMI_MAX_PRE_OUTPUT; q++) { if(q < numRev) { asGlobal(g.outPre[q])[bi] = 0.0f; } }
-            #pragma unroll
-            for(uint32_t m = 0; m < GENNMI_MAX_PSM; m++) {
-                if(m < numPSM) {
-                    const uint32_t D = g.psm[m].maxDenDelay;
-                    if(D) { asGlobal(g.psm[m].denDelay)[((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i] = 0.0f; }
-                    asGlobal(g.psm[m].outPost)[bi] = lin[m];
-                }
-            }
             if(g.model == GENNMI_NEURON_LIF) {
                 if(l1 <= 0.0f) {
                     const float alpha = ((Isyn + g.params[0]) * g.params[1]) + g.params[2];
@@ -256,7 +249,6 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
                 if(l0 > 30.0f) { l0 = 30.0f; }
             }
         }
-        float preTrace = 0, postTrace = 0;
         if(g.preTrace) { preTrace = g.preTrace[bi] * g.preDecay; }
         if(g.postTrace) { postTrace = g.postTrace[bi] * g.postDecay; }
         if(g.model == GENNMI_NEURON_LIF) { spiked = (l1 <= 0.0f && l0 >= g.params[4]); }
@@ -265,24 +257,44 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
         vEvent = l0;           // spike-like event conditions see the updated V before any reset (neuronUpdateGroupMerged.cc:677-683)
         if(spiked) {
             preTrace += 1.0f; postTrace += 1.0f;
-            if(g.sT) { g.sT[bi] = t; }
             if(g.model == GENNMI_NEURON_LIF) { l0 = g.params[5]; l1 = g.params[6]; }
-            else if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
-                startSpike = g.startSpike[bi] + 1;
-                g.startSpike[bi] = startSpike;
-                G.nextSpikeTime[bi] = (startSpike != g.endSpike[bi]) ? g.spikeTimes[startSpike] : INFINITY;
-            }
         }
-        if(g.preTrace) { g.preTrace[bi] = preTrace; }
-        if(g.postTrace) { g.postTrace[bi] = postTrace; }
-        if(g.model != GENNMI_NEURON_SPIKE_SOURCE_ARRAY) { g.var0[bi] = l0; g.var1[bi] = l1; }
     }
-
-    // keep the user-visible ring pointers current (nothing in the kernels reads them)
-    if(localBlock == 0 && batch == 0 && threadIdx.x < g.numPSM) {
-        const gennmi_psm_t &psm = g.psm[threadIdx.x];
-        if(psm.maxDenDelay && psm.denDelayPtr) { *psm.denDelayPtr = modStep(st.epoch + 1, psm.maxDenDelay); }
-    }
+    // The stores of the update, issued once the block's spike count is on its way (the work-groups behind this one wait for
+    // that count; a wavefront queued behind the chip's store traffic before it can vote would keep them waiting).
+    auto storeState = [&]() {
+        if(i < n) {
+            if(g.model == GENNMI_NEURON_SPIKE_SOURCE_ARRAY) {
+                if(spiked) {
+                    const uint32_t startSpike = g.startSpike[bi] + 1;
+                    g.startSpike[bi] = startSpike;
+                    G.nextSpikeTime[bi] = (startSpike != g.endSpike[bi]) ? g.spikeTimes[startSpike] : INFINITY;
+                }
+            }
+            else {
+                const uint32_t numPSM = g.numPSM, numRev = g.numPreOutput;
+                #pragma unroll
+                for(uint32_t q = 0; q < GENNMI_MAX_PRE_OUTPUT; q++) { if(q < numRev) { asGlobal(g.outPre[q])[bi] = 0.0f; } }
+                #pragma unroll
+                for(uint32_t m = 0; m < GENNMI_MAX_PSM; m++) {
+                    if(m < numPSM) {
+                        const uint32_t D = g.psm[m].maxDenDelay;
+                        if(D) { asGlobal(g.psm[m].denDelay)[((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i] = 0.0f; }
+                        asGlobal(g.psm[m].outPost)[bi] = lin[m];
+                    }
+                }
+                g.var0[bi] = l0; g.var1[bi] = l1;
+            }
+            if(spiked && g.sT) { g.sT[bi] = t; }
+            if(g.preTrace) { g.preTrace[bi] = preTrace; }
+            if(g.postTrace) { g.postTrace[bi] = postTrace; }
+        }
+        // keep the user-visible ring pointers current (nothing in the kernels reads them)
+        if(localBlock == 0 && batch == 0 && threadIdx.x < g.numPSM) {
+            const gennmi_psm_t &psm = g.psm[threadIdx.x];
+            if(psm.maxDenDelay && psm.denDelayPtr) { *psm.denDelayPtr = modStep(st.epoch + 1, psm.maxDenDelay); }
+        }
+    };
 
     // ---- spike-like events: one ordered queue per event condition ----------------------------------
     if(g.numSpkEvent) {
@@ -327,6 +339,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
         __hip_atomic_store(&agg[aggBase + localBlock], ((unsigned long long)tag << 32) | blockCount,
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    storeState();
     const bool last = (localBlock == G.numBlocks - 1);
     const bool groupLeader = ((localBlock % WAVE) == WAVE - 1) || last;
     if(blockCount == 0 && !groupLeader) { return; }
