@@ -426,6 +426,9 @@ int gennmi_init_sparse_fixed_number_pre(uint32_t numPre, uint32_t numPost, uint3
     }
     uint32_t capacity = 2;
     while(capacity < rowStride) { capacity <<= 1; }
+    if(capacity * sizeof(uint32_t) > 48 * 1024) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(rowSortKernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)(capacity * sizeof(uint32_t))));
+    }
     hipLaunchKernelGGL(rowSortKernel, dim3(numPre), dim3(BLOCK), capacity * sizeof(uint32_t), 0, rowStride, rowLength, ind, capacity);
     return finishConnectivity(overflowRows);
 }
