@@ -83,8 +83,12 @@ def test_izhikevich_full_run():
     This network fires in population bursts, about one spike per neuron each and a dozen per second, and parts from the
     oracle at the first of them (step 66: a threshold crossing flipped by the order of fp32 atomic additions).  Whether the
     window's last burst falls inside it then moves the rate over the configuration's one simulated second by a few
-    per cent from run to run of the very same kernels (two runs: 0.45 % and 3.1 % from the oracle), so one second cannot
-    carry a 2 % gate; four seconds (some fifty bursts) can.  The first second is held to 8 %, one burst's worth."""
+    per cent from run to run of the very same kernels (three runs: 0.45 %, 2.5 % and 3.1 % from the oracle), and the
+    intervals between bursts vary from run to run as well: over four seconds (some fifty bursts) two runs of the same
+    build were 0.4 % and 2.0 % from the oracle.  A 2 % gate on this configuration would fail every other run for a reason
+    that has nothing to do with the kernels, so the rate over four seconds is held to 5 % and the first second to 8 %
+    (one burst's worth); what pins the arithmetic of this configuration is the lock-step comparison and the bit-identical
+    ordered run of test_gpu_full_size.py."""
     steps, second = 4000, 1000
     net = configs.izhikevich_fanout(steps=steps, noise_steps=1000)
     n = net.pops[0].n
@@ -101,7 +105,7 @@ def test_izhikevich_full_run():
     report = []
     for name, first, last, count in (("excitatory", 0, n_e // 32, n_e), ("inhibitory", n_e // 32, words, n - n_e)):
         per_step_got, per_step_want = _spikes_per_step(got, steps, words, first, last), _spikes_per_step(want, steps, words, first, last)
-        for label, upto, tol in (("first second", second, 0.08), ("four seconds", steps, RATE_TOL)):
+        for label, upto, tol in (("first second", second, 0.08), ("four seconds", steps, 0.05)):
             rate_got, rate_want = per_step_got[:upto].sum() / count / (upto / 1000.0), per_step_want[:upto].sum() / count / (upto / 1000.0)
             report.append(f"{name} {label}: {rate_got:.3f} / {rate_want:.3f} Hz")
             assert rate_want > 1.0, f"{name} neurons are silent in the oracle"
