@@ -148,6 +148,8 @@ SYMBOLS = {
     "gennmi_program_set_timing": (C.c_int, [C.c_void_p, C.c_int]),
     "gennmi_program_get_time": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_double)]),
     "gennmi_program_get_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_ulonglong * 4)]),
+    "gennmi_host_malloc": (C.c_int, [C.POINTER(C.c_void_p), C.c_size_t, C.c_int, C.POINTER(C.c_void_p)]),
+    "gennmi_host_free": (C.c_int, [C.c_void_p]),
     "gennmi_profiler_range_push": (C.c_int, [C.c_char_p]),
     "gennmi_profiler_range_pop": (C.c_int, []),
     "gennmi_init_var": (C.c_int, [C.c_void_p, C.c_uint32, C.c_size_t, C.c_uint32, C.POINTER(C.c_double * 4), C.c_uint64, C.c_uint32]),

@@ -50,7 +50,8 @@ void check(int rc, const char *what)
 // Array classes of the reference's backends (hip/backend.cc:61-236).  An array the model places on the device only
 // (VarLocation::DEVICE) gets no host memory there; here it gets address space that is committed only where host code
 // touches it and given back after every upload (gennmi_register_device_array), so a 4 GB index array that the device
-// generates never exists on the host.
+// generates never exists on the host.  Host sides of moderate size are pinned, and a zero-copy array (HOST_DEVICE_ZERO_COPY)
+// is one piece of pinned memory that both sides address.
 //--------------------------------------------------------------------------
 class Array : public Runtime::ArrayBase
 {
@@ -73,8 +74,23 @@ public:
     {
         setCount(count);
         m_Reserved = !(getLocation() & VarLocationAttribute::HOST);
+        m_ZeroCopy = !m_Reserved && (getLocation() & VarLocationAttribute::ZERO_COPY);
+        // pinned host memory where copies recur (recording buffers, state a user pulls while the model runs); the largest arrays,
+        // which are uploaded once, stay pageable: pinning gigabytes costs more than their one copy saves
+        m_Pinned = m_ZeroCopy || (!m_Reserved && getSizeBytes() <= PINNED_LIMIT);
         std::byte *host = nullptr;
-        if(m_Reserved) {
+        if(m_Pinned) {
+            void *p = nullptr, *mapped = nullptr;
+            check(gennmi_host_malloc(&p, getSizeBytes(), m_ZeroCopy ? 1 : 0, &mapped), "pinned host allocation");
+            host = static_cast<std::byte*>(p);
+            if(m_ZeroCopy) {
+                setHostPointer(host);
+                m_Device = mapped;
+                check(gennmi_register_mirror(host, m_Device, getSizeBytes()), "array registration");
+                return;
+            }
+        }
+        else if(m_Reserved) {
             void *space = mmap(nullptr, getSizeBytes(), PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
             if(space == MAP_FAILED) { throw std::bad_alloc(); }
             host = static_cast<std::byte*>(space);
@@ -92,8 +108,9 @@ public:
     virtual void free() final
     {
         check(gennmi_unregister_mirror(getHostPointer()), "array deregistration");
-        check(gennmi_free(m_Device), "array release");
-        if(m_Reserved) { munmap(getHostPointer(), getSizeBytes()); }
+        if(!m_ZeroCopy) { check(gennmi_free(m_Device), "array release"); }
+        if(m_Pinned) { check(gennmi_host_free(getHostPointer()), "pinned host release"); }
+        else if(m_Reserved) { munmap(getHostPointer(), getSizeBytes()); }
         else { std::free(getHostPointer()); }
         m_Device = nullptr;
         setHostPointer(nullptr);
@@ -104,11 +121,17 @@ public:
     virtual void pushSlice1DToDevice(size_t offset, size_t count) final
     {
         const auto [o, b] = slice(offset, count);
+        if(m_ZeroCopy) { return; }          // one memory: nothing to copy (hip/backend.cc:131-136)
         check(gennmi_memcpy_to_device(static_cast<char*>(m_Device) + o, getHostPointer() + o, b), "push");
     }
     virtual void pullSlice1DFromDevice(size_t offset, size_t count) final
     {
         const auto [o, b] = slice(offset, count);
+        if(m_ZeroCopy) {
+            // one memory: what the device wrote is there once the steps still queued have run
+            check(gennmi_synchronize(), "pull");
+            return;
+        }
         check(gennmi_memcpy_from_device(getHostPointer() + o, static_cast<const char*>(m_Device) + o, b), "pull");
     }
     virtual void memsetDeviceObject(int value) final
@@ -142,8 +165,11 @@ private:
         return {offset * elem, count * elem};
     }
 
+    static constexpr size_t PINNED_LIMIT = 64u << 20;
     void *m_Device;
     bool m_Reserved = false;    // the host side is address space without memory behind it (device-only array)
+    bool m_Pinned = false;      // the host side is pinned memory
+    bool m_ZeroCopy = false;    // ... mapped into the device's address space: host and device side are one memory
 };
 
 //--------------------------------------------------------------------------

@@ -236,6 +236,20 @@ int gennmi_malloc(void **devPtr, size_t bytes)
     HIP_TRY(hipMalloc(devPtr, bytes ? bytes : 4));
     return GENNMI_OK;
 }
+int gennmi_host_malloc(void **hostPtr, size_t bytes, int zeroCopy, void **devPtr)
+{
+    if(!hostPtr || (zeroCopy && !devPtr)) { return fail(GENNMI_EINVAL, "host_malloc: null result pointer"); }
+    HIP_TRY(hipHostMalloc(hostPtr, bytes ? bytes : 4, zeroCopy ? hipHostMallocMapped : hipHostMallocPortable));
+    std::memset(*hostPtr, 0, bytes);
+    if(devPtr) { *devPtr = nullptr; }
+    if(zeroCopy) { HIP_TRY(hipHostGetDevicePointer(devPtr, *hostPtr, 0)); }
+    return GENNMI_OK;
+}
+int gennmi_host_free(void *hostPtr)
+{
+    if(hostPtr) { HIP_TRY(hipHostFree(hostPtr)); }
+    return GENNMI_OK;
+}
 int gennmi_free(void *devPtr) { FLUSH_QUEUED(); HIP_TRY(hipFree(devPtr)); return GENNMI_OK; }
 int gennmi_memcpy_to_device(void *dev, const void *host, size_t bytes)
 {
@@ -297,7 +311,8 @@ namespace
 // deviceInitialised: a device generator filled the buffer since initialisation began, so the host copy is not the one to
 // upload; hostStale: ... and has not been copied back since.  releaseHost: the host side is lazily committed address space
 // (an array the model places on the device only) whose pages are given back after every upload.
-struct Mirror { void *dev; size_t bytes; bool deviceInitialised = false, hostStale = false, releaseHost = false; };
+// zeroCopy: host and device side are the same pinned memory (VarLocation::HOST_DEVICE_ZERO_COPY): nothing is ever copied.
+struct Mirror { void *dev; size_t bytes; bool deviceInitialised = false, hostStale = false, releaseHost = false, zeroCopy = false; };
 std::map<uintptr_t, Mirror> g_mirrors;      // keyed by host base address
 std::mutex g_mirrorMutex;
 // the registered buffer `host` points into (g_mirrorMutex held)
@@ -316,7 +331,11 @@ int gennmi_register_mirror(const void *host, void *dev, size_t bytes)
 {
     if(!host || !dev || bytes == 0) { return fail(GENNMI_EINVAL, "register_mirror: null pointer or empty buffer"); }
     std::lock_guard<std::mutex> lock(g_mirrorMutex);
-    g_mirrors[reinterpret_cast<uintptr_t>(host)] = Mirror{dev, bytes};
+    Mirror m{dev, bytes};
+    hipPointerAttribute_t attributes{};
+    if(hipPointerGetAttributes(&attributes, dev) == hipSuccess) { m.zeroCopy = (attributes.type == hipMemoryTypeHost); }
+    else { (void)hipGetLastError(); }
+    g_mirrors[reinterpret_cast<uintptr_t>(host)] = m;
     return GENNMI_OK;
 }
 int gennmi_register_device_array(const void *host, void *dev, size_t bytes)
@@ -350,6 +369,7 @@ int gennmi_mirror_ensure_host(const void *host)
     uintptr_t base = 0;
     Mirror *m = findMirror(host, &base);
     if(!m) { return fail(GENNMI_EINVAL, "mirror_ensure_host: host pointer is not inside a registered buffer"); }
+    if(m->hostStale && m->zeroCopy) { HIP_TRY(hipDeviceSynchronize()); m->hostStale = false; }
     if(m->hostStale) {
         HIP_TRY(hipMemcpy(reinterpret_cast<void*>(base), m->dev, m->bytes, hipMemcpyDeviceToHost));
         m->hostStale = false;
@@ -398,7 +418,7 @@ int gennmi_push_mirrors(void)
     FLUSH_QUEUED();
     std::lock_guard<std::mutex> lock(g_mirrorMutex);
     for(const auto &m : g_mirrors) {
-        if(!m.second.deviceInitialised) {
+        if(!m.second.deviceInitialised && !m.second.zeroCopy) {
             HIP_TRY(hipMemcpy(m.second.dev, reinterpret_cast<const void*>(m.first), m.second.bytes, hipMemcpyHostToDevice));
             noteDeviceWrite(m.second.dev, m.second.bytes);
         }

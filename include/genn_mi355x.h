@@ -78,6 +78,12 @@ int gennmi_init(int device);                                   /* hip/backend.cc
 const char *gennmi_last_error(void);
 int gennmi_device_name(char *buf, size_t len);
 int gennmi_malloc(void **devPtr, size_t bytes);                 /* Array::allocate  hip/backend.cc:86-108 */
+/* Pinned, zero-filled host memory for an array's host side (hipHostMalloc in Array::allocate, hip/backend.cc:90-97).  With
+ * `zeroCopy` (VarLocation::HOST_DEVICE_ZERO_COPY) the memory is mapped into the device's address space and *devPtr receives
+ * the address kernels use (hipHostGetDevicePointer, :101-103): such an array has no device buffer of its own and needs no
+ * copies.  Without it devPtr may be NULL.  gennmi_host_free releases the memory. */
+int gennmi_host_malloc(void **hostPtr, size_t bytes, int zeroCopy, void **devPtr);
+int gennmi_host_free(void *hostPtr);
 int gennmi_free(void *devPtr);                                  /* Array::free      hip/backend.cc:110-128 */
 int gennmi_memcpy_to_device(void *dev, const void *host, size_t bytes);    /* pushToDevice / pushSlice1DToDevice   :130-176 */
 int gennmi_memcpy_from_device(void *host, const void *dev, size_t bytes);  /* pullFromDevice / pullSlice1DFromDevice :142-198 */

@@ -416,7 +416,7 @@ int main(int argc, char *argv[])
         bool generateOnly = false;
         std::string userCxxFlags;
         std::vector<std::string> dynamicParams;
-        bool timing = false, ordered = false, deviceInit = false, doublePrecision = false, narrowInd = false, deviceArrays = false, profilerRanges = false;
+        bool timing = false, ordered = false, deviceInit = false, doublePrecision = false, narrowInd = false, deviceArrays = false, profilerRanges = false, zeroCopyRecording = false;
         int stepQueue = -1;
         std::string kernels = "auto";
         for(int a = 4; a < argc; a++) {
@@ -428,6 +428,7 @@ int main(int argc, char *argv[])
             else if(opt.rfind("--dynamic=", 0) == 0) { dynamicParams.push_back(opt.substr(10)); }
             else if(opt.rfind("--kernels=", 0) == 0) { kernels = opt.substr(10); }    // MI355X backend: library | generated | auto (Preferences::kernelSource)
             else if(opt.rfind("--step-queue=", 0) == 0) { stepQueue = std::stoi(opt.substr(13)); }      // MI355X backend: Preferences::stepQueueLength
+            else if(opt == "--zero-copy-recording") { zeroCopyRecording = true; }  // NeuronGroup::setRecordingZeroCopyEnabled for every population
             else if(opt == "--profiler-ranges") { profilerRanges = true; }         // MI355X backend: Preferences::profilerRanges
             else if(opt == "--device-init") { deviceInit = true; }                  // MI355X backend: Preferences::deviceInitialisation
             // matrices built by snippets are placed on the device only (VarLocation::DEVICE) and not written to the out directory
@@ -557,6 +558,7 @@ int main(int argc, char *argv[])
             }
             else throw std::runtime_error("pop model " + p.model);
             p.ng->setSpikeRecordingEnabled(true);
+            if(zeroCopyRecording) { p.ng->setRecordingZeroCopyEnabled(true); }
             popByName[p.name] = &p;
         }
         // populations that drive graded projections also record their spike-like events

@@ -919,6 +919,31 @@ def test_adapter_dense_kernel_and_neuron_variables_initialised_on_the_device():
         shutil.rmtree(tmp, ignore_errors=True)
 
 
+def test_adapter_zero_copy_recording_buffers():
+    """VarLocation::HOST_DEVICE_ZERO_COPY (hip/backend.cc:90-103): with NeuronGroup::setRecordingZeroCopyEnabled the recording
+    buffers are pinned host memory mapped into the device's address space — the kernels write the spike words straight into
+    them, pulls copy nothing — and the rasters must be those of the reference CPU backend's fixture, on the resident plan with
+    its step queue and with every step launched when asked for."""
+    net, snap = CASES["va_small"]()
+    net.snap = snap
+    golden = np.load(os.path.join(HERE, "golden", "va_small.npz"))
+    tmp = tempfile.mkdtemp(prefix="adapter_zero_copy_")
+    try:
+        spec = os.path.join(tmp, "spec")
+        write_netspec(net, spec)
+        for label, options in (("queued", []), ("eager", ["--step-queue=0"])):
+            work, out = os.path.join(tmp, "work_" + label), os.path.join(tmp, "out_" + label)
+            os.makedirs(work); os.makedirs(out)
+            print(f"adapter zero-copy recording ({label}): running {DRIVER}", flush=True)
+            res = subprocess.run([DRIVER, spec, work, out, "--zero-copy-recording"] + options, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
+            assert res.returncode == 0, res.stdout[-3000:]
+            for p in net.pops:
+                got = np.fromfile(os.path.join(out, f"{p.name}.spikes.u32"), np.uint32).reshape(-1, 2)
+                assert np.array_equal(got, golden[f"spikes.{p.name}"]), f"{label}: raster of {p.name} differs"
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
 def _first_difference(a, b):
     """First timestep at which two rasters ((step, neuron) pairs in ascending order) differ, or None."""
     if np.array_equal(a, b):
