@@ -1442,6 +1442,8 @@ int gennmi_runner_finalise(gennmi_runner *r)
             const uint32_t budget = blocksPerCUTile * numCU * BLOCK / r->tileThreads;
             // ... several groups share two such rounds in proportion to their synapse counts: a launch's floor is the
             // dispatch of its blocks, and the quiet steps of a network with many projections should not pay for a round each
+            const char *envPerSplit = getenv("GENNMI_TILE_SPIKES_PER_SPLIT");
+            const uint32_t spikesPerSplit = envPerSplit ? (uint32_t)std::max(1, atoi(envPerSplit)) : 4096u;
             double totalWeight = 0.0;
             for(const auto &t : tileGroups) { totalWeight += (double)t.g.numSrcNeurons * t.g.rowStride; }
             for(auto &t : tileGroups) {
@@ -1449,6 +1451,7 @@ int gennmi_runner_finalise(gennmi_runner *r)
                 const uint32_t groupBudget = std::max(t.numTiles, (uint32_t)(share * budget));
                 const uint32_t numSplits = std::max(1u, std::min(256u, groupBudget / t.numTiles));
                 t.numSplits = numSplits;
+                t.spikesPerSplit = spikesPerSplit;
                 for(uint32_t tile = 0; tile < t.numTiles; tile++) {
                     for(uint32_t split = 0; split < numSplits; split++) { t.tile = tile; t.split = split; tiles.push_back(t); }
                 }

@@ -145,6 +145,7 @@ struct TileGroupDev
     uint32_t tile, split, numSplits;    // this block: which tile, which share of the spikes
     uint32_t lanes;                     // lanes per (spike, tile) segment, power of two
     uint32_t threshold;
+    uint32_t spikesPerSplit;            // a step's spikes are shared between max(2, numSpikes / spikesPerSplit) of a tile's blocks (record path)
     uint32_t recLanes;                  // != 0: the projection has segment records (below), read by this many lanes each (5 or 10)
     const uint8_t *records;             // [numTiles][numSrc] records of 24 * recLanes + 8 bytes (128 or 256), or NULL
     const uint8_t *overflow;            // [numTiles][numSrc] 64-byte records of the 8 synapses that follow a full record, or NULL
@@ -241,24 +242,50 @@ __device__ __forceinline__ void ldsAddF32(float *addr, float v)
 }
 
 // four adds of one lane with their LDS round trips overlapped: all reads, then all swaps, then whatever lost a race
-// (including two of the four that name the same element) one by one
+// (including two of the four that name the same element) one by one.  Straight-line code: an add that is switched off
+// goes to a word of the lane's own instead of being branched around — with a branch per add the compiler waits for each
+// swap before it issues the next, five dependent LDS round trips and a dozen changes of the execution mask per call, which
+// is what bounded the tile kernels' main loops (a wavefront's pass, not memory, set their pace).
+__device__ __forceinline__ float *ldsOwnWord()
+{
+    __shared__ float unused[1024];          // (one word per thread of the largest work-group)
+    return &unused[threadIdx.x];
+}
+
 __device__ __forceinline__ void ldsAddF32x4(float *a0, float v0, bool p0, float *a1, float v1, bool p1, float *a2, float v2, bool p2, float *a3, float v3, bool p3)
 {
-    uint32_t *q0 = reinterpret_cast<uint32_t*>(a0), *q1 = reinterpret_cast<uint32_t*>(a1), *q2 = reinterpret_cast<uint32_t*>(a2), *q3 = reinterpret_cast<uint32_t*>(a3);
-    uint32_t o0 = 0, o1 = 0, o2 = 0, o3 = 0;
-    if(p0) { o0 = __hip_atomic_load(q0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
-    if(p1) { o1 = __hip_atomic_load(q1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
-    if(p2) { o2 = __hip_atomic_load(q2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
-    if(p3) { o3 = __hip_atomic_load(q3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
-    uint32_t r0 = o0, r1 = o1, r2 = o2, r3 = o3;
-    if(p0) { r0 = atomicCAS(q0, o0, __float_as_uint(__uint_as_float(o0) + v0)); }
-    if(p1) { r1 = atomicCAS(q1, o1, __float_as_uint(__uint_as_float(o1) + v1)); }
-    if(p2) { r2 = atomicCAS(q2, o2, __float_as_uint(__uint_as_float(o2) + v2)); }
-    if(p3) { r3 = atomicCAS(q3, o3, __float_as_uint(__uint_as_float(o3) + v3)); }
-    if(p0 && r0 != o0) { ldsAddF32(a0, v0); }
-    if(p1 && r1 != o1) { ldsAddF32(a1, v1); }
-    if(p2 && r2 != o2) { ldsAddF32(a2, v2); }
-    if(p3 && r3 != o3) { ldsAddF32(a3, v3); }
+    float *own = ldsOwnWord();
+    uint32_t *q0 = reinterpret_cast<uint32_t*>(p0 ? a0 : own), *q1 = reinterpret_cast<uint32_t*>(p1 ? a1 : own);
+    uint32_t *q2 = reinterpret_cast<uint32_t*>(p2 ? a2 : own), *q3 = reinterpret_cast<uint32_t*>(p3 ? a3 : own);
+    const uint32_t o0 = __hip_atomic_load(q0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t o1 = __hip_atomic_load(q1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t o2 = __hip_atomic_load(q2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t o3 = __hip_atomic_load(q3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t r0 = atomicCAS(q0, o0, __float_as_uint(__uint_as_float(o0) + v0));
+    const uint32_t r1 = atomicCAS(q1, o1, __float_as_uint(__uint_as_float(o1) + v1));
+    const uint32_t r2 = atomicCAS(q2, o2, __float_as_uint(__uint_as_float(o2) + v2));
+    const uint32_t r3 = atomicCAS(q3, o3, __float_as_uint(__uint_as_float(o3) + v3));
+    if(((r0 ^ o0) | (r1 ^ o1) | (r2 ^ o2) | (r3 ^ o3)) != 0u) {
+        if(r0 != o0) { ldsAddF32(reinterpret_cast<float*>(q0), v0); }
+        if(r1 != o1) { ldsAddF32(reinterpret_cast<float*>(q1), v1); }
+        if(r2 != o2) { ldsAddF32(reinterpret_cast<float*>(q2), v2); }
+        if(r3 != o3) { ldsAddF32(reinterpret_cast<float*>(q3), v3); }
+    }
+}
+
+// the same for two adds
+__device__ __forceinline__ void ldsAddF32x2(float *a0, float v0, bool p0, float *a1, float v1, bool p1)
+{
+    float *own = ldsOwnWord();
+    uint32_t *q0 = reinterpret_cast<uint32_t*>(p0 ? a0 : own), *q1 = reinterpret_cast<uint32_t*>(p1 ? a1 : own);
+    const uint32_t o0 = __hip_atomic_load(q0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t o1 = __hip_atomic_load(q1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t r0 = atomicCAS(q0, o0, __float_as_uint(__uint_as_float(o0) + v0));
+    const uint32_t r1 = atomicCAS(q1, o1, __float_as_uint(__uint_as_float(o1) + v1));
+    if(((r0 ^ o0) | (r1 ^ o1)) != 0u) {
+        if(r0 != o0) { ldsAddF32(reinterpret_cast<float*>(q0), v0); }
+        if(r1 != o1) { ldsAddF32(reinterpret_cast<float*>(q1), v1); }
+    }
 }
 
 }   // namespace

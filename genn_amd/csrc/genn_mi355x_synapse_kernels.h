@@ -416,47 +416,75 @@ __device__ __forceinline__ unsigned long long tileRecordLoop(const TileGroupDev 
         return r;
     };
     // DEPTH records in flight per lane group (a pass of the block is one dependent chain spike id -> record -> adds, and a
-    // step of a few thousand spikes is only a handful of passes per block): ids are fetched DEPTH passes ahead of their
-    // records, records DEPTH passes ahead of their adds
+    // step of a few thousand spikes is only a handful of passes per block): ids are fetched 2 * DEPTH passes ahead of their
+    // adds, records DEPTH passes ahead.  Every value that is loaded keeps ONE place for the whole loop — id slot v, record
+    // slot v % DEPTH, used up before it is loaded again, the round written out 2 * DEPTH passes long so that no id moves
+    // from slot to slot: a loaded value that changes its register where the loop closes is copied there, and that copy
+    // waits for every load issued before it, i.e. drains the pipeline once per round (the loop ran at a quarter of its
+    // present speed that way).
     constexpr uint32_t DEPTH = 4;
     uint32_t s = G.split * perBlock + (threadIdx.x / WAVE) * GROUPS + min(group, GROUPS - 1);
     uint32_t ids[2 * DEPTH];
     Rec recs[DEPTH];
+    // A segment longer than a record (one in seven where segments average 16 synapses, so nearly every pass of a
+    // wavefront's twelve records holds one) has its next 8 synapses in an overflow record.  That record is asked for when
+    // the segment's length is known and added DEPTH passes later, when the slot comes round again: read and added on the
+    // spot, it cost every pass a whole trip to memory, and with it every load in flight was waited for.
+    struct Ovf { float w0, w1; uint32_t t0, t1, m; };
+    Ovf ovf[DEPTH];
     #pragma unroll
-    for(uint32_t u = 0; u < 2 * DEPTH; u++) { ids[u] = spk[min(s + u * stride, lastSrc)]; }
+    for(uint32_t u = 0; u < DEPTH; u++) { ovf[u].w0 = ovf[u].w1 = 0.0f; ovf[u].t0 = ovf[u].t1 = 0u; ovf[u].m = 0u; }
+    auto addOverflow = [&](Ovf &o) {
+        if(o.m) {
+            ldsAddF32x2(&shTile[o.t0], o.w0, k < o.m, &shTile[o.t1], o.w1, k + L < o.m);
+            o.m = 0u;
+        }
+    };
+    #pragma unroll
+    for(uint32_t v = 0; v < 2 * DEPTH; v++) { ids[v] = spk[min(s + v * stride, lastSrc)]; }
     #pragma unroll
     for(uint32_t u = 0; u < DEPTH; u++) { recs[u] = fetch(ids[u]); }
-    for(; s < numSpikes; s += DEPTH * stride) {
+    // (the loop is entered with no load pending: the waits inside it are then counted from the loop's own order of loads
+    // alone; merged with this prologue's order they come out as "all but the last two or three" on every round)
+    __builtin_amdgcn_s_waitcnt(0);
+    for(; s < numSpikes; s += 2 * DEPTH * stride) {
         #pragma unroll
-        for(uint32_t u = 0; u < DEPTH; u++) {
-            const Rec cur = recs[u];
-            const uint32_t idPre = ids[u];
-            ids[u] = ids[u + DEPTH];
-            ids[u + DEPTH] = spk[min(s + (u + 2 * DEPTH) * stride, lastSrc)];
-            recs[u] = fetch(ids[u]);
-            if(!live || s + u * stride >= numSpikes) { continue; }
-            const uint32_t n = cur.meta & 0xFFFFu;
-            const uint32_t j = 4 * k;
-            ldsAddF32x4(&shTile[cur.t01 & 0xFFFFu], cur.w.x, j < n, &shTile[cur.t01 >> 16], cur.w.y, j + 1 < n,
-                        &shTile[cur.t23 & 0xFFFFu], cur.w.z, j + 2 < n, &shTile[cur.t23 >> 16], cur.w.w, j + 3 < n);
-            if(n > C) {
-                // a segment longer than a record: the next 8 synapses from its overflow record, the rest from the row itself
-                uint32_t done = C;
-                if(overflow) {
-                    GLOBAL_AS const uint8_t *ovf = overflow + (size_t)idPre * 64;
-                    for(uint32_t jj = k; jj < min(n - C, REC_OVERFLOW); jj += L) {
-                        ldsAddF32(&shTile[reinterpret_cast<GLOBAL_AS const uint16_t*>(ovf + 32)[jj]], reinterpret_cast<GLOBAL_AS const float*>(ovf)[jj]);
+        for(uint32_t v = 0; v < 2 * DEPTH; v++) {
+            Rec &cur = recs[v % DEPTH];
+            Ovf &pend = ovf[v % DEPTH];
+            addOverflow(pend);
+            if(live && s + v * stride < numSpikes) {
+                const uint32_t idPre = ids[v];
+                const uint32_t n = cur.meta & 0xFFFFu;
+                const uint32_t j = 4 * k;
+                ldsAddF32x4(&shTile[cur.t01 & 0xFFFFu], cur.w.x, j < n, &shTile[cur.t01 >> 16], cur.w.y, j + 1 < n,
+                            &shTile[cur.t23 & 0xFFFFu], cur.w.z, j + 2 < n, &shTile[cur.t23 >> 16], cur.w.w, j + 3 < n);
+                if(n > C) {
+                    uint32_t done = C;
+                    if(overflow) {
+                        GLOBAL_AS const uint8_t *rec = overflow + (size_t)idPre * 64;
+                        const uint32_t m = min(n - C, REC_OVERFLOW);
+                        if(k < m) { pend.w0 = reinterpret_cast<GLOBAL_AS const float*>(rec)[k]; pend.t0 = reinterpret_cast<GLOBAL_AS const uint16_t*>(rec + 32)[k]; }
+                        if(k + L < m) { pend.w1 = reinterpret_cast<GLOBAL_AS const float*>(rec)[k + L]; pend.t1 = reinterpret_cast<GLOBAL_AS const uint16_t*>(rec + 32)[k + L]; }
+                        pend.m = m;
+                        done = C + REC_OVERFLOW;
                     }
-                    done = C + REC_OVERFLOW;
+                    if(n > done) {
+                        // beyond both records (rare): from the row itself, on the spot
+                        const size_t base = (size_t)idPre * g.rowStride + (cur.meta >> 16);
+                        for(uint32_t jj = done + k; jj < n; jj += L) {
+                            ldsAddF32(&shTile[asGlobal(g.ind)[base + jj] - tileStart], asGlobal(g.g)[base + jj]);
+                        }
+                    }
                 }
-                const size_t base = (size_t)idPre * g.rowStride + (cur.meta >> 16);
-                for(uint32_t jj = done + k; jj < n; jj += L) {
-                    ldsAddF32(&shTile[asGlobal(g.ind)[base + jj] - tileStart], asGlobal(g.g)[base + jj]);
-                }
+                if(k == 0) { events += n; }
             }
-            if(k == 0) { events += n; }
+            cur = fetch(ids[(v + DEPTH) % (2 * DEPTH)]);
+            ids[v] = spk[min(s + (v + 2 * DEPTH) * stride, lastSrc)];
         }
     }
+    #pragma unroll
+    for(uint32_t u = 0; u < DEPTH; u++) { addOverflow(ovf[u]); }
     return events;
 }
 
@@ -471,7 +499,7 @@ __device__ __forceinline__ void presynapticTileBody(const TileGroupDev &G, float
         // touched with global atomics, which costs more than the adds themselves while a block's share of the tile is
         // sparsely filled.  Measured on 10^6 rows x 1000 synapses (us per step with 2 / 4 / 8 / 16 blocks per tile): 3 x 10^3
         // spikes 49 / 54 / 73 / 102, 2 x 10^4 spikes 171 / 114 / 111 / 159, 3 x 10^5 spikes 2281 / 1190 / 754 / 766.
-        const uint32_t activeSplits = min(G.numSplits, max(2u, numSpikes / 4096u));
+        const uint32_t activeSplits = min(G.numSplits, max(2u, numSpikes / G.spikesPerSplit));
         if(G.split >= activeSplits) { return; }
         const uint32_t tileStart = G.tile * G.tileSize;
         const uint32_t tileLen = min(G.tileSize, g.numTrgNeurons - tileStart);
