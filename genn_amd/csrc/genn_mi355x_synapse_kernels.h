@@ -20,6 +20,19 @@ __device__ __forceinline__ float learnPostOnSynapse(const LearnPostDev &L, const
     }
     return w;
 }
+// the same rule with what it reads of the presynaptic neuron (last spike time, trace) already in registers: the same for every
+// synapse of a row
+__device__ __forceinline__ float learnPostOnSynapseWith(const LearnPostDev &L, const gennmi_presynaptic_update_group_t &g, float stRaw, float trace,
+                                                        float w, float t, float dt)
+{
+    const float stPre = dt + stRaw;
+    const float dtSpike = t - stPre;
+    if(dtSpike > 0) {
+        const float factor = (L.tauPlus > 0.0f) ? (float)exp((double)(-dtSpike / L.tauPlus)) : trace;
+        return fminf(g.wMax, fmaxf(g.wMin, w + (L.aPlus * factor)));
+    }
+    return w;
+}
 __device__ __forceinline__ bool bitmapTest(GLOBAL_AS const uint32_t *bitmap, uint32_t i) { return (bitmap[i >> 5] >> (i & 31)) & 1u; }
 
 // ------------------------------------------------------------------------------------------------
@@ -201,7 +214,11 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
                 GLOBAL_AS float *wPtr = weight + (size_t)batch * g.numSrcNeurons * g.rowStride + rowBase + j;
                 const float w = *wPtr;
                 const size_t post = (size_t)batch * numTrg + idPost;
-                const float stPost = dt + asGlobal(g.trgST)[post];   // st_post = DT*(backPropSteps+1) + trgST (synapseUpdateGroupMerged.cc:134-142)
+                // (everything the rule reads of the target is asked for at once: one trip to memory after the index, not three)
+                const float stRaw = asGlobal(g.trgST)[post];
+                const float trace = (g.wum == GENNMI_WUM_STDP) ? 0.0f : asGlobal(g.postTrace)[post];
+                const uint32_t firedBits = G.learn.enabled ? asGlobal(G.learn.trgBitmap)[(size_t)batch * ((numTrg + 31) / 32) + (idPost >> 5)] : 0u;
+                const float stPost = dt + stRaw;   // st_post = DT*(backPropSteps+1) + trgST (synapseUpdateGroupMerged.cc:134-142)
                 atomicAddF32(&outPost[idPost], w);
                 const float dtSpike = st.t - stPost;
                 float newWeight = w;
@@ -209,11 +226,11 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
                 if(dtSpike > 0) {
                     // trace rule: the target's trace; built-in additive rule (weightUpdateModels.h:352-359): the exponential
                     // of the time since the target's last spike, evaluated in double and rounded once as the reference does
-                    const float factor = (g.wum == GENNMI_WUM_STDP) ? (float)exp((double)(-dtSpike / g.tauMinus)) : asGlobal(g.postTrace)[post];
+                    const float factor = (g.wum == GENNMI_WUM_STDP) ? (float)exp((double)(-dtSpike / g.tauMinus)) : trace;
                     newWeight = fminf(g.wMax, fmaxf(g.wMin, w - (g.aMinus * factor)));
                     changed = true;
                 }
-                if(G.learn.enabled && bitmapTest(asGlobal(G.learn.trgBitmap) + (size_t)batch * ((numTrg + 31) / 32), idPost)) {
+                if((firedBits >> (idPost & 31u)) & 1u) {
                     newWeight = learnPostOnSynapse(G.learn, g, batch, idPre, newWeight, st.t, dt, changed);
                 }
                 if(changed) { *wPtr = newWeight; }
@@ -537,16 +554,36 @@ __device__ __forceinline__ void presynapticTileBody(const TileGroupDev &G, float
     GLOBAL_AS const float *postTrace = asGlobal(g.postTrace) + (size_t)batch * g.numTrgNeurons;
     GLOBAL_AS const uint32_t *trgBitmap = asGlobal(G.learn.trgBitmap) + (size_t)batch * ((g.numTrgNeurons + 31) / 32);
     const bool paired = (G.learn.enabled != 0);
-    auto depress = [&](uint32_t idPre, uint32_t idPost, float w) -> float {
-        const float stPost = dt + trgST[idPost];
+    // the rule on one synapse, given what it reads of its target: last spike time, trace, word of the spike bitmap
+    // (what the postsynaptic-spike rule reads of the row's own neuron — rowST, rowTrace — is loaded once per row, one row ahead:
+    // in a burst most targets have just fired, and two dependent loads per synapse were the longest chain of such a step)
+    float rowST = 0.0f, rowTrace = 0.0f;
+    auto depressWith = [&](uint32_t idPre, uint32_t idPost, float w, float st, float trace, uint32_t bits) -> float {
+        const float stPost = dt + st;
         const float dtSpike = t - stPost;
         float nw = w;
         if(dtSpike > 0) {
-            const float factor = additive ? (float)exp((double)(-dtSpike / g.tauMinus)) : postTrace[idPost];
+            const float factor = additive ? (float)exp((double)(-dtSpike / g.tauMinus)) : trace;
             nw = fminf(g.wMax, fmaxf(g.wMin, w - (g.aMinus * factor)));
         }
         // the target fired in the last update too: its postsynaptic-spike rule follows here (see LearnPostDev)
-        if(paired && bitmapTest(trgBitmap, idPost)) { bool changed = false; nw = learnPostOnSynapse(G.learn, g, batch, idPre, nw, t, dt, changed); }
+        if(paired && ((bits >> (idPost & 31u)) & 1u)) { nw = learnPostOnSynapseWith(G.learn, g, rowST, rowTrace, nw, t, dt); }
+        return nw;
+    };
+    auto depress = [&](uint32_t idPre, uint32_t idPost, float w) -> float {
+        return depressWith(idPre, idPost, w, trgST[idPost], additive ? 0.0f : postTrace[idPost], paired ? trgBitmap[idPost >> 5] : 0u);
+    };
+    // four synapses of a lane: all their gathers are issued before the first is used (one synapse at a time, each waits
+    // for its own two or three dependent loads: twelve trips to L2 in a row per lane and pass)
+    auto depress4 = [&](uint32_t idPre, const u32x4u &ip, const f32x4u &w) -> f32x4u {
+        const float st0 = trgST[ip.x], st1 = trgST[ip.y], st2 = trgST[ip.z], st3 = trgST[ip.w];
+        float tr0 = 0.0f, tr1 = 0.0f, tr2 = 0.0f, tr3 = 0.0f;
+        if(!additive) { tr0 = postTrace[ip.x]; tr1 = postTrace[ip.y]; tr2 = postTrace[ip.z]; tr3 = postTrace[ip.w]; }
+        uint32_t b0 = 0, b1 = 0, b2 = 0, b3 = 0;
+        if(paired) { b0 = trgBitmap[ip.x >> 5]; b1 = trgBitmap[ip.y >> 5]; b2 = trgBitmap[ip.z >> 5]; b3 = trgBitmap[ip.w >> 5]; }
+        f32x4u nw;
+        nw.x = depressWith(idPre, ip.x, w.x, st0, tr0, b0); nw.y = depressWith(idPre, ip.y, w.y, st1, tr1, b1);
+        nw.z = depressWith(idPre, ip.z, w.z, st2, tr2, b2); nw.w = depressWith(idPre, ip.w, w.w, st3, tr3, b3);
         return nw;
     };
     const uint32_t L = G.lanes;
@@ -561,22 +598,25 @@ __device__ __forceinline__ void presynapticTileBody(const TileGroupDev &G, float
     uint32_t id0 = spk[min(s, lastSrc)], id1 = spk[min(s + stride, lastSrc)];
     size_t o0 = (size_t)id0 * (G.numTiles + 1) + G.tile;
     uint32_t a0 = off[o0], b0 = off[o0 + 1];
+    GLOBAL_AS const float *srcST = asGlobal(G.learn.srcST) + (size_t)batch * g.numSrcNeurons;
+    GLOBAL_AS const float *preTrace = asGlobal(G.learn.preTrace) + (size_t)batch * g.numSrcNeurons;
+    const bool rowTraceWanted = paired && !(G.learn.tauPlus > 0.0f);
+    float st0 = paired ? srcST[id0] : 0.0f, tr0 = rowTraceWanted ? preTrace[id0] : 0.0f;
     for(; s < numSpikes; s += stride) {
         const uint32_t idPre = id0, a = a0, b = b0;
+        rowST = st0; rowTrace = tr0;
         id0 = id1;
         id1 = spk[min(s + 2 * stride, lastSrc)];
         o0 = (size_t)id0 * (G.numTiles + 1) + G.tile;
         a0 = off[o0]; b0 = off[o0 + 1];
+        if(paired) { st0 = srcST[id0]; }
+        if(rowTraceWanted) { tr0 = preTrace[id0]; }
         const size_t rowBase = (size_t)idPre * g.rowStride;
         for(uint32_t j = a + 4 * lis; j < b; j += 4 * L) {
             if(j + 4 <= b) {
                 const u32x4u ip = *reinterpret_cast<GLOBAL_AS const u32x4u*>(ind + rowBase + j);
                 const f32x4u w = *reinterpret_cast<GLOBAL_AS const f32x4u*>(weight + rowBase + j);
-                if(stdp) {
-                    f32x4u nw;
-                    nw.x = depress(idPre, ip.x, w.x); nw.y = depress(idPre, ip.y, w.y); nw.z = depress(idPre, ip.z, w.z); nw.w = depress(idPre, ip.w, w.w);
-                    *reinterpret_cast<GLOBAL_AS f32x4u*>(weight + rowBase + j) = nw;
-                }
+                if(stdp) { *reinterpret_cast<GLOBAL_AS f32x4u*>(weight + rowBase + j) = depress4(idPre, ip, w); }
                 ldsAddF32x4(&shTile[ip.x - tileStart], w.x, true, &shTile[ip.y - tileStart], w.y, true,
                             &shTile[ip.z - tileStart], w.z, true, &shTile[ip.w - tileStart], w.w, true);
             }
