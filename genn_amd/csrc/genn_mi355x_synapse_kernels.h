@@ -1136,15 +1136,21 @@ __device__ __forceinline__ void postsynapticBody(const PostGroupDev &G, uint32_t
                 live[u] = (i < npre);
                 rowMajorIndex[u] = live[u] ? remap[colBase + i] : 0u;
             }
+            // second trip: everything an entry needs, for all four entries at once and whether the entry is live or not (a
+            // dead one reads row 0 and synapse 0: readable) — loads that wait for the bitmap's answer, or sit behind a
+            // branch per entry, are issued one entry after the other and the walk becomes nine trips long instead of three
             float stPre[INFLIGHT], trace[INFLIGHT], w[INFLIGHT];
+            uint32_t firedBits[INFLIGHT], idPre[INFLIGHT];
             #pragma unroll
             for(int u = 0; u < INFLIGHT; u++) {
-                const uint32_t idPre = rowMajorIndex[u] / g.rowStride;
-                live[u] = live[u] && !(paired && bitmapTest(srcBitmap, idPre));
-                stPre[u] = live[u] ? srcST[idPre] : 0.0f;
-                trace[u] = (live[u] && !additive) ? preTrace[idPre] : 0.0f;
-                w[u] = live[u] ? weight[rowMajorIndex[u]] : 0.0f;
+                idPre[u] = rowMajorIndex[u] / g.rowStride;
+                firedBits[u] = paired ? srcBitmap[idPre[u] >> 5] : 0u;
+                stPre[u] = srcST[idPre[u]];
+                trace[u] = additive ? 0.0f : preTrace[idPre[u]];
+                w[u] = weight[rowMajorIndex[u]];
             }
+            #pragma unroll
+            for(int u = 0; u < INFLIGHT; u++) { live[u] = live[u] && !((firedBits[u] >> (idPre[u] & 31u)) & 1u); }
             #pragma unroll
             for(int u = 0; u < INFLIGHT; u++) {
                 const float dtSpike = st.t - (dt + stPre[u]);
