@@ -206,13 +206,15 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
                     }
                 }
             }
-            else if(j < npost) {
+            else {
                 // trace STDP presynaptic-spike code (pygenn/genn_model.py:1456-1463); every synapse of
                 // the row is owned by exactly one lane, so the read-modify-write of g needs no atomic
-                // (plastic weights, spike times and traces are per batch: VarAccess::READ_WRITE variables are duplicated)
-                const uint32_t idPost = ind[rowBase + j];
+                // (plastic weights, spike times and traces are per batch: VarAccess::READ_WRITE variables are duplicated).
+                // Index and weight are read with the row's length, not after it (rows are padded: any j < rowStride is readable).
                 GLOBAL_AS float *wPtr = weight + (size_t)batch * g.numSrcNeurons * g.rowStride + rowBase + j;
-                const float w = *wPtr;
+                uint32_t idPost = 0; float w = 0.0f;
+                if(inRow) { idPost = ind[rowBase + j]; w = *wPtr; }
+                if(j >= npost) { if(lis == 0 && chunk == 0) { events += npost; } continue; }
                 const size_t post = (size_t)batch * numTrg + idPost;
                 // (everything the rule reads of the target is asked for at once: one trip to memory after the index, not three)
                 const float stRaw = asGlobal(g.trgST)[post];
