@@ -488,8 +488,8 @@ int gennmi_runner_create(gennmi_runner **runner, float dt, uint32_t batchSize)
     HIP_TRY(hipMemset(r->dError, 0, sizeof(uint32_t)));
     HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&r->hError), sizeof(uint32_t), hipHostMallocDefault));
     *r->hError = 0;
-    HIP_TRY(hipMalloc(&r->dEvents, sizeof(unsigned long long)));
-    HIP_TRY(hipMemset(r->dEvents, 0, sizeof(unsigned long long)));
+    HIP_TRY(hipMalloc(&r->dEvents, sizeof(unsigned long long) * EVENT_SLOTS * EVENT_SLOT_STRIDE));
+    HIP_TRY(hipMemset(r->dEvents, 0, sizeof(unsigned long long) * EVENT_SLOTS * EVENT_SLOT_STRIDE));
     HIP_TRY(hipMalloc(&r->dState, sizeof(StepState)));
     HIP_TRY(hipMemset(r->dState, 0, sizeof(StepState)));
     {
@@ -2119,7 +2119,12 @@ int gennmi_runner_event_count(gennmi_runner *r, unsigned long long *events)
     if(!r || !events) { return fail(GENNMI_EINVAL, "runner_event_count: null argument"); }
     FLUSH_QUEUED();
     HIP_TRY(hipStreamSynchronize(r->stream));
-    HIP_TRY(hipMemcpy(events, r->dEvents, sizeof(*events), hipMemcpyDeviceToHost));
+    // (partial counts a cache line apart: see addEvents)
+    unsigned long long slots[EVENT_SLOTS * EVENT_SLOT_STRIDE];
+    HIP_TRY(hipMemcpy(slots, r->dEvents, sizeof(slots), hipMemcpyDeviceToHost));
+    unsigned long long total = 0;
+    for(uint32_t k = 0; k < EVENT_SLOTS; k++) { total += slots[k * EVENT_SLOT_STRIDE]; }
+    *events = total;
     return GENNMI_OK;
 }
 

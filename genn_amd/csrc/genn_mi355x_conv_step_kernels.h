@@ -94,6 +94,7 @@ void convStepKernel(const ConvMfmaDev * __restrict__ conv, const NeuronGroupDev 
     extern __shared__ float shConvM[];
     __shared__ uint32_t shWaveTotal[CONV_STEP_THREADS / WAVE];
     __shared__ uint32_t shPrefix;
+    __shared__ unsigned long long shWaveEvents[CONV_STEP_THREADS / WAVE];
     const Resolved st = resolve(args, dt);
     const ConvMfmaDev &G = conv[0];
     const uint32_t ow = (uint32_t)G.g.conv[6], oc = (uint32_t)G.g.conv[7], oh = (uint32_t)G.g.conv[5];
@@ -121,7 +122,7 @@ void convStepKernel(const ConvMfmaDev * __restrict__ conv, const NeuronGroupDev 
     ConvStepEpilogue epilogue{plainNeuronOf(t), t.psm[0].kind, t.numCS, t.psm[0].init, t.psm[0].expDecay, asGlobal(t.var0) + (size_t)batch * n,
                               asGlobal(t.var1) + (size_t)batch * n, asGlobal(t.psm[0].outPost) + (size_t)batch * n,
                               spikeBits, ow, oc, dt, t.numCS ? t.cs[0].amp : 0.0f, {}, {}, {}};
-    convMfmaBlock<CONV_STEP_THREADS>(G, rowGroup, batch, st.epoch, shConvM, epilogue, eventCounter);
+    convMfmaBlock<CONV_STEP_THREADS>(G, rowGroup, batch, st.epoch, shConvM, epilogue, eventCounter, shWaveEvents);
     __syncthreads();
 
     // ---- the block's spikes, in ascending neuron index: thread k owns the words [k * per, (k + 1) * per) of the bitmap
@@ -160,5 +161,13 @@ void convStepKernel(const ConvMfmaDev * __restrict__ conv, const NeuronGroupDev 
         }
     }
     if(rowGroup == convBlocks - 1 && threadIdx.x == 0) { t.spkCnt[batch] = prefix + blockCount; }
+    // the work-group's synaptic events, one atomic, behind which nothing waits (shWaveEvents was written before the barrier
+    // that followed the products)
+    if(threadIdx.x == 0) {
+        unsigned long long events = 0;
+        #pragma unroll
+        for(uint32_t w = 0; w < CONV_STEP_THREADS / WAVE; w++) { events += shWaveEvents[w]; }
+        if(events) { addEvents(eventCounter, events); }
+    }
 }
 }   // namespace

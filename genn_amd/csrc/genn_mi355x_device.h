@@ -241,6 +241,17 @@ __device__ __forceinline__ void ldsAddF32(float *addr, float v)
     } while(old != assumed);
 }
 
+// The runner's count of synaptic events is kept as EVENT_SLOTS partial counts a cache line apart (the host adds them up):
+// atomics on ONE address complete one after the other, about 8 ns each, so a launch whose thousand wavefronts each add
+// their share to a single counter ends 8 us after its last useful instruction — and any barrier behind such an add waits
+// that long.  A wavefront adds to the slot its work-group and wavefront numbers select.
+constexpr uint32_t EVENT_SLOTS = 64, EVENT_SLOT_STRIDE = 16;        // (16 x 8 bytes = 128 bytes)
+__device__ __forceinline__ void addEvents(unsigned long long *eventCounter, unsigned long long events)
+{
+    const uint32_t slot = (blockIdx.x * 5u + blockIdx.y * 3u + (threadIdx.x / WAVE)) & (EVENT_SLOTS - 1);
+    atomicAdd(&eventCounter[(size_t)slot * EVENT_SLOT_STRIDE], events);
+}
+
 // four adds of one lane with their LDS round trips overlapped: all reads, then all swaps, then whatever lost a race
 // (including two of the four that name the same element) one by one.  Straight-line code: an add that is switched off
 // goes to a word of the lane's own instead of being branched around — with a branch per add the compiler waits for each

@@ -146,7 +146,7 @@ void presynapticOrderedKernel(OrderedGroupDev G, StepArgs args, float dt, unsign
             if(slot < D) { denDelay[(size_t)slot * g.numTrgNeurons + idPost] = acc[q]; }
         }
     }
-    if(lane == 0 && events) { atomicAdd(eventCounter, events); }
+    if(lane == 0 && events) { addEvents(eventCounter, events); }
 }
 }   // namespace
 

@@ -640,7 +640,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         if(G.shadowSpk) { G.shadowCnt[shadowParity] = offset + ownCount; }
     }
     for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
-    if(lane == 0 && events) { atomicAdd(eventCounter, events); }
+    if(lane == 0 && events) { addEvents(eventCounter, events); }
 }
 
 

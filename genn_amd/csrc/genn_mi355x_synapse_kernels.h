@@ -243,7 +243,7 @@ __device__ __forceinline__ void presynapticBody(const PreGroupDev &G, uint32_t b
 
     // one counter update per wave
     for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
-    if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+    if((threadIdx.x & (WAVE - 1)) == 0 && events) { addEvents(eventCounter, events); }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -313,7 +313,7 @@ void presynapticDenseKernel(const DenseGroupDev * __restrict__ blocks, unsigned 
         else if(acc != 0.0f) { atomicAddF32(&outPost[j], acc); }
     }
     for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
-    if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+    if((threadIdx.x & (WAVE - 1)) == 0 && events) { addEvents(eventCounter, events); }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -394,7 +394,7 @@ void presynapticProceduralKernel(const ProcGroupDev * __restrict__ blocks, unsig
         }
     }
     for(int off = WAVE / 2; off > 0; off >>= 1) { events += __shfl_down(events, off, WAVE); }
-    if(lane == 0 && events) { atomicAdd(eventCounter, events); }
+    if(lane == 0 && events) { addEvents(eventCounter, events); }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -534,7 +534,7 @@ __device__ __forceinline__ void presynapticTileBody(const TileGroupDev &G, float
             if(v != 0.0f) { atomicAddF32(&outPost[k], v); }
         }
         for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
-        if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+        if((threadIdx.x & (WAVE - 1)) == 0 && events) { addEvents(eventCounter, events); }
         return;
     }
     const uint32_t tileStart = G.tile * G.tileSize;
@@ -640,7 +640,7 @@ __device__ __forceinline__ void presynapticTileBody(const TileGroupDev &G, float
         if(v != 0.0f) { atomicAddF32(&outPost[k], v); }
     }
     for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
-    if((threadIdx.x & (WAVE - 1)) == 0 && events) { atomicAdd(eventCounter, events); }
+    if((threadIdx.x & (WAVE - 1)) == 0 && events) { addEvents(eventCounter, events); }
 }
 
 __global__ __launch_bounds__(1024)
@@ -753,7 +753,7 @@ void presynapticConvTileKernel(const ConvTileDev * __restrict__ blocks, unsigned
         }
     }
     for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
-    if(lane == 0 && events) { atomicAdd(eventCounter, events); }
+    if(lane == 0 && events) { addEvents(eventCounter, events); }
 }
 
 // Segment boundaries of every row for the tile kernel; also verifies that rows are sorted by target.
@@ -855,7 +855,7 @@ __device__ __forceinline__ uint32_t convMfmaLdsFloats(const ConvMfmaDev &G)
 // the output rows [rowGroup * rowsPerBlock, ...) of one batch, by all THREADS threads of a block; `epoch`: completed steps
 template<int THREADS, typename Epilogue>
 __device__ __forceinline__ void convMfmaBlock(const ConvMfmaDev &G, uint32_t rowGroup, uint32_t batch, unsigned long long epoch, float *lds,
-                                              Epilogue &epilogue, unsigned long long *eventCounter)
+                                              Epilogue &epilogue, unsigned long long *eventCounter, unsigned long long *waveEvents = nullptr)
 {
     const gennmi_presynaptic_update_group_t &g = G.g;
     const int kh = g.conv[0], kw = g.conv[1], ih = g.conv[2], iw = g.conv[3], ic = g.conv[4];
@@ -1005,7 +1005,12 @@ __device__ __forceinline__ void convMfmaBlock(const ConvMfmaDev &G, uint32_t row
         epilogue.finish(acc, r, y, x0, o, half);
     }
     for(int o2 = WAVE / 2; o2 > 0; o2 >>= 1) { events += __shfl_down(events, o2, WAVE); }
-    if(lane == 0 && events) { atomicAdd(eventCounter, events); }
+    // (a caller with barriers still to come takes the wavefronts' sums in LDS and adds them itself when it is done: a barrier
+    // waits for the wavefront's memory operations, and a thousand atomics on the one counter complete one after the other)
+    if(lane == 0) {
+        if(waveEvents) { waveEvents[wave] = events; }
+        else if(events) { addEvents(eventCounter, events); }
+    }
 }
 
 __global__ __launch_bounds__(CONV_MFMA_THREADS)
