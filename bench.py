@@ -42,9 +42,9 @@ MEASURED_TRAFFIC_BYTES = {
                          "kernel_source": ("genn_amd/csrc/genn_mi355x_resident_kernels.h", "6e38adb29614848d"),
                          "source": "rocprofv3 --pmc FETCH_SIZE (67852.50 x 2 KiB) + WRITE_SIZE (16193.69 x 1 KiB) of the timed 20-step "
                                    "launch, profiles/residentKernel_potjans_full.md"},
-    ("conv", 1000, 100): {"plan": "stepped", "requires": "conv_step_in_one_launch", "bytes_per_launch": 66207078,
-                          "kernel_source": ("genn_amd/csrc/genn_mi355x_conv_step_kernels.h", "2914660ba1d4438d"),
-                          "source": "rocprofv3 --pmc FETCH_SIZE (18922.75 x 2 KiB) + WRITE_SIZE (26809.85 x 1 KiB), average over the "
+    ("conv", 1000, 100): {"plan": "stepped", "requires": "conv_step_in_one_launch", "bytes_per_launch": 66118287,
+                          "kernel_source": ("genn_amd/csrc/genn_mi355x_conv_step_kernels.h", "b33aec4cfae473d9"),
+                          "source": "rocprofv3 --pmc FETCH_SIZE (18888.04 x 2 KiB) + WRITE_SIZE (26792.56 x 1 KiB), average over the "
                                     "run's 1,100 launches, profiles/convStepKernel_conv_batch16.md"},
 }
 FP32_MFMA_PEAK_TFLOPS = 157.3
