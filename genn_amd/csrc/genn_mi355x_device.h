@@ -272,10 +272,12 @@ __device__ __forceinline__ void ldsAddF32x4(float *a0, float v0, bool p0, float 
     const uint32_t o1 = __hip_atomic_load(q1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     const uint32_t o2 = __hip_atomic_load(q2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     const uint32_t o3 = __hip_atomic_load(q3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __builtin_amdgcn_sched_barrier(0);      // (all four reads are issued before the first swap waits for its own)
     const uint32_t r0 = atomicCAS(q0, o0, __float_as_uint(__uint_as_float(o0) + v0));
     const uint32_t r1 = atomicCAS(q1, o1, __float_as_uint(__uint_as_float(o1) + v1));
     const uint32_t r2 = atomicCAS(q2, o2, __float_as_uint(__uint_as_float(o2) + v2));
     const uint32_t r3 = atomicCAS(q3, o3, __float_as_uint(__uint_as_float(o3) + v3));
+    __builtin_amdgcn_sched_barrier(0);
     if(((r0 ^ o0) | (r1 ^ o1) | (r2 ^ o2) | (r3 ^ o3)) != 0u) {
         if(r0 != o0) { ldsAddF32(reinterpret_cast<float*>(q0), v0); }
         if(r1 != o1) { ldsAddF32(reinterpret_cast<float*>(q1), v1); }
