@@ -1488,7 +1488,9 @@ int gennmi_runner_finalise(gennmi_runner *r)
     const uint32_t synThreads = r->tileBlocks ? r->tileThreads : (uint32_t)BLOCK;
     r->synapseThreads = synThreads;
     const char *envBudget = getenv("GENNMI_PRESYN_BLOCKS_PER_CU");
-    const uint32_t blocksPerCU = envBudget ? std::max(1, atoi(envBudget)) : 4u;
+    // (2, not more: measured with 4 / 2 / 1 — 100 k-neuron plastic network 23.8 / 22.6 / 22.6 us per step, 10^6-neuron fan-out network
+    // 45.6 / 44.0 / 44.8, microcircuit stepped launch by launch 11.8 / 11.4 / 12.2: a quiet step pays for every block it dispatches)
+    const uint32_t blocksPerCU = envBudget ? std::max(1, atoi(envBudget)) : 2u;
     // the launch has one grid row per batch, so the budget is per batch (at least one block per compute unit in all)
     const uint64_t budget = std::max<uint64_t>((numCU + r->batch - 1) / r->batch, (uint64_t)numCU * blocksPerCU * BLOCK / synThreads / r->batch);
     std::vector<uint64_t> wantBlocks;
@@ -1523,7 +1525,9 @@ int gennmi_runner_finalise(gennmi_runner *r)
     for(auto &p : r->post) {
         p.lanesPerSpike = std::min<uint32_t>(WAVE, std::max(4u, pow2Ceil((p.g.colStride + 3) / 4)));
         const uint64_t wantSubGroups = std::max<uint64_t>(8, p.g.numTrgNeurons / 16);
-        const uint32_t cap = std::max(1u, (numCU * 4u * BLOCK / synThreads) / (uint32_t)r->post.size());
+        const char *envPost = getenv("GENNMI_POST_BLOCKS_PER_CU");
+        const uint32_t postPerCU = envPost ? (uint32_t)std::max(1, atoi(envPost)) : 4u;
+        const uint32_t cap = std::max(1u, (numCU * postPerCU * BLOCK / synThreads) / (uint32_t)r->post.size());
         p.startBlock = block;
         p.numBlocks = std::max(1u, (uint32_t)std::min<uint64_t>((wantSubGroups * p.lanesPerSpike + synThreads - 1) / synThreads, cap));
         block += p.numBlocks;
