@@ -173,18 +173,23 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     const uint32_t numProj = T.numProj;
     if(tid < numProj) { shProj[tid] = T.proj[tid]; }
     __syncthreads();
-    if(tid == 0) {
-        // projections grouped by source group (counting sort; a handful of entries, read from the LDS copy: one thread
-        // chasing them through global memory costs tens of microseconds per launch)
-        for(uint32_t s = 0; s <= RES_MAX_GROUPS; s++) { shProjStart[s] = 0; }
-        for(uint32_t p = 0; p < numProj; p++) { shProjStart[shProj[p].srcGroup + 1]++; }
-        for(uint32_t s = 0; s < RES_MAX_GROUPS; s++) { shProjStart[s + 1] += shProjStart[s]; }
-        for(uint32_t p = 0; p < numProj; p++) {
-            const uint32_t s = shProj[p].srcGroup;
-            uint32_t before = 0;
-            for(uint32_t q = 0; q < p; q++) { before += (shProj[q].srcGroup == s) ? 1u : 0u; }
-            shProjIdx[shProjStart[s] + before] = (uint8_t)p;
+    // projections grouped by source group (a counting sort of a handful of entries, read from the LDS copy; every thread
+    // finds one entry's place by itself — one thread doing all of it is a chain of a hundred dependent LDS reads, 3 us
+    // of every launch)
+    if(tid <= RES_MAX_GROUPS) {
+        uint32_t below = 0;
+        for(uint32_t q = 0; q < numProj; q++) { below += (shProj[q].srcGroup < tid) ? 1u : 0u; }
+        shProjStart[tid] = below;
+    }
+    if(tid < numProj) {
+        const uint32_t s = shProj[tid].srcGroup;
+        uint32_t below = 0, before = 0;
+        for(uint32_t q = 0; q < numProj; q++) {
+            const uint32_t sq = shProj[q].srcGroup;
+            below += (sq < s) ? 1u : 0u;
+            before += (q < tid && sq == s) ? 1u : 0u;
         }
+        shProjIdx[below + before] = (uint8_t)tid;
     }
 
     // ---- state: neuron variables in registers, inSyn and ring slices in LDS
