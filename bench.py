@@ -239,19 +239,13 @@ def run_net_workload(args, workload, steps, warmup, profile_steps, with_cpu, wit
     model.run(warmup)
     model.synchronize()
     ev0 = model.synaptic_event_count
-    # Device time of the timed region from HIP events on the runner's stream: recorded around the region, or — on the
-    # resident plan, whose region is one launch — bound to that launch itself (its own begin and end, the duration a kernel
-    # trace shows; nothing is added to the stream)
-    launch_bound_events = model.runner_info()["resident_plan"] and steps >= 4
     t0 = time.perf_counter()
-    if not launch_bound_events:
-        model.stream_mark(0)
+    model.stream_mark(0)
     model.run(steps)
-    if not launch_bound_events:
-        model.stream_mark(1)
+    model.stream_mark(1)
     model.synchronize()
     wall = time.perf_counter() - t0
-    region_s = model.resident_launch_seconds() if launch_bound_events else model.stream_elapsed()
+    region_s = model.stream_elapsed()          # HIP events on the runner's stream around the timed region
     events = model.synaptic_event_count - ev0
     events_with_warmup = events + ev0
 
@@ -365,14 +359,12 @@ def run_net_workload(args, workload, steps, warmup, profile_steps, with_cpu, wit
         model.synchronize()
         ev0s = model.synaptic_event_count
         t0 = time.perf_counter()
-        if not info["resident_plan"]:
-            model.stream_mark(0)
+        model.stream_mark(0)
         model.run(args.steady_steps)
-        if not info["resident_plan"]:
-            model.stream_mark(1)
+        model.stream_mark(1)
         model.synchronize()
         wall_s = time.perf_counter() - t0
-        region = model.resident_launch_seconds() if info["resident_plan"] else model.stream_elapsed()
+        region = model.stream_elapsed()
         ev_s = model.synaptic_event_count - ev0s
         bpe = bytes_per_event or max(BYTES_PER_EVENT[k] for k in kinds)
         nbytes = batch * sum(p.n * (0 if p.model == "ssa" else 32) for p in net.pops)

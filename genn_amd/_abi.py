@@ -174,7 +174,6 @@ SYMBOLS = {
     "gennmi_runner_kernel_stats": (C.c_int, [C.c_void_p, C.POINTER(C.c_double * 8)]),
     "gennmi_runner_stream_mark": (C.c_int, [C.c_void_p, C.c_int]),
     "gennmi_runner_stream_elapsed": (C.c_int, [C.c_void_p, C.POINTER(C.c_double)]),
-    "gennmi_runner_resident_launch_seconds": (C.c_int, [C.c_void_p, C.POINTER(C.c_double)]),
     "gennmi_runner_get_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint32 * 4)]),
     "gennmi_runner_event_count": (C.c_int, [C.c_void_p, C.POINTER(_ULL)]),
 }

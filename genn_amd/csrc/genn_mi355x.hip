@@ -25,7 +25,6 @@
 #include <dlfcn.h>
 #include <sys/mman.h>
 #include <hip/hip_runtime.h>
-#include <hip/hip_ext.h>
 
 #include <algorithm>
 #include <atomic>
@@ -121,8 +120,6 @@ struct gennmi_runner
     struct Pending { hipEvent_t a, b; int kind; };          // kind: 0 presynaptic, 1 postsynaptic, 2 neuron, 3 single-launch step
     std::vector<hipEvent_t> eventPool; size_t eventNext = 0; std::vector<Pending> pending;
     hipEvent_t marks[2] = {nullptr, nullptr};               // gennmi_runner_stream_mark
-    hipEvent_t resEvents[2] = {nullptr, nullptr};           // start and end of the latest resident launch(es) of one call (bound to the launches)
-    bool resEventsSet = false;
     // step queue (gennmi_runner_set_step_queue): steps asked for one at a time and not yet launched
     struct QueuedStep { float t; uint32_t recordingTimestep; };
     uint32_t stepQueueLimit = 0;
@@ -515,7 +512,6 @@ int gennmi_runner_destroy(gennmi_runner *r)
     if(r->graphExec) { hipGraphExecDestroy(r->graphExec); }
     for(hipEvent_t e : r->eventPool) { hipEventDestroy(e); }
     for(hipEvent_t e : r->marks) { if(e) { hipEventDestroy(e); } }
-    for(hipEvent_t e : r->resEvents) { if(e) { hipEventDestroy(e); } }
     for(void *q : r->owned) { hipFree(q); }
     for(void *q : r->zeroOwned) { hipFree(q); }
     for(void *q : r->orderedOwned) { hipFree(q); }
@@ -885,19 +881,13 @@ static int launchResident(gennmi_runner *r, unsigned long long timestep, unsigne
         }
         HIP_TRY(hipGetLastError());
     }
-    // the call's first launch carries a start event and its last one a stop event, bound to the launches themselves (their
-    // own begin and end on the device, no marker of its own in the stream): gennmi_runner_resident_launch_seconds
-    if(!r->resEvents[0]) { HIP_TRY(hipEventCreate(&r->resEvents[0])); HIP_TRY(hipEventCreate(&r->resEvents[1])); }
     for(unsigned long long done = 0; done < numSteps; ) {
         const uint32_t chunk = (uint32_t)std::min(MAX_STEPS, numSteps - done);
         auto launch = r->resPoisson ? residentKernel<true> : residentKernel<false>;
-        hipExtLaunchKernelGGL(launch, dim3(r->resTiles), dim3(BLOCK), (uint32_t)r->resLdsBytes, r->stream,
-            done == 0 ? r->resEvents[0] : nullptr, done + chunk == numSteps ? r->resEvents[1] : nullptr, 0u,
-            (const ResTile*)r->dResTiles, r->resTiles, (const NeuronGroupDev*)r->dResGroups, (const uint8_t*)r->dResTileGroup, r->dResTags, r->dResSide,
-            (unsigned long long)(timestep + done), (unsigned long long)r->epoch, (unsigned long long)numRecordingTimesteps,
-            chunk, r->dt, r->fusedStep ? 1u : 0u, r->dError, r->dEvents, r->resReplicaStride, (unsigned long long)r->resSeq);
+        launch<<<dim3(r->resTiles), dim3(BLOCK), r->resLdsBytes, r->stream>>>(
+            r->dResTiles, r->resTiles, r->dResGroups, r->dResTileGroup, r->dResTags, r->dResSide, timestep + done, r->epoch, numRecordingTimesteps,
+            chunk, r->dt, r->fusedStep ? 1u : 0u, r->dError, r->dEvents, r->resReplicaStride, r->resSeq);
         HIP_TRY(hipGetLastError());
-        r->resEventsSet = true;
         r->resSeq += chunk + 1u;                                   // the launch used sequence numbers resSeq + 1 ... resSeq + chunk + 1 (words hold them modulo 2^23)
         done += chunk;
         r->epoch += chunk;
@@ -2115,18 +2105,6 @@ int gennmi_runner_stream_elapsed(gennmi_runner *r, double *seconds)
     HIP_TRY(hipEventSynchronize(r->marks[1]));
     float ms = 0;
     HIP_TRY(hipEventElapsedTime(&ms, r->marks[0], r->marks[1]));
-    *seconds = ms * 1e-3;
-    return GENNMI_OK;
-}
-
-int gennmi_runner_resident_launch_seconds(gennmi_runner *r, double *seconds)
-{
-    if(!r || !seconds) { return fail(GENNMI_EINVAL, "runner_resident_launch_seconds: null argument"); }
-    FLUSH_QUEUED();
-    if(!r->resEventsSet) { return fail(GENNMI_ESTATE, "runner_resident_launch_seconds: no launch of the resident plan so far"); }
-    HIP_TRY(hipEventSynchronize(r->resEvents[1]));
-    float ms = 0;
-    HIP_TRY(hipEventElapsedTime(&ms, r->resEvents[0], r->resEvents[1]));
     *seconds = ms * 1e-3;
     return GENNMI_OK;
 }

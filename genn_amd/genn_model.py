@@ -1055,12 +1055,6 @@ class GeNNModel:
         _abi.check(_abi.load().gennmi_runner_stream_elapsed(self._runner, C.byref(v)))
         return v.value
 
-    def resident_launch_seconds(self):
-        """Device time of the latest resident-plan call, from events bound to its launches (include/genn_mi355x.h)."""
-        v = C.c_double()
-        _abi.check(_abi.load().gennmi_runner_resident_launch_seconds(self._runner, C.byref(v)))
-        return v.value
-
     def runner_info(self):
         info = (C.c_uint32 * 4)()
         _abi.check(_abi.load().gennmi_runner_get_info(self._runner, C.byref(info)))

@@ -445,13 +445,6 @@ int gennmi_runner_kernel_stats(gennmi_runner *runner, double stats[8]);
  * backendCUDAHIP.cc:36-76 for a caller-chosen region, e.g. a whole gennmi_run_steps replay. */
 int gennmi_runner_stream_mark(gennmi_runner *runner, int which);
 int gennmi_runner_stream_elapsed(gennmi_runner *runner, double *seconds);
-/* Device time of the latest call that stepped the network on the resident plan (gennmi_run_steps, or a flush of queued
- * single steps): from the begin of its first launch to the end of its last, taken from HIP events bound to the launches
- * themselves (hipExtLaunchKernel's start and stop events), so nothing is added to the stream and the figure is the
- * kernel's own duration, the one a kernel trace shows.  Blocks until that launch has completed; GENNMI_ESTATE before the
- * first such launch.  No counterpart in the reference (its Timer brackets a kernel with two recorded events,
- * backendCUDAHIP.cc:36-76). */
-int gennmi_runner_resident_launch_seconds(gennmi_runner *runner, double *seconds);
 /* Launch plan chosen by gennmi_runner_finalise: bit 1 of info[0] is set if gennmi_run_steps keeps the network resident on
  * the chip (many steps per launch: batch 1, static SPARSE projections with ascending rows between LIF / Izhikevich
  * populations, all tiles of 256 neurons resident at once, and room in device memory for a per-(row, tile) table of 32 bytes

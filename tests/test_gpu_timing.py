@@ -74,33 +74,6 @@ def test_counters_under_the_single_launch_and_resident_plans():
     model.unload()
 
 
-def test_duration_of_a_resident_launch_from_events_bound_to_it():
-    """gennmi_runner_resident_launch_seconds: the device time of the latest run() on the resident plan, from start and stop
-    events bound to the launch itself.  It must lie inside what two events recorded around the same call measure (those add a
-    marker on either side of the kernel), inside the wall clock, and it is refused before the first such launch."""
-    import time
-    from genn_amd import _abi
-    net = configs.potjans(neuron_scale=0.05, connectivity_scale=1.0, steps=400)
-    model = model_from_net(net)
-    model.load(num_recording_timesteps=400)
-    assert model.runner_info()["resident_plan"]
-    with pytest.raises(_abi.GennmiError):
-        model.resident_launch_seconds()
-    model.run(100)
-    model.synchronize()
-    t0 = time.perf_counter()
-    model.stream_mark(0)
-    model.run(200)
-    model.stream_mark(1)
-    model.synchronize()
-    wall = time.perf_counter() - t0
-    around = model.stream_elapsed()
-    bound = model.resident_launch_seconds()
-    assert 0.0 < bound <= around <= wall, (bound, around, wall)
-    assert bound > 200 * 1e-6, "two hundred steps of this network take more than a microsecond each"
-    model.unload()
-
-
 def test_counters_through_the_reference_runtime():
     """ModelSpec::setTimingEnabled through the adapter: the generated runner's exported doubles, read by
     Runtime::get*Time (runtime.h:324-333)."""
