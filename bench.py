@@ -235,8 +235,11 @@ def run_net_workload(args, workload, steps, warmup, profile_steps, with_cpu, wit
     model.synchronize()
     load_s = time.time() - t0
 
-    # ---- warm-up (also captures the step graph), then the timed region
+    # ---- warm-up (also captures the step graph; the events are recorded around it too, so that creating them and
+    # recording for the first time — 30 us of host time — is not part of the timed region), then the timed region
+    model.stream_mark(0)
     model.run(warmup)
+    model.stream_mark(1)
     model.synchronize()
     ev0 = model.synaptic_event_count
     t0 = time.perf_counter()
