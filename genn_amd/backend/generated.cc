@@ -447,9 +447,25 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
         os << "if(threadIdx.x == 0u)";
         {
             CodeStream::Scope b(os);
-            os << "const unsigned int arrived = __hip_atomic_fetch_add(gennmiArgs.finished, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);" << std::endl;
-            os << "gennmiLastToFinish = (arrived == gridDim.x * gridDim.y - 1u);" << std::endl;
-            os << "if(gennmiLastToFinish) { __hip_atomic_store(gennmiArgs.finished, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }" << std::endl;
+            // counted in two levels, sixteen work-groups to a word and one word per cache line: atomics on one address complete
+            // one after the other (about 8 ns each), and every work-group waits for the answer to its own
+            os << "const unsigned int linear = blockIdx.y * gridDim.x + blockIdx.x, total = gridDim.x * gridDim.y;" << std::endl;
+            os << "const unsigned int group = linear >> 4, groups = (total + 15u) >> 4;" << std::endl;
+            os << "const unsigned int inGroup = (total - (group << 4) < 16u) ? total - (group << 4) : 16u;" << std::endl;
+            os << "uint32_t *groupWord = gennmiArgs.finished + 32u * (1u + group);" << std::endl;
+            os << "bool last = false;" << std::endl;
+            os << "if(__hip_atomic_fetch_add(groupWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == inGroup - 1u)";
+            {
+                CodeStream::Scope b2(os);
+                os << "__hip_atomic_store(groupWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);" << std::endl;
+                os << "if(__hip_atomic_fetch_add(gennmiArgs.finished, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1u)";
+                {
+                    CodeStream::Scope b3(os);
+                    os << "__hip_atomic_store(gennmiArgs.finished, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);" << std::endl;
+                    os << "last = true;" << std::endl;
+                }
+            }
+            os << "gennmiLastToFinish = last;" << std::endl;
         }
         os << "__syncthreads();" << std::endl;
         os << "if(gennmiLastToFinish)";
@@ -501,8 +517,9 @@ void Backend::genNeuronUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMer
             os << "GENNMI_CHECK(gennmi_memset(p, 0, " << 2 * std::max<size_t>(1, table.numBlocks) * batchSize * (1 + maxEventGroups) << " * sizeof(unsigned long long)));" << std::endl;
             os << "gennmiNeuronAgg = (unsigned long long*)p;" << std::endl;
             if(anyDenDelay) {
-                os << "GENNMI_CHECK(gennmi_malloc(&p, sizeof(uint32_t)));" << std::endl;
-                os << "GENNMI_CHECK(gennmi_memset(p, 0, sizeof(uint32_t)));" << std::endl;
+                const size_t finishedWords = 32 * (2 + (std::max<size_t>(1, table.numBlocks) * batchSize + 15) / 16);       // (a cache line per word: see the kernel's end)
+                os << "GENNMI_CHECK(gennmi_malloc(&p, " << finishedWords << " * sizeof(uint32_t)));" << std::endl;
+                os << "GENNMI_CHECK(gennmi_memset(p, 0, " << finishedWords << " * sizeof(uint32_t)));" << std::endl;
                 os << "gennmiNeuronFinished = (uint32_t*)p;" << std::endl;
             }
             os << "uint32_t module = 0;" << std::endl;
@@ -699,7 +716,10 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
         for(const auto &sg : model.getSynapseGroups()) {
             if(sg.second.isPreSpikeRequired() || sg.second.isPreSpikeEventRequired()) { wanted += presynapticBlocks(sg.second); }
         }
-        constexpr size_t oneRound = 256 * 8;        // work-groups of 256 threads the chip holds at once
+        const char *envRound = std::getenv("GENNMI_GENERATED_PRESYN_BLOCKS_PER_CU");
+        // (work-groups of 256 threads per compute unit that all projections share; the full microcircuit through
+        // Runtime::stepTime with 1 / 2 / 4 / 8 / 16 / 32: 38.2 / 26.8 / 20.6 / 18.3 / 17.8 / 18.0 us per step)
+        const size_t oneRound = 256 * (envRound ? (size_t)std::max(1, std::atoi(envRound)) : 16);
         if(wanted > oneRound) { presynapticScale = (double)oneRound / (double)wanted; }
     }
     {
