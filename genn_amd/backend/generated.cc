@@ -778,14 +778,23 @@ void Backend::genSynapseUpdateGenerated(CodeStream &os, ModelSpecMerged &modelMe
                         // (axonal delay: the slot of the source's ring written `delay` steps ago, presynapticUpdateStrategySIMT.cc:224-247)
                         const bool preDelay = src->isDelayRequired() && (trueSpike ? src->isSpikeQueueRequired() : src->isSpikeEventQueueRequired());
                         CodeStream::Scope b1(groupEnv.getStream());
+                        // (the queue entry of an item is asked for one item ahead, the first one together with the count: the queue
+                        // always holds num_pre entries, so any index below that is readable, and an item's chain of dependent loads
+                        // is row -> synapses instead of count -> entry -> row -> synapses)
+                        groupEnv.getStream() << "unsigned long long item = entry.blockInGroup * 4u + (threadIdx.x / 64u);" << std::endl;
+                        groupEnv.printLine("unsigned int spikeNext = (unsigned int)min(item / chunksPerRow, (unsigned long long)($(num_pre) - 1u));");
+                        groupEnv.printLine("unsigned int idPreNext = $(_src_spk" + suffix + ")[" + s.getPreVarIndex(preDelay, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "spikeNext") + "];");
                         groupEnv.printLine("const unsigned int numSpikes = $(_src_spk_cnt" + suffix + ")[" + s.getPreSlot(preDelay, batchSize) + "];");
                         groupEnv.getStream() << "const unsigned long long numItems = (unsigned long long)numSpikes * chunksPerRow;" << std::endl;
-                        groupEnv.getStream() << "for(unsigned long long item = entry.blockInGroup * 4u + (threadIdx.x / 64u); item < numItems; item += numWaves)";
+                        groupEnv.getStream() << "while(item < numItems)";
                         CodeStream::Scope b2(groupEnv.getStream());
                         EnvironmentGroupMergedField<PresynapticUpdateGroupMerged> synEnv(groupEnv, s);
                         synEnv.getStream() << "const unsigned int spike = (unsigned int)(item / chunksPerRow);" << std::endl;
                         synEnv.getStream() << "const unsigned int j = (unsigned int)(item % chunksPerRow) * 64u + (threadIdx.x & 63u);" << std::endl;
-                        synEnv.printLine("const unsigned int idPre = $(_src_spk" + suffix + ")[" + s.getPreVarIndex(preDelay, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "spike") + "];");
+                        synEnv.getStream() << "const unsigned int idPre = idPreNext;" << std::endl;
+                        synEnv.getStream() << "item += numWaves;" << std::endl;
+                        synEnv.printLine("spikeNext = (unsigned int)min(item / chunksPerRow, (unsigned long long)($(num_pre) - 1u));");
+                        synEnv.printLine("idPreNext = $(_src_spk" + suffix + ")[" + s.getPreVarIndex(preDelay, batchSize, VarAccessDim::BATCH | VarAccessDim::ELEMENT, "spikeNext") + "];");
                         synEnv.add(Type::Uint32.addConst(), "id_pre", "idPre");
                         if(procedural) {
                             // A row of a PROCEDURAL matrix is the connectivity snippet's row build code, run afresh for every spike:

@@ -295,7 +295,7 @@ def test_generated_kernels_take_the_batch_from_the_grid():
         assert "u, 2u, 256u, &a, sizeof(a)" in neuron and "u, 2u, 256u, &a, sizeof(a)" in synapse
         assert "group->A[batchOffset + id]" in neuron and "[blockIdx.y] = slot.total" in neuron
         assert "(size_t)recordingTimestep * 2u + blockIdx.y" in neuron
-        assert "group->srcSpk[preBatchOffset + spike]" in synapse and "group->wPost[synBatchOffset + idSyn]" in synapse
+        assert "group->srcSpk[preBatchOffset + spikeNext]" in synapse and "group->wPost[synBatchOffset + idSyn]" in synapse
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
 
