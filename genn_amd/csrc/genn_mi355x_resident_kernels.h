@@ -579,12 +579,6 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         const unsigned long long ballot = __ballot(spiked);
         const uint32_t laneRank = __popcll(ballot & ((1ull << lane) - 1ull));
         if(lane == 0) { shWave[wave] = __popcll(ballot); }
-        if(recordSpk && (lane & 31) == 0 && mine) {
-            const unsigned long long ts = timestep0 + k;
-            const uint32_t recT = numRecordingTimesteps ? (((ts | numRecordingTimesteps) >> 32) ? (uint32_t)(ts % numRecordingTimesteps)
-                                                                                                : ((uint32_t)ts % (uint32_t)numRecordingTimesteps)) : 0u;
-            recordSpk[(size_t)recT * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
-        }
         __syncthreads();
         uint32_t waveOffset = 0;
         ownCount = 0;
@@ -597,7 +591,14 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         if(spiked) { shOwn[waveOffset + laneRank] = i; }
         __syncthreads();
         publish(k + 2, ownCount);
-        // while the words of this step travel: the synapses of the previous step's spikes that are not due yet
+        // while the words of this step travel: the step's recording words, and the synapses of the previous step's spikes
+        // that are not due yet
+        if(recordSpk && (lane & 31) == 0 && mine) {
+            const unsigned long long ts = timestep0 + k;
+            const uint32_t recT = numRecordingTimesteps ? (((ts | numRecordingTimesteps) >> 32) ? (uint32_t)(ts % numRecordingTimesteps)
+                                                                                                : ((uint32_t)ts % (uint32_t)numRecordingTimesteps)) : 0u;
+            recordSpk[(size_t)recT * ((n + 31) / 32) + (i >> 5)] = (uint32_t)(ballot >> (lane & 32));
+        }
         deliverLater(later);
     }
 
