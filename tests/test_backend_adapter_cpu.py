@@ -181,7 +181,7 @@ def _generate_with(case, *options):
 
 
 @pytest.mark.parametrize("case, options", [("custom_update_small", ("--kernels=generated",)), ("va_double_small", ()), ("post_events_small", ()), ("custom_small", ()), ("dynamic_small", ()), ("poisson_input_small", ()), ("synapse_dynamics_small", ()), ("prev_times_small", ()), ("stdp_delay_small", ()), ("graded_small", ("--kernels=generated",)), ("conv_small", ("--kernels=generated",)), ("procedural", ("--kernels=generated",)), ("dense_small", ("--kernels=generated",)), ("stdp_small", ("--kernels=generated",)),
-                                           ("va_small", ("--dynamic=neuron:E.Ioffset",))])
+                                           ("va_small", ("--dynamic=neuron:E.Ioffset",)), ("potjans_small", ("--kernels=generated",))])
 def test_generated_kernels_are_chosen_and_build(case, options):
     """Models of the driver's own, dynamic parameters, or Preferences::kernelSource = GENERATED: the modules then hold device
     code (the model's snippets inside this backend's kernel skeletons), built into gfx950 code objects by the runner's own
@@ -219,6 +219,13 @@ def test_generated_kernels_are_chosen_and_build(case, options):
             assert "group->variableTranspose[" in custom and "gennmiTile[tx][ty + j]" in custom
             assert "if(col < group->rowLength[row])" in custom
             assert "gennmiUploadCustomUpdateGroups();" in open(os.path.join(code, "runner.cc")).read()
+        if case == "potjans_small":
+            # dendritic delay: the neuron update's last work-group moves the ring pointers on; it is found by a count in two
+            # levels (sixteen work-groups to a word, a cache line per word), not by every work-group adding to one word
+            assert "gennmiLastToFinish = last;" in neuron and "gennmiArgs.finished + 32u * (1u + group)" in neuron
+            assert "* sizeof(uint32_t)));" in neuron and "GENNMI_CHECK(gennmi_malloc(&p, sizeof(uint32_t)));" not in neuron
+            # the presynaptic walk asks for an item's queue entry one item ahead
+            assert "idPreNext = group->srcSpk[" in synapse and "const unsigned int idPre = idPreNext;" in synapse
         if case == "custom_small":
             # the extra state variable and the weight-update variables are in the kernels under the reference's names
             assert "group->A[id]" in neuron and "sPreOutSynWUMPre" in neuron and "sPostInSynWUMPost" in neuron
