@@ -652,7 +652,9 @@ __device__ __forceinline__ void neuronBulkBody(const NeuronGroupDev &G, uint32_t
             if(m < numPSM) {
                 const uint32_t D = psmD[m];
                 if(D) { psmRing[m][((size_t)batch * D + modStep(st.epoch + 1, D)) * n + i] = 0.0f; }
-                psmOut[m][bi] = outLin[j][m];
+                // (an input that is the same bits as it was read — a DeltaCurr input that received nothing: zero in, zero out —
+                // is not written again: in a quiet step that is most of a population's 4 bytes per neuron)
+                if(__float_as_uint(outLin[j][m]) != __float_as_uint(lin[j][m])) { psmOut[m][bi] = outLin[j][m]; }
             }
         }
         var0[bi] = l0[j]; var1[bi] = l1[j];
