@@ -38,9 +38,9 @@ BYTES_PER_EVENT = {"dense": 4,          # one weight read per (spike, target); o
 # its seed and therefore its activity are then identical); any other run reports null.
 # The kernel's source is named with a digest: a figure measured on another version of the kernel is not attached.
 MEASURED_TRAFFIC_BYTES = {
-    ("potjans", 20, 5): {"plan": "resident", "bytes_per_launch": 155167200,
-                         "kernel_source": ("genn_amd/csrc/genn_mi355x_resident_kernels.h", "16ddbf08db441d1c"),
-                         "source": "rocprofv3 --pmc FETCH_SIZE (67668.13 x 2 KiB) + WRITE_SIZE (16194.22 x 1 KiB) of the timed 20-step "
+    ("potjans", 20, 5): {"plan": "resident", "bytes_per_launch": 155216672,
+                         "kernel_source": ("genn_amd/csrc/genn_mi355x_resident_kernels.h", "861e3def22045d8a"),
+                         "source": "rocprofv3 --pmc FETCH_SIZE (67692.56 x 2 KiB) + WRITE_SIZE (16193.66 x 1 KiB) of the timed 20-step "
                                    "launch, profiles/residentKernel_potjans_full.md"},
     ("conv", 1000, 100): {"plan": "stepped", "requires": "conv_step_in_one_launch", "bytes_per_launch": 66118287,
                           "kernel_source": ("genn_amd/csrc/genn_mi355x_conv_step_kernels.h", "b33aec4cfae473d9"),

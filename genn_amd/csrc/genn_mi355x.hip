@@ -61,7 +61,7 @@ struct gennmi_runner
     NeuronGroupDev *dNeuron = nullptr; PreGroupDev *dPre = nullptr; PostGroupDev *dPost = nullptr;
     uint32_t neuronBlocks = 0, preBlocks = 0, postBlocks = 0;
     unsigned long long *dAgg = nullptr; uint32_t *dError = nullptr; unsigned long long *dEvents = nullptr;
-    uint32_t *hError = nullptr;     // pinned host word that the error flag is copied into on the runner's stream, ahead of a wait
+    uint32_t *hError = nullptr;     // the error flag: a pinned host word; dError is the same word's device address
     StepState *dState = nullptr;
     unsigned long long epoch = 0;       // completed steps (host mirror)
     bool synapsesDone = false;          // updateSynapses ran for the current step
@@ -484,10 +484,11 @@ int gennmi_runner_create(gennmi_runner **runner, float dt, uint32_t batchSize)
     gennmi_runner *r = new gennmi_runner;
     r->dt = dt; r->batch = batchSize;
     HIP_TRY(hipStreamCreate(&r->stream));       // blocking stream: ordered against null-stream copies
-    HIP_TRY(hipMalloc(&r->dError, sizeof(uint32_t)));
-    HIP_TRY(hipMemset(r->dError, 0, sizeof(uint32_t)));
-    HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&r->hError), sizeof(uint32_t), hipHostMallocDefault));
+
+    // the error flag: one pinned host word, which the kernels reach through its device address (raiseErrorFlag)
+    HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&r->hError), sizeof(uint32_t), hipHostMallocMapped | hipHostMallocCoherent));
     *r->hError = 0;
+    HIP_TRY(hipHostGetDevicePointer(reinterpret_cast<void**>(&r->dError), r->hError, 0));
     HIP_TRY(hipMalloc(&r->dEvents, sizeof(unsigned long long) * EVENT_SLOTS * EVENT_SLOT_STRIDE));
     HIP_TRY(hipMemset(r->dEvents, 0, sizeof(unsigned long long) * EVENT_SLOTS * EVENT_SLOT_STRIDE));
     HIP_TRY(hipMalloc(&r->dState, sizeof(StepState)));
@@ -517,7 +518,7 @@ int gennmi_runner_destroy(gennmi_runner *r)
     for(void *q : r->orderedOwned) { hipFree(q); }
     hipFree(r->dOrderedSources); hipFree(r->dOrderedBitmaps);
     hipFree(r->dTile); hipFree(r->dConvTile);
-    hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dDense); hipFree(r->dProc); hipFree(r->dAgg); hipFree(r->dError); if(r->hError) { hipHostFree(r->hError); } hipFree(r->dEvents); hipFree(r->dState);
+    hipFree(r->dNeuron); hipFree(r->dPre); hipFree(r->dPost); hipFree(r->dDense); hipFree(r->dProc); hipFree(r->dAgg); if(r->hError) { hipHostFree(r->hError); } hipFree(r->dEvents); hipFree(r->dState);
     hipStreamDestroy(r->stream);
     delete r;
     return GENNMI_OK;
@@ -857,6 +858,7 @@ static int setupResident(gennmi_runner *r, uint32_t numCU)
 static int launchResident(gennmi_runner *r, unsigned long long timestep, unsigned long long numSteps, unsigned long long numRecordingTimesteps)
 {
     constexpr unsigned long long MAX_STEPS = 1ull << 20;
+    if(*r->hError) { return fail(GENNMI_EDEVICE, "a kernel's bounded wait for other work-groups expired earlier; the runner's state is undefined"); }
     bool stale;
     std::vector<uint8_t> staleProj;
     {
@@ -2041,9 +2043,7 @@ int gennmi_runner_synchronize(gennmi_runner *r)
 {
     if(!r) { return fail(GENNMI_EINVAL, "runner_synchronize: null runner"); }
     FLUSH_QUEUED();
-    // (the flag travels on the stream behind the queued work, so that one wait covers both: a blocking copy after the wait
-    // would cost a second round trip, as long as several steps of a small model)
-    HIP_TRY(hipMemcpyAsync(r->hError, r->dError, sizeof(uint32_t), hipMemcpyDeviceToHost, r->stream));
+    // (the flag is host memory the kernels write: nothing to copy, it is read below once the stream has drained)
     // (short waits are polled: a blocking wait wakes up some tens of microseconds after the work has ended; GENNMI_POLL_US=0 blocks at once)
     static const long pollMicroseconds = [] { const char *e = getenv("GENNMI_POLL_US"); return e ? atol(e) : 500l; }();
     if(pollMicroseconds > 0) {

@@ -241,6 +241,14 @@ __device__ __forceinline__ void ldsAddF32(float *addr, float v)
     } while(old != assumed);
 }
 
+// The runner's error flag lives in pinned host memory that the device sees too: a bounded wait that expires stores 1 there
+// (the flag only ever goes from 0 to 1, so a store does what an atomic OR would, on any kind of memory), and the host reads
+// the word after waiting for the stream — no copy command behind every launch (3.5 us per launch and wait).
+__device__ __forceinline__ void raiseErrorFlag(uint32_t *errorFlag)
+{
+    __hip_atomic_store(errorFlag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // The runner's count of synaptic events is kept as EVENT_SLOTS partial counts a cache line apart (the host adds them up):
 // atomics on ONE address complete one after the other, about 8 ns each, so a launch whose thousand wavefronts each add
 // their share to a single counter ends 8 us after its last useful instruction — and any barrier behind such an add waits

@@ -92,7 +92,7 @@ __device__ __forceinline__ uint32_t blockQueueOffset(uint32_t blockCount, uint32
         }
         const bool allOk = (__ballot(!ok) == 0ull);
         if(lane == 0) {
-            if(!allOk) { atomicOr(errorFlag, 1u); sum = 0xFFFFFFFFu; }
+            if(!allOk) { raiseErrorFlag(errorFlag); sum = 0xFFFFFFFFu; }
             *shOffset = sum;
         }
     }
@@ -404,7 +404,7 @@ __device__ __forceinline__ void neuronBody(const NeuronGroupDev &G, uint32_t blo
         }
         const bool allOk = (__ballot(!ok) == 0ull);
         if(lane == 0) {
-            if(!allOk) { atomicOr(errorFlag, 1u); sum = 0xFFFFFFFFu; }
+            if(!allOk) { raiseErrorFlag(errorFlag); sum = 0xFFFFFFFFu; }
             shPrefix = sum;
         }
     }

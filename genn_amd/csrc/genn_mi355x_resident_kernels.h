@@ -163,10 +163,10 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
     const bool mine = tid < T.count;
     const uint32_t numPSM = g.numPSM, numCS = g.numCS;
 
-    // a launch that finds the error flag raised (an earlier work-group gave up waiting) leaves at once, as one
-    if(tid == 0) { shScalar[3] = __hip_atomic_load(errorFlag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    // (a runner whose error flag is raised launches nothing more: the host looks at the flag before every launch; the flag
+    // is host memory, and reading it here would put a trip over the bus in front of every launch)
+    if(tid == 0) { shScalar[3] = 0u; }
     __syncthreads();
-    if(shScalar[3]) { return; }
 
     // ---- tables into LDS
     for(uint32_t k = tid; k < numTiles; k += BLOCK) { shTileGroup[k] = tileGroup[k]; }
@@ -325,7 +325,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         if(!ok) { shScalar[3] = 1u; }                  // (zero since the launch began: a launch that finds the error flag raised has left)
         __syncthreads();
         if(shScalar[3]) {
-            if(tid == 0) { atomicOr(errorFlag, 1u); }
+            if(tid == 0) { raiseErrorFlag(errorFlag); }
             return false;
         }
         // front slot of every projection's ring in the step this exchange feeds
@@ -358,7 +358,7 @@ void residentKernel(const ResTile * __restrict__ tiles, uint32_t numTiles, const
         if(!ok) { shScalar[3] = 1u; }
         __syncthreads();
         if(shScalar[3]) {
-            if(tid == 0) { atomicOr(errorFlag, 1u); }
+            if(tid == 0) { raiseErrorFlag(errorFlag); }
             return false;
         }
         return true;
